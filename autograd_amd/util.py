@@ -1,0 +1,68 @@
+"""Small helpers shared by the tracer and the rule tables.
+
+Behavioural counterpart of the reference's autograd/util.py:4-40 (tuple
+substitution helpers and the reverse topological ordering used by the backward
+replay).
+"""
+
+from operator import attrgetter
+
+__all__ = ["subvals", "subval", "func", "toposort"]
+
+
+def subvals(seq, index_value_pairs):
+    """Return ``tuple(seq)`` with ``seq[i]`` replaced by ``v`` for each ``(i, v)``."""
+    out = list(seq)
+    for i, v in index_value_pairs:
+        out[i] = v
+    return tuple(out)
+
+
+def subval(seq, index, value):
+    """Single-position form of :func:`subvals`."""
+    out = list(seq)
+    out[index] = value
+    return tuple(out)
+
+
+def func(f):
+    """Identity; lets ``func(Class.method)`` read the same for bound primitives."""
+    return f
+
+
+_get_parents = attrgetter("parents")
+
+
+def toposort(end_node, parents=_get_parents):
+    """Yield the nodes reachable from ``end_node``, every node after all of its children.
+
+    The visiting order is part of the contract (reference autograd/util.py:21-40):
+    the order in which cotangent contributions reach a node fixes the floating
+    point order of their accumulation.  Phase one counts, by a depth-first walk
+    with an explicit LIFO stack, how many times each node is reached as a
+    parent.  Phase two keeps a LIFO stack of nodes whose children have all been
+    emitted; a parent is pushed when its last child is emitted, so for a node
+    with several parents the subtree of the last-listed parent that became
+    ready is replayed first.
+    """
+    pending_children = {}
+    work = [end_node]
+    while work:
+        node = work.pop()
+        seen = pending_children.get(node)
+        if seen is None:
+            pending_children[node] = 1
+            work.extend(parents(node))
+        else:
+            pending_children[node] = seen + 1
+
+    ready = [end_node]
+    while ready:
+        node = ready.pop()
+        yield node
+        for parent in parents(node):
+            remaining = pending_children[parent]
+            if remaining == 1:
+                ready.append(parent)
+            else:
+                pending_children[parent] = remaining - 1
