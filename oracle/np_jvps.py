@@ -112,7 +112,7 @@ for _name, _rule in _unary.items():
 
 defjvp(anp.clip, lambda g, ans, x, a_min, a_max: g * anp.logical_and(ans != a_min, ans != a_max))
 defjvp(
-    anp.where,
+    anp._raw_where,
     None,
     lambda g, ans, c, x=None, y=None: anp.where(c, g, anp.zeros(anp.shape(g))),
     lambda g, ans, c, x=None, y=None: anp.where(c, anp.zeros(g.shape), g),
@@ -122,6 +122,34 @@ defjvp(
     lambda g, ans, x, axis=None, keepdims=False, **kwargs: ans * anp.sum(g / x, axis=axis, keepdims=keepdims),
 )
 defjvp(anp._astype, lambda g, ans, A, dtype, *a, **k: anp._astype(g, dtype))
+
+
+def _num_reps(g, axis):
+    if axis is None:
+        return anp.size(g)
+    if isinstance(axis, int):
+        return anp.shape(g)[axis]
+    return anp.prod(anp.array(anp.shape(g))[list(axis)])
+
+
+def _fwd_var(g, ans, x, axis=None, ddof=0, keepdims=False, **kwargs):
+    # numpy_jvps.py:165-177
+    num_reps = _num_reps(g, axis)
+    x_minus_mean = anp.conj(x - anp.mean(x, axis=axis, keepdims=True))
+    return 2.0 * anp.sum(anp.real(g * x_minus_mean), axis=axis, keepdims=keepdims) / (num_reps - ddof)
+
+
+def _fwd_std(g, ans, x, axis=None, ddof=0, keepdims=False, **kwargs):
+    # numpy_jvps.py:180-193
+    num_reps = _num_reps(g, axis)
+    if num_reps <= 1:
+        return anp.zeros_like(ans)
+    x_minus_mean = anp.conj(x - anp.mean(x, axis=axis, keepdims=True))
+    return anp.sum(anp.real(g * x_minus_mean), axis=axis, keepdims=keepdims) / ((num_reps - ddof) * ans)
+
+
+defjvp(anp._primitive_var, _fwd_var)
+defjvp(anp._primitive_std, _fwd_std)
 
 
 def _fwd_chooser(g, ans, x, axis=None, keepdims=False, **kwargs):

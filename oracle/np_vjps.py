@@ -158,7 +158,7 @@ defvjp(anp.triu, lambda ans, x, k=0: lambda g: anp.triu(g, k=k))
 defvjp(anp.tril, lambda ans, x, k=0: lambda g: anp.tril(g, k=k))
 defvjp(anp.clip, lambda ans, x, a_min, a_max: lambda g: g * anp.logical_and(ans != a_min, ans != a_max))
 defvjp(
-    anp.where,
+    anp._raw_where,
     None,
     lambda ans, c, x=None, y=None: lambda g: anp.where(c, g, anp.zeros(g.shape)),
     lambda ans, c, x=None, y=None: lambda g: anp.where(c, anp.zeros(g.shape), g),
