@@ -1,0 +1,301 @@
+"""ctypes binding of ``libagmi.so`` (the C ABI declared in ``include/agmi.h``).
+
+This module is the only place that touches the native library.  Everything above
+it works with ``torch.Tensor`` objects, which are used purely as device-memory
+handles (allocation through torch's caching allocator, views as metadata,
+``data_ptr()`` + element strides handed to the kernels, launches on torch's
+current HIP stream).  No arithmetic is ever done by torch.
+
+There is NO fallback: if the library is missing or a launch is rejected, the
+call raises.
+"""
+
+import ctypes
+import os
+
+import numpy as onp
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.environ.get("AGMI_LIBRARY", os.path.join(_HERE, "libagmi.so"))
+
+MAX_DIMS = 8
+MAX_IN = 4
+MAX_OUT = 2
+
+# agmi_dtype
+F32, F64, BOOL, I64, I32 = 0, 1, 2, 3, 4
+DTYPE_CODE = {
+    onp.dtype("float32"): F32,
+    onp.dtype("float64"): F64,
+    onp.dtype("bool"): BOOL,
+    onp.dtype("int64"): I64,
+    onp.dtype("int32"): I32,
+}
+TORCH_DTYPE = {
+    onp.dtype("float32"): torch.float32,
+    onp.dtype("float64"): torch.float64,
+    onp.dtype("bool"): torch.bool,
+    onp.dtype("int64"): torch.int64,
+    onp.dtype("int32"): torch.int32,
+}
+NUMPY_DTYPE = {v: k for k, v in TORCH_DTYPE.items()}
+
+
+# agmi_op (values fixed by include/agmi.h)
+class Op:
+    COPY, NEG, EXP, LOG, TANH, SINH, COSH, SIN, COS, SQRT, SQUARE, ABS, SIGN, RECIPROCAL, LOG1P, EXPM1 = range(16)
+    ADD, SUB, MUL, DIV, POW, MAXIMUM, MINIMUM = range(32, 39)
+    WHERE = 64
+    (
+        DIV_VJP1,
+        TANH_VJP,
+        POW_VJP0,
+        POW_VJP1,
+        LSE_VJP,
+        RECIPROCAL_VJP,
+        SQRT_VJP,
+        SIN_VJP,
+        COS_VJP,
+        SINH_VJP,
+        COSH_VJP,
+        SQUARE_VJP,
+        ABS_VJP,
+        CHOOSE_VJP,
+        LOG1P_VJP,
+        EXPM1_VJP,
+        DIV_VJP_BOTH,
+        MUL_ADD,
+    ) = range(96, 114)
+
+
+class Cmp:
+    EQ, NE, LT, LE, GT, GE = range(6)
+
+
+class Red:
+    SUM, MAX, MIN, PROD, LOGSUMEXP = range(5)
+
+
+# ops agmi_map_reduce can fuse in front of a sum (reduce.hip: AGMI_FOR_EACH_REDUCE_OP)
+REDUCE_FUSABLE = frozenset(
+    {Op.COPY, Op.NEG, Op.MUL, Op.DIV, Op.SQUARE, Op.ABS, Op.DIV_VJP1, Op.TANH_VJP, Op.POW_VJP0, Op.POW_VJP1,
+     Op.LSE_VJP, Op.CHOOSE_VJP}
+)
+
+
+class AgmiArray(ctypes.Structure):
+    _fields_ = [("data", ctypes.c_void_p), ("strides", ctypes.c_int64 * MAX_DIMS)]
+
+
+class AgmiError(RuntimeError):
+    pass
+
+
+_LIB = None
+
+
+def lib():
+    """Load ``libagmi.so`` once.  Raises ImportError when it has not been built."""
+    global _LIB
+    if _LIB is not None:
+        return _LIB
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} not found: the HIP library is not built. Run `make -C autograd_amd/csrc` "
+            "(or `python -c 'import __graft_entry__ as g; g.build()'`). There is no CPU fallback."
+        )
+    L = ctypes.CDLL(LIB_PATH)
+    c_i, c_i64, c_d, c_p, c_sz = ctypes.c_int, ctypes.c_int64, ctypes.c_double, ctypes.c_void_p, ctypes.c_size_t
+    p_i64 = ctypes.POINTER(ctypes.c_int64)
+    p_arr = ctypes.POINTER(AgmiArray)
+    p_d = ctypes.POINTER(ctypes.c_double)
+    p_u8 = ctypes.POINTER(ctypes.c_uint8)
+    L.agmi_last_error.restype = ctypes.c_char_p
+    L.agmi_last_error.argtypes = []
+    L.agmi_version.restype = c_i
+    L.agmi_version.argtypes = []
+    L.agmi_elementwise.restype = c_i
+    L.agmi_elementwise.argtypes = [c_i, c_i, c_i, p_i64, c_i, p_arr, c_i, p_arr, p_d, c_p]
+    L.agmi_compare.restype = c_i
+    L.agmi_compare.argtypes = [c_i, c_i, c_i, p_i64, p_arr, p_arr, p_d, c_p]
+    L.agmi_cast.restype = c_i
+    L.agmi_cast.argtypes = [c_i, c_i, c_i, p_i64, p_arr, p_arr, c_p]
+    L.agmi_map_reduce.restype = c_i
+    L.agmi_map_reduce.argtypes = [c_i, c_i, c_i, c_i, p_i64, p_u8, p_arr, c_i, p_arr, p_d, c_p, c_sz, c_p]
+    L.agmi_map_reduce_workspace_bytes.restype = c_sz
+    L.agmi_map_reduce_workspace_bytes.argtypes = [c_i, c_i, c_i, p_i64, p_u8]
+    L.agmi_gemm.restype = c_i
+    L.agmi_gemm.argtypes = [c_i, c_i64, c_i64, c_i64, c_i64, c_d, c_p, c_i64, c_i64, c_i64, c_p, c_i64, c_i64,
+                            c_i64, c_d, c_p, c_i64, c_i64, c_p]
+    L.agmi_fill.restype = c_i
+    L.agmi_fill.argtypes = [c_i, c_p, c_i64, c_d, c_p]
+    L.agmi_take_rows.restype = c_i
+    L.agmi_take_rows.argtypes = [c_i, c_p, c_i64, c_i64, c_p, c_i64, c_p, c_p]
+    L.agmi_scatter_add_rows.restype = c_i
+    L.agmi_scatter_add_rows.argtypes = [c_i, c_p, c_i64, c_i64, c_p, c_p, c_p, c_p, c_i64, c_p]
+    _LIB = L
+    return L
+
+
+EXPORTS = (
+    "agmi_last_error agmi_version agmi_elementwise agmi_compare agmi_cast agmi_map_reduce "
+    "agmi_map_reduce_workspace_bytes agmi_gemm agmi_fill agmi_take_rows agmi_scatter_add_rows"
+).split()
+
+
+def _check(rc, what):
+    if rc != 0:
+        msg = lib().agmi_last_error().decode("utf-8", "replace")
+        raise AgmiError(f"{what} failed (code {rc}): {msg}")
+
+
+# ---- device / stream ---------------------------------------------------------------------
+_DEVICE = None
+
+
+def device():
+    """The GPU all device arrays live on.  Raises when no GPU is visible."""
+    global _DEVICE
+    if _DEVICE is None:
+        if not torch.cuda.is_available():
+            raise RuntimeError(
+                "autograd_amd needs an AMD GPU (MI355X / gfx950) visible to PyTorch-ROCm; none found. "
+                "There is no CPU fallback."
+            )
+        _DEVICE = torch.device("cuda", torch.cuda.current_device())
+        lib()
+    return _DEVICE
+
+
+def _stream():
+    return torch._C._cuda_getCurrentRawStream(_DEVICE.index)
+
+
+def empty(shape, np_dtype):
+    return torch.empty(tuple(shape), dtype=TORCH_DTYPE[np_dtype], device=device())
+
+
+def synchronize():
+    torch.cuda.synchronize(device())
+
+
+# ---- argument marshalling (buffers reused: single-threaded by contract) ----------------------
+_outs = (AgmiArray * MAX_OUT)()
+_ins = (AgmiArray * MAX_IN)()
+_shape = (ctypes.c_int64 * MAX_DIMS)()
+_scalars = (ctypes.c_double * MAX_IN)()
+_mask = (ctypes.c_uint8 * MAX_DIMS)()
+
+
+def _set_array(slot, t):
+    slot.data = t.data_ptr()
+    st = slot.strides
+    for d, s in enumerate(t.stride()):
+        st[d] = s
+
+
+def _set_shape(shape):
+    n = len(shape)
+    if n > MAX_DIMS:
+        raise AgmiError(f"rank {n} arrays are not supported (max {MAX_DIMS})")
+    for d, s in enumerate(shape):
+        _shape[d] = s
+    return n
+
+
+def _set_inputs(ins):
+    for k, x in enumerate(ins):
+        if isinstance(x, torch.Tensor):
+            _set_array(_ins[k], x)
+        else:
+            _ins[k].data = None
+            _scalars[k] = x
+    return len(ins)
+
+
+def elementwise(op, code, shape, outs, ins):
+    """``outs[k][idx] = op(ins...)`` over ``shape``.
+
+    ``outs`` are tensors of exactly ``shape``; ``ins`` are tensors already expanded to
+    ``shape`` (stride 0 on broadcast axes) or Python floats (by-value scalars).
+    """
+    nd = _set_shape(shape)
+    for k, t in enumerate(outs):
+        _set_array(_outs[k], t)
+    n_in = _set_inputs(ins)
+    rc = _LIB.agmi_elementwise(op, code, nd, _shape, len(outs), _outs, n_in, _ins, _scalars, _stream())
+    if rc:
+        _check(rc, "agmi_elementwise")
+
+
+def compare(cmp, code, shape, out, ins):
+    nd = _set_shape(shape)
+    _set_array(_outs[0], out)
+    _set_inputs(ins)
+    _check(_LIB.agmi_compare(cmp, code, nd, _shape, _outs, _ins, _scalars, _stream()), "agmi_compare")
+
+
+def cast(src_code, dst_code, shape, out, src):
+    nd = _set_shape(shape)
+    _set_array(_outs[0], out)
+    _set_array(_ins[0], src)
+    _check(_LIB.agmi_cast(src_code, dst_code, nd, _shape, _outs, _ins, _stream()), "agmi_cast")
+
+
+_WORKSPACE = None
+_WORKSPACE_BYTES = 32 << 20
+
+
+def _workspace():
+    global _WORKSPACE
+    if _WORKSPACE is None:
+        _WORKSPACE = torch.empty(_WORKSPACE_BYTES, dtype=torch.uint8, device=device())
+    return _WORKSPACE
+
+
+def map_reduce(op, red, code, shape, reduce_mask, out, ins):
+    """``out[kept] = RED over masked axes of op(ins...)``.
+
+    ``out`` is a tensor whose strides are given for ALL axes of ``shape`` (any value on the
+    reduced ones); ``ins`` as in :func:`elementwise`.  Returns False when the reduced axes do
+    not form one group after merging (caller then reduces in two steps).
+    """
+    nd = _set_shape(shape)
+    for d, m in enumerate(reduce_mask):
+        _mask[d] = 1 if m else 0
+    _set_array(_outs[0], out)
+    n_in = _set_inputs(ins)
+    ws = _workspace()
+    rc = _LIB.agmi_map_reduce(op, red, code, nd, _shape, _mask, _outs, n_in, _ins, _scalars, ws.data_ptr(),
+                              _WORKSPACE_BYTES, _stream())
+    if rc == -2:  # AGMI_ERR_UNSUPPORTED
+        return False
+    if rc:
+        _check(rc, "agmi_map_reduce")
+    return True
+
+
+def gemm(code, batch, M, N, K, alpha, A, a_rs, a_cs, a_bs, B, b_rs, b_cs, b_bs, beta, C, ldc, c_bs):
+    rc = _LIB.agmi_gemm(code, batch, M, N, K, alpha, A.data_ptr(), a_rs, a_cs, a_bs, B.data_ptr(), b_rs, b_cs, b_bs,
+                        beta, C.data_ptr(), ldc, c_bs, _stream())
+    if rc:
+        _check(rc, "agmi_gemm")
+
+
+def fill(code, t, value):
+    """Fill a CONTIGUOUS tensor."""
+    rc = _LIB.agmi_fill(code, t.data_ptr(), t.numel(), float(value), _stream())
+    if rc:
+        _check(rc, "agmi_fill")
+
+
+def take_rows(code, src, n_rows, inner, index, n_index, out):
+    _check(_LIB.agmi_take_rows(code, src.data_ptr(), n_rows, inner, index.data_ptr(), n_index, out.data_ptr(),
+                               _stream()), "agmi_take_rows")
+
+
+def scatter_add_rows(code, dst, n_rows, inner, src, index, order, seg_start, n_seg):
+    _check(_LIB.agmi_scatter_add_rows(code, dst.data_ptr(), n_rows, inner, src.data_ptr(), index.data_ptr(),
+                                      order.data_ptr(), seg_start.data_ptr(), n_seg, _stream()),
+           "agmi_scatter_add_rows")

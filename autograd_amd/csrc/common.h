@@ -1,0 +1,54 @@
+// Host-side helpers shared by the kernel files of libagmi.so: error reporting, dtype
+// dispatch and the axis-merging planner that turns an N-d strided index space into the
+// smallest equivalent one.  gfx950 only; no other target is considered anywhere.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "agmi.h"
+
+namespace agmi {
+
+void set_error(const char *fmt, ...);
+int hip_check(hipError_t e, const char *what);
+
+constexpr int kBlock = 256;        // 4 wavefronts of 64 lanes
+constexpr int kMaxMerged = 6;      // rank the strided kernels index with div/mod
+constexpr int kMaxOperands = AGMI_MAX_INPUTS + AGMI_MAX_OUTPUTS;
+
+inline size_t dtype_size(int dtype) {
+    switch (dtype) {
+        case AGMI_F32: return 4;
+        case AGMI_F64: return 8;
+        case AGMI_BOOL: return 1;
+        case AGMI_I64: return 8;
+        case AGMI_I32: return 4;
+        default: return 0;
+    }
+}
+
+// An index space after dropping size-1 axes and fusing neighbours that every operand walks
+// contiguously (stride[d] == stride[d+1] * shape[d+1], which also holds for two broadcast
+// axes).  `group[d]`, when given, forbids fusing axes of different groups (kept vs reduced).
+struct Merged {
+    int ndim;
+    int64_t n;  // number of points
+    int64_t shape[AGMI_MAX_DIMS];
+    uint8_t group[AGMI_MAX_DIMS];
+    int64_t stride[kMaxOperands][AGMI_MAX_DIMS];
+};
+
+// Returns false (and sets the error) on rank/shape errors.  `strides[k]` may be nullptr for a
+// by-value scalar slot (all zeros are stored).
+bool merge_axes(int ndim, const int64_t *shape, const uint8_t *group, int n_operands,
+                const int64_t *const *strides, Merged *out);
+
+inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
+
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+}  // namespace agmi

@@ -1,0 +1,463 @@
+// Elementwise ("map") kernels: out[k][idx] = op(in[0][idx], ...) over a strided index space.
+//
+// All of these are HBM-bound on MI355X, so the design goal is one pass with full-width,
+// coalesced accesses: every thread moves one 16-byte vector per array operand and there is
+// no loop (measured on the target: one vector per thread, 256-thread blocks, grid = exactly
+// the element count saturates HBM; unrolled variants were slower).  Three layouts:
+//   flat  - after axis merging every array operand is contiguous or a single element;
+//   rows  - two merged axes whose inner stride is 1 or 0 for every operand
+//           (A * b[None, :], x + c[:, None], row slices): vectors along the inner axis,
+//           broadcast operands cost one scalar load;
+//   nd    - anything else up to 6 merged axes, one element per thread with div/mod indexing.
+// A by-value scalar operand lives in kernel arguments (SGPRs); which slots are scalars is a
+// run-time, wave-uniform mask, so one kernel serves array/scalar combinations.
+#include "common.h"
+#include "functors.h"
+
+namespace agmi {
+
+struct EwParams {
+    void *out[AGMI_MAX_OUTPUTS];
+    const void *in[AGMI_MAX_INPUTS];
+    double scalar[AGMI_MAX_INPUTS];
+    unsigned scalar_mask;
+    int ndim;
+    int64_t n;
+    int64_t shape[kMaxMerged];
+    int64_t ostr[AGMI_MAX_OUTPUTS][kMaxMerged];
+    int64_t istr[AGMI_MAX_INPUTS][kMaxMerged];
+};
+
+template <typename T>
+struct Vec {
+    static constexpr int N = 16 / sizeof(T);
+    // element-aligned vector: 16-byte global accesses that only need sizeof(T) alignment, so
+    // views that start at an odd element (x[1:]) still move 16 bytes per lane
+    typedef T type __attribute__((ext_vector_type(N), aligned(sizeof(T))));
+};
+
+// ---- flat ------------------------------------------------------------------------------
+template <template <typename> class F, typename T>
+__global__ __launch_bounds__(kBlock) void ew_flat(const EwParams p) {
+    using Fn = F<T>;
+    constexpr int V = Vec<T>::N;
+    using vec_t = typename Vec<T>::type;
+    const int64_t i0 = (static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x) * V;
+    if (i0 >= p.n) return;
+    T x[Fn::NIN][V];
+    T o[Fn::NOUT][V];
+    if (i0 + V <= p.n) {
+#pragma unroll
+        for (int k = 0; k < Fn::NIN; ++k) {
+            if (p.scalar_mask & (1u << k)) {
+                const T s = static_cast<T>(p.scalar[k]);
+#pragma unroll
+                for (int j = 0; j < V; ++j) x[k][j] = s;
+            } else if (p.istr[k][0] == 0) {
+                const T s = *static_cast<const T *>(p.in[k]);
+#pragma unroll
+                for (int j = 0; j < V; ++j) x[k][j] = s;
+            } else {
+                const vec_t v = *reinterpret_cast<const vec_t *>(static_cast<const T *>(p.in[k]) + i0);
+#pragma unroll
+                for (int j = 0; j < V; ++j) x[k][j] = v[j];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            T xi[Fn::NIN], oi[Fn::NOUT];
+#pragma unroll
+            for (int k = 0; k < Fn::NIN; ++k) xi[k] = x[k][j];
+            Fn::apply(xi, oi);
+#pragma unroll
+            for (int k = 0; k < Fn::NOUT; ++k) o[k][j] = oi[k];
+        }
+#pragma unroll
+        for (int k = 0; k < Fn::NOUT; ++k) {
+            vec_t v;
+#pragma unroll
+            for (int j = 0; j < V; ++j) v[j] = o[k][j];
+            *reinterpret_cast<vec_t *>(static_cast<T *>(p.out[k]) + i0) = v;
+        }
+    } else {
+        for (int64_t i = i0; i < p.n; ++i) {
+            T xi[Fn::NIN], oi[Fn::NOUT];
+#pragma unroll
+            for (int k = 0; k < Fn::NIN; ++k) {
+                if (p.scalar_mask & (1u << k))
+                    xi[k] = static_cast<T>(p.scalar[k]);
+                else
+                    xi[k] = static_cast<const T *>(p.in[k])[p.istr[k][0] == 0 ? 0 : i];
+            }
+            Fn::apply(xi, oi);
+#pragma unroll
+            for (int k = 0; k < Fn::NOUT; ++k) static_cast<T *>(p.out[k])[i] = oi[k];
+        }
+    }
+}
+
+// ---- rows ------------------------------------------------------------------------------
+// shape = (R, C); every operand has inner stride 1 or 0.  `tpr` = threads per row.
+template <template <typename> class F, typename T, typename Index>
+__global__ __launch_bounds__(kBlock) void ew_rows(const EwParams p, const Index tpr, const Index total) {
+    using Fn = F<T>;
+    constexpr int V = Vec<T>::N;
+    using vec_t = typename Vec<T>::type;
+    const Index t = static_cast<Index>(blockIdx.x) * kBlock + threadIdx.x;
+    if (t >= total) return;
+    const Index row = t / tpr;
+    const int64_t c0 = static_cast<int64_t>(t - row * tpr) * V;
+    const int64_t C = p.shape[1];
+    const bool full = c0 + V <= C;
+    const int nvalid = full ? V : static_cast<int>(C - c0);
+    T x[Fn::NIN][V];
+#pragma unroll
+    for (int k = 0; k < Fn::NIN; ++k) {
+        if (p.scalar_mask & (1u << k)) {
+            const T s = static_cast<T>(p.scalar[k]);
+#pragma unroll
+            for (int j = 0; j < V; ++j) x[k][j] = s;
+        } else {
+            const T *base = static_cast<const T *>(p.in[k]) + static_cast<int64_t>(row) * p.istr[k][0];
+            if (p.istr[k][1] == 0) {
+                const T s = *base;
+#pragma unroll
+                for (int j = 0; j < V; ++j) x[k][j] = s;
+            } else if (full) {
+                const vec_t v = *reinterpret_cast<const vec_t *>(base + c0);
+#pragma unroll
+                for (int j = 0; j < V; ++j) x[k][j] = v[j];
+            } else {
+#pragma unroll
+                for (int j = 0; j < V; ++j) x[k][j] = j < nvalid ? base[c0 + j] : T(1);
+            }
+        }
+    }
+    T o[Fn::NOUT][V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+        T xi[Fn::NIN], oi[Fn::NOUT];
+#pragma unroll
+        for (int k = 0; k < Fn::NIN; ++k) xi[k] = x[k][j];
+        Fn::apply(xi, oi);
+#pragma unroll
+        for (int k = 0; k < Fn::NOUT; ++k) o[k][j] = oi[k];
+    }
+#pragma unroll
+    for (int k = 0; k < Fn::NOUT; ++k) {
+        T *base = static_cast<T *>(p.out[k]) + static_cast<int64_t>(row) * p.ostr[k][0];
+        if (full) {
+            vec_t v;
+#pragma unroll
+            for (int j = 0; j < V; ++j) v[j] = o[k][j];
+            *reinterpret_cast<vec_t *>(base + c0) = v;
+        } else {
+#pragma unroll
+            for (int j = 0; j < V; ++j)
+                if (j < nvalid) base[c0 + j] = o[k][j];
+        }
+    }
+}
+
+// ---- nd --------------------------------------------------------------------------------
+template <template <typename> class F, typename T, typename Index>
+__global__ __launch_bounds__(kBlock) void ew_nd(const EwParams p) {
+    using Fn = F<T>;
+    Index rem = static_cast<Index>(blockIdx.x) * kBlock + threadIdx.x;
+    if (static_cast<int64_t>(rem) >= p.n) return;
+    int64_t ioff[Fn::NIN];
+    int64_t ooff[Fn::NOUT];
+#pragma unroll
+    for (int k = 0; k < Fn::NIN; ++k) ioff[k] = 0;
+#pragma unroll
+    for (int k = 0; k < Fn::NOUT; ++k) ooff[k] = 0;
+    for (int d = p.ndim - 1; d >= 0; --d) {
+        const Index extent = static_cast<Index>(p.shape[d]);
+        const Index q = rem / extent;
+        const int64_t c = static_cast<int64_t>(rem - q * extent);
+        rem = q;
+#pragma unroll
+        for (int k = 0; k < Fn::NIN; ++k) ioff[k] += c * p.istr[k][d];
+#pragma unroll
+        for (int k = 0; k < Fn::NOUT; ++k) ooff[k] += c * p.ostr[k][d];
+    }
+    T xi[Fn::NIN], oi[Fn::NOUT];
+#pragma unroll
+    for (int k = 0; k < Fn::NIN; ++k)
+        xi[k] = (p.scalar_mask & (1u << k)) ? static_cast<T>(p.scalar[k]) : static_cast<const T *>(p.in[k])[ioff[k]];
+    Fn::apply(xi, oi);
+#pragma unroll
+    for (int k = 0; k < Fn::NOUT; ++k) static_cast<T *>(p.out[k])[ooff[k]] = oi[k];
+}
+
+// ---- host side -------------------------------------------------------------------------
+static int check_blocks(int64_t blocks) {
+    if (blocks > 0x7fffffffLL) {
+        set_error("elementwise: index space too large for one launch");
+        return AGMI_ERR_UNSUPPORTED;
+    }
+    return 0;
+}
+
+template <template <typename> class F, typename T>
+static int launch_ew(const Merged &m, int n_out, const agmi_array *outs, int n_in, const agmi_array *ins,
+                     const double *scalars, hipStream_t s) {
+    using Fn = F<T>;
+    if (n_in != Fn::NIN || n_out != Fn::NOUT) {
+        set_error("elementwise: op takes %d inputs and %d outputs, got %d and %d", Fn::NIN, Fn::NOUT, n_in, n_out);
+        return AGMI_ERR_ARG;
+    }
+    if (m.ndim > kMaxMerged) {
+        set_error("elementwise: %d axes remain after merging, at most %d are supported", m.ndim, kMaxMerged);
+        return AGMI_ERR_UNSUPPORTED;
+    }
+    EwParams p = {};
+    p.ndim = m.ndim;
+    p.n = m.n;
+    for (int d = 0; d < m.ndim; ++d) p.shape[d] = m.shape[d];
+    for (int k = 0; k < n_out; ++k) {
+        p.out[k] = outs[k].data;
+        for (int d = 0; d < m.ndim; ++d) {
+            p.ostr[k][d] = m.stride[k][d];
+            if (m.stride[k][d] == 0 && m.shape[d] > 1) {
+                set_error("elementwise: output %d has stride 0 on an axis of extent %lld", k, (long long)m.shape[d]);
+                return AGMI_ERR_ARG;
+            }
+        }
+    }
+    for (int k = 0; k < n_in; ++k) {
+        p.in[k] = ins[k].data;
+        if (ins[k].data == nullptr) {
+            if (scalars == nullptr) {
+                set_error("elementwise: scalar slot %d without scalars array", k);
+                return AGMI_ERR_ARG;
+            }
+            p.scalar_mask |= 1u << k;
+            p.scalar[k] = scalars[k];
+        }
+        for (int d = 0; d < m.ndim; ++d) p.istr[k][d] = m.stride[n_out + k][d];
+    }
+
+    constexpr int V = Vec<T>::N;
+    bool inner_unit = true;  // every operand's innermost stride is 1 (outputs) or 0/1 (inputs)
+    const int last = m.ndim - 1;
+    for (int k = 0; k < n_out; ++k) inner_unit &= (p.ostr[k][last] == 1 || m.shape[last] == 1);
+    for (int k = 0; k < n_in; ++k)
+        inner_unit &= (p.scalar_mask & (1u << k)) || p.istr[k][last] == 1 || p.istr[k][last] == 0;
+
+    if (m.ndim == 1 && inner_unit) {
+        const int64_t blocks = ceil_div(ceil_div(m.n, V), kBlock);
+        if (int rc = check_blocks(blocks)) return rc;
+        hipLaunchKernelGGL((ew_flat<F, T>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p);
+    } else if (m.ndim == 2 && inner_unit) {
+        const int64_t tpr = ceil_div(m.shape[1], V);
+        const int64_t total = tpr * m.shape[0];
+        const int64_t blocks = ceil_div(total, kBlock);
+        if (int rc = check_blocks(blocks)) return rc;
+        if (total < 0x7fffffffLL)
+            hipLaunchKernelGGL((ew_rows<F, T, unsigned>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p,
+                               (unsigned)tpr, (unsigned)total);
+        else
+            hipLaunchKernelGGL((ew_rows<F, T, int64_t>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p, tpr, total);
+    } else {
+        const int64_t blocks = ceil_div(m.n, kBlock);
+        if (int rc = check_blocks(blocks)) return rc;
+        if (m.n < 0x7fffffffLL)
+            hipLaunchKernelGGL((ew_nd<F, T, unsigned>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p);
+        else
+            hipLaunchKernelGGL((ew_nd<F, T, int64_t>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p);
+    }
+    return hip_check(hipGetLastError(), "elementwise launch");
+}
+
+// ---- compare and cast (not on the bandwidth-critical path: nd indexing only) -----------------
+struct MixParams {
+    void *out;
+    const void *in[2];
+    double scalar[2];
+    unsigned scalar_mask;
+    int ndim;
+    int64_t n;
+    int64_t shape[kMaxMerged];
+    int64_t ostr[kMaxMerged];
+    int64_t istr[2][kMaxMerged];
+};
+
+template <typename Index>
+__device__ __forceinline__ void nd_offsets(const MixParams &p, Index rem, int n_in, int64_t *ioff, int64_t *ooff) {
+    for (int d = p.ndim - 1; d >= 0; --d) {
+        const Index extent = static_cast<Index>(p.shape[d]);
+        const Index q = rem / extent;
+        const int64_t c = static_cast<int64_t>(rem - q * extent);
+        rem = q;
+        for (int k = 0; k < n_in; ++k) ioff[k] += c * p.istr[k][d];
+        *ooff += c * p.ostr[d];
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void compare_nd(const MixParams p, const int cmp) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (i >= p.n) return;
+    int64_t ioff[2] = {0, 0}, ooff = 0;
+    nd_offsets<int64_t>(p, i, 2, ioff, &ooff);
+    const T a = (p.scalar_mask & 1u) ? static_cast<T>(p.scalar[0]) : static_cast<const T *>(p.in[0])[ioff[0]];
+    const T b = (p.scalar_mask & 2u) ? static_cast<T>(p.scalar[1]) : static_cast<const T *>(p.in[1])[ioff[1]];
+    bool r;
+    switch (cmp) {
+        case AGMI_EQ: r = a == b; break;
+        case AGMI_NE: r = a != b; break;
+        case AGMI_LT: r = a < b; break;
+        case AGMI_LE: r = a <= b; break;
+        case AGMI_GT: r = a > b; break;
+        default: r = a >= b; break;
+    }
+    static_cast<uint8_t *>(p.out)[ooff] = r ? 1 : 0;
+}
+
+template <typename S, typename D>
+__global__ __launch_bounds__(kBlock) void cast_nd(const MixParams p) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (i >= p.n) return;
+    int64_t ioff[2] = {0, 0}, ooff = 0;
+    nd_offsets<int64_t>(p, i, 1, ioff, &ooff);
+    const S v = static_cast<const S *>(p.in[0])[ioff[0]];
+    D r;
+    if constexpr (sizeof(D) == 1)
+        r = static_cast<D>(v != S(0) ? 1 : 0);  // to bool
+    else
+        r = static_cast<D>(v);
+    static_cast<D *>(p.out)[ooff] = r;
+}
+
+static bool fill_mix(const Merged &m, const agmi_array *out, int n_in, const agmi_array *ins, const double *scalars,
+                     MixParams *p) {
+    if (m.ndim > kMaxMerged) {
+        set_error("%d axes remain after merging, at most %d are supported", m.ndim, kMaxMerged);
+        return false;
+    }
+    *p = MixParams{};
+    p->ndim = m.ndim;
+    p->n = m.n;
+    p->out = out->data;
+    for (int d = 0; d < m.ndim; ++d) {
+        p->shape[d] = m.shape[d];
+        p->ostr[d] = m.stride[0][d];
+    }
+    for (int k = 0; k < n_in; ++k) {
+        p->in[k] = ins[k].data;
+        if (ins[k].data == nullptr) {
+            if (!scalars) {
+                set_error("scalar slot %d without scalars array", k);
+                return false;
+            }
+            p->scalar_mask |= 1u << k;
+            p->scalar[k] = scalars[k];
+        }
+        for (int d = 0; d < m.ndim; ++d) p->istr[k][d] = m.stride[1 + k][d];
+    }
+    return true;
+}
+
+template <typename S>
+static int launch_cast_from(int dst_dtype, const MixParams &p, unsigned blocks, hipStream_t s) {
+    switch (dst_dtype) {
+        case AGMI_F32: hipLaunchKernelGGL((cast_nd<S, float>), dim3(blocks), dim3(kBlock), 0, s, p); break;
+        case AGMI_F64: hipLaunchKernelGGL((cast_nd<S, double>), dim3(blocks), dim3(kBlock), 0, s, p); break;
+        case AGMI_BOOL: hipLaunchKernelGGL((cast_nd<S, uint8_t>), dim3(blocks), dim3(kBlock), 0, s, p); break;
+        case AGMI_I64: hipLaunchKernelGGL((cast_nd<S, int64_t>), dim3(blocks), dim3(kBlock), 0, s, p); break;
+        case AGMI_I32: hipLaunchKernelGGL((cast_nd<S, int32_t>), dim3(blocks), dim3(kBlock), 0, s, p); break;
+        default: set_error("cast: unknown destination dtype %d", dst_dtype); return AGMI_ERR_ARG;
+    }
+    return hip_check(hipGetLastError(), "cast launch");
+}
+
+}  // namespace agmi
+
+using namespace agmi;
+
+extern "C" int agmi_elementwise(int op, int dtype, int ndim, const int64_t *shape, int n_out,
+                                const agmi_array *outs, int n_in, const agmi_array *ins,
+                                const double *scalars, void *stream) {
+    if (n_out < 1 || n_out > AGMI_MAX_OUTPUTS || n_in < 1 || n_in > AGMI_MAX_INPUTS || !outs || !ins) {
+        set_error("elementwise: bad operand counts or null operand arrays");
+        return AGMI_ERR_ARG;
+    }
+    const int64_t *strides[kMaxOperands];
+    for (int k = 0; k < n_out; ++k) {
+        if (outs[k].data == nullptr) {
+            set_error("elementwise: output %d is null", k);
+            return AGMI_ERR_ARG;
+        }
+        strides[k] = outs[k].strides;
+    }
+    for (int k = 0; k < n_in; ++k) strides[n_out + k] = ins[k].data ? ins[k].strides : nullptr;
+    Merged m;
+    if (!merge_axes(ndim, shape, nullptr, n_out + n_in, strides, &m)) return AGMI_ERR_ARG;
+    if (m.n == 0) return 0;
+    hipStream_t s = as_stream(stream);
+#define AGMI_CASE(OP, FN)                                                                    \
+    case OP:                                                                                 \
+        if (dtype == AGMI_F32) return launch_ew<FN, float>(m, n_out, outs, n_in, ins, scalars, s);  \
+        if (dtype == AGMI_F64) return launch_ew<FN, double>(m, n_out, outs, n_in, ins, scalars, s); \
+        break;
+    switch (op) {
+        AGMI_FOR_EACH_OP(AGMI_CASE)
+        default: set_error("elementwise: unknown op %d", op); return AGMI_ERR_ARG;
+    }
+#undef AGMI_CASE
+    set_error("elementwise: dtype %d is not a floating type", dtype);
+    return AGMI_ERR_ARG;
+}
+
+extern "C" int agmi_compare(int cmp, int dtype, int ndim, const int64_t *shape, const agmi_array *out,
+                            const agmi_array *ins, const double *scalars, void *stream) {
+    if (!out || !ins || !out->data || cmp < AGMI_EQ || cmp > AGMI_GE) {
+        set_error("compare: bad arguments");
+        return AGMI_ERR_ARG;
+    }
+    const int64_t *strides[3] = {out->strides, ins[0].data ? ins[0].strides : nullptr,
+                                 ins[1].data ? ins[1].strides : nullptr};
+    Merged m;
+    if (!merge_axes(ndim, shape, nullptr, 3, strides, &m)) return AGMI_ERR_ARG;
+    if (m.n == 0) return 0;
+    MixParams p;
+    if (!fill_mix(m, out, 2, ins, scalars, &p)) return AGMI_ERR_UNSUPPORTED;
+    const int64_t blocks = ceil_div(m.n, kBlock);
+    if (int rc = check_blocks(blocks)) return rc;
+    hipStream_t s = as_stream(stream);
+    if (dtype == AGMI_F32)
+        hipLaunchKernelGGL(compare_nd<float>, dim3((unsigned)blocks), dim3(kBlock), 0, s, p, cmp);
+    else if (dtype == AGMI_F64)
+        hipLaunchKernelGGL(compare_nd<double>, dim3((unsigned)blocks), dim3(kBlock), 0, s, p, cmp);
+    else {
+        set_error("compare: dtype %d is not a floating type", dtype);
+        return AGMI_ERR_ARG;
+    }
+    return hip_check(hipGetLastError(), "compare launch");
+}
+
+extern "C" int agmi_cast(int src_dtype, int dst_dtype, int ndim, const int64_t *shape, const agmi_array *out,
+                         const agmi_array *in, void *stream) {
+    if (!out || !in || !out->data || !in->data) {
+        set_error("cast: null operand");
+        return AGMI_ERR_ARG;
+    }
+    const int64_t *strides[2] = {out->strides, in->strides};
+    Merged m;
+    if (!merge_axes(ndim, shape, nullptr, 2, strides, &m)) return AGMI_ERR_ARG;
+    if (m.n == 0) return 0;
+    MixParams p;
+    if (!fill_mix(m, out, 1, in, nullptr, &p)) return AGMI_ERR_UNSUPPORTED;
+    const int64_t blocks = ceil_div(m.n, kBlock);
+    if (int rc = check_blocks(blocks)) return rc;
+    hipStream_t s = as_stream(stream);
+    switch (src_dtype) {
+        case AGMI_F32: return launch_cast_from<float>(dst_dtype, p, (unsigned)blocks, s);
+        case AGMI_F64: return launch_cast_from<double>(dst_dtype, p, (unsigned)blocks, s);
+        case AGMI_BOOL: return launch_cast_from<uint8_t>(dst_dtype, p, (unsigned)blocks, s);
+        case AGMI_I64: return launch_cast_from<int64_t>(dst_dtype, p, (unsigned)blocks, s);
+        case AGMI_I32: return launch_cast_from<int32_t>(dst_dtype, p, (unsigned)blocks, s);
+        default: set_error("cast: unknown source dtype %d", src_dtype); return AGMI_ERR_ARG;
+    }
+}

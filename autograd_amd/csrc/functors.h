@@ -1,0 +1,176 @@
+// Elementwise operation table: one functor per agmi_op, shared by the map kernels
+// (elementwise.hip) and the map-reduce kernels (reduce.hip).
+//
+// Each functor states its arity and computes one point from its inputs.  Fused derivative
+// rules keep the operation order of the reference rule they replace (cited in agmi.h) so
+// that results differ from NumPy's only by the last-bit behaviour of transcendental
+// functions; the library is compiled with -ffp-contract=off so products and sums are not
+// fused into FMAs that NumPy would not perform.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "agmi.h"
+
+namespace agmi {
+
+// math on T in {float, double}
+__device__ __forceinline__ float m_exp(float x) { return expf(x); }
+__device__ __forceinline__ double m_exp(double x) { return exp(x); }
+__device__ __forceinline__ float m_log(float x) { return logf(x); }
+__device__ __forceinline__ double m_log(double x) { return log(x); }
+__device__ __forceinline__ float m_log1p(float x) { return log1pf(x); }
+__device__ __forceinline__ double m_log1p(double x) { return log1p(x); }
+__device__ __forceinline__ float m_expm1(float x) { return expm1f(x); }
+__device__ __forceinline__ double m_expm1(double x) { return expm1(x); }
+__device__ __forceinline__ float m_tanh(float x) { return tanhf(x); }
+__device__ __forceinline__ double m_tanh(double x) { return tanh(x); }
+__device__ __forceinline__ float m_sinh(float x) { return sinhf(x); }
+__device__ __forceinline__ double m_sinh(double x) { return sinh(x); }
+__device__ __forceinline__ float m_cosh(float x) { return coshf(x); }
+__device__ __forceinline__ double m_cosh(double x) { return cosh(x); }
+__device__ __forceinline__ float m_sin(float x) { return sinf(x); }
+__device__ __forceinline__ double m_sin(double x) { return sin(x); }
+__device__ __forceinline__ float m_cos(float x) { return cosf(x); }
+__device__ __forceinline__ double m_cos(double x) { return cos(x); }
+__device__ __forceinline__ float m_sqrt(float x) { return sqrtf(x); }
+__device__ __forceinline__ double m_sqrt(double x) { return sqrt(x); }
+__device__ __forceinline__ float m_abs(float x) { return fabsf(x); }
+__device__ __forceinline__ double m_abs(double x) { return fabs(x); }
+__device__ __forceinline__ float m_pow(float x, float y) { return powf(x, y); }
+__device__ __forceinline__ double m_pow(double x, double y) { return pow(x, y); }
+
+// x**y with the exponents NumPy short-cuts (1, 2, 0, -1, 0.5) computed the same exact way.
+template <typename T>
+__device__ __forceinline__ T pow_like_numpy(T x, T y) {
+    if (y == T(2)) return x * x;
+    if (y == T(1)) return x;
+    if (y == T(0)) return T(1);
+    if (y == T(-1)) return T(1) / x;
+    if (y == T(0.5)) return m_sqrt(x);
+    return m_pow(x, y);
+}
+
+// NumPy's maximum/minimum propagate NaN from either operand.
+template <typename T>
+__device__ __forceinline__ T max_nan(T a, T b) {
+    return (a >= b || a != a) ? a : b;
+}
+template <typename T>
+__device__ __forceinline__ T min_nan(T a, T b) {
+    return (a <= b || a != a) ? a : b;
+}
+
+#define AGMI_FUNCTOR(NAME, N_IN, N_OUT, ...)                                      \
+    template <typename T>                                                         \
+    struct NAME {                                                                 \
+        static constexpr int NIN = N_IN;                                          \
+        static constexpr int NOUT = N_OUT;                                        \
+        __device__ __forceinline__ static void apply(const T *x, T *o) { __VA_ARGS__ } \
+    };
+
+AGMI_FUNCTOR(FCopy, 1, 1, o[0] = x[0];)
+AGMI_FUNCTOR(FNeg, 1, 1, o[0] = -x[0];)
+AGMI_FUNCTOR(FExp, 1, 1, o[0] = m_exp(x[0]);)
+AGMI_FUNCTOR(FLog, 1, 1, o[0] = m_log(x[0]);)
+AGMI_FUNCTOR(FTanh, 1, 1, o[0] = m_tanh(x[0]);)
+AGMI_FUNCTOR(FSinh, 1, 1, o[0] = m_sinh(x[0]);)
+AGMI_FUNCTOR(FCosh, 1, 1, o[0] = m_cosh(x[0]);)
+AGMI_FUNCTOR(FSin, 1, 1, o[0] = m_sin(x[0]);)
+AGMI_FUNCTOR(FCos, 1, 1, o[0] = m_cos(x[0]);)
+AGMI_FUNCTOR(FSqrt, 1, 1, o[0] = m_sqrt(x[0]);)
+AGMI_FUNCTOR(FSquare, 1, 1, o[0] = x[0] * x[0];)
+AGMI_FUNCTOR(FAbs, 1, 1, o[0] = m_abs(x[0]);)
+AGMI_FUNCTOR(FSign, 1, 1, o[0] = x[0] > T(0) ? T(1) : (x[0] < T(0) ? T(-1) : x[0]);)
+AGMI_FUNCTOR(FReciprocal, 1, 1, o[0] = T(1) / x[0];)
+AGMI_FUNCTOR(FLog1p, 1, 1, o[0] = m_log1p(x[0]);)
+AGMI_FUNCTOR(FExpm1, 1, 1, o[0] = m_expm1(x[0]);)
+
+AGMI_FUNCTOR(FAdd, 2, 1, o[0] = x[0] + x[1];)
+AGMI_FUNCTOR(FSub, 2, 1, o[0] = x[0] - x[1];)
+AGMI_FUNCTOR(FMul, 2, 1, o[0] = x[0] * x[1];)
+AGMI_FUNCTOR(FDiv, 2, 1, o[0] = x[0] / x[1];)
+AGMI_FUNCTOR(FPow, 2, 1, o[0] = pow_like_numpy(x[0], x[1]);)
+AGMI_FUNCTOR(FMaximum, 2, 1, o[0] = max_nan(x[0], x[1]);)
+AGMI_FUNCTOR(FMinimum, 2, 1, o[0] = min_nan(x[0], x[1]);)
+
+AGMI_FUNCTOR(FWhere, 3, 1, o[0] = (x[0] != T(0)) ? x[1] : x[2];)
+
+// (g, x, y): -g * x / y**2
+AGMI_FUNCTOR(FDivVjp1, 3, 1, o[0] = ((-x[0]) * x[1]) / (x[2] * x[2]);)
+// (g, x): g / cosh(x)**2
+AGMI_FUNCTOR(FTanhVjp, 2, 1, T c = m_cosh(x[1]); o[0] = x[0] / (c * c);)
+// (g, x, y): g * y * x**where(y, y - 1, 1)
+AGMI_FUNCTOR(FPowVjp0, 3, 1, T e = (x[2] != T(0)) ? x[2] - T(1) : T(1);
+             o[0] = (x[0] * x[2]) * pow_like_numpy(x[1], e);)
+// (g, x, ans): g * log(where(x, x, 1)) * ans
+AGMI_FUNCTOR(FPowVjp1, 3, 1, T b = (x[1] != T(0)) ? x[1] : T(1); o[0] = (x[0] * m_log(b)) * x[2];)
+// (g, b, x, ans): g * b * exp(x - ans)
+AGMI_FUNCTOR(FLseVjp, 4, 1, o[0] = (x[0] * x[1]) * m_exp(x[2] - x[3]);)
+// (g, x): -g / x**2
+AGMI_FUNCTOR(FReciprocalVjp, 2, 1, o[0] = (-x[0]) / (x[1] * x[1]);)
+// (g, x): g * 0.5 * x**-0.5
+AGMI_FUNCTOR(FSqrtVjp, 2, 1, o[0] = (x[0] * T(0.5)) * m_pow(x[1], T(-0.5));)
+AGMI_FUNCTOR(FSinVjp, 2, 1, o[0] = x[0] * m_cos(x[1]);)
+AGMI_FUNCTOR(FCosVjp, 2, 1, o[0] = (-x[0]) * m_sin(x[1]);)
+AGMI_FUNCTOR(FSinhVjp, 2, 1, o[0] = x[0] * m_cosh(x[1]);)
+AGMI_FUNCTOR(FCoshVjp, 2, 1, o[0] = x[0] * m_sinh(x[1]);)
+AGMI_FUNCTOR(FSquareVjp, 2, 1, o[0] = (x[0] * T(2)) * x[1];)
+// (g, x, ans): g * where(x, x, 0) / where(ans, ans, 1)
+AGMI_FUNCTOR(FAbsVjp, 3, 1, T d = (x[2] != T(0)) ? x[2] : T(1); o[0] = (x[0] * x[1]) / d;)
+// (g, x, ans, y): g * ((x == ans) / (1 + (x == y)))
+AGMI_FUNCTOR(FChooseVjp, 4, 1, T num = (x[1] == x[2]) ? T(1) : T(0); T den = (x[1] == x[3]) ? T(2) : T(1);
+             o[0] = x[0] * (num / den);)
+AGMI_FUNCTOR(FLog1pVjp, 2, 1, o[0] = x[0] / (x[1] + T(1));)
+AGMI_FUNCTOR(FExpm1Vjp, 2, 1, o[0] = (x[1] + T(1)) * x[0];)
+// (g, x, y) -> g / y, -g * x / y**2
+AGMI_FUNCTOR(FDivVjpBoth, 3, 2, o[0] = x[0] / x[2]; o[1] = ((-x[0]) * x[1]) / (x[2] * x[2]);)
+// (a, x, y): a * x + y, two roundings
+AGMI_FUNCTOR(FMulAdd, 3, 1, T t = x[0] * x[1]; o[0] = t + x[2];)
+
+// X(op enum, functor)
+#define AGMI_FOR_EACH_OP(X)                     \
+    X(AGMI_OP_COPY, FCopy)                      \
+    X(AGMI_OP_NEG, FNeg)                        \
+    X(AGMI_OP_EXP, FExp)                        \
+    X(AGMI_OP_LOG, FLog)                        \
+    X(AGMI_OP_TANH, FTanh)                      \
+    X(AGMI_OP_SINH, FSinh)                      \
+    X(AGMI_OP_COSH, FCosh)                      \
+    X(AGMI_OP_SIN, FSin)                        \
+    X(AGMI_OP_COS, FCos)                        \
+    X(AGMI_OP_SQRT, FSqrt)                      \
+    X(AGMI_OP_SQUARE, FSquare)                  \
+    X(AGMI_OP_ABS, FAbs)                        \
+    X(AGMI_OP_SIGN, FSign)                      \
+    X(AGMI_OP_RECIPROCAL, FReciprocal)          \
+    X(AGMI_OP_LOG1P, FLog1p)                    \
+    X(AGMI_OP_EXPM1, FExpm1)                    \
+    X(AGMI_OP_ADD, FAdd)                        \
+    X(AGMI_OP_SUB, FSub)                        \
+    X(AGMI_OP_MUL, FMul)                        \
+    X(AGMI_OP_DIV, FDiv)                        \
+    X(AGMI_OP_POW, FPow)                        \
+    X(AGMI_OP_MAXIMUM, FMaximum)                \
+    X(AGMI_OP_MINIMUM, FMinimum)                \
+    X(AGMI_OP_WHERE, FWhere)                    \
+    X(AGMI_OP_DIV_VJP1, FDivVjp1)               \
+    X(AGMI_OP_TANH_VJP, FTanhVjp)               \
+    X(AGMI_OP_POW_VJP0, FPowVjp0)               \
+    X(AGMI_OP_POW_VJP1, FPowVjp1)               \
+    X(AGMI_OP_LSE_VJP, FLseVjp)                 \
+    X(AGMI_OP_RECIPROCAL_VJP, FReciprocalVjp)   \
+    X(AGMI_OP_SQRT_VJP, FSqrtVjp)               \
+    X(AGMI_OP_SIN_VJP, FSinVjp)                 \
+    X(AGMI_OP_COS_VJP, FCosVjp)                 \
+    X(AGMI_OP_SINH_VJP, FSinhVjp)               \
+    X(AGMI_OP_COSH_VJP, FCoshVjp)               \
+    X(AGMI_OP_SQUARE_VJP, FSquareVjp)           \
+    X(AGMI_OP_ABS_VJP, FAbsVjp)                 \
+    X(AGMI_OP_CHOOSE_VJP, FChooseVjp)           \
+    X(AGMI_OP_LOG1P_VJP, FLog1pVjp)             \
+    X(AGMI_OP_EXPM1_VJP, FExpm1Vjp)             \
+    X(AGMI_OP_DIV_VJP_BOTH, FDivVjpBoth)        \
+    X(AGMI_OP_MUL_ADD, FMulAdd)
+
+}  // namespace agmi

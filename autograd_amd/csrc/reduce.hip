@@ -1,0 +1,607 @@
+// Map-reduce kernels: out[kept] = REDUCE_{reduced axes} op(in[0][idx], in[1][idx], ...).
+//
+// One kernel family serves unbroadcast (sum of a rule's cotangent over broadcast axes, fused
+// with the rule itself), numpy.sum/max/min/prod, scipy's logsumexp (as a reduction over
+// (max, scaled-sum) pairs, single pass over memory), inner products and matrix-vector dot.
+//
+// After axis merging the index space is (O, R, I): outer kept, reduced, inner kept.
+//   I == 1  "row" form : red_row_block (one 256-thread block per row chunk, 16-byte loads
+//                        along R) or red_row_group (G <= 64 lanes per row for short rows);
+//   I  > 1  "col" form : red_cols, threads along I (coalesced, 16-byte loads when possible),
+//                        a TX x TY block walks R, LDS tree over TY.
+// When one pass cannot fill 256 CUs, R is cut into chunks whose partial accumulators go to a
+// caller-provided workspace and red_finish combines them.  Combination order is a fixed
+// function of the shapes: wave-level butterflies (__shfl_xor over 64 lanes), then an LDS
+// tree over the block's 4 waves, then chunks in index order - never atomics - so results
+// are reproducible run to run.
+#include <algorithm>
+
+#include "common.h"
+#include "functors.h"
+
+namespace agmi {
+
+// ---- accumulators ----------------------------------------------------------------------
+template <typename T>
+struct AccSum {
+    typedef T type;
+    __device__ __forceinline__ static T identity() { return T(0); }
+    __device__ __forceinline__ static T lift(T v) { return v; }
+    __device__ __forceinline__ static T combine(T a, T b) { return a + b; }
+    __device__ __forceinline__ static T finish(T a) { return a; }
+    __device__ __forceinline__ static T shfl_xor(T a, int m) { return __shfl_xor(a, m, 64); }
+};
+template <typename T>
+struct AccProd : AccSum<T> {
+    __device__ __forceinline__ static T identity() { return T(1); }
+    __device__ __forceinline__ static T combine(T a, T b) { return a * b; }
+};
+template <typename T>
+struct AccMax : AccSum<T> {
+    __device__ __forceinline__ static T identity() { return -INFINITY; }
+    __device__ __forceinline__ static T combine(T a, T b) { return max_nan(a, b); }
+};
+template <typename T>
+struct AccMin : AccSum<T> {
+    __device__ __forceinline__ static T identity() { return INFINITY; }
+    __device__ __forceinline__ static T combine(T a, T b) { return min_nan(a, b); }
+};
+
+// log-sum-exp as an associative reduction over (m, s) with value = m + log(s),
+// s = sum exp(x - m).  Infinite and equal maxima are combined without forming inf - inf.
+template <typename T>
+struct LsePair {
+    T m, s;
+};
+template <typename T>
+struct AccLse {
+    typedef LsePair<T> type;
+    __device__ __forceinline__ static type identity() { return {T(-INFINITY), T(0)}; }
+    __device__ __forceinline__ static type lift(T v) { return {v, T(1)}; }
+    __device__ __forceinline__ static type combine(type a, type b) {
+        if (a.m == b.m) return {a.m, a.s + b.s};
+        if (a.m > b.m) return {a.m, a.s + b.s * m_exp(b.m - a.m)};
+        if (b.m > a.m) return {b.m, b.s + a.s * m_exp(a.m - b.m)};
+        return {a.m + b.m, a.s + b.s};  // a NaN is involved: propagate it
+    }
+    __device__ __forceinline__ static T finish(type a) {
+        if (a.s == T(0) || a.m == T(INFINITY)) return a.m;  // all -inf, or a +inf present
+        return a.m + m_log(a.s);
+    }
+    __device__ __forceinline__ static type shfl_xor(type a, int m) {
+        return {__shfl_xor(a.m, m, 64), __shfl_xor(a.s, m, 64)};
+    }
+};
+
+struct RedParams {
+    void *out;  // T* when final, Acc* (chunk-major) when partial
+    const void *in[AGMI_MAX_INPUTS];
+    double scalar[AGMI_MAX_INPUTS];
+    unsigned scalar_mask;
+    int n_chunks;
+    int64_t O, R, I;
+    int64_t r_chunk;
+    int64_t ostr_o, ostr_i;
+    int64_t istr[AGMI_MAX_INPUTS][3];  // (o, r, i)
+};
+
+template <typename T>
+struct RVec {
+    static constexpr int N = 16 / sizeof(T);
+    typedef T type __attribute__((ext_vector_type(N), aligned(sizeof(T))));
+};
+
+// load V consecutive points along axis `ax` (1 = r, 2 = i) starting at element offsets given
+template <template <typename> class F, typename T, int V, int AX>
+__device__ __forceinline__ void load_points(const RedParams &p, int64_t o, int64_t r, int64_t i, T (&x)[F<T>::NIN][V]) {
+    using vec_t = typename RVec<T>::type;
+#pragma unroll
+    for (int k = 0; k < F<T>::NIN; ++k) {
+        if (p.scalar_mask & (1u << k)) {
+            const T s = static_cast<T>(p.scalar[k]);
+#pragma unroll
+            for (int j = 0; j < V; ++j) x[k][j] = s;
+        } else {
+            const T *base = static_cast<const T *>(p.in[k]) + o * p.istr[k][0] + r * p.istr[k][1] + i * p.istr[k][2];
+            if (V == 1) {
+                x[k][0] = *base;
+            } else if (p.istr[k][AX] == 0) {
+                const T s = *base;
+#pragma unroll
+                for (int j = 0; j < V; ++j) x[k][j] = s;
+            } else {  // stride 1 along AX, guaranteed by the planner when V > 1
+                const vec_t v = *reinterpret_cast<const vec_t *>(base);
+#pragma unroll
+                for (int j = 0; j < V; ++j) x[k][j] = v[j];
+            }
+        }
+    }
+}
+
+template <template <typename> class F, typename T, int V>
+__device__ __forceinline__ T map_point(const T (&x)[F<T>::NIN][V], int j) {
+    T xi[F<T>::NIN], oi[F<T>::NOUT];
+#pragma unroll
+    for (int k = 0; k < F<T>::NIN; ++k) xi[k] = x[k][j];
+    F<T>::apply(xi, oi);
+    return oi[0];
+}
+
+template <class Acc>
+__device__ __forceinline__ typename Acc::type wave_reduce(typename Acc::type a, int lanes) {
+    for (int m = lanes >> 1; m > 0; m >>= 1) a = Acc::combine(a, Acc::shfl_xor(a, m));
+    return a;
+}
+
+// all 256 threads call; result valid in thread 0
+template <class Acc>
+__device__ __forceinline__ typename Acc::type block_reduce(typename Acc::type a) {
+    __shared__ typename Acc::type wave_part[kBlock / 64];
+    a = wave_reduce<Acc>(a, 64);
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) wave_part[wave] = a;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int w = 1; w < kBlock / 64; ++w) a = Acc::combine(a, wave_part[w]);
+    }
+    return a;
+}
+
+template <class Acc, typename T, bool FINAL>
+__device__ __forceinline__ void store_result(const RedParams &p, typename Acc::type a, int64_t o, int64_t i, int chunk) {
+    if (FINAL)
+        static_cast<T *>(p.out)[o * p.ostr_o + i * p.ostr_i] = Acc::finish(a);
+    else
+        static_cast<typename Acc::type *>(p.out)[(static_cast<int64_t>(chunk) * p.O + o) * p.I + i] = a;
+}
+
+// ---- row form, one block per (row, chunk) ----------------------------------------------------
+template <template <typename> class F, template <typename> class AccT, typename T, int V, bool FINAL>
+__global__ __launch_bounds__(kBlock) void red_row_block(const RedParams p) {
+    using Acc = AccT<T>;
+    const int64_t o = blockIdx.x;
+    const int chunk = blockIdx.y;
+    const int64_t r_begin = static_cast<int64_t>(chunk) * p.r_chunk;
+    const int64_t r_end = min(r_begin + p.r_chunk, p.R);
+    typename Acc::type acc = Acc::identity();
+    const int64_t n_vec = (r_end - r_begin) / V;
+    for (int64_t v = threadIdx.x; v < n_vec; v += kBlock) {
+        T x[F<T>::NIN][V];
+        load_points<F, T, V, 1>(p, o, r_begin + v * V, 0, x);
+#pragma unroll
+        for (int j = 0; j < V; ++j) acc = Acc::combine(acc, Acc::lift(map_point<F, T, V>(x, j)));
+    }
+    if (V > 1) {  // ragged tail, fewer than V points
+        const int64_t r = r_begin + n_vec * V + threadIdx.x;
+        if (r < r_end) {
+            T x[F<T>::NIN][1];
+            load_points<F, T, 1, 1>(p, o, r, 0, x);
+            acc = Acc::combine(acc, Acc::lift(map_point<F, T, 1>(x, 0)));
+        }
+    }
+    acc = block_reduce<Acc>(acc);
+    if (threadIdx.x == 0) store_result<Acc, T, FINAL>(p, acc, o, 0, chunk);
+}
+
+// ---- row form, G lanes per row (short rows) --------------------------------------------------
+template <template <typename> class F, template <typename> class AccT, typename T>
+__global__ __launch_bounds__(kBlock) void red_row_group(const RedParams p, const int G) {
+    using Acc = AccT<T>;
+    const int rows_per_block = kBlock / G;
+    const int64_t o = static_cast<int64_t>(blockIdx.x) * rows_per_block + threadIdx.x / G;
+    const int lane = threadIdx.x % G;
+    typename Acc::type acc = Acc::identity();
+    if (o < p.O) {
+        for (int64_t r = lane; r < p.R; r += G) {
+            T x[F<T>::NIN][1];
+            load_points<F, T, 1, 1>(p, o, r, 0, x);
+            acc = Acc::combine(acc, Acc::lift(map_point<F, T, 1>(x, 0)));
+        }
+    }
+    acc = wave_reduce<Acc>(acc, G);  // every lane of the wave takes part (rows past O hold identities)
+    if (o < p.O && lane == 0) store_result<Acc, T, true>(p, acc, o, 0, 0);
+}
+
+// ---- col form ----------------------------------------------------------------------------------
+// block = TX x TY threads (TX * TY == 256); a thread owns V consecutive i and walks r with step TY.
+template <template <typename> class F, template <typename> class AccT, typename T, int V, bool FINAL>
+__global__ __launch_bounds__(kBlock) void red_cols(const RedParams p, const int TX) {
+    using Acc = AccT<T>;
+    using acc_t = typename Acc::type;
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    acc_t *smem = reinterpret_cast<acc_t *>(smem_raw);
+    const int TY = kBlock / TX;
+    const int tx = threadIdx.x % TX;
+    const int ty = threadIdx.x / TX;
+    const int64_t i0 = (static_cast<int64_t>(blockIdx.x) * TX + tx) * V;
+    const int64_t o = blockIdx.y / p.n_chunks;
+    const int chunk = blockIdx.y % p.n_chunks;
+    const int64_t r_begin = static_cast<int64_t>(chunk) * p.r_chunk;
+    const int64_t r_end = min(r_begin + p.r_chunk, p.R);
+    const bool active = i0 < p.I;  // planner guarantees I % V == 0 when V > 1
+    acc_t acc[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) acc[j] = Acc::identity();
+    if (active) {
+#pragma unroll 4
+        for (int64_t r = r_begin + ty; r < r_end; r += TY) {
+            T x[F<T>::NIN][V];
+            load_points<F, T, V, 2>(p, o, r, i0, x);
+#pragma unroll
+            for (int j = 0; j < V; ++j) acc[j] = Acc::combine(acc[j], Acc::lift(map_point<F, T, V>(x, j)));
+        }
+    }
+    if (TY > 1) {
+#pragma unroll
+        for (int j = 0; j < V; ++j) smem[(ty * TX + tx) * V + j] = acc[j];
+        __syncthreads();
+        for (int half = TY >> 1; half > 0; half >>= 1) {
+            if (ty < half) {
+#pragma unroll
+                for (int j = 0; j < V; ++j) {
+                    acc[j] = Acc::combine(acc[j], smem[((ty + half) * TX + tx) * V + j]);
+                    smem[(ty * TX + tx) * V + j] = acc[j];
+                }
+            }
+            __syncthreads();
+        }
+    }
+    if (active && ty == 0) {
+#pragma unroll
+        for (int j = 0; j < V; ++j) store_result<Acc, T, FINAL>(p, acc[j], o, i0 + j, chunk);
+    }
+}
+
+// ---- second stage: combine chunk partials in chunk order -----------------------------------------
+template <template <typename> class AccT, typename T>
+__global__ __launch_bounds__(kBlock) void red_finish(const void *partial, T *out, const int n_chunks, const int64_t O,
+                                                     const int64_t I, const int64_t ostr_o, const int64_t ostr_i,
+                                                     const int G) {
+    using Acc = AccT<T>;
+    const typename Acc::type *part = static_cast<const typename Acc::type *>(partial);
+    const int per_block = kBlock / G;
+    const int64_t e = static_cast<int64_t>(blockIdx.x) * per_block + threadIdx.x / G;
+    const int lane = threadIdx.x % G;
+    const int64_t n_out = O * I;
+    typename Acc::type acc = Acc::identity();
+    if (e < n_out)
+        for (int c = lane; c < n_chunks; c += G) acc = Acc::combine(acc, part[static_cast<int64_t>(c) * n_out + e]);
+    acc = wave_reduce<Acc>(acc, G);
+    if (e < n_out && lane == 0) out[(e / I) * ostr_o + (e % I) * ostr_i] = Acc::finish(acc);
+}
+
+// ---- planning ------------------------------------------------------------------------------------
+struct RedPlan {
+    bool row_form;
+    bool block_per_row;
+    int G;         // row_group lanes per row, or finish lanes per output
+    int V;         // vector width in elements (1 or 16 / sizeof(T))
+    int TX;        // col form
+    int n_chunks;
+    int64_t r_chunk;
+};
+
+static int pow2_ceil(int64_t v) {
+    int p = 1;
+    while (p < v && p < (1 << 30)) p <<= 1;
+    return p;
+}
+
+// enough blocks to give each of the 256 CUs several
+constexpr int64_t kTargetBlocks = 2048;
+
+static RedPlan plan_reduce(int64_t O, int64_t R, int64_t I, int vec, bool vec_ok, size_t acc_size,
+                           size_t workspace_bytes) {
+    RedPlan pl = {};
+    pl.n_chunks = 1;
+    pl.r_chunk = R;
+    pl.V = 1;
+    const int64_t max_chunks_ws = static_cast<int64_t>(workspace_bytes / (acc_size * (size_t)(O * I)));
+    if (I == 1) {
+        pl.row_form = true;
+        if (R > 1024 || (R > 64 && O < 64)) {
+            pl.block_per_row = true;
+            pl.V = vec_ok ? vec : 1;
+            const int64_t per_block_min = static_cast<int64_t>(kBlock) * pl.V * 4;  // >= 4 vectors per thread
+            int64_t chunks = std::min<int64_t>(ceil_div(kTargetBlocks, O), ceil_div(R, per_block_min));
+            chunks = std::min<int64_t>(chunks, std::min<int64_t>(max_chunks_ws, 65535));
+            if (chunks > 1) {
+                int64_t rc = ceil_div(R, chunks);
+                rc = ceil_div(rc, pl.V) * pl.V;  // chunk starts stay vector-aligned within the row
+                pl.r_chunk = rc;
+                pl.n_chunks = static_cast<int>(ceil_div(R, rc));
+            }
+        } else {
+            pl.G = std::min(64, pow2_ceil(ceil_div(R, 4)));
+        }
+    } else {
+        pl.row_form = false;
+        pl.V = (vec_ok && I % vec == 0) ? vec : 1;
+        pl.TX = std::min<int>(kBlock, pow2_ceil(ceil_div(I, pl.V)));
+        const int TY = kBlock / pl.TX;
+        const int64_t blocks_x = ceil_div(ceil_div(I, pl.V), pl.TX);
+        int64_t chunks = std::min<int64_t>(ceil_div(kTargetBlocks, blocks_x * O), ceil_div(R, static_cast<int64_t>(TY) * 8));
+        chunks = std::min<int64_t>(chunks, max_chunks_ws);
+        if (O * chunks > 65535) chunks = std::max<int64_t>(1, 65535 / O);
+        if (chunks > 1) {
+            pl.r_chunk = ceil_div(R, chunks);
+            pl.n_chunks = static_cast<int>(ceil_div(R, pl.r_chunk));
+        }
+    }
+    if (pl.n_chunks > 1) pl.G = (O * I <= 4096) ? 64 : 1;
+    return pl;
+}
+
+template <template <typename> class F, template <typename> class AccT, typename T>
+static int launch_reduce(const RedParams &base, bool vec_ok, void *workspace, size_t workspace_bytes,
+                         hipStream_t s) {
+    using Acc = AccT<T>;
+    using acc_t = typename Acc::type;
+    constexpr int VEC = RVec<T>::N;
+    const RedPlan pl = plan_reduce(base.O, base.R, base.I, VEC, vec_ok, sizeof(acc_t), workspace ? workspace_bytes : 0);
+    RedParams p = base;
+    p.n_chunks = pl.n_chunks;
+    p.r_chunk = pl.r_chunk;
+    const bool two_stage = pl.n_chunks > 1;
+    void *final_out = p.out;
+    if (two_stage) p.out = workspace;
+
+    if (pl.row_form && !pl.block_per_row) {
+        const int rows_per_block = kBlock / pl.G;
+        const int64_t blocks = ceil_div(p.O, rows_per_block);
+        if (blocks > 0x7fffffffLL) {
+            set_error("map_reduce: too many rows");
+            return AGMI_ERR_UNSUPPORTED;
+        }
+        hipLaunchKernelGGL((red_row_group<F, AccT, T>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p, pl.G);
+    } else if (pl.row_form) {
+        if (p.O > 0x7fffffffLL) {
+            set_error("map_reduce: too many rows");
+            return AGMI_ERR_UNSUPPORTED;
+        }
+        const dim3 grid((unsigned)p.O, (unsigned)pl.n_chunks);
+#define AGMI_ROW(VV)                                                                                          \
+    do {                                                                                                      \
+        if (two_stage)                                                                                        \
+            hipLaunchKernelGGL((red_row_block<F, AccT, T, VV, false>), grid, dim3(kBlock), 0, s, p);          \
+        else                                                                                                  \
+            hipLaunchKernelGGL((red_row_block<F, AccT, T, VV, true>), grid, dim3(kBlock), 0, s, p);           \
+    } while (0)
+        if (pl.V > 1)
+            AGMI_ROW(VEC);
+        else
+            AGMI_ROW(1);
+#undef AGMI_ROW
+    } else {
+        const int64_t blocks_x = ceil_div(ceil_div(p.I, pl.V), pl.TX);
+        if (blocks_x > 0x7fffffffLL || p.O * pl.n_chunks > 65535) {
+            set_error("map_reduce: grid too large (outer extent %lld)", (long long)p.O);
+            return AGMI_ERR_UNSUPPORTED;
+        }
+        const dim3 grid((unsigned)blocks_x, (unsigned)(p.O * pl.n_chunks));
+        const size_t smem = (kBlock / pl.TX > 1) ? sizeof(acc_t) * kBlock * pl.V : 0;
+#define AGMI_COL(VV)                                                                                          \
+    do {                                                                                                      \
+        if (two_stage)                                                                                        \
+            hipLaunchKernelGGL((red_cols<F, AccT, T, VV, false>), grid, dim3(kBlock), smem, s, p, pl.TX);     \
+        else                                                                                                  \
+            hipLaunchKernelGGL((red_cols<F, AccT, T, VV, true>), grid, dim3(kBlock), smem, s, p, pl.TX);      \
+    } while (0)
+        if (pl.V > 1)
+            AGMI_COL(VEC);
+        else
+            AGMI_COL(1);
+#undef AGMI_COL
+    }
+    if (int rc = hip_check(hipGetLastError(), "map_reduce launch")) return rc;
+    if (two_stage) {
+        const int per_block = kBlock / pl.G;
+        const int64_t blocks = ceil_div(p.O * p.I, per_block);
+        hipLaunchKernelGGL((red_finish<AccT, T>), dim3((unsigned)blocks), dim3(kBlock), 0, s, workspace,
+                           static_cast<T *>(final_out), pl.n_chunks, p.O, p.I, p.ostr_o, p.ostr_i, pl.G);
+        if (int rc = hip_check(hipGetLastError(), "map_reduce finish launch")) return rc;
+    }
+    return 0;
+}
+
+// Canonical (O, R, I) view of a merged index space, or failure for patterns such as
+// reduced-kept-reduced that need two passes.
+static bool canonical_ori(const Merged &m, int n_operands, RedParams *p, int64_t (*ostr)[3]) {
+    // pattern of groups after merging: sequences K, R, KR, RK, KRK
+    int idx_o = -1, idx_r = -1, idx_i = -1;
+    if (m.ndim == 1) {
+        (m.group[0] ? idx_r : idx_i) = 0;
+    } else if (m.ndim == 2) {
+        if (!m.group[0] && m.group[1]) {
+            idx_o = 0;
+            idx_r = 1;
+        } else if (m.group[0] && !m.group[1]) {
+            idx_r = 0;
+            idx_i = 1;
+        } else {
+            return false;
+        }
+    } else if (m.ndim == 3 && !m.group[0] && m.group[1] && !m.group[2]) {
+        idx_o = 0;
+        idx_r = 1;
+        idx_i = 2;
+    } else {
+        return false;
+    }
+    p->O = idx_o >= 0 ? m.shape[idx_o] : 1;
+    p->R = idx_r >= 0 ? m.shape[idx_r] : 1;
+    p->I = idx_i >= 0 ? m.shape[idx_i] : 1;
+    for (int k = 0; k < n_operands; ++k) {
+        ostr[k][0] = idx_o >= 0 ? m.stride[k][idx_o] : 0;
+        ostr[k][1] = idx_r >= 0 ? m.stride[k][idx_r] : 0;
+        ostr[k][2] = idx_i >= 0 ? m.stride[k][idx_i] : 0;
+    }
+    return true;
+}
+
+struct RedSetup {
+    RedParams p;
+    bool vec_ok;
+};
+
+static int setup_reduce(int ndim, const int64_t *shape, const uint8_t *reduce_axes, const agmi_array *out, int n_in,
+                        const agmi_array *ins, const double *scalars, RedSetup *st, bool *empty) {
+    if (!out || !ins || !reduce_axes || n_in < 1 || n_in > AGMI_MAX_INPUTS) {
+        set_error("map_reduce: bad arguments");
+        return AGMI_ERR_ARG;
+    }
+    int64_t out_strides[AGMI_MAX_DIMS];
+    uint8_t group[AGMI_MAX_DIMS];
+    if (ndim > AGMI_MAX_DIMS || ndim < 0) {
+        set_error("map_reduce: rank %d", ndim);
+        return AGMI_ERR_ARG;
+    }
+    for (int d = 0; d < ndim; ++d) {
+        group[d] = reduce_axes[d] ? 1 : 0;
+        out_strides[d] = group[d] ? 0 : out->strides[d];
+    }
+    const int64_t *strides[kMaxOperands];
+    strides[0] = out_strides;
+    for (int k = 0; k < n_in; ++k) strides[1 + k] = ins[k].data ? ins[k].strides : nullptr;
+    Merged m;
+    if (!merge_axes(ndim, shape, group, 1 + n_in, strides, &m)) return AGMI_ERR_ARG;
+    *empty = false;
+    if (m.n == 0) {
+        // an empty reduced axis still produces identities; callers handle that case with fill
+        *empty = true;
+        return 0;
+    }
+    RedParams &p = st->p;
+    p = RedParams{};
+    int64_t ori[kMaxOperands][3];
+    if (!canonical_ori(m, 1 + n_in, &p, ori)) {
+        set_error("map_reduce: reduced axes are not one contiguous group after merging; reduce in two calls");
+        return AGMI_ERR_UNSUPPORTED;
+    }
+    p.out = out->data;
+    p.ostr_o = ori[0][0];
+    p.ostr_i = ori[0][2];
+    st->vec_ok = true;
+    const int ax = (p.I == 1) ? 1 : 2;
+    for (int k = 0; k < n_in; ++k) {
+        p.in[k] = ins[k].data;
+        if (!ins[k].data) {
+            if (!scalars) {
+                set_error("map_reduce: scalar slot %d without scalars array", k);
+                return AGMI_ERR_ARG;
+            }
+            p.scalar_mask |= 1u << k;
+            p.scalar[k] = scalars[k];
+        } else {
+            for (int a = 0; a < 3; ++a) p.istr[k][a] = ori[1 + k][a];
+            if (p.istr[k][ax] != 0 && p.istr[k][ax] != 1) st->vec_ok = false;
+        }
+    }
+    if (p.out == nullptr) {
+        set_error("map_reduce: output is null");
+        return AGMI_ERR_ARG;
+    }
+    return 0;
+}
+
+template <typename T>
+static size_t acc_size_of(int red) {
+    return red == AGMI_RED_LOGSUMEXP ? sizeof(LsePair<T>) : sizeof(T);
+}
+
+template <template <typename> class F, typename T>
+static int dispatch_red(int red, const RedSetup &st, void *ws, size_t ws_bytes, hipStream_t s) {
+    if (F<T>::NOUT != 1) {
+        set_error("map_reduce: op has %d outputs", F<T>::NOUT);
+        return AGMI_ERR_ARG;
+    }
+    switch (red) {
+        case AGMI_RED_SUM: return launch_reduce<F, AccSum, T>(st.p, st.vec_ok, ws, ws_bytes, s);
+        default: break;
+    }
+    set_error("map_reduce: reduction %d is only available with AGMI_OP_COPY", red);
+    return AGMI_ERR_UNSUPPORTED;
+}
+
+template <typename T>
+static int dispatch_red_copy(int red, const RedSetup &st, void *ws, size_t ws_bytes, hipStream_t s) {
+    switch (red) {
+        case AGMI_RED_SUM: return launch_reduce<FCopy, AccSum, T>(st.p, st.vec_ok, ws, ws_bytes, s);
+        case AGMI_RED_MAX: return launch_reduce<FCopy, AccMax, T>(st.p, st.vec_ok, ws, ws_bytes, s);
+        case AGMI_RED_MIN: return launch_reduce<FCopy, AccMin, T>(st.p, st.vec_ok, ws, ws_bytes, s);
+        case AGMI_RED_PROD: return launch_reduce<FCopy, AccProd, T>(st.p, st.vec_ok, ws, ws_bytes, s);
+        case AGMI_RED_LOGSUMEXP: return launch_reduce<FCopy, AccLse, T>(st.p, st.vec_ok, ws, ws_bytes, s);
+        default: set_error("map_reduce: unknown reduction %d", red); return AGMI_ERR_ARG;
+    }
+}
+
+}  // namespace agmi
+
+using namespace agmi;
+
+// ops that may feed a sum: the rules whose cotangent is unbroadcast, the logsumexp JVP, products
+#define AGMI_FOR_EACH_REDUCE_OP(X) \
+    X(AGMI_OP_NEG, FNeg)           \
+    X(AGMI_OP_MUL, FMul)           \
+    X(AGMI_OP_DIV, FDiv)           \
+    X(AGMI_OP_SQUARE, FSquare)     \
+    X(AGMI_OP_ABS, FAbs)           \
+    X(AGMI_OP_DIV_VJP1, FDivVjp1)  \
+    X(AGMI_OP_TANH_VJP, FTanhVjp)  \
+    X(AGMI_OP_POW_VJP0, FPowVjp0)  \
+    X(AGMI_OP_POW_VJP1, FPowVjp1)  \
+    X(AGMI_OP_LSE_VJP, FLseVjp)    \
+    X(AGMI_OP_CHOOSE_VJP, FChooseVjp)
+
+extern "C" int agmi_map_reduce(int op, int red, int dtype, int ndim, const int64_t *shape,
+                               const uint8_t *reduce_axes, const agmi_array *out, int n_in,
+                               const agmi_array *ins, const double *scalars, void *workspace,
+                               size_t workspace_bytes, void *stream) {
+    RedSetup st;
+    bool empty = false;
+    if (int rc = setup_reduce(ndim, shape, reduce_axes, out, n_in, ins, scalars, &st, &empty)) return rc;
+    if (empty) return 0;
+    hipStream_t s = as_stream(stream);
+    if (dtype != AGMI_F32 && dtype != AGMI_F64) {
+        set_error("map_reduce: dtype %d is not a floating type", dtype);
+        return AGMI_ERR_ARG;
+    }
+    if (op == AGMI_OP_COPY) {
+        if (n_in != 1) {
+            set_error("map_reduce: AGMI_OP_COPY takes one input");
+            return AGMI_ERR_ARG;
+        }
+        return dtype == AGMI_F32 ? dispatch_red_copy<float>(red, st, workspace, workspace_bytes, s)
+                                 : dispatch_red_copy<double>(red, st, workspace, workspace_bytes, s);
+    }
+#define AGMI_CASE(OP, FN)                                                                        \
+    case OP:                                                                                     \
+        if (n_in != FN<float>::NIN) {                                                            \
+            set_error("map_reduce: op takes %d inputs, got %d", FN<float>::NIN, n_in);           \
+            return AGMI_ERR_ARG;                                                                 \
+        }                                                                                        \
+        return dtype == AGMI_F32 ? dispatch_red<FN, float>(red, st, workspace, workspace_bytes, s) \
+                                 : dispatch_red<FN, double>(red, st, workspace, workspace_bytes, s);
+    switch (op) {
+        AGMI_FOR_EACH_REDUCE_OP(AGMI_CASE)
+        default: break;
+    }
+#undef AGMI_CASE
+    set_error("map_reduce: op %d cannot be fused into a reduction", op);
+    return AGMI_ERR_UNSUPPORTED;
+}
+
+extern "C" size_t agmi_map_reduce_workspace_bytes(int red, int dtype, int ndim, const int64_t *shape,
+                                                  const uint8_t *reduce_axes) {
+    // Upper bound over every layout: partials for kTargetBlocks chunks can never be needed for
+    // more than kTargetBlocks * (number of outputs) accumulators, and never more chunks than
+    // there are reduced points.
+    if (ndim < 0 || ndim > AGMI_MAX_DIMS || !shape || !reduce_axes) return 0;
+    int64_t kept = 1, reduced = 1;
+    for (int d = 0; d < ndim; ++d) (reduce_axes[d] ? reduced : kept) *= shape[d];
+    if (kept <= 0 || reduced <= 1) return 0;
+    const size_t acc = dtype == AGMI_F64 ? acc_size_of<double>(red) : acc_size_of<float>(red);
+    const int64_t chunks = std::min<int64_t>(kTargetBlocks, reduced);
+    return static_cast<size_t>(chunks) * static_cast<size_t>(kept) * acc;
+}

@@ -1,0 +1,429 @@
+"""``DevArray``: the device-resident array value type, and the raw (untraced) operations on it.
+
+A ``DevArray`` is an immutable n-d array in MI355X HBM.  It is a thin wrapper around a
+``torch.Tensor`` used only as a memory handle: shape, strides and offset are the tensor's
+view metadata (slicing, reshaping, transposing and broadcasting are views and launch
+nothing), and every arithmetic operation launches a kernel of ``libagmi.so`` on torch's
+current stream.  It plays the role ``numpy.ndarray`` plays for the reference
+(autograd/numpy/numpy_boxes.py:12-189 boxes ndarrays; ``DevArrayBox`` boxes these).
+
+dtype promotion follows NumPy 2 (NEP 50): Python scalars are weak, arrays and NumPy
+scalars are strong.
+"""
+
+import numbers
+
+import numpy as onp
+import torch
+
+from .. import _lib
+from .._lib import Cmp, Op, Red
+
+_FLOATS = (onp.dtype("float32"), onp.dtype("float64"))
+_F64 = onp.dtype("float64")
+_BOOL = onp.dtype("bool")
+_I64 = onp.dtype("int64")
+
+
+class DevArray:
+    """n-d array in GPU memory; arithmetic is hand-written HIP kernels."""
+
+    __slots__ = ("_t", "dtype")
+    __array_ufunc__ = None  # NumPy binary operators defer to ours (ndarray * DevArray -> __rmul__)
+    __array_priority__ = 200.0
+
+    def __init__(self, tensor, dtype=None):
+        self._t = tensor
+        self.dtype = dtype if dtype is not None else _lib.NUMPY_DTYPE[tensor.dtype]
+
+    # ---- metadata ----------------------------------------------------------------------
+    @property
+    def shape(self):
+        return tuple(self._t.shape)
+
+    @property
+    def ndim(self):
+        return self._t.dim()
+
+    @property
+    def size(self):
+        return self._t.numel()
+
+    @property
+    def strides(self):
+        item = self.dtype.itemsize
+        return tuple(s * item for s in self._t.stride())
+
+    @property
+    def T(self):
+        from . import wrapper
+
+        return wrapper.transpose(self)
+
+    def __len__(self):
+        if self._t.dim() == 0:
+            raise TypeError("len() of unsized object")
+        return self._t.shape[0]
+
+    def __iter__(self):
+        if self._t.dim() == 0:
+            raise TypeError("iteration over a 0-d array")
+        return (self[i] for i in range(self._t.shape[0]))
+
+    # ---- host transfer (synchronises) ------------------------------------------------------
+    def numpy(self):
+        """Copy to a host ``numpy.ndarray`` (blocks until the stream has produced the data)."""
+        return self._t.cpu().numpy()
+
+    def __array__(self, dtype=None, copy=None):
+        a = self.numpy()
+        return a.astype(dtype) if dtype is not None else a
+
+    def item(self):
+        if self._t.numel() != 1:
+            raise ValueError("can only convert an array of size 1 to a Python scalar")
+        return self._t.item()
+
+    def __float__(self):
+        return float(self.item())
+
+    def __int__(self):
+        return int(self.item())
+
+    def __bool__(self):
+        if self._t.numel() != 1:
+            raise ValueError("The truth value of an array with more than one element is ambiguous.")
+        return bool(self.item())
+
+    def __repr__(self):
+        return f"DevArray({self.numpy()!r}, device='{self._t.device}')"
+
+    __str__ = __repr__
+    __hash__ = object.__hash__
+
+    def __setitem__(self, idx, value):
+        raise TypeError("DevArray is immutable: item assignment is not supported")
+
+    # ---- operators and methods are attached by wrapper.py (they are traced primitives) ------
+
+
+def is_scalar(x):
+    return isinstance(x, (numbers.Number, onp.generic)) and not isinstance(x, DevArray)
+
+
+# --------------------------------------------------------------------------------------------
+# construction
+# --------------------------------------------------------------------------------------------
+def _np_dtype(dtype):
+    return None if dtype is None else onp.dtype(dtype)
+
+
+def from_numpy(a, dtype=None):
+    """Upload a host array (one H2D copy; no arithmetic)."""
+    a = onp.asarray(a, dtype=dtype)
+    if a.dtype not in _lib.DTYPE_CODE:
+        if a.dtype.kind == "f":
+            a = a.astype(onp.float64 if a.dtype.itemsize > 4 else onp.float32)
+        elif a.dtype.kind in "iu":
+            a = a.astype(onp.int64)
+        else:
+            raise TypeError(f"dtype {a.dtype} is not supported on the device")
+    a = onp.ascontiguousarray(a)
+    t = torch.from_numpy(a.copy() if not a.flags.writeable else a).to(_lib.device())
+    return DevArray(t, a.dtype)
+
+
+def asarray(x, dtype=None):
+    """Device array from a DevArray (no copy), host array, nested list or scalar."""
+    dtype = _np_dtype(dtype)
+    if isinstance(x, DevArray):
+        return x if dtype is None or dtype == x.dtype else astype(x, dtype)
+    if isinstance(x, (numbers.Number, onp.generic)):
+        dt = dtype or (onp.asarray(x).dtype if isinstance(x, onp.generic) else (_F64 if not isinstance(x, (bool, int)) else onp.asarray(x).dtype))
+        if dt in _FLOATS:
+            return full((), float(x), dt)
+        return from_numpy(onp.asarray(x), dt)
+    if isinstance(x, (list, tuple)) and any(isinstance(e, DevArray) for e in x):
+        from . import wrapper
+
+        return wrapper.stack([asarray(e) for e in x])
+    return from_numpy(x, dtype)
+
+
+def to_numpy(x):
+    if isinstance(x, DevArray):
+        return x.numpy()
+    return onp.asarray(x)
+
+
+def empty(shape, dtype=_F64):
+    shape = (shape,) if isinstance(shape, numbers.Integral) else tuple(shape)
+    dtype = onp.dtype(dtype)
+    return DevArray(_lib.empty(shape, dtype), dtype)
+
+
+def full(shape, fill_value, dtype=None):
+    dtype = onp.dtype(dtype) if dtype is not None else onp.asarray(fill_value).dtype
+    if dtype.kind == "i" and dtype not in _lib.DTYPE_CODE:
+        dtype = _I64
+    out = empty(shape, dtype)
+    _lib.fill(_lib.DTYPE_CODE[dtype], out._t, fill_value)
+    return out
+
+
+def zeros(shape, dtype=_F64):
+    return full(shape, 0.0, onp.dtype(dtype))
+
+
+def ones(shape, dtype=_F64):
+    return full(shape, 1.0, onp.dtype(dtype))
+
+
+# --------------------------------------------------------------------------------------------
+# operand preparation
+# --------------------------------------------------------------------------------------------
+def result_dtype(*operands):
+    """NumPy-2 result type of an operation on ``operands`` (Python scalars are weak)."""
+    args = []
+    first = None
+    same = True
+    for x in operands:
+        if isinstance(x, DevArray):
+            if first is None:
+                first = x.dtype
+            elif x.dtype != first:
+                same = False
+            args.append(x.dtype)
+        elif isinstance(x, onp.ndarray):
+            same = False
+            args.append(x.dtype)
+        elif isinstance(x, onp.generic):
+            same = False
+            args.append(x.dtype)
+        elif isinstance(x, (bool, int, float)):
+            args.append(x)
+        else:
+            same = False
+            args.append(onp.asarray(x).dtype)
+    if first is not None and same and first in _FLOATS:
+        return first  # fast path: weak scalars never change a float array's dtype
+    return onp.result_type(*args)
+
+
+def _float_dtype(dt):
+    """dtype a floating ufunc (exp, true_divide, ...) computes in for input dtype ``dt``."""
+    if dt in _FLOATS:
+        return dt
+    if dt.kind == "f":
+        return onp.dtype("float32") if dt.itemsize <= 4 else _F64
+    return _F64
+
+
+def astype(x, dtype):
+    dtype = onp.dtype(dtype)
+    if not isinstance(x, DevArray):
+        return asarray(x, dtype)
+    if dtype == x.dtype:
+        return copy(x)
+    if dtype not in _lib.DTYPE_CODE:
+        raise TypeError(f"dtype {dtype} is not supported on the device")
+    out = empty(x.shape, dtype)
+    _lib.cast(_lib.DTYPE_CODE[x.dtype], _lib.DTYPE_CODE[dtype], x.shape, out._t, x._t)
+    return out
+
+
+def _operand(x, dtype):
+    """tensor (of ``dtype``) or Python float for a kernel input slot."""
+    if isinstance(x, DevArray):
+        if x.dtype != dtype:
+            x = astype(x, dtype)
+        return x._t
+    if isinstance(x, (numbers.Number, onp.generic)):
+        return float(x)
+    return asarray(x, dtype)._t
+
+
+def _bshape(operands):
+    shape = None
+    for t in operands:
+        if isinstance(t, torch.Tensor):
+            s = tuple(t.shape)
+            if shape is None:
+                shape = s
+            elif s != shape:
+                shape = tuple(onp.broadcast_shapes(shape, s))
+    return shape
+
+
+def _expand(t, shape):
+    if isinstance(t, torch.Tensor) and tuple(t.shape) != shape:
+        return t.expand(shape)
+    return t
+
+
+def _lift_scalars(operands, dtype):
+    """All operands are by-value scalars: put the first on the device as a 0-d array."""
+    return (full((), operands[0], dtype)._t,) + tuple(operands[1:])
+
+
+def map_op(op, dtype, *xs, out=None, n_out=1):
+    """Launch elementwise ``op`` on broadcast operands; returns DevArray (or a tuple)."""
+    ops = tuple(_operand(x, dtype) for x in xs)
+    shape = _bshape(ops)
+    if shape is None:
+        ops = _lift_scalars(ops, dtype)
+        shape = ()
+    ops = tuple(_expand(t, shape) for t in ops)
+    code = _lib.DTYPE_CODE[dtype]
+    if out is not None:
+        _lib.elementwise(op, code, shape, (out._t,), ops)
+        return out
+    outs = tuple(_lib.empty(shape, dtype) for _ in range(n_out))
+    _lib.elementwise(op, code, shape, outs, ops)
+    if n_out == 1:
+        return DevArray(outs[0], dtype)
+    return tuple(DevArray(t, dtype) for t in outs)
+
+
+def float_map(op, *xs):
+    """Floating ufunc: compute in the promoted floating dtype."""
+    return map_op(op, _float_dtype(result_dtype(*xs)), *xs)
+
+
+def arith_map(op, *xs):
+    """add/subtract/multiply/...: promoted dtype, computed in floating point.
+
+    Integer and bool arrays are promoted to float64 (integer arithmetic has no kernels:
+    the differentiable path is floating point)."""
+    return map_op(op, _float_dtype(result_dtype(*xs)), *xs)
+
+
+def copy(x):
+    return map_op(Op.COPY, x.dtype, x) if x.dtype in _FLOATS else astype_copy(x)
+
+
+def astype_copy(x):
+    out = empty(x.shape, x.dtype)
+    code = _lib.DTYPE_CODE[x.dtype]
+    _lib.cast(code, code, x.shape, out._t, x._t)
+    return out
+
+
+def contiguous(x):
+    return x if x._t.is_contiguous() else copy(x)
+
+
+def compare(cmp, a, b):
+    dt = _float_dtype(result_dtype(a, b))
+    ops = (_operand(a, dt), _operand(b, dt))
+    shape = _bshape(ops)
+    if shape is None:
+        ops = _lift_scalars(ops, dt)
+        shape = ()
+    ops = tuple(_expand(t, shape) for t in ops)
+    out = empty(shape, _BOOL)
+    _lib.compare(cmp, _lib.DTYPE_CODE[dt], shape, out._t, ops)
+    return out
+
+
+# --------------------------------------------------------------------------------------------
+# reductions
+# --------------------------------------------------------------------------------------------
+def normalize_axes(axis, ndim):
+    if axis is None:
+        return tuple(range(ndim))
+    if isinstance(axis, (numbers.Integral, onp.integer)):
+        axis = (int(axis),)
+    axes = tuple(sorted({int(a) % ndim if ndim else 0 for a in axis}))
+    for a in axis:
+        if not -max(ndim, 1) <= int(a) < max(ndim, 1):
+            raise ValueError(f"axis {a} is out of bounds for array of dimension {ndim}")
+    return axes
+
+
+def reduce_shape(shape, axes, keepdims):
+    if keepdims:
+        return tuple(1 if d in axes else s for d, s in enumerate(shape))
+    return tuple(s for d, s in enumerate(shape) if d not in axes)
+
+
+_IDENTITY = {Red.SUM: 0.0, Red.PROD: 1.0}
+
+
+def map_reduce(op, red, dtype, xs, axes, keepdims, shape=None):
+    """``RED_axes op(xs...)`` with ``xs`` broadcast to ``shape`` (default: their broadcast)."""
+    ops = tuple(_operand(x, dtype) for x in xs)
+    if shape is None:
+        shape = _bshape(ops)
+    if shape is None:
+        ops = _lift_scalars(ops, dtype)
+        shape = ()
+    ops = tuple(_expand(t, shape) for t in ops)
+    nd = len(shape)
+    axes = tuple(axes)
+    mask = [d in axes for d in range(nd)]
+    kept_shape = reduce_shape(shape, axes, True)
+    out_t = _lib.empty(kept_shape, dtype)
+    n_reduced = 1
+    for d in axes:
+        n_reduced *= shape[d]
+    code = _lib.DTYPE_CODE[dtype]
+    if out_t.numel() == 0:
+        pass
+    elif n_reduced == 0:
+        if red not in _IDENTITY:
+            raise ValueError("zero-size array to reduction operation which has no identity")
+        _lib.fill(code, out_t, _IDENTITY[red])
+    elif not _lib.map_reduce(op, red, code, shape, mask, out_t, ops):
+        # reduced axes interleaved with kept ones: one group of adjacent axes at a time
+        if red == Red.LOGSUMEXP:
+            raise NotImplementedError("logsumexp over non-adjacent axes of a non-contiguous layout")
+        cur = map_op(op, dtype, *[DevArray(t, dtype) if isinstance(t, torch.Tensor) else t for t in ops])
+        for group in _adjacent_groups(axes):
+            cur = map_reduce(Op.COPY, red, dtype, (cur,), group, True)
+        out_t = cur._t
+    out = DevArray(out_t, dtype)
+    if not keepdims and axes:
+        out = DevArray(out_t.reshape(reduce_shape(shape, axes, False)), dtype)
+    return out
+
+
+def _adjacent_groups(axes):
+    groups, cur = [], []
+    for a in axes:
+        if cur and a != cur[-1] + 1:
+            groups.append(tuple(cur))
+            cur = []
+        cur.append(a)
+    if cur:
+        groups.append(tuple(cur))
+    return groups
+
+
+# --------------------------------------------------------------------------------------------
+# contractions
+# --------------------------------------------------------------------------------------------
+def gemm2d(a, b, dtype, out=None, beta=0.0):
+    """``a @ b`` for 2-d tensors of ``dtype`` (any strides) -> contiguous (M, N) tensor."""
+    M, K = a.shape
+    K2, N = b.shape
+    if K != K2:
+        raise ValueError(f"shapes {tuple(a.shape)} and {tuple(b.shape)} not aligned: {K} (dim 1) != {K2} (dim 0)")
+    c = out if out is not None else _lib.empty((M, N), dtype)
+    if M and N:
+        _lib.gemm(_lib.DTYPE_CODE[dtype], 1, M, N, K, 1.0, a, a.stride(0), a.stride(1), 0, b, b.stride(0),
+                  b.stride(1), 0, beta, c, max(N, 1), 0)
+    return c
+
+
+def gemm_batched(a, b, dtype):
+    """(B, M, K) @ (B, K, N) with broadcastable (possibly stride-0) batch axes."""
+    Bn, M, K = a.shape
+    _, K2, N = b.shape
+    if K != K2:
+        raise ValueError(f"matmul: inner dimensions differ ({K} vs {K2})")
+    c = _lib.empty((Bn, M, N), dtype)
+    if Bn and M and N:
+        _lib.gemm(_lib.DTYPE_CODE[dtype], Bn, M, N, K, 1.0, a, a.stride(1), a.stride(2), a.stride(0), b,
+                  b.stride(1), b.stride(2), b.stride(0), 0.0, c, max(N, 1), M * N)
+    return c

@@ -1,0 +1,615 @@
+"""Reverse-mode rules of the device namespace.
+
+Every rule computes what the cited rule of the reference's autograd/numpy/numpy_vjps.py
+computes.  Each has two forms:
+
+* concrete - when the cotangent and the saved values are plain ``DevArray`` s (the outermost
+  backward pass, which is where the time goes), the whole rule, including the ``unbroadcast``
+  sum that follows a broadcasting ufunc, is ONE fused kernel launch;
+* traced - when any of them is a box (an outer differentiation is recording this backward
+  pass), the rule is written with namespace primitives exactly like the reference's, so that
+  it can itself be differentiated to any order.
+"""
+
+from functools import partial
+
+import numpy as onp
+
+from .._lib import REDUCE_FUSABLE, Op, Red
+from ..extend import SparseObject, VJPNode, defvjp, defvjp_argnum, primitive, register_notrace, vspace
+from ..tracer import isbox
+from ..util import func
+from . import devarray as D
+from . import wrapper as anp
+from .boxes import DevArrayBox
+from .devarray import DevArray
+
+# ---- functions with no derivative (numpy_vjps.py:13-68) -------------------------------------
+nograd_functions = [
+    anp.sign,
+    anp.equal,
+    anp.not_equal,
+    anp.less,
+    anp.less_equal,
+    anp.greater,
+    anp.greater_equal,
+]
+for _f in nograd_functions:
+    register_notrace(VJPNode, _f)
+
+
+def _concrete(*xs):
+    """True when no argument is a box: the fused kernels may be used."""
+    for x in xs:
+        if isbox(x):
+            return False
+    return True
+
+
+def _shape_of(x):
+    return x.shape if isinstance(x, DevArray) else onp.shape(x)
+
+
+# ---- unbroadcast (numpy_vjps.py:883-897) -----------------------------------------------------
+def unbroadcast(x, target_meta, broadcast_idx=0):
+    """Traced form: sum ``x`` down to the shape it was broadcast from."""
+    target_shape, target_ndim, _dtype, target_iscomplex = target_meta
+    while anp.ndim(x) > target_ndim:
+        x = anp.sum(x, axis=broadcast_idx)
+    for axis, size in enumerate(target_shape):
+        if size == 1:
+            x = anp.sum(x, axis=axis, keepdims=True)
+    return x
+
+
+def _fused_unbroadcast(op, target_meta, *operands):
+    """Concrete form: ``unbroadcast(op(*operands), target_meta)`` in one launch.
+
+    When the operands' broadcast shape equals the target shape this is a plain elementwise
+    kernel; otherwise the sum over the broadcast axes runs in the same pass (map-reduce), so
+    the full-size intermediate is never written.
+    """
+    target_shape, target_ndim, _dt, _c = target_meta
+    if op == Op.COPY and _shape_of(operands[0]) == tuple(target_shape):
+        return operands[0]  # add/subtract without broadcasting: the cotangent is `g` itself, no copy
+    dt = D._float_dtype(D.result_dtype(*operands))
+    shape = ()
+    for x in operands:
+        s = _shape_of(x)
+        if s != shape:
+            shape = tuple(onp.broadcast_shapes(shape, s))
+    if shape == tuple(target_shape):
+        return D.map_op(op, dt, *operands)
+    lead = len(shape) - target_ndim
+    axes = list(range(lead)) + [lead + a for a, size in enumerate(target_shape) if size == 1]
+    if op not in REDUCE_FUSABLE:
+        full = D.map_op(op, dt, *operands)
+        out = D.map_reduce(Op.COPY, Red.SUM, dt, (full,), axes, True)
+    else:
+        out = D.map_reduce(op, Red.SUM, dt, operands, axes, True, shape=shape)
+    return DevArray(out._t.reshape(tuple(target_shape)), dt) if lead else out
+
+
+def unbroadcast_f(target, f):
+    target_meta = anp.metadata(target)
+    return lambda g: unbroadcast(f(g), target_meta)
+
+
+def _binary_rule(fun, traced0, traced1, fused0, fused1):
+    """Register both cotangents of a broadcasting ufunc.
+
+    ``traced*(ans, x, y)`` return ``g -> cotangent`` written with primitives (reference form);
+    ``fused*(g, ans, x, y)`` return ``(op, operands)`` for the single-kernel form.
+    """
+
+    def maker(traced, fused, which):
+        def make(ans, x, y):
+            target = (x, y)[which]
+            meta = anp.metadata(target)
+            slow = traced(ans, x, y)
+
+            def vjp(g):
+                if _concrete(g, ans, x, y):
+                    op, operands = fused(g, ans, x, y)
+                    return _fused_unbroadcast(op, meta, *operands)
+                return unbroadcast(slow(g), meta)
+
+            return vjp
+
+        return make
+
+    defvjp(fun, maker(traced0, fused0, 0), maker(traced1, fused1, 1))
+
+
+# ---- binary ufuncs (numpy_vjps.py:76-143) ----------------------------------------------------
+_binary_rule(
+    anp.add,
+    lambda ans, x, y: lambda g: g,
+    lambda ans, x, y: lambda g: g,
+    lambda g, ans, x, y: (Op.COPY, (g,)),
+    lambda g, ans, x, y: (Op.COPY, (g,)),
+)
+_binary_rule(
+    anp.subtract,
+    lambda ans, x, y: lambda g: g,
+    lambda ans, x, y: lambda g: -g,
+    lambda g, ans, x, y: (Op.COPY, (g,)),
+    lambda g, ans, x, y: (Op.NEG, (g,)),
+)
+_binary_rule(
+    anp.multiply,
+    lambda ans, x, y: lambda g: y * g,
+    lambda ans, x, y: lambda g: x * g,
+    lambda g, ans, x, y: (Op.MUL, (y, g)),
+    lambda g, ans, x, y: (Op.MUL, (x, g)),
+)
+_binary_rule(
+    anp.true_divide,
+    lambda ans, x, y: lambda g: g / y,
+    lambda ans, x, y: lambda g: -g * x / y**2,
+    lambda g, ans, x, y: (Op.DIV, (g, y)),
+    lambda g, ans, x, y: (Op.DIV_VJP1, (g, x, y)),
+)
+_binary_rule(
+    anp.power,
+    lambda ans, x, y: lambda g: g * y * x ** anp.where(y, y - 1, 1.0),
+    lambda ans, x, y: lambda g: g * anp.log(replace_zero(x, 1.0)) * ans,
+    lambda g, ans, x, y: (Op.POW_VJP0, (g, x, y)),
+    lambda g, ans, x, y: (Op.POW_VJP1, (g, x, ans)),
+)
+for _chooser in (anp.maximum, anp.minimum):
+    _binary_rule(
+        _chooser,
+        lambda ans, x, y: lambda g: g * balanced_eq(x, ans, y),
+        lambda ans, x, y: lambda g: g * balanced_eq(y, ans, x),
+        lambda g, ans, x, y: (Op.CHOOSE_VJP, (g, x, ans, y)),
+        lambda g, ans, x, y: (Op.CHOOSE_VJP, (g, y, ans, x)),
+    )
+
+def balanced_eq(x, z, y):
+    return (x == z) / (1.0 + (x == y))
+
+
+def replace_zero(x, val):
+    return anp.where(x, x, val)
+
+
+# ---- unary ufuncs (numpy_vjps.py:157-191) ----------------------------------------------------
+def _unary_rule(fun, traced, fused):
+    """``traced(ans, x)`` -> ``g -> cotangent`` with primitives; ``fused(g, ans, x)`` -> (op, operands)."""
+
+    def make(ans, x):
+        slow = traced(ans, x)
+
+        def vjp(g):
+            if _concrete(g, ans, x):
+                op, operands = fused(g, ans, x)
+                return D.float_map(op, *operands)
+            return slow(g)
+
+        return vjp
+
+    defvjp(fun, make)
+
+
+_unary_rule(anp.negative, lambda ans, x: lambda g: -g, lambda g, ans, x: (Op.NEG, (g,)))
+_unary_rule(anp.exp, lambda ans, x: lambda g: ans * g, lambda g, ans, x: (Op.MUL, (ans, g)))
+_unary_rule(anp.log, lambda ans, x: lambda g: g / x, lambda g, ans, x: (Op.DIV, (g, x)))
+_unary_rule(anp.tanh, lambda ans, x: lambda g: g / anp.cosh(x) ** 2, lambda g, ans, x: (Op.TANH_VJP, (g, x)))
+_unary_rule(anp.sinh, lambda ans, x: lambda g: g * anp.cosh(x), lambda g, ans, x: (Op.SINH_VJP, (g, x)))
+_unary_rule(anp.cosh, lambda ans, x: lambda g: g * anp.sinh(x), lambda g, ans, x: (Op.COSH_VJP, (g, x)))
+_unary_rule(anp.sin, lambda ans, x: lambda g: g * anp.cos(x), lambda g, ans, x: (Op.SIN_VJP, (g, x)))
+_unary_rule(anp.cos, lambda ans, x: lambda g: -g * anp.sin(x), lambda g, ans, x: (Op.COS_VJP, (g, x)))
+_unary_rule(anp.sqrt, lambda ans, x: lambda g: g * 0.5 * x**-0.5, lambda g, ans, x: (Op.SQRT_VJP, (g, x)))
+_unary_rule(anp.square, lambda ans, x: lambda g: g * 2 * x, lambda g, ans, x: (Op.SQUARE_VJP, (g, x)))
+_unary_rule(anp.reciprocal, lambda ans, x: lambda g: -g / x**2, lambda g, ans, x: (Op.RECIPROCAL_VJP, (g, x)))
+_unary_rule(anp.log1p, lambda ans, x: lambda g: g / (x + 1), lambda g, ans, x: (Op.LOG1P_VJP, (g, x)))
+_unary_rule(anp.expm1, lambda ans, x: lambda g: (ans + 1) * g, lambda g, ans, x: (Op.EXPM1_VJP, (g, ans)))
+_unary_rule(
+    anp.abs,
+    lambda ans, x: lambda g: g * replace_zero(x, 0.0) / replace_zero(ans, 1.0),
+    lambda g, ans, x: (Op.ABS_VJP, (g, x, ans)),
+)
+
+defvjp(
+    anp._where3,
+    None,
+    lambda ans, c, x, y: lambda g: anp.where(c, g, anp.zeros_like(g)),
+    lambda ans, c, x, y: lambda g: anp.where(c, anp.zeros_like(g), g),
+)
+defvjp(
+    anp.astype,
+    lambda ans, A, dtype, order="K", casting="unsafe", subok=True, copy=True: lambda g: anp.astype(g, anp.result_type(A)),
+)
+
+# ---- shape-only functions (numpy_vjps.py:192-217, 407-413, 804-812) --------------------------
+defvjp(anp.reshape, lambda ans, x, shape, order=None: lambda g: anp.reshape(g, anp.shape(x), order=order))
+defvjp(anp.ravel, lambda ans, x, order=None: lambda g: anp.reshape(g, anp.shape(x), order=order))
+defvjp(anp.expand_dims, lambda ans, x, axis: lambda g: anp.reshape(g, anp.shape(x)))
+defvjp(anp.squeeze, lambda ans, x, axis=None: lambda g: anp.reshape(g, anp.shape(x)))
+defvjp(anp.swapaxes, lambda ans, x, axis1, axis2: lambda g: anp.swapaxes(g, axis2, axis1))
+defvjp(anp.moveaxis, lambda ans, a, source, destination: lambda g: anp.moveaxis(g, destination, source))
+
+
+def _grad_transpose(ans, x, axes=None):
+    if axes is not None:
+        axes = tuple(int(i) for i in onp.argsort(axes))
+    return lambda g: anp.transpose(g, axes)
+
+
+defvjp(anp.transpose, _grad_transpose)
+
+
+def _grad_atleast(ans, *arys):
+    if len(arys) > 1:
+        raise NotImplementedError("Can't handle multiple arguments yet.")
+    return lambda g: anp.reshape(g, anp.shape(arys[0]))
+
+
+for _f in (anp.atleast_1d, anp.atleast_2d, anp.atleast_3d):
+    defvjp(_f, _grad_atleast)
+
+
+def _grad_broadcast_to(ans, x, new_shape):
+    old_shape = anp.shape(x)
+    assert len(old_shape) == len(new_shape), "Can't handle extra leading dims"
+    axes = tuple(i for i, (o, n) in enumerate(zip(old_shape, new_shape)) if o == 1 and n > 1)
+    return lambda g: anp.sum(g, axis=axes, keepdims=True) if axes else g
+
+
+defvjp(anp.broadcast_to, _grad_broadcast_to)
+
+
+# ---- reductions (numpy_vjps.py:416-461) ------------------------------------------------------
+def repeat_to_match_shape(g, shape, dtype, axis, keepdims):
+    """Broadcast a reduction's cotangent back over the reduced axes; returns ``(array, num_reps)``.
+
+    The reference materialises the broadcast by adding a zeros array (numpy_vjps.py:416-427).
+    Here it is a stride-0 view (``broadcast_to`` is a primitive with its own rules), so nothing
+    is written; consumers read the small array through broadcast strides.  ``num_reps`` is a
+    NumPy integer scalar as in the reference, which keeps its promotion behaviour: a float32
+    cotangent divided by it becomes float64.
+    """
+    if shape == ():
+        return g, 1
+    axes = D.normalize_axes(axis, len(shape))
+    new_shape = tuple(1 if d in axes else s for d, s in enumerate(shape))
+    num_reps = onp.prod(onp.array(shape)[list(axes)])
+    out = anp.broadcast_to(anp.reshape(g, new_shape), shape)
+    if anp.result_type(g) != onp.result_type(anp.result_type(g), dtype):
+        out = anp.astype(out, onp.result_type(anp.result_type(g), dtype))
+    return out, num_reps
+
+
+def _grad_sum(ans, x, axis=None, keepdims=False, dtype=None, **kwargs):
+    shape, dtype = anp.shape(x), anp.result_type(x)
+    return lambda g: repeat_to_match_shape(g, shape, dtype, axis, keepdims)[0]
+
+
+defvjp(anp.sum, _grad_sum)
+
+
+def _grad_mean(ans, x, axis=None, keepdims=False, **kwargs):
+    shape, dtype = anp.shape(x), anp.result_type(x)
+
+    def vjp(g):
+        g_repeated, num_reps = repeat_to_match_shape(g, shape, dtype, axis, keepdims)
+        return g_repeated / num_reps
+
+    return vjp
+
+
+defvjp(anp._primitive_mean, _grad_mean)
+
+
+def _grad_var(ans, x, axis=None, ddof=0, keepdims=False, **kwargs):
+    # numpy_vjps.py:477-490
+    shape, dtype = anp.shape(x), anp.result_type(x)
+
+    def vjp(g):
+        g_repeated, num_reps = repeat_to_match_shape(g, shape, dtype, axis, keepdims)
+        x_minus_mean = x - anp.mean(x, axis=axis, keepdims=True)
+        return 2.0 * g_repeated * x_minus_mean / (num_reps - ddof)
+
+    return vjp
+
+
+defvjp(anp._primitive_var, _grad_var)
+
+
+def _grad_std(ans, x, axis=None, ddof=0, keepdims=False, **kwargs):
+    # numpy_vjps.py:493-512
+    shape, dtype = anp.shape(x), anp.result_type(x)
+
+    def vjp(g):
+        g_repeated, num_reps = repeat_to_match_shape(g, shape, dtype, axis, keepdims)
+        if num_reps <= 1:
+            return g_repeated * 0.0
+        g_repeated, num_reps = repeat_to_match_shape(g / ans, shape, dtype, axis, keepdims)
+        x_minus_mean = x - anp.mean(x, axis=axis, keepdims=True)
+        return g_repeated * x_minus_mean / (num_reps - ddof)
+
+    return vjp
+
+
+defvjp(anp._primitive_std, _grad_std)
+
+
+def _grad_prod(ans, x, axis=None, keepdims=False, **kwargs):
+    shape, dtype = anp.shape(x), anp.result_type(x)
+
+    def vjp(g):
+        g_repeated, _ = repeat_to_match_shape(g * ans, shape, dtype, axis, keepdims)
+        return g_repeated / x
+
+    return vjp
+
+
+defvjp(anp.prod, _grad_prod)
+
+
+def _grad_chooser(ans, x, axis=None, keepdims=None, **kwargs):
+    """max/min: the cotangent is shared equally by the positions that attain the extremum
+    (numpy_vjps.py:515-530)."""
+    shape, dtype = anp.shape(x), anp.result_type(x)
+
+    def vjp(g):
+        g_repeated, _ = repeat_to_match_shape(g, shape, dtype, axis, keepdims)
+        ans_repeated, _ = repeat_to_match_shape(ans, shape, dtype, axis, keepdims)
+        hits = anp.astype(x == ans_repeated, dtype)
+        return g_repeated * hits / anp.sum(hits, axis=axis, keepdims=True)
+
+    return vjp
+
+
+defvjp(anp.max, _grad_chooser)
+defvjp(anp.min, _grad_chooser)
+
+
+def _grad_repeat(ans, x, repeats, axis=None):
+    shape = anp.shape(x)
+
+    def vjp(g):
+        if axis is None:
+            expanded = anp.reshape(g, (int(onp.prod(shape)),) + (repeats,))
+            return anp.reshape(anp.sum(expanded, axis=1, keepdims=False), shape)
+        ax = axis % len(shape)
+        if shape[ax] == 1:
+            return anp.sum(g, axis=ax, keepdims=True)
+        expanded = anp.reshape(g, shape[0 : ax + 1] + (repeats,) + shape[ax + 1 :])
+        return anp.sum(expanded, axis=ax + 1, keepdims=False)
+
+    return vjp
+
+
+defvjp(anp.repeat, _grad_repeat)
+
+
+# ---- dense contractions (numpy_vjps.py:552-747) ----------------------------------------------
+def _as_dtype(x, dtype):
+    return x if x.dtype == dtype else D.astype(x, dtype)
+
+
+@primitive
+def dot_adjoint_0(B, G, A_meta, B_meta):
+    """Cotangent of ``dot(A, B)`` with respect to ``A`` (numpy_vjps.py:615-624): for matrices
+    ``G . B^T``, read through swapped strides - B is never transposed in memory."""
+    _, A_ndim, A_dtype, _ = A_meta
+    _, B_ndim, _, _ = B_meta
+    if A_ndim == 2 and B_ndim == 2:
+        B, G = D.asarray(B), D.asarray(G)
+        dt = D._float_dtype(D.result_dtype(B, G))
+        out = DevArray(D.gemm2d(_as_dtype(G, dt)._t, _as_dtype(B, dt)._t.t(), dt), dt)
+        return _as_dtype(out, onp.dtype(A_dtype))
+    if B_ndim == 0 or B_ndim == 1 or A_ndim == 0:
+        contract_num = max(0, B_ndim - (A_ndim != 0))
+        out = anp.tensordot.fun(G, B, contract_num)
+    else:
+        out = anp.tensordot.fun(G, anp.swapaxes.fun(D.asarray(B), -1, -2), B_ndim - 1)
+    return _as_dtype(out, onp.dtype(A_dtype))
+
+
+@primitive
+def dot_adjoint_1(A, G, A_meta, B_meta):
+    """Cotangent of ``dot(A, B)`` with respect to ``B`` (numpy_vjps.py:627-638): for matrices
+    ``A^T . G`` computed directly (the reference forms ``(G^T A)^T`` and returns a transposed
+    view; the values are the same, the result here is contiguous)."""
+    _, A_ndim, _, _ = A_meta
+    _, B_ndim, B_dtype, _ = B_meta
+    A, G = D.asarray(A), D.asarray(G)
+    if A_ndim == 2 and B_ndim == 2:
+        dt = D._float_dtype(D.result_dtype(A, G))
+        out = DevArray(D.gemm2d(_as_dtype(A, dt)._t.t(), _as_dtype(G, dt)._t, dt), dt)
+        return _as_dtype(out, onp.dtype(B_dtype))
+    needs_transpose = B_ndim > 1 and A_ndim != 0
+    swap = (lambda x: anp.swapaxes.fun(x, -1, -2)) if needs_transpose else (lambda x: x)
+    if A_ndim == 0 or A_ndim == 1 or B_ndim == 0:
+        contract_num = max(0, A_ndim - (B_ndim != 0))
+        out = swap(anp.tensordot.fun(G, A, contract_num))
+    else:
+        out = swap(
+            anp.tensordot.fun(G, A, [list(range(-A_ndim - B_ndim + 2, -B_ndim + 1)), list(range(A_ndim - 1))])
+        )
+    return _as_dtype(out, onp.dtype(B_dtype))
+
+
+def _dot_vjp_0(ans, A, B):
+    A_meta, B_meta = anp.metadata(A), anp.metadata(B)
+    return lambda g: dot_adjoint_0(B, g, A_meta, B_meta)
+
+
+def _dot_vjp_1(ans, A, B):
+    A_meta, B_meta = anp.metadata(A), anp.metadata(B)
+    return lambda g: dot_adjoint_1(A, g, A_meta, B_meta)
+
+
+defvjp(anp.dot, _dot_vjp_0, _dot_vjp_1)
+defvjp(
+    dot_adjoint_0,
+    lambda ans, B, g, An, Bn: lambda A: dot_adjoint_1(A, g, An, Bn),
+    lambda ans, B, g, An, Bn: lambda A: anp.dot(A, B),
+)
+defvjp(
+    dot_adjoint_1,
+    lambda ans, A, g, An, Bn: lambda B: dot_adjoint_0(B, g, An, Bn),
+    lambda ans, A, g, An, Bn: lambda B: anp.dot(A, B),
+)
+
+
+def _matmul_adjoint_0(B, G, A_meta, B_ndim):
+    if anp.ndim(G) == 0:
+        return unbroadcast(G * B, A_meta)
+    _, A_ndim, _, _ = A_meta
+    if A_ndim == 1:
+        G = anp.expand_dims(G, anp.ndim(G) - 1)
+    if B_ndim == 1:
+        B = anp.expand_dims(B, 0)
+        G = anp.expand_dims(G, anp.ndim(G))
+    else:
+        B = anp.swapaxes(B, B_ndim - 2, B_ndim - 1)
+    return unbroadcast(anp.matmul(G, B), A_meta)
+
+
+def _matmul_adjoint_1(A, G, A_ndim, B_meta):
+    if anp.ndim(G) == 0:
+        return unbroadcast(G * A, B_meta)
+    _, B_ndim, _, _ = B_meta
+    B_is_vec = B_ndim == 1
+    if B_is_vec:
+        G = anp.expand_dims(G, anp.ndim(G))
+    if A_ndim == 1:
+        A = anp.expand_dims(A, 1)
+        G = anp.expand_dims(G, anp.ndim(G) - 1)
+    else:
+        A = anp.swapaxes(A, A_ndim - 2, A_ndim - 1)
+    result = anp.matmul(A, G)
+    if B_is_vec:
+        result = anp.squeeze(result, anp.ndim(G) - 1)
+    return unbroadcast(result, B_meta)
+
+
+def _matmul_vjp_0(ans, A, B):
+    A_meta, B_ndim = anp.metadata(A), anp.ndim(B)
+    return lambda g: _matmul_adjoint_0(B, g, A_meta, B_ndim)
+
+
+def _matmul_vjp_1(ans, A, B):
+    A_ndim, B_meta = anp.ndim(A), anp.metadata(B)
+    return lambda g: _matmul_adjoint_1(A, g, A_ndim, B_meta)
+
+
+defvjp(anp.matmul, _matmul_vjp_0, _matmul_vjp_1)
+
+
+def _split_axes(axes, A_ndim, B_ndim):
+    axes0 = [axes[0]] if type(axes[0]) is int else list(axes[0])
+    axes1 = [axes[1]] if type(axes[1]) is int else list(axes[1])
+    summed = [onp.asarray(axes0, dtype="int64") % A_ndim, onp.asarray(axes1, dtype="int64") % B_ndim]
+    other = [onp.delete(onp.arange(A_ndim), summed[0]), onp.delete(onp.arange(B_ndim), summed[1])]
+    return summed, other
+
+
+def _ints(a):
+    return [int(i) for i in a]
+
+
+@primitive
+def tensordot_adjoint_0(B, G, axes, A_ndim, B_ndim):
+    """Adjoint of ``A -> tensordot(A, B, axes)`` (numpy_vjps.py:666-691): one MFMA contraction
+    of permuted views plus a final axis permutation (a view)."""
+    if B_ndim == 0:
+        return D.arith_map(Op.MUL, G, B)
+    G_axes = list(range(anp.ndim(G)))
+    if type(axes) is int:
+        axes = max(axes, 0)
+        return anp.tensordot.fun(G, B, [G_axes[A_ndim - axes :], list(range(B_ndim))[axes:]])
+    summed, other = _split_axes(axes, A_ndim, B_ndim)
+    out = anp.tensordot.fun(G, B, [G_axes[len(other[0]) :], _ints(other[1])])
+    perm = onp.argsort(onp.concatenate((other[0], summed[0][onp.argsort(summed[1])])))
+    return anp.transpose.fun(out, _ints(perm))
+
+
+@primitive
+def tensordot_adjoint_1(A, G, axes, A_ndim, B_ndim):
+    """Adjoint of ``B -> tensordot(A, B, axes)`` (numpy_vjps.py:694-719)."""
+    if A_ndim == 0:
+        return D.arith_map(Op.MUL, G, A)
+    G_axes = list(range(anp.ndim(G)))
+    if type(axes) is int:
+        axes = max(axes, 0)
+        A_axes = list(range(A_ndim))
+        return anp.tensordot.fun(A, G, [A_axes[: A_ndim - axes], G_axes[: A_ndim - axes]])
+    summed, other = _split_axes(axes, A_ndim, B_ndim)
+    out = anp.tensordot.fun(A, G, [_ints(other[0]), G_axes[: len(other[0])]])
+    perm = onp.argsort(onp.concatenate((summed[1][onp.argsort(summed[0])], other[1])))
+    return anp.transpose.fun(out, _ints(perm))
+
+
+def _tensordot_vjp_0(ans, A, B, axes=2):
+    A_ndim, B_ndim = anp.ndim(A), anp.ndim(B)
+    return lambda G: tensordot_adjoint_0(B, G, axes, A_ndim, B_ndim)
+
+
+def _tensordot_vjp_1(ans, A, B, axes=2):
+    A_ndim, B_ndim = anp.ndim(A), anp.ndim(B)
+    return lambda G: tensordot_adjoint_1(A, G, axes, A_ndim, B_ndim)
+
+
+defvjp(anp.tensordot, _tensordot_vjp_0, _tensordot_vjp_1)
+defvjp(
+    tensordot_adjoint_0,
+    lambda ans, B, G, axes, An, Bn: lambda A: tensordot_adjoint_1(A, G, axes, An, Bn),
+    lambda ans, B, G, axes, An, Bn: lambda A: anp.tensordot(A, B, axes),
+)
+defvjp(
+    tensordot_adjoint_1,
+    lambda ans, A, G, axes, An, Bn: lambda B: tensordot_adjoint_0(B, G, axes, An, Bn),
+    lambda ans, A, G, axes, An, Bn: lambda B: anp.tensordot(A, B, axes),
+)
+defvjp(
+    anp.outer,
+    lambda ans, a, b: lambda g: anp.dot(g, anp.ravel(b)),
+    lambda ans, a, b: lambda g: anp.dot(anp.ravel(a), g),
+)
+
+
+# ---- concatenate / array construction (numpy_vjps.py:750-759, 922-938) -----------------------
+def _grad_concatenate_args(argnum, ans, axis_args, kwargs):
+    axis, args = axis_args[0], axis_args[1:]
+    sizes = [anp.shape(a)[axis] for a in args[:argnum]]
+    start = sum(sizes[:-1])
+    idxs = [slice(None)] * anp.ndim(ans)
+    idxs[axis] = slice(start, start + sizes[-1])
+    return lambda g: g[tuple(idxs)]
+
+
+defvjp_argnum(anp.concatenate_args, _grad_concatenate_args)
+defvjp_argnum(anp.array_from_args, lambda argnum, ans, args, kwargs: lambda g: g[argnum - 2])
+
+
+def _grad_array_from_scalar_or_array(ans, array_args, array_kwargs, scarray):
+    ndmin = array_kwargs.get("ndmin", 0)
+    scarray_ndim = anp.ndim(scarray)
+    if ndmin > scarray_ndim:
+        return lambda g: anp.squeeze(g, axis=tuple(range(ndmin - scarray_ndim)))
+    return lambda g: g
+
+
+defvjp(anp._array_from_scalar_or_array, _grad_array_from_scalar_or_array, argnums=(2, 3))
+
+
+# ---- indexing (numpy_vjps.py:941-954) --------------------------------------------------------
+@primitive
+def untake(x, idx, vs):
+    """Cotangent of ``A[idx]``: a sparse object whose ``mut_add`` scatters ``x`` into a dense
+    buffer - a strided in-place add for slices, the ordered scatter-add kernel (numpy.add.at
+    order, bit for bit) for integer-array indices."""
+
+    def mut_add(A):
+        return anp.scatter_add(A, idx, x)
+
+    return SparseObject(vs, mut_add)
+
+
+defvjp(func(DevArrayBox.__getitem__), lambda ans, A, idx: lambda g: untake(g, idx, vspace(A)))
+defvjp(untake, lambda ans, x, idx, _: lambda g: g[idx])

@@ -1,0 +1,73 @@
+"""``DevArrayVSpace``: the vector space of device arrays.
+
+Counterpart of the reference's ArrayVSpace (autograd/numpy/numpy_vspaces.py:7-37).  The
+accumulation hooks used by ``add_outgrads`` (autograd/core.py:185-205) launch kernels:
+``_add`` allocates a fresh buffer, ``_mut_add`` updates the (always freshly allocated,
+never aliased) accumulator in place.
+"""
+
+import numpy as onp
+
+from .. import _lib
+from .._lib import Op, Red
+from ..extend import VSpace
+from . import devarray as D
+from .devarray import DevArray
+
+
+class DevArrayVSpace(VSpace):
+    def __init__(self, value):
+        if isinstance(value, DevArray):
+            self.shape = value.shape
+            self.dtype = value.dtype
+        else:
+            value = onp.asarray(value)
+            self.shape = value.shape
+            self.dtype = value.dtype
+
+    @property
+    def size(self):
+        return int(onp.prod(self.shape))
+
+    @property
+    def ndim(self):
+        return len(self.shape)
+
+    def zeros(self):
+        return D.zeros(self.shape, self.dtype)
+
+    def ones(self):
+        return D.ones(self.shape, self.dtype)
+
+    def standard_basis(self):
+        for idxs in onp.ndindex(*self.shape):
+            vect = D.zeros(self.shape, self.dtype)
+            cell = vect._t[idxs] if idxs else vect._t
+            _lib.fill(_lib.DTYPE_CODE[self.dtype], cell, 1.0)  # a single element is always contiguous
+            yield vect
+
+    def randn(self):
+        # host RNG (numpy.random, as the reference) so seeded tests see the same draws
+        return D.from_numpy(onp.array(onp.random.randn(*self.shape)).astype(self.dtype))
+
+    def _add(self, x, y):
+        return D.map_op(Op.ADD, D._float_dtype(D.result_dtype(x, y)), x, y)
+
+    def _mut_add(self, x, y):
+        if not isinstance(x, DevArray):
+            return self._add(x, y)
+        if isinstance(y, DevArray) and y.shape != x.shape and onp.broadcast_shapes(x.shape, y.shape) != x.shape:
+            return self._add(x, y)
+        return D.map_op(Op.ADD, x.dtype, x, y, out=x)
+
+    def _scalar_mul(self, x, a):
+        return D.arith_map(Op.MUL, x, a)
+
+    def _inner_prod(self, x, y):
+        x, y = D.asarray(x), D.asarray(y)
+        dt = D._float_dtype(D.result_dtype(x, y))
+        return D.map_reduce(Op.MUL, Red.SUM, dt, (x, y), tuple(range(max(x.ndim, y.ndim))), False)
+
+
+DevArrayVSpace.register(DevArray)
+DevArrayVSpace.register(float)

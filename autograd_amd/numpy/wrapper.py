@@ -1,0 +1,782 @@
+"""The device array namespace: NumPy-named functions on ``DevArray`` wrapped as primitives.
+
+Counterpart of the reference's autograd/numpy/numpy_wrapper.py:25-236 for the part of NumPy the
+hot path uses.  Each differentiable function is a ``primitive`` whose raw implementation
+launches HIP kernels; shape queries are never traced; list-taking functions are routed through
+``concatenate_args`` / ``array_from_args`` so boxes inside Python lists are seen.
+"""
+
+import numbers
+
+import numpy as onp
+import torch
+
+from .. import _lib
+from ..extend import notrace_primitive, primitive
+from . import devarray as D
+from .._lib import Cmp, Op, Red
+from .devarray import DevArray
+
+# constants and dtypes
+pi, e, inf, nan, newaxis = onp.pi, onp.e, onp.inf, onp.nan, None
+euler_gamma = onp.euler_gamma
+float32, float64, int32, int64, bool_ = onp.float32, onp.float64, onp.int32, onp.int64, onp.bool_
+ndarray = DevArray
+
+
+def _wrap(raw, name):
+    raw.__name__ = name
+    raw.__qualname__ = name
+    return primitive(raw)
+
+
+# ---- elementwise ----------------------------------------------------------------------------
+def _unary(op, name):
+    def raw(x):
+        return D.float_map(op, x)
+
+    return _wrap(raw, name)
+
+
+negative = _wrap(lambda x: D.arith_map(Op.NEG, x), "negative")
+exp = _unary(Op.EXP, "exp")
+log = _unary(Op.LOG, "log")
+tanh = _unary(Op.TANH, "tanh")
+sinh = _unary(Op.SINH, "sinh")
+cosh = _unary(Op.COSH, "cosh")
+sin = _unary(Op.SIN, "sin")
+cos = _unary(Op.COS, "cos")
+sqrt = _unary(Op.SQRT, "sqrt")
+log1p = _unary(Op.LOG1P, "log1p")
+expm1 = _unary(Op.EXPM1, "expm1")
+reciprocal = _unary(Op.RECIPROCAL, "reciprocal")
+square = _wrap(lambda x: D.arith_map(Op.SQUARE, x), "square")
+abs = absolute = _wrap(lambda x: D.arith_map(Op.ABS, x), "abs")  # noqa: A001
+sign = _wrap(lambda x: D.arith_map(Op.SIGN, x), "sign")
+
+
+def _binary(op, name, floating=False):
+    fn = D.float_map if floating else D.arith_map
+
+    def raw(x, y):
+        return fn(op, x, y)
+
+    return _wrap(raw, name)
+
+
+add = _binary(Op.ADD, "add")
+subtract = _binary(Op.SUB, "subtract")
+multiply = _binary(Op.MUL, "multiply")
+divide = true_divide = _binary(Op.DIV, "true_divide", floating=True)
+power = _binary(Op.POW, "power")
+maximum = _binary(Op.MAXIMUM, "maximum")
+minimum = _binary(Op.MINIMUM, "minimum")
+
+
+def _compare(cmp, name):
+    def raw(x, y):
+        return D.compare(cmp, x, y)
+
+    return _wrap(raw, name)
+
+
+equal = _compare(Cmp.EQ, "equal")
+not_equal = _compare(Cmp.NE, "not_equal")
+less = _compare(Cmp.LT, "less")
+less_equal = _compare(Cmp.LE, "less_equal")
+greater = _compare(Cmp.GT, "greater")
+greater_equal = _compare(Cmp.GE, "greater_equal")
+
+
+@primitive
+def _where3(c, x, y):
+    dt = D._float_dtype(D.result_dtype(x, y))
+    if isinstance(c, DevArray):
+        c = D.astype(c, dt) if c.dtype != dt else c
+    else:
+        c = 1.0 if c else 0.0
+    return D.map_op(Op.WHERE, dt, c, x, y)
+
+
+def where(condition, x, y):
+    """``numpy.where(c, x, y)``.  Keeps native Python types when no operand is an array or a
+    box, as the reference does (autograd/numpy/__init__.py:13-39): the ``power`` rule calls
+    ``where(y, y - 1, 1.0)`` with a Python exponent and needs a Python float back."""
+    from ..tracer import isbox
+
+    def arrayish(v):
+        return isinstance(v, (DevArray, onp.ndarray, onp.generic)) or isbox(v)
+
+    if not (arrayish(condition) or arrayish(x) or arrayish(y)):
+        return x if condition else y
+    return _where3(condition, x, y)
+
+
+def logical_and(a, b):
+    return _wrap_bool(D.map_op(Op.MUL, onp.dtype("float64"), _truth(a), _truth(b)))
+
+
+def logical_not(a):
+    return D.compare(Cmp.EQ, _truth(a), 0.0)
+
+
+def _truth(a):
+    from ..tracer import getval
+
+    a = getval(a)
+    return D.astype(D.compare(Cmp.NE, a, 0.0), onp.float64) if isinstance(a, DevArray) else (1.0 if a else 0.0)
+
+
+def _wrap_bool(x):
+    return D.compare(Cmp.NE, x, 0.0)
+
+
+# ---- astype / copies --------------------------------------------------------------------------
+@primitive
+def astype(A, dtype, order="K", casting="unsafe", subok=True, copy=True):
+    return D.astype(A, dtype)
+
+
+_astype = astype
+
+
+# ---- reductions ---------------------------------------------------------------------------------
+def _reduction(red, name):
+    def raw(x, axis=None, keepdims=False, dtype=None, out=None, **kwargs):
+        x = D.asarray(x)
+        dt = D._float_dtype(x.dtype) if dtype is None else onp.dtype(dtype)
+        return D.map_reduce(Op.COPY, red, dt, (x,), D.normalize_axes(axis, x.ndim), keepdims)
+
+    return _wrap(raw, name)
+
+
+sum = _reduction(Red.SUM, "sum")  # noqa: A001
+prod = _reduction(Red.PROD, "prod")
+max = amax = _reduction(Red.MAX, "max")  # noqa: A001
+min = amin = _reduction(Red.MIN, "min")  # noqa: A001
+
+
+@primitive
+def _primitive_mean(x, axis=None, keepdims=False, dtype=None, out=None, **kwargs):
+    x = D.asarray(x)
+    axes = D.normalize_axes(axis, x.ndim)
+    dt = D._float_dtype(x.dtype)
+    total = D.map_reduce(Op.COPY, Red.SUM, dt, (x,), axes, keepdims)
+    count = 1
+    for a in axes:
+        count *= x.shape[a]
+    return D.map_op(Op.DIV, dt, total, float(count))
+
+
+_primitive_mean.__name__ = "mean"
+
+
+def mean(a, *args, **kwargs):
+    if type(a) in (list, tuple):
+        a = array(a)
+    return _primitive_mean(a, *args, **kwargs)
+
+
+# ---- shape-only functions (views: no kernel unless a copy is unavoidable) -----------------------
+def _view_or_copy(x, shape):
+    try:
+        return DevArray(x._t.view(shape), x.dtype)
+    except RuntimeError:
+        return DevArray(D.contiguous(x)._t.view(shape), x.dtype)
+
+
+def _norm_shape(shape, size):
+    if isinstance(shape, (numbers.Integral, onp.integer)):
+        shape = (int(shape),)
+    shape = [int(s) for s in shape]
+    if shape.count(-1) > 1:
+        raise ValueError("can only specify one unknown dimension")
+    if -1 in shape:
+        known = 1
+        for s in shape:
+            if s != -1:
+                known *= s
+        if known == 0 or size % known:
+            raise ValueError(f"cannot reshape array of size {size} into shape {tuple(shape)}")
+        shape[shape.index(-1)] = size // known
+    total = 1
+    for s in shape:
+        total *= s
+    if total != size:
+        raise ValueError(f"cannot reshape array of size {size} into shape {tuple(shape)}")
+    return tuple(shape)
+
+
+def _check_order(order):
+    if order not in (None, "C"):
+        raise NotImplementedError("only C order is supported on the device")
+
+
+@primitive
+def reshape(x, shape, order=None):
+    _check_order(order)
+    x = D.asarray(x)
+    return _view_or_copy(x, _norm_shape(shape, x.size))
+
+
+@primitive
+def ravel(x, order=None):
+    _check_order(order)
+    x = D.asarray(x)
+    return _view_or_copy(x, (x.size,))
+
+
+@primitive
+def expand_dims(x, axis):
+    x = D.asarray(x)
+    axes = (axis,) if isinstance(axis, (numbers.Integral, onp.integer)) else tuple(axis)
+    nd = x.ndim + len(axes)
+    axes = sorted(a % nd for a in axes)
+    t = x._t
+    for a in axes:
+        t = t.unsqueeze(a)
+    return DevArray(t, x.dtype)
+
+
+@primitive
+def squeeze(x, axis=None):
+    x = D.asarray(x)
+    if axis is None:
+        return DevArray(x._t.squeeze(), x.dtype)
+    axes = (axis,) if isinstance(axis, (numbers.Integral, onp.integer)) else tuple(axis)
+    axes = sorted((a % x.ndim for a in axes), reverse=True)
+    t = x._t
+    for a in axes:
+        if t.shape[a] != 1:
+            raise ValueError("cannot select an axis to squeeze out which has size not equal to one")
+        t = t.squeeze(a)
+    return DevArray(t, x.dtype)
+
+
+@primitive
+def transpose(x, axes=None):
+    x = D.asarray(x)
+    if axes is None:
+        axes = tuple(range(x.ndim))[::-1]
+    axes = tuple(int(a) % x.ndim for a in axes) if x.ndim else ()
+    return DevArray(x._t.permute(axes) if x.ndim else x._t, x.dtype)
+
+
+@primitive
+def swapaxes(x, axis1, axis2):
+    x = D.asarray(x)
+    return DevArray(x._t.transpose(axis1, axis2), x.dtype)
+
+
+@primitive
+def moveaxis(x, source, destination):
+    x = D.asarray(x)
+    return DevArray(torch.movedim(x._t, source, destination), x.dtype)
+
+
+@primitive
+def broadcast_to(x, shape):
+    x = D.asarray(x)
+    shape = (shape,) if isinstance(shape, numbers.Integral) else tuple(shape)
+    return DevArray(x._t.expand(shape), x.dtype)
+
+
+def _atleast(n):
+    def raw(*arys):
+        res = []
+        for a in arys:
+            a = D.asarray(a)
+            t = a._t
+            if n >= 1 and t.dim() == 0:
+                t = t.reshape(1)
+            if n >= 2 and t.dim() == 1:
+                t = t.unsqueeze(0)
+            if n >= 3 and t.dim() == 2:
+                t = t.unsqueeze(2)
+            res.append(DevArray(t, a.dtype))
+        return res[0] if len(res) == 1 else res
+
+    return _wrap(raw, f"atleast_{n}d")
+
+
+atleast_1d, atleast_2d, atleast_3d = _atleast(1), _atleast(2), _atleast(3)
+
+
+@primitive
+def repeat(x, repeats, axis=None):
+    x = D.asarray(x)
+    if not isinstance(repeats, (numbers.Integral, onp.integer)):
+        raise NotImplementedError("repeat: only an integer repeat count is supported on the device")
+    repeats = int(repeats)
+    if axis is None:
+        x = ravel.fun(x)
+        axis = 0
+    axis %= x.ndim
+    # out viewed as (..., n, repeats, ...) = x broadcast along a new axis
+    src = x._t.unsqueeze(axis + 1)
+    wide = src.shape[: axis + 1] + (repeats,) + src.shape[axis + 2 :]
+    out = D.map_op(Op.COPY, x.dtype, DevArray(src.expand(wide), x.dtype)) if x.dtype in D._FLOATS else D.astype_copy(
+        DevArray(src.expand(wide), x.dtype))
+    final = x.shape[:axis] + (x.shape[axis] * repeats,) + x.shape[axis + 1 :]
+    return DevArray(out._t.view(final), x.dtype)
+
+
+@primitive
+def concatenate_args(axis, *args):
+    arrs = [D.asarray(a) for a in args]
+    dt = D.result_dtype(*arrs)
+    if axis is None:
+        arrs = [ravel.fun(a) for a in arrs]
+        axis = 0
+    nd = arrs[0].ndim
+    if nd == 0:
+        raise ValueError("zero-dimensional arrays cannot be concatenated")
+    axis %= nd
+    total = 0
+    for a in arrs:
+        if a.ndim != nd or a.shape[:axis] != arrs[0].shape[:axis] or a.shape[axis + 1 :] != arrs[0].shape[axis + 1 :]:
+            raise ValueError("all the input array dimensions except for the concatenation axis must match exactly")
+        total += a.shape[axis]
+    shape = arrs[0].shape[:axis] + (total,) + arrs[0].shape[axis + 1 :]
+    out = D.empty(shape, dt)
+    start = 0
+    for a in arrs:
+        n = a.shape[axis]
+        if n:
+            dst = DevArray(out._t.narrow(axis, start, n), dt)
+            if dt in D._FLOATS:
+                D.map_op(Op.COPY, dt, a, out=dst)
+            else:
+                _lib.cast(_lib.DTYPE_CODE[a.dtype], _lib.DTYPE_CODE[dt], dst.shape, dst._t, a._t)
+        start += n
+    return out
+
+
+def concatenate(arr_list, axis=0):
+    return concatenate_args(axis, *arr_list)
+
+
+def vstack(tup):
+    return concatenate([atleast_2d(m) for m in tup], axis=0)
+
+
+row_stack = vstack
+
+
+def hstack(tup):
+    arrs = [atleast_1d(m) for m in tup]
+    if arrs[0].ndim == 1:
+        return concatenate(arrs, 0)
+    return concatenate(arrs, 1)
+
+
+@primitive
+def _array_from_scalar_or_array(array_args, array_kwargs, scalar):
+    dtype = array_kwargs.get("dtype", array_args[0] if array_args else None)
+    out = D.asarray(scalar, dtype)
+    ndmin = array_kwargs.get("ndmin", 0)
+    while out.ndim < ndmin:
+        out = DevArray(out._t.unsqueeze(0), out.dtype)
+    return out
+
+
+@primitive
+def array_from_args(array_args, array_kwargs, *args):
+    dtype = array_kwargs.get("dtype", array_args[0] if array_args else None)
+    parts = [D.asarray(a) for a in args]
+    dt = onp.dtype(dtype) if dtype is not None else D.result_dtype(*parts)
+    return concatenate_args.fun(0, *[DevArray(p._t.unsqueeze(0), p.dtype) for p in parts]) if parts else D.empty((0,), dt)
+
+
+def array(A, *args, **kwargs):
+    """``numpy.array``: host data is uploaded; lists that contain boxes stay differentiable."""
+    from ..tracer import isbox
+
+    if type(A) in (list, tuple):
+        flat_has_dev = _contains_dev_or_box(A)
+        if flat_has_dev:
+            return array_from_args(args, kwargs, *map(array, A))
+        return D.asarray(onp.array(A, *args, **kwargs))
+    if isbox(A) or isinstance(A, DevArray):
+        return _array_from_scalar_or_array(args, kwargs, A)
+    return D.asarray(onp.array(A, *args, **kwargs))
+
+
+def _contains_dev_or_box(seq):
+    from ..tracer import isbox
+
+    for item in seq:
+        if isinstance(item, DevArray) or isbox(item):
+            return True
+        if isinstance(item, (list, tuple)) and _contains_dev_or_box(item):
+            return True
+    return False
+
+
+def asarray(a, dtype=None):
+    from ..tracer import isbox
+
+    if isbox(a):
+        return a if dtype is None else astype(a, dtype)
+    return D.asarray(a, dtype)
+
+
+def stack(arrays, axis=0):
+    arrays = [array(a) for a in arrays]
+    if not arrays:
+        raise ValueError("need at least one array to stack")
+    if len({a.shape for a in arrays}) != 1:
+        raise ValueError("all input arrays must have the same shape")
+    nd = arrays[0].ndim + 1
+    if not -nd <= axis < nd:
+        raise IndexError(f"axis {axis} out of bounds [-{nd}, {nd})")
+    axis %= nd
+    sl = (slice(None),) * axis + (None,)
+    return concatenate([a[sl] for a in arrays], axis=axis)
+
+
+# ---- indexing -----------------------------------------------------------------------------------
+def _is_basic_index(idx):
+    items = idx if isinstance(idx, tuple) else (idx,)
+    for it in items:
+        if it is None or it is Ellipsis or isinstance(it, (numbers.Integral, onp.integer)):
+            continue
+        if isinstance(it, slice):
+            if it.step is not None and it.step <= 0:
+                raise NotImplementedError("slices with a non-positive step are not supported on the device")
+            continue
+        return False
+    return True
+
+
+def _plain(idx):
+    items = idx if isinstance(idx, tuple) else (idx,)
+    return tuple(int(i) if isinstance(i, (numbers.Integral, onp.integer)) else i for i in items)
+
+
+def _host_index(idx):
+    """1-d int64 host array for an integer-array index on the leading axis, else None."""
+    if isinstance(idx, list):
+        if len(idx) and isinstance(idx[0], slice):
+            return None
+        arr = onp.asarray(idx)
+    elif isinstance(idx, onp.ndarray):
+        arr = idx
+    elif isinstance(idx, DevArray):
+        arr = idx.numpy()
+    else:
+        return None
+    if arr.dtype == bool:
+        arr = onp.nonzero(arr)[0]
+    if arr.size == 0:
+        arr = arr.astype(onp.int64)
+    if arr.dtype.kind not in "iu" or arr.ndim != 1:
+        return None
+    return arr.astype(onp.int64)
+
+
+def take(A, idx):
+    """``A[idx]``: views for basic indices, a gather kernel for an integer array on axis 0."""
+    if _is_basic_index(idx):
+        return DevArray(A._t[_plain(idx)], A.dtype)
+    rows = _host_index(idx)
+    if rows is None:
+        raise NotImplementedError(
+            f"index {idx!r}: only basic indexing and a 1-d integer array on the leading axis are supported on the device"
+        )
+    if A.ndim == 0:
+        raise IndexError("too many indices for array")
+    n_rows = A.shape[0]
+    if rows.size and (rows.max() >= n_rows or rows.min() < -n_rows):
+        raise IndexError(f"index out of bounds for axis 0 with size {n_rows}")
+    src = D.contiguous(A)
+    inner = 1
+    for s in A.shape[1:]:
+        inner *= s
+    out = D.empty((rows.size,) + A.shape[1:], A.dtype)
+    if A.dtype not in D._FLOATS:
+        raise NotImplementedError("gather of non-floating arrays")
+    index = D.from_numpy(rows)
+    _lib.take_rows(_lib.DTYPE_CODE[A.dtype], src._t, n_rows, inner, index._t, rows.size, out._t)
+    return out
+
+
+def scatter_add(A, idx, x):
+    """In place ``numpy.add.at(A, idx, x)`` on a freshly allocated, contiguous ``A``.
+
+    Basic indices: a strided in-place add on the view (every destination gets exactly one
+    addend).  Integer array on axis 0: the ordered scatter kernel, which adds repeated
+    destinations sequentially in index order like ``numpy.add.at``.
+    """
+    if _is_basic_index(idx):
+        view = DevArray(A._t[_plain(idx)], A.dtype)
+        D.map_op(Op.ADD, A.dtype, view, x, out=view)
+        return A
+    rows = _host_index(idx)
+    if rows is None:
+        raise NotImplementedError(f"scatter with index {idx!r} is not supported on the device")
+    n_rows = A.shape[0]
+    if rows.size == 0:
+        return A
+    wrapped = onp.where(rows < 0, rows + n_rows, rows)
+    order = onp.argsort(wrapped, kind="stable").astype(onp.int64)
+    sorted_rows = wrapped[order]
+    boundaries = onp.flatnonzero(onp.diff(sorted_rows)) + 1
+    seg_start = onp.concatenate(([0], boundaries, [rows.size])).astype(onp.int64)
+    inner = 1
+    for s in A.shape[1:]:
+        inner *= s
+    target = (rows.size,) + A.shape[1:]
+    src = D.asarray(x, A.dtype)
+    if src.shape != target:
+        src = DevArray(src._t.expand(target), src.dtype)
+    src = D.contiguous(src)
+    if not A._t.is_contiguous():
+        raise AssertionError("scatter destination must be contiguous")
+    _lib.scatter_add_rows(_lib.DTYPE_CODE[A.dtype], A._t, n_rows, inner, src._t, D.from_numpy(rows)._t,
+                          D.from_numpy(order)._t, D.from_numpy(seg_start)._t, len(seg_start) - 1)
+    return A
+
+
+# ---- contractions -------------------------------------------------------------------------------
+def _dot_raw(a, b):
+    a, b = D.asarray(a) if not D.is_scalar(a) else a, D.asarray(b) if not D.is_scalar(b) else b
+    if D.is_scalar(a) or D.is_scalar(b) or a.ndim == 0 or b.ndim == 0:
+        return D.arith_map(Op.MUL, a, b)
+    dt = D._float_dtype(D.result_dtype(a, b))
+    a = D.astype(a, dt) if a.dtype != dt else a
+    b = D.astype(b, dt) if b.dtype != dt else b
+    if a.ndim == 1 and b.ndim == 1:
+        if a.shape != b.shape:
+            raise ValueError(f"shapes {a.shape} and {b.shape} not aligned")
+        return D.map_reduce(Op.MUL, Red.SUM, dt, (a, b), (0,), False)
+    if b.ndim == 1:  # (..., K) . (K,) -> (...): row map-reduce, bandwidth bound
+        if a.shape[-1] != b.shape[0]:
+            raise ValueError(f"shapes {a.shape} and {b.shape} not aligned")
+        return D.map_reduce(Op.MUL, Red.SUM, dt, (a, b), (a.ndim - 1,), False)
+    if a.ndim == 1:  # (K,) . (..., K, N) -> (..., N)
+        if a.shape[0] != b.shape[-2]:
+            raise ValueError(f"shapes {a.shape} and {b.shape} not aligned")
+        a_col = DevArray(a._t.reshape((1,) * (b.ndim - 2) + (a.shape[0], 1)), dt)
+        return D.map_reduce(Op.MUL, Red.SUM, dt, (a_col, b), (b.ndim - 2,), False)
+    if a.shape[-1] != b.shape[-2]:
+        raise ValueError(f"shapes {a.shape} and {b.shape} not aligned: {a.shape[-1]} (dim {a.ndim - 1}) != {b.shape[-2]} (dim {b.ndim - 2})")
+    if a.ndim == 2 and b.ndim == 2:
+        return DevArray(D.gemm2d(a._t, b._t, dt), dt)
+    # numpy.dot on higher ranks: sum over last axis of a and second-to-last of b
+    return _tensordot_raw(a, b, axes=((a.ndim - 1,), (b.ndim - 2,)))
+
+
+dot = _wrap(_dot_raw, "dot")
+
+
+def _matmul_raw(a, b):
+    a, b = D.asarray(a), D.asarray(b)
+    if a.ndim == 0 or b.ndim == 0:
+        raise ValueError("matmul: Input operand does not have enough dimensions")
+    if a.ndim <= 2 and b.ndim <= 2:
+        return _dot_raw(a, b)
+    dt = D._float_dtype(D.result_dtype(a, b))
+    a = D.astype(a, dt) if a.dtype != dt else a
+    b = D.astype(b, dt) if b.dtype != dt else b
+    ta, tb = a._t, b._t
+    a_vec, b_vec = ta.dim() == 1, tb.dim() == 1
+    if a_vec:
+        ta = ta.unsqueeze(0)
+    if b_vec:
+        tb = tb.unsqueeze(1)
+    batch = tuple(onp.broadcast_shapes(tuple(ta.shape[:-2]), tuple(tb.shape[:-2])))
+    ta = ta.expand(batch + tuple(ta.shape[-2:]))
+    tb = tb.expand(batch + tuple(tb.shape[-2:]))
+    M, K = ta.shape[-2:]
+    N = tb.shape[-1]
+
+    def flat(t, rows, cols):
+        # (batch..., rows, cols) -> (B, rows, cols) keeping stride-0 batch axes when one axis suffices
+        try:
+            return t.view((-1, rows, cols)) if len(batch) != 1 else t
+        except RuntimeError:
+            return D.contiguous(DevArray(t, dt))._t.view((-1, rows, cols))
+
+    fa, fb = flat(ta, M, K), flat(tb, K, N)
+    c = D.gemm_batched(fa, fb, dt).view(batch + (M, N))
+    if a_vec:
+        c = c.squeeze(-2)
+    if b_vec:
+        c = c.squeeze(-1)
+    return DevArray(c, dt)
+
+
+matmul = _wrap(_matmul_raw, "matmul")
+
+
+def _tensordot_raw(a, b, axes=2):
+    a, b = D.asarray(a), D.asarray(b)
+    dt = D._float_dtype(D.result_dtype(a, b))
+    a = D.astype(a, dt) if a.dtype != dt else a
+    b = D.astype(b, dt) if b.dtype != dt else b
+    if isinstance(axes, (numbers.Integral, onp.integer)):
+        n = int(axes)
+        if n < 0:
+            n = 0
+        axes_a, axes_b = list(range(a.ndim - n, a.ndim)), list(range(n))
+    else:
+        axes_a, axes_b = axes
+        axes_a = [axes_a] if isinstance(axes_a, (numbers.Integral, onp.integer)) else list(axes_a)
+        axes_b = [axes_b] if isinstance(axes_b, (numbers.Integral, onp.integer)) else list(axes_b)
+    axes_a = [int(x) % a.ndim for x in axes_a] if a.ndim else []
+    axes_b = [int(x) % b.ndim for x in axes_b] if b.ndim else []
+    if len(axes_a) != len(axes_b) or any(a.shape[i] != b.shape[j] for i, j in zip(axes_a, axes_b)):
+        raise ValueError("shape-mismatch for sum")
+    free_a = [d for d in range(a.ndim) if d not in axes_a]
+    free_b = [d for d in range(b.ndim) if d not in axes_b]
+    M = 1
+    for d in free_a:
+        M *= a.shape[d]
+    N = 1
+    for d in free_b:
+        N *= b.shape[d]
+    K = 1
+    for d in axes_a:
+        K *= a.shape[d]
+    at = a._t.permute(free_a + axes_a) if a.ndim else a._t
+    bt = b._t.permute(axes_b + free_b) if b.ndim else b._t
+    a2 = _view_or_copy(DevArray(at, dt), (M, K))._t
+    b2 = _view_or_copy(DevArray(bt, dt), (K, N))._t
+    out_shape = tuple(a.shape[d] for d in free_a) + tuple(b.shape[d] for d in free_b)
+    c = D.gemm2d(a2, b2, dt)
+    return DevArray(c.view(out_shape), dt)
+
+
+tensordot = _wrap(_tensordot_raw, "tensordot")
+
+
+@primitive
+def outer(a, b):
+    a, b = ravel.fun(D.asarray(a)), ravel.fun(D.asarray(b))
+    return D.arith_map(Op.MUL, DevArray(a._t.unsqueeze(1), a.dtype), DevArray(b._t.unsqueeze(0), b.dtype))
+
+
+# ---- non-differentiable helpers ---------------------------------------------------------------
+def _meta_of(A):
+    if isinstance(A, DevArray):
+        return A.shape, A.ndim, A.dtype, False
+    return onp.shape(A), onp.ndim(A), onp.result_type(A), onp.iscomplexobj(A)
+
+
+@notrace_primitive
+def metadata(A):
+    return _meta_of(A)
+
+
+@notrace_primitive
+def shape(A):
+    return _meta_of(A)[0]
+
+
+@notrace_primitive
+def ndim(A):
+    return _meta_of(A)[1]
+
+
+@notrace_primitive
+def result_type(*xs):
+    return D.result_dtype(*xs) if len(xs) > 1 else _meta_of(xs[0])[2]
+
+
+@notrace_primitive
+def size(A):
+    return A.size if isinstance(A, DevArray) else onp.size(A)
+
+
+@notrace_primitive
+def iscomplexobj(A):
+    return False if isinstance(A, DevArray) else onp.iscomplexobj(A)
+
+
+@notrace_primitive
+def isscalar(A):
+    return onp.isscalar(A)
+
+
+def zeros(shape, dtype=float):
+    return D.zeros(shape, dtype)
+
+
+def ones(shape, dtype=float):
+    return D.ones(shape, dtype)
+
+
+def full(shape, fill_value, dtype=None):
+    return D.full(shape, fill_value, dtype)
+
+
+def empty(shape, dtype=float):
+    return D.empty(shape, dtype)
+
+
+@notrace_primitive
+def zeros_like(a, dtype=None):
+    s, _, dt, _ = _meta_of(a)
+    return D.zeros(s, dtype or dt)
+
+
+@notrace_primitive
+def ones_like(a, dtype=None):
+    s, _, dt, _ = _meta_of(a)
+    return D.ones(s, dtype or dt)
+
+
+def linspace(start, stop, num=50, endpoint=True, dtype=None):
+    return D.from_numpy(onp.linspace(start, stop, num, endpoint=endpoint), dtype)
+
+
+def arange(*args, **kwargs):
+    return D.from_numpy(onp.arange(*args, **kwargs))
+
+
+def eye(N, M=None, k=0, dtype=float):
+    return D.from_numpy(onp.eye(N, M, k, dtype=dtype))
+
+
+to_numpy = D.to_numpy
+
+
+def synchronize():
+    _lib.synchronize()
+
+
+def allclose(a, b, rtol=1e-05, atol=1e-08):
+    from ..tracer import getval
+
+    return bool(onp.allclose(to_numpy(getval(a)), to_numpy(getval(b)), rtol=rtol, atol=atol))
+
+
+def _var_forward(x, axis=None, ddof=0, keepdims=False, **kwargs):
+    x = D.asarray(x)
+    axes = D.normalize_axes(axis, x.ndim)
+    dt = D._float_dtype(x.dtype)
+    n = 1
+    for d in axes:
+        n *= x.shape[d]
+    mu = _primitive_mean.fun(x, axis=axis, keepdims=True)
+    centered = D.map_op(Op.SUB, dt, x, mu)
+    total = D.map_reduce(Op.SQUARE, Red.SUM, dt, (centered,), axes, keepdims)
+    return D.map_op(Op.DIV, dt, total, float(n - ddof))
+
+
+_primitive_var = _wrap(_var_forward, "var")
+_primitive_std = _wrap(lambda x, axis=None, ddof=0, keepdims=False, **kw: D.float_map(
+    Op.SQRT, _var_forward(x, axis=axis, ddof=ddof, keepdims=keepdims)), "std")
+
+
+def var(a, *args, **kwargs):
+    if type(a) in (list, tuple):
+        a = array(a)
+    return _primitive_var(a, *args, **kwargs)
+
+
+def std(a, *args, **kwargs):
+    if type(a) in (list, tuple):
+        a = array(a)
+    return _primitive_std(a, *args, **kwargs)

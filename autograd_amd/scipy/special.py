@@ -1,0 +1,75 @@
+"""``logsumexp`` on device arrays, with its reverse- and forward-mode rules.
+
+Counterpart of the reference's autograd/scipy/special.py:119-147, whose forward is
+``scipy.special.logsumexp``.  Forward: one single-pass reduction kernel over (max, scaled sum)
+pairs.  Reverse, concrete operands: one fused kernel ``g * b * exp(x - ans)`` that reads ``g``
+and ``ans`` through broadcast strides, so neither is ever materialised at full size (the
+reference materialises both).  Forward mode: the same functor fused into a sum.
+"""
+
+import numbers
+
+import numpy as onp
+
+from .._lib import Op, Red
+from ..extend import defjvp, defvjp, primitive
+from ..numpy import devarray as D
+from ..numpy import wrapper as np
+from ..numpy.devarray import DevArray
+from ..numpy.vjps import _concrete, repeat_to_match_shape
+
+
+@primitive
+def logsumexp(x, axis=None, b=1.0, keepdims=False):
+    x = D.asarray(x)
+    if not (isinstance(b, numbers.Number) and b == 1.0):
+        # weighted form: log(sum(b * exp(x))) = logsumexp(x + log(b)) for positive weights
+        x = np.add.fun(x, np.log.fun(D.asarray(b) if not isinstance(b, numbers.Number) else b))
+    dt = D._float_dtype(x.dtype)
+    return D.map_reduce(Op.COPY, Red.LOGSUMEXP, dt, (x,), D.normalize_axes(axis, x.ndim), keepdims)
+
+
+def _keep(a, shape, axis, keepdims):
+    """Reduced-shape array ``a`` viewed with the reduced axes kept as size 1."""
+    if keepdims or len(shape) == 0:
+        return a
+    axes = D.normalize_axes(axis, len(shape))
+    new_shape = tuple(1 if d in axes else s for d, s in enumerate(shape))
+    return DevArray(a._t.reshape(new_shape), a.dtype)
+
+
+def _make_grad_logsumexp(ans, x, axis=None, b=1.0, keepdims=False):
+    shape, dtype = np.shape(x), np.result_type(x)
+
+    def vjp(g):
+        if _concrete(g, ans, x, b):
+            g_k = _keep(D.asarray(g), shape, axis, keepdims)
+            ans_k = _keep(ans, shape, axis, keepdims)
+            dt = D._float_dtype(D.result_dtype(g_k, x, ans_k))
+            return D.map_op(Op.LSE_VJP, dt, g_k, b, x, ans_k)
+        g_repeated, _ = repeat_to_match_shape(g, shape, dtype, axis, keepdims)
+        ans_repeated, _ = repeat_to_match_shape(ans, shape, dtype, axis, keepdims)
+        return g_repeated * b * np.exp(x - ans_repeated)
+
+    return vjp
+
+
+defvjp(logsumexp, _make_grad_logsumexp)
+
+
+def _fwd_grad_logsumexp(g, ans, x, axis=None, b=1.0, keepdims=False):
+    shape = np.shape(x)
+    if _concrete(g, ans, x, b):
+        ans_k = _keep(ans, shape, axis, keepdims)
+        dt = D._float_dtype(D.result_dtype(g, x, ans_k))
+        return D.map_reduce(Op.LSE_VJP, Red.SUM, dt, (g, b, x, ans_k), D.normalize_axes(axis, len(shape)), keepdims)
+    if not keepdims:
+        if isinstance(axis, int):
+            ans = np.expand_dims(ans, axis)
+        elif isinstance(axis, tuple):
+            for ax in sorted(axis):
+                ans = np.expand_dims(ans, ax)
+    return np.sum(g * b * np.exp(x - ans), axis=axis, keepdims=keepdims)
+
+
+defjvp(logsumexp, _fwd_grad_logsumexp)

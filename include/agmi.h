@@ -1,0 +1,191 @@
+/*
+ * agmi.h - C ABI of libagmi.so: the MI355X (gfx950) kernels under the VJP/JVP hot path.
+ *
+ * The reference (HIPS/autograd) is pure Python; the arithmetic of its hot path is the
+ * NumPy / SciPy / BLAS call inside each derivative rule.  Each entry point below replaces
+ * one family of those calls; the comment on each names the reference call sites it stands
+ * in for (paths relative to the reference tree).
+ *
+ * Conventions
+ *  - Every pointer named "device" is GPU memory owned by the caller.  The library never
+ *    allocates, frees or synchronises; work is enqueued on `stream` (a hipStream_t passed
+ *    as void*, NULL = the default stream) and the call returns immediately.
+ *  - Strides are in ELEMENTS, may be 0 (broadcast axis) and may be negative.
+ *  - Return value: 0 on success; AGMI_ERR_* (negative) for a rejected argument, in which
+ *    case nothing was launched; a positive value is a hipError_t from the launch.
+ *    agmi_last_error() returns a static, thread-local description of the last failure.
+ *  - Operands may alias only where a function says so.
+ */
+#ifndef AGMI_H
+#define AGMI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AGMI_MAX_DIMS 8      /* rank accepted at the ABI (before axis merging) */
+#define AGMI_MAX_INPUTS 4
+#define AGMI_MAX_OUTPUTS 2
+
+#define AGMI_ERR_ARG (-1)          /* null pointer, bad enum, rank > AGMI_MAX_DIMS, negative size */
+#define AGMI_ERR_UNSUPPORTED (-2)  /* layout the kernels do not cover (e.g. > 6 unmergeable axes) */
+#define AGMI_ERR_WORKSPACE (-3)    /* workspace smaller than agmi_*_workspace_bytes() asked for */
+
+typedef enum agmi_dtype {
+    AGMI_F32 = 0,
+    AGMI_F64 = 1,
+    AGMI_BOOL = 2, /* one byte per element, 0 or 1: comparison results, masks */
+    AGMI_I64 = 3,  /* index arrays */
+    AGMI_I32 = 4
+} agmi_dtype;
+
+/* One strided operand.  data == NULL in an INPUT slot means "scalar passed by value": the
+ * value is taken from scalars[slot] and converted to the array dtype (a weak Python scalar
+ * in NumPy's promotion rules). */
+typedef struct agmi_array {
+    void *data;                     /* device pointer to the element at index (0, ..., 0) */
+    int64_t strides[AGMI_MAX_DIMS]; /* elements */
+} agmi_array;
+
+/* Elementwise operations.  Unary/binary/ternary ufuncs are the forward primitives
+ * (autograd/numpy/numpy_wrapper.py:25-52 wraps numpy.add, numpy.exp, ...); the *_VJP entries
+ * are whole derivative rules of autograd/numpy/numpy_vjps.py fused into one pass, with the
+ * reference's operation order kept inside. */
+typedef enum agmi_op {
+    /* one input */
+    AGMI_OP_COPY = 0, /* out = x                    (materialise a view / broadcast)          */
+    AGMI_OP_NEG,      /* -x                         numpy_vjps.py:157, 87                     */
+    AGMI_OP_EXP,
+    AGMI_OP_LOG,
+    AGMI_OP_TANH,
+    AGMI_OP_SINH,
+    AGMI_OP_COSH,
+    AGMI_OP_SIN,
+    AGMI_OP_COS,
+    AGMI_OP_SQRT,
+    AGMI_OP_SQUARE,
+    AGMI_OP_ABS,
+    AGMI_OP_SIGN,
+    AGMI_OP_RECIPROCAL,
+    AGMI_OP_LOG1P,
+    AGMI_OP_EXPM1,
+    /* two inputs */
+    AGMI_OP_ADD = 32, /* also VSpace._add / _mut_add, autograd/core.py:259-264 (out may alias in0) */
+    AGMI_OP_SUB,
+    AGMI_OP_MUL,      /* y*g, x*g                   numpy_vjps.py:79-83, 163                  */
+    AGMI_OP_DIV,      /* g/y                        numpy_vjps.py:91, 126, 166                */
+    AGMI_OP_POW,
+    AGMI_OP_MAXIMUM,
+    AGMI_OP_MINIMUM,
+    /* three inputs */
+    AGMI_OP_WHERE = 64, /* c != 0 ? x : y  (c in the array dtype)                             */
+    /* fused derivative rules; inputs in the order listed */
+    AGMI_OP_DIV_VJP1 = 96, /* (g, x, y)      -g * x / y**2            numpy_vjps.py:92, 127       */
+    AGMI_OP_TANH_VJP,      /* (g, x)         g / cosh(x)**2           numpy_vjps.py:178           */
+    AGMI_OP_POW_VJP0,      /* (g, x, y)      g * y * x**where(y, y-1, 1)   numpy_vjps.py:141      */
+    AGMI_OP_POW_VJP1,      /* (g, x, ans)    g * log(where(x, x, 1)) * ans numpy_vjps.py:142      */
+    AGMI_OP_LSE_VJP,       /* (g, b, x, ans) g * b * exp(x - ans)     scipy/special.py:123-134    */
+    AGMI_OP_RECIPROCAL_VJP,/* (g, x)         -g / x**2                numpy_vjps.py:162           */
+    AGMI_OP_SQRT_VJP,      /* (g, x)         g * 0.5 * x**-0.5        numpy_vjps.py:187           */
+    AGMI_OP_SIN_VJP,       /* (g, x)         g * cos(x)               numpy_vjps.py:170           */
+    AGMI_OP_COS_VJP,       /* (g, x)         -g * sin(x)              numpy_vjps.py:171           */
+    AGMI_OP_SINH_VJP,      /* (g, x)         g * cosh(x)              numpy_vjps.py:176           */
+    AGMI_OP_COSH_VJP,      /* (g, x)         g * sinh(x)              numpy_vjps.py:177           */
+    AGMI_OP_SQUARE_VJP,    /* (g, x)         g * 2 * x                numpy_vjps.py:186           */
+    AGMI_OP_ABS_VJP,       /* (g, x, ans)    g * where(x,x,0) / where(ans,ans,1)  numpy_vjps.py:158 */
+    AGMI_OP_CHOOSE_VJP,    /* (g, x, ans, y) g * (x==ans) / (1 + (x==y))   numpy_vjps.py:94-113, 911 */
+    AGMI_OP_LOG1P_VJP,     /* (g, x)         g / (x + 1)              numpy_vjps.py:169           */
+    AGMI_OP_EXPM1_VJP,     /* (g, ans)       (ans + 1) * g            numpy_vjps.py:165           */
+    AGMI_OP_DIV_VJP_BOTH,  /* (g, x, y) -> two outputs: g / y and -g * x / y**2  (91-92)          */
+    AGMI_OP_MUL_ADD        /* (a, x, y)      a * x + y  (two roundings; scalar_mul + add)         */
+} agmi_op;
+
+/* comparison producing AGMI_BOOL: numpy.equal ... (non-differentiable, numpy_vjps.py:13-68) */
+typedef enum agmi_cmp { AGMI_EQ = 0, AGMI_NE, AGMI_LT, AGMI_LE, AGMI_GT, AGMI_GE } agmi_cmp;
+
+/* reduction kinds of agmi_map_reduce */
+typedef enum agmi_reduce_kind {
+    AGMI_RED_SUM = 0, /* numpy.sum: unbroadcast (numpy_vjps.py:883-892), repeat VJP (345-362)   */
+    AGMI_RED_MAX,
+    AGMI_RED_MIN,
+    AGMI_RED_PROD,
+    AGMI_RED_LOGSUMEXP /* scipy.special.logsumexp wrapped at autograd/scipy/special.py:120      */
+} agmi_reduce_kind;
+
+const char *agmi_last_error(void);
+int agmi_version(void);
+
+/* out[k][idx] = op(in[0][idx], in[1][idx], ...) over the index space `shape` (rank `ndim`).
+ * dtype is AGMI_F32 or AGMI_F64 for all operands.  An output may alias an input only when
+ * both have identical strides (in-place update: VSpace._mut_add, core.py:262-264).
+ * Replaces: one NumPy ufunc pass per arithmetic step of a rule in numpy_vjps.py:76-230. */
+int agmi_elementwise(int op, int dtype, int ndim, const int64_t *shape,
+                     int n_out, const agmi_array *outs,
+                     int n_in, const agmi_array *ins, const double *scalars,
+                     void *stream);
+
+/* out[idx] = (in0[idx] <cmp> in1[idx]) as AGMI_BOOL; inputs as in agmi_elementwise. */
+int agmi_compare(int cmp, int dtype, int ndim, const int64_t *shape,
+                 const agmi_array *out, const agmi_array *ins, const double *scalars,
+                 void *stream);
+
+/* out[idx] = (dst_dtype) in[idx] for any pair of dtypes (numpy astype, numpy_vjps.py:246-251;
+ * the dtype=A_dtype casts of dot_adjoint_*, 624, 638). */
+int agmi_cast(int src_dtype, int dst_dtype, int ndim, const int64_t *shape,
+              const agmi_array *out, const agmi_array *in, void *stream);
+
+/* out[kept idx] = REDUCE over the axes with reduce_axes[d] != 0 of op(in[0][idx], ...).
+ * `out->strides` are given for all `ndim` axes and are ignored on reduced axes.  `op` is any
+ * single-output agmi_op (AGMI_OP_COPY for a plain reduction).  Deterministic: the summation
+ * tree depends only on shapes, never on timing.  Large reductions run in two stages through
+ * `workspace` (device memory, at least agmi_map_reduce_workspace_bytes() bytes; may be NULL
+ * when that returns 0).
+ * Replaces: anp.sum inside unbroadcast (numpy_vjps.py:883-892) fused with the rule that feeds
+ * it (x*g then sum: 79-83), numpy.sum/max/min forward, scipy.special.logsumexp forward,
+ * the logsumexp JVP (scipy/special.py:137-147), ArrayVSpace._inner_prod (numpy_vspaces.py:36-37),
+ * and matrix-vector numpy.dot. */
+int agmi_map_reduce(int op, int red, int dtype, int ndim, const int64_t *shape,
+                    const uint8_t *reduce_axes, const agmi_array *out,
+                    int n_in, const agmi_array *ins, const double *scalars,
+                    void *workspace, size_t workspace_bytes, void *stream);
+size_t agmi_map_reduce_workspace_bytes(int red, int dtype, int ndim, const int64_t *shape,
+                                       const uint8_t *reduce_axes);
+
+/* C[m,n] = alpha * sum_k A[m,k] B[k,n] + beta * C[m,n] on the matrix cores (MFMA), dtype
+ * AGMI_F32 or AGMI_F64.  A and B are addressed as A[m*a_rs + k*a_cs], B[k*b_rs + n*b_cs], so
+ * the transposed operands of the adjoints need no copy; C is row-major with leading
+ * dimension ldc.  `batch` independent products with element strides *_bs (batch >= 1).
+ * Replaces: numpy.dot forward (numpy_wrapper.py:39-40), onp.tensordot in dot_adjoint_0/1
+ * (numpy_vjps.py:615-638: G.B^T and A^T.G), matmul adjoints (567-612), tensordot_adjoint_0/1
+ * (666-719) after axis permutation. */
+int agmi_gemm(int dtype, int64_t batch, int64_t M, int64_t N, int64_t K, double alpha,
+              const void *A, int64_t a_rs, int64_t a_cs, int64_t a_bs,
+              const void *B, int64_t b_rs, int64_t b_cs, int64_t b_bs,
+              double beta, void *C, int64_t ldc, int64_t c_bs, void *stream);
+
+/* ptr[0..n) = value (vspace zeros/ones, numpy_vspaces.py:21-25; sparse_add's zero fill,
+ * core.py:212-215). */
+int agmi_fill(int dtype, void *ptr, int64_t n, double value, void *stream);
+
+/* Gather rows: out[i, :] = src[index[i], :] for i in [0, n_index); rows have `inner` elements,
+ * src has `n_rows` rows.  Negative indices count from the end.  Forward of A[idx] with an
+ * integer-array idx on the leading axis (numpy_boxes.py:16-18). */
+int agmi_take_rows(int dtype, const void *src, int64_t n_rows, int64_t inner,
+                   const int64_t *index, int64_t n_index, void *out, void *stream);
+
+/* Ordered scatter-add: for i = 0 .. n_index-1 IN THIS ORDER: dst[index[i], :] += src[i, :].
+ * Bit-identical to numpy.add.at (numpy_vjps.py:941-950): a destination row that occurs several
+ * times receives its addends sequentially in index order.  `order` is the stable argsort of
+ * the (wrapped) index values and `seg_start[s] .. seg_start[s+1]` delimit runs of equal
+ * destination in that order (n_seg runs); both are device arrays prepared by the caller. */
+int agmi_scatter_add_rows(int dtype, void *dst, int64_t n_rows, int64_t inner,
+                          const void *src, const int64_t *index, const int64_t *order,
+                          const int64_t *seg_start, int64_t n_seg, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AGMI_H */

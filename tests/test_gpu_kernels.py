@@ -1,0 +1,364 @@
+"""Kernel-level parity on the GPU, through the C ABI (ctypes) on torch device memory.
+
+Each kernel family is compared with the NumPy/SciPy library routine it replaces, on seeded
+inputs, over every layout path of the planner (flat / rows / nd; row / column / middle / full
+and two-stage reductions; GEMM operand layouts and ragged sizes).  Tolerances: elementwise
+float ops 4 ulp-ish (rtol 1e-6 f32 / 1e-14 f64 of the element, they are single roundings plus
+device libm); reductions and GEMM rtol 1e-5 (f32) / 1e-12 (f64) of |ref| + max|ref|; integer /
+index / copy / scatter work bit-exact.
+"""
+
+import numpy as onp
+import pytest
+import scipy.special
+
+pytestmark = pytest.mark.gpu
+
+F32, F64 = onp.float32, onp.float64
+
+
+@pytest.fixture(scope="module")
+def dnp():
+    import autograd_amd.numpy as dnp
+
+    return dnp
+
+
+def P(dnp, a):
+    return dnp.asarray(a)
+
+
+def close(got, want, rtol):
+    got = onp.asarray(got)
+    want = onp.asarray(want)
+    assert got.shape == want.shape, (got.shape, want.shape)
+    assert got.dtype == want.dtype, (got.dtype, want.dtype)
+    g, w = got.astype(F64), want.astype(F64)
+    scale = onp.max(onp.abs(w)) if w.size else 0.0
+    tol = rtol * onp.abs(w) + rtol * scale
+    bad = ~((onp.abs(g - w) <= tol) | (onp.isnan(g) & onp.isnan(w)) | (g == w))
+    assert not bad.any(), f"max err {onp.max(onp.abs(g - w)[bad])} at {onp.argwhere(bad)[:3].tolist()}"
+
+
+RT = {F32: 1e-5, F64: 1e-12}
+RT_EW = {F32: 2e-6, F64: 2e-15}
+
+
+# ---- elementwise --------------------------------------------------------------------------------
+UNARY = [
+    ("negative", onp.negative, False), ("exp", onp.exp, False), ("log", onp.log, True), ("tanh", onp.tanh, False),
+    ("sinh", onp.sinh, False), ("cosh", onp.cosh, False), ("sin", onp.sin, False), ("cos", onp.cos, False),
+    ("sqrt", onp.sqrt, True), ("square", onp.square, False), ("abs", onp.abs, False), ("sign", onp.sign, False),
+    ("reciprocal", onp.reciprocal, True), ("log1p", onp.log1p, True), ("expm1", onp.expm1, False),
+]
+
+
+@pytest.mark.parametrize("dtype", [F32, F64])
+@pytest.mark.parametrize("name,ref,positive", UNARY)
+def test_unary(dnp, dtype, name, ref, positive):
+    rs = onp.random.RandomState(0)
+    for shape in [(), (1,), (7,), (1031,), (33, 65)]:
+        x = (rs.rand(*shape) * 3 + 0.1 if positive else rs.randn(*shape) * 2).astype(dtype)
+        close(getattr(dnp, name)(P(dnp, x)).numpy(), ref(x), RT_EW[dtype] * 8)
+
+
+BINARY = [("add", onp.add), ("subtract", onp.subtract), ("multiply", onp.multiply), ("true_divide", onp.true_divide),
+          ("maximum", onp.maximum), ("minimum", onp.minimum), ("power", onp.power)]
+
+
+@pytest.mark.parametrize("dtype", [F32, F64])
+@pytest.mark.parametrize("name,ref", BINARY)
+def test_binary_layouts(dnp, dtype, name, ref):
+    rs = onp.random.RandomState(1)
+    op = getattr(dnp, name)
+
+    def mk(*shape):
+        a = rs.rand(*shape) + 0.5 if name in ("power", "true_divide") else rs.randn(*shape)
+        return a.astype(dtype)
+
+    cases = [
+        (mk(1000), mk(1000)),             # flat
+        (mk(37, 29), mk(29)),             # rows: broadcast along rows
+        (mk(37, 29), mk(37, 1)),          # rows: per-row scalar
+        (mk(37, 1), mk(1, 29)),           # both broadcast
+        (mk(5, 6, 7), mk(6, 1)),          # nd
+        (mk(8, 9), mk(9, 8).T),           # transposed operand: nd path
+        (mk(3, 1, 5), mk(4, 1)),
+        (mk(6), mk()),                    # 0-d operand
+    ]
+    for a, b in cases:
+        close(op(P(dnp, a), P(dnp, b)).numpy(), ref(a, b), RT_EW[dtype] * 8)
+    a = mk(50, 20)
+    for s in (2.0, 0.5, 3, -1.25):
+        close(op(P(dnp, a), s).numpy(), ref(a, dtype(s) if False else s).astype(dtype), RT_EW[dtype] * 8)
+        close(op(s, P(dnp, a)).numpy(), ref(s, a).astype(dtype), RT_EW[dtype] * 8)
+
+
+def test_power_shortcuts_are_exact(dnp):
+    x = onp.random.RandomState(2).randn(4099)
+    for e in (2, 1, 0, -1, 0.5, 2.0):
+        xx = onp.abs(x) + 0.1 if e == 0.5 else x
+        assert onp.array_equal(dnp.power(P(dnp, xx), e).numpy(), xx**e), e
+
+
+def test_views_and_slices(dnp):
+    rs = onp.random.RandomState(3)
+    x = rs.randn(2**12 + 3)
+    X = P(dnp, x)
+    assert onp.array_equal((X[1:] - X[:-1] ** 2).numpy(), x[1:] - x[:-1] ** 2)  # misaligned 16-byte vectors
+    assert onp.array_equal((X[3:-5:2] * 2.0).numpy(), x[3:-5:2] * 2.0)
+    A = rs.randn(6, 8, 10).astype(F32)
+    DA = P(dnp, A)
+    assert onp.array_equal(dnp.transpose(DA, (2, 0, 1)).numpy(), A.transpose(2, 0, 1))
+    assert onp.array_equal((dnp.swapaxes(DA, 0, 2) + 1.0).numpy(), A.swapaxes(0, 2) + F32(1.0))
+    assert onp.array_equal(dnp.reshape(dnp.swapaxes(DA, 0, 1), (8, 60)).numpy(), A.swapaxes(0, 1).reshape(8, 60))
+    assert onp.array_equal(DA[2, :, None, 3].numpy(), A[2, :, None, 3])
+    assert onp.array_equal(dnp.repeat(DA[:, :1], 4, axis=1).numpy(), onp.repeat(A[:, :1], 4, axis=1))
+    assert onp.array_equal(dnp.repeat(DA, 3, axis=2).numpy(), onp.repeat(A, 3, axis=2))
+    assert onp.array_equal(dnp.concatenate((DA, DA[:, :2]), axis=1).numpy(), onp.concatenate((A, A[:, :2]), axis=1))
+    assert onp.array_equal(dnp.hstack((DA[0], DA[1, :, :3])).numpy(), onp.hstack((A[0], A[1, :, :3])))
+    assert onp.array_equal(dnp.astype(DA, F64).numpy(), A.astype(F64))
+    assert onp.array_equal((DA > 0.3).numpy(), A > 0.3)
+    assert onp.array_equal(dnp.where(DA > 0, DA, 0.0).numpy(), onp.where(A > 0, A, F32(0)))
+    assert onp.array_equal(dnp.ones((3, 5), dtype=F32).numpy(), onp.ones((3, 5), F32))
+    assert onp.array_equal(dnp.full((1027,), 2.5).numpy(), onp.full((1027,), 2.5))
+    assert [r.shape for r in DA] == [(8, 10)] * 6
+
+
+FUSED = [
+    ("DIV_VJP1", 3, lambda g, x, y: -g * x / y**2),
+    ("TANH_VJP", 2, lambda g, x: g / onp.cosh(x) ** 2),
+    ("POW_VJP1", 3, lambda g, x, a: g * onp.log(onp.where(x, x, 1.0)) * a),
+    ("LSE_VJP", 4, lambda g, b, x, a: g * b * onp.exp(x - a)),
+    ("RECIPROCAL_VJP", 2, lambda g, x: -g / x**2),
+    ("SQRT_VJP", 2, lambda g, x: g * 0.5 * x**-0.5),
+    ("SIN_VJP", 2, lambda g, x: g * onp.cos(x)),
+    ("COS_VJP", 2, lambda g, x: -g * onp.sin(x)),
+    ("SINH_VJP", 2, lambda g, x: g * onp.cosh(x)),
+    ("COSH_VJP", 2, lambda g, x: g * onp.sinh(x)),
+    ("SQUARE_VJP", 2, lambda g, x: g * 2 * x),
+    ("LOG1P_VJP", 2, lambda g, x: g / (x + 1)),
+    ("EXPM1_VJP", 2, lambda g, a: (a + 1) * g),
+    ("MUL_ADD", 3, lambda a, x, y: a * x + y),
+]
+
+
+@pytest.mark.parametrize("dtype", [F32, F64])
+@pytest.mark.parametrize("opname,nin,ref", FUSED)
+def test_fused_rule_kernels(dnp, dtype, opname, nin, ref):
+    from autograd_amd._lib import Op
+    from autograd_amd.numpy import devarray as D
+
+    rs = onp.random.RandomState(4)
+    xs = [(rs.rand(513, 40) + 0.5).astype(dtype) for _ in range(nin)]
+    got = D.map_op(getattr(Op, opname), onp.dtype(dtype), *[P(dnp, x) for x in xs]).numpy()
+    close(got, ref(*xs).astype(dtype), RT_EW[dtype] * 16)
+
+
+def test_pow_vjp0_and_choose(dnp):
+    from autograd_amd._lib import Op
+    from autograd_amd.numpy import devarray as D
+
+    rs = onp.random.RandomState(5)
+    g, x = rs.randn(999), rs.rand(999) + 0.5
+    for y in (2.0, 3.0, 0.0, 1.0, -1.5):
+        want = g * y * x ** onp.where(y, y - 1, 1.0)
+        close(D.map_op(Op.POW_VJP0, onp.dtype(F64), P(dnp, g), P(dnp, x), y).numpy(), want, 1e-14)
+    a, b = rs.randint(0, 3, 999).astype(F64), rs.randint(0, 3, 999).astype(F64)
+    ans = onp.maximum(a, b)
+    want = g * ((a == ans) / (1.0 + (a == b)))
+    assert onp.array_equal(D.map_op(Op.CHOOSE_VJP, onp.dtype(F64), P(dnp, g), P(dnp, a), P(dnp, ans), P(dnp, b)).numpy(), want)
+    gy, gx = D.map_op(Op.DIV_VJP_BOTH, onp.dtype(F64), P(dnp, g), P(dnp, a), P(dnp, x), n_out=2)
+    assert onp.array_equal(gy.numpy(), g / x) and onp.array_equal(gx.numpy(), -g * a / x**2)
+
+
+# ---- reductions ---------------------------------------------------------------------------------
+RED_SHAPES = [
+    ((7,), None), ((5000,), None), ((300000,), None),             # full: group, block, two-stage
+    ((33, 10), 1), ((33, 10), 0), ((1024, 10), 1), ((1024, 10), 0),
+    ((64, 300), 1), ((64, 300), 0), ((20, 5000), 1), ((20, 5000), 0),
+    ((3000, 260), 0), ((3000, 256), 0), ((2, 70000), 1),          # two-stage column / row
+    ((6, 50, 8), 1), ((6, 50, 8), (0, 2)), ((6, 50, 8), (1, 2)), ((6, 50, 8), (0, 1)), ((6, 50, 8), None),
+    ((4, 1, 9), 1), ((0, 5), 0), ((5, 0), 0),
+]
+
+
+@pytest.mark.parametrize("dtype", [F32, F64])
+@pytest.mark.parametrize("shape,axis", RED_SHAPES)
+def test_sum_max_min(dnp, dtype, shape, axis):
+    rs = onp.random.RandomState(6)
+    x = rs.randn(*shape).astype(dtype)
+    X = P(dnp, x)
+    for keepdims in (False, True):
+        close(dnp.sum(X, axis=axis, keepdims=keepdims).numpy(), onp.sum(x, axis=axis, keepdims=keepdims), RT[dtype])
+        if x.size and all(s for s in shape):
+            assert onp.array_equal(dnp.max(X, axis=axis, keepdims=keepdims).numpy(), onp.max(x, axis=axis, keepdims=keepdims))
+            assert onp.array_equal(dnp.min(X, axis=axis, keepdims=keepdims).numpy(), onp.min(x, axis=axis, keepdims=keepdims))
+            close(dnp.mean(X, axis=axis, keepdims=keepdims).numpy(), onp.mean(x, axis=axis, keepdims=keepdims), RT[dtype])
+
+
+def test_sum_of_small_integers_is_exact_in_any_order(dnp):
+    # integer-valued floats: every partial sum is exact, so any summation tree must agree bit for bit
+    rs = onp.random.RandomState(7)
+    x = rs.randint(-8, 9, (777, 513)).astype(F32)
+    X = P(dnp, x)
+    for axis in (None, 0, 1):
+        assert onp.array_equal(dnp.sum(X, axis=axis).numpy(), onp.sum(x, axis=axis, dtype=F64).astype(F32))
+    assert onp.array_equal(dnp.sum(dnp.transpose(X), axis=0).numpy(), onp.sum(x.T, axis=0, dtype=F64).astype(F32))
+
+
+def test_reductions_are_deterministic(dnp):
+    x = P(dnp, onp.random.RandomState(8).randn(4096, 600).astype(F32))
+    for axis in (None, 0, 1):
+        a = dnp.sum(x, axis=axis).numpy()
+        for _ in range(3):
+            assert onp.array_equal(a, dnp.sum(x, axis=axis).numpy())
+
+
+@pytest.mark.parametrize("dtype", [F32, F64])
+def test_fused_map_reduce_is_unbroadcast(dnp, dtype):
+    from autograd_amd._lib import Op, Red
+    from autograd_amd.numpy import devarray as D
+
+    rs = onp.random.RandomState(9)
+    x, g = rs.randn(300, 170).astype(dtype), rs.randn(300, 170).astype(dtype)
+    dt = onp.dtype(dtype)
+    close(D.map_reduce(Op.MUL, Red.SUM, dt, (P(dnp, x), P(dnp, g)), (0,), True).numpy(),
+          onp.sum(x * g, axis=0, keepdims=True), RT[dtype])
+    close(D.map_reduce(Op.MUL, Red.SUM, dt, (P(dnp, x), P(dnp, g)), (1,), True).numpy(),
+          onp.sum(x * g, axis=1, keepdims=True), RT[dtype])
+    b = rs.rand(170).astype(dtype) + 0.5
+    close(D.map_reduce(Op.DIV_VJP1, Red.SUM, dt, (P(dnp, g), P(dnp, x), P(dnp, b)), (0,), True, shape=(300, 170)).numpy(),
+          onp.sum(-g * x / b**2, axis=0, keepdims=True), RT[dtype])
+    close(D.map_reduce(Op.NEG, Red.SUM, dt, (P(dnp, g),), (0, 1), False).numpy(), onp.sum(-g), RT[dtype])
+
+
+@pytest.mark.parametrize("dtype", [F32, F64])
+@pytest.mark.parametrize("shape,axis", [((1024, 10), 1), ((256, 128), 1), ((37, 4096), 1), ((37, 4096), 0),
+                                        ((5, 4), None), ((6, 50, 8), 1), ((3, 70000), 1), ((4, 5), (0, 1))])
+def test_logsumexp_forward(dnp, dtype, shape, axis):
+    from autograd_amd.scipy.special import logsumexp
+
+    rs = onp.random.RandomState(10)
+    x = (rs.randn(*shape) * 5).astype(dtype)
+    for keepdims in (False, True):
+        want = scipy.special.logsumexp(x, axis=axis, keepdims=keepdims)
+        close(logsumexp(P(dnp, x), axis=axis, keepdims=keepdims).numpy(), onp.asarray(want, dtype=dtype), RT[dtype])
+
+
+def test_logsumexp_special_values(dnp):
+    from autograd_amd.scipy.special import logsumexp
+
+    x = onp.array([[-onp.inf, -onp.inf, -onp.inf], [0.0, -onp.inf, 0.0], [1000.0, 1000.0, 999.0],
+                   [onp.inf, 1.0, 2.0], [-1000.0, -1001.0, -1002.0], [onp.nan, 1.0, 2.0]])
+    with onp.errstate(all="ignore"):
+        want = scipy.special.logsumexp(x, axis=1)
+    got = logsumexp(P(dnp, x), axis=1).numpy()
+    assert onp.allclose(got, want, rtol=1e-13, equal_nan=True), (got, want)
+
+
+# ---- contractions -------------------------------------------------------------------------------
+GEMM_SHAPES = [(1, 1, 1), (5, 7, 3), (64, 64, 16), (65, 63, 17), (130, 70, 33), (256, 128, 641), (1024, 10, 1024),
+               (10, 1024, 300), (300, 300, 1), (129, 257, 100), (512, 512, 512)]
+
+
+@pytest.mark.parametrize("dtype", [F32, F64])
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
+def test_dot_all_operand_layouts(dnp, dtype, M, N, K):
+    rs = onp.random.RandomState(11)
+    a, b = rs.randn(M, K).astype(dtype), rs.randn(K, N).astype(dtype)
+    want = (a.astype(F64) @ b.astype(F64)).astype(dtype)
+    rt = RT[dtype] * max(1.0, onp.sqrt(K) / 8)
+    A, B = P(dnp, a), P(dnp, b)
+    close(dnp.dot(A, B).numpy(), want, rt)                                                  # NN
+    At, Bt = P(dnp, onp.ascontiguousarray(a.T)), P(dnp, onp.ascontiguousarray(b.T))
+    close(dnp.dot(dnp.transpose(At), B).numpy(), want, rt)                                  # TN  (A^T . G)
+    close(dnp.dot(A, dnp.transpose(Bt)).numpy(), want, rt)                                  # NT  (G . B^T)
+    close(dnp.dot(dnp.transpose(At), dnp.transpose(Bt)).numpy(), want, rt)                  # TT
+    if M > 4 and K > 4:
+        close(dnp.dot(A[1:-1, 2:], B[2:]).numpy(), (a[1:-1, 2:].astype(F64) @ b[2:].astype(F64)).astype(dtype), rt)
+    if M >= 8 and N >= 8 and K >= 8:
+        close(dnp.dot(A[::2, ::2], B[::2, ::2]).numpy(),
+              (a[::2, ::2].astype(F64) @ b[::2, ::2].astype(F64)).astype(dtype), rt)        # generic strides
+
+
+def test_dot_small_integers_exact(dnp):
+    rs = onp.random.RandomState(12)
+    a = rs.randint(-4, 5, (200, 333)).astype(F32)
+    b = rs.randint(-4, 5, (333, 150)).astype(F32)
+    assert onp.array_equal(dnp.dot(P(dnp, a), P(dnp, b)).numpy(), a @ b)
+    assert onp.array_equal(dnp.dot(P(dnp, a.astype(F64)), P(dnp, b.astype(F64))).numpy(), a.astype(F64) @ b.astype(F64))
+
+
+@pytest.mark.parametrize("dtype", [F32, F64])
+def test_dot_vector_forms_matmul_tensordot(dnp, dtype):
+    rs = onp.random.RandomState(13)
+    rt = RT[dtype] * 4
+    A, v, u = rs.randn(30, 40).astype(dtype), rs.randn(40).astype(dtype), rs.randn(30).astype(dtype)
+    close(dnp.dot(P(dnp, A), P(dnp, v)).numpy(), A @ v, rt)
+    close(dnp.dot(P(dnp, u), P(dnp, A)).numpy(), u @ A, rt)
+    close(dnp.dot(P(dnp, v), P(dnp, v)).numpy(), onp.asarray(v @ v), rt)
+    close(dnp.dot(P(dnp, A), 2.0).numpy(), A * dtype(2.0), rt)
+    B3, C3 = rs.randn(4, 30, 40).astype(dtype), rs.randn(4, 40, 20).astype(dtype)
+    close(dnp.matmul(P(dnp, B3), P(dnp, C3)).numpy(), onp.matmul(B3, C3), rt)
+    close(dnp.matmul(P(dnp, B3), P(dnp, C3[0])).numpy(), onp.matmul(B3, C3[0]), rt)
+    close(dnp.matmul(P(dnp, A), P(dnp, C3)).numpy(), onp.matmul(A, C3), rt)
+    close(dnp.matmul(P(dnp, B3), P(dnp, v)).numpy(), onp.matmul(B3, v), rt)
+    T1, T2 = rs.randn(2, 3, 5, 4).astype(dtype), rs.randn(5, 4, 2, 3).astype(dtype)
+    close(dnp.tensordot(P(dnp, T1), P(dnp, T2), 2).numpy(), onp.tensordot(T1, T2, 2), rt)
+    close(dnp.tensordot(P(dnp, T1), P(dnp, T2), [[0, 1], [2, 3]]).numpy(), onp.tensordot(T1, T2, [[0, 1], [2, 3]]), rt)
+    close(dnp.tensordot(P(dnp, T1), P(dnp, T2), [[3, 0], [1, 2]]).numpy(), onp.tensordot(T1, T2, [[3, 0], [1, 2]]), rt)
+    close(dnp.tensordot(P(dnp, A), P(dnp, v), 0).numpy(), onp.tensordot(A, v, 0), rt)
+    close(dnp.dot(P(dnp, B3), P(dnp, C3[0])).numpy(), onp.dot(B3, C3[0]), rt)
+    close(dnp.outer(P(dnp, u), P(dnp, v)).numpy(), onp.outer(u, v), rt)
+
+
+# ---- index / scatter: bit exact -----------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [F32, F64])
+def test_take_and_ordered_scatter_add(dnp, dtype):
+    from autograd_amd.numpy import wrapper as W
+
+    rs = onp.random.RandomState(14)
+    A = rs.randn(50, 7).astype(dtype)
+    for idx in ([0, 0], [0, 1, 0], [3, -1, 3, 3, 49, -50], list(rs.randint(-50, 50, 500)), []):
+        got = P(dnp, A)[idx].numpy()
+        assert onp.array_equal(got, A[onp.array(idx, dtype="int64")])
+        x = (rs.randn(len(idx), 7) * 1e3).astype(dtype)
+        dst = rs.randn(50, 7).astype(dtype)
+        want = dst.copy()
+        onp.add.at(want, onp.array(idx, dtype="int64"), x)
+        got = W.scatter_add(dnp.asarray(dst) + 0.0, idx, P(dnp, x)).numpy()
+        assert onp.array_equal(got, want), idx[:6]
+    v = rs.randn(1000).astype(dtype)
+    idx = list(rs.randint(0, 10, 4000))           # long runs: sequential order matters in floating point
+    x = (rs.randn(4000) * onp.exp(rs.randn(4000) * 5)).astype(dtype)
+    want = v[:10].copy()
+    onp.add.at(want, onp.array(idx), x)
+    assert onp.array_equal(W.scatter_add(dnp.asarray(v[:10]) + 0.0, idx, P(dnp, x)).numpy(), want)
+    for sl in (slice(1, None), slice(None, -1), slice(2, 9, 3), 4, (slice(None), 2), (Ellipsis, slice(1, 3))):
+        dst = rs.randn(12, 5).astype(dtype)
+        x = rs.randn(*onp.shape(dst[sl])).astype(dtype)
+        want = dst.copy()
+        onp.add.at(want, sl, x)
+        assert onp.array_equal(W.scatter_add(dnp.asarray(dst) + 0.0, sl, P(dnp, x)).numpy(), want)
+
+
+def test_vspace_axioms(dnp):
+    # tests/test_vspaces.py:10-159 of the reference, for the device vspace
+    from autograd_amd.extend import vspace
+
+    x = P(dnp, onp.random.RandomState(15).randn(4, 3))
+    vs = vspace(x)
+    assert vs.shape == (4, 3) and vs.dtype == onp.float64 and vs.size == 12 and vs.ndim == 2
+    assert vs == vspace(vs.zeros()) and vs == vspace(vs.ones()) and vs == vspace(vs.randn())
+    a, b = vs.randn(), vs.randn()
+    assert onp.array_equal(vs.add(a, b).numpy(), a.numpy() + b.numpy())
+    assert onp.array_equal(vs.add(a, vs.zeros()).numpy(), a.numpy())
+    assert onp.array_equal(vs.scalar_mul(a, 2.5).numpy(), a.numpy() * 2.5)
+    assert abs(float(vs.inner_prod(a, b)) - onp.sum(a.numpy() * b.numpy())) < 1e-12
+    basis = list(vs.standard_basis())
+    assert len(basis) == 12 and onp.array_equal(onp.sum([e.numpy() for e in basis], axis=0), onp.ones((4, 3)))
+    acc = vs.mut_add(None, a)
+    acc2 = vs.mut_add(acc, b)
+    assert acc2 is acc and onp.array_equal(acc.numpy(), (0.0 + a.numpy()) + b.numpy())
+    assert vspace(dnp.ones((2,), dtype=F32)).dtype == onp.float32

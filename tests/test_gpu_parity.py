@@ -1,0 +1,229 @@
+"""Parity of the MI355X path with the CPU oracle (and through it the reference), on the GPU.
+
+* small sizes: against the golden vectors the real reference wrote (tests/golden);
+* medium / full sizes: against the oracle run in this process on the same seeded inputs, and
+  against float64 closed forms, with the tolerance north-star states (rtol 1e-12 f64 / 1e-5
+  f32, applied as |got - ref| <= rtol * |ref| + rtol * max|ref|: a pure relative bound is
+  meaningless at the zeros of a derivative);
+* index / scatter results bit-exact;
+* size-independent properties at full size (linearity of the VJP in its cotangent, symmetry of
+  the Hessian-vector product, agreement of the two HVP constructions).
+"""
+
+import os
+
+import numpy as onp
+import pytest
+
+from autograd_amd import configs
+from cases import SMALL, extra_cases, flatten
+from conftest import oracle_backend
+from oracle import closed_forms as cf
+
+pytestmark = pytest.mark.gpu
+
+GOLD = onp.load(os.path.join(os.path.dirname(__file__), "golden", "reference_vectors.npz"))
+
+
+def check(name, got, want, rtol=None, exact=False):
+    got, want = onp.asarray(got), onp.asarray(want)
+    assert got.dtype == want.dtype, f"{name}: dtype {got.dtype} != {want.dtype}"
+    assert got.shape == want.shape, f"{name}: shape {got.shape} != {want.shape}"
+    if exact:
+        assert onp.array_equal(got, want), f"{name}: not bit-exact, max diff {onp.max(onp.abs(got - want))}"
+        return
+    if rtol is None:
+        rtol = 1e-5 if want.dtype == onp.float32 else 1e-12
+    g, w = got.astype(onp.float64), want.astype(onp.float64)
+    tol = rtol * onp.abs(w) + rtol * onp.max(onp.abs(w))
+    err = onp.abs(g - w)
+    assert onp.all(err <= tol), f"{name}: max err/tol {onp.max(err / (tol + 1e-300)):.3g}"
+
+
+@pytest.fixture(scope="module")
+def dev():
+    return configs.device_backend()
+
+
+@pytest.mark.parametrize("name", list(SMALL))
+def test_small_workloads_match_reference_vectors(dev, name):
+    inputs = configs.CONFIG_INPUTS[name](**SMALL[name])
+    store = {}
+    flatten(name, configs.run_config(name, dev, inputs), store)
+    for key, value in store.items():
+        check(key, value, GOLD[key])
+
+
+# cases whose inputs are float32 but whose result is float64 through NumPy-2 promotion in the rule
+_F32_INPUT = {"extra/mean_f32_all", "extra/mean_f32_axis0", "extra/var_f32"}
+_BIT_EXACT = {"extra/dup_index_00"}
+
+
+def test_extra_cases_match_reference_vectors(dev):
+    store = {}
+    flatten("extra", extra_cases(dev), store)
+    assert set(store) == {k for k in GOLD.files if k.startswith("extra/")}
+    for key, value in store.items():
+        check(key, value, GOLD[key], rtol=1e-5 if key in _F32_INPUT else None, exact=key in _BIT_EXACT)
+
+
+MEDIUM = {
+    "tanh": dict(n=200003),
+    "bcast": dict(rows=1024, cols=515),
+    "mlp": dict(batch=256, layer_sizes=(784, 300, 257, 10)),
+    "rnn": dict(seq_len=8, batch=32, input_size=24, state_size=40, output_size=24),
+    "rosen": dict(n=100001),
+}
+
+
+@pytest.mark.parametrize("name", list(MEDIUM))
+def test_medium_workloads_match_oracle(dev, name):
+    inputs = configs.CONFIG_INPUTS[name](**MEDIUM[name])
+    got, want = {}, {}
+    flatten(name, configs.run_config(name, dev, inputs), got)
+    flatten(name, configs.run_config(name, oracle_backend(), inputs), want)
+    assert set(got) == set(want)
+    for key in want:
+        check(key, got[key], want[key])
+
+
+def test_full_tanh(dev):
+    inputs = configs.tanh_inputs()
+    got = configs.run_config("tanh", dev, inputs)
+    want = configs.run_config("tanh", oracle_backend(), inputs)
+    exact = cf.tanh_derivatives(inputs["x"])
+    for k in ("d1", "d2", "d3"):
+        check(f"tanh/{k} vs oracle", got[k], want[k])
+        check(f"tanh/{k} vs closed form", got[k], exact[k], rtol=1e-11)
+
+
+def test_full_bcast(dev):
+    inputs = configs.bcast_inputs()
+    got = configs.run_config("bcast", dev, inputs)
+    want = configs.run_config("bcast", oracle_backend(), inputs)
+    exact = cf.bcast_grads(**inputs)
+    for k in ("dA", "db", "dc"):
+        check(f"bcast/{k} vs oracle", got[k], want[k])
+        check(f"bcast/{k} vs f64 closed form", got[k], exact[k].astype(onp.float32))
+        # and the device result is at least as close to the float64 answer as NumPy's float32 one
+        e_dev = onp.max(onp.abs(got[k].astype(onp.float64) - exact[k]))
+        e_ref = onp.max(onp.abs(want[k].astype(onp.float64) - exact[k]))
+        assert e_dev <= 4 * e_ref + 1e-6 * onp.max(onp.abs(exact[k])), (k, e_dev, e_ref)
+
+
+def test_full_mlp(dev):
+    inputs = configs.mlp_inputs()
+    got = configs.run_config("mlp", dev, inputs)["grad"]
+    want = configs.run_config("mlp", oracle_backend(), inputs)["grad"]
+    exact = cf.mlp_grads(inputs["params"], inputs["X"], inputs["T"])
+    for layer in range(3):
+        for j, nm in enumerate(("W", "b")):
+            check(f"mlp/{layer}/{nm} vs oracle", got[layer][j], want[layer][j])
+            check(f"mlp/{layer}/{nm} vs f64 backprop", got[layer][j], exact[layer][j].astype(onp.float32))
+
+
+def test_full_rnn(dev):
+    inputs = configs.rnn_inputs()
+    got = configs.run_config("rnn", dev, inputs)["grad"]
+    want = configs.run_config("rnn", oracle_backend(), inputs)["grad"]
+    for k in want:
+        check(f"rnn/{k} vs oracle", got[k], want[k])
+
+
+def test_full_rosen_hvp(dev):
+    inputs = configs.rosen_inputs()
+    got = configs.run_config("rosen", dev, inputs)
+    check("rosen/grad vs closed form", got["grad"], cf.rosen_grad(inputs["x"]), rtol=1e-12)
+    exact = cf.rosen_hvp(inputs["x"], inputs["v"])
+    check("rosen/hvp_rev vs closed form", got["hvp_rev"], exact, rtol=1e-12)
+    check("rosen/hvp_fwd vs closed form", got["hvp_fwd"], exact, rtol=1e-12)
+    want = configs.run_config("rosen", oracle_backend(), configs.rosen_inputs(n=2**20))
+    got_s = configs.run_config("rosen", dev, configs.rosen_inputs(n=2**20))
+    for k in ("grad", "hvp_rev", "hvp_fwd"):
+        check(f"rosen/{k} vs oracle (2^20)", got_s[k], want[k])
+
+
+def test_vjp_is_linear_and_hvp_is_symmetric(dev):
+    import autograd_amd as ag
+
+    np = dev.np
+    prog = configs.rosen_program(dev)
+    inp = configs.rosen_inputs(n=2**22)
+    x, v = dev.put(inp["x"]), dev.put(inp["v"])
+    w = dev.put(onp.random.RandomState(3).randn(2**22))
+    hvp = ag.make_hvp(prog["f"])(x)[0]
+    hv, hw = hvp(v), hvp(w)
+    # <w, H v> == <v, H w>
+    a, b = float(np.sum(w * hv)), float(np.sum(v * hw))
+    assert abs(a - b) <= 1e-9 * max(abs(a), abs(b))
+    # H (2v - 3w) == 2 H v - 3 H w
+    lhs = hvp(2.0 * v - 3.0 * w).numpy()
+    rhs = (2.0 * hv - 3.0 * hw).numpy()
+    check("hvp linearity", lhs, rhs, rtol=1e-11)
+
+
+def test_containers_exact_answers(dev):
+    # tests/test_tuple.py:11-24, test_list.py:11-24, test_dict.py:13-26 of the reference
+    import autograd_amd as ag
+
+    np = dev.np
+    rs = onp.random.RandomState(5)
+    A, B, C = (dev.put(rs.randn(*s)) for s in ((5, 6), (4, 3), (2, 4)))
+    for arg, keys in (((A, B, C), (0, 1, 2)), ([A, B, C], (0, 1, 2)), ({"a": A, "b": B, "c": C}, ("a", "b", "c"))):
+        res = ag.grad(lambda c: np.sum(c[keys[0]]) + 2.0 * np.sum(c[keys[1]]))(arg)
+        assert type(res) is type(arg)
+        assert onp.array_equal(res[keys[0]].numpy(), onp.ones((5, 6)))
+        assert onp.array_equal(res[keys[1]].numpy(), 2 * onp.ones((4, 3)))
+        assert onp.array_equal(res[keys[2]].numpy(), onp.zeros((2, 4)))
+
+
+def test_known_answers_on_device(dev):
+    import autograd_amd as ag
+
+    np = dev.np
+    # README.md:27-34 and tests/test_direct.py:13-24 of the reference
+    assert abs(float(ag.grad(np.tanh)(1.0)) - 0.419974341614026) < 1e-14
+    assert abs(float(ag.grad(lambda x: (x + np.sin(x**2)) * x)(1.3)) - 3.190948746871) < 1e-6
+    assert float(ag.grad(lambda x: x**0)(0.0)) == 0.0
+    x32 = dev.put(onp.arange(4, dtype=onp.float32) + 1)
+    assert ag.grad(lambda x: np.sum(np.sin(x) * 3.0))(x32).dtype == onp.float32
+    with pytest.raises(TypeError):
+        ag.grad(lambda x: x * 2.0)(dev.put(onp.ones(3)))
+
+
+def test_check_grads_on_device(dev):
+    # the reference's own checker (autograd/test_util.py:60-78) run against the device value type
+    from autograd_amd.scipy.special import logsumexp
+    from autograd_amd.test_util import check_grads
+
+    np = dev.np
+    rs = onp.random.RandomState(6)
+    P = dev.put
+    for sa in [(), (4,), (3, 4), (1, 4)]:
+        for sb in [(), (4,), (3, 4), (1, 4)]:
+            a, b = P(rs.randn(*sa)), P(onp.abs(rs.randn(*sb)) + 1.1)
+            for op in (np.add, np.subtract, np.multiply, np.true_divide, np.maximum):
+                check_grads(lambda a, b: op(a, b), (0, 1))(a, b)
+            check_grads(lambda a, b: np.power(b, a), (0, 1))(a, b)
+    x = P(rs.randn(3, 4))
+    for f in (np.exp, np.tanh, np.sin, np.cos, np.sinh, np.cosh, np.square, np.negative):
+        check_grads(f)(x)
+    for f in (np.log, np.sqrt, np.reciprocal, np.log1p, np.abs):
+        check_grads(f)(P(onp.abs(rs.randn(3, 4)) + 1.1))
+    for axis in (None, 0, 1):
+        for keepdims in (False, True):
+            for red in (np.sum, np.mean, np.max, np.var, np.std, np.prod):
+                check_grads(lambda x: red(x, axis=axis, keepdims=keepdims))(x)
+            check_grads(lambda x: logsumexp(x, axis=axis, keepdims=keepdims))(x)
+    A, B = P(rs.randn(3, 4)), P(rs.randn(4, 5))
+    check_grads(np.dot, (0, 1), order=3)(A, B)
+    check_grads(np.dot, (0, 1))(A, P(rs.randn(4)))
+    check_grads(np.dot, (0, 1))(P(rs.randn(3)), A)
+    check_grads(np.matmul, (0, 1))(P(rs.randn(2, 3, 4)), P(rs.randn(2, 4, 5)))
+    check_grads(np.matmul, (0, 1))(P(rs.randn(2, 3, 4)), B)
+    T1, T2 = P(rs.randn(2, 3, 4)), P(rs.randn(4, 3, 5))
+    check_grads(lambda a, b: np.tensordot(a, b, axes=[[1, 2], [1, 0]]), (0, 1), order=3)(T1, T2)
+    check_grads(lambda x: np.sum(np.sin(x[[0, 1, 0]]) * x[0, 1]))(x)
+    check_grads(lambda x: np.hstack((x[0], x[1, 1:])))(x)
+    check_grads(lambda x: np.repeat(x[:, :1], 3, axis=1) * np.reshape(x, (4, 3)).T)(x)
+    check_grads(lambda x: np.concatenate((x, x * 2.0), axis=0))(x)

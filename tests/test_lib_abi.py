@@ -1,0 +1,86 @@
+"""The C-ABI library loads without a GPU and exports every symbol ``include/agmi.h`` declares."""
+
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "agmi.h")
+LIB = os.path.join(ROOT, "autograd_amd", "libagmi.so")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(agmi_[a-z0-9_]+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(LIB):
+        pytest.fail(f"{LIB} is not built; run `make -C autograd_amd/csrc`")
+    return ctypes.CDLL(LIB)
+
+
+def test_header_declares_entry_points():
+    names = declared_symbols()
+    assert "agmi_elementwise" in names and "agmi_gemm" in names and len(names) >= 10
+
+
+def test_every_declared_symbol_is_exported(lib):
+    missing = [n for n in declared_symbols() if not hasattr(lib, n)]
+    assert not missing, missing
+
+
+def test_binding_covers_the_header():
+    from autograd_amd import _lib
+
+    assert sorted(_lib.EXPORTS) == declared_symbols()
+    L = _lib.lib()
+    assert L.agmi_version() >= 100
+    assert _lib.AgmiArray.strides.size == 8 * 8  # AGMI_MAX_DIMS int64 strides
+
+
+def test_op_codes_match_header():
+    from autograd_amd import _lib
+
+    text = open(HEADER).read()
+    body = re.search(r"typedef enum agmi_op \{(.*?)\} agmi_op;", text, flags=re.S).group(1)
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    value = -1
+    for item in body.split(","):
+        item = item.strip()
+        if not item:
+            continue
+        if "=" in item:
+            name, v = [s.strip() for s in item.split("=")]
+            value = int(v)
+        else:
+            name, value = item, value + 1
+        py = name.replace("AGMI_OP_", "")
+        assert getattr(_lib.Op, py) == value, (name, value)
+
+
+def test_argument_errors_are_reported_without_a_gpu(lib):
+    # argument validation happens on the host before any launch
+    lib.agmi_last_error.restype = ctypes.c_char_p
+    rc = lib.agmi_fill(0, None, ctypes.c_int64(16), ctypes.c_double(0.0), None)
+    assert rc == -1 and b"fill" in lib.agmi_last_error()
+    rc = lib.agmi_gemm(0, ctypes.c_int64(1), ctypes.c_int64(-1), ctypes.c_int64(1), ctypes.c_int64(1),
+                       ctypes.c_double(1.0), None, ctypes.c_int64(0), ctypes.c_int64(0), ctypes.c_int64(0), None,
+                       ctypes.c_int64(0), ctypes.c_int64(0), ctypes.c_int64(0), ctypes.c_double(0.0), None,
+                       ctypes.c_int64(1), ctypes.c_int64(0), None)
+    assert rc == -1
+
+
+def test_device_path_fails_loudly_without_gpu():
+    import torch
+
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    import autograd_amd.numpy as np
+
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        np.ones((2, 2))
