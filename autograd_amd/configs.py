@@ -131,16 +131,16 @@ def mlp_program(be):
 # --------------------------------------------------------------------------------------
 # config 4: vanilla tanh RNN driven by a Python loop, float32
 # --------------------------------------------------------------------------------------
-def rnn_inputs(seq_len=64, batch=256, input_size=128, state_size=512, output_size=128, seed=0):
+def rnn_inputs(seq_len=64, batch=256, input_size=128, state_size=512, output_size=128, seed=0, dtype=onp.float32):
     rs = onp.random.RandomState(seed)
     ids = rs.randint(0, input_size, (seq_len, batch))
-    inputs = (ids[:, :, None] == onp.arange(input_size)[None, None, :]).astype(onp.float32)
+    inputs = (ids[:, :, None] == onp.arange(input_size)[None, None, :]).astype(dtype)
     tids = rs.randint(0, output_size, (seq_len, batch))
-    targets = (tids[:, :, None] == onp.arange(output_size)[None, None, :]).astype(onp.float32)
+    targets = (tids[:, :, None] == onp.arange(output_size)[None, None, :]).astype(dtype)
     params = {
-        "init hiddens": (0.1 * rs.randn(1, state_size)).astype(onp.float32),
-        "change": (0.1 * rs.randn(input_size + state_size + 1, state_size)).astype(onp.float32),
-        "predict": (0.1 * rs.randn(state_size + 1, output_size)).astype(onp.float32),
+        "init hiddens": (0.1 * rs.randn(1, state_size)).astype(dtype),
+        "change": (0.1 * rs.randn(input_size + state_size + 1, state_size)).astype(dtype),
+        "predict": (0.1 * rs.randn(state_size + 1, output_size)).astype(dtype),
     }
     return {"inputs": inputs, "targets": targets, "params": params}
 
@@ -149,7 +149,7 @@ def rnn_program(be):
     np, logsumexp = be.np, be.logsumexp
 
     def concat_and_multiply(weights, *args):
-        cat_state = np.hstack(args + (np.ones((args[0].shape[0], 1), dtype=np.float32),))
+        cat_state = np.hstack(args + (np.ones((args[0].shape[0], 1), dtype=args[0].dtype),))
         return np.dot(cat_state, weights)
 
     def rnn_predict(params, inputs):

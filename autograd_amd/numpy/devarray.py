@@ -128,8 +128,9 @@ def from_numpy(a, dtype=None):
             a = a.astype(onp.int64)
         else:
             raise TypeError(f"dtype {a.dtype} is not supported on the device")
-    a = onp.ascontiguousarray(a)
-    t = torch.from_numpy(a.copy() if not a.flags.writeable else a).to(_lib.device())
+    if not a.flags.c_contiguous or not a.flags.writeable:
+        a = onp.array(a, order="C")  # (ascontiguousarray would turn a 0-d array into 1-d)
+    t = torch.from_numpy(a).to(_lib.device())
     return DevArray(t, a.dtype)
 
 

@@ -58,7 +58,7 @@ UNARY = [
 def test_unary(dnp, dtype, name, ref, positive):
     rs = onp.random.RandomState(0)
     for shape in [(), (1,), (7,), (1031,), (33, 65)]:
-        x = (rs.rand(*shape) * 3 + 0.1 if positive else rs.randn(*shape) * 2).astype(dtype)
+        x = onp.asarray(rs.rand(*shape) * 3 + 0.1 if positive else rs.randn(*shape) * 2).astype(dtype)
         close(getattr(dnp, name)(P(dnp, x)).numpy(), ref(x), RT_EW[dtype] * 8)
 
 
@@ -74,7 +74,7 @@ def test_binary_layouts(dnp, dtype, name, ref):
 
     def mk(*shape):
         a = rs.rand(*shape) + 0.5 if name in ("power", "true_divide") else rs.randn(*shape)
-        return a.astype(dtype)
+        return onp.asarray(a).astype(dtype)
 
     cases = [
         (mk(1000), mk(1000)),             # flat
