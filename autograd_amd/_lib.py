@@ -115,6 +115,8 @@ def lib():
     L.agmi_last_error.argtypes = []
     L.agmi_version.restype = c_i
     L.agmi_version.argtypes = []
+    L.agmi_last_kernel.restype = ctypes.c_char_p
+    L.agmi_last_kernel.argtypes = []
     L.agmi_elementwise.restype = c_i
     L.agmi_elementwise.argtypes = [c_i, c_i, c_i, p_i64, c_i, p_arr, c_i, p_arr, p_d, c_p]
     L.agmi_compare.restype = c_i
@@ -139,7 +141,7 @@ def lib():
 
 
 EXPORTS = (
-    "agmi_last_error agmi_version agmi_elementwise agmi_compare agmi_cast agmi_map_reduce "
+    "agmi_last_error agmi_version agmi_last_kernel agmi_elementwise agmi_compare agmi_cast agmi_map_reduce "
     "agmi_map_reduce_workspace_bytes agmi_gemm agmi_fill agmi_take_rows agmi_scatter_add_rows"
 ).split()
 
@@ -178,6 +180,79 @@ def empty(shape, np_dtype):
 
 def synchronize():
     torch.cuda.synchronize(device())
+
+
+# ---- optional per-launch timing (HIP events on the launch stream) ------------------------------
+class KernelTimer:
+    """Times launches with HIP events recorded on the stream the kernels run on.
+
+    ``with KernelTimer() as kt: ...`` brackets every launch whose ``(entry point, op)`` key is in
+    ``only`` (all launches when ``only`` is None).  ``summary()`` (after a device synchronise)
+    gives, per kernel name, the launch count, the average duration and the average algorithmic
+    traffic: every distinct input element read once plus every output element written once
+    (2*M*N*K flops for a contraction).
+    """
+
+    def __init__(self, only=None):
+        self.only = only
+        self.records = []
+
+    def __enter__(self):
+        global _TIMER
+        self._prev, _TIMER = _TIMER, self
+        return self
+
+    def __exit__(self, *exc):
+        global _TIMER
+        _TIMER = self._prev
+
+    def begin(self, key):
+        if self.only is not None and key not in self.only:
+            return None
+        ev = torch.cuda.Event(enable_timing=True)
+        ev.record()
+        return ev
+
+    def end(self, ev0, key, nbytes, flops=0.0):
+        ev1 = torch.cuda.Event(enable_timing=True)
+        ev1.record()
+        name = _LIB.agmi_last_kernel().decode()
+        self.records.append((name, key, ev0, ev1, nbytes, flops))
+
+    def summary(self):
+        synchronize()
+        out = {}
+        for name, key, ev0, ev1, nbytes, flops in self.records:
+            r = out.setdefault(name, {"key": key, "launches": 0, "ms": 0.0, "bytes": 0.0, "flops": 0.0})
+            r["launches"] += 1
+            r["ms"] += ev0.elapsed_time(ev1)
+            r["bytes"] += nbytes
+            r["flops"] += flops
+        for r in out.values():
+            n = r["launches"]
+            r["avg_ms"], r["avg_bytes"], r["avg_flops"] = r["ms"] / n, r["bytes"] / n, r["flops"] / n
+        return out
+
+
+_TIMER = None
+
+
+def _distinct_bytes(t):
+    n = 1
+    for extent, stride in zip(t.shape, t.stride()):
+        if stride != 0:
+            n *= extent
+    return n * t.element_size()
+
+
+def _traffic(outs, ins):
+    total = 0
+    for t in outs:
+        total += t.numel() * t.element_size()
+    for t in ins:
+        if isinstance(t, torch.Tensor):
+            total += _distinct_bytes(t)
+    return total
 
 
 # ---- argument marshalling (buffers reused: single-threaded by contract) ----------------------
@@ -224,9 +299,12 @@ def elementwise(op, code, shape, outs, ins):
     for k, t in enumerate(outs):
         _set_array(_outs[k], t)
     n_in = _set_inputs(ins)
+    ev = _TIMER.begin(("elementwise", op)) if _TIMER is not None else None
     rc = _LIB.agmi_elementwise(op, code, nd, _shape, len(outs), _outs, n_in, _ins, _scalars, _stream())
     if rc:
         _check(rc, "agmi_elementwise")
+    if ev is not None:
+        _TIMER.end(ev, ("elementwise", op), _traffic(outs, ins))
 
 
 def compare(cmp, code, shape, out, ins):
@@ -267,20 +345,27 @@ def map_reduce(op, red, code, shape, reduce_mask, out, ins):
     _set_array(_outs[0], out)
     n_in = _set_inputs(ins)
     ws = _workspace()
+    ev = _TIMER.begin(("map_reduce", op, red)) if _TIMER is not None else None
     rc = _LIB.agmi_map_reduce(op, red, code, nd, _shape, _mask, _outs, n_in, _ins, _scalars, ws.data_ptr(),
                               _WORKSPACE_BYTES, _stream())
     if rc == -2:  # AGMI_ERR_UNSUPPORTED
         return False
     if rc:
         _check(rc, "agmi_map_reduce")
+    if ev is not None:
+        _TIMER.end(ev, ("map_reduce", op, red), _traffic((out,), ins))
     return True
 
 
 def gemm(code, batch, M, N, K, alpha, A, a_rs, a_cs, a_bs, B, b_rs, b_cs, b_bs, beta, C, ldc, c_bs):
+    ev = _TIMER.begin(("gemm",)) if _TIMER is not None else None
     rc = _LIB.agmi_gemm(code, batch, M, N, K, alpha, A.data_ptr(), a_rs, a_cs, a_bs, B.data_ptr(), b_rs, b_cs, b_bs,
                         beta, C.data_ptr(), ldc, c_bs, _stream())
     if rc:
         _check(rc, "agmi_gemm")
+    if ev is not None:
+        es = A.element_size()
+        _TIMER.end(ev, ("gemm",), batch * (M * K + K * N + M * N) * es, 2.0 * batch * M * N * K)
 
 
 def fill(code, t, value):

@@ -14,6 +14,8 @@
 namespace agmi {
 
 void set_error(const char *fmt, ...);
+// name of the kernel family the last successful entry point launched (for profilers' labels)
+void set_kernel_name(const char *fmt, ...);
 int hip_check(hipError_t e, const char *what);
 
 constexpr int kBlock = 256;        // 4 wavefronts of 64 lanes

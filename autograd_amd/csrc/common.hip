@@ -14,6 +14,15 @@ void set_error(const char *fmt, ...) {
     va_end(ap);
 }
 
+static thread_local char g_kernel[128] = "";
+
+void set_kernel_name(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_kernel, sizeof(g_kernel), fmt, ap);
+    va_end(ap);
+}
+
 int hip_check(hipError_t e, const char *what) {
     if (e == hipSuccess) return 0;
     set_error("%s: %s", what, hipGetErrorString(e));
@@ -106,6 +115,7 @@ static int launch_fill(void *ptr, int64_t n, double value, hipStream_t s) {
         set_error("fill: too many elements");
         return AGMI_ERR_UNSUPPORTED;
     }
+    set_kernel_name("fill_kernel");
     hipLaunchKernelGGL(fill_kernel<T>, dim3((unsigned)blocks), dim3(kBlock), 0, s, static_cast<T *>(ptr), n,
                        static_cast<T>(value));
     return hip_check(hipGetLastError(), "fill launch");
@@ -116,6 +126,8 @@ static int launch_fill(void *ptr, int64_t n, double value, hipStream_t s) {
 using namespace agmi;
 
 extern "C" const char *agmi_last_error(void) { return g_error; }
+
+extern "C" const char *agmi_last_kernel(void) { return g_kernel; }
 
 extern "C" int agmi_version(void) { return 100; }
 

@@ -200,8 +200,8 @@ static int check_blocks(int64_t blocks) {
 }
 
 template <template <typename> class F, typename T>
-static int launch_ew(const Merged &m, int n_out, const agmi_array *outs, int n_in, const agmi_array *ins,
-                     const double *scalars, hipStream_t s) {
+static int launch_ew(const char *fname, const Merged &m, int n_out, const agmi_array *outs, int n_in,
+                     const agmi_array *ins, const double *scalars, hipStream_t s) {
     using Fn = F<T>;
     if (n_in != Fn::NIN || n_out != Fn::NOUT) {
         set_error("elementwise: op takes %d inputs and %d outputs, got %d and %d", Fn::NIN, Fn::NOUT, n_in, n_out);
@@ -248,12 +248,14 @@ static int launch_ew(const Merged &m, int n_out, const agmi_array *outs, int n_i
     if (m.ndim == 1 && inner_unit) {
         const int64_t blocks = ceil_div(ceil_div(m.n, V), kBlock);
         if (int rc = check_blocks(blocks)) return rc;
+        set_kernel_name("ew_flat<%s>", fname);
         hipLaunchKernelGGL((ew_flat<F, T>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p);
     } else if (m.ndim == 2 && inner_unit) {
         const int64_t tpr = ceil_div(m.shape[1], V);
         const int64_t total = tpr * m.shape[0];
         const int64_t blocks = ceil_div(total, kBlock);
         if (int rc = check_blocks(blocks)) return rc;
+        set_kernel_name("ew_rows<%s>", fname);
         if (total < 0x7fffffffLL)
             hipLaunchKernelGGL((ew_rows<F, T, unsigned>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p,
                                (unsigned)tpr, (unsigned)total);
@@ -262,6 +264,7 @@ static int launch_ew(const Merged &m, int n_out, const agmi_array *outs, int n_i
     } else {
         const int64_t blocks = ceil_div(m.n, kBlock);
         if (int rc = check_blocks(blocks)) return rc;
+        set_kernel_name("ew_nd<%s>", fname);
         if (m.n < 0x7fffffffLL)
             hipLaunchKernelGGL((ew_nd<F, T, unsigned>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p);
         else
@@ -398,8 +401,8 @@ extern "C" int agmi_elementwise(int op, int dtype, int ndim, const int64_t *shap
     hipStream_t s = as_stream(stream);
 #define AGMI_CASE(OP, FN)                                                                    \
     case OP:                                                                                 \
-        if (dtype == AGMI_F32) return launch_ew<FN, float>(m, n_out, outs, n_in, ins, scalars, s);  \
-        if (dtype == AGMI_F64) return launch_ew<FN, double>(m, n_out, outs, n_in, ins, scalars, s); \
+        if (dtype == AGMI_F32) return launch_ew<FN, float>(#FN, m, n_out, outs, n_in, ins, scalars, s);  \
+        if (dtype == AGMI_F64) return launch_ew<FN, double>(#FN, m, n_out, outs, n_in, ins, scalars, s); \
         break;
     switch (op) {
         AGMI_FOR_EACH_OP(AGMI_CASE)
@@ -426,6 +429,7 @@ extern "C" int agmi_compare(int cmp, int dtype, int ndim, const int64_t *shape, 
     const int64_t blocks = ceil_div(m.n, kBlock);
     if (int rc = check_blocks(blocks)) return rc;
     hipStream_t s = as_stream(stream);
+    set_kernel_name("compare_nd");
     if (dtype == AGMI_F32)
         hipLaunchKernelGGL(compare_nd<float>, dim3((unsigned)blocks), dim3(kBlock), 0, s, p, cmp);
     else if (dtype == AGMI_F64)
@@ -452,6 +456,7 @@ extern "C" int agmi_cast(int src_dtype, int dst_dtype, int ndim, const int64_t *
     const int64_t blocks = ceil_div(m.n, kBlock);
     if (int rc = check_blocks(blocks)) return rc;
     hipStream_t s = as_stream(stream);
+    set_kernel_name("cast_nd");
     switch (src_dtype) {
         case AGMI_F32: return launch_cast_from<float>(dst_dtype, p, (unsigned)blocks, s);
         case AGMI_F64: return launch_cast_from<double>(dst_dtype, p, (unsigned)blocks, s);

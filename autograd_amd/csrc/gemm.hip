@@ -252,6 +252,7 @@ static int launch_gemm(GemmParams p, int64_t batch, hipStream_t s) {
     }
     p.tiles_m = static_cast<int>(tm);
     p.tiles_n = static_cast<int>(tn);
+    set_kernel_name("gemm_mfma<%s,%d,%d,%d>", sizeof(T) == 4 ? "f32" : "f64", BM, BN, BK);
     hipLaunchKernelGGL((gemm_mfma<T, BM, BN, BK>), dim3((unsigned)(tm * tn), (unsigned)batch), dim3(kBlock), 0, s, p);
     return hip_check(hipGetLastError(), "gemm launch");
 }

@@ -62,6 +62,7 @@ extern "C" int agmi_take_rows(int dtype, const void *src, int64_t n_rows, int64_
         return AGMI_ERR_UNSUPPORTED;
     }
     hipStream_t s = as_stream(stream);
+    set_kernel_name("take_rows_kernel");
     if (dtype == AGMI_F32)
         hipLaunchKernelGGL(take_rows_kernel<float>, dim3((unsigned)blocks), dim3(kBlock), 0, s,
                            static_cast<const float *>(src), n_rows, inner, index, n_index, static_cast<float *>(out));
@@ -94,6 +95,7 @@ extern "C" int agmi_scatter_add_rows(int dtype, void *dst, int64_t n_rows, int64
         return AGMI_ERR_UNSUPPORTED;
     }
     hipStream_t s = as_stream(stream);
+    set_kernel_name("scatter_add_rows_kernel");
     if (dtype == AGMI_F32)
         hipLaunchKernelGGL(scatter_add_rows_kernel<float>, dim3((unsigned)blocks), dim3(kBlock), 0, s,
                            static_cast<float *>(dst), n_rows, inner, static_cast<const float *>(src), index, order,

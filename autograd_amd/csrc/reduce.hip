@@ -334,8 +334,8 @@ static RedPlan plan_reduce(int64_t O, int64_t R, int64_t I, int vec, bool vec_ok
 }
 
 template <template <typename> class F, template <typename> class AccT, typename T>
-static int launch_reduce(const RedParams &base, bool vec_ok, void *workspace, size_t workspace_bytes,
-                         hipStream_t s) {
+static int launch_reduce(const char *fname, const RedParams &base, bool vec_ok, void *workspace,
+                         size_t workspace_bytes, hipStream_t s) {
     using Acc = AccT<T>;
     using acc_t = typename Acc::type;
     constexpr int VEC = RVec<T>::N;
@@ -354,6 +354,7 @@ static int launch_reduce(const RedParams &base, bool vec_ok, void *workspace, si
             set_error("map_reduce: too many rows");
             return AGMI_ERR_UNSUPPORTED;
         }
+        set_kernel_name("red_row_group<%s>", fname);
         hipLaunchKernelGGL((red_row_group<F, AccT, T>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p, pl.G);
     } else if (pl.row_form) {
         if (p.O > 0x7fffffffLL) {
@@ -361,6 +362,7 @@ static int launch_reduce(const RedParams &base, bool vec_ok, void *workspace, si
             return AGMI_ERR_UNSUPPORTED;
         }
         const dim3 grid((unsigned)p.O, (unsigned)pl.n_chunks);
+        set_kernel_name("red_row_block<%s>%s", fname, two_stage ? "+red_finish" : "");
 #define AGMI_ROW(VV)                                                                                          \
     do {                                                                                                      \
         if (two_stage)                                                                                        \
@@ -381,6 +383,7 @@ static int launch_reduce(const RedParams &base, bool vec_ok, void *workspace, si
         }
         const dim3 grid((unsigned)blocks_x, (unsigned)(p.O * pl.n_chunks));
         const size_t smem = (kBlock / pl.TX > 1) ? sizeof(acc_t) * kBlock * pl.V : 0;
+        set_kernel_name("red_cols<%s>%s", fname, two_stage ? "+red_finish" : "");
 #define AGMI_COL(VV)                                                                                          \
     do {                                                                                                      \
         if (two_stage)                                                                                        \
@@ -511,13 +514,13 @@ static size_t acc_size_of(int red) {
 }
 
 template <template <typename> class F, typename T>
-static int dispatch_red(int red, const RedSetup &st, void *ws, size_t ws_bytes, hipStream_t s) {
+static int dispatch_red(const char *fname, int red, const RedSetup &st, void *ws, size_t ws_bytes, hipStream_t s) {
     if (F<T>::NOUT != 1) {
         set_error("map_reduce: op has %d outputs", F<T>::NOUT);
         return AGMI_ERR_ARG;
     }
     switch (red) {
-        case AGMI_RED_SUM: return launch_reduce<F, AccSum, T>(st.p, st.vec_ok, ws, ws_bytes, s);
+        case AGMI_RED_SUM: return launch_reduce<F, AccSum, T>(fname, st.p, st.vec_ok, ws, ws_bytes, s);
         default: break;
     }
     set_error("map_reduce: reduction %d is only available with AGMI_OP_COPY", red);
@@ -527,11 +530,11 @@ static int dispatch_red(int red, const RedSetup &st, void *ws, size_t ws_bytes, 
 template <typename T>
 static int dispatch_red_copy(int red, const RedSetup &st, void *ws, size_t ws_bytes, hipStream_t s) {
     switch (red) {
-        case AGMI_RED_SUM: return launch_reduce<FCopy, AccSum, T>(st.p, st.vec_ok, ws, ws_bytes, s);
-        case AGMI_RED_MAX: return launch_reduce<FCopy, AccMax, T>(st.p, st.vec_ok, ws, ws_bytes, s);
-        case AGMI_RED_MIN: return launch_reduce<FCopy, AccMin, T>(st.p, st.vec_ok, ws, ws_bytes, s);
-        case AGMI_RED_PROD: return launch_reduce<FCopy, AccProd, T>(st.p, st.vec_ok, ws, ws_bytes, s);
-        case AGMI_RED_LOGSUMEXP: return launch_reduce<FCopy, AccLse, T>(st.p, st.vec_ok, ws, ws_bytes, s);
+        case AGMI_RED_SUM: return launch_reduce<FCopy, AccSum, T>("sum", st.p, st.vec_ok, ws, ws_bytes, s);
+        case AGMI_RED_MAX: return launch_reduce<FCopy, AccMax, T>("max", st.p, st.vec_ok, ws, ws_bytes, s);
+        case AGMI_RED_MIN: return launch_reduce<FCopy, AccMin, T>("min", st.p, st.vec_ok, ws, ws_bytes, s);
+        case AGMI_RED_PROD: return launch_reduce<FCopy, AccProd, T>("prod", st.p, st.vec_ok, ws, ws_bytes, s);
+        case AGMI_RED_LOGSUMEXP: return launch_reduce<FCopy, AccLse, T>("logsumexp", st.p, st.vec_ok, ws, ws_bytes, s);
         default: set_error("map_reduce: unknown reduction %d", red); return AGMI_ERR_ARG;
     }
 }
@@ -581,8 +584,8 @@ extern "C" int agmi_map_reduce(int op, int red, int dtype, int ndim, const int64
             set_error("map_reduce: op takes %d inputs, got %d", FN<float>::NIN, n_in);           \
             return AGMI_ERR_ARG;                                                                 \
         }                                                                                        \
-        return dtype == AGMI_F32 ? dispatch_red<FN, float>(red, st, workspace, workspace_bytes, s) \
-                                 : dispatch_red<FN, double>(red, st, workspace, workspace_bytes, s);
+        return dtype == AGMI_F32 ? dispatch_red<FN, float>(#FN, red, st, workspace, workspace_bytes, s) \
+                                 : dispatch_red<FN, double>(#FN, red, st, workspace, workspace_bytes, s);
     switch (op) {
         AGMI_FOR_EACH_REDUCE_OP(AGMI_CASE)
         default: break;

@@ -117,6 +117,9 @@ typedef enum agmi_reduce_kind {
 
 const char *agmi_last_error(void);
 int agmi_version(void);
+/* Name of the kernel the calling thread's last entry point launched, e.g. "ew_rows<FMul>"
+ * (static storage; for labelling profiles). */
+const char *agmi_last_kernel(void);
 
 /* out[k][idx] = op(in[0][idx], in[1][idx], ...) over the index space `shape` (rank `ndim`).
  * dtype is AGMI_F32 or AGMI_F64 for all operands.  An output may alias an input only when
