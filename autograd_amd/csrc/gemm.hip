@@ -24,11 +24,8 @@ namespace agmi {
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef double v4d __attribute__((ext_vector_type(4)));
 
-template <typename T>
-struct Mfma;
-
-template <>
-struct Mfma<float> {
+struct MfmaF32x32 {
+    typedef float elem_t;
     static constexpr int TM = 32;   // rows = cols of one MFMA block
     static constexpr int TK = 2;    // K depth of one instruction
     static constexpr int NACC = 16; // accumulator registers per lane
@@ -39,8 +36,22 @@ struct Mfma<float> {
     __device__ __forceinline__ static int d_row(int v, int lane) { return 8 * (v / 4) + 4 * (lane / 32) + (v % 4); }
 };
 
-template <>
-struct Mfma<double> {
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+struct MfmaF32x16 {  // 16x16x4: four independent accumulators per 32x32 wave tile instead of one chain
+    typedef float elem_t;
+    static constexpr int TM = 16;
+    static constexpr int TK = 4;
+    static constexpr int NACC = 4;
+    typedef v4f acc_t;
+    __device__ __forceinline__ static acc_t mma(float a, float b, acc_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+    }
+    __device__ __forceinline__ static int d_row(int v, int lane) { return 4 * (lane / 16) + v; }
+};
+
+struct MfmaF64x16 {
+    typedef double elem_t;
     static constexpr int TM = 16;
     static constexpr int TK = 4;
     static constexpr int NACC = 4;
@@ -68,71 +79,62 @@ constexpr int kXcds = 8;
 
 // Copy one K-slab of an operand into LDS as S[k][x] (x = m for A, n for B).
 //   xs: element stride along x, ks: element stride along k in global memory.
-// Each thread owns LOADS groups of 4 elements: contiguous along x when xs == 1, along k when
-// ks == 1 (then written transposed), and falls back to scalar loads otherwise.
-template <typename T, int BX, int BK, int LOADS>
+// MODE fixes, at compile time, how a thread's groups of 4 elements lie in global memory:
+//   kXC - 4 consecutive x at one k (xs == 1, X % 4 == 0): one 16-byte load, one 16-byte LDS store
+//   kKC - 4 consecutive k at one x (ks == 1, K % 4 == 0): one 16-byte load, stored transposed
+//   kGen - any strides / ragged extents: four 4-byte loads
+// Loads are branch-free (out-of-range groups read a clamped address and are zeroed by a select),
+// so the number of loads in flight is the same on every path and the compiler can wait for
+// exactly the slab it needs (s_waitcnt vmcnt(n)) while younger prefetches stay in flight.
+enum LoadMode { kXC = 0, kKC = 1, kGen = 2 };
+
+template <typename T, int BX, int BK, int LOADS, int MODE, int NT>
 struct SlabLoader {
     T reg[LOADS][4];
 
     __device__ __forceinline__ void load(const T *__restrict__ g, int64_t xs, int64_t ks, int64_t x0, int64_t X,
                                          int64_t k0, int64_t K, int tid) {
         typedef T vec_t __attribute__((ext_vector_type(4), aligned(sizeof(T))));
-        if (xs == 1) {  // 4 consecutive x at one k
 #pragma unroll
-            for (int i = 0; i < LOADS; ++i) {
-                const int e = tid + i * kBlock;
-                const int kk = e / (BX / 4), xx = (e % (BX / 4)) * 4;
-                const int64_t k = k0 + kk, x = x0 + xx;
-                if (k < K && x + 3 < X) {
-                    const vec_t v = *reinterpret_cast<const vec_t *>(g + k * ks + x);
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) reg[i][j] = v[j];
-                } else {
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) reg[i][j] = (k < K && x + j < X) ? g[k * ks + x + j] : T(0);
-                }
-            }
-        } else if (ks == 1) {  // 4 consecutive k at one x
-#pragma unroll
-            for (int i = 0; i < LOADS; ++i) {
-                const int e = tid + i * kBlock;
+        for (int i = 0; i < LOADS; ++i) {
+            const int e = tid + i * NT;
+            if (MODE == kKC) {
                 const int xx = e / (BK / 4), kk = (e % (BK / 4)) * 4;
                 const int64_t k = k0 + kk, x = x0 + xx;
-                if (x < X && k + 3 < K) {
-                    const vec_t v = *reinterpret_cast<const vec_t *>(g + x * xs + k);
+                const bool ok = x < X && k < K;  // K % 4 == 0: the group is all in or all out
+                const vec_t v = *reinterpret_cast<const vec_t *>(ok ? g + x * xs + k : g);
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) reg[i][j] = v[j];
-                } else {
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) reg[i][j] = (x < X && k + j < K) ? g[x * xs + k + j] : T(0);
-                }
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < LOADS; ++i) {
-                const int e = tid + i * kBlock;
+                for (int j = 0; j < 4; ++j) reg[i][j] = ok ? v[j] : T(0);
+            } else {
                 const int kk = e / (BX / 4), xx = (e % (BX / 4)) * 4;
                 const int64_t k = k0 + kk, x = x0 + xx;
+                if (MODE == kXC) {
+                    const bool ok = k < K && x < X;  // X % 4 == 0
+                    const vec_t v = *reinterpret_cast<const vec_t *>(ok ? g + k * ks + x : g);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) reg[i][j] = (k < K && x + j < X) ? g[k * ks + (x + j) * xs] : T(0);
+                    for (int j = 0; j < 4; ++j) reg[i][j] = ok ? v[j] : T(0);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const bool ok = k < K && x + j < X;
+                        const T v = *(ok ? g + k * ks + (x + j) * xs : g);
+                        reg[i][j] = ok ? v : T(0);
+                    }
+                }
             }
         }
     }
 
     template <int LDX>
-    __device__ __forceinline__ void store(T (*S)[LDX], int64_t xs, int64_t ks, int tid) const {
-        if (xs != 1 && ks == 1) {
+    __device__ __forceinline__ void store(T (*S)[LDX], int tid) const {
 #pragma unroll
-            for (int i = 0; i < LOADS; ++i) {
-                const int e = tid + i * kBlock;
+        for (int i = 0; i < LOADS; ++i) {
+            const int e = tid + i * NT;
+            if (MODE == kKC) {
                 const int xx = e / (BK / 4), kk = (e % (BK / 4)) * 4;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) S[kk + j][xx] = reg[i][j];
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < LOADS; ++i) {
-                const int e = tid + i * kBlock;
+            } else {
                 const int kk = e / (BX / 4), xx = (e % (BX / 4)) * 4;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) S[kk][xx + j] = reg[i][j];
@@ -141,19 +143,28 @@ struct SlabLoader {
     }
 };
 
-template <typename T, int BM, int BN, int BK>
-__global__ __launch_bounds__(kBlock) void gemm_mfma(const GemmParams p) {
-    using MF = Mfma<T>;
+template <class MF, int BM, int BN, int BK, int DEPTH, int MODE_A, int MODE_B, int KS>
+__global__ __launch_bounds__(kBlock *KS) void gemm_mfma(const GemmParams p) {
+    using T = typename MF::elem_t;
     constexpr int TM = MF::TM, TK = MF::TK;
     constexpr int WM = BM / 2, WN = BN / 2;      // wave tile
     constexpr int FM = WM / TM, FN = WN / TM;    // MFMA blocks per wave
-    constexpr int PAD = 4;
-    constexpr int LA = (BM * BK) / (kBlock * 4), LB = (BN * BK) / (kBlock * 4);
-    static_assert(LA >= 1 && LB >= 1, "slab too small for 256 threads");
+    // row padding of the LDS images: 16-byte rows for vector stores, or (transposed 4-byte stores)
+    // a pitch that spreads a wave's stores over all 32 banks
+    constexpr int PAD_A = MODE_A == kKC ? 2 : 4, PAD_B = MODE_B == kKC ? 2 : 4;
+    // KS groups of 4 waves share one C tile and split every K-slab between them (two waves per
+    // SIMD keep the matrix core fed while the other waits on LDS or the barrier); their partial
+    // accumulators are summed through LDS once, in group order, before the epilogue.
+    constexpr int NT = kBlock * KS;
+    constexpr int LA = (BM * BK) / (NT * 4), LB = (BN * BK) / (NT * 4);
+    static_assert(LA >= 1 && LB >= 1, "slab too small for the thread count");
+    constexpr int STEPS = BK / TK / KS;  // MFMA k-steps per wave per slab
+    static_assert(STEPS >= 1 && (BK / TK) % KS == 0, "K split");
     static_assert(WM % TM == 0 && WN % TM == 0 && BK % TK == 0 && BK % 4 == 0, "tile shape");
+    static_assert(DEPTH >= 1, "prefetch depth");
 
-    __shared__ T As[2][BK][BM + PAD];
-    __shared__ T Bs[2][BK][BN + PAD];
+    __shared__ T As[2][BK][BM + PAD_A];
+    __shared__ T Bs[2][BK][BN + PAD_B];
 
     // XCD-aware tile order
     const int n_tiles = p.tiles_m * p.tiles_n;
@@ -177,7 +188,9 @@ __global__ __launch_bounds__(kBlock) void gemm_mfma(const GemmParams p) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
+    const int kgroup = wave >> 2, quad = wave & 3;
+    const int wm0 = (quad >> 1) * WM, wn0 = (quad & 1) * WN;
+    const int ks0 = kgroup * STEPS * TK;  // this wave's first k inside a slab
     const int64_t m0 = static_cast<int64_t>(tile_m) * BM, n0 = static_cast<int64_t>(tile_n) * BN;
     const int op_x = lane % TM, op_k = lane / TM;
 
@@ -189,38 +202,81 @@ __global__ __launch_bounds__(kBlock) void gemm_mfma(const GemmParams p) {
 #pragma unroll
             for (int v = 0; v < MF::NACC; ++v) acc[i][j][v] = T(0);
 
-    SlabLoader<T, BM, BK, LA> la;
-    SlabLoader<T, BN, BK, LB> lb;
-    la.load(A, p.a_rs, p.a_cs, m0, p.M, 0, p.K, tid);
-    lb.load(B, p.b_cs, p.b_rs, n0, p.N, 0, p.K, tid);
-    la.template store<BM + PAD>(As[0], p.a_rs, p.a_cs, tid);
-    lb.template store<BN + PAD>(Bs[0], p.b_cs, p.b_rs, tid);
+    // Global loads run DEPTH slabs ahead of the matrix cores: with one 4-wave block per CU there
+    // is nothing else to hide HBM/L2 latency behind, and a slab is only ~1 us of MFMA work.
+    SlabLoader<T, BM, BK, LA, MODE_A, NT> la[DEPTH];
+    SlabLoader<T, BN, BK, LB, MODE_B, NT> lb[DEPTH];
+    const int64_t n_slabs = (p.K + BK - 1) / BK;
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+        // slabs past the end load zeros (their k range fails the bounds test), harmless and branch-free
+        la[d].load(A, p.a_rs, p.a_cs, m0, p.M, static_cast<int64_t>(d) * BK, p.K, tid);
+        lb[d].load(B, p.b_cs, p.b_rs, n0, p.N, static_cast<int64_t>(d) * BK, p.K, tid);
+    }
+    la[0].template store<BM + PAD_A>(As[0], tid);
+    lb[0].template store<BN + PAD_B>(Bs[0], tid);
     __syncthreads();
 
-    const int64_t n_slabs = (p.K + BK - 1) / BK;
-    for (int64_t t = 0; t < n_slabs; ++t) {
-        const int cur = t & 1;
-        if (t + 1 < n_slabs) {
-            la.load(A, p.a_rs, p.a_cs, m0, p.M, (t + 1) * BK, p.K, tid);
-            lb.load(B, p.b_cs, p.b_rs, n0, p.N, (t + 1) * BK, p.K, tid);
+    for (int64_t t0 = 0; t0 < n_slabs; t0 += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            const int64_t t = t0 + d;
+            if (t < n_slabs) {  // uniform across the block
+                const int cur = (DEPTH % 2 == 0) ? (d & 1) : static_cast<int>(t & 1);
+                // register slot d held slab t (already in LDS): refill it with slab t + DEPTH
+                la[d].load(A, p.a_rs, p.a_cs, m0, p.M, (t + DEPTH) * BK, p.K, tid);
+                lb[d].load(B, p.b_cs, p.b_rs, n0, p.N, (t + DEPTH) * BK, p.K, tid);
+                // all operand fragments of the slab are read from LDS first, so the MFMAs issue
+                // back to back instead of each waiting for its own LDS round trip
+                T a[STEPS][FM], b[STEPS][FN];
+#pragma unroll
+                for (int s = 0; s < STEPS; ++s) {
+#pragma unroll
+                    for (int i = 0; i < FM; ++i) a[s][i] = As[cur][ks0 + s * TK + op_k][wm0 + i * TM + op_x];
+#pragma unroll
+                    for (int j = 0; j < FN; ++j) b[s][j] = Bs[cur][ks0 + s * TK + op_k][wn0 + j * TM + op_x];
+                }
+#pragma unroll
+                for (int s = 0; s < STEPS; ++s)
+#pragma unroll
+                    for (int i = 0; i < FM; ++i)
+#pragma unroll
+                        for (int j = 0; j < FN; ++j) acc[i][j] = MF::mma(a[s][i], b[s][j], acc[i][j]);
+                if (t + 1 < n_slabs) {
+                    const int slot = (d + 1) % DEPTH;  // compile-time after unrolling
+                    la[slot].template store<BM + PAD_A>(As[cur ^ 1], tid);
+                    lb[slot].template store<BN + PAD_B>(Bs[cur ^ 1], tid);
+                }
+                __syncthreads();
+            }
         }
-#pragma unroll
-        for (int kk = 0; kk < BK; kk += TK) {
-            T a[FM], b[FN];
-#pragma unroll
-            for (int i = 0; i < FM; ++i) a[i] = As[cur][kk + op_k][wm0 + i * TM + op_x];
-#pragma unroll
-            for (int j = 0; j < FN; ++j) b[j] = Bs[cur][kk + op_k][wn0 + j * TM + op_x];
+    }
+
+    if (KS > 1) {
+        // sum the K-split partial accumulators: groups 1.. park theirs in LDS (the slab buffers are
+        // free after the last barrier), group 0 adds them in group order
+        T *scratch = &As[0][0][0];
+        static_assert(sizeof(As) + 0 >= sizeof(T) * (KS - 1) * 4 * FM * FN * MF::NACC * 64 || KS == 1, "scratch fits in As");
+        if (kgroup > 0) {
 #pragma unroll
             for (int i = 0; i < FM; ++i)
 #pragma unroll
-                for (int j = 0; j < FN; ++j) acc[i][j] = MF::mma(a[i], b[j], acc[i][j]);
-        }
-        if (t + 1 < n_slabs) {
-            la.template store<BM + PAD>(As[cur ^ 1], p.a_rs, p.a_cs, tid);
-            lb.template store<BN + PAD>(Bs[cur ^ 1], p.b_cs, p.b_rs, tid);
+                for (int j = 0; j < FN; ++j)
+#pragma unroll
+                    for (int v = 0; v < MF::NACC; ++v)
+                        scratch[((((kgroup - 1) * 4 + quad) * FM * FN + i * FN + j) * MF::NACC + v) * 64 + lane] = acc[i][j][v];
         }
         __syncthreads();
+        if (kgroup > 0) return;
+#pragma unroll
+        for (int g = 1; g < KS; ++g)
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+#pragma unroll
+                    for (int v = 0; v < MF::NACC; ++v)
+                        acc[i][j][v] += scratch[((((g - 1) * 4 + quad) * FM * FN + i * FN + j) * MF::NACC + v) * 64 + lane];
     }
 
     const T alpha = static_cast<T>(p.alpha), beta = static_cast<T>(p.beta);
@@ -243,7 +299,24 @@ __global__ __launch_bounds__(kBlock) void gemm_mfma(const GemmParams p) {
         }
 }
 
-template <typename T, int BM, int BN, int BK>
+template <class MF, int BM, int BN, int BK, int DEPTH, int KS, int MODE_A, int MODE_B>
+static void launch_modes(const GemmParams &p, dim3 grid, hipStream_t s) {
+    hipLaunchKernelGGL((gemm_mfma<MF, BM, BN, BK, DEPTH, MODE_A, MODE_B, KS>), grid, dim3(kBlock * KS), 0, s, p);
+}
+
+template <class MF, int BM, int BN, int BK, int DEPTH, int KS, int MODE_A>
+static void launch_mode_b(int mode_b, const GemmParams &p, dim3 grid, hipStream_t s) {
+    if (mode_b == kXC)
+        launch_modes<MF, BM, BN, BK, DEPTH, KS, MODE_A, kXC>(p, grid, s);
+    else if (mode_b == kKC)
+        launch_modes<MF, BM, BN, BK, DEPTH, KS, MODE_A, kKC>(p, grid, s);
+    else
+        launch_modes<MF, BM, BN, BK, DEPTH, KS, MODE_A, kGen>(p, grid, s);
+}
+
+static const char *mode_name(int m) { return m == kXC ? "x" : (m == kKC ? "k" : "g"); }
+
+template <class MF, int BM, int BN, int BK, int DEPTH, int KS = 1>
 static int launch_gemm(GemmParams p, int64_t batch, hipStream_t s) {
     const int64_t tm = ceil_div(p.M, BM), tn = ceil_div(p.N, BN);
     if (tm * tn > 0x7fffffffLL || batch > 65535) {
@@ -252,8 +325,18 @@ static int launch_gemm(GemmParams p, int64_t batch, hipStream_t s) {
     }
     p.tiles_m = static_cast<int>(tm);
     p.tiles_n = static_cast<int>(tn);
-    set_kernel_name("gemm_mfma<%s,%d,%d,%d>", sizeof(T) == 4 ? "f32" : "f64", BM, BN, BK);
-    hipLaunchKernelGGL((gemm_mfma<T, BM, BN, BK>), dim3((unsigned)(tm * tn), (unsigned)batch), dim3(kBlock), 0, s, p);
+    // how each operand's 4-element groups lie in memory (see SlabLoader)
+    const int mode_a = (p.a_rs == 1 && p.M % 4 == 0) ? kXC : ((p.a_cs == 1 && p.K % 4 == 0) ? kKC : kGen);
+    const int mode_b = (p.b_cs == 1 && p.N % 4 == 0) ? kXC : ((p.b_rs == 1 && p.K % 4 == 0) ? kKC : kGen);
+    set_kernel_name("gemm_mfma<%s,%d,%d,%d,%s%s>", sizeof(typename MF::elem_t) == 4 ? "f32" : "f64", BM, BN, BK, mode_name(mode_a),
+                    mode_name(mode_b));
+    const dim3 grid((unsigned)(tm * tn), (unsigned)batch);
+    if (mode_a == kXC)
+        launch_mode_b<MF, BM, BN, BK, DEPTH, KS, kXC>(mode_b, p, grid, s);
+    else if (mode_a == kKC)
+        launch_mode_b<MF, BM, BN, BK, DEPTH, KS, kKC>(mode_b, p, grid, s);
+    else
+        launch_mode_b<MF, BM, BN, BK, DEPTH, KS, kGen>(mode_b, p, grid, s);
     return hip_check(hipGetLastError(), "gemm launch");
 }
 
@@ -287,12 +370,14 @@ extern "C" int agmi_gemm(int dtype, int64_t batch, int64_t M, int64_t N, int64_t
     p.alpha = alpha; p.beta = beta;
     hipStream_t s = as_stream(stream);
     if (dtype == AGMI_F32) {
-        // 128x128 tiles once they alone give every CU work, 64x64 otherwise
+        // 64x64 tiles, 8 waves (two K-groups), prefetch 4 slabs: best measured on the 1024-cubed
+        // contractions of the MLP workload (one tile per CU).  128x128 tiles only once they alone
+        // give every CU two tiles (less L2 traffic per flop for large problems).
         const int64_t big_tiles = ceil_div(M, 128) * ceil_div(N, 128) * batch;
-        if (big_tiles >= 256) return launch_gemm<float, 128, 128, 16>(p, batch, s);
-        return launch_gemm<float, 64, 64, 16>(p, batch, s);
+        if (big_tiles >= 512) return launch_gemm<MfmaF32x32, 128, 128, 16, 2, 1>(p, batch, s);
+        return launch_gemm<MfmaF32x32, 64, 64, 32, 4, 2>(p, batch, s);
     }
-    if (dtype == AGMI_F64) return launch_gemm<double, 64, 64, 16>(p, batch, s);
+    if (dtype == AGMI_F64) return launch_gemm<MfmaF64x16, 64, 64, 16, 2, 1>(p, batch, s);
     set_error("gemm: dtype %d is not a floating type", dtype);
     return AGMI_ERR_ARG;
 }

@@ -15,6 +15,7 @@
 // tree over the block's 4 waves, then chunks in index order - never atomics - so results
 // are reproducible run to run.
 #include <algorithm>
+#include <type_traits>
 
 #include "common.h"
 #include "functors.h"
@@ -184,6 +185,54 @@ __global__ __launch_bounds__(kBlock) void red_row_block(const RedParams p) {
     if (threadIdx.x == 0) store_result<Acc, T, FINAL>(p, acc, o, 0, chunk);
 }
 
+// ---- logsumexp of a row chunk held in registers ------------------------------------------------
+// The generic pair accumulator costs one exp per element on a serial dependency chain.  When a
+// row chunk fits in registers (<= 256 * V * ITERS elements) each thread instead takes the plain
+// maximum of its elements and then sums exp(x - max) with independent exps, and only the
+// per-thread (max, sum) pairs go through the pair reduction: one pass over memory.
+template <typename T, int V, int ITERS, bool FINAL>
+__global__ __launch_bounds__(kBlock) void lse_row_block(const RedParams p) {
+    using Acc = AccLse<T>;
+    using vec_t = typename RVec<T>::type;
+    const int64_t o = blockIdx.x;
+    const int chunk = blockIdx.y;
+    const int64_t r_begin = static_cast<int64_t>(chunk) * p.r_chunk;
+    const int64_t r_end = min(r_begin + p.r_chunk, p.R);
+    const int64_t n = r_end - r_begin;
+    const T *row = static_cast<const T *>(p.in[0]) + o * p.istr[0][0] + r_begin * p.istr[0][1];
+    const int64_t sr = p.istr[0][1];
+    T x[ITERS][V];
+    T m = T(-INFINITY);
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+        const int64_t e0 = (static_cast<int64_t>(it) * kBlock + threadIdx.x) * V;
+        if (V > 1 && e0 + V <= n) {
+            const vec_t v = *reinterpret_cast<const vec_t *>(row + e0);
+#pragma unroll
+            for (int j = 0; j < V; ++j) x[it][j] = v[j];
+        } else {
+#pragma unroll
+            for (int j = 0; j < V; ++j) x[it][j] = (e0 + j < n) ? row[(e0 + j) * sr] : T(-INFINITY);
+        }
+#pragma unroll
+        for (int j = 0; j < V; ++j) m = max_nan(x[it][j], m);
+    }
+    T s = T(0);
+    if (m == T(INFINITY)) {
+        s = T(1);
+    } else if (m != T(-INFINITY)) {  // also taken for NaN, which then propagates through exp
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+            for (int j = 0; j < V; ++j) s += m_exp(x[it][j] - m);
+    }
+    typename Acc::type acc = {m, s};
+    acc = block_reduce<Acc>(acc);
+    if (threadIdx.x == 0) store_result<Acc, T, FINAL>(p, acc, o, 0, chunk);
+}
+
+constexpr int kLseIters = 8;
+
 // ---- row form, G lanes per row (short rows) --------------------------------------------------
 template <template <typename> class F, template <typename> class AccT, typename T>
 __global__ __launch_bounds__(kBlock) void red_row_group(const RedParams p, const int G) {
@@ -253,22 +302,36 @@ __global__ __launch_bounds__(kBlock) void red_cols(const RedParams p, const int 
     }
 }
 
-// ---- second stage: combine chunk partials in chunk order -----------------------------------------
+// ---- second stage: combine chunk partials ---------------------------------------------------------
+// block = FX x FY threads: FX consecutive outputs (coalesced reads of one chunk's partials), FY
+// strided walkers over the chunks, LDS tree over FY.  The order is fixed by (n_chunks, FY).
+constexpr int kFinishX = 32, kFinishY = kBlock / kFinishX;
+
 template <template <typename> class AccT, typename T>
 __global__ __launch_bounds__(kBlock) void red_finish(const void *partial, T *out, const int n_chunks, const int64_t O,
-                                                     const int64_t I, const int64_t ostr_o, const int64_t ostr_i,
-                                                     const int G) {
+                                                     const int64_t I, const int64_t ostr_o, const int64_t ostr_i) {
     using Acc = AccT<T>;
-    const typename Acc::type *part = static_cast<const typename Acc::type *>(partial);
-    const int per_block = kBlock / G;
-    const int64_t e = static_cast<int64_t>(blockIdx.x) * per_block + threadIdx.x / G;
-    const int lane = threadIdx.x % G;
+    using acc_t = typename Acc::type;
+    __shared__ acc_t smem[kFinishY][kFinishX];
+    const acc_t *part = static_cast<const acc_t *>(partial);
+    const int tx = threadIdx.x % kFinishX, ty = threadIdx.x / kFinishX;
+    const int64_t e = static_cast<int64_t>(blockIdx.x) * kFinishX + tx;
     const int64_t n_out = O * I;
-    typename Acc::type acc = Acc::identity();
-    if (e < n_out)
-        for (int c = lane; c < n_chunks; c += G) acc = Acc::combine(acc, part[static_cast<int64_t>(c) * n_out + e]);
-    acc = wave_reduce<Acc>(acc, G);
-    if (e < n_out && lane == 0) out[(e / I) * ostr_o + (e % I) * ostr_i] = Acc::finish(acc);
+    acc_t acc = Acc::identity();
+    if (e < n_out) {
+#pragma unroll 4
+        for (int c = ty; c < n_chunks; c += kFinishY) acc = Acc::combine(acc, part[static_cast<int64_t>(c) * n_out + e]);
+    }
+    smem[ty][tx] = acc;
+    __syncthreads();
+    for (int half = kFinishY >> 1; half > 0; half >>= 1) {
+        if (ty < half) {
+            acc = Acc::combine(acc, smem[ty + half][tx]);
+            smem[ty][tx] = acc;
+        }
+        __syncthreads();
+    }
+    if (ty == 0 && e < n_out) out[(e / I) * ostr_o + (e % I) * ostr_i] = Acc::finish(acc);
 }
 
 // ---- planning ------------------------------------------------------------------------------------
@@ -291,7 +354,7 @@ static int pow2_ceil(int64_t v) {
 // enough blocks to give each of the 256 CUs several
 constexpr int64_t kTargetBlocks = 2048;
 
-static RedPlan plan_reduce(int64_t O, int64_t R, int64_t I, int vec, bool vec_ok, size_t acc_size,
+static RedPlan plan_reduce(int64_t O, int64_t R, int64_t I, int vec, bool vec_ok, size_t acc_size, size_t elem_size,
                            size_t workspace_bytes) {
     RedPlan pl = {};
     pl.n_chunks = 1;
@@ -318,7 +381,10 @@ static RedPlan plan_reduce(int64_t O, int64_t R, int64_t I, int vec, bool vec_ok
     } else {
         pl.row_form = false;
         pl.V = (vec_ok && I % vec == 0) ? vec : 1;
-        pl.TX = std::min<int>(kBlock, pow2_ceil(ceil_div(I, pl.V)));
+        // a thread-row covers ~256 contiguous bytes of one row of the operands; the rest of the
+        // block's threads walk different rows, so many blocks fit across I and few chunks are needed
+        const int tx_full = std::max<int>(1, 256 / (pl.V * static_cast<int>(elem_size)));
+        pl.TX = std::min<int>(tx_full, pow2_ceil(ceil_div(I, pl.V)));
         const int TY = kBlock / pl.TX;
         const int64_t blocks_x = ceil_div(ceil_div(I, pl.V), pl.TX);
         int64_t chunks = std::min<int64_t>(ceil_div(kTargetBlocks, blocks_x * O), ceil_div(R, static_cast<int64_t>(TY) * 8));
@@ -329,7 +395,6 @@ static RedPlan plan_reduce(int64_t O, int64_t R, int64_t I, int vec, bool vec_ok
             pl.n_chunks = static_cast<int>(ceil_div(R, pl.r_chunk));
         }
     }
-    if (pl.n_chunks > 1) pl.G = (O * I <= 4096) ? 64 : 1;
     return pl;
 }
 
@@ -339,7 +404,7 @@ static int launch_reduce(const char *fname, const RedParams &base, bool vec_ok, 
     using Acc = AccT<T>;
     using acc_t = typename Acc::type;
     constexpr int VEC = RVec<T>::N;
-    const RedPlan pl = plan_reduce(base.O, base.R, base.I, VEC, vec_ok, sizeof(acc_t), workspace ? workspace_bytes : 0);
+    const RedPlan pl = plan_reduce(base.O, base.R, base.I, VEC, vec_ok, sizeof(acc_t), sizeof(T), workspace ? workspace_bytes : 0);
     RedParams p = base;
     p.n_chunks = pl.n_chunks;
     p.r_chunk = pl.r_chunk;
@@ -362,6 +427,35 @@ static int launch_reduce(const char *fname, const RedParams &base, bool vec_ok, 
             return AGMI_ERR_UNSUPPORTED;
         }
         const dim3 grid((unsigned)p.O, (unsigned)pl.n_chunks);
+        if constexpr (std::is_same<AccT<T>, AccLse<T>>::value && std::is_same<F<T>, FCopy<T>>::value) {
+            const bool unit = p.istr[0][1] == 1 || p.r_chunk == 1;
+            const int v = (pl.V > 1 && unit) ? VEC : 1;
+            if (!(p.scalar_mask & 1u) && p.r_chunk <= static_cast<int64_t>(kBlock) * v * kLseIters) {
+                set_kernel_name("lse_row_block%s", two_stage ? "+red_finish" : "");
+                const int64_t need = ceil_div(p.r_chunk, static_cast<int64_t>(kBlock) * v);
+#define AGMI_LSE(VV, IT)                                                                                   \
+    do {                                                                                                   \
+        if (two_stage)                                                                                     \
+            hipLaunchKernelGGL((lse_row_block<T, VV, IT, false>), grid, dim3(kBlock), 0, s, p);            \
+        else                                                                                               \
+            hipLaunchKernelGGL((lse_row_block<T, VV, IT, true>), grid, dim3(kBlock), 0, s, p);             \
+    } while (0)
+#define AGMI_LSE_IT(VV)                      \
+    do {                                     \
+        if (need <= 1) AGMI_LSE(VV, 1);      \
+        else if (need <= 2) AGMI_LSE(VV, 2); \
+        else if (need <= 4) AGMI_LSE(VV, 4); \
+        else AGMI_LSE(VV, kLseIters);        \
+    } while (0)
+                if (v > 1)
+                    AGMI_LSE_IT(VEC);
+                else
+                    AGMI_LSE_IT(1);
+#undef AGMI_LSE_IT
+#undef AGMI_LSE
+                goto launched;
+            }
+        }
         set_kernel_name("red_row_block<%s>%s", fname, two_stage ? "+red_finish" : "");
 #define AGMI_ROW(VV)                                                                                          \
     do {                                                                                                      \
@@ -397,12 +491,12 @@ static int launch_reduce(const char *fname, const RedParams &base, bool vec_ok, 
             AGMI_COL(1);
 #undef AGMI_COL
     }
+launched:
     if (int rc = hip_check(hipGetLastError(), "map_reduce launch")) return rc;
     if (two_stage) {
-        const int per_block = kBlock / pl.G;
-        const int64_t blocks = ceil_div(p.O * p.I, per_block);
+        const int64_t blocks = ceil_div(p.O * p.I, kFinishX);
         hipLaunchKernelGGL((red_finish<AccT, T>), dim3((unsigned)blocks), dim3(kBlock), 0, s, workspace,
-                           static_cast<T *>(final_out), pl.n_chunks, p.O, p.I, p.ostr_o, p.ostr_i, pl.G);
+                           static_cast<T *>(final_out), pl.n_chunks, p.O, p.I, p.ostr_o, p.ostr_i);
         if (int rc = hip_check(hipGetLastError(), "map_reduce finish launch")) return rc;
     }
     return 0;

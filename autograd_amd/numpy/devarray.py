@@ -28,13 +28,16 @@ _I64 = onp.dtype("int64")
 class DevArray:
     """n-d array in GPU memory; arithmetic is hand-written HIP kernels."""
 
-    __slots__ = ("_t", "dtype")
+    __slots__ = ("_t", "dtype", "_borrowed")
     __array_ufunc__ = None  # NumPy binary operators defer to ours (ndarray * DevArray -> __rmul__)
     __array_priority__ = 200.0
 
     def __init__(self, tensor, dtype=None):
         self._t = tensor
         self.dtype = dtype if dtype is not None else _lib.NUMPY_DTYPE[tensor.dtype]
+        # True on an accumulator that shares its memory with a cotangent it was initialised from
+        # (0 + g kept as g): in-place accumulation must then go to fresh memory instead
+        self._borrowed = False
 
     # ---- metadata ----------------------------------------------------------------------
     @property

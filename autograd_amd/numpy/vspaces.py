@@ -15,6 +15,32 @@ from . import devarray as D
 from .devarray import DevArray
 
 
+_ZEROS = {}
+
+
+def _shared_zero(dtype):
+    z = _ZEROS.get(dtype)
+    if z is None:
+        z = _ZEROS[dtype] = D.zeros((), dtype)
+    return z
+
+
+def is_broadcast_view(x):
+    """True when some axis of extent > 1 has stride 0: several indices share one element."""
+    t = x._t
+    if t.numel() <= 1:
+        return False
+    for extent, stride in zip(t.shape, t.stride()):
+        if stride == 0 and extent > 1:
+            return True
+    return False
+
+
+def is_shared_zero(x):
+    z = _ZEROS.get(x.dtype)
+    return z is not None and x._t.data_ptr() == z._t.data_ptr()
+
+
 class DevArrayVSpace(VSpace):
     def __init__(self, value):
         if isinstance(value, DevArray):
@@ -34,7 +60,14 @@ class DevArrayVSpace(VSpace):
         return len(self.shape)
 
     def zeros(self):
-        return D.zeros(self.shape, self.dtype)
+        """A zero cotangent.  Accumulators start from it (core.py:212-215, 238-241 of the
+        reference: ``vs.zeros()`` then ``+=``), so it is returned as a stride-0 view of one shared
+        zero: creating it writes nothing, and the first ``x_prev + x_new`` reads it from a
+        register instead of streaming a zero-filled buffer.  It is never written in place:
+        ``_mut_add`` and the scatter rule allocate the real buffer when they meet it."""
+        if self.size <= 1:
+            return D.zeros(self.shape, self.dtype)
+        return DevArray(_shared_zero(self.dtype)._t.expand(self.shape), self.dtype)
 
     def ones(self):
         return D.ones(self.shape, self.dtype)
@@ -54,7 +87,19 @@ class DevArrayVSpace(VSpace):
         return D.map_op(Op.ADD, D._float_dtype(D.result_dtype(x, y)), x, y)
 
     def _mut_add(self, x, y):
+        """``x += y`` for an accumulator ``x`` (reference core.py:262-264).
+
+        ``zeros() + y`` is ``y``: instead of streaming ``y`` through an add with zero, the
+        accumulator borrows ``y``'s memory and is marked ``_borrowed``; the next contribution
+        then goes out of place (same traffic as an in-place add), so the borrowed array - which
+        may also be a tape value or another node's cotangent - is never written."""
         if not isinstance(x, DevArray):
+            return self._add(x, y)
+        if is_shared_zero(x) and isinstance(y, DevArray) and y.shape == x.shape and y.dtype == x.dtype:
+            acc = DevArray(y._t, y.dtype)
+            acc._borrowed = True
+            return acc
+        if x._borrowed or is_broadcast_view(x):
             return self._add(x, y)
         if isinstance(y, DevArray) and y.shape != x.shape and onp.broadcast_shapes(x.shape, y.shape) != x.shape:
             return self._add(x, y)

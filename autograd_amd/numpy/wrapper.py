@@ -508,9 +508,16 @@ def scatter_add(A, idx, x):
     addend).  Integer array on axis 0: the ordered scatter kernel, which adds repeated
     destinations sequentially in index order like ``numpy.add.at``.
     """
+    from .vspaces import is_broadcast_view, is_shared_zero
+
+    fresh_zero = False
+    if A._borrowed or is_broadcast_view(A):  # not this accumulator's own memory yet: allocate it
+        fresh_zero = is_shared_zero(A)
+        A = D.zeros(A.shape, A.dtype) if fresh_zero else D.copy(A)
     if _is_basic_index(idx):
         view = DevArray(A._t[_plain(idx)], A.dtype)
-        D.map_op(Op.ADD, A.dtype, view, x, out=view)
+        # into fresh zeros the sum is 0 + x: no need to read the destination back
+        D.map_op(Op.ADD, A.dtype, 0.0 if fresh_zero else view, x, out=view)
         return A
     rows = _host_index(idx)
     if rows is None:
