@@ -34,6 +34,9 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing")
     ap.add_argument("--no-extras", action="store_true", help="skip the other workloads")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget for the CPU baseline sample")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch plain copies of a (8192,4096) f32 array (134.2 MB read + 134.2 MB written "
+                         "each): the reference dispatch that hardware traffic counters are scaled by")
     return ap.parse_args()
 
 
@@ -81,6 +84,22 @@ def cpu_baseline(seconds):
         "ms_per_eval_min": best * 1e3,
         "ms_per_eval_median": float(onp.median(times)) * 1e3,
     }
+
+
+def measured_traffic(kernel):
+    """HBM bytes per launch of ``kernel`` from the committed rocprofv3 counter summary
+    (profiles/bcast_grad_hbm_traffic.md: FETCH_SIZE + WRITE_SIZE scaled by a plain copy), or None."""
+    path = os.path.join(ROOT, "profiles", "bcast_grad_hbm_traffic.md")
+    family, _, functor = kernel.partition("<")
+    functor = functor.split(">")[0]
+    try:
+        for line in open(path):
+            cells = [c.strip() for c in line.split("|")]
+            if len(cells) > 8 and family in cells[1] and (not functor or functor in cells[1]):
+                return float(cells[7]) * 1e6
+    except (OSError, ValueError):
+        pass
+    return None
 
 
 def main():
@@ -146,7 +165,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": None,
+            "traffic": measured_traffic(dominant),
             "algorithmic_bytes_per_launch": dom["avg_bytes"],
             "avg_launch_ms": dom["avg_ms"],
             "launches_timed": dom["launches"],
@@ -158,6 +177,13 @@ def main():
         },
     }
 
+    if args.calibrate_copy:
+        from autograd_amd._lib import Op
+        from autograd_amd.numpy import devarray as D
+
+        for _ in range(5):
+            D.map_op(Op.COPY, A.dtype, A)
+        be.sync()
     if not args.no_extras:
         result["extras"] = extras(be)
     if not args.no_cpu_baseline:
