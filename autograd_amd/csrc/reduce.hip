@@ -303,31 +303,33 @@ __global__ __launch_bounds__(kBlock) void red_cols(const RedParams p, const int 
 }
 
 // ---- second stage: combine chunk partials ---------------------------------------------------------
-// block = FX x FY threads: FX consecutive outputs (coalesced reads of one chunk's partials), FY
-// strided walkers over the chunks, LDS tree over FY.  The order is fixed by (n_chunks, FY).
-constexpr int kFinishX = 32, kFinishY = kBlock / kFinishX;
-
+// block = FX x FY threads (FX * FY = 256): FX consecutive outputs (coalesced reads of one chunk's
+// partials), FY strided walkers over the chunks, LDS tree over FY.  FX shrinks with the number of
+// outputs so that a full reduction (one output) still uses all 256 threads.  The order of
+// combination is fixed by (n_chunks, FY).
 template <template <typename> class AccT, typename T>
 __global__ __launch_bounds__(kBlock) void red_finish(const void *partial, T *out, const int n_chunks, const int64_t O,
-                                                     const int64_t I, const int64_t ostr_o, const int64_t ostr_i) {
+                                                     const int64_t I, const int64_t ostr_o, const int64_t ostr_i,
+                                                     const int FX) {
     using Acc = AccT<T>;
     using acc_t = typename Acc::type;
-    __shared__ acc_t smem[kFinishY][kFinishX];
+    __shared__ acc_t smem[kBlock];
     const acc_t *part = static_cast<const acc_t *>(partial);
-    const int tx = threadIdx.x % kFinishX, ty = threadIdx.x / kFinishX;
-    const int64_t e = static_cast<int64_t>(blockIdx.x) * kFinishX + tx;
+    const int FY = kBlock / FX;
+    const int tx = threadIdx.x % FX, ty = threadIdx.x / FX;
+    const int64_t e = static_cast<int64_t>(blockIdx.x) * FX + tx;
     const int64_t n_out = O * I;
     acc_t acc = Acc::identity();
     if (e < n_out) {
 #pragma unroll 4
-        for (int c = ty; c < n_chunks; c += kFinishY) acc = Acc::combine(acc, part[static_cast<int64_t>(c) * n_out + e]);
+        for (int c = ty; c < n_chunks; c += FY) acc = Acc::combine(acc, part[static_cast<int64_t>(c) * n_out + e]);
     }
-    smem[ty][tx] = acc;
+    smem[ty * FX + tx] = acc;
     __syncthreads();
-    for (int half = kFinishY >> 1; half > 0; half >>= 1) {
+    for (int half = FY >> 1; half > 0; half >>= 1) {
         if (ty < half) {
-            acc = Acc::combine(acc, smem[ty + half][tx]);
-            smem[ty][tx] = acc;
+            acc = Acc::combine(acc, smem[(ty + half) * FX + tx]);
+            smem[ty * FX + tx] = acc;
         }
         __syncthreads();
     }
@@ -366,7 +368,7 @@ static RedPlan plan_reduce(int64_t O, int64_t R, int64_t I, int vec, bool vec_ok
         if (R > 1024 || (R > 64 && O < 64)) {
             pl.block_per_row = true;
             pl.V = vec_ok ? vec : 1;
-            const int64_t per_block_min = static_cast<int64_t>(kBlock) * pl.V * 4;  // >= 4 vectors per thread
+            const int64_t per_block_min = static_cast<int64_t>(kBlock) * pl.V * 16;  // >= 16 vectors per thread
             int64_t chunks = std::min<int64_t>(ceil_div(kTargetBlocks, O), ceil_div(R, per_block_min));
             chunks = std::min<int64_t>(chunks, std::min<int64_t>(max_chunks_ws, 65535));
             if (chunks > 1) {
@@ -494,9 +496,10 @@ static int launch_reduce(const char *fname, const RedParams &base, bool vec_ok, 
 launched:
     if (int rc = hip_check(hipGetLastError(), "map_reduce launch")) return rc;
     if (two_stage) {
-        const int64_t blocks = ceil_div(p.O * p.I, kFinishX);
+        const int fx = static_cast<int>(std::min<int64_t>(32, pow2_ceil(p.O * p.I)));
+        const int64_t blocks = ceil_div(p.O * p.I, fx);
         hipLaunchKernelGGL((red_finish<AccT, T>), dim3((unsigned)blocks), dim3(kBlock), 0, s, workspace,
-                           static_cast<T *>(final_out), pl.n_chunks, p.O, p.I, p.ostr_o, p.ostr_i);
+                           static_cast<T *>(final_out), pl.n_chunks, p.O, p.I, p.ostr_o, p.ostr_i, fx);
         if (int rc = hip_check(hipGetLastError(), "map_reduce finish launch")) return rc;
     }
     return 0;

@@ -510,14 +510,24 @@ def scatter_add(A, idx, x):
     """
     from .vspaces import is_broadcast_view, is_shared_zero
 
-    fresh_zero = False
+    basic = _is_basic_index(idx)
     if A._borrowed or is_broadcast_view(A):  # not this accumulator's own memory yet: allocate it
-        fresh_zero = is_shared_zero(A)
-        A = D.zeros(A.shape, A.dtype) if fresh_zero else D.copy(A)
-    if _is_basic_index(idx):
+        if is_shared_zero(A):
+            if basic:
+                # into zeros the sum is 0 + x, so the destination is never read back; and when the
+                # view covers every element (b[None, :], c[:, None], full slices) the zero fill
+                # is skipped as well
+                probe = A._t[_plain(idx)]
+                full_cover = probe.numel() == A._t.numel() and probe.dim() >= A._t.dim()
+                A = D.empty(A.shape, A.dtype) if full_cover else D.zeros(A.shape, A.dtype)
+                D.map_op(Op.ADD, A.dtype, 0.0, x, out=DevArray(A._t[_plain(idx)], A.dtype))
+                return A
+            A = D.zeros(A.shape, A.dtype)
+        else:
+            A = D.copy(A)
+    if basic:
         view = DevArray(A._t[_plain(idx)], A.dtype)
-        # into fresh zeros the sum is 0 + x: no need to read the destination back
-        D.map_op(Op.ADD, A.dtype, 0.0 if fresh_zero else view, x, out=view)
+        D.map_op(Op.ADD, A.dtype, view, x, out=view)
         return A
     rows = _host_index(idx)
     if rows is None:
