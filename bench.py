@@ -34,6 +34,9 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing")
     ap.add_argument("--no-extras", action="store_true", help="skip the other workloads")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget for the CPU baseline sample")
+    ap.add_argument("--workload", default="bcast", choices=["bcast", "tanh", "mlp", "rnn", "rosen"],
+                    help="bcast (default) is the headline workload, BASELINE configs[1]; the others are the "
+                         "remaining BASELINE configs, selectable for profiling")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch plain copies of a (8192,4096) f32 array (134.2 MB read + 134.2 MB written "
                          "each): the reference dispatch that hardware traffic counters are scaled by")
@@ -86,6 +89,48 @@ def cpu_baseline(seconds):
     }
 
 
+def make_workload(name, be):
+    """(step function, config description, arithmetic dtype) for one BASELINE workload; inputs are
+    uploaded here, before any timing."""
+    from autograd_amd import configs
+
+    if name == "bcast":
+        inp = configs.bcast_inputs()
+        A, b, c = be.put(inp["A"]), be.put(inp["b"]), be.put(inp["c"])
+        g = configs.bcast_program(be)["grad"]
+        cfg = {"workload": "configs[1] broadcast+reduction VJPs: grad wrt (A,b,c) of "
+                           "sum(logsumexp(A*b[None,:]+c[:,None],axis=1))",
+               "A": [8192, 4096], "b": [4096], "c": [8192], "seed": 0}
+        return (lambda: g(A, b, c)), cfg, "f32"
+    if name == "tanh":
+        x = be.put(configs.tanh_inputs()["x"])
+        prog = configs.tanh_program(be)
+        cfg = {"workload": "configs[0] elementwise tanh: egrad, egrad^2 and egrad^3 of (1-exp(-2x))/(1+exp(-2x)); "
+                           "one step = the three calls", "x": [4194304]}
+        return (lambda: (prog["d1"](x), prog["d2"](x), prog["d3"](x))), cfg, "f64"
+    if name == "mlp":
+        inp = configs.mlp_inputs()
+        params = configs.tree_map(be.put, inp["params"])
+        X, T = be.put(inp["X"]), be.put(inp["T"])
+        g = configs.mlp_program(be)["grad"]
+        cfg = {"workload": "configs[2] MLP 784-1024-1024-10 tanh, log-softmax loss, grad wrt [(W,b)]",
+               "batch": 1024, "seed": 0}
+        return (lambda: g(params, X, T)), cfg, "f32"
+    if name == "rnn":
+        inp = configs.rnn_inputs()
+        params = configs.tree_map(be.put, inp["params"])
+        xs, ts = be.put(inp["inputs"]), be.put(inp["targets"])
+        g = configs.rnn_program(be)["grad"]
+        cfg = {"workload": "configs[3] tanh RNN T=64 B=256 H=512, grad wrt params dict", "seed": 0}
+        return (lambda: g(params, xs, ts)), cfg, "f32"
+    inp = configs.rosen_inputs()
+    x, v = be.put(inp["x"]), be.put(inp["v"])
+    prog = configs.rosen_program(be)
+    cfg = {"workload": "configs[4] Rosenbrock HVP n=2^24: one step = make_hvp(f)(x)[0](v) and make_jvp(grad(f))(x)(v)",
+           "seed": 0}
+    return (lambda: (prog["hvp_rev"](x, v), prog["hvp_fwd"](x, v))), cfg, "f64"
+
+
 def measured_traffic(kernel):
     """HBM bytes per launch of ``kernel`` from the committed rocprofv3 counter summary
     (profiles/bcast_grad_hbm_traffic.md: FETCH_SIZE + WRITE_SIZE scaled by a plain copy), or None."""
@@ -112,12 +157,7 @@ def main():
     from autograd_amd import _lib, configs
 
     be = configs.device_backend()
-    inp = configs.bcast_inputs()
-    A, b, c = be.put(inp["A"]), be.put(inp["b"]), be.put(inp["c"])
-    grad_fn = configs.bcast_program(be)["grad"]
-
-    def step():
-        return grad_fn(A, b, c)
+    step, config, dtype = make_workload(args.workload, be)
 
     # warm-up, with every launch timed once to find the kernel that dominates the step
     for _ in range(max(1, args.warmup)):
@@ -139,7 +179,19 @@ def main():
         elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
     dom = kt.summary()[dominant]
-    achieved = dom["avg_bytes"] / (dom["avg_ms"] * 1e-3) / 1e9
+    if dominant.startswith("gemm_mfma"):
+        achieved = dom["avg_flops"] / (dom["avg_ms"] * 1e-3) / 1e12
+        roofline = {"bound": "mfma", "kernel": dominant, "achieved": achieved, "peak": MFMA_F32_PEAK_TFLOPS,
+                    "unit": "TFLOP/s", "frac": achieved / MFMA_F32_PEAK_TFLOPS, "traffic": None,
+                    "algorithmic_flops_per_launch": dom["avg_flops"]}
+    else:
+        achieved = dom["avg_bytes"] / (dom["avg_ms"] * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": achieved / HBM_PEAK_GBS,
+                    "traffic": measured_traffic(dominant) if args.workload == "bcast" else None,
+                    "algorithmic_bytes_per_launch": dom["avg_bytes"]}
+    roofline["avg_launch_ms"] = dom["avg_ms"]
+    roofline["launches_timed"] = dom["launches"]
 
     result = {
         "metric": "grad evals/sec",
@@ -152,24 +204,10 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": dtype,
         "data": "synthetic",
-        "config": {
-            "workload": "configs[1] broadcast+reduction VJPs: grad wrt (A,b,c) of sum(logsumexp(A*b[None,:]+c[:,None],axis=1))",
-            "A": [8192, 4096], "b": [4096], "c": [8192], "seed": 0,
-        },
-        "roofline": {
-            "bound": "hbm",
-            "kernel": dominant,
-            "achieved": achieved,
-            "peak": HBM_PEAK_GBS,
-            "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS,
-            "traffic": measured_traffic(dominant),
-            "algorithmic_bytes_per_launch": dom["avg_bytes"],
-            "avg_launch_ms": dom["avg_ms"],
-            "launches_timed": dom["launches"],
-        },
+        "config": config,
+        "roofline": roofline,
         "kernels_per_step": {
             name: {"launches": r["launches"], "avg_ms": round(r["avg_ms"], 5),
                    "GB/s": round(r["avg_bytes"] / (r["avg_ms"] * 1e-3) / 1e9, 1) if r["avg_ms"] > 0 else None}
@@ -178,13 +216,16 @@ def main():
     }
 
     if args.calibrate_copy:
+        import numpy as onp
+
         from autograd_amd._lib import Op
         from autograd_amd.numpy import devarray as D
 
+        ref = D.zeros((8192, 4096), onp.float32)
         for _ in range(5):
-            D.map_op(Op.COPY, A.dtype, A)
+            D.map_op(Op.COPY, ref.dtype, ref)
         be.sync()
-    if not args.no_extras:
+    if not args.no_extras and args.workload == "bcast":
         result["extras"] = extras(be)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.cpu_seconds)
