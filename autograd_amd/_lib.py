@@ -265,17 +265,17 @@ _mask = (ctypes.c_uint8 * MAX_DIMS)()
 
 def _set_array(slot, t):
     slot.data = t.data_ptr()
-    st = slot.strides
-    for d, s in enumerate(t.stride()):
-        st[d] = s
+    st = t.stride()
+    if st:
+        slot.strides[: len(st)] = st
 
 
 def _set_shape(shape):
     n = len(shape)
     if n > MAX_DIMS:
         raise AgmiError(f"rank {n} arrays are not supported (max {MAX_DIMS})")
-    for d, s in enumerate(shape):
-        _shape[d] = s
+    if n:
+        _shape[:n] = shape
     return n
 
 

@@ -247,6 +247,25 @@ def _operand(x, dtype):
     return asarray(x, dtype)._t
 
 
+def broadcast_shapes(a, b):
+    """NumPy broadcasting of two shape tuples (plain tuple arithmetic: this sits on the launch path)."""
+    if a == b:
+        return a
+    if len(a) < len(b):
+        a, b = b, a
+    pad = len(a) - len(b)
+    out = list(a)
+    for i, sb in enumerate(b):
+        sa = a[pad + i]
+        if sa == sb or sb == 1:
+            continue
+        if sa == 1:
+            out[pad + i] = sb
+        else:
+            raise ValueError(f"operands could not be broadcast together with shapes {a} {b}")
+    return tuple(out)
+
+
 def _bshape(operands):
     shape = None
     for t in operands:
@@ -255,7 +274,7 @@ def _bshape(operands):
             if shape is None:
                 shape = s
             elif s != shape:
-                shape = tuple(onp.broadcast_shapes(shape, s))
+                shape = broadcast_shapes(shape, s)
     return shape
 
 

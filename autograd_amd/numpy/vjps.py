@@ -77,7 +77,7 @@ def _fused_unbroadcast(op, target_meta, *operands):
     for x in operands:
         s = _shape_of(x)
         if s != shape:
-            shape = tuple(onp.broadcast_shapes(shape, s))
+            shape = D.broadcast_shapes(shape, s)
     if shape == tuple(target_shape):
         return D.map_op(op, dt, *operands)
     lead = len(shape) - target_ndim

@@ -53,7 +53,10 @@ class DevArrayVSpace(VSpace):
 
     @property
     def size(self):
-        return int(onp.prod(self.shape))
+        n = 1
+        for s in self.shape:
+            n *= s
+        return n
 
     @property
     def ndim(self):
@@ -101,7 +104,7 @@ class DevArrayVSpace(VSpace):
             return acc
         if x._borrowed or is_broadcast_view(x):
             return self._add(x, y)
-        if isinstance(y, DevArray) and y.shape != x.shape and onp.broadcast_shapes(x.shape, y.shape) != x.shape:
+        if isinstance(y, DevArray) and y.shape != x.shape and D.broadcast_shapes(x.shape, y.shape) != x.shape:
             return self._add(x, y)
         return D.map_op(Op.ADD, x.dtype, x, y, out=x)
 

@@ -602,7 +602,7 @@ def _matmul_raw(a, b):
         ta = ta.unsqueeze(0)
     if b_vec:
         tb = tb.unsqueeze(1)
-    batch = tuple(onp.broadcast_shapes(tuple(ta.shape[:-2]), tuple(tb.shape[:-2])))
+    batch = D.broadcast_shapes(tuple(ta.shape[:-2]), tuple(tb.shape[:-2]))
     ta = ta.expand(batch + tuple(ta.shape[-2:]))
     tb = tb.expand(batch + tuple(tb.shape[-2:]))
     M, K = ta.shape[-2:]
