@@ -129,7 +129,7 @@ def lib():
     L.agmi_map_reduce_workspace_bytes.argtypes = [c_i, c_i, c_i, p_i64, p_u8]
     L.agmi_gemm.restype = c_i
     L.agmi_gemm.argtypes = [c_i, c_i64, c_i64, c_i64, c_i64, c_d, c_p, c_i64, c_i64, c_i64, c_p, c_i64, c_i64,
-                            c_i64, c_d, c_p, c_i64, c_i64, c_p]
+                            c_i64, c_d, c_p, c_i64, c_i64, c_p, c_sz, c_p]
     L.agmi_fill.restype = c_i
     L.agmi_fill.argtypes = [c_i, c_p, c_i64, c_d, c_p]
     L.agmi_take_rows.restype = c_i
@@ -360,7 +360,7 @@ def map_reduce(op, red, code, shape, reduce_mask, out, ins):
 def gemm(code, batch, M, N, K, alpha, A, a_rs, a_cs, a_bs, B, b_rs, b_cs, b_bs, beta, C, ldc, c_bs):
     ev = _TIMER.begin(("gemm",)) if _TIMER is not None else None
     rc = _LIB.agmi_gemm(code, batch, M, N, K, alpha, A.data_ptr(), a_rs, a_cs, a_bs, B.data_ptr(), b_rs, b_cs, b_bs,
-                        beta, C.data_ptr(), ldc, c_bs, _stream())
+                        beta, C.data_ptr(), ldc, c_bs, _workspace().data_ptr(), _WORKSPACE_BYTES, _stream())
     if rc:
         _check(rc, "agmi_gemm")
     if ev is not None:

@@ -49,6 +49,14 @@ struct Merged {
 bool merge_axes(int ndim, const int64_t *shape, const uint8_t *group, int n_operands,
                 const int64_t *const *strides, Merged *out);
 
+// true when some extent is 0 (valid rank and shape pointer assumed checked elsewhere)
+inline bool index_space_is_empty(int ndim, const int64_t *shape) {
+    if (ndim <= 0 || ndim > AGMI_MAX_DIMS || shape == nullptr) return false;
+    for (int d = 0; d < ndim; ++d)
+        if (shape[d] == 0) return true;
+    return false;
+}
+
 inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }

@@ -386,6 +386,7 @@ extern "C" int agmi_elementwise(int op, int dtype, int ndim, const int64_t *shap
         set_error("elementwise: bad operand counts or null operand arrays");
         return AGMI_ERR_ARG;
     }
+    if (index_space_is_empty(ndim, shape)) return 0;  // nothing to compute; empty arrays have null data
     const int64_t *strides[kMaxOperands];
     for (int k = 0; k < n_out; ++k) {
         if (outs[k].data == nullptr) {
@@ -415,6 +416,7 @@ extern "C" int agmi_elementwise(int op, int dtype, int ndim, const int64_t *shap
 
 extern "C" int agmi_compare(int cmp, int dtype, int ndim, const int64_t *shape, const agmi_array *out,
                             const agmi_array *ins, const double *scalars, void *stream) {
+    if (index_space_is_empty(ndim, shape)) return 0;
     if (!out || !ins || !out->data || cmp < AGMI_EQ || cmp > AGMI_GE) {
         set_error("compare: bad arguments");
         return AGMI_ERR_ARG;
@@ -443,6 +445,7 @@ extern "C" int agmi_compare(int cmp, int dtype, int ndim, const int64_t *shape, 
 
 extern "C" int agmi_cast(int src_dtype, int dst_dtype, int ndim, const int64_t *shape, const agmi_array *out,
                          const agmi_array *in, void *stream) {
+    if (index_space_is_empty(ndim, shape)) return 0;
     if (!out || !in || !out->data || !in->data) {
         set_error("cast: null operand");
         return AGMI_ERR_ARG;

@@ -17,6 +17,8 @@
 // Workgroup ids are dealt round-robin to the 8 XCDs (each with its own L2), so the tile
 // order is remapped: XCD x works on a contiguous range of tiles, walked in column-major
 // groups of kGroupM tile-rows, which keeps one XCD's A rows and B columns resident in its L2.
+#include <algorithm>
+
 #include "common.h"
 
 namespace agmi {
@@ -72,6 +74,11 @@ struct GemmParams {
     int64_t ldc, c_bs;
     double alpha, beta;
     int tiles_m, tiles_n;
+    // cross-block K split (blockIdx.z): split z covers k in [z * k_per_split, min(K, (z+1) * k_per_split))
+    // and writes its raw partial tile to ws[(z * batch + b) * M * N + row * N + col]
+    int splits;
+    int64_t k_per_split;
+    void *ws;
 };
 
 constexpr int kGroupM = 8;
@@ -163,8 +170,13 @@ __global__ __launch_bounds__(kBlock *KS) void gemm_mfma(const GemmParams p) {
     static_assert(WM % TM == 0 && WN % TM == 0 && BK % TK == 0 && BK % 4 == 0, "tile shape");
     static_assert(DEPTH >= 1, "prefetch depth");
 
-    __shared__ T As[2][BK][BM + PAD_A];
-    __shared__ T Bs[2][BK][BN + PAD_B];
+    // one LDS allocation: the two double-buffered slab images, reused as scratch by the K-group sum
+    constexpr int kAsElems = 2 * BK * (BM + PAD_A), kBsElems = 2 * BK * (BN + PAD_B);
+    constexpr int kScratchElems = (KS - 1) * 4 * FM * FN * MF::NACC * 64;
+    constexpr int kLdsElems = (kAsElems + kBsElems) > kScratchElems ? (kAsElems + kBsElems) : kScratchElems;
+    __shared__ T lds[kLdsElems];
+    T(*As)[BK][BM + PAD_A] = reinterpret_cast<T(*)[BK][BM + PAD_A]>(lds);
+    T(*Bs)[BK][BN + PAD_B] = reinterpret_cast<T(*)[BK][BN + PAD_B]>(lds + kAsElems);
 
     // XCD-aware tile order
     const int n_tiles = p.tiles_m * p.tiles_n;
@@ -206,12 +218,14 @@ __global__ __launch_bounds__(kBlock *KS) void gemm_mfma(const GemmParams p) {
     // is nothing else to hide HBM/L2 latency behind, and a slab is only ~1 us of MFMA work.
     SlabLoader<T, BM, BK, LA, MODE_A, NT> la[DEPTH];
     SlabLoader<T, BN, BK, LB, MODE_B, NT> lb[DEPTH];
-    const int64_t n_slabs = (p.K + BK - 1) / BK;
+    const int64_t k_first = static_cast<int64_t>(blockIdx.z) * p.k_per_split;   // multiple of BK
+    const int64_t k_limit = min(p.K, k_first + p.k_per_split);
+    const int64_t n_slabs = (k_limit - k_first + BK - 1) / BK;
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
         // slabs past the end load zeros (their k range fails the bounds test), harmless and branch-free
-        la[d].load(A, p.a_rs, p.a_cs, m0, p.M, static_cast<int64_t>(d) * BK, p.K, tid);
-        lb[d].load(B, p.b_cs, p.b_rs, n0, p.N, static_cast<int64_t>(d) * BK, p.K, tid);
+        la[d].load(A, p.a_rs, p.a_cs, m0, p.M, k_first + static_cast<int64_t>(d) * BK, k_limit, tid);
+        lb[d].load(B, p.b_cs, p.b_rs, n0, p.N, k_first + static_cast<int64_t>(d) * BK, k_limit, tid);
     }
     la[0].template store<BM + PAD_A>(As[0], tid);
     lb[0].template store<BN + PAD_B>(Bs[0], tid);
@@ -224,8 +238,8 @@ __global__ __launch_bounds__(kBlock *KS) void gemm_mfma(const GemmParams p) {
             if (t < n_slabs) {  // uniform across the block
                 const int cur = (DEPTH % 2 == 0) ? (d & 1) : static_cast<int>(t & 1);
                 // register slot d held slab t (already in LDS): refill it with slab t + DEPTH
-                la[d].load(A, p.a_rs, p.a_cs, m0, p.M, (t + DEPTH) * BK, p.K, tid);
-                lb[d].load(B, p.b_cs, p.b_rs, n0, p.N, (t + DEPTH) * BK, p.K, tid);
+                la[d].load(A, p.a_rs, p.a_cs, m0, p.M, k_first + (t + DEPTH) * BK, k_limit, tid);
+                lb[d].load(B, p.b_cs, p.b_rs, n0, p.N, k_first + (t + DEPTH) * BK, k_limit, tid);
                 // all operand fragments of the slab are read from LDS first, so the MFMAs issue
                 // back to back instead of each waiting for its own LDS round trip
                 T a[STEPS][FM], b[STEPS][FN];
@@ -255,8 +269,7 @@ __global__ __launch_bounds__(kBlock *KS) void gemm_mfma(const GemmParams p) {
     if (KS > 1) {
         // sum the K-split partial accumulators: groups 1.. park theirs in LDS (the slab buffers are
         // free after the last barrier), group 0 adds them in group order
-        T *scratch = &As[0][0][0];
-        static_assert(sizeof(As) + 0 >= sizeof(T) * (KS - 1) * 4 * FM * FN * MF::NACC * 64 || KS == 1, "scratch fits in As");
+        T *scratch = lds;
         if (kgroup > 0) {
 #pragma unroll
             for (int i = 0; i < FM; ++i)
@@ -279,6 +292,22 @@ __global__ __launch_bounds__(kBlock *KS) void gemm_mfma(const GemmParams p) {
                         acc[i][j][v] += scratch[((((g - 1) * 4 + quad) * FM * FN + i * FN + j) * MF::NACC + v) * 64 + lane];
     }
 
+    if (p.splits > 1) {  // raw partial tile; gemm_split_finish applies alpha / beta
+        T *W = static_cast<T *>(p.ws) + (static_cast<int64_t>(blockIdx.z) * gridDim.y + batch) * p.M * p.N;
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j) {
+                const int64_t col = n0 + wn0 + j * TM + op_x;
+#pragma unroll
+                for (int v = 0; v < MF::NACC; ++v) {
+                    const int64_t row = m0 + wm0 + i * TM + MF::d_row(v, lane);
+                    if (row < p.M && col < p.N) W[row * p.N + col] = acc[i][j][v];
+                }
+            }
+        return;
+    }
+
     const T alpha = static_cast<T>(p.alpha), beta = static_cast<T>(p.beta);
 #pragma unroll
     for (int i = 0; i < FM; ++i)
@@ -299,6 +328,45 @@ __global__ __launch_bounds__(kBlock *KS) void gemm_mfma(const GemmParams p) {
         }
 }
 
+// C = alpha * (sum over splits, in split order) + beta * C
+template <typename T>
+__global__ __launch_bounds__(kBlock) void gemm_split_finish(const T *__restrict__ ws, T *__restrict__ C, int splits,
+                                                            int64_t batch, int64_t M, int64_t N, int64_t ldc, int64_t c_bs,
+                                                            T alpha, T beta) {
+    const int64_t e = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    const int64_t per = M * N;
+    if (e >= batch * per) return;
+    const int64_t b = e / per, r = (e - b * per) / N, c = e - b * per - r * N;
+    T acc = ws[e];
+    for (int s = 1; s < splits; ++s) acc += ws[static_cast<int64_t>(s) * batch * per + e];
+    T *dst = C + b * c_bs + r * ldc + c;
+    T v = alpha * acc;
+    if (beta != T(0)) v = v + beta * *dst;
+    *dst = v;
+}
+
+// K == 0: the product is empty, C = beta * C.  Handled apart because the tile kernel's branch-free
+// loads read the operand base address for out-of-range elements, and empty operands have none.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void gemm_empty_k(T *__restrict__ C, int64_t batch, int64_t M, int64_t N, int64_t ldc,
+                                                       int64_t c_bs, T beta) {
+    const int64_t e = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    const int64_t per = M * N;
+    if (e >= batch * per) return;
+    const int64_t b = e / per, r = (e - b * per) / N, c = e - b * per - r * N;
+    T *dst = C + b * c_bs + r * ldc + c;
+    *dst = beta != T(0) ? beta * *dst : T(0);
+}
+
+template <typename T>
+static int launch_empty_k(const GemmParams &p, int64_t batch, hipStream_t s) {
+    const int64_t n = batch * p.M * p.N;
+    set_kernel_name("gemm_empty_k");
+    hipLaunchKernelGGL(gemm_empty_k<T>, dim3((unsigned)ceil_div(n, kBlock)), dim3(kBlock), 0, s, static_cast<T *>(p.C), batch,
+                       p.M, p.N, p.ldc, p.c_bs, static_cast<T>(p.beta));
+    return hip_check(hipGetLastError(), "gemm launch");
+}
+
 template <class MF, int BM, int BN, int BK, int DEPTH, int KS, int MODE_A, int MODE_B>
 static void launch_modes(const GemmParams &p, dim3 grid, hipStream_t s) {
     hipLaunchKernelGGL((gemm_mfma<MF, BM, BN, BK, DEPTH, MODE_A, MODE_B, KS>), grid, dim3(kBlock * KS), 0, s, p);
@@ -317,7 +385,8 @@ static void launch_mode_b(int mode_b, const GemmParams &p, dim3 grid, hipStream_
 static const char *mode_name(int m) { return m == kXC ? "x" : (m == kKC ? "k" : "g"); }
 
 template <class MF, int BM, int BN, int BK, int DEPTH, int KS = 1>
-static int launch_gemm(GemmParams p, int64_t batch, hipStream_t s) {
+static int launch_gemm(GemmParams p, int64_t batch, hipStream_t s, void *ws = nullptr, size_t ws_bytes = 0) {
+    using T = typename MF::elem_t;
     const int64_t tm = ceil_div(p.M, BM), tn = ceil_div(p.N, BN);
     if (tm * tn > 0x7fffffffLL || batch > 65535) {
         set_error("gemm: problem too large for one launch");
@@ -330,13 +399,38 @@ static int launch_gemm(GemmParams p, int64_t batch, hipStream_t s) {
     const int mode_b = (p.b_cs == 1 && p.N % 4 == 0) ? kXC : ((p.b_rs == 1 && p.K % 4 == 0) ? kKC : kGen);
     set_kernel_name("gemm_mfma<%s,%d,%d,%d,%s%s>", sizeof(typename MF::elem_t) == 4 ? "f32" : "f64", BM, BN, BK, mode_name(mode_a),
                     mode_name(mode_b));
-    const dim3 grid((unsigned)(tm * tn), (unsigned)batch);
+    // Few tiles but a long K (skinny outputs, small batches of a recurrent net): cut K across blocks so
+    // the machine fills up; partial tiles go to the workspace and are summed in split order.
+    p.splits = 1;
+    p.k_per_split = ceil_div(p.K, BK) * BK;
+    const int64_t tiles = tm * tn * batch;
+    if (ws != nullptr && tiles < 128 && p.K >= 8 * BK) {
+        int64_t splits = std::min<int64_t>(ceil_div(256, tiles), p.K / (4 * BK));
+        splits = std::min<int64_t>(splits, static_cast<int64_t>(ws_bytes / (sizeof(T) * (size_t)(batch * p.M * p.N))));
+        splits = std::min<int64_t>(splits, 64);
+        if (splits > 1) {
+            p.k_per_split = ceil_div(ceil_div(p.K, splits), BK) * BK;
+            p.splits = static_cast<int>(ceil_div(p.K, p.k_per_split));
+            p.ws = ws;
+        }
+    }
+    const dim3 grid((unsigned)(tm * tn), (unsigned)batch, (unsigned)p.splits);
+    if (p.splits > 1)
+        set_kernel_name("gemm_mfma<%s,%d,%d,%d,%s%s>+split%d", sizeof(T) == 4 ? "f32" : "f64", BM, BN, BK,
+                        mode_name(mode_a), mode_name(mode_b), p.splits);
     if (mode_a == kXC)
         launch_mode_b<MF, BM, BN, BK, DEPTH, KS, kXC>(mode_b, p, grid, s);
     else if (mode_a == kKC)
         launch_mode_b<MF, BM, BN, BK, DEPTH, KS, kKC>(mode_b, p, grid, s);
     else
         launch_mode_b<MF, BM, BN, BK, DEPTH, KS, kGen>(mode_b, p, grid, s);
+    if (int rc = hip_check(hipGetLastError(), "gemm launch")) return rc;
+    if (p.splits > 1) {
+        const int64_t n = batch * p.M * p.N;
+        hipLaunchKernelGGL(gemm_split_finish<T>, dim3((unsigned)ceil_div(n, kBlock)), dim3(kBlock), 0, s,
+                           static_cast<const T *>(p.ws), static_cast<T *>(p.C), p.splits, batch, p.M, p.N, p.ldc,
+                           p.c_bs, static_cast<T>(p.alpha), static_cast<T>(p.beta));
+    }
     return hip_check(hipGetLastError(), "gemm launch");
 }
 
@@ -347,7 +441,8 @@ using namespace agmi;
 extern "C" int agmi_gemm(int dtype, int64_t batch, int64_t M, int64_t N, int64_t K, double alpha,
                          const void *A, int64_t a_rs, int64_t a_cs, int64_t a_bs,
                          const void *B, int64_t b_rs, int64_t b_cs, int64_t b_bs,
-                         double beta, void *C, int64_t ldc, int64_t c_bs, void *stream) {
+                         double beta, void *C, int64_t ldc, int64_t c_bs, void *workspace,
+                         size_t workspace_bytes, void *stream) {
     if (M < 0 || N < 0 || K < 0 || batch < 0) {
         set_error("gemm: negative extent");
         return AGMI_ERR_ARG;
@@ -369,15 +464,25 @@ extern "C" int agmi_gemm(int dtype, int64_t batch, int64_t M, int64_t N, int64_t
     p.ldc = ldc; p.c_bs = c_bs;
     p.alpha = alpha; p.beta = beta;
     hipStream_t s = as_stream(stream);
+    if (batch * M * N > 0x7fffffffLL * kBlock) {
+        set_error("gemm: output too large for one launch");
+        return AGMI_ERR_UNSUPPORTED;
+    }
+    if (K == 0) {
+        if (dtype == AGMI_F32) return launch_empty_k<float>(p, batch, s);
+        if (dtype == AGMI_F64) return launch_empty_k<double>(p, batch, s);
+        set_error("gemm: dtype %d is not a floating type", dtype);
+        return AGMI_ERR_ARG;
+    }
     if (dtype == AGMI_F32) {
         // 64x64 tiles, 8 waves (two K-groups), prefetch 4 slabs: best measured on the 1024-cubed
         // contractions of the MLP workload (one tile per CU).  128x128 tiles only once they alone
         // give every CU two tiles (less L2 traffic per flop for large problems).
         const int64_t big_tiles = ceil_div(M, 128) * ceil_div(N, 128) * batch;
         if (big_tiles >= 512) return launch_gemm<MfmaF32x32, 128, 128, 16, 2, 1>(p, batch, s);
-        return launch_gemm<MfmaF32x32, 64, 64, 32, 4, 2>(p, batch, s);
+        return launch_gemm<MfmaF32x32, 64, 64, 32, 4, 2>(p, batch, s, workspace, workspace_bytes);
     }
-    if (dtype == AGMI_F64) return launch_gemm<MfmaF64x16, 64, 64, 16, 2, 1>(p, batch, s);
+    if (dtype == AGMI_F64) return launch_gemm<MfmaF64x16, 64, 64, 16, 2, 1>(p, batch, s, workspace, workspace_bytes);
     set_error("gemm: dtype %d is not a floating type", dtype);
     return AGMI_ERR_ARG;
 }

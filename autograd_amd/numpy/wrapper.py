@@ -112,23 +112,27 @@ def where(condition, x, y):
     return _where3(condition, x, y)
 
 
+def _truth(a):
+    """Operand for a logical op: 1.0 / 0.0 array (or Python float) from any array or scalar."""
+    from ..tracer import getval
+
+    a = getval(a)
+    if isinstance(a, DevArray):
+        return D.astype(D.compare(Cmp.NE, a, 0.0) if a.dtype != D._BOOL else a, onp.float64)
+    return 1.0 if a else 0.0
+
+
 def logical_and(a, b):
-    return _wrap_bool(D.map_op(Op.MUL, onp.dtype("float64"), _truth(a), _truth(b)))
+    """Non-differentiable (numpy_vjps.py:13-68); used by the ``clip`` rule."""
+    return D.compare(Cmp.NE, D.map_op(Op.MUL, onp.dtype("float64"), _truth(a), _truth(b)), 0.0)
+
+
+def logical_or(a, b):
+    return D.compare(Cmp.NE, D.map_op(Op.ADD, onp.dtype("float64"), _truth(a), _truth(b)), 0.0)
 
 
 def logical_not(a):
     return D.compare(Cmp.EQ, _truth(a), 0.0)
-
-
-def _truth(a):
-    from ..tracer import getval
-
-    a = getval(a)
-    return D.astype(D.compare(Cmp.NE, a, 0.0), onp.float64) if isinstance(a, DevArray) else (1.0 if a else 0.0)
-
-
-def _wrap_bool(x):
-    return D.compare(Cmp.NE, x, 0.0)
 
 
 # ---- astype / copies --------------------------------------------------------------------------

@@ -161,13 +161,16 @@ size_t agmi_map_reduce_workspace_bytes(int red, int dtype, int ndim, const int64
  * AGMI_F32 or AGMI_F64.  A and B are addressed as A[m*a_rs + k*a_cs], B[k*b_rs + n*b_cs], so
  * the transposed operands of the adjoints need no copy; C is row-major with leading
  * dimension ldc.  `batch` independent products with element strides *_bs (batch >= 1).
+ * `workspace` (device memory, may be NULL) lets problems with few output tiles and a long K be
+ * cut across workgroups along K; partial tiles are then summed in a fixed order (deterministic).
  * Replaces: numpy.dot forward (numpy_wrapper.py:39-40), onp.tensordot in dot_adjoint_0/1
  * (numpy_vjps.py:615-638: G.B^T and A^T.G), matmul adjoints (567-612), tensordot_adjoint_0/1
  * (666-719) after axis permutation. */
 int agmi_gemm(int dtype, int64_t batch, int64_t M, int64_t N, int64_t K, double alpha,
               const void *A, int64_t a_rs, int64_t a_cs, int64_t a_bs,
               const void *B, int64_t b_rs, int64_t b_cs, int64_t b_bs,
-              double beta, void *C, int64_t ldc, int64_t c_bs, void *stream);
+              double beta, void *C, int64_t ldc, int64_t c_bs,
+              void *workspace, size_t workspace_bytes, void *stream);
 
 /* ptr[0..n) = value (vspace zeros/ones, numpy_vspaces.py:21-25; sparse_add's zero fill,
  * core.py:212-215). */

@@ -365,3 +365,66 @@ def test_vspace_axioms(dnp):
     assert onp.array_equal(acc.numpy(), a.numpy())
     assert onp.array_equal(acc3.numpy(), ((0.0 + a.numpy()) + b.numpy()) + b.numpy())
     assert vspace(dnp.ones((2,), dtype=F32)).dtype == onp.float32
+
+
+# ---- edge cases: empty, single-element and ragged extents, special values ------------------------
+def test_empty_and_degenerate_shapes(dnp):
+    for shape in [(0,), (0, 5), (5, 0), (3, 0, 2)]:
+        x = onp.zeros(shape, F32)
+        X = P(dnp, x)
+        assert (X + 1.0).shape == shape and dnp.exp(X).shape == shape
+        assert onp.array_equal(dnp.sum(X).numpy(), onp.sum(x))
+        assert dnp.sum(X, axis=0).shape == onp.sum(x, axis=0).shape
+        assert onp.array_equal(dnp.sum(X, axis=-1).numpy(), onp.sum(x, axis=-1))
+        assert dnp.reshape(X, (-1,)).shape == (0,)
+    a, b = onp.ones((0, 4), F32), onp.ones((4, 3), F32)
+    assert onp.array_equal(dnp.dot(P(dnp, a), P(dnp, b)).numpy(), a @ b)
+    a, b = onp.ones((2, 0), F32), onp.ones((0, 3), F32)
+    assert onp.array_equal(dnp.dot(P(dnp, a), P(dnp, b)).numpy(), a @ b)  # K = 0: zeros
+    assert onp.array_equal(dnp.concatenate((P(dnp, onp.ones((0, 3))), P(dnp, onp.ones((2, 3)))), axis=0).numpy(), onp.ones((2, 3)))
+    s = P(dnp, onp.float64(3.0))
+    assert (s * s).shape == () and float(s * s) == 9.0 and float(dnp.sum(s)) == 3.0
+
+
+@pytest.mark.parametrize("n", [1, 3, 4, 5, 255, 256, 257, 1023, 1025, 4099])
+def test_ragged_lengths_every_vector_tail(dnp, n):
+    rs = onp.random.RandomState(n)
+    for dtype in (F32, F64):
+        x, y = rs.randn(n).astype(dtype), rs.randn(n).astype(dtype)
+        assert onp.array_equal((P(dnp, x) * P(dnp, y)).numpy(), x * y)
+        assert onp.array_equal((P(dnp, x)[1:] + 2.0).numpy(), x[1:] + dtype(2.0))
+        close(dnp.sum(P(dnp, x)).numpy(), onp.sum(x), RT[dtype])
+        m = rs.randn(7, n).astype(dtype)
+        assert onp.array_equal((P(dnp, m) - P(dnp, y)).numpy(), m - y)
+        close(dnp.sum(P(dnp, m), axis=0).numpy(), m.sum(axis=0), RT[dtype])
+        close(dnp.sum(P(dnp, m), axis=1).numpy(), m.sum(axis=1), RT[dtype])
+        assert onp.array_equal(dnp.max(P(dnp, m), axis=1).numpy(), m.max(axis=1))
+
+
+def test_special_values_propagate_like_numpy(dnp):
+    x = onp.array([0.0, -0.0, onp.inf, -onp.inf, onp.nan, 1.0, -1.0])
+    X = P(dnp, x)
+    with onp.errstate(all="ignore"):
+        for name in ("exp", "tanh", "negative", "abs", "square", "sign"):
+            got, want = getattr(dnp, name)(X).numpy(), getattr(onp, name)(x)
+            assert onp.array_equal(got, want, equal_nan=True), name
+        assert onp.array_equal(dnp.maximum(X, 0.5).numpy(), onp.maximum(x, 0.5), equal_nan=True)
+        assert onp.array_equal(dnp.minimum(X, X[::1] * 0.0).numpy(), onp.minimum(x, x * 0.0), equal_nan=True)
+        assert onp.isnan(dnp.max(X).numpy()) and onp.isnan(dnp.sum(X).numpy())
+        assert dnp.max(X[:4]).numpy() == onp.inf and dnp.min(X[:4]).numpy() == -onp.inf
+        assert onp.array_equal((X / 0.0).numpy(), x / 0.0, equal_nan=True)
+    assert onp.array_equal(dnp.logical_and(X[5:] > 0, X[5:] < 2).numpy(), [True, False])
+    assert onp.array_equal(dnp.logical_or(X[5:] > 0, X[5:] < 0).numpy(), [True, True])
+    assert onp.array_equal(dnp.logical_not(X[5:] > 0).numpy(), [False, True])
+
+
+def test_rank_limits_are_reported(dnp):
+    from autograd_amd._lib import AgmiError
+
+    x = P(dnp, onp.zeros((2,) * 8, F32))
+    assert (x + 1.0).shape == (2,) * 8                      # rank 8 merges to one axis
+    y = dnp.transpose(x)                                    # fully reversed: 8 unmergeable axes
+    with pytest.raises(AgmiError, match="axes remain after merging"):
+        y + x
+    with pytest.raises(AgmiError):
+        P(dnp, onp.zeros((1,) * 9, F32)) + 1.0

@@ -1,0 +1,102 @@
+"""Host-side logic of the device layer that needs no GPU: shape/axis/dtype planning.
+
+``DevArray`` only needs a tensor for its metadata, so CPU tensors stand in here; nothing is
+launched (any launch would raise: there is no CPU fallback).
+"""
+
+import numpy as onp
+import pytest
+import torch
+
+from autograd_amd.numpy import devarray as D
+from autograd_amd.numpy import wrapper as W
+from autograd_amd.numpy.devarray import DevArray
+
+
+def meta(shape, dtype=torch.float32):
+    return DevArray(torch.empty(shape, dtype=dtype))
+
+
+def test_broadcast_shapes_matches_numpy():
+    cases = [((), ()), ((3,), ()), ((3, 4), (4,)), ((3, 1), (1, 4)), ((2, 1, 5), (7, 1)), ((0, 4), (1, 4)), ((5,), (5,))]
+    for a, b in cases:
+        assert D.broadcast_shapes(a, b) == onp.broadcast_shapes(a, b)
+        assert D.broadcast_shapes(b, a) == onp.broadcast_shapes(a, b)
+    with pytest.raises(ValueError):
+        D.broadcast_shapes((3, 4), (3,))
+
+
+def test_result_dtype_follows_numpy2_promotion():
+    f32, f64, i64 = meta((2,)), meta((2,), torch.float64), meta((2,), torch.int64)
+    assert D.result_dtype(f32, 2.0) == onp.float32            # weak Python scalar
+    assert D.result_dtype(f32, 3) == onp.float32
+    assert D.result_dtype(f32, onp.float64(2.0)) == onp.float64  # strong NumPy scalar
+    assert D.result_dtype(f32, onp.int64(3)) == onp.float64      # the mean-rule promotion of the reference
+    assert D.result_dtype(f32, f64) == onp.float64
+    assert D.result_dtype(f32, i64) == onp.float64
+    assert D.result_dtype(f32, f32, 1.5) == onp.float32
+    assert D.result_dtype(i64, 2.0) == onp.float64
+    for args in [(onp.float32(1), 2.0), (onp.ones(2, onp.float32), onp.int64(3)), (onp.ones(2, onp.float32), 2)]:
+        ours = D.result_dtype(*[meta((2,)) if isinstance(a, onp.ndarray) else a for a in args])
+        assert ours == onp.result_type(*args)
+
+
+def test_normalize_axes_and_reduce_shape():
+    assert D.normalize_axes(None, 3) == (0, 1, 2)
+    assert D.normalize_axes(-1, 3) == (2,)
+    assert D.normalize_axes((2, 0), 3) == (0, 2)
+    assert D.normalize_axes(None, 0) == ()
+    with pytest.raises(ValueError):
+        D.normalize_axes(3, 3)
+    assert D.reduce_shape((2, 3, 4), (1,), False) == (2, 4)
+    assert D.reduce_shape((2, 3, 4), (0, 2), True) == (1, 3, 1)
+    assert D._adjacent_groups((0, 1, 3)) == [(0, 1), (3,)]
+
+
+def test_reshape_shape_normalisation():
+    assert W._norm_shape((-1, 4), 12) == (3, 4)
+    assert W._norm_shape(12, 12) == (12,)
+    assert W._norm_shape((), 1) == ()
+    for bad in [((5,), 12), ((-1, -1), 12), ((-1, 5), 12)]:
+        with pytest.raises(ValueError):
+            W._norm_shape(*bad)
+
+
+def test_index_classification():
+    assert W._is_basic_index((slice(1, None), None, 3, Ellipsis))
+    assert W._is_basic_index(onp.int64(2))
+    assert not W._is_basic_index([0, 1])
+    assert not W._is_basic_index((slice(None), onp.array([0, 1])))
+    with pytest.raises(NotImplementedError):
+        W._is_basic_index(slice(None, None, -1))
+    assert onp.array_equal(W._host_index([0, 2, 0]), [0, 2, 0])
+    assert onp.array_equal(W._host_index(onp.array([True, False, True])), [0, 2])
+    assert W._host_index([]).dtype == onp.int64 and W._host_index([]).size == 0
+    assert W._host_index([slice(0, 1)]) is None
+    assert W._host_index(onp.ones((2, 2), int)) is None
+
+
+def test_views_are_metadata_only():
+    x = meta((4, 6))
+    assert W.transpose(x).shape == (6, 4) and W.transpose(x)._t.data_ptr() == x._t.data_ptr()
+    assert W.reshape(x, (2, 12)).shape == (2, 12)
+    assert W.expand_dims(x, (0, 3)).shape == (1, 4, 6, 1)
+    assert W.squeeze(W.expand_dims(x, 1)).shape == (4, 6)
+    assert W.broadcast_to(meta((1, 6)), (5, 6))._t.stride() == (0, 1)
+    assert W.swapaxes(x, 0, 1).shape == (6, 4)
+    assert W.atleast_2d(meta((3,))).shape == (1, 3) and W.atleast_1d(meta(())).shape == (1,)
+    assert x[1:, ::2].shape == (3, 3) and x[None, 2].shape == (1, 6)
+    assert W.shape(x) == (4, 6) and W.ndim(x) == 2 and W.size(x) == 24 and W.result_type(x) == onp.float32
+    with pytest.raises(TypeError):
+        x[0] = 1.0
+
+
+def test_vspace_metadata_and_laziness():
+    from autograd_amd.extend import vspace
+    from autograd_amd.numpy.vspaces import DevArrayVSpace
+
+    vs = vspace(meta((3, 4)))
+    assert isinstance(vs, DevArrayVSpace) and vs.shape == (3, 4) and vs.size == 12 and vs.ndim == 2
+    assert vs == vspace(meta((3, 4))) and vs != vspace(meta((3, 4), torch.float64))
+    fs = vspace(1.5)
+    assert fs.shape == () and fs.dtype == onp.float64 and fs.size == 1

@@ -71,7 +71,7 @@ def test_argument_errors_are_reported_without_a_gpu(lib):
     rc = lib.agmi_gemm(0, ctypes.c_int64(1), ctypes.c_int64(-1), ctypes.c_int64(1), ctypes.c_int64(1),
                        ctypes.c_double(1.0), None, ctypes.c_int64(0), ctypes.c_int64(0), ctypes.c_int64(0), None,
                        ctypes.c_int64(0), ctypes.c_int64(0), ctypes.c_int64(0), ctypes.c_double(0.0), None,
-                       ctypes.c_int64(1), ctypes.c_int64(0), None)
+                       ctypes.c_int64(1), ctypes.c_int64(0), None, ctypes.c_size_t(0), None)
     assert rc == -1
 
 
