@@ -85,7 +85,17 @@ REDUCE_FUSABLE = frozenset(
 
 
 class AgmiArray(ctypes.Structure):
-    _fields_ = [("data", ctypes.c_void_p), ("strides", ctypes.c_int64 * MAX_DIMS)]
+    _fields_ = [("data", ctypes.c_void_p), ("strides", ctypes.c_int64 * MAX_DIMS), ("scale", ctypes.c_double),
+                ("shift", ctypes.c_double), ("affine", ctypes.c_uint32)]
+
+
+class Affine:
+    """Kernel input slot ``t * scale + shift`` (``shift`` None: no add), applied on load."""
+
+    __slots__ = ("t", "scale", "shift")
+
+    def __init__(self, t, scale, shift):
+        self.t, self.scale, self.shift = t, scale, shift
 
 
 class AgmiError(RuntimeError):
@@ -250,6 +260,8 @@ def _traffic(outs, ins):
     for t in outs:
         total += t.numel() * t.element_size()
     for t in ins:
+        if type(t) is Affine:
+            t = t.t
         if isinstance(t, torch.Tensor):
             total += _distinct_bytes(t)
     return total
@@ -281,10 +293,22 @@ def _set_shape(shape):
 
 def _set_inputs(ins):
     for k, x in enumerate(ins):
+        slot = _ins[k]
         if isinstance(x, torch.Tensor):
-            _set_array(_ins[k], x)
+            _set_array(slot, x)
+            slot.affine = 0
+        elif type(x) is Affine:
+            _set_array(slot, x.t)
+            flags = 0
+            if x.scale != 1.0:
+                slot.scale = x.scale
+                flags = 1
+            if x.shift is not None:
+                slot.shift = x.shift
+                flags |= 2
+            slot.affine = flags
         else:
-            _ins[k].data = None
+            slot.data = None
             _scalars[k] = x
     return len(ins)
 
@@ -318,6 +342,7 @@ def cast(src_code, dst_code, shape, out, src):
     nd = _set_shape(shape)
     _set_array(_outs[0], out)
     _set_array(_ins[0], src)
+    _ins[0].affine = 0
     _check(_LIB.agmi_cast(src_code, dst_code, nd, _shape, _outs, _ins, _stream()), "agmi_cast")
 
 

@@ -20,13 +20,28 @@ struct EwParams {
     void *out[AGMI_MAX_OUTPUTS];
     const void *in[AGMI_MAX_INPUTS];
     double scalar[AGMI_MAX_INPUTS];
+    double scale[AGMI_MAX_INPUTS];  // pending affine map of an input: value = mem * scale + shift
+    double shift[AGMI_MAX_INPUTS];
     unsigned scalar_mask;
+    unsigned scale_mask, shift_mask;
     int ndim;
     int64_t n;
     int64_t shape[kMaxMerged];
     int64_t ostr[AGMI_MAX_OUTPUTS][kMaxMerged];
     int64_t istr[AGMI_MAX_INPUTS][kMaxMerged];
 };
+
+// Apply the inputs' pending affine maps to one gathered point: multiply, then add, each rounded
+// on its own (the masks are wave-uniform, so plain operands pay one scalar branch).
+template <typename T, int NIN, class P>
+__device__ __forceinline__ void apply_affine(const P &p, T *xi) {
+    if ((p.scale_mask | p.shift_mask) == 0) return;
+#pragma unroll
+    for (int k = 0; k < NIN; ++k) {
+        if (p.scale_mask & (1u << k)) xi[k] = xi[k] * static_cast<T>(p.scale[k]);
+        if (p.shift_mask & (1u << k)) xi[k] = xi[k] + static_cast<T>(p.shift[k]);
+    }
+}
 
 template <typename T>
 struct Vec {
@@ -68,6 +83,7 @@ __global__ __launch_bounds__(kBlock) void ew_flat(const EwParams p) {
             T xi[Fn::NIN], oi[Fn::NOUT];
 #pragma unroll
             for (int k = 0; k < Fn::NIN; ++k) xi[k] = x[k][j];
+            apply_affine<T, Fn::NIN>(p, xi);
             Fn::apply(xi, oi);
 #pragma unroll
             for (int k = 0; k < Fn::NOUT; ++k) o[k][j] = oi[k];
@@ -89,6 +105,7 @@ __global__ __launch_bounds__(kBlock) void ew_flat(const EwParams p) {
                 else
                     xi[k] = static_cast<const T *>(p.in[k])[p.istr[k][0] == 0 ? 0 : i];
             }
+            apply_affine<T, Fn::NIN>(p, xi);
             Fn::apply(xi, oi);
 #pragma unroll
             for (int k = 0; k < Fn::NOUT; ++k) static_cast<T *>(p.out[k])[i] = oi[k];
@@ -139,6 +156,7 @@ __global__ __launch_bounds__(kBlock) void ew_rows(const EwParams p, const Index 
         T xi[Fn::NIN], oi[Fn::NOUT];
 #pragma unroll
         for (int k = 0; k < Fn::NIN; ++k) xi[k] = x[k][j];
+        apply_affine<T, Fn::NIN>(p, xi);
         Fn::apply(xi, oi);
 #pragma unroll
         for (int k = 0; k < Fn::NOUT; ++k) o[k][j] = oi[k];
@@ -185,6 +203,7 @@ __global__ __launch_bounds__(kBlock) void ew_nd(const EwParams p) {
 #pragma unroll
     for (int k = 0; k < Fn::NIN; ++k)
         xi[k] = (p.scalar_mask & (1u << k)) ? static_cast<T>(p.scalar[k]) : static_cast<const T *>(p.in[k])[ioff[k]];
+    apply_affine<T, Fn::NIN>(p, xi);
     Fn::apply(xi, oi);
 #pragma unroll
     for (int k = 0; k < Fn::NOUT; ++k) static_cast<T *>(p.out[k])[ooff[k]] = oi[k];
@@ -234,6 +253,15 @@ static int launch_ew(const char *fname, const Merged &m, int n_out, const agmi_a
             }
             p.scalar_mask |= 1u << k;
             p.scalar[k] = scalars[k];
+        } else {
+            if (ins[k].affine & AGMI_AFFINE_SCALE) {
+                p.scale_mask |= 1u << k;
+                p.scale[k] = ins[k].scale;
+            }
+            if (ins[k].affine & AGMI_AFFINE_SHIFT) {
+                p.shift_mask |= 1u << k;
+                p.shift[k] = ins[k].shift;
+            }
         }
         for (int d = 0; d < m.ndim; ++d) p.istr[k][d] = m.stride[n_out + k][d];
     }

@@ -78,7 +78,10 @@ struct RedParams {
     void *out;  // T* when final, Acc* (chunk-major) when partial
     const void *in[AGMI_MAX_INPUTS];
     double scalar[AGMI_MAX_INPUTS];
+    double scale[AGMI_MAX_INPUTS];  // pending affine map of an input: value = mem * scale + shift
+    double shift[AGMI_MAX_INPUTS];
     unsigned scalar_mask;
+    unsigned scale_mask, shift_mask;
     int n_chunks;
     int64_t O, R, I;
     int64_t r_chunk;
@@ -120,10 +123,17 @@ __device__ __forceinline__ void load_points(const RedParams &p, int64_t o, int64
 }
 
 template <template <typename> class F, typename T, int V>
-__device__ __forceinline__ T map_point(const T (&x)[F<T>::NIN][V], int j) {
+__device__ __forceinline__ T map_point(const RedParams &p, const T (&x)[F<T>::NIN][V], int j) {
     T xi[F<T>::NIN], oi[F<T>::NOUT];
 #pragma unroll
     for (int k = 0; k < F<T>::NIN; ++k) xi[k] = x[k][j];
+    if (p.scale_mask | p.shift_mask) {  // wave-uniform
+#pragma unroll
+        for (int k = 0; k < F<T>::NIN; ++k) {
+            if (p.scale_mask & (1u << k)) xi[k] = xi[k] * static_cast<T>(p.scale[k]);
+            if (p.shift_mask & (1u << k)) xi[k] = xi[k] + static_cast<T>(p.shift[k]);
+        }
+    }
     F<T>::apply(xi, oi);
     return oi[0];
 }
@@ -171,14 +181,14 @@ __global__ __launch_bounds__(kBlock) void red_row_block(const RedParams p) {
         T x[F<T>::NIN][V];
         load_points<F, T, V, 1>(p, o, r_begin + v * V, 0, x);
 #pragma unroll
-        for (int j = 0; j < V; ++j) acc = Acc::combine(acc, Acc::lift(map_point<F, T, V>(x, j)));
+        for (int j = 0; j < V; ++j) acc = Acc::combine(acc, Acc::lift(map_point<F, T, V>(p, x, j)));
     }
     if (V > 1) {  // ragged tail, fewer than V points
         const int64_t r = r_begin + n_vec * V + threadIdx.x;
         if (r < r_end) {
             T x[F<T>::NIN][1];
             load_points<F, T, 1, 1>(p, o, r, 0, x);
-            acc = Acc::combine(acc, Acc::lift(map_point<F, T, 1>(x, 0)));
+            acc = Acc::combine(acc, Acc::lift(map_point<F, T, 1>(p, x, 0)));
         }
     }
     acc = block_reduce<Acc>(acc);
@@ -245,7 +255,7 @@ __global__ __launch_bounds__(kBlock) void red_row_group(const RedParams p, const
         for (int64_t r = lane; r < p.R; r += G) {
             T x[F<T>::NIN][1];
             load_points<F, T, 1, 1>(p, o, r, 0, x);
-            acc = Acc::combine(acc, Acc::lift(map_point<F, T, 1>(x, 0)));
+            acc = Acc::combine(acc, Acc::lift(map_point<F, T, 1>(p, x, 0)));
         }
     }
     acc = wave_reduce<Acc>(acc, G);  // every lane of the wave takes part (rows past O hold identities)
@@ -278,7 +288,7 @@ __global__ __launch_bounds__(kBlock) void red_cols(const RedParams p, const int 
             T x[F<T>::NIN][V];
             load_points<F, T, V, 2>(p, o, r, i0, x);
 #pragma unroll
-            for (int j = 0; j < V; ++j) acc[j] = Acc::combine(acc[j], Acc::lift(map_point<F, T, V>(x, j)));
+            for (int j = 0; j < V; ++j) acc[j] = Acc::combine(acc[j], Acc::lift(map_point<F, T, V>(p, x, j)));
         }
     }
     if (TY > 1) {
@@ -432,7 +442,7 @@ static int launch_reduce(const char *fname, const RedParams &base, bool vec_ok, 
         if constexpr (std::is_same<AccT<T>, AccLse<T>>::value && std::is_same<F<T>, FCopy<T>>::value) {
             const bool unit = p.istr[0][1] == 1 || p.r_chunk == 1;
             const int v = (pl.V > 1 && unit) ? VEC : 1;
-            if (!(p.scalar_mask & 1u) && p.r_chunk <= static_cast<int64_t>(kBlock) * v * kLseIters) {
+            if (!(p.scalar_mask & 1u) && !((p.scale_mask | p.shift_mask) & 1u) && p.r_chunk <= static_cast<int64_t>(kBlock) * v * kLseIters) {
                 set_kernel_name("lse_row_block%s", two_stage ? "+red_finish" : "");
                 const int64_t need = ceil_div(p.r_chunk, static_cast<int64_t>(kBlock) * v);
 #define AGMI_LSE(VV, IT)                                                                                   \
@@ -594,6 +604,14 @@ static int setup_reduce(int ndim, const int64_t *shape, const uint8_t *reduce_ax
             p.scalar_mask |= 1u << k;
             p.scalar[k] = scalars[k];
         } else {
+            if (ins[k].affine & AGMI_AFFINE_SCALE) {
+                p.scale_mask |= 1u << k;
+                p.scale[k] = ins[k].scale;
+            }
+            if (ins[k].affine & AGMI_AFFINE_SHIFT) {
+                p.shift_mask |= 1u << k;
+                p.shift[k] = ins[k].shift;
+            }
             for (int a = 0; a < 3; ++a) p.istr[k][a] = ori[1 + k][a];
             if (p.istr[k][ax] != 0 && p.istr[k][ax] != 1) st->vec_ok = false;
         }

@@ -9,7 +9,7 @@ primitives (and therefore the same kernels).
 
 from ..extend import Box, primitive
 from . import wrapper as anp
-from .devarray import DevArray
+from .devarray import DevArray, LazyDevArray
 
 
 def _route(name, swap=False):
@@ -102,4 +102,5 @@ DevArray.__hash__ = object.__hash__
 DevArrayBox.__hash__ = lambda self: id(self)
 
 DevArrayBox.register(DevArray)
+DevArrayBox.register(LazyDevArray)
 DevArrayBox.register(float)

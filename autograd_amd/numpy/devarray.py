@@ -11,6 +11,7 @@ dtype promotion follows NumPy 2 (NEP 50): Python scalars are weak, arrays and Nu
 scalars are strong.
 """
 
+import math
 import numbers
 
 import numpy as onp
@@ -107,7 +108,164 @@ class DevArray:
     def __setitem__(self, idx, value):
         raise TypeError("DevArray is immutable: item assignment is not supported")
 
+    # ---- view helpers ---------------------------------------------------------------------
+    def _h(self):
+        """The tensor that carries shape, strides and storage (metadata only: never its values)."""
+        return self._t
+
+    def _like(self, t):
+        """A view ``t`` of this array's storage as an array of the same kind."""
+        return DevArray(t, self.dtype)
+
     # ---- operators and methods are attached by wrapper.py (they are traced primitives) ------
+
+
+class LazyDevArray(DevArray):
+    """``raw * scale + shift`` not yet written to memory.
+
+    Negation and arithmetic with a Python scalar return one of these instead of launching a
+    kernel (see ``_fold``); the next kernel that reads it applies the map on load, as two
+    separately rounded operations, so the value is bit-for-bit what the eager passes would have
+    stored.  Code that is unaware of it reads ``_t`` as on any ``DevArray``: the first such read
+    writes the value to a fresh buffer (one copy kernel) and keeps it.
+    """
+
+    __slots__ = ("_raw", "_scale", "_shift")
+
+    def __init__(self, raw, dtype, scale, shift):
+        self._raw = raw
+        self.dtype = dtype
+        self._borrowed = False
+        self._scale = scale  # Python float, representable in dtype; 1.0 = no multiply
+        self._shift = shift  # Python float, or None = no add (x + 0.0 is not x for x = -0.0)
+
+    def __getattr__(self, name):
+        # only reached when a slot is unset: `_t` before the value has been written out
+        if name != "_t":
+            raise AttributeError(name)
+        raw = self._raw
+        out = _lib.empty(tuple(raw.shape), self.dtype)
+        _lib.elementwise(Op.COPY, _lib.DTYPE_CODE[self.dtype], tuple(raw.shape), (out,),
+                         (_lib.Affine(raw, self._scale, self._shift),))
+        self._t = out
+        return out
+
+    @property
+    def shape(self):
+        return tuple(self._raw.shape)
+
+    @property
+    def ndim(self):
+        return self._raw.dim()
+
+    @property
+    def size(self):
+        return self._raw.numel()
+
+    @property
+    def strides(self):
+        item = self.dtype.itemsize
+        return tuple(s * item for s in self._raw.stride())
+
+    def __len__(self):
+        if self._raw.dim() == 0:
+            raise TypeError("len() of unsized object")
+        return self._raw.shape[0]
+
+    def __iter__(self):
+        if self._raw.dim() == 0:
+            raise TypeError("iteration over a 0-d array")
+        return (self[i] for i in range(self._raw.shape[0]))
+
+    def _h(self):
+        return self._raw
+
+    def _like(self, t):
+        return LazyDevArray(t, self.dtype, self._scale, self._shift)
+
+
+def plain(x):
+    """``x`` with any pending map written out (a no-op for everything else)."""
+    return DevArray(x._t, x.dtype) if type(x) is LazyDevArray else x
+
+
+def alias(x):
+    """A second handle on ``x``'s storage (and pending map)."""
+    return x._like(x._h())
+
+
+def _is_pow2(c):
+    return c != 0.0 and math.isfinite(c) and math.frexp(c)[0] in (0.5, -0.5) and 2.0**-60 <= abs(c) <= 2.0**60
+
+
+def _representable(v, dtype):
+    return math.isfinite(v) and (dtype == _F64 or float(onp.float32(v)) == v)
+
+
+def _fold(op, dtype, xs):
+    """``op(xs)`` as a pending affine map of its one array operand, or None.
+
+    Folded only when the composed map gives bit-for-bit the value of the eager passes:
+    negation always (it commutes with rounding); a scalar factor when it or the pending scale is a
+    power of two (that multiply is then exact); a scalar offset when no offset is pending.  Scalars are
+    Python floats/ints (weak in NumPy's promotion: converted to the array's dtype first).
+    """
+    if op == Op.NEG:
+        (a,) = xs
+        c = None
+    elif len(xs) == 2:
+        a, c = xs
+        swapped = False
+        if type(c) is not float and type(c) is not int:
+            a, c, swapped = c, a, True
+            if type(c) is not float and type(c) is not int:
+                return None
+    else:
+        return None
+    if not isinstance(a, DevArray) or a.dtype != dtype:
+        return None
+    if type(a) is LazyDevArray:
+        raw, s, t = a._raw, a._scale, a._shift
+    else:
+        raw, s, t = a._t, 1.0, None
+    if c is not None:
+        c = float(c) if dtype == _F64 else float(onp.float32(c))
+    if op == Op.NEG:
+        s, t = -s, (None if t is None else -t)
+    elif op == Op.MUL or (op == Op.DIV and not swapped and _is_pow2(c)):
+        if op == Op.DIV:
+            c = 1.0 / c
+        if t is None:
+            if not (_is_pow2(s) or _is_pow2(c)):  # one of the two multiplies is exact
+                return None
+            s = s * c
+        elif _is_pow2(c):
+            s, t = s * c, t * c
+            if not _representable(t, dtype) or (t == 0.0) != (a._shift == 0.0):
+                return None
+        else:
+            return None
+        if s != s or not (_representable(s, dtype) or math.isinf(s)):
+            return None
+    elif op == Op.ADD:
+        if t is not None:
+            return None
+        t = c
+    elif op == Op.SUB:
+        if t is not None:
+            return None
+        if swapped:  # c - x = (-x) + c
+            s, t = -s, c
+        else:  # x - c = x + (-c)
+            t = -c
+    else:
+        return None
+    if s == 1.0 and t is None:
+        return DevArray(raw, dtype)
+    return LazyDevArray(raw, dtype, s, t)
+
+
+_FOLDABLE = frozenset({Op.NEG, Op.MUL, Op.ADD, Op.SUB, Op.DIV})
 
 
 def is_scalar(x):
@@ -241,6 +399,8 @@ def _operand(x, dtype):
     if isinstance(x, DevArray):
         if x.dtype != dtype:
             x = astype(x, dtype)
+        elif type(x) is LazyDevArray:
+            return _lib.Affine(x._raw, x._scale, x._shift)
         return x._t
     if isinstance(x, (numbers.Number, onp.generic)):
         return float(x)
@@ -269,6 +429,8 @@ def broadcast_shapes(a, b):
 def _bshape(operands):
     shape = None
     for t in operands:
+        if type(t) is _lib.Affine:
+            t = t.t
         if isinstance(t, torch.Tensor):
             s = tuple(t.shape)
             if shape is None:
@@ -279,8 +441,11 @@ def _bshape(operands):
 
 
 def _expand(t, shape):
-    if isinstance(t, torch.Tensor) and tuple(t.shape) != shape:
-        return t.expand(shape)
+    if isinstance(t, torch.Tensor):
+        if tuple(t.shape) != shape:
+            return t.expand(shape)
+    elif type(t) is _lib.Affine and tuple(t.t.shape) != shape:
+        return _lib.Affine(t.t.expand(shape), t.scale, t.shift)
     return t
 
 
@@ -290,7 +455,17 @@ def _lift_scalars(operands, dtype):
 
 
 def map_op(op, dtype, *xs, out=None, n_out=1):
-    """Launch elementwise ``op`` on broadcast operands; returns DevArray (or a tuple)."""
+    """Launch elementwise ``op`` on broadcast operands; returns DevArray (or a tuple).
+
+    Negation and arithmetic with one Python scalar launch nothing when the result can be kept as
+    a pending affine map of the operand (``_fold``)."""
+    if out is None:
+        if op in _FOLDABLE:
+            folded = _fold(op, dtype, xs)
+            if folded is not None:
+                return folded
+    elif type(out) is not DevArray:
+        raise TypeError("map_op: `out` must be a plain device array")
     ops = tuple(_operand(x, dtype) for x in xs)
     shape = _bshape(ops)
     if shape is None:
@@ -333,12 +508,13 @@ def astype_copy(x):
 
 
 def contiguous(x):
-    return x if x._t.is_contiguous() else copy(x)
+    return x if type(x) is DevArray and x._t.is_contiguous() else copy(x)
 
 
 def compare(cmp, a, b):
     dt = _float_dtype(result_dtype(a, b))
-    ops = (_operand(a, dt), _operand(b, dt))
+    ops = tuple(x.t if type(x) is _lib.Affine else x
+                for x in (_operand(plain(a), dt), _operand(plain(b), dt)))  # the compare kernel applies no map
     shape = _bshape(ops)
     if shape is None:
         ops = _lift_scalars(ops, dt)
@@ -401,7 +577,7 @@ def map_reduce(op, red, dtype, xs, axes, keepdims, shape=None):
         # reduced axes interleaved with kept ones: one group of adjacent axes at a time
         if red == Red.LOGSUMEXP:
             raise NotImplementedError("logsumexp over non-adjacent axes of a non-contiguous layout")
-        cur = map_op(op, dtype, *[DevArray(t, dtype) if isinstance(t, torch.Tensor) else t for t in ops])
+        cur = map_op(op, dtype, *[_rewrap(t, dtype) for t in ops])
         for group in _adjacent_groups(axes):
             cur = map_reduce(Op.COPY, red, dtype, (cur,), group, True)
         out_t = cur._t
@@ -409,6 +585,14 @@ def map_reduce(op, red, dtype, xs, axes, keepdims, shape=None):
     if not keepdims and axes:
         out = DevArray(out_t.reshape(reduce_shape(shape, axes, False)), dtype)
     return out
+
+
+def _rewrap(t, dtype):
+    if isinstance(t, torch.Tensor):
+        return DevArray(t, dtype)
+    if type(t) is _lib.Affine:
+        return LazyDevArray(t.t, dtype, t.scale, t.shift)
+    return t
 
 
 def _adjacent_groups(axes):

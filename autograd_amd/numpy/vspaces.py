@@ -12,7 +12,7 @@ from .. import _lib
 from .._lib import Op, Red
 from ..extend import VSpace
 from . import devarray as D
-from .devarray import DevArray
+from .devarray import DevArray, LazyDevArray
 
 
 _ZEROS = {}
@@ -27,7 +27,7 @@ def _shared_zero(dtype):
 
 def is_broadcast_view(x):
     """True when some axis of extent > 1 has stride 0: several indices share one element."""
-    t = x._t
+    t = x._h()
     if t.numel() <= 1:
         return False
     for extent, stride in zip(t.shape, t.stride()):
@@ -37,6 +37,8 @@ def is_broadcast_view(x):
 
 
 def is_shared_zero(x):
+    if type(x) is not DevArray:
+        return False
     z = _ZEROS.get(x.dtype)
     return z is not None and x._t.data_ptr() == z._t.data_ptr()
 
@@ -99,10 +101,10 @@ class DevArrayVSpace(VSpace):
         if not isinstance(x, DevArray):
             return self._add(x, y)
         if is_shared_zero(x) and isinstance(y, DevArray) and y.shape == x.shape and y.dtype == x.dtype:
-            acc = DevArray(y._t, y.dtype)
+            acc = D.alias(y)
             acc._borrowed = True
             return acc
-        if x._borrowed or is_broadcast_view(x):
+        if x._borrowed or type(x) is not DevArray or is_broadcast_view(x):
             return self._add(x, y)
         if isinstance(y, DevArray) and y.shape != x.shape and D.broadcast_shapes(x.shape, y.shape) != x.shape:
             return self._add(x, y)
@@ -118,4 +120,5 @@ class DevArrayVSpace(VSpace):
 
 
 DevArrayVSpace.register(DevArray)
+DevArrayVSpace.register(LazyDevArray)
 DevArrayVSpace.register(float)

@@ -184,7 +184,7 @@ def mean(a, *args, **kwargs):
 # ---- shape-only functions (views: no kernel unless a copy is unavoidable) -----------------------
 def _view_or_copy(x, shape):
     try:
-        return DevArray(x._t.view(shape), x.dtype)
+        return x._like(x._h().view(shape))
     except RuntimeError:
         return DevArray(D.contiguous(x)._t.view(shape), x.dtype)
 
@@ -236,25 +236,25 @@ def expand_dims(x, axis):
     axes = (axis,) if isinstance(axis, (numbers.Integral, onp.integer)) else tuple(axis)
     nd = x.ndim + len(axes)
     axes = sorted(a % nd for a in axes)
-    t = x._t
+    t = x._h()
     for a in axes:
         t = t.unsqueeze(a)
-    return DevArray(t, x.dtype)
+    return x._like(t)
 
 
 @primitive
 def squeeze(x, axis=None):
     x = D.asarray(x)
     if axis is None:
-        return DevArray(x._t.squeeze(), x.dtype)
+        return x._like(x._h().squeeze())
     axes = (axis,) if isinstance(axis, (numbers.Integral, onp.integer)) else tuple(axis)
     axes = sorted((a % x.ndim for a in axes), reverse=True)
-    t = x._t
+    t = x._h()
     for a in axes:
         if t.shape[a] != 1:
             raise ValueError("cannot select an axis to squeeze out which has size not equal to one")
         t = t.squeeze(a)
-    return DevArray(t, x.dtype)
+    return x._like(t)
 
 
 @primitive
@@ -263,26 +263,26 @@ def transpose(x, axes=None):
     if axes is None:
         axes = tuple(range(x.ndim))[::-1]
     axes = tuple(int(a) % x.ndim for a in axes) if x.ndim else ()
-    return DevArray(x._t.permute(axes) if x.ndim else x._t, x.dtype)
+    return x._like(x._h().permute(axes) if x.ndim else x._h())
 
 
 @primitive
 def swapaxes(x, axis1, axis2):
     x = D.asarray(x)
-    return DevArray(x._t.transpose(axis1, axis2), x.dtype)
+    return x._like(x._h().transpose(axis1, axis2))
 
 
 @primitive
 def moveaxis(x, source, destination):
     x = D.asarray(x)
-    return DevArray(torch.movedim(x._t, source, destination), x.dtype)
+    return x._like(torch.movedim(x._h(), source, destination))
 
 
 @primitive
 def broadcast_to(x, shape):
     x = D.asarray(x)
     shape = (shape,) if isinstance(shape, numbers.Integral) else tuple(shape)
-    return DevArray(x._t.expand(shape), x.dtype)
+    return x._like(x._h().expand(shape))
 
 
 def _atleast(n):
@@ -290,14 +290,14 @@ def _atleast(n):
         res = []
         for a in arys:
             a = D.asarray(a)
-            t = a._t
+            t = a._h()
             if n >= 1 and t.dim() == 0:
                 t = t.reshape(1)
             if n >= 2 and t.dim() == 1:
                 t = t.unsqueeze(0)
             if n >= 3 and t.dim() == 2:
                 t = t.unsqueeze(2)
-            res.append(DevArray(t, a.dtype))
+            res.append(a._like(t))
         return res[0] if len(res) == 1 else res
 
     return _wrap(raw, f"atleast_{n}d")
@@ -317,9 +317,9 @@ def repeat(x, repeats, axis=None):
         axis = 0
     axis %= x.ndim
     # out viewed as (..., n, repeats, ...) = x broadcast along a new axis
-    src = x._t.unsqueeze(axis + 1)
+    src = x._h().unsqueeze(axis + 1)
     wide = src.shape[: axis + 1] + (repeats,) + src.shape[axis + 2 :]
-    out = D.map_op(Op.COPY, x.dtype, DevArray(src.expand(wide), x.dtype)) if x.dtype in D._FLOATS else D.astype_copy(
+    out = D.map_op(Op.COPY, x.dtype, x._like(src.expand(wide))) if x.dtype in D._FLOATS else D.astype_copy(
         DevArray(src.expand(wide), x.dtype))
     final = x.shape[:axis] + (x.shape[axis] * repeats,) + x.shape[axis + 1 :]
     return DevArray(out._t.view(final), x.dtype)
@@ -482,7 +482,7 @@ def _host_index(idx):
 def take(A, idx):
     """``A[idx]``: views for basic indices, a gather kernel for an integer array on axis 0."""
     if _is_basic_index(idx):
-        return DevArray(A._t[_plain(idx)], A.dtype)
+        return A._like(A._h()[_plain(idx)])
     rows = _host_index(idx)
     if rows is None:
         raise NotImplementedError(
@@ -515,7 +515,7 @@ def scatter_add(A, idx, x):
     from .vspaces import is_broadcast_view, is_shared_zero
 
     basic = _is_basic_index(idx)
-    if A._borrowed or is_broadcast_view(A):  # not this accumulator's own memory yet: allocate it
+    if A._borrowed or type(A) is not DevArray or is_broadcast_view(A):  # not this accumulator's own memory yet: allocate it
         if is_shared_zero(A):
             if basic:
                 # into zeros the sum is 0 + x, so the destination is never read back; and when the

@@ -44,10 +44,21 @@ typedef enum agmi_dtype {
 
 /* One strided operand.  data == NULL in an INPUT slot means "scalar passed by value": the
  * value is taken from scalars[slot] and converted to the array dtype (a weak Python scalar
- * in NumPy's promotion rules). */
+ * in NumPy's promotion rules).
+ * An INPUT may carry a pending affine map: its element value is then mem * scale + shift,
+ * computed on load as two separately rounded operations (exactly what the NumPy passes
+ * `x * scale` and `+ shift` would have produced), so that negation, scalar multiples and
+ * scalar offsets of an array (numpy_vjps.py:87, 157; `2 * g`, `1.0 - e` in user code) cost no
+ * pass of their own.  `affine` is a bit set: AGMI_AFFINE_SCALE, AGMI_AFFINE_SHIFT; 0 = plain
+ * (zero-initialised structs are plain).  Ignored for outputs and by agmi_gemm/cast/compare. */
+#define AGMI_AFFINE_SCALE 1u
+#define AGMI_AFFINE_SHIFT 2u
 typedef struct agmi_array {
     void *data;                     /* device pointer to the element at index (0, ..., 0) */
     int64_t strides[AGMI_MAX_DIMS]; /* elements */
+    double scale;
+    double shift;
+    uint32_t affine;
 } agmi_array;
 
 /* Elementwise operations.  Unary/binary/ternary ufuncs are the forward primitives

@@ -422,9 +422,89 @@ def test_rank_limits_are_reported(dnp):
     from autograd_amd._lib import AgmiError
 
     x = P(dnp, onp.zeros((2,) * 8, F32))
-    assert (x + 1.0).shape == (2,) * 8                      # rank 8 merges to one axis
+    assert dnp.exp(x).shape == (2,) * 8                      # rank 8 merges to one axis
     y = dnp.transpose(x)                                    # fully reversed: 8 unmergeable axes
     with pytest.raises(AgmiError, match="axes remain after merging"):
         y + x
     with pytest.raises(AgmiError):
-        P(dnp, onp.zeros((1,) * 9, F32)) + 1.0
+        dnp.exp(P(dnp, onp.zeros((1,) * 9, F32)))
+
+
+# ---- pending affine maps (negation / scalar factor / scalar offset folded into the consumer) -----
+def _lazy_cases(dnp, x):
+    """(device expression, NumPy expression) pairs whose device side is a pending map."""
+    X = P(dnp, x)
+    one = x.dtype.type(1)
+    return [
+        (-X, -x), (X * 3.0, x * one * x.dtype.type(3.0)), (0.1 * X, x.dtype.type(0.1) * x), (X + 1.5, x + x.dtype.type(1.5)),
+        (1.0 - X, one - x), (1.0 - 2.0 * X, one - x.dtype.type(2) * x), (-(X * 0.3), -(x * x.dtype.type(0.3))),
+        ((X + 0.7) * 4.0, (x + x.dtype.type(0.7)) * x.dtype.type(4)), (X + 0.0, x + x.dtype.type(0)),
+        ((X * 3.0) * 0.5, (x * x.dtype.type(3)) * x.dtype.type(0.5)),
+    ]
+
+
+@pytest.mark.parametrize("dtype", [F32, F64])
+def test_pending_maps_are_bit_exact_on_every_kernel_path(dnp, dtype):
+    from autograd_amd.numpy.devarray import LazyDevArray
+
+    rng = onp.random.RandomState(11)
+    x = rng.randn(67, 130).astype(dtype)
+    x[0, :4] = [0.0, -0.0, onp.inf, onp.nan]
+    y = rng.randn(67, 130).astype(dtype)
+    Y = P(dnp, y)
+    for k, (L, ref) in enumerate(_lazy_cases(dnp, x)):
+        assert type(L) is LazyDevArray, k
+        assert ref.dtype == dtype
+        # written out by the copy kernel (flat path), bit for bit incl. signed zeros
+        got = L.numpy()
+        nan = onp.isnan(ref)  # (the sign of a NaN is not specified: compare bits everywhere else)
+        assert got.dtype == dtype and onp.array_equal(onp.isnan(got), nan), k
+        assert onp.array_equal(got[~nan].view(onp.uint8), ref[~nan].view(onp.uint8)), k
+        # as an operand: flat, row-broadcast, strided (nd) and transposed consumers
+        assert onp.array_equal((L * Y).numpy(), ref * y, equal_nan=True), k
+        assert onp.array_equal((Y[:, :1] + L).numpy(), y[:, :1] + ref, equal_nan=True), k
+        assert onp.array_equal((L[::2, 1::3] - Y[::2, 1::3]).numpy(), ref[::2, 1::3] - y[::2, 1::3], equal_nan=True), k
+        assert onp.array_equal((L.T * Y.T).numpy(), ref.T * y.T, equal_nan=True), k
+        assert onp.array_equal((L[3] * Y).numpy(), ref[3] * y, equal_nan=True), k  # row operand pending
+        # two pending operands in one launch
+        assert onp.array_equal((L * (1.0 - Y)).numpy(), ref * (dtype(1) - y), equal_nan=True), k
+        # compare / cast / gather / contraction consumers see the written-out value
+        assert onp.array_equal((L > Y).numpy(), ref > y), k
+        assert onp.array_equal(dnp.take(L, onp.array([5, 1, 5])).numpy(), ref[[5, 1, 5]], equal_nan=True), k
+    # reductions: row / column / full, fused map, logsumexp (finite rows)
+    xf, yf = x[1:], y[1:]
+    for k, (L, ref) in enumerate(_lazy_cases(dnp, xf)):
+        close(dnp.sum(L, axis=1).numpy(), ref.sum(axis=1), RT[dtype])
+        close(dnp.sum(L, axis=0).numpy(), ref.sum(axis=0), RT[dtype])
+        close(dnp.sum(L).numpy(), ref.sum(), RT[dtype])
+        close(dnp.max(L, axis=1).numpy(), ref.max(axis=1), 0.0)
+        close(dnp.sum(L * Y[1:], axis=0).numpy(), (ref * yf).sum(axis=0), RT[dtype])
+        from autograd_amd.scipy.special import logsumexp
+
+        close(logsumexp(L, axis=1).numpy(), scipy.special.logsumexp(ref, axis=1), RT[dtype])
+        close(logsumexp(L, axis=0).numpy(), scipy.special.logsumexp(ref, axis=0), RT[dtype])
+        A, B = rng.randn(5, 66).astype(dtype), rng.randn(130, 3).astype(dtype)
+        close(dnp.dot(P(dnp, A), L).numpy(), A @ ref, RT[dtype])
+        close(dnp.dot(L, P(dnp, B)).numpy(), ref @ B, RT[dtype])
+
+
+def test_pending_maps_through_grad_match_eager_numpy(dnp):
+    """Differentiating through folded operations gives what NumPy gives op by op."""
+    from autograd_amd import elementwise_grad, grad
+
+    x = onp.linspace(-1.5, 1.5, 4099)
+    X = P(dnp, x)
+
+    def f(np):
+        return lambda v: np.sum((1.0 - np.exp(-2.0 * v)) / (1.0 + np.exp(-(2 * v))) * 0.5 - (3.0 - v) ** 2)
+
+    g = grad(f(dnp))(X)
+    e = onp.exp(-2.0 * x)
+    want = 0.5 * (2.0 * e / (1.0 + e) + (1.0 - e) * 2.0 * e / (1.0 + e) ** 2) + 2.0 * (3.0 - x)
+    close(g.numpy(), want, 1e-13)
+    h = elementwise_grad(elementwise_grad(lambda v: -dnp.tanh(-v) * 2.0))(X)
+    t = onp.tanh(x)
+    close(h.numpy(), 2.0 * (-2.0 * t * (1.0 - t * t)), 1e-13)
+    # accumulation over a fan-out whose contributions are pending maps of one array
+    k = grad(lambda v: dnp.sum(-v) + dnp.sum(2.0 * v) + dnp.sum(v + 1.0) + dnp.sum(v * v))(X)
+    close(k.numpy(), 2.0 + 2.0 * x, 1e-15)

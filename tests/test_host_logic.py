@@ -100,3 +100,62 @@ def test_vspace_metadata_and_laziness():
     assert vs == vspace(meta((3, 4))) and vs != vspace(meta((3, 4), torch.float64))
     fs = vspace(1.5)
     assert fs.shape == () and fs.dtype == onp.float64 and fs.size == 1
+
+
+def test_scalar_arithmetic_folds_into_a_pending_map_only_when_exact():
+    """negative / scalar multiply / scalar offset keep the operand's memory and record
+    ``raw * scale + shift``; they fold only where the composed map rounds exactly like the
+    eager passes (reference semantics: numpy_vjps.py:87 ``-g``, :73-78 ``y * g``)."""
+    from autograd_amd._lib import Op
+    from autograd_amd.numpy.devarray import LazyDevArray
+
+    x = meta((4, 6), torch.float64)
+
+    def state(a):
+        return (a._scale, a._shift) if type(a) is LazyDevArray else (1.0, None)
+
+    n = W.negative(x)
+    assert type(n) is LazyDevArray and state(n) == (-1.0, None) and n._raw.data_ptr() == x._t.data_ptr()
+    assert type(W.negative(n)) is DevArray and W.negative(n)._t.data_ptr() == x._t.data_ptr()
+    assert state(x * 3.0) == (3.0, None) and state(3 * x) == (3.0, None)
+    assert state(-(x * 3.0)) == (-3.0, None)
+    assert state(n * 3.0) == (-3.0, None)  # (-x) * 3 == x * (-3) exactly
+    assert state((x * 3.0) * 2.0) == (6.0, None)  # power-of-two factor commutes with rounding
+    assert state((x * 2.0) * 3.0) == (6.0, None)
+    assert state(x + 1.5) == (1.0, 1.5) and state(1.5 + x) == (1.0, 1.5)
+    assert state(x - 1.5) == (1.0, -1.5) and state(1.5 - x) == (-1.0, 1.5)
+    assert state(1.0 - 2.0 * x) == (-2.0, 1.0)
+    assert state(-(1.0 - 2.0 * x)) == (2.0, -1.0)
+    assert state((x + 1.0) * 4.0) == (4.0, 4.0) and state((x + 1.0) / 4.0) == (0.25, 0.25)
+    assert state(x + 0.0) == (1.0, 0.0)  # kept: -0.0 + 0.0 is +0.0
+    # not exact in general: these must launch (and there is no device here, so they raise)
+    for expr in (lambda: (x * 3.0) * 5.0, lambda: (x + 1.0) * 3.0, lambda: (x + 1.0) + 1.0, lambda: 2.0 / x,
+                 lambda: x / 3.0, lambda: x * onp.float64(3.0)):
+        with pytest.raises(Exception):
+            expr()
+    # float32: scalars are rounded to the array's dtype first, as NumPy's weak scalars are
+    y = meta((5,), torch.float32)
+    assert state(y * 0.1) == (float(onp.float32(0.1)), None) and (y * 0.1).dtype == onp.float32
+    # views keep the pending map and the metadata comes from the raw storage
+    v = W.transpose((1.0 - x))[1:, :2]
+    assert type(v) is LazyDevArray and v.shape == (5, 2) and state(v) == (-1.0, 1.0) and v.ndim == 2 and v.size == 10
+    assert len(v) == 5 and v.strides == (8, 48)
+    assert D._fold(Op.EXP, x.dtype, (x,)) is None
+
+
+def test_accumulators_never_write_through_a_pending_map(monkeypatch):
+    from autograd_amd.numpy import vspaces
+    from autograd_amd.numpy.devarray import LazyDevArray
+    from autograd_amd.numpy.vspaces import DevArrayVSpace, is_shared_zero
+
+    monkeypatch.setitem(vspaces._ZEROS, onp.dtype("float64"), DevArray(torch.zeros((), dtype=torch.float64)))
+    x = meta((3, 4), torch.float64)
+    vs = DevArrayVSpace(x)
+    g = W.negative(x)
+    acc = vs._mut_add(vs.zeros(), g)  # 0 + g borrows g, pending map included
+    assert type(acc) is LazyDevArray and acc._borrowed and acc._raw.data_ptr() == x._t.data_ptr()
+    assert not is_shared_zero(acc)
+    with pytest.raises(Exception):  # next contribution goes out of place -> needs a launch -> no device here
+        vs._mut_add(acc, x)
+    with pytest.raises(TypeError):
+        D.map_op(0, x.dtype, x, out=g)
