@@ -33,5 +33,6 @@ from .differential_operators import (  # noqa: F401
     vector_jacobian_product,
 )
 from .extend import primitive  # noqa: F401
+from .graphs import capture  # noqa: F401
 
 __version__ = "0.1.0"

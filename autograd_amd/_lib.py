@@ -192,6 +192,18 @@ def synchronize():
     torch.cuda.synchronize(device())
 
 
+# True while a HIP graph is being recorded: only kernel launches are legal then
+CAPTURING = False
+
+
+def check_not_capturing(what):
+    if CAPTURING:
+        raise RuntimeError(
+            f"{what} moves data between host and device, which cannot be recorded into a HIP graph; "
+            "do it outside the captured function"
+        )
+
+
 # ---- optional per-launch timing (HIP events on the launch stream) ------------------------------
 class KernelTimer:
     """Times launches with HIP events recorded on the stream the kernels run on.

@@ -77,6 +77,7 @@ class DevArray:
     # ---- host transfer (synchronises) ------------------------------------------------------
     def numpy(self):
         """Copy to a host ``numpy.ndarray`` (blocks until the stream has produced the data)."""
+        _lib.check_not_capturing("DevArray.numpy()")
         return self._t.cpu().numpy()
 
     def __array__(self, dtype=None, copy=None):
@@ -86,6 +87,7 @@ class DevArray:
     def item(self):
         if self._t.numel() != 1:
             raise ValueError("can only convert an array of size 1 to a Python scalar")
+        _lib.check_not_capturing("DevArray.item()")
         return self._t.item()
 
     def __float__(self):
@@ -291,6 +293,7 @@ def from_numpy(a, dtype=None):
             raise TypeError(f"dtype {a.dtype} is not supported on the device")
     if not a.flags.c_contiguous or not a.flags.writeable:
         a = onp.array(a, order="C")  # (ascontiguousarray would turn a 0-d array into 1-d)
+    _lib.check_not_capturing("uploading a host array")
     t = torch.from_numpy(a).to(_lib.device())
     return DevArray(t, a.dtype)
 

@@ -37,6 +37,9 @@ def parse():
     ap.add_argument("--workload", default="bcast", choices=["bcast", "tanh", "mlp", "rnn", "rosen"],
                     help="bcast (default) is the headline workload, BASELINE configs[1]; the others are the "
                          "remaining BASELINE configs, selectable for profiling")
+    ap.add_argument("--graph", action="store_true",
+                    help="time the workload replayed from a HIP graph (autograd_amd.capture) instead of the eager "
+                         "tracer; no per-kernel events in this mode")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch plain copies of a (8192,4096) f32 array (134.2 MB read + 134.2 MB written "
                          "each): the reference dispatch that hardware traffic counters are scaled by")
@@ -90,8 +93,8 @@ def cpu_baseline(seconds):
 
 
 def make_workload(name, be):
-    """(step function, config description, arithmetic dtype) for one BASELINE workload; inputs are
-    uploaded here, before any timing."""
+    """(function, device arguments, config description, arithmetic dtype) for one BASELINE workload;
+    inputs are uploaded here, before any timing."""
     from autograd_amd import configs
 
     if name == "bcast":
@@ -101,13 +104,13 @@ def make_workload(name, be):
         cfg = {"workload": "configs[1] broadcast+reduction VJPs: grad wrt (A,b,c) of "
                            "sum(logsumexp(A*b[None,:]+c[:,None],axis=1))",
                "A": [8192, 4096], "b": [4096], "c": [8192], "seed": 0}
-        return (lambda: g(A, b, c)), cfg, "f32"
+        return g, (A, b, c), cfg, "f32"
     if name == "tanh":
         x = be.put(configs.tanh_inputs()["x"])
         prog = configs.tanh_program(be)
         cfg = {"workload": "configs[0] elementwise tanh: egrad, egrad^2 and egrad^3 of (1-exp(-2x))/(1+exp(-2x)); "
                            "one step = the three calls", "x": [4194304]}
-        return (lambda: (prog["d1"](x), prog["d2"](x), prog["d3"](x))), cfg, "f64"
+        return (lambda x: (prog["d1"](x), prog["d2"](x), prog["d3"](x))), (x,), cfg, "f64"
     if name == "mlp":
         inp = configs.mlp_inputs()
         params = configs.tree_map(be.put, inp["params"])
@@ -115,20 +118,20 @@ def make_workload(name, be):
         g = configs.mlp_program(be)["grad"]
         cfg = {"workload": "configs[2] MLP 784-1024-1024-10 tanh, log-softmax loss, grad wrt [(W,b)]",
                "batch": 1024, "seed": 0}
-        return (lambda: g(params, X, T)), cfg, "f32"
+        return g, (params, X, T), cfg, "f32"
     if name == "rnn":
         inp = configs.rnn_inputs()
         params = configs.tree_map(be.put, inp["params"])
         xs, ts = be.put(inp["inputs"]), be.put(inp["targets"])
         g = configs.rnn_program(be)["grad"]
         cfg = {"workload": "configs[3] tanh RNN T=64 B=256 H=512, grad wrt params dict", "seed": 0}
-        return (lambda: g(params, xs, ts)), cfg, "f32"
+        return g, (params, xs, ts), cfg, "f32"
     inp = configs.rosen_inputs()
     x, v = be.put(inp["x"]), be.put(inp["v"])
     prog = configs.rosen_program(be)
     cfg = {"workload": "configs[4] Rosenbrock HVP n=2^24: one step = make_hvp(f)(x)[0](v) and make_jvp(grad(f))(x)(v)",
            "seed": 0}
-    return (lambda: (prog["hvp_rev"](x, v), prog["hvp_fwd"](x, v))), cfg, "f64"
+    return (lambda x, v: (prog["hvp_rev"](x, v), prog["hvp_fwd"](x, v))), (x, v), cfg, "f64"
 
 
 def measured_traffic(kernel):
@@ -157,7 +160,12 @@ def main():
     from autograd_amd import _lib, configs
 
     be = configs.device_backend()
-    step, config, dtype = make_workload(args.workload, be)
+    fun, fun_args, config, dtype = make_workload(args.workload, be)
+    if args.graph:
+        return main_graph(args, be, fun, fun_args, config, dtype)
+
+    def step():
+        return fun(*fun_args)
 
     # warm-up, with every launch timed once to find the kernel that dominates the step
     for _ in range(max(1, args.warmup)):
@@ -232,6 +240,32 @@ def main():
     print(json.dumps(result))
 
 
+def main_graph(args, be, fun, fun_args, config, dtype):
+    """--graph: the step is one replay of the workload recorded as a HIP graph (no per-kernel events:
+    nothing is launched from the host but the graph)."""
+    import autograd_amd as ag
+
+    graphed = ag.capture(fun, *fun_args)
+    sec = time_steps(lambda: graphed(*fun_args), be.sync, args.steps, max(1, args.warmup))
+    config = dict(config, execution="HIP graph replay of the recorded evaluation")
+    print(json.dumps({
+        "metric": "grad evals/sec", "value": 1.0 / sec, "unit": "grad evals/sec", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": sec * 1e3, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": dtype, "data": "synthetic", "config": config, "roofline": None,
+        "cpu_baseline": None,
+    }))
+
+
+def graph_rate(fun, args, sync, steps):
+    """grad evals/sec of ``fun(*args)`` replayed from a HIP graph; the graph is dropped afterwards."""
+    import autograd_amd as ag
+
+    graphed = ag.capture(fun, *args)
+    sec = time_steps(lambda: graphed(*args), sync, steps, 2)
+    del graphed
+    return 1.0 / sec
+
+
 def extras(be):
     """The other workloads (grad evals/sec each) and the MLP contraction rate; short runs."""
     from autograd_amd import _lib, configs
@@ -243,6 +277,7 @@ def extras(be):
     for k in ("d1", "d2", "d3"):
         ms = time_steps(lambda: prog[k](x), be.sync, 10, 2) * 1e3
         out[f"tanh_{k}_evals_per_sec"] = 1e3 / ms
+        out[f"tanh_{k}_graph_evals_per_sec"] = graph_rate(prog[k], (x,), be.sync, 10)
     # config 3: MLP gradient, f32; MFMA rate over the GEMMs whose dimensions are all >= 784
     inp = configs.mlp_inputs()
     params = configs.tree_map(be.put, inp["params"])
@@ -250,6 +285,7 @@ def extras(be):
     g = configs.mlp_program(be)["grad"]
     ms = time_steps(lambda: g(params, X, T), be.sync, 20, 3) * 1e3
     out["mlp_grad_evals_per_sec"] = 1e3 / ms
+    out["mlp_grad_graph_evals_per_sec"] = graph_rate(g, (params, X, T), be.sync, 20)
     with _lib.KernelTimer(only={("gemm",)}) as kt:
         for _ in range(5):
             g(params, X, T)
@@ -271,14 +307,17 @@ def extras(be):
     g4 = configs.rnn_program(be)["grad"]
     ms = time_steps(lambda: g4(params, xs, ts), be.sync, 5, 1) * 1e3
     out["rnn_grad_evals_per_sec"] = 1e3 / ms
+    out["rnn_grad_graph_evals_per_sec"] = graph_rate(g4, (params, xs, ts), be.sync, 5)
     # config 5: Rosenbrock HVP, f64
     inp = configs.rosen_inputs()
     x5, v5 = be.put(inp["x"]), be.put(inp["v"])
     p5 = configs.rosen_program(be)
     ms = time_steps(lambda: p5["hvp_rev"](x5, v5), be.sync, 5, 1) * 1e3
     out["rosen_hvp_rev_evals_per_sec"] = 1e3 / ms
+    out["rosen_hvp_rev_graph_evals_per_sec"] = graph_rate(p5["hvp_rev"], (x5, v5), be.sync, 5)
     ms = time_steps(lambda: p5["hvp_fwd"](x5, v5), be.sync, 5, 1) * 1e3
     out["rosen_hvp_fwd_evals_per_sec"] = 1e3 / ms
+    out["rosen_hvp_fwd_graph_evals_per_sec"] = graph_rate(p5["hvp_fwd"], (x5, v5), be.sync, 5)
     return out
 
 
