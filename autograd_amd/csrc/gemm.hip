@@ -90,9 +90,11 @@ constexpr int kXcds = 8;
 //   kXC - 4 consecutive x at one k (xs == 1, X % 4 == 0): one 16-byte load, one 16-byte LDS store
 //   kKC - 4 consecutive k at one x (ks == 1, K % 4 == 0): one 16-byte load, stored transposed
 //   kGen - any strides / ragged extents: four 4-byte loads
-// Loads are branch-free (out-of-range groups read a clamped address and are zeroed by a select),
-// so the number of loads in flight is the same on every path and the compiler can wait for
-// exactly the slab it needs (s_waitcnt vmcnt(n)) while younger prefetches stay in flight.
+// Loads are branch-free (out-of-range groups read a clamped address), so the number of loads in
+// flight is the same on every path and the compiler can wait for exactly the slab it needs
+// (s_waitcnt vmcnt(n)) while younger prefetches stay in flight.  Out-of-range groups are zeroed
+// when the slab is copied to LDS, not when it is loaded: a select right after the load would
+// make every iteration wait for the load it has just issued.
 enum LoadMode { kXC = 0, kKC = 1, kGen = 2 };
 
 template <typename T, int BX, int BK, int LOADS, int MODE, int NT>
@@ -111,7 +113,7 @@ struct SlabLoader {
                 const bool ok = x < X && k < K;  // K % 4 == 0: the group is all in or all out
                 const vec_t v = *reinterpret_cast<const vec_t *>(ok ? g + x * xs + k : g);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) reg[i][j] = ok ? v[j] : T(0);
+                for (int j = 0; j < 4; ++j) reg[i][j] = v[j];
             } else {
                 const int kk = e / (BX / 4), xx = (e % (BX / 4)) * 4;
                 const int64_t k = k0 + kk, x = x0 + xx;
@@ -119,32 +121,34 @@ struct SlabLoader {
                     const bool ok = k < K && x < X;  // X % 4 == 0
                     const vec_t v = *reinterpret_cast<const vec_t *>(ok ? g + k * ks + x : g);
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) reg[i][j] = ok ? v[j] : T(0);
+                    for (int j = 0; j < 4; ++j) reg[i][j] = v[j];
                 } else {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         const bool ok = k < K && x + j < X;
-                        const T v = *(ok ? g + k * ks + (x + j) * xs : g);
-                        reg[i][j] = ok ? v : T(0);
+                        reg[i][j] = *(ok ? g + k * ks + (x + j) * xs : g);
                     }
                 }
             }
         }
     }
 
+    // (x0, X, k0, K): the bounds the slab in `reg` was loaded with
     template <int LDX>
-    __device__ __forceinline__ void store(T (*S)[LDX], int tid) const {
+    __device__ __forceinline__ void store(T (*S)[LDX], int64_t x0, int64_t X, int64_t k0, int64_t K, int tid) const {
 #pragma unroll
         for (int i = 0; i < LOADS; ++i) {
             const int e = tid + i * NT;
             if (MODE == kKC) {
                 const int xx = e / (BK / 4), kk = (e % (BK / 4)) * 4;
+                const bool ok = x0 + xx < X && k0 + kk < K;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) S[kk + j][xx] = reg[i][j];
+                for (int j = 0; j < 4; ++j) S[kk + j][xx] = ok ? reg[i][j] : T(0);
             } else {
                 const int kk = e / (BX / 4), xx = (e % (BX / 4)) * 4;
+                const bool k_ok = k0 + kk < K;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) S[kk][xx + j] = reg[i][j];
+                for (int j = 0; j < 4; ++j) S[kk][xx + j] = (k_ok && x0 + xx + (MODE == kXC ? 0 : j) < X) ? reg[i][j] : T(0);
             }
         }
     }
@@ -168,7 +172,7 @@ __global__ __launch_bounds__(kBlock *KS) void gemm_mfma(const GemmParams p) {
     constexpr int STEPS = BK / TK / KS;  // MFMA k-steps per wave per slab
     static_assert(STEPS >= 1 && (BK / TK) % KS == 0, "K split");
     static_assert(WM % TM == 0 && WN % TM == 0 && BK % TK == 0 && BK % 4 == 0, "tile shape");
-    static_assert(DEPTH >= 1, "prefetch depth");
+    static_assert(DEPTH >= 2 && DEPTH % 2 == 0, "prefetch depth must be even (buffer parity is fixed at compile time)");
 
     // one LDS allocation: the two double-buffered slab images, reused as scratch by the K-group sum
     constexpr int kAsElems = 2 * BK * (BM + PAD_A), kBsElems = 2 * BK * (BN + PAD_B);
@@ -227,43 +231,79 @@ __global__ __launch_bounds__(kBlock *KS) void gemm_mfma(const GemmParams p) {
         la[d].load(A, p.a_rs, p.a_cs, m0, p.M, k_first + static_cast<int64_t>(d) * BK, k_limit, tid);
         lb[d].load(B, p.b_cs, p.b_rs, n0, p.N, k_first + static_cast<int64_t>(d) * BK, k_limit, tid);
     }
-    la[0].template store<BM + PAD_A>(As[0], tid);
-    lb[0].template store<BN + PAD_B>(Bs[0], tid);
+    // Register slot s % DEPTH holds slab s until it has been copied to LDS (two iterations before
+    // the matrix cores reach it), then is refilled with slab s + DEPTH.  Operand fragments are double-buffered in registers as well: the fragments
+    // of slab t + 1 are read from LDS while the matrix cores work on slab t, so that LDS latency
+    // is not paid in front of every group of MFMAs.
+    T fa[2][STEPS][FM], fb[2][STEPS][FN];
+    auto read_fragment = [&](int f, int buf, int s) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < FM; ++i) fa[f][s][i] = As[buf][ks0 + s * TK + op_k][wm0 + i * TM + op_x];
+#pragma unroll
+        for (int j = 0; j < FN; ++j) fb[f][s][j] = Bs[buf][ks0 + s * TK + op_k][wn0 + j * TM + op_x];
+    };
+    auto read_fragments = [&](int f, int buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) read_fragment(f, buf, s);
+    };
+    auto slab_k = [&](int64_t slab) { return k_first + slab * BK; };
+    la[0].template store<BM + PAD_A>(As[0], m0, p.M, slab_k(0), k_limit, tid);
+    lb[0].template store<BN + PAD_B>(Bs[0], n0, p.N, slab_k(0), k_limit, tid);
     __syncthreads();
+    read_fragments(0, 0);
+    if (n_slabs > 1) {
+        la[1 % DEPTH].template store<BM + PAD_A>(As[1], m0, p.M, slab_k(1), k_limit, tid);
+        lb[1 % DEPTH].template store<BN + PAD_B>(Bs[1], n0, p.N, slab_k(1), k_limit, tid);
+    }
 
-    for (int64_t t0 = 0; t0 < n_slabs; t0 += DEPTH) {
+    // One slab step.  `d` = t % DEPTH and `guarded` are compile-time constants after unrolling.
+    // A wave's MFMAs form one dependent chain per accumulator, so each one issues only when the
+    // previous has finished; everything else the step has to do (the global loads of slab
+    // t + DEPTH, the LDS reads of slab t + 1's fragments, the LDS writes of slab t + 2) is placed
+    // between the MFMAs and runs in their shadow.  The scheduling barriers pin that order (the
+    // scheduler would otherwise sink each LDS read next to its use, one step later).  Reads and
+    // writes of one step go to different LDS buffers, so their order within the step is free.
+    auto step = [&](const int d, const int64_t t, const bool guarded) __attribute__((always_inline)) {
+        const int cur = d & 1;  // DEPTH is even: slab t lives in LDS buffer t % 2
+        constexpr int kStoreAt = STEPS / 2;
+        // slab t + 1 is complete in LDS, and every wave is done reading buffer `cur`
+        __syncthreads();
 #pragma unroll
-        for (int d = 0; d < DEPTH; ++d) {
-            const int64_t t = t0 + d;
-            if (t < n_slabs) {  // uniform across the block
-                const int cur = (DEPTH % 2 == 0) ? (d & 1) : static_cast<int>(t & 1);
-                // register slot d held slab t (already in LDS): refill it with slab t + DEPTH
-                la[d].load(A, p.a_rs, p.a_cs, m0, p.M, k_first + (t + DEPTH) * BK, k_limit, tid);
-                lb[d].load(B, p.b_cs, p.b_rs, n0, p.N, k_first + (t + DEPTH) * BK, k_limit, tid);
-                // all operand fragments of the slab are read from LDS first, so the MFMAs issue
-                // back to back instead of each waiting for its own LDS round trip
-                T a[STEPS][FM], b[STEPS][FN];
+        for (int s = 0; s < STEPS; ++s) {
 #pragma unroll
-                for (int s = 0; s < STEPS; ++s) {
+            for (int i = 0; i < FM; ++i)
 #pragma unroll
-                    for (int i = 0; i < FM; ++i) a[s][i] = As[cur][ks0 + s * TK + op_k][wm0 + i * TM + op_x];
-#pragma unroll
-                    for (int j = 0; j < FN; ++j) b[s][j] = Bs[cur][ks0 + s * TK + op_k][wn0 + j * TM + op_x];
-                }
-#pragma unroll
-                for (int s = 0; s < STEPS; ++s)
-#pragma unroll
-                    for (int i = 0; i < FM; ++i)
-#pragma unroll
-                        for (int j = 0; j < FN; ++j) acc[i][j] = MF::mma(a[s][i], b[s][j], acc[i][j]);
-                if (t + 1 < n_slabs) {
-                    const int slot = (d + 1) % DEPTH;  // compile-time after unrolling
-                    la[slot].template store<BM + PAD_A>(As[cur ^ 1], tid);
-                    lb[slot].template store<BN + PAD_B>(Bs[cur ^ 1], tid);
-                }
-                __syncthreads();
+                for (int j = 0; j < FN; ++j) acc[i][j] = MF::mma(fa[cur][s][i], fb[cur][s][j], acc[i][j]);
+            // two fragment reads per MFMA in the first half of the step: every read has returned
+            // long before the wave reaches the barrier
+            if ((!guarded || t + 1 < n_slabs) && 2 * s < STEPS) {
+                read_fragment(cur ^ 1, cur ^ 1, 2 * s);
+                if (2 * s + 1 < STEPS) read_fragment(cur ^ 1, cur ^ 1, 2 * s + 1);
             }
+            if (s == 0) {
+                // slot d held slab t, which went to LDS two steps ago: refill it
+                la[d].load(A, p.a_rs, p.a_cs, m0, p.M, slab_k(t + DEPTH), k_limit, tid);
+                lb[d].load(B, p.b_cs, p.b_rs, n0, p.N, slab_k(t + DEPTH), k_limit, tid);
+            }
+            if (s == kStoreAt && (!guarded || t + 2 < n_slabs)) {
+                const int slot = (d + 2) % DEPTH;
+                la[slot].template store<BM + PAD_A>(As[cur], m0, p.M, slab_k(t + 2), k_limit, tid);
+                lb[slot].template store<BN + PAD_B>(Bs[cur], n0, p.N, slab_k(t + 2), k_limit, tid);
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
+    };
+    // main loop: groups of DEPTH steps that need no bounds tests form one straight-line block, so
+    // the count of loads in flight is known exactly at every wait; the last steps are guarded
+    int64_t t0 = 0;
+    for (; t0 + DEPTH + 2 <= n_slabs; t0 += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) step(d, t0 + d, false);
+    }
+    for (; t0 < n_slabs; t0 += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d)
+            if (t0 + d < n_slabs) step(d, t0 + d, true);  // uniform across the block
     }
 
     if (KS > 1) {
@@ -480,7 +520,7 @@ extern "C" int agmi_gemm(int dtype, int64_t batch, int64_t M, int64_t N, int64_t
         // give every CU two tiles (less L2 traffic per flop for large problems).
         const int64_t big_tiles = ceil_div(M, 128) * ceil_div(N, 128) * batch;
         if (big_tiles >= 512) return launch_gemm<MfmaF32x32, 128, 128, 16, 2, 1>(p, batch, s);
-        return launch_gemm<MfmaF32x32, 64, 64, 32, 4, 2>(p, batch, s, workspace, workspace_bytes);
+        return launch_gemm<MfmaF32x32, 64, 64, 32, 2, 2>(p, batch, s, workspace, workspace_bytes);
     }
     if (dtype == AGMI_F64) return launch_gemm<MfmaF64x16, 64, 64, 16, 2, 1>(p, batch, s, workspace, workspace_bytes);
     set_error("gemm: dtype %d is not a floating type", dtype);
