@@ -195,6 +195,13 @@ __global__ __launch_bounds__(kBlock) void red_row_block(const RedParams p) {
     if (threadIdx.x == 0) store_result<Acc, T, FINAL>(p, acc, o, 0, chunk);
 }
 
+// exp(d) for d <= 0 (or NaN) as a term of a sum that contains exp(0) = 1.  float: one v_exp_f32 on
+// d * log2(e); the rounding of that product perturbs the term by at most |d| e^d 2^-24 <= 0.37 * 2^-24
+// of the sum, below the rounding of the sum itself, and results under the normal range flush to
+// zero (they are below 1e-38 of the sum).  double: the library routine.
+__device__ __forceinline__ float exp_nonpositive(float d) { return __builtin_amdgcn_exp2f(d * 1.44269504088896340736f); }
+__device__ __forceinline__ double exp_nonpositive(double d) { return exp(d); }
+
 // ---- logsumexp of a row chunk held in registers ------------------------------------------------
 // The generic pair accumulator costs one exp per element on a serial dependency chain.  When a
 // row chunk fits in registers (<= 256 * V * ITERS elements) each thread instead takes the plain
@@ -234,7 +241,7 @@ __global__ __launch_bounds__(kBlock) void lse_row_block(const RedParams p) {
 #pragma unroll
         for (int it = 0; it < ITERS; ++it)
 #pragma unroll
-            for (int j = 0; j < V; ++j) s += m_exp(x[it][j] - m);
+            for (int j = 0; j < V; ++j) s += exp_nonpositive(x[it][j] - m);
     }
     typename Acc::type acc = {m, s};
     acc = block_reduce<Acc>(acc);
