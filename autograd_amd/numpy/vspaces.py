@@ -25,6 +25,16 @@ def _shared_zero(dtype):
     return z
 
 
+_ONES = {}
+
+
+def _shared_one(dtype):
+    o = _ONES.get(dtype)
+    if o is None:
+        o = _ONES[dtype] = D.ones((), dtype)
+    return o
+
+
 def is_broadcast_view(x):
     """True when some axis of extent > 1 has stride 0: several indices share one element."""
     t = x._h()
@@ -75,7 +85,12 @@ class DevArrayVSpace(VSpace):
         return DevArray(_shared_zero(self.dtype)._t.expand(self.shape), self.dtype)
 
     def ones(self):
-        return D.ones(self.shape, self.dtype)
+        """The seed cotangent of ``elementwise_grad`` (differential_operators.py:41-49 of the reference
+        seeds ``vs.ones()``): like ``zeros``, a stride-0 view of one shared element, so seeding a
+        backward pass writes nothing and the first rule reads the seed from a register."""
+        if self.size <= 1:
+            return D.ones(self.shape, self.dtype)
+        return DevArray(_shared_one(self.dtype)._t.expand(self.shape), self.dtype)
 
     def standard_basis(self):
         for idxs in onp.ndindex(*self.shape):
