@@ -146,13 +146,15 @@ def lib():
     L.agmi_take_rows.argtypes = [c_i, c_p, c_i64, c_i64, c_p, c_i64, c_p, c_p]
     L.agmi_scatter_add_rows.restype = c_i
     L.agmi_scatter_add_rows.argtypes = [c_i, c_p, c_i64, c_i64, c_p, c_p, c_p, c_p, c_i64, c_p]
+    L.agmi_optimizer_step.restype = c_i
+    L.agmi_optimizer_step.argtypes = [c_i, c_i, c_i, c_i64, c_p, c_p, c_p, c_p, c_p, p_d, c_p]
     _LIB = L
     return L
 
 
 EXPORTS = (
     "agmi_last_error agmi_version agmi_last_kernel agmi_elementwise agmi_compare agmi_cast agmi_map_reduce "
-    "agmi_map_reduce_workspace_bytes agmi_gemm agmi_fill agmi_take_rows agmi_scatter_add_rows"
+    "agmi_map_reduce_workspace_bytes agmi_gemm agmi_fill agmi_take_rows agmi_scatter_add_rows agmi_optimizer_step"
 ).split()
 
 
@@ -421,3 +423,25 @@ def scatter_add_rows(code, dst, n_rows, inner, src, index, order, seg_start, n_s
     _check(_LIB.agmi_scatter_add_rows(code, dst.data_ptr(), n_rows, inner, src.data_ptr(), index.data_ptr(),
                                       order.data_ptr(), seg_start.data_ptr(), n_seg, _stream()),
            "agmi_scatter_add_rows")
+
+
+OPT_SGD, OPT_RMSPROP, OPT_ADAM = 0, 1, 2
+_hyper = (ctypes.c_double * 8)()
+
+
+def optimizer_step(kind, x_in, g, s0, s1, x_out, hyper):
+    """One fused optimizer update on flat contiguous tensors (state and ``x_out`` float64)."""
+    n = x_in.numel()
+    for t in (x_in, g, s0, s1, x_out):
+        if t is not None and (t.numel() != n or not t.is_contiguous()):
+            raise AgmiError("optimizer_step: operands must be contiguous and of equal length")
+    _hyper[: len(hyper)] = hyper
+    ev = _TIMER.begin(("optimizer_step", kind)) if _TIMER is not None else None
+    rc = _LIB.agmi_optimizer_step(kind, DTYPE_CODE[NUMPY_DTYPE[x_in.dtype]], DTYPE_CODE[NUMPY_DTYPE[g.dtype]], n,
+                                  x_in.data_ptr(), g.data_ptr(), s0.data_ptr(), s1.data_ptr() if s1 is not None else None,
+                                  x_out.data_ptr(), _hyper, _stream())
+    if rc:
+        _check(rc, "agmi_optimizer_step")
+    if ev is not None:
+        _TIMER.end(ev, ("optimizer_step", kind), _traffic((x_out, s0) + ((s1,) if s1 is not None else ()),
+                                                           (x_in, g, s0) + ((s1,) if s1 is not None else ())))

@@ -1,0 +1,4 @@
+"""Helpers either side of the gradient evaluation: container flattening and optimizers
+(autograd/misc/__init__.py of the reference exports ``flatten``)."""
+
+from .flatten import flatten, flatten_func  # noqa: F401

@@ -119,6 +119,11 @@ class DevArrayVSpace(VSpace):
             acc = D.alias(y)
             acc._borrowed = True
             return acc
+        if isinstance(y, DevArray) and y.dtype != x.dtype and D.result_dtype(x, y) != x.dtype:
+            # numpy.add(x, y, out=x) of the reference (numpy_vspaces.py:33-34 through core.py:262-264)
+            # adds in the promoted dtype and stores in x's: a float64 cotangent accumulated into a
+            # float32 leaf comes out float32
+            return D.astype(self._add(x, y), x.dtype)
         if x._borrowed or type(x) is not DevArray or is_broadcast_view(x):
             return self._add(x, y)
         if isinstance(y, DevArray) and y.shape != x.shape and D.broadcast_shapes(x.shape, y.shape) != x.shape:

@@ -202,6 +202,20 @@ int agmi_scatter_add_rows(int dtype, void *dst, int64_t n_rows, int64_t inner,
                           const void *src, const int64_t *index, const int64_t *order,
                           const int64_t *seg_start, int64_t n_seg, void *stream);
 
+/* One fused update of a flat, contiguous parameter vector of n elements: the whole-array NumPy
+ * passes of the reference's optimizers (misc/optimizers.py: sgd 40-47, rmsprop 54-59, adam 66-75)
+ * in one pass, element arithmetic in the reference's order.
+ *   AGMI_OPT_SGD:     s0 = velocity;             hyper = {mass, 1-mass, step_size}
+ *   AGMI_OPT_RMSPROP: s0 = avg_sq_grad;          hyper = {gamma, 1-gamma, step_size, eps}
+ *   AGMI_OPT_ADAM:    s0 = m, s1 = v;            hyper = {1-b1, b1, 1-b2, b2, 1-b1**t, 1-b2**t, step_size, eps}
+ * x_in has dtype x_dtype, g has g_dtype (float32 or float64); the state arrays and x_out are
+ * float64, as in the reference (its state starts as np.zeros/np.ones, float64, and NumPy promotion
+ * carries that into the parameters).  State is updated in place; x_out may be x_in when x_dtype is
+ * float64. */
+enum agmi_optimizer { AGMI_OPT_SGD = 0, AGMI_OPT_RMSPROP = 1, AGMI_OPT_ADAM = 2 };
+int agmi_optimizer_step(int kind, int x_dtype, int g_dtype, int64_t n, const void *x_in, const void *g,
+                        void *s0, void *s1, void *x_out, const double *hyper, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,69 @@
+"""Small seeded cases for the components either side of the hot path: container flattening,
+optimizers, Jacobians/Hessians, and the rest of the elementwise rule table.
+
+``next_cases(be, ext)`` is written against a ``configs.Backend`` plus a namespace ``ext`` with
+``flatten, sgd, rmsprop, adam, jacobian, hessian`` so the same code runs on the reference (when
+writing fixtures), the CPU oracle and the device.
+"""
+
+import numpy as onp
+
+
+def _params(rs, P):
+    return {
+        "layers": [(P((0.3 * rs.randn(4, 3)).astype(onp.float32)), P(onp.zeros(3, onp.float32))),
+                   (P((0.3 * rs.randn(3, 2)).astype(onp.float32)), P((0.1 * rs.randn(2)).astype(onp.float32)))],
+        "scale": P(onp.asarray(1.5)),
+    }
+
+
+def next_cases(be, ext):
+    np, grad, P = be.np, be.grad, be.put
+    rs = onp.random.RandomState(11)
+    out = {}
+
+    # ---- flatten / unflatten (misc/flatten.py:11-35) ------------------------------------------
+    params = _params(rs, P)
+    flat, unflatten = ext.flatten(params)
+    out["flatten/flat"] = flat
+    out["flatten/roundtrip"] = unflatten(flat * 2.0)
+    out["flatten/grad"] = grad(lambda p: np.sum(ext.flatten(p)[0] ** 2))(params)
+    f32 = [P(rs.randn(3).astype(onp.float32)), (P(rs.randn(2, 2).astype(onp.float32)),)]
+    flat32, un32 = ext.flatten(f32)
+    out["flatten/f32_flat"] = flat32
+    out["flatten/f32_roundtrip"] = un32(flat32)
+
+    # ---- optimizers (misc/optimizers.py:33-75) on a small two-layer regression ---------------------
+    X = P(rs.randn(5, 4).astype(onp.float32))
+    Y = P(rs.randn(5, 2).astype(onp.float32))
+
+    def loss(p, i):
+        h = np.tanh(np.dot(X, p["layers"][0][0]) + p["layers"][0][1])
+        y = np.dot(h, p["layers"][1][0]) + p["layers"][1][1]
+        return np.sum((y * p["scale"] - Y) ** 2) * (1.0 + 0.1 * i)
+
+    seen = {}
+
+    def callback(x, i, g):
+        if i == 2:
+            seen["x"], seen["g"] = x, g
+
+    out["opt/sgd"] = ext.sgd(grad(loss), params, num_iters=4, step_size=0.05, mass=0.8)
+    out["opt/rmsprop"] = ext.rmsprop(grad(loss), params, num_iters=4, step_size=0.02)
+    out["opt/adam"] = ext.adam(grad(loss), params, callback=callback, num_iters=5, step_size=0.01)
+    out["opt/adam_callback_x"] = seen["x"]
+    out["opt/adam_callback_g"] = seen["g"]
+    # float64 parameters from the start
+    p64 = [P(rs.randn(6)), P(rs.randn(2, 3))]
+    q = lambda p, i: np.sum(np.sin(p[0]) * np.sum(p[1] ** 2)) + np.sum(p[1])  # noqa: E731
+    out["opt/adam_f64"] = ext.adam(grad(q), p64, num_iters=3)
+    out["opt/sgd_f64"] = ext.sgd(grad(q), p64, num_iters=3)
+    out["opt/rmsprop_f64"] = ext.rmsprop(grad(q), p64, num_iters=3)
+
+    # ---- jacobian / hessian (differential_operators.py:57-91) -------------------------------------
+    A = P(rs.randn(3, 4))
+    x = P(rs.randn(4))
+    out["jac/matvec"] = ext.jacobian(lambda v: np.tanh(np.dot(A, v)))(x)
+    out["jac/matrix_in"] = ext.jacobian(lambda M: np.dot(M, x) ** 2)(A)
+    out["hess/quartic"] = ext.hessian(lambda v: np.sum(np.dot(A, v) ** 4) + np.sum(np.sin(v) * v))(x)
+    return out
