@@ -40,6 +40,52 @@ __device__ __forceinline__ double m_abs(double x) { return fabs(x); }
 __device__ __forceinline__ float m_pow(float x, float y) { return powf(x, y); }
 __device__ __forceinline__ double m_pow(double x, double y) { return pow(x, y); }
 
+__device__ __forceinline__ float m_exp2(float x) { return exp2f(x); }
+__device__ __forceinline__ double m_exp2(double x) { return exp2(x); }
+__device__ __forceinline__ float m_log2(float x) { return log2f(x); }
+__device__ __forceinline__ double m_log2(double x) { return log2(x); }
+__device__ __forceinline__ float m_log10(float x) { return log10f(x); }
+__device__ __forceinline__ double m_log10(double x) { return log10(x); }
+__device__ __forceinline__ float m_tan(float x) { return tanf(x); }
+__device__ __forceinline__ double m_tan(double x) { return tan(x); }
+__device__ __forceinline__ float m_asin(float x) { return asinf(x); }
+__device__ __forceinline__ double m_asin(double x) { return asin(x); }
+__device__ __forceinline__ float m_acos(float x) { return acosf(x); }
+__device__ __forceinline__ double m_acos(double x) { return acos(x); }
+__device__ __forceinline__ float m_atan(float x) { return atanf(x); }
+__device__ __forceinline__ double m_atan(double x) { return atan(x); }
+__device__ __forceinline__ float m_asinh(float x) { return asinhf(x); }
+__device__ __forceinline__ double m_asinh(double x) { return asinh(x); }
+__device__ __forceinline__ float m_acosh(float x) { return acoshf(x); }
+__device__ __forceinline__ double m_acosh(double x) { return acosh(x); }
+__device__ __forceinline__ float m_atanh(float x) { return atanhf(x); }
+__device__ __forceinline__ double m_atanh(double x) { return atanh(x); }
+__device__ __forceinline__ float m_atan2(float y, float x) { return atan2f(y, x); }
+__device__ __forceinline__ double m_atan2(double y, double x) { return atan2(y, x); }
+__device__ __forceinline__ float m_hypot(float x, float y) { return hypotf(x, y); }
+__device__ __forceinline__ double m_hypot(double x, double y) { return hypot(x, y); }
+
+// numpy.logaddexp (npy_math: equal operands -> x + log 2; otherwise the larger one plus log1p of
+// the exponential of the negative distance; a NaN distance is returned as it is)
+template <typename T>
+__device__ __forceinline__ T logaddexp_like_numpy(T x, T y) {
+    if (x == y) return x + T(0.693147180559945309417232121458176568);
+    const T d = x - y;
+    if (d > T(0)) return x + m_log1p(m_exp(-d));
+    if (d <= T(0)) return y + m_log1p(m_exp(d));
+    return d;
+}
+
+// numpy.fmax / fmin: a NaN operand is ignored when the other one is a number
+template <typename T>
+__device__ __forceinline__ T fmax_like_numpy(T a, T b) {
+    return (a >= b || b != b) ? a : b;
+}
+template <typename T>
+__device__ __forceinline__ T fmin_like_numpy(T a, T b) {
+    return (a <= b || b != b) ? a : b;
+}
+
 // x**y with the exponents NumPy short-cuts (1, 2, 0, -1, 0.5) computed the same exact way.
 template <typename T>
 __device__ __forceinline__ T pow_like_numpy(T x, T y) {
@@ -86,6 +132,17 @@ AGMI_FUNCTOR(FReciprocal, 1, 1, o[0] = T(1) / x[0];)
 AGMI_FUNCTOR(FLog1p, 1, 1, o[0] = m_log1p(x[0]);)
 AGMI_FUNCTOR(FExpm1, 1, 1, o[0] = m_expm1(x[0]);)
 
+AGMI_FUNCTOR(FExp2, 1, 1, o[0] = m_exp2(x[0]);)
+AGMI_FUNCTOR(FLog2, 1, 1, o[0] = m_log2(x[0]);)
+AGMI_FUNCTOR(FLog10, 1, 1, o[0] = m_log10(x[0]);)
+AGMI_FUNCTOR(FTan, 1, 1, o[0] = m_tan(x[0]);)
+AGMI_FUNCTOR(FArcsin, 1, 1, o[0] = m_asin(x[0]);)
+AGMI_FUNCTOR(FArccos, 1, 1, o[0] = m_acos(x[0]);)
+AGMI_FUNCTOR(FArctan, 1, 1, o[0] = m_atan(x[0]);)
+AGMI_FUNCTOR(FArcsinh, 1, 1, o[0] = m_asinh(x[0]);)
+AGMI_FUNCTOR(FArccosh, 1, 1, o[0] = m_acosh(x[0]);)
+AGMI_FUNCTOR(FArctanh, 1, 1, o[0] = m_atanh(x[0]);)
+
 AGMI_FUNCTOR(FAdd, 2, 1, o[0] = x[0] + x[1];)
 AGMI_FUNCTOR(FSub, 2, 1, o[0] = x[0] - x[1];)
 AGMI_FUNCTOR(FMul, 2, 1, o[0] = x[0] * x[1];)
@@ -93,6 +150,12 @@ AGMI_FUNCTOR(FDiv, 2, 1, o[0] = x[0] / x[1];)
 AGMI_FUNCTOR(FPow, 2, 1, o[0] = pow_like_numpy(x[0], x[1]);)
 AGMI_FUNCTOR(FMaximum, 2, 1, o[0] = max_nan(x[0], x[1]);)
 AGMI_FUNCTOR(FMinimum, 2, 1, o[0] = min_nan(x[0], x[1]);)
+
+AGMI_FUNCTOR(FFmax, 2, 1, o[0] = fmax_like_numpy(x[0], x[1]);)
+AGMI_FUNCTOR(FFmin, 2, 1, o[0] = fmin_like_numpy(x[0], x[1]);)
+AGMI_FUNCTOR(FArctan2, 2, 1, o[0] = m_atan2(x[0], x[1]);)
+AGMI_FUNCTOR(FHypot, 2, 1, o[0] = m_hypot(x[0], x[1]);)
+AGMI_FUNCTOR(FLogaddexp, 2, 1, o[0] = logaddexp_like_numpy(x[0], x[1]);)
 
 AGMI_FUNCTOR(FWhere, 3, 1, o[0] = (x[0] != T(0)) ? x[1] : x[2];)
 
@@ -146,6 +209,16 @@ AGMI_FUNCTOR(FMulAdd, 3, 1, T t = x[0] * x[1]; o[0] = t + x[2];)
     X(AGMI_OP_RECIPROCAL, FReciprocal)          \
     X(AGMI_OP_LOG1P, FLog1p)                    \
     X(AGMI_OP_EXPM1, FExpm1)                    \
+    X(AGMI_OP_EXP2, FExp2)                      \
+    X(AGMI_OP_LOG2, FLog2)                      \
+    X(AGMI_OP_LOG10, FLog10)                    \
+    X(AGMI_OP_TAN, FTan)                        \
+    X(AGMI_OP_ARCSIN, FArcsin)                  \
+    X(AGMI_OP_ARCCOS, FArccos)                  \
+    X(AGMI_OP_ARCTAN, FArctan)                  \
+    X(AGMI_OP_ARCSINH, FArcsinh)                \
+    X(AGMI_OP_ARCCOSH, FArccosh)                \
+    X(AGMI_OP_ARCTANH, FArctanh)                \
     X(AGMI_OP_ADD, FAdd)                        \
     X(AGMI_OP_SUB, FSub)                        \
     X(AGMI_OP_MUL, FMul)                        \
@@ -153,6 +226,11 @@ AGMI_FUNCTOR(FMulAdd, 3, 1, T t = x[0] * x[1]; o[0] = t + x[2];)
     X(AGMI_OP_POW, FPow)                        \
     X(AGMI_OP_MAXIMUM, FMaximum)                \
     X(AGMI_OP_MINIMUM, FMinimum)                \
+    X(AGMI_OP_FMAX, FFmax)                      \
+    X(AGMI_OP_FMIN, FFmin)                      \
+    X(AGMI_OP_ARCTAN2, FArctan2)                \
+    X(AGMI_OP_HYPOT, FHypot)                    \
+    X(AGMI_OP_LOGADDEXP, FLogaddexp)            \
     X(AGMI_OP_WHERE, FWhere)                    \
     X(AGMI_OP_DIV_VJP1, FDivVjp1)               \
     X(AGMI_OP_TANH_VJP, FTanhVjp)               \

@@ -77,7 +77,7 @@ defjvp(
     lambda g, ans, x, y: _fused_or(Op.POW_VJP0, (g, x, y), lambda: g * y * x ** anp.where(y, y - 1, 1.0)),
     lambda g, ans, x, y: _fused_or(Op.POW_VJP1, (g, x, ans), lambda: g * anp.log(replace_zero(x, 1.0)) * ans),
 )
-for _chooser in (anp.maximum, anp.minimum):
+for _chooser in (anp.maximum, anp.minimum, anp.fmax, anp.fmin):
     defjvp(
         _chooser,
         lambda g, ans, x, y: g * balanced_eq(x, ans, y),
@@ -110,6 +110,25 @@ defjvp(
         Op.ABS_VJP, (g, x, ans), lambda: g * replace_zero(x, 0.0) / replace_zero(ans, 1.0)
     ),
 )
+# the rest of the table (numpy_jvps.py:63-73, 108-147)
+defjvp(anp.logaddexp, lambda g, ans, x, y: g * anp.exp(x - ans), lambda g, ans, x, y: g * anp.exp(y - ans))
+defjvp(anp.arctan2, lambda g, ans, x, y: g * y / (x**2 + y**2), lambda g, ans, x, y: g * -x / (x**2 + y**2))
+defjvp(anp.hypot, lambda g, ans, x, y: g * x / ans, lambda g, ans, x, y: g * y / ans)
+defjvp(anp.fabs, lambda g, ans, x: anp.sign(x) * g)
+defjvp(anp.exp2, lambda g, ans, x: ans * anp.log(2) * g)
+defjvp(anp.log2, lambda g, ans, x: g / x / anp.log(2))
+defjvp(anp.log10, lambda g, ans, x: g / x / anp.log(10))
+defjvp(anp.tan, lambda g, ans, x: g / anp.cos(x) ** 2)
+defjvp(anp.arcsin, lambda g, ans, x: g / anp.sqrt(1 - x**2))
+defjvp(anp.arccos, lambda g, ans, x: -g / anp.sqrt(1 - x**2))
+defjvp(anp.arctan, lambda g, ans, x: g / (1 + x**2))
+defjvp(anp.arcsinh, lambda g, ans, x: g / anp.sqrt(x**2 + 1))
+defjvp(anp.arccosh, lambda g, ans, x: g / anp.sqrt(x**2 - 1))
+defjvp(anp.arctanh, lambda g, ans, x: g / (1 - x**2))
+defjvp(anp.rad2deg, lambda g, ans, x: g / anp.pi * 180.0)
+defjvp(anp.deg2rad, lambda g, ans, x: g * anp.pi / 180.0)
+defjvp(anp.clip, lambda g, ans, x, a_min, a_max: g * anp.logical_and(ans != a_min, ans != a_max))
+
 defjvp(
     anp._where3,
     None,

@@ -38,6 +38,9 @@ for _f in nograd_functions:
     register_notrace(VJPNode, _f)
 
 
+_F64 = onp.dtype("float64")
+
+
 def _concrete(*xs):
     """True when no argument is a box: the fused kernels may be used."""
     for x in xs:
@@ -110,8 +113,13 @@ def _binary_rule(fun, traced0, traced1, fused0, fused1):
 
             def vjp(g):
                 if _concrete(g, ans, x, y):
-                    op, operands = fused(g, ans, x, y)
-                    return _fused_unbroadcast(op, meta, *operands)
+                    op, operands, *promote = fused(g, ans, x, y)
+                    out = _fused_unbroadcast(op, meta, *operands)
+                    if promote and out.dtype != promote[0]:
+                        # the reference's expression has a float64 factor (see the rule): same
+                        # values, NumPy's result dtype
+                        out = D.astype(out, promote[0])
+                    return out
                 return unbroadcast(slow(g), meta)
 
             return vjp
@@ -157,13 +165,15 @@ _binary_rule(
     lambda g, ans, x, y: (Op.POW_VJP0, (g, x, y)),
     lambda g, ans, x, y: (Op.POW_VJP1, (g, x, ans)),
 )
-for _chooser in (anp.maximum, anp.minimum):
+for _chooser in (anp.maximum, anp.minimum, anp.fmax, anp.fmin):
     _binary_rule(
         _chooser,
         lambda ans, x, y: lambda g: g * balanced_eq(x, ans, y),
         lambda ans, x, y: lambda g: g * balanced_eq(y, ans, x),
-        lambda g, ans, x, y: (Op.CHOOSE_VJP, (g, x, ans, y)),
-        lambda g, ans, x, y: (Op.CHOOSE_VJP, (g, y, ans, x)),
+        # balanced_eq divides a bool array by a float64 one, so `g * balanced_eq(...)` is float64
+        # whatever g is; its factors 0, 1/2, 1 are exact in any precision
+        lambda g, ans, x, y: (Op.CHOOSE_VJP, (g, x, ans, y), _F64),
+        lambda g, ans, x, y: (Op.CHOOSE_VJP, (g, y, ans, x), _F64),
     )
 
 def balanced_eq(x, z, y):
@@ -210,6 +220,37 @@ _unary_rule(
     lambda ans, x: lambda g: g * replace_zero(x, 0.0) / replace_zero(ans, 1.0),
     lambda g, ans, x: (Op.ABS_VJP, (g, x, ans)),
 )
+
+# the rest of the table (numpy_vjps.py:114-135, 160-185, 215): reference compositions, one launch per primitive
+defvjp(
+    anp.logaddexp,
+    lambda ans, x, y: unbroadcast_f(x, lambda g: g * anp.exp(x - ans)),
+    lambda ans, x, y: unbroadcast_f(y, lambda g: g * anp.exp(y - ans)),
+)
+defvjp(
+    anp.arctan2,
+    lambda ans, x, y: unbroadcast_f(x, lambda g: g * y / (x**2 + y**2)),
+    lambda ans, x, y: unbroadcast_f(y, lambda g: g * -x / (x**2 + y**2)),
+)
+defvjp(
+    anp.hypot,
+    lambda ans, x, y: unbroadcast_f(x, lambda g: g * x / ans),
+    lambda ans, x, y: unbroadcast_f(y, lambda g: g * y / ans),
+)
+defvjp(anp.fabs, lambda ans, x: lambda g: anp.sign(x) * g)
+defvjp(anp.exp2, lambda ans, x: lambda g: ans * anp.log(2) * g)
+defvjp(anp.log2, lambda ans, x: lambda g: g / x / anp.log(2))
+defvjp(anp.log10, lambda ans, x: lambda g: g / x / anp.log(10))
+defvjp(anp.tan, lambda ans, x: lambda g: g / anp.cos(x) ** 2)
+defvjp(anp.arcsin, lambda ans, x: lambda g: g / anp.sqrt(1 - x**2))
+defvjp(anp.arccos, lambda ans, x: lambda g: -g / anp.sqrt(1 - x**2))
+defvjp(anp.arctan, lambda ans, x: lambda g: g / (1 + x**2))
+defvjp(anp.arcsinh, lambda ans, x: lambda g: g / anp.sqrt(x**2 + 1))
+defvjp(anp.arccosh, lambda ans, x: lambda g: g / anp.sqrt(x**2 - 1))
+defvjp(anp.arctanh, lambda ans, x: lambda g: g / (1 - x**2))
+defvjp(anp.rad2deg, lambda ans, x: lambda g: g / anp.pi * 180.0)
+defvjp(anp.deg2rad, lambda ans, x: lambda g: g * anp.pi / 180.0)
+defvjp(anp.clip, lambda ans, x, a_min, a_max: lambda g: g * anp.logical_and(ans != a_min, ans != a_max))
 
 defvjp(
     anp._where3,

@@ -50,6 +50,20 @@ sqrt = _unary(Op.SQRT, "sqrt")
 log1p = _unary(Op.LOG1P, "log1p")
 expm1 = _unary(Op.EXPM1, "expm1")
 reciprocal = _unary(Op.RECIPROCAL, "reciprocal")
+exp2 = _unary(Op.EXP2, "exp2")
+log2 = _unary(Op.LOG2, "log2")
+log10 = _unary(Op.LOG10, "log10")
+tan = _unary(Op.TAN, "tan")
+arcsin = _unary(Op.ARCSIN, "arcsin")
+arccos = _unary(Op.ARCCOS, "arccos")
+arctan = _unary(Op.ARCTAN, "arctan")
+arcsinh = _unary(Op.ARCSINH, "arcsinh")
+arccosh = _unary(Op.ARCCOSH, "arccosh")
+arctanh = _unary(Op.ARCTANH, "arctanh")
+fabs = _wrap(lambda x: D.float_map(Op.ABS, x), "fabs")
+# numpy's loops multiply by the constant 180/pi resp. pi/180
+rad2deg = degrees = _wrap(lambda x: D.float_map(Op.MUL, x, 180.0 / onp.pi), "rad2deg")
+deg2rad = radians = _wrap(lambda x: D.float_map(Op.MUL, x, onp.pi / 180.0), "deg2rad")
 square = _wrap(lambda x: D.arith_map(Op.SQUARE, x), "square")
 abs = absolute = _wrap(lambda x: D.arith_map(Op.ABS, x), "abs")  # noqa: A001
 sign = _wrap(lambda x: D.arith_map(Op.SIGN, x), "sign")
@@ -71,6 +85,19 @@ divide = true_divide = _binary(Op.DIV, "true_divide", floating=True)
 power = _binary(Op.POW, "power")
 maximum = _binary(Op.MAXIMUM, "maximum")
 minimum = _binary(Op.MINIMUM, "minimum")
+fmax = _binary(Op.FMAX, "fmax")
+fmin = _binary(Op.FMIN, "fmin")
+arctan2 = _binary(Op.ARCTAN2, "arctan2", floating=True)
+hypot = _binary(Op.HYPOT, "hypot", floating=True)
+logaddexp = _binary(Op.LOGADDEXP, "logaddexp", floating=True)
+
+
+@primitive
+def clip(a, a_min, a_max):
+    """``numpy.clip`` with scalar or array bounds: minimum(maximum(a, a_min), a_max)."""
+    a = D.asarray(a)
+    dt = D._float_dtype(D.result_dtype(a, a_min, a_max))
+    return D.map_op(Op.MINIMUM, dt, D.map_op(Op.MAXIMUM, dt, a, a_min), a_max)
 
 
 def _compare(cmp, name):

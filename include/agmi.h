@@ -83,6 +83,16 @@ typedef enum agmi_op {
     AGMI_OP_RECIPROCAL,
     AGMI_OP_LOG1P,
     AGMI_OP_EXPM1,
+    AGMI_OP_EXP2,     /* the rest of the unary ufunc table, numpy_vjps.py:164-182 (forward passes) */
+    AGMI_OP_LOG2,
+    AGMI_OP_LOG10,
+    AGMI_OP_TAN,
+    AGMI_OP_ARCSIN,
+    AGMI_OP_ARCCOS,
+    AGMI_OP_ARCTAN,
+    AGMI_OP_ARCSINH,
+    AGMI_OP_ARCCOSH,
+    AGMI_OP_ARCTANH,
     /* two inputs */
     AGMI_OP_ADD = 32, /* also VSpace._add / _mut_add, autograd/core.py:259-264 (out may alias in0) */
     AGMI_OP_SUB,
@@ -91,6 +101,11 @@ typedef enum agmi_op {
     AGMI_OP_POW,
     AGMI_OP_MAXIMUM,
     AGMI_OP_MINIMUM,
+    AGMI_OP_FMAX,     /* NaN-ignoring choosers        numpy_vjps.py:104-113                     */
+    AGMI_OP_FMIN,
+    AGMI_OP_ARCTAN2,  /* (y, x)                       numpy_vjps.py:131-135                     */
+    AGMI_OP_HYPOT,
+    AGMI_OP_LOGADDEXP,/* numpy_vjps.py:114-118 */
     /* three inputs */
     AGMI_OP_WHERE = 64, /* c != 0 ? x : y  (c in the array dtype)                             */
     /* fused derivative rules; inputs in the order listed */

@@ -17,6 +17,7 @@ add subtract multiply divide true_divide power negative positive mod remainder
 exp exp2 expm1 log log2 log10 log1p sin cos tan sinh cosh tanh arcsin arccos arctan
 arcsinh arccosh arctanh sqrt square abs absolute fabs reciprocal sign maximum minimum
 fmax fmin logaddexp hypot arctan2 where clip nan_to_num real imag conj conjugate
+rad2deg degrees deg2rad radians
 sum mean prod max min amax amin var std cumsum
 reshape ravel expand_dims squeeze transpose swapaxes moveaxis atleast_1d atleast_2d
 atleast_3d repeat tile broadcast_to roll flipud fliplr diag diagonal trace tril triu

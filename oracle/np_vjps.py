@@ -142,6 +142,11 @@ _unary = {
 }
 for _name, _maker in _unary.items():
     defvjp(getattr(anp, _name), _maker)
+# numpy_vjps.py:182-185
+defvjp(anp.rad2deg, lambda ans, x: lambda g: g / anp.pi * 180.0)
+defvjp(anp.degrees, lambda ans, x: lambda g: g / anp.pi * 180.0)
+defvjp(anp.deg2rad, lambda ans, x: lambda g: g * anp.pi / 180.0)
+defvjp(anp.radians, lambda ans, x: lambda g: g * anp.pi / 180.0)
 
 # ---- shape-only functions (numpy_vjps.py:192-217, 407-413, 804-812) ---------------
 defvjp(anp.reshape, lambda ans, x, shape, order=None: lambda g: anp.reshape(g, anp.shape(x), order=order))

@@ -66,4 +66,30 @@ def next_cases(be, ext):
     out["jac/matvec"] = ext.jacobian(lambda v: np.tanh(np.dot(A, v)))(x)
     out["jac/matrix_in"] = ext.jacobian(lambda M: np.dot(M, x) ** 2)(A)
     out["hess/quartic"] = ext.hessian(lambda v: np.sum(np.dot(A, v) ** 4) + np.sum(np.sin(v) * v))(x)
+
+    # ---- the rest of the elementwise rule table (numpy_vjps.py:104-135, 160-185, 215) ------------------
+    u = rs.uniform(0.1, 0.9, (3, 4))          # inside every domain below
+    w = rs.uniform(1.1, 3.0, (3, 4))
+    for dtype in (onp.float64, onp.float32):
+        tag = "f32" if dtype == onp.float32 else "f64"
+        U, W = P(u.astype(dtype)), P(w.astype(dtype))
+        for name in "exp2 log2 log10 tan arcsin arccos arctan arcsinh arctanh fabs rad2deg deg2rad".split():
+            f = getattr(np, name)
+            out[f"ufunc/{name}_{tag}/value"] = f(U)
+            out[f"ufunc/{name}_{tag}/grad"] = grad(lambda z: np.sum(f(z) * W))(U)
+        out[f"ufunc/arccosh_{tag}/grad"] = grad(lambda z: np.sum(np.arccosh(z) * U))(W)
+        row = P(rs.uniform(0.2, 2.0, (1, 4)).astype(dtype))
+        for name in "fmax fmin arctan2 hypot logaddexp".split():
+            f = getattr(np, name)
+            out[f"ufunc/{name}_{tag}/value"] = f(U, row)
+            out[f"ufunc/{name}_{tag}/grad"] = grad(lambda a, b: np.sum(f(a, b) * W), (0, 1))(U, row)
+        out[f"ufunc/clip_{tag}/grad"] = grad(lambda z: np.sum(np.clip(z, 0.3, 0.6) * W))(U)
+        # single-argument grads keep the dtype the rule produces (no container accumulation casts it back)
+        out[f"ufunc/maximum_{tag}/grad_single"] = grad(lambda z: np.sum(np.maximum(z, 0.5) * W))(U)
+        out[f"ufunc/fmin_{tag}/grad_single"] = grad(lambda z: np.sum(np.fmin(z, row) * W))(U)
+    second = P(rs.uniform(0.2, 0.8, 5))
+    out["ufunc/second_order"] = grad(lambda z: np.sum(grad(lambda t: np.sum(np.arctan(t) * np.log2(t) + np.tan(t)))(z)))(second)
+    tie = P(onp.array([1.0, 2.0, 2.0, onp.nan, 3.0]))
+    other = P(onp.array([1.0, 1.0, 3.0, 2.0, onp.nan]))
+    out["ufunc/fmax_ties_nan"] = grad(lambda a, b: np.sum(np.fmax(a, b) * P(onp.arange(1.0, 6.0))), (0, 1))(tie, other)
     return out

@@ -50,7 +50,44 @@ UNARY = [
     ("sinh", onp.sinh, False), ("cosh", onp.cosh, False), ("sin", onp.sin, False), ("cos", onp.cos, False),
     ("sqrt", onp.sqrt, True), ("square", onp.square, False), ("abs", onp.abs, False), ("sign", onp.sign, False),
     ("reciprocal", onp.reciprocal, True), ("log1p", onp.log1p, True), ("expm1", onp.expm1, False),
+    ("exp2", onp.exp2, False), ("log2", onp.log2, True), ("log10", onp.log10, True), ("tan", onp.tan, False),
+    ("arctan", onp.arctan, False), ("arcsinh", onp.arcsinh, False), ("fabs", onp.fabs, False),
+    ("rad2deg", onp.rad2deg, False), ("deg2rad", onp.deg2rad, False), ("degrees", onp.degrees, False),
 ]
+
+
+@pytest.mark.parametrize("dtype", [F32, F64])
+def test_unary_bounded_domains(dnp, dtype):
+    rs = onp.random.RandomState(4)
+    inside = (rs.rand(1031) * 1.9 - 0.95).astype(dtype)     # (-1, 1)
+    above = (rs.rand(1031) * 5 + 1.01).astype(dtype)        # (1, 6)
+    for name, x in (("arcsin", inside), ("arccos", inside), ("arctanh", inside), ("arccosh", above)):
+        close(getattr(dnp, name)(P(dnp, x)).numpy(), getattr(onp, name)(x), RT_EW[dtype] * 8)
+    edge = onp.array([0.0, -0.0, 1.0, -1.0, 2.0, onp.nan, onp.inf, -onp.inf], dtype)
+    with onp.errstate(all="ignore"):
+        for name in ("arcsin", "arccos", "arctanh", "arccosh", "log2", "exp2", "arctan", "tan"):
+            close(getattr(dnp, name)(P(dnp, edge)).numpy(), getattr(onp, name)(edge), RT_EW[dtype] * 8)
+
+
+@pytest.mark.parametrize("dtype", [F32, F64])
+def test_fmax_fmin_clip_and_two_argument_functions(dnp, dtype):
+    rs = onp.random.RandomState(5)
+    a, b = rs.randn(37, 29).astype(dtype), rs.randn(29).astype(dtype)
+    a[0, :3] = onp.nan
+    b[2] = onp.nan
+    A, B = P(dnp, a), P(dnp, b)
+    for name in ("fmax", "fmin", "maximum", "minimum"):          # NaN handling differs between the pairs
+        assert onp.array_equal(getattr(dnp, name)(A, B).numpy(), getattr(onp, name)(a, b), equal_nan=True), name
+    assert onp.array_equal(dnp.clip(A, -0.5, 0.25).numpy(), onp.clip(a, -0.5, 0.25), equal_nan=True)
+    lo = (rs.randn(29) - 1).astype(dtype)
+    assert onp.array_equal(dnp.clip(A, P(dnp, lo), 0.25).numpy(), onp.clip(a, lo, 0.25), equal_nan=True)
+    x, y = rs.randn(37, 29).astype(dtype), rs.randn(37, 1).astype(dtype)
+    for name in ("arctan2", "hypot", "logaddexp"):
+        close(getattr(dnp, name)(P(dnp, x), P(dnp, y)).numpy(), getattr(onp, name)(x, y), RT_EW[dtype] * 8)
+    big = onp.array([1000.0, -1000.0, 5.0, onp.inf, -onp.inf, onp.nan], dtype)
+    oth = onp.array([1000.0, 3.0, 5.0, 1.0, -onp.inf, 1.0], dtype)
+    with onp.errstate(all="ignore"):
+        close(dnp.logaddexp(P(dnp, big), P(dnp, oth)).numpy(), onp.logaddexp(big, oth), RT_EW[dtype] * 8)
 
 
 @pytest.mark.parametrize("dtype", [F32, F64])
