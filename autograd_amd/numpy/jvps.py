@@ -84,6 +84,8 @@ for _chooser in (anp.maximum, anp.minimum, anp.fmax, anp.fmin):
         lambda g, ans, x, y: g * balanced_eq(y, ans, x),
     )
 
+def_linear(anp.einsum)  # numpy_jvps.py:287
+
 # linear one-argument functions (77-105, 150-162)
 for _name in (
     "negative reshape ravel expand_dims squeeze swapaxes moveaxis broadcast_to repeat transpose sum "

@@ -614,6 +614,42 @@ defvjp(
 )
 
 
+# ---- einsum (numpy_vjps.py:815-860, subscript-string convention) ------------------------------------
+def _grad_einsum(argnum, ans, operands_, kwargs):
+    result_meta = anp.metadata(operands_[argnum])
+
+    def vjp(g):
+        operands = operands_
+        in_subs, out_subs, _ = anp.parse_einsum_input(*operands)
+        operands = operands[1:]
+        in_subs_list = in_subs.split(",")
+        op_num = argnum - 1
+        subs_wrt = in_subs_list[op_num]
+        rest_of_ops = operands[:op_num] + operands[op_num + 1 :]
+        rest_of_subs = in_subs_list[:op_num] + in_subs_list[op_num + 1 :]
+        # subscripts that appear only in subs_wrt are summed out in the forward pass, as if contracted
+        # against a tensor of ones; the reference makes that tensor explicit for the broadcast back
+        other_named_subs = set("".join([out_subs] + rest_of_subs))
+        naked_summed = [(i, sub) for i, sub in enumerate(subs_wrt) if sub not in other_named_subs]
+        if naked_summed:
+            naked_summed_dims, ones_subs = zip(*naked_summed)
+            ones_subs = "".join(ones_subs)
+            wrt_shape = anp.shape(operands[op_num])
+            ones = anp.ones(tuple(wrt_shape[d] for d in naked_summed_dims))
+            new_input_subs = ",".join([out_subs, ones_subs] + rest_of_subs)
+            new_operands = (g, ones) + rest_of_ops
+        else:
+            new_input_subs = ",".join([out_subs] + rest_of_subs)
+            new_operands = (g,) + rest_of_ops
+        new_subscripts = new_input_subs + "->" + subs_wrt
+        return unbroadcast(anp.einsum(new_subscripts, *new_operands), result_meta)
+
+    return vjp
+
+
+defvjp_argnum(anp.einsum, _grad_einsum)
+
+
 # ---- concatenate / array construction (numpy_vjps.py:750-759, 922-938) -----------------------
 def _grad_concatenate_args(argnum, ans, axis_args, kwargs):
     axis, args = axis_args[0], axis_args[1:]

@@ -705,6 +705,102 @@ def outer(a, b):
     return D.arith_map(Op.MUL, DevArray(a._t.unsqueeze(1), a.dtype), DevArray(b._t.unsqueeze(0), b.dtype))
 
 
+# ---- einsum (subscript-string convention) -> sums, permutations and batched MFMA GEMMs ----------------
+def parse_einsum_input(*args):
+    """NumPy's own subscript parser (the reference wraps the same routine, numpy_wrapper.py:194-195)
+    run on shape-only stand-ins, so no operand is copied to the host."""
+    try:
+        from numpy._core.einsumfunc import _parse_einsum_input
+    except ImportError:  # NumPy 1.x
+        from numpy.core.einsumfunc import _parse_einsum_input
+    from ..tracer import getval
+
+    if not isinstance(args[0], str):
+        raise NotImplementedError("einsum: only the subscript-string convention is supported on the device")
+    stand_ins = [onp.broadcast_to(onp.zeros((), onp.float32), shape(getval(a))) for a in args[1:]]
+    in_subs, out_subs, _ = _parse_einsum_input([args[0]] + stand_ins)
+    return in_subs, out_subs, args[1:]
+
+
+def _einsum_sum_out(x, subs, drop):
+    """Sum the axes of ``x`` labelled by the letters in ``drop``."""
+    axes = tuple(i for i, c in enumerate(subs) if c in drop)
+    if not axes:
+        return x, subs
+    x = D.map_reduce(Op.COPY, Red.SUM, x.dtype, (x,), axes, False)
+    return x, "".join(c for c in subs if c not in drop)
+
+
+def _einsum_pair(a, sa, b, sb, keep):
+    """Contract two labelled operands; letters in ``keep`` survive.  Returns (array, labels)."""
+    a, sa = _einsum_sum_out(a, sa, {c for c in sa if c not in sb and c not in keep})
+    b, sb = _einsum_sum_out(b, sb, {c for c in sb if c not in sa and c not in keep})
+    size = {}
+    for x, sx in ((a, sa), (b, sb)):
+        for c, n in zip(sx, x.shape):
+            if size.get(c, 1) == 1:
+                size[c] = n
+            elif n not in (1, size[c]):
+                raise ValueError(f"einsum: operands could not be broadcast together on subscript {c!r}")
+    batch = [c for c in sa if c in sb and c in keep]
+    contracted = [c for c in sa if c in sb and c not in keep]
+    free_a = [c for c in sa if c not in sb]
+    free_b = [c for c in sb if c not in sa]
+
+    def arrange(x, sx, order):
+        x = transpose.fun(x, [sx.index(c) for c in order])
+        full = tuple(size[c] for c in order)
+        return broadcast_to.fun(x, full) if x.shape != full else x
+
+    def prod(letters):
+        n = 1
+        for c in letters:
+            n *= size[c]
+        return n
+
+    Bn, M, K, N = prod(batch), prod(free_a), prod(contracted), prod(free_b)
+    a3 = _view_or_copy(arrange(a, sa, batch + free_a + contracted), (Bn, M, K))
+    b3 = _view_or_copy(arrange(b, sb, batch + contracted + free_b), (Bn, K, N))
+    dt = a.dtype
+    c = D.gemm_batched(D.plain(a3)._t, D.plain(b3)._t, dt)
+    out_subs = batch + free_a + free_b
+    return DevArray(c.view(tuple(size[c_] for c_ in out_subs)), dt), "".join(out_subs)
+
+
+@primitive
+def einsum(*operands, **kwargs):
+    """``numpy.einsum`` for the subscript-string convention: operands are contracted pairwise from
+    the left, each pair as a batched GEMM on permuted views; letters that appear nowhere else are
+    summed out first.  Repeated letters within one operand or in the output (diagonals) are not
+    supported."""
+    if kwargs:
+        raise NotImplementedError(f"einsum: keyword arguments {sorted(kwargs)} are not supported on the device")
+    in_subs, out_subs, arrays = parse_einsum_input(*operands)
+    subs = in_subs.split(",")
+    arrays = [D.asarray(a) for a in arrays]
+    dt = D._float_dtype(D.result_dtype(*arrays))
+    arrays = [D.astype(a, dt) if a.dtype != dt else a for a in arrays]
+    for sx in subs + [out_subs]:
+        if len(set(sx)) != len(sx):
+            raise NotImplementedError("einsum: repeated subscripts within one operand (diagonals) are not supported")
+    cur, cur_subs = arrays[0], subs[0]
+    for k in range(1, len(arrays)):
+        keep = set(out_subs).union(*subs[k + 1:]) if k + 1 < len(arrays) else set(out_subs)
+        cur, cur_subs = _einsum_pair(cur, cur_subs, arrays[k], subs[k], keep)
+    cur, cur_subs = _einsum_sum_out(cur, cur_subs, {c for c in cur_subs if c not in out_subs})
+    if cur_subs != out_subs:
+        cur = transpose.fun(cur, [cur_subs.index(c) for c in out_subs])
+    return copy_if_input(cur, arrays)
+
+
+def copy_if_input(x, inputs):
+    """``x`` itself unless it is one of ``inputs`` (a primitive must not return its argument object)."""
+    for a in inputs:
+        if x is a:
+            return D.alias(x)
+    return x
+
+
 # ---- non-differentiable helpers ---------------------------------------------------------------
 def _meta_of(A):
     if isinstance(A, DevArray):

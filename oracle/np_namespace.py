@@ -54,6 +54,12 @@ _primitive_mean, _primitive_var, _primitive_std = mean, var, std  # noqa: F821
 _astype = astype  # noqa: F821
 
 
+def parse_einsum_input(*args):  # numpy_wrapper.py:194-195
+    from numpy._core.einsumfunc import _parse_einsum_input
+
+    return _parse_einsum_input(args)
+
+
 @notrace_primitive
 def metadata(A):
     return _np.shape(A), _np.ndim(A), _np.result_type(A), _np.iscomplexobj(A)

@@ -92,4 +92,22 @@ def next_cases(be, ext):
     tie = P(onp.array([1.0, 2.0, 2.0, onp.nan, 3.0]))
     other = P(onp.array([1.0, 1.0, 3.0, 2.0, onp.nan]))
     out["ufunc/fmax_ties_nan"] = grad(lambda a, b: np.sum(np.fmax(a, b) * P(onp.arange(1.0, 6.0))), (0, 1))(tie, other)
+
+    # ---- einsum (numpy_vjps.py:815-848): contraction, batch, summed-out, three operands, ellipsis ------
+    for dtype in (onp.float64, onp.float32):
+        tag = "f32" if dtype == onp.float32 else "f64"
+        E = {k: P(rs.randn(*shp).astype(dtype)) for k, shp in
+             dict(a=(3, 4), b=(4, 5), c=(5, 2), t=(2, 3, 4), u=(2, 4, 5), v=(6, 4), w=(1, 4, 5)).items()}
+        cases = [
+            ("mm", "ij,jk->ik", ("a", "b")), ("implicit", "ij,jk", ("a", "b")), ("batched", "bij,bjk->bik", ("t", "u")),
+            ("summed_out", "ij,kj->i", ("a", "v")), ("three", "ij,jk,kl->il", ("a", "b", "c")),
+            ("transpose", "ij->ji", ("a",)), ("total", "ij->", ("a",)), ("outer", "ij,kl->ijkl", ("a", "c")),
+            ("ellipsis", "...ij,...jk->...ik", ("t", "w")), ("inner_batch", "bij,bij->b", ("t", "t")),
+        ]
+        for name, spec, ops in cases:
+            args = tuple(E[o] for o in ops)
+            out[f"einsum/{name}_{tag}/value"] = np.einsum(spec, *args)
+            weights = P(onp.asarray(rs.randn(*onp.shape(be.get(out[f"einsum/{name}_{tag}/value"])))).astype(dtype))
+            f = lambda *xs: np.sum(np.einsum(spec, *xs) * weights)  # noqa: E731,B023
+            out[f"einsum/{name}_{tag}/grad"] = grad(f, tuple(range(len(args))))(*args)
     return out

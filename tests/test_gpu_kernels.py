@@ -545,3 +545,24 @@ def test_pending_maps_through_grad_match_eager_numpy(dnp):
     # accumulation over a fan-out whose contributions are pending maps of one array
     k = grad(lambda v: dnp.sum(-v) + dnp.sum(2.0 * v) + dnp.sum(v + 1.0) + dnp.sum(v * v))(X)
     close(k.numpy(), 2.0 + 2.0 * x, 1e-15)
+
+
+@pytest.mark.parametrize("dtype", [F32, F64])
+def test_einsum_matches_numpy(dnp, dtype):
+    rs = onp.random.RandomState(9)
+    shapes = dict(a=(33, 20), b=(20, 17), c=(17, 5), t=(3, 33, 20), u=(3, 20, 17), w=(1, 20, 17), v=(9, 20), x=(20,))
+    H = {k: rs.randn(*s).astype(dtype) for k, s in shapes.items()}
+    Dv = {k: P(dnp, h) for k, h in H.items()}
+    specs = [("ij,jk->ik", "ab"), ("ij,jk", "ab"), ("ij,jk->ki", "ab"), ("bij,bjk->bik", "tu"), ("bij,bjk->kbi", "tu"),
+             ("ij,kj->i", "av"), ("ij,kj->ik", "av"), ("ij,jk,kl->il", "abc"), ("ij->ji", "a"), ("ij->", "a"), ("ij->j", "a"),
+             ("ij,j->i", "ax"), ("i,i->", "xx"), ("i,j->ij", "xx"), ("...ij,...jk->...ik", "tw"), ("bij,bij->b", "tt"),
+             ("bij,ij->b", "ta"), ("ij,kl->", "ac")]
+    for spec, ops in specs:
+        got = dnp.einsum(spec, *[Dv[o] for o in ops]).numpy()
+        want = onp.einsum(spec, *[H[o] for o in ops])
+        close(got, onp.asarray(want, dtype), RT[dtype] * 4)
+    close(dnp.einsum("ij,jk->ik", Dv["a"].T.T, Dv["b"][:, ::2]).numpy(), H["a"] @ H["b"][:, ::2], RT[dtype] * 4)
+    with pytest.raises(NotImplementedError):
+        dnp.einsum("ii->i", P(dnp, onp.eye(3, dtype=dtype)))
+    with pytest.raises(NotImplementedError):
+        dnp.einsum(Dv["a"], [0, 1], Dv["b"], [1, 2], [0, 2])
