@@ -280,15 +280,15 @@ def extras(be):
         out[f"tanh_{k}_graph_evals_per_sec"] = graph_rate(prog[k], (x,), be.sync, 10)
     # config 3: MLP gradient, f32; MFMA rate over the GEMMs whose dimensions are all >= 784
     inp = configs.mlp_inputs()
-    params = configs.tree_map(be.put, inp["params"])
-    X, T = be.put(inp["X"]), be.put(inp["T"])
-    g = configs.mlp_program(be)["grad"]
-    ms = time_steps(lambda: g(params, X, T), be.sync, 20, 3) * 1e3
+    params3 = configs.tree_map(be.put, inp["params"])
+    X3, T3 = be.put(inp["X"]), be.put(inp["T"])
+    g3 = configs.mlp_program(be)["grad"]
+    ms = time_steps(lambda: g3(params3, X3, T3), be.sync, 20, 3) * 1e3
     out["mlp_grad_evals_per_sec"] = 1e3 / ms
-    out["mlp_grad_graph_evals_per_sec"] = graph_rate(g, (params, X, T), be.sync, 20)
+    out["mlp_grad_graph_evals_per_sec"] = graph_rate(g3, (params3, X3, T3), be.sync, 20)
     with _lib.KernelTimer(only={("gemm",)}) as kt:
         for _ in range(5):
-            g(params, X, T)
+            g3(params3, X3, T3)
     gemm_ms, gemm_flops = 0.0, 0.0
     for name, key, ev0, ev1, nbytes, flops in kt.records:
         if flops >= 2.0 * 784 * 1024 * 1024:  # skip the three GEMMs with a 10-wide dimension (memory-bound)
@@ -318,6 +318,27 @@ def extras(be):
     ms = time_steps(lambda: p5["hvp_fwd"](x5, v5), be.sync, 5, 1) * 1e3
     out["rosen_hvp_fwd_evals_per_sec"] = 1e3 / ms
     out["rosen_hvp_fwd_graph_evals_per_sec"] = graph_rate(p5["hvp_fwd"], (x5, v5), be.sync, 5)
+    # training-loop residency: one fused Adam update of a flat 2^24-element float64 parameter vector
+    # (reads x, g, m, v; writes m, v, x: 56 bytes per element), and whole MLP training steps
+    # (gradient + flatten + update, nothing leaves HBM)
+    import numpy as onp
+
+    from autograd_amd._lib import OPT_ADAM
+    from autograd_amd.misc.optimizers import adam
+    from autograd_amd.numpy import devarray as D
+
+    n = 1 << 24
+    xs = [D.zeros((n,), onp.float64) for _ in range(5)]
+    hyper = (0.1, 0.9, 0.001, 0.999, 0.5, 0.5, 0.001, 1e-8)
+    sec = time_steps(lambda: _lib.optimizer_step(OPT_ADAM, xs[0]._t, xs[1]._t, xs[2]._t, xs[3]._t, xs[4]._t, hyper),
+                     be.sync, 20, 3)
+    out["adam_update_GBps"] = 56.0 * n / sec / 1e9
+    del xs
+    steps = 20
+    t0 = time.perf_counter()
+    adam(lambda p, i: g3(p, X3, T3), params3, num_iters=steps)
+    be.sync()
+    out["mlp_adam_training_steps_per_sec"] = steps / (time.perf_counter() - t0)
     return out
 
 
