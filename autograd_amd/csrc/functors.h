@@ -143,6 +143,12 @@ AGMI_FUNCTOR(FArcsinh, 1, 1, o[0] = m_asinh(x[0]);)
 AGMI_FUNCTOR(FArccosh, 1, 1, o[0] = m_acosh(x[0]);)
 AGMI_FUNCTOR(FArctanh, 1, 1, o[0] = m_atanh(x[0]);)
 
+// rounding functions (no derivative, numpy_vjps.py:13-20)
+AGMI_FUNCTOR(FFloor, 1, 1, o[0] = floor(x[0]);)
+AGMI_FUNCTOR(FCeil, 1, 1, o[0] = ceil(x[0]);)
+AGMI_FUNCTOR(FRint, 1, 1, o[0] = rint(x[0]);)
+AGMI_FUNCTOR(FTrunc, 1, 1, o[0] = trunc(x[0]);)
+
 AGMI_FUNCTOR(FAdd, 2, 1, o[0] = x[0] + x[1];)
 AGMI_FUNCTOR(FSub, 2, 1, o[0] = x[0] - x[1];)
 AGMI_FUNCTOR(FMul, 2, 1, o[0] = x[0] * x[1];)
@@ -219,6 +225,10 @@ AGMI_FUNCTOR(FMulAdd, 3, 1, T t = x[0] * x[1]; o[0] = t + x[2];)
     X(AGMI_OP_ARCSINH, FArcsinh)                \
     X(AGMI_OP_ARCCOSH, FArccosh)                \
     X(AGMI_OP_ARCTANH, FArctanh)                \
+    X(AGMI_OP_FLOOR, FFloor)                    \
+    X(AGMI_OP_CEIL, FCeil)                      \
+    X(AGMI_OP_RINT, FRint)                      \
+    X(AGMI_OP_TRUNC, FTrunc)                    \
     X(AGMI_OP_ADD, FAdd)                        \
     X(AGMI_OP_SUB, FSub)                        \
     X(AGMI_OP_MUL, FMul)                        \

@@ -26,6 +26,11 @@ from .devarray import DevArray
 
 # ---- functions with no derivative (numpy_vjps.py:13-68) -------------------------------------
 nograd_functions = [
+    anp.floor,
+    anp.ceil,
+    anp.rint,
+    anp.round,
+    anp.trunc,
     anp.sign,
     anp.equal,
     anp.not_equal,

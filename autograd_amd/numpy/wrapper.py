@@ -69,6 +69,23 @@ abs = absolute = _wrap(lambda x: D.arith_map(Op.ABS, x), "abs")  # noqa: A001
 sign = _wrap(lambda x: D.arith_map(Op.SIGN, x), "sign")
 
 
+def _rounding(op, name):
+    def raw(x, decimals=0, out=None):
+        if decimals != 0:
+            raise NotImplementedError(f"{name}: only decimals=0 is supported on the device")
+        x = D.asarray(x)
+        return D.map_op(op, x.dtype, x) if x.dtype in D._FLOATS else x
+
+    return _wrap(raw, name)
+
+
+floor = _rounding(Op.FLOOR, "floor")
+ceil = _rounding(Op.CEIL, "ceil")
+rint = _rounding(Op.RINT, "rint")
+round = around = _rounding(Op.RINT, "round")  # noqa: A001
+trunc = fix = _rounding(Op.TRUNC, "trunc")
+
+
 def _binary(op, name, floating=False):
     fn = D.float_map if floating else D.arith_map
 
@@ -160,6 +177,66 @@ def logical_or(a, b):
 
 def logical_not(a):
     return D.compare(Cmp.EQ, _truth(a), 0.0)
+
+
+def logical_xor(a, b):
+    return D.compare(Cmp.NE, _truth(a), _truth(b))
+
+
+def isnan(x):
+    from ..tracer import getval
+
+    x = D.asarray(getval(x))
+    return D.compare(Cmp.NE, x, x)
+
+
+def isinf(x):
+    from ..tracer import getval
+
+    x = D.asarray(getval(x))
+    return D.compare(Cmp.EQ, D.float_map(Op.ABS, x), onp.inf)
+
+
+def isfinite(x):
+    from ..tracer import getval
+
+    x = D.asarray(getval(x))
+    return D.compare(Cmp.LT, D.float_map(Op.ABS, x), onp.inf)  # NaN compares false
+
+
+def _arg_extreme(red, name):
+    def raw(a, axis=None, out=None, keepdims=False):
+        """Index of the first extreme element: min over the axis of where(x == extreme, position, n)
+        (positions are exact in float64 below 2**53).  Non-differentiable (numpy_vjps.py:22-23)."""
+        from ..tracer import getval
+
+        x = D.asarray(getval(a))
+        if x.dtype not in D._FLOATS:
+            x = D.astype(x, onp.float64)
+        if axis is None:
+            x = ravel.fun(x)
+            ax = 0
+        else:
+            ax = int(axis) % x.ndim
+        n = x.shape[ax]
+        if n == 0:
+            raise ValueError(f"attempt to get {name} of an empty sequence")
+        best = D.map_reduce(Op.COPY, red, x.dtype, (x,), (ax,), True)
+        hit = D.compare(Cmp.EQ, x, best)
+        view = [1] * x.ndim
+        view[ax] = n
+        pos = D.from_numpy(onp.arange(n, dtype=onp.float64).reshape(view))
+        f64 = onp.dtype("float64")
+        cand = D.map_op(Op.WHERE, f64, D.astype(hit, f64), pos, float(n))
+        idx = D.map_reduce(Op.COPY, Red.MIN, f64, (cand,), (ax,), bool(keepdims) and axis is not None)
+        return D.astype(idx, onp.int64)
+
+    raw.__name__ = raw.__qualname__ = name
+    return raw
+
+
+argmax = _arg_extreme(Red.MAX, "argmax")
+argmin = _arg_extreme(Red.MIN, "argmin")
 
 
 # ---- astype / copies --------------------------------------------------------------------------

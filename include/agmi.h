@@ -93,6 +93,10 @@ typedef enum agmi_op {
     AGMI_OP_ARCSINH,
     AGMI_OP_ARCCOSH,
     AGMI_OP_ARCTANH,
+    AGMI_OP_FLOOR,    /* rounding functions: no derivative (numpy_vjps.py:13-20)                   */
+    AGMI_OP_CEIL,
+    AGMI_OP_RINT,     /* round half to even: numpy.rint, numpy.round(x) with decimals=0            */
+    AGMI_OP_TRUNC,
     /* two inputs */
     AGMI_OP_ADD = 32, /* also VSpace._add / _mut_add, autograd/core.py:259-264 (out may alias in0) */
     AGMI_OP_SUB,
