@@ -233,6 +233,10 @@ def main():
         for _ in range(5):
             D.map_op(Op.COPY, ref.dtype, ref)
         be.sync()
+    # the same evaluation recorded once and replayed as a HIP graph (autograd_amd.capture): same kernels,
+    # no per-step Python tracing; reported beside the eager figure, never as `value`
+    rate = graph_rate(fun, fun_args, be.sync, args.steps)
+    result["graph_replay"] = {"value": rate, "unit": "grad evals/sec", "ms_per_step": 1e3 / rate}
     if not args.no_extras and args.workload == "bcast":
         result["extras"] = extras(be)
     if not args.no_cpu_baseline:
@@ -339,6 +343,18 @@ def extras(be):
     adam(lambda p, i: g3(p, X3, T3), params3, num_iters=steps)
     be.sync()
     out["mlp_adam_training_steps_per_sec"] = steps / (time.perf_counter() - t0)
+    # the same loop with the gradient replayed from a HIP graph (parameters are copied into the recorded
+    # input buffers every step, the update stays a separate kernel)
+    import autograd_amd as ag
+
+    graphed = ag.capture(g3, params3, X3, T3)
+    adam(lambda p, i: graphed(p, X3, T3), params3, num_iters=3)
+    be.sync()
+    t0 = time.perf_counter()
+    adam(lambda p, i: graphed(p, X3, T3), params3, num_iters=steps)
+    be.sync()
+    out["mlp_adam_training_graph_steps_per_sec"] = steps / (time.perf_counter() - t0)
+    del graphed
     return out
 
 
