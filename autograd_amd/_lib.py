@@ -21,6 +21,7 @@ LIB_PATH = os.environ.get("AGMI_LIBRARY", os.path.join(_HERE, "libagmi.so"))
 
 MAX_DIMS = 8
 MAX_IN = 4
+MAX_AUX = 2  # auxiliary operands (array-valued factors / offsets of pending maps) per launch
 MAX_OUT = 2
 
 # agmi_dtype
@@ -88,16 +89,19 @@ REDUCE_FUSABLE = frozenset(
 
 class AgmiArray(ctypes.Structure):
     _fields_ = [("data", ctypes.c_void_p), ("strides", ctypes.c_int64 * MAX_DIMS), ("scale", ctypes.c_double),
-                ("shift", ctypes.c_double), ("affine", ctypes.c_uint32)]
+                ("shift", ctypes.c_double), ("affine", ctypes.c_uint32), ("scale_slot", ctypes.c_int32),
+                ("shift_slot", ctypes.c_int32)]
 
 
 class Affine:
-    """Kernel input slot ``t * scale + shift`` (``shift`` None: no add), applied on load."""
+    """Kernel input slot ``t * scale * ascale + shift``, applied on load in that order, each step
+    rounded on its own.  ``scale`` is a Python float (1.0: no multiply); ``ascale`` is None or a tensor
+    of ``t``'s shape (a broadcast view); ``shift`` is None (no add), a Python float or such a tensor."""
 
-    __slots__ = ("t", "scale", "shift")
+    __slots__ = ("t", "scale", "shift", "ascale")
 
-    def __init__(self, t, scale, shift):
-        self.t, self.scale, self.shift = t, scale, shift
+    def __init__(self, t, scale, shift, ascale=None):
+        self.t, self.scale, self.shift, self.ascale = t, scale, shift, ascale
 
 
 class AgmiError(RuntimeError):
@@ -277,6 +281,9 @@ def _traffic(outs, ins):
         total += t.numel() * t.element_size()
     for t in ins:
         if type(t) is Affine:
+            for aux in (t.ascale, t.shift):
+                if isinstance(aux, torch.Tensor):
+                    total += _distinct_bytes(aux)
             t = t.t
         if isinstance(t, torch.Tensor):
             total += _distinct_bytes(t)
@@ -285,7 +292,7 @@ def _traffic(outs, ins):
 
 # ---- argument marshalling (buffers reused: single-threaded by contract) ----------------------
 _outs = (AgmiArray * MAX_OUT)()
-_ins = (AgmiArray * MAX_IN)()
+_ins = (AgmiArray * (MAX_IN + MAX_AUX))()
 _shape = (ctypes.c_int64 * MAX_DIMS)()
 _scalars = (ctypes.c_double * MAX_IN)()
 _mask = (ctypes.c_uint8 * MAX_DIMS)()
@@ -308,6 +315,9 @@ def _set_shape(shape):
 
 
 def _set_inputs(ins):
+    """Fill the input slots; array-valued factors / offsets of pending maps go to auxiliary slots
+    after the op's own inputs.  Returns the total number of slots used."""
+    n = len(ins)
     for k, x in enumerate(ins):
         slot = _ins[k]
         if isinstance(x, torch.Tensor):
@@ -319,14 +329,32 @@ def _set_inputs(ins):
             if x.scale != 1.0:
                 slot.scale = x.scale
                 flags = 1
-            if x.shift is not None:
-                slot.shift = x.shift
-                flags |= 2
+            if x.ascale is not None:
+                if n >= MAX_IN + MAX_AUX:
+                    raise AgmiError("too many array-valued pending maps in one launch")
+                _set_array(_ins[n], x.ascale)
+                _ins[n].affine = 0
+                slot.scale_slot = n
+                flags |= 4
+                n += 1
+            sh = x.shift
+            if sh is not None:
+                if type(sh) is float:
+                    slot.shift = sh
+                    flags |= 2
+                else:
+                    if n >= MAX_IN + MAX_AUX:
+                        raise AgmiError("too many array-valued pending maps in one launch")
+                    _set_array(_ins[n], sh)
+                    _ins[n].affine = 0
+                    slot.shift_slot = n
+                    flags |= 8
+                    n += 1
             slot.affine = flags
         else:
             slot.data = None
             _scalars[k] = x
-    return len(ins)
+    return n
 
 
 def elementwise(op, code, shape, outs, ins):

@@ -39,9 +39,24 @@ def make_vjp(fun, x):
     else:
 
         def vjp(g):
-            return backward_pass(g, end_node)
+            return settle(backward_pass(g, end_node))
 
     return vjp, end_value
+
+
+def settle(value):
+    """A derivative as it is handed to the caller: value types whose arithmetic may be deferred
+    (they define ``_settled``) complete it here, inside whatever is timing the evaluation;
+    containers are walked, boxes and everything else pass through."""
+    t = type(value)
+    done = getattr(t, "_settled", None)
+    if done is not None:
+        return done(value)
+    if t is tuple or t is list:
+        return t(settle(v) for v in value)
+    if t is dict:
+        return {k: settle(v) for k, v in value.items()}
+    return value
 
 
 def backward_pass(g, end_node):
@@ -159,7 +174,7 @@ def make_jvp(fun, x):
         end_value, end_node = trace(start_node, fun, x)
         if end_node is None:
             return end_value, vspace(end_value).zeros()
-        return end_value, end_node.g
+        return end_value, settle(end_node.g)
 
     return jvp
 

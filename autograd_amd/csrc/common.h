@@ -20,7 +20,8 @@ int hip_check(hipError_t e, const char *what);
 
 constexpr int kBlock = 256;        // 4 wavefronts of 64 lanes
 constexpr int kMaxMerged = 6;      // rank the strided kernels index with div/mod
-constexpr int kMaxOperands = AGMI_MAX_INPUTS + AGMI_MAX_OUTPUTS;
+constexpr int kMaxPhysIn = AGMI_MAX_INPUTS + AGMI_MAX_AUX;  // an op's own inputs + auxiliary operands of pending maps
+constexpr int kMaxOperands = kMaxPhysIn + AGMI_MAX_OUTPUTS;
 
 inline size_t dtype_size(int dtype) {
     switch (dtype) {
@@ -55,6 +56,34 @@ inline bool index_space_is_empty(int ndim, const int64_t *shape) {
     for (int d = 0; d < ndim; ++d)
         if (shape[d] == 0) return true;
     return false;
+}
+
+// Copy input k's pending map into the kernel parameters; auxiliary slots must lie in [arity, n_in).
+template <class P>
+inline bool read_affine(const agmi_array &a, int arity, int n_in, int k, P *p) {
+    if (a.affine & AGMI_AFFINE_SCALE) {
+        p->scale_mask |= 1u << k;
+        p->scale[k] = a.scale;
+    }
+    if (a.affine & AGMI_AFFINE_SHIFT) {
+        p->shift_mask |= 1u << k;
+        p->shift[k] = a.shift;
+    }
+    if (a.affine & AGMI_AFFINE_SCALE_AUX) {
+        if (a.scale_slot < arity || a.scale_slot >= n_in) {
+            set_error("input %d: scale_slot %d is not an auxiliary input", k, a.scale_slot);
+            return false;
+        }
+        p->scale_aux[k] = static_cast<signed char>(a.scale_slot);
+    }
+    if (a.affine & AGMI_AFFINE_SHIFT_AUX) {
+        if (a.shift_slot < arity || a.shift_slot >= n_in) {
+            set_error("input %d: shift_slot %d is not an auxiliary input", k, a.shift_slot);
+            return false;
+        }
+        p->shift_aux[k] = static_cast<signed char>(a.shift_slot);
+    }
+    return true;
 }
 
 inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }

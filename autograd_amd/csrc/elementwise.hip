@@ -11,6 +11,8 @@
 //   nd    - anything else up to 6 merged axes, one element per thread with div/mod indexing.
 // A by-value scalar operand lives in kernel arguments (SGPRs); which slots are scalars is a
 // run-time, wave-uniform mask, so one kernel serves array/scalar combinations.
+#include <type_traits>
+
 #include "common.h"
 #include "functors.h"
 
@@ -18,28 +20,57 @@ namespace agmi {
 
 struct EwParams {
     void *out[AGMI_MAX_OUTPUTS];
-    const void *in[AGMI_MAX_INPUTS];
+    const void *in[kMaxPhysIn];
     double scalar[AGMI_MAX_INPUTS];
     double scale[AGMI_MAX_INPUTS];  // pending affine map of an input: value = mem * scale + shift
     double shift[AGMI_MAX_INPUTS];
     unsigned scalar_mask;
     unsigned scale_mask, shift_mask;
+    // pending maps whose factor / offset is an array: index (>= the op's arity) of the auxiliary
+    // input that holds it, or -1
+    signed char scale_aux[AGMI_MAX_INPUTS], shift_aux[AGMI_MAX_INPUTS];
     int ndim;
     int64_t n;
     int64_t shape[kMaxMerged];
     int64_t ostr[AGMI_MAX_OUTPUTS][kMaxMerged];
-    int64_t istr[AGMI_MAX_INPUTS][kMaxMerged];
+    int64_t istr[kMaxPhysIn][kMaxMerged];
 };
 
-// Apply the inputs' pending affine maps to one gathered point: multiply, then add, each rounded
-// on its own (the masks are wave-uniform, so plain operands pay one scalar branch).
-template <typename T, int NIN, class P>
-__device__ __forceinline__ void apply_affine(const P &p, T *xi) {
-    if ((p.scale_mask | p.shift_mask) == 0) return;
+// Apply the inputs' pending affine maps to the V points a thread has gathered: multiply, then
+// add, each rounded on its own.  `x` holds the op's NIN inputs followed by NAUX auxiliary
+// operands (array-valued factors / offsets).  All tests are wave-uniform and made once per
+// input, not once per point, so plain operands pay a few scalar branches per thread.
+template <typename T, int NIN, int NAUX, int V, class P>
+__device__ __forceinline__ void apply_affine(const P &p, T (&x)[NIN + NAUX][V]) {
+    if (NAUX == 0 && (p.scale_mask | p.shift_mask) == 0) return;
 #pragma unroll
     for (int k = 0; k < NIN; ++k) {
-        if (p.scale_mask & (1u << k)) xi[k] = xi[k] * static_cast<T>(p.scale[k]);
-        if (p.shift_mask & (1u << k)) xi[k] = xi[k] + static_cast<T>(p.shift[k]);
+        if (p.scale_mask & (1u << k)) {
+            const T s = static_cast<T>(p.scale[k]);
+#pragma unroll
+            for (int j = 0; j < V; ++j) x[k][j] = x[k][j] * s;
+        }
+        if (NAUX > 0 && p.scale_aux[k] >= 0) {
+#pragma unroll
+            for (int a = 0; a < NAUX; ++a)
+                if (p.scale_aux[k] == NIN + a) {
+#pragma unroll
+                    for (int j = 0; j < V; ++j) x[k][j] = x[k][j] * x[NIN + a][j];
+                }
+        }
+        if (p.shift_mask & (1u << k)) {
+            const T s = static_cast<T>(p.shift[k]);
+#pragma unroll
+            for (int j = 0; j < V; ++j) x[k][j] = x[k][j] + s;
+        }
+        if (NAUX > 0 && p.shift_aux[k] >= 0) {
+#pragma unroll
+            for (int a = 0; a < NAUX; ++a)
+                if (p.shift_aux[k] == NIN + a) {
+#pragma unroll
+                    for (int j = 0; j < V; ++j) x[k][j] = x[k][j] + x[NIN + a][j];
+                }
+        }
     }
 }
 
@@ -52,18 +83,19 @@ struct Vec {
 };
 
 // ---- flat ------------------------------------------------------------------------------
-template <template <typename> class F, typename T>
+template <template <typename> class F, typename T, int NAUX>
 __global__ __launch_bounds__(kBlock) void ew_flat(const EwParams p) {
     using Fn = F<T>;
+    constexpr int NP = Fn::NIN + NAUX;
     constexpr int V = Vec<T>::N;
     using vec_t = typename Vec<T>::type;
     const int64_t i0 = (static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x) * V;
     if (i0 >= p.n) return;
-    T x[Fn::NIN][V];
+    T x[NP][V];
     T o[Fn::NOUT][V];
     if (i0 + V <= p.n) {
 #pragma unroll
-        for (int k = 0; k < Fn::NIN; ++k) {
+        for (int k = 0; k < NP; ++k) {
             if (p.scalar_mask & (1u << k)) {
                 const T s = static_cast<T>(p.scalar[k]);
 #pragma unroll
@@ -78,12 +110,12 @@ __global__ __launch_bounds__(kBlock) void ew_flat(const EwParams p) {
                 for (int j = 0; j < V; ++j) x[k][j] = v[j];
             }
         }
+        apply_affine<T, Fn::NIN, NAUX, V>(p, x);
 #pragma unroll
         for (int j = 0; j < V; ++j) {
             T xi[Fn::NIN], oi[Fn::NOUT];
 #pragma unroll
             for (int k = 0; k < Fn::NIN; ++k) xi[k] = x[k][j];
-            apply_affine<T, Fn::NIN>(p, xi);
             Fn::apply(xi, oi);
 #pragma unroll
             for (int k = 0; k < Fn::NOUT; ++k) o[k][j] = oi[k];
@@ -97,15 +129,17 @@ __global__ __launch_bounds__(kBlock) void ew_flat(const EwParams p) {
         }
     } else {
         for (int64_t i = i0; i < p.n; ++i) {
-            T xi[Fn::NIN], oi[Fn::NOUT];
+            T x1[NP][1], xi[Fn::NIN], oi[Fn::NOUT];
 #pragma unroll
-            for (int k = 0; k < Fn::NIN; ++k) {
+            for (int k = 0; k < NP; ++k) {
                 if (p.scalar_mask & (1u << k))
-                    xi[k] = static_cast<T>(p.scalar[k]);
+                    x1[k][0] = static_cast<T>(p.scalar[k]);
                 else
-                    xi[k] = static_cast<const T *>(p.in[k])[p.istr[k][0] == 0 ? 0 : i];
+                    x1[k][0] = static_cast<const T *>(p.in[k])[p.istr[k][0] == 0 ? 0 : i];
             }
-            apply_affine<T, Fn::NIN>(p, xi);
+            apply_affine<T, Fn::NIN, NAUX, 1>(p, x1);
+#pragma unroll
+            for (int k = 0; k < Fn::NIN; ++k) xi[k] = x1[k][0];
             Fn::apply(xi, oi);
 #pragma unroll
             for (int k = 0; k < Fn::NOUT; ++k) static_cast<T *>(p.out[k])[i] = oi[k];
@@ -115,9 +149,10 @@ __global__ __launch_bounds__(kBlock) void ew_flat(const EwParams p) {
 
 // ---- rows ------------------------------------------------------------------------------
 // shape = (R, C); every operand has inner stride 1 or 0.  `tpr` = threads per row.
-template <template <typename> class F, typename T, typename Index>
+template <template <typename> class F, typename T, typename Index, int NAUX>
 __global__ __launch_bounds__(kBlock) void ew_rows(const EwParams p, const Index tpr, const Index total) {
     using Fn = F<T>;
+    constexpr int NP = Fn::NIN + NAUX;
     constexpr int V = Vec<T>::N;
     using vec_t = typename Vec<T>::type;
     const Index t = static_cast<Index>(blockIdx.x) * kBlock + threadIdx.x;
@@ -127,9 +162,9 @@ __global__ __launch_bounds__(kBlock) void ew_rows(const EwParams p, const Index 
     const int64_t C = p.shape[1];
     const bool full = c0 + V <= C;
     const int nvalid = full ? V : static_cast<int>(C - c0);
-    T x[Fn::NIN][V];
+    T x[NP][V];
 #pragma unroll
-    for (int k = 0; k < Fn::NIN; ++k) {
+    for (int k = 0; k < NP; ++k) {
         if (p.scalar_mask & (1u << k)) {
             const T s = static_cast<T>(p.scalar[k]);
 #pragma unroll
@@ -150,13 +185,13 @@ __global__ __launch_bounds__(kBlock) void ew_rows(const EwParams p, const Index 
             }
         }
     }
+    apply_affine<T, Fn::NIN, NAUX, V>(p, x);
     T o[Fn::NOUT][V];
 #pragma unroll
     for (int j = 0; j < V; ++j) {
         T xi[Fn::NIN], oi[Fn::NOUT];
 #pragma unroll
         for (int k = 0; k < Fn::NIN; ++k) xi[k] = x[k][j];
-        apply_affine<T, Fn::NIN>(p, xi);
         Fn::apply(xi, oi);
 #pragma unroll
         for (int k = 0; k < Fn::NOUT; ++k) o[k][j] = oi[k];
@@ -178,15 +213,16 @@ __global__ __launch_bounds__(kBlock) void ew_rows(const EwParams p, const Index 
 }
 
 // ---- nd --------------------------------------------------------------------------------
-template <template <typename> class F, typename T, typename Index>
+template <template <typename> class F, typename T, typename Index, int NAUX>
 __global__ __launch_bounds__(kBlock) void ew_nd(const EwParams p) {
     using Fn = F<T>;
+    constexpr int NP = Fn::NIN + NAUX;
     Index rem = static_cast<Index>(blockIdx.x) * kBlock + threadIdx.x;
     if (static_cast<int64_t>(rem) >= p.n) return;
-    int64_t ioff[Fn::NIN];
+    int64_t ioff[NP];
     int64_t ooff[Fn::NOUT];
 #pragma unroll
-    for (int k = 0; k < Fn::NIN; ++k) ioff[k] = 0;
+    for (int k = 0; k < NP; ++k) ioff[k] = 0;
 #pragma unroll
     for (int k = 0; k < Fn::NOUT; ++k) ooff[k] = 0;
     for (int d = p.ndim - 1; d >= 0; --d) {
@@ -195,15 +231,17 @@ __global__ __launch_bounds__(kBlock) void ew_nd(const EwParams p) {
         const int64_t c = static_cast<int64_t>(rem - q * extent);
         rem = q;
 #pragma unroll
-        for (int k = 0; k < Fn::NIN; ++k) ioff[k] += c * p.istr[k][d];
+        for (int k = 0; k < NP; ++k) ioff[k] += c * p.istr[k][d];
 #pragma unroll
         for (int k = 0; k < Fn::NOUT; ++k) ooff[k] += c * p.ostr[k][d];
     }
-    T xi[Fn::NIN], oi[Fn::NOUT];
+    T x1[NP][1], xi[Fn::NIN], oi[Fn::NOUT];
 #pragma unroll
-    for (int k = 0; k < Fn::NIN; ++k)
-        xi[k] = (p.scalar_mask & (1u << k)) ? static_cast<T>(p.scalar[k]) : static_cast<const T *>(p.in[k])[ioff[k]];
-    apply_affine<T, Fn::NIN>(p, xi);
+    for (int k = 0; k < NP; ++k)
+        x1[k][0] = (p.scalar_mask & (1u << k)) ? static_cast<T>(p.scalar[k]) : static_cast<const T *>(p.in[k])[ioff[k]];
+    apply_affine<T, Fn::NIN, NAUX, 1>(p, x1);
+#pragma unroll
+    for (int k = 0; k < Fn::NIN; ++k) xi[k] = x1[k][0];
     Fn::apply(xi, oi);
 #pragma unroll
     for (int k = 0; k < Fn::NOUT; ++k) static_cast<T *>(p.out[k])[ooff[k]] = oi[k];
@@ -222,8 +260,10 @@ template <template <typename> class F, typename T>
 static int launch_ew(const char *fname, const Merged &m, int n_out, const agmi_array *outs, int n_in,
                      const agmi_array *ins, const double *scalars, hipStream_t s) {
     using Fn = F<T>;
-    if (n_in != Fn::NIN || n_out != Fn::NOUT) {
-        set_error("elementwise: op takes %d inputs and %d outputs, got %d and %d", Fn::NIN, Fn::NOUT, n_in, n_out);
+    const int n_aux = n_in - Fn::NIN;
+    if (n_aux < 0 || n_aux > AGMI_MAX_AUX || n_out != Fn::NOUT) {
+        set_error("elementwise: op takes %d inputs (+ at most %d auxiliary) and %d outputs, got %d and %d", Fn::NIN,
+                  AGMI_MAX_AUX, Fn::NOUT, n_in, n_out);
         return AGMI_ERR_ARG;
     }
     if (m.ndim > kMaxMerged) {
@@ -244,24 +284,18 @@ static int launch_ew(const char *fname, const Merged &m, int n_out, const agmi_a
             }
         }
     }
+    for (int k = 0; k < AGMI_MAX_INPUTS; ++k) p.scale_aux[k] = p.shift_aux[k] = -1;
     for (int k = 0; k < n_in; ++k) {
         p.in[k] = ins[k].data;
         if (ins[k].data == nullptr) {
-            if (scalars == nullptr) {
-                set_error("elementwise: scalar slot %d without scalars array", k);
+            if (scalars == nullptr || k >= Fn::NIN) {
+                set_error("elementwise: scalar slot %d without scalars array (auxiliary inputs must be arrays)", k);
                 return AGMI_ERR_ARG;
             }
             p.scalar_mask |= 1u << k;
             p.scalar[k] = scalars[k];
-        } else {
-            if (ins[k].affine & AGMI_AFFINE_SCALE) {
-                p.scale_mask |= 1u << k;
-                p.scale[k] = ins[k].scale;
-            }
-            if (ins[k].affine & AGMI_AFFINE_SHIFT) {
-                p.shift_mask |= 1u << k;
-                p.shift[k] = ins[k].shift;
-            }
+        } else if (k < Fn::NIN) {
+            if (!read_affine(ins[k], Fn::NIN, n_in, k, &p)) return AGMI_ERR_ARG;
         }
         for (int d = 0; d < m.ndim; ++d) p.istr[k][d] = m.stride[n_out + k][d];
     }
@@ -272,12 +306,19 @@ static int launch_ew(const char *fname, const Merged &m, int n_out, const agmi_a
     for (int k = 0; k < n_out; ++k) inner_unit &= (p.ostr[k][last] == 1 || m.shape[last] == 1);
     for (int k = 0; k < n_in; ++k)
         inner_unit &= (p.scalar_mask & (1u << k)) || p.istr[k][last] == 1 || p.istr[k][last] == 0;
-
+    // the kernels are instantiated for 0, 1 and 2 auxiliary operands
+    auto with_naux = [&](auto launch) {
+        if (n_aux == 0) launch(std::integral_constant<int, 0>{});
+        else if (n_aux == 1) launch(std::integral_constant<int, 1>{});
+        else launch(std::integral_constant<int, 2>{});
+    };
     if (m.ndim == 1 && inner_unit) {
         const int64_t blocks = ceil_div(ceil_div(m.n, V), kBlock);
         if (int rc = check_blocks(blocks)) return rc;
         set_kernel_name("ew_flat<%s>", fname);
-        hipLaunchKernelGGL((ew_flat<F, T>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p);
+        with_naux([&](auto na) {
+            hipLaunchKernelGGL((ew_flat<F, T, decltype(na)::value>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p);
+        });
     } else if (m.ndim == 2 && inner_unit) {
         const int64_t tpr = ceil_div(m.shape[1], V);
         const int64_t total = tpr * m.shape[0];
@@ -285,18 +326,27 @@ static int launch_ew(const char *fname, const Merged &m, int n_out, const agmi_a
         if (int rc = check_blocks(blocks)) return rc;
         set_kernel_name("ew_rows<%s>", fname);
         if (total < 0x7fffffffLL)
-            hipLaunchKernelGGL((ew_rows<F, T, unsigned>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p,
-                               (unsigned)tpr, (unsigned)total);
+            with_naux([&](auto na) {
+                hipLaunchKernelGGL((ew_rows<F, T, unsigned, decltype(na)::value>), dim3((unsigned)blocks), dim3(kBlock), 0,
+                                   s, p, (unsigned)tpr, (unsigned)total);
+            });
         else
-            hipLaunchKernelGGL((ew_rows<F, T, int64_t>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p, tpr, total);
+            with_naux([&](auto na) {
+                hipLaunchKernelGGL((ew_rows<F, T, int64_t, decltype(na)::value>), dim3((unsigned)blocks), dim3(kBlock), 0,
+                                   s, p, tpr, total);
+            });
     } else {
         const int64_t blocks = ceil_div(m.n, kBlock);
         if (int rc = check_blocks(blocks)) return rc;
         set_kernel_name("ew_nd<%s>", fname);
         if (m.n < 0x7fffffffLL)
-            hipLaunchKernelGGL((ew_nd<F, T, unsigned>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p);
+            with_naux([&](auto na) {
+                hipLaunchKernelGGL((ew_nd<F, T, unsigned, decltype(na)::value>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p);
+            });
         else
-            hipLaunchKernelGGL((ew_nd<F, T, int64_t>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p);
+            with_naux([&](auto na) {
+                hipLaunchKernelGGL((ew_nd<F, T, int64_t, decltype(na)::value>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p);
+            });
     }
     return hip_check(hipGetLastError(), "elementwise launch");
 }
@@ -410,7 +460,7 @@ using namespace agmi;
 extern "C" int agmi_elementwise(int op, int dtype, int ndim, const int64_t *shape, int n_out,
                                 const agmi_array *outs, int n_in, const agmi_array *ins,
                                 const double *scalars, void *stream) {
-    if (n_out < 1 || n_out > AGMI_MAX_OUTPUTS || n_in < 1 || n_in > AGMI_MAX_INPUTS || !outs || !ins) {
+    if (n_out < 1 || n_out > AGMI_MAX_OUTPUTS || n_in < 1 || n_in > kMaxPhysIn || !outs || !ins) {
         set_error("elementwise: bad operand counts or null operand arrays");
         return AGMI_ERR_ARG;
     }

@@ -76,17 +76,19 @@ struct AccLse {
 
 struct RedParams {
     void *out;  // T* when final, Acc* (chunk-major) when partial
-    const void *in[AGMI_MAX_INPUTS];
+    const void *in[kMaxPhysIn];     // the op's inputs, then n_aux auxiliary operands of pending maps
     double scalar[AGMI_MAX_INPUTS];
     double scale[AGMI_MAX_INPUTS];  // pending affine map of an input: value = mem * scale + shift
     double shift[AGMI_MAX_INPUTS];
     unsigned scalar_mask;
     unsigned scale_mask, shift_mask;
+    signed char scale_aux[AGMI_MAX_INPUTS], shift_aux[AGMI_MAX_INPUTS];  // index of the auxiliary input, or -1
+    int n_aux;
     int n_chunks;
     int64_t O, R, I;
     int64_t r_chunk;
     int64_t ostr_o, ostr_i;
-    int64_t istr[AGMI_MAX_INPUTS][3];  // (o, r, i)
+    int64_t istr[kMaxPhysIn][3];  // (o, r, i)
 };
 
 template <typename T>
@@ -97,11 +99,13 @@ struct RVec {
 
 // load V consecutive points along axis `ax` (1 = r, 2 = i) starting at element offsets given
 template <template <typename> class F, typename T, int V, int AX>
-__device__ __forceinline__ void load_points(const RedParams &p, int64_t o, int64_t r, int64_t i, T (&x)[F<T>::NIN][V]) {
+__device__ __forceinline__ void load_points(const RedParams &p, int64_t o, int64_t r, int64_t i,
+                                            T (&x)[F<T>::NIN + AGMI_MAX_AUX][V]) {
     using vec_t = typename RVec<T>::type;
 #pragma unroll
-    for (int k = 0; k < F<T>::NIN; ++k) {
-        if (p.scalar_mask & (1u << k)) {
+    for (int k = 0; k < F<T>::NIN + AGMI_MAX_AUX; ++k) {
+        if (k >= F<T>::NIN + p.n_aux) {  // wave-uniform: no auxiliary operand in this slot
+        } else if (p.scalar_mask & (1u << k)) {
             const T s = static_cast<T>(p.scalar[k]);
 #pragma unroll
             for (int j = 0; j < V; ++j) x[k][j] = s;
@@ -120,20 +124,47 @@ __device__ __forceinline__ void load_points(const RedParams &p, int64_t o, int64
             }
         }
     }
-}
-
-template <template <typename> class F, typename T, int V>
-__device__ __forceinline__ T map_point(const RedParams &p, const T (&x)[F<T>::NIN][V], int j) {
-    T xi[F<T>::NIN], oi[F<T>::NOUT];
+    // pending affine maps: multiply, then add, each rounded on its own (wave-uniform tests, once per input)
+    if ((p.scale_mask | p.shift_mask) == 0 && p.n_aux == 0) return;
+    constexpr int NIN = F<T>::NIN;
 #pragma unroll
-    for (int k = 0; k < F<T>::NIN; ++k) xi[k] = x[k][j];
-    if (p.scale_mask | p.shift_mask) {  // wave-uniform
+    for (int k = 0; k < NIN; ++k) {
+        if (p.scale_mask & (1u << k)) {
+            const T s = static_cast<T>(p.scale[k]);
 #pragma unroll
-        for (int k = 0; k < F<T>::NIN; ++k) {
-            if (p.scale_mask & (1u << k)) xi[k] = xi[k] * static_cast<T>(p.scale[k]);
-            if (p.shift_mask & (1u << k)) xi[k] = xi[k] + static_cast<T>(p.shift[k]);
+            for (int j = 0; j < V; ++j) x[k][j] = x[k][j] * s;
+        }
+        if (p.scale_aux[k] >= 0) {
+#pragma unroll
+            for (int a = 0; a < AGMI_MAX_AUX; ++a)
+                if (p.scale_aux[k] == NIN + a) {
+#pragma unroll
+                    for (int j = 0; j < V; ++j) x[k][j] = x[k][j] * x[NIN + a][j];
+                }
+        }
+        if (p.shift_mask & (1u << k)) {
+            const T s = static_cast<T>(p.shift[k]);
+#pragma unroll
+            for (int j = 0; j < V; ++j) x[k][j] = x[k][j] + s;
+        }
+        if (p.shift_aux[k] >= 0) {
+#pragma unroll
+            for (int a = 0; a < AGMI_MAX_AUX; ++a)
+                if (p.shift_aux[k] == NIN + a) {
+#pragma unroll
+                    for (int j = 0; j < V; ++j) x[k][j] = x[k][j] + x[NIN + a][j];
+                }
         }
     }
+}
+
+// one point of the mapped operand (pending maps have been applied by load_points)
+template <template <typename> class F, typename T, int V>
+__device__ __forceinline__ T map_point(const RedParams &p, const T (&x)[F<T>::NIN + AGMI_MAX_AUX][V], int j) {
+    constexpr int NIN = F<T>::NIN;
+    T xi[NIN], oi[F<T>::NOUT];
+#pragma unroll
+    for (int k = 0; k < NIN; ++k) xi[k] = x[k][j];
     F<T>::apply(xi, oi);
     return oi[0];
 }
@@ -178,7 +209,7 @@ __global__ __launch_bounds__(kBlock) void red_row_block(const RedParams p) {
     typename Acc::type acc = Acc::identity();
     const int64_t n_vec = (r_end - r_begin) / V;
     for (int64_t v = threadIdx.x; v < n_vec; v += kBlock) {
-        T x[F<T>::NIN][V];
+        T x[F<T>::NIN + AGMI_MAX_AUX][V];
         load_points<F, T, V, 1>(p, o, r_begin + v * V, 0, x);
 #pragma unroll
         for (int j = 0; j < V; ++j) acc = Acc::combine(acc, Acc::lift(map_point<F, T, V>(p, x, j)));
@@ -186,7 +217,7 @@ __global__ __launch_bounds__(kBlock) void red_row_block(const RedParams p) {
     if (V > 1) {  // ragged tail, fewer than V points
         const int64_t r = r_begin + n_vec * V + threadIdx.x;
         if (r < r_end) {
-            T x[F<T>::NIN][1];
+            T x[F<T>::NIN + AGMI_MAX_AUX][1];
             load_points<F, T, 1, 1>(p, o, r, 0, x);
             acc = Acc::combine(acc, Acc::lift(map_point<F, T, 1>(p, x, 0)));
         }
@@ -207,33 +238,92 @@ __device__ __forceinline__ double exp_nonpositive(double d) { return exp(d); }
 // row chunk fits in registers (<= 256 * V * ITERS elements) each thread instead takes the plain
 // maximum of its elements and then sums exp(x - max) with independent exps, and only the
 // per-thread (max, sum) pairs go through the pair reduction: one pass over memory.
-template <typename T, int V, int ITERS, bool FINAL>
+// V elements of physical input k of row o, starting at reduced index r0 (n_left of them in range);
+// out-of-range lanes get `fill`
+template <typename T, int V>
+__device__ __forceinline__ void lse_load(const RedParams &p, int k, int64_t o, int64_t r0, int64_t n_left, T fill,
+                                         T (&dst)[V]) {
+    using vec_t = typename RVec<T>::type;
+    const int64_t sr = p.istr[k][1];
+    const T *base = static_cast<const T *>(p.in[k]) + o * p.istr[k][0] + r0 * sr;
+    if (sr == 0) {
+        const T v = n_left > 0 ? *base : fill;
+#pragma unroll
+        for (int j = 0; j < V; ++j) dst[j] = j < n_left ? v : fill;
+    } else if (V > 1 && sr == 1 && n_left >= V) {
+        const vec_t v = *reinterpret_cast<const vec_t *>(base);
+#pragma unroll
+        for (int j = 0; j < V; ++j) dst[j] = v[j];
+    } else {
+#pragma unroll
+        for (int j = 0; j < V; ++j) dst[j] = j < n_left ? base[j * sr] : fill;
+    }
+}
+
+// AFFINE: the input carries a pending map (scalar or auxiliary-array factor / offset), applied on load
+template <typename T, int V, int ITERS, bool FINAL, bool AFFINE>
 __global__ __launch_bounds__(kBlock) void lse_row_block(const RedParams p) {
     using Acc = AccLse<T>;
-    using vec_t = typename RVec<T>::type;
     const int64_t o = blockIdx.x;
     const int chunk = blockIdx.y;
     const int64_t r_begin = static_cast<int64_t>(chunk) * p.r_chunk;
     const int64_t r_end = min(r_begin + p.r_chunk, p.R);
     const int64_t n = r_end - r_begin;
-    const T *row = static_cast<const T *>(p.in[0]) + o * p.istr[0][0] + r_begin * p.istr[0][1];
-    const int64_t sr = p.istr[0][1];
     T x[ITERS][V];
     T m = T(-INFINITY);
+    // every load is issued before the first use (memory-level parallelism: 1 + aux loads per iteration)
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
         const int64_t e0 = (static_cast<int64_t>(it) * kBlock + threadIdx.x) * V;
-        if (V > 1 && e0 + V <= n) {
-            const vec_t v = *reinterpret_cast<const vec_t *>(row + e0);
+        lse_load<T, V>(p, 0, o, r_begin + e0, n - e0, T(-INFINITY), x[it]);
+    }
+    if (AFFINE) {
+        T a[ITERS][V], b[ITERS][V];
+        const bool has_a = p.scale_aux[0] >= 0, has_b = p.shift_aux[0] >= 0;
+        if (has_a) {
 #pragma unroll
-            for (int j = 0; j < V; ++j) x[it][j] = v[j];
-        } else {
-#pragma unroll
-            for (int j = 0; j < V; ++j) x[it][j] = (e0 + j < n) ? row[(e0 + j) * sr] : T(-INFINITY);
+            for (int it = 0; it < ITERS; ++it) {
+                const int64_t e0 = (static_cast<int64_t>(it) * kBlock + threadIdx.x) * V;
+                lse_load<T, V>(p, p.scale_aux[0], o, r_begin + e0, n - e0, T(1), a[it]);
+            }
         }
+        if (has_b) {
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it) {
+                const int64_t e0 = (static_cast<int64_t>(it) * kBlock + threadIdx.x) * V;
+                lse_load<T, V>(p, p.shift_aux[0], o, r_begin + e0, n - e0, T(0), b[it]);
+            }
+        }
+        if (!has_a) {
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+                for (int j = 0; j < V; ++j) a[it][j] = T(1);
+        }
+        if (!has_b) {
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+                for (int j = 0; j < V; ++j) b[it][j] = T(0);
+        }
+        // absent steps are the neutral element (x * 1 is exact; x + 0 only loses the sign of a
+        // zero, which neither max nor exp can see), so the arithmetic is branch-free
+        const T sc = (p.scale_mask & 1u) ? static_cast<T>(p.scale[0]) : T(1);
+        const T sh = (p.shift_mask & 1u) ? static_cast<T>(p.shift[0]) : T(0);
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+            const int64_t n_left = n - (static_cast<int64_t>(it) * kBlock + threadIdx.x) * V;
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                const T v = ((x[it][j] * sc) * a[it][j] + sh) + b[it][j];
+                x[it][j] = j < n_left ? v : T(-INFINITY);  // padding stays neutral
+            }
+        }
+    }
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it)
 #pragma unroll
         for (int j = 0; j < V; ++j) m = max_nan(x[it][j], m);
-    }
     T s = T(0);
     if (m == T(INFINITY)) {
         s = T(1);
@@ -260,7 +350,7 @@ __global__ __launch_bounds__(kBlock) void red_row_group(const RedParams p, const
     typename Acc::type acc = Acc::identity();
     if (o < p.O) {
         for (int64_t r = lane; r < p.R; r += G) {
-            T x[F<T>::NIN][1];
+            T x[F<T>::NIN + AGMI_MAX_AUX][1];
             load_points<F, T, 1, 1>(p, o, r, 0, x);
             acc = Acc::combine(acc, Acc::lift(map_point<F, T, 1>(p, x, 0)));
         }
@@ -292,7 +382,7 @@ __global__ __launch_bounds__(kBlock) void red_cols(const RedParams p, const int 
     if (active) {
 #pragma unroll 4
         for (int64_t r = r_begin + ty; r < r_end; r += TY) {
-            T x[F<T>::NIN][V];
+            T x[F<T>::NIN + AGMI_MAX_AUX][V];
             load_points<F, T, V, 2>(p, o, r, i0, x);
 #pragma unroll
             for (int j = 0; j < V; ++j) acc[j] = Acc::combine(acc[j], Acc::lift(map_point<F, T, V>(p, x, j)));
@@ -449,15 +539,20 @@ static int launch_reduce(const char *fname, const RedParams &base, bool vec_ok, 
         if constexpr (std::is_same<AccT<T>, AccLse<T>>::value && std::is_same<F<T>, FCopy<T>>::value) {
             const bool unit = p.istr[0][1] == 1 || p.r_chunk == 1;
             const int v = (pl.V > 1 && unit) ? VEC : 1;
-            if (!(p.scalar_mask & 1u) && !((p.scale_mask | p.shift_mask) & 1u) && p.r_chunk <= static_cast<int64_t>(kBlock) * v * kLseIters) {
+            if (!(p.scalar_mask & 1u) && p.r_chunk <= static_cast<int64_t>(kBlock) * v * kLseIters) {
                 set_kernel_name("lse_row_block%s", two_stage ? "+red_finish" : "");
                 const int64_t need = ceil_div(p.r_chunk, static_cast<int64_t>(kBlock) * v);
+                const bool affine = ((p.scale_mask | p.shift_mask) & 1u) || p.n_aux > 0;
 #define AGMI_LSE(VV, IT)                                                                                   \
     do {                                                                                                   \
-        if (two_stage)                                                                                     \
-            hipLaunchKernelGGL((lse_row_block<T, VV, IT, false>), grid, dim3(kBlock), 0, s, p);            \
+        if (two_stage && affine)                                                                           \
+            hipLaunchKernelGGL((lse_row_block<T, VV, IT, false, true>), grid, dim3(kBlock), 0, s, p);      \
+        else if (two_stage)                                                                                \
+            hipLaunchKernelGGL((lse_row_block<T, VV, IT, false, false>), grid, dim3(kBlock), 0, s, p);     \
+        else if (affine)                                                                                   \
+            hipLaunchKernelGGL((lse_row_block<T, VV, IT, true, true>), grid, dim3(kBlock), 0, s, p);       \
         else                                                                                               \
-            hipLaunchKernelGGL((lse_row_block<T, VV, IT, true>), grid, dim3(kBlock), 0, s, p);             \
+            hipLaunchKernelGGL((lse_row_block<T, VV, IT, true, false>), grid, dim3(kBlock), 0, s, p);      \
     } while (0)
 #define AGMI_LSE_IT(VV)                      \
     do {                                     \
@@ -562,9 +657,10 @@ struct RedSetup {
     bool vec_ok;
 };
 
-static int setup_reduce(int ndim, const int64_t *shape, const uint8_t *reduce_axes, const agmi_array *out, int n_in,
-                        const agmi_array *ins, const double *scalars, RedSetup *st, bool *empty) {
-    if (!out || !ins || !reduce_axes || n_in < 1 || n_in > AGMI_MAX_INPUTS) {
+// `arity` = number of inputs of the op itself; ins[arity .. n_in) are auxiliary operands of pending maps
+static int setup_reduce(int ndim, const int64_t *shape, const uint8_t *reduce_axes, const agmi_array *out, int arity,
+                        int n_in, const agmi_array *ins, const double *scalars, RedSetup *st, bool *empty) {
+    if (!out || !ins || !reduce_axes || n_in < 1 || n_in > kMaxPhysIn || arity < 1 || arity > n_in || n_in - arity > AGMI_MAX_AUX) {
         set_error("map_reduce: bad arguments");
         return AGMI_ERR_ARG;
     }
@@ -601,24 +697,19 @@ static int setup_reduce(int ndim, const int64_t *shape, const uint8_t *reduce_ax
     p.ostr_i = ori[0][2];
     st->vec_ok = true;
     const int ax = (p.I == 1) ? 1 : 2;
+    p.n_aux = n_in - arity;
+    for (int k = 0; k < AGMI_MAX_INPUTS; ++k) p.scale_aux[k] = p.shift_aux[k] = -1;
     for (int k = 0; k < n_in; ++k) {
         p.in[k] = ins[k].data;
         if (!ins[k].data) {
-            if (!scalars) {
-                set_error("map_reduce: scalar slot %d without scalars array", k);
+            if (!scalars || k >= arity) {
+                set_error("map_reduce: scalar slot %d without scalars array (auxiliary inputs must be arrays)", k);
                 return AGMI_ERR_ARG;
             }
             p.scalar_mask |= 1u << k;
             p.scalar[k] = scalars[k];
         } else {
-            if (ins[k].affine & AGMI_AFFINE_SCALE) {
-                p.scale_mask |= 1u << k;
-                p.scale[k] = ins[k].scale;
-            }
-            if (ins[k].affine & AGMI_AFFINE_SHIFT) {
-                p.shift_mask |= 1u << k;
-                p.shift[k] = ins[k].shift;
-            }
+            if (k < arity && !read_affine(ins[k], arity, n_in, k, &p)) return AGMI_ERR_ARG;
             for (int a = 0; a < 3; ++a) p.istr[k][a] = ori[1 + k][a];
             if (p.istr[k][ax] != 0 && p.istr[k][ax] != 1) st->vec_ok = false;
         }
@@ -683,9 +774,18 @@ extern "C" int agmi_map_reduce(int op, int red, int dtype, int ndim, const int64
                                const uint8_t *reduce_axes, const agmi_array *out, int n_in,
                                const agmi_array *ins, const double *scalars, void *workspace,
                                size_t workspace_bytes, void *stream) {
+    int arity = op == AGMI_OP_COPY ? 1 : -1;
+#define AGMI_CASE(OP, FN) \
+    if (op == OP) arity = FN<float>::NIN;
+    AGMI_FOR_EACH_REDUCE_OP(AGMI_CASE)
+#undef AGMI_CASE
+    if (arity < 0) {
+        set_error("map_reduce: op %d cannot be fused into a reduction", op);
+        return AGMI_ERR_UNSUPPORTED;
+    }
     RedSetup st;
     bool empty = false;
-    if (int rc = setup_reduce(ndim, shape, reduce_axes, out, n_in, ins, scalars, &st, &empty)) return rc;
+    if (int rc = setup_reduce(ndim, shape, reduce_axes, out, arity, n_in, ins, scalars, &st, &empty)) return rc;
     if (empty) return 0;
     hipStream_t s = as_stream(stream);
     if (dtype != AGMI_F32 && dtype != AGMI_F64) {
@@ -693,19 +793,11 @@ extern "C" int agmi_map_reduce(int op, int red, int dtype, int ndim, const int64
         return AGMI_ERR_ARG;
     }
     if (op == AGMI_OP_COPY) {
-        if (n_in != 1) {
-            set_error("map_reduce: AGMI_OP_COPY takes one input");
-            return AGMI_ERR_ARG;
-        }
         return dtype == AGMI_F32 ? dispatch_red_copy<float>(red, st, workspace, workspace_bytes, s)
                                  : dispatch_red_copy<double>(red, st, workspace, workspace_bytes, s);
     }
 #define AGMI_CASE(OP, FN)                                                                        \
     case OP:                                                                                     \
-        if (n_in != FN<float>::NIN) {                                                            \
-            set_error("map_reduce: op takes %d inputs, got %d", FN<float>::NIN, n_in);           \
-            return AGMI_ERR_ARG;                                                                 \
-        }                                                                                        \
         return dtype == AGMI_F32 ? dispatch_red<FN, float>(#FN, red, st, workspace, workspace_bytes, s) \
                                  : dispatch_red<FN, double>(#FN, red, st, workspace, workspace_bytes, s);
     switch (op) {

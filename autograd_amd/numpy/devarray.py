@@ -115,31 +115,39 @@ class DevArray:
         """The tensor that carries shape, strides and storage (metadata only: never its values)."""
         return self._t
 
-    def _like(self, t):
-        """A view ``t`` of this array's storage as an array of the same kind."""
-        return DevArray(t, self.dtype)
+    def _view(self, fn):
+        """``fn`` (a view operation on a tensor: slicing, reshaping, permuting ...) applied to this array."""
+        return DevArray(fn(self._t), self.dtype)
+
+    def _settled(self):
+        """This array with no arithmetic pending (see ``core.settle``)."""
+        return self
 
     # ---- operators and methods are attached by wrapper.py (they are traced primitives) ------
 
 
 class LazyDevArray(DevArray):
-    """``raw * scale + shift`` not yet written to memory.
+    """``raw * scale * ascale + shift`` not yet written to memory.
 
-    Negation and arithmetic with a Python scalar return one of these instead of launching a
-    kernel (see ``_fold``); the next kernel that reads it applies the map on load, as two
-    separately rounded operations, so the value is bit-for-bit what the eager passes would have
-    stored.  Code that is unaware of it reads ``_t`` as on any ``DevArray``: the first such read
-    writes the value to a fresh buffer (one copy kernel) and keeps it.
+    Negation, arithmetic with a Python scalar, and products / sums with a BROADCAST array operand
+    (``A * b[None, :] + c[:, None]``, a bias added to a matrix product) return one of these instead
+    of launching a kernel (see ``_fold``); the next kernel that reads it applies the steps on load,
+    each one rounded on its own, so the value is bit-for-bit what the eager passes would have
+    stored.  ``scale`` is a Python float; ``ascale`` is None or a tensor of ``raw``'s shape (a
+    stride-0 view of the broadcast operand); ``shift`` is None, a Python float or such a tensor.
+    Code that is unaware of all this reads ``_t`` as on any ``DevArray``: the first such read writes
+    the value to a fresh buffer (one copy kernel) and keeps it.
     """
 
-    __slots__ = ("_raw", "_scale", "_shift")
+    __slots__ = ("_raw", "_scale", "_shift", "_ascale")
 
-    def __init__(self, raw, dtype, scale, shift):
+    def __init__(self, raw, dtype, scale, shift, ascale=None):
         self._raw = raw
         self.dtype = dtype
         self._borrowed = False
-        self._scale = scale  # Python float, representable in dtype; 1.0 = no multiply
-        self._shift = shift  # Python float, or None = no add (x + 0.0 is not x for x = -0.0)
+        self._scale = scale    # Python float, representable in dtype; 1.0 = no multiply
+        self._ascale = ascale  # tensor shaped like raw, or None
+        self._shift = shift    # Python float or tensor shaped like raw; None = no add (x + 0.0 is not x for -0.0)
 
     def __getattr__(self, name):
         # only reached when a slot is unset: `_t` before the value has been written out
@@ -147,10 +155,12 @@ class LazyDevArray(DevArray):
             raise AttributeError(name)
         raw = self._raw
         out = _lib.empty(tuple(raw.shape), self.dtype)
-        _lib.elementwise(Op.COPY, _lib.DTYPE_CODE[self.dtype], tuple(raw.shape), (out,),
-                         (_lib.Affine(raw, self._scale, self._shift),))
+        _lib.elementwise(Op.COPY, _lib.DTYPE_CODE[self.dtype], tuple(raw.shape), (out,), (self._affine(),))
         self._t = out
         return out
+
+    def _affine(self):
+        return _lib.Affine(self._raw, self._scale, self._shift, self._ascale)
 
     @property
     def shape(self):
@@ -182,8 +192,19 @@ class LazyDevArray(DevArray):
     def _h(self):
         return self._raw
 
-    def _like(self, t):
-        return LazyDevArray(t, self.dtype, self._scale, self._shift)
+    def _settled(self):
+        return DevArray(self._t, self.dtype)
+
+    def _view(self, fn):
+        """The same view operation on the storage and on the array-valued steps (they have the
+        storage's shape); when one of them cannot be viewed that way the value is written out."""
+        asc, sh = self._ascale, self._shift
+        try:
+            return LazyDevArray(fn(self._raw), self.dtype, self._scale,
+                                fn(sh) if isinstance(sh, torch.Tensor) else sh,
+                                fn(asc) if asc is not None else None)
+        except RuntimeError:
+            return DevArray(fn(self._t), self.dtype)
 
 
 def plain(x):
@@ -193,7 +214,7 @@ def plain(x):
 
 def alias(x):
     """A second handle on ``x``'s storage (and pending map)."""
-    return x._like(x._h())
+    return x._view(lambda t: t)
 
 
 def _is_pow2(c):
@@ -204,20 +225,38 @@ def _representable(v, dtype):
     return math.isfinite(v) and (dtype == _F64 or float(onp.float32(v)) == v)
 
 
-def _fold(op, dtype, xs):
-    """``op(xs)`` as a pending affine map of its one array operand, or None.
+def _state(a):
+    """(raw tensor, scalar scale, array scale, shift) of a device array."""
+    if type(a) is LazyDevArray:
+        return a._raw, a._scale, a._ascale, a._shift
+    return a._t, 1.0, None, None
 
-    Folded only when the composed map gives bit-for-bit the value of the eager passes:
-    negation always (it commutes with rounding); a scalar factor when it or the pending scale is a
-    power of two (that multiply is then exact); a scalar offset when no offset is pending.  Scalars are
-    Python floats/ints (weak in NumPy's promotion: converted to the array's dtype first).
+
+def _fold(op, dtype, xs):
+    """``op(xs)`` as a pending map ``raw * scale * ascale + shift`` of its array operand, or None.
+
+    Folded only when the kernel's fixed step order (scalar factor, array factor, offset), each step
+    rounded on its own, gives bit-for-bit the value of the eager passes:
+    * negation: always (it commutes with rounding), unless an array-valued offset is pending;
+    * a Python-scalar factor: when it, or the pending scalar factor, is a power of two (that
+      multiply is then exact) - and only a power of two once an array factor or an offset is pending;
+    * a Python-scalar offset, or an array offset: when no offset is pending;
+    * an array factor: when no array factor and no offset is pending.
+    Scalars are Python floats/ints (weak in NumPy's promotion: converted to the array's dtype
+    first).  An array operand qualifies when it is BROADCAST against the other one (strictly fewer
+    elements, same dtype): the other operand's storage stays the `raw` of the result.
     """
     if op == Op.NEG:
         (a,) = xs
         c = None
+        swapped = False
     elif len(xs) == 2:
         a, c = xs
         swapped = False
+        if isinstance(c, DevArray) and isinstance(a, DevArray):
+            if c.size > a.size:
+                a, c, swapped = c, a, True
+            return _fold_array(op, dtype, a, c, swapped)
         if type(c) is not float and type(c) is not int:
             a, c, swapped = c, a, True
             if type(c) is not float and type(c) is not int:
@@ -226,25 +265,28 @@ def _fold(op, dtype, xs):
         return None
     if not isinstance(a, DevArray) or a.dtype != dtype:
         return None
-    if type(a) is LazyDevArray:
-        raw, s, t = a._raw, a._scale, a._shift
-    else:
-        raw, s, t = a._t, 1.0, None
+    raw, s, asc, t = _state(a)
+    array_shift = isinstance(t, torch.Tensor)
     if c is not None:
         c = float(c) if dtype == _F64 else float(onp.float32(c))
     if op == Op.NEG:
+        if array_shift:
+            return None
         s, t = -s, (None if t is None else -t)
     elif op == Op.MUL or (op == Op.DIV and not swapped and _is_pow2(c)):
         if op == Op.DIV:
             c = 1.0 / c
-        if t is None:
+        if t is None and asc is None:
             if not (_is_pow2(s) or _is_pow2(c)):  # one of the two multiplies is exact
                 return None
             s = s * c
-        elif _is_pow2(c):
-            s, t = s * c, t * c
-            if not _representable(t, dtype) or (t == 0.0) != (a._shift == 0.0):
-                return None
+        elif _is_pow2(c) and not array_shift:
+            s = s * c
+            if t is not None:
+                t2 = t * c
+                if not _representable(t2, dtype) or (t2 == 0.0) != (t == 0.0):
+                    return None
+                t = t2
         else:
             return None
         if s != s or not (_representable(s, dtype) or math.isinf(s)):
@@ -262,9 +304,33 @@ def _fold(op, dtype, xs):
             t = -c
     else:
         return None
-    if s == 1.0 and t is None:
+    if s == 1.0 and t is None and asc is None:
         return DevArray(raw, dtype)
-    return LazyDevArray(raw, dtype, s, t)
+    return LazyDevArray(raw, dtype, s, t, asc)
+
+
+def _fold_array(op, dtype, a, c, swapped):
+    """``_fold`` for two array operands: ``c`` is broadcast against ``a`` (``swapped``: ``c`` was the
+    left operand)."""
+    if a.dtype != dtype or c.dtype != dtype or dtype not in _FLOATS:
+        return None
+    if c.size >= a.size or a.size == 0 or broadcast_shapes(a.shape, c.shape) != a.shape:
+        return None
+    raw, s, asc, t = _state(a)
+    if t is not None:
+        return None  # an offset is the last step
+    if type(c) is LazyDevArray or c.ndim > a.ndim:
+        c = plain(c)
+    vec = c._t.expand(a.shape)
+    if op == Op.MUL:
+        if asc is not None:
+            return None
+        return LazyDevArray(raw, dtype, s, None, vec)
+    if op == Op.ADD:
+        return LazyDevArray(raw, dtype, s, vec, asc)
+    if op == Op.SUB and swapped:  # c - a = (-a) + c
+        return LazyDevArray(raw, dtype, -s, vec, asc)
+    return None
 
 
 _FOLDABLE = frozenset({Op.NEG, Op.MUL, Op.ADD, Op.SUB, Op.DIV})
@@ -403,7 +469,7 @@ def _operand(x, dtype):
         if x.dtype != dtype:
             x = astype(x, dtype)
         elif type(x) is LazyDevArray:
-            return _lib.Affine(x._raw, x._scale, x._shift)
+            return x._affine()
         return x._t
     if isinstance(x, (numbers.Number, onp.generic)):
         return float(x)
@@ -448,8 +514,28 @@ def _expand(t, shape):
         if tuple(t.shape) != shape:
             return t.expand(shape)
     elif type(t) is _lib.Affine and tuple(t.t.shape) != shape:
-        return _lib.Affine(t.t.expand(shape), t.scale, t.shift)
+        sh, asc = t.shift, t.ascale
+        return _lib.Affine(t.t.expand(shape), t.scale, sh.expand(shape) if isinstance(sh, torch.Tensor) else sh,
+                           asc.expand(shape) if asc is not None else None)
     return t
+
+
+def _limit_aux(ops, dtype):
+    """A launch takes at most ``_lib.MAX_AUX`` array-valued steps: write out the operands that carry
+    the most of them until the rest fits."""
+    def n_aux(t):
+        return (t.ascale is not None) + isinstance(t.shift, torch.Tensor) if type(t) is _lib.Affine else 0
+
+    total = sum(n_aux(t) for t in ops)
+    if total <= _lib.MAX_AUX:
+        return ops
+    ops = list(ops)
+    while total > _lib.MAX_AUX:
+        k = max(range(len(ops)), key=lambda i: n_aux(ops[i]))
+        total -= n_aux(ops[k])
+        t = ops[k]
+        ops[k] = LazyDevArray(t.t, dtype, t.scale, t.shift, t.ascale)._t
+    return tuple(ops)
 
 
 def _lift_scalars(operands, dtype):
@@ -469,7 +555,7 @@ def map_op(op, dtype, *xs, out=None, n_out=1):
                 return folded
     elif type(out) is not DevArray:
         raise TypeError("map_op: `out` must be a plain device array")
-    ops = tuple(_operand(x, dtype) for x in xs)
+    ops = _limit_aux(tuple(_operand(x, dtype) for x in xs), dtype)
     shape = _bshape(ops)
     if shape is None:
         ops = _lift_scalars(ops, dtype)
@@ -554,7 +640,7 @@ _IDENTITY = {Red.SUM: 0.0, Red.PROD: 1.0}
 
 def map_reduce(op, red, dtype, xs, axes, keepdims, shape=None):
     """``RED_axes op(xs...)`` with ``xs`` broadcast to ``shape`` (default: their broadcast)."""
-    ops = tuple(_operand(x, dtype) for x in xs)
+    ops = _limit_aux(tuple(_operand(x, dtype) for x in xs), dtype)
     if shape is None:
         shape = _bshape(ops)
     if shape is None:
@@ -594,7 +680,7 @@ def _rewrap(t, dtype):
     if isinstance(t, torch.Tensor):
         return DevArray(t, dtype)
     if type(t) is _lib.Affine:
-        return LazyDevArray(t.t, dtype, t.scale, t.shift)
+        return LazyDevArray(t.t, dtype, t.scale, t.shift, t.ascale)
     return t
 
 

@@ -80,7 +80,7 @@ class DevArrayVSpace(VSpace):
         zero: creating it writes nothing, and the first ``x_prev + x_new`` reads it from a
         register instead of streaming a zero-filled buffer.  It is never written in place:
         ``_mut_add`` and the scatter rule allocate the real buffer when they meet it."""
-        if self.size <= 1:
+        if self.size == 0:
             return D.zeros(self.shape, self.dtype)
         return DevArray(_shared_zero(self.dtype)._t.expand(self.shape), self.dtype)
 
@@ -88,7 +88,7 @@ class DevArrayVSpace(VSpace):
         """The seed cotangent of ``elementwise_grad`` (differential_operators.py:41-49 of the reference
         seeds ``vs.ones()``): like ``zeros``, a stride-0 view of one shared element, so seeding a
         backward pass writes nothing and the first rule reads the seed from a register."""
-        if self.size <= 1:
+        if self.size == 0:
             return D.ones(self.shape, self.dtype)
         return DevArray(_shared_one(self.dtype)._t.expand(self.shape), self.dtype)
 
@@ -115,10 +115,13 @@ class DevArrayVSpace(VSpace):
         may also be a tape value or another node's cotangent - is never written."""
         if not isinstance(x, DevArray):
             return self._add(x, y)
-        if is_shared_zero(x) and isinstance(y, DevArray) and y.shape == x.shape and y.dtype == x.dtype:
-            acc = D.alias(y)
-            acc._borrowed = True
-            return acc
+        if is_shared_zero(x):
+            if isinstance(y, DevArray) and y.shape == x.shape and y.dtype == x.dtype:
+                acc = D.alias(y)
+                acc._borrowed = True
+                return acc
+            res = self._add(x, y)  # the shared zero is never written
+            return D.astype(res, x.dtype) if isinstance(res, DevArray) and res.dtype != x.dtype else res
         if isinstance(y, DevArray) and y.dtype != x.dtype and D.result_dtype(x, y) != x.dtype:
             # numpy.add(x, y, out=x) of the reference (numpy_vspaces.py:33-34 through core.py:262-264)
             # adds in the promoted dtype and stores in x's: a float64 cotangent accumulated into a

@@ -288,7 +288,7 @@ def mean(a, *args, **kwargs):
 # ---- shape-only functions (views: no kernel unless a copy is unavoidable) -----------------------
 def _view_or_copy(x, shape):
     try:
-        return x._like(x._h().view(shape))
+        return x._view(lambda t: t.view(shape))
     except RuntimeError:
         return DevArray(D.contiguous(x)._t.view(shape), x.dtype)
 
@@ -340,25 +340,31 @@ def expand_dims(x, axis):
     axes = (axis,) if isinstance(axis, (numbers.Integral, onp.integer)) else tuple(axis)
     nd = x.ndim + len(axes)
     axes = sorted(a % nd for a in axes)
-    t = x._h()
-    for a in axes:
-        t = t.unsqueeze(a)
-    return x._like(t)
+    def expand(t):
+        for a in axes:
+            t = t.unsqueeze(a)
+        return t
+
+    return x._view(expand)
 
 
 @primitive
 def squeeze(x, axis=None):
     x = D.asarray(x)
     if axis is None:
-        return x._like(x._h().squeeze())
+        return x._view(lambda t: t.squeeze())
     axes = (axis,) if isinstance(axis, (numbers.Integral, onp.integer)) else tuple(axis)
     axes = sorted((a % x.ndim for a in axes), reverse=True)
-    t = x._h()
     for a in axes:
-        if t.shape[a] != 1:
+        if x.shape[a] != 1:
             raise ValueError("cannot select an axis to squeeze out which has size not equal to one")
-        t = t.squeeze(a)
-    return x._like(t)
+
+    def drop(t):
+        for a in axes:
+            t = t.squeeze(a)
+        return t
+
+    return x._view(drop)
 
 
 @primitive
@@ -367,26 +373,26 @@ def transpose(x, axes=None):
     if axes is None:
         axes = tuple(range(x.ndim))[::-1]
     axes = tuple(int(a) % x.ndim for a in axes) if x.ndim else ()
-    return x._like(x._h().permute(axes) if x.ndim else x._h())
+    return x._view(lambda t: t.permute(axes) if t.dim() else t)
 
 
 @primitive
 def swapaxes(x, axis1, axis2):
     x = D.asarray(x)
-    return x._like(x._h().transpose(axis1, axis2))
+    return x._view(lambda t: t.transpose(axis1, axis2))
 
 
 @primitive
 def moveaxis(x, source, destination):
     x = D.asarray(x)
-    return x._like(torch.movedim(x._h(), source, destination))
+    return x._view(lambda t: torch.movedim(t, source, destination))
 
 
 @primitive
 def broadcast_to(x, shape):
     x = D.asarray(x)
     shape = (shape,) if isinstance(shape, numbers.Integral) else tuple(shape)
-    return x._like(x._h().expand(shape))
+    return x._view(lambda t: t.expand(shape))
 
 
 def _atleast(n):
@@ -394,14 +400,16 @@ def _atleast(n):
         res = []
         for a in arys:
             a = D.asarray(a)
-            t = a._h()
-            if n >= 1 and t.dim() == 0:
-                t = t.reshape(1)
-            if n >= 2 and t.dim() == 1:
-                t = t.unsqueeze(0)
-            if n >= 3 and t.dim() == 2:
-                t = t.unsqueeze(2)
-            res.append(a._like(t))
+            def lift(t):
+                if n >= 1 and t.dim() == 0:
+                    t = t.reshape(1)
+                if n >= 2 and t.dim() == 1:
+                    t = t.unsqueeze(0)
+                if n >= 3 and t.dim() == 2:
+                    t = t.unsqueeze(2)
+                return t
+
+            res.append(a._view(lift))
         return res[0] if len(res) == 1 else res
 
     return _wrap(raw, f"atleast_{n}d")
@@ -421,10 +429,10 @@ def repeat(x, repeats, axis=None):
         axis = 0
     axis %= x.ndim
     # out viewed as (..., n, repeats, ...) = x broadcast along a new axis
-    src = x._h().unsqueeze(axis + 1)
-    wide = src.shape[: axis + 1] + (repeats,) + src.shape[axis + 2 :]
-    out = D.map_op(Op.COPY, x.dtype, x._like(src.expand(wide))) if x.dtype in D._FLOATS else D.astype_copy(
-        DevArray(src.expand(wide), x.dtype))
+    shp = x.shape
+    wide = shp[: axis + 1] + (repeats,) + shp[axis + 1 :]
+    widened = x._view(lambda t: t.unsqueeze(axis + 1).expand(wide))
+    out = D.map_op(Op.COPY, x.dtype, widened) if x.dtype in D._FLOATS else D.astype_copy(D.plain(widened))
     final = x.shape[:axis] + (x.shape[axis] * repeats,) + x.shape[axis + 1 :]
     return DevArray(out._t.view(final), x.dtype)
 
@@ -586,7 +594,8 @@ def _host_index(idx):
 def take(A, idx):
     """``A[idx]``: views for basic indices, a gather kernel for an integer array on axis 0."""
     if _is_basic_index(idx):
-        return A._like(A._h()[_plain(idx)])
+        pidx = _plain(idx)
+        return A._view(lambda t: t[pidx])
     rows = _host_index(idx)
     if rows is None:
         raise NotImplementedError(
@@ -619,7 +628,7 @@ def scatter_add(A, idx, x):
     from .vspaces import is_broadcast_view, is_shared_zero
 
     basic = _is_basic_index(idx)
-    if A._borrowed or type(A) is not DevArray or is_broadcast_view(A):  # not this accumulator's own memory yet: allocate it
+    if A._borrowed or type(A) is not DevArray or is_broadcast_view(A) or is_shared_zero(A):  # not this accumulator's own memory yet: allocate it
         if is_shared_zero(A):
             if basic:
                 # into zeros the sum is 0 + x, so the destination is never read back; and when the
@@ -627,6 +636,13 @@ def scatter_add(A, idx, x):
                 # is skipped as well
                 probe = A._t[_plain(idx)]
                 full_cover = probe.numel() == A._t.numel() and probe.dim() >= A._t.dim()
+                if full_cover and isinstance(x, DevArray) and x.dtype == A.dtype and x.shape == tuple(probe.shape):
+                    # basic indices cannot permute: the view is A with unit axes inserted, so 0 + x is x
+                    # with A's shape.  Borrowed like any `zeros + g` (vspaces._mut_add): nothing is launched
+                    shape = A.shape
+                    acc = x._view(lambda t: t.reshape(shape))
+                    acc._borrowed = True
+                    return acc
                 A = D.empty(A.shape, A.dtype) if full_cover else D.zeros(A.shape, A.dtype)
                 D.map_op(Op.ADD, A.dtype, 0.0, x, out=DevArray(A._t[_plain(idx)], A.dtype))
                 return A

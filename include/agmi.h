@@ -48,17 +48,29 @@ typedef enum agmi_dtype {
  * An INPUT may carry a pending affine map: its element value is then mem * scale + shift,
  * computed on load as two separately rounded operations (exactly what the NumPy passes
  * `x * scale` and `+ shift` would have produced), so that negation, scalar multiples and
- * scalar offsets of an array (numpy_vjps.py:87, 157; `2 * g`, `1.0 - e` in user code) cost no
- * pass of their own.  `affine` is a bit set: AGMI_AFFINE_SCALE, AGMI_AFFINE_SHIFT; 0 = plain
- * (zero-initialised structs are plain).  Ignored for outputs and by agmi_gemm/cast/compare. */
-#define AGMI_AFFINE_SCALE 1u
-#define AGMI_AFFINE_SHIFT 2u
+ * scalar offsets of an array (numpy_vjps.py:87, 157; `2 * g`, `1.0 - e` in user code) and
+ * products / sums with a BROADCAST operand (`A * b[None, :] + c[:, None]`, a bias added to a
+ * matrix product: examples/neural_net.py:34) cost no pass of their own.  `affine` is a bit set;
+ * 0 = plain (zero-initialised structs are plain).  A scale or shift that is itself an array is
+ * passed as an AUXILIARY input: an extra entry of the `ins` array after the op's own inputs
+ * (at most AGMI_MAX_AUX of them per call), named by `scale_slot` / `shift_slot` = its index in
+ * `ins`; it is read with its own strides (stride 0 on the axes it is broadcast along).  When several
+ * bits are set the steps run in the order of the bit values: * scale, * ins[scale_slot],
+ * + shift, + ins[shift_slot].
+ * Ignored for outputs and by agmi_gemm / agmi_cast / agmi_compare. */
+#define AGMI_AFFINE_SCALE 1u      /* multiply by `scale` */
+#define AGMI_AFFINE_SHIFT 2u      /* then add `shift` */
+#define AGMI_AFFINE_SCALE_AUX 4u  /* multiply by ins[scale_slot] */
+#define AGMI_AFFINE_SHIFT_AUX 8u  /* then add ins[shift_slot] */
+#define AGMI_MAX_AUX 2
 typedef struct agmi_array {
     void *data;                     /* device pointer to the element at index (0, ..., 0) */
     int64_t strides[AGMI_MAX_DIMS]; /* elements */
     double scale;
     double shift;
     uint32_t affine;
+    int32_t scale_slot;
+    int32_t shift_slot;
 } agmi_array;
 
 /* Elementwise operations.  Unary/binary/ternary ufuncs are the forward primitives
