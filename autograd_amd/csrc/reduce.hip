@@ -260,8 +260,14 @@ __device__ __forceinline__ void lse_load(const RedParams &p, int k, int64_t o, i
     }
 }
 
-// AFFINE: the input carries a pending map (scalar or auxiliary-array factor / offset), applied on load
-template <typename T, int V, int ITERS, bool FINAL, bool AFFINE>
+// MODE: 0 = plain input; otherwise the input carries a pending map applied on load:
+//   kLseAffine        scalar steps and auxiliary operands that are constant along the row (one value per block)
+//   | kLseVecScale    the auxiliary factor varies along the row (registers for it)
+//   | kLseVecShift    the auxiliary offset varies along the row
+// Separate instantiations keep the register count (and so the blocks per CU) of the plain form.
+constexpr int kLseAffine = 1, kLseVecScale = 2, kLseVecShift = 4;
+
+template <typename T, int V, int ITERS, bool FINAL, int MODE>
 __global__ __launch_bounds__(kBlock) void lse_row_block(const RedParams p) {
     using Acc = AccLse<T>;
     const int64_t o = blockIdx.x;
@@ -271,43 +277,36 @@ __global__ __launch_bounds__(kBlock) void lse_row_block(const RedParams p) {
     const int64_t n = r_end - r_begin;
     T x[ITERS][V];
     T m = T(-INFINITY);
-    // every load is issued before the first use (memory-level parallelism: 1 + aux loads per iteration)
+    // every load is issued before the first use (memory-level parallelism)
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
         const int64_t e0 = (static_cast<int64_t>(it) * kBlock + threadIdx.x) * V;
         lse_load<T, V>(p, 0, o, r_begin + e0, n - e0, T(-INFINITY), x[it]);
     }
-    if (AFFINE) {
-        T a[ITERS][V], b[ITERS][V];
-        const bool has_a = p.scale_aux[0] >= 0, has_b = p.shift_aux[0] >= 0;
-        if (has_a) {
+    if (MODE != 0) {
+        constexpr bool VEC_A = (MODE & kLseVecScale) != 0, VEC_B = (MODE & kLseVecShift) != 0;
+        T a[VEC_A ? ITERS : 1][V], b[VEC_B ? ITERS : 1][V];
+        // steps that are absent are the neutral element (x * 1 is exact; x + 0 only loses the sign
+        // of a zero, which neither max nor exp can see), so the arithmetic below is branch-free
+        T ua = T(1), ub = T(0);  // auxiliary operands that do not vary along the row
+        if (VEC_A) {
 #pragma unroll
             for (int it = 0; it < ITERS; ++it) {
                 const int64_t e0 = (static_cast<int64_t>(it) * kBlock + threadIdx.x) * V;
                 lse_load<T, V>(p, p.scale_aux[0], o, r_begin + e0, n - e0, T(1), a[it]);
             }
+        } else if (p.scale_aux[0] >= 0) {
+            ua = static_cast<const T *>(p.in[p.scale_aux[0]])[o * p.istr[p.scale_aux[0]][0]];
         }
-        if (has_b) {
+        if (VEC_B) {
 #pragma unroll
             for (int it = 0; it < ITERS; ++it) {
                 const int64_t e0 = (static_cast<int64_t>(it) * kBlock + threadIdx.x) * V;
                 lse_load<T, V>(p, p.shift_aux[0], o, r_begin + e0, n - e0, T(0), b[it]);
             }
+        } else if (p.shift_aux[0] >= 0) {
+            ub = static_cast<const T *>(p.in[p.shift_aux[0]])[o * p.istr[p.shift_aux[0]][0]];
         }
-        if (!has_a) {
-#pragma unroll
-            for (int it = 0; it < ITERS; ++it)
-#pragma unroll
-                for (int j = 0; j < V; ++j) a[it][j] = T(1);
-        }
-        if (!has_b) {
-#pragma unroll
-            for (int it = 0; it < ITERS; ++it)
-#pragma unroll
-                for (int j = 0; j < V; ++j) b[it][j] = T(0);
-        }
-        // absent steps are the neutral element (x * 1 is exact; x + 0 only loses the sign of a
-        // zero, which neither max nor exp can see), so the arithmetic is branch-free
         const T sc = (p.scale_mask & 1u) ? static_cast<T>(p.scale[0]) : T(1);
         const T sh = (p.shift_mask & 1u) ? static_cast<T>(p.shift[0]) : T(0);
 #pragma unroll
@@ -315,7 +314,10 @@ __global__ __launch_bounds__(kBlock) void lse_row_block(const RedParams p) {
             const int64_t n_left = n - (static_cast<int64_t>(it) * kBlock + threadIdx.x) * V;
 #pragma unroll
             for (int j = 0; j < V; ++j) {
-                const T v = ((x[it][j] * sc) * a[it][j] + sh) + b[it][j];
+                T v = x[it][j] * sc;
+                v = v * (VEC_A ? a[it][j] : ua);
+                v = v + sh;
+                v = v + (VEC_B ? b[it][j] : ub);
                 x[it][j] = j < n_left ? v : T(-INFINITY);  // padding stays neutral
             }
         }
@@ -542,17 +544,37 @@ static int launch_reduce(const char *fname, const RedParams &base, bool vec_ok, 
             if (!(p.scalar_mask & 1u) && p.r_chunk <= static_cast<int64_t>(kBlock) * v * kLseIters) {
                 set_kernel_name("lse_row_block%s", two_stage ? "+red_finish" : "");
                 const int64_t need = ceil_div(p.r_chunk, static_cast<int64_t>(kBlock) * v);
-                const bool affine = ((p.scale_mask | p.shift_mask) & 1u) || p.n_aux > 0;
-#define AGMI_LSE(VV, IT)                                                                                   \
-    do {                                                                                                   \
-        if (two_stage && affine)                                                                           \
-            hipLaunchKernelGGL((lse_row_block<T, VV, IT, false, true>), grid, dim3(kBlock), 0, s, p);      \
-        else if (two_stage)                                                                                \
-            hipLaunchKernelGGL((lse_row_block<T, VV, IT, false, false>), grid, dim3(kBlock), 0, s, p);     \
-        else if (affine)                                                                                   \
-            hipLaunchKernelGGL((lse_row_block<T, VV, IT, true, true>), grid, dim3(kBlock), 0, s, p);       \
-        else                                                                                               \
-            hipLaunchKernelGGL((lse_row_block<T, VV, IT, true, false>), grid, dim3(kBlock), 0, s, p);      \
+                // form of the pending map: auxiliary operands that vary along the reduced axis need registers
+                int mode = 0;
+                if (((p.scale_mask | p.shift_mask) & 1u) || p.n_aux > 0) mode = kLseAffine;
+                if (p.scale_aux[0] >= 0 && p.istr[p.scale_aux[0]][1] != 0) mode |= kLseVecScale;
+                if (p.shift_aux[0] >= 0 && p.istr[p.shift_aux[0]][1] != 0) mode |= kLseVecShift;
+#define AGMI_LSE_MODE(VV, IT, FIN)                                                                                    \
+    do {                                                                                                              \
+        switch (mode) {                                                                                               \
+            case 0: hipLaunchKernelGGL((lse_row_block<T, VV, IT, FIN, 0>), grid, dim3(kBlock), 0, s, p); break;       \
+            case kLseAffine:                                                                                          \
+                hipLaunchKernelGGL((lse_row_block<T, VV, IT, FIN, kLseAffine>), grid, dim3(kBlock), 0, s, p);         \
+                break;                                                                                                \
+            case kLseAffine | kLseVecScale:                                                                           \
+                hipLaunchKernelGGL((lse_row_block<T, VV, IT, FIN, kLseAffine | kLseVecScale>), grid, dim3(kBlock), 0, \
+                                   s, p);                                                                             \
+                break;                                                                                                \
+            case kLseAffine | kLseVecShift:                                                                           \
+                hipLaunchKernelGGL((lse_row_block<T, VV, IT, FIN, kLseAffine | kLseVecShift>), grid, dim3(kBlock), 0, \
+                                   s, p);                                                                             \
+                break;                                                                                                \
+            default:                                                                                                  \
+                hipLaunchKernelGGL((lse_row_block<T, VV, IT, FIN, kLseAffine | kLseVecScale | kLseVecShift>), grid,   \
+                                   dim3(kBlock), 0, s, p);                                                            \
+        }                                                                                                             \
+    } while (0)
+#define AGMI_LSE(VV, IT)                     \
+    do {                                     \
+        if (two_stage)                       \
+            AGMI_LSE_MODE(VV, IT, false);    \
+        else                                 \
+            AGMI_LSE_MODE(VV, IT, true);     \
     } while (0)
 #define AGMI_LSE_IT(VV)                      \
     do {                                     \
@@ -567,6 +589,7 @@ static int launch_reduce(const char *fname, const RedParams &base, bool vec_ok, 
                     AGMI_LSE_IT(1);
 #undef AGMI_LSE_IT
 #undef AGMI_LSE
+#undef AGMI_LSE_MODE
                 goto launched;
             }
         }
