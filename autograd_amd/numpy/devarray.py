@@ -663,6 +663,11 @@ def map_reduce(op, red, dtype, xs, axes, keepdims, shape=None):
             raise ValueError("zero-size array to reduction operation which has no identity")
         _lib.fill(code, out_t, _IDENTITY[red])
     elif not _lib.map_reduce(op, red, code, shape, mask, out_t, ops):
+        if any(type(t) is _lib.Affine and (t.ascale is not None or isinstance(t.shift, torch.Tensor)) for t in ops):
+            # broadcast operands of pending maps can keep reduced axes from merging: write those out, retry
+            settled = [LazyDevArray(t.t, dtype, t.scale, t.shift, t.ascale)._settled() if type(t) is _lib.Affine
+                       else _rewrap(t, dtype) for t in ops]
+            return map_reduce(op, red, dtype, settled, axes, keepdims, shape=shape)
         # reduced axes interleaved with kept ones: one group of adjacent axes at a time
         if red == Red.LOGSUMEXP:
             raise NotImplementedError("logsumexp over non-adjacent axes of a non-contiguous layout")

@@ -566,3 +566,73 @@ def test_einsum_matches_numpy(dnp, dtype):
         dnp.einsum("ii->i", P(dnp, onp.eye(3, dtype=dtype)))
     with pytest.raises(NotImplementedError):
         dnp.einsum(Dv["a"], [0, 1], Dv["b"], [1, 2], [0, 2])
+
+
+@pytest.mark.parametrize("dtype", [F32, F64])
+def test_pending_maps_with_broadcast_operands_are_bit_exact(dnp, dtype):
+    """``A * b[None, :] + c[:, None]`` and friends launch nothing; every consumer kernel applies the
+    steps on load and must round exactly like the NumPy passes."""
+    from autograd_amd.numpy.devarray import LazyDevArray
+    from autograd_amd.scipy.special import logsumexp
+
+    rs = onp.random.RandomState(21)
+    a = rs.randn(67, 130).astype(dtype)
+    b = rs.uniform(0.5, 1.5, 130).astype(dtype)
+    c = rs.randn(67).astype(dtype)
+    y = rs.randn(67, 130).astype(dtype)
+    a[0, :3] = [0.0, -0.0, onp.inf]
+    A, B, C, Y = P(dnp, a), P(dnp, b), P(dnp, c), P(dnp, y)
+    one = dtype(1)
+    cases = [
+        (A * B[None, :], a * b[None, :]),
+        (A + C[:, None], a + c[:, None]),
+        (A * B[None, :] + C[:, None], a * b[None, :] + c[:, None]),
+        (C[:, None] + B * A, c[:, None] + b * a),
+        (-(A * B), -(a * b)),
+        ((A * B) * 2.0 + 1.0, (a * b) * dtype(2) + one),
+        (C[:, None] - A, c[:, None] - a),
+        (2.0 * A * C[:, None], dtype(2) * a * c[:, None]),
+        (A * B[0], a * b[0]),                                     # 0-d array operand
+    ]
+    for k, (L, ref) in enumerate(cases):
+        assert type(L) is LazyDevArray, k
+        nan = onp.isnan(ref)
+        got = L.numpy()
+        assert got.dtype == dtype and onp.array_equal(onp.isnan(got), nan), k
+        assert onp.array_equal(got[~nan].view(onp.uint8), ref[~nan].view(onp.uint8)), k
+        with onp.errstate(all="ignore"):
+            assert onp.array_equal((L * Y).numpy(), ref * y, equal_nan=True), k                 # flat / rows consumer
+            assert onp.array_equal((L.T + Y.T).numpy(), ref.T + y.T, equal_nan=True), k         # transposed view keeps the steps
+            assert onp.array_equal((L[1::2, 3:99] - Y[1::2, 3:99]).numpy(), ref[1::2, 3:99] - y[1::2, 3:99], equal_nan=True), k
+            assert onp.array_equal(dnp.reshape(L, (67, 10, 13)).numpy(), ref.reshape(67, 10, 13), equal_nan=True), k
+            assert onp.array_equal(dnp.exp(L[5]).numpy()[:0], onp.exp(ref[5])[:0]), k
+            close(dnp.exp(L[5] * 0.01).numpy(), onp.exp(ref[5] * dtype(0.01)), RT_EW[dtype] * 8)
+        # more array-valued steps than one launch takes: operands are written out as needed
+        M = (A * B[None, :] + C[:, None]) * (Y * B + C[:, None])
+        with onp.errstate(all="ignore"):
+            assert onp.array_equal(M.numpy(), (a * b[None, :] + c[:, None]) * (y * b + c[:, None]), equal_nan=True)
+    # reductions over finite data: row / column / full sums, fused map, logsumexp in every form
+    af = a[1:]
+    Af, Cf, Yf = P(dnp, af), P(dnp, c[1:]), P(dnp, y[1:])
+    forms = [
+        (Af * B[None, :] + Cf[:, None], af * b[None, :] + c[1:, None]),   # row-varying factor, row-constant offset
+        (Af * Cf[:, None] + B[None, :], af * c[1:, None] + b[None, :]),   # the other way round
+        (Af * B[None, :], af * b[None, :]),
+        (Af + Cf[:, None], af + c[1:, None]),
+        (Af * 0.5 + B, af * dtype(0.5) + b),
+    ]
+    for L, ref in forms:
+        assert type(L) is LazyDevArray
+        close(dnp.sum(L, axis=1).numpy(), ref.sum(axis=1), RT[dtype])
+        close(dnp.sum(L, axis=0).numpy(), ref.sum(axis=0), RT[dtype])
+        close(dnp.sum(L).numpy(), ref.sum(), RT[dtype])
+        close(dnp.max(L, axis=0).numpy(), ref.max(axis=0), 0.0)
+        close(dnp.sum(L * Yf, axis=0).numpy(), (ref * y[1:]).sum(axis=0), RT[dtype])
+        close(logsumexp(L, axis=1).numpy(), scipy.special.logsumexp(ref, axis=1), RT[dtype])
+        close(logsumexp(L, axis=0).numpy(), scipy.special.logsumexp(ref, axis=0), RT[dtype])
+        close(logsumexp(L[:, :37], axis=1).numpy(), scipy.special.logsumexp(ref[:, :37], axis=1), RT[dtype])
+        close(logsumexp(L).numpy(), scipy.special.logsumexp(ref), RT[dtype])
+    wide = rs.randn(9, 5000).astype(dtype)  # rows longer than one block pass: chunked logsumexp
+    wb = rs.uniform(0.5, 1.5, 5000).astype(dtype)
+    close(logsumexp(P(dnp, wide) * P(dnp, wb) + 0.25, axis=1).numpy(),
+          scipy.special.logsumexp(wide * wb + dtype(0.25), axis=1), RT[dtype])

@@ -159,3 +159,36 @@ def test_accumulators_never_write_through_a_pending_map(monkeypatch):
         vs._mut_add(acc, x)
     with pytest.raises(TypeError):
         D.map_op(0, x.dtype, x, out=g)
+
+
+def test_broadcast_operands_fold_into_pending_maps():
+    """Products / sums with a broadcast array operand keep the big operand's storage; the small one
+    becomes an array-valued step (a stride-0 view of the big shape).  Folded only in the kernel's
+    fixed step order: scalar factor, array factor, offset."""
+    from autograd_amd.numpy.devarray import LazyDevArray
+
+    A = meta((8, 6), torch.float64)
+    b = meta((6,), torch.float64)
+    c = meta((8, 1), torch.float64)
+
+    L = A * b
+    assert type(L) is LazyDevArray and L._raw.data_ptr() == A._t.data_ptr() and L._scale == 1.0 and L._shift is None
+    assert tuple(L._ascale.shape) == (8, 6) and L._ascale.stride() == (0, 1) and L._ascale.data_ptr() == b._t.data_ptr()
+    M = b * A + c
+    assert type(M) is LazyDevArray and M._ascale.stride() == (0, 1) and M._shift.stride() == (1, 0)
+    assert M.shape == (8, 6) and M._raw.data_ptr() == A._t.data_ptr()
+    N = -(A * b)
+    assert type(N) is LazyDevArray and N._scale == -1.0 and N._ascale is not None   # (-x) * v == -(x * v) exactly
+    assert type((A * b) * 4.0) is LazyDevArray and ((A * b) * 4.0)._scale == 4.0     # power of two commutes
+    R = c - A
+    assert type(R) is LazyDevArray and R._scale == -1.0 and R._shift.stride() == (1, 0)
+    # views carry the array-valued steps along
+    V = W.transpose(M)[1:4]
+    assert type(V) is LazyDevArray and V.shape == (3, 8) and V._ascale.stride() == (1, 0) and V._shift.stride() == (0, 1)
+    V2 = W.reshape(A * b, (4, 2, 6))
+    assert type(V2) is LazyDevArray and V2._ascale.stride() == (0, 0, 1)
+    # not exact or not expressible in that order: these must launch (no device here -> raise)
+    for expr in (lambda: (A * b) * 3.0, lambda: (A + c) * b, lambda: (A + c) + b, lambda: (A * b) * b, lambda: A - c,
+                 lambda: A / b, lambda: -(A + c), lambda: A * meta((8, 6), torch.float64), lambda: A * meta((6,), torch.float32)):
+        with pytest.raises(Exception):
+            expr()
