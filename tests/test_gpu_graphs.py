@@ -99,3 +99,25 @@ def test_capture_contract_errors():
     with pytest.raises(RuntimeError, match="cannot be recorded"):
         ag.capture(lambda v: dnp.exp(v) * float(dnp.sum(v)), x)
     assert onp.allclose(dnp.exp(x).numpy(), onp.exp(onp.linspace(-1.0, 1.0, 64)), rtol=1e-14)
+
+
+def test_replay_of_random_programs_equals_eager():
+    """Gradients of 40 random programs (pending maps, views, fan-out accumulation) recorded and replayed."""
+    import autograd_amd as ag
+    import autograd_amd.numpy as dnp
+    from autograd_amd.scipy.special import logsumexp
+    from tests.test_gpu_random_programs import make_program
+
+    for seed in range(300, 340):
+        program, inputs = make_program(seed)
+        fun = ag.grad(lambda *xs: program(dnp, logsumexp, *xs), tuple(range(len(inputs))))  # noqa: B023
+        args = [dnp.asarray(a) for a in inputs]
+        graphed = ag.capture(fun, *args)
+        for trial in range(2):
+            if trial:
+                rs = onp.random.RandomState(seed + 1000)
+                args = [dnp.asarray(a + 0.1 * rs.standard_normal(a.shape)) for a in inputs]
+            got = [g.numpy() for g in graphed(*args)]
+            want = [g.numpy() for g in fun(*args)]
+            for g, w in zip(got, want):
+                assert g.dtype == w.dtype and onp.array_equal(g, w, equal_nan=True), (seed, trial)
