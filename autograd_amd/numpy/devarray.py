@@ -254,6 +254,8 @@ def _fold(op, dtype, xs):
         a, c = xs
         swapped = False
         if isinstance(c, DevArray) and isinstance(a, DevArray):
+            if a._h().shape == c._h().shape:
+                return None  # a true elementwise binary operation
             if c.size > a.size:
                 a, c, swapped = c, a, True
             return _fold_array(op, dtype, a, c, swapped)
@@ -520,19 +522,23 @@ def _expand(t, shape):
     return t
 
 
+def _n_aux(t):
+    return (t.ascale is not None) + isinstance(t.shift, torch.Tensor)
+
+
 def _limit_aux(ops, dtype):
     """A launch takes at most ``_lib.MAX_AUX`` array-valued steps: write out the operands that carry
     the most of them until the rest fits."""
-    def n_aux(t):
-        return (t.ascale is not None) + isinstance(t.shift, torch.Tensor) if type(t) is _lib.Affine else 0
-
-    total = sum(n_aux(t) for t in ops)
+    total = 0
+    for t in ops:
+        if type(t) is _lib.Affine:
+            total += _n_aux(t)
     if total <= _lib.MAX_AUX:
         return ops
     ops = list(ops)
     while total > _lib.MAX_AUX:
-        k = max(range(len(ops)), key=lambda i: n_aux(ops[i]))
-        total -= n_aux(ops[k])
+        k = max(range(len(ops)), key=lambda i: _n_aux(ops[i]) if type(ops[i]) is _lib.Affine else 0)
+        total -= _n_aux(ops[k])
         t = ops[k]
         ops[k] = LazyDevArray(t.t, dtype, t.scale, t.shift, t.ascale)._t
     return tuple(ops)

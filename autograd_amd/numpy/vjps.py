@@ -693,5 +693,34 @@ def untake(x, idx, vs):
     return SparseObject(vs, mut_add)
 
 
-defvjp(func(DevArrayBox.__getitem__), lambda ans, A, idx: lambda g: untake(g, idx, vspace(A)))
+def _only_inserts_unit_axes(idx):
+    """True for indices made of ``None``, ``...`` and full slices: ``b[None, :]``, ``c[:, None]``."""
+    items = idx if isinstance(idx, tuple) else (idx,)
+    for it in items:
+        if it is None or it is Ellipsis:
+            continue
+        if isinstance(it, slice) and it.start is None and it.stop is None and it.step is None:
+            continue
+        return False
+    return True
+
+
+def _grad_getitem(ans, A, idx):
+    # numpy_vjps.py:954: untake(g, idx, vspace(A)), a sparse cotangent that add_outgrads scatters into zeros.
+    # An index that only inserts unit axes selects every element exactly once, so that scatter is
+    # `zeros + g` with A's shape: the cotangent itself, reshaped (nothing is launched).
+    vs = vspace(A)
+    if _only_inserts_unit_axes(idx):
+        shape, dtype = vs.shape, vs.dtype
+
+        def vjp(g):
+            if isinstance(g, DevArray) and g.dtype == dtype:
+                return anp.reshape.fun(g, shape)
+            return untake(g, idx, vs)
+
+        return vjp
+    return lambda g: untake(g, idx, vs)
+
+
+defvjp(func(DevArrayBox.__getitem__), _grad_getitem)
 defvjp(untake, lambda ans, x, idx, _: lambda g: g[idx])
