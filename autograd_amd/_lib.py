@@ -93,6 +93,20 @@ class AgmiArray(ctypes.Structure):
                 ("shift_slot", ctypes.c_int32)]
 
 
+class AgmiWindowOperand(ctypes.Structure):
+    _fields_ = [("data", ctypes.c_void_p), ("batch_stride", ctypes.c_int64), ("dot_stride", ctypes.c_int64),
+                ("strides", ctypes.c_int64 * 3)]
+
+
+class AgmiCorrelation(ctypes.Structure):
+    _fields_ = [("n_conv", ctypes.c_int32), ("filter_batch", ctypes.c_int64), ("signal_batch", ctypes.c_int64),
+                ("dot", ctypes.c_int64), ("window", ctypes.c_int64 * 3), ("extent", ctypes.c_int64 * 3),
+                ("pad_before", ctypes.c_int64 * 3), ("out_extent", ctypes.c_int64 * 3),
+                ("filter", AgmiWindowOperand), ("signal", AgmiWindowOperand), ("out", ctypes.c_void_p),
+                ("out_filter_stride", ctypes.c_int64), ("out_signal_stride", ctypes.c_int64),
+                ("out_strides", ctypes.c_int64 * 3)]
+
+
 class Affine:
     """Kernel input slot ``t * scale * ascale + shift``, applied on load in that order, each step
     rounded on its own.  ``scale`` is a Python float (1.0: no multiply); ``ascale`` is None or a tensor
@@ -154,13 +168,16 @@ def lib():
     L.agmi_scatter_add_rows.argtypes = [c_i, c_p, c_i64, c_i64, c_p, c_p, c_p, c_p, c_i64, c_p]
     L.agmi_optimizer_step.restype = c_i
     L.agmi_optimizer_step.argtypes = [c_i, c_i, c_i, c_i64, c_p, c_p, c_p, c_p, c_p, p_d, c_p]
+    L.agmi_correlate.restype = c_i
+    L.agmi_correlate.argtypes = [c_i, ctypes.POINTER(AgmiCorrelation), c_p]
     _LIB = L
     return L
 
 
 EXPORTS = (
     "agmi_last_error agmi_version agmi_last_kernel agmi_elementwise agmi_compare agmi_cast agmi_map_reduce "
-    "agmi_map_reduce_workspace_bytes agmi_gemm agmi_fill agmi_take_rows agmi_scatter_add_rows agmi_optimizer_step"
+    "agmi_map_reduce_workspace_bytes agmi_gemm agmi_fill agmi_take_rows agmi_scatter_add_rows agmi_optimizer_step "
+    "agmi_correlate"
 ).split()
 
 
@@ -453,6 +470,16 @@ def scatter_add_rows(code, dst, n_rows, inner, src, index, order, seg_start, n_s
     _check(_LIB.agmi_scatter_add_rows(code, dst.data_ptr(), n_rows, inner, src.data_ptr(), index.data_ptr(),
                                       order.data_ptr(), seg_start.data_ptr(), n_seg, _stream()),
            "agmi_scatter_add_rows")
+
+
+def correlate(code, args, n_bytes, n_flops):
+    """Launch the sliding-window contraction described by the ``AgmiCorrelation`` block ``args``."""
+    ev = _TIMER.begin(("correlate",)) if _TIMER is not None else None
+    rc = _LIB.agmi_correlate(code, ctypes.byref(args), _stream())
+    if rc:
+        _check(rc, "agmi_correlate")
+    if ev is not None:
+        _TIMER.end(ev, ("correlate",), n_bytes, n_flops)
 
 
 OPT_SGD, OPT_RMSPROP, OPT_ADAM = 0, 1, 2

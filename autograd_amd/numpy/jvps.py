@@ -85,6 +85,7 @@ for _chooser in (anp.maximum, anp.minimum, anp.fmax, anp.fmin):
     )
 
 def_linear(anp.einsum)  # numpy_jvps.py:287
+defjvp(anp.pad, lambda g, ans, array, width, mode, **kwargs: anp.pad(g, width, mode))  # numpy_jvps.py:303
 
 # linear one-argument functions (77-105, 150-162)
 for _name in (

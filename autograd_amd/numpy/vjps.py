@@ -724,3 +724,18 @@ def _grad_getitem(ans, A, idx):
 
 defvjp(func(DevArrayBox.__getitem__), _grad_getitem)
 defvjp(untake, lambda ans, x, idx, _: lambda g: g[idx])
+
+
+def _unpad(array, width):
+    # numpy_vjps.py:957-967
+    idxs = tuple(slice(l, -u or None) for l, u in anp.pad_widths(width, anp.ndim(array)))
+    return array[idxs]
+
+
+def pad_vjp(ans, array, pad_width, mode, **kwargs):
+    # numpy_vjps.py:970-975
+    assert mode == "constant", "Only constant mode padding is supported."
+    return lambda g: _unpad(g, pad_width)
+
+
+defvjp(anp.pad, pad_vjp)

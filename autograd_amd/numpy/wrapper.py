@@ -679,6 +679,34 @@ def scatter_add(A, idx, x):
     return A
 
 
+def pad_widths(pad_width, ndim):
+    """``pad_width`` in any of numpy.pad's spellings -> ((before, after),) * ndim of Python ints."""
+    w = onp.asarray(pad_width)
+    if w.dtype.kind not in "iu":
+        raise TypeError("`pad_width` must be of integral type.")
+    return tuple((int(b), int(a)) for b, a in onp.broadcast_to(w, (ndim, 2)))
+
+
+@primitive
+def pad(array, pad_width, mode="constant", **kwargs):
+    """Zero padding (numpy.pad, constant mode): one fill and one strided copy into the interior."""
+    if mode != "constant" or any(v != 0 for v in onp.ravel(kwargs.get("constant_values", 0))) or set(kwargs) - {"constant_values"}:
+        raise NotImplementedError("pad: only mode='constant' with zeros is supported on the device")
+    x = D.asarray(array)
+    widths = pad_widths(pad_width, x.ndim)
+    if any(b < 0 or a < 0 for b, a in widths):
+        raise ValueError("index can't contain negative values")
+    out = D.zeros(tuple(n + b + a for n, (b, a) in zip(x.shape, widths)), x.dtype)
+    if x.size:
+        inner = out._t[tuple(slice(b, b + n) for n, (b, _) in zip(x.shape, widths))]
+        if x.dtype in D._FLOATS:
+            D.map_op(Op.COPY, x.dtype, x, out=DevArray(inner, x.dtype))
+        else:
+            code = _lib.DTYPE_CODE[x.dtype]
+            _lib.cast(code, code, x.shape, inner, x._t)
+    return out
+
+
 # ---- contractions -------------------------------------------------------------------------------
 def _dot_raw(a, b):
     a, b = D.asarray(a) if not D.is_scalar(a) else a, D.asarray(b) if not D.is_scalar(b) else b

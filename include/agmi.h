@@ -247,6 +247,42 @@ enum agmi_optimizer { AGMI_OPT_SGD = 0, AGMI_OPT_RMSPROP = 1, AGMI_OPT_ADAM = 2 
 int agmi_optimizer_step(int kind, int x_dtype, int g_dtype, int64_t n, const void *x_in, const void *g,
                         void *s0, void *s1, void *x_out, const double *hyper, void *stream);
 
+/* Sliding-window contraction: the strided window view + einsum of the reference's N-d convolution
+ * (scipy/signal.py:45-65; its cotangents, 153-214, are the same contraction on other operands):
+ *
+ *   out[i, j, p] = sum over d and k of  filter[i, d, k] * signal[j, d, p + k - pad_before]
+ *
+ * where p, k and pad_before are multi-indices over n_conv <= AGMI_MAX_CONV_DIMS convolved axes,
+ * 0 <= k < window, 0 <= p < out_extent, and terms whose signal position falls outside
+ * [0, extent) are zero (the reference's explicit zero padding, never written out).  i runs over
+ * the filter's free axes (merged to one, filter_batch values), j over the signal's
+ * (signal_batch), d over the contracted non-convolved axes (dot).  Strides are in elements and
+ * may be negative: an operand read back to front along an axis (the flip of the convolution
+ * proper) passes the address of its LAST element on that axis and a negated stride.  Entries of
+ * window / extent / pad_before / out_extent / strides beyond n_conv are ignored.  Products are
+ * accumulated with fused multiply-adds in the operand type; the summation order is fixed for a
+ * given problem shape (no atomics).  float32 and float64 only. */
+#define AGMI_MAX_CONV_DIMS 3
+typedef struct agmi_window_operand {
+    const void *data;
+    int64_t batch_stride;
+    int64_t dot_stride;
+    int64_t strides[AGMI_MAX_CONV_DIMS];
+} agmi_window_operand;
+typedef struct agmi_correlation {
+    int32_t n_conv;
+    int64_t filter_batch, signal_batch, dot;
+    int64_t window[AGMI_MAX_CONV_DIMS];
+    int64_t extent[AGMI_MAX_CONV_DIMS];
+    int64_t pad_before[AGMI_MAX_CONV_DIMS];
+    int64_t out_extent[AGMI_MAX_CONV_DIMS];
+    agmi_window_operand filter, signal;
+    void *out;
+    int64_t out_filter_stride, out_signal_stride;
+    int64_t out_strides[AGMI_MAX_CONV_DIMS];
+} agmi_correlation;
+int agmi_correlate(int dtype, const agmi_correlation *c, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -596,3 +596,24 @@ def untake(x, idx, vs):
 
 defvjp(func(ArrayBox.__getitem__), lambda ans, A, idx: lambda g: untake(g, idx, vspace(A)))
 defvjp(untake, lambda ans, x, idx, _: lambda g: g[idx])
+
+
+# ---- zero padding (numpy_vjps.py:957-975) ------------------------------------------------------
+def _unpad(array, width):
+    if anp.isscalar(width):
+        width = [[width, width]]
+    elif anp.shape(width) == (1,):
+        width = [anp.concatenate((width, width))]
+    elif anp.shape(width) == (2,):
+        width = [width]
+    if anp.shape(width)[0] == 1:
+        width = anp.repeat(width, anp.ndim(array), 0)
+    return array[tuple(slice(lo, -hi or None) for lo, hi in width)]
+
+
+def _pad_vjp(ans, array, pad_width, mode, **kwargs):
+    assert mode == "constant", "Only constant mode padding is supported."
+    return lambda g: _unpad(g, pad_width)
+
+
+defvjp(anp.pad, _pad_vjp)

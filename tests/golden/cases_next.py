@@ -2,7 +2,7 @@
 optimizers, Jacobians/Hessians, and the rest of the elementwise rule table.
 
 ``next_cases(be, ext)`` is written against a ``configs.Backend`` plus a namespace ``ext`` with
-``flatten, sgd, rmsprop, adam, jacobian, hessian`` so the same code runs on the reference (when
+``flatten, sgd, rmsprop, adam, jacobian, hessian, convolve`` so the same code runs on the reference (when
 writing fixtures), the CPU oracle and the device.
 """
 
@@ -110,4 +110,39 @@ def next_cases(be, ext):
             weights = P(onp.asarray(rs.randn(*onp.shape(be.get(out[f"einsum/{name}_{tag}/value"])))).astype(dtype))
             f = lambda *xs: np.sum(np.einsum(spec, *xs) * weights)  # noqa: E731,B023
             out[f"einsum/{name}_{tag}/grad"] = grad(f, tuple(range(len(args))))(*args)
+
+    # ---- scipy.signal.convolve (scipy/signal.py:10-217): modes, operand orders, free / contracted axes ----
+    conv = ext.convolve
+    for dtype in (onp.float64, onp.float32):
+        tag = "f32" if dtype == onp.float32 else "f64"
+        C = {k: P(rs.randn(*shp).astype(dtype)) for k, shp in
+             dict(v5=(5,), v3=(3,), v4=(4,), img=(2, 3, 6, 5), filt=(3, 4, 3, 2), m45=(4, 5), m23=(2, 3), m62=(6, 2),
+                  m33=(3, 3), vol=(3, 4, 3), cube=(2, 2, 2), bat=(2, 5, 4), bank=(3, 2, 2)).items()}
+        specs = []
+        for mode in ("full", "valid", "same"):
+            specs += [(f"1d_{mode}", ("v5", "v3"), dict(mode=mode)), (f"1d_swapped_{mode}", ("v3", "v5"), dict(mode=mode)),
+                      (f"1d_even_{mode}", ("v5", "v4"), dict(mode=mode)),
+                      (f"2d_{mode}", ("m45", "m23"), dict(mode=mode)), (f"2d_swapped_{mode}", ("m23", "m45"), dict(mode=mode)),
+                      (f"3d_{mode}", ("vol", "cube"), dict(mode=mode)),
+                      (f"free_axes_{mode}", ("bat", "bank"), dict(axes=([1, 2], [1, 2]), mode=mode)),
+                      (f"convnet_{mode}", ("img", "filt"), dict(axes=([2, 3], [2, 3]), dot_axes=([1], [0]), mode=mode))]
+        specs += [("2d_mixed_full", ("m45", "m62"), dict(mode="full")), ("2d_mixed_same", ("m45", "m62"), dict(mode="same")),
+                  ("2d_equal_full", ("m33", "m33"), dict(mode="full")), ("2d_equal_valid", ("m33", "m33"), dict(mode="valid")),
+                  ("one_axis_of_two", ("m45", "m23"), dict(axes=([1], [1]), mode="full")),
+                  ("dot_first", ("m45", "m45"), dict(axes=([1], [1]), dot_axes=([0], [0]), mode="full"))]
+        for name, ops, kw in specs:
+            a, b = C[ops[0]], C[ops[1]]
+            value = conv(a, b, **kw)
+            out[f"conv/{name}_{tag}/value"] = value
+            weights = P(rs.randn(*onp.shape(be.get(value))).astype(dtype))
+            f = lambda x, y: np.sum(conv(x, y, **kw) * weights)  # noqa: E731,B023
+            out[f"conv/{name}_{tag}/grad"] = grad(f, (0, 1))(a, b)
+    # second order: the cotangent rules differentiated again (every flip of operands and result occurs)
+    for mode in ("full", "valid", "same"):
+        for name, ops, kw in [("1d", ("v5", "v4"), {}), ("1d_swapped", ("v3", "v5"), {}),
+                              ("convnet", ("img", "filt"), dict(axes=([2, 3], [2, 3]), dot_axes=([1], [0])))]:
+            a, b = C[ops[0]], C[ops[1]]
+            first = lambda x, y: np.sum(np.sin(conv(x, y, mode=mode, **kw)))  # noqa: E731,B023
+            second = lambda x, y: sum(np.sum(np.tanh(d)) for d in grad(first, (0, 1))(x, y))  # noqa: E731,B023
+            out[f"conv/second_{name}_{mode}"] = grad(second, (0, 1))(a, b)
     return out

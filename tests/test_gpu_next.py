@@ -24,9 +24,10 @@ def device_ext():
     import autograd_amd as ag
     import autograd_amd.misc.optimizers as opt
     from autograd_amd.misc import flatten as dflatten
+    from autograd_amd.scipy.signal import convolve
 
     return SimpleNamespace(flatten=dflatten, sgd=opt.sgd, rmsprop=opt.rmsprop, adam=opt.adam, jacobian=ag.jacobian,
-                           hessian=ag.hessian)
+                           hessian=ag.hessian, convolve=convolve)
 
 
 def test_next_cases_match_reference_vectors():

@@ -19,9 +19,10 @@ GOLD = np.load(os.path.join(os.path.dirname(__file__), "golden", "reference_next
 
 def oracle_ext():
     import oracle.misc as M
+    from oracle.convolution import convolve
 
     return SimpleNamespace(flatten=M.flatten, sgd=M.sgd, rmsprop=M.rmsprop, adam=M.adam, jacobian=ag.jacobian,
-                           hessian=ag.hessian)
+                           hessian=ag.hessian, convolve=convolve)
 
 
 def test_next_cases_bit_identical():
