@@ -210,6 +210,42 @@ def rosen_program(be):
 
 
 # --------------------------------------------------------------------------------------
+# beside the five configs: the LeNet-style stack of examples/convnet.py (conv 5x5x6, 2x2 max pool,
+# conv 5x5x16, 2x2 max pool, tanh 120, tanh 84, log-softmax 10) on 28x28 images
+# --------------------------------------------------------------------------------------
+def convnet_inputs(batch=256, seed=0, dtype=onp.float64):
+    rs = onp.random.RandomState(seed)
+    shapes = {"c1": (1, 6, 5, 5), "b1": (1, 6, 1, 1), "c2": (6, 16, 5, 5), "b2": (1, 16, 1, 1),
+              "w3": (256, 120), "b3": (120,), "w4": (120, 84), "b4": (84,), "w5": (84, 10), "b5": (10,)}
+    params = {k: (0.1 * rs.randn(*shp)).astype(dtype) for k, shp in shapes.items()}
+    X = rs.rand(batch, 1, 28, 28).astype(dtype)
+    T = (rs.randint(0, 10, batch)[:, None] == onp.arange(10)[None, :]).astype(dtype)
+    return {"params": params, "X": X, "T": T}
+
+
+def convnet_program(be, convolve):
+    np, logsumexp = be.np, be.logsumexp
+
+    def pool(x):  # examples/convnet.py:112-119
+        n, c, h, w = x.shape
+        return np.max(np.max(x.reshape((n, c, h // 2, 2, w // 2, 2)), axis=3), axis=4)
+
+    def predict(p, X):
+        h = pool(convolve(X, p["c1"], axes=([2, 3], [2, 3]), dot_axes=([1], [0]), mode="valid") + p["b1"])
+        h = pool(convolve(h, p["c2"], axes=([2, 3], [2, 3]), dot_axes=([1], [0]), mode="valid") + p["b2"])
+        h = h.reshape((h.shape[0], 256))
+        h = np.tanh(np.dot(h, p["w3"]) + p["b3"])
+        h = np.tanh(np.dot(h, p["w4"]) + p["b4"])
+        out = np.dot(h, p["w5"]) + p["b5"]
+        return out - logsumexp(out, axis=1, keepdims=True)
+
+    def loss(p, X, T):
+        return -np.sum(predict(p, X) * T)
+
+    return {"loss": loss, "grad": be.grad(loss)}
+
+
+# --------------------------------------------------------------------------------------
 # uniform runner: name -> {output name -> host array tree}
 # --------------------------------------------------------------------------------------
 def run_config(name, be, inputs):

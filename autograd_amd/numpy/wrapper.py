@@ -251,6 +251,9 @@ _astype = astype
 # ---- reductions ---------------------------------------------------------------------------------
 def _reduction(red, name):
     def raw(x, axis=None, keepdims=False, dtype=None, out=None, **kwargs):
+        if type(x) in (tuple, list) and all(isinstance(e, (int, onp.integer)) for e in x):
+            # shape arithmetic on a tuple of Python ints (np.prod(shape)) stays a host integer, usable in slices
+            return getattr(onp, name)(x, axis=axis, dtype=dtype, keepdims=keepdims)
         x = D.asarray(x)
         dt = D._float_dtype(x.dtype) if dtype is None else onp.dtype(dtype)
         return D.map_reduce(Op.COPY, red, dt, (x,), D.normalize_axes(axis, x.ndim), keepdims)

@@ -1,7 +1,7 @@
 """``autograd_amd.scipy.signal.convolve`` and ``numpy.pad`` on the device against the CPU oracle
 (oracle/convolution.py, itself bit-identical to the reference on tests/golden/reference_next.npz)
-at sizes that reach every launch shape of the window-contraction kernel (1, 8, 64 and 256 lanes
-per output) and the operand-copy path.
+at sizes that reach both window-contraction kernels (one thread per position with filter-batch
+tiles of 1, 2, 4 and 8; one block per output) and the operand-copy path.
 
 Tolerance: |got - want| <= rtol * (|want| + max|want|), rtol 1e-5 (float32) / 1e-12 (float64); the
 summation order of a device contraction differs from numpy.einsum's.
@@ -48,7 +48,7 @@ def test_convnet_layer_forward_and_both_cotangents(dtype):
     rs = onp.random.RandomState(0)
     img, filt = rs.randn(8, 3, 14, 14).astype(dtype), rs.randn(3, 5, 5, 5).astype(dtype)
     kernel = _both(dict(axes=([2, 3], [2, 3]), dot_axes=([1], [0]), mode="valid"), img, filt, dtype)
-    assert kernel.startswith("correlate_kernel")
+    assert kernel.startswith("correlate_reduce")
 
 
 @pytest.mark.parametrize("mode", ["full", "valid", "same"])
@@ -58,20 +58,20 @@ def test_long_one_dimensional_windows(mode):
     _both(dict(mode=mode), rs.randn(2000).astype(onp.float32), rs.randn(700).astype(onp.float32), onp.float32)
 
 
-def test_one_lane_per_output_on_a_large_image():
+@pytest.mark.parametrize("filters,tile", [(1, 1), (2, 2), (4, 4), (6, 8), (16, 8)])
+def test_one_thread_per_position_with_filter_batch_tiles(filters, tile):
     import autograd_amd.numpy as dnp
     from autograd_amd import _lib
     from autograd_amd.scipy.signal import convolve as dconv
     from oracle.convolution import convolve as oconv
 
     rs = onp.random.RandomState(2)
-    img, filt = rs.randn(16, 2, 96, 96).astype(onp.float32), rs.randn(2, 2, 3, 3).astype(onp.float32)
-    kw = dict(axes=([2, 3], [2, 3]), dot_axes=([1], [0]), mode="valid")
-    got = dconv(dnp.asarray(img), dnp.asarray(filt), **kw)
-    assert _lib.lib().agmi_last_kernel().decode() == "correlate_kernel<float, 1>"
-    _close(got.numpy(), oconv(img, filt, **kw), onp.float32)
-    same = dconv(dnp.asarray(img), dnp.asarray(filt), axes=([2, 3], [2, 3]), dot_axes=([1], [0]), mode="same")
-    _close(same.numpy(), oconv(img, filt, axes=([2, 3], [2, 3]), dot_axes=([1], [0]), mode="same"), onp.float32)
+    img, filt = rs.randn(64, 2, 36, 36).astype(onp.float32), rs.randn(2, filters, 5, 5).astype(onp.float32)
+    for mode in ("valid", "same"):
+        kw = dict(axes=([2, 3], [2, 3]), dot_axes=([1], [0]), mode=mode)
+        got = dconv(dnp.asarray(img), dnp.asarray(filt), **kw)
+        assert _lib.lib().agmi_last_kernel().decode() == f"correlate_positions<float, {tile}>"
+        _close(got.numpy(), oconv(img, filt, **kw), onp.float32)
 
 
 def test_free_axes_that_do_not_merge_are_copied_once():
