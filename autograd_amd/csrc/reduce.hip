@@ -462,6 +462,30 @@ __global__ __launch_bounds__(kBlock) void red_cols(const RedParams p, const int 
     }
 }
 
+// ---- short form ------------------------------------------------------------------------------
+// Few reduced elements per output and many outputs (a 2x2 pooling window, a short middle axis): a
+// thread owns V consecutive i of one o and walks the R reduced elements itself, so no lane idles.
+template <template <typename> class F, template <typename> class AccT, typename T, int V>
+__global__ __launch_bounds__(kBlock) void red_short(const RedParams p, const int64_t i_vecs) {
+    using Acc = AccT<T>;
+    using acc_t = typename Acc::type;
+    const int64_t e = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (e >= p.O * i_vecs) return;
+    const int64_t o = e / i_vecs, i0 = (e - o * i_vecs) * V;
+    acc_t acc[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) acc[j] = Acc::identity();
+#pragma unroll 2
+    for (int64_t r = 0; r < p.R; ++r) {
+        T x[F<T>::NIN + AGMI_MAX_AUX][V];
+        load_points<F, T, V, 2>(p, o, r, i0, x);
+#pragma unroll
+        for (int j = 0; j < V; ++j) acc[j] = Acc::combine(acc[j], Acc::lift(map_point<F, T, V>(p, x, j)));
+    }
+#pragma unroll
+    for (int j = 0; j < V; ++j) store_result<Acc, T, true>(p, acc[j], o, i0 + j, 0);
+}
+
 // ---- second stage: combine chunk partials ---------------------------------------------------------
 // block = FX x FY threads (FX * FY = 256): FX consecutive outputs (coalesced reads of one chunk's
 // partials), FY strided walkers over the chunks, LDS tree over FY.  FX shrinks with the number of
@@ -497,9 +521,12 @@ __global__ __launch_bounds__(kBlock) void red_finish(const void *partial, T *out
 }
 
 // ---- planning ------------------------------------------------------------------------------------
+constexpr int64_t kShortReduce = 16;  // reduced extents up to this are walked by one thread (column form)
+
 struct RedPlan {
     bool row_form;
     bool block_per_row;
+    bool short_form;
     int G;         // row_group lanes per row, or finish lanes per output
     int V;         // vector width in elements (1 or 16 / sizeof(T))
     int TX;        // col form
@@ -543,6 +570,10 @@ static RedPlan plan_reduce(int64_t O, int64_t R, int64_t I, int vec, bool vec_ok
     } else {
         pl.row_form = false;
         pl.V = (vec_ok && I % vec == 0) ? vec : 1;
+        if (R <= kShortReduce) {
+            pl.short_form = true;
+            return pl;
+        }
         // a thread-row covers ~256 contiguous bytes of one row of the operands; the rest of the
         // block's threads walk different rows, so many blocks fit across I and few chunks are needed
         const int tx_full = std::max<int>(1, 256 / (pl.V * static_cast<int>(elem_size)));
@@ -662,6 +693,18 @@ static int launch_reduce(const char *fname, const RedParams &base, bool vec_ok, 
         else
             AGMI_ROW(1);
 #undef AGMI_ROW
+    } else if (pl.short_form) {
+        const int64_t i_vecs = p.I / pl.V;
+        const int64_t blocks = ceil_div(p.O * i_vecs, kBlock);
+        if (blocks > 0x7fffffffLL) {
+            set_error("map_reduce: too many outputs");
+            return AGMI_ERR_UNSUPPORTED;
+        }
+        set_kernel_name("red_short<%s>", fname);
+        if (pl.V > 1)
+            hipLaunchKernelGGL((red_short<F, AccT, T, VEC>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p, i_vecs);
+        else
+            hipLaunchKernelGGL((red_short<F, AccT, T, 1>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p, i_vecs);
     } else {
         const int64_t blocks_x = ceil_div(ceil_div(p.I, pl.V), pl.TX);
         if (blocks_x > 0x7fffffffLL || p.O * pl.n_chunks > 65535) {

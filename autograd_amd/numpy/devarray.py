@@ -677,7 +677,10 @@ def map_reduce(op, red, dtype, xs, axes, keepdims, shape=None):
         # reduced axes interleaved with kept ones: one group of adjacent axes at a time
         if red == Red.LOGSUMEXP:
             raise NotImplementedError("logsumexp over non-adjacent axes of a non-contiguous layout")
-        cur = map_op(op, dtype, *[_rewrap(t, dtype) for t in ops])
+        if op == Op.COPY and isinstance(ops[0], torch.Tensor) and ops[0].is_contiguous():
+            cur = DevArray(ops[0], dtype)  # nothing to apply or lay out first: reduce the operand itself
+        else:
+            cur = map_op(op, dtype, *[_rewrap(t, dtype) for t in ops])
         for group in _adjacent_groups(axes):
             cur = map_reduce(Op.COPY, red, dtype, (cur,), group, True)
         out_t = cur._t

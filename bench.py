@@ -34,9 +34,9 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing")
     ap.add_argument("--no-extras", action="store_true", help="skip the other workloads")
     ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget for the CPU baseline sample")
-    ap.add_argument("--workload", default="bcast", choices=["bcast", "tanh", "mlp", "rnn", "rosen"],
+    ap.add_argument("--workload", default="bcast", choices=["bcast", "tanh", "mlp", "rnn", "rosen", "convnet"],
                     help="bcast (default) is the headline workload, BASELINE configs[1]; the others are the "
-                         "remaining BASELINE configs, selectable for profiling")
+                         "remaining BASELINE configs and the convnet example, selectable for profiling")
     ap.add_argument("--graph", action="store_true",
                     help="time the workload replayed from a HIP graph (autograd_amd.capture) instead of the eager "
                          "tracer; no per-kernel events in this mode")
@@ -126,6 +126,16 @@ def make_workload(name, be):
         g = configs.rnn_program(be)["grad"]
         cfg = {"workload": "configs[3] tanh RNN T=64 B=256 H=512, grad wrt params dict", "seed": 0}
         return g, (params, xs, ts), cfg, "f32"
+    if name == "convnet":
+        from autograd_amd.scipy.signal import convolve
+
+        inp = configs.convnet_inputs(dtype="float32")
+        params = configs.tree_map(be.put, inp["params"])
+        X, T = be.put(inp["X"]), be.put(inp["T"])
+        g = configs.convnet_program(be, convolve)["grad"]
+        cfg = {"workload": "examples/convnet.py LeNet stack (conv5x5x6, pool, conv5x5x16, pool, 120, 84, 10) on 28x28, "
+                           "grad wrt params dict", "batch": 256, "seed": 0}
+        return g, (params, X, T), cfg, "f32"
     inp = configs.rosen_inputs()
     x, v = be.put(inp["x"]), be.put(inp["v"])
     prog = configs.rosen_program(be)
@@ -187,9 +197,10 @@ def main():
         elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
     dom = kt.summary()[dominant]
-    if dominant.startswith("gemm_mfma"):
+    if dominant.startswith(("gemm_mfma", "correlate")):
         achieved = dom["avg_flops"] / (dom["avg_ms"] * 1e-3) / 1e12
-        roofline = {"bound": "mfma", "kernel": dominant, "achieved": achieved, "peak": MFMA_F32_PEAK_TFLOPS,
+        # the window contraction runs on the vector ALUs, whose published fp32 peak equals the MFMA one
+        roofline = {"bound": "mfma" if dominant.startswith("gemm") else "valu", "kernel": dominant, "achieved": achieved, "peak": MFMA_F32_PEAK_TFLOPS,
                     "unit": "TFLOP/s", "frac": achieved / MFMA_F32_PEAK_TFLOPS, "traffic": None,
                     "algorithmic_flops_per_launch": dom["avg_flops"]}
     else:

@@ -217,6 +217,9 @@ RED_SHAPES = [
     ((3000, 260), 0), ((3000, 256), 0), ((2, 70000), 1),          # two-stage column / row
     ((6, 50, 8), 1), ((6, 50, 8), (0, 2)), ((6, 50, 8), (1, 2)), ((6, 50, 8), (0, 1)), ((6, 50, 8), None),
     ((4, 1, 9), 1), ((0, 5), 0), ((5, 0), 0),
+    # few reduced elements per output (one thread walks them): pooling windows, short middle axes, vector tails
+    ((64, 2, 24), 1), ((18, 3, 6, 2, 12, 2), 3), ((18, 3, 6, 2, 12, 2), 5), ((500, 16, 7), 1), ((500, 17, 8), 1),
+    ((2, 300000), 0), ((5, 3), 0), ((16, 4099), 0),
 ]
 
 
@@ -272,7 +275,7 @@ def test_fused_map_reduce_is_unbroadcast(dnp, dtype):
 
 @pytest.mark.parametrize("dtype", [F32, F64])
 @pytest.mark.parametrize("shape,axis", [((1024, 10), 1), ((256, 128), 1), ((37, 4096), 1), ((37, 4096), 0),
-                                        ((5, 4), None), ((6, 50, 8), 1), ((3, 70000), 1), ((4, 5), (0, 1))])
+                                        ((5, 4), None), ((6, 50, 8), 1), ((3, 70000), 1), ((4, 5), (0, 1)), ((9, 700), 0), ((6, 12, 8), 1)])
 def test_logsumexp_forward(dnp, dtype, shape, axis):
     from autograd_amd.scipy.special import logsumexp
 
