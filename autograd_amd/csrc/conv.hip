@@ -86,7 +86,7 @@ __global__ __launch_bounds__(kBlock) void correlate_positions(const T *__restric
                 for (int64_t k2 = 0; k2 < c.K[2]; ++k2) {
                     const int64_t s2 = b2 + k2;
                     const bool in = in1 && static_cast<uint64_t>(s2) < static_cast<uint64_t>(c.N[2]);
-                    const T sv = in ? sr[s2 * c.s_s[2]] : T(0);
+                    const T sv = in ? sr[s2 * c.s_s[2]] : T(0);  // a tap that falls off the signal is padding
                     const int64_t fo = fr + k2 * c.f_s[2];
 #pragma unroll
                     for (int t = 0; t < TI; ++t) acc[t] = fused_mul_add(f[t][fo], sv, acc[t]);
@@ -238,6 +238,8 @@ extern "C" int agmi_correlate(int dtype, const agmi_correlation *a, void *stream
     }
     const int64_t outputs = c.I * c.J * p_total;
     if (outputs == 0) return 0;
+    for (int d = 0; d < 3; ++d)
+        if (c.N[d] == 0) c.D = 0;  // an empty signal: every tap is padding, the result is all zeros
     const int64_t r_total = c.D * k_total;
     if (r_total > 0x7fffffffLL || c.I > 0x7fffffffLL || c.J > 0x7fffffffLL) {
         set_error("correlate: reduction of %lld terms is too long", static_cast<long long>(r_total));
@@ -255,8 +257,8 @@ extern "C" int agmi_correlate(int dtype, const agmi_correlation *a, void *stream
     c.o_ss = a->out_signal_stride;
     c.p_total = static_cast<uint32_t>(p_total);
 
-    // Widest filter-batch tile that still leaves 256 blocks of position threads; when even single
-    // entries do not give 64 blocks and the reduction is long enough to share, one block per output.
+    // Widest filter-batch tile that still leaves four waves per SIMD of position threads; when even
+    // single entries do not give 64 blocks and the reduction is long enough to share, one block per output.
     const int64_t pairs = c.J * p_total;
     if (pairs > 0x7fffffffLL) {
         set_error("correlate: too many output positions for one launch");

@@ -66,7 +66,7 @@ def test_one_thread_per_position_with_filter_batch_tiles(filters, tile):
     from oracle.convolution import convolve as oconv
 
     rs = onp.random.RandomState(2)
-    img, filt = rs.randn(64, 2, 36, 36).astype(onp.float32), rs.randn(2, filters, 5, 5).astype(onp.float32)
+    img, filt = rs.randn(64, 2, 68, 68).astype(onp.float32), rs.randn(2, filters, 5, 5).astype(onp.float32)
     for mode in ("valid", "same"):
         kw = dict(axes=([2, 3], [2, 3]), dot_axes=([1], [0]), mode=mode)
         got = dconv(dnp.asarray(img), dnp.asarray(filt), **kw)
