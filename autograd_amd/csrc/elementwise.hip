@@ -36,37 +36,56 @@ struct EwParams {
     int64_t istr[kMaxPhysIn][kMaxMerged];
 };
 
+// The pending affine maps of an op's inputs, read out of the launch parameters in one go.  Every
+// field is read unconditionally, so the reads become a few wide scalar loads at the top of the
+// kernel whose latency overlaps with the operand loads, instead of one dependent scalar load
+// behind each branch.
+template <typename T, int NIN>
+struct AffineRegs {
+    unsigned scale_mask, shift_mask;
+    T scale[NIN], shift[NIN];
+    int scale_aux[NIN], shift_aux[NIN];
+    template <class P>
+    __device__ __forceinline__ explicit AffineRegs(const P &p) : scale_mask(p.scale_mask), shift_mask(p.shift_mask) {
+#pragma unroll
+        for (int k = 0; k < NIN; ++k) {
+            scale[k] = static_cast<T>(p.scale[k]);
+            shift[k] = static_cast<T>(p.shift[k]);
+            scale_aux[k] = p.scale_aux[k];
+            shift_aux[k] = p.shift_aux[k];
+        }
+    }
+};
+
 // Apply the inputs' pending affine maps to the V points a thread has gathered: multiply, then
 // add, each rounded on its own.  `x` holds the op's NIN inputs followed by NAUX auxiliary
 // operands (array-valued factors / offsets).  All tests are wave-uniform and made once per
 // input, not once per point, so plain operands pay a few scalar branches per thread.
-template <typename T, int NIN, int NAUX, int V, class P>
-__device__ __forceinline__ void apply_affine(const P &p, T (&x)[NIN + NAUX][V]) {
-    if (NAUX == 0 && (p.scale_mask | p.shift_mask) == 0) return;
+template <typename T, int NIN, int NAUX, int V>
+__device__ __forceinline__ void apply_affine(const AffineRegs<T, NIN> &r, T (&x)[NIN + NAUX][V]) {
+    if (NAUX == 0 && (r.scale_mask | r.shift_mask) == 0) return;
 #pragma unroll
     for (int k = 0; k < NIN; ++k) {
-        if (p.scale_mask & (1u << k)) {
-            const T s = static_cast<T>(p.scale[k]);
+        if (r.scale_mask & (1u << k)) {
 #pragma unroll
-            for (int j = 0; j < V; ++j) x[k][j] = x[k][j] * s;
+            for (int j = 0; j < V; ++j) x[k][j] = x[k][j] * r.scale[k];
         }
-        if (NAUX > 0 && p.scale_aux[k] >= 0) {
+        if (NAUX > 0 && r.scale_aux[k] >= 0) {
 #pragma unroll
             for (int a = 0; a < NAUX; ++a)
-                if (p.scale_aux[k] == NIN + a) {
+                if (r.scale_aux[k] == NIN + a) {
 #pragma unroll
                     for (int j = 0; j < V; ++j) x[k][j] = x[k][j] * x[NIN + a][j];
                 }
         }
-        if (p.shift_mask & (1u << k)) {
-            const T s = static_cast<T>(p.shift[k]);
+        if (r.shift_mask & (1u << k)) {
 #pragma unroll
-            for (int j = 0; j < V; ++j) x[k][j] = x[k][j] + s;
+            for (int j = 0; j < V; ++j) x[k][j] = x[k][j] + r.shift[k];
         }
-        if (NAUX > 0 && p.shift_aux[k] >= 0) {
+        if (NAUX > 0 && r.shift_aux[k] >= 0) {
 #pragma unroll
             for (int a = 0; a < NAUX; ++a)
-                if (p.shift_aux[k] == NIN + a) {
+                if (r.shift_aux[k] == NIN + a) {
 #pragma unroll
                     for (int j = 0; j < V; ++j) x[k][j] = x[k][j] + x[NIN + a][j];
                 }
@@ -91,12 +110,13 @@ __global__ __launch_bounds__(kBlock) void ew_flat(const EwParams p) {
     using vec_t = typename Vec<T>::type;
     const int64_t i0 = (static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x) * V;
     if (i0 >= p.n) return;
+    const AffineRegs<T, Fn::NIN> affine(p);
     T x[NP][V];
     T o[Fn::NOUT][V];
     if (i0 + V <= p.n) {
 #pragma unroll
         for (int k = 0; k < NP; ++k) {
-            if (p.scalar_mask & (1u << k)) {
+            if (k < Fn::NIN && (p.scalar_mask & (1u << k))) {
                 const T s = static_cast<T>(p.scalar[k]);
 #pragma unroll
                 for (int j = 0; j < V; ++j) x[k][j] = s;
@@ -110,7 +130,7 @@ __global__ __launch_bounds__(kBlock) void ew_flat(const EwParams p) {
                 for (int j = 0; j < V; ++j) x[k][j] = v[j];
             }
         }
-        apply_affine<T, Fn::NIN, NAUX, V>(p, x);
+        apply_affine<T, Fn::NIN, NAUX, V>(affine, x);
 #pragma unroll
         for (int j = 0; j < V; ++j) {
             T xi[Fn::NIN], oi[Fn::NOUT];
@@ -132,12 +152,12 @@ __global__ __launch_bounds__(kBlock) void ew_flat(const EwParams p) {
             T x1[NP][1], xi[Fn::NIN], oi[Fn::NOUT];
 #pragma unroll
             for (int k = 0; k < NP; ++k) {
-                if (p.scalar_mask & (1u << k))
+                if (k < Fn::NIN && (p.scalar_mask & (1u << k)))
                     x1[k][0] = static_cast<T>(p.scalar[k]);
                 else
                     x1[k][0] = static_cast<const T *>(p.in[k])[p.istr[k][0] == 0 ? 0 : i];
             }
-            apply_affine<T, Fn::NIN, NAUX, 1>(p, x1);
+            apply_affine<T, Fn::NIN, NAUX, 1>(affine, x1);
 #pragma unroll
             for (int k = 0; k < Fn::NIN; ++k) xi[k] = x1[k][0];
             Fn::apply(xi, oi);
@@ -150,28 +170,52 @@ __global__ __launch_bounds__(kBlock) void ew_flat(const EwParams p) {
 // ---- rows ------------------------------------------------------------------------------
 // shape = (R, C); every operand has inner stride 1 or 0.  `tpr` = threads per row.
 template <template <typename> class F, typename T, typename Index, int NAUX>
-__global__ __launch_bounds__(kBlock) void ew_rows(const EwParams p, const Index tpr, const Index total) {
+__global__ __launch_bounds__(kBlock) void ew_rows(const EwParams p, const Index tpr, const Index total,
+                                                  const int tile_shift) {
     using Fn = F<T>;
     constexpr int NP = Fn::NIN + NAUX;
     constexpr int V = Vec<T>::N;
     using vec_t = typename Vec<T>::type;
-    const Index t = static_cast<Index>(blockIdx.x) * kBlock + threadIdx.x;
-    if (t >= total) return;
-    const Index row = t / tpr;
-    const int64_t c0 = static_cast<int64_t>(t - row * tpr) * V;
+    Index row, in_row;
+    if (tile_shift >= 0) {
+        // a row spans 2^tile_shift whole blocks: the row comes from the block index with scalar shifts,
+        // where the general mapping below spends some 25 vector instructions on an integer division
+        row = static_cast<Index>(blockIdx.x >> tile_shift);
+        in_row = static_cast<Index>(((blockIdx.x & ((1u << tile_shift) - 1u)) * kBlock) + threadIdx.x);
+        if (in_row >= tpr) return;
+    } else {
+        const Index t = static_cast<Index>(blockIdx.x) * kBlock + threadIdx.x;
+        if (t >= total) return;
+        row = t / tpr;
+        in_row = t - row * tpr;
+    }
+    const int64_t c0 = static_cast<int64_t>(in_row) * V;
     const int64_t C = p.shape[1];
     const bool full = c0 + V <= C;
     const int nvalid = full ? V : static_cast<int>(C - c0);
+    // every operand's descriptor is read before the first load is issued (see AffineRegs)
+    const unsigned scalar_mask = p.scalar_mask;
+    const AffineRegs<T, Fn::NIN> affine(p);
+    const T *bases[NP];
+    bool broadcast[NP];
+#pragma unroll
+    for (int k = 0; k < NP; ++k) {
+        bases[k] = static_cast<const T *>(p.in[k]) + static_cast<int64_t>(row) * p.istr[k][0];
+        const int64_t inner = p.istr[k][1];
+        // keep the compiler from sinking these reads back behind the branches that use them
+        asm volatile("" : : "v"(bases[k]), "s"(inner));
+        broadcast[k] = inner == 0;
+    }
     T x[NP][V];
 #pragma unroll
     for (int k = 0; k < NP; ++k) {
-        if (p.scalar_mask & (1u << k)) {
+        if (k < Fn::NIN && (scalar_mask & (1u << k))) {
             const T s = static_cast<T>(p.scalar[k]);
 #pragma unroll
             for (int j = 0; j < V; ++j) x[k][j] = s;
         } else {
-            const T *base = static_cast<const T *>(p.in[k]) + static_cast<int64_t>(row) * p.istr[k][0];
-            if (p.istr[k][1] == 0) {
+            const T *base = bases[k];
+            if (broadcast[k]) {
                 const T s = *base;
 #pragma unroll
                 for (int j = 0; j < V; ++j) x[k][j] = s;
@@ -185,7 +229,7 @@ __global__ __launch_bounds__(kBlock) void ew_rows(const EwParams p, const Index 
             }
         }
     }
-    apply_affine<T, Fn::NIN, NAUX, V>(p, x);
+    apply_affine<T, Fn::NIN, NAUX, V>(affine, x);
     T o[Fn::NOUT][V];
 #pragma unroll
     for (int j = 0; j < V; ++j) {
@@ -235,11 +279,12 @@ __global__ __launch_bounds__(kBlock) void ew_nd(const EwParams p) {
 #pragma unroll
         for (int k = 0; k < Fn::NOUT; ++k) ooff[k] += c * p.ostr[k][d];
     }
+    const AffineRegs<T, Fn::NIN> affine(p);
     T x1[NP][1], xi[Fn::NIN], oi[Fn::NOUT];
 #pragma unroll
     for (int k = 0; k < NP; ++k)
-        x1[k][0] = (p.scalar_mask & (1u << k)) ? static_cast<T>(p.scalar[k]) : static_cast<const T *>(p.in[k])[ioff[k]];
-    apply_affine<T, Fn::NIN, NAUX, 1>(p, x1);
+        x1[k][0] = (k < Fn::NIN && (p.scalar_mask & (1u << k))) ? static_cast<T>(p.scalar[k]) : static_cast<const T *>(p.in[k])[ioff[k]];
+    apply_affine<T, Fn::NIN, NAUX, 1>(affine, x1);
 #pragma unroll
     for (int k = 0; k < Fn::NIN; ++k) xi[k] = x1[k][0];
     Fn::apply(xi, oi);
@@ -322,18 +367,26 @@ static int launch_ew(const char *fname, const Merged &m, int n_out, const agmi_a
     } else if (m.ndim == 2 && inner_unit) {
         const int64_t tpr = ceil_div(m.shape[1], V);
         const int64_t total = tpr * m.shape[0];
-        const int64_t blocks = ceil_div(total, kBlock);
+        int64_t blocks = ceil_div(total, kBlock);
+        // whole blocks per row, a power of two of them, and little idle tail: block index -> row by shifts
+        const int64_t tiles = ceil_div(tpr, kBlock);
+        int tile_shift = -1;
+        if ((tiles & (tiles - 1)) == 0 && (tpr % kBlock == 0 || tiles >= 4) && tiles * m.shape[0] < 0x7fffffffLL) {
+            tile_shift = 0;
+            while ((int64_t(1) << tile_shift) < tiles) ++tile_shift;
+            blocks = tiles * m.shape[0];
+        }
         if (int rc = check_blocks(blocks)) return rc;
         set_kernel_name("ew_rows<%s>", fname);
         if (total < 0x7fffffffLL)
             with_naux([&](auto na) {
                 hipLaunchKernelGGL((ew_rows<F, T, unsigned, decltype(na)::value>), dim3((unsigned)blocks), dim3(kBlock), 0,
-                                   s, p, (unsigned)tpr, (unsigned)total);
+                                   s, p, (unsigned)tpr, (unsigned)total, tile_shift);
             });
         else
             with_naux([&](auto na) {
                 hipLaunchKernelGGL((ew_rows<F, T, int64_t, decltype(na)::value>), dim3((unsigned)blocks), dim3(kBlock), 0,
-                                   s, p, tpr, total);
+                                   s, p, tpr, total, tile_shift);
             });
     } else {
         const int64_t blocks = ceil_div(m.n, kBlock);

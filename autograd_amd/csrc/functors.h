@@ -17,6 +17,19 @@ namespace agmi {
 // math on T in {float, double}
 __device__ __forceinline__ float m_exp(float x) { return expf(x); }
 __device__ __forceinline__ double m_exp(double x) { return exp(x); }
+// exp(d) for d <= 0 (an element minus the logsumexp of its row) to within 1 ulp of expf, without the
+// overflow handling: d*log2(e) is split into an integer n and a remainder whose rounding error is
+// recovered with fused multiply-adds (log2(e) as a float pair), the hardware exp2 sees |r| <= 1/2,
+// and ldexp scales, also into the subnormals.  n is clamped so that d = -inf (and anything whose exp
+// underflows) arrives at exp2(-inf) = 0; a NaN passes through the clamp's other operand into the fma.
+__device__ __forceinline__ float exp_of_nonpositive(float d) {
+    const float kLog2eHi = 1.44269502162933349609375f, kLog2eLo = 1.92596299112661746e-8f;
+    const float n = fmaxf(rintf(d * kLog2eHi), -160.0f);
+    float r = __builtin_fmaf(d, kLog2eHi, -n);
+    r = __builtin_fmaf(d, kLog2eLo, r);
+    return ldexpf(__builtin_amdgcn_exp2f(r), static_cast<int>(n));
+}
+__device__ __forceinline__ double exp_of_nonpositive(double d) { return exp(d); }
 __device__ __forceinline__ float m_log(float x) { return logf(x); }
 __device__ __forceinline__ double m_log(double x) { return log(x); }
 __device__ __forceinline__ float m_log1p(float x) { return log1pf(x); }
@@ -175,7 +188,7 @@ AGMI_FUNCTOR(FPowVjp0, 3, 1, T e = (x[2] != T(0)) ? x[2] - T(1) : T(1);
 // (g, x, ans): g * log(where(x, x, 1)) * ans
 AGMI_FUNCTOR(FPowVjp1, 3, 1, T b = (x[1] != T(0)) ? x[1] : T(1); o[0] = (x[0] * m_log(b)) * x[2];)
 // (g, b, x, ans): g * b * exp(x - ans)
-AGMI_FUNCTOR(FLseVjp, 4, 1, o[0] = (x[0] * x[1]) * m_exp(x[2] - x[3]);)
+AGMI_FUNCTOR(FLseVjp, 4, 1, o[0] = (x[0] * x[1]) * exp_of_nonpositive(x[2] - x[3]);)
 // (g, x): -g / x**2
 AGMI_FUNCTOR(FReciprocalVjp, 2, 1, o[0] = (-x[0]) / (x[1] * x[1]);)
 // (g, x): g * 0.5 * x**-0.5

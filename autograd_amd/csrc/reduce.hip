@@ -105,7 +105,7 @@ __device__ __forceinline__ void load_points(const RedParams &p, int64_t o, int64
 #pragma unroll
     for (int k = 0; k < F<T>::NIN + AGMI_MAX_AUX; ++k) {
         if (k >= F<T>::NIN + p.n_aux) {  // wave-uniform: no auxiliary operand in this slot
-        } else if (p.scalar_mask & (1u << k)) {
+        } else if (k < F<T>::NIN && (p.scalar_mask & (1u << k))) {
             const T s = static_cast<T>(p.scalar[k]);
 #pragma unroll
             for (int j = 0; j < V; ++j) x[k][j] = s;
