@@ -267,127 +267,95 @@ __device__ __forceinline__ void lse_load(const RedParams &p, int k, int64_t o, i
 // Separate instantiations keep the register count (and so the blocks per CU) of the plain form.
 constexpr int kLseAffine = 1, kLseVecScale = 2, kLseVecShift = 4;
 
-// ROWS = rows per block, reduced side by side (2 when an auxiliary operand that varies along the
-// row is the same for every row: it is loaded once per block instead of once per row, and the two
-// rows share one barrier).
-template <typename T, int V, int ITERS, bool FINAL, int MODE, int ROWS>
+template <typename T, int V, int ITERS, bool FINAL, int MODE>
 __global__ __launch_bounds__(kBlock) void lse_row_block(const RedParams p) {
     using Acc = AccLse<T>;
-    const int64_t o0 = static_cast<int64_t>(blockIdx.x) * ROWS;
+    const int64_t o = blockIdx.x;
     const int chunk = blockIdx.y;
     const int64_t r_begin = static_cast<int64_t>(chunk) * p.r_chunk;
     const int64_t r_end = min(r_begin + p.r_chunk, p.R);
     const int64_t n = r_end - r_begin;
-    T x[ROWS][ITERS][V];
+    T x[ITERS][V];
     // every load is issued before the first use (memory-level parallelism)
 #pragma unroll
-    for (int rr = 0; rr < ROWS; ++rr) {
-        const int64_t o = min(o0 + rr, p.O - 1);  // a row past the end repeats the last one; it is not stored
-#pragma unroll
-        for (int it = 0; it < ITERS; ++it) {
-            const int64_t e0 = (static_cast<int64_t>(it) * kBlock + threadIdx.x) * V;
-            lse_load<T, V>(p, 0, o, r_begin + e0, n - e0, T(-INFINITY), x[rr][it]);
-        }
+    for (int it = 0; it < ITERS; ++it) {
+        const int64_t e0 = (static_cast<int64_t>(it) * kBlock + threadIdx.x) * V;
+        lse_load<T, V>(p, 0, o, r_begin + e0, n - e0, T(-INFINITY), x[it]);
     }
     if (MODE != 0) {
         constexpr bool VEC_A = (MODE & kLseVecScale) != 0, VEC_B = (MODE & kLseVecShift) != 0;
         T a[VEC_A ? ITERS : 1][V], b[VEC_B ? ITERS : 1][V];
         // steps that are absent are the neutral element (x * 1 is exact; x + 0 only loses the sign
         // of a zero, which neither max nor exp can see), so the arithmetic below is branch-free
-        T ua[ROWS], ub[ROWS];  // auxiliary operands that do not vary along the row
-#pragma unroll
-        for (int rr = 0; rr < ROWS; ++rr) {
-            ua[rr] = T(1);
-            ub[rr] = T(0);
-        }
-        // with ROWS > 1 the launcher guarantees that row-varying auxiliary operands have stride 0 across rows
+        T ua = T(1), ub = T(0);  // auxiliary operands that do not vary along the row
         if (VEC_A) {
 #pragma unroll
             for (int it = 0; it < ITERS; ++it) {
                 const int64_t e0 = (static_cast<int64_t>(it) * kBlock + threadIdx.x) * V;
-                lse_load<T, V>(p, p.scale_aux[0], o0, r_begin + e0, n - e0, T(1), a[it]);
+                lse_load<T, V>(p, p.scale_aux[0], o, r_begin + e0, n - e0, T(1), a[it]);
             }
         } else if (p.scale_aux[0] >= 0) {
-#pragma unroll
-            for (int rr = 0; rr < ROWS; ++rr)
-                ua[rr] = static_cast<const T *>(p.in[p.scale_aux[0]])[min(o0 + rr, p.O - 1) * p.istr[p.scale_aux[0]][0]];
+            ua = static_cast<const T *>(p.in[p.scale_aux[0]])[o * p.istr[p.scale_aux[0]][0]];
         }
         if (VEC_B) {
 #pragma unroll
             for (int it = 0; it < ITERS; ++it) {
                 const int64_t e0 = (static_cast<int64_t>(it) * kBlock + threadIdx.x) * V;
-                lse_load<T, V>(p, p.shift_aux[0], o0, r_begin + e0, n - e0, T(0), b[it]);
+                lse_load<T, V>(p, p.shift_aux[0], o, r_begin + e0, n - e0, T(0), b[it]);
             }
         } else if (p.shift_aux[0] >= 0) {
-#pragma unroll
-            for (int rr = 0; rr < ROWS; ++rr)
-                ub[rr] = static_cast<const T *>(p.in[p.shift_aux[0]])[min(o0 + rr, p.O - 1) * p.istr[p.shift_aux[0]][0]];
+            ub = static_cast<const T *>(p.in[p.shift_aux[0]])[o * p.istr[p.shift_aux[0]][0]];
         }
         const T sc = (p.scale_mask & 1u) ? static_cast<T>(p.scale[0]) : T(1);
         const T sh = (p.shift_mask & 1u) ? static_cast<T>(p.shift[0]) : T(0);
         if (n == static_cast<int64_t>(ITERS) * kBlock * V) {  // the chunk fills every lane: no padding to protect
 #pragma unroll
-            for (int rr = 0; rr < ROWS; ++rr)
+            for (int it = 0; it < ITERS; ++it)
 #pragma unroll
-                for (int it = 0; it < ITERS; ++it)
-#pragma unroll
-                    for (int j = 0; j < V; ++j) {
-                        T v = x[rr][it][j] * sc;
-                        v = v * (VEC_A ? a[it][j] : ua[rr]);
-                        v = v + sh;
-                        x[rr][it][j] = v + (VEC_B ? b[it][j] : ub[rr]);
-                    }
+                for (int j = 0; j < V; ++j) {
+                    T v = x[it][j] * sc;
+                    v = v * (VEC_A ? a[it][j] : ua);
+                    v = v + sh;
+                    x[it][j] = v + (VEC_B ? b[it][j] : ub);
+                }
         } else {
 #pragma unroll
-            for (int rr = 0; rr < ROWS; ++rr)
+            for (int it = 0; it < ITERS; ++it) {
+                const int64_t n_left = n - (static_cast<int64_t>(it) * kBlock + threadIdx.x) * V;
 #pragma unroll
-                for (int it = 0; it < ITERS; ++it) {
-                    const int64_t n_left = n - (static_cast<int64_t>(it) * kBlock + threadIdx.x) * V;
-#pragma unroll
-                    for (int j = 0; j < V; ++j) {
-                        T v = x[rr][it][j] * sc;
-                        v = v * (VEC_A ? a[it][j] : ua[rr]);
-                        v = v + sh;
-                        v = v + (VEC_B ? b[it][j] : ub[rr]);
-                        x[rr][it][j] = j < n_left ? v : T(-INFINITY);  // padding stays neutral
-                    }
+                for (int j = 0; j < V; ++j) {
+                    T v = x[it][j] * sc;
+                    v = v * (VEC_A ? a[it][j] : ua);
+                    v = v + sh;
+                    v = v + (VEC_B ? b[it][j] : ub);
+                    x[it][j] = j < n_left ? v : T(-INFINITY);  // padding stays neutral
                 }
+            }
         }
     }
-    typename Acc::type acc[ROWS];
+    T m = T(-INFINITY);
 #pragma unroll
-    for (int rr = 0; rr < ROWS; ++rr) {
-        T m = T(-INFINITY);
+    for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+        for (int j = 0; j < V; ++j) m = max_nan(x[it][j], m);
+    T sum = T(0);
+    if (m == T(INFINITY)) {
+        sum = T(1);
+    } else if (m != T(-INFINITY)) {  // also taken for NaN, which then propagates through exp
 #pragma unroll
         for (int it = 0; it < ITERS; ++it)
 #pragma unroll
-            for (int j = 0; j < V; ++j) m = max_nan(x[rr][it][j], m);
-        T s = T(0);
-        if (m == T(INFINITY)) {
-            s = T(1);
-        } else if (m != T(-INFINITY)) {  // also taken for NaN, which then propagates through exp
-#pragma unroll
-            for (int it = 0; it < ITERS; ++it)
-#pragma unroll
-                for (int j = 0; j < V; ++j) s += exp_nonpositive(x[rr][it][j] - m);
-        }
-        acc[rr] = wave_reduce<Acc>({m, s}, 64);
+            for (int j = 0; j < V; ++j) sum += exp_nonpositive(x[it][j] - m);
     }
-    __shared__ typename Acc::type part[ROWS][kBlock / 64];
-    if ((threadIdx.x & 63) == 0) {
-#pragma unroll
-        for (int rr = 0; rr < ROWS; ++rr) part[rr][threadIdx.x >> 6] = acc[rr];
-    }
+    const typename Acc::type acc = wave_reduce<Acc>({m, sum}, 64);
+    __shared__ typename Acc::type part[kBlock / 64];
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
     __syncthreads();
     if (threadIdx.x == 0) {
+        typename Acc::type t = acc;
 #pragma unroll
-        for (int rr = 0; rr < ROWS; ++rr) {
-            if (o0 + rr >= p.O) break;
-            typename Acc::type t = acc[rr];
-#pragma unroll
-            for (int w = 1; w < kBlock / 64; ++w) t = Acc::combine(t, part[rr][w]);
-            store_result<Acc, T, FINAL>(p, t, o0 + rr, 0, chunk);
-        }
+        for (int w = 1; w < kBlock / 64; ++w) t = Acc::combine(t, part[w]);
+        store_result<Acc, T, FINAL>(p, t, o, 0, chunk);
     }
 }
 
@@ -631,29 +599,17 @@ static int launch_reduce(const char *fname, const RedParams &base, bool vec_ok, 
                 if (((p.scale_mask | p.shift_mask) & 1u) || p.n_aux > 0) mode = kLseAffine;
                 if (p.scale_aux[0] >= 0 && p.istr[p.scale_aux[0]][1] != 0) mode |= kLseVecScale;
                 if (p.shift_aux[0] >= 0 && p.istr[p.shift_aux[0]][1] != 0) mode |= kLseVecShift;
-                // two rows per block when a row-varying auxiliary operand is shared by all rows
-                bool pair_rows = (mode & (kLseVecScale | kLseVecShift)) != 0 && p.O >= 2;
-                if ((mode & kLseVecScale) && p.istr[p.scale_aux[0]][0] != 0) pair_rows = false;
-                if ((mode & kLseVecShift) && p.istr[p.shift_aux[0]][0] != 0) pair_rows = false;
-                const dim3 grid2((unsigned)ceil_div(p.O, 2), (unsigned)pl.n_chunks);
-#define AGMI_LSE_ONE(VV, IT, FIN, MD)                                                                                \
-    do {                                                                                                             \
-        if (pair_rows && IT <= 4)                                                                                    \
-            hipLaunchKernelGGL((lse_row_block<T, VV, (IT <= 4 ? IT : 4), FIN, MD, 2>), grid2, dim3(kBlock), 0, s, p); \
-        else                                                                                                         \
-            hipLaunchKernelGGL((lse_row_block<T, VV, IT, FIN, MD, 1>), grid, dim3(kBlock), 0, s, p);                 \
-    } while (0)
-#define AGMI_LSE_MODE(VV, IT, FIN)                                                                                   \
-    do {                                                                                                             \
-        switch (mode) {                                                                                              \
-            case 0: hipLaunchKernelGGL((lse_row_block<T, VV, IT, FIN, 0, 1>), grid, dim3(kBlock), 0, s, p); break;   \
-            case kLseAffine:                                                                                         \
-                hipLaunchKernelGGL((lse_row_block<T, VV, IT, FIN, kLseAffine, 1>), grid, dim3(kBlock), 0, s, p);     \
-                break;                                                                                               \
-            case kLseAffine | kLseVecScale: AGMI_LSE_ONE(VV, IT, FIN, kLseAffine | kLseVecScale); break;             \
-            case kLseAffine | kLseVecShift: AGMI_LSE_ONE(VV, IT, FIN, kLseAffine | kLseVecShift); break;             \
-            default: AGMI_LSE_ONE(VV, IT, FIN, kLseAffine | kLseVecScale | kLseVecShift);                            \
-        }                                                                                                            \
+#define AGMI_LSE_ONE(VV, IT, FIN, MD) \
+    hipLaunchKernelGGL((lse_row_block<T, VV, IT, FIN, MD>), grid, dim3(kBlock), 0, s, p)
+#define AGMI_LSE_MODE(VV, IT, FIN)                                                                        \
+    do {                                                                                                  \
+        switch (mode) {                                                                                   \
+            case 0: AGMI_LSE_ONE(VV, IT, FIN, 0); break;                                                  \
+            case kLseAffine: AGMI_LSE_ONE(VV, IT, FIN, kLseAffine); break;                                \
+            case kLseAffine | kLseVecScale: AGMI_LSE_ONE(VV, IT, FIN, kLseAffine | kLseVecScale); break;  \
+            case kLseAffine | kLseVecShift: AGMI_LSE_ONE(VV, IT, FIN, kLseAffine | kLseVecShift); break;  \
+            default: AGMI_LSE_ONE(VV, IT, FIN, kLseAffine | kLseVecScale | kLseVecShift);                 \
+        }                                                                                                 \
     } while (0)
 #define AGMI_LSE(VV, IT)                     \
     do {                                     \

@@ -342,6 +342,28 @@ def extras(be):
     from autograd_amd.misc.optimizers import adam
     from autograd_amd.numpy import devarray as D
 
+    # what this part streams on cold data: (8192,4096) f32 buffers in rotation (1 GiB of sources, far more than the
+    # 256 MB last-level cache holds), a plain copy (read + write), a row sum (read only) and a fill (write only)
+    from autograd_amd._lib import Op
+
+    src = [D.zeros((8192, 4096), onp.float32) for _ in range(8)]
+    dst = [D.empty((8192, 4096), onp.float32) for _ in range(8)]
+    nbytes = 8192 * 4096 * 4
+    turn = [0]
+
+    def rotate(fn):
+        def step():
+            turn[0] += 1
+            fn(turn[0] % 8)
+        return step
+
+    sec = time_steps(rotate(lambda i: D.map_op(Op.COPY, src[0].dtype, src[i], out=dst[i])), be.sync, 40, 8)
+    ceil_copy = 2 * nbytes / sec / 1e9
+    sec = time_steps(rotate(lambda i: be.np.sum(src[i], axis=1)), be.sync, 40, 8)
+    ceil_read = nbytes / sec / 1e9
+    sec = time_steps(rotate(lambda i: _lib.fill(_lib.DTYPE_CODE[dst[0].dtype], dst[i]._t, 1.0)), be.sync, 40, 8)
+    out["stream_ceiling_GBps"] = {"copy": ceil_copy, "read": ceil_read, "write": nbytes / sec / 1e9}
+    del src, dst
     n = 1 << 24
     xs = [D.zeros((n,), onp.float64) for _ in range(5)]
     hyper = (0.1, 0.9, 0.001, 0.999, 0.5, 0.5, 0.001, 1e-8)
