@@ -69,7 +69,9 @@ class Op:
         EXPM1_VJP,
         DIV_VJP_BOTH,
         MUL_ADD,
-    ) = range(96, 114)
+        EQUAL_AS_FLOAT,
+        EXTREMUM_VJP,
+    ) = range(96, 116)
 
 
 class Cmp:
@@ -83,7 +85,7 @@ class Red:
 # ops agmi_map_reduce can fuse in front of a sum (reduce.hip: AGMI_FOR_EACH_REDUCE_OP)
 REDUCE_FUSABLE = frozenset(
     {Op.COPY, Op.NEG, Op.MUL, Op.DIV, Op.SQUARE, Op.ABS, Op.DIV_VJP1, Op.TANH_VJP, Op.POW_VJP0, Op.POW_VJP1,
-     Op.LSE_VJP, Op.CHOOSE_VJP}
+     Op.LSE_VJP, Op.CHOOSE_VJP, Op.EQUAL_AS_FLOAT}
 )
 
 

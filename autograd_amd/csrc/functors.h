@@ -209,6 +209,10 @@ AGMI_FUNCTOR(FExpm1Vjp, 2, 1, o[0] = (x[1] + T(1)) * x[0];)
 AGMI_FUNCTOR(FDivVjpBoth, 3, 2, o[0] = x[0] / x[2]; o[1] = ((-x[0]) * x[1]) / (x[2] * x[2]);)
 // (a, x, y): a * x + y, two roundings
 AGMI_FUNCTOR(FMulAdd, 3, 1, T t = x[0] * x[1]; o[0] = t + x[2];)
+// (x, y): astype(x == y, dtype)
+AGMI_FUNCTOR(FEqualAsFloat, 2, 1, o[0] = (x[0] == x[1]) ? T(1) : T(0);)
+// (g, x, ans, n): g * astype(x == ans, dtype) / n
+AGMI_FUNCTOR(FExtremumVjp, 4, 1, o[0] = (x[0] * ((x[1] == x[2]) ? T(1) : T(0))) / x[3];)
 
 // X(op enum, functor)
 #define AGMI_FOR_EACH_OP(X)                     \
@@ -272,6 +276,8 @@ AGMI_FUNCTOR(FMulAdd, 3, 1, T t = x[0] * x[1]; o[0] = t + x[2];)
     X(AGMI_OP_LOG1P_VJP, FLog1pVjp)             \
     X(AGMI_OP_EXPM1_VJP, FExpm1Vjp)             \
     X(AGMI_OP_DIV_VJP_BOTH, FDivVjpBoth)        \
-    X(AGMI_OP_MUL_ADD, FMulAdd)
+    X(AGMI_OP_MUL_ADD, FMulAdd)                 \
+    X(AGMI_OP_EQUAL_AS_FLOAT, FEqualAsFloat)    \
+    X(AGMI_OP_EXTREMUM_VJP, FExtremumVjp)
 
 }  // namespace agmi

@@ -846,7 +846,8 @@ using namespace agmi;
     X(AGMI_OP_POW_VJP0, FPowVjp0)  \
     X(AGMI_OP_POW_VJP1, FPowVjp1)  \
     X(AGMI_OP_LSE_VJP, FLseVjp)    \
-    X(AGMI_OP_CHOOSE_VJP, FChooseVjp)
+    X(AGMI_OP_CHOOSE_VJP, FChooseVjp) \
+    X(AGMI_OP_EQUAL_AS_FLOAT, FEqualAsFloat)
 
 extern "C" int agmi_map_reduce(int op, int red, int dtype, int ndim, const int64_t *shape,
                                const uint8_t *reduce_axes, const agmi_array *out, int n_in,

@@ -396,13 +396,24 @@ defvjp(anp.prod, _grad_prod)
 
 def _grad_chooser(ans, x, axis=None, keepdims=None, **kwargs):
     """max/min: the cotangent is shared equally by the positions that attain the extremum
-    (numpy_vjps.py:515-530)."""
+    (numpy_vjps.py:515-530).  The reference multiplies by the boolean hit mask and divides by its
+    integer sum, so the result is float64 whatever the operand's precision; the mask is taken as
+    float64 here (0 and 1 are exact), which promotes the same way."""
     shape, dtype = anp.shape(x), anp.result_type(x)
 
     def vjp(g):
+        if (_concrete(g, ans, x) and isinstance(x, DevArray) and isinstance(g, DevArray) and isinstance(ans, DevArray)
+                and x.dtype == _F64 and g.dtype == _F64 and ans.dtype == _F64 and x.size and shape):
+            # the same arithmetic in two launches: the number of hits per group (a comparison fused
+            # into a sum), then (g * hit) / hits with g, ans and the count read through broadcast strides
+            axes = D.normalize_axes(axis, len(shape))
+            kept = D.reduce_shape(shape, axes, True)
+            g_kept, ans_kept = (a._view(lambda t: t.reshape(kept)) for a in (g, ans))
+            n_hits = D.map_reduce(Op.EQUAL_AS_FLOAT, Red.SUM, _F64, (x, ans_kept), axes, True, shape=shape)
+            return D.map_op(Op.EXTREMUM_VJP, _F64, g_kept, x, ans_kept, n_hits)
         g_repeated, _ = repeat_to_match_shape(g, shape, dtype, axis, keepdims)
         ans_repeated, _ = repeat_to_match_shape(ans, shape, dtype, axis, keepdims)
-        hits = anp.astype(x == ans_repeated, dtype)
+        hits = anp.astype(x == ans_repeated, _F64)
         return g_repeated * hits / anp.sum(hits, axis=axis, keepdims=True)
 
     return vjp

@@ -129,13 +129,13 @@ def make_workload(name, be):
     if name == "convnet":
         from autograd_amd.scipy.signal import convolve
 
-        inp = configs.convnet_inputs(dtype="float32")
+        inp = configs.convnet_inputs()  # float64, as the example's npr.randn weights and /255.0 images are
         params = configs.tree_map(be.put, inp["params"])
         X, T = be.put(inp["X"]), be.put(inp["T"])
         g = configs.convnet_program(be, convolve)["grad"]
         cfg = {"workload": "examples/convnet.py LeNet stack (conv5x5x6, pool, conv5x5x16, pool, 120, 84, 10) on 28x28, "
                            "grad wrt params dict", "batch": 256, "seed": 0}
-        return g, (params, X, T), cfg, "f32"
+        return g, (params, X, T), cfg, "f64"
     inp = configs.rosen_inputs()
     x, v = be.put(inp["x"]), be.put(inp["v"])
     prog = configs.rosen_program(be)

@@ -142,7 +142,10 @@ typedef enum agmi_op {
     AGMI_OP_LOG1P_VJP,     /* (g, x)         g / (x + 1)              numpy_vjps.py:169           */
     AGMI_OP_EXPM1_VJP,     /* (g, ans)       (ans + 1) * g            numpy_vjps.py:165           */
     AGMI_OP_DIV_VJP_BOTH,  /* (g, x, y) -> two outputs: g / y and -g * x / y**2  (91-92)          */
-    AGMI_OP_MUL_ADD        /* (a, x, y)      a * x + y  (two roundings; scalar_mul + add)         */
+    AGMI_OP_MUL_ADD,       /* (a, x, y)      a * x + y  (two roundings; scalar_mul + add)         */
+    AGMI_OP_EQUAL_AS_FLOAT,/* (x, y)         1.0 where x == y else 0.0: astype(x == ans, dtype)   numpy_vjps.py:524 */
+    AGMI_OP_EXTREMUM_VJP   /* (g, x, ans, n) g * (x == ans) / n, n = number of positions that attain the
+                              extremum of their group (max / min over axes)  numpy_vjps.py:515-530 */
 } agmi_op;
 
 /* comparison producing AGMI_BOOL: numpy.equal ... (non-differentiable, numpy_vjps.py:13-68) */

@@ -93,6 +93,20 @@ def next_cases(be, ext):
     other = P(onp.array([1.0, 1.0, 3.0, 2.0, onp.nan]))
     out["ufunc/fmax_ties_nan"] = grad(lambda a, b: np.sum(np.fmax(a, b) * P(onp.arange(1.0, 6.0))), (0, 1))(tie, other)
 
+    # ---- max / min over axes with ties (numpy_vjps.py:515-530; float64 results whatever the operand) ------
+    tied = rs.randint(-2, 3, (4, 3, 5)).astype(onp.float64)
+    tied[0] += rs.randn(3, 5)
+    for dtype in (onp.float64, onp.float32):
+        tag = "f32" if dtype == onp.float32 else "f64"
+        Z = P(tied.astype(dtype))
+        for fname in ("max", "min"):
+            f = getattr(np, fname)
+            for axis, keepdims in ((None, False), (0, False), (1, True), (2, False), ((0, 2), True)):
+                value = f(Z, axis=axis, keepdims=keepdims)
+                wts = P(onp.asarray(rs.randn(*onp.shape(be.get(value)))).astype(dtype))
+                out[f"extremum/{fname}_{tag}_{axis}_{keepdims}/grad"] = grad(
+                    lambda z: np.sum(f(z, axis=axis, keepdims=keepdims) * wts))(Z)  # noqa: B023
+
     # ---- einsum (numpy_vjps.py:815-848): contraction, batch, summed-out, three operands, ellipsis ------
     for dtype in (onp.float64, onp.float32):
         tag = "f32" if dtype == onp.float32 else "f64"

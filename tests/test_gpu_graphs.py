@@ -25,6 +25,10 @@ def _programs(name, be):
         return configs.mlp_program(be)["grad"], ("params", "X", "T")
     if name == "rnn":
         return configs.rnn_program(be)["grad"], ("params", "inputs", "targets")
+    if name == "convnet":
+        from autograd_amd.scipy.signal import convolve
+
+        return configs.convnet_program(be, convolve)["grad"], ("params", "X", "T")
     prog = configs.rosen_program(be)
     return (lambda x, v: (prog["grad"](x), prog["hvp_rev"](x, v), prog["hvp_fwd"](x, v))), ("x", "v")
 
@@ -39,14 +43,14 @@ def _perturb(tree, rng):
     return configs.tree_map(leaf, tree)
 
 
-@pytest.mark.parametrize("name", ["tanh", "bcast", "mlp", "rnn", "rosen"])
+@pytest.mark.parametrize("name", ["tanh", "bcast", "mlp", "rnn", "rosen", "convnet"])
 def test_replay_equals_eager_on_every_workload(name):
     import autograd_amd as ag
     import autograd_amd.numpy as dnp
 
     be = configs.device_backend()
     fun, keys = _programs(name, be)
-    host = configs.CONFIG_INPUTS[name](**SMALL[name])
+    host = configs.convnet_inputs(batch=5) if name == "convnet" else configs.CONFIG_INPUTS[name](**SMALL[name])
     args = [configs.tree_map(be.put, host[k]) for k in keys]
     graphed = ag.capture(fun, *args)
     rng = onp.random.default_rng(5)

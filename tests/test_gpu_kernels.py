@@ -639,3 +639,29 @@ def test_pending_maps_with_broadcast_operands_are_bit_exact(dnp, dtype):
     wb = rs.uniform(0.5, 1.5, 5000).astype(dtype)
     close(logsumexp(P(dnp, wide) * P(dnp, wb) + 0.25, axis=1).numpy(),
           scipy.special.logsumexp(wide * wb + dtype(0.25), axis=1), RT[dtype])
+
+
+@pytest.mark.parametrize("dtype", [F32, F64])
+def test_max_min_reduction_rules_share_the_cotangent_between_ties(dnp, dtype):
+    """numpy_vjps.py:515-530: g * (x == ans) / count, here one fused count and one fused product;
+    the arithmetic is the reference's, so the result is compared bit for bit with the oracle."""
+    import autograd_amd as ag
+    import oracle.anp as anp
+
+    rs = onp.random.RandomState(21)
+    x = rs.randint(-3, 4, (6, 5, 8)).astype(dtype)  # many ties
+    x[0] += rs.randn(5, 8).astype(dtype)            # and a slab without
+    X = P(dnp, x)
+    for fname in ("max", "min"):
+        for axis in (None, 0, 1, 2, (0, 2), (1, 2)):
+            for keepdims in (False, True):
+                w = onp.asarray(rs.randn(*onp.shape(getattr(onp, fname)(x, axis=axis, keepdims=keepdims)))).astype(dtype)
+                got = ag.grad(lambda z: dnp.sum(getattr(dnp, fname)(z, axis=axis, keepdims=keepdims) * P(dnp, w)))(X)
+                want = ag.grad(lambda z: anp.sum(getattr(anp, fname)(z, axis=axis, keepdims=keepdims) * w))(x)
+                assert got.dtype == want.dtype and onp.array_equal(got.numpy(), want), (fname, axis, keepdims)
+    # second order goes through the traced form of the rule
+    v = P(dnp, rs.randn(7).astype(dtype))
+    h = ag.grad(lambda z: dnp.sum(ag.grad(lambda t: dnp.max(t * t) * dnp.sum(t))(z)))(v)
+    vo = v.numpy()
+    ho = ag.grad(lambda z: anp.sum(ag.grad(lambda t: anp.max(t * t) * anp.sum(t))(z)))(vo)
+    close(h.numpy(), ho, RT[dtype])
