@@ -6,6 +6,8 @@ applied to the tangent, i.e. the same kernels); non-linear ufuncs reuse the fuse
 single-kernel forms of the reverse rules when their operands are concrete.
 """
 
+import numpy as onp
+
 from .._lib import Op
 from ..extend import JVPNode, def_linear, defjvp, defjvp_argnum, register_notrace, vspace
 from ..tracer import isbox
@@ -14,6 +16,7 @@ from . import devarray as D
 from . import wrapper as anp
 from .boxes import DevArrayBox
 from .vjps import (
+    _float64_zeros,
     balanced_eq,
     dot_adjoint_0,
     dot_adjoint_1,
@@ -128,15 +131,16 @@ defjvp(anp.arctan, lambda g, ans, x: g / (1 + x**2))
 defjvp(anp.arcsinh, lambda g, ans, x: g / anp.sqrt(x**2 + 1))
 defjvp(anp.arccosh, lambda g, ans, x: g / anp.sqrt(x**2 - 1))
 defjvp(anp.arctanh, lambda g, ans, x: g / (1 - x**2))
-defjvp(anp.rad2deg, lambda g, ans, x: g / anp.pi * 180.0)
-defjvp(anp.deg2rad, lambda g, ans, x: g * anp.pi / 180.0)
+defjvp(anp.rad2deg, "same")  # numpy_jvps.py:78-81: the function itself applied to the tangent
+defjvp(anp.deg2rad, "same")
 defjvp(anp.clip, lambda g, ans, x, a_min, a_max: g * anp.logical_and(ans != a_min, ans != a_max))
 
 defjvp(
     anp._where3,
     None,
-    lambda g, ans, c, x, y: anp.where(c, g, anp.zeros_like(g)),
-    lambda g, ans, c, x, y: anp.where(c, anp.zeros_like(g), g),
+    # numpy_jvps.py:150-151: float64 zeros, so a float32 tangent comes out float64
+    lambda g, ans, c, x, y: anp.where(c, g, _float64_zeros(anp.shape(g))),
+    lambda g, ans, c, x, y: anp.where(c, _float64_zeros(anp.shape(g)), g),
 )
 defjvp(anp.astype, lambda g, ans, A, dtype, *a, **k: anp.astype(g, dtype))
 defjvp(
@@ -183,7 +187,8 @@ def _fwd_chooser(g, ans, x, axis=None, keepdims=False, **kwargs):
                 ans = anp.expand_dims(ans, ax)
         elif axis is None:
             ans = anp.reshape(ans, (1,) * anp.ndim(x))
-    chosen = anp.astype(x == ans, anp.result_type(x))
+    # the reference multiplies by the boolean mask and divides by its integer sum: float64 results
+    chosen = anp.astype(x == ans, onp.float64)
     return anp.sum(g * chosen, axis=axis, keepdims=keepdims) / anp.sum(chosen, axis=axis, keepdims=keepdims)
 
 

@@ -257,11 +257,19 @@ defvjp(anp.rad2deg, lambda ans, x: lambda g: g / anp.pi * 180.0)
 defvjp(anp.deg2rad, lambda ans, x: lambda g: g * anp.pi / 180.0)
 defvjp(anp.clip, lambda ans, x, a_min, a_max: lambda g: g * anp.logical_and(ans != a_min, ans != a_max))
 
+def _float64_zeros(shape):
+    """``numpy.zeros(shape)`` without the fill: a stride-0 view of the shared float64 zero."""
+    from .vspaces import _shared_zero
+
+    return DevArray(_shared_zero(_F64)._t.expand(tuple(shape)), _F64) if all(shape) else D.zeros(shape, _F64)
+
+
 defvjp(
     anp._where3,
     None,
-    lambda ans, c, x, y: lambda g: anp.where(c, g, anp.zeros_like(g)),
-    lambda ans, c, x, y: lambda g: anp.where(c, anp.zeros_like(g), g),
+    # numpy_vjps.py:228-229: the zeros are float64 (anp.zeros(g.shape)), so a float32 cotangent comes out float64
+    lambda ans, c, x, y: lambda g: anp.where(c, g, _float64_zeros(anp.shape(g))),
+    lambda ans, c, x, y: lambda g: anp.where(c, _float64_zeros(anp.shape(g)), g),
 )
 defvjp(
     anp.astype,

@@ -110,10 +110,8 @@ _unary = {
 for _name, _rule in _unary.items():
     defjvp(getattr(anp, _name), _rule)
 
-defjvp(anp.rad2deg, lambda g, ans, x: g / anp.pi * 180.0)  # numpy_jvps.py:129-132
-defjvp(anp.degrees, lambda g, ans, x: g / anp.pi * 180.0)
-defjvp(anp.deg2rad, lambda g, ans, x: g * anp.pi / 180.0)
-defjvp(anp.radians, lambda g, ans, x: g * anp.pi / 180.0)
+for _f in (anp.rad2deg, anp.degrees, anp.deg2rad, anp.radians):  # numpy_jvps.py:78-81: the ufunc itself on the tangent
+    defjvp(_f, "same")
 defjvp(anp.clip, lambda g, ans, x, a_min, a_max: g * anp.logical_and(ans != a_min, ans != a_max))
 defjvp(
     anp._raw_where,

@@ -87,6 +87,10 @@ def next_cases(be, ext):
         # single-argument grads keep the dtype the rule produces (no container accumulation casts it back)
         out[f"ufunc/maximum_{tag}/grad_single"] = grad(lambda z: np.sum(np.maximum(z, 0.5) * W))(U)
         out[f"ufunc/fmin_{tag}/grad_single"] = grad(lambda z: np.sum(np.fmin(z, row) * W))(U)
+    # where: the rule's zeros are float64, so a float32 operand's cotangent is promoted (numpy_vjps.py:226-230)
+    W32 = P(u.astype(onp.float32))
+    out["ufunc/where_f32/grad_single"] = grad(lambda z: np.sum(np.where(z > 0.5, z, 2.0 * z) * z))(W32)
+    out["ufunc/where_f64/grad_single"] = grad(lambda z: np.sum(np.where(z > 0.5, z, 2.0 * z) * z))(P(u))
     second = P(rs.uniform(0.2, 0.8, 5))
     out["ufunc/second_order"] = grad(lambda z: np.sum(grad(lambda t: np.sum(np.arctan(t) * np.log2(t) + np.tan(t)))(z)))(second)
     tie = P(onp.array([1.0, 2.0, 2.0, onp.nan, 3.0]))
@@ -106,6 +110,45 @@ def next_cases(be, ext):
                 wts = P(onp.asarray(rs.randn(*onp.shape(be.get(value)))).astype(dtype))
                 out[f"extremum/{fname}_{tag}_{axis}_{keepdims}/grad"] = grad(
                     lambda z: np.sum(f(z, axis=axis, keepdims=keepdims) * wts))(Z)  # noqa: B023
+
+    # ---- dtype and value of every rule on a float32 operand: reverse, forward and second order ------------
+    # (NumPy-2 promotion inside the reference's rule bodies decides the dtype: bool masks, integer counts,
+    # float64 zeros and Python scalars all behave differently)
+    xs = rs.uniform(0.2, 0.9, (3, 4)).astype(onp.float32)
+    ys = rs.uniform(0.2, 0.9, (3, 4)).astype(onp.float32)
+    ts = rs.randn(3, 4).astype(onp.float32)
+    X32, Y32, T32 = P(xs), P(ys), P(ts)
+    sweep = {}
+    for name in ("exp log tanh sinh cosh sin cos sqrt square abs reciprocal log1p expm1 exp2 log2 log10 tan arcsin "
+                 "arccos arctan arcsinh arctanh fabs negative sign rad2deg deg2rad").split():
+        sweep[name] = lambda a, n=name: np.sum(getattr(np, n)(a))
+    for name in "sum mean prod max min var std".split():
+        for axis in (None, 0, 1):
+            sweep[f"{name}_ax{axis}"] = lambda a, n=name, ax=axis: np.sum(getattr(np, n)(a, axis=ax))
+    sweep["var_ddof1"] = lambda a: np.sum(np.var(a, axis=0, ddof=1))
+    sweep["std_keepdims"] = lambda a: np.sum(np.std(a, axis=1, keepdims=True))
+    for name in "add subtract multiply divide power maximum minimum fmax fmin arctan2 hypot logaddexp".split():
+        sweep[f"{name}_array"] = lambda a, n=name: np.sum(getattr(np, n)(a, Y32))
+        sweep[f"{name}_scalar"] = lambda a, n=name: np.sum(getattr(np, n)(a, 0.5))
+        sweep[f"{name}_second_arg"] = lambda a, n=name: np.sum(getattr(np, n)(Y32, a))
+    sweep["clip"] = lambda a: np.sum(np.clip(a, 0.3, 0.6))
+    sweep["where"] = lambda a: np.sum(np.where(a > 0.5, a, 2.0 * a))
+    sweep["reshape_T"] = lambda a: np.sum(np.reshape(a, (4, 3)).T * 2.0)
+    sweep["getitem"] = lambda a: np.sum(a[1:, ::2] ** 2)
+    sweep["dot"] = lambda a: np.sum(np.dot(a, Y32.T))
+    sweep["int_power"] = lambda a: np.sum(a ** 3)
+    sweep["divide_by_int"] = lambda a: np.sum(a / 3)
+    sweep["mean_times_two"] = lambda a: np.mean(a) * 2
+    sweep["concatenate"] = lambda a: np.sum(np.concatenate([a, a * 2], axis=0))
+    sweep["repeat"] = lambda a: np.sum(np.repeat(a, 2, axis=1))
+    sweep["expand_squeeze"] = lambda a: np.sum(np.squeeze(np.expand_dims(a, 0)))
+    sweep["logsumexp_rows"] = lambda a: np.sum(be.logsumexp(a, axis=1))
+    for name, f in sweep.items():
+        out[f"sweep/{name}/grad"] = grad(f)(X32)
+        if not name.startswith("hypot"):  # the reference defines no forward rule for hypot
+            value, tangent = be.make_jvp(f)(X32)(T32)
+            out[f"sweep/{name}/jvp_value"], out[f"sweep/{name}/jvp_tangent"] = value, tangent
+        out[f"sweep/{name}/second"] = grad(lambda a: np.sum(grad(f)(a) * T32))(X32)  # noqa: B023
 
     # ---- einsum (numpy_vjps.py:815-848): contraction, batch, summed-out, three operands, ellipsis ------
     for dtype in (onp.float64, onp.float32):
