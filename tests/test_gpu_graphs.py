@@ -110,7 +110,7 @@ def test_replay_of_random_programs_equals_eager():
     import autograd_amd as ag
     import autograd_amd.numpy as dnp
     from autograd_amd.scipy.special import logsumexp
-    from tests.test_gpu_random_programs import make_program
+    from cases_random import make_program
 
     for seed in range(300, 340):
         program, inputs = make_program(seed)

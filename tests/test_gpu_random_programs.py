@@ -15,80 +15,7 @@ import pytest
 
 pytestmark = pytest.mark.gpu
 
-UNARY = ["tanh", "sin", "cos", "exp_small", "square", "negative", "sqrt_abs", "log1p_sq", "abs_shift"]
-
-
-def _apply_unary(np, name, x):
-    if name == "exp_small":
-        return np.exp(x * 0.25)
-    if name == "sqrt_abs":
-        return np.sqrt(np.abs(x) + 1.0)
-    if name == "log1p_sq":
-        return np.log1p(x * x)
-    if name == "abs_shift":
-        return np.abs(x + 0.37)
-    return getattr(np, name)(x)
-
-
-def make_program(seed):
-    """Returns (program(np, logsumexp, *arrays) -> scalar, list of host input arrays)."""
-    rs = onp.random.RandomState(seed)
-    m, n = int(rs.randint(2, 7)), int(rs.randint(2, 9))
-    inputs = [rs.randn(m, n), rs.uniform(0.5, 1.5, n), rs.randn(m), rs.randn(n, m), rs.randn(m, n)]
-    steps = []
-    for _ in range(int(rs.randint(3, 12))):
-        kind = rs.choice(["bin_full", "bin_row", "bin_col", "bin_scalar", "unary", "view", "dot", "mix"])
-        steps.append((kind, int(rs.randint(0, 1 << 30))))
-    tail = rs.choice(["sum", "lse_rows", "lse_cols", "mean_sq", "rowsum_weighted", "max_rows"])
-
-    def program(np, logsumexp, A, b, c, D, E):
-        x = A  # (m, n) throughout
-        for kind, r in steps:
-            q = onp.random.RandomState(r)
-            op = q.choice(["add", "sub", "mul", "div"])
-            if kind == "bin_full":
-                other = E if q.rand() < 0.5 else np.transpose(D)
-                x = {"add": x + other, "sub": other - x, "mul": x * other, "div": x / (other * other + 1.0)}[op]
-            elif kind == "bin_row":
-                x = {"add": x + b, "sub": b[None, :] - x, "mul": b * x, "div": x / b}[op]
-            elif kind == "bin_col":
-                col = c[:, None]
-                x = {"add": col + x, "sub": x - col, "mul": x * col, "div": x / (col * col + 0.5)}[op]
-            elif kind == "bin_scalar":
-                s = float(q.choice([2.0, 0.5, -1.0, 3.0, 0.1, -0.75]))
-                x = {"add": x + s, "sub": s - x, "mul": s * x, "div": x / s}[op]
-            elif kind == "unary":
-                x = _apply_unary(np, UNARY[q.randint(len(UNARY))], x)
-            elif kind == "view":
-                v = q.randint(4)
-                if v == 0:
-                    x = np.transpose(np.transpose(x) * 1.5)
-                elif v == 1:
-                    x = np.reshape(np.reshape(x, (x.shape[0] * x.shape[1],)) + 0.25, x.shape)
-                elif v == 2:
-                    x = x + np.sum(x[1:, :], axis=0) * 0.1 - x[0:1, :]
-                else:
-                    x = x * np.expand_dims(np.sum(x[:, ::2], axis=1), 1)
-                    x = np.tanh(x * 0.1)
-            elif kind == "dot":
-                x = np.dot(np.dot(x, D), E) * 0.05 if q.rand() < 0.5 else np.dot(x, np.dot(D, x)) * 0.05
-                x = np.tanh(x)
-            else:  # the same value consumed several times in different forms (fan-out accumulation)
-                y = x * b + c[:, None]
-                x = y * 0.5 - np.transpose(np.transpose(y)) * y * 0.01 + np.sum(y, axis=1, keepdims=True) * 0.01
-        if tail == "sum":
-            return np.sum(x)
-        if tail == "lse_rows":
-            return np.sum(logsumexp(x, axis=1))
-        if tail == "lse_cols":
-            return np.sum(logsumexp(x * b + c[:, None], axis=0) * b)
-        if tail == "mean_sq":
-            return np.mean(x * x)
-        if tail == "rowsum_weighted":
-            return np.sum(np.sum(x, axis=1) * c)
-        return np.sum(np.max(x, axis=1))
-
-    return program, inputs
+from cases_random import make_program  # noqa: E402  (tests/golden is on sys.path, see conftest.py)
 
 
 @pytest.mark.parametrize("dtype,rtol", [(onp.float64, 1e-9), (onp.float32, 1e-4)])
@@ -149,3 +76,28 @@ def test_random_programs_hessian_vector_products_match_the_oracle():
             assert onp.all(onp.abs(got - want) <= 1e-8 * onp.abs(want) + 1e-8 * scale), (seed, float(onp.abs(got - want).max()), scale)
         checked += 1
     assert checked >= 30
+
+
+def test_random_programs_match_the_reference_vectors():
+    """The same generator, seeds the reference itself evaluated (tests/golden/reference_random.npz)."""
+    import os
+
+    import autograd_amd as ag
+    import autograd_amd.numpy as dnp
+    from autograd_amd.scipy.special import logsumexp as dlse
+    from cases_random import random_program_cases
+
+    gold = onp.load(os.path.join(os.path.dirname(__file__), "golden", "reference_random.npz"))
+    seeds = sorted({int(k.split("/")[2]) for k in gold.files})
+    for dtype, rtol in ((onp.float64, 1e-9), (onp.float32, 1e-4)):
+        got = random_program_cases(dnp, dlse, ag.grad, dnp.asarray, seeds, dtype)
+        for seed in seeds:
+            keys = [k for k in got if k.split("/")[2] == str(seed)]
+            want = [gold[k] for k in keys]
+            if not all(onp.all(onp.isfinite(w)) for w in want):
+                continue
+            scale = max(float(onp.max(onp.abs(w))) if w.size else 0.0 for w in want)
+            for k, w in zip(keys, want):
+                g = got[k].numpy()
+                assert g.dtype == w.dtype and g.shape == w.shape, k
+                assert onp.all(onp.abs(g.astype(onp.float64) - w) <= rtol * (onp.abs(w) + scale)), k
