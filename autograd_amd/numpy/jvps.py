@@ -17,6 +17,7 @@ from . import wrapper as anp
 from .boxes import DevArrayBox
 from .vjps import (
     _float64_zeros,
+    _strong_scalar,
     balanced_eq,
     dot_adjoint_0,
     dot_adjoint_1,
@@ -78,7 +79,8 @@ defjvp(
 defjvp(
     anp.power,
     lambda g, ans, x, y: _fused_or(Op.POW_VJP0, (g, x, y), lambda: g * y * x ** anp.where(y, y - 1, 1.0)),
-    lambda g, ans, x, y: _fused_or(Op.POW_VJP1, (g, x, ans), lambda: g * anp.log(replace_zero(x, 1.0)) * ans),
+    lambda g, ans, x, y: _fused_or(Op.POW_VJP1, (g, _strong_scalar(x), ans),
+                                   lambda: g * anp.log(replace_zero(x, 1.0)) * ans),
 )
 for _chooser in (anp.maximum, anp.minimum, anp.fmax, anp.fmin):
     defjvp(

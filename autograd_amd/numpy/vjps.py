@@ -103,6 +103,12 @@ def unbroadcast_f(target, f):
     return lambda g: unbroadcast(f(g), target_meta)
 
 
+def _strong_scalar(x):
+    """A scalar base of ``power`` as NumPy sees it inside the exponent's rule: ``anp.log(2.0)`` is a
+    numpy.float64, which (unlike the Python float it came from) promotes a float32 array."""
+    return onp.float64(x) if isinstance(x, (int, float)) and not isinstance(x, bool) else x
+
+
 def _binary_rule(fun, traced0, traced1, fused0, fused1):
     """Register both cotangents of a broadcasting ufunc.
 
@@ -168,7 +174,7 @@ _binary_rule(
     lambda ans, x, y: lambda g: g * y * x ** anp.where(y, y - 1, 1.0),
     lambda ans, x, y: lambda g: g * anp.log(replace_zero(x, 1.0)) * ans,
     lambda g, ans, x, y: (Op.POW_VJP0, (g, x, y)),
-    lambda g, ans, x, y: (Op.POW_VJP1, (g, x, ans)),
+    lambda g, ans, x, y: (Op.POW_VJP1, (g, _strong_scalar(x), ans)),
 )
 for _chooser in (anp.maximum, anp.minimum, anp.fmax, anp.fmin):
     _binary_rule(

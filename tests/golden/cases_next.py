@@ -143,12 +143,80 @@ def next_cases(be, ext):
     sweep["repeat"] = lambda a: np.sum(np.repeat(a, 2, axis=1))
     sweep["expand_squeeze"] = lambda a: np.sum(np.squeeze(np.expand_dims(a, 0)))
     sweep["logsumexp_rows"] = lambda a: np.sum(be.logsumexp(a, axis=1))
+    sweep["power_scalar_base"] = lambda a: np.sum(2.0 ** a)  # log(2.0) is a numpy.float64 inside the rule: float64 out
+    for name in "subtract divide arctan2 hypot logaddexp maximum fmin".split():
+        sweep[f"{name}_scalar_first"] = lambda a, n=name: np.sum(getattr(np, n)(0.5, a))
+        sweep[f"{name}_numpy_scalar"] = lambda a, n=name: np.sum(getattr(np, n)(a, onp.float64(0.5)))
     for name, f in sweep.items():
         out[f"sweep/{name}/grad"] = grad(f)(X32)
         if not name.startswith("hypot"):  # the reference defines no forward rule for hypot
             value, tangent = be.make_jvp(f)(X32)(T32)
             out[f"sweep/{name}/jvp_value"], out[f"sweep/{name}/jvp_tangent"] = value, tangent
         out[f"sweep/{name}/second"] = grad(lambda a: np.sum(grad(f)(a) * T32))(X32)  # noqa: B023
+
+    # ---- the namespace's other forms on (3,4) operands, both precisions: stacking, indexing, contractions of every
+    # rank, methods and operators, multi-axis statistics, mixed operand types; reverse, forward, second order ----
+    hA, hB, hv, hT = rs.uniform(0.2, 0.9, (3, 4)), rs.randn(4, 5), rs.randn(4), rs.randn(2, 3, 4)
+    ramp = onp.arange(16.0).reshape(4, 4)
+    rows = onp.array([2, 0, 2, 1])
+    for dtype in (onp.float64, onp.float32):
+        tag = "f32" if dtype == onp.float32 else "f64"
+        A_, B_, v_, T_ = P(hA.astype(dtype)), P(hB.astype(dtype)), P(hv.astype(dtype)), P(hT.astype(dtype))
+        R_, A64, I_ = P(ramp.astype(dtype)), P(hA), P(onp.arange(12).reshape(3, 4))
+        forms = {
+            "stack": lambda a: np.sum(np.stack([a, a * 2.0, np.sin(a)], axis=1) ** 2),
+            "vstack": lambda a: np.sum(np.vstack([a, a * 3.0]) ** 2),
+            "hstack": lambda a: np.sum(np.hstack([a, a * a]) * 1.5),
+            "array_of_rows": lambda a: np.sum(np.array([a[0], a[1] * 2.0, a[2]]) ** 2),
+            "array_of_scalars": lambda a: np.sum(np.array([a[0, 0], a[1, 1] * 2.0, 3.0]) ** 2),
+            "moveaxis": lambda a: np.sum(np.moveaxis(np.expand_dims(a, 0), 0, 2) * 2.0),
+            "swapaxes": lambda a: np.sum(np.dot(np.swapaxes(a, 0, 1), a)),
+            "ravel": lambda a: np.sum(np.ravel(a)[::2] ** 2),
+            "outer": lambda a: np.sum(np.outer(a[0], v_) * np.outer(a[0], v_)),
+            "matmul_2d": lambda a: np.sum(np.matmul(a, B_) ** 2),
+            "matmul_vec": lambda a: np.sum(np.matmul(a, v_) ** 2),
+            "matmul_vec_left": lambda a: np.sum(np.matmul(v_[:3], a) ** 2),
+            "matmul_batched": lambda a: np.sum(np.matmul(T_, a.T) ** 2),
+            "dot_vec_vec": lambda a: np.dot(a[0], v_) * 2.0,
+            "dot_mat_vec": lambda a: np.sum(np.dot(a, v_)),
+            "dot_nd": lambda a: np.sum(np.dot(T_, a.T) * 0.5),
+            "tensordot_2": lambda a: np.tensordot(a, a, axes=2) * 1.0,
+            "tensordot_axes": lambda a: np.sum(np.tensordot(T_, a, axes=([2], [1])) ** 2),
+            "tensordot_0": lambda a: np.sum(np.tensordot(a[0], v_, axes=0)),
+            "take_rows": lambda a: np.sum(a[rows] * R_),
+            "take_negative_slices": lambda a: np.sum(a[-2:, 1:-1] ** 3),
+            "take_int": lambda a: np.sum(a[1] * a[-1]),
+            "take_newaxis": lambda a: np.sum(a[:, None, :] * a[None, :, :]),
+            "take_ellipsis": lambda a: np.sum(a[..., 1] ** 2),
+            "broadcast_to": lambda a: np.sum(np.broadcast_to(a[:1], (5, 4)) * R_[0]),
+            "atleast_2d": lambda a: np.sum(np.atleast_2d(a[0]) * 2.0),
+            "var_two_axes": lambda a: np.sum(np.var(np.expand_dims(a, 0) * T_[:1], axis=(0, 2))),
+            "mean_two_axes_keepdims": lambda a: np.sum(np.mean(a, axis=(0, 1), keepdims=True) * 3.0),
+            "sum_negative_axis": lambda a: np.sum(np.sum(a, axis=-1) ** 2),
+            "astype_float64": lambda a: np.sum(a.astype(onp.float64) ** 2),
+            "astype_float32": lambda a: np.sum(a.astype(onp.float32) ** 2),
+            "methods": lambda a: ((a.T.sum(axis=1) * a.mean(axis=0)).sum() + a.reshape(2, 6).max() + a.ravel().min()
+                                  + np.dot(a, v_).prod()),
+            "operators": lambda a: np.sum((-a) ** 2 / (a + 2.0) - (1.0 - a) * (2 - a) + 3 / (a * a + 1)),
+            "powers": lambda a: np.sum(2.0 ** a + a ** 2.0 + a ** 0.5 + a ** -1),
+            "where_and_mask": lambda a: np.sum(np.where(a > 0.5, np.exp(a), -a) * (a < 0.8)),
+            "logical": lambda a: np.sum(a * np.logical_and(a > 0.3, a < 0.7) + a * np.logical_or(a > 0.8, a < 0.25) * 2.0),
+            "abs_sign": lambda a: np.sum(np.abs(a - 0.5) * np.sign(a - 0.5)),
+            "std_var_all": lambda a: np.std(a) + np.var(a, ddof=1),
+            "times_float64_array": lambda a: np.sum(a * A64),
+            "times_integer_array": lambda a: np.sum(a * I_),
+            "squeeze_axis": lambda a: np.sum(np.squeeze(a[:, :1], axis=1) * v_[:3]),
+            "repeat_axis0": lambda a: np.sum(np.repeat(a, 3, axis=0) * 0.5),
+            "concatenate_axis1": lambda a: np.sum(np.concatenate((a, a[:, :2]), axis=1) ** 2),
+            "prod_axis": lambda a: np.sum(np.prod(a, axis=1)),
+            "softmax_shift": lambda a: np.sum(np.exp(a - np.max(a, axis=1, keepdims=True))),
+        }
+        tangent_in, weights2 = P((hA * 0.3).astype(dtype)), P(hA[::-1].copy().astype(dtype))
+        for name, f in forms.items():
+            out[f"forms/{name}_{tag}/grad"] = grad(f)(A_)
+            if name not in ("astype_float64", "astype_float32", "var_two_axes"):  # no forward rule / a NameError there
+                out[f"forms/{name}_{tag}/jvp_tangent"] = be.make_jvp(f)(A_)(tangent_in)[1]
+            out[f"forms/{name}_{tag}/second"] = grad(lambda a: np.sum(grad(f)(a) * weights2))(A_)  # noqa: B023
 
     # ---- einsum (numpy_vjps.py:815-848): contraction, batch, summed-out, three operands, ellipsis ------
     for dtype in (onp.float64, onp.float32):
