@@ -67,6 +67,32 @@ def next_cases(be, ext):
     out["jac/matrix_in"] = ext.jacobian(lambda M: np.dot(M, x) ** 2)(A)
     out["hess/quartic"] = ext.hessian(lambda v: np.sum(np.dot(A, v) ** 4) + np.sum(np.sin(v) * v))(x)
 
+    # ---- the other differential operators (differential_operators.py:95-200), through ``ext.ag`` -------------
+    ag = ext.ag
+    for dtype in (onp.float64, onp.float32):
+        tag = "f32" if dtype == onp.float32 else "f64"
+        M, xv, vv = P(rs.randn(3, 4).astype(dtype)), P(rs.randn(4).astype(dtype)), P(rs.randn(4).astype(dtype))
+        tv = P(rs.randn(3).astype(dtype))
+        f = lambda z: np.sum(np.tanh(np.dot(M, z)) ** 2)  # noqa: E731,B023
+        h = lambda z: np.tanh(np.dot(M, z))  # noqa: E731,B023
+        out[f"operators/value_and_grad_{tag}"] = ag.value_and_grad(f)(xv)
+        out[f"operators/grad_and_aux_{tag}"] = ag.grad_and_aux(lambda z: (f(z), np.sin(z)))(xv)  # noqa: B023
+        out[f"operators/elementwise_grad_{tag}"] = ag.elementwise_grad(lambda z: np.sin(z) * z)(xv)
+        out[f"operators/hessian_vector_product_{tag}"] = ag.hessian_vector_product(f)(xv, vv)
+        out[f"operators/hessian_tensor_product_{tag}"] = ag.hessian_tensor_product(
+            lambda Z: np.sum(np.tanh(Z) ** 2 * Z))(M, M * 0.5)
+        out[f"operators/make_hvp_{tag}"] = ag.make_hvp(f)(xv)[0](vv)
+        out[f"operators/vector_jacobian_product_{tag}"] = ag.vector_jacobian_product(h)(xv, tv)
+        out[f"operators/tensor_jacobian_product_{tag}"] = ag.tensor_jacobian_product(lambda Z: np.sin(Z) * xv)(M, M * 2.0)  # noqa: B023
+        out[f"operators/make_jvp_reversemode_{tag}"] = ext.make_jvp_reversemode(h)(xv)(vv)
+        out[f"operators/make_jvp_{tag}"] = ag.make_jvp(h)(xv)(vv)
+        out[f"operators/make_vjp_{tag}"] = ag.make_vjp(h)(xv)[0](tv)
+        out[f"operators/make_ggnvp_{tag}"] = ag.make_ggnvp(h)(xv)(vv)
+        out[f"operators/checkpoint_{tag}"] = grad(lambda z: np.sum(ag.checkpoint(h)(z) * tv))(xv)  # noqa: B023
+        out[f"operators/grad_named_{tag}"] = ag.grad_named(lambda a, b: np.sum(np.dot(a, b) ** 2), "b")(M, xv)
+        out[f"operators/jacobian_matrix_out_{tag}"] = ext.jacobian(lambda z: np.outer(np.sin(z), z))(xv)
+        out[f"operators/grad_argnum_tuple_{tag}"] = grad(lambda a, b: np.sum(np.dot(a, b) ** 2), (1, 0))(M, xv)
+
     # ---- the rest of the elementwise rule table (numpy_vjps.py:104-135, 160-185, 215) ------------------
     u = rs.uniform(0.1, 0.9, (3, 4))          # inside every domain below
     w = rs.uniform(1.1, 3.0, (3, 4))

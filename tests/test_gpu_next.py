@@ -27,7 +27,7 @@ def device_ext():
     from autograd_amd.scipy.signal import convolve
 
     return SimpleNamespace(flatten=dflatten, sgd=opt.sgd, rmsprop=opt.rmsprop, adam=opt.adam, jacobian=ag.jacobian,
-                           hessian=ag.hessian, convolve=convolve)
+                           hessian=ag.hessian, convolve=convolve, ag=ag, make_jvp_reversemode=ag.make_jvp_reversemode)
 
 
 def test_next_cases_match_reference_vectors():

@@ -22,7 +22,7 @@ def oracle_ext():
     from oracle.convolution import convolve
 
     return SimpleNamespace(flatten=M.flatten, sgd=M.sgd, rmsprop=M.rmsprop, adam=M.adam, jacobian=ag.jacobian,
-                           hessian=ag.hessian, convolve=convolve)
+                           hessian=ag.hessian, convolve=convolve, ag=ag, make_jvp_reversemode=ag.make_jvp_reversemode)
 
 
 def test_next_cases_bit_identical():
