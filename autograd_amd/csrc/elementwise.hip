@@ -510,6 +510,37 @@ static int launch_cast_from(int dst_dtype, const MixParams &p, unsigned blocks, 
 
 using namespace agmi;
 
+// This file is compiled twice, once per precision (-DAGMI_PART=32 / 64), so that the two halves of
+// the functor x layout instantiations build in parallel; the entry points live in the float32 half.
+#ifndef AGMI_PART
+#error "compile with -DAGMI_PART=32 or -DAGMI_PART=64"
+#endif
+namespace agmi {
+int elementwise_part_f32(int op, const Merged &m, int n_out, const agmi_array *outs, int n_in, const agmi_array *ins,
+                         const double *scalars, hipStream_t s);
+int elementwise_part_f64(int op, const Merged &m, int n_out, const agmi_array *outs, int n_in, const agmi_array *ins,
+                         const double *scalars, hipStream_t s);
+#if AGMI_PART == 32
+#define AGMI_PART_FN elementwise_part_f32
+using PartT = float;
+#else
+#define AGMI_PART_FN elementwise_part_f64
+using PartT = double;
+#endif
+int AGMI_PART_FN(int op, const Merged &m, int n_out, const agmi_array *outs, int n_in, const agmi_array *ins,
+                 const double *scalars, hipStream_t s) {
+#define AGMI_CASE(OP, FN) \
+    case OP: return launch_ew<FN, PartT>(#FN, m, n_out, outs, n_in, ins, scalars, s);
+    switch (op) {
+        AGMI_FOR_EACH_OP(AGMI_CASE)
+        default: set_error("elementwise: unknown op %d", op); return AGMI_ERR_ARG;
+    }
+#undef AGMI_CASE
+}
+#undef AGMI_PART_FN
+}  // namespace agmi
+
+#if AGMI_PART == 32
 extern "C" int agmi_elementwise(int op, int dtype, int ndim, const int64_t *shape, int n_out,
                                 const agmi_array *outs, int n_in, const agmi_array *ins,
                                 const double *scalars, void *stream) {
@@ -531,16 +562,8 @@ extern "C" int agmi_elementwise(int op, int dtype, int ndim, const int64_t *shap
     if (!merge_axes(ndim, shape, nullptr, n_out + n_in, strides, &m)) return AGMI_ERR_ARG;
     if (m.n == 0) return 0;
     hipStream_t s = as_stream(stream);
-#define AGMI_CASE(OP, FN)                                                                    \
-    case OP:                                                                                 \
-        if (dtype == AGMI_F32) return launch_ew<FN, float>(#FN, m, n_out, outs, n_in, ins, scalars, s);  \
-        if (dtype == AGMI_F64) return launch_ew<FN, double>(#FN, m, n_out, outs, n_in, ins, scalars, s); \
-        break;
-    switch (op) {
-        AGMI_FOR_EACH_OP(AGMI_CASE)
-        default: set_error("elementwise: unknown op %d", op); return AGMI_ERR_ARG;
-    }
-#undef AGMI_CASE
+    if (dtype == AGMI_F32) return elementwise_part_f32(op, m, n_out, outs, n_in, ins, scalars, s);
+    if (dtype == AGMI_F64) return elementwise_part_f64(op, m, n_out, outs, n_in, ins, scalars, s);
     set_error("elementwise: dtype %d is not a floating type", dtype);
     return AGMI_ERR_ARG;
 }
@@ -600,3 +623,4 @@ extern "C" int agmi_cast(int src_dtype, int dst_dtype, int ndim, const int64_t *
         default: set_error("cast: unknown source dtype %d", src_dtype); return AGMI_ERR_ARG;
     }
 }
+#endif  // AGMI_PART == 32

@@ -849,6 +849,37 @@ using namespace agmi;
     X(AGMI_OP_CHOOSE_VJP, FChooseVjp) \
     X(AGMI_OP_EQUAL_AS_FLOAT, FEqualAsFloat)
 
+// This file is compiled twice, once per precision (-DAGMI_PART=32 / 64), so that the two halves of
+// the kernel instantiations build in parallel; the entry points live in the float32 half.
+#ifndef AGMI_PART
+#error "compile with -DAGMI_PART=32 or -DAGMI_PART=64"
+#endif
+namespace agmi {
+int reduce_part_f32(int op, int red, const RedSetup &st, void *ws, size_t ws_bytes, hipStream_t s);
+int reduce_part_f64(int op, int red, const RedSetup &st, void *ws, size_t ws_bytes, hipStream_t s);
+#if AGMI_PART == 32
+#define AGMI_PART_FN reduce_part_f32
+using PartT = float;
+#else
+#define AGMI_PART_FN reduce_part_f64
+using PartT = double;
+#endif
+int AGMI_PART_FN(int op, int red, const RedSetup &st, void *ws, size_t ws_bytes, hipStream_t s) {
+    if (op == AGMI_OP_COPY) return dispatch_red_copy<PartT>(red, st, ws, ws_bytes, s);
+#define AGMI_CASE(OP, FN) \
+    case OP: return dispatch_red<FN, PartT>(#FN, red, st, ws, ws_bytes, s);
+    switch (op) {
+        AGMI_FOR_EACH_REDUCE_OP(AGMI_CASE)
+        default: break;
+    }
+#undef AGMI_CASE
+    set_error("map_reduce: op %d cannot be fused into a reduction", op);
+    return AGMI_ERR_UNSUPPORTED;
+}
+#undef AGMI_PART_FN
+}  // namespace agmi
+
+#if AGMI_PART == 32
 extern "C" int agmi_map_reduce(int op, int red, int dtype, int ndim, const int64_t *shape,
                                const uint8_t *reduce_axes, const agmi_array *out, int n_in,
                                const agmi_array *ins, const double *scalars, void *workspace,
@@ -871,21 +902,8 @@ extern "C" int agmi_map_reduce(int op, int red, int dtype, int ndim, const int64
         set_error("map_reduce: dtype %d is not a floating type", dtype);
         return AGMI_ERR_ARG;
     }
-    if (op == AGMI_OP_COPY) {
-        return dtype == AGMI_F32 ? dispatch_red_copy<float>(red, st, workspace, workspace_bytes, s)
-                                 : dispatch_red_copy<double>(red, st, workspace, workspace_bytes, s);
-    }
-#define AGMI_CASE(OP, FN)                                                                        \
-    case OP:                                                                                     \
-        return dtype == AGMI_F32 ? dispatch_red<FN, float>(#FN, red, st, workspace, workspace_bytes, s) \
-                                 : dispatch_red<FN, double>(#FN, red, st, workspace, workspace_bytes, s);
-    switch (op) {
-        AGMI_FOR_EACH_REDUCE_OP(AGMI_CASE)
-        default: break;
-    }
-#undef AGMI_CASE
-    set_error("map_reduce: op %d cannot be fused into a reduction", op);
-    return AGMI_ERR_UNSUPPORTED;
+    return dtype == AGMI_F32 ? reduce_part_f32(op, red, st, workspace, workspace_bytes, s)
+                             : reduce_part_f64(op, red, st, workspace, workspace_bytes, s);
 }
 
 extern "C" size_t agmi_map_reduce_workspace_bytes(int red, int dtype, int ndim, const int64_t *shape,
@@ -901,3 +919,4 @@ extern "C" size_t agmi_map_reduce_workspace_bytes(int red, int dtype, int ndim, 
     const int64_t chunks = std::min<int64_t>(kTargetBlocks, reduced);
     return static_cast<size_t>(chunks) * static_cast<size_t>(kept) * acc;
 }
+#endif  // AGMI_PART == 32

@@ -631,7 +631,7 @@ def normalize_axes(axis, ndim):
     axes = tuple(sorted({int(a) % ndim if ndim else 0 for a in axis}))
     for a in axis:
         if not -max(ndim, 1) <= int(a) < max(ndim, 1):
-            raise ValueError(f"axis {a} is out of bounds for array of dimension {ndim}")
+            raise onp.exceptions.AxisError(int(a), ndim)  # NumPy's own exception (a ValueError and an IndexError)
     return axes
 
 
