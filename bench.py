@@ -33,7 +33,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing")
     ap.add_argument("--no-extras", action="store_true", help="skip the other workloads")
-    ap.add_argument("--cpu-seconds", type=float, default=20.0, help="budget for the CPU baseline sample")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget for the CPU baseline sample")
     ap.add_argument("--workload", default="bcast", choices=["bcast", "tanh", "mlp", "rnn", "rosen", "convnet"],
                     help="bcast (default) is the headline workload, BASELINE configs[1]; the others are the "
                          "remaining BASELINE configs and the convnet example, selectable for profiling")
@@ -74,7 +74,7 @@ def cpu_baseline(seconds):
     first = time.perf_counter() - t0
     times = []
     deadline = time.perf_counter() + max(0.0, seconds - first)
-    while len(times) < 5 and (not times or time.perf_counter() + min(times) < deadline):
+    while len(times) < 50 and (not times or time.perf_counter() + min(times) < deadline):
         t0 = time.perf_counter()
         g(inp["A"], inp["b"], inp["c"])
         times.append(time.perf_counter() - t0)
