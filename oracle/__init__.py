@@ -10,6 +10,9 @@ What is here
   numpy_boxes.py, numpy_vspaces.py, numpy_wrapper.py, scipy/special.py), so
   that on the same seeded inputs it reproduces what reference autograd+NumPy
   computes on the host.
+* ``misc`` / ``convolution``: container flattening and the optimizers (autograd/misc/flatten.py,
+  optimizers.py) and the N-d convolution with its cotangents (autograd/scipy/signal.py), restated
+  the same way.
 * ``closed_forms``: answers that do not come from any tracer at all (textbook
   derivatives, brute-force sums, dense Hessians) for the five workloads and the
   rule families; they are what pins the restatement where the reference's own
@@ -31,8 +34,11 @@ tests/test_scalar_ops.py:134-143, tests/test_numpy.py:881-890,1032-1038, ...),
 (2) ``closed_forms``, (3) central finite differences (the reference's
 ``check_grads`` construction) over the shape lists of the reference's
 systematic tests, and (4) fixtures under ``tests/golden/`` written by the real
-reference in the build container (whole-workload outputs at reduced sizes and
-result dtypes), against which the restatement is bit-identical.
+reference in the build container (whole-workload outputs at reduced sizes, a
+sweep of every rule and namespace form in reverse mode, forward mode and second
+order with their result dtypes, the differential operators, convolutions in
+every mode, gradients of seeded random programs), against which the restatement
+is bit-identical.  No function here is "parity unpinned".
 
 Python ``float`` is deliberately NOT registered as an oracle value type (the
 device namespace owns it); use ``numpy.float64`` scalars or 0-d arrays.
