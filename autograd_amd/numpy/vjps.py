@@ -335,6 +335,9 @@ def repeat_to_match_shape(g, shape, dtype, axis, keepdims):
     axes = D.normalize_axes(axis, len(shape))
     new_shape = tuple(1 if d in axes else s for d, s in enumerate(shape))
     num_reps = onp.prod(onp.array(shape)[list(axes)])
+    if isinstance(g, DevArray) and (g.dtype == dtype or g.dtype == _F64):
+        # a concrete cotangent that needs no promotion: the view itself, without the two primitive calls
+        return g._view(lambda t: t.reshape(new_shape).expand(shape)), num_reps
     out = anp.broadcast_to(anp.reshape(g, new_shape), shape)
     if anp.result_type(g) != onp.result_type(anp.result_type(g), dtype):
         out = anp.astype(out, onp.result_type(anp.result_type(g), dtype))
