@@ -9,7 +9,7 @@ primitives (and therefore the same kernels).
 
 from ..extend import Box, primitive
 from . import wrapper as anp
-from .devarray import DevArray, LazyDevArray
+from .devarray import DevArray, LazyDevArray, PendingProduct
 
 
 def _route(name, swap=False):
@@ -103,4 +103,5 @@ DevArrayBox.__hash__ = lambda self: id(self)
 
 DevArrayBox.register(DevArray)
 DevArrayBox.register(LazyDevArray)
+DevArrayBox.register(PendingProduct)
 DevArrayBox.register(float)

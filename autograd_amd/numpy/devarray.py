@@ -207,9 +207,74 @@ class LazyDevArray(DevArray):
             return DevArray(fn(self._t), self.dtype)
 
 
+class PendingProduct(DevArray):
+    """The matrix product ``left @ right`` of two 2-d tensors, not yet computed.
+
+    The cotangent rules of ``dot`` return one of these for matrix operands.  A cotangent usually
+    ends up added to an accumulator (the weight matrix of a recurrent net receives one per time
+    step); ``DevArrayVSpace._mut_add`` then runs the contraction with beta = 1 straight into the
+    accumulator (``add_into``) instead of writing a temporary that an add kernel reads back.  The
+    sum is the same to the bit: the kernel's epilogue adds C to the very accumulators it would
+    otherwise have stored.  Anything else that touches the value reads ``_t`` as on any
+    ``DevArray``; the first such read computes the product and keeps it.
+    """
+
+    __slots__ = ("_left", "_right", "_shape")
+
+    def __init__(self, left, right, dtype):
+        self._left, self._right = left, right
+        self._shape = (left.shape[0], right.shape[1])
+        self.dtype = dtype
+        self._borrowed = False
+
+    def __getattr__(self, name):
+        # only reached when a slot is unset: `_t` before the product has been computed
+        if name != "_t":
+            raise AttributeError(name)
+        self._t = out = gemm2d(self._left, self._right, self.dtype)
+        self._left = self._right = None
+        return out
+
+    def computed(self):
+        return self._left is None
+
+    def fresh(self):
+        """The product in a buffer of the caller's own (nothing is kept here)."""
+        return DevArray(gemm2d(self._left, self._right, self.dtype), self.dtype)
+
+    def add_into(self, acc):
+        """``acc += left @ right`` for a contiguous tensor ``acc`` of this shape and dtype."""
+        gemm2d(self._left, self._right, self.dtype, out=acc, beta=1.0)
+
+    @property
+    def shape(self):
+        return self._shape
+
+    @property
+    def ndim(self):
+        return 2
+
+    @property
+    def size(self):
+        return self._shape[0] * self._shape[1]
+
+    @property
+    def strides(self):
+        return (self._shape[1] * self.dtype.itemsize, self.dtype.itemsize)
+
+    def __len__(self):
+        return self._shape[0]
+
+    def __iter__(self):
+        return (self[i] for i in range(self._shape[0]))
+
+    def _settled(self):
+        return DevArray(self._t, self.dtype)
+
+
 def plain(x):
-    """``x`` with any pending map written out (a no-op for everything else)."""
-    return DevArray(x._t, x.dtype) if type(x) is LazyDevArray else x
+    """``x`` with any pending arithmetic written out (a no-op for everything else)."""
+    return DevArray(x._t, x.dtype) if type(x) in (LazyDevArray, PendingProduct) else x
 
 
 def alias(x):
@@ -603,6 +668,7 @@ def astype_copy(x):
 
 
 def contiguous(x):
+    x = plain(x) if type(x) is PendingProduct else x  # a computed product is contiguous already
     return x if type(x) is DevArray and x._t.is_contiguous() else copy(x)
 
 

@@ -507,14 +507,36 @@ def dot_adjoint_1(A, G, A_meta, B_meta):
     return _as_dtype(out, onp.dtype(B_dtype))
 
 
+def _matrix_operands(dtype_wanted, *xs):
+    """The operands as plain tensors when all are concrete 2-d float device arrays of one dtype."""
+    for x in xs:
+        if not isinstance(x, DevArray) or x.ndim != 2 or x.dtype != dtype_wanted or x.dtype not in D._FLOATS:
+            return None
+    return tuple(x._t for x in xs)
+
+
 def _dot_vjp_0(ans, A, B):
     A_meta, B_meta = anp.metadata(A), anp.metadata(B)
-    return lambda g: dot_adjoint_0(B, g, A_meta, B_meta)
+
+    def vjp(g):
+        ts = _matrix_operands(A_meta[2], g, B) if A_meta[1] == 2 and B_meta[1] == 2 and _concrete(g, B) else None
+        if ts is not None:
+            return D.PendingProduct(ts[0], ts[1].t(), A_meta[2])  # added into A's accumulator by the contraction itself
+        return dot_adjoint_0(B, g, A_meta, B_meta)
+
+    return vjp
 
 
 def _dot_vjp_1(ans, A, B):
     A_meta, B_meta = anp.metadata(A), anp.metadata(B)
-    return lambda g: dot_adjoint_1(A, g, A_meta, B_meta)
+
+    def vjp(g):
+        ts = _matrix_operands(B_meta[2], A, g) if A_meta[1] == 2 and B_meta[1] == 2 and _concrete(A, g) else None
+        if ts is not None:
+            return D.PendingProduct(ts[0].t(), ts[1], B_meta[2])
+        return dot_adjoint_1(A, g, A_meta, B_meta)
+
+    return vjp
 
 
 defvjp(anp.dot, _dot_vjp_0, _dot_vjp_1)

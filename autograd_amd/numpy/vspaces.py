@@ -115,6 +115,13 @@ class DevArrayVSpace(VSpace):
         may also be a tape value or another node's cotangent - is never written."""
         if not isinstance(x, DevArray):
             return self._add(x, y)
+        if type(y) is D.PendingProduct and not y.computed() and y.dtype == x.dtype and y.shape == x.shape:
+            # a matrix cotangent whose contraction has not run yet: run it into the accumulator
+            if is_shared_zero(x):
+                return y.fresh()  # 0 + G: a buffer of the accumulator's own, so later contributions add in place
+            if type(x) is DevArray and not x._borrowed and not is_broadcast_view(x) and x._t.is_contiguous():
+                y.add_into(x._t)
+                return x
         if is_shared_zero(x):
             if isinstance(y, DevArray) and y.shape == x.shape and y.dtype == x.dtype:
                 acc = D.alias(y)
@@ -144,4 +151,5 @@ class DevArrayVSpace(VSpace):
 
 DevArrayVSpace.register(DevArray)
 DevArrayVSpace.register(LazyDevArray)
+DevArrayVSpace.register(D.PendingProduct)
 DevArrayVSpace.register(float)

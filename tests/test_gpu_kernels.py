@@ -665,3 +665,30 @@ def test_max_min_reduction_rules_share_the_cotangent_between_ties(dnp, dtype):
     vo = v.numpy()
     ho = ag.grad(lambda z: anp.sum(ag.grad(lambda t: anp.max(t * t) * anp.sum(t))(z)))(vo)
     close(h.numpy(), ho, RT[dtype])
+
+
+@pytest.mark.parametrize("dtype", [F32, F64])
+@pytest.mark.parametrize("rows,inner,cols", [(256, 641, 512), (1024, 784, 1024), (64, 33, 10), (7, 5, 3)])
+def test_matrix_cotangents_accumulate_inside_the_contraction(dnp, dtype, rows, inner, cols):
+    """A weight used by several products: from the second contribution on, the cotangent's contraction
+    runs with beta = 1 into the accumulator.  Bit for bit the same as contracting and adding separately,
+    for both operands, whether the contraction is split over K or not."""
+    import autograd_amd as ag
+
+    rs = onp.random.RandomState(31)
+    X1, X2, X3 = (P(dnp, rs.randn(rows, inner).astype(dtype)) for _ in range(3))
+    C1, C2, C3 = (P(dnp, rs.randn(rows, cols).astype(dtype)) for _ in range(3))
+    W = P(dnp, rs.randn(inner, cols).astype(dtype))
+    f = lambda w: dnp.sum(dnp.dot(X1, w) * C1) + dnp.sum(dnp.dot(X2, w) * C2)  # noqa: E731
+    got = ag.grad(f)(W).numpy()
+    want = (dnp.dot(X1.T, C1) + dnp.dot(X2.T, C2)).numpy()
+    assert onp.array_equal(got, want)
+    # three uses, and the left operand of the product this time
+    V1, V2, V3 = (P(dnp, rs.randn(inner, cols).astype(dtype)) for _ in range(3))
+    h = lambda x: dnp.sum(dnp.dot(x, V1) * C1) + dnp.sum(dnp.dot(x, V2) * C2) + dnp.sum(dnp.dot(x, V3) * C3)  # noqa: E731
+    got = ag.grad(h)(X1).numpy()
+    parts = [dnp.dot(C, V.T).numpy().astype(onp.float64) for C, V in ((C1, V1), (C2, V2), (C3, V3))]
+    ref = parts[0] + parts[1] + parts[2]
+    close(got, ref.astype(dtype), RT[dtype])
+    # against NumPy as well
+    close(ag.grad(f)(W).numpy(), X1.numpy().T @ C1.numpy() + X2.numpy().T @ C2.numpy(), RT[dtype] * 10)
