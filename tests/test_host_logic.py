@@ -192,3 +192,41 @@ def test_broadcast_operands_fold_into_pending_maps():
                  lambda: A / b, lambda: -(A + c), lambda: A * meta((8, 6), torch.float64), lambda: A * meta((6,), torch.float32)):
         with pytest.raises(Exception):
             expr()
+
+
+def test_pending_products_are_contracted_into_an_accumulator_of_its_own(monkeypatch):
+    """The accumulation protocol for matrix cotangents, with the contraction replaced by a recorder:
+    0 + G computes G into a buffer the accumulator owns; an owned accumulator takes the next
+    product with beta = 1; a borrowed accumulator (it shares memory with a cotangent) is never
+    written, the product is computed on its own and added out of place."""
+    from autograd_amd.numpy import vspaces
+
+    calls = []
+
+    def fake_gemm2d(a, b, dtype, out=None, beta=0.0):
+        calls.append(("gemm", out is not None, beta))
+        return out if out is not None else torch.zeros((a.shape[0], b.shape[1]), dtype=torch.float64)
+
+    monkeypatch.setattr(D, "gemm2d", fake_gemm2d)
+    monkeypatch.setitem(vspaces._ZEROS, onp.dtype("float64"), DevArray(torch.zeros((), dtype=torch.float64)))
+    left, right = torch.zeros((3, 5), dtype=torch.float64), torch.zeros((5, 4), dtype=torch.float64)
+    vs = vspaces.DevArrayVSpace(DevArray(torch.zeros((3, 4), dtype=torch.float64)))
+    first = D.PendingProduct(left, right, onp.dtype("float64"))
+    assert first.shape == (3, 4) and first.ndim == 2 and first.size == 12 and not first.computed()
+    acc = vs._mut_add(vs.zeros(), first)
+    assert type(acc) is DevArray and not acc._borrowed and calls == [("gemm", False, 0.0)]
+    assert not first.computed()  # the product went to the accumulator, nothing was cached on the cotangent
+    second = D.PendingProduct(left, right, onp.dtype("float64"))
+    assert vs._mut_add(acc, second) is acc and calls[-1] == ("gemm", True, 1.0) and not second.computed()
+    # a borrowed accumulator must not be written: no beta = 1 call on it
+    borrowed = D.alias(acc)
+    borrowed._borrowed = True
+    third = D.PendingProduct(left, right, onp.dtype("float64"))
+    with pytest.raises(Exception):  # the out-of-place add would launch a kernel: there is no CPU fallback
+        vs._mut_add(borrowed, third)
+    assert ("gemm", True, 1.0) not in calls[2:] and third.computed()
+    # reading the value computes it once and keeps it
+    fourth = D.PendingProduct(left, right, onp.dtype("float64"))
+    n = len(calls)
+    t = fourth._t
+    assert fourth._t is t and len(calls) == n + 1 and fourth.computed() and D.plain(fourth)._t is t
