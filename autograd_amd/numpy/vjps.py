@@ -586,12 +586,26 @@ def _matmul_adjoint_1(A, G, A_ndim, B_meta):
 
 def _matmul_vjp_0(ans, A, B):
     A_meta, B_ndim = anp.metadata(A), anp.ndim(B)
-    return lambda g: _matmul_adjoint_0(B, g, A_meta, B_ndim)
+
+    def vjp(g):
+        ts = _matrix_operands(A_meta[2], g, B) if A_meta[1] == 2 and B_ndim == 2 and _concrete(g, B) else None
+        if ts is not None:  # matrices: the same pending product as for dot
+            return D.PendingProduct(ts[0], ts[1].t(), A_meta[2])
+        return _matmul_adjoint_0(B, g, A_meta, B_ndim)
+
+    return vjp
 
 
 def _matmul_vjp_1(ans, A, B):
     A_ndim, B_meta = anp.ndim(A), anp.metadata(B)
-    return lambda g: _matmul_adjoint_1(A, g, A_ndim, B_meta)
+
+    def vjp(g):
+        ts = _matrix_operands(B_meta[2], A, g) if A_ndim == 2 and B_meta[1] == 2 and _concrete(A, g) else None
+        if ts is not None:
+            return D.PendingProduct(ts[0].t(), ts[1], B_meta[2])
+        return _matmul_adjoint_1(A, g, A_ndim, B_meta)
+
+    return vjp
 
 
 defvjp(anp.matmul, _matmul_vjp_0, _matmul_vjp_1)

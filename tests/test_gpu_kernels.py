@@ -692,3 +692,8 @@ def test_matrix_cotangents_accumulate_inside_the_contraction(dnp, dtype, rows, i
     close(got, ref.astype(dtype), RT[dtype])
     # against NumPy as well
     close(ag.grad(f)(W).numpy(), X1.numpy().T @ C1.numpy() + X2.numpy().T @ C2.numpy(), RT[dtype] * 10)
+    # the @ operator takes the same route
+    fm = lambda w: dnp.sum((X1 @ w) * C1) + dnp.sum(dnp.matmul(X2, w) * C2)  # noqa: E731
+    assert onp.array_equal(ag.grad(fm)(W).numpy(), want)
+    hm = lambda x: dnp.sum((x @ V1) * C1) + dnp.sum((x @ V2) * C2)  # noqa: E731
+    assert onp.array_equal(ag.grad(hm)(X1).numpy(), (dnp.dot(C1, V1.T) + dnp.dot(C2, V2.T)).numpy())
