@@ -621,6 +621,21 @@ def take(A, idx):
     return out
 
 
+def _leading_rows(idx, shape):
+    """(start, stop) when the basic index ``idx`` selects rows start:stop of the leading axis with
+    step 1 and every other axis in full; None otherwise."""
+    if isinstance(idx, slice):
+        first, rest = idx, ()
+    elif isinstance(idx, tuple) and idx and isinstance(idx[0], slice):
+        first, rest = idx[0], idx[1:]
+    else:
+        return None
+    if not shape or any(not (isinstance(r, slice) and r == slice(None)) for r in rest):
+        return None
+    start, stop, step = first.indices(shape[0])
+    return (start, stop if stop > start else start) if step == 1 else None  # (this module's max is the array reduction)
+
+
 def scatter_add(A, idx, x):
     """In place ``numpy.add.at(A, idx, x)`` on a freshly allocated, contiguous ``A``.
 
@@ -646,7 +661,18 @@ def scatter_add(A, idx, x):
                     acc = x._view(lambda t: t.reshape(shape))
                     acc._borrowed = True
                     return acc
-                A = D.empty(A.shape, A.dtype) if full_cover else D.zeros(A.shape, A.dtype)
+                rows = None if full_cover else _leading_rows(idx, A.shape)
+                if full_cover or rows is not None:
+                    A = D.empty(A.shape, A.dtype)
+                    if rows is not None:
+                        # x[1:], x[:-1], x[a:b]: only the rows outside the range need zeros (two short fills),
+                        # not the whole array
+                        code = _lib.DTYPE_CODE[A.dtype]
+                        for part in (A._t[:rows[0]], A._t[rows[1]:]):
+                            if part.numel():
+                                _lib.fill(code, part, 0.0)
+                else:
+                    A = D.zeros(A.shape, A.dtype)
                 D.map_op(Op.ADD, A.dtype, 0.0, x, out=DevArray(A._t[_plain(idx)], A.dtype))
                 return A
             A = D.zeros(A.shape, A.dtype)
