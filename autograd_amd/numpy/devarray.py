@@ -18,7 +18,7 @@ import numpy as onp
 import torch
 
 from .. import _lib
-from .._lib import Cmp, Op, Red
+from .._lib import Op, Red
 
 _FLOATS = (onp.dtype("float32"), onp.dtype("float64"))
 _F64 = onp.dtype("float64")

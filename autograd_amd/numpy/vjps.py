@@ -11,8 +11,6 @@ computes.  Each has two forms:
   it can itself be differentiated to any order.
 """
 
-from functools import partial
-
 import numpy as onp
 
 from .._lib import REDUCE_FUSABLE, Op, Red

@@ -9,13 +9,10 @@ reference materialises both).  Forward mode: the same functor fused into a sum.
 
 import numbers
 
-import numpy as onp
-
 from .._lib import Op, Red
 from ..extend import defjvp, defvjp, primitive
 from ..numpy import devarray as D
 from ..numpy import wrapper as np
-from ..numpy.devarray import DevArray
 from ..numpy.vjps import _concrete, repeat_to_match_shape
 
 
