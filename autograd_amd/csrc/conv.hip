@@ -7,9 +7,9 @@
 // is walked in place and the taps that fall off the signal are skipped.  Flips arrive as negative
 // strides.
 //
-// Two shapes of problem occur, and each has its kernel.
+// Two shapes of problem occur, and each has its kernels.
 //
-// correlate_positions: the forward pass and the signal's cotangent have many output positions and
+// correlate_tiled / correlate_positions: the forward pass and the signal's cotangent have many output positions and
 // a short reduction (channels x window).  A thread owns one (signal batch, position) pair and a
 // tile of TI filter-batch entries (output channels): each signal element it loads feeds TI
 // multiply-adds whose filter operands are wave-uniform.
@@ -32,7 +32,16 @@ struct CorrParams {
     uint32_t p_total;    // P[0] * P[1] * P[2]
     uint32_t tiles;      // correlate_positions: blocks per filter-batch tile
     uint32_t lane_bits;  // correlate_reduce: log2 of the lanes that share the innermost window axis
+    // correlate_tiled: a block covers 2^jt_bits images x 2^p1_bits rows x 2^p2_bits columns of output
+    // (256 positions) and stages the H x W window of signal they read, per image, in LDS
+    int jt_bits, p1_bits, p2_bits, H, W;
+    int DT;                     // contracted indices staged per step
+    uint32_t n_tj, n_t1, n_t2;  // tiles along each
+    uint32_t s_elems_padded;    // LDS elements reserved for the signal tile (a multiple of 8)
 };
+
+constexpr int kTileLoads = 8;    // signal elements a thread stages per step: tiles of up to 2048 elements
+constexpr int kFilterLoads = 4;  // filter elements a thread stages per step: DT * K1 * K2 * TI up to 1024
 
 template <typename T>
 __device__ __forceinline__ T fused_mul_add(T a, T b, T c);
@@ -95,6 +104,156 @@ __global__ __launch_bounds__(kBlock) void correlate_positions(const T *__restric
         }
     }
     if (!live) return;
+    T *o = out + j * c.o_ss + p0 * c.o_s[0] + p1 * c.o_s[1] + p2 * c.o_s[2];
+#pragma unroll
+    for (int t = 0; t < TI; ++t)
+        if (i0 + t < c.I) o[(i0 + t) * c.o_fs] = acc[t];
+}
+
+// The same contraction with the operands staged in LDS.  A block owns 256 output positions (a tile of
+// images x rows x columns) and TI filter-batch entries.  For every contracted index d (and tap k0 of
+// a third convolved axis) it copies the window of signal its positions read (zero where the window
+// leaves the signal: the padding is made here, once per element, not tested per tap) and the
+// K1 x K2 x TI filter taps into LDS (several d per step while they fit), then every thread walks the
+// window row by row: the LDS reads of a row (signal and broadcast taps) are issued together, then its
+// K2 x TI multiply-adds (rows of width 2, 3, 5, 7 are unrolled; LDS latency, not bandwidth, is what a
+// tap-by-tap loop pays for).  Which
+// global element each thread stages is fixed for the whole kernel and computed once; the loads
+// of step n+1 are issued before the multiply-adds of step n.
+template <typename T, int TI, int K2T>
+__global__ __launch_bounds__(kBlock) void correlate_tiled(const T *__restrict__ filter, const T *__restrict__ signal,
+                                                          T *__restrict__ out, const CorrParams c) {
+    extern __shared__ __align__(64) unsigned char lds_raw[];
+    T *S = reinterpret_cast<T *>(lds_raw);  // [DT][2^jt_bits][H][W]
+    T *F = S + c.s_elems_padded;            // [DT][K1 * K2][TI]
+    uint32_t q = blockIdx.x;
+    const uint32_t t2 = q % c.n_t2;
+    q /= c.n_t2;
+    const uint32_t t1 = q % c.n_t1;
+    q /= c.n_t1;
+    const uint32_t tj = q % c.n_tj;
+    q /= c.n_tj;
+    const int64_t p0 = q % static_cast<uint32_t>(c.P[0]);
+    const int64_t i0 = static_cast<int64_t>(q / static_cast<uint32_t>(c.P[0])) * TI;
+    const int tid = threadIdx.x;
+    const int x = tid & ((1 << c.p2_bits) - 1);
+    const int y = (tid >> c.p2_bits) & ((1 << c.p1_bits) - 1);
+    const int jj = tid >> (c.p2_bits + c.p1_bits);
+    const int64_t j0 = static_cast<int64_t>(tj) << c.jt_bits;
+    const int64_t r0 = static_cast<int64_t>(t1) << c.p1_bits, c0 = static_cast<int64_t>(t2) << c.p2_bits;
+    const int HW = c.H * c.W, s_slice = HW << c.jt_bits, s_elems = s_slice * c.DT;
+    const int K1 = static_cast<int>(c.K[1]), K2 = K2T > 0 ? K2T : static_cast<int>(c.K[2]);
+    const int f_slice = K1 * K2 * TI, f_elems = f_slice * c.DT;
+
+    // what this thread stages: LDS slot tid + n * 256 of either tile.  Slots that fall on padding
+    // (or past the last contracted index) read a valid address and store zero.
+    int64_t s_off[kTileLoads], f_off[kFilterLoads];
+    int s_dd[kTileLoads], f_dd[kFilterLoads];
+    unsigned s_ok = 0;
+#pragma unroll
+    for (int n = 0; n < kTileLoads; ++n) {
+        const int e = tid + n * kBlock;
+        s_off[n] = 0;
+        s_dd[n] = 0;
+        if (e < s_elems) {
+            const int dd = e / s_slice, e1 = e - dd * s_slice;
+            const int ej = e1 / HW, rem = e1 - ej * HW, h = rem / c.W, w = rem - h * c.W;
+            const int64_t j = j0 + ej, s1 = r0 + h - c.pad[1], s2 = c0 + w - c.pad[2];
+            s_dd[n] = dd;
+            if (j < c.J && static_cast<uint64_t>(s1) < static_cast<uint64_t>(c.N[1]) &&
+                static_cast<uint64_t>(s2) < static_cast<uint64_t>(c.N[2])) {
+                s_ok |= 1u << n;
+                s_off[n] = j * c.s_bs + s1 * c.s_s[1] + s2 * c.s_s[2];
+            }
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < kFilterLoads; ++m) {
+        const int e = tid + m * kBlock;
+        f_off[m] = 0;
+        f_dd[m] = 0;
+        if (e < f_elems) {
+            const int dd = e / f_slice, e1 = e - dd * f_slice;
+            const int kk = e1 / TI, t = e1 - kk * TI, k1 = kk / K2, k2 = kk - k1 * K2;
+            const int64_t i = i0 + t < c.I ? i0 + t : c.I - 1;  // rows past the last repeat it (computed, never stored)
+            f_dd[m] = dd;
+            f_off[m] = i * c.f_bs + k1 * c.f_s[1] + k2 * c.f_s[2];
+        }
+    }
+    // taps of the third convolved axis that meet the signal (the same for the whole block)
+    const int64_t b0 = p0 - c.pad[0];
+    const int k0_lo = static_cast<int>(b0 < 0 ? -b0 : 0);
+    const int k0_hi = static_cast<int>(c.N[0] - b0 < c.K[0] ? c.N[0] - b0 : c.K[0]);
+    const int d_groups = k0_hi > k0_lo ? static_cast<int>((c.D + c.DT - 1) / c.DT) : 0;
+
+    // a step = DT contracted indices (group g) at one tap k0 of the third axis.  Every thread issues all
+    // its loads unconditionally (slots it does not own read element 0 again), so none waits on another.
+    T s_reg[kTileLoads], f_reg[kFilterLoads];
+    auto fetch = [&](int g, int k0) {
+        const int64_t d0 = static_cast<int64_t>(g) * c.DT;
+        const int last = static_cast<int>(c.D - 1 - d0 < c.DT ? c.D - 1 - d0 : c.DT);  // indices past the end repeat the last
+        const T *sg = signal + d0 * c.s_ds + (b0 + k0) * c.s_s[0];
+        const T *fg = filter + d0 * c.f_ds + k0 * c.f_s[0];
+#pragma unroll
+        for (int n = 0; n < kTileLoads; ++n) s_reg[n] = sg[(s_dd[n] < last ? s_dd[n] : last) * c.s_ds + s_off[n]];
+#pragma unroll
+        for (int m = 0; m < kFilterLoads; ++m) f_reg[m] = fg[(f_dd[m] < last ? f_dd[m] : last) * c.f_ds + f_off[m]];
+    };
+    T acc[TI];
+#pragma unroll
+    for (int t = 0; t < TI; ++t) acc[t] = T(0);
+    const T *Sp = S + jj * HW + y * c.W + x;
+    int g = 0, k0 = k0_lo;
+    if (d_groups > 0) fetch(g, k0);
+    while (g < d_groups) {
+        const int64_t left = c.D - static_cast<int64_t>(g) * c.DT;
+        const int live = static_cast<int>(left < c.DT ? left : c.DT);  // contracted indices in this step
+        __syncthreads();  // everyone has finished reading the previous step's tiles
+#pragma unroll
+        for (int n = 0; n < kTileLoads; ++n)
+            if (tid + n * kBlock < s_elems)
+                S[tid + n * kBlock] = ((s_ok >> n & 1u) && s_dd[n] < live) ? s_reg[n] : T(0);
+#pragma unroll
+        for (int m = 0; m < kFilterLoads; ++m)
+            if (tid + m * kBlock < f_elems) F[tid + m * kBlock] = f_reg[m];
+        __syncthreads();
+        int g_next = g, k0_next = k0 + 1;
+        if (k0_next >= k0_hi) {
+            k0_next = k0_lo;
+            ++g_next;
+        }
+        if (g_next < d_groups) fetch(g_next, k0_next);  // in flight during the multiply-adds below
+        for (int dd = 0; dd < live; ++dd) {
+            for (int k1 = 0; k1 < K1; ++k1) {
+                const T *row = Sp + dd * s_slice + k1 * c.W;
+                const T *taps = F + dd * f_slice + k1 * K2 * TI;
+                if constexpr (K2T > 0) {
+                    // a window row of known width: its LDS reads are issued together, then the multiply-adds
+                    T sv[K2T], fv[K2T][TI];
+#pragma unroll
+                    for (int k2 = 0; k2 < K2T; ++k2) {
+                        sv[k2] = row[k2];
+#pragma unroll
+                        for (int t = 0; t < TI; ++t) fv[k2][t] = taps[k2 * TI + t];
+                    }
+#pragma unroll
+                    for (int k2 = 0; k2 < K2T; ++k2)
+#pragma unroll
+                        for (int t = 0; t < TI; ++t) acc[t] = fused_mul_add(fv[k2][t], sv[k2], acc[t]);
+                } else {
+                    for (int k2 = 0; k2 < K2; ++k2) {
+                        const T sv = row[k2];
+#pragma unroll
+                        for (int t = 0; t < TI; ++t) acc[t] = fused_mul_add(taps[k2 * TI + t], sv, acc[t]);
+                    }
+                }
+            }
+        }
+        g = g_next;
+        k0 = k0_next;
+    }
+    const int64_t j = j0 + jj, p1 = r0 + y, p2 = c0 + x;
+    if (j >= c.J || p1 >= c.P[1] || p2 >= c.P[2]) return;
     T *o = out + j * c.o_ss + p0 * c.o_s[0] + p1 * c.o_s[1] + p2 * c.o_s[2];
 #pragma unroll
     for (int t = 0; t < TI; ++t)
@@ -170,8 +329,38 @@ void launch_positions(const agmi_correlation *a, CorrParams &c, hipStream_t s) {
                        static_cast<T *>(a->out), c);
 }
 
+template <typename T, int TI, int K2T>
+void launch_tiled_width(const agmi_correlation *a, CorrParams &c, hipStream_t s) {
+    const int64_t blocks = ceil_div(c.I, TI) * c.P[0] * c.n_tj * c.n_t1 * c.n_t2;
+    const size_t lds = (static_cast<size_t>(c.s_elems_padded) + static_cast<size_t>(c.K[1] * c.K[2]) * TI * c.DT) * sizeof(T);
+    hipLaunchKernelGGL((correlate_tiled<T, TI, K2T>), dim3(static_cast<unsigned>(blocks)), dim3(kBlock), lds, s,
+                       static_cast<const T *>(a->filter.data), static_cast<const T *>(a->signal.data),
+                       static_cast<T *>(a->out), c);
+}
+
+// the common window widths get a fully unrolled row; any other width runs the generic loop
+template <typename T, int TI>
+void launch_tiled(const agmi_correlation *a, CorrParams &c, hipStream_t s) {
+    switch (c.K[2]) {
+        case 2: launch_tiled_width<T, TI, 2>(a, c, s); break;
+        case 3: launch_tiled_width<T, TI, 3>(a, c, s); break;
+        case 5: launch_tiled_width<T, TI, 5>(a, c, s); break;
+        case 7: launch_tiled_width<T, TI, 7>(a, c, s); break;
+        default: launch_tiled_width<T, TI, 0>(a, c, s); break;
+    }
+}
+
 template <typename T>
-void launch(const agmi_correlation *a, CorrParams &c, int tile, hipStream_t s) {
+void launch(const agmi_correlation *a, CorrParams &c, int tile, bool tiled, hipStream_t s) {
+    if (tiled) {
+        switch (tile) {
+            case 1: launch_tiled<T, 1>(a, c, s); break;
+            case 2: launch_tiled<T, 2>(a, c, s); break;
+            case 4: launch_tiled<T, 4>(a, c, s); break;
+            default: launch_tiled<T, 8>(a, c, s); break;
+        }
+        return;
+    }
     switch (tile) {
         case 0:
             hipLaunchKernelGGL((correlate_reduce<T>), dim3(static_cast<unsigned>(c.I * c.J * c.p_total)), dim3(kBlock),
@@ -273,19 +462,55 @@ extern "C" int agmi_correlate(int dtype, const agmi_correlation *a, void *stream
         c.lane_bits = 0;
         while (c.lane_bits < 8 && (int64_t(1) << c.lane_bits) < c.K[2]) ++c.lane_bits;
     }
-    const int64_t blocks = tile == 0 ? outputs : ceil_div(pairs, kBlock) * ceil_div(c.I, tile);
+    // The LDS-staged kernel when its tiles fit: 256 positions per block shaped to the output (columns
+    // first), the window of signal they read within kTileLoads x 256 elements, the taps within
+    // kFilterLoads x 256.
+    bool tiled = false;
+    if (tile != 0 && c.D > 0) {
+        // tile shape: columns first (up to 32: whole LDS rows per wave), then rows, then images.  A shape fitted
+        // to the output (12 x 12 as 4 x 4 x 16 images instead of 16 x 16 x 1) wastes fewer threads but was slower
+        // when measured: narrow rows mean more steps and LDS bank conflicts.
+        auto bits_for = [](int64_t n, int cap) {
+            int b = 0;
+            while (b < cap && (int64_t(1) << b) < n) ++b;
+            return b;
+        };
+        c.p2_bits = bits_for(c.P[2], 5);
+        c.p1_bits = bits_for(c.P[1], 8 - c.p2_bits);
+        c.jt_bits = 8 - c.p2_bits - c.p1_bits;
+        const int64_t H = (int64_t(1) << c.p1_bits) + c.K[1] - 1, W = (int64_t(1) << c.p2_bits) + c.K[2] - 1;
+        const int64_t s_elems = (H * W) << c.jt_bits;
+        if (s_elems <= kTileLoads * kBlock && c.K[1] * c.K[2] * tile <= kFilterLoads * kBlock) {
+            tiled = true;
+            c.H = static_cast<int>(H);
+            c.W = static_cast<int>(W);
+            // several contracted indices per step while both tiles still fit: fewer barriers and more loads in flight
+            c.DT = 1;
+            while (c.DT < 8 && c.DT * 2 <= c.D && s_elems * c.DT * 2 <= kTileLoads * kBlock &&
+                   c.K[1] * c.K[2] * tile * c.DT * 2 <= kFilterLoads * kBlock)
+                c.DT *= 2;
+            c.s_elems_padded = static_cast<uint32_t>((s_elems * c.DT + 7) / 8 * 8);
+            c.n_tj = static_cast<uint32_t>(ceil_div(c.J, int64_t(1) << c.jt_bits));
+            c.n_t1 = static_cast<uint32_t>(ceil_div(c.P[1], int64_t(1) << c.p1_bits));
+            c.n_t2 = static_cast<uint32_t>(ceil_div(c.P[2], int64_t(1) << c.p2_bits));
+        }
+    }
+    const int64_t blocks = tile == 0 ? outputs
+                           : tiled   ? ceil_div(c.I, tile) * c.P[0] * c.n_tj * c.n_t1 * c.n_t2
+                                     : ceil_div(pairs, kBlock) * ceil_div(c.I, tile);
     if (blocks > 0x7fffffffLL) {
         set_error("correlate: too many outputs for one launch");
         return AGMI_ERR_UNSUPPORTED;
     }
     hipStream_t s = as_stream(stream);
+    const char *tname = dtype == AGMI_F32 ? "float" : "double";
     if (tile == 0)
-        set_kernel_name("correlate_reduce<%s>", dtype == AGMI_F32 ? "float" : "double");
+        set_kernel_name("correlate_reduce<%s>", tname);
     else
-        set_kernel_name("correlate_positions<%s, %d>", dtype == AGMI_F32 ? "float" : "double", tile);
+        set_kernel_name("correlate_%s<%s, %d>", tiled ? "tiled" : "positions", tname, tile);
     if (dtype == AGMI_F32)
-        launch<float>(a, c, tile, s);
+        launch<float>(a, c, tile, tiled, s);
     else
-        launch<double>(a, c, tile, s);
+        launch<double>(a, c, tile, tiled, s);
     return hip_check(hipGetLastError(), "correlate launch");
 }

@@ -1,7 +1,7 @@
 """``autograd_amd.scipy.signal.convolve`` and ``numpy.pad`` on the device against the CPU oracle
 (oracle/convolution.py, itself bit-identical to the reference on tests/golden/reference_next.npz)
-at sizes that reach both window-contraction kernels (one thread per position with filter-batch
-tiles of 1, 2, 4 and 8; one block per output) and the operand-copy path.
+at sizes that reach every window-contraction kernel (LDS-staged tiles and one thread per position,
+with filter-batch tiles of 1, 2, 4 and 8; one block per output) and the operand-copy path.
 
 Tolerance: |got - want| <= rtol * (|want| + max|want|), rtol 1e-5 (float32) / 1e-12 (float64); the
 summation order of a device contraction differs from numpy.einsum's.
@@ -59,7 +59,7 @@ def test_long_one_dimensional_windows(mode):
 
 
 @pytest.mark.parametrize("filters,tile", [(1, 1), (2, 2), (4, 4), (6, 8), (16, 8)])
-def test_one_thread_per_position_with_filter_batch_tiles(filters, tile):
+def test_staged_tiles_with_filter_batch_tiles(filters, tile):
     import autograd_amd.numpy as dnp
     from autograd_amd import _lib
     from autograd_amd.scipy.signal import convolve as dconv
@@ -70,8 +70,34 @@ def test_one_thread_per_position_with_filter_batch_tiles(filters, tile):
     for mode in ("valid", "same"):
         kw = dict(axes=([2, 3], [2, 3]), dot_axes=([1], [0]), mode=mode)
         got = dconv(dnp.asarray(img), dnp.asarray(filt), **kw)
-        assert _lib.lib().agmi_last_kernel().decode() == f"correlate_positions<float, {tile}>"
+        assert _lib.lib().agmi_last_kernel().decode() == f"correlate_tiled<float, {tile}>"
         _close(got.numpy(), oconv(img, filt, **kw), onp.float32)
+
+
+@pytest.mark.parametrize("dtype", [onp.float32, onp.float64])
+def test_windows_too_large_to_stage_run_one_thread_per_position(dtype):
+    import autograd_amd.numpy as dnp
+    from autograd_amd import _lib
+    from autograd_amd.scipy.signal import convolve as dconv
+    from oracle.convolution import convolve as oconv
+
+    rs = onp.random.RandomState(7)
+    img, filt = rs.randn(200, 200).astype(dtype), rs.randn(40, 40).astype(dtype)
+    got = dconv(dnp.asarray(img), dnp.asarray(filt), mode="valid")
+    assert _lib.lib().agmi_last_kernel().decode().startswith("correlate_positions<")
+    _close(got.numpy(), oconv(img, filt, mode="valid"), dtype)
+
+
+@pytest.mark.parametrize("mode", ["full", "valid", "same"])
+def test_staged_tiles_on_ragged_shapes(mode):
+    """Tile edges: outputs that are not multiples of the tile, images fewer than a tile holds, a third
+    convolved axis, negative strides (the flips) and padding on every side."""
+    rs = onp.random.RandomState(8)
+    _both(dict(axes=([1, 2], [1, 2]), mode=mode), rs.randn(3, 13, 9), rs.randn(2, 4, 3), onp.float64)
+    _both(dict(mode=mode), rs.randn(5, 7, 9).astype(onp.float32), rs.randn(2, 3, 2).astype(onp.float32), onp.float32)
+    _both(dict(axes=([2, 3], [2, 3]), dot_axes=([1], [0]), mode=mode), rs.randn(5, 3, 17, 33), rs.randn(3, 7, 4, 6),
+          onp.float64)
+    _both(dict(mode=mode), rs.randn(1000), rs.randn(9), onp.float64)
 
 
 def test_free_axes_that_do_not_merge_are_copied_once():
