@@ -47,8 +47,8 @@ NUMPY_DTYPE = {v: k for k, v in TORCH_DTYPE.items()}
 class Op:
     COPY, NEG, EXP, LOG, TANH, SINH, COSH, SIN, COS, SQRT, SQUARE, ABS, SIGN, RECIPROCAL, LOG1P, EXPM1 = range(16)
     EXP2, LOG2, LOG10, TAN, ARCSIN, ARCCOS, ARCTAN, ARCSINH, ARCCOSH, ARCTANH = range(16, 26)
-    FLOOR, CEIL, RINT, TRUNC = range(26, 30)
-    ADD, SUB, MUL, DIV, POW, MAXIMUM, MINIMUM, FMAX, FMIN, ARCTAN2, HYPOT, LOGADDEXP = range(32, 44)
+    FLOOR, CEIL, RINT, TRUNC, NAN_TO_NUM = range(26, 31)
+    ADD, SUB, MUL, DIV, POW, MAXIMUM, MINIMUM, FMAX, FMIN, ARCTAN2, HYPOT, LOGADDEXP, REMAINDER = range(32, 45)
     WHERE = 64
     (
         DIV_VJP1,

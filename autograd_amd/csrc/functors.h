@@ -89,6 +89,34 @@ __device__ __forceinline__ T logaddexp_like_numpy(T x, T y) {
     return d;
 }
 
+// numpy.remainder for floating point (npy_divmod): fmod, then moved by one divisor when its sign
+// differs from the divisor's; an exact multiple gives a zero with the divisor's sign; b == 0 -> NaN.
+__device__ __forceinline__ float m_fmod(float a, float b) { return fmodf(a, b); }
+__device__ __forceinline__ double m_fmod(double a, double b) { return fmod(a, b); }
+__device__ __forceinline__ float m_copysign(float a, float b) { return copysignf(a, b); }
+__device__ __forceinline__ double m_copysign(double a, double b) { return copysign(a, b); }
+template <typename T>
+__device__ __forceinline__ T remainder_like_numpy(T a, T b) {
+    T m = m_fmod(a, b);
+    if (b == T(0)) return m;
+    if (m != T(0)) {
+        if ((b < T(0)) != (m < T(0))) m += b;
+    } else {
+        m = m_copysign(T(0), b);
+    }
+    return m;
+}
+
+// numpy.nan_to_num with its defaults: NaN -> 0, infinities -> the largest finite values
+template <typename T>
+__device__ __forceinline__ T nan_to_num_like_numpy(T x) {
+    const T big = sizeof(T) == 4 ? T(__FLT_MAX__) : T(__DBL_MAX__);
+    if (x != x) return T(0);
+    if (x > big) return big;
+    if (x < -big) return -big;
+    return x;
+}
+
 // numpy.fmax / fmin: a NaN operand is ignored when the other one is a number
 template <typename T>
 __device__ __forceinline__ T fmax_like_numpy(T a, T b) {
@@ -161,6 +189,7 @@ AGMI_FUNCTOR(FFloor, 1, 1, o[0] = floor(x[0]);)
 AGMI_FUNCTOR(FCeil, 1, 1, o[0] = ceil(x[0]);)
 AGMI_FUNCTOR(FRint, 1, 1, o[0] = rint(x[0]);)
 AGMI_FUNCTOR(FTrunc, 1, 1, o[0] = trunc(x[0]);)
+AGMI_FUNCTOR(FNanToNum, 1, 1, o[0] = nan_to_num_like_numpy(x[0]);)
 
 AGMI_FUNCTOR(FAdd, 2, 1, o[0] = x[0] + x[1];)
 AGMI_FUNCTOR(FSub, 2, 1, o[0] = x[0] - x[1];)
@@ -175,6 +204,7 @@ AGMI_FUNCTOR(FFmin, 2, 1, o[0] = fmin_like_numpy(x[0], x[1]);)
 AGMI_FUNCTOR(FArctan2, 2, 1, o[0] = m_atan2(x[0], x[1]);)
 AGMI_FUNCTOR(FHypot, 2, 1, o[0] = m_hypot(x[0], x[1]);)
 AGMI_FUNCTOR(FLogaddexp, 2, 1, o[0] = logaddexp_like_numpy(x[0], x[1]);)
+AGMI_FUNCTOR(FRemainder, 2, 1, o[0] = remainder_like_numpy(x[0], x[1]);)
 
 AGMI_FUNCTOR(FWhere, 3, 1, o[0] = (x[0] != T(0)) ? x[1] : x[2];)
 
@@ -258,6 +288,8 @@ AGMI_FUNCTOR(FExtremumVjp, 4, 1, o[0] = (x[0] * ((x[1] == x[2]) ? T(1) : T(0))) 
     X(AGMI_OP_ARCTAN2, FArctan2)                \
     X(AGMI_OP_HYPOT, FHypot)                    \
     X(AGMI_OP_LOGADDEXP, FLogaddexp)            \
+    X(AGMI_OP_REMAINDER, FRemainder)            \
+    X(AGMI_OP_NAN_TO_NUM, FNanToNum)            \
     X(AGMI_OP_WHERE, FWhere)                    \
     X(AGMI_OP_DIV_VJP1, FDivVjp1)               \
     X(AGMI_OP_TANH_VJP, FTanhVjp)               \

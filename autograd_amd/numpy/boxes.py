@@ -33,6 +33,8 @@ _OPERATORS = {
     "__rtruediv__": _route("true_divide", True),
     "__pow__": _route("power"),
     "__rpow__": _route("power", True),
+    "__mod__": _route("remainder"),
+    "__rmod__": _route("remainder", True),
     "__matmul__": _route("matmul"),
     "__rmatmul__": _route("matmul", True),
     "__eq__": _route("equal"),
@@ -53,7 +55,7 @@ def _reshape_method(x, *args, **kwargs):
 
 _METHODS = {
     name: getattr(anp, name)
-    for name in "sum mean max min prod ravel repeat reshape squeeze swapaxes transpose astype dot".split()
+    for name in "sum mean max min prod ravel repeat reshape squeeze swapaxes transpose astype dot diagonal trace".split()
 }
 _METHODS["reshape"] = _reshape_method
 _METHODS["flatten"] = anp.ravel

@@ -82,6 +82,13 @@ defjvp(
     lambda g, ans, x, y: _fused_or(Op.POW_VJP1, (g, _strong_scalar(x), ans),
                                    lambda: g * anp.log(replace_zero(x, 1.0)) * ans),
 )
+defjvp(  # numpy_jvps.py:67-68 (numpy.mod is the same function)
+    anp.remainder,
+    lambda g, ans, x, y: broadcast(g, ans),
+    lambda g, ans, x, y: -g * anp.floor(x / y),
+)
+defjvp(anp.nan_to_num, lambda g, ans, x: anp.where(anp.isfinite(x), g, 0.0))  # numpy_jvps.py:35
+defjvp(anp.kron, "same", "same")  # numpy_jvps.py:155
 for _chooser in (anp.maximum, anp.minimum, anp.fmax, anp.fmin):
     defjvp(
         _chooser,
@@ -95,7 +102,7 @@ defjvp(anp.pad, lambda g, ans, array, width, mode, **kwargs: anp.pad(g, width, m
 # linear one-argument functions (77-105, 150-162)
 for _name in (
     "negative reshape ravel expand_dims squeeze swapaxes moveaxis broadcast_to repeat transpose sum "
-    "_primitive_mean"
+    "_primitive_mean roll diag diagonal make_diagonal trace triu tril tile real real_if_close conjugate"
 ).split():
     defjvp(getattr(anp, _name), "same")
 
@@ -198,7 +205,7 @@ defjvp(anp.max, _fwd_chooser)
 defjvp(anp.min, _fwd_chooser)
 
 # contractions (230-240)
-for _f in (anp.matmul, anp.dot, anp.tensordot, anp.outer):
+for _f in (anp.matmul, anp.dot, anp.tensordot, anp.outer, anp.inner):
     def_linear(_f)
 for _f in (dot_adjoint_0, dot_adjoint_1, tensordot_adjoint_0, tensordot_adjoint_1):
     def_linear(_f)

@@ -11,6 +11,8 @@ computes.  Each has two forms:
   it can itself be differentiated to any order.
 """
 
+from functools import partial
+
 import numpy as onp
 
 from .._lib import REDUCE_FUSABLE, Op, Red
@@ -237,6 +239,12 @@ defvjp(
     lambda ans, x, y: unbroadcast_f(y, lambda g: g * anp.exp(y - ans)),
 )
 defvjp(
+    anp.remainder,  # numpy.mod is the same function (numpy_vjps.py:128-137)
+    lambda ans, x, y: unbroadcast_f(x, lambda g: g),
+    lambda ans, x, y: unbroadcast_f(y, lambda g: -g * anp.floor(x / y)),
+)
+defvjp(anp.nan_to_num, lambda ans, x: lambda g: anp.where(anp.isfinite(x), g, 0.0))  # 216
+defvjp(
     anp.arctan2,
     lambda ans, x, y: unbroadcast_f(x, lambda g: g * y / (x**2 + y**2)),
     lambda ans, x, y: unbroadcast_f(y, lambda g: g * -x / (x**2 + y**2)),
@@ -455,6 +463,68 @@ def _grad_repeat(ans, x, repeats, axis=None):
 
 
 defvjp(anp.repeat, _grad_repeat)
+
+
+def _grad_tile(ans, x, reps):
+    """numpy_vjps.py:352-362: the copies along every axis are added up, first axis first."""
+    reps = (reps,) if anp.isscalar(reps) else tuple(reps)
+    x_shape = anp.shape(x)
+
+    def vjp(g):
+        reps_full = (1,) * (anp.ndim(g) - len(reps)) + reps
+        for axis, rep in enumerate(reps_full):
+            shp = anp.shape(g)
+            g = anp.sum(anp.reshape(g, shp[:axis] + (rep, shp[axis] // rep) + shp[axis + 1 :]), axis=axis)
+        return anp.reshape(g, x_shape)
+
+    return vjp
+
+
+defvjp(anp.tile, _grad_tile)
+
+
+def _grad_kron(argnum, ans, orig_A, orig_B):
+    """numpy_vjps.py:368-392: G viewed with the two operands' axes side by side, then contracted
+    with the other operand over all of its axes."""
+    orig_A_shape, orig_B_shape = anp.shape(orig_A), anp.shape(orig_B)
+
+    def vjp(G):
+        A, B = anp.atleast_2d(orig_A), anp.atleast_2d(orig_B)
+        shape = list(anp.shape(A) + anp.shape(B))
+        n = anp.ndim(A)
+        shape[n - 1], shape[n] = shape[n], shape[n - 1]
+        paired = anp.swapaxes(anp.reshape(G, shape), n - 1, n)
+        if argnum == 0:
+            return anp.reshape(anp.tensordot(paired, B, axes=anp.ndim(B)), orig_A_shape)
+        return anp.reshape(anp.tensordot(A, paired, axes=anp.ndim(A)), orig_B_shape)
+
+    return vjp
+
+
+defvjp(anp.kron, partial(_grad_kron, 0), partial(_grad_kron, 1))
+
+# diagonals and triangles (numpy_vjps.py:193, 201, 205-213, 863-870)
+defvjp(anp.roll, lambda ans, x, shift, axis=None: lambda g: anp.roll(g, -shift, axis=axis))
+defvjp(anp.diag, lambda ans, x, k=0: lambda g: anp.diag(g, k))
+defvjp(anp.triu, lambda ans, x, k=0: lambda g: anp.triu(g, k=k))
+defvjp(anp.tril, lambda ans, x, k=0: lambda g: anp.tril(g, k=k))
+defvjp(
+    anp.trace,  # the reference's einsum("ij,...->ij...", eye, g) has no summed index: a broadcast product
+    lambda ans, x, offset=0: lambda g: anp.reshape(
+        anp.eye(anp.shape(x)[0], anp.shape(x)[1], k=offset), anp.shape(x)[:2] + (1,) * anp.ndim(g)
+    )
+    * g,
+)
+defvjp(
+    anp.diagonal,
+    lambda ans, A, offset=0, axis1=0, axis2=1: lambda g: anp.make_diagonal(g, offset, axis1, axis2),
+)
+defvjp(
+    anp.make_diagonal,
+    lambda ans, D_, offset=0, axis1=0, axis2=1: lambda g: anp.diagonal(g, offset, axis1, axis2),
+)
+for _identity in (anp.real, anp.real_if_close, anp.conjugate):
+    defvjp(_identity, lambda ans, x: lambda g: g)
 
 
 # ---- dense contractions (numpy_vjps.py:552-747) ----------------------------------------------
@@ -679,6 +749,17 @@ defvjp(
     lambda ans, a, b: lambda g: anp.dot(g, anp.ravel(b)),
     lambda ans, a, b: lambda g: anp.dot(anp.ravel(a), g),
 )
+
+
+def _grad_inner(argnum, ans, A, B):  # numpy_vjps.py:552-563
+    A_ndim, B_ndim = anp.ndim(A), anp.ndim(B)
+    axes = ([], []) if A_ndim == 0 or B_ndim == 0 else ([A_ndim - 1], [B_ndim - 1])
+    if argnum == 0:
+        return lambda G: tensordot_adjoint_0(B, G, axes, A_ndim, B_ndim)
+    return lambda G: tensordot_adjoint_1(A, G, axes, A_ndim, B_ndim)
+
+
+defvjp(anp.inner, partial(_grad_inner, 0), partial(_grad_inner, 1))
 
 
 # ---- einsum (numpy_vjps.py:815-860, subscript-string convention) ------------------------------------

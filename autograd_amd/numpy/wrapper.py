@@ -6,6 +6,7 @@ launches HIP kernels; shape queries are never traced; list-taking functions are 
 ``concatenate_args`` / ``array_from_args`` so boxes inside Python lists are seen.
 """
 
+import builtins
 import numbers
 
 import numpy as onp
@@ -107,6 +108,8 @@ fmin = _binary(Op.FMIN, "fmin")
 arctan2 = _binary(Op.ARCTAN2, "arctan2", floating=True)
 hypot = _binary(Op.HYPOT, "hypot", floating=True)
 logaddexp = _binary(Op.LOGADDEXP, "logaddexp", floating=True)
+mod = remainder = _binary(Op.REMAINDER, "remainder", floating=True)
+nan_to_num = _unary(Op.NAN_TO_NUM, "nan_to_num")
 
 
 @primitive
@@ -853,6 +856,150 @@ tensordot = _wrap(_tensordot_raw, "tensordot")
 def outer(a, b):
     a, b = ravel.fun(D.asarray(a)), ravel.fun(D.asarray(b))
     return D.arith_map(Op.MUL, DevArray(a._t.unsqueeze(1), a.dtype), DevArray(b._t.unsqueeze(0), b.dtype))
+
+
+# ---- the remaining array functions with rules in the reference's table (numpy_vjps.py:193-216, 352-405,
+# ---- 552-566, 855-872): views where NumPy gives views, one copy kernel otherwise ------------------------
+def _identity_primitive(name):
+    return _wrap(lambda x: D.asarray(x), name)
+
+
+# real arrays only: these are the identity (numpy_vjps.py:207-213 reduce to passing g through)
+real = _identity_primitive("real")
+real_if_close = _identity_primitive("real_if_close")
+conj = conjugate = _identity_primitive("conjugate")
+
+
+def _copy_into(dst, src):
+    """dst[...] = src with the device copy kernel (cast when the types differ)."""
+    if dst.dtype in D._FLOATS and src.dtype in D._FLOATS:
+        D.map_op(Op.COPY, dst.dtype, src, out=dst)
+    else:
+        _lib.cast(_lib.DTYPE_CODE[src.dtype], _lib.DTYPE_CODE[dst.dtype], dst.shape, dst._t, D.plain(src)._t)
+
+
+@primitive
+def roll(x, shift, axis=None):
+    x = D.asarray(x)
+    if not isinstance(shift, (numbers.Integral, onp.integer)) or not (axis is None or isinstance(axis, numbers.Integral)):
+        raise NotImplementedError("roll: one integer shift along one axis (or the flattened array) is supported")
+    if axis is None:
+        return reshape.fun(roll.fun(ravel.fun(x), shift, 0), x.shape)
+    axis = D.normalize_axes(axis, x.ndim)[0]
+    n = x.shape[axis]
+    out = D.empty(x.shape, x.dtype)
+    s = int(shift) % n if n else 0
+    for dst0, src0, m in ((s, 0, n - s), (0, n - s, s)):
+        if m and x.size:
+            _copy_into(DevArray(out._t.narrow(axis, dst0, m), x.dtype), DevArray(D.plain(x)._t.narrow(axis, src0, m), x.dtype))
+    return out
+
+
+@primitive
+def diagonal(A, offset=0, axis1=0, axis2=1):
+    A = D.asarray(A)
+    return D.plain(A)._view(lambda t: torch.diagonal(t, int(offset), axis1, axis2))
+
+
+@primitive
+def make_diagonal(D_, offset=0, axis1=0, axis2=1):
+    """Zeros with ``D_`` written on the diagonal of the last two axes (numpy_wrapper.py:172-185: only that
+    placement exists, and the zeros are float64 whatever ``D_`` is)."""
+    if not (offset == 0 and axis1 == -1 and axis2 == -2):
+        raise NotImplementedError(
+            "Currently make_diagonal only supports offset=0, axis1=-1, axis2=-2"
+        )
+    d = D.asarray(D_)
+    out = D.zeros(d.shape + (d.shape[-1],), onp.dtype(onp.float64))
+    if d.size:
+        _copy_into(DevArray(torch.diagonal(out._t, 0, -1, -2), out.dtype), d)
+    return out
+
+
+@primitive
+def diag(x, k=0):
+    x = D.asarray(x)
+    k = int(k)
+    if x.ndim == 2:
+        return D.plain(x)._view(lambda t: torch.diagonal(t, k))
+    if x.ndim != 1:
+        raise ValueError("Input must be 1- or 2-d.")
+    n = x.shape[0] + (k if k >= 0 else -k)
+    out = D.zeros((n, n), x.dtype)
+    if x.size:
+        _copy_into(DevArray(torch.diagonal(out._t, k), x.dtype), x)
+    return out
+
+
+@primitive
+def trace(x, offset=0):
+    x = D.asarray(x)
+    if x.ndim < 2:
+        raise ValueError("diag requires an array of at least two dimensions")
+    return sum.fun(diagonal.fun(x, offset), axis=-1)
+
+
+_TRIANGLES = {}
+
+
+def _triangle(x, k, lower):
+    x = D.asarray(x)
+    if x.ndim < 2:
+        x = D.asarray(broadcast_to.fun(x, (x.shape[0] if x.ndim else 1,) * 2))
+    n, m = x.shape[-2:]
+    dt = x.dtype if x.dtype in D._FLOATS else onp.dtype(onp.float64)
+    key = (n, m, int(k), dt, lower)
+    keep = _TRIANGLES.get(key)
+    if keep is None:
+        tri = onp.tri(n, m, k if lower else k - 1, dtype=bool)
+        keep = _TRIANGLES[key] = D.from_numpy((tri if lower else ~tri).astype(dt))
+    if x.dtype not in D._FLOATS:
+        raise NotImplementedError("tril/triu: floating-point arrays only on the device")
+    return D.map_op(Op.WHERE, dt, keep, x, 0.0)
+
+
+tril = _wrap(lambda x, k=0: _triangle(x, k, True), "tril")
+triu = _wrap(lambda x, k=0: _triangle(x, k, False), "triu")
+
+
+@primitive
+def tile(x, reps):
+    x = D.asarray(x)
+    reps = (int(reps),) if isinstance(reps, (numbers.Integral, onp.integer)) else tuple(int(r) for r in reps)
+    nd = builtins.max(len(reps), x.ndim)
+    reps = (1,) * (nd - len(reps)) + reps
+    shp = (1,) * (nd - x.ndim) + x.shape
+    # out viewed as (r0, n0, r1, n1, ...) = x broadcast along the r axes
+    lifted, wide, final = [], [], []
+    for r, n in zip(reps, shp):
+        lifted += [1, n]
+        wide += [r, n]
+        final.append(r * n)
+    widened = D.plain(x)._view(lambda t: t.reshape(lifted).expand(wide))
+    out = D.copy(widened) if onp.prod(wide) else D.empty(tuple(wide), x.dtype)
+    return DevArray(out._t.view(final), x.dtype)
+
+
+@primitive
+def kron(a, b):
+    a, b = D.asarray(a), D.asarray(b)
+    nd = builtins.max(a.ndim, b.ndim)
+    sa, sb = (1,) * (nd - a.ndim) + a.shape, (1,) * (nd - b.ndim) + b.shape
+    la, lb, final = [], [], []
+    for n, m in zip(sa, sb):
+        la += [n, 1]
+        lb += [1, m]
+        final.append(n * m)
+    out = D.arith_map(Op.MUL, D.plain(a)._view(lambda t: t.reshape(la)), D.plain(b)._view(lambda t: t.reshape(lb)))
+    return DevArray(D.contiguous(out)._t.view(final), out.dtype)
+
+
+@primitive
+def inner(a, b):
+    if onp.ndim(a) == 0 or onp.ndim(b) == 0:  # a Python scalar stays weakly typed in the product
+        return D.arith_map(Op.MUL, a, b)
+    a, b = D.asarray(a), D.asarray(b)
+    return _tensordot_raw(a, b, axes=([a.ndim - 1], [b.ndim - 1]))
 
 
 # ---- einsum (subscript-string convention) -> sums, permutations and batched MFMA GEMMs ----------------

@@ -109,6 +109,7 @@ typedef enum agmi_op {
     AGMI_OP_CEIL,
     AGMI_OP_RINT,     /* round half to even: numpy.rint, numpy.round(x) with decimals=0            */
     AGMI_OP_TRUNC,
+    AGMI_OP_NAN_TO_NUM, /* NaN -> 0, +-inf -> +-largest finite (numpy.nan_to_num defaults), numpy_vjps.py:216 */
     /* two inputs */
     AGMI_OP_ADD = 32, /* also VSpace._add / _mut_add, autograd/core.py:259-264 (out may alias in0) */
     AGMI_OP_SUB,
@@ -122,6 +123,7 @@ typedef enum agmi_op {
     AGMI_OP_ARCTAN2,  /* (y, x)                       numpy_vjps.py:131-135                     */
     AGMI_OP_HYPOT,
     AGMI_OP_LOGADDEXP,/* numpy_vjps.py:114-118 */
+    AGMI_OP_REMAINDER,/* numpy.mod / numpy.remainder: result takes the sign of the divisor, numpy_vjps.py:128-137 */
     /* three inputs */
     AGMI_OP_WHERE = 64, /* c != 0 ? x : y  (c in the array dtype)                             */
     /* fused derivative rules; inputs in the order listed */

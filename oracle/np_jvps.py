@@ -76,6 +76,8 @@ for _name in (
 ).split():
     defjvp(getattr(anp, _name), "same")
 defjvp(anp.full, "same", argnums=(1,))
+defjvp(anp.make_diagonal, "same")  # numpy_jvps.py:94
+defjvp(anp.kron, "same", "same")  # numpy_jvps.py:155
 
 # unary ufuncs (108-134)
 _unary = {

@@ -20,7 +20,7 @@ fmax fmin logaddexp hypot arctan2 where clip nan_to_num real imag conj conjugate
 rad2deg degrees deg2rad radians
 sum mean prod max min amax amin var std cumsum
 reshape ravel expand_dims squeeze transpose swapaxes moveaxis atleast_1d atleast_2d
-atleast_3d repeat tile broadcast_to roll flipud fliplr diag diagonal trace tril triu
+atleast_3d repeat tile split broadcast_to roll flipud fliplr diag diagonal trace tril triu
 dot matmul tensordot inner outer einsum kron
 astype
 floor ceil round rint around fix trunc all any argmax argmin argsort nonzero
@@ -114,6 +114,17 @@ def stack(arrays, axis=0):
 
 
 _raw_where = where  # noqa: F821
+
+
+@primitive
+def make_diagonal(D, offset=0, axis1=0, axis2=1):  # numpy_wrapper.py:172-185
+    if not (offset == 0 and axis1 == -1 and axis2 == -2):
+        raise NotImplementedError("Currently make_diagonal only supports offset=0, axis1=-1, axis2=-2")
+    out = _np.zeros(D.shape + (D.shape[-1],))
+    out_diagonal = _np.diagonal(out, offset, axis1, axis2)
+    out_diagonal.flags.writeable = True
+    out_diagonal[...] = D
+    return out
 
 
 def where(condition, *args, **kwargs):  # noqa: F811

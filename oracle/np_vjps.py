@@ -322,6 +322,53 @@ def _grad_repeat(ans, x, repeats, axis=None):
 
 
 defvjp(anp.repeat, _grad_repeat)
+defvjp(anp.split, lambda ans, ary, idxs, axis=0: lambda g: anp.concatenate(g, axis=axis))  # numpy_vjps.py:195
+
+
+def _grad_tile(ans, x, reps):  # numpy_vjps.py:352-364
+    reps = [reps] if anp.isscalar(reps) else reps
+    x_shape = anp.shape(x)
+
+    def vjp(g):
+        for axis, rep in enumerate(reps):
+            g = sum(anp.split(g, rep, axis))
+        return anp.reshape(g, x_shape)
+
+    return vjp
+
+
+defvjp(anp.tile, _grad_tile)
+
+
+def _grad_kron(argnum, ans, orig_A, orig_B):  # numpy_vjps.py:367-392
+    orig_A_shape, orig_B_shape = anp.shape(orig_A), anp.shape(orig_B)
+
+    def vjp(G):
+        A, B = anp.atleast_2d(orig_A), anp.atleast_2d(orig_B)
+        shape = list(A.shape + B.shape)
+        n = anp.ndim(A)
+        shape[n - 1], shape[n] = shape[n], shape[n - 1]
+        reshaped_G = anp.swapaxes(anp.reshape(G, shape), n - 1, n)
+        if argnum == 0:
+            return match_complex(orig_A, anp.reshape(anp.tensordot(reshaped_G, B, axes=anp.ndim(B)), orig_A_shape))
+        return match_complex(orig_B, anp.reshape(anp.tensordot(A, reshaped_G, axes=anp.ndim(A)), orig_B_shape))
+
+    return vjp
+
+
+defvjp(anp.kron, partial(_grad_kron, 0), partial(_grad_kron, 1))
+defvjp(  # numpy_vjps.py:205-210
+    anp.trace,
+    lambda ans, x, offset=0: lambda g: anp.einsum("ij,...->ij...", anp.eye(x.shape[0], x.shape[1], k=offset), g),
+)
+defvjp(  # numpy_vjps.py:863-870
+    anp.diagonal,
+    lambda ans, A, offset=0, axis1=0, axis2=1: lambda g: anp.make_diagonal(g, offset, axis1, axis2),
+)
+defvjp(
+    anp.make_diagonal,
+    lambda ans, D, offset=0, axis1=0, axis2=1: lambda g: anp.diagonal(g, offset, axis1, axis2),
+)
 
 
 def _reverse_axis(x, axis):

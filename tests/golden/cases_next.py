@@ -296,4 +296,64 @@ def next_cases(be, ext):
             first = lambda x, y: np.sum(np.sin(conv(x, y, mode=mode, **kw)))  # noqa: E731,B023
             second = lambda x, y: sum(np.sum(np.tanh(d)) for d in grad(first, (0, 1))(x, y))  # noqa: E731,B023
             out[f"conv/second_{name}_{mode}"] = grad(second, (0, 1))(a, b)
+    
+
+    # ---- the rest of the array-function table (numpy_vjps.py:128-137, 193-216, 352-405, 552-566, 863-870): remainder,
+    # nan_to_num, roll, diagonals and triangles, tile, kron, inner; reverse, forward, second order, both precisions ----
+    tA, tQ, tV, tT = rs.uniform(-0.9, 0.9, (3, 4)), rs.randn(4, 4), rs.randn(4), rs.randn(2, 3, 4)
+    tB, tY = rs.randn(2, 3), rs.uniform(0.2, 0.6, (3, 4)) * rs.choice([-1.0, 1.0], (3, 4))
+    tS = rs.randn(2, 3, 3)
+    special = tA.copy()
+    special[0, 1], special[1, 2], special[2, 0] = onp.nan, onp.inf, -onp.inf
+    for dtype in (onp.float64, onp.float32):
+        tag = "f32" if dtype == onp.float32 else "f64"
+        A_, Q_, v_, T_, B_, Y_ = (P(h.astype(dtype)) for h in (tA, tQ, tV, tT, tB, tY))
+        S_, C_ = P(special.astype(dtype)), P(tS.astype(dtype))
+        W34, W44, W55 = (P(rs.randn(n, m).astype(dtype)) for n, m in ((3, 4), (4, 4), (5, 5)))
+        table = {
+            "remainder_array": (lambda a: np.sum(np.remainder(a, Y_) * W34), A_),
+            "mod_scalar": (lambda a: np.sum(np.mod(a, 0.3) * W34), A_),
+            "mod_negative_scalar": (lambda a: np.sum(np.mod(a, -0.4) * W34), A_),
+            "mod_second_arg": (lambda a: np.sum(np.mod(Q_[:3] * 3.0, a) * W34), Y_),
+            "mod_operator": (lambda a: np.sum((a % Y_) * W34), A_),
+            "nan_to_num": (lambda a: np.sum(np.nan_to_num(a * 2.0) * W34), S_),
+            "roll_axis0": (lambda a: np.sum(np.roll(a, 1, axis=0) * W34), A_),
+            "roll_axis1_negative": (lambda a: np.sum(np.roll(a, -2, axis=1) * W34), A_),
+            "roll_flat": (lambda a: np.sum(np.roll(a, 5) * W34), A_),
+            "roll_wraps": (lambda a: np.sum(np.roll(a, 9, axis=-1) * W34), A_),
+            "diag_of_matrix": (lambda q: np.sum(np.diag(q, 1) ** 2), Q_),
+            "diag_of_vector": (lambda q: np.sum(np.diag(q[0], -1) ** 2 * W55), Q_),
+            "diag_twice": (lambda q: np.sum(np.diag(np.diag(q)) * W44), Q_),
+            "diagonal_last_axes": (lambda t: np.sum(np.diagonal(t, 0, -1, -2) ** 2), C_),
+            "make_diagonal": (lambda a: np.sum(np.make_diagonal(a, 0, -1, -2) * W44[None, :, :] * 2.0), A_),
+            "trace": (lambda q: np.trace(q) * 2.0, Q_),
+            "trace_offset": (lambda q: np.trace(q, offset=1) ** 2, Q_),
+            "trace_rectangle": (lambda a: np.trace(a, offset=-1) * 3.0, A_),
+            "trace_of_stack": (lambda t: np.sum(np.trace(t) * v_), T_),
+            "tril": (lambda q: np.sum(np.tril(q) * W44), Q_),
+            "triu_offset": (lambda q: np.sum(np.triu(q, 1) ** 2), Q_),
+            "tril_rectangle": (lambda a: np.sum(np.tril(a, -1) * W34), A_),
+            "triu_batched": (lambda t: np.sum(np.triu(t, -1) ** 2), T_),
+            "tile_2d": (lambda a: np.sum(np.tile(a, (2, 3)) ** 2), A_),
+            "tile_more_reps": (lambda a: np.sum(np.tile(a, (2, 1, 2)) * T_[:, :, :1] * 0.5), A_),
+            "tile_vector_scalar_reps": (lambda q: np.sum(np.tile(q[1], 3) ** 3), Q_),
+            "kron_2d": (lambda a: np.sum(np.kron(a, B_) ** 2), A_),
+            "kron_2d_second": (lambda a: np.sum(np.kron(B_, a) ** 2), A_),
+            "kron_1d": (lambda q: np.sum(np.kron(q[0], v_) ** 2), Q_),
+            "kron_2d_1d": (lambda a: np.sum(np.kron(a, v_) ** 2), A_),
+            "kron_both": (lambda a: np.sum(np.kron(a, a.T) * 0.5), A_),
+            "inner_matrices": (lambda a: np.sum(np.inner(a, Q_) ** 2), A_),
+            "inner_vectors": (lambda q: np.inner(q[0], v_) ** 2, Q_),
+            "inner_stack_vector": (lambda t: np.sum(np.inner(t, v_) ** 2), T_),
+            "inner_second": (lambda a: np.sum(np.inner(T_, a) ** 2), A_),
+            "real_conj": (lambda a: np.sum(np.real(a) * np.conj(a) * 2.0), A_),
+        }
+        for name, (f, x) in table.items():
+            out[f"table/{name}_{tag}/value"] = f(x)
+            out[f"table/{name}_{tag}/grad"] = grad(f)(x)
+            tangent_in = P(rs.randn(*onp.shape(be.get(x))).astype(dtype))
+            out[f"table/{name}_{tag}/jvp_tangent"] = be.make_jvp(f)(x)(tangent_in)[1]
+            if not name.startswith(("mod", "remainder_array", "nan_to_num")):  # piecewise linear in x: no second order
+                weights2 = P(rs.randn(*onp.shape(be.get(x))).astype(dtype))
+                out[f"table/{name}_{tag}/second"] = grad(lambda a: np.sum(grad(f)(a) * weights2))(x)  # noqa: B023
     return out

@@ -697,3 +697,80 @@ def test_matrix_cotangents_accumulate_inside_the_contraction(dnp, dtype, rows, i
     assert onp.array_equal(ag.grad(fm)(W).numpy(), want)
     hm = lambda x: dnp.sum((x @ V1) * C1) + dnp.sum((x @ V2) * C2)  # noqa: E731
     assert onp.array_equal(ag.grad(hm)(X1).numpy(), (dnp.dot(C1, V1.T) + dnp.dot(C2, V2.T)).numpy())
+
+
+# ---- remainder, nan_to_num and the array functions built on views and copy kernels: bit-exact ---------------
+@pytest.mark.parametrize("dtype", [F32, F64])
+def test_remainder_and_nan_to_num_are_bit_exact(dnp, dtype):
+    rs = onp.random.RandomState(31)
+    a = (rs.randn(257, 33) * 7).astype(dtype)
+    b = (rs.uniform(0.2, 3.0, (257, 33)) * rs.choice([-1.0, 1.0], (257, 33))).astype(dtype)
+    # exact multiples (signed zero results), zero dividends and divisors, infinities and NaN
+    a[0, :8] = onp.array([6.0, -6.0, 0.0, -0.0, 5.0, -5.0, onp.inf, onp.nan], dtype)
+    b[0, :8] = onp.array([3.0, 3.0, -2.0, 2.0, 0.0, onp.inf, 2.0, 2.0], dtype)
+    b[1, :4] = onp.array([-3.0, -3.0, onp.inf, -onp.inf], dtype)
+    a[1, :4] = onp.array([6.0, -6.0, -5.0, 5.0], dtype)
+    with onp.errstate(all="ignore"):
+        want = onp.remainder(a, b)
+        got = dnp.remainder(P(dnp, a), P(dnp, b)).numpy()
+        assert got.dtype == want.dtype and onp.array_equal(got, want, equal_nan=True)
+        ok = ~onp.isnan(want)  # the sign of a zero result is the divisor's; a NaN's sign means nothing
+        assert onp.array_equal(onp.signbit(got[ok]), onp.signbit(want[ok]))
+        assert onp.array_equal(dnp.mod(P(dnp, a), 0.75).numpy(), onp.mod(a, dtype(0.75)), equal_nan=True)
+        assert onp.array_equal((P(dnp, a) % P(dnp, b)).numpy(), want, equal_nan=True)
+        assert onp.array_equal((2.5 % P(dnp, b)).numpy(), 2.5 % b, equal_nan=True)
+    x = a.copy()
+    x[2, :3] = [onp.nan, onp.inf, -onp.inf]
+    got = dnp.nan_to_num(P(dnp, x)).numpy()
+    assert got.dtype == dtype and onp.array_equal(got, onp.nan_to_num(x))
+
+
+@pytest.mark.parametrize("dtype", [F32, F64])
+def test_array_functions_on_views_and_copies_are_bit_exact(dnp, dtype):
+    rs = onp.random.RandomState(32)
+    a, q, v, t = (rs.randn(*s).astype(dtype) for s in ((5, 7), (6, 6), (7,), (3, 5, 7)))
+    A, Q, V, T = (P(dnp, h) for h in (a, q, v, t))
+
+    def same(got, want):
+        got = got.numpy()
+        assert got.shape == want.shape and got.dtype == want.dtype, (got.shape, want.shape, got.dtype, want.dtype)
+        assert onp.array_equal(got, want, equal_nan=True)
+
+    for shift, axis in ((1, 0), (-2, 1), (9, -1), (0, 0), (5, None), (-3, None)):
+        same(dnp.roll(A, shift, axis=axis), onp.roll(a, shift, axis=axis))
+    same(dnp.roll(T[:, ::2], 2, axis=1), onp.roll(t[:, ::2], 2, axis=1))
+    for k in (-2, 0, 1, 3):
+        same(dnp.diag(Q, k), onp.diag(q, k))
+        same(dnp.diag(A, k), onp.diag(a, k))
+        same(dnp.diag(V, k), onp.diag(v, k))
+        same(dnp.tril(A, k), onp.tril(a, k))
+        same(dnp.triu(A, k), onp.triu(a, k))
+        same(dnp.triu(T, k), onp.triu(t, k))
+        same(dnp.diagonal(T, k, 1, 2), onp.diagonal(t, k, 1, 2))
+        same(dnp.diagonal(T, k, -1, 0), onp.diagonal(t, k, -1, 0))
+    same(Q.diagonal(), q.diagonal())
+    same(dnp.tril(dnp.asarray(onp.array([[onp.nan, onp.inf], [1.0, -onp.inf]], dtype))),
+         onp.tril(onp.array([[onp.nan, onp.inf], [1.0, -onp.inf]], dtype)))  # masked entries are zeros, not NaN
+    for reps in (3, (2,), (2, 3), (2, 1, 2), (1, 1), (0, 2)):
+        same(dnp.tile(A, reps), onp.tile(a, reps))
+    same(dnp.tile(V, 4), onp.tile(v, 4))
+    same(dnp.tile(T.T, (2, 1, 3)), onp.tile(t.T, (2, 1, 3)))
+    for x, y, hx, hy in ((A, Q, a, q), (V, V, v, v), (A, V, a, v), (V, A, v, a), (T, A, t, a), (A.T, Q[:2], a.T, q[:2])):
+        same(dnp.kron(x, y), onp.kron(hx, hy))
+    wide = onp.zeros(a.shape + (a.shape[-1],))
+    for i in range(a.shape[0]):
+        wide[i] = onp.diag(a[i].astype(F64))
+    same(dnp.make_diagonal(A, 0, -1, -2), wide)  # float64 zeros whatever the operand, as the reference builds them
+    with pytest.raises(NotImplementedError):
+        dnp.make_diagonal(A)
+    same(dnp.real(A), a)
+    same(dnp.conj(A), a)
+    # traces and inner products accumulate: tolerance of the reductions / contractions
+    for k in (-1, 0, 2):
+        close(dnp.trace(Q, k).numpy(), onp.asarray(onp.trace(q, k)), RT[dtype])
+        close(dnp.trace(T, k).numpy(), onp.trace(t, k), RT[dtype])
+    close(Q.trace().numpy(), onp.asarray(q.trace()), RT[dtype])
+    close(dnp.inner(A, T).numpy(), onp.inner(a, t), RT[dtype])
+    close(dnp.inner(V, V).numpy(), onp.asarray(onp.inner(v, v)), RT[dtype])
+    close(dnp.inner(T, V).numpy(), onp.inner(t, v), RT[dtype])
+    same(dnp.inner(A, 2.0), onp.inner(a, dtype(2.0)))
