@@ -48,7 +48,7 @@ class Op:
     COPY, NEG, EXP, LOG, TANH, SINH, COSH, SIN, COS, SQRT, SQUARE, ABS, SIGN, RECIPROCAL, LOG1P, EXPM1 = range(16)
     EXP2, LOG2, LOG10, TAN, ARCSIN, ARCCOS, ARCTAN, ARCSINH, ARCCOSH, ARCTANH = range(16, 26)
     FLOOR, CEIL, RINT, TRUNC, NAN_TO_NUM = range(26, 31)
-    ADD, SUB, MUL, DIV, POW, MAXIMUM, MINIMUM, FMAX, FMIN, ARCTAN2, HYPOT, LOGADDEXP, REMAINDER = range(32, 45)
+    ADD, SUB, MUL, DIV, POW, MAXIMUM, MINIMUM, FMAX, FMIN, ARCTAN2, HYPOT, LOGADDEXP, REMAINDER, LOGADDEXP2 = range(32, 46)
     WHERE = 64
     (
         DIV_VJP1,
@@ -164,6 +164,8 @@ def lib():
                             c_i64, c_d, c_p, c_i64, c_i64, c_p, c_sz, c_p]
     L.agmi_fill.restype = c_i
     L.agmi_fill.argtypes = [c_i, c_p, c_i64, c_d, c_p]
+    L.agmi_cumsum.restype = c_i
+    L.agmi_cumsum.argtypes = [c_i, c_p, c_i64, c_i64, c_i64, c_p, c_p]
     L.agmi_take_rows.restype = c_i
     L.agmi_take_rows.argtypes = [c_i, c_p, c_i64, c_i64, c_p, c_i64, c_p, c_p]
     L.agmi_scatter_add_rows.restype = c_i
@@ -178,7 +180,7 @@ def lib():
 
 EXPORTS = (
     "agmi_last_error agmi_version agmi_last_kernel agmi_elementwise agmi_compare agmi_cast agmi_map_reduce "
-    "agmi_map_reduce_workspace_bytes agmi_gemm agmi_fill agmi_take_rows agmi_scatter_add_rows agmi_optimizer_step "
+    "agmi_map_reduce_workspace_bytes agmi_gemm agmi_fill agmi_take_rows agmi_cumsum agmi_scatter_add_rows agmi_optimizer_step "
     "agmi_correlate"
 ).split()
 
@@ -466,6 +468,10 @@ def fill(code, t, value):
 def take_rows(code, src, n_rows, inner, index, n_index, out):
     _check(_LIB.agmi_take_rows(code, src.data_ptr(), n_rows, inner, index.data_ptr(), n_index, out.data_ptr(),
                                _stream()), "agmi_take_rows")
+
+
+def cumsum(code, src, outer, n, inner, out):
+    _check(_LIB.agmi_cumsum(code, src.data_ptr(), outer, n, inner, out.data_ptr(), _stream()), "agmi_cumsum")
 
 
 def scatter_add_rows(code, dst, n_rows, inner, src, index, order, seg_start, n_seg):

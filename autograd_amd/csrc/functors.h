@@ -89,6 +89,17 @@ __device__ __forceinline__ T logaddexp_like_numpy(T x, T y) {
     return d;
 }
 
+// numpy.logaddexp2 (npy_math): like logaddexp with exp2 and log1p scaled by log2(e)
+template <typename T>
+__device__ __forceinline__ T logaddexp2_like_numpy(T x, T y) {
+    const T kLog2e = T(1.442695040888963407359924681001892137);
+    if (x == y) return x + T(1);
+    const T d = x - y;
+    if (d > T(0)) return x + kLog2e * m_log1p(m_exp2(-d));
+    if (d <= T(0)) return y + kLog2e * m_log1p(m_exp2(d));
+    return d;
+}
+
 // numpy.remainder for floating point (npy_divmod): fmod, then moved by one divisor when its sign
 // differs from the divisor's; an exact multiple gives a zero with the divisor's sign; b == 0 -> NaN.
 __device__ __forceinline__ float m_fmod(float a, float b) { return fmodf(a, b); }
@@ -205,6 +216,7 @@ AGMI_FUNCTOR(FArctan2, 2, 1, o[0] = m_atan2(x[0], x[1]);)
 AGMI_FUNCTOR(FHypot, 2, 1, o[0] = m_hypot(x[0], x[1]);)
 AGMI_FUNCTOR(FLogaddexp, 2, 1, o[0] = logaddexp_like_numpy(x[0], x[1]);)
 AGMI_FUNCTOR(FRemainder, 2, 1, o[0] = remainder_like_numpy(x[0], x[1]);)
+AGMI_FUNCTOR(FLogaddexp2, 2, 1, o[0] = logaddexp2_like_numpy(x[0], x[1]);)
 
 AGMI_FUNCTOR(FWhere, 3, 1, o[0] = (x[0] != T(0)) ? x[1] : x[2];)
 
@@ -289,6 +301,7 @@ AGMI_FUNCTOR(FExtremumVjp, 4, 1, o[0] = (x[0] * ((x[1] == x[2]) ? T(1) : T(0))) 
     X(AGMI_OP_HYPOT, FHypot)                    \
     X(AGMI_OP_LOGADDEXP, FLogaddexp)            \
     X(AGMI_OP_REMAINDER, FRemainder)            \
+    X(AGMI_OP_LOGADDEXP2, FLogaddexp2)          \
     X(AGMI_OP_NAN_TO_NUM, FNanToNum)            \
     X(AGMI_OP_WHERE, FWhere)                    \
     X(AGMI_OP_DIV_VJP1, FDivVjp1)               \

@@ -40,6 +40,57 @@ __global__ __launch_bounds__(kBlock) void scatter_add_rows_kernel(T *__restrict_
     dst[r * inner + c] = acc;
 }
 
+// Running sums along the middle axis of a contiguous (outer, n, inner) array, added in index order like
+// numpy.add.accumulate, so the result is bit-identical to NumPy's.  One thread owns one (outer, inner) line;
+// neighbouring threads read neighbouring `inner` positions.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void cumsum_lines(const T *__restrict__ src, int64_t outer, int64_t n,
+                                                       int64_t inner, T *__restrict__ out) {
+    const int64_t line = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (line >= outer * inner) return;
+    const int64_t o = line / inner, c = line - o * inner;
+    const T *p = src + o * n * inner + c;
+    T *q = out + o * n * inner + c;
+    T acc = p[0];
+    q[0] = acc;
+    for (int64_t k = 1; k < n; ++k) {
+        acc = acc + p[k * inner];
+        q[k * inner] = acc;
+    }
+}
+
+// The same along the last axis (inner == 1): one wavefront takes 64 rows and walks them in chunks of 64
+// columns staged through LDS, so that global loads and stores run along the rows (coalesced) while each
+// lane still adds its own row's elements one after the other.
+constexpr int kScanTile = 64;
+
+template <typename T>
+__global__ __launch_bounds__(kScanTile) void cumsum_rows(const T *__restrict__ src, int64_t rows, int64_t n,
+                                                         T *__restrict__ out) {
+    __shared__ T tile[kScanTile][kScanTile + 1];
+    const int lane = threadIdx.x;
+    const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kScanTile;
+    const int live = static_cast<int>(rows - row0 < kScanTile ? rows - row0 : kScanTile);
+    T acc = T(0);
+    for (int64_t c0 = 0; c0 < n; c0 += kScanTile) {
+        const bool in_col = c0 + lane < n;
+        for (int r = 0; r < live; ++r)
+            if (in_col) tile[r][lane] = src[(row0 + r) * n + c0 + lane];
+        __syncthreads();
+        if (lane < live) {
+            const int width = static_cast<int>(n - c0 < kScanTile ? n - c0 : kScanTile);
+            for (int j = 0; j < width; ++j) {
+                acc = (c0 == 0 && j == 0) ? tile[lane][0] : acc + tile[lane][j];
+                tile[lane][j] = acc;
+            }
+        }
+        __syncthreads();
+        for (int r = 0; r < live; ++r)
+            if (in_col) out[(row0 + r) * n + c0 + lane] = tile[r][lane];
+        __syncthreads();
+    }
+}
+
 }  // namespace agmi
 
 using namespace agmi;
@@ -109,4 +160,45 @@ extern "C" int agmi_scatter_add_rows(int dtype, void *dst, int64_t n_rows, int64
         return AGMI_ERR_ARG;
     }
     return hip_check(hipGetLastError(), "scatter_add_rows launch");
+}
+
+extern "C" int agmi_cumsum(int dtype, const void *src, int64_t outer, int64_t n, int64_t inner, void *out,
+                           void *stream) {
+    if (outer < 0 || n < 0 || inner < 0) {
+        set_error("cumsum: negative extent");
+        return AGMI_ERR_ARG;
+    }
+    if (outer == 0 || n == 0 || inner == 0) return 0;
+    if (!src || !out) {
+        set_error("cumsum: null operand");
+        return AGMI_ERR_ARG;
+    }
+    if (dtype != AGMI_F32 && dtype != AGMI_F64) {
+        set_error("cumsum: dtype %d is not a floating type", dtype);
+        return AGMI_ERR_ARG;
+    }
+    const bool rows = inner == 1;
+    const int64_t blocks = rows ? ceil_div(outer, kScanTile) : ceil_div(outer * inner, kBlock);
+    if (blocks > 0x7fffffffLL) {
+        set_error("cumsum: too many lines");
+        return AGMI_ERR_UNSUPPORTED;
+    }
+    hipStream_t s = as_stream(stream);
+    set_kernel_name(rows ? "cumsum_rows" : "cumsum_lines");
+    if (dtype == AGMI_F32) {
+        if (rows)
+            hipLaunchKernelGGL(cumsum_rows<float>, dim3((unsigned)blocks), dim3(kScanTile), 0, s,
+                               static_cast<const float *>(src), outer, n, static_cast<float *>(out));
+        else
+            hipLaunchKernelGGL(cumsum_lines<float>, dim3((unsigned)blocks), dim3(kBlock), 0, s,
+                               static_cast<const float *>(src), outer, n, inner, static_cast<float *>(out));
+    } else {
+        if (rows)
+            hipLaunchKernelGGL(cumsum_rows<double>, dim3((unsigned)blocks), dim3(kScanTile), 0, s,
+                               static_cast<const double *>(src), outer, n, static_cast<double *>(out));
+        else
+            hipLaunchKernelGGL(cumsum_lines<double>, dim3((unsigned)blocks), dim3(kBlock), 0, s,
+                               static_cast<const double *>(src), outer, n, inner, static_cast<double *>(out));
+    }
+    return hip_check(hipGetLastError(), "cumsum launch");
 }

@@ -89,6 +89,12 @@ defjvp(  # numpy_jvps.py:67-68 (numpy.mod is the same function)
 )
 defjvp(anp.nan_to_num, lambda g, ans, x: anp.where(anp.isfinite(x), g, 0.0))  # numpy_jvps.py:35
 defjvp(anp.kron, "same", "same")  # numpy_jvps.py:155
+def_linear(anp.cross)  # numpy_jvps.py:106
+defjvp(anp.logaddexp2, lambda g, ans, x, y: g * 2 ** (x - ans), lambda g, ans, x, y: g * 2 ** (y - ans))  # 65
+defjvp(  # numpy_jvps.py:135-138
+    anp.sinc,
+    lambda g, ans, x: g * (anp.cos(anp.pi * x) * anp.pi * x - anp.sin(anp.pi * x)) / (anp.pi * x**2),
+)
 for _chooser in (anp.maximum, anp.minimum, anp.fmax, anp.fmin):
     defjvp(
         _chooser,
@@ -102,7 +108,8 @@ defjvp(anp.pad, lambda g, ans, array, width, mode, **kwargs: anp.pad(g, width, m
 # linear one-argument functions (77-105, 150-162)
 for _name in (
     "negative reshape ravel expand_dims squeeze swapaxes moveaxis broadcast_to repeat transpose sum "
-    "_primitive_mean roll diag diagonal make_diagonal trace triu tril tile real real_if_close conjugate"
+    "_primitive_mean roll diag diagonal make_diagonal trace triu tril tile real real_if_close conjugate flipud fliplr flip rot90 "
+    "array_split split vsplit hsplit dsplit rollaxis diff cumsum"
 ).split():
     defjvp(getattr(anp, _name), "same")
 

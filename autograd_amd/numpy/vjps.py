@@ -239,6 +239,20 @@ defvjp(
     lambda ans, x, y: unbroadcast_f(y, lambda g: g * anp.exp(y - ans)),
 )
 defvjp(
+    anp.logaddexp2,  # numpy_vjps.py:119-123
+    lambda ans, x, y: unbroadcast_f(x, lambda g: g * 2 ** (x - ans)),
+    lambda ans, x, y: unbroadcast_f(y, lambda g: g * 2 ** (y - ans)),
+)
+defvjp(
+    anp.sinc,  # numpy_vjps.py:188-191
+    lambda ans, x: lambda g: g * (anp.cos(anp.pi * x) * anp.pi * x - anp.sin(anp.pi * x)) / (anp.pi * x**2),
+)
+defvjp(
+    anp.cross,  # numpy_vjps.py:231-239
+    lambda ans, a, b, axisa=-1, axisb=-1, axisc=-1, axis=None: lambda g: anp.cross(b, g, axisb, axisc, axisa, axis),
+    lambda ans, a, b, axisa=-1, axisb=-1, axisc=-1, axis=None: lambda g: anp.cross(g, a, axisc, axisa, axisb, axis),
+)
+defvjp(
     anp.remainder,  # numpy.mod is the same function (numpy_vjps.py:128-137)
     lambda ans, x, y: unbroadcast_f(x, lambda g: g),
     lambda ans, x, y: unbroadcast_f(y, lambda g: -g * anp.floor(x / y)),
@@ -506,6 +520,71 @@ defvjp(anp.kron, partial(_grad_kron, 0), partial(_grad_kron, 1))
 # diagonals and triangles (numpy_vjps.py:193, 201, 205-213, 863-870)
 defvjp(anp.roll, lambda ans, x, shift, axis=None: lambda g: anp.roll(g, -shift, axis=axis))
 defvjp(anp.diag, lambda ans, x, k=0: lambda g: anp.diag(g, k))
+# pieces of an array (numpy_vjps.py:194-198): the cotangent is the list of the pieces' cotangents, joined again
+defvjp(anp.array_split, lambda ans, ary, idxs, axis=0: lambda g: anp.concatenate(g, axis=axis))
+defvjp(anp.split, lambda ans, ary, idxs, axis=0: lambda g: anp.concatenate(g, axis=axis))
+defvjp(anp.vsplit, lambda ans, ary, idxs: lambda g: anp.concatenate(g, axis=0))
+defvjp(anp.hsplit, lambda ans, ary, idxs: lambda g: anp.concatenate(g, axis=1))
+defvjp(anp.dsplit, lambda ans, ary, idxs: lambda g: anp.concatenate(g, axis=2))
+
+
+def _grad_rollaxis(ans, a, axis, start=0):  # numpy_vjps.py:255-267
+    if axis < 0:
+        raise NotImplementedError("Gradient of rollaxis not implemented for axis < 0. Please use moveaxis instead.")
+    if start < 0:
+        raise NotImplementedError("Gradient of rollaxis not implemented for start < 0. Please use moveaxis instead.")
+    return lambda g: anp.rollaxis(g, start - 1, axis) if start > axis else anp.rollaxis(g, start, axis + 1)
+
+
+defvjp(anp.rollaxis, _grad_rollaxis)
+
+
+def _grad_diff(ans, a, n=1, axis=-1):
+    """numpy_vjps.py:270-294: each differencing is undone by joining minus the first cotangent, minus the
+    differences of the cotangents, and the last cotangent."""
+    nd = anp.ndim(a)
+    ans_shape = anp.shape(ans)
+    first, last = [slice(None)] * nd, [slice(None)] * nd
+    first[axis], last[axis] = slice(None, 1), slice(-1, None)
+
+    def undiff(g):
+        if anp.shape(g)[axis] > 0:
+            return anp.concatenate((-g[tuple(first)], -anp.diff(g, axis=axis), g[tuple(last)]), axis=axis)
+        shape = list(ans_shape)
+        shape[axis] = 1
+        return anp.zeros(shape)
+
+    def vjp(g):
+        for _ in range(n):
+            g = undiff(g)
+        return g
+
+    return vjp
+
+
+defvjp(anp.diff, _grad_diff)
+
+
+def _reverse_axis(x, axis):  # numpy_vjps.py:533-536
+    x = anp.swapaxes(x, axis, 0)
+    x = x[::-1, ...]
+    return anp.swapaxes(x, 0, axis)
+
+
+def _grad_cumsum(ans, x, axis=None):  # numpy_vjps.py:539-549
+    def vjp(g):
+        if axis:
+            return _reverse_axis(anp.cumsum(_reverse_axis(g, axis), axis), axis)
+        return anp.reshape(anp.cumsum(g[::-1], axis)[::-1], anp.shape(x))
+
+    return vjp
+
+
+defvjp(anp.cumsum, _grad_cumsum)
+defvjp(anp.flipud, lambda ans, x: lambda g: anp.flipud(g))
+defvjp(anp.fliplr, lambda ans, x: lambda g: anp.fliplr(g))
+defvjp(anp.flip, lambda ans, x, axis=None: lambda g: anp.flip(g, axis))  # not in the reference's table: its own inverse
+defvjp(anp.rot90, lambda ans, x, k=1: lambda g: anp.rot90(g, -k))
 defvjp(anp.triu, lambda ans, x, k=0: lambda g: anp.triu(g, k=k))
 defvjp(anp.tril, lambda ans, x, k=0: lambda g: anp.tril(g, k=k))
 defvjp(

@@ -109,6 +109,7 @@ arctan2 = _binary(Op.ARCTAN2, "arctan2", floating=True)
 hypot = _binary(Op.HYPOT, "hypot", floating=True)
 logaddexp = _binary(Op.LOGADDEXP, "logaddexp", floating=True)
 mod = remainder = _binary(Op.REMAINDER, "remainder", floating=True)
+logaddexp2 = _binary(Op.LOGADDEXP2, "logaddexp2", floating=True)
 nan_to_num = _unary(Op.NAN_TO_NUM, "nan_to_num")
 
 
@@ -564,8 +565,6 @@ def _is_basic_index(idx):
         if it is None or it is Ellipsis or isinstance(it, (numbers.Integral, onp.integer)):
             continue
         if isinstance(it, slice):
-            if it.step is not None and it.step <= 0:
-                raise NotImplementedError("slices with a non-positive step are not supported on the device")
             continue
         return False
     return True
@@ -597,11 +596,66 @@ def _host_index(idx):
     return arr.astype(onp.int64)
 
 
+def _positive_steps(idx, shape):
+    """``(idx_up, axes)``: a basic index whose slices all step upwards and select the same elements as
+    ``idx``, and the axes of the result along which that selection is reversed to give ``A[idx]``
+    (device views cannot have negative strides; a reversal is one gather)."""
+    items = list(idx if isinstance(idx, tuple) else (idx,))
+    if not any(isinstance(it, slice) and it.step is not None and it.step < 0 for it in items):
+        return idx, ()
+    if any(it is Ellipsis for it in items):
+        k = [it is Ellipsis for it in items].index(True)
+        consumed = len([it for it in items if it is not None and it is not Ellipsis])
+        items[k : k + 1] = [slice(None)] * (len(shape) - consumed)
+    up, axes, src_axis, res_axis = [], [], 0, 0
+    for it in items:
+        if it is None:
+            up.append(None)
+            res_axis += 1
+            continue
+        if src_axis >= len(shape):
+            raise IndexError("too many indices for array")
+        if isinstance(it, slice):
+            if it.step is not None and it.step < 0:
+                picked = range(*it.indices(shape[src_axis]))
+                it = slice(picked[-1], picked[0] + 1, -picked.step) if len(picked) else slice(0, 0, 1)
+                axes.append(res_axis)
+            res_axis += 1
+        up.append(it)
+        src_axis += 1
+    return tuple(up), tuple(axes)
+
+
+_REVERSED_ROWS = {}
+
+
+def _reverse_axes(x, axes):
+    """``x`` reversed along ``axes`` (a new contiguous array): the row gather with a cached descending index."""
+    for axis in axes:
+        n = x.shape[axis]
+        if n <= 1 or x.size == 0:
+            continue
+        if x.dtype not in D._FLOATS:
+            raise NotImplementedError("reversal of non-floating arrays")
+        outer, inner = int(onp.prod(x.shape[:axis], dtype=onp.int64)), int(onp.prod(x.shape[axis + 1 :], dtype=onp.int64))
+        index = _REVERSED_ROWS.get((outer, n))
+        if index is None:
+            host = (onp.arange(outer, dtype=onp.int64)[:, None] * n + onp.arange(n - 1, -1, -1, dtype=onp.int64)).ravel()
+            index = _REVERSED_ROWS[(outer, n)] = D.from_numpy(host)
+        src = D.contiguous(D.plain(x))
+        out = D.empty(x.shape, x.dtype)
+        _lib.take_rows(_lib.DTYPE_CODE[x.dtype], src._t, outer * n, inner, index._t, outer * n, out._t)
+        x = out
+    return x
+
+
 def take(A, idx):
-    """``A[idx]``: views for basic indices, a gather kernel for an integer array on axis 0."""
+    """``A[idx]``: views for basic indices (plus one gather per axis sliced backwards), a gather kernel for an
+    integer array on axis 0."""
     if _is_basic_index(idx):
-        pidx = _plain(idx)
-        return A._view(lambda t: t[pidx])
+        pidx, backwards = _positive_steps(_plain(idx), A.shape)
+        picked = A._view(lambda t: t[pidx])
+        return _reverse_axes(picked, backwards) if backwards else picked
     rows = _host_index(idx)
     if rows is None:
         raise NotImplementedError(
@@ -649,6 +703,10 @@ def scatter_add(A, idx, x):
     from .vspaces import is_broadcast_view, is_shared_zero
 
     basic = _is_basic_index(idx)
+    if basic:
+        idx, backwards = _positive_steps(_plain(idx), A.shape)
+        if backwards:  # A[::-1] += x  is  A[::1] += x reversed
+            x = _reverse_axes(D.asarray(broadcast_to.fun(D.asarray(x, A.dtype), tuple(A._t[idx].shape))), backwards)
     if A._borrowed or type(A) is not DevArray or is_broadcast_view(A) or is_shared_zero(A):  # not this accumulator's own memory yet: allocate it
         if is_shared_zero(A):
             if basic:
@@ -893,6 +951,155 @@ def roll(x, shift, axis=None):
         if m and x.size:
             _copy_into(DevArray(out._t.narrow(axis, dst0, m), x.dtype), DevArray(D.plain(x)._t.narrow(axis, src0, m), x.dtype))
     return out
+
+
+@primitive
+def cumsum(x, axis=None):
+    """Running sums, added in index order like NumPy's (bit-identical): one line per thread."""
+    x = D.asarray(x)
+    if x.dtype not in D._FLOATS:
+        raise NotImplementedError("cumsum: floating-point arrays only on the device")
+    if axis is None:
+        x, axis = D.asarray(ravel.fun(x)), 0
+    (axis,) = D.normalize_axes(axis, x.ndim)
+    src = D.contiguous(D.plain(x))
+    out = D.empty(x.shape, x.dtype)
+    outer, inner = int(onp.prod(x.shape[:axis], dtype=onp.int64)), int(onp.prod(x.shape[axis + 1 :], dtype=onp.int64))
+    _lib.cumsum(_lib.DTYPE_CODE[x.dtype], src._t, outer, x.shape[axis], inner, out._t)
+    return out
+
+
+def _split_views(ary, sections, axis, even):
+    ary = D.asarray(ary)
+    (axis,) = D.normalize_axes(axis, ary.ndim)
+    n = ary.shape[axis]
+    if isinstance(sections, (numbers.Integral, onp.integer)):
+        k = int(sections)
+        if k <= 0:
+            raise ValueError("number sections must be larger than 0.")
+        if even and n % k:
+            raise ValueError("array split does not result in an equal division")
+        each, extra = divmod(n, k)
+        bounds = [0]
+        for i in range(k):
+            bounds.append(bounds[-1] + each + (1 if i < extra else 0))
+    else:
+        bounds = [0] + [int(b) for b in sections] + [n]
+    pieces = []
+    for lo, hi in zip(bounds[:-1], bounds[1:]):
+        lo, hi = slice(lo, hi).indices(n)[:2]
+        pieces.append(D.plain(ary)._view(lambda t, lo=lo, hi=hi: t.narrow(axis, lo, hi - lo if hi > lo else 0)))
+    return pieces
+
+
+split = _wrap(lambda ary, indices_or_sections, axis=0: _split_views(ary, indices_or_sections, axis, True), "split")
+array_split = _wrap(lambda ary, indices_or_sections, axis=0: _split_views(ary, indices_or_sections, axis, False),
+                    "array_split")
+vsplit = _wrap(lambda ary, indices_or_sections: _split_views(ary, indices_or_sections, 0, True), "vsplit")
+hsplit = _wrap(lambda ary, indices_or_sections: _split_views(
+    ary, indices_or_sections, 1 if D.asarray(ary).ndim > 1 else 0, True), "hsplit")
+dsplit = _wrap(lambda ary, indices_or_sections: _split_views(ary, indices_or_sections, 2, True), "dsplit")
+
+
+@primitive
+def diff(a, n=1, axis=-1):
+    a = D.asarray(a)
+    (axis,) = D.normalize_axes(axis, a.ndim)
+    if n < 0:
+        raise ValueError("order must be non-negative but got " + repr(n))
+    for _ in range(int(n)):
+        m = a.shape[axis]
+        hi = D.plain(a)._view(lambda t: t.narrow(axis, 1, m - 1) if m else t)
+        lo = D.plain(a)._view(lambda t: t.narrow(axis, 0, m - 1) if m else t)
+        a = D.arith_map(Op.SUB, hi, lo)
+    return a
+
+
+@primitive
+def sinc(x):
+    """sin(pi x) / (pi x) the way NumPy evaluates it: x == 0 is moved to 1e-20 first."""
+    x = D.asarray(x)
+    dt = D._float_dtype(x.dtype)
+    moved = D.map_op(Op.WHERE, dt, D.astype(D.compare(Cmp.EQ, x, 0.0), dt), 1.0e-20, x)
+    y = D.map_op(Op.MUL, dt, onp.pi, moved)
+    return D.map_op(Op.DIV, dt, D.map_op(Op.SIN, dt, y), y)
+
+
+@primitive
+def cross(a, b, axisa=-1, axisb=-1, axisc=-1, axis=None):
+    """Vector product of 3-vectors (NumPy's own evaluation order: each component is one product minus another)."""
+    if axis is not None:
+        axisa = axisb = axisc = axis
+    a, b = D.asarray(a), D.asarray(b)
+    a, b = D.asarray(moveaxis.fun(a, axisa, -1)), D.asarray(moveaxis.fun(b, axisb, -1))
+    if a.shape[-1] != 3 or b.shape[-1] != 3:
+        raise NotImplementedError("cross: 3-vectors only on the device")
+    part = lambda v, k: v._view(lambda t: t[..., k])  # noqa: E731
+    comps = []
+    for i, j in ((1, 2), (2, 0), (0, 1)):
+        comps.append(D.arith_map(Op.SUB, D.arith_map(Op.MUL, part(a, i), part(b, j)),
+                                 D.arith_map(Op.MUL, part(a, j), part(b, i))))
+    out = stack(comps, axis=-1)
+    return moveaxis.fun(out, -1, axisc)
+
+
+@primitive
+def rollaxis(a, axis, start=0):
+    a = D.asarray(a)
+    n = a.ndim
+    (axis,) = D.normalize_axes(axis, n)
+    if start < 0:
+        start += n
+    if not 0 <= start < n + 1:
+        raise onp.exceptions.AxisError(f"'start' arg requires {-n} <= start < {n + 1}, but {start - n if start < 0 else start} was passed in")
+    if axis < start:
+        start -= 1
+    if axis == start:
+        return a
+    order = list(range(n))
+    order.remove(axis)
+    order.insert(start, axis)
+    return transpose.fun(a, order)
+
+
+@primitive
+def flip(m, axis=None):
+    m = D.asarray(m)
+    return _reverse_axes(m, D.normalize_axes(axis, m.ndim))
+
+
+@primitive
+def flipud(m):
+    m = D.asarray(m)
+    if m.ndim < 1:
+        raise ValueError("Input must be >= 1-d.")
+    return flip.fun(m, 0)
+
+
+@primitive
+def fliplr(m):
+    m = D.asarray(m)
+    if m.ndim < 2:
+        raise ValueError("Input must be >= 2-d.")
+    return flip.fun(m, 1)
+
+
+@primitive
+def rot90(m, k=1, axes=(0, 1)):
+    m = D.asarray(m)
+    if len(axes) != 2:
+        raise ValueError("len(axes) must be 2.")
+    (a0,), (a1,) = D.normalize_axes(axes[0], m.ndim), D.normalize_axes(axes[1], m.ndim)
+    if a0 == a1:
+        raise ValueError("Axes must be different.")
+    k = int(k) % 4
+    if k == 0:
+        return m
+    if k == 2:
+        return flip.fun(m, (a0, a1))
+    turned = D.asarray(swapaxes.fun(m, a0, a1))
+    # a quarter turn is a transposition and one reversal (numpy.rot90: k=1 reverses axis a1 first, k=3 reverses it after)
+    return flip.fun(turned, a0 if k == 1 else a1)
 
 
 @primitive

@@ -124,6 +124,7 @@ typedef enum agmi_op {
     AGMI_OP_HYPOT,
     AGMI_OP_LOGADDEXP,/* numpy_vjps.py:114-118 */
     AGMI_OP_REMAINDER,/* numpy.mod / numpy.remainder: result takes the sign of the divisor, numpy_vjps.py:128-137 */
+    AGMI_OP_LOGADDEXP2,/* log2(2**x + 2**y) the way NumPy evaluates it, numpy_vjps.py:119-123 */
     /* three inputs */
     AGMI_OP_WHERE = 64, /* c != 0 ? x : y  (c in the array dtype)                             */
     /* fused derivative rules; inputs in the order listed */
@@ -228,6 +229,13 @@ int agmi_fill(int dtype, void *ptr, int64_t n, double value, void *stream);
  * integer-array idx on the leading axis (numpy_boxes.py:16-18). */
 int agmi_take_rows(int dtype, const void *src, int64_t n_rows, int64_t inner,
                    const int64_t *index, int64_t n_index, void *out, void *stream);
+
+/* Running sums along the middle axis of a contiguous (outer, n, inner) array:
+ * out[o, k, c] = src[o, 0, c] + ... + src[o, k, c], added in that order (bit-identical to
+ * numpy.cumsum).  Forward of numpy.cumsum and, on reversed operands, its cotangent
+ * (numpy_vjps.py:533-549).  src and out must not overlap. */
+int agmi_cumsum(int dtype, const void *src, int64_t outer, int64_t n, int64_t inner, void *out,
+                void *stream);
 
 /* Ordered scatter-add: for i = 0 .. n_index-1 IN THIS ORDER: dst[index[i], :] += src[i, :].
  * Bit-identical to numpy.add.at (numpy_vjps.py:941-950): a destination row that occurs several

@@ -62,6 +62,7 @@ for _chooser in (anp.maximum, anp.minimum, anp.fmax, anp.fmin):
     )
 defjvp(anp.logaddexp, lambda g, ans, x, y: g * anp.exp(x - ans), lambda g, ans, x, y: g * anp.exp(y - ans))
 defjvp(anp.mod, lambda g, ans, x, y: broadcast(g, ans), lambda g, ans, x, y: -g * anp.floor(x / y))
+defjvp(anp.logaddexp2, lambda g, ans, x, y: g * 2 ** (x - ans), lambda g, ans, x, y: g * 2 ** (y - ans))  # 65
 defjvp(
     anp.power,
     lambda g, ans, x, y: g * y * x ** anp.where(y, y - 1, 1.0),
@@ -72,7 +73,8 @@ defjvp(anp.arctan2, lambda g, ans, x, y: g * y / (x**2 + y**2), lambda g, ans, x
 # linear one-argument functions (77-105, 150-162)
 for _name in (
     "negative reshape ravel expand_dims squeeze swapaxes moveaxis roll flipud fliplr diag diagonal "
-    "trace triu tril broadcast_to repeat tile transpose sum _primitive_mean cumsum"
+    "trace triu tril broadcast_to repeat tile transpose sum _primitive_mean cumsum "
+    "array_split split vsplit hsplit dsplit rollaxis rot90 diff"
 ).split():
     defjvp(getattr(anp, _name), "same")
 defjvp(anp.full, "same", argnums=(1,))
@@ -108,6 +110,7 @@ _unary = {
     "real": lambda g, ans, x: anp.real(g),
     "conj": lambda g, ans, x: anp.conj(g),
     "nan_to_num": lambda g, ans, x: anp.where(anp.isfinite(x), g, 0.0),
+    "sinc": lambda g, ans, x: g * (anp.cos(anp.pi * x) * anp.pi * x - anp.sin(anp.pi * x)) / (anp.pi * x**2),
 }
 for _name, _rule in _unary.items():
     defjvp(getattr(anp, _name), _rule)
@@ -173,7 +176,7 @@ for _f in (anp.max, anp.min, anp.amax, anp.amin):
     defjvp(_f, _fwd_chooser)
 
 # contractions (230-240)
-for _f in (anp.inner, anp.matmul, anp.dot, anp.tensordot, anp.outer, anp.einsum):
+for _f in (anp.inner, anp.matmul, anp.dot, anp.tensordot, anp.outer, anp.einsum, anp.cross):
     def_linear(_f)
 for _f in (dot_adjoint_0, dot_adjoint_1, tensordot_adjoint_0, tensordot_adjoint_1):
     def_linear(_f)

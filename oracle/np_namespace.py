@@ -20,7 +20,7 @@ fmax fmin logaddexp hypot arctan2 where clip nan_to_num real imag conj conjugate
 rad2deg degrees deg2rad radians
 sum mean prod max min amax amin var std cumsum
 reshape ravel expand_dims squeeze transpose swapaxes moveaxis atleast_1d atleast_2d
-atleast_3d repeat tile split broadcast_to roll flipud fliplr diag diagonal trace tril triu
+atleast_3d repeat tile split array_split vsplit hsplit dsplit rollaxis rot90 diff cross sinc logaddexp2 broadcast_to roll flipud fliplr diag diagonal trace tril triu
 dot matmul tensordot inner outer einsum kron
 astype
 floor ceil round rint around fix trunc all any argmax argmin argsort nonzero

@@ -97,6 +97,11 @@ _binary(
     lambda ans, x, y: lambda g: g * anp.exp(y - ans),
 )
 _binary(anp.mod, lambda ans, x, y: lambda g: g, lambda ans, x, y: lambda g: -g * anp.floor(x / y))
+_binary(  # numpy_vjps.py:119-123
+    anp.logaddexp2,
+    lambda ans, x, y: lambda g: g * 2 ** (x - ans),
+    lambda ans, x, y: lambda g: g * 2 ** (y - ans),
+)
 _binary(
     anp.power,
     lambda ans, x, y: lambda g: g * y * x ** anp.where(y, y - 1, 1.0),
@@ -139,6 +144,7 @@ _unary = {
     "real": lambda ans, x: lambda g: match_complex(x, g),
     "conj": lambda ans, x: lambda g: anp.conj(g),
     "nan_to_num": lambda ans, x: lambda g: anp.where(anp.isfinite(x), g, 0.0),
+    "sinc": lambda ans, x: lambda g: g * (anp.cos(anp.pi * x) * anp.pi * x - anp.sin(anp.pi * x)) / (anp.pi * x**2),
 }
 for _name, _maker in _unary.items():
     defvjp(getattr(anp, _name), _maker)
@@ -322,7 +328,53 @@ def _grad_repeat(ans, x, repeats, axis=None):
 
 
 defvjp(anp.repeat, _grad_repeat)
-defvjp(anp.split, lambda ans, ary, idxs, axis=0: lambda g: anp.concatenate(g, axis=axis))  # numpy_vjps.py:195
+# numpy_vjps.py:194-198, 204
+defvjp(anp.array_split, lambda ans, ary, idxs, axis=0: lambda g: anp.concatenate(g, axis=axis))
+defvjp(anp.split, lambda ans, ary, idxs, axis=0: lambda g: anp.concatenate(g, axis=axis))
+defvjp(anp.vsplit, lambda ans, ary, idxs: lambda g: anp.concatenate(g, axis=0))
+defvjp(anp.hsplit, lambda ans, ary, idxs: lambda g: anp.concatenate(g, axis=1))
+defvjp(anp.dsplit, lambda ans, ary, idxs: lambda g: anp.concatenate(g, axis=2))
+defvjp(anp.rot90, lambda ans, x, k=1: lambda g: anp.rot90(g, -k))
+defvjp(  # numpy_vjps.py:231-239
+    anp.cross,
+    lambda ans, a, b, axisa=-1, axisb=-1, axisc=-1, axis=None: lambda g: anp.cross(b, g, axisb, axisc, axisa, axis),
+    lambda ans, a, b, axisa=-1, axisb=-1, axisc=-1, axis=None: lambda g: anp.cross(g, a, axisc, axisa, axisb, axis),
+)
+
+
+def _grad_rollaxis(ans, a, axis, start=0):  # numpy_vjps.py:255-267
+    if axis < 0:
+        raise NotImplementedError("Gradient of rollaxis not implemented for axis < 0. Please use moveaxis instead.")
+    elif start < 0:
+        raise NotImplementedError("Gradient of rollaxis not implemented for start < 0. Please use moveaxis instead.")
+    return lambda g: anp.rollaxis(g, start - 1, axis) if start > axis else anp.rollaxis(g, start, axis + 1)
+
+
+defvjp(anp.rollaxis, _grad_rollaxis)
+
+
+def _grad_diff(ans, a, n=1, axis=-1):  # numpy_vjps.py:270-294
+    nd = anp.ndim(a)
+    ans_shape = anp.shape(ans)
+    sl1 = [slice(None)] * nd
+    sl1[axis] = slice(None, 1)
+    sl2 = [slice(None)] * nd
+    sl2[axis] = slice(-1, None)
+
+    def undiff(g):
+        if g.shape[axis] > 0:
+            return anp.concatenate((-g[tuple(sl1)], -anp.diff(g, axis=axis), g[tuple(sl2)]), axis=axis)
+        shape = list(ans_shape)
+        shape[axis] = 1
+        return anp.zeros(shape)
+
+    def helper(g, n):
+        return g if n == 0 else helper(undiff(g), n - 1)
+
+    return lambda g: helper(g, n)
+
+
+defvjp(anp.diff, _grad_diff)
 
 
 def _grad_tile(ans, x, reps):  # numpy_vjps.py:352-364

@@ -316,7 +316,7 @@ def next_cases(be, ext):
             "mod_negative_scalar": (lambda a: np.sum(np.mod(a, -0.4) * W34), A_),
             "mod_second_arg": (lambda a: np.sum(np.mod(Q_[:3] * 3.0, a) * W34), Y_),
             "mod_operator": (lambda a: np.sum((a % Y_) * W34), A_),
-            "nan_to_num": (lambda a: np.sum(np.nan_to_num(a * 2.0) * W34), S_),
+            "nan_to_num": (lambda a: np.sum(np.nan_to_num(a * 2.0) * 1e-30 * W34), S_),
             "roll_axis0": (lambda a: np.sum(np.roll(a, 1, axis=0) * W34), A_),
             "roll_axis1_negative": (lambda a: np.sum(np.roll(a, -2, axis=1) * W34), A_),
             "roll_flat": (lambda a: np.sum(np.roll(a, 5) * W34), A_),
@@ -346,6 +346,40 @@ def next_cases(be, ext):
             "inner_vectors": (lambda q: np.inner(q[0], v_) ** 2, Q_),
             "inner_stack_vector": (lambda t: np.sum(np.inner(t, v_) ** 2), T_),
             "inner_second": (lambda a: np.sum(np.inner(T_, a) ** 2), A_),
+            "flipud": (lambda a: np.sum(np.flipud(a) * W34), A_),
+            "fliplr": (lambda a: np.sum(np.fliplr(a) ** 2 * W34), A_),
+            "fliplr_of_stack": (lambda t: np.sum(np.fliplr(t) * W34), T_),
+            "rot90": (lambda q: np.sum(np.rot90(q) * W44), Q_),
+            "rot90_half_turn": (lambda q: np.sum(np.rot90(q, 2) ** 2 * W44), Q_),
+            "rot90_back": (lambda a: np.sum(np.rot90(a, -1) * W34.T), A_),
+            "reversed_rows": (lambda a: np.sum(a[::-1] * W34), A_),
+            "reversed_strided_columns": (lambda a: np.sum(a[:, ::-2] ** 2 * W34[:, :2]), A_),
+            "reversed_both_partial": (lambda a: np.sum(a[2:0:-1, ::-1] * W34[:2]), A_),
+            "reversed_after_ellipsis": (lambda t: np.sum(t[..., ::-1] ** 2 * W34), T_),
+            "reversed_with_newaxis_and_int": (lambda t: np.sum(t[1, None, ::-1] * W34), T_),
+            "cumsum_flat": (lambda a: np.sum(np.cumsum(a) ** 2), A_),
+            "cumsum_axis0": (lambda a: np.sum(np.cumsum(a, axis=0) * W34), A_),
+            "cumsum_axis1": (lambda a: np.sum(np.cumsum(a, axis=1) ** 2), A_),
+            "cumsum_middle_axis": (lambda t: np.sum(np.cumsum(t, axis=1) * W34), T_),
+            "cumsum_last_axis_of_stack": (lambda t: np.sum(np.cumsum(t, axis=-1) ** 2), T_),
+            "split_even": (lambda a: np.sum(np.split(a, 2, axis=1)[0] * np.split(a, 2, axis=1)[1]), A_),
+            "split_at_indices": (lambda a: np.sum(np.split(a, [1, 3], axis=1)[1] ** 2) + np.sum(np.split(a, [1, 3], 1)[2]), A_),
+            "array_split_uneven": (lambda a: np.sum(np.array_split(a, 3, axis=1)[0] ** 2) + np.sum(np.array_split(a, 3, 1)[2] ** 3), A_),
+            "vsplit": (lambda q: np.sum(np.vsplit(q, 2)[1] * W44[:2]), Q_),
+            "hsplit": (lambda q: np.sum(np.hsplit(q, 2)[0] ** 2), Q_),
+            "dsplit": (lambda t: np.sum(np.dsplit(t, 2)[1] ** 2 * W34[:, :2]), T_),
+            "rollaxis": (lambda t: np.sum(np.rollaxis(t, 2) * W34.T[:, None, :]), T_),
+            "rollaxis_to_end": (lambda t: np.sum(np.rollaxis(t, 0, 3) ** 2 * W34[:, :, None]), T_),
+            "diff": (lambda a: np.sum(np.diff(a) ** 2), A_),
+            "diff_twice_axis0": (lambda q: np.sum(np.diff(q, n=2, axis=0) * W44[:2]), Q_),
+            "diff_vector_thrice": (lambda q: np.sum(np.diff(q[0], 3) ** 2), Q_),
+            "cross_first": (lambda t: np.sum(np.cross(t[0].T, C_[0][:1] * 2.0) ** 2), T_),
+            "cross_second": (lambda t: np.sum(np.cross(C_[1][None, :, :], t[:, :, :3]) ** 2), T_),
+            "cross_axis": (lambda a: np.sum(np.cross(a, W34, axis=0) * Y_), A_),
+            "sinc": (lambda a: np.sum(np.sinc(a) * W34), A_),
+            "logaddexp2_array": (lambda a: np.sum(np.logaddexp2(a, Y_) * W34), A_),
+            "logaddexp2_scalar": (lambda a: np.sum(np.logaddexp2(a, 0.5) ** 2), A_),
+            "logaddexp2_second_arg": (lambda a: np.sum(np.logaddexp2(Y_ * 3.0, a) * W34), A_),
             "real_conj": (lambda a: np.sum(np.real(a) * np.conj(a) * 2.0), A_),
         }
         for name, (f, x) in table.items():

@@ -774,3 +774,80 @@ def test_array_functions_on_views_and_copies_are_bit_exact(dnp, dtype):
     close(dnp.inner(V, V).numpy(), onp.asarray(onp.inner(v, v)), RT[dtype])
     close(dnp.inner(T, V).numpy(), onp.inner(t, v), RT[dtype])
     same(dnp.inner(A, 2.0), onp.inner(a, dtype(2.0)))
+
+
+@pytest.mark.parametrize("dtype", [F32, F64])
+def test_reversals_running_sums_and_pieces_are_bit_exact(dnp, dtype):
+    import autograd_amd as ag
+
+    rs = onp.random.RandomState(33)
+    a, q, t = (rs.randn(*s).astype(dtype) for s in ((5, 7), (6, 6), (3, 5, 7)))
+    A, Q, T = (P(dnp, h) for h in (a, q, t))
+
+    def same(got, want):
+        got = got.numpy()
+        assert got.shape == want.shape and got.dtype == want.dtype, (got.shape, want.shape, got.dtype, want.dtype)
+        assert onp.array_equal(got, want)
+
+    # slices that step backwards: one gather per reversed axis on top of the forward-stepping view
+    for idx in ((slice(None, None, -1),), (slice(None), slice(None, None, -2)), (slice(3, 0, -1), slice(None, None, -1)),
+                (Ellipsis, slice(None, None, -1)), (1, None, slice(None, None, -1)), (slice(-2, None, -1),),
+                (slice(0, 3, -1),), (slice(None, None, -3), 2), (slice(10, -10, -1), slice(5, 1, -2))):
+        same(T[idx], t[idx])
+        same(A[idx[:2]] if Ellipsis not in idx and None not in idx else A[idx], a[idx[:2]] if Ellipsis not in idx and None not in idx else a[idx])
+    w = rs.randn(3, 5, 7).astype(dtype)
+    got = ag.grad(lambda x: dnp.sum(x[::-1, 1:4, ::-2] * P(dnp, w[:, 1:4, ::2])))(T).numpy()
+    want = onp.zeros_like(t)
+    want[::-1, 1:4, ::-2] = w[:, 1:4, ::2]
+    assert onp.array_equal(got, want)
+    same(dnp.flipud(A), onp.flipud(a))
+    same(dnp.fliplr(T), onp.fliplr(t))
+    same(dnp.flip(T), onp.flip(t))
+    same(dnp.flip(T, (0, 2)), onp.flip(t, (0, 2)))
+    same(dnp.flip(A.T, 1), onp.flip(a.T, 1))
+    for k in range(-3, 5):
+        same(dnp.rot90(A, k), onp.rot90(a, k))
+        same(dnp.rot90(T, k, axes=(2, 0)), onp.rot90(t, k, axes=(2, 0)))
+    # running sums: every layout path of both kernels, ragged against the 64-wide tiles
+    for shape, axis in (((1000,), 0), ((130, 4100), 1), ((130, 4100), 0), ((7, 300, 65), 1), ((7, 300, 65), 2),
+                        ((7, 300, 65), None), ((5, 7), -1), ((1, 1), 0), ((64, 64), 1), ((65, 129), -1), ((3, 0, 4), 1)):
+        x = rs.randn(*shape).astype(dtype)
+        if x.size:
+            x.flat[0] = -0.0
+        same(dnp.cumsum(P(dnp, x), axis=axis), onp.cumsum(x, axis=axis))
+    same(dnp.cumsum(Q.T, axis=1), onp.cumsum(q.T, axis=1))  # a transposed view is copied first
+    big = (rs.randn(300, 5000) * 1e3).astype(dtype)
+    same(dnp.cumsum(P(dnp, big), axis=1), onp.cumsum(big, axis=1))
+    # pieces are views of the operand
+    for fn, args in (("split", (2, 0)), ("split", ([1, 4], 1)), ("array_split", (4, 1)), ("array_split", ([2, 2, 9], 1)),
+                     ("vsplit", (3,)), ("hsplit", ([1, 2],)), ("split", ([-2], 1))):
+        got, want = getattr(dnp, fn)(Q, *args), getattr(onp, fn)(q, *args)
+        assert len(got) == len(want)
+        for g_, w_ in zip(got, want):
+            same(g_, w_)
+    for g_, w_ in zip(dnp.dsplit(T, [3]), onp.dsplit(t, [3])):
+        same(g_, w_)
+    with pytest.raises(ValueError):
+        dnp.split(A, 2, axis=1)
+    for n_, axis in ((1, -1), (2, 0), (3, 1), (0, 0), (7, 1)):
+        same(dnp.diff(A, n_, axis), onp.diff(a, n_, axis))
+    for axis, start in ((2, 0), (0, 3), (1, 1), (-1, 1), (0, -1)):
+        same(dnp.rollaxis(T, axis, start), onp.rollaxis(t, axis, start))
+    u, v = rs.randn(4, 3).astype(dtype), rs.randn(4, 3).astype(dtype)
+    same(dnp.cross(P(dnp, u), P(dnp, v)), onp.cross(u, v))
+    same(dnp.cross(P(dnp, u.T), P(dnp, v[0]), axisa=0), onp.cross(u.T, v[0], axisa=0))
+    same(dnp.cross(P(dnp, u.T), P(dnp, v.T), axis=0), onp.cross(u.T, v.T, axis=0))
+    z = a.copy()
+    z[0, 0] = 0.0
+    close(dnp.sinc(P(dnp, z)).numpy(), onp.sinc(z), RT_EW[dtype] * 8)
+    assert dnp.sinc(P(dnp, z)).numpy()[0, 0] == 1.0
+    b = rs.randn(5, 7).astype(dtype)
+    b[0, :3] = a[0, :3]
+    a2 = a.copy()
+    a2[1, :3], b[1, :3] = [onp.inf, -onp.inf, onp.nan], [onp.inf, 1.0, 1.0]
+    with onp.errstate(all="ignore"):
+        for x in (a2, a2 * 50):
+            got, want = dnp.logaddexp2(P(dnp, x), P(dnp, b)).numpy(), onp.logaddexp2(x, b)
+            special = ~onp.isfinite(want)
+            assert onp.array_equal(got[special], want[special], equal_nan=True)
+            close(got[~special], want[~special], RT_EW[dtype] * 8)

@@ -67,8 +67,18 @@ def test_index_classification():
     assert W._is_basic_index(onp.int64(2))
     assert not W._is_basic_index([0, 1])
     assert not W._is_basic_index((slice(None), onp.array([0, 1])))
-    with pytest.raises(NotImplementedError):
-        W._is_basic_index(slice(None, None, -1))
+    assert W._is_basic_index(slice(None, None, -1))
+    # slices that step backwards become the forward-stepping slice over the same elements + the result axes to reverse
+    for shape, idx in (((5,), (slice(None, None, -1),)), ((5, 6), (slice(3, 0, -1), slice(None, None, -2))),
+                       ((4, 5, 6), (Ellipsis, slice(4, None, -3))), ((4, 5, 6), (1, None, slice(None, None, -1))),
+                       ((5,), (slice(0, 3, -1),)), ((4, 5, 6), (slice(None, None, 2), slice(10, -10, -1)))):
+        up, axes = W._positive_steps(idx, shape)
+        x = onp.arange(int(onp.prod(shape))).reshape(shape)
+        assert all(not isinstance(i, slice) or i.step is None or i.step > 0 for i in up)
+        assert onp.array_equal(onp.flip(x[up], axes) if axes else x[up], x[idx]), (shape, idx)
+    assert W._positive_steps((slice(1, 3), 2), (5, 6)) == ((slice(1, 3), 2), ())
+    with pytest.raises(IndexError):
+        W._positive_steps((0, 0, slice(None, None, -1)), (5, 6))
     assert onp.array_equal(W._host_index([0, 2, 0]), [0, 2, 0])
     assert onp.array_equal(W._host_index(onp.array([True, False, True])), [0, 2])
     assert W._host_index([]).dtype == onp.int64 and W._host_index([]).size == 0
