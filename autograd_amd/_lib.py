@@ -164,6 +164,10 @@ def lib():
                             c_i64, c_d, c_p, c_i64, c_i64, c_p, c_sz, c_p]
     L.agmi_fill.restype = c_i
     L.agmi_fill.argtypes = [c_i, c_p, c_i64, c_d, c_p]
+    L.agmi_reverse.restype = c_i
+    L.agmi_reverse.argtypes = [c_i, c_p, c_i64, c_i64, c_i64, c_p, c_p]
+    L.agmi_triangle.restype = c_i
+    L.agmi_triangle.argtypes = [c_i, c_p, c_i64, c_i64, c_i64, c_i64, c_i, c_p, c_p]
     L.agmi_cumsum.restype = c_i
     L.agmi_cumsum.argtypes = [c_i, c_p, c_i64, c_i64, c_i64, c_p, c_p]
     L.agmi_take_rows.restype = c_i
@@ -180,7 +184,7 @@ def lib():
 
 EXPORTS = (
     "agmi_last_error agmi_version agmi_last_kernel agmi_elementwise agmi_compare agmi_cast agmi_map_reduce "
-    "agmi_map_reduce_workspace_bytes agmi_gemm agmi_fill agmi_take_rows agmi_cumsum agmi_scatter_add_rows agmi_optimizer_step "
+    "agmi_map_reduce_workspace_bytes agmi_gemm agmi_fill agmi_take_rows agmi_cumsum agmi_reverse agmi_triangle agmi_scatter_add_rows agmi_optimizer_step "
     "agmi_correlate"
 ).split()
 
@@ -468,6 +472,15 @@ def fill(code, t, value):
 def take_rows(code, src, n_rows, inner, index, n_index, out):
     _check(_LIB.agmi_take_rows(code, src.data_ptr(), n_rows, inner, index.data_ptr(), n_index, out.data_ptr(),
                                _stream()), "agmi_take_rows")
+
+
+def reverse(code, src, outer, n, inner, out):
+    _check(_LIB.agmi_reverse(code, src.data_ptr(), outer, n, inner, out.data_ptr(), _stream()), "agmi_reverse")
+
+
+def triangle(code, src, batch, rows, cols, k, lower, out):
+    _check(_LIB.agmi_triangle(code, src.data_ptr(), batch, rows, cols, k, 1 if lower else 0, out.data_ptr(), _stream()),
+           "agmi_triangle")
 
 
 def cumsum(code, src, outer, n, inner, out):

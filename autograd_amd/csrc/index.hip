@@ -91,6 +91,31 @@ __global__ __launch_bounds__(kScanTile) void cumsum_rows(const T *__restrict__ s
     }
 }
 
+// out[o, k, c] = src[o, n - 1 - k, c] on contiguous (outer, n, inner) arrays: the copy behind a slice
+// that steps backwards (device views cannot carry negative strides).
+template <typename T>
+__global__ __launch_bounds__(kBlock) void reverse_axis_kernel(const T *__restrict__ src, int64_t total, int64_t n,
+                                                              int64_t inner, T *__restrict__ out) {
+    const int64_t e = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (e >= total) return;
+    const int64_t line = e / inner, c = e - line * inner;
+    const int64_t o = line / n, k = line - o * n;
+    out[e] = src[(o * n + (n - 1 - k)) * inner + c];
+}
+
+// out[b, i, j] = src[b, i, j] where j - i <= k (lower) or j - i >= k (upper), else 0: numpy.tril / triu on
+// contiguous (batch, rows, cols) arrays.  Masked entries are zeros whatever the source holds (NaN included).
+template <typename T>
+__global__ __launch_bounds__(kBlock) void triangle_kernel(const T *__restrict__ src, int64_t total, int64_t rows,
+                                                          int64_t cols, int64_t k, int lower, T *__restrict__ out) {
+    const int64_t e = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (e >= total) return;
+    const int64_t line = e / cols, j = e - line * cols;
+    const int64_t i = line % rows;
+    const bool keep = lower ? (j - i <= k) : (j - i >= k);
+    out[e] = keep ? src[e] : T(0);
+}
+
 }  // namespace agmi
 
 using namespace agmi;
@@ -201,4 +226,68 @@ extern "C" int agmi_cumsum(int dtype, const void *src, int64_t outer, int64_t n,
                                static_cast<const double *>(src), outer, n, inner, static_cast<double *>(out));
     }
     return hip_check(hipGetLastError(), "cumsum launch");
+}
+
+namespace {
+
+// shared argument checks of the two copy-shaped entry points below; returns the block count or a negative error
+int64_t plan_copy(const char *what, int dtype, const void *src, const void *out, int64_t total) {
+    if (!src || !out) {
+        set_error("%s: null operand", what);
+        return AGMI_ERR_ARG;
+    }
+    if (dtype != AGMI_F32 && dtype != AGMI_F64) {
+        set_error("%s: dtype %d is not a floating type", what, dtype);
+        return AGMI_ERR_ARG;
+    }
+    const int64_t blocks = ceil_div(total, kBlock);
+    if (blocks > 0x7fffffffLL) {
+        set_error("%s: too many elements", what);
+        return AGMI_ERR_UNSUPPORTED;
+    }
+    return blocks;
+}
+
+}  // namespace
+
+extern "C" int agmi_reverse(int dtype, const void *src, int64_t outer, int64_t n, int64_t inner, void *out,
+                            void *stream) {
+    if (outer < 0 || n < 0 || inner < 0) {
+        set_error("reverse: negative extent");
+        return AGMI_ERR_ARG;
+    }
+    const int64_t total = outer * n * inner;
+    if (total == 0) return 0;
+    const int64_t blocks = plan_copy("reverse", dtype, src, out, total);
+    if (blocks < 0) return static_cast<int>(blocks);
+    hipStream_t s = as_stream(stream);
+    set_kernel_name("reverse_axis_kernel");
+    if (dtype == AGMI_F32)
+        hipLaunchKernelGGL(reverse_axis_kernel<float>, dim3((unsigned)blocks), dim3(kBlock), 0, s,
+                           static_cast<const float *>(src), total, n, inner, static_cast<float *>(out));
+    else
+        hipLaunchKernelGGL(reverse_axis_kernel<double>, dim3((unsigned)blocks), dim3(kBlock), 0, s,
+                           static_cast<const double *>(src), total, n, inner, static_cast<double *>(out));
+    return hip_check(hipGetLastError(), "reverse launch");
+}
+
+extern "C" int agmi_triangle(int dtype, const void *src, int64_t batch, int64_t rows, int64_t cols, int64_t k,
+                             int lower, void *out, void *stream) {
+    if (batch < 0 || rows < 0 || cols < 0) {
+        set_error("triangle: negative extent");
+        return AGMI_ERR_ARG;
+    }
+    const int64_t total = batch * rows * cols;
+    if (total == 0) return 0;
+    const int64_t blocks = plan_copy("triangle", dtype, src, out, total);
+    if (blocks < 0) return static_cast<int>(blocks);
+    hipStream_t s = as_stream(stream);
+    set_kernel_name("triangle_kernel");
+    if (dtype == AGMI_F32)
+        hipLaunchKernelGGL(triangle_kernel<float>, dim3((unsigned)blocks), dim3(kBlock), 0, s,
+                           static_cast<const float *>(src), total, rows, cols, k, lower, static_cast<float *>(out));
+    else
+        hipLaunchKernelGGL(triangle_kernel<double>, dim3((unsigned)blocks), dim3(kBlock), 0, s,
+                           static_cast<const double *>(src), total, rows, cols, k, lower, static_cast<double *>(out));
+    return hip_check(hipGetLastError(), "triangle launch");
 }

@@ -626,11 +626,8 @@ def _positive_steps(idx, shape):
     return tuple(up), tuple(axes)
 
 
-_REVERSED_ROWS = {}
-
-
 def _reverse_axes(x, axes):
-    """``x`` reversed along ``axes`` (a new contiguous array): the row gather with a cached descending index."""
+    """``x`` reversed along ``axes`` (a new contiguous array), one copy kernel per axis."""
     for axis in axes:
         n = x.shape[axis]
         if n <= 1 or x.size == 0:
@@ -638,13 +635,9 @@ def _reverse_axes(x, axes):
         if x.dtype not in D._FLOATS:
             raise NotImplementedError("reversal of non-floating arrays")
         outer, inner = int(onp.prod(x.shape[:axis], dtype=onp.int64)), int(onp.prod(x.shape[axis + 1 :], dtype=onp.int64))
-        index = _REVERSED_ROWS.get((outer, n))
-        if index is None:
-            host = (onp.arange(outer, dtype=onp.int64)[:, None] * n + onp.arange(n - 1, -1, -1, dtype=onp.int64)).ravel()
-            index = _REVERSED_ROWS[(outer, n)] = D.from_numpy(host)
         src = D.contiguous(D.plain(x))
         out = D.empty(x.shape, x.dtype)
-        _lib.take_rows(_lib.DTYPE_CODE[x.dtype], src._t, outer * n, inner, index._t, outer * n, out._t)
+        _lib.reverse(_lib.DTYPE_CODE[x.dtype], src._t, outer, n, inner, out._t)
         x = out
     return x
 
@@ -1146,23 +1139,18 @@ def trace(x, offset=0):
     return sum.fun(diagonal.fun(x, offset), axis=-1)
 
 
-_TRIANGLES = {}
-
-
 def _triangle(x, k, lower):
     x = D.asarray(x)
     if x.ndim < 2:
         x = D.asarray(broadcast_to.fun(x, (x.shape[0] if x.ndim else 1,) * 2))
-    n, m = x.shape[-2:]
-    dt = x.dtype if x.dtype in D._FLOATS else onp.dtype(onp.float64)
-    key = (n, m, int(k), dt, lower)
-    keep = _TRIANGLES.get(key)
-    if keep is None:
-        tri = onp.tri(n, m, k if lower else k - 1, dtype=bool)
-        keep = _TRIANGLES[key] = D.from_numpy((tri if lower else ~tri).astype(dt))
     if x.dtype not in D._FLOATS:
         raise NotImplementedError("tril/triu: floating-point arrays only on the device")
-    return D.map_op(Op.WHERE, dt, keep, x, 0.0)
+    rows, cols = x.shape[-2:]
+    src = D.contiguous(D.plain(x))
+    out = D.empty(x.shape, x.dtype)
+    _lib.triangle(_lib.DTYPE_CODE[x.dtype], src._t, int(onp.prod(x.shape[:-2], dtype=onp.int64)), rows, cols, int(k), lower,
+                  out._t)
+    return out
 
 
 tril = _wrap(lambda x, k=0: _triangle(x, k, True), "tril")

@@ -230,6 +230,18 @@ int agmi_fill(int dtype, void *ptr, int64_t n, double value, void *stream);
 int agmi_take_rows(int dtype, const void *src, int64_t n_rows, int64_t inner,
                    const int64_t *index, int64_t n_index, void *out, void *stream);
 
+/* out[o, k, c] = src[o, n-1-k, c] on contiguous (outer, n, inner) arrays: numpy.flipud / fliplr / rot90
+ * (numpy_vjps.py:202-204) and slices that step backwards, A[::-1] (numpy_boxes.py:16-18), whose
+ * NumPy form is a view with a negative stride.  src and out must not overlap. */
+int agmi_reverse(int dtype, const void *src, int64_t outer, int64_t n, int64_t inner, void *out,
+                 void *stream);
+
+/* numpy.tril (lower != 0) / numpy.triu (lower == 0) with diagonal offset k on contiguous
+ * (batch, rows, cols) arrays (numpy_vjps.py:212-213): entries on the other side are written as
+ * zeros.  src and out may be the same buffer. */
+int agmi_triangle(int dtype, const void *src, int64_t batch, int64_t rows, int64_t cols, int64_t k,
+                  int lower, void *out, void *stream);
+
 /* Running sums along the middle axis of a contiguous (outer, n, inner) array:
  * out[o, k, c] = src[o, 0, c] + ... + src[o, k, c], added in that order (bit-identical to
  * numpy.cumsum).  Forward of numpy.cumsum and, on reversed operands, its cotangent
