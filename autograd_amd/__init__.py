@@ -9,30 +9,16 @@ derivative rules launch hand-written HIP kernels.
     from autograd_amd import grad, elementwise_grad, make_hvp
 """
 
+from . import differential_operators as _operators
 from .builtins import dict, isinstance, list, tuple, type  # noqa: A004,F401
-from .differential_operators import (  # noqa: F401
-    checkpoint,
-    deriv,
-    elementwise_grad,
-    grad,
-    grad_and_aux,
-    grad_named,
-    hessian,
-    hessian_tensor_product,
-    hessian_vector_product,
-    holomorphic_grad,
-    jacobian,
-    make_ggnvp,
-    make_hvp,
-    make_jvp,
-    make_jvp_reversemode,
-    make_vjp,
-    multigrad_dict,
-    tensor_jacobian_product,
-    value_and_grad,
-    vector_jacobian_product,
-)
 from .extend import primitive  # noqa: F401
 from .graphs import capture  # noqa: F401
+
+# the differential operators of autograd/__init__.py:1-22, under the same names
+_OPERATORS = ("grad elementwise_grad value_and_grad grad_and_aux grad_named multigrad_dict deriv holomorphic_grad "
+              "jacobian hessian make_vjp make_jvp make_jvp_reversemode make_hvp make_ggnvp hessian_tensor_product "
+              "hessian_vector_product tensor_jacobian_product vector_jacobian_product checkpoint").split()
+for _name in _OPERATORS:
+    globals()[_name] = getattr(_operators, _name)
 
 __version__ = "0.1.0"

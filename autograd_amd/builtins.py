@@ -1,50 +1,67 @@
 """Differentiable tuples, lists and dicts.
 
-Contract of the reference's autograd/builtins.py:24-286: containers are boxed
-(``SequenceBox``, ``DictBox``), indexing a boxed container is the primitive
-``container_take`` whose cotangent is the sparse object built by
-``container_untake``, and container vector spaces map the leaf vspaces over the
-structure.  Pure host-side bookkeeping; leaves do the arithmetic.
+Contract of the reference's autograd/builtins.py:24-286 (same names and behaviour): containers are
+boxed (``SequenceBox``, ``DictBox``); indexing a boxed container is the primitive
+``container_take``, whose cotangent is the scatter-form object built by ``container_untake``;
+container vector spaces apply the leaves' vector spaces across the structure.  Pure host-side
+bookkeeping: the leaves do the arithmetic.
 """
 
-from .extend import (
-    Box,
-    SparseObject,
-    VSpace,
-    defjvp,
-    defjvp_argnum,
-    defvjp,
-    defvjp_argnum,
-    notrace_primitive,
-    primitive,
-    vspace,
-)
+from .extend import Box, SparseObject, VSpace, defjvp, defjvp_argnum, defvjp, defvjp_argnum, notrace_primitive, primitive
+from .extend import vspace
 from .util import subvals
 
-isinstance_ = isinstance
-isinstance = notrace_primitive(isinstance)
+# the Python builtins this module shadows with traceable versions
+isinstance_, type_, tuple_, list_, dict_ = isinstance, type, tuple, list, dict
 
-type_ = type
-type = notrace_primitive(type)
+# type queries see through boxes and are never traced (builtins.py:18-22)
+isinstance = notrace_primitive(isinstance_)
+type = notrace_primitive(type_)
 
-tuple_, list_, dict_ = tuple, list, dict
 
-
+# ---- taking an element out of a container, and its cotangent (builtins.py:24-34, 99-109) ---------
 @primitive
 def container_take(A, idx):
     return A[idx]
 
 
+@primitive
+def container_untake(x, idx, vs):
+    """Cotangent of ``container_take``: a zero container with ``x`` added at ``idx``, in scatter form.
+
+    ``idx`` is a key / position, or a slice of a sequence (then ``x`` is the matching run of
+    elements).  The addition happens leaf by leaf with the leaf vspaces' ``_mut_add``; the container
+    itself is rebuilt with the entry replaced."""
+    leaf_spaces = vs.shape[idx]
+    if isinstance_(idx, slice):
+        merged = lambda old: [s._mut_add(o, new) for s, o, new in zip(leaf_spaces, old, x)]  # noqa: E731
+    else:
+        merged = lambda old: leaf_spaces._mut_add(old, x)  # noqa: E731
+    return SparseObject(vs, lambda A: vs._subval(A, idx, merged(A[idx])))
+
+
 defvjp(container_take, lambda ans, A, idx: lambda g: container_untake(g, idx, vspace(A)))
-defjvp(container_take, "same")
+defvjp(container_untake, lambda ans, x, idx, _: lambda g: container_take(g, idx))
+for _linear in (container_take, container_untake):
+    defjvp(_linear, "same")
 
 
-class SequenceBox(Box):
+# ---- boxes (builtins.py:37-96) -------------------------------------------------------------------
+class _ContainerBox(Box):
+    """What tuples, lists and dicts share when boxed: traced item access, untraced size and membership."""
+
     __slots__ = []
     __getitem__ = container_take
 
     def __len__(self):
         return len(self._value)
+
+    def __contains__(self, item):
+        return item in self._value
+
+
+class SequenceBox(_ContainerBox):
+    __slots__ = []
 
     def __add__(self, other):
         return sequence_extend_right(self, *other)
@@ -52,93 +69,48 @@ class SequenceBox(Box):
     def __radd__(self, other):
         return sequence_extend_left(self, *other)
 
-    def __contains__(self, elt):
-        return elt in self._value
-
-    def index(self, elt):
-        return self._value.index(elt)
+    def index(self, item):
+        return self._value.index(item)
 
 
-SequenceBox.register(tuple_)
-SequenceBox.register(list_)
+class DictBox(_ContainerBox):
+    """Keys are plain values; every way of reaching a value goes through the traced item access."""
 
-
-class DictBox(Box):
     __slots__ = []
-    __getitem__ = container_take
-
-    def __len__(self):
-        return len(self._value)
 
     def __iter__(self):
         return iter(self._value)
 
-    def __contains__(self, elt):
-        return elt in self._value
-
-    def iterkeys(self):
-        return iter(self)
+    iterkeys = __iter__
 
     def itervalues(self):
-        return (self[k] for k in self)
+        return (self[key] for key in self._value)
 
     def iteritems(self):
-        return ((k, self[k]) for k in self)
+        return ((key, self[key]) for key in self._value)
 
     def keys(self):
-        return list(self.iterkeys())
+        return list_(self._value)
 
     def values(self):
-        return list(self.itervalues())
+        return list_(self.itervalues())
 
     def items(self):
-        return list(self.iteritems())
+        return list_(self.iteritems())
 
     def get(self, k, d=None):
-        return self[k] if k in self else d
+        return self[k] if k in self._value else d
 
 
+for _seq in (tuple_, list_):
+    SequenceBox.register(_seq)
 DictBox.register(dict_)
 
 
-@primitive
-def container_untake(x, idx, vs):
-    """Cotangent of ``container_take``: add ``x`` into leaf (or slice) ``idx``.
-
-    The leaf update uses the leaf vspace's ``_mut_add`` and the container is
-    rebuilt with that one entry replaced (reference builtins.py:99-109).
-    """
-    if isinstance_(idx, slice):
-
-        def accum(current):
-            return [leaf_vs._mut_add(a, b) for leaf_vs, a, b in zip(vs.shape[idx], current, x)]
-
-    else:
-
-        def accum(current):
-            return vs.shape[idx]._mut_add(current, x)
-
-    def mut_add(A):
-        return vs._subval(A, idx, accum(A[idx]))
-
-    return SparseObject(vs, mut_add)
-
-
-defvjp(container_untake, lambda ans, x, idx, _: lambda g: container_take(g, idx))
-defjvp(container_untake, "same")
-
-
+# ---- building containers out of (possibly boxed) elements (builtins.py:112-195) -------------------
 @primitive
 def sequence_extend_right(seq, *elts):
     return seq + type_(seq)(elts)
-
-
-def _grad_sequence_extend_right(argnum, ans, args, kwargs):
-    n = len(args[0])
-    return lambda g: g[:n] if argnum == 0 else g[n + argnum - 1]
-
-
-defvjp_argnum(sequence_extend_right, _grad_sequence_extend_right)
 
 
 @primitive
@@ -146,63 +118,9 @@ def sequence_extend_left(seq, *elts):
     return type_(seq)(elts) + seq
 
 
-def _grad_sequence_extend_left(argnum, ans, args, kwargs):
-    n_new = len(args) - 1
-    return lambda g: g[n_new:] if argnum == 0 else g[argnum - 1]
-
-
-defvjp_argnum(sequence_extend_left, _grad_sequence_extend_left)
-
-
 @primitive
 def make_sequence(seq_type, *args):
     return seq_type(args)
-
-
-defvjp_argnum(make_sequence, lambda argnum, *args: lambda g: g[argnum - 1])
-defjvp_argnum(
-    make_sequence,
-    lambda argnum, g, ans, args, kwargs: container_untake(g, argnum - 1, vspace(ans)),
-)
-
-
-class _TupleMeta(type_(tuple_)):
-    def __instancecheck__(self, instance):
-        return isinstance_(instance, tuple_)
-
-
-class tuple(tuple_, metaclass=_TupleMeta):
-    """``tuple(xs)`` that keeps boxed elements traceable."""
-
-    def __new__(cls, xs):
-        return make_sequence(tuple_, *xs)
-
-
-class _ListMeta(type_):
-    def __instancecheck__(self, instance):
-        return isinstance_(instance, list_)
-
-
-class list(list_, metaclass=_ListMeta):
-    """``list(xs)`` that keeps boxed elements traceable."""
-
-    def __new__(cls, xs):
-        return make_sequence(list_, *xs)
-
-
-class _DictMeta(type_):
-    def __instancecheck__(self, instance):
-        return isinstance_(instance, dict_)
-
-
-class dict(dict_, metaclass=_DictMeta):
-    """``dict(...)`` that keeps boxed values traceable."""
-
-    def __new__(cls, *args, **kwargs):
-        result = dict_(*args, **kwargs)
-        if result:
-            return _make_dict(result.keys(), list(result.values()))
-        return result
 
 
 @primitive
@@ -210,63 +128,130 @@ def _make_dict(keys, vals):
     return dict_(zip(keys, vals))
 
 
+def _cotangent_of_extend_right(argnum, ans, args, kwargs):
+    # argument 0 is the sequence (the head of the result), argument k > 0 its k-th appended element
+    head = len(args[0])
+    if argnum == 0:
+        return lambda g: g[:head]
+    return lambda g: g[head + argnum - 1]
+
+
+def _cotangent_of_extend_left(argnum, ans, args, kwargs):
+    # the new elements come first, the sequence (argument 0) is the tail
+    n_new = len(args) - 1
+    if argnum == 0:
+        return lambda g: g[n_new:]
+    return lambda g: g[argnum - 1]
+
+
+defvjp_argnum(sequence_extend_right, _cotangent_of_extend_right)
+defvjp_argnum(sequence_extend_left, _cotangent_of_extend_left)
+defvjp_argnum(make_sequence, lambda argnum, *args: lambda g: g[argnum - 1])
+defjvp_argnum(make_sequence, lambda argnum, g, ans, args, kwargs: container_untake(g, argnum - 1, vspace(ans)))
 defvjp(_make_dict, lambda ans, keys, vals: lambda g: list(g[key] for key in keys), argnums=(1,))
 
 
+def _looks_like(builtin):
+    """Metaclass making ``isinstance(x, traced_type)`` answer for the builtin it stands in for."""
+
+    class Meta(type_(builtin)):
+        def __instancecheck__(cls, instance):
+            return isinstance_(instance, builtin)
+
+    return Meta
+
+
+class tuple(tuple_, metaclass=_looks_like(tuple_)):
+    """``tuple(xs)`` that keeps boxed elements traceable."""
+
+    def __new__(cls, xs):
+        return make_sequence(tuple_, *xs)
+
+
+class list(list_, metaclass=_looks_like(list_)):
+    """``list(xs)`` that keeps boxed elements traceable."""
+
+    def __new__(cls, xs):
+        return make_sequence(list_, *xs)
+
+
+class dict(dict_, metaclass=_looks_like(dict_)):
+    """``dict(...)`` that keeps boxed values traceable."""
+
+    def __new__(cls, *args, **kwargs):
+        plain = dict_(*args, **kwargs)
+        return _make_dict(plain.keys(), list(plain.values())) if plain else plain
+
+
+# ---- vector spaces (builtins.py:198-286) ----------------------------------------------------------
 class ContainerVSpace(VSpace):
-    """Vspace of a container: ``self.shape`` holds the container of leaf vspaces."""
+    """Vspace of a container: ``self.shape`` is the same container holding the leaves' vspaces.
+
+    Subclasses say how to walk and rebuild their kind of container: ``_values``, ``_kv_pairs``,
+    ``_map(f, *containers)`` (``f`` gets the leaf vspace first) and ``_subval(xs, key, x)``."""
 
     def __init__(self, value):
-        self.shape = value
+        self.shape = value  # _map walks self.shape: first the values themselves, then their vspaces
         self.shape = self._map(vspace)
+
+    def _leafwise(self, method, *containers, extra=()):
+        return self._map(lambda leaf_vs, *leaves: getattr(leaf_vs, method)(*leaves, *extra), *containers)
+
+    def _total(self, per_leaf):
+        return sum(self._values(per_leaf))
 
     @property
     def size(self):
-        return sum(self._values(self._map(lambda vs: vs.size)))
+        return self._total(self._map(lambda leaf_vs: leaf_vs.size))
 
     def zeros(self):
-        return self._map(lambda vs: vs.zeros())
+        return self._leafwise("zeros")
 
     def ones(self):
-        return self._map(lambda vs: vs.ones())
+        return self._leafwise("ones")
 
     def randn(self):
-        return self._map(lambda vs: vs.randn())
+        return self._leafwise("randn")
 
     def standard_basis(self):
-        zero = self.zeros()
+        origin = self.zeros()
         for key, leaf_vs in self._kv_pairs(self.shape):
-            for basis_vector in leaf_vs.standard_basis():
-                yield self._subval(zero, key, basis_vector)
+            for unit in leaf_vs.standard_basis():
+                yield self._subval(origin, key, unit)
 
     def _add(self, xs, ys):
-        return self._map(lambda vs, x, y: vs._add(x, y), xs, ys)
+        return self._leafwise("_add", xs, ys)
 
     def _mut_add(self, xs, ys):
-        return self._map(lambda vs, x, y: vs._mut_add(x, y), xs, ys)
+        return self._leafwise("_mut_add", xs, ys)
 
     def _scalar_mul(self, xs, a):
-        return self._map(lambda vs, x: vs._scalar_mul(x, a), xs)
-
-    def _inner_prod(self, xs, ys):
-        return sum(self._values(self._map(lambda vs, x, y: vs._inner_prod(x, y), xs, ys)))
+        return self._leafwise("_scalar_mul", xs, extra=(a,))
 
     def _covector(self, xs):
-        return self._map(lambda vs, x: vs._covector(x), xs)
+        return self._leafwise("_covector", xs)
+
+    def _inner_prod(self, xs, ys):
+        return self._total(self._leafwise("_inner_prod", xs, ys))
 
 
 class SequenceVSpace(ContainerVSpace):
+    seq_type = None  # set by the concrete classes
+
     def _values(self, x):
         return x
 
     def _kv_pairs(self, x):
         return enumerate(x)
 
+    def _build(self, items):
+        return self.seq_type(items)
+
     def _map(self, f, *args):
-        return self.seq_type(map(f, self.shape, *args))
+        return self._build(map(f, self.shape, *args))
 
     def _subval(self, xs, idx, x):
-        return self.seq_type(subvals(xs, [(idx, x)]))
+        return self._build(subvals(xs, [(idx, x)]))
 
 
 class ListVSpace(SequenceVSpace):
@@ -277,6 +262,13 @@ class TupleVSpace(SequenceVSpace):
     seq_type = tuple_
 
 
+class NamedTupleVSpace(SequenceVSpace):
+    """For namedtuple types (a subclass sets ``seq_type``): built from positional fields."""
+
+    def _build(self, items):
+        return self.seq_type(*items)
+
+
 class DictVSpace(ContainerVSpace):
     def _values(self, x):
         return x.values()
@@ -285,22 +277,14 @@ class DictVSpace(ContainerVSpace):
         return x.items()
 
     def _map(self, f, *args):
-        return {k: f(vs, *[x[k] for x in args]) for k, vs in self.shape.items()}
+        return {key: f(leaf_vs, *(x[key] for x in args)) for key, leaf_vs in self.shape.items()}
 
     def _subval(self, xs, idx, x):
-        d = dict_(xs.items())
-        d[idx] = x
-        return d
+        out = dict_(xs)
+        out[idx] = x
+        return out
 
 
 ListVSpace.register(list_)
 TupleVSpace.register(tuple_)
 DictVSpace.register(dict_)
-
-
-class NamedTupleVSpace(SequenceVSpace):
-    def _map(self, f, *args):
-        return self.seq_type(*map(f, self.shape, *args))
-
-    def _subval(self, xs, idx, x):
-        return self.seq_type(*subvals(xs, [(idx, x)]))

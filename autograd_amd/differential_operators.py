@@ -1,30 +1,32 @@
-"""User-facing differential operators, all thin closures over ``make_vjp`` / ``make_jvp``.
+"""User-facing differential operators: closures over ``make_vjp`` / ``make_jvp``.
 
-Same surface and semantics as the reference's
-autograd/differential_operators.py:19-242.  Nothing here touches array data
-directly: seeds come from the value's ``VSpace`` and every array operation goes
-through the device namespace (``autograd_amd.numpy``).
+Same surface and semantics as the reference's autograd/differential_operators.py:19-242 (names,
+argument meaning, error messages).  Nothing here touches array data directly: seeds come from the
+value's ``VSpace`` and every array operation goes through the value type's array namespace, by
+default the device namespace ``autograd_amd.numpy``.
+
+Operators decorated with ``unary_to_nary`` are written for a function of one argument and a point;
+the decorator makes them ``op(fun, argnum=0)(*args, **kwargs)`` for any argument position(s).
 """
 
+import inspect
 import warnings
-from inspect import getfullargspec as _getargspec
+from collections import OrderedDict
 
+from . import core
 from .builtins import tuple as atuple
-from .core import make_jvp as _make_jvp
-from .core import make_vjp as _make_vjp
 from .extend import defvjp_argnum, primitive, vspace
 from .wrap_util import unary_to_nary
 
-make_vjp = unary_to_nary(_make_vjp)
-make_jvp = unary_to_nary(_make_jvp)
+make_vjp = unary_to_nary(core.make_vjp)
+make_jvp = unary_to_nary(core.make_jvp)
 
 
 def _anp(*values):
     """Array namespace to use for ``values``.
 
-    A box class may name the namespace its value type lives in through a
-    ``_namespace`` attribute (a callable returning the module); the default is
-    the device namespace ``autograd_amd.numpy``.
+    A box class may name the namespace its value type lives in through a ``_namespace`` attribute
+    (a callable returning the module); the default is the device namespace ``autograd_amd.numpy``.
     """
     from .tracer import Box, getval
 
@@ -38,58 +40,65 @@ def _anp(*values):
     return anp
 
 
-_SCALAR_ONLY = (
-    "{name} only applies to real scalar-output functions. "
-    "Try jacobian, elementwise_grad or holomorphic_grad."
-)
+def _seeded_with_ones(fun, x, who=None):
+    """``(fun(x), cotangent of x for a cotangent of ones on fun(x))``.  With ``who`` given the output
+    has to be a single real number, and ``who`` is named in the error otherwise."""
+    pull_back, ans = core.make_vjp(fun, x)
+    out_space = vspace(ans)
+    if who is not None and out_space.size != 1:
+        raise TypeError(
+            f"{who} only applies to real scalar-output functions. "
+            "Try jacobian, elementwise_grad or holomorphic_grad."
+        )
+    return ans, pull_back(out_space.ones())
 
 
 @unary_to_nary
 def grad(fun, x):
-    """
-    Returns a function which computes the gradient of `fun` with respect to
-    positional argument number `argnum`. The returned function takes the same
-    arguments as `fun`, but returns the gradient instead. The function `fun`
-    should be scalar-valued. The gradient has the same type as the argument."""
-    vjp, ans = _make_vjp(fun, x)
-    if not vspace(ans).size == 1:
-        raise TypeError(_SCALAR_ONLY.format(name="Grad"))
-    return vjp(vspace(ans).ones())
+    """Gradient of a scalar-valued ``fun`` with respect to its argument number ``argnum``: a function
+    of the same arguments as ``fun`` whose result has the type and structure of that argument."""
+    return _seeded_with_ones(fun, x, "Grad")[1]
+
+
+@unary_to_nary
+def value_and_grad(fun, x):
+    """Like ``grad``, returning ``(fun's value, gradient)`` from the one forward pass."""
+    return _seeded_with_ones(fun, x, "value_and_grad")
 
 
 @unary_to_nary
 def elementwise_grad(fun, x):
-    """
-    Returns a function that computes the sum of each column of the Jacobian of
-    `fun`, in one pass. If the Jacobian is diagonal, then this is the diagonal
-    of the Jacobian.
-    """
-    vjp, ans = _make_vjp(fun, x)
-    if vspace(ans).iscomplex:
+    """Column sums of the Jacobian of ``fun`` in one backward pass (the cotangent seed is all ones);
+    for a function acting element by element this is its derivative at every element."""
+    pull_back, ans = core.make_vjp(fun, x)
+    out_space = vspace(ans)
+    if out_space.iscomplex:
         raise TypeError("Elementwise_grad only applies to real-output functions.")
-    return vjp(vspace(ans).ones())
+    return pull_back(out_space.ones())
 
 
 @unary_to_nary
 def deriv(fun, x):
-    return _make_jvp(fun, x)(vspace(x).ones())[1]
+    """Forward-mode derivative along the all-ones direction of the input."""
+    return core.make_jvp(fun, x)(vspace(x).ones())[1]
 
 
 @unary_to_nary
 def jacobian(fun, x):
-    """
-    Returns a function which computes the Jacobian of `fun` with respect to
-    positional argument number `argnum`, which must be a scalar or array. If the
-    input has shape (in1, in2, ...) and the output (out1, out2, ...), the
-    Jacobian has shape (out1, out2, ..., in1, in2, ...).  One VJP per output
-    element (reference differential_operators.py:57-73).
-    """
-    vjp, ans = _make_vjp(fun, x)
+    """Jacobian of an array-valued ``fun`` of an array (or scalar): output axes first, input axes
+    last.  One backward pass per output element, each seeded with a standard basis vector of the
+    output space (reference differential_operators.py:57-73)."""
+    pull_back, ans = core.make_vjp(fun, x)
     np = _anp(ans, x)
-    ans_vspace = vspace(ans)
-    jacobian_shape = ans_vspace.shape + vspace(x).shape
-    grads = map(vjp, ans_vspace.standard_basis())
-    return np.reshape(np.stack(grads), jacobian_shape)
+    out_space = vspace(ans)
+    rows = [pull_back(unit) for unit in out_space.standard_basis()]
+    return np.reshape(np.stack(rows), out_space.shape + vspace(x).shape)
+
+
+@unary_to_nary
+def hessian(fun, x):
+    """Exact Hessian: the Jacobian of the Jacobian (for scalar ``fun``, of the gradient)."""
+    return jacobian(jacobian(fun))(x)
 
 
 @unary_to_nary
@@ -97,145 +106,127 @@ def holomorphic_grad(fun, x):
     if not vspace(x).iscomplex:
         warnings.warn("Input to holomorphic_grad is not complex")
     np = _anp(x)
-    return grad(lambda x: np.real(fun(x)))(x)
+    return grad(lambda z: np.real(fun(z)))(x)
 
 
 def grad_named(fun, argname):
-    """Gradient with respect to a named argument (not *args / **kwargs)."""
-    return grad(fun, _getargspec(fun).args.index(argname))
-
-
-@unary_to_nary
-def hessian(fun, x):
-    "Returns a function that computes the exact Hessian."
-    return jacobian(jacobian(fun))(x)
+    """Gradient with respect to the positional argument called ``argname``."""
+    position = inspect.getfullargspec(fun).args.index(argname)
+    return grad(fun, position)
 
 
 @unary_to_nary
 def make_hvp(fun, x):
-    """Builds a function for evaluating the Hessian-vector product at a point:
-    the VJP of ``grad(fun)`` (reverse-over-reverse), so the forward pass is
-    shared between many products at the same point."""
-    return _make_vjp(grad(fun), x)
+    """``(hvp, gradient at x)`` where ``hvp(v)`` is the Hessian of ``fun`` at ``x`` times ``v``:
+    the VJP of ``grad(fun)`` (reverse over reverse), so one forward pass serves many products."""
+    return core.make_vjp(grad(fun), x)
+
+
+def _split_last(args):
+    return args[:-1], args[-1]
 
 
 def hessian_tensor_product(fun, argnum=0):
-    """Returns a function of (*args, tensor, **kwargs) giving the exact
-    Hessian-tensor product."""
-    fun_grad = grad(fun, argnum)
+    """Function of ``(*args, tensor, **kwargs)``: the Hessian of ``fun`` contracted with ``tensor``,
+    as the gradient of <grad fun, tensor> (no Hessian is formed)."""
+    first_derivative = grad(fun, argnum)
 
-    def vector_dot_grad(*args, **kwargs):
-        args, vector = args[:-1], args[-1]
-        np = _anp(vector)
-        return np.tensordot(fun_grad(*args, **kwargs), vector, np.ndim(vector))
+    def contracted_gradient(*args, **kwargs):
+        point, tensor = _split_last(args)
+        np = _anp(tensor)
+        return np.tensordot(first_derivative(*point, **kwargs), tensor, np.ndim(tensor))
 
-    return grad(vector_dot_grad, argnum)
-
-
-hessian_vector_product = hessian_tensor_product
+    return grad(contracted_gradient, argnum)
 
 
 def tensor_jacobian_product(fun, argnum=0):
-    """Returns a function of (*args, tensor, **kwargs) giving the Jacobian
-    left-multiplied by tensor."""
+    """Function of ``(*args, tensor, **kwargs)``: ``tensor`` contracted with the output axes of the
+    Jacobian of ``fun``."""
 
-    def vector_dot_fun(*args, **kwargs):
-        args, vector = args[:-1], args[-1]
-        np = _anp(vector)
-        return np.tensordot(vector, fun(*args, **kwargs), axes=np.ndim(vector))
+    def contracted_output(*args, **kwargs):
+        point, tensor = _split_last(args)
+        np = _anp(tensor)
+        return np.tensordot(tensor, fun(*point, **kwargs), axes=np.ndim(tensor))
 
-    return jacobian(vector_dot_fun, argnum)
+    return jacobian(contracted_output, argnum)
 
 
+hessian_vector_product = hessian_tensor_product
 vector_jacobian_product = tensor_jacobian_product
+
+
+def _transpose_of(linear_map, like):
+    """The VJP of a linear map (linear maps are their own derivative), seeded at zero."""
+    return core.make_vjp(linear_map, vspace(like).zeros())[0]
 
 
 @unary_to_nary
 def make_jvp_reversemode(fun, x):
-    """Jacobian-vector product built from two reverse passes (the VJP is linear
-    in its argument, so the VJP of the VJP is the JVP)."""
-    vjp, y = _make_vjp(fun, x)
-    vjp_vjp, _ = _make_vjp(vjp, vspace(y).zeros())
-    return vjp_vjp
+    """Jacobian-vector products from reverse mode only: the VJP is linear in its cotangent, so its
+    own VJP is multiplication by the Jacobian.  Pays off when many products are taken at one point."""
+    pull_back, y = core.make_vjp(fun, x)
+    return _transpose_of(pull_back, y)
 
 
 def make_ggnvp(f, g=None, f_argnum=0):
-    """Generalized-Gauss-Newton-vector products at a point."""
+    """Generalized Gauss-Newton vector products of ``g(f(x))`` at a point: ``v -> J' H_g J v``.
+    ``g`` defaults to half the squared norm along the last axis."""
     if g is None:
 
-        def g(x):
-            np = _anp(x)
-            return 1.0 / 2 * np.sum(x**2, axis=-1)
+        def g(y):
+            return 1.0 / 2 * _anp(y).sum(y**2, axis=-1)
 
     @unary_to_nary
-    def _make_ggnvp(f, x):
-        f_vjp, f_x = _make_vjp(f, x)
-        g_hvp, grad_g_x = _make_vjp(grad(g), f_x)
-        f_jvp, _ = _make_vjp(f_vjp, vspace(grad_g_x).zeros())
+    def at_point(f, x):
+        j_transposed, y = core.make_vjp(f, x)
+        hessian_of_g, dg = core.make_vjp(grad(g), y)
+        j = _transpose_of(j_transposed, dg)
+        return lambda v: j_transposed(hessian_of_g(j(v)))
 
-        def ggnvp(v):
-            return f_vjp(g_hvp(f_jvp(v)))
-
-        return ggnvp
-
-    return _make_ggnvp(f, f_argnum)
-
-
-@unary_to_nary
-def value_and_grad(fun, x):
-    """Returns a function that returns both value and gradient."""
-    vjp, ans = _make_vjp(fun, x)
-    if not vspace(ans).size == 1:
-        raise TypeError(_SCALAR_ONLY.format(name="value_and_grad"))
-    return ans, vjp(vspace(ans).ones())
+    return at_point(f, f_argnum)
 
 
 @unary_to_nary
 def grad_and_aux(fun, x):
-    """Gradient of the first output of a two-output function, plus the
-    (unmodified) second output."""
-    vjp, (ans, aux) = _make_vjp(lambda x: atuple(fun(x)), x)
-    return vjp((vspace(ans).ones(), vspace(aux).zeros())), aux
+    """For ``fun`` returning ``(value, aux)``: the gradient of ``value`` and ``aux`` as it is."""
+    pull_back, (ans, aux) = core.make_vjp(lambda arg: atuple(fun(arg)), x)
+    seed = (vspace(ans).ones(), vspace(aux).zeros())
+    return pull_back(seed), aux
 
 
 def multigrad_dict(fun):
-    "Takes gradients wrt all arguments simultaneously; returns {argname: grad}."
-    import inspect
-    from collections import OrderedDict
+    """Gradients with respect to all arguments at once, as an ordered ``{argument name: gradient}``;
+    ``*args`` / ``**kwargs`` of ``fun`` appear under their own names as a tuple / dict of gradients."""
+    signature = inspect.signature(fun)
+    kinds = {name: p.kind for name, p in signature.parameters.items()}
+    star = [n for n, k in kinds.items() if k == inspect.Parameter.VAR_POSITIONAL]
+    double_star = [n for n, k in kinds.items() if k == inspect.Parameter.VAR_KEYWORD]
+    named = [n for n in kinds if n not in star + double_star]
 
-    sig = inspect.signature(fun)
-    params = sig.parameters
-    var_pos = [n for n, p in params.items() if p.kind == p.VAR_POSITIONAL]
-    var_kwd = [n for n, p in params.items() if p.kind == p.VAR_KEYWORD]
-    plain = [n for n in params if n not in var_pos + var_kwd]
+    def call_with(values):
+        positional = tuple(values[n] for n in named)
+        if star:
+            positional += tuple(values[star[0]])
+        keywords = {k: values[double_star[0]][k] for k in values[double_star[0]]} if double_star else {}
+        return fun(*positional, **keywords)
 
     def gradfun(*args, **kwargs):
-        bound = sig.bind(*args, **kwargs)
-        argdict = OrderedDict()
-        for name, p in params.items():
-            if name in bound.arguments:
-                argdict[name] = bound.arguments[name]
+        given = signature.bind(*args, **kwargs).arguments
+        values = OrderedDict()
+        for name, p in signature.parameters.items():
+            if name in given:
+                values[name] = given[name]
             elif p.default is not p.empty:
-                argdict[name] = p.default
-
-        def newfun(dct):
-            pos = tuple(dct[n] for n in plain) + (tuple(dct[var_pos[0]]) if var_pos else ())
-            kw = {k: dct[var_kwd[0]][k] for k in dct[var_kwd[0]]} if var_kwd else {}
-            return fun(*pos, **kw)
-
-        grad_dict = grad(newfun)(dict(argdict))
-        return OrderedDict((name, grad_dict[name]) for name in argdict)
+                values[name] = p.default
+        gradients = grad(call_with)(dict(values))
+        return OrderedDict((name, gradients[name]) for name in values)
 
     return gradfun
 
 
 def checkpoint(fun):
-    """Gradient checkpointing: intermediate values of ``fun`` are dropped after
-    the forward pass and recomputed when its VJP is needed."""
-
-    def wrapped_grad(argnum, ans, args, kwargs):
-        return make_vjp(fun, argnum)(*args, **kwargs)[0]
-
-    wrapped = primitive(fun)
-    defvjp_argnum(wrapped, wrapped_grad)
-    return wrapped
+    """``fun`` as a primitive that keeps no intermediate values: its VJP traces ``fun`` again when
+    the backward pass gets there (memory for recomputation)."""
+    as_primitive = primitive(fun)
+    defvjp_argnum(as_primitive, lambda argnum, ans, args, kwargs: make_vjp(fun, argnum)(*args, **kwargs)[0])
+    return as_primitive

@@ -12,29 +12,40 @@ from autograd_amd import make_vjp
 from autograd_amd.builtins import type
 
 
-def flatten(value):
-    """Flattens any nesting of tuples, lists, or dicts, with device arrays or scalars inside.
-    Returns a 1-d device array and an unflatten function."""
-    unflatten, flat_value = make_vjp(_flatten)(value)
-    return flat_value, unflatten
+def _leaves_in_order(value):
+    """The leaves of ``value`` from left to right, each as a 1-d array (boxes stay boxes)."""
+    kind = type(value)  # sees through boxes
+    if kind is dict:
+        children = [value[key] for key in sorted(value)]
+    elif kind is list or kind is tuple:
+        children = value
+    else:
+        return [np.ravel(value)]
+    found = []
+    for child in children:
+        found.extend(_leaves_in_order(child))
+    # an empty container flattens to an empty float64 vector (and promotes its neighbours like one)
+    return found if found else [np.array([])]
 
 
 def _flatten(value):
-    t = type(value)
-    if t in (list, tuple):
-        return _concatenate(map(_flatten, value))
-    elif t is dict:
-        return _concatenate(_flatten(value[k]) for k in sorted(value))
-    else:
-        return np.ravel(value)
+    pieces = _leaves_in_order(value)
+    return pieces[0] if len(pieces) == 1 and type(value) not in (list, tuple, dict) else np.concatenate(pieces)
 
 
-def _concatenate(lst):
-    lst = list(lst)
-    return np.concatenate(lst) if lst else np.array([])
+def flatten(value):
+    """Flattens any nesting of tuples, lists, or dicts, with device arrays or scalars inside.
+    Returns a 1-d device array and an unflatten function: unflattening a vector is the cotangent map
+    of flattening, which hands every leaf its slice in the leaf's shape."""
+    unflatten, flat = make_vjp(_flatten)(value)
+    return flat, unflatten
 
 
 def flatten_func(func, example):
-    _ex, unflatten = flatten(example)
-    _func = lambda _x, *args: flatten(func(unflatten(_x), *args))[0]  # noqa: E731
-    return _func, unflatten, _ex
+    """``func`` on containers -> the same function on flat vectors (and the flat example)."""
+    flat_example, unflatten = flatten(example)
+
+    def on_vectors(flat, *args):
+        return flatten(func(unflatten(flat), *args))[0]
+
+    return on_vectors, unflatten, flat_example

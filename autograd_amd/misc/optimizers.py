@@ -19,21 +19,26 @@ from .flatten import flatten
 
 
 def unflatten_optimizer(optimize):
-    """Takes an optimizer that operates on flat 1-d device arrays and returns a wrapped version
-    that handles trees of nested containers (lists/tuples/dicts) with arrays/scalars at the
-    leaves (optimizers.py:15-31)."""
+    """An optimizer written for flat 1-d device vectors -> one that takes any nest of lists, tuples and dicts
+    with arrays or scalars at the leaves: the point, the gradients and what the callback sees are flattened
+    and unflattened at the boundary (optimizers.py:15-31)."""
 
     @wraps(optimize)
-    def _optimize(grad, x0, callback=None, *args, **kwargs):
-        _x0, unflatten = flatten(x0)
-        _grad = lambda x, i: flatten(grad(unflatten(x), i))[0]  # noqa: E731
-        if callback:
-            _callback = lambda x, i, g: callback(unflatten(x), i, unflatten(g))  # noqa: E731
-        else:
-            _callback = None
-        return unflatten(optimize(_grad, _x0, _callback, *args, **kwargs))
+    def on_containers(grad, x0, callback=None, *args, **kwargs):
+        flat_x0, unflatten = flatten(x0)
 
-    return _optimize
+        def flat_grad(x, i):
+            return flatten(grad(unflatten(x), i))[0]
+
+        flat_callback = None
+        if callback:
+
+            def flat_callback(x, i, g):
+                return callback(unflatten(x), i, unflatten(g))
+
+        return unflatten(optimize(flat_grad, flat_x0, flat_callback, *args, **kwargs))
+
+    return on_containers
 
 
 _F64 = onp.dtype("float64")
@@ -57,41 +62,39 @@ def _step(kind, x, g, s0, s1, hyper):
     return out
 
 
-@unflatten_optimizer
-def sgd(grad, x, callback=None, num_iters=200, step_size=0.1, mass=0.9):
-    """Stochastic gradient descent with momentum.
-    grad() must have signature grad(x, i), where i is the iteration number."""
-    velocity = D.zeros((len(x),), _F64)
+def _descend(grad, x, callback, num_iters, kind, state, hyper_at):
+    """The loop all three optimizers share: gradient at (x, i), the callback sees (x, i, g) before the
+    update, then one fused update kernel; ``hyper_at(i)`` gives the iteration's scalars."""
     for i in range(num_iters):
         g = grad(x, i)
         if callback:
             callback(x, i, g)
-        x = _step(_lib.OPT_SGD, x, g, velocity, None, (mass, 1.0 - mass, step_size))
+        x = _step(kind, x, g, state[0], state[1], hyper_at(i))
     return x
+
+
+@unflatten_optimizer
+def sgd(grad, x, callback=None, num_iters=200, step_size=0.1, mass=0.9):
+    """Gradient descent with momentum: velocity = mass * velocity - (1 - mass) * g; x += step_size * velocity.
+    ``grad(x, i)`` receives the iteration number (optimizers.py:33-45)."""
+    velocity = D.zeros((len(x),), _F64)
+    return _descend(grad, x, callback, num_iters, _lib.OPT_SGD, (velocity, None),
+                    lambda i: (mass, 1.0 - mass, step_size))
 
 
 @unflatten_optimizer
 def rmsprop(grad, x, callback=None, num_iters=100, step_size=0.1, gamma=0.9, eps=10**-8):
-    """Root mean squared prop: See Adagrad paper for details."""
-    avg_sq_grad = D.ones((len(x),), _F64)
-    for i in range(num_iters):
-        g = grad(x, i)
-        if callback:
-            callback(x, i, g)
-        x = _step(_lib.OPT_RMSPROP, x, g, avg_sq_grad, None, (gamma, 1 - gamma, step_size, eps))
-    return x
+    """RMSprop: a running average of squared gradients (started at one) scales each step
+    (optimizers.py:48-59)."""
+    mean_square = D.ones((len(x),), _F64)
+    return _descend(grad, x, callback, num_iters, _lib.OPT_RMSPROP, (mean_square, None),
+                    lambda i: (gamma, 1 - gamma, step_size, eps))
 
 
 @unflatten_optimizer
 def adam(grad, x, callback=None, num_iters=100, step_size=0.001, b1=0.9, b2=0.999, eps=10**-8):
-    """Adam as described in http://arxiv.org/pdf/1412.6980.pdf.
-    It's basically RMSprop with momentum and some correction terms."""
-    m = D.zeros((len(x),), _F64)
-    v = D.zeros((len(x),), _F64)
-    for i in range(num_iters):
-        g = grad(x, i)
-        if callback:
-            callback(x, i, g)
-        x = _step(_lib.OPT_ADAM, x, g, m, v,
-                  (1 - b1, b1, 1 - b2, b2, 1 - b1 ** (i + 1), 1 - b2 ** (i + 1), step_size, eps))
-    return x
+    """Adam (Kingma & Ba, arXiv:1412.6980): bias-corrected running first and second moments
+    (optimizers.py:62-75)."""
+    moments = (D.zeros((len(x),), _F64), D.zeros((len(x),), _F64))
+    return _descend(grad, x, callback, num_iters, _lib.OPT_ADAM, moments,
+                    lambda i: (1 - b1, b1, 1 - b2, b2, 1 - b1 ** (i + 1), 1 - b2 ** (i + 1), step_size, eps))

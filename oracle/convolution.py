@@ -22,15 +22,38 @@ def _mode_ok(mode):
     assert mode in _MODES, f"Mode {mode} undefined, it can be one of 'valid', 'full', and 'same'"
 
 
-def _labelled_contraction(X, Y, paired_axes):
-    """einsum with integer labels: axis k of X is label k, of Y label X.ndim + k, and each
-    (x_axis, y_axis) pair shares a label beyond those, so it is summed.  signal.py:68-76"""
-    x_labels = list(range(X.ndim))
-    y_labels = list(range(X.ndim, X.ndim + Y.ndim))
-    shared = X.ndim + Y.ndim
-    for n, (ax, ay) in enumerate(zip(*paired_axes)):
-        x_labels[ax] = y_labels[ay] = shared + n
-    return onp.einsum(X, x_labels, Y, y_labels)
+def _out_size(a, b, mode):  # signal.py:135-143
+    if mode == "full":
+        return a + b - 1
+    if mode == "same":
+        return a
+    if mode == "valid":
+        return abs(a - b) + 1
+    raise ValueError(f"Mode {mode} not recognized")
+
+
+def _roles(A_shape, B_shape, conv_axes, dot_axes, mode):
+    """signal.py:91-132"""
+    if conv_axes is None:
+        conv_axes = (tuple(range(len(A_shape))), tuple(range(len(A_shape))))
+    ax = {}
+    for name, shape, n in (("A", A_shape, 0), ("B", B_shape, 1)):
+        ax[name] = {"conv": tuple(conv_axes[n]), "dot": tuple(dot_axes[n]),
+                    "ignore": tuple(i for i in range(len(shape)) if i not in conv_axes[n] and i not in dot_axes[n])}
+    assert len(ax["A"]["dot"]) == len(ax["B"]["dot"])
+    assert len(ax["A"]["conv"]) == len(ax["B"]["conv"])
+    a, b, c = len(ax["A"]["ignore"]), len(ax["B"]["ignore"]), len(ax["A"]["conv"])
+    ax["out"] = {"ignore_A": tuple(range(a)), "ignore_B": tuple(range(a, a + b)), "conv": tuple(range(a + b, a + b + c))}
+    sh = {"A": {k: tuple(A_shape[i] for i in v) for k, v in ax["A"].items()},
+          "B": {k: tuple(B_shape[i] for i in v) for k, v in ax["B"].items()}}
+    return ax, sh
+
+
+def _reversed(ndim, axes):
+    idx = [slice(None)] * ndim
+    for a in axes:
+        idx[a] = slice(None, None, -1)
+    return tuple(idx)
 
 
 def _zero_pad(S, W, axes, mode):
@@ -44,6 +67,17 @@ def _zero_pad(S, W, axes, mode):
             after = (k - 1) // 2
             widths[a_s] = (k - 1 - after, after)
     return onp.pad(S, widths, mode="constant")
+
+
+def _labelled_contraction(X, Y, paired_axes):
+    """einsum with integer labels: axis k of X is label k, of Y label X.ndim + k, and each
+    (x_axis, y_axis) pair shares a label beyond those, so it is summed.  signal.py:68-76"""
+    x_labels = list(range(X.ndim))
+    y_labels = list(range(X.ndim, X.ndim + Y.ndim))
+    shared = X.ndim + Y.ndim
+    for n, (ax, ay) in enumerate(zip(*paired_axes)):
+        x_labels[ax] = y_labels[ay] = shared + n
+    return onp.einsum(X, x_labels, Y, y_labels)
 
 
 @primitive
@@ -91,40 +125,6 @@ def convolve(A, B, axes=None, dot_axes=None, mode="full"):
         free_W = list(range(n_free_S + n_conv, n_free_S + n_conv + n_free_W))
         return _labelled_contraction(windows, window, paired[::-1]).transpose(free_S + free_W + conv)
     return _labelled_contraction(window, windows, paired)
-
-
-def _out_size(a, b, mode):  # signal.py:135-143
-    if mode == "full":
-        return a + b - 1
-    if mode == "same":
-        return a
-    if mode == "valid":
-        return abs(a - b) + 1
-    raise ValueError(f"Mode {mode} not recognized")
-
-
-def _roles(A_shape, B_shape, conv_axes, dot_axes, mode):
-    """signal.py:91-132"""
-    if conv_axes is None:
-        conv_axes = (tuple(range(len(A_shape))), tuple(range(len(A_shape))))
-    ax = {}
-    for name, shape, n in (("A", A_shape, 0), ("B", B_shape, 1)):
-        ax[name] = {"conv": tuple(conv_axes[n]), "dot": tuple(dot_axes[n]),
-                    "ignore": tuple(i for i in range(len(shape)) if i not in conv_axes[n] and i not in dot_axes[n])}
-    assert len(ax["A"]["dot"]) == len(ax["B"]["dot"])
-    assert len(ax["A"]["conv"]) == len(ax["B"]["conv"])
-    a, b, c = len(ax["A"]["ignore"]), len(ax["B"]["ignore"]), len(ax["A"]["conv"])
-    ax["out"] = {"ignore_A": tuple(range(a)), "ignore_B": tuple(range(a, a + b)), "conv": tuple(range(a + b, a + b + c))}
-    sh = {"A": {k: tuple(A_shape[i] for i in v) for k, v in ax["A"].items()},
-          "B": {k: tuple(B_shape[i] for i in v) for k, v in ax["B"].items()}}
-    return ax, sh
-
-
-def _reversed(ndim, axes):
-    idx = [slice(None)] * ndim
-    for a in axes:
-        idx[a] = slice(None, None, -1)
-    return tuple(idx)
 
 
 def _grad_convolve(argnum, ans, A, B, axes=None, dot_axes=None, mode="full"):

@@ -38,97 +38,11 @@ def broadcast(x, target):
     return x
 
 
-# indexing and array construction (23-32)
-defjvp(func(ArrayBox.__getitem__), "same")
-defjvp(untake, "same")
-defjvp_argnum(anp.array_from_args, lambda argnum, g, ans, args, kwargs: untake(g, argnum - 2, vspace(ans)))
-defjvp(
-    anp._array_from_scalar_or_array,
-    None,
-    None,
-    lambda g, ans, args, kwargs, _: anp._array_from_scalar_or_array(args, kwargs, g),
-)
-
-# binary ufuncs (38-74)
-def_linear(anp.multiply)
-defjvp(anp.add, lambda g, ans, x, y: broadcast(g, ans), lambda g, ans, x, y: broadcast(g, ans))
-defjvp(anp.subtract, lambda g, ans, x, y: broadcast(g, ans), lambda g, ans, x, y: broadcast(-g, ans))
-defjvp(anp.true_divide, "same", lambda g, ans, x, y: -g * x / y**2)
-for _chooser in (anp.maximum, anp.minimum, anp.fmax, anp.fmin):
-    defjvp(
-        _chooser,
-        lambda g, ans, x, y: g * balanced_eq(x, ans, y),
-        lambda g, ans, x, y: g * balanced_eq(y, ans, x),
-    )
-defjvp(anp.logaddexp, lambda g, ans, x, y: g * anp.exp(x - ans), lambda g, ans, x, y: g * anp.exp(y - ans))
-defjvp(anp.mod, lambda g, ans, x, y: broadcast(g, ans), lambda g, ans, x, y: -g * anp.floor(x / y))
-defjvp(anp.logaddexp2, lambda g, ans, x, y: g * 2 ** (x - ans), lambda g, ans, x, y: g * 2 ** (y - ans))  # 65
-defjvp(
-    anp.power,
-    lambda g, ans, x, y: g * y * x ** anp.where(y, y - 1, 1.0),
-    lambda g, ans, x, y: g * anp.log(replace_zero(x, 1.0)) * ans,
-)
-defjvp(anp.arctan2, lambda g, ans, x, y: g * y / (x**2 + y**2), lambda g, ans, x, y: g * -x / (x**2 + y**2))
-
-# linear one-argument functions (77-105, 150-162)
-for _name in (
-    "negative reshape ravel expand_dims squeeze swapaxes moveaxis roll flipud fliplr diag diagonal "
-    "trace triu tril broadcast_to repeat tile transpose sum _primitive_mean cumsum "
-    "array_split split vsplit hsplit dsplit rollaxis rot90 diff"
-).split():
-    defjvp(getattr(anp, _name), "same")
-defjvp(anp.full, "same", argnums=(1,))
-defjvp(anp.make_diagonal, "same")  # numpy_jvps.py:94
-defjvp(anp.kron, "same", "same")  # numpy_jvps.py:155
-
-# unary ufuncs (108-134)
-_unary = {
-    "abs": lambda g, ans, x: anp.real(g * replace_zero(anp.conj(x), 0.0)) / replace_zero(ans, 1.0),
-    "fabs": lambda g, ans, x: anp.sign(x) * g,
-    "reciprocal": lambda g, ans, x: -g / x**2,
-    "exp": lambda g, ans, x: ans * g,
-    "exp2": lambda g, ans, x: ans * anp.log(2) * g,
-    "expm1": lambda g, ans, x: (ans + 1) * g,
-    "log": lambda g, ans, x: g / x,
-    "log2": lambda g, ans, x: g / x / anp.log(2),
-    "log10": lambda g, ans, x: g / x / anp.log(10),
-    "log1p": lambda g, ans, x: g / (x + 1),
-    "sin": lambda g, ans, x: g * anp.cos(x),
-    "cos": lambda g, ans, x: -g * anp.sin(x),
-    "tan": lambda g, ans, x: g / anp.cos(x) ** 2,
-    "arcsin": lambda g, ans, x: g / anp.sqrt(1 - x**2),
-    "arccos": lambda g, ans, x: -g / anp.sqrt(1 - x**2),
-    "arctan": lambda g, ans, x: g / (1 + x**2),
-    "sinh": lambda g, ans, x: g * anp.cosh(x),
-    "cosh": lambda g, ans, x: g * anp.sinh(x),
-    "tanh": lambda g, ans, x: g / anp.cosh(x) ** 2,
-    "arcsinh": lambda g, ans, x: g / anp.sqrt(x**2 + 1),
-    "arccosh": lambda g, ans, x: g / anp.sqrt(x**2 - 1),
-    "arctanh": lambda g, ans, x: g / (1 - x**2),
-    "square": lambda g, ans, x: g * 2 * x,
-    "sqrt": lambda g, ans, x: g * 0.5 * x**-0.5,
-    "real": lambda g, ans, x: anp.real(g),
-    "conj": lambda g, ans, x: anp.conj(g),
-    "nan_to_num": lambda g, ans, x: anp.where(anp.isfinite(x), g, 0.0),
-    "sinc": lambda g, ans, x: g * (anp.cos(anp.pi * x) * anp.pi * x - anp.sin(anp.pi * x)) / (anp.pi * x**2),
-}
-for _name, _rule in _unary.items():
-    defjvp(getattr(anp, _name), _rule)
-
-for _f in (anp.rad2deg, anp.degrees, anp.deg2rad, anp.radians):  # numpy_jvps.py:78-81: the ufunc itself on the tangent
-    defjvp(_f, "same")
-defjvp(anp.clip, lambda g, ans, x, a_min, a_max: g * anp.logical_and(ans != a_min, ans != a_max))
-defjvp(
-    anp._raw_where,
-    None,
-    lambda g, ans, c, x=None, y=None: anp.where(c, g, anp.zeros(anp.shape(g))),
-    lambda g, ans, c, x=None, y=None: anp.where(c, anp.zeros(g.shape), g),
-)
-defjvp(
-    anp.prod,
-    lambda g, ans, x, axis=None, keepdims=False, **kwargs: ans * anp.sum(g / x, axis=axis, keepdims=keepdims),
-)
-defjvp(anp._astype, lambda g, ans, A, dtype, *a, **k: anp._astype(g, dtype))
+# contractions (230-240)
+for _f in (anp.inner, anp.matmul, anp.dot, anp.tensordot, anp.outer, anp.einsum, anp.cross):
+    def_linear(_f)
+for _f in (dot_adjoint_0, dot_adjoint_1, tensordot_adjoint_0, tensordot_adjoint_1):
+    def_linear(_f)
 
 
 def _num_reps(g, axis):
@@ -175,11 +89,16 @@ def _fwd_chooser(g, ans, x, axis=None, keepdims=False, **kwargs):
 for _f in (anp.max, anp.min, anp.amax, anp.amin):
     defjvp(_f, _fwd_chooser)
 
-# contractions (230-240)
-for _f in (anp.inner, anp.matmul, anp.dot, anp.tensordot, anp.outer, anp.einsum, anp.cross):
-    def_linear(_f)
-for _f in (dot_adjoint_0, dot_adjoint_1, tensordot_adjoint_0, tensordot_adjoint_1):
-    def_linear(_f)
+# linear one-argument functions (77-105, 150-162)
+for _name in (
+    "negative reshape ravel expand_dims squeeze swapaxes moveaxis roll flipud fliplr diag diagonal "
+    "trace triu tril broadcast_to repeat tile transpose sum _primitive_mean cumsum "
+    "array_split split vsplit hsplit dsplit rollaxis rot90 diff"
+).split():
+    defjvp(getattr(anp, _name), "same")
+defjvp(anp.full, "same", argnums=(1,))
+defjvp(anp.make_diagonal, "same")  # numpy_jvps.py:94
+defjvp(anp.kron, "same", "same")  # numpy_jvps.py:155
 
 
 def _fwd_concatenate_args(argnum, g, ans, axis_args, kwargs):
@@ -203,3 +122,84 @@ for _f in (anp.atleast_1d, anp.atleast_2d, anp.atleast_3d):
     defjvp(_f, _atleast_jvp(_f))
 
 defjvp(anp.pad, lambda g, ans, array, width, mode, **kwargs: anp.pad(g, width, mode))  # numpy_jvps.py:303
+
+# unary ufuncs (108-134)
+_unary = {
+    "abs": lambda g, ans, x: anp.real(g * replace_zero(anp.conj(x), 0.0)) / replace_zero(ans, 1.0),
+    "arccos": lambda g, ans, x: -g / anp.sqrt(1 - x**2),
+    "arccosh": lambda g, ans, x: g / anp.sqrt(x**2 - 1),
+    "arcsin": lambda g, ans, x: g / anp.sqrt(1 - x**2),
+    "arcsinh": lambda g, ans, x: g / anp.sqrt(x**2 + 1),
+    "arctan": lambda g, ans, x: g / (1 + x**2),
+    "arctanh": lambda g, ans, x: g / (1 - x**2),
+    "conj": lambda g, ans, x: anp.conj(g),
+    "cos": lambda g, ans, x: -g * anp.sin(x),
+    "cosh": lambda g, ans, x: g * anp.sinh(x),
+    "exp": lambda g, ans, x: ans * g,
+    "exp2": lambda g, ans, x: ans * anp.log(2) * g,
+    "expm1": lambda g, ans, x: (ans + 1) * g,
+    "fabs": lambda g, ans, x: anp.sign(x) * g,
+    "log": lambda g, ans, x: g / x,
+    "log10": lambda g, ans, x: g / x / anp.log(10),
+    "log1p": lambda g, ans, x: g / (x + 1),
+    "log2": lambda g, ans, x: g / x / anp.log(2),
+    "nan_to_num": lambda g, ans, x: anp.where(anp.isfinite(x), g, 0.0),
+    "real": lambda g, ans, x: anp.real(g),
+    "reciprocal": lambda g, ans, x: -g / x**2,
+    "sin": lambda g, ans, x: g * anp.cos(x),
+    "sinc": lambda g, ans, x: g * (anp.cos(anp.pi * x) * anp.pi * x - anp.sin(anp.pi * x)) / (anp.pi * x**2),
+    "sinh": lambda g, ans, x: g * anp.cosh(x),
+    "sqrt": lambda g, ans, x: g * 0.5 * x**-0.5,
+    "square": lambda g, ans, x: g * 2 * x,
+    "tan": lambda g, ans, x: g / anp.cos(x) ** 2,
+    "tanh": lambda g, ans, x: g / anp.cosh(x) ** 2,
+}
+for _name, _rule in _unary.items():
+    defjvp(getattr(anp, _name), _rule)
+
+for _f in (anp.rad2deg, anp.degrees, anp.deg2rad, anp.radians):  # numpy_jvps.py:78-81: the ufunc itself on the tangent
+    defjvp(_f, "same")
+defjvp(anp.clip, lambda g, ans, x, a_min, a_max: g * anp.logical_and(ans != a_min, ans != a_max))
+defjvp(
+    anp._raw_where,
+    None,
+    lambda g, ans, c, x=None, y=None: anp.where(c, g, anp.zeros(anp.shape(g))),
+    lambda g, ans, c, x=None, y=None: anp.where(c, anp.zeros(g.shape), g),
+)
+defjvp(
+    anp.prod,
+    lambda g, ans, x, axis=None, keepdims=False, **kwargs: ans * anp.sum(g / x, axis=axis, keepdims=keepdims),
+)
+defjvp(anp._astype, lambda g, ans, A, dtype, *a, **k: anp._astype(g, dtype))
+
+# binary ufuncs (38-74)
+def_linear(anp.multiply)
+defjvp(anp.add, lambda g, ans, x, y: broadcast(g, ans), lambda g, ans, x, y: broadcast(g, ans))
+defjvp(anp.subtract, lambda g, ans, x, y: broadcast(g, ans), lambda g, ans, x, y: broadcast(-g, ans))
+defjvp(anp.true_divide, "same", lambda g, ans, x, y: -g * x / y**2)
+for _chooser in (anp.maximum, anp.minimum, anp.fmax, anp.fmin):
+    defjvp(
+        _chooser,
+        lambda g, ans, x, y: g * balanced_eq(x, ans, y),
+        lambda g, ans, x, y: g * balanced_eq(y, ans, x),
+    )
+defjvp(anp.logaddexp, lambda g, ans, x, y: g * anp.exp(x - ans), lambda g, ans, x, y: g * anp.exp(y - ans))
+defjvp(anp.mod, lambda g, ans, x, y: broadcast(g, ans), lambda g, ans, x, y: -g * anp.floor(x / y))
+defjvp(anp.logaddexp2, lambda g, ans, x, y: g * 2 ** (x - ans), lambda g, ans, x, y: g * 2 ** (y - ans))  # 65
+defjvp(
+    anp.power,
+    lambda g, ans, x, y: g * y * x ** anp.where(y, y - 1, 1.0),
+    lambda g, ans, x, y: g * anp.log(replace_zero(x, 1.0)) * ans,
+)
+defjvp(anp.arctan2, lambda g, ans, x, y: g * y / (x**2 + y**2), lambda g, ans, x, y: g * -x / (x**2 + y**2))
+
+# indexing and array construction (23-32)
+defjvp(func(ArrayBox.__getitem__), "same")
+defjvp(untake, "same")
+defjvp_argnum(anp.array_from_args, lambda argnum, g, ans, args, kwargs: untake(g, argnum - 2, vspace(ans)))
+defjvp(
+    anp._array_from_scalar_or_array,
+    None,
+    None,
+    lambda g, ans, args, kwargs, _: anp._array_from_scalar_or_array(args, kwargs, g),
+)
