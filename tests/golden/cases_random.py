@@ -1,6 +1,7 @@
 """Seeded generator of small random programs over the traced NumPy namespace (broadcasting arithmetic
 with arrays, row / column vectors and Python scalars; unary ufuncs; views; axis reductions;
-logsumexp; matrix products; fan-out).  The same Python function runs on the reference (when
+logsumexp; matrix products; fan-out; reversals, rolls, running sums, triangles, pieces and
+diagonals).  The same Python function runs on the reference (when
 writing fixtures), the CPU oracle and the device.
 """
 
@@ -28,7 +29,7 @@ def make_program(seed):
     inputs = [rs.randn(m, n), rs.uniform(0.5, 1.5, n), rs.randn(m), rs.randn(n, m), rs.randn(m, n)]
     steps = []
     for _ in range(int(rs.randint(3, 12))):
-        kind = rs.choice(["bin_full", "bin_row", "bin_col", "bin_scalar", "unary", "view", "dot", "mix"])
+        kind = rs.choice(["bin_full", "bin_row", "bin_col", "bin_scalar", "unary", "view", "dot", "mix", "rearrange"])
         steps.append((kind, int(rs.randint(0, 1 << 30))))
     tail = rs.choice(["sum", "lse_rows", "lse_cols", "mean_sq", "rowsum_weighted", "max_rows"])
 
@@ -64,6 +65,30 @@ def make_program(seed):
             elif kind == "dot":
                 x = np.dot(np.dot(x, D), E) * 0.05 if q.rand() < 0.5 else np.dot(x, np.dot(D, x)) * 0.05
                 x = np.tanh(x)
+            elif kind == "rearrange":  # shape-preserving uses of the array-function table
+                v = q.randint(10)
+                rows = x.shape[0]
+                if v == 0:
+                    x = np.roll(x, int(q.randint(-3, 4)), axis=int(q.randint(2))) + np.roll(x, 2) * 0.5
+                elif v == 1:
+                    x = x[::-1] * 0.5 + np.fliplr(x) - np.rot90(x, 2) * 0.25
+                elif v == 2:
+                    x = np.cumsum(x, axis=int(q.randint(2))) * 0.3 + np.reshape(np.cumsum(x), x.shape) * 0.01
+                elif v == 3:
+                    x = np.tile(x, (2, 1))[1 : 1 + rows] * b - x[:, ::-1]
+                elif v == 4:
+                    x = np.concatenate([np.diff(x, axis=1), x[:, :1]], axis=1) + np.tril(x) - 0.5 * np.triu(x, 1)
+                elif v == 5:
+                    head, rest = np.split(x, [1], axis=0)
+                    x = np.concatenate([rest * 2.0, head], axis=0) + np.flipud(x) * 0.1
+                elif v == 6:
+                    x = np.dot(np.inner(x, x) * 0.05, x) + np.trace(np.dot(x, D)) * 0.01
+                elif v == 7:
+                    x = x + np.diag(np.dot(x, D))[:, None] * 0.1 + np.diag(np.diag(np.dot(x, D)))[:, :1] * 0.1
+                elif v == 8:
+                    x = np.sinc(x * 0.3) + np.logaddexp2(x, E) * 0.1
+                else:
+                    x = np.kron(x, b[:2])[:, ::2] * 0.5 + np.moveaxis(np.rollaxis(np.transpose(x), 1), 0, 0)
             else:  # the same value consumed several times in different forms (fan-out accumulation)
                 y = x * b + c[:, None]
                 x = y * 0.5 - np.transpose(np.transpose(y)) * y * 0.01 + np.sum(y, axis=1, keepdims=True) * 0.01
