@@ -631,6 +631,8 @@ def map_op(op, dtype, *xs, out=None, n_out=1):
     if shape is None:
         ops = _lift_scalars(ops, dtype)
         shape = ()
+    if out is not None:
+        shape = out.shape  # the operands are broadcast to the destination (they may all be smaller)
     ops = tuple(_expand(t, shape) for t in ops)
     code = _lib.DTYPE_CODE[dtype]
     if out is not None:

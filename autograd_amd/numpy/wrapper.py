@@ -1372,7 +1372,16 @@ def arange(*args, **kwargs):
 
 
 def eye(N, M=None, k=0, dtype=float):
-    return D.from_numpy(onp.eye(N, M, k, dtype=dtype))
+    """Made on the device (a zero fill and ones written along the diagonal view), so that rules that need an
+    identity, like the cotangent of ``trace``, launch kernels only and can be recorded into a graph."""
+    dt = onp.dtype(dtype)
+    if dt not in D._FLOATS:
+        return D.from_numpy(onp.eye(N, M, k, dtype=dtype))
+    out = D.zeros((int(N), int(N if M is None else M)), dt)
+    diagonal_view = torch.diagonal(out._t, int(k))
+    if diagonal_view.numel():
+        D.map_op(Op.COPY, dt, D.ones((), dt), out=DevArray(diagonal_view, dt))
+    return out
 
 
 to_numpy = D.to_numpy

@@ -851,3 +851,11 @@ def test_reversals_running_sums_and_pieces_are_bit_exact(dnp, dtype):
             special = ~onp.isfinite(want)
             assert onp.array_equal(got[special], want[special], equal_nan=True)
             close(got[~special], want[~special], RT_EW[dtype] * 8)
+
+
+def test_identity_matrices_are_made_on_the_device(dnp):
+    for args in ((3,), (3, 5), (4, 2, 1), (4, 4, -2), (2, 3, 5), (1, 1), (5, 3, -1)):
+        got = dnp.eye(*args).numpy()
+        assert got.dtype == onp.float64 and onp.array_equal(got, onp.eye(*args)), args
+    assert onp.array_equal(dnp.eye(4, 6, 1, dtype=F32).numpy(), onp.eye(4, 6, 1, dtype=F32))
+    assert dnp.eye(3, dtype=F32).numpy().dtype == F32
