@@ -248,29 +248,46 @@ class KernelTimer:
     (2*M*N*K flops for a contraction).
     """
 
-    def __init__(self, only=None):
+    def __init__(self, only=None, events=0):
         self.only = only
         self.records = []
+        self._traffic = {}  # (key, shape of the first result) -> algorithmic bytes, computed once
+        # events made ahead of time keep the cost inside a timed region to the two records per launch
+        self._spare = [torch.cuda.Event(enable_timing=True) for _ in range(events)]
+        self._stream = None
 
     def __enter__(self):
         global _TIMER
         self._prev, _TIMER = _TIMER, self
+        self._stream = torch.cuda.current_stream(device())
         return self
 
     def __exit__(self, *exc):
         global _TIMER
         _TIMER = self._prev
 
+    def _event(self):
+        ev = self._spare.pop() if self._spare else torch.cuda.Event(enable_timing=True)
+        ev.record(self._stream)
+        return ev
+
     def begin(self, key):
         if self.only is not None and key not in self.only:
             return None
-        ev = torch.cuda.Event(enable_timing=True)
-        ev.record()
-        return ev
+        return self._event()
 
     def end(self, ev0, key, nbytes, flops=0.0):
-        ev1 = torch.cuda.Event(enable_timing=True)
-        ev1.record()
+        """``nbytes``: the algorithmic bytes, or ``(outs, ins)`` to have them counted (once per key and shape)."""
+        ev1 = self._event()
+        if type(nbytes) is tuple:
+            outs, ins = nbytes
+            if self.only is None:
+                nbytes = _traffic(outs, ins)
+            else:  # a few selected kernels of a step that repeats: count once per key and shape
+                sig = (key, tuple(outs[0].shape))
+                nbytes = self._traffic.get(sig)
+                if nbytes is None:
+                    nbytes = self._traffic[sig] = _traffic(outs, ins)
         name = _LIB.agmi_last_kernel().decode()
         self.records.append((name, key, ev0, ev1, nbytes, flops))
 
@@ -397,7 +414,7 @@ def elementwise(op, code, shape, outs, ins):
     if rc:
         _check(rc, "agmi_elementwise")
     if ev is not None:
-        _TIMER.end(ev, ("elementwise", op), _traffic(outs, ins))
+        _TIMER.end(ev, ("elementwise", op), (outs, ins))
 
 
 def compare(cmp, code, shape, out, ins):
@@ -447,7 +464,7 @@ def map_reduce(op, red, code, shape, reduce_mask, out, ins):
     if rc:
         _check(rc, "agmi_map_reduce")
     if ev is not None:
-        _TIMER.end(ev, ("map_reduce", op, red), _traffic((out,), ins))
+        _TIMER.end(ev, ("map_reduce", op, red), ((out,), ins))
     return True
 
 

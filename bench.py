@@ -189,7 +189,7 @@ def main():
 
     # timed region: K steps bracketed by synchronise; only the dominant kernel carries events
     be.sync()
-    with _lib.KernelTimer(only={dom_key}) as kt:
+    with _lib.KernelTimer(only={dom_key}, events=2 * args.steps * per_kernel[dominant]["launches"]) as kt:
         t0 = time.perf_counter()
         for _ in range(args.steps):
             step()
