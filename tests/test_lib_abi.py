@@ -73,6 +73,19 @@ def test_argument_errors_are_reported_without_a_gpu(lib):
                        ctypes.c_int64(0), ctypes.c_int64(0), ctypes.c_int64(0), ctypes.c_double(0.0), None,
                        ctypes.c_int64(1), ctypes.c_int64(0), None, ctypes.c_size_t(0), None)
     assert rc == -1
+    i64, c_int = ctypes.c_int64, ctypes.c_int
+    # the copy-shaped index entry points: empty extents are a no-op, everything else is checked before the launch
+    for name, args in (("agmi_cumsum", (i64(2), i64(0), i64(3))), ("agmi_reverse", (i64(0), i64(4), i64(3)))):
+        assert getattr(lib, name)(0, None, *args, None, None) == 0
+    assert lib.agmi_triangle(0, None, i64(1), i64(0), i64(5), i64(0), c_int(1), None, None) == 0
+    for name, args in (("agmi_cumsum", (i64(2), i64(4), i64(3))), ("agmi_reverse", (i64(2), i64(4), i64(3)))):
+        assert getattr(lib, name)(0, None, *args, None, None) == -1 and b"null" in lib.agmi_last_error()
+        assert getattr(lib, name)(0, None, i64(-1), i64(4), i64(3), None, None) == -1 and b"negative" in lib.agmi_last_error()
+    assert lib.agmi_triangle(0, None, i64(1), i64(3), i64(5), i64(0), c_int(1), None, None) == -1
+    buf = (ctypes.c_double * 8)()
+    for name, args in (("agmi_cumsum", (i64(1), i64(8), i64(1))), ("agmi_reverse", (i64(1), i64(8), i64(1)))):
+        assert getattr(lib, name)(7, buf, *args, buf, None) == -1 and b"floating" in lib.agmi_last_error()
+    assert lib.agmi_triangle(7, buf, i64(1), i64(2), i64(4), i64(0), c_int(0), buf, None) == -1
 
 
 def test_device_path_fails_loudly_without_gpu():
