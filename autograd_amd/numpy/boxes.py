@@ -95,8 +95,7 @@ class DevArrayBox(Box):
 
 for _name, _fn in {**_OPERATORS, **_METHODS}.items():
     setattr(DevArrayBox, _name, _fn)
-    if _name != "__eq__" or True:
-        setattr(DevArray, _name, _fn)
+    setattr(DevArray, _name, _fn)  # plain device arrays take the same operators and methods (nothing to trace)
 
 # unboxed values index through the same function (a plain call: nothing to trace)
 DevArray.__getitem__ = lambda self, idx: anp.take(self, idx)
