@@ -260,6 +260,8 @@ class KernelTimer:
         global _TIMER
         self._prev, _TIMER = _TIMER, self
         self._stream = torch.cuda.current_stream(device())
+        for ev in self._spare:  # the underlying HIP event is only created by the first record: do that now
+            ev.record(self._stream)
         return self
 
     def __exit__(self, *exc):

@@ -125,22 +125,25 @@ def defvjp(fun, *vjpmakers, **kwargs):
     traced arguments, nearly all of them, get closures without a loop."""
     makers = {n: translate_vjp(m, fun, n) for n, m in zip(kwargs.get("argnums", count()), vjpmakers)}
 
-    def pick(argnums):
-        try:
-            return [makers[n] for n in argnums]
-        except KeyError:
-            listed = "argnum 0" if len(argnums) == 1 else "argnums 0, 1"
-            raise NotImplementedError(f"VJP of {fun.__name__} wrt {listed} not defined") from None
+    def undefined(n):
+        listed = "argnum 0" if n == 1 else "argnums 0, 1"
+        return NotImplementedError(f"VJP of {fun.__name__} wrt {listed} not defined")
 
     def for_all(argnums, ans, args, kwargs):
-        if len(argnums) == 1:
-            (only,) = pick(argnums)
+        n = len(argnums)
+        if n == 1:
+            only = makers.get(argnums[0])
+            if only is None:
+                raise undefined(1)
             closure = only(ans, *args, **kwargs)
             return lambda g: (closure(g),)
-        if len(argnums) == 2:
-            first, second = (m(ans, *args, **kwargs) for m in pick(argnums))
+        if n == 2:
+            first, second = makers.get(argnums[0]), makers.get(argnums[1])
+            if first is None or second is None:
+                raise undefined(2)
+            first, second = first(ans, *args, **kwargs), second(ans, *args, **kwargs)
             return lambda g: (first(g), second(g))
-        closures = [makers[n](ans, *args, **kwargs) for n in argnums]
+        closures = [makers[k](ans, *args, **kwargs) for k in argnums]
         return lambda g: (c(g) for c in closures)
 
     defvjp_argnums(fun, for_all)

@@ -404,7 +404,7 @@ _FOLDABLE = frozenset({Op.NEG, Op.MUL, Op.ADD, Op.SUB, Op.DIV})
 
 
 def is_scalar(x):
-    return isinstance(x, (numbers.Number, onp.generic)) and not isinstance(x, DevArray)
+    return type(x) is float or type(x) is int or (isinstance(x, (numbers.Number, onp.generic)) and not isinstance(x, DevArray))
 
 
 # --------------------------------------------------------------------------------------------
@@ -538,7 +538,7 @@ def _operand(x, dtype):
         elif type(x) is LazyDevArray:
             return x._affine()
         return x._t
-    if isinstance(x, (numbers.Number, onp.generic)):
+    if type(x) is float or type(x) is int or isinstance(x, (numbers.Number, onp.generic)):  # (exact types first: the ABC test is slow)
         return float(x)
     return asarray(x, dtype)._t
 
@@ -694,7 +694,7 @@ def compare(cmp, a, b):
 def normalize_axes(axis, ndim):
     if axis is None:
         return tuple(range(ndim))
-    if isinstance(axis, (numbers.Integral, onp.integer)):
+    if type(axis) is int or isinstance(axis, (numbers.Integral, onp.integer)):
         axis = (int(axis),)
     axes = tuple(sorted({int(a) % ndim if ndim else 0 for a in axis}))
     for a in axis:

@@ -562,9 +562,9 @@ def stack(arrays, axis=0):
 def _is_basic_index(idx):
     items = idx if isinstance(idx, tuple) else (idx,)
     for it in items:
-        if it is None or it is Ellipsis or isinstance(it, (numbers.Integral, onp.integer)):
+        if it is None or it is Ellipsis or type(it) is slice or type(it) is int:
             continue
-        if isinstance(it, slice):
+        if isinstance(it, (numbers.Integral, onp.integer, slice)):
             continue
         return False
     return True
@@ -572,7 +572,8 @@ def _is_basic_index(idx):
 
 def _plain(idx):
     items = idx if isinstance(idx, tuple) else (idx,)
-    return tuple(int(i) if isinstance(i, (numbers.Integral, onp.integer)) else i for i in items)
+    return tuple(i if (i is None or type(i) is slice or type(i) is int or i is Ellipsis)
+                 else (int(i) if isinstance(i, (numbers.Integral, onp.integer)) else i) for i in items)
 
 
 def _host_index(idx):

@@ -19,7 +19,7 @@ from ..numpy.vjps import _concrete, repeat_to_match_shape
 @primitive
 def logsumexp(x, axis=None, b=1.0, keepdims=False):
     x = D.asarray(x)
-    if not (isinstance(b, numbers.Number) and b == 1.0):
+    if not ((type(b) is float or isinstance(b, numbers.Number)) and b == 1.0):
         # weighted form: log(sum(b * exp(x))) = logsumexp(x + log(b)) for positive weights
         x = np.add.fun(x, np.log.fun(D.asarray(b) if not isinstance(b, numbers.Number) else b))
     dt = D._float_dtype(x.dtype)
