@@ -184,17 +184,36 @@ def primitive(f_raw):
 
     @wraps(f_raw)
     def f_wrapped(*args, **kwargs):
-        boxed_args, level, node_constructor = find_top_boxed_args(args)
-        if not boxed_args:
+        # this wrapper runs for every array operation of a traced program, so it scans the arguments itself:
+        # first for the highest trace level present, then to unbox the arguments of that level
+        top = -1
+        for arg in args:
+            if type(arg) in box_types and arg._trace > top:
+                top = arg._trace
+        if top < 0:
             return f_raw(*args, **kwargs)
-        argvals = subvals(args, [(argnum, box._value) for argnum, box in boxed_args])
+        argvals, argnums, parents = list(args), [], []
+        nested = False  # a box of an outer trace remains among the values: they go through the wrapper again
+        for argnum, arg in enumerate(args):
+            if type(arg) in box_types:
+                if arg._trace == top:
+                    value = argvals[argnum] = arg._value
+                    argnums.append(argnum)
+                    parents.append(arg._node)
+                    if type(value) in box_types:
+                        nested = True
+                else:
+                    nested = True
+        argvals = tuple(argvals)
+        node_constructor = type(parents[0])
         if f_wrapped in notrace_primitives[node_constructor]:
             return f_wrapped(*argvals, **kwargs)
-        parents = tuple(box._node for _, box in boxed_args)
-        argnums = tuple(argnum for argnum, _ in boxed_args)
-        ans = f_wrapped(*argvals, **kwargs)
-        node = node_constructor(ans, f_wrapped, argvals, kwargs, argnums, parents)
-        return new_box(ans, level, node)
+        ans = f_wrapped(*argvals, **kwargs) if nested else f_raw(*argvals, **kwargs)
+        node = node_constructor(ans, f_wrapped, argvals, kwargs, tuple(argnums), tuple(parents))
+        box_cls = box_type_mappings.get(type(ans))
+        if box_cls is None:
+            return new_box(ans, top, node)  # raises the type error
+        return box_cls(ans, top, node)
 
     f_wrapped.fun = f_raw
     f_wrapped._is_autograd_primitive = True
