@@ -168,6 +168,8 @@ def lib():
     L.agmi_reverse.argtypes = [c_i, c_p, c_i64, c_i64, c_i64, c_p, c_p]
     L.agmi_triangle.restype = c_i
     L.agmi_triangle.argtypes = [c_i, c_p, c_i64, c_i64, c_i64, c_i64, c_i, c_p, c_p]
+    L.agmi_sort_rows.restype = c_i
+    L.agmi_sort_rows.argtypes = [c_i, c_p, c_i64, c_i64, c_p, c_p, c_p, c_p]
     L.agmi_cumsum.restype = c_i
     L.agmi_cumsum.argtypes = [c_i, c_p, c_i64, c_i64, c_i64, c_p, c_p]
     L.agmi_take_rows.restype = c_i
@@ -184,7 +186,7 @@ def lib():
 
 EXPORTS = (
     "agmi_last_error agmi_version agmi_last_kernel agmi_elementwise agmi_compare agmi_cast agmi_map_reduce "
-    "agmi_map_reduce_workspace_bytes agmi_gemm agmi_fill agmi_take_rows agmi_cumsum agmi_reverse agmi_triangle agmi_scatter_add_rows agmi_optimizer_step "
+    "agmi_map_reduce_workspace_bytes agmi_gemm agmi_fill agmi_take_rows agmi_sort_rows agmi_cumsum agmi_reverse agmi_triangle agmi_scatter_add_rows agmi_optimizer_step "
     "agmi_correlate"
 ).split()
 
@@ -500,6 +502,14 @@ def reverse(code, src, outer, n, inner, out):
 def triangle(code, src, batch, rows, cols, k, lower, out):
     _check(_LIB.agmi_triangle(code, src.data_ptr(), batch, rows, cols, k, 1 if lower else 0, out.data_ptr(), _stream()),
            "agmi_triangle")
+
+
+def sort_rows(code, src, rows, n, sorted_out=None, order=None, rank=None):
+    ptr = lambda t: None if t is None else t.data_ptr()  # noqa: E731
+    rc = _LIB.agmi_sort_rows(code, src.data_ptr(), rows, n, ptr(sorted_out), ptr(order), ptr(rank), _stream())
+    if rc == -2:  # AGMI_ERR_UNSUPPORTED
+        raise NotImplementedError(_LIB.agmi_last_error().decode())
+    _check(rc, "agmi_sort_rows")
 
 
 def cumsum(code, src, outer, n, inner, out):

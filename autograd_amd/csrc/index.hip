@@ -116,6 +116,44 @@ __global__ __launch_bounds__(kBlock) void triangle_kernel(const T *__restrict__ 
     out[e] = keep ? src[e] : T(0);
 }
 
+// Stable sort of each row of a contiguous (rows, n) array by counting: the rank of an element is the number
+// of elements ordered before it (smaller; equal and earlier; any number before a NaN), so no element moves
+// until its final place is known and equal elements keep their order.  O(n^2) comparisons per row, tiles of
+// the row staged through LDS; meant for the vector lengths sort rules are used on (see kMaxSortLength).
+constexpr int64_t kMaxSortLength = 65536;
+
+template <typename T>
+__device__ __forceinline__ bool ordered_before(T a, int64_t ja, T b, int64_t jb) {
+    const bool a_nan = a != a, b_nan = b != b;
+    if (a_nan || b_nan) return (!a_nan && b_nan) || (a_nan && b_nan && ja < jb);
+    return a < b || (a == b && ja < jb);
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void rank_sort_rows(const T *__restrict__ src, int64_t n, T *__restrict__ sorted,
+                                                         int64_t *__restrict__ order, int64_t *__restrict__ rank) {
+    __shared__ T tile[kBlock];
+    const int64_t row = blockIdx.y;
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    const T *line = src + row * n;
+    const bool live = i < n;
+    const T mine = live ? line[i] : T(0);
+    int64_t before = 0;
+    for (int64_t j0 = 0; j0 < n; j0 += kBlock) {
+        const int64_t j = j0 + threadIdx.x;
+        tile[threadIdx.x] = j < n ? line[j] : T(0);
+        __syncthreads();
+        const int width = static_cast<int>(n - j0 < kBlock ? n - j0 : kBlock);
+        if (live)
+            for (int t = 0; t < width; ++t) before += ordered_before(tile[t], j0 + t, mine, i) ? 1 : 0;
+        __syncthreads();
+    }
+    if (!live) return;
+    if (sorted) sorted[row * n + before] = mine;
+    if (order) order[row * n + before] = i;
+    if (rank) rank[row * n + i] = before;
+}
+
 }  // namespace agmi
 
 using namespace agmi;
@@ -290,4 +328,36 @@ extern "C" int agmi_triangle(int dtype, const void *src, int64_t batch, int64_t 
         hipLaunchKernelGGL(triangle_kernel<double>, dim3((unsigned)blocks), dim3(kBlock), 0, s,
                            static_cast<const double *>(src), total, rows, cols, k, lower, static_cast<double *>(out));
     return hip_check(hipGetLastError(), "triangle launch");
+}
+
+extern "C" int agmi_sort_rows(int dtype, const void *src, int64_t rows, int64_t n, void *sorted, int64_t *order,
+                              int64_t *rank, void *stream) {
+    if (rows < 0 || n < 0) {
+        set_error("sort_rows: negative extent");
+        return AGMI_ERR_ARG;
+    }
+    if (rows == 0 || n == 0) return 0;
+    if (!src || (!sorted && !order && !rank)) {
+        set_error("sort_rows: null source, or no result asked for");
+        return AGMI_ERR_ARG;
+    }
+    if (dtype != AGMI_F32 && dtype != AGMI_F64) {
+        set_error("sort_rows: dtype %d is not a floating type", dtype);
+        return AGMI_ERR_ARG;
+    }
+    if (n > kMaxSortLength || rows > 65535) {
+        set_error("sort_rows: %lld rows of %lld elements; at most 65535 rows of %lld are supported", (long long)rows,
+                  (long long)n, (long long)kMaxSortLength);
+        return AGMI_ERR_UNSUPPORTED;
+    }
+    const dim3 grid((unsigned)ceil_div(n, kBlock), (unsigned)rows);
+    hipStream_t s = as_stream(stream);
+    set_kernel_name("rank_sort_rows");
+    if (dtype == AGMI_F32)
+        hipLaunchKernelGGL(rank_sort_rows<float>, grid, dim3(kBlock), 0, s, static_cast<const float *>(src), n,
+                           static_cast<float *>(sorted), order, rank);
+    else
+        hipLaunchKernelGGL(rank_sort_rows<double>, grid, dim3(kBlock), 0, s, static_cast<const double *>(src), n,
+                           static_cast<double *>(sorted), order, rank);
+    return hip_check(hipGetLastError(), "sort_rows launch");
 }

@@ -89,6 +89,16 @@ defjvp(  # numpy_jvps.py:67-68 (numpy.mod is the same function)
 )
 defjvp(anp.nan_to_num, lambda g, ans, x: anp.where(anp.isfinite(x), g, 0.0))  # numpy_jvps.py:35
 defjvp(anp.kron, "same", "same")  # numpy_jvps.py:155
+
+
+def _fwd_sort(g, ans, x, *args, **kwargs):  # numpy_jvps.py:256-271 (sort and partition alike): the tangent in sorted order
+    order_, rank = anp.sort_permutations(x)
+    return anp._reorder(g, order_, rank)
+
+
+defjvp(anp.sort, _fwd_sort)
+defjvp(anp.partition, _fwd_sort)
+defjvp(anp._reorder, "same")
 def_linear(anp.cross)  # numpy_jvps.py:106
 defjvp(anp.logaddexp2, lambda g, ans, x, y: g * 2 ** (x - ans), lambda g, ans, x, y: g * 2 ** (y - ans))  # 65
 defjvp(  # numpy_jvps.py:135-138

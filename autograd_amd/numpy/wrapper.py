@@ -1056,6 +1056,79 @@ def rollaxis(a, axis, start=0):
     return transpose.fun(a, order)
 
 
+# ---- sorting (numpy_vjps.py:773-802): a stable counting sort on the device; rules move cotangents and tangents
+# ---- through the permutation with `_reorder`, whose own rule is the inverse permutation --------------------
+def _sorted_lines(x, axis, want):
+    """Sort along ``axis``; ``want`` names the results: "sorted", "order" (argsort), "rank" (its inverse)."""
+    x = D.asarray(x)
+    if x.dtype not in D._FLOATS:
+        raise NotImplementedError("sort: floating-point arrays only on the device")
+    if axis is None:
+        x, axis = D.asarray(ravel.fun(x)), 0
+    if x.ndim == 0:
+        raise onp.exceptions.AxisError(axis, 0)
+    (axis,) = D.normalize_axes(axis, x.ndim)
+    last = x.ndim - 1
+    lines = D.contiguous(D.plain(D.asarray(moveaxis.fun(x, axis, last))))
+    n = lines.shape[-1]
+    rows = lines.size // n if n else 0
+    i64 = onp.dtype(onp.int64)
+    outs = {"sorted": D.empty(lines.shape, x.dtype) if "sorted" in want else None,
+            "order": D.empty(lines.shape, i64) if "order" in want else None,
+            "rank": D.empty(lines.shape, i64) if "rank" in want else None}
+    if lines.size:
+        _lib.sort_rows(_lib.DTYPE_CODE[x.dtype], lines._t, rows, n, *(None if outs[k] is None else outs[k]._t
+                                                                      for k in ("sorted", "order", "rank")))
+    back = lambda a: a if axis == last else D.asarray(moveaxis.fun(a, last, axis))  # noqa: E731
+    return tuple(back(outs[k]) for k in want)
+
+
+@primitive
+def sort(a, axis=-1, kind=None, order=None):
+    if order is not None:
+        raise NotImplementedError("sort: structured-array fields are not supported on the device")
+    return _sorted_lines(a, axis, ("sorted",))[0]
+
+
+@primitive
+def partition(a, kth, axis=-1, kind="introselect", order=None):
+    """A full sort: it satisfies numpy.partition's contract for every ``kth``."""
+    if order is not None:
+        raise NotImplementedError("partition: structured-array fields are not supported on the device")
+    return _sorted_lines(a, axis, ("sorted",))[0]
+
+
+def argsort(a, axis=-1, kind=None, order=None):
+    from ..tracer import getval
+
+    return _sorted_lines(getval(a), axis, ("order",))[0]
+
+
+def argpartition(a, kth, axis=-1, kind="introselect", order=None):
+    from ..tracer import getval
+
+    return _sorted_lines(getval(a), axis, ("order",))[0]
+
+
+def sort_permutations(x):
+    """(order, rank) of a vector: ``x[order]`` is sorted and ``rank`` is the inverse permutation."""
+    from ..tracer import getval
+
+    return _sorted_lines(getval(x), 0, ("order", "rank"))
+
+
+@primitive
+def _reorder(x, index, inverse):
+    """``x[index]`` for a permutation ``index`` of a vector that is already on the device (``inverse`` is its
+    inverse, used by the rule).  The index comes from the sort kernel, so it is not read back for a bounds check."""
+    x = D.contiguous(D.plain(D.asarray(x)))
+    n = x.shape[0]
+    out = D.empty(x.shape, x.dtype)
+    if x.size:
+        _lib.take_rows(_lib.DTYPE_CODE[x.dtype], x._t, n, x.size // n, index._t, n, out._t)
+    return out
+
+
 @primitive
 def flip(m, axis=None):
     m = D.asarray(m)

@@ -242,6 +242,16 @@ int agmi_reverse(int dtype, const void *src, int64_t outer, int64_t n, int64_t i
 int agmi_triangle(int dtype, const void *src, int64_t batch, int64_t rows, int64_t cols, int64_t k,
                   int lower, void *out, void *stream);
 
+/* Stable ascending sort of every row of a contiguous (rows, n) array, NaNs last: any of
+ *   sorted[r, k]  the k-th smallest element of row r,
+ *   order[r, k]   its position in the row (numpy.argsort, kind="stable"),
+ *   rank[r, i]    the place element i of the row takes (the inverse permutation)
+ * (null pointers are skipped).  Forward of numpy.sort / partition and the permutations their
+ * rules route cotangents and tangents through (numpy_vjps.py:773-802, numpy_jvps.py:256-271).
+ * n is limited to 65536 (the ranks are found by counting), rows to 65535. */
+int agmi_sort_rows(int dtype, const void *src, int64_t rows, int64_t n, void *sorted, int64_t *order,
+                   int64_t *rank, void *stream);
+
 /* Running sums along the middle axis of a contiguous (outer, n, inner) array:
  * out[o, k, c] = src[o, 0, c] + ... + src[o, k, c], added in that order (bit-identical to
  * numpy.cumsum).  Forward of numpy.cumsum and, on reversed operands, its cotangent

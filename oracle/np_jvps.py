@@ -122,6 +122,12 @@ for _f in (anp.atleast_1d, anp.atleast_2d, anp.atleast_3d):
     defjvp(_f, _atleast_jvp(_f))
 
 defjvp(anp.pad, lambda g, ans, array, width, mode, **kwargs: anp.pad(g, width, mode))  # numpy_jvps.py:303
+# numpy_jvps.py:256-271: the tangent taken in sorted (partitioned) order
+defjvp(anp.sort, lambda g, ans, x, axis=-1, kind="quicksort", order=None: g[anp.argsort(x, axis, kind, order)])
+defjvp(
+    anp.partition,
+    lambda g, ans, x, kth, axis=-1, kind="introselect", order=None: g[anp.argpartition(x, kth, axis, kind, order)],
+)
 
 # unary ufuncs (108-134)
 _unary = {

@@ -23,7 +23,7 @@ reshape ravel expand_dims squeeze transpose swapaxes moveaxis atleast_1d atleast
 atleast_3d repeat tile split array_split vsplit hsplit dsplit rollaxis rot90 diff cross sinc logaddexp2 broadcast_to roll flipud fliplr diag diagonal trace tril triu
 dot matmul tensordot inner outer einsum kron
 astype
-floor ceil round rint around fix trunc all any argmax argmin argsort nonzero
+floor ceil round rint around fix trunc all any argmax argmin argsort argpartition sort partition nonzero
 count_nonzero searchsorted floor_divide logical_and logical_or logical_not logical_xor
 isfinite isinf isnan allclose isclose array_equal greater greater_equal less less_equal
 equal not_equal iscomplex size isscalar isreal zeros_like ones_like empty_like full_like

@@ -22,7 +22,7 @@ from .np_boxes import ArrayBox
 nograd_functions = [
     getattr(anp, n)
     for n in (
-        "floor ceil round rint around fix trunc all any argmax argmin argsort nonzero "
+        "floor ceil round rint around fix trunc all any argmax argmin argsort argpartition nonzero "
         "count_nonzero searchsorted sign ndim shape floor_divide logical_and logical_or "
         "logical_not logical_xor isfinite isinf isnan allclose isclose array_equal greater "
         "greater_equal less less_equal equal not_equal iscomplexobj iscomplex size isscalar "
@@ -375,6 +375,30 @@ def _grad_diff(ans, a, n=1, axis=-1):  # numpy_vjps.py:270-294
 
 
 defvjp(anp.diff, _grad_diff)
+
+
+def _unpermuter(g, permutation):  # numpy_vjps.py:798-801
+    unsort = anp.zeros(len(permutation), dtype=int)
+    unsort[permutation] = list(range(len(permutation)))
+    return g[unsort]
+
+
+def _grad_sort(ans, x, axis=-1, kind="quicksort", order=None):  # numpy_vjps.py:773-779
+    if len(x.shape) > 1:
+        raise NotImplementedError("Gradient of sort not implemented for multi-dimensional arrays.")
+    sort_perm = anp.argsort(x, axis, kind, order)
+    return lambda g: _unpermuter(g, sort_perm)
+
+
+def _grad_partition(ans, x, kth, axis=-1, kind="introselect", order=None):  # numpy_vjps.py:787-792
+    if len(x.shape) > 1:
+        raise NotImplementedError("Gradient of partition not implemented for multi-dimensional arrays.")
+    partition_perm = anp.argpartition(x, kth, axis, kind, order)
+    return lambda g: _unpermuter(g, partition_perm)
+
+
+defvjp(anp.sort, _grad_sort)
+defvjp(anp.partition, _grad_partition)
 
 
 def _grad_tile(ans, x, reps):  # numpy_vjps.py:352-364

@@ -380,6 +380,10 @@ def next_cases(be, ext):
             "logaddexp2_array": (lambda a: np.sum(np.logaddexp2(a, Y_) * W34), A_),
             "logaddexp2_scalar": (lambda a: np.sum(np.logaddexp2(a, 0.5) ** 2), A_),
             "logaddexp2_second_arg": (lambda a: np.sum(np.logaddexp2(Y_ * 3.0, a) * W34), A_),
+            "sort": (lambda q: np.sum(np.sort(q[1] * q[2]) * v_ ** 2), Q_),
+            "sort_through_take": (lambda a: np.sum(np.sort(np.ravel(a))[::3] ** 2), A_),
+            # (which of the two smallest comes first is the selection algorithm's business: weigh them alike)
+            "partition": (lambda q: np.sum(np.partition(q[0] * q[3], 2)[:2]) * 2.0 + np.partition(q[0] * q[3], 2)[2] ** 2, Q_),
             "real_conj": (lambda a: np.sum(np.real(a) * np.conj(a) * 2.0), A_),
         }
         for name, (f, x) in table.items():

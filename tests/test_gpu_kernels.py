@@ -859,3 +859,46 @@ def test_identity_matrices_are_made_on_the_device(dnp):
         assert got.dtype == onp.float64 and onp.array_equal(got, onp.eye(*args)), args
     assert onp.array_equal(dnp.eye(4, 6, 1, dtype=F32).numpy(), onp.eye(4, 6, 1, dtype=F32))
     assert dnp.eye(3, dtype=F32).numpy().dtype == F32
+
+
+@pytest.mark.parametrize("dtype", [F32, F64])
+def test_sort_is_stable_and_puts_nans_last(dnp, dtype):
+    import autograd_amd as ag
+
+    rs = onp.random.RandomState(51)
+    for n in (1, 2, 7, 255, 256, 257, 1000, 5003):
+        x = rs.randn(n).astype(dtype)
+        if n > 6:
+            x[rs.randint(0, n, n // 5)] = x[0]          # ties
+            x[rs.randint(0, n, 3)] = onp.nan            # NaNs sort last, in their original order
+            x[rs.randint(0, n, 2)] = onp.inf
+            x[rs.randint(0, n, 2)] = -onp.inf
+        want_order = onp.argsort(x, kind="stable")
+        assert onp.array_equal(dnp.sort(P(dnp, x)).numpy(), x[want_order], equal_nan=True)
+        order = dnp.argsort(P(dnp, x)).numpy()
+        assert order.dtype == onp.int64 and onp.array_equal(order, want_order)
+        part = dnp.partition(P(dnp, x), n // 2).numpy()
+        assert onp.array_equal(part, onp.sort(x), equal_nan=True)
+    a = rs.randn(5, 33, 7).astype(dtype)
+    for axis in (0, 1, 2, -1, None):
+        got = dnp.sort(P(dnp, a), axis=axis).numpy()
+        assert got.dtype == dtype and onp.array_equal(got, onp.sort(a, axis=axis))
+        if axis is not None:
+            assert onp.array_equal(dnp.argsort(P(dnp, a), axis=axis).numpy(), onp.argsort(a, axis=axis, kind="stable"))
+    assert onp.array_equal(dnp.sort(P(dnp, a).T[::2], axis=1).numpy(), onp.sort(a.T[::2], axis=1))
+    assert dnp.sort(P(dnp, onp.zeros((0, 4), dtype))).shape == (0, 4)
+    with pytest.raises(NotImplementedError):
+        dnp.sort(P(dnp, onp.zeros(70000, dtype)))
+    # cotangents go back to where the sorted elements came from; second order exists
+    x = rs.randn(300).astype(dtype)
+    w = rs.randn(300).astype(dtype)
+    g = ag.grad(lambda v: dnp.sum(dnp.sort(v) * P(dnp, w)))(P(dnp, x)).numpy()
+    want = onp.empty_like(x)
+    want[onp.argsort(x, kind="stable")] = w
+    assert onp.array_equal(g, want)
+    with pytest.raises(NotImplementedError):
+        ag.grad(lambda v: dnp.sum(dnp.sort(v, axis=0)))(P(dnp, a))
+    h = ag.grad(lambda v: dnp.sum(ag.grad(lambda u: dnp.sum(dnp.sort(u * u) * P(dnp, w)))(v) * P(dnp, w)))(P(dnp, x)).numpy()
+    want2 = onp.empty_like(x)
+    want2[onp.argsort(x * x, kind="stable")] = w
+    close(h, (dtype(2.0) * want2 * w).astype(dtype), RT_EW[dtype] * 4)

@@ -86,6 +86,10 @@ def test_argument_errors_are_reported_without_a_gpu(lib):
     for name, args in (("agmi_cumsum", (i64(1), i64(8), i64(1))), ("agmi_reverse", (i64(1), i64(8), i64(1)))):
         assert getattr(lib, name)(7, buf, *args, buf, None) == -1 and b"floating" in lib.agmi_last_error()
     assert lib.agmi_triangle(7, buf, i64(1), i64(2), i64(4), i64(0), c_int(0), buf, None) == -1
+    assert lib.agmi_sort_rows(0, None, i64(0), i64(5), None, None, None, None) == 0
+    assert lib.agmi_sort_rows(1, buf, i64(1), i64(8), None, None, None, None) == -1 and b"no result" in lib.agmi_last_error()
+    assert lib.agmi_sort_rows(1, buf, i64(1), i64(70000), buf, None, None, None) == -2 and b"65536" in lib.agmi_last_error()
+    assert lib.agmi_sort_rows(7, buf, i64(1), i64(8), buf, None, None, None) == -1 and b"floating" in lib.agmi_last_error()
 
 
 def test_device_path_fails_loudly_without_gpu():
