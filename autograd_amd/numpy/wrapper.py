@@ -208,6 +208,76 @@ def isfinite(x):
     return D.compare(Cmp.LT, D.float_map(Op.ABS, x), onp.inf)  # NaN compares false
 
 
+def isposinf(x):
+    from ..tracer import getval
+
+    return D.compare(Cmp.EQ, D.asarray(getval(x)), onp.inf)
+
+
+def isneginf(x):
+    from ..tracer import getval
+
+    return D.compare(Cmp.EQ, D.asarray(getval(x)), -onp.inf)
+
+
+def _truth_reduced(a, red, axis, keepdims):
+    truth = _truth(a)
+    if not isinstance(truth, DevArray):
+        truth = D.full((), truth, onp.dtype(onp.float64))
+    axes = D.normalize_axes(axis, truth.ndim)
+    return D.map_reduce(Op.COPY, red, truth.dtype, (truth,), axes, keepdims)
+
+
+def all(a, axis=None, keepdims=False):  # noqa: A001
+    """Non-differentiable truth tests (numpy_vjps.py:13-68): the minimum / maximum / sum of the 0-1 array."""
+    return D.compare(Cmp.NE, _truth_reduced(a, Red.MIN, axis, keepdims), 0.0)
+
+
+def any(a, axis=None, keepdims=False):  # noqa: A001
+    return D.compare(Cmp.NE, _truth_reduced(a, Red.MAX, axis, keepdims), 0.0)
+
+
+def count_nonzero(a, axis=None, keepdims=False):
+    """Counts are exact in float64 below 2**53; returned as int64 like NumPy's."""
+    return D.astype(_truth_reduced(a, Red.SUM, axis, keepdims), onp.int64)
+
+
+def isclose(a, b, rtol=1e-05, atol=1e-08, equal_nan=False):
+    """|a - b| <= atol + rtol * |b| where both are finite, equality elsewhere (numpy.isclose)."""
+    from ..tracer import getval
+
+    a, b = D.asarray(getval(a)), D.asarray(getval(b))
+    dt = D._float_dtype(D.result_dtype(a, b))
+    f64 = onp.dtype(onp.float64)
+    gap = D.map_op(Op.ABS, dt, D.map_op(Op.SUB, dt, a, b))
+    bound = D.map_op(Op.ADD, dt, D.map_op(Op.MUL, dt, D.map_op(Op.ABS, dt, b), float(rtol)), float(atol))
+    near = D.astype(D.compare(Cmp.LE, gap, bound), f64)
+    finite = D.map_op(Op.MUL, f64, D.astype(isfinite(a), f64), D.astype(isfinite(b), f64))
+    same = D.astype(D.compare(Cmp.EQ, a, b), f64)
+    # finite pairs by the tolerance, the rest (infinities) by equality
+    verdict = D.map_op(Op.WHERE, f64, finite, near, same)
+    if equal_nan:
+        both_nan = D.map_op(Op.MUL, f64, D.astype(isnan(a), f64), D.astype(isnan(b), f64))
+        verdict = D.map_op(Op.MAXIMUM, f64, verdict, both_nan)
+    return D.compare(Cmp.NE, verdict, 0.0)
+
+
+def array_equal(a1, a2, equal_nan=False):
+    """A Python bool (reads one element back): same shape and all elements equal."""
+    from ..tracer import getval
+
+    a1, a2 = D.asarray(getval(a1)), D.asarray(getval(a2))
+    if a1.shape != a2.shape:
+        return False
+    if a1.size == 0:
+        return True
+    f64 = onp.dtype(onp.float64)
+    same = D.astype(D.compare(Cmp.EQ, a1, a2), f64)
+    if equal_nan:
+        same = D.map_op(Op.MAXIMUM, f64, same, D.map_op(Op.MUL, f64, D.astype(isnan(a1), f64), D.astype(isnan(a2), f64)))
+    return bool(all(same))
+
+
 def _arg_extreme(red, name):
     def raw(a, axis=None, out=None, keepdims=False):
         """Index of the first extreme element: min over the axis of where(x == extreme, position, n)
@@ -255,7 +325,7 @@ _astype = astype
 # ---- reductions ---------------------------------------------------------------------------------
 def _reduction(red, name):
     def raw(x, axis=None, keepdims=False, dtype=None, out=None, **kwargs):
-        if type(x) in (tuple, list) and all(isinstance(e, (int, onp.integer)) for e in x):
+        if type(x) in (tuple, list) and builtins.all(isinstance(e, (int, onp.integer)) for e in x):
             # shape arithmetic on a tuple of Python ints (np.prod(shape)) stays a host integer, usable in slices
             return getattr(onp, name)(x, axis=axis, dtype=dtype, keepdims=keepdims)
         x = D.asarray(x)
@@ -602,9 +672,9 @@ def _positive_steps(idx, shape):
     ``idx``, and the axes of the result along which that selection is reversed to give ``A[idx]``
     (device views cannot have negative strides; a reversal is one gather)."""
     items = list(idx if isinstance(idx, tuple) else (idx,))
-    if not any(isinstance(it, slice) and it.step is not None and it.step < 0 for it in items):
+    if not builtins.any(isinstance(it, slice) and it.step is not None and it.step < 0 for it in items):
         return idx, ()
-    if any(it is Ellipsis for it in items):
+    if builtins.any(it is Ellipsis for it in items):
         k = [it is Ellipsis for it in items].index(True)
         consumed = len([it for it in items if it is not None and it is not Ellipsis])
         items[k : k + 1] = [slice(None)] * (len(shape) - consumed)
@@ -681,7 +751,7 @@ def _leading_rows(idx, shape):
         first, rest = idx[0], idx[1:]
     else:
         return None
-    if not shape or any(not (isinstance(r, slice) and r == slice(None)) for r in rest):
+    if not shape or builtins.any(not (isinstance(r, slice) and r == slice(None)) for r in rest):
         return None
     start, stop, step = first.indices(shape[0])
     return (start, stop if stop > start else start) if step == 1 else None  # (this module's max is the array reduction)
@@ -774,11 +844,11 @@ def pad_widths(pad_width, ndim):
 @primitive
 def pad(array, pad_width, mode="constant", **kwargs):
     """Zero padding (numpy.pad, constant mode): one fill and one strided copy into the interior."""
-    if mode != "constant" or any(v != 0 for v in onp.ravel(kwargs.get("constant_values", 0))) or set(kwargs) - {"constant_values"}:
+    if mode != "constant" or builtins.any(v != 0 for v in onp.ravel(kwargs.get("constant_values", 0))) or set(kwargs) - {"constant_values"}:
         raise NotImplementedError("pad: only mode='constant' with zeros is supported on the device")
     x = D.asarray(array)
     widths = pad_widths(pad_width, x.ndim)
-    if any(b < 0 or a < 0 for b, a in widths):
+    if builtins.any(b < 0 or a < 0 for b, a in widths):
         raise ValueError("index can't contain negative values")
     out = D.zeros(tuple(n + b + a for n, (b, a) in zip(x.shape, widths)), x.dtype)
     if x.size:
@@ -879,7 +949,7 @@ def _tensordot_raw(a, b, axes=2):
         axes_b = [axes_b] if isinstance(axes_b, (numbers.Integral, onp.integer)) else list(axes_b)
     axes_a = [int(x) % a.ndim for x in axes_a] if a.ndim else []
     axes_b = [int(x) % b.ndim for x in axes_b] if b.ndim else []
-    if len(axes_a) != len(axes_b) or any(a.shape[i] != b.shape[j] for i, j in zip(axes_a, axes_b)):
+    if len(axes_a) != len(axes_b) or builtins.any(a.shape[i] != b.shape[j] for i, j in zip(axes_a, axes_b)):
         raise ValueError("shape-mismatch for sum")
     free_a = [d for d in range(a.ndim) if d not in axes_a]
     free_b = [d for d in range(b.ndim) if d not in axes_b]
@@ -1429,6 +1499,18 @@ def empty(shape, dtype=float):
 def zeros_like(a, dtype=None):
     s, _, dt, _ = _meta_of(a)
     return D.zeros(s, dtype or dt)
+
+
+@notrace_primitive
+def full_like(a, fill_value, dtype=None):
+    s, _, dt, _ = _meta_of(a)
+    return D.full(s, fill_value, onp.dtype(dtype or dt))
+
+
+@notrace_primitive
+def empty_like(a, dtype=None):
+    s, _, dt, _ = _meta_of(a)
+    return D.empty(s, onp.dtype(dtype or dt))
 
 
 @notrace_primitive

@@ -902,3 +902,28 @@ def test_sort_is_stable_and_puts_nans_last(dnp, dtype):
     want2 = onp.empty_like(x)
     want2[onp.argsort(x * x, kind="stable")] = w
     close(h, (dtype(2.0) * want2 * w).astype(dtype), RT_EW[dtype] * 4)
+
+
+def test_truth_tests_and_closeness(dnp):
+    rs = onp.random.RandomState(61)
+    a = rs.randn(6, 9)
+    a[a < -0.5] = 0.0
+    A = P(dnp, a)
+    for axis in (None, 0, 1, (0, 1)):
+        for keepdims in (False, True):
+            for mine, ref in ((dnp.all, onp.all), (dnp.any, onp.any), (dnp.count_nonzero, onp.count_nonzero)):
+                got, want = mine(A, axis=axis, keepdims=keepdims).numpy(), onp.asarray(ref(a, axis=axis, keepdims=keepdims))
+                assert got.dtype == want.dtype and got.shape == want.shape and onp.array_equal(got, want), (ref.__name__, axis)
+    assert bool(dnp.all(A * 0.0 + 1.0)) and not bool(dnp.any(A * 0.0)) and bool(dnp.any(A > 1.0))
+    x = onp.array([1.0, 1.0 + 1e-9, 1.1, onp.inf, onp.inf, -onp.inf, onp.nan, onp.nan, 0.0, 1e-9])
+    y = onp.array([1.0, 1.0, 1.0, onp.inf, -onp.inf, -onp.inf, onp.nan, 1.0, 1e-9, 0.0])
+    for kw in ({}, {"equal_nan": True}, {"rtol": 0.2}, {"atol": 0.0, "rtol": 0.0}):
+        assert onp.array_equal(dnp.isclose(P(dnp, x), P(dnp, y), **kw).numpy(), onp.isclose(x, y, **kw)), kw
+    assert onp.array_equal(dnp.isclose(P(dnp, x.astype(F32)), 1.0).numpy(), onp.isclose(x.astype(F32), 1.0))
+    assert dnp.array_equal(A, P(dnp, a.copy())) and not dnp.array_equal(A, A + 1.0) and not dnp.array_equal(A, A[:, :3])
+    assert not dnp.array_equal(P(dnp, x), P(dnp, x)) and dnp.array_equal(P(dnp, x), P(dnp, x), equal_nan=True)
+    assert onp.array_equal(dnp.isposinf(P(dnp, x)).numpy(), onp.isposinf(x))
+    assert onp.array_equal(dnp.isneginf(P(dnp, x)).numpy(), onp.isneginf(x))
+    f = dnp.full_like(A, 2.5)
+    assert f.shape == (6, 9) and f.dtype == onp.float64 and onp.all(f.numpy() == 2.5)
+    assert dnp.full_like(P(dnp, a.astype(F32)), 1.5).numpy().dtype == F32 and dnp.empty_like(A).shape == (6, 9)
