@@ -29,7 +29,7 @@ _I64 = onp.dtype("int64")
 class DevArray:
     """n-d array in GPU memory; arithmetic is hand-written HIP kernels."""
 
-    __slots__ = ("_t", "dtype", "_borrowed")
+    __slots__ = ("_t", "dtype", "_borrowed", "_shape_tuple")
     __array_ufunc__ = None  # NumPy binary operators defer to ours (ndarray * DevArray -> __rmul__)
     __array_priority__ = 200.0
 
@@ -39,11 +39,15 @@ class DevArray:
         # True on an accumulator that shares its memory with a cotangent it was initialised from
         # (0 + g kept as g): in-place accumulation must then go to fresh memory instead
         self._borrowed = False
+        self._shape_tuple = None  # filled by the first `shape` (asked many times per launch; arrays never change)
 
     # ---- metadata ----------------------------------------------------------------------
     @property
     def shape(self):
-        return tuple(self._t.shape)
+        s = self._shape_tuple
+        if s is None:
+            s = self._shape_tuple = tuple(self._t.shape)
+        return s
 
     @property
     def ndim(self):
@@ -148,6 +152,7 @@ class LazyDevArray(DevArray):
         self._scale = scale    # Python float, representable in dtype; 1.0 = no multiply
         self._ascale = ascale  # tensor shaped like raw, or None
         self._shift = shift    # Python float or tensor shaped like raw; None = no add (x + 0.0 is not x for -0.0)
+        self._shape_tuple = None
 
     def __getattr__(self, name):
         # only reached when a slot is unset: `_t` before the value has been written out
@@ -164,7 +169,10 @@ class LazyDevArray(DevArray):
 
     @property
     def shape(self):
-        return tuple(self._raw.shape)
+        s = self._shape_tuple
+        if s is None:
+            s = self._shape_tuple = tuple(self._raw.shape)
+        return s
 
     @property
     def ndim(self):
