@@ -7,6 +7,8 @@
 // addition is not associative, so the kernel reproduces exactly that order: the caller
 // supplies the stable argsort of the destinations and the run boundaries, one thread owns
 // one (destination row, column) pair and walks its run sequentially.  No atomics.
+#include <algorithm>
+
 #include "common.h"
 
 namespace agmi {
@@ -51,42 +53,79 @@ __global__ __launch_bounds__(kBlock) void cumsum_lines(const T *__restrict__ src
     const int64_t o = line / inner, c = line - o * inner;
     const T *p = src + o * n * inner + c;
     T *q = out + o * n * inner + c;
+    // the additions form one chain, but the loads do not depend on it: fetch kLineChunk elements at once
+    constexpr int kLineChunk = 16;
     T acc = p[0];
     q[0] = acc;
-    for (int64_t k = 1; k < n; ++k) {
+    int64_t k = 1;
+    for (; k + kLineChunk <= n; k += kLineChunk) {
+        T v[kLineChunk];
+#pragma unroll
+        for (int u = 0; u < kLineChunk; ++u) v[u] = p[(k + u) * inner];
+#pragma unroll
+        for (int u = 0; u < kLineChunk; ++u) {
+            acc = acc + v[u];
+            q[(k + u) * inner] = acc;
+        }
+    }
+    for (; k < n; ++k) {
         acc = acc + p[k * inner];
         q[k * inner] = acc;
     }
 }
 
-// The same along the last axis (inner == 1): one wavefront takes 64 rows and walks them in chunks of 64
-// columns staged through LDS, so that global loads and stores run along the rows (coalesced) while each
-// lane still adds its own row's elements one after the other.
-constexpr int kScanTile = 64;
+// The same along the last axis (inner == 1): one wavefront takes kScanRows rows and walks them in chunks of
+// kScanCols columns staged through LDS, so that global loads and stores run along the rows (coalesced, all of a
+// chunk's loads in flight together) while one lane per row still adds that row's elements one after the other.
+// Few rows per wavefront and wide chunks: the chain of additions is short next to the memory latency of a
+// chunk, so throughput comes from the number of wavefronts in flight.
+constexpr int kScanRows = 16, kScanCols = 256, kScanGroups = kScanCols / 64;
 
 template <typename T>
-__global__ __launch_bounds__(kScanTile) void cumsum_rows(const T *__restrict__ src, int64_t rows, int64_t n,
-                                                         T *__restrict__ out) {
-    __shared__ T tile[kScanTile][kScanTile + 1];
+__global__ __launch_bounds__(64) void cumsum_rows(const T *__restrict__ src, int64_t rows, int64_t n,
+                                                  T *__restrict__ out) {
+    __shared__ T tile[kScanRows][kScanCols + 1];
     const int lane = threadIdx.x;
-    const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kScanTile;
-    const int live = static_cast<int>(rows - row0 < kScanTile ? rows - row0 : kScanTile);
+    const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kScanRows;
+    const int live = static_cast<int>(rows - row0 < kScanRows ? rows - row0 : kScanRows);
     T acc = T(0);
-    for (int64_t c0 = 0; c0 < n; c0 += kScanTile) {
-        const bool in_col = c0 + lane < n;
-        for (int r = 0; r < live; ++r)
-            if (in_col) tile[r][lane] = src[(row0 + r) * n + c0 + lane];
+    for (int64_t c0 = 0; c0 < n; c0 += kScanCols) {
+        {
+            T v[kScanRows * kScanGroups];
+#pragma unroll
+            for (int r = 0; r < kScanRows; ++r)
+#pragma unroll
+                for (int g = 0; g < kScanGroups; ++g) {
+                    const int64_t col = c0 + g * 64 + lane;
+                    v[r * kScanGroups + g] = (r < live && col < n) ? src[(row0 + r) * n + col] : T(0);
+                }
+#pragma unroll
+            for (int r = 0; r < kScanRows; ++r)
+#pragma unroll
+                for (int g = 0; g < kScanGroups; ++g) tile[r][g * 64 + lane] = v[r * kScanGroups + g];
+        }
         __syncthreads();
         if (lane < live) {
-            const int width = static_cast<int>(n - c0 < kScanTile ? n - c0 : kScanTile);
-            for (int j = 0; j < width; ++j) {
-                acc = (c0 == 0 && j == 0) ? tile[lane][0] : acc + tile[lane][j];
+            const int width = static_cast<int>(n - c0 < kScanCols ? n - c0 : kScanCols);
+            int j = 0;
+            if (c0 == 0) {  // the row's first element starts the chain as it is (0 + x would turn -0.0 into +0.0)
+                acc = tile[lane][0];
+                j = 1;
+            }
+#pragma unroll 8
+            for (; j < width; ++j) {
+                acc = acc + tile[lane][j];
                 tile[lane][j] = acc;
             }
         }
         __syncthreads();
-        for (int r = 0; r < live; ++r)
-            if (in_col) out[(row0 + r) * n + c0 + lane] = tile[r][lane];
+#pragma unroll
+        for (int r = 0; r < kScanRows; ++r)
+#pragma unroll
+            for (int g = 0; g < kScanGroups; ++g) {
+                const int64_t col = c0 + g * 64 + lane;
+                if (r < live && col < n) out[(row0 + r) * n + col] = tile[r][g * 64 + lane];
+            }
         __syncthreads();
     }
 }
@@ -152,6 +191,51 @@ __global__ __launch_bounds__(kBlock) void rank_sort_rows(const T *__restrict__ s
     if (sorted) sorted[row * n + before] = mine;
     if (order) order[row * n + before] = i;
     if (rank) rank[row * n + i] = before;
+}
+
+// The same count split over `slices` parts of the row (blockIdx.z), so that a long row fills the chip: every
+// block adds its partial count to rank[] with an integer atomic (exact in any order); rank[] starts at zero and
+// `place_by_rank` moves the elements once all counts are in.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void rank_count_slices(const T *__restrict__ src, int64_t n, int64_t tiles_per_slice,
+                                                            int64_t *__restrict__ rank) {
+    __shared__ T tile[kBlock];
+    const int64_t row = blockIdx.y;
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    const T *line = src + row * n;
+    const bool live = i < n;
+    const T mine = live ? line[i] : T(0);
+    const int64_t j_begin = static_cast<int64_t>(blockIdx.z) * tiles_per_slice * kBlock;
+    const int64_t j_end = j_begin + tiles_per_slice * kBlock < n ? j_begin + tiles_per_slice * kBlock : n;
+    int64_t before = 0;
+    for (int64_t j0 = j_begin; j0 < j_end; j0 += kBlock) {
+        const int64_t j = j0 + threadIdx.x;
+        tile[threadIdx.x] = j < j_end ? line[j] : T(0);
+        __syncthreads();
+        const int width = static_cast<int>(j_end - j0 < kBlock ? j_end - j0 : kBlock);
+        if (live)
+            for (int t = 0; t < width; ++t) before += ordered_before(tile[t], j0 + t, mine, i) ? 1 : 0;
+        __syncthreads();
+    }
+    if (live && before)
+        atomicAdd(reinterpret_cast<unsigned long long *>(rank + row * n + i), static_cast<unsigned long long>(before));
+}
+
+__global__ __launch_bounds__(kBlock) void zero_ranks(int64_t *__restrict__ rank, int64_t total) {
+    const int64_t e = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (e < total) rank[e] = 0;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void place_by_rank(const T *__restrict__ src, int64_t n, int64_t total,
+                                                        const int64_t *__restrict__ rank, T *__restrict__ sorted,
+                                                        int64_t *__restrict__ order) {
+    const int64_t e = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (e >= total) return;
+    const int64_t row = e / n, i = e - row * n;
+    const int64_t k = rank[e];
+    if (sorted) sorted[row * n + k] = src[e];
+    if (order) order[row * n + k] = i;
 }
 
 }  // namespace agmi
@@ -241,7 +325,7 @@ extern "C" int agmi_cumsum(int dtype, const void *src, int64_t outer, int64_t n,
         return AGMI_ERR_ARG;
     }
     const bool rows = inner == 1;
-    const int64_t blocks = rows ? ceil_div(outer, kScanTile) : ceil_div(outer * inner, kBlock);
+    const int64_t blocks = rows ? ceil_div(outer, kScanRows) : ceil_div(outer * inner, kBlock);
     if (blocks > 0x7fffffffLL) {
         set_error("cumsum: too many lines");
         return AGMI_ERR_UNSUPPORTED;
@@ -250,14 +334,14 @@ extern "C" int agmi_cumsum(int dtype, const void *src, int64_t outer, int64_t n,
     set_kernel_name(rows ? "cumsum_rows" : "cumsum_lines");
     if (dtype == AGMI_F32) {
         if (rows)
-            hipLaunchKernelGGL(cumsum_rows<float>, dim3((unsigned)blocks), dim3(kScanTile), 0, s,
+            hipLaunchKernelGGL(cumsum_rows<float>, dim3((unsigned)blocks), dim3(64), 0, s,
                                static_cast<const float *>(src), outer, n, static_cast<float *>(out));
         else
             hipLaunchKernelGGL(cumsum_lines<float>, dim3((unsigned)blocks), dim3(kBlock), 0, s,
                                static_cast<const float *>(src), outer, n, inner, static_cast<float *>(out));
     } else {
         if (rows)
-            hipLaunchKernelGGL(cumsum_rows<double>, dim3((unsigned)blocks), dim3(kScanTile), 0, s,
+            hipLaunchKernelGGL(cumsum_rows<double>, dim3((unsigned)blocks), dim3(64), 0, s,
                                static_cast<const double *>(src), outer, n, static_cast<double *>(out));
         else
             hipLaunchKernelGGL(cumsum_lines<double>, dim3((unsigned)blocks), dim3(kBlock), 0, s,
@@ -350,8 +434,32 @@ extern "C" int agmi_sort_rows(int dtype, const void *src, int64_t rows, int64_t 
                   (long long)n, (long long)kMaxSortLength);
         return AGMI_ERR_UNSUPPORTED;
     }
-    const dim3 grid((unsigned)ceil_div(n, kBlock), (unsigned)rows);
     hipStream_t s = as_stream(stream);
+    const int64_t tiles = ceil_div(n, kBlock);
+    if (rank && tiles >= 8) {
+        // long rows: the count is split over slices of the row; rank[] is both a result and the accumulator
+        const int64_t slices = std::min<int64_t>(32, tiles);
+        const int64_t tiles_per_slice = ceil_div(tiles, slices);
+        const int64_t total = rows * n;
+        const dim3 grid3((unsigned)tiles, (unsigned)rows, (unsigned)ceil_div(tiles, tiles_per_slice));
+        set_kernel_name("rank_count_slices+place_by_rank");
+        hipLaunchKernelGGL(zero_ranks, dim3((unsigned)ceil_div(total, kBlock)), dim3(kBlock), 0, s, rank, total);
+        if (dtype == AGMI_F32) {
+            hipLaunchKernelGGL(rank_count_slices<float>, grid3, dim3(kBlock), 0, s, static_cast<const float *>(src), n,
+                               tiles_per_slice, rank);
+            if (sorted || order)
+                hipLaunchKernelGGL(place_by_rank<float>, dim3((unsigned)ceil_div(total, kBlock)), dim3(kBlock), 0, s,
+                                   static_cast<const float *>(src), n, total, rank, static_cast<float *>(sorted), order);
+        } else {
+            hipLaunchKernelGGL(rank_count_slices<double>, grid3, dim3(kBlock), 0, s, static_cast<const double *>(src), n,
+                               tiles_per_slice, rank);
+            if (sorted || order)
+                hipLaunchKernelGGL(place_by_rank<double>, dim3((unsigned)ceil_div(total, kBlock)), dim3(kBlock), 0, s,
+                                   static_cast<const double *>(src), n, total, rank, static_cast<double *>(sorted), order);
+        }
+        return hip_check(hipGetLastError(), "sort_rows launch");
+    }
+    const dim3 grid((unsigned)tiles, (unsigned)rows);
     set_kernel_name("rank_sort_rows");
     if (dtype == AGMI_F32)
         hipLaunchKernelGGL(rank_sort_rows<float>, grid, dim3(kBlock), 0, s, static_cast<const float *>(src), n,

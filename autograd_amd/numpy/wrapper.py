@@ -697,19 +697,37 @@ def _positive_steps(idx, shape):
     return tuple(up), tuple(axes)
 
 
+def _in_memory_order(x, axis):
+    """``(tensor, axis, restore)`` for a kernel that wants a contiguous operand and works along one axis.
+
+    A transposed (axis-permuted) view of a contiguous array is handed over in its memory order, with the
+    axis renamed accordingly, so that no transposing copy is made; ``restore`` turns the kernel's result
+    (same layout) back into an array with ``x``'s shape.  Anything else is copied to row-major order first."""
+    x = D.plain(x)
+    t = x._t
+    if not t.is_contiguous() and t.dim() > 1 and 0 not in t.stride():
+        order = sorted(range(t.dim()), key=lambda d: -t.stride(d))
+        tm = t.permute(order)
+        if tm.is_contiguous():
+            back = [order.index(d) for d in range(t.dim())]
+            return tm, order.index(axis), lambda out: DevArray(out.permute(back), x.dtype)
+    return D.contiguous(x)._t, axis, lambda out: DevArray(out, x.dtype)
+
+
 def _reverse_axes(x, axes):
-    """``x`` reversed along ``axes`` (a new contiguous array), one copy kernel per axis."""
+    """``x`` reversed along ``axes`` (a new array), one copy kernel per axis."""
     for axis in axes:
         n = x.shape[axis]
         if n <= 1 or x.size == 0:
             continue
         if x.dtype not in D._FLOATS:
             raise NotImplementedError("reversal of non-floating arrays")
-        outer, inner = int(onp.prod(x.shape[:axis], dtype=onp.int64)), int(onp.prod(x.shape[axis + 1 :], dtype=onp.int64))
-        src = D.contiguous(D.plain(x))
-        out = D.empty(x.shape, x.dtype)
-        _lib.reverse(_lib.DTYPE_CODE[x.dtype], src._t, outer, n, inner, out._t)
-        x = out
+        src, ax, restore = _in_memory_order(x, axis)
+        shp = tuple(src.shape)
+        outer, inner = int(onp.prod(shp[:ax], dtype=onp.int64)), int(onp.prod(shp[ax + 1 :], dtype=onp.int64))
+        out = _lib.empty(shp, x.dtype)
+        _lib.reverse(_lib.DTYPE_CODE[x.dtype], src, outer, n, inner, out)
+        x = restore(out)
     return x
 
 
@@ -1026,11 +1044,14 @@ def cumsum(x, axis=None):
     if axis is None:
         x, axis = D.asarray(ravel.fun(x)), 0
     (axis,) = D.normalize_axes(axis, x.ndim)
-    src = D.contiguous(D.plain(x))
-    out = D.empty(x.shape, x.dtype)
-    outer, inner = int(onp.prod(x.shape[:axis], dtype=onp.int64)), int(onp.prod(x.shape[axis + 1 :], dtype=onp.int64))
-    _lib.cumsum(_lib.DTYPE_CODE[x.dtype], src._t, outer, x.shape[axis], inner, out._t)
-    return out
+    if x.size == 0:
+        return D.empty(x.shape, x.dtype)
+    src, ax, restore = _in_memory_order(x, axis)
+    shp = tuple(src.shape)
+    out = _lib.empty(shp, x.dtype)
+    outer, inner = int(onp.prod(shp[:ax], dtype=onp.int64)), int(onp.prod(shp[ax + 1 :], dtype=onp.int64))
+    _lib.cumsum(_lib.DTYPE_CODE[x.dtype], src, outer, shp[ax], inner, out)
+    return restore(out)
 
 
 def _split_views(ary, sections, axis, even):
@@ -1145,7 +1166,8 @@ def _sorted_lines(x, axis, want):
     i64 = onp.dtype(onp.int64)
     outs = {"sorted": D.empty(lines.shape, x.dtype) if "sorted" in want else None,
             "order": D.empty(lines.shape, i64) if "order" in want else None,
-            "rank": D.empty(lines.shape, i64) if "rank" in want else None}
+            # long rows are counted in slices that accumulate into the rank array: it is always handed over then
+            "rank": D.empty(lines.shape, i64) if "rank" in want or n >= 2048 else None}
     if lines.size:
         _lib.sort_rows(_lib.DTYPE_CODE[x.dtype], lines._t, rows, n, *(None if outs[k] is None else outs[k]._t
                                                                       for k in ("sorted", "order", "rank")))

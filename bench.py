@@ -34,7 +34,7 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing")
     ap.add_argument("--no-extras", action="store_true", help="skip the other workloads")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget for the CPU baseline sample")
-    ap.add_argument("--workload", default="bcast", choices=["bcast", "tanh", "mlp", "rnn", "rosen", "convnet"],
+    ap.add_argument("--workload", default="bcast", choices=["bcast", "tanh", "mlp", "rnn", "rosen", "convnet", "arrayfuncs"],
                     help="bcast (default) is the headline workload, BASELINE configs[1]; the others are the "
                          "remaining BASELINE configs and the convnet example, selectable for profiling")
     ap.add_argument("--graph", action="store_true",
@@ -136,6 +136,24 @@ def make_workload(name, be):
         cfg = {"workload": "examples/convnet.py LeNet stack (conv5x5x6, pool, conv5x5x16, pool, 120, 84, 10) on 28x28, "
                            "grad wrt params dict", "batch": 256, "seed": 0}
         return g, (params, X, T), cfg, "f64"
+    if name == "arrayfuncs":
+        # not a BASELINE config: the index-shaped kernels of the array-function table (running sums, reversal,
+        # triangle, roll, sort) on one 4096 x 4096 matrix and one 16384-vector, forward and cotangent
+        import numpy as onp
+
+        np = be.np
+        rs = onp.random.RandomState(0)
+        x = be.put(rs.randn(4096, 4096).astype(onp.float32))
+        v, w = be.put(rs.randn(16384).astype(onp.float32)), be.put(rs.randn(16384).astype(onp.float32))
+
+        def f(x, v):
+            y = np.cumsum(x, axis=1) * 1e-3 + np.cumsum(x, axis=0) * 1e-3
+            y = y + np.tril(x) - x[::-1] + np.roll(x, 3, axis=1) + np.fliplr(x)
+            return np.sum(y * y) + np.sum(np.sort(v) * w)
+
+        cfg = {"workload": "array functions: grad wrt (x, v) of cumsum (both axes), tril, reversed rows and columns, "
+                           "roll on x (4096,4096) and sort on v (16384,)", "seed": 0}
+        return be.grad(f, (0, 1)), (x, v), cfg, "f32"
     inp = configs.rosen_inputs()
     x, v = be.put(inp["x"]), be.put(inp["v"])
     prog = configs.rosen_program(be)

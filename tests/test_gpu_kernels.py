@@ -815,7 +815,7 @@ def test_reversals_running_sums_and_pieces_are_bit_exact(dnp, dtype):
         if x.size:
             x.flat[0] = -0.0
         same(dnp.cumsum(P(dnp, x), axis=axis), onp.cumsum(x, axis=axis))
-    same(dnp.cumsum(Q.T, axis=1), onp.cumsum(q.T, axis=1))  # a transposed view is copied first
+    same(dnp.cumsum(Q.T, axis=1), onp.cumsum(q.T, axis=1))  # a transposed view: summed in its memory order
     big = (rs.randn(300, 5000) * 1e3).astype(dtype)
     same(dnp.cumsum(P(dnp, big), axis=1), onp.cumsum(big, axis=1))
     # pieces are views of the operand
