@@ -125,3 +125,31 @@ def test_replay_of_random_programs_equals_eager():
             want = [g.numpy() for g in fun(*args)]
             for g, w in zip(got, want):
                 assert g.dtype == w.dtype and onp.array_equal(g, w, equal_nan=True), (seed, trial)
+
+
+def test_replay_of_array_functions_equals_eager():
+    """Running sums, reversals, triangles, rolls, pieces and the counting sort (with its atomically accumulated
+    ranks) launch kernels only, so they can be recorded; every replay must equal the eager evaluation bit for bit."""
+    import autograd_amd as ag
+    import autograd_amd.numpy as dnp
+
+    rs = onp.random.RandomState(17)
+    w = dnp.asarray(rs.randn(3000))
+
+    def f(x, v):
+        y = dnp.cumsum(x, axis=1) * 1e-2 + dnp.cumsum(x, axis=0) * 1e-2 + dnp.reshape(dnp.cumsum(x), x.shape) * 1e-3
+        y = y + dnp.tril(x) - x[::-1] + dnp.roll(x, 3, axis=1) + dnp.fliplr(x) + dnp.rot90(x, 2) * 0.5
+        head, tail = dnp.split(y, [7], axis=0)
+        y = dnp.concatenate([tail, head], axis=0) + dnp.trace(x) * 1e-2 + dnp.tile(x[:1], (x.shape[0], 1))
+        return dnp.sum(y * y) + dnp.sum(dnp.sort(v) * w) + dnp.sum(dnp.diff(x, axis=1) ** 2)
+
+    fun = ag.grad(f, (0, 1))
+    hx, hv = rs.randn(70, 70), rs.randn(3000)
+    graphed = ag.capture(fun, dnp.asarray(hx), dnp.asarray(hv))
+    for trial in range(3):
+        x, v = dnp.asarray(hx + 0.1 * trial * rs.randn(70, 70)), dnp.asarray(hv + trial * rs.randn(3000))
+        got = [g.numpy() for g in graphed(x, v)]
+        dnp.synchronize()
+        want = [g.numpy() for g in fun(x, v)]
+        for g, w_ in zip(got, want):
+            assert g.dtype == w_.dtype and onp.array_equal(g, w_), trial
