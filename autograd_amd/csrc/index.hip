@@ -8,6 +8,7 @@
 // supplies the stable argsort of the destinations and the run boundaries, one thread owns
 // one (destination row, column) pair and walks its run sequentially.  No atomics.
 #include <algorithm>
+#include <cstdint>
 
 #include "common.h"
 
@@ -140,6 +141,60 @@ __global__ __launch_bounds__(kBlock) void reverse_axis_kernel(const T *__restric
     const int64_t line = e / inner, c = e - line * inner;
     const int64_t o = line / n, k = line - o * n;
     out[e] = src[(o * n + (n - 1 - k)) * inner + c];
+}
+
+// 16-byte variants of the reversal: V = 16 / sizeof(T) consecutive elements per thread.  `reverse_axis_vec_inner`
+// copies V neighbours of one line position (inner % V == 0); `reverse_axis_vec_last` is the reversal of the
+// contiguous axis itself (inner == 1, n % V == 0): V results come from one aligned vector read backwards.
+template <typename T>
+struct IndexVec {
+    static constexpr int N = 16 / sizeof(T);
+    typedef T type __attribute__((ext_vector_type(N)));
+};
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void reverse_axis_vec_inner(const T *__restrict__ src, int64_t total_vecs, int64_t n,
+                                                                 int64_t inner_vecs, T *__restrict__ out) {
+    using vec_t = typename IndexVec<T>::type;
+    const int64_t e = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (e >= total_vecs) return;
+    const int64_t line = e / inner_vecs, c = e - line * inner_vecs;
+    const int64_t o = line / n, k = line - o * n;
+    reinterpret_cast<vec_t *>(out)[e] = reinterpret_cast<const vec_t *>(src)[(o * n + (n - 1 - k)) * inner_vecs + c];
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void reverse_axis_vec_last(const T *__restrict__ src, int64_t total_vecs,
+                                                                int64_t n_vecs, T *__restrict__ out) {
+    using vec_t = typename IndexVec<T>::type;
+    constexpr int V = IndexVec<T>::N;
+    const int64_t e = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (e >= total_vecs) return;
+    const int64_t o = e / n_vecs, kv = e - o * n_vecs;
+    const vec_t v = reinterpret_cast<const vec_t *>(src)[o * n_vecs + (n_vecs - 1 - kv)];
+    vec_t r;
+#pragma unroll
+    for (int j = 0; j < V; ++j) r[j] = v[V - 1 - j];
+    reinterpret_cast<vec_t *>(out)[e] = r;
+}
+
+// tril / triu with V columns per thread (cols % V == 0)
+template <typename T>
+__global__ __launch_bounds__(kBlock) void triangle_vec_kernel(const T *__restrict__ src, int64_t total_vecs, int64_t rows,
+                                                              int64_t col_vecs, int64_t k, int lower, T *__restrict__ out) {
+    using vec_t = typename IndexVec<T>::type;
+    constexpr int V = IndexVec<T>::N;
+    const int64_t e = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (e >= total_vecs) return;
+    const int64_t line = e / col_vecs, j0 = (e - line * col_vecs) * V;
+    const int64_t i = line % rows;
+    vec_t v = reinterpret_cast<const vec_t *>(src)[e];
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+        const int64_t d = j0 + j - i;
+        if (!(lower ? (d <= k) : (d >= k))) v[j] = T(0);
+    }
+    reinterpret_cast<vec_t *>(out)[e] = v;
 }
 
 // out[b, i, j] = src[b, i, j] where j - i <= k (lower) or j - i >= k (upper), else 0: numpy.tril / triu on
@@ -380,9 +435,35 @@ extern "C" int agmi_reverse(int dtype, const void *src, int64_t outer, int64_t n
     }
     const int64_t total = outer * n * inner;
     if (total == 0) return 0;
-    const int64_t blocks = plan_copy("reverse", dtype, src, out, total);
+    int64_t blocks = plan_copy("reverse", dtype, src, out, total);
     if (blocks < 0) return static_cast<int>(blocks);
     hipStream_t s = as_stream(stream);
+    {
+        const int64_t V = dtype == AGMI_F32 ? 4 : 2;
+        const bool aligned = ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+        const bool vec_inner = aligned && inner % V == 0, vec_last = aligned && inner == 1 && n % V == 0;
+        if (vec_inner || vec_last) {
+            const int64_t vecs = total / V;
+            const dim3 grid((unsigned)ceil_div(vecs, kBlock));
+            set_kernel_name(vec_inner ? "reverse_axis_vec_inner" : "reverse_axis_vec_last");
+            if (dtype == AGMI_F32) {
+                if (vec_inner)
+                    hipLaunchKernelGGL(reverse_axis_vec_inner<float>, grid, dim3(kBlock), 0, s, static_cast<const float *>(src),
+                                       vecs, n, inner / V, static_cast<float *>(out));
+                else
+                    hipLaunchKernelGGL(reverse_axis_vec_last<float>, grid, dim3(kBlock), 0, s, static_cast<const float *>(src),
+                                       vecs, n / V, static_cast<float *>(out));
+            } else {
+                if (vec_inner)
+                    hipLaunchKernelGGL(reverse_axis_vec_inner<double>, grid, dim3(kBlock), 0, s,
+                                       static_cast<const double *>(src), vecs, n, inner / V, static_cast<double *>(out));
+                else
+                    hipLaunchKernelGGL(reverse_axis_vec_last<double>, grid, dim3(kBlock), 0, s,
+                                       static_cast<const double *>(src), vecs, n / V, static_cast<double *>(out));
+            }
+            return hip_check(hipGetLastError(), "reverse launch");
+        }
+    }
     set_kernel_name("reverse_axis_kernel");
     if (dtype == AGMI_F32)
         hipLaunchKernelGGL(reverse_axis_kernel<float>, dim3((unsigned)blocks), dim3(kBlock), 0, s,
@@ -404,6 +485,22 @@ extern "C" int agmi_triangle(int dtype, const void *src, int64_t batch, int64_t 
     const int64_t blocks = plan_copy("triangle", dtype, src, out, total);
     if (blocks < 0) return static_cast<int>(blocks);
     hipStream_t s = as_stream(stream);
+    {
+        const int64_t V = dtype == AGMI_F32 ? 4 : 2;
+        const bool aligned = ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+        if (aligned && cols % V == 0) {
+            const int64_t vecs = total / V;
+            const dim3 grid((unsigned)ceil_div(vecs, kBlock));
+            set_kernel_name("triangle_vec_kernel");
+            if (dtype == AGMI_F32)
+                hipLaunchKernelGGL(triangle_vec_kernel<float>, grid, dim3(kBlock), 0, s, static_cast<const float *>(src), vecs,
+                                   rows, cols / V, k, lower, static_cast<float *>(out));
+            else
+                hipLaunchKernelGGL(triangle_vec_kernel<double>, grid, dim3(kBlock), 0, s, static_cast<const double *>(src), vecs,
+                                   rows, cols / V, k, lower, static_cast<double *>(out));
+            return hip_check(hipGetLastError(), "triangle launch");
+        }
+    }
     set_kernel_name("triangle_kernel");
     if (dtype == AGMI_F32)
         hipLaunchKernelGGL(triangle_kernel<float>, dim3((unsigned)blocks), dim3(kBlock), 0, s,

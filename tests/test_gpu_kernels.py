@@ -927,3 +927,26 @@ def test_truth_tests_and_closeness(dnp):
     f = dnp.full_like(A, 2.5)
     assert f.shape == (6, 9) and f.dtype == onp.float64 and onp.all(f.numpy() == 2.5)
     assert dnp.full_like(P(dnp, a.astype(F32)), 1.5).numpy().dtype == F32 and dnp.empty_like(A).shape == (6, 9)
+
+
+@pytest.mark.parametrize("dtype", [F32, F64])
+def test_reversal_and_triangle_vector_paths(dnp, dtype):
+    """Extents that are multiples of the 16-byte vector length take the vector kernels; offset views whose start is not
+    16-byte aligned fall back to the element kernels.  All are copies: bit-exact."""
+    rs = onp.random.RandomState(71)
+    for shape in ((8, 12), (4, 6, 8), (16, 4), (3, 8, 4), (2, 2, 2, 8), (260, 516)):
+        a = rs.randn(*shape).astype(dtype)
+        a.flat[::7] = onp.nan
+        A = P(dnp, a)
+        for axis in range(len(shape)):
+            assert onp.array_equal(dnp.flip(A, axis).numpy(), onp.flip(a, axis), equal_nan=True), (shape, axis)
+        assert onp.array_equal(dnp.flip(A).numpy(), onp.flip(a), equal_nan=True)
+        assert onp.array_equal(dnp.flip(A[1:], 0).numpy(), onp.flip(a[1:], 0), equal_nan=True)       # offset start
+        assert onp.array_equal(dnp.flip(A[..., 1:], -1).numpy(), onp.flip(a[..., 1:], -1), equal_nan=True)
+        for k in (-3, -1, 0, 1, 2, 5):
+            assert onp.array_equal(dnp.tril(A, k).numpy(), onp.where(onp.tri(*shape[-2:], k, dtype=bool), a, 0),
+                                   equal_nan=True), (shape, k)
+            assert onp.array_equal(dnp.triu(A, k).numpy(), onp.where(~onp.tri(*shape[-2:], k - 1, dtype=bool), a, 0),
+                                   equal_nan=True), (shape, k)
+            assert onp.array_equal(dnp.tril(A[1:], k).numpy(), onp.where(onp.tri(*a[1:].shape[-2:], k, dtype=bool), a[1:], 0),
+                                   equal_nan=True)
