@@ -703,15 +703,16 @@ def _in_memory_order(x, axis):
     A transposed (axis-permuted) view of a contiguous array is handed over in its memory order, with the
     axis renamed accordingly, so that no transposing copy is made; ``restore`` turns the kernel's result
     (same layout) back into an array with ``x``'s shape.  Anything else is copied to row-major order first."""
-    x = D.plain(x)
-    t = x._t
+    t = x._h()  # layout only: pending arithmetic, if any, is written out below, already in memory order
+    dtype = x.dtype
     if not t.is_contiguous() and t.dim() > 1 and 0 not in t.stride():
         order = sorted(range(t.dim()), key=lambda d: -t.stride(d))
-        tm = t.permute(order)
-        if tm.is_contiguous():
+        if t.permute(order).is_contiguous():
             back = [order.index(d) for d in range(t.dim())]
-            return tm, order.index(axis), lambda out: DevArray(out.permute(back), x.dtype)
-    return D.contiguous(x)._t, axis, lambda out: DevArray(out, x.dtype)
+            tm = D.plain(x._view(lambda u: u.permute(order)))._t
+            if tm.is_contiguous():
+                return tm, order.index(axis), lambda out: DevArray(out.permute(back), dtype)
+    return D.contiguous(D.plain(x))._t, axis, lambda out: DevArray(out, dtype)
 
 
 def _reverse_axes(x, axes):
