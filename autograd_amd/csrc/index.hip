@@ -54,8 +54,8 @@ __global__ __launch_bounds__(kBlock) void cumsum_lines(const T *__restrict__ src
     const int64_t o = line / inner, c = line - o * inner;
     const T *p = src + o * n * inner + c;
     T *q = out + o * n * inner + c;
-    // the additions form one chain, but the loads do not depend on it: fetch kLineChunk elements at once
-    constexpr int kLineChunk = 16;
+    // the additions form one chain, but the loads do not depend on it: fetch kLineChunk elements at once (the bytes in flight per thread set the rate)
+    constexpr int kLineChunk = 64;
     T acc = p[0];
     q[0] = acc;
     int64_t k = 1;
