@@ -157,6 +157,8 @@ def lib():
     L.agmi_cast.argtypes = [c_i, c_i, c_i, p_i64, p_arr, p_arr, c_p]
     L.agmi_map_reduce.restype = c_i
     L.agmi_map_reduce.argtypes = [c_i, c_i, c_i, c_i, p_i64, p_u8, p_arr, c_i, p_arr, p_d, c_p, c_sz, c_p]
+    L.agmi_map_reduce_static.restype = c_i
+    L.agmi_map_reduce_static.argtypes = [c_i, c_i, c_i, c_i, p_i64, p_u8, p_arr, c_i, p_arr, p_d, c_p]
     L.agmi_map_reduce_workspace_bytes.restype = c_sz
     L.agmi_map_reduce_workspace_bytes.argtypes = [c_i, c_i, c_i, p_i64, p_u8]
     L.agmi_gemm.restype = c_i
@@ -186,7 +188,7 @@ def lib():
 
 EXPORTS = (
     "agmi_last_error agmi_version agmi_last_kernel agmi_elementwise agmi_compare agmi_cast agmi_map_reduce "
-    "agmi_map_reduce_workspace_bytes agmi_gemm agmi_fill agmi_take_rows agmi_sort_rows agmi_cumsum agmi_reverse agmi_triangle agmi_scatter_add_rows agmi_optimizer_step "
+    "agmi_map_reduce_workspace_bytes agmi_map_reduce_static agmi_gemm agmi_fill agmi_take_rows agmi_sort_rows agmi_cumsum agmi_reverse agmi_triangle agmi_scatter_add_rows agmi_optimizer_step "
     "agmi_correlate"
 ).split()
 
@@ -469,6 +471,26 @@ def map_reduce(op, red, code, shape, reduce_mask, out, ins):
         _check(rc, "agmi_map_reduce")
     if ev is not None:
         _TIMER.end(ev, ("map_reduce", op, red), ((out,), ins))
+    return True
+
+
+STATIC_SCRATCH_BYTES = 1 << 20
+
+
+def map_reduce_static(op, red, code, shape, reduce_mask, out, ins):
+    """:func:`map_reduce` through ``agmi_map_reduce_static``: partial results are staged in the
+    library's built-in scratch array, nothing is allocated.  Raises :class:`AgmiError` when the
+    reduction's partial results exceed ``STATIC_SCRATCH_BYTES``."""
+    nd = _set_shape(shape)
+    for d, m in enumerate(reduce_mask):
+        _mask[d] = 1 if m else 0
+    _set_array(_outs[0], out)
+    n_in = _set_inputs(ins)
+    rc = _LIB.agmi_map_reduce_static(op, red, code, nd, _shape, _mask, _outs, n_in, _ins, _scalars, _stream())
+    if rc == -2:  # AGMI_ERR_UNSUPPORTED
+        return False
+    if rc:
+        _check(rc, "agmi_map_reduce_static")
     return True
 
 

@@ -15,6 +15,7 @@
 // tree over the block's 4 waves, then chunks in index order - never atomics - so results
 // are reproducible run to run.
 #include <algorithm>
+#include <mutex>
 #include <type_traits>
 
 #include "common.h"
@@ -559,13 +560,24 @@ static RedPlan plan_reduce(int64_t O, int64_t R, int64_t I, int vec, bool vec_ok
     return pl;
 }
 
+// `strict`: the workspace has a fixed size that must not change the plan (the summation tree would
+// differ from the one a roomy workspace gives); a problem whose partials do not fit is rejected.
 template <template <typename> class F, template <typename> class AccT, typename T>
 static int launch_reduce(const char *fname, const RedParams &base, bool vec_ok, void *workspace,
-                         size_t workspace_bytes, hipStream_t s) {
+                         size_t workspace_bytes, bool strict, hipStream_t s) {
     using Acc = AccT<T>;
     using acc_t = typename Acc::type;
     constexpr int VEC = RVec<T>::N;
-    const RedPlan pl = plan_reduce(base.O, base.R, base.I, VEC, vec_ok, sizeof(acc_t), sizeof(T), workspace ? workspace_bytes : 0);
+    const RedPlan pl = plan_reduce(base.O, base.R, base.I, VEC, vec_ok, sizeof(acc_t), sizeof(T),
+                                   strict ? SIZE_MAX : (workspace ? workspace_bytes : 0));
+    if (strict && pl.n_chunks > 1) {
+        const size_t need = sizeof(acc_t) * static_cast<size_t>(pl.n_chunks) * static_cast<size_t>(base.O * base.I);
+        if (need > workspace_bytes) {
+            set_error("map_reduce: this reduction stages %zu bytes of partial results; the built-in scratch holds %zu",
+                      need, workspace_bytes);
+            return AGMI_ERR_WORKSPACE;
+        }
+    }
     RedParams p = base;
     p.n_chunks = pl.n_chunks;
     p.r_chunk = pl.r_chunk;
@@ -733,6 +745,7 @@ static bool canonical_ori(const Merged &m, int n_operands, RedParams *p, int64_t
 struct RedSetup {
     RedParams p;
     bool vec_ok;
+    bool ws_strict = false;  // see launch_reduce
 };
 
 // `arity` = number of inputs of the op itself; ins[arity .. n_in) are auxiliary operands of pending maps
@@ -811,7 +824,7 @@ static int dispatch_red(const char *fname, int red, const RedSetup &st, void *ws
         return AGMI_ERR_ARG;
     }
     switch (red) {
-        case AGMI_RED_SUM: return launch_reduce<F, AccSum, T>(fname, st.p, st.vec_ok, ws, ws_bytes, s);
+        case AGMI_RED_SUM: return launch_reduce<F, AccSum, T>(fname, st.p, st.vec_ok, ws, ws_bytes, st.ws_strict, s);
         default: break;
     }
     set_error("map_reduce: reduction %d is only available with AGMI_OP_COPY", red);
@@ -821,11 +834,11 @@ static int dispatch_red(const char *fname, int red, const RedSetup &st, void *ws
 template <typename T>
 static int dispatch_red_copy(int red, const RedSetup &st, void *ws, size_t ws_bytes, hipStream_t s) {
     switch (red) {
-        case AGMI_RED_SUM: return launch_reduce<FCopy, AccSum, T>("sum", st.p, st.vec_ok, ws, ws_bytes, s);
-        case AGMI_RED_MAX: return launch_reduce<FCopy, AccMax, T>("max", st.p, st.vec_ok, ws, ws_bytes, s);
-        case AGMI_RED_MIN: return launch_reduce<FCopy, AccMin, T>("min", st.p, st.vec_ok, ws, ws_bytes, s);
-        case AGMI_RED_PROD: return launch_reduce<FCopy, AccProd, T>("prod", st.p, st.vec_ok, ws, ws_bytes, s);
-        case AGMI_RED_LOGSUMEXP: return launch_reduce<FCopy, AccLse, T>("logsumexp", st.p, st.vec_ok, ws, ws_bytes, s);
+        case AGMI_RED_SUM: return launch_reduce<FCopy, AccSum, T>("sum", st.p, st.vec_ok, ws, ws_bytes, st.ws_strict, s);
+        case AGMI_RED_MAX: return launch_reduce<FCopy, AccMax, T>("max", st.p, st.vec_ok, ws, ws_bytes, st.ws_strict, s);
+        case AGMI_RED_MIN: return launch_reduce<FCopy, AccMin, T>("min", st.p, st.vec_ok, ws, ws_bytes, st.ws_strict, s);
+        case AGMI_RED_PROD: return launch_reduce<FCopy, AccProd, T>("prod", st.p, st.vec_ok, ws, ws_bytes, st.ws_strict, s);
+        case AGMI_RED_LOGSUMEXP: return launch_reduce<FCopy, AccLse, T>("logsumexp", st.p, st.vec_ok, ws, ws_bytes, st.ws_strict, s);
         default: set_error("map_reduce: unknown reduction %d", red); return AGMI_ERR_ARG;
     }
 }
@@ -880,10 +893,10 @@ int AGMI_PART_FN(int op, int red, const RedSetup &st, void *ws, size_t ws_bytes,
 }  // namespace agmi
 
 #if AGMI_PART == 32
-extern "C" int agmi_map_reduce(int op, int red, int dtype, int ndim, const int64_t *shape,
-                               const uint8_t *reduce_axes, const agmi_array *out, int n_in,
-                               const agmi_array *ins, const double *scalars, void *workspace,
-                               size_t workspace_bytes, void *stream) {
+static int map_reduce_entry(int op, int red, int dtype, int ndim, const int64_t *shape, const uint8_t *reduce_axes,
+                            const agmi_array *out, int n_in, const agmi_array *ins, const double *scalars,
+                            void *(*workspace_of)(void *), void *workspace, size_t workspace_bytes, bool strict,
+                            void *stream) {
     int arity = op == AGMI_OP_COPY ? 1 : -1;
 #define AGMI_CASE(OP, FN) \
     if (op == OP) arity = FN<float>::NIN;
@@ -897,13 +910,63 @@ extern "C" int agmi_map_reduce(int op, int red, int dtype, int ndim, const int64
     bool empty = false;
     if (int rc = setup_reduce(ndim, shape, reduce_axes, out, arity, n_in, ins, scalars, &st, &empty)) return rc;
     if (empty) return 0;
+    st.ws_strict = strict;
     hipStream_t s = as_stream(stream);
     if (dtype != AGMI_F32 && dtype != AGMI_F64) {
         set_error("map_reduce: dtype %d is not a floating type", dtype);
         return AGMI_ERR_ARG;
     }
+    if (workspace_of) {  // resolved only once the arguments have been accepted
+        workspace = workspace_of(nullptr);
+        if (!workspace) return AGMI_ERR_WORKSPACE;
+    }
     return dtype == AGMI_F32 ? reduce_part_f32(op, red, st, workspace, workspace_bytes, s)
                              : reduce_part_f64(op, red, st, workspace, workspace_bytes, s);
+}
+
+extern "C" int agmi_map_reduce(int op, int red, int dtype, int ndim, const int64_t *shape,
+                               const uint8_t *reduce_axes, const agmi_array *out, int n_in,
+                               const agmi_array *ins, const double *scalars, void *workspace,
+                               size_t workspace_bytes, void *stream) {
+    return map_reduce_entry(op, red, dtype, ndim, shape, reduce_axes, out, n_in, ins, scalars, nullptr, workspace,
+                            workspace_bytes, false, stream);
+}
+
+// Staging memory of agmi_map_reduce_static: part of the library's device image, one copy on every
+// GPU the process uses, held until the process ends.  Two-stage reductions write every partial
+// result they later read, so nothing in it has to start at zero.
+static __device__ __align__(256) unsigned char scratch[AGMI_STATIC_SCRATCH_BYTES];
+
+// Device address of `scratch` on the current GPU.  In host code the array's name is only a handle
+// for this lookup, never an address a kernel may be given.
+static void *static_scratch(void *) {
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static void *ptr[kMaxDevices] = {};
+    int dev = -1;
+    if (hip_check(hipGetDevice(&dev), "hipGetDevice")) return nullptr;
+    if (dev < 0 || dev >= kMaxDevices) {
+        set_error("map_reduce_static: device ordinal %d out of range", dev);
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptr[dev]) {
+        void *p = nullptr;
+        if (hip_check(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)")) return nullptr;
+        if (!p) {
+            set_error("map_reduce_static: the scratch symbol has no address on device %d", dev);
+            return nullptr;
+        }
+        ptr[dev] = p;
+    }
+    return ptr[dev];
+}
+
+extern "C" int agmi_map_reduce_static(int op, int red, int dtype, int ndim, const int64_t *shape,
+                                      const uint8_t *reduce_axes, const agmi_array *out, int n_in,
+                                      const agmi_array *ins, const double *scalars, void *stream) {
+    return map_reduce_entry(op, red, dtype, ndim, shape, reduce_axes, out, n_in, ins, scalars, static_scratch, nullptr,
+                            AGMI_STATIC_SCRATCH_BYTES, true, stream);
 }
 
 extern "C" size_t agmi_map_reduce_workspace_bytes(int red, int dtype, int ndim, const int64_t *shape,

@@ -205,6 +205,23 @@ int agmi_map_reduce(int op, int red, int dtype, int ndim, const int64_t *shape,
 size_t agmi_map_reduce_workspace_bytes(int red, int dtype, int ndim, const int64_t *shape,
                                        const uint8_t *reduce_axes);
 
+/* agmi_map_reduce for callers that cannot allocate device memory (code under HIP graph capture,
+ * serving loops and harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * Same arguments and results as agmi_map_reduce given a roomy workspace (bit for bit: the
+ * summation tree is the same), but the partial results of a two-stage reduction are staged in a
+ * fixed array of AGMI_STATIC_SCRATCH_BYTES bytes that is part of the library's device image (each
+ * GPU the process uses holds its own copy until the process ends).  The call allocates and frees
+ * nothing.  A reduction whose partial results need more than that is rejected with
+ * AGMI_ERR_WORKSPACE and nothing is launched.  All calls on one GPU share the array: calls that
+ * overlap in time (different streams, or graphs replayed concurrently) race; calls on one
+ * stream are ordered and safe.  The first call on each GPU looks the array's device address up
+ * (hipGetSymbolAddress); make that call outside stream capture. */
+#define AGMI_STATIC_SCRATCH_BYTES (1u << 20)
+int agmi_map_reduce_static(int op, int red, int dtype, int ndim, const int64_t *shape,
+                           const uint8_t *reduce_axes, const agmi_array *out,
+                           int n_in, const agmi_array *ins, const double *scalars,
+                           void *stream);
+
 /* C[m,n] = alpha * sum_k A[m,k] B[k,n] + beta * C[m,n] on the matrix cores (MFMA), dtype
  * AGMI_F32 or AGMI_F64.  A and B are addressed as A[m*a_rs + k*a_cs], B[k*b_rs + n*b_cs], so
  * the transposed operands of the adjoints need no copy; C is row-major with leading
