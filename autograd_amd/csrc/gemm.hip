@@ -14,6 +14,12 @@
 // B[k=l/32][col=l%32]; accumulator register v of lane l is C[8*(v/4)+4*(l/32)+v%4][l%32].
 // fp64 16x16x4 - lane l supplies A[l%16][l/16], B[l/16][l%16]; register v is C[4*v+l/16][l%16].
 //
+// Two kernels share that scheme.  gemm_mfma stages operands through registers (any strides, both
+// precisions).  gemm_direct (fp32, operands with a unit stride and 16-byte aligned rows) lets the
+// memory pipeline write each K-slab straight into LDS (buffer_load ... lds): no staging registers,
+// no LDS store instructions, no wait for global data in the middle of the MFMA stream; a ring of
+// four slab buffers keeps three slabs in flight ahead of the matrix cores.
+//
 // Workgroup ids are dealt round-robin to the 8 XCDs (each with its own L2), so the tile
 // order is remapped: XCD x works on a contiguous range of tiles, walked in column-major
 // groups of kGroupM tile-rows, which keeps one XCD's A rows and B columns resident in its L2.
@@ -79,6 +85,9 @@ struct GemmParams {
     int splits;
     int64_t k_per_split;
     void *ws;
+    // gemm_direct only: bytes from element (0, 0) of one matrix of the batch to one past its last
+    // element (the extent of the buffer descriptor the loads are range-checked against)
+    uint32_t a_span_bytes, b_span_bytes;
 };
 
 constexpr int kGroupM = 8;
@@ -368,6 +377,278 @@ __global__ __launch_bounds__(kBlock *KS) void gemm_mfma(const GemmParams p) {
         }
 }
 
+
+// ---- direct-to-LDS kernel ------------------------------------------------------------------------
+//
+// Tile 64 x 64 x 32, 512 threads = 8 waves: two K-groups of 2 x 2 waves, each wave one 32 x 32
+// accumulator over its half of every slab (two waves per SIMD keep the matrix core fed).
+//
+// Loads.  One wave-wide `buffer_load_dwordx4 ... lds` moves 1 KB; lane e's 16 bytes land at LDS
+// offset 16 e of the chunk, so the LDS image is fixed by which global address each lane reads:
+//   x-contiguous operand (kXC): slab image [k][x], 64 x per row; chunk c = k rows 4c .. 4c+3;
+//                               lane e reads k = 4c + e/16, x = 4 (e%16)
+//   k-contiguous operand (kKC): slab image [x][k], 32 k per row in eight 16-byte groups; chunk c =
+//                               x rows 8c .. 8c+7; the group that holds k-group g of row x sits at
+//                               position g ^ (x % 8), so that the 16-byte fragment reads of 8
+//                               consecutive rows fall on 8 different bank groups
+// Wave w loads chunk w of both operands, behind two different MFMAs of the step (sixteen loads
+// issued together right after the barrier queue up in the CU's one address unit and hold back the
+// MFMAs behind them).  Out-of-range lanes (x beyond the matrix edge, k beyond this block's K range)
+// get an offset beyond the descriptor's extent: the hardware then writes zeros, which is exactly
+// the padding the product needs, so ragged edges cost one select per load and no extra code.
+// Offsets are 32-bit: operands must span less than 2 GiB (the caller checks).
+//
+// MFMA k order.  Within a group q of 8 k, instruction j (0..3) multiplies k = 8q + 4h + j in lane
+// half h: a k-contiguous operand delivers a lane's four j values with one 16-byte LDS read, an
+// x-contiguous one with four 4-byte reads at a fixed row pitch.
+//
+// Pipeline per step t (slab t):  wait until this wave's loads of slab t+1 have landed; barrier
+// (now slab t+1 is complete for everyone, and everyone is done reading slab t-1's buffer); 8 MFMAs
+// on slab t's fragments (in registers since step t-1) with, in their shadow, the loads of slab t+3
+// into slab t-1's buffer and the LDS reads of slab t+1's fragments.
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+constexpr int kDirectThreads = 512;
+constexpr uint32_t kDirectOob = 0x80000000u;  // beyond any extent the caller admits
+
+// The destination of an LDS-direct load is M0 (wave-uniform LDS byte address) + 16 * lane.  Written
+// as inline assembly so that the compiler's wait-count bookkeeping does not make every later LDS
+// read wait for all loads in flight; the kernel waits with explicit s_waitcnt vmcnt(n) instead.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"  // M0 is written on purpose: it is the load's destination register
+__device__ __forceinline__ void load_to_lds_16(v4i rsrc, uint32_t byte_offset, uint32_t lds_byte_addr) {
+    asm volatile(
+        "s_mov_b32 m0, %0\n\t"
+        "s_nop 0\n\t"
+        "buffer_load_dwordx4 %1, %2, 0 offen lds"
+        :
+        : "s"(lds_byte_addr), "v"(byte_offset), "s"(rsrc)
+        : "memory", "m0");
+}
+#pragma clang diagnostic pop
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    static_assert(N >= 0 && N < 64, "vmcnt range");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+__device__ __forceinline__ v4i raw_buffer(const void *base, uint32_t bytes) {
+    const uint64_t b = reinterpret_cast<uint64_t>(base);
+    v4i r;
+    r[0] = static_cast<int>(b & 0xffffffffu);
+    r[1] = static_cast<int>((b >> 32) & 0xffffu);  // stride 0: raw buffer, offsets checked against `bytes`
+    r[2] = static_cast<int>(bytes);
+    r[3] = 0x00020000;                             // 32-bit raw data format
+    return r;
+}
+
+template <int MODE_A, int MODE_B>
+__global__ __launch_bounds__(kDirectThreads) void gemm_direct(const GemmParams p) {
+    constexpr int BM = 64, BN = 64, BK = 32, NBUF = 4;
+    constexpr int kOpFloats = 64 * BK;         // one operand slab
+    constexpr int kBufFloats = 2 * kOpFloats;  // A then B
+    constexpr int NQ = BK / 16;                // groups of 8 k per K-group per slab
+    constexpr int G = BK / 4;                  // 16-byte groups per row of a k-contiguous operand
+    constexpr int kDist = NBUF - 1;            // slabs in flight ahead of the matrix cores
+    constexpr int kSlotA = 1, kSlotB = 5;      // MFMAs of the step the two loads are issued behind
+    __shared__ __attribute__((aligned(1024))) float lds[NBUF * kBufFloats];
+
+    const int n_tiles = p.tiles_m * p.tiles_n;
+    int bid = blockIdx.x;
+    {
+        const int per_xcd = n_tiles / kXcds;
+        if (bid < per_xcd * kXcds) bid = (bid % kXcds) * per_xcd + bid / kXcds;
+    }
+    const int group_size = kGroupM * p.tiles_n;
+    const int group = bid / group_size;
+    const int first_m = group * kGroupM;
+    const int rows_in_group = min(p.tiles_m - first_m, kGroupM);
+    const int tile_m = first_m + (bid % group_size) % rows_in_group;
+    const int tile_n = (bid % group_size) / rows_in_group;
+
+    const int64_t batch = blockIdx.y;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int kgroup = wave >> 2, quad = wave & 3;
+    const int wm0 = (quad >> 1) * 32, wn0 = (quad & 1) * 32;
+    const int64_t m0 = static_cast<int64_t>(tile_m) * BM, n0 = static_cast<int64_t>(tile_n) * BN;
+    const int r = lane & 31, h = lane >> 5;
+
+    const int64_t k_first = static_cast<int64_t>(blockIdx.z) * p.k_per_split;  // multiple of BK
+    const int64_t k_limit = min(p.K, k_first + p.k_per_split);
+    const int n_slabs = static_cast<int>((k_limit - k_first + BK - 1) / BK);
+
+    const v4i rsrc_a = raw_buffer(static_cast<const float *>(p.A) + batch * p.a_bs, p.a_span_bytes);
+    const v4i rsrc_b = raw_buffer(static_cast<const float *>(p.B) + batch * p.b_bs, p.b_span_bytes);
+
+    // this lane's 16 bytes of chunk `wave`: byte offset of slab 0, advance per slab, and how many k
+    // remain from its k position to the end of the block's range (<= 0: load zeros)
+    uint32_t off_a, off_b, step_a, step_b;
+    int krem_a, krem_b;
+    if (MODE_A == kXC) {
+        const int kl = 4 * wave + lane / 16, xl = 4 * (lane % 16);
+        off_a = static_cast<uint32_t>(((k_first + kl) * p.a_cs + (m0 + xl)) * 4);
+        step_a = static_cast<uint32_t>(BK * p.a_cs * 4);
+        krem_a = (m0 + xl < p.M) ? static_cast<int>(k_limit - k_first) - kl : 0;
+    } else {
+        const int xl = (64 / G) * wave + lane / G, k4 = (lane % G) ^ (xl & 7);
+        off_a = static_cast<uint32_t>(((m0 + xl) * p.a_rs + k_first + 4 * k4) * 4);
+        step_a = BK * 4;
+        krem_a = (m0 + xl < p.M) ? static_cast<int>(k_limit - k_first) - 4 * k4 : 0;
+    }
+    if (MODE_B == kXC) {
+        const int kl = 4 * wave + lane / 16, xl = 4 * (lane % 16);
+        off_b = static_cast<uint32_t>(((k_first + kl) * p.b_rs + (n0 + xl)) * 4);
+        step_b = static_cast<uint32_t>(BK * p.b_rs * 4);
+        krem_b = (n0 + xl < p.N) ? static_cast<int>(k_limit - k_first) - kl : 0;
+    } else {
+        const int xl = (64 / G) * wave + lane / G, k4 = (lane % G) ^ (xl & 7);
+        off_b = static_cast<uint32_t>(((n0 + xl) * p.b_cs + k_first + 4 * k4) * 4);
+        step_b = BK * 4;
+        krem_b = (n0 + xl < p.N) ? static_cast<int>(k_limit - k_first) - 4 * k4 : 0;
+    }
+    const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));  // LDS byte address
+    auto issue_a = [&](int buf) __attribute__((always_inline)) {
+        load_to_lds_16(rsrc_a, krem_a > 0 ? off_a : kDirectOob,
+                       lds_base + static_cast<uint32_t>(buf * kBufFloats + wave * 256) * 4u);
+        off_a += step_a;
+        krem_a -= BK;
+    };
+    auto issue_b = [&](int buf) __attribute__((always_inline)) {
+        load_to_lds_16(rsrc_b, krem_b > 0 ? off_b : kDirectOob,
+                       lds_base + static_cast<uint32_t>(buf * kBufFloats + kOpFloats + wave * 256) * 4u);
+        off_b += step_b;
+        krem_b -= BK;
+    };
+
+    // fragment addresses (floats within one operand slab) of this wave's groups q = NQ * kgroup + qq
+    int fa_addr[NQ], fb_addr[NQ];
+#pragma unroll
+    for (int qq = 0; qq < NQ; ++qq) {
+        const int q = NQ * kgroup + qq;
+        fa_addr[qq] = MODE_A == kXC ? (8 * q + 4 * h) * 64 + wm0 + r : (wm0 + r) * BK + (((2 * q + h) ^ (r & 7)) * 4);
+        fb_addr[qq] = MODE_B == kXC ? (8 * q + 4 * h) * 64 + wn0 + r : (wn0 + r) * BK + (((2 * q + h) ^ (r & 7)) * 4);
+    }
+    float fa[2][NQ][4], fb[2][NQ][4];
+    auto read_frag = [&](int f, int buf, int qq) __attribute__((always_inline)) {
+        const float *sa = lds + buf * kBufFloats;
+        const float *sb = sa + kOpFloats;
+        if (MODE_A == kXC) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) fa[f][qq][j] = sa[fa_addr[qq] + j * 64];
+        } else {
+            const v4f v = *reinterpret_cast<const v4f *>(sa + fa_addr[qq]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) fa[f][qq][j] = v[j];
+        }
+        if (MODE_B == kXC) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) fb[f][qq][j] = sb[fb_addr[qq] + j * 64];
+        } else {
+            const v4f v = *reinterpret_cast<const v4f *>(sb + fb_addr[qq]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) fb[f][qq][j] = v[j];
+        }
+    };
+
+    v16f acc;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+
+    // prologue: kDist slabs in flight (slabs past the end load zeros); slab 0's fragments to registers
+#pragma unroll
+    for (int d = 0; d < kDist; ++d) {
+        issue_a(d);
+        issue_b(d);
+    }
+    wait_vmcnt<(kDist - 1) * 2>();
+    __syncthreads();
+#pragma unroll
+    for (int qq = 0; qq < NQ; ++qq) read_frag(0, 0, qq);
+
+    auto step = [&](const int tb /* t % NBUF */, const int f /* t % 2 */) __attribute__((always_inline)) {
+        wait_vmcnt<(kDist - 2) * 2>();  // all but the youngest slab's two loads: slab t+1 is in LDS
+        __syncthreads();
+#pragma unroll
+        for (int qq = 0; qq < NQ; ++qq) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[f][qq][j], fb[f][qq][j], acc, 0, 0, 0);
+                const int slot = qq * 4 + j;
+                if (slot == kSlotA) issue_a((tb + kDist) % NBUF);
+                if (slot == kSlotB) issue_b((tb + kDist) % NBUF);
+                if (slot % 2 == 0 && slot / 2 < NQ) read_frag(f ^ 1, (tb + 1) % NBUF, slot / 2);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    };
+    static_assert(NBUF % 2 == 0, "the fragment register set alternates with the buffer index");
+    int t = 0;
+    for (; t + NBUF <= n_slabs; t += NBUF) {
+#pragma unroll
+        for (int d = 0; d < NBUF; ++d) step(d, d & 1);
+    }
+#pragma unroll
+    for (int d = 0; d < NBUF - 1; ++d)
+        if (t + d < n_slabs) step(d, d & 1);  // uniform across the block
+
+    // the loads still in flight (zeros for slabs past the end) must land before LDS is reused
+    wait_vmcnt<0>();
+    __syncthreads();
+    float *scratch = lds;
+    if (kgroup > 0) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) scratch[(quad * 16 + v) * 64 + lane] = acc[v];
+    }
+    __syncthreads();
+    if (kgroup > 0) return;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[v] += scratch[(quad * 16 + v) * 64 + lane];
+
+    // accumulator register v of lane (r, h) is C[8 (v/4) + 4 h + v%4][r] of the wave's 32 x 32 block
+    const int64_t col = n0 + wn0 + r;
+    const int64_t row0 = m0 + wm0 + 4 * h;
+    const bool interior = m0 + BM <= p.M && n0 + BN <= p.N;  // uniform: no per-element bounds tests
+    if (p.splits > 1) {  // raw partial tile; gemm_split_finish applies alpha / beta
+        float *W = static_cast<float *>(p.ws) + (static_cast<int64_t>(blockIdx.z) * gridDim.y + batch) * p.M * p.N +
+                   row0 * p.N + col;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int dr = 8 * (v / 4) + (v % 4);
+            if (interior || (row0 + dr < p.M && col < p.N)) W[dr * p.N] = acc[v];
+        }
+        return;
+    }
+    float *C = static_cast<float *>(p.C) + batch * p.c_bs + row0 * p.ldc + col;
+    const float alpha = static_cast<float>(p.alpha), beta = static_cast<float>(p.beta);
+    if (p.alpha != 1.0) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[v] = alpha * acc[v];
+    }
+    if (p.beta != 0.0) {
+        float old[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int dr = 8 * (v / 4) + (v % 4);
+            old[v] = (interior || (row0 + dr < p.M && col < p.N)) ? C[dr * p.ldc] : 0.f;
+        }
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[v] = acc[v] + beta * old[v];
+    }
+    if (interior) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) C[(8 * (v / 4) + (v % 4)) * p.ldc] = acc[v];
+    } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int dr = 8 * (v / 4) + (v % 4);
+            if (row0 + dr < p.M && col < p.N) C[dr * p.ldc] = acc[v];
+        }
+    }
+}
+
 // C = alpha * (sum over splits, in split order) + beta * C
 template <typename T>
 __global__ __launch_bounds__(kBlock) void gemm_split_finish(const T *__restrict__ ws, T *__restrict__ C, int splits,
@@ -474,6 +755,73 @@ static int launch_gemm(GemmParams p, int64_t batch, hipStream_t s, void *ws = nu
     return hip_check(hipGetLastError(), "gemm launch");
 }
 
+// Operand layouts gemm_direct accepts: a unit stride along x or k, the other stride a positive
+// multiple of 4 elements, and whole 16-byte groups (so a lane's group is entirely inside the
+// matrix or entirely outside).  Returns kXC, kKC or -1.
+static int direct_mode(int64_t x_stride, int64_t k_stride, int64_t X, int64_t K) {
+    if (x_stride == 1 && X % 4 == 0 && (K == 1 || (k_stride > 0 && k_stride % 4 == 0))) return kXC;
+    if (k_stride == 1 && K % 4 == 0 && (X == 1 || (x_stride > 0 && x_stride % 4 == 0))) return kKC;
+    return -1;
+}
+
+static bool aligned16(const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
+
+// fp32 product through gemm_direct; returns 1 when the operands do not qualify (nothing launched).
+static int launch_direct(GemmParams p, int64_t batch, hipStream_t s, void *ws, size_t ws_bytes) {
+    constexpr int BM = 64, BN = 64, BK = 32;
+    constexpr int64_t kMaxSpan = 0x7fff0000LL;  // 32-bit byte offsets, with room for the slabs issued past the end
+    const int mode_a = direct_mode(p.a_rs, p.a_cs, p.M, p.K);
+    const int mode_b = direct_mode(p.b_cs, p.b_rs, p.N, p.K);
+    if (mode_a < 0 || mode_b < 0) return 1;
+    if (!aligned16(p.A) || !aligned16(p.B)) return 1;
+    if (batch > 1 && (p.a_bs % 4 != 0 || p.b_bs % 4 != 0 || p.a_bs < 0 || p.b_bs < 0)) return 1;
+    const int64_t a_span = ((p.M - 1) * p.a_rs + (p.K - 1) * p.a_cs + 1) * 4;
+    const int64_t b_span = ((p.K - 1) * p.b_rs + (p.N - 1) * p.b_cs + 1) * 4;
+    if (a_span > kMaxSpan || b_span > kMaxSpan || BK * p.a_cs * 4 > kMaxSpan || BK * p.b_rs * 4 > kMaxSpan) return 1;
+    const int64_t tm = ceil_div(p.M, BM), tn = ceil_div(p.N, BN);
+    if (tm * tn > 0x7fffffffLL || batch > 65535) return 1;
+    p.a_span_bytes = static_cast<uint32_t>(a_span);
+    p.b_span_bytes = static_cast<uint32_t>(b_span);
+    p.tiles_m = static_cast<int>(tm);
+    p.tiles_n = static_cast<int>(tn);
+    p.splits = 1;
+    p.k_per_split = ceil_div(p.K, BK) * BK;
+    const int64_t tiles = tm * tn * batch;
+    if (ws != nullptr && tiles < 128 && p.K >= 8 * BK) {  // few tiles, long K: cut K across blocks
+        int64_t splits = std::min<int64_t>(ceil_div(256, tiles), p.K / (4 * BK));
+        splits = std::min<int64_t>(splits, static_cast<int64_t>(ws_bytes / (sizeof(float) * (size_t)(batch * p.M * p.N))));
+        splits = std::min<int64_t>(splits, 64);
+        if (splits > 1) {
+            p.k_per_split = ceil_div(ceil_div(p.K, splits), BK) * BK;
+            p.splits = static_cast<int>(ceil_div(p.K, p.k_per_split));
+            p.ws = ws;
+        }
+    }
+    if (p.splits > 1)
+        set_kernel_name("gemm_direct<f32,64,64,32,%s%s>+split%d", mode_name(mode_a), mode_name(mode_b), p.splits);
+    else
+        set_kernel_name("gemm_direct<f32,64,64,32,%s%s>", mode_name(mode_a), mode_name(mode_b));
+    const dim3 grid((unsigned)(tm * tn), (unsigned)batch, (unsigned)p.splits);
+    const dim3 block(kDirectThreads);
+    if (mode_a == kXC && mode_b == kXC)
+        hipLaunchKernelGGL((gemm_direct<kXC, kXC>), grid, block, 0, s, p);
+    else if (mode_a == kXC)
+        hipLaunchKernelGGL((gemm_direct<kXC, kKC>), grid, block, 0, s, p);
+    else if (mode_b == kXC)
+        hipLaunchKernelGGL((gemm_direct<kKC, kXC>), grid, block, 0, s, p);
+    else
+        hipLaunchKernelGGL((gemm_direct<kKC, kKC>), grid, block, 0, s, p);
+    if (int rc = hip_check(hipGetLastError(), "gemm launch")) return rc;
+    if (p.splits > 1) {
+        const int64_t n = batch * p.M * p.N;
+        hipLaunchKernelGGL(gemm_split_finish<float>, dim3((unsigned)ceil_div(n, kBlock)), dim3(kBlock), 0, s,
+                           static_cast<const float *>(p.ws), static_cast<float *>(p.C), p.splits, batch, p.M, p.N, p.ldc,
+                           p.c_bs, static_cast<float>(p.alpha), static_cast<float>(p.beta));
+        return hip_check(hipGetLastError(), "gemm launch");
+    }
+    return 0;
+}
+
 }  // namespace agmi
 
 using namespace agmi;
@@ -520,6 +868,10 @@ extern "C" int agmi_gemm(int dtype, int64_t batch, int64_t M, int64_t N, int64_t
         // give every CU two tiles (less L2 traffic per flop for large problems).
         const int64_t big_tiles = ceil_div(M, 128) * ceil_div(N, 128) * batch;
         if (big_tiles >= 512) return launch_gemm<MfmaF32x32, 128, 128, 16, 2, 1>(p, batch, s);
+        {
+            const int rc = launch_direct(p, batch, s, workspace, workspace_bytes);
+            if (rc != 1) return rc;  // launched (0) or failed; 1 = operands do not qualify
+        }
         return launch_gemm<MfmaF32x32, 64, 64, 32, 2, 2>(p, batch, s, workspace, workspace_bytes);
     }
     if (dtype == AGMI_F64) return launch_gemm<MfmaF64x16, 64, 64, 16, 2, 1>(p, batch, s, workspace, workspace_bytes);
