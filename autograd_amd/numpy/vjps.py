@@ -80,6 +80,10 @@ def _fused_unbroadcast(op, target_meta, *operands):
     target_shape, target_ndim, _dt, _c = target_meta
     if op == Op.COPY and _shape_of(operands[0]) == tuple(target_shape):
         return operands[0]  # add/subtract without broadcasting: the cotangent is `g` itself, no copy
+    if type(operands[-1]) is D.LseCotangent and not operands[-1].computed():
+        out = _consume_lse_cotangent(op, tuple(target_shape), operands)
+        if out is not None:
+            return out
     dt = D._float_dtype(D.result_dtype(*operands))
     shape = ()
     for x in operands:
@@ -96,6 +100,26 @@ def _fused_unbroadcast(op, target_meta, *operands):
     else:
         out = D.map_reduce(op, Red.SUM, dt, operands, axes, True, shape=shape)
     return DevArray(out._t.reshape(tuple(target_shape)), dt) if lead else out
+
+
+def _consume_lse_cotangent(op, target_shape, operands):
+    """``unbroadcast(op(*operands))`` when the cotangent (last operand) is an unwritten logsumexp cotangent
+    and the request is one its fused pass serves; None otherwise."""
+    s = operands[-1]
+    rows, cols = s.shape
+    if op == Op.COPY and target_shape in ((rows, 1), (rows,)):
+        out = s.row_sums()
+        return out if target_shape == (rows, 1) else out._view(lambda t: t.reshape(rows))
+    if op == Op.MUL and len(operands) == 2 and isinstance(operands[0], DevArray) and operands[0].dtype == s.dtype:
+        y = operands[0]
+        if target_shape == (rows, cols) and type(y) is DevArray and y.shape in ((1, cols), (cols,)):
+            return s.scaled_by(y._t.reshape(1, cols).expand(rows, cols))
+        if target_shape in ((1, cols), (cols,)) and y.shape == (rows, cols):
+            out = s.col_sums_with(y)
+            if out is not None and target_shape == (cols,):
+                out = out._view(lambda t: t.reshape(cols))
+            return out
+    return None
 
 
 def unbroadcast_f(target, f):

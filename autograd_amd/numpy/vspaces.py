@@ -152,4 +152,6 @@ class DevArrayVSpace(VSpace):
 DevArrayVSpace.register(DevArray)
 DevArrayVSpace.register(LazyDevArray)
 DevArrayVSpace.register(D.PendingProduct)
+DevArrayVSpace.register(D.LseCotangent)
+DevArrayVSpace.register(D.FusedResult)
 DevArrayVSpace.register(float)

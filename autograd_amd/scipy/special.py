@@ -4,7 +4,8 @@ Counterpart of the reference's autograd/scipy/special.py:119-147, whose forward 
 ``scipy.special.logsumexp``.  Forward: one single-pass reduction kernel over (max, scaled sum)
 pairs.  Reverse, concrete operands: one fused kernel ``g * b * exp(x - ans)`` that reads ``g``
 and ``ans`` through broadcast strides, so neither is ever materialised at full size (the
-reference materialises both).  Forward mode: the same functor fused into a sum.
+reference materialises both); for the rows of a matrix the cotangent is not written at all until
+the rules that consume it have run (``devarray.LseCotangent``).  Forward mode: the same functor fused into a sum.
 """
 
 import numbers
@@ -43,6 +44,11 @@ def _make_grad_logsumexp(ans, x, axis=None, b=1.0, keepdims=False):
             g_k = _keep(D.asarray(g), shape, axis, keepdims)
             ans_k = _keep(ans, shape, axis, keepdims)
             dt = D._float_dtype(D.result_dtype(g_k, x, ans_k))
+            if (type(b) is float and b == 1.0 and len(shape) == 2 and D.normalize_axes(axis, 2) == (1,)
+                    and D.LseCotangent.eligible(g_k, x, ans_k, dt)):
+                # rows of a matrix: the cotangent stays unwritten until its consumers are known; the usual
+                # ones (row sums, a rescaled copy, column sums of a product) then come out of one pass
+                return D.LseCotangent(g_k, x, ans_k, dt)
             return D.map_op(Op.LSE_VJP, dt, g_k, b, x, ans_k)
         g_repeated, _ = repeat_to_match_shape(g, shape, dtype, axis, keepdims)
         ans_repeated, _ = repeat_to_match_shape(ans, shape, dtype, axis, keepdims)

@@ -7,7 +7,11 @@ Workload (N=1): BASELINE.json configs[1], "Broadcast and reduction VJPs":
     one step = one grad(L, (0, 1, 2))(A, b, c) call (forward trace + backward replay), inputs
     resident in HBM before the timed region.
 metric = grad evals/sec.  `roofline` describes the kernel that takes most of the step, timed
-with HIP events on the launch stream during the timed steps; `cpu_baseline` is the CPU oracle
+with HIP events on the launch stream, once during the timed steps (`avg_launch_ms_in_timed_region`:
+the eager tracer leaves the GPU waiting for the host, so the event pair also holds the host's
+dispatch latency) and once over the same number of steps with the stream kept busy ahead of each
+step (`avg_launch_ms`, the figure `achieved` uses: the events then bracket GPU execution only, which
+is what a rocprofv3 kernel trace reports); `cpu_baseline` is the CPU oracle
 (the NumPy restatement of reference autograd) timed on this machine's host cores on a
 bounded sample of the same workload.  `extras` holds the other four workloads and the MLP
 contraction rate, measured after the timed region (never part of `value`).
@@ -57,6 +61,32 @@ def time_steps(fn, sync, steps, warmup):
     return (time.perf_counter() - t0) / steps
 
 
+class HeadStart:
+    """Keeps the launch stream busy for about ``ms`` milliseconds (fills of a 256 MiB scratch array), so that
+    the launches the host enqueues meanwhile run back to back on the GPU and HIP events around one of
+    them measure its execution, not the host's dispatch latency."""
+
+    def __init__(self):
+        import numpy as onp
+
+        from autograd_amd import _lib
+        from autograd_amd.numpy import devarray as D
+
+        self._lib = _lib
+        self.buf = D.empty((64 << 20,), onp.float32)
+        self.code = _lib.DTYPE_CODE[self.buf.dtype]
+        _lib.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(20):
+            _lib.fill(self.code, self.buf._t, 0.0)
+        _lib.synchronize()
+        self.ms_per_fill = (time.perf_counter() - t0) / 20 * 1e3
+
+    def __call__(self, ms):
+        for _ in range(max(1, int(ms / self.ms_per_fill) + 1)):
+            self._lib.fill(self.code, self.buf._t, 0.0)
+
+
 def cpu_baseline(seconds):
     """Time the CPU oracle on the same full-size workload; bounded by ``seconds``."""
     import numpy as onp
@@ -90,6 +120,45 @@ def cpu_baseline(seconds):
         "ms_per_eval_min": best * 1e3,
         "ms_per_eval_median": float(onp.median(times)) * 1e3,
     }
+
+
+def cpu_baseline_contractions(seconds):
+    """The CPU oracle on the two workloads whose time goes into BLAS (MLP and RNN gradients, full size): NumPy's
+    BLAS uses every host core it is given, so these are all-core figures; each is bounded by ``seconds`` / 2."""
+    import numpy as onp
+
+    import autograd_amd as ag
+    import oracle.anp as anp
+    from autograd_amd import configs
+
+    try:
+        from threadpoolctl import threadpool_info
+
+        blas = [f"{d.get('internal_api')} x{d.get('num_threads')}" for d in threadpool_info() if d.get("user_api") == "blas"]
+    except Exception:  # threadpoolctl is optional
+        blas = []
+    be = configs.Backend("oracle", anp, anp.logsumexp, ag.grad, ag.elementwise_grad, ag.make_hvp, ag.make_jvp,
+                         lambda a: a, onp.asarray, lambda: None)
+    out = {}
+    for name, inputs, program in (("mlp", configs.mlp_inputs, configs.mlp_program),
+                                  ("rnn", configs.rnn_inputs, configs.rnn_program)):
+        inp = inputs()
+        g = program(be)["grad"]
+        call_args = (inp["params"], inp["X"], inp["T"]) if name == "mlp" else (inp["params"], inp["inputs"], inp["targets"])
+        t0 = time.perf_counter()
+        g(*call_args)
+        first = time.perf_counter() - t0
+        times = []
+        deadline = time.perf_counter() + max(0.0, seconds / 2 - first)
+        while len(times) < 20 and (not times or time.perf_counter() + min(times) < deadline):
+            t0 = time.perf_counter()
+            g(*call_args)
+            times.append(time.perf_counter() - t0)
+        out[name] = {"value": 1.0 / min(times), "unit": "grad evals/sec", "cores": os.cpu_count(), "kind": "port",
+                     "blas_threads": blas,
+                     "sample": f"{len(times)} full-size grad evals after 1 warm-up, best of them",
+                     "ms_per_eval_min": min(times) * 1e3}
+    return out
 
 
 def make_workload(name, be):
@@ -164,18 +233,26 @@ def make_workload(name, be):
 
 def measured_traffic(kernel):
     """HBM bytes per launch of ``kernel`` from the committed rocprofv3 counter summary
-    (profiles/bcast_grad_hbm_traffic.md: FETCH_SIZE + WRITE_SIZE scaled by a plain copy), or None."""
-    path = os.path.join(ROOT, "profiles", "bcast_grad_hbm_traffic.md")
+    (profiles/bcast_grad_hbm_traffic.md: FETCH_SIZE + WRITE_SIZE scaled by a plain copy) and where the figure
+    comes from (file and the commit that last changed it); (None, None) when the file has no row for this kernel."""
+    import subprocess
+
+    rel = os.path.join("profiles", "bcast_grad_hbm_traffic.md")
     family, _, functor = kernel.partition("<")
-    functor = functor.split(">")[0]
+    functor = functor.split(">")[0].split(",")[0]
     try:
-        for line in open(path):
+        for line in open(os.path.join(ROOT, rel)):
             cells = [c.strip() for c in line.split("|")]
             if len(cells) > 8 and family in cells[1] and (not functor or functor in cells[1]):
-                return float(cells[7]) * 1e6
+                try:
+                    rev = subprocess.run(["git", "-C", ROOT, "log", "-1", "--format=%h", "--", rel], capture_output=True,
+                                         text=True, timeout=10).stdout.strip() or "unknown"
+                except (OSError, subprocess.SubprocessError):
+                    rev = "unknown"
+                return float(cells[7]) * 1e6, f"{rel} @ {rev} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not measured in this run)"
     except (OSError, ValueError):
         pass
-    return None
+    return None, None
 
 
 def main():
@@ -195,27 +272,44 @@ def main():
     def step():
         return fun(*fun_args)
 
-    # warm-up, with every launch timed once to find the kernel that dominates the step
+    # warm-up, then PROBE_STEPS steps with every launch timed (stream kept busy ahead of each step) to find
+    # the kernel that dominates the step and to report every kernel's average duration
+    PROBE_STEPS = 5
+    t0 = time.perf_counter()
     for _ in range(max(1, args.warmup)):
         step()
     be.sync()
+    host_ms = (time.perf_counter() - t0) / max(1, args.warmup) * 1e3
+    ahead = HeadStart()
     with _lib.KernelTimer() as probe:
-        step()
+        for _ in range(PROBE_STEPS):
+            be.sync()
+            ahead(1.5 * host_ms + 0.2)
+            step()
     per_kernel = probe.summary()
     dominant = max(per_kernel, key=lambda k: per_kernel[k]["ms"])
     dom_key = per_kernel[dominant]["key"]
+    dom_launches = max(1, per_kernel[dominant]["launches"] // PROBE_STEPS)
 
     # timed region: K steps bracketed by synchronise; only the dominant kernel carries events
     be.sync()
-    with _lib.KernelTimer(only={dom_key}, events=2 * args.steps * per_kernel[dominant]["launches"]) as kt:
+    with _lib.KernelTimer(only={dom_key}, events=2 * args.steps * dom_launches) as kt:
         t0 = time.perf_counter()
         for _ in range(args.steps):
             step()
         be.sync()
         elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
+    dom_eager = kt.summary()[dominant]
+    # the same K steps again, each behind a busy stream: the events bracket GPU execution only
+    with _lib.KernelTimer(only={dom_key}, events=2 * args.steps * dom_launches) as kt:
+        for _ in range(args.steps):
+            be.sync()
+            ahead(1.5 * ms_per_step + 0.2)
+            step()
+        be.sync()
     dom = kt.summary()[dominant]
-    if dominant.startswith(("gemm_mfma", "correlate")):
+    if dominant.startswith(("gemm_", "correlate")):
         achieved = dom["avg_flops"] / (dom["avg_ms"] * 1e-3) / 1e12
         # the window contraction runs on the vector ALUs, whose published fp32 peak equals the MFMA one
         roofline = {"bound": "mfma" if dominant.startswith("gemm") else "valu", "kernel": dominant, "achieved": achieved, "peak": MFMA_F32_PEAK_TFLOPS,
@@ -223,12 +317,15 @@ def main():
                     "algorithmic_flops_per_launch": dom["avg_flops"]}
     else:
         achieved = dom["avg_bytes"] / (dom["avg_ms"] * 1e-3) / 1e9
+        traffic, source = measured_traffic(dominant) if args.workload == "bcast" else (None, None)
         roofline = {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                    "frac": achieved / HBM_PEAK_GBS,
-                    "traffic": measured_traffic(dominant) if args.workload == "bcast" else None,
+                    "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "traffic_source": source,
                     "algorithmic_bytes_per_launch": dom["avg_bytes"]}
     roofline["avg_launch_ms"] = dom["avg_ms"]
+    roofline["avg_launch_ms_in_timed_region"] = dom_eager["avg_ms"]
     roofline["launches_timed"] = dom["launches"]
+    roofline["timing"] = ("HIP events on the launch stream around every launch of this kernel over `steps` steps, the stream "
+                          "kept busy ahead of each step so that the pair brackets GPU execution only")
 
     result = {
         "metric": "grad evals/sec",
@@ -246,7 +343,7 @@ def main():
         "config": config,
         "roofline": roofline,
         "kernels_per_step": {
-            name: {"launches": r["launches"], "avg_ms": round(r["avg_ms"], 5),
+            name: {"launches": r["launches"] / PROBE_STEPS, "avg_ms": round(r["avg_ms"], 5),
                    "GB/s": round(r["avg_bytes"] / (r["avg_ms"] * 1e-3) / 1e9, 1) if r["avg_ms"] > 0 else None}
             for name, r in sorted(per_kernel.items(), key=lambda kv: -kv[1]["ms"])
         },
@@ -270,6 +367,8 @@ def main():
         result["extras"] = extras(be)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args.cpu_seconds)
+        if "extras" in result:
+            result["extras"]["cpu_baselines"] = cpu_baseline_contractions(args.cpu_seconds)
     print(json.dumps(result))
 
 
@@ -319,20 +418,26 @@ def extras(be):
     ms = time_steps(lambda: g3(params3, X3, T3), be.sync, 20, 3) * 1e3
     out["mlp_grad_evals_per_sec"] = 1e3 / ms
     out["mlp_grad_graph_evals_per_sec"] = graph_rate(g3, (params3, X3, T3), be.sync, 20)
+    ahead = HeadStart()
     with _lib.KernelTimer(only={("gemm",)}) as kt:
         for _ in range(5):
+            be.sync()
+            ahead(1.5 * ms + 0.2)  # the five big contractions then run back to back with their neighbours
             g3(params3, X3, T3)
-    gemm_ms, gemm_flops = 0.0, 0.0
+    be.sync()
+    gemm_ms, gemm_flops, worst = 0.0, 0.0, None
     for name, key, ev0, ev1, nbytes, flops in kt.records:
         if flops >= 2.0 * 784 * 1024 * 1024:  # skip the three GEMMs with a 10-wide dimension (memory-bound)
+            t = ev0.elapsed_time(ev1)
             gemm_flops += flops
-    be.sync()
-    for name, key, ev0, ev1, nbytes, flops in kt.records:
-        if flops >= 2.0 * 784 * 1024 * 1024:
-            gemm_ms += ev0.elapsed_time(ev1)
+            gemm_ms += t
+            rate = flops / (t * 1e-3) / 1e12
+            worst = rate if worst is None else min(worst, rate)
     tflops = gemm_flops / (gemm_ms * 1e-3) / 1e12 if gemm_ms else 0.0
     out["mlp_gemm"] = {"bound": "mfma", "achieved": tflops, "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s",
-                       "frac": tflops / MFMA_F32_PEAK_TFLOPS, "gemms_timed": 5 * 5}
+                       "frac": tflops / MFMA_F32_PEAK_TFLOPS, "gemms_timed": 5 * 5, "slowest_single_launch_TFLOPs": worst,
+                       "timing": "HIP events around each contraction, stream kept busy ahead of each evaluation"}
+    del ahead
     # config 4: RNN, f32
     inp = configs.rnn_inputs()
     params = configs.tree_map(be.put, inp["params"])

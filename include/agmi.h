@@ -222,6 +222,45 @@ int agmi_map_reduce_static(int op, int red, int dtype, int ndim, const int64_t *
                            int n_in, const agmi_array *ins, const double *scalars,
                            void *stream);
 
+/* The cotangent of a row-wise logsumexp together with the rules that consume it, in one pass.
+ * With x[r,k] = mem[r,k] * scale * scale_vec + shift + shift_vec (the steps selected by `affine`,
+ * AGMI_AFFINE_* bits, in that order, each rounded on its own: a matrix that carries a pending map,
+ * e.g. A * b[None, :] + c[:, None]), ans[r] = logsumexp(x[r, :]) and the incoming cotangent g[r],
+ *     S[r,k] = g[r] * exp(x[r,k] - ans[r])                      autograd/scipy/special.py:123-134
+ * is never written; any of its consumers (null pointer = not wanted) is produced instead:
+ *     row_sums[r]  = sum_k S[r,k]              unbroadcast of S to an operand broadcast along the row
+ *                                              (add rule, autograd/numpy/numpy_vjps.py:77, 883-892)
+ *     scaled[r,k]  = col_factor[k] * S[r,k]    multiply rule for mem * col_factor[None, :] (79)
+ *     col_sums[k]  = sum_r mem[r,k] * S[r,k]   multiply rule for the broadcast factor (80-83, 883-892)
+ * mem is row-major with unit column stride; scale_vec / shift_vec vary along rows only (column
+ * stride 0) or along columns only (row stride 0, column stride 1); cols must be a multiple of the
+ * 16-byte vector (4 float32 / 2 float64) and at most 8192 float32 / 4096 float64.  Column sums
+ * are staged per band of rows in `workspace` (cols * ceil(rows / 64) elements always suffice) and
+ * added in a fixed order; nothing is atomic.  Returns AGMI_ERR_UNSUPPORTED for layouts outside
+ * this (the caller then forms S with AGMI_OP_LSE_VJP and reduces it with agmi_map_reduce). */
+typedef struct agmi_lse_cotangent {
+    int64_t rows, cols;
+    const void *x;              /* mem */
+    int64_t x_row_stride;
+    uint32_t affine;
+    double scale, shift;
+    const void *scale_vec;
+    int64_t scale_row_stride, scale_col_stride;
+    const void *shift_vec;
+    int64_t shift_row_stride, shift_col_stride;
+    const void *ans;
+    int64_t ans_stride;
+    const void *g;
+    int64_t g_stride;           /* 0: one value for every row */
+    void *row_sums;             /* [rows], contiguous */
+    const void *col_factor;     /* [cols], contiguous */
+    void *scaled;               /* [rows][cols] */
+    int64_t scaled_row_stride;
+    void *col_sums;             /* [cols], contiguous */
+} agmi_lse_cotangent;
+int agmi_lse_cotangent_fused(int dtype, const agmi_lse_cotangent *c, void *workspace, size_t workspace_bytes,
+                             void *stream);
+
 /* C[m,n] = alpha * sum_k A[m,k] B[k,n] + beta * C[m,n] on the matrix cores (MFMA), dtype
  * AGMI_F32 or AGMI_F64.  A and B are addressed as A[m*a_rs + k*a_cs], B[k*b_rs + n*b_cs], so
  * the transposed operands of the adjoints need no copy; C is row-major with leading

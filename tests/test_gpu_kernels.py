@@ -950,3 +950,141 @@ def test_reversal_and_triangle_vector_paths(dnp, dtype):
                                    equal_nan=True), (shape, k)
             assert onp.array_equal(dnp.tril(A[1:], k).numpy(), onp.where(onp.tri(*a[1:].shape[-2:], k, dtype=bool), a[1:], 0),
                                    equal_nan=True)
+
+
+# ---- logsumexp cotangent with its consumers fused (agmi_lse_cotangent_fused) ---------------------------
+def _lse_cotangent_reference(mem, scale, svec, shift, hvec, g):
+    x = mem.astype(F64)
+    if scale is not None:
+        x = x * scale
+    if svec is not None:
+        x = x * svec
+    if shift is not None:
+        x = x + shift
+    if hvec is not None:
+        x = x + hvec
+    ans = scipy.special.logsumexp(x, axis=1, keepdims=True)
+    return ans, g * onp.exp(x - ans)
+
+
+@pytest.mark.parametrize("dtype", [F32, F64])
+@pytest.mark.parametrize("rows,cols", [(37, 8), (300, 64), (129, 1028), (1000, 4096), (64, 2)])
+def test_lse_cotangent_fused_entry_point(dnp, dtype, rows, cols):
+    import torch
+
+    from autograd_amd import _lib
+
+    if cols % (16 // onp.dtype(dtype).itemsize):
+        pytest.skip("not a whole number of 16-byte vectors")
+    rs = onp.random.RandomState(rows + cols)
+    dev = _lib.device()
+    code = _lib.DTYPE_CODE[onp.dtype(dtype)]
+    mem = rs.randn(rows, cols).astype(dtype)
+    by_col = rs.uniform(0.5, 1.5, (1, cols)).astype(dtype)
+    by_row = rs.randn(rows, 1).astype(dtype)
+    put = lambda a: torch.from_numpy(onp.ascontiguousarray(a)).to(dev)
+    t_mem, t_col, t_row = put(mem), put(by_col), put(by_row)
+    g_rows = rs.randn(rows, 1).astype(dtype)
+    layouts = [
+        ("plain", t_mem, (None, None, None, None)),
+        ("A*b+c", _lib.Affine(t_mem, 1.0, t_row.expand(rows, cols), t_col.expand(rows, cols)), (None, by_col, None, by_row)),
+        ("2A*c+b", _lib.Affine(t_mem, 2.0, t_col.expand(rows, cols), t_row.expand(rows, cols)), (2.0, by_row, None, by_col)),
+        ("-A+0.5", _lib.Affine(t_mem, -1.0, 0.5, None), (-1.0, None, 0.5, None)),
+    ]
+    for name, operand, (scale, svec, shift, hvec) in layouts:
+        for g in (g_rows, onp.full((1, 1), 0.75, dtype)):
+            ans, S = _lse_cotangent_reference(mem, scale, svec, shift, hvec, g.astype(F64))
+            t_ans = put(ans.astype(dtype))
+            t_g = put(g).expand(rows, 1)
+            for want in range(1, 8):
+                row_sums = torch.full((rows, 1), float("nan"), dtype=t_mem.dtype, device=dev) if want & 2 else None
+                scaled = torch.full((rows, cols), float("nan"), dtype=t_mem.dtype, device=dev) if want & 1 else None
+                col_sums = torch.full((1, cols), float("nan"), dtype=t_mem.dtype, device=dev) if want & 4 else None
+                assert _lib.lse_cotangent(code, operand, t_ans, t_g, row_sums=row_sums,
+                                          col_factor=t_col.reshape(cols) if want & 1 else None, scaled=scaled, col_sums=col_sums)
+                label = f"{name} want={want}"
+                if want & 1:
+                    close(scaled.cpu().numpy(), (by_col * S).astype(dtype), RT[dtype])
+                if want & 2:
+                    close(row_sums.cpu().numpy(), onp.sum(S, axis=1, keepdims=True).astype(dtype), RT[dtype])
+                if want & 4:
+                    close(col_sums.cpu().numpy(), onp.sum(mem.astype(F64) * S, axis=0, keepdims=True).astype(dtype), RT[dtype]), label
+
+
+def test_lse_cotangent_layouts_outside_the_kernel_are_reported(dnp):
+    import torch
+
+    from autograd_amd import _lib
+
+    dev = _lib.device()
+    code = _lib.DTYPE_CODE[onp.dtype(F32)]
+    ans, g = torch.zeros((6, 1), device=dev), torch.ones((6, 1), device=dev)
+    out = torch.zeros((6, 1), device=dev)
+    assert not _lib.lse_cotangent(code, torch.zeros((6, 10), device=dev), ans, g, row_sums=out)        # 10 % 4 != 0
+    assert not _lib.lse_cotangent(code, torch.zeros((6, 8200), device=dev), ans, g, row_sums=out)      # > 8192 columns
+    assert not _lib.lse_cotangent(code, torch.zeros((16, 6), device=dev).t(), ans, g, row_sums=out)    # column stride != 1
+    diag = _lib.Affine(torch.zeros((6, 8), device=dev), 1.0, None, torch.zeros((6, 8), device=dev))    # factor varies both ways
+    assert not _lib.lse_cotangent(code, diag, ans, g, row_sums=out)
+
+
+@pytest.mark.parametrize("dtype", [F32, F64])
+def test_deferred_logsumexp_cotangent_serves_any_subset_of_consumers(dnp, dtype):
+    """The rules after a row-wise logsumexp ask its cotangent for row sums, a rescaled copy and column sums of a
+    product; whichever subset a program needs, values and dtypes must be what the stored-cotangent path gives."""
+    import autograd_amd as ag
+    import oracle.anp as anp
+    from autograd_amd.numpy import devarray as D
+    from autograd_amd.scipy.special import logsumexp
+
+    rs = onp.random.RandomState(5)
+    rows, cols = 260, 72
+    A = rs.randn(rows, cols).astype(dtype)
+    b = rs.uniform(0.5, 1.5, cols).astype(dtype)
+    c = rs.randn(rows).astype(dtype)
+    w = rs.randn(rows).astype(dtype)
+
+    def programs(np_, lse):
+        return {
+            "A*b+c": (lambda A, b, c: np_.sum(lse(A * b[None, :] + c[:, None], axis=1) * w), (0, 1, 2)),
+            "A*b+c wrt b": (lambda A, b, c: np_.sum(lse(A * b[None, :] + c[:, None], axis=1)), (1,)),
+            "A*b+c wrt c,A": (lambda A, b, c: np_.sum(lse(A * b[None, :] + c[:, None], axis=1)), (2, 0)),
+            "A+c": (lambda A, b, c: np_.sum(lse(A + c[:, None], axis=1, keepdims=True)), (0, 2)),
+            "A*b": (lambda A, b, c: np_.sum(lse(A * b, axis=-1)), (0, 1)),
+            "plain": (lambda A, b, c: np_.sum(lse(A, axis=1) * w), (0,)),
+            "twice": (lambda A, b, c: np_.sum(lse(A * b[None, :] + c[:, None], axis=1)) + np_.sum(lse(A * b[None, :], axis=1) ** 2), (0, 1, 2)),
+            "axis0": (lambda A, b, c: np_.sum(lse(A * b[None, :] + c[:, None], axis=0)), (0, 1, 2)),
+            "used twice": (lambda A, b, c: np_.sum(np_.exp(lse(A * b[None, :], axis=1)[:, None] - A * b[None, :])), (0, 1)),
+        }
+
+    dev_args = (dnp.asarray(A), dnp.asarray(b), dnp.asarray(c))
+    w_host = w
+    for name in programs(anp, anp.logsumexp):
+        w = w_host
+        f_ref, argnums = programs(anp, anp.logsumexp)[name]
+        want = ag.grad(f_ref, argnums)(A, b, c)
+        w = dnp.asarray(w_host)
+        f_dev, _ = programs(dnp, logsumexp)[name]
+        got = ag.grad(f_dev, argnums)(*dev_args)
+        for gd, wr in zip(got, want):
+            assert type(gd) is D.DevArray, (name, type(gd))  # settled: no pending object leaves grad
+            close(gd.numpy(), wr, RT[dtype])
+
+
+def test_deferred_logsumexp_cotangent_survives_accumulation_and_second_order(dnp):
+    import autograd_amd as ag
+    import oracle.anp as anp
+    from autograd_amd.scipy.special import logsumexp
+
+    rs = onp.random.RandomState(9)
+    A = rs.randn(48, 16)
+    b = rs.uniform(0.5, 1.5, 16)
+
+    def make(np_, lse):
+        # b reaches the loss twice (fan-in on its cotangent), and the outer derivative traces the inner backward pass
+        f = lambda A, b: np_.sum(lse(A * b[None, :], axis=1)) + np_.sum(b * b)
+        return ag.grad(lambda A, b: np_.sum(ag.grad(f, 1)(A, b) ** 2), (0, 1))
+
+    want = make(anp, anp.logsumexp)(A, b)
+    got = make(dnp, logsumexp)(dnp.asarray(A), dnp.asarray(b))
+    for gd, wr in zip(got, want):
+        close(gd.numpy(), wr, 1e-10)
