@@ -17,7 +17,7 @@ predecessor that was not owned.
 from itertools import count
 
 from .tracer import Box, Node, getval, isbox, primitive, toposort, trace
-from .util import func, subval
+from .util import collector_paused, func, subval
 
 
 def _undefined(mode, fun, argnums):
@@ -67,10 +67,11 @@ def backward_pass(g, end_node):
     what comes back is folded into the parents' entries."""
     table = {end_node: (g, False)}
     cotangent = g
-    for node in toposort(end_node):
-        cotangent = table.pop(node)[0]
-        for parent, share in zip(node.parents, node.vjp(cotangent)):
-            table[parent] = add_outgrads(table.get(parent), share)
+    with collector_paused():
+        for node in toposort(end_node):
+            cotangent = table.pop(node)[0]
+            for parent, share in zip(node.parents, node.vjp(cotangent)):
+                table[parent] = add_outgrads(table.get(parent), share)
     return cotangent
 
 

@@ -162,6 +162,8 @@ class LazyDevArray(DevArray):
         out = _lib.empty(tuple(raw.shape), self.dtype)
         _lib.elementwise(Op.COPY, _lib.DTYPE_CODE[self.dtype], tuple(raw.shape), (out,), (self._affine(),))
         self._t = out
+        # from here on the value lives in `out`: later readers take it from there (an identity map)
+        self._raw, self._scale, self._shift, self._ascale = out, 1.0, None, None
         return out
 
     def _affine(self):
@@ -696,6 +698,30 @@ def zeros(shape, dtype=_F64):
 
 def ones(shape, dtype=_F64):
     return full(shape, 1.0, onp.dtype(dtype))
+
+
+_CONSTANTS = {}
+
+
+def constant(shape, value, dtype):
+    """An array of ``shape`` filled with ``value`` that costs no launch to make: a stride-0 view of one
+    shared element, wrapped as a pending map (``LazyDevArray``) so that kernels read it through broadcast
+    strides and only code that needs the memory itself (an in-place update, a contiguous operand) has
+    it written out, once, on its first ``_t``.  Floating dtypes only; others get a real fill."""
+    shape = (shape,) if isinstance(shape, numbers.Integral) else tuple(int(s) for s in shape)
+    dtype = onp.dtype(dtype)
+    n = 1
+    for extent in shape:
+        n *= extent
+    if dtype not in _FLOATS or n == 0 or not shape:
+        return full(shape, value, dtype)
+    key = (dtype, float(value))
+    one = _CONSTANTS.get(key)
+    if one is None:
+        if len(_CONSTANTS) > 64:
+            return full(shape, value, dtype)
+        one = _CONSTANTS[key] = full((), float(value), dtype)._t
+    return LazyDevArray(one.expand(shape), dtype, 1.0, None)
 
 
 # --------------------------------------------------------------------------------------------

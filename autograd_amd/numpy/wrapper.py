@@ -1503,15 +1503,17 @@ def isscalar(A):
 
 
 def zeros(shape, dtype=float):
-    return D.zeros(shape, dtype)
+    return D.constant(shape, 0.0, dtype)
 
 
 def ones(shape, dtype=float):
-    return D.ones(shape, dtype)
+    return D.constant(shape, 1.0, dtype)
 
 
 def full(shape, fill_value, dtype=None):
-    return D.full(shape, fill_value, dtype)
+    if dtype is None or not isinstance(fill_value, (int, float)) or isinstance(fill_value, bool):
+        return D.full(shape, fill_value, dtype)
+    return D.constant(shape, fill_value, dtype)
 
 
 def empty(shape, dtype=float):
@@ -1521,7 +1523,7 @@ def empty(shape, dtype=float):
 @notrace_primitive
 def zeros_like(a, dtype=None):
     s, _, dt, _ = _meta_of(a)
-    return D.zeros(s, dtype or dt)
+    return D.constant(s, 0.0, dtype or dt)
 
 
 @notrace_primitive
@@ -1539,7 +1541,7 @@ def empty_like(a, dtype=None):
 @notrace_primitive
 def ones_like(a, dtype=None):
     s, _, dt, _ = _meta_of(a)
-    return D.ones(s, dtype or dt)
+    return D.constant(s, 1.0, dtype or dt)
 
 
 def linspace(start, stop, num=50, endpoint=True, dtype=None):

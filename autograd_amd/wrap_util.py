@@ -9,7 +9,7 @@ those arguments).
 
 from contextlib import suppress
 
-from .util import subvals
+from .util import collector_paused, subvals
 
 __all__ = ["unary_to_nary", "wraps", "wrap_nary_f", "get_name", "get_doc"]
 
@@ -57,7 +57,8 @@ def unary_to_nary(unary_operator):
                 return fun(*subvals(args, pairs), **kwargs)
 
             x0 = args[argnum] if single else tuple(args[i] for i in argnum)
-            return unary_operator(unary_f, x0, *op_args, **op_kwargs)
+            with collector_paused():  # see util.collector_paused: tapes hold no cycles
+                return unary_operator(unary_f, x0, *op_args, **op_kwargs)
 
         return nary_f
 
