@@ -59,6 +59,17 @@ def make_vjp(fun, x):
     return (lambda g: settle(backward_pass(g, last))), value
 
 
+def make_vjp_and_batched(fun, x):
+    """One trace, two pull-backs: ``(vjp, batched_vjp, fun(x))``.  ``batched_vjp(G, n, unstack, stack)`` replays
+    the tape once for ``n`` cotangents stacked along axis 0 of ``G`` (see ``batched_backward_pass``); it is
+    None when nothing was traced."""
+    value, last = trace(VJPNode.new_root(), fun, x)
+    if last is None:
+        return (lambda g: vspace(x).zeros()), None, value
+    return ((lambda g: settle(backward_pass(g, last))),
+            (lambda G, n, unstack, stack: settle(batched_backward_pass(G, last, n, unstack, stack))), value)
+
+
 def backward_pass(g, end_node):
     """Replay the tape from ``end_node`` and return the root's cotangent.
 
@@ -79,20 +90,83 @@ def _no_cotangents(g):
     return ()
 
 
+# ---- one backward pass for a whole batch of cotangents -----------------------------------------
+# `jacobian` (reference differential_operators.py:57-73) replays the tape once per element of the
+# output, each time with a standard basis vector as the cotangent.  Here the basis vectors are
+# stacked along a new leading axis and go through the tape together: rules registered with
+# `batch_safe` accept cotangents with that extra axis (the value type's rule table says how, see
+# `BatchMode`); any other node's rule is applied to the slices one by one and the results are
+# stacked again, so every tape can be replayed this way and the number of kernel launches no longer
+# grows with the output size when all its rules are batch-safe.
+batch_safe_vjps = set()
+
+
+def batch_safe(*funs):
+    """Declare that the reverse rules of ``funs`` accept cotangents with a leading batch axis while
+    ``BatchMode.active`` is set (they raise ``NotBatchable`` for argument forms they do not cover)."""
+    batch_safe_vjps.update(funs)
+
+
+class NotBatchable(Exception):
+    """Raised by a batch-safe rule for a call it cannot treat with the batch axis in place."""
+
+
+class BatchMode:
+    """Dynamic state of a batched replay: ``active`` is 1 while a rule runs on stacked cotangents."""
+
+    active = 0
+
+
+def batched_backward_pass(G, end_node, n, unstack, stack):
+    """``backward_pass`` for ``n`` cotangents stacked along axis 0 of ``G``.  ``unstack(value, i)``
+    gives the i-th cotangent of a stacked value, ``stack(list)`` puts rule results back together (both
+    come from the value type's namespace); raises ``NotBatchable`` when a result is not stackable."""
+    table = {end_node: (G, False)}
+    cotangent = G
+    with collector_paused():
+        for node in toposort(end_node):
+            cotangent = table.pop(node)[0]
+            if not node.parents:
+                continue
+            shares = None
+            if getattr(node, "fun", None) in batch_safe_vjps:
+                BatchMode.active = 1
+                try:
+                    shares = tuple(node.vjp(cotangent))
+                except NotBatchable:
+                    shares = None
+                finally:
+                    BatchMode.active = 0
+            if shares is None:
+                per_slice = [tuple(node.vjp(unstack(cotangent, i))) for i in range(n)]
+                shares = tuple(stack([dense(row[k]) for row in per_slice]) for k in range(len(node.parents)))
+            for parent, share in zip(node.parents, shares):
+                table[parent] = add_outgrads(table.get(parent), share)
+    return cotangent
+
+
+def dense(share):
+    """A rule's result as a dense value (sparse scatter objects are added into zeros)."""
+    if type(share) in sparse_object_types:
+        return sparse_add(vspace(share), None, share)
+    return share
+
+
 class VJPNode(Node):
     """Tape node of reverse mode: its parents and the closure mapping its cotangent to theirs."""
 
-    __slots__ = ["parents", "vjp"]
+    __slots__ = ["parents", "vjp", "fun"]
 
     def __init__(self, value, fun, args, kwargs, parent_argnums, parents):
         maker = primitive_vjps.get(fun)
         if maker is None:
             raise NotImplementedError(_undefined("VJP", fun, parent_argnums))
         self.parents = parents
+        self.fun = fun  # which rule table entry made `vjp` (a batched replay asks whether it is batch-safe)
         self.vjp = maker(parent_argnums, value, args, kwargs)
 
     def initialize_root(self):
-        self.parents, self.vjp = [], _no_cotangents
+        self.parents, self.vjp, self.fun = [], _no_cotangents, None
 
 
 def defvjp_argnums(fun, vjpmaker):

@@ -86,13 +86,23 @@ def deriv(fun, x):
 @unary_to_nary
 def jacobian(fun, x):
     """Jacobian of an array-valued ``fun`` of an array (or scalar): output axes first, input axes
-    last.  One backward pass per output element, each seeded with a standard basis vector of the
-    output space (reference differential_operators.py:57-73)."""
-    pull_back, ans = core.make_vjp(fun, x)
+    last.  The reference runs one backward pass per output element, each seeded with a standard basis
+    vector of the output space (differential_operators.py:57-73); here the basis vectors go through the
+    tape together, stacked along a leading axis (``core.batched_backward_pass``), when the value type
+    offers ``stacked_standard_basis``; the per-element loop remains for value types that do not."""
+    pull_back, pull_back_all, ans = core.make_vjp_and_batched(fun, x)
     np = _anp(ans, x)
-    out_space = vspace(ans)
+    out_space, in_space = vspace(ans), vspace(x)
+    stacked_basis = getattr(out_space, "stacked_standard_basis", None)
+    if pull_back_all is not None and stacked_basis is not None and out_space.size > 0 and type(in_space) is type(out_space):
+        # all basis cotangents in ONE replay of the tape, stacked along a leading axis
+        try:
+            rows = pull_back_all(stacked_basis(), out_space.size, lambda value, i: value[i], np.stack)
+            return np.reshape(rows, out_space.shape + in_space.shape)
+        except core.NotBatchable:
+            pass
     rows = [pull_back(unit) for unit in out_space.standard_basis()]
-    return np.reshape(np.stack(rows), out_space.shape + vspace(x).shape)
+    return np.reshape(np.stack(rows), out_space.shape + in_space.shape)
 
 
 @unary_to_nary

@@ -16,6 +16,7 @@ from functools import partial
 import numpy as onp
 
 from .._lib import REDUCE_FUSABLE, Op, Red
+from ..core import BatchMode, NotBatchable, batch_safe
 from ..extend import SparseObject, VJPNode, defvjp, defvjp_argnum, primitive, register_notrace, vspace
 from ..tracer import isbox
 from ..util import func
@@ -62,11 +63,12 @@ def _shape_of(x):
 def unbroadcast(x, target_meta, broadcast_idx=0):
     """Traced form: sum ``x`` down to the shape it was broadcast from."""
     target_shape, target_ndim, _dtype, target_iscomplex = target_meta
-    while anp.ndim(x) > target_ndim:
-        x = anp.sum(x, axis=broadcast_idx)
+    lead = BatchMode.active  # 1 while cotangents carry a leading batch axis, which is never summed away
+    while anp.ndim(x) > target_ndim + lead:
+        x = anp.sum(x, axis=broadcast_idx + lead)
     for axis, size in enumerate(target_shape):
         if size == 1:
-            x = anp.sum(x, axis=axis, keepdims=True)
+            x = anp.sum(x, axis=axis + lead, keepdims=True)
     return x
 
 
@@ -78,10 +80,12 @@ def _fused_unbroadcast(op, target_meta, *operands):
     the full-size intermediate is never written.
     """
     target_shape, target_ndim, _dt, _c = target_meta
-    if op == Op.COPY and _shape_of(operands[0]) == tuple(target_shape):
+    target_shape = tuple(target_shape)
+    batch = BatchMode.active  # the cotangent (and so the broadcast of the operands) has a leading batch axis
+    if op == Op.COPY and _shape_of(operands[0])[batch:] == target_shape:
         return operands[0]  # add/subtract without broadcasting: the cotangent is `g` itself, no copy
-    if type(operands[-1]) is D.LseCotangent and not operands[-1].computed():
-        out = _consume_lse_cotangent(op, tuple(target_shape), operands)
+    if not batch and type(operands[-1]) is D.LseCotangent and not operands[-1].computed():
+        out = _consume_lse_cotangent(op, target_shape, operands)
         if out is not None:
             return out
     dt = D._float_dtype(D.result_dtype(*operands))
@@ -90,16 +94,16 @@ def _fused_unbroadcast(op, target_meta, *operands):
         s = _shape_of(x)
         if s != shape:
             shape = D.broadcast_shapes(shape, s)
-    if shape == tuple(target_shape):
+    if shape[batch:] == target_shape:
         return D.map_op(op, dt, *operands)
-    lead = len(shape) - target_ndim
-    axes = list(range(lead)) + [lead + a for a, size in enumerate(target_shape) if size == 1]
+    lead = len(shape) - target_ndim - batch
+    axes = [batch + i for i in range(lead)] + [batch + lead + a for a, size in enumerate(target_shape) if size == 1]
     if op not in REDUCE_FUSABLE:
         full = D.map_op(op, dt, *operands)
         out = D.map_reduce(Op.COPY, Red.SUM, dt, (full,), axes, True)
     else:
         out = D.map_reduce(op, Red.SUM, dt, operands, axes, True, shape=shape)
-    return DevArray(out._t.reshape(tuple(target_shape)), dt) if lead else out
+    return DevArray(out._t.reshape(shape[:batch] + target_shape), dt) if lead else out
 
 
 def _consume_lse_cotangent(op, target_shape, operands):
@@ -327,18 +331,40 @@ defvjp(
 )
 
 # ---- shape-only functions (numpy_vjps.py:192-217, 407-413, 804-812) --------------------------
-defvjp(anp.reshape, lambda ans, x, shape, order=None: lambda g: anp.reshape(g, anp.shape(x), order=order))
-defvjp(anp.ravel, lambda ans, x, order=None: lambda g: anp.reshape(g, anp.shape(x), order=order))
-defvjp(anp.expand_dims, lambda ans, x, axis: lambda g: anp.reshape(g, anp.shape(x)))
-defvjp(anp.squeeze, lambda ans, x, axis=None: lambda g: anp.reshape(g, anp.shape(x)))
-defvjp(anp.swapaxes, lambda ans, x, axis1, axis2: lambda g: anp.swapaxes(g, axis2, axis1))
-defvjp(anp.moveaxis, lambda ans, a, source, destination: lambda g: anp.moveaxis(g, destination, source))
+def _shaped_like(g, shape, order=None):
+    """The cotangent ``g`` of a reshaping function, given the operand's shape again (a leading batch axis stays)."""
+    if BatchMode.active:
+        shape = (anp.shape(g)[0],) + tuple(shape)
+    return anp.reshape(g, shape, order=order)
+
+
+defvjp(anp.reshape, lambda ans, x, shape, order=None: lambda g: _shaped_like(g, anp.shape(x), order))
+defvjp(anp.ravel, lambda ans, x, order=None: lambda g: _shaped_like(g, anp.shape(x), order))
+defvjp(anp.expand_dims, lambda ans, x, axis: lambda g: _shaped_like(g, anp.shape(x)))
+defvjp(anp.squeeze, lambda ans, x, axis=None: lambda g: _shaped_like(g, anp.shape(x)))
+def _behind_batch(axis, ndim):
+    """Axis number(s) of an ``ndim``-d operand as they are in a cotangent that has a leading batch axis."""
+    if isinstance(axis, (tuple, list)):
+        return tuple(_behind_batch(a, ndim) for a in axis)
+    return int(axis) % ndim + BatchMode.active
+
+
+defvjp(anp.swapaxes, lambda ans, x, axis1, axis2: lambda g: anp.swapaxes(
+    g, _behind_batch(axis2, anp.ndim(x)), _behind_batch(axis1, anp.ndim(x))))
+defvjp(anp.moveaxis, lambda ans, a, source, destination: lambda g: anp.moveaxis(
+    g, _behind_batch(destination, anp.ndim(a)), _behind_batch(source, anp.ndim(a))))
 
 
 def _grad_transpose(ans, x, axes=None):
-    if axes is not None:
-        axes = tuple(int(i) for i in onp.argsort(axes))
-    return lambda g: anp.transpose(g, axes)
+    nd = anp.ndim(x)
+    back = tuple(int(i) for i in onp.argsort(axes)) if axes is not None else tuple(reversed(range(nd)))
+
+    def vjp(g):
+        if BatchMode.active:
+            return anp.transpose(g, (0,) + tuple(i + 1 for i in back))
+        return anp.transpose(g, back if axes is not None else None)
+
+    return vjp
 
 
 defvjp(anp.transpose, _grad_transpose)
@@ -347,7 +373,7 @@ defvjp(anp.transpose, _grad_transpose)
 def _grad_atleast(ans, *arys):
     if len(arys) > 1:
         raise NotImplementedError("Can't handle multiple arguments yet.")
-    return lambda g: anp.reshape(g, anp.shape(arys[0]))
+    return lambda g: _shaped_like(g, anp.shape(arys[0]))
 
 
 for _f in (anp.atleast_1d, anp.atleast_2d, anp.atleast_3d):
@@ -358,7 +384,7 @@ def _grad_broadcast_to(ans, x, new_shape):
     old_shape = anp.shape(x)
     assert len(old_shape) == len(new_shape), "Can't handle extra leading dims"
     axes = tuple(i for i, (o, n) in enumerate(zip(old_shape, new_shape)) if o == 1 and n > 1)
-    return lambda g: anp.sum(g, axis=axes, keepdims=True) if axes else g
+    return lambda g: anp.sum(g, axis=tuple(a + BatchMode.active for a in axes), keepdims=True) if axes else g
 
 
 defvjp(anp.broadcast_to, _grad_broadcast_to)
@@ -379,6 +405,9 @@ def repeat_to_match_shape(g, shape, dtype, axis, keepdims):
     axes = D.normalize_axes(axis, len(shape))
     new_shape = tuple(1 if d in axes else s for d, s in enumerate(shape))
     num_reps = onp.prod(onp.array(shape)[list(axes)])
+    if BatchMode.active:  # cotangents stacked along a leading axis: it is carried along
+        n = anp.shape(g)[0]
+        new_shape, shape = (n,) + new_shape, (n,) + shape
     if isinstance(g, DevArray) and (g.dtype == dtype or g.dtype == _F64):
         # a concrete cotangent that needs no promotion: the view itself, without the two primitive calls
         return g._view(lambda t: t.reshape(new_shape).expand(shape)), num_reps
@@ -709,6 +738,10 @@ def _dot_vjp_0(ans, A, B):
     A_meta, B_meta = anp.metadata(A), anp.metadata(B)
 
     def vjp(g):
+        if BatchMode.active:  # stacked matrix cotangents: one batched product with B^T shared by the batch
+            if A_meta[1] != 2 or B_meta[1] != 2:
+                raise NotBatchable
+            return anp.astype(anp.matmul(g, anp.swapaxes(B, -1, -2)), A_meta[2])
         ts = _matrix_operands(A_meta[2], g, B) if A_meta[1] == 2 and B_meta[1] == 2 and _concrete(g, B) else None
         if ts is not None:
             return D.PendingProduct(ts[0], ts[1].t(), A_meta[2])  # added into A's accumulator by the contraction itself
@@ -721,6 +754,10 @@ def _dot_vjp_1(ans, A, B):
     A_meta, B_meta = anp.metadata(A), anp.metadata(B)
 
     def vjp(g):
+        if BatchMode.active:
+            if A_meta[1] != 2 or B_meta[1] != 2:
+                raise NotBatchable
+            return anp.astype(anp.matmul(anp.swapaxes(A, -1, -2), g), B_meta[2])
         ts = _matrix_operands(B_meta[2], A, g) if A_meta[1] == 2 and B_meta[1] == 2 and _concrete(A, g) else None
         if ts is not None:
             return D.PendingProduct(ts[0].t(), ts[1], B_meta[2])
@@ -927,11 +964,11 @@ def _grad_concatenate_args(argnum, ans, axis_args, kwargs):
     start = sum(sizes[:-1])
     idxs = [slice(None)] * anp.ndim(ans)
     idxs[axis] = slice(start, start + sizes[-1])
-    return lambda g: g[tuple(idxs)]
+    return lambda g: g[(slice(None),) * BatchMode.active + tuple(idxs)]
 
 
 defvjp_argnum(anp.concatenate_args, _grad_concatenate_args)
-defvjp_argnum(anp.array_from_args, lambda argnum, ans, args, kwargs: lambda g: g[argnum - 2])
+defvjp_argnum(anp.array_from_args, lambda argnum, ans, args, kwargs: lambda g: g[(slice(None),) * BatchMode.active + (argnum - 2,)])
 
 
 def _grad_array_from_scalar_or_array(ans, array_args, array_kwargs, scarray):
@@ -975,16 +1012,28 @@ def _grad_getitem(ans, A, idx):
     # An index that only inserts unit axes selects every element exactly once, so that scatter is
     # `zeros + g` with A's shape: the cotangent itself, reshaped (nothing is launched).
     vs = vspace(A)
+
+    def stacked(g):
+        # cotangents stacked along a leading axis: the same selection behind a full slice, scattered into a
+        # buffer with the batch axis in front (basic indices only: array indices would reorder result axes)
+        if not anp._is_basic_index(idx):
+            raise NotBatchable
+        items = idx if isinstance(idx, tuple) else (idx,)
+        wide = vspace(anp.zeros((anp.shape(g)[0],) + tuple(vs.shape), dtype=vs.dtype))
+        return untake(g, (slice(None),) + tuple(items), wide)
+
     if _only_inserts_unit_axes(idx):
         shape, dtype = vs.shape, vs.dtype
 
         def vjp(g):
+            if BatchMode.active:
+                return _shaped_like(g, shape) if isinstance(g, DevArray) and g.dtype == dtype else stacked(g)
             if isinstance(g, DevArray) and g.dtype == dtype:
                 return anp.reshape.fun(g, shape)
             return untake(g, idx, vs)
 
         return vjp
-    return lambda g: untake(g, idx, vs)
+    return lambda g: stacked(g) if BatchMode.active else untake(g, idx, vs)
 
 
 defvjp(func(DevArrayBox.__getitem__), _grad_getitem)
@@ -1004,3 +1053,20 @@ def pad_vjp(ans, array, pad_width, mode, **kwargs):
 
 
 defvjp(anp.pad, pad_vjp)
+
+
+# ---- rules that take cotangents stacked along a leading batch axis (core.batched_backward_pass) --------
+# Elementwise rules broadcast the saved operands against the stacked cotangent as they are; the helpers
+# they share (unbroadcast, repeat_to_match_shape, _shaped_like) leave the batch axis alone while
+# BatchMode.active is set.  Everything not listed is replayed slice by slice.
+batch_safe(
+    anp.add, anp.subtract, anp.multiply, anp.true_divide, anp.power, anp.maximum, anp.minimum, anp.fmax, anp.fmin,
+    anp.negative, anp.exp, anp.log, anp.tanh, anp.sinh, anp.cosh, anp.sin, anp.cos, anp.sqrt, anp.square,
+    anp.reciprocal, anp.log1p, anp.expm1, anp.abs, anp.fabs, anp.logaddexp, anp.logaddexp2, anp.sinc, anp.remainder,
+    anp.arctan2, anp.hypot, anp.exp2, anp.log2, anp.log10, anp.tan, anp.arcsin, anp.arccos, anp.arctan, anp.arcsinh,
+    anp.arccosh, anp.arctanh, anp.rad2deg, anp.deg2rad, anp.clip, anp.nan_to_num, anp._where3, anp.astype,
+    anp.reshape, anp.ravel, anp.expand_dims, anp.squeeze, anp.sum, anp._primitive_mean, anp.dot,
+    anp.real, anp.real_if_close, anp.conjugate, anp.swapaxes, anp.moveaxis, anp.transpose, anp.atleast_1d,
+    anp.atleast_2d, anp.atleast_3d, anp.broadcast_to, func(DevArrayBox.__getitem__), anp.concatenate_args,
+    anp.array_from_args,
+)

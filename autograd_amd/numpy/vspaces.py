@@ -99,6 +99,14 @@ class DevArrayVSpace(VSpace):
             _lib.fill(_lib.DTYPE_CODE[self.dtype], cell, 1.0)  # a single element is always contiguous
             yield vect
 
+    def stacked_standard_basis(self):
+        """All ``size`` standard basis vectors stacked along a new leading axis: an identity matrix viewed
+        as ``(size,) + shape`` (one launch instead of ``size`` fills)."""
+        from . import wrapper as anp
+
+        eye = anp.eye(self.size, dtype=self.dtype)
+        return eye._view(lambda t: t.reshape((self.size,) + tuple(self.shape)))
+
     def randn(self):
         # host RNG (numpy.random, as the reference) so seeded tests see the same draws
         return D.from_numpy(onp.array(onp.random.randn(*self.shape)).astype(self.dtype))

@@ -11,6 +11,7 @@ the rules that consume it have run (``devarray.LseCotangent``).  Forward mode: t
 import numbers
 
 from .._lib import Op, Red
+from ..core import BatchMode, batch_safe
 from ..extend import defjvp, defvjp, primitive
 from ..numpy import devarray as D
 from ..numpy import wrapper as np
@@ -40,6 +41,12 @@ def _make_grad_logsumexp(ans, x, axis=None, b=1.0, keepdims=False):
     shape, dtype = np.shape(x), np.result_type(x)
 
     def vjp(g):
+        if BatchMode.active:
+            # cotangents stacked along a leading axis: plain broadcasting against the kept-dims form of `ans`
+            g_repeated, _ = repeat_to_match_shape(g, shape, dtype, axis, keepdims)
+            axes = D.normalize_axes(axis, len(shape))
+            ans_kept = ans if keepdims or not shape else np.reshape(ans, tuple(1 if d in axes else n for d, n in enumerate(shape)))
+            return g_repeated * b * np.exp(x - ans_kept)
         if _concrete(g, ans, x, b):
             g_k = _keep(D.asarray(g), shape, axis, keepdims)
             ans_k = _keep(ans, shape, axis, keepdims)
@@ -58,6 +65,7 @@ def _make_grad_logsumexp(ans, x, axis=None, b=1.0, keepdims=False):
 
 
 defvjp(logsumexp, _make_grad_logsumexp)
+batch_safe(logsumexp)
 
 
 def _fwd_grad_logsumexp(g, ans, x, axis=None, b=1.0, keepdims=False):
