@@ -599,8 +599,10 @@ def cumsum(code, src, outer, n, inner, out):
 
 
 def scatter_add_rows(code, dst, n_rows, inner, src, index, order, seg_start, n_seg):
+    """``seg_start`` None: the runs of equal destination are found on the device and ``n_seg`` counts index entries."""
     _check(_LIB.agmi_scatter_add_rows(code, dst.data_ptr(), n_rows, inner, src.data_ptr(), index.data_ptr(),
-                                      order.data_ptr(), seg_start.data_ptr(), n_seg, _stream()),
+                                      order.data_ptr(), None if seg_start is None else seg_start.data_ptr(), n_seg,
+                                      _stream()),
            "agmi_scatter_add_rows")
 
 

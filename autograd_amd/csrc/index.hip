@@ -26,6 +26,35 @@ __global__ __launch_bounds__(kBlock) void take_rows_kernel(const T *__restrict__
     out[e] = src[r * inner + c];
 }
 
+// The same accumulation when the runs of equal destination are not listed: one thread per position of the
+// sorted order (and column); a thread whose position starts a run (its destination differs from the
+// previous position's) adds the whole run in order, the others leave.  Nothing about the index has to be
+// known on the host, so the call can be recorded into a graph with a device-resident index.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void scatter_add_runs_kernel(T *__restrict__ dst, int64_t n_rows, int64_t inner,
+                                                                  const T *__restrict__ src,
+                                                                  const int64_t *__restrict__ index,
+                                                                  const int64_t *__restrict__ order, int64_t n_index) {
+    const int64_t e = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (e >= n_index * inner) return;
+    const int64_t pos = e / inner, c = e - pos * inner;
+    int64_t r = index[order[pos]];
+    if (r < 0) r += n_rows;
+    if (pos > 0) {
+        int64_t before = index[order[pos - 1]];
+        if (before < 0) before += n_rows;
+        if (before == r) return;  // inside a run: its first position does the work
+    }
+    T acc = dst[r * inner + c];
+    for (int64_t k = pos; k < n_index; ++k) {
+        int64_t rk = index[order[k]];
+        if (rk < 0) rk += n_rows;
+        if (rk != r) break;
+        acc = acc + src[order[k] * inner + c];
+    }
+    dst[r * inner + c] = acc;
+}
+
 template <typename T>
 __global__ __launch_bounds__(kBlock) void scatter_add_rows_kernel(T *__restrict__ dst, int64_t n_rows, int64_t inner,
                                                                   const T *__restrict__ src,
@@ -338,8 +367,12 @@ extern "C" int agmi_scatter_add_rows(int dtype, void *dst, int64_t n_rows, int64
     }
     const int64_t n = n_seg * inner;
     if (n == 0) return 0;
-    if (!dst || !src || !index || !order || !seg_start) {
+    if (!dst || !src || !index || !order) {
         set_error("scatter_add_rows: null operand");
+        return AGMI_ERR_ARG;
+    }
+    if (dtype != AGMI_F32 && dtype != AGMI_F64) {
+        set_error("scatter_add_rows: dtype %d is not a floating type", dtype);
         return AGMI_ERR_ARG;
     }
     const int64_t blocks = ceil_div(n, kBlock);
@@ -348,19 +381,25 @@ extern "C" int agmi_scatter_add_rows(int dtype, void *dst, int64_t n_rows, int64
         return AGMI_ERR_UNSUPPORTED;
     }
     hipStream_t s = as_stream(stream);
+    if (!seg_start) {  // runs found on the device: n_seg counts index entries
+        set_kernel_name("scatter_add_runs_kernel");
+        if (dtype == AGMI_F32)
+            hipLaunchKernelGGL(scatter_add_runs_kernel<float>, dim3((unsigned)blocks), dim3(kBlock), 0, s,
+                               static_cast<float *>(dst), n_rows, inner, static_cast<const float *>(src), index, order, n_seg);
+        else
+            hipLaunchKernelGGL(scatter_add_runs_kernel<double>, dim3((unsigned)blocks), dim3(kBlock), 0, s,
+                               static_cast<double *>(dst), n_rows, inner, static_cast<const double *>(src), index, order, n_seg);
+        return hip_check(hipGetLastError(), "scatter_add_rows launch");
+    }
     set_kernel_name("scatter_add_rows_kernel");
     if (dtype == AGMI_F32)
         hipLaunchKernelGGL(scatter_add_rows_kernel<float>, dim3((unsigned)blocks), dim3(kBlock), 0, s,
                            static_cast<float *>(dst), n_rows, inner, static_cast<const float *>(src), index, order,
                            seg_start, n_seg);
-    else if (dtype == AGMI_F64)
+    else
         hipLaunchKernelGGL(scatter_add_rows_kernel<double>, dim3((unsigned)blocks), dim3(kBlock), 0, s,
                            static_cast<double *>(dst), n_rows, inner, static_cast<const double *>(src), index, order,
                            seg_start, n_seg);
-    else {
-        set_error("scatter_add_rows: dtype %d is not a floating type", dtype);
-        return AGMI_ERR_ARG;
-    }
     return hip_check(hipGetLastError(), "scatter_add_rows launch");
 }
 

@@ -646,25 +646,105 @@ def _plain(idx):
                  else (int(i) if isinstance(i, (numbers.Integral, onp.integer)) else i) for i in items)
 
 
-def _host_index(idx):
-    """1-d int64 host array for an integer-array index on the leading axis, else None."""
-    if isinstance(idx, list):
-        if len(idx) and isinstance(idx[0], slice):
+_INDEX_PLANS = {}
+_INDEX_PLAN_LIMIT = 512
+
+
+def _index_key(idx):
+    """Hashable identity of an index made of host data (ints, slices, None, Ellipsis, lists, NumPy arrays);
+    None when it holds anything else (a device array)."""
+    items = idx if isinstance(idx, tuple) else (idx,)
+    key = []
+    for it in items:
+        if it is None or it is Ellipsis or isinstance(it, (int, onp.integer, bool, onp.bool_)):
+            key.append(it)
+        elif isinstance(it, slice):
+            key.append(("s", it.start, it.stop, it.step))
+        elif isinstance(it, (list, onp.ndarray)):
+            arr = onp.asarray(it)
+            if arr.dtype.kind not in "iub":
+                raise IndexError("arrays used as indices must be of integer (or boolean) type")
+            key.append(("a", arr.shape, arr.dtype.str, arr.tobytes()))
+        else:
             return None
-        arr = onp.asarray(idx)
-    elif isinstance(idx, onp.ndarray):
-        arr = idx
-    elif isinstance(idx, DevArray):
-        arr = idx.numpy()
-    else:
-        return None
-    if arr.dtype == bool:
-        arr = onp.nonzero(arr)[0]
-    if arr.size == 0:
-        arr = arr.astype(onp.int64)
-    if arr.dtype.kind not in "iu" or arr.ndim != 1:
-        return None
-    return arr.astype(onp.int64)
+    return (isinstance(idx, tuple), tuple(key))
+
+
+def _to_host_index(idx):
+    """``idx`` with lists turned into NumPy arrays (an empty one is an empty INTEGER index, as NumPy reads it)
+    and device arrays brought to the host (a synchronising transfer: their VALUES decide which elements are
+    taken, and for boolean masks even how many)."""
+    def one(it):
+        if isinstance(it, DevArray):
+            return it.numpy()
+        if isinstance(it, list):
+            if builtins.any(isinstance(e, DevArray) for e in it):
+                it = [e.numpy() if isinstance(e, DevArray) else e for e in it]
+            arr = onp.asarray(it)
+            return arr.astype(onp.int64) if arr.size == 0 else arr
+        return it
+
+    return tuple(one(it) for it in idx) if isinstance(idx, tuple) else one(idx)
+
+
+def _flat_positions(shape, idx):
+    """int64 array shaped like ``A[idx]`` (for ``A`` of ``shape``) holding the flat (row-major) position in ``A``
+    of every selected element.  NumPy itself applies the index, to stride-0 views of the axis coordinates: that
+    costs memory for the RESULT only and brings NumPy's indexing rules along (broadcast of index arrays, where
+    their axes land in the result, boolean masks, out-of-range errors)."""
+    flat = None
+    stride = 1
+    strides = []
+    for extent in reversed(shape):
+        strides.append(stride)
+        stride *= extent
+    strides.reverse()
+    for axis, extent in enumerate(shape):
+        coords = onp.arange(extent, dtype=onp.int64).reshape((1,) * axis + (extent,) + (1,) * (len(shape) - axis - 1))
+        picked = onp.broadcast_to(coords, shape)[idx]
+        flat = picked * strides[axis] if flat is None else flat + picked * strides[axis]
+    if flat is None:  # 0-d array: only (), ... and None can index it
+        flat = onp.zeros((), dtype=onp.int64)[idx]
+    return onp.asarray(flat, dtype=onp.int64, order="C")
+
+
+class _IndexPlan:
+    """What ``A[idx]`` with an advanced index selects from an array of one shape: the flat position in ``A`` of
+    every element of the result, resident on the device, and the stable order of those positions that the
+    ordered scatter of the cotangent needs.  Built once per (shape, index) and kept, so repeated evaluations
+    and recorded graphs do no host work and no transfers for it."""
+
+    __slots__ = ("shape", "positions", "n", "_order")
+
+    def __init__(self, shape, idx):
+        flat = _flat_positions(shape, idx)
+        self.shape = flat.shape
+        self.n = flat.size
+        self.positions = D.from_numpy(flat.reshape(-1))
+        # equal destinations keep their order of appearance, which is the order numpy.add.at adds them in
+        self._order = D.from_numpy(onp.argsort(flat.reshape(-1), kind="stable").astype(onp.int64))
+
+    def order(self):
+        return self._order
+
+
+def _index_plan(shape, idx):
+    idx = _to_host_index(idx)
+    key = (tuple(shape), _index_key(idx))
+    plan = _INDEX_PLANS.get(key)
+    if plan is None:
+        if len(_INDEX_PLANS) >= _INDEX_PLAN_LIMIT:
+            _INDEX_PLANS.clear()
+        plan = _INDEX_PLANS[key] = _IndexPlan(tuple(shape), idx)
+    return plan
+
+
+def _device_rows(idx):
+    """The index when it is a device-resident 1-d integer array (rows of the leading axis, chosen by data that
+    never leaves the device); None otherwise."""
+    if isinstance(idx, DevArray) and idx.ndim == 1 and idx.dtype in (D._I64, onp.dtype("int32")):
+        return idx if idx.dtype == D._I64 else D.astype(idx, D._I64)
+    return None
 
 
 def _positive_steps(idx, shape):
@@ -732,33 +812,34 @@ def _reverse_axes(x, axes):
     return x
 
 
+def _gather(A, positions, n_rows, inner, out_shape):
+    if A.dtype not in D._FLOATS:
+        raise NotImplementedError("gather of non-floating arrays")
+    src = D.contiguous(A)
+    out = D.empty(out_shape, A.dtype)
+    if out.size:
+        _lib.take_rows(_lib.DTYPE_CODE[A.dtype], src._t, n_rows, inner, positions._t, positions.size, out._t)
+    return out
+
+
 def take(A, idx):
-    """``A[idx]``: views for basic indices (plus one gather per axis sliced backwards), a gather kernel for an
-    integer array on axis 0."""
+    """``A[idx]``: views for basic indices (plus one gather per axis sliced backwards); one gather kernel for
+    every other NumPy index form (integer arrays and lists on any axes, mixed with slices and integers, boolean
+    masks), driven by a device-resident table of flat positions that is built once per (shape, index)."""
     if _is_basic_index(idx):
         pidx, backwards = _positive_steps(_plain(idx), A.shape)
         picked = A._view(lambda t: t[pidx])
         return _reverse_axes(picked, backwards) if backwards else picked
-    rows = _host_index(idx)
-    if rows is None:
-        raise NotImplementedError(
-            f"index {idx!r}: only basic indexing and a 1-d integer array on the leading axis are supported on the device"
-        )
     if A.ndim == 0:
         raise IndexError("too many indices for array")
-    n_rows = A.shape[0]
-    if rows.size and (rows.max() >= n_rows or rows.min() < -n_rows):
-        raise IndexError(f"index out of bounds for axis 0 with size {n_rows}")
-    src = D.contiguous(A)
-    inner = 1
-    for s in A.shape[1:]:
-        inner *= s
-    out = D.empty((rows.size,) + A.shape[1:], A.dtype)
-    if A.dtype not in D._FLOATS:
-        raise NotImplementedError("gather of non-floating arrays")
-    index = D.from_numpy(rows)
-    _lib.take_rows(_lib.DTYPE_CODE[A.dtype], src._t, n_rows, inner, index._t, rows.size, out._t)
-    return out
+    rows = _device_rows(idx)
+    if rows is not None:  # data-dependent rows: the index stays on the device (out-of-range values are the caller's to avoid)
+        inner = 1
+        for s in A.shape[1:]:
+            inner *= s
+        return _gather(A, rows, A.shape[0], inner, (rows.size,) + A.shape[1:])
+    plan = _index_plan(A.shape, idx)
+    return _gather(A, plan.positions, A.size, 1, plan.shape)
 
 
 def _leading_rows(idx, shape):
@@ -826,29 +907,40 @@ def scatter_add(A, idx, x):
         view = DevArray(A._t[_plain(idx)], A.dtype)
         D.map_op(Op.ADD, A.dtype, view, x, out=view)
         return A
-    rows = _host_index(idx)
-    if rows is None:
-        raise NotImplementedError(f"scatter with index {idx!r} is not supported on the device")
-    n_rows = A.shape[0]
-    if rows.size == 0:
-        return A
-    wrapped = onp.where(rows < 0, rows + n_rows, rows)
-    order = onp.argsort(wrapped, kind="stable").astype(onp.int64)
-    sorted_rows = wrapped[order]
-    boundaries = onp.flatnonzero(onp.diff(sorted_rows)) + 1
-    seg_start = onp.concatenate(([0], boundaries, [rows.size])).astype(onp.int64)
-    inner = 1
-    for s in A.shape[1:]:
-        inner *= s
-    target = (rows.size,) + A.shape[1:]
-    src = D.asarray(x, A.dtype)
-    if src.shape != target:
-        src = DevArray(src._t.expand(target), src.dtype)
-    src = D.contiguous(src)
     if not A._t.is_contiguous():
         raise AssertionError("scatter destination must be contiguous")
-    _lib.scatter_add_rows(_lib.DTYPE_CODE[A.dtype], A._t, n_rows, inner, src._t, D.from_numpy(rows)._t,
-                          D.from_numpy(order)._t, D.from_numpy(seg_start)._t, len(seg_start) - 1)
+    code = _lib.DTYPE_CODE[A.dtype]
+    rows = _device_rows(idx)
+    if rows is not None:
+        # a device-resident index: its stable order comes from the counting sort on the device (keys as float64,
+        # exact below 2^53), the runs of equal destination are found by the scatter kernel itself
+        n = rows.size
+        if n == 0:
+            return A
+        inner = 1
+        for s in A.shape[1:]:
+            inner *= s
+        if n > 65536:
+            raise NotImplementedError("scatter through a device-resident index of more than 65536 entries")
+        wrapped = D.map_op(Op.REMAINDER, D._F64, D.astype(rows, D._F64), float(A.shape[0]))  # negative rows count from the end
+        keys = D.astype(wrapped, D._I64)
+        order = D.empty((n,), D._I64)
+        _lib.sort_rows(_lib.DTYPE_CODE[D._F64], D.contiguous(wrapped)._t, 1, n, None, order._t, None)
+        target = (n,) + A.shape[1:]
+        src = D.asarray(x, A.dtype)
+        if src.shape != target:
+            src = DevArray(src._h().expand(target), src.dtype) if type(src) is DevArray else broadcast_to.fun(src, target)
+        src = D.contiguous(src)
+        _lib.scatter_add_rows(code, A._t, A.shape[0], inner, src._t, keys._t, order._t, None, n)
+        return A
+    plan = _index_plan(A.shape, idx)
+    if plan.n == 0:
+        return A
+    src = D.asarray(x, A.dtype)
+    if src.shape != plan.shape:
+        src = broadcast_to.fun(src, plan.shape)
+    src = D.contiguous(D.plain(src))
+    _lib.scatter_add_rows(code, A._t, A.size, 1, src._t, plan.positions._t, plan.order()._t, None, plan.n)
     return A
 
 

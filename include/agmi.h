@@ -319,7 +319,10 @@ int agmi_cumsum(int dtype, const void *src, int64_t outer, int64_t n, int64_t in
  * Bit-identical to numpy.add.at (numpy_vjps.py:941-950): a destination row that occurs several
  * times receives its addends sequentially in index order.  `order` is the stable argsort of
  * the (wrapped) index values and `seg_start[s] .. seg_start[s+1]` delimit runs of equal
- * destination in that order (n_seg runs); both are device arrays prepared by the caller. */
+ * destination in that order (n_seg runs); both are device arrays prepared by the caller.
+ * seg_start may be NULL: n_seg then counts the index entries and the runs are found on the device
+ * (nothing about the index needs to be known on the host: agmi_sort_rows on the index values gives
+ * `order`, so a device-resident index can be scattered from inside a recorded graph). */
 int agmi_scatter_add_rows(int dtype, void *dst, int64_t n_rows, int64_t inner,
                           const void *src, const int64_t *index, const int64_t *order,
                           const int64_t *seg_start, int64_t n_seg, void *stream);

@@ -153,3 +153,34 @@ def test_replay_of_array_functions_equals_eager():
         want = [g.numpy() for g in fun(x, v)]
         for g, w_ in zip(got, want):
             assert g.dtype == w_.dtype and onp.array_equal(g, w_), trial
+
+
+def test_gather_and_ordered_scatter_replay_from_a_graph():
+    """``x[[0, 1, 0]]`` (the reference's repeated-index case, tests/test_numpy.py:887-890) and a device-resident
+    row index inside a recorded evaluation: the index tables live on the device, so the replay needs no host
+    work, and repeated destinations are still added in index order."""
+    import autograd_amd as ag
+    import autograd_amd.numpy as dnp
+
+    rs = onp.random.default_rng(3)
+    rows = dnp.asarray(onp.array([4, 0, 4, 2, 4], dtype=onp.int64))
+    w = dnp.asarray(rs.standard_normal((5, 3)) * 1e3)
+
+    def f(x, M):
+        return dnp.sum(x[[0, 1, 0]] ** 2) + dnp.sum(M[rows] * w) + dnp.sum(M[[1, 1, 3], 1:] ** 3)
+
+    g = ag.grad(f, (0, 1))
+    x0, M0 = rs.standard_normal(3), rs.standard_normal((6, 3))
+    graphed = ag.capture(g, dnp.asarray(x0), dnp.asarray(M0))
+    for replay in range(4):
+        x0, M0 = rs.standard_normal(3), rs.standard_normal((6, 3))
+        got = graphed(dnp.asarray(x0), dnp.asarray(M0))
+        got = [a.numpy().copy() for a in got]
+        dnp.sum(dnp.asarray(M0) * 2.0).numpy()  # eager work and a synchronisation between replays
+        want = g(dnp.asarray(x0), dnp.asarray(M0))
+        for a, b in zip(got, want):
+            assert onp.array_equal(a, b.numpy())
+        dM = onp.zeros_like(M0)
+        onp.add.at(dM, onp.array([4, 0, 4, 2, 4]), w.numpy())
+        onp.add.at(dM, (onp.array([1, 1, 3]), slice(1, None)), 3 * M0[[1, 1, 3], 1:] ** 2)
+        assert onp.allclose(got[1], dM, rtol=1e-12)

@@ -1088,3 +1088,95 @@ def test_deferred_logsumexp_cotangent_survives_accumulation_and_second_order(dnp
     got = make(dnp, logsumexp)(dnp.asarray(A), dnp.asarray(b))
     for gd, wr in zip(got, want):
         close(gd.numpy(), wr, 1e-10)
+
+
+# ---- every NumPy index form: one gather forward, the ordered scatter backward --------------------------
+def _index_forms(rs):
+    return [
+        [0, 1, 2], ([0, 1, 2], slice(None), slice(None)), (3, slice(2, None), [1, 3]),       # tests/test_numpy.py:304-321
+        (slice(None), [0, 5, 0]), (slice(None, None, -1), [1, 1], slice(1, 3)), ([[0, 1], [2, 3]], [[1], [2]]),
+        (Ellipsis, [3, 0, 3]), (None, [4, 0], None, 2), ([0, 4, 0], slice(None), [1, 2, 1]), (onp.array([4, -1, 0, -1]),),
+        rs.rand(5, 6, 4) > 0.5, (onp.array([True, False, True, False, True]),), (slice(1, 4), rs.rand(6, 4) > 0.3),
+        (onp.array([1, 2, 0]), onp.array([True] * 3 + [False] * 3)), onp.zeros((0, 2), dtype=onp.int64),
+    ]
+
+
+@pytest.mark.parametrize("dtype", [F32, F64])
+def test_advanced_indexing_matches_numpy_bit_for_bit(dnp, dtype):
+    import autograd_amd as ag
+    from autograd_amd.numpy import wrapper as W
+
+    rs = onp.random.RandomState(21)
+    x = rs.randn(5, 6, 4).astype(dtype)
+    dx = dnp.asarray(x)
+    for idx in _index_forms(rs):
+        want = x[idx]
+        got = dx[idx].numpy()
+        assert got.shape == want.shape and onp.array_equal(got, want), idx
+        # cotangent: numpy.add.at order, duplicates included (numpy_vjps.py:941-950)
+        w = (rs.randn(*want.shape) * onp.exp(3 * rs.randn(*want.shape))).astype(dtype)
+        dst = onp.zeros_like(x)
+        onp.add.at(dst, idx, w)
+        g = ag.grad(lambda a: dnp.sum(a[idx] * dnp.asarray(w)))(dx).numpy()
+        assert g.dtype == dst.dtype and onp.array_equal(g, dst), idx
+        # accumulation into an array that already holds values
+        base = rs.randn(*x.shape).astype(dtype)
+        ref = base.copy()
+        onp.add.at(ref, idx, w)
+        assert onp.array_equal(W.scatter_add(dnp.asarray(base) + 0.0, idx, dnp.asarray(w)).numpy(), ref), idx
+    v = rs.randn(3).astype(dtype)
+    for idx in ([0, 0], [0, 1, 0]):                                                        # tests/test_numpy.py:881-890
+        g = ag.grad(lambda a: dnp.sum(a[idx]))(dnp.asarray(v)).numpy()
+        dst = onp.zeros_like(v)
+        onp.add.at(dst, idx, 1.0)
+        assert onp.array_equal(g, dst)
+    with pytest.raises(IndexError):
+        dx[[5]]
+    with pytest.raises(IndexError):
+        dx[onp.array([True, False])]
+
+
+def test_boolean_masks_select_elements_like_numpy(dnp):
+    import autograd_amd as ag
+
+    rs = onp.random.RandomState(2)
+    A = rs.randn(7, 5)
+    dA = dnp.asarray(A)
+    mask = A > 0.1
+    assert onp.array_equal(dA[mask].numpy(), A[mask])                     # N-d mask: the selected elements, 1-d
+    assert onp.array_equal(dA[dA > 0.1].numpy(), A[A > 0.1])               # a mask computed on the device
+    rows = onp.array([True, False, True, True, False, False, True])
+    assert onp.array_equal(dA[rows].numpy(), A[rows])
+    g = ag.grad(lambda a: dnp.sum(a[a > 0.1] ** 2))(dA).numpy()
+    assert onp.array_equal(g, onp.where(mask, 2 * A, 0.0))
+    with pytest.raises(IndexError):
+        dA[onp.array([True, False, True])]                                   # wrong length, as NumPy
+
+
+def test_reference_index_cases_pass_check_grads(dnp):
+    from autograd_amd.test_util import check_grads
+
+    rs = onp.random.RandomState(0)
+    A = dnp.asarray(rs.randn(5, 6, 4))
+    for fun in (lambda x: x[3, 0, 1], lambda x: x[::-1, 2:4, :], lambda x: x[[0, 1, 2], :, :], lambda x: x[3, 2:, [1, 3]],
+                lambda x: x[::-1, 2:4, :] + x[::-1, 3:5, :]):
+        check_grads(fun)(A)
+    v = dnp.asarray(rs.randn(7))
+    check_grads(lambda x: x[2:6][1:3])(v)
+    check_grads(lambda x: dnp.sum(x[[0, 1, 0]]))(dnp.asarray(rs.randn(3)))
+
+
+@pytest.mark.parametrize("dtype", [F32, F64])
+def test_device_resident_row_index_gathers_and_scatters_in_order(dnp, dtype):
+    from autograd_amd.numpy import wrapper as W
+
+    rs = onp.random.RandomState(8)
+    A = rs.randn(40, 6).astype(dtype)
+    for n in (1, 7, 300, 5000):
+        idx = rs.randint(-40, 40, n)
+        d_idx = dnp.asarray(idx)                                             # int64 on the device
+        assert onp.array_equal(dnp.asarray(A)[d_idx].numpy(), A[idx])
+        x = (rs.randn(n, 6) * onp.exp(3 * rs.randn(n, 6))).astype(dtype)
+        want = A.copy()
+        onp.add.at(want, idx, x)
+        assert onp.array_equal(W.scatter_add(dnp.asarray(A) + 0.0, d_idx, dnp.asarray(x)).numpy(), want), n
