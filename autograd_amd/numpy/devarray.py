@@ -506,7 +506,12 @@ def alias(x):
 
 
 def _is_pow2(c):
-    return c != 0.0 and math.isfinite(c) and math.frexp(c)[0] in (0.5, -0.5) and 2.0**-60 <= abs(c) <= 2.0**60
+    """A power of two of modest size.  Multiplying by one is exact unless the product leaves the normal
+    range, so merging it into a pending factor is bit-for-bit the eager result for every element whose
+    eager intermediates stay normal; keeping the exponent within +-8 keeps a chain of merged factors from
+    carrying values across the underflow or overflow threshold that the eager passes would have hit
+    (``(x * 2**-60) * 2**60`` is two real passes, as in NumPy)."""
+    return c != 0.0 and math.isfinite(c) and math.frexp(c)[0] in (0.5, -0.5) and 2.0**-8 <= abs(c) <= 2.0**8
 
 
 def _representable(v, dtype):
@@ -524,7 +529,8 @@ def _fold(op, dtype, xs):
     """``op(xs)`` as a pending map ``raw * scale * ascale + shift`` of its array operand, or None.
 
     Folded only when the kernel's fixed step order (scalar factor, array factor, offset), each step
-    rounded on its own, gives bit-for-bit the value of the eager passes:
+    rounded on its own, gives bit-for-bit the value of the eager passes (for elements whose eager
+    intermediates are neither subnormal nor overflowing; see ``_is_pow2``):
     * negation: always (it commutes with rounding), unless an array-valued offset is pending;
     * a Python-scalar factor: when it, or the pending scalar factor, is a power of two (that
       multiply is then exact) - and only a power of two once an array factor or an offset is pending;

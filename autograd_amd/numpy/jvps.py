@@ -67,6 +67,13 @@ defjvp(
     lambda g, ans, args, kwargs, _: anp._array_from_scalar_or_array(args, kwargs, g),
 )
 
+defjvp(anp.full, "same", argnums=(1,))  # numpy_jvps.py:33
+defjvp(  # numpy_jvps.py:169-173
+    anp.linspace,
+    lambda g, ans, start, stop, *args, **kwargs: anp.linspace(g, 0, *args, **kwargs),
+    lambda g, ans, start, stop, *args, **kwargs: anp.linspace(0, g, *args, **kwargs),
+)
+
 # binary ufuncs (38-74)
 def_linear(anp.multiply)
 defjvp(anp.add, lambda g, ans, x, y: broadcast(g, ans), lambda g, ans, x, y: broadcast(g, ans))

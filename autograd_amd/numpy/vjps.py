@@ -779,36 +779,36 @@ defvjp(
 )
 
 
+def _matmul_cotangent(wrt_left, other, g, other_ndim, target_meta):
+    """Cotangent of ``matmul(A, B)`` (numpy_vjps.py:567-612) for the left (``wrt_left``) or right operand, the
+    other one being ``other``.  matmul treats a 1-d left operand as a single row and a 1-d right operand as a
+    single column and drops that unit axis from its result; here the axis is put back on ``g`` (and on a 1-d
+    ``other``), the cotangent is one stacked matrix product, ``g . B^T`` or ``A^T . g``, and the unit axis of a
+    1-d target is dropped again.  Stacks that were broadcast are summed by ``unbroadcast``."""
+    target_ndim = target_meta[1]
+    if anp.ndim(g) == 0:  # vector times vector
+        return unbroadcast(g * other, target_meta)
+    left_is_vector = (target_ndim if wrt_left else other_ndim) == 1
+    right_is_vector = (other_ndim if wrt_left else target_ndim) == 1
+    if right_is_vector:
+        g = anp.expand_dims(g, -1)              # the column axis of the result
+    if left_is_vector:
+        g = anp.expand_dims(g, -2)              # the row axis of the result
+    if other_ndim == 1:
+        other = anp.expand_dims(other, -1 if wrt_left else 0)   # B as a column / A as a row
+    other_t = anp.swapaxes(other, -1, -2)
+    out = anp.matmul(g, other_t) if wrt_left else anp.matmul(other_t, g)
+    if target_ndim == 1:
+        out = anp.squeeze(out, -2 if wrt_left else -1)
+    return unbroadcast(out, target_meta)
+
+
 def _matmul_adjoint_0(B, G, A_meta, B_ndim):
-    if anp.ndim(G) == 0:
-        return unbroadcast(G * B, A_meta)
-    _, A_ndim, _, _ = A_meta
-    if A_ndim == 1:
-        G = anp.expand_dims(G, anp.ndim(G) - 1)
-    if B_ndim == 1:
-        B = anp.expand_dims(B, 0)
-        G = anp.expand_dims(G, anp.ndim(G))
-    else:
-        B = anp.swapaxes(B, B_ndim - 2, B_ndim - 1)
-    return unbroadcast(anp.matmul(G, B), A_meta)
+    return _matmul_cotangent(True, B, G, B_ndim, A_meta)
 
 
 def _matmul_adjoint_1(A, G, A_ndim, B_meta):
-    if anp.ndim(G) == 0:
-        return unbroadcast(G * A, B_meta)
-    _, B_ndim, _, _ = B_meta
-    B_is_vec = B_ndim == 1
-    if B_is_vec:
-        G = anp.expand_dims(G, anp.ndim(G))
-    if A_ndim == 1:
-        A = anp.expand_dims(A, 1)
-        G = anp.expand_dims(G, anp.ndim(G) - 1)
-    else:
-        A = anp.swapaxes(A, A_ndim - 2, A_ndim - 1)
-    result = anp.matmul(A, G)
-    if B_is_vec:
-        result = anp.squeeze(result, anp.ndim(G) - 1)
-    return unbroadcast(result, B_meta)
+    return _matmul_cotangent(False, A, G, A_ndim, B_meta)
 
 
 def _matmul_vjp_0(ans, A, B):
@@ -922,34 +922,54 @@ defvjp(anp.inner, partial(_grad_inner, 0), partial(_grad_inner, 1))
 
 
 # ---- einsum (numpy_vjps.py:815-860, subscript-string convention) ------------------------------------
+def _einsum_spread(cot, have, want, extents):
+    """The cotangent ``cot`` (axes named by the distinct letters ``have``) laid out with the axes ``want`` of an
+    einsum operand of shape ``extents``.  A letter of ``want`` missing from ``have`` was summed over by the forward
+    pass without meeting any other operand: every position along it receives the same value (a broadcast).  A
+    letter that ``want`` repeats read a diagonal going forward: its cotangent goes back onto that diagonal, zeros
+    elsewhere (a product with an identity matrix placed on the two axes)."""
+    distinct = "".join(dict.fromkeys(want))
+    size = {c: extents[want.index(c)] for c in distinct}
+    if have != distinct:
+        cot = anp.reshape(cot, tuple(size[c] if c in have else 1 for c in distinct))
+        cot = anp.broadcast_to(cot, tuple(size[c] for c in distinct))
+    labels = list(distinct)
+    for c in distinct:
+        times = want.count(c)
+        if times == 1:
+            continue
+        if times > 2:
+            raise NotImplementedError(f"einsum: index {c!r} repeated {times} times in one operand")
+        at = labels.index(c)
+        # x[..., i, ...] -> y[..., i, j, ...] = x[..., i, ...] * (i == j)
+        delta = anp.reshape(anp.eye(size[c]), (1,) * at + (size[c], size[c]) + (1,) * (len(labels) - at - 1))
+        cot = anp.expand_dims(cot, at + 1) * delta
+        labels.insert(at + 1, c)
+    # labels now holds every axis of `want`, repeated letters adjacent: permute into `want`'s order
+    order, used = [], [False] * len(labels)
+    for c in want:
+        k = next(i for i, (l, u) in enumerate(zip(labels, used)) if l == c and not u)
+        used[k] = True
+        order.append(k)
+    return cot if order == list(range(len(order))) else anp.transpose(cot, order)
+
+
 def _grad_einsum(argnum, ans, operands_, kwargs):
-    result_meta = anp.metadata(operands_[argnum])
+    """numpy_vjps.py:815-857, both calling conventions at once: the cotangent of operand k is the einsum of the
+    output cotangent with all other operands, onto k's own letters."""
+    target_meta = anp.metadata(operands_[argnum])
+    position = argnum - 1 if isinstance(operands_[0], str) else argnum // 2
 
     def vjp(g):
-        operands = operands_
-        in_subs, out_subs, _ = anp.parse_einsum_input(*operands)
-        operands = operands[1:]
-        in_subs_list = in_subs.split(",")
-        op_num = argnum - 1
-        subs_wrt = in_subs_list[op_num]
-        rest_of_ops = operands[:op_num] + operands[op_num + 1 :]
-        rest_of_subs = in_subs_list[:op_num] + in_subs_list[op_num + 1 :]
-        # subscripts that appear only in subs_wrt are summed out in the forward pass, as if contracted
-        # against a tensor of ones; the reference makes that tensor explicit for the broadcast back
-        other_named_subs = set("".join([out_subs] + rest_of_subs))
-        naked_summed = [(i, sub) for i, sub in enumerate(subs_wrt) if sub not in other_named_subs]
-        if naked_summed:
-            naked_summed_dims, ones_subs = zip(*naked_summed)
-            ones_subs = "".join(ones_subs)
-            wrt_shape = anp.shape(operands[op_num])
-            ones = anp.ones(tuple(wrt_shape[d] for d in naked_summed_dims))
-            new_input_subs = ",".join([out_subs, ones_subs] + rest_of_subs)
-            new_operands = (g, ones) + rest_of_ops
-        else:
-            new_input_subs = ",".join([out_subs] + rest_of_subs)
-            new_operands = (g,) + rest_of_ops
-        new_subscripts = new_input_subs + "->" + subs_wrt
-        return unbroadcast(anp.einsum(new_subscripts, *new_operands), result_meta)
+        in_subs, out_subs, arrays = anp.parse_einsum_input(*operands_)
+        subs = in_subs.split(",")
+        wanted = subs[position]
+        others = [a for k, a in enumerate(arrays) if k != position]
+        other_subs = [sx for k, sx in enumerate(subs) if k != position]
+        seen_elsewhere = set(out_subs).union(*other_subs)
+        reachable = "".join(dict.fromkeys(c for c in wanted if c in seen_elsewhere))
+        cot = anp.einsum(",".join([out_subs] + other_subs) + "->" + reachable, g, *others)
+        return unbroadcast(_einsum_spread(cot, reachable, wanted, target_meta[0]), target_meta)
 
     return vjp
 
@@ -980,6 +1000,15 @@ def _grad_array_from_scalar_or_array(ans, array_args, array_kwargs, scarray):
 
 
 defvjp(anp._array_from_scalar_or_array, _grad_array_from_scalar_or_array, argnums=(2, 3))
+# numpy_vjps.py:240-244: each sample is a fixed mix of the two end points; the mixing weights come from linspace itself
+# (float64, as there, whatever the end points' precision)
+defvjp(
+    anp.linspace,
+    lambda ans, start, stop, num=50, endpoint=True, dtype=None: lambda g: anp.dot(anp.linspace(1.0, 0.0, num, endpoint), g),
+    lambda ans, start, stop, num=50, endpoint=True, dtype=None: lambda g: anp.dot(anp.linspace(0.0, 1.0, num, endpoint), g),
+)
+# numpy_vjps.py:88-89: every output element is the fill value, so its cotangent is their sum
+defvjp(anp.full, lambda ans, shape, fill_value, dtype=None: lambda g: anp.sum(g), argnums=(1,))
 
 
 # ---- indexing (numpy_vjps.py:941-954) --------------------------------------------------------

@@ -280,8 +280,9 @@ def array_equal(a1, a2, equal_nan=False):
 
 def _arg_extreme(red, name):
     def raw(a, axis=None, out=None, keepdims=False):
-        """Index of the first extreme element: min over the axis of where(x == extreme, position, n)
-        (positions are exact in float64 below 2**53).  Non-differentiable (numpy_vjps.py:22-23)."""
+        """Index of the first extreme element, or of the first NaN if there is one: min over the axis of
+        where(x == extreme or x is NaN, position, n) (positions are exact in float64 below 2**53).
+        Non-differentiable (numpy_vjps.py:22-23)."""
         from ..tracer import getval
 
         x = D.asarray(getval(a))
@@ -302,6 +303,8 @@ def _arg_extreme(red, name):
         pos = D.from_numpy(onp.arange(n, dtype=onp.float64).reshape(view))
         f64 = onp.dtype("float64")
         cand = D.map_op(Op.WHERE, f64, D.astype(hit, f64), pos, float(n))
+        # a NaN makes the extreme NaN, which equals nothing: NumPy then reports the first NaN
+        cand = D.map_op(Op.WHERE, f64, D.astype(D.compare(Cmp.NE, x, x), f64), pos, cand)
         idx = D.map_reduce(Op.COPY, Red.MIN, f64, (cand,), (ax,), bool(keepdims) and axis is not None)
         return D.astype(idx, onp.int64)
 
@@ -1458,19 +1461,43 @@ def inner(a, b):
 
 # ---- einsum (subscript-string convention) -> sums, permutations and batched MFMA GEMMs ----------------
 def parse_einsum_input(*args):
-    """NumPy's own subscript parser (the reference wraps the same routine, numpy_wrapper.py:194-195)
-    run on shape-only stand-ins, so no operand is copied to the host."""
+    """``(input subscripts, output subscripts, array operands)`` of an einsum call in either convention
+    (subscript string, or operands alternating with sublists), letters only: NumPy's own parser (the
+    reference wraps the same routine, numpy_wrapper.py:194-195) run on shape-only stand-ins, so no operand
+    is copied to the host; it also spells out an ellipsis as letters."""
     try:
         from numpy._core.einsumfunc import _parse_einsum_input
     except ImportError:  # NumPy 1.x
         from numpy.core.einsumfunc import _parse_einsum_input
     from ..tracer import getval
 
-    if not isinstance(args[0], str):
-        raise NotImplementedError("einsum: only the subscript-string convention is supported on the device")
-    stand_ins = [onp.broadcast_to(onp.zeros((), onp.float32), shape(getval(a))) for a in args[1:]]
-    in_subs, out_subs, _ = _parse_einsum_input([args[0]] + stand_ins)
-    return in_subs, out_subs, args[1:]
+    def stand_in(a):
+        return onp.broadcast_to(onp.zeros((), onp.float32), shape(getval(a)))
+
+    if isinstance(args[0], str):
+        arrays = tuple(args[1:])
+        spec = [args[0]] + [stand_in(a) for a in arrays]
+    else:
+        n = len(args) // 2
+        arrays = tuple(args[0:2 * n:2])
+        spec = [stand_in(a) if i % 2 == 0 and i < 2 * n else a for i, a in enumerate(args)]
+    in_subs, out_subs, _ = _parse_einsum_input(spec)
+    return in_subs, out_subs, arrays
+
+
+def _einsum_diagonals(x, subs):
+    """A letter repeated within one operand's subscripts reads a diagonal: the operand as a strided view with
+    that letter once (its axis last, as ``torch.diagonal`` puts it).  Returns (view, subscripts)."""
+    while True:
+        dup = next((c for c in subs if subs.count(c) > 1), None)
+        if dup is None:
+            return x, subs
+        p = subs.index(dup)
+        q = subs.index(dup, p + 1)
+        if x.shape[p] != x.shape[q]:
+            raise ValueError(f"einsum: dimensions in operand for collapsing index {dup!r} don't match ({x.shape[p]} != {x.shape[q]})")
+        x = x._view(lambda t: torch.diagonal(t, 0, p, q))
+        subs = "".join(c for i, c in enumerate(subs) if i not in (p, q)) + dup
 
 
 def _einsum_sum_out(x, subs, drop):
@@ -1520,10 +1547,10 @@ def _einsum_pair(a, sa, b, sb, keep):
 
 @primitive
 def einsum(*operands, **kwargs):
-    """``numpy.einsum`` for the subscript-string convention: operands are contracted pairwise from
-    the left, each pair as a batched GEMM on permuted views; letters that appear nowhere else are
-    summed out first.  Repeated letters within one operand or in the output (diagonals) are not
-    supported."""
+    """``numpy.einsum`` in both calling conventions (subscript string; operands alternating with sublists):
+    a letter repeated within one operand is read as a diagonal (a strided view), then operands are
+    contracted pairwise from the left, each pair as a batched GEMM on permuted views; letters that appear
+    nowhere else are summed out first."""
     if kwargs:
         raise NotImplementedError(f"einsum: keyword arguments {sorted(kwargs)} are not supported on the device")
     in_subs, out_subs, arrays = parse_einsum_input(*operands)
@@ -1531,9 +1558,10 @@ def einsum(*operands, **kwargs):
     arrays = [D.asarray(a) for a in arrays]
     dt = D._float_dtype(D.result_dtype(*arrays))
     arrays = [D.astype(a, dt) if a.dtype != dt else a for a in arrays]
-    for sx in subs + [out_subs]:
-        if len(set(sx)) != len(sx):
-            raise NotImplementedError("einsum: repeated subscripts within one operand (diagonals) are not supported")
+    if len(set(out_subs)) != len(out_subs):
+        raise ValueError("einsum: output subscripts may name an index only once")
+    for k in range(len(arrays)):
+        arrays[k], subs[k] = _einsum_diagonals(arrays[k], subs[k])
     cur, cur_subs = arrays[0], subs[0]
     for k in range(1, len(arrays)):
         keep = set(out_subs).union(*subs[k + 1:]) if k + 1 < len(arrays) else set(out_subs)
@@ -1541,6 +1569,8 @@ def einsum(*operands, **kwargs):
     cur, cur_subs = _einsum_sum_out(cur, cur_subs, {c for c in cur_subs if c not in out_subs})
     if cur_subs != out_subs:
         cur = transpose.fun(cur, [cur_subs.index(c) for c in out_subs])
+    if type(cur) is not DevArray or not cur._t.is_contiguous():
+        cur = D.copy(cur) if cur.dtype in D._FLOATS else cur  # a diagonal or permuted view of an input: NumPy returns a new array
     return copy_if_input(cur, arrays)
 
 
@@ -1602,7 +1632,13 @@ def ones(shape, dtype=float):
     return D.constant(shape, 1.0, dtype)
 
 
+@primitive
 def full(shape, fill_value, dtype=None):
+    """``numpy.full``; differentiable in ``fill_value`` (argument 1), which may be a 0-d device array."""
+    if isinstance(fill_value, DevArray):
+        shape = (shape,) if isinstance(shape, numbers.Integral) else tuple(shape)
+        src = fill_value if dtype is None else astype(fill_value, dtype)
+        return D.contiguous(broadcast_to(reshape(src, ()), shape))
     if dtype is None or not isinstance(fill_value, (int, float)) or isinstance(fill_value, bool):
         return D.full(shape, fill_value, dtype)
     return D.constant(shape, fill_value, dtype)
@@ -1636,8 +1672,62 @@ def ones_like(a, dtype=None):
     return D.constant(s, 1.0, dtype or dt)
 
 
+@primitive
 def linspace(start, stop, num=50, endpoint=True, dtype=None):
-    return D.from_numpy(onp.linspace(start, stop, num, endpoint=endpoint), dtype)
+    """``numpy.linspace``.  Host numbers give an uploaded constant; a device-resident end point is
+    taken through NumPy's own arithmetic, ``arange(num) * ((stop - start) / div) + start`` with the
+    last sample set to ``stop``, in the dtype NumPy would choose."""
+    if not (isinstance(start, DevArray) or isinstance(stop, DevArray)):
+        return D.from_numpy(onp.linspace(start, stop, num, endpoint=endpoint), dtype)
+    num = int(num)
+    if num < 0:
+        raise ValueError("Number of samples, %s, must be non-negative." % num)
+    div = num - 1 if endpoint else num
+    ends = [v.dtype if isinstance(v, DevArray) else v for v in (start, stop)]
+    steps = D.from_numpy(onp.arange(num, dtype=onp.result_type(ends[0], ends[1], float(num))))
+    step = (stop - start) / div if div > 0 else (stop - start)
+    samples = steps * step + start
+    if endpoint and num > 1:
+        samples = concatenate([samples[:-1], reshape(stop + 0.0 * start, (1,))])
+    return samples if dtype is None else astype(samples, dtype)
+
+
+def gradient(f, *varargs, axis=None, edge_order=1):
+    """``numpy.gradient`` with unit spacing: central differences inside, one-sided ones at both
+    ends, built from slices so that it differentiates to any order (the reference gives it a
+    hand-written cotangent, numpy_vjps.py:297-342, and only supports ``axis`` too)."""
+    if varargs or edge_order != 1:
+        raise NotImplementedError("The only optional argument currently supported for np.gradient is axis.")
+    nd = ndim(f)
+    if axis is None:
+        axes = tuple(range(nd))
+    elif isinstance(axis, numbers.Integral):
+        axes = (int(axis),)
+    else:
+        axes = tuple(int(a) for a in axis)
+    axes = tuple(a + nd if a < 0 else a for a in axes)
+    extents = shape(f)
+    outs = []
+    for a in axes:
+        if not 0 <= a < nd:
+            raise onp.exceptions.AxisError(a, nd)
+        if extents[a] < 2:
+            raise ValueError(
+                "Shape of array too small to calculate a numerical gradient, "
+                "at least (edge_order + 1) elements are required."
+            )
+
+        def cut(lo, hi, a=a):
+            return f[(slice(None),) * a + (slice(lo, hi),)]
+
+        pieces = [cut(1, 2) - cut(0, 1)]
+        if extents[a] > 2:
+            pieces.append((cut(2, None) - cut(None, -2)) / 2.0)
+        pieces.append(cut(-1, None) - cut(-2, -1))
+        outs.append(concatenate(pieces, axis=a))
+    if len(axes) == 1 and (axis is None or isinstance(axis, numbers.Integral)):
+        return outs[0]
+    return tuple(outs)
 
 
 def arange(*args, **kwargs):

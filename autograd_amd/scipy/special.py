@@ -21,11 +21,25 @@ from ..numpy.vjps import _concrete, repeat_to_match_shape
 @primitive
 def logsumexp(x, axis=None, b=1.0, keepdims=False):
     x = D.asarray(x)
-    if not ((type(b) is float or isinstance(b, numbers.Number)) and b == 1.0):
-        # weighted form: log(sum(b * exp(x))) = logsumexp(x + log(b)) for positive weights
-        x = np.add.fun(x, np.log.fun(D.asarray(b) if not isinstance(b, numbers.Number) else b))
-    dt = D._float_dtype(x.dtype)
-    return D.map_reduce(Op.COPY, Red.LOGSUMEXP, dt, (x,), D.normalize_axes(axis, x.ndim), keepdims)
+    axes = D.normalize_axes(axis, x.ndim)
+    if (type(b) is float or isinstance(b, numbers.Number)) and b == 1.0:
+        return D.map_reduce(Op.COPY, Red.LOGSUMEXP, D._float_dtype(x.dtype), (x,), axes, keepdims)
+    # weighted form, the way scipy evaluates it: m = max(x), log(sum(b * exp(x - m))) + m, with weights of either
+    # sign (a negative total gives NaN, as there).  Two passes over x: the maximum, then the weighted sum
+    # fused into its reduction.
+    if not isinstance(b, numbers.Number):
+        b = D.asarray(b)
+        if D.broadcast_shapes(x.shape, b.shape) != x.shape:
+            x = np.broadcast_to.fun(x, D.broadcast_shapes(x.shape, b.shape))
+            axes = D.normalize_axes(axis, x.ndim)
+    dt = D._float_dtype(D.result_dtype(x, b))
+    top = D.map_reduce(Op.COPY, Red.MAX, dt, (x,), axes, True)
+    top = np._where3.fun(np.isfinite(top), top, 0.0)  # all -inf, or an inf / NaN present: no shift
+    total = D.map_reduce(Op.LSE_VJP, Red.SUM, dt, (1.0, b, x, top), axes, True)
+    out = np.add.fun(np.log.fun(total), top)
+    if keepdims:
+        return out
+    return np.reshape.fun(out, tuple(n for d, n in enumerate(x.shape) if d not in axes))
 
 
 def _keep(a, shape, axis, keepdims):

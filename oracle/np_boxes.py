@@ -132,38 +132,6 @@ class ArrayVSpace(VSpace):
         return np.dot(np.ravel(x), np.ravel(y))
 
 
-class ComplexArrayVSpace(ArrayVSpace):
-    iscomplex = True
-
-    @property
-    def size(self):
-        return np.prod(self.shape) * 2
-
-    def ones(self):
-        one = np.ones(self.shape, dtype=self.dtype)
-        return one + 1.0j * one
-
-    def standard_basis(self):
-        for idxs in np.ndindex(*self.shape):
-            for v in (1.0, 1.0j):
-                vect = np.zeros(self.shape, dtype=self.dtype)
-                vect[idxs] = v
-                yield vect
-
-    def randn(self):
-        re = np.array(np.random.randn(*self.shape)).astype(self.dtype)
-        im = np.array(np.random.randn(*self.shape)).astype(self.dtype)
-        return re + 1.0j * im
-
-    def _inner_prod(self, x, y):
-        return np.real(np.dot(np.conj(np.ravel(x)), np.ravel(y)))
-
-    def _covector(self, x):
-        return np.conj(x)
-
-
-VSpace.register(np.ndarray, lambda x: ComplexArrayVSpace(x) if np.iscomplexobj(x) else ArrayVSpace(x))
+VSpace.register(np.ndarray, ArrayVSpace)  # real arrays only: no workload of the path is complex
 for _t in (np.float64, np.float32, np.float16, np.longdouble):
     ArrayVSpace.register(_t)
-for _t in (np.complex64, np.complex128):
-    ComplexArrayVSpace.register(_t)

@@ -122,6 +122,12 @@ for _f in (anp.atleast_1d, anp.atleast_2d, anp.atleast_3d):
     defjvp(_f, _atleast_jvp(_f))
 
 defjvp(anp.pad, lambda g, ans, array, width, mode, **kwargs: anp.pad(g, width, mode))  # numpy_jvps.py:303
+defjvp(anp.gradient, "same")  # numpy_jvps.py:157
+defjvp(  # numpy_jvps.py:169-173
+    anp.linspace,
+    lambda g, ans, start, stop, *args, **kwargs: anp.linspace(g, 0, *args, **kwargs),
+    lambda g, ans, start, stop, *args, **kwargs: anp.linspace(0, g, *args, **kwargs),
+)
 # numpy_jvps.py:256-271: the tangent taken in sorted (partitioned) order
 defjvp(anp.sort, lambda g, ans, x, axis=-1, kind="quicksort", order=None: g[anp.argsort(x, axis, kind, order)])
 defjvp(
@@ -176,7 +182,6 @@ defjvp(
     anp.prod,
     lambda g, ans, x, axis=None, keepdims=False, **kwargs: ans * anp.sum(g / x, axis=axis, keepdims=keepdims),
 )
-defjvp(anp._astype, lambda g, ans, A, dtype, *a, **k: anp._astype(g, dtype))
 
 # binary ufuncs (38-74)
 def_linear(anp.multiply)

@@ -27,7 +27,7 @@ floor ceil round rint around fix trunc all any argmax argmin argsort argpartitio
 count_nonzero searchsorted floor_divide logical_and logical_or logical_not logical_xor
 isfinite isinf isnan allclose isclose array_equal greater greater_equal less less_equal
 equal not_equal iscomplex size isscalar isreal zeros_like ones_like empty_like full_like
-zeros ones empty full eye identity arange linspace asarray copy pad
+zeros ones empty full eye identity arange linspace asarray copy pad gradient
 """.split()
 
 _by_identity = {}

@@ -642,14 +642,29 @@ defvjp(
 )
 
 
-# ---- einsum, subscript-string convention (numpy_vjps.py:815-848) ---------------------------
+# ---- einsum, both calling conventions (numpy_vjps.py:815-857, 900-908) -------------------------
+def _unbroadcast_einsum(x, target_meta, subscript):
+    if Ellipsis not in subscript:
+        return x
+    if subscript[0] == Ellipsis:
+        return unbroadcast(x, target_meta, 0)
+    if subscript[-1] == Ellipsis:
+        return unbroadcast(x, target_meta, -1)
+    return unbroadcast(x, target_meta, subscript.index(Ellipsis))
+
+
 def _grad_einsum(argnum, ans, operands_, kwargs):
     result_meta = anp.metadata(operands_[argnum])
 
     def vjp(g):
         operands = operands_
         if not isinstance(operands[0], str):
-            raise NotImplementedError("oracle: only the subscript-string convention is restated")
+            # (op0, sublist0, op1, sublist1, ..., sublistout) convention, numpy_vjps.py:848-857
+            if len(operands) % 2 == 0:
+                raise NotImplementedError("Need sublistout argument")
+            operands = list(operands)
+            rest_of_ops = [operands[-1]] + operands[:argnum] + operands[(argnum + 2) : -1] + [operands[argnum + 1]]
+            return _unbroadcast_einsum(anp.einsum(g, *rest_of_ops), result_meta, operands[argnum + 1])
         in_subs, out_subs, _ = anp.parse_einsum_input(*operands)
         string, operands = operands[0], operands[1:]
         in_subs_list = in_subs.split(",")
@@ -740,3 +755,48 @@ def _pad_vjp(ans, array, pad_width, mode, **kwargs):
 
 
 defvjp(anp.pad, _pad_vjp)
+
+
+# ---- linspace (numpy_vjps.py:240-244) and gradient (297-342) ------------------------------------------
+defvjp(
+    anp.linspace,
+    lambda ans, start, stop, num: lambda g: anp.dot(anp.linspace(1.0, 0.0, num), g),
+    lambda ans, start, stop, num: lambda g: anp.dot(anp.linspace(0.0, 1.0, num), g),
+)
+
+
+def _grad_gradient(ans, x, *vargs, **kwargs):
+    axis = kwargs.pop("axis", None)
+    if vargs or kwargs:
+        raise NotImplementedError("The only optional argument currently supported for np.gradient is axis.")
+    if axis is None:
+        axis = range(x.ndim)
+    elif type(axis) is int:
+        axis = [axis]
+    else:
+        axis = list(axis)
+    x_dtype, x_shape, nd = x.dtype, x.shape, x.ndim
+
+    def vjp(g):
+        if anp.ndim(g) == nd:
+            g = g[anp.newaxis]  # a single axis: numpy returned one array, not a list
+        out = anp.zeros(x_shape, dtype=x_dtype)
+        for i, a in enumerate(axis):
+            g_swap = anp.swapaxes(g[i], 0, a)[:, anp.newaxis]
+            out_axis = anp.concatenate(
+                (
+                    -g_swap[0] - 0.5 * g_swap[1],
+                    g_swap[0] - 0.5 * g_swap[2],
+                    (-1.0) * anp.gradient(g_swap, axis=0)[2:-2, 0],
+                    0.5 * g_swap[-3] - g_swap[-1],
+                    0.5 * g_swap[-2] + g_swap[-1],
+                ),
+                axis=0,
+            )
+            out = out + anp.swapaxes(out_axis, 0, a)
+        return out
+
+    return vjp
+
+
+defvjp(anp.gradient, _grad_gradient)

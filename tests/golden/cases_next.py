@@ -394,4 +394,56 @@ def next_cases(be, ext):
             if not name.startswith(("mod", "remainder_array", "nan_to_num")):  # piecewise linear in x: no second order
                 weights2 = P(rs.randn(*onp.shape(be.get(x))).astype(dtype))
                 out[f"table/{name}_{tag}/second"] = grad(lambda a: np.sum(grad(f)(a) * weights2))(x)  # noqa: B023
+    # ---- rules that nothing above exercises: degrees/radians (numpy_vjps.py:112-115, numpy_jvps.py:78-81), full
+    # (88-89; 33), array(ndmin=) (665-670), the pad and arccosh tangents (numpy_jvps.py:303, 105), einsum in the
+    # sublist convention and with repeated subscripts (numpy_vjps.py:790-854), linspace (240-244) and gradient
+    # (297-342).  A generator of their own, so that the draws above stay what they were. ----
+    rs2 = onp.random.RandomState(23)
+    hA, hQ, hv = rs2.randn(3, 4), rs2.randn(4, 4), rs2.randn(4)
+    hT, hC = rs2.randn(2, 3, 4), rs2.uniform(1.2, 3.0, (3, 4))
+    hG = rs2.randn(6, 5)
+    for dtype in (onp.float64, onp.float32):
+        tag = "f32" if dtype == onp.float32 else "f64"
+        A_, Q_, v_, T_, C_, G_ = (P(h.astype(dtype)) for h in (hA, hQ, hv, hT, hC, hG))
+        W34, W44 = P(rs2.randn(3, 4).astype(dtype)), P(rs2.randn(4, 4).astype(dtype))
+        s0, s1 = P(onp.asarray(0.7, dtype)), P(onp.asarray(-1.9, dtype))
+        lin_w = P(rs2.randn(7).astype(dtype))
+        more = {
+            "degrees": (lambda a: np.sum(np.degrees(a) ** 2 * W34), A_),
+            "radians": (lambda a: np.sum(np.sin(np.radians(a * 50.0)) * W34), A_),
+            "rad2deg": (lambda a: np.sum(np.rad2deg(a) * W34), A_),
+            "deg2rad": (lambda a: np.sum(np.deg2rad(a) ** 3 * W34), A_),
+            "full": (lambda f: np.sum(np.full((3, 4), f) ** 2 * W34), s0),
+            "full_with_dtype": (lambda f: np.sum(np.full(4, np.sin(f), dtype=dtype) * v_), s1),  # noqa: B023
+            "array_ndmin": (lambda a: np.sum(np.array(a, ndmin=4)[0, 0] ** 2 * W34), A_),
+            "array_ndmin_of_scalar": (lambda f: np.sum(np.array(f, ndmin=2) ** 3), s0),
+            "pad_constant": (lambda a: np.sum(np.pad(a, ((1, 2), (0, 1)), "constant") ** 2), A_),
+            "pad_one_width": (lambda q: np.sum(np.pad(q, 1, "constant")[1:, :-1] * W44[0, 0] * np.pad(q, 1, "constant")[:-1, 1:]), Q_),
+            "arccosh": (lambda c: np.sum(np.arccosh(c) * W34), C_),
+            "arccosh_composed": (lambda c: np.sum(np.arccosh(c * c) ** 2), C_),
+            "einsum_sublist": (lambda a: np.sum(np.einsum(a, [0, 1], Q_, [1, 2], [0, 2]) ** 2 * W34), A_),
+            "einsum_sublist_second": (lambda q: np.sum(np.einsum(A_, [0, 1], q, [1, 2], [0, 2]) * W34), Q_),
+            "einsum_sublist_ellipsis": (lambda t: np.sum(np.einsum(t, [Ellipsis, 0, 1], Q_, [1, 2], [Ellipsis, 0, 2]) ** 2), T_),
+            # (the reference's rule cannot differentiate the operand that carries a repeated subscript; the others it can)
+            "einsum_repeated_other_operand": (lambda w: np.sum(np.einsum("ii,ij->j", Q_, w) ** 2), W44),
+            "einsum_repeated_other_operand_first": (lambda a: np.sum(np.einsum("ij,jj->i", a, Q_) ** 2), A_),
+            "einsum_repeated_three_operands": (lambda a: np.sum(np.einsum("ij,jj,j->i", a, Q_, v_) * a[:, 0]), A_),
+            "linspace_start": (lambda f: np.sum(np.linspace(f, 2.5, 7) ** 2 * lin_w), s0),  # noqa: B023
+            "linspace_stop": (lambda f: np.sum(np.sin(np.linspace(-0.5, f, 7)) * lin_w), s1),  # noqa: B023
+            "linspace_both": (lambda f: np.sum(np.linspace(f, f * f, 7) ** 2), s0),
+            # (the reference's cotangent needs at least four samples along each differentiated axis)
+            "gradient_vector": (lambda q: np.sum(np.gradient(q[0]) ** 2), Q_),
+            "gradient_axis0": (lambda m: np.sum(np.gradient(m, axis=0) * np.sin(m)), G_),
+            "gradient_axis1": (lambda a: np.sum(np.gradient(a, axis=1) ** 2 * W34), A_),
+            "gradient_last_axis_of_stack": (lambda t: np.sum(np.gradient(t, axis=-1) ** 2), T_),
+            "gradient_all_axes": (lambda m: np.sum(np.gradient(m)[0] * np.gradient(m)[1]), G_),
+            "gradient_axis_pair": (lambda m: np.sum(np.gradient(m, axis=(1, 0))[0] ** 2) + np.sum(np.gradient(m, axis=(1, 0))[1]), G_),
+        }
+        for name, (f, x) in more.items():
+            out[f"more/{name}_{tag}/value"] = f(x)
+            out[f"more/{name}_{tag}/grad"] = grad(f)(x)
+            tangent_in = P(onp.asarray(rs2.randn(*onp.shape(be.get(x)))).astype(dtype))
+            out[f"more/{name}_{tag}/jvp_tangent"] = be.make_jvp(f)(x)(tangent_in)[1]
+            weights2 = P(onp.asarray(rs2.randn(*onp.shape(be.get(x)))).astype(dtype))
+            out[f"more/{name}_{tag}/second"] = grad(lambda a: np.sum(grad(f)(a) * weights2))(x)  # noqa: B023
     return out

@@ -249,6 +249,11 @@ def test_random_argmax_rounding_helpers():
         assert onp.array_equal(dnp.argmax(X, axis=axis).numpy(), onp.argmax(x, axis=axis))
         assert onp.array_equal(dnp.argmin(X, axis=axis).numpy(), onp.argmin(x, axis=axis))
     assert dnp.argmax(X, axis=1).dtype == onp.int64
+    x[1, 4] = x[1, 7] = x[5, 0] = onp.nan  # a NaN wins over every number, the first one in its line
+    X = dnp.asarray(x)
+    for axis in (0, 1, None):
+        assert onp.array_equal(dnp.argmax(X, axis=axis).numpy(), onp.argmax(x, axis=axis))
+        assert onp.array_equal(dnp.argmin(X, axis=axis).numpy(), onp.argmin(x, axis=axis))
     y = onp.array([-2.5, -1.5, -0.5, 0.5, 1.5, 2.5, 2.4999, -0.0, onp.inf, onp.nan])
     Y = dnp.asarray(y)
     for name in ("floor", "ceil", "rint", "round", "trunc", "fix"):

@@ -297,6 +297,40 @@ def test_logsumexp_special_values(dnp):
     assert onp.allclose(got, want, rtol=1e-13, equal_nan=True), (got, want)
 
 
+def test_weighted_logsumexp_follows_scipy(dnp):
+    """The ``b=`` form (reference tests/test_scipy.py:237-255: positive weights of shapes (4,), (3, 4), (2, 3, 4)
+    over axis None/0/1, keepdims both ways) and weights of either sign, which scipy sums before the logarithm."""
+    from autograd_amd.scipy.special import logsumexp
+    from autograd_amd.test_util import check_grads
+
+    rs = onp.random.RandomState(21)
+    for shape in ((4,), (3, 4), (2, 3, 4)):
+        x, w = rs.randn(*shape), onp.exp(rs.randn(*shape))
+        signed = w.copy()
+        signed.flat[1::5] *= -0.02  # a few negative weights, every total still positive
+        for axis in (None, 0, 1)[: 2 + (len(shape) > 1)]:
+            for keepdims in (True, False):
+                for b in (w, signed, 2.5):
+                    want = scipy.special.logsumexp(x, axis=axis, b=b, keepdims=keepdims)
+                    assert onp.all(onp.isfinite(want))
+                    B = b if isinstance(b, float) else dnp.asarray(b)
+                    got = logsumexp(dnp.asarray(x), axis=axis, b=B, keepdims=keepdims)
+                    assert got.shape == onp.shape(want)
+                    close(got.numpy(), want, 1e-13)
+                    check_grads(lambda a: logsumexp(a, axis=axis, b=B, keepdims=keepdims), modes=["fwd", "rev"])(dnp.asarray(x))  # noqa: B023
+    # weights broadcast against x, a total below zero (NaN, as in scipy), float32
+    x, w = rs.randn(3, 4), onp.exp(rs.randn(4))
+    close(logsumexp(dnp.asarray(x), axis=1, b=dnp.asarray(w)).numpy(), scipy.special.logsumexp(x, axis=1, b=w), 1e-13)
+    with onp.errstate(all="ignore"):
+        want = scipy.special.logsumexp(x, axis=1, b=onp.array([1.0, -50.0, 1.0, 1.0]))
+    got = logsumexp(dnp.asarray(x), axis=1, b=dnp.asarray(onp.array([1.0, -50.0, 1.0, 1.0]))).numpy()
+    assert onp.isnan(want).any() and onp.array_equal(onp.isnan(got), onp.isnan(want))
+    x32, w32 = x.astype(onp.float32), onp.exp(rs.randn(3, 4)).astype(onp.float32)
+    got = logsumexp(dnp.asarray(x32), axis=0, b=dnp.asarray(w32))
+    assert got.dtype == onp.float32
+    close(got.numpy(), scipy.special.logsumexp(x32, axis=0, b=w32), 1e-5)
+
+
 # ---- contractions -------------------------------------------------------------------------------
 GEMM_SHAPES = [(1, 1, 1), (5, 7, 3), (64, 64, 16), (65, 63, 17), (130, 70, 33), (256, 128, 641), (1024, 10, 1024),
                (10, 1024, 300), (300, 300, 1), (129, 257, 100), (512, 512, 512)]
@@ -565,10 +599,74 @@ def test_einsum_matches_numpy(dnp, dtype):
         want = onp.einsum(spec, *[H[o] for o in ops])
         close(got, onp.asarray(want, dtype), RT[dtype] * 4)
     close(dnp.einsum("ij,jk->ik", Dv["a"].T.T, Dv["b"][:, ::2]).numpy(), H["a"] @ H["b"][:, ::2], RT[dtype] * 4)
+    # repeated subscripts (diagonals) and the operand/sublist convention
+    H["q"], H["s"] = rs.randn(6, 6).astype(dtype), rs.randn(3, 5, 5).astype(dtype)
+    Dv["q"], Dv["s"] = P(dnp, H["q"]), P(dnp, H["s"])
+    for spec, ops in [("ii->i", "q"), ("ii->", "q"), ("ii", "q"), ("bii->bi", "s"), ("bjj->b", "s"), ("ii,ij->j", "qq"), ("ij,jj->i", "qq")]:
+        close(dnp.einsum(spec, *[Dv[o] for o in ops]).numpy(), onp.asarray(onp.einsum(spec, *[H[o] for o in ops]), dtype), RT[dtype] * 4)
+    close(dnp.einsum(Dv["a"], [0, 1], Dv["b"], [1, 2], [0, 2]).numpy(), H["a"] @ H["b"], RT[dtype] * 4)
+    close(dnp.einsum(Dv["a"], [0, 1], Dv["b"], [1, 2]).numpy(), H["a"] @ H["b"], RT[dtype] * 4)
+    close(dnp.einsum(Dv["t"], [Ellipsis, 0, 1], Dv["b"], [1, 2], [Ellipsis, 2, 0]).numpy(),
+          onp.einsum("...ij,jk->...ki", H["t"], H["b"]), RT[dtype] * 4)
+    with pytest.raises(ValueError):
+        dnp.einsum("ij->ii", Dv["q"])
+
+
+def test_einsum_rules_beyond_the_reference_agree_with_finite_differences(dnp):
+    """The reference's einsum cotangent (numpy_vjps.py:790-854) raises for an operand that carries a repeated
+    subscript, and for the operand/sublist form without an output sublist, so no reference vector exists for
+    these: they are checked against numerical differentiation."""
+    from autograd_amd.test_util import check_grads
+
+    rs = onp.random.RandomState(12)
+    Q, W, T = (dnp.asarray(rs.randn(*s)) for s in ((4, 4), (4, 4), (2, 3, 3)))
+    for fun, x in [(lambda q: dnp.einsum("ii->", q) ** 2, Q), (lambda q: dnp.einsum("ii->i", q) ** 2, Q),
+                   (lambda q: dnp.einsum("ii,ij->j", q, W) ** 2, Q), (lambda q: dnp.einsum("ij,jj->i", W, q) ** 2, Q),
+                   (lambda t: dnp.einsum("bii->bi", t) ** 2, T), (lambda t: dnp.einsum("bii->", t) ** 2, T),
+                   (lambda q: dnp.einsum(q, [0, 0], W, [0, 1], [1]) ** 2, Q), (lambda q: dnp.einsum(q, [0, 1], W, [1, 2]) ** 2, Q),
+                   (lambda q: dnp.einsum(W, [1, 0], q, [0, 2]) ** 2, Q)]:
+        check_grads(fun, modes=["fwd", "rev"], order=2)(x)
+
+
+def test_gradient_and_linspace_follow_numpy_and_differentiate(dnp):
+    """Values are NumPy's bit for bit (the same subtractions, halvings and affine steps).  The reference's
+    gradient cotangent needs four samples along the axis and its linspace rules take no ``endpoint``; the
+    shorter axes and ``endpoint=False`` are checked against numerical differentiation."""
+    from autograd_amd.test_util import check_grads
+
+    rs = onp.random.RandomState(13)
+    for shp, ax in [((6,), None), ((4, 5), None), ((2, 5), 0), ((3, 5), 0), ((4, 5), -1), ((3, 4, 5), (0, 2))]:
+        x = rs.randn(*shp)
+        want, got = onp.gradient(x, axis=ax), dnp.gradient(dnp.asarray(x), axis=ax)
+        if isinstance(want, (tuple, list)):
+            assert len(want) == len(got) and all(onp.array_equal(w, g.numpy()) for w, g in zip(want, got))
+            check_grads(lambda a: sum(dnp.sum(dnp.sin(p)) for p in dnp.gradient(a, axis=ax)), modes=["fwd", "rev"], order=2)(dnp.asarray(x))  # noqa: B023
+        else:
+            assert onp.array_equal(want, got.numpy()), (shp, ax)
+            check_grads(lambda a: dnp.gradient(a, axis=ax), modes=["fwd", "rev"], order=2)(dnp.asarray(x))  # noqa: B023
+    with pytest.raises(ValueError):
+        dnp.gradient(dnp.asarray(rs.randn(1, 4)), axis=0)
     with pytest.raises(NotImplementedError):
-        dnp.einsum("ii->i", P(dnp, onp.eye(3, dtype=dtype)))
-    with pytest.raises(NotImplementedError):
-        dnp.einsum(Dv["a"], [0, 1], Dv["b"], [1, 2], [0, 2])
+        dnp.gradient(dnp.asarray(rs.randn(5)), 2.0)
+    for num in (1, 2, 5, 50):
+        for endpoint in (True, False):
+            want = onp.linspace(1.3, -0.7, num, endpoint=endpoint)
+            got = dnp.linspace(dnp.asarray(1.3), dnp.asarray(-0.7), num, endpoint=endpoint)
+            assert onp.array_equal(want, got.numpy()), (num, endpoint)
+            check_grads(lambda s, t: dnp.linspace(s, t, num, endpoint=endpoint), modes=["fwd", "rev"], order=2)(  # noqa: B023
+                dnp.asarray(1.3), dnp.asarray(-0.7))
+    assert dnp.linspace(dnp.asarray(onp.float32(0.5)), 2.0, 4).dtype == onp.float32
+    assert onp.array_equal(dnp.linspace(0.0, 1.0, 5).numpy(), onp.linspace(0.0, 1.0, 5))
+
+
+def test_astype_tangent_is_the_cast_of_the_tangent(dnp):
+    """The reference defines no forward-mode rule for ``astype`` (numpy_jvps.py has none); this one does, so
+    it is checked against numerical differentiation instead of a reference vector."""
+    from autograd_amd.test_util import check_grads
+
+    x = dnp.asarray(onp.random.RandomState(14).randn(3, 4))
+    check_grads(lambda a: dnp.sin(a).astype(onp.float64) ** 2, modes=["fwd", "rev"], order=2)(x)
+    check_grads(lambda a: dnp.astype(a * a, onp.float64), modes=["fwd"], order=1)(x)
 
 
 @pytest.mark.parametrize("dtype", [F32, F64])

@@ -164,8 +164,12 @@ def test_scalar_arithmetic_folds_into_a_pending_map_only_when_exact():
     assert state((x + 1.0) * 4.0) == (4.0, 4.0) and state((x + 1.0) / 4.0) == (0.25, 0.25)
     assert state(x + 0.0) == (1.0, 0.0)  # kept: -0.0 + 0.0 is +0.0
     # not exact in general: these must launch (and there is no device here, so they raise)
+    # (a far power of two is exact by itself, but merged with its inverse it would hide the eager underflow:
+    # (x * 2**-60) * 2**60 is 0 for a float32 1e-30 in NumPy, and must be two passes here too)
+    assert state(x * 2.0**-60) == (2.0**-60, None)
     for expr in (lambda: (x * 3.0) * 5.0, lambda: (x + 1.0) * 3.0, lambda: (x + 1.0) + 1.0, lambda: 2.0 / x,
-                 lambda: x / 3.0, lambda: x * onp.float64(3.0)):
+                 lambda: x / 3.0, lambda: x * onp.float64(3.0), lambda: (x * 2.0**-60) * 2.0**60,
+                 lambda: (x * 3.0) * 2.0**40, lambda: (x + 1.0) * 2.0**9):
         with pytest.raises(Exception):
             expr()
     # float32: scalars are rounded to the array's dtype first, as NumPy's weak scalars are
