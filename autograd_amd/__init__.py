@@ -9,10 +9,14 @@ derivative rules launch hand-written HIP kernels.
     from autograd_amd import grad, elementwise_grad, make_hvp
 """
 
-from . import differential_operators as _operators
-from .builtins import dict, isinstance, list, tuple, type  # noqa: A004,F401
-from .extend import primitive  # noqa: F401
-from .graphs import capture  # noqa: F401
+from . import _host
+
+_host.install()  # an installed HIPS/autograd may host the value type instead of this package's own tracer
+
+from . import differential_operators as _operators  # noqa: E402
+from .builtins import dict, isinstance, list, tuple, type  # noqa: A004,E402,F401
+from .extend import primitive  # noqa: E402,F401
+from .graphs import capture  # noqa: E402,F401
 
 # the differential operators of autograd/__init__.py:1-22, under the same names
 _OPERATORS = ("grad elementwise_grad value_and_grad grad_and_aux grad_named multigrad_dict deriv holomorphic_grad "

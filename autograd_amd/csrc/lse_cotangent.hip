@@ -111,7 +111,7 @@ __global__ __launch_bounds__(kBlock) void lse_cotangent_rows(const LseCotParams 
         const T *base = static_cast<const T *>(p.x) + r * p.x_rs;
 #pragma unroll
         for (int it = 0; it < ITERS; ++it)
-            if (ok[it]) a[it] = __builtin_nontemporal_load(reinterpret_cast<const vec_t *>(base + col[it]));  // read once
+            if (ok[it]) a[it] = __builtin_nontemporal_load(reinterpret_cast<const vec_t *>(base + col[it]));  // last reader
     };
     auto process_row = [&](int64_t r, const vec_t (&a)[ITERS]) __attribute__((always_inline)) {
         const T sr = scale_row ? static_cast<const T *>(p.scale_vec)[r * p.scale_rs] : T(1);

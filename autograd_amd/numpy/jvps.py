@@ -98,13 +98,16 @@ defjvp(anp.nan_to_num, lambda g, ans, x: anp.where(anp.isfinite(x), g, 0.0))  # 
 defjvp(anp.kron, "same", "same")  # numpy_jvps.py:155
 
 
-def _fwd_sort(g, ans, x, *args, **kwargs):  # numpy_jvps.py:256-271 (sort and partition alike): the tangent in sorted order
-    order_, rank = anp.sort_permutations(x)
-    return anp._reorder(g, order_, rank)
+def _sort_tangent(g, x, axis):  # numpy_jvps.py:256-271 (sort and partition alike): the tangent in sorted order
+    if axis is None:
+        order_, rank = anp.sort_permutations(anp.ravel(x), 0)
+        return anp._reorder(anp.ravel(g), order_, rank, 0)
+    order_, rank = anp.sort_permutations(x, axis)
+    return anp._reorder(g, order_, rank, axis)
 
 
-defjvp(anp.sort, _fwd_sort)
-defjvp(anp.partition, _fwd_sort)
+defjvp(anp.sort, lambda g, ans, x, axis=-1, kind=None, order=None: _sort_tangent(g, x, axis))
+defjvp(anp.partition, lambda g, ans, x, kth, axis=-1, kind="introselect", order=None: _sort_tangent(g, x, axis))
 defjvp(anp._reorder, "same")
 def_linear(anp.cross)  # numpy_jvps.py:106
 defjvp(anp.logaddexp2, lambda g, ans, x, y: g * 2 ** (x - ans), lambda g, ans, x, y: g * 2 ** (y - ans))  # 65

@@ -636,23 +636,20 @@ def _grad_cumsum(ans, x, axis=None):  # numpy_vjps.py:539-549
 defvjp(anp.cumsum, _grad_cumsum)
 
 
-def _grad_sort(ans, x, axis=-1, kind="quicksort", order=None):  # numpy_vjps.py:773-780
-    if len(anp.shape(x)) > 1:
-        raise NotImplementedError("Gradient of sort not implemented for multi-dimensional arrays.")
-    order_, rank = anp.sort_permutations(x)
-    return lambda g: anp._reorder(g, rank, order_)  # (the reference's unpermuter: g[inverse of argsort])
-
-
-def _grad_partition(ans, x, kth, axis=-1, kind="introselect", order=None):  # numpy_vjps.py:787-795
-    if len(anp.shape(x)) > 1:
-        raise NotImplementedError("Gradient of partition not implemented for multi-dimensional arrays.")
-    order_, rank = anp.sort_permutations(x)
-    return lambda g: anp._reorder(g, rank, order_)
+def _grad_sort(ans, x, axis=-1, kind="quicksort", order=None, *_):
+    """numpy_vjps.py:773-795 (sort and partition alike): the cotangent goes back through the inverse of the
+    sorting permutation.  The reference does this for vectors only and raises for anything else; here every
+    line along ``axis`` is un-permuted (``axis=None`` sorts the flattened array)."""
+    if axis is None:
+        order_, rank = anp.sort_permutations(anp.ravel(x), 0)
+        return lambda g: anp.reshape(anp._reorder(g, rank, order_, 0), anp.shape(x))
+    order_, rank = anp.sort_permutations(x, axis)
+    return lambda g: anp._reorder(g, rank, order_, axis)
 
 
 defvjp(anp.sort, _grad_sort)
-defvjp(anp.partition, _grad_partition)
-defvjp(anp._reorder, lambda ans, x, index, inverse: lambda g: anp._reorder(g, inverse, index))
+defvjp(anp.partition, lambda ans, x, kth, axis=-1, kind="introselect", order=None: _grad_sort(ans, x, axis))
+defvjp(anp._reorder, lambda ans, x, index, inverse, axis=0: lambda g: anp._reorder(g, inverse, index, axis))
 defvjp(anp.flipud, lambda ans, x: lambda g: anp.flipud(g))
 defvjp(anp.fliplr, lambda ans, x: lambda g: anp.fliplr(g))
 defvjp(anp.flip, lambda ans, x, axis=None: lambda g: anp.flip(g, axis))  # not in the reference's table: its own inverse

@@ -1298,18 +1298,36 @@ def argpartition(a, kth, axis=-1, kind="introselect", order=None):
     return _sorted_lines(getval(a), axis, ("order",))[0]
 
 
-def sort_permutations(x):
-    """(order, rank) of a vector: ``x[order]`` is sorted and ``rank`` is the inverse permutation."""
+def sort_permutations(x, axis=-1):
+    """(order, rank) along ``axis``: ``take_along_axis(x, order, axis)`` is sorted and ``rank`` is the inverse
+    permutation of every line."""
     from ..tracer import getval
 
-    return _sorted_lines(getval(x), 0, ("order", "rank"))
+    return _sorted_lines(getval(x), axis, ("order", "rank"))
 
 
 @primitive
-def _reorder(x, index, inverse):
-    """``x[index]`` for a permutation ``index`` of a vector that is already on the device (``inverse`` is its
-    inverse, used by the rule).  The index comes from the sort kernel, so it is not read back for a bounds check."""
-    x = D.contiguous(D.plain(D.asarray(x)))
+def _reorder(x, index, inverse, axis=0):
+    """``take_along_axis(x, index, axis)`` for an ``index`` that permutes every line and is already on the device
+    (``inverse`` holds the inverse permutations, used by the rule).  The index comes from the sort kernel, so it
+    is not read back for a bounds check."""
+    x = D.asarray(x)
+    if x.ndim > 1:
+        (axis,) = D.normalize_axes(axis, x.ndim)
+        last = x.ndim - 1
+        lines = D.contiguous(D.plain(D.asarray(moveaxis.fun(x, axis, last))))
+        n = lines.shape[-1]
+        rows = lines.size // n if n else 0
+        # flat positions: the line's offset plus the place within it (exact in float64 below 2**53)
+        f64 = onp.dtype(onp.float64)
+        within = D.astype(D.contiguous(D.asarray(moveaxis.fun(index, axis, last))), f64)
+        starts = D.from_numpy((onp.arange(rows, dtype=onp.float64) * n).reshape(lines.shape[:-1] + (1,)))
+        flat = D.astype(D.map_op(Op.ADD, f64, within, starts), onp.int64)
+        out = D.empty(lines.shape, x.dtype)
+        if lines.size:
+            _lib.take_rows(_lib.DTYPE_CODE[x.dtype], lines._t, lines.size, 1, flat._t, lines.size, out._t)
+        return out if axis == last else D.asarray(moveaxis.fun(out, last, axis))
+    x = D.contiguous(D.plain(x))
     n = x.shape[0]
     out = D.empty(x.shape, x.dtype)
     if x.size:

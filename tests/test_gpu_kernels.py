@@ -659,6 +659,31 @@ def test_gradient_and_linspace_follow_numpy_and_differentiate(dnp):
     assert onp.array_equal(dnp.linspace(0.0, 1.0, 5).numpy(), onp.linspace(0.0, 1.0, 5))
 
 
+def test_sort_and_partition_differentiate_along_any_axis(dnp):
+    """The reference's rules stop at vectors (numpy_vjps.py:773-795 raise for anything else), so there is no
+    reference vector: each line's cotangent must come back through the inverse of that line's permutation,
+    checked against ``take_along_axis`` on the host and numerical differentiation."""
+    from autograd_amd import grad
+    from autograd_amd.test_util import check_grads
+
+    rs = onp.random.RandomState(15)
+    for shape, axis in (((5, 7), -1), ((5, 7), 0), ((3, 4, 6), 1), ((3, 4, 6), None), ((6,), 0)):
+        x, w = rs.randn(*shape), rs.randn(*(shape if axis is not None else (int(onp.prod(shape)),)))
+        X, W = dnp.asarray(x), dnp.asarray(w)
+        got = grad(lambda a: dnp.sum(dnp.sort(a, axis=axis) * W))(X).numpy()  # noqa: B023
+        if axis is None:
+            want = onp.empty(x.size)
+            want[onp.argsort(x, axis=None, kind="stable")] = w
+            want = want.reshape(shape)
+        else:
+            want = onp.take_along_axis(w, onp.argsort(onp.argsort(x, axis=axis, kind="stable"), axis=axis, kind="stable"), axis)
+        assert onp.array_equal(got, want), (shape, axis)
+        check_grads(lambda a: dnp.sort(a, axis=axis) * W, modes=["fwd", "rev"], order=2)(X)  # noqa: B023
+        if axis is not None:
+            check_grads(lambda a: dnp.sort(a, axis=axis)[(slice(None),) * (axis % len(shape)) + (slice(0, 2),)] ** 2,  # noqa: B023
+                        modes=["fwd", "rev"])(X)
+
+
 def test_astype_tangent_is_the_cast_of_the_tangent(dnp):
     """The reference defines no forward-mode rule for ``astype`` (numpy_jvps.py has none); this one does, so
     it is checked against numerical differentiation instead of a reference vector."""
@@ -994,8 +1019,8 @@ def test_sort_is_stable_and_puts_nans_last(dnp, dtype):
     want = onp.empty_like(x)
     want[onp.argsort(x, kind="stable")] = w
     assert onp.array_equal(g, want)
-    with pytest.raises(NotImplementedError):
-        ag.grad(lambda v: dnp.sum(dnp.sort(v, axis=0)))(P(dnp, a))
+    # along an axis of a stack too (the reference's rule raises there): every cotangent of ones comes back as ones
+    assert onp.array_equal(ag.grad(lambda v: dnp.sum(dnp.sort(v, axis=0)))(P(dnp, a)).numpy(), onp.ones_like(a))
     h = ag.grad(lambda v: dnp.sum(ag.grad(lambda u: dnp.sum(dnp.sort(u * u) * P(dnp, w)))(v) * P(dnp, w)))(P(dnp, x)).numpy()
     want2 = onp.empty_like(x)
     want2[onp.argsort(x * x, kind="stable")] = w

@@ -123,12 +123,24 @@ def test_full_mlp(dev):
 
 
 def test_full_rnn(dev):
-    """The T=64, H=512 recurrence with 0.1*N(0,1) weights is chaotic (recurrent gain ~2.3): float32
-    rounding differences grow ~30x per doubling of T, and at T=64 reference autograd+NumPy itself
-    is ~20% away from the float64 answer.  So at full size: (1) in float32 the device result must be
-    as close to the float64 answer as the NumPy float32 one is (same conditioning, no extra error);
-    (2) the same full-length tape in float64 must match the float64 oracle tightly; (3) at T=8,
-    where rounding has not been amplified yet, float32 parity holds at the stated rtol 1e-5."""
+    """The H=512 recurrence with 0.1*N(0,1) weights is chaotic (recurrent gain ~2.3): a rounding difference
+    grows about 30x per doubling of T, in either precision.  Measured against the oracle at full width
+    (B=256, H=512), relative to |ref| + max|ref|:
+        float32  T=8 1.5e-6   T=12 4.1e-6   T=14 7.7e-6   T=16 1.3e-5   T=32 4.0e-4   T=64 ~0.2
+        float64  T=16 2.1e-14  T=32 1.1e-12  T=64 5.9e-10
+    and NumPy's own float32 result is as far from the float64 answer as the device's at every T.  The two
+    precisions differ by the ratio of their unit roundoffs at every T, so this is the conditioning of the
+    program and not an error of a kernel: any evaluation that sums a GEMM in another order than the host BLAS
+    lands this far away.  Hence: (1) the stated rtol 1e-5 is asserted in float32 at full width up to T=14, the
+    longest sequence for which it holds; (2) at T=64 in float32 the device result must be as close to the float64
+    answer as the NumPy float32 one is; (3) the full-length tape in float64 is held to 2e-9, T=32 to 1e-11 and
+    T=16 to the stated 1e-12."""
+    for seq_len in (8, 12, 14):
+        short = configs.rnn_inputs(seq_len=seq_len)
+        got_s = configs.run_config("rnn", dev, short)["grad"]
+        want_s = configs.run_config("rnn", oracle_backend(), short)["grad"]
+        for k in want_s:
+            check(f"rnn(f32, T={seq_len})/{k} vs oracle", got_s[k], want_s[k], rtol=1e-5)
     inputs = configs.rnn_inputs()
     got = configs.run_config("rnn", dev, inputs)["grad"]
     want = configs.run_config("rnn", oracle_backend(), inputs)["grad"]
@@ -139,18 +151,14 @@ def test_full_rnn(dev):
         e_dev = onp.max(onp.abs(got[k] - exact[k])) / scale
         e_ref = onp.max(onp.abs(want[k] - exact[k])) / scale
         assert e_dev <= 3.0 * e_ref + 1e-5, (k, e_dev, e_ref)
-    inputs64 = configs.rnn_inputs(dtype=onp.float64)
-    got64 = configs.run_config("rnn", dev, inputs64)["grad"]
-    want64 = configs.run_config("rnn", oracle_backend(), inputs64)["grad"]
-    exact64 = cf.rnn_grads(inputs64["params"], inputs64["inputs"], inputs64["targets"])
-    for k in want64:
-        check(f"rnn(f64, T=64)/{k} vs oracle", got64[k], want64[k], rtol=1e-8)
-        check(f"rnn(f64, T=64)/{k} vs hand-written BPTT", got64[k], exact64[k], rtol=1e-8)
-    short = configs.rnn_inputs(seq_len=8)
-    got8 = configs.run_config("rnn", dev, short)["grad"]
-    want8 = configs.run_config("rnn", oracle_backend(), short)["grad"]
-    for k in want8:
-        check(f"rnn(T=8)/{k} vs oracle", got8[k], want8[k])
+    for seq_len, rtol in ((16, 1e-12), (32, 1e-11), (64, 2e-9)):
+        inputs64 = configs.rnn_inputs(seq_len=seq_len, dtype=onp.float64)
+        got64 = configs.run_config("rnn", dev, inputs64)["grad"]
+        want64 = configs.run_config("rnn", oracle_backend(), inputs64)["grad"]
+        exact64 = cf.rnn_grads(inputs64["params"], inputs64["inputs"], inputs64["targets"])
+        for k in want64:
+            check(f"rnn(f64, T={seq_len})/{k} vs oracle", got64[k], want64[k], rtol=rtol)
+            check(f"rnn(f64, T={seq_len})/{k} vs hand-written BPTT", got64[k], exact64[k], rtol=rtol)
 
 
 def test_full_rosen_hvp(dev):
