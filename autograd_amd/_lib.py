@@ -327,6 +327,19 @@ class KernelTimer:
 _TIMER = None
 
 
+class untimed:
+    """``with untimed(): ...``: launches inside are not seen by the active ``KernelTimer`` (filler work of a
+    measurement, for instance)."""
+
+    def __enter__(self):
+        global _TIMER
+        self._prev, _TIMER = _TIMER, None
+
+    def __exit__(self, *exc):
+        global _TIMER
+        _TIMER = self._prev
+
+
 def _distinct_bytes(t):
     n = 1
     for extent, stride in zip(t.shape, t.stride()):
