@@ -64,7 +64,8 @@ def time_steps(fn, sync, steps, warmup):
 class HeadStart:
     """Keeps the launch stream busy for about ``ms`` milliseconds, so that the launches the host enqueues
     meanwhile run back to back on the GPU and HIP events around one of them measure its execution, not the
-    host's dispatch latency.  The filler only READS (sums of a 256 MiB array): what it leaves in the caches is
+    host's dispatch latency.  The filler only READS (minima of a 256 MiB array, a reduction no workload here
+    launches, so a kernel trace tells it apart by its `AccMin` kernels): what it leaves in the caches is
     clean, as after the reads that end a real evaluation; a filler that writes leaves 256 MiB of dirty lines
     whose write-back is then charged to the first kernels of the measured step (measured: +10 us on the
     134 MB forward reduction)."""
@@ -79,7 +80,7 @@ class HeadStart:
         self._lib = _lib
         self.buf = D.empty((64 << 20,), onp.float32)
         _lib.fill(_lib.DTYPE_CODE[self.buf.dtype], self.buf._t, 0.0)
-        self.read = lambda: D.map_reduce(Op.COPY, Red.SUM, self.buf.dtype, (self.buf,), (0,), False)
+        self.read = lambda: D.map_reduce(Op.COPY, Red.MIN, self.buf.dtype, (self.buf,), (0,), False)
         self.read()
         _lib.synchronize()
         t0 = time.perf_counter()
@@ -95,16 +96,19 @@ class HeadStart:
 
 
 def event_pair_overhead_ms(ahead, pairs=40):
-    """What a HIP event pair adds to the kernel it brackets, measured live: pairs around ONE tiny launch give
-    overhead + k, pairs around TWO of them overhead + 2k, so overhead = 2 * t1 - t2.  Taken behind a busy
-    stream, like the kernel timings it corrects."""
+    """What a HIP event pair adds to the kernel it brackets, measured live: pairs around ONE launch of a probe
+    kernel give overhead + k, pairs around TWO of them overhead + 2k, so overhead = 2 * t1 - t2.  The probe
+    is a 64 MiB fill (about 10 us, the scale of the kernels being timed): around a tiny launch the same
+    arithmetic gives 4.5 us instead of about 2, because a tiny kernel hides none of the pair's cost, and
+    subtracting that from a 20-50 us kernel would flatter it.  Taken behind a busy stream, like the kernel
+    timings it corrects."""
     import numpy as onp
     import torch
 
     from autograd_amd import _lib
     from autograd_amd.numpy import devarray as D
 
-    cell = D.empty((64,), onp.float32)
+    cell = D.empty((16 << 20,), onp.float32)
     code = _lib.DTYPE_CODE[cell.dtype]
     stream = torch.cuda.current_stream(_lib.device())
     events = [torch.cuda.Event(enable_timing=True) for _ in range(4 * pairs)]
@@ -274,22 +278,21 @@ def make_workload(name, be):
 def measured_traffic(kernel):
     """HBM bytes per launch of ``kernel`` from the committed rocprofv3 counter summary
     (profiles/bcast_grad_hbm_traffic.md: FETCH_SIZE + WRITE_SIZE scaled by a plain copy) and where the figure
-    comes from (file and the commit that last changed it); (None, None) when the file has no row for this kernel."""
-    import subprocess
+    comes from (the file and a hash of its contents, which also identifies it where there is no git history);
+    (None, None) when the file has no row for this kernel."""
+    import hashlib
 
     rel = os.path.join("profiles", "bcast_grad_hbm_traffic.md")
     family, _, functor = kernel.partition("<")
     functor = functor.split(">")[0].split(",")[0]
     try:
-        for line in open(os.path.join(ROOT, rel)):
+        text = open(os.path.join(ROOT, rel)).read()
+        for line in text.splitlines():
             cells = [c.strip() for c in line.split("|")]
-            if len(cells) > 8 and family in cells[1] and (not functor or functor in cells[1]):
-                try:
-                    rev = subprocess.run(["git", "-C", ROOT, "log", "-1", "--format=%h", "--", rel], capture_output=True,
-                                         text=True, timeout=10).stdout.strip() or "unknown"
-                except (OSError, subprocess.SubprocessError):
-                    rev = "unknown"
-                return float(cells[7]) * 1e6, f"{rel} @ {rev} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not measured in this run)"
+            # (a functor name, `F...`, tells rows of one kernel family apart; other template arguments do not matter)
+            if len(cells) > 8 and family in cells[1] and (not functor.startswith("F") or functor in cells[1]):
+                digest = hashlib.sha256(text.encode()).hexdigest()[:12]
+                return float(cells[7]) * 1e6, f"{rel} sha256:{digest} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not measured in this run)"
     except (OSError, ValueError):
         pass
     return None, None
@@ -370,7 +373,7 @@ def main():
     roofline["launches_timed"] = dom["launches"]
     roofline["timing"] = ("HIP events on the launch stream around every launch of this kernel over `steps` steps, the stream "
                           "kept busy ahead of each step so that the pair brackets GPU execution only; the pair's own cost "
-                          "(measured live: 2 x pair around one tiny launch - pair around two) is subtracted")
+                          "(measured live: 2 x pair around one 64 MiB fill - pair around two) is subtracted")
 
     result = {
         "metric": "grad evals/sec",
