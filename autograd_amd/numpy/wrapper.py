@@ -1666,6 +1666,23 @@ def empty(shape, dtype=float):
     return D.empty(shape, dtype)
 
 
+def settle(x):
+    """``x`` with any deferred arithmetic done (a pending affine map written out, a deferred contraction or
+    logsumexp cotangent computed); tuples, lists and dicts are walked.  The package's own differential operators do
+    this to every derivative they hand back; it is for callers that obtained a value some other way (a tracer of
+    another package hosting the value type) and want its kernels inside their own timed region."""
+    from ..tracer import getval
+
+    x = getval(x)
+    kind = type(x)
+    if kind is tuple or kind is list:
+        return kind(settle(item) for item in x)
+    if kind is dict:
+        return {key: settle(item) for key, item in x.items()}
+    finish = getattr(kind, "_settled", None)
+    return finish(x) if finish is not None else x
+
+
 @notrace_primitive
 def zeros_like(a, dtype=None):
     s, _, dt, _ = _meta_of(a)
