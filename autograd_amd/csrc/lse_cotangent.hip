@@ -9,14 +9,18 @@
 //     scaled copy   col_factor[k] * S[r, k]         (cotangent of mem when x = mem * col_factor)
 //     column sums   sum_r mem[r, k] * S[r, k]       (cotangent of the factor broadcast along the column)
 // Launched one by one these are four passes over matrix-sized data (write S, read it three times,
-// read mem again for the product).  Here a block walks a band of rows; each thread keeps its
-// columns' factors and column accumulators in registers, forms S from mem on the fly, writes the
-// scaled copy, and S itself never reaches memory: read mem once, write the scaled copy once.
+// read mem again for the product).  Here a block owns a tile of 16 (or a multiple of 16) rows by
+// 256 vectors of columns; each thread keeps its columns' factors and column accumulators in
+// registers, walks the tile's rows with four rows of loads in flight, forms S from mem on the fly and
+// writes the scaled copy; S itself never reaches memory: read mem once, write the scaled copy once.
+// Tiles this small give thousands of blocks (2048 for 8192 x 4096 float32), which streams measurably
+// better than a few hundred long-lived ones, at the price of partial results in both directions:
 //
-// Row sums: per-thread sum in column order, wave butterfly, the four wave partials added in wave
-// order.  Column sums: a thread adds its rows in row order; each block writes one partial row to the
-// workspace and a second kernel adds the blocks' partials in a fixed order.  Nothing is atomic, so
-// results depend only on the shape.
+// Row sums: per-thread sum over its vector, wave butterfly, the block's wave partials added in wave
+// order; with more than one tile across, the tiles' partials go to the workspace and are added in tile
+// order by the finishing kernel.  Column sums: a thread adds its rows in row order; each band of rows
+// writes one partial row to the workspace and the finishing kernel adds the bands' partials in a
+// fixed order.  Nothing is atomic, so results depend only on the shape.
 #include <algorithm>
 
 #include "common.h"
@@ -24,8 +28,9 @@
 
 namespace agmi {
 
-constexpr int kLseCotMaxRowsPerBlock = 64;
-constexpr int kLseCotMaxIters = 8;
+constexpr int kLseCotRowGroup = 16;         // rows of a tile are taken in groups of this many
+constexpr int kLseCotMaxRowsPerBlock = 64;  // wave partials of a tile's rows are held in LDS
+constexpr int kLseCotDepth = 4;             // rows of loads in flight per thread
 
 struct LseCotParams {
     int64_t rows, cols;
@@ -42,123 +47,134 @@ struct LseCotParams {
     int64_t ans_rs;
     const void *g;
     int64_t g_rs;
-    void *row_sums;
+    void *row_sums;      // final row sums (one tile across) ...
+    void *row_partials;  // ... or [tiles across][rows] partial sums
     const void *col_factor;
     void *scaled;
     int64_t scaled_rs;
-    void *partials;  // [blocks][cols]
+    void *partials;  // [bands][cols]
     int rows_per_block;
 };
 
 enum { kWantScaled = 1, kWantRowSums = 2, kWantColSums = 4 };
 
-template <typename T, int ITERS, int WANT>
-__global__ __launch_bounds__(kBlock) void lse_cotangent_rows(const LseCotParams p) {
+// the value lane `q` holds, as a wave-uniform scalar (q is the same for the whole wave)
+__device__ __forceinline__ float from_lane(float v, int q) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), q));
+}
+__device__ __forceinline__ double from_lane(double v, int q) {
+    const unsigned long long bits = __builtin_bit_cast(unsigned long long, v);
+    const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(bits), q));
+    const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(bits >> 32), q));
+    return __builtin_bit_cast(double, (static_cast<unsigned long long>(hi) << 32) | lo);
+}
+
+template <typename T, int WANT>
+__global__ __launch_bounds__(kBlock) void lse_cotangent_tile(const LseCotParams p) {
     constexpr int V = 16 / sizeof(T);
+    constexpr int D = kLseCotDepth;
     typedef T vec_t __attribute__((ext_vector_type(V), aligned(sizeof(T))));
     __shared__ T wave_sums[kLseCotMaxRowsPerBlock][kBlock / 64];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int64_t row_begin = static_cast<int64_t>(blockIdx.x) * p.rows_per_block;
+    const int64_t own_col = (static_cast<int64_t>(blockIdx.x) * kBlock + tid) * V;  // cols % V == 0: a vector is all in or all out
+    const bool ok = own_col < p.cols;
+    // lanes past the last column work on column 0 and throw the result away: a load under a per-lane condition
+    // makes the compiler wait for it where the branches join, which would serialise the rows in flight
+    const int64_t col = ok ? own_col : 0;
+    const int64_t row_begin = static_cast<int64_t>(blockIdx.y) * p.rows_per_block;
     const int64_t row_end = min(p.rows, row_begin + p.rows_per_block);
 
-    int64_t col[ITERS];
-    bool ok[ITERS];
-#pragma unroll
-    for (int it = 0; it < ITERS; ++it) {
-        col[it] = (static_cast<int64_t>(it) * kBlock + tid) * V;  // cols % V == 0: a vector is all in or all out
-        ok[it] = col[it] < p.cols;
-    }
     // absent steps are neutral elements (x * 1 is exact; x + 0 can only change the sign of a zero,
     // which exp(x - ans) cannot see), so the arithmetic below has no branches
     const T sc = static_cast<T>(p.scale), sh = static_cast<T>(p.shift);
     const bool scale_col = p.scale_vec != nullptr && p.scale_by_col, scale_row = p.scale_vec != nullptr && !p.scale_by_col;
     const bool shift_col = p.shift_vec != nullptr && p.shift_by_col, shift_row = p.shift_vec != nullptr && !p.shift_by_col;
-    T sv[ITERS][V], hv[ITERS][V], fv[(WANT & kWantScaled) ? ITERS : 1][V];
+    vec_t sv, hv, fv, colacc;
 #pragma unroll
-    for (int it = 0; it < ITERS; ++it) {
+    for (int j = 0; j < V; ++j) {
+        sv[j] = T(1);
+        hv[j] = T(0);
+        fv[j] = T(0);
+        colacc[j] = T(0);
+    }
+    if (scale_col) sv = *reinterpret_cast<const vec_t *>(static_cast<const T *>(p.scale_vec) + col);
+    if (shift_col) hv = *reinterpret_cast<const vec_t *>(static_cast<const T *>(p.shift_vec) + col);
+    if (WANT & kWantScaled) fv = *reinterpret_cast<const vec_t *>(static_cast<const T *>(p.col_factor) + col);
+
+    const auto load_row = [&](int64_t r, vec_t &a) __attribute__((always_inline)) {
+        // last reader of this operand: a streaming load (the row test is the same for the whole block)
+        if (r < row_end) a = __builtin_nontemporal_load(reinterpret_cast<const vec_t *>(static_cast<const T *>(p.x) + r * p.x_rs + col));
+    };
+    // The per-row operands (ans, g, a factor / offset that varies along rows) of a group of 16 rows: lane l of every
+    // wave fetches those of row l with ONE load each, ahead of the group's matrix loads, and the rows read them
+    // back as wave-uniform scalars.  Fetched row by row instead they are vector loads issued after the prefetched
+    // matrix rows, and waiting for one of them waits for every load before it: no rows in flight any more.
+    T ans_v, g_v, sr_v = T(1), hr_v = T(0);
+    const auto load_row_operands = [&](int64_t r) __attribute__((always_inline)) {
+        const int64_t rr = min(r + (lane & (kLseCotRowGroup - 1)), row_end - 1);
+        ans_v = static_cast<const T *>(p.ans)[rr * p.ans_rs];
+        g_v = static_cast<const T *>(p.g)[rr * p.g_rs];
+        if (scale_row) sr_v = static_cast<const T *>(p.scale_vec)[rr * p.scale_rs];
+        if (shift_row) hr_v = static_cast<const T *>(p.shift_vec)[rr * p.shift_rs];
+    };
+    const auto process_row = [&](int64_t r, int q, const vec_t &a) __attribute__((always_inline)) {
+        const T sr = from_lane(sr_v, q), hr = from_lane(hr_v, q), ans_r = from_lane(ans_v, q), g_r = from_lane(g_v, q);
+        T rsum = T(0);
+        vec_t o;
 #pragma unroll
         for (int j = 0; j < V; ++j) {
-            sv[it][j] = T(1);
-            hv[it][j] = T(0);
+            T xv = a[j] * sc;
+            xv = xv * (scale_col ? sv[j] : sr);
+            xv = xv + sh;
+            xv = xv + (shift_col ? hv[j] : hr);
+            const T s = g_r * exp_of_nonpositive(xv - ans_r);
+            if (WANT & kWantRowSums) rsum += s;
+            if (WANT & kWantColSums) colacc[j] += a[j] * s;
+            if (WANT & kWantScaled) o[j] = fv[j] * s;
         }
-        if (ok[it]) {
-            if (scale_col) {
-                const vec_t v = *reinterpret_cast<const vec_t *>(static_cast<const T *>(p.scale_vec) + col[it]);
-#pragma unroll
-                for (int j = 0; j < V; ++j) sv[it][j] = v[j];
-            }
-            if (shift_col) {
-                const vec_t v = *reinterpret_cast<const vec_t *>(static_cast<const T *>(p.shift_vec) + col[it]);
-#pragma unroll
-                for (int j = 0; j < V; ++j) hv[it][j] = v[j];
-            }
-            if (WANT & kWantScaled) {
-                const vec_t v = *reinterpret_cast<const vec_t *>(static_cast<const T *>(p.col_factor) + col[it]);
-#pragma unroll
-                for (int j = 0; j < V; ++j) fv[it][j] = v[j];
-            }
-        }
-    }
-    T colacc[(WANT & kWantColSums) ? ITERS : 1][V];
-    if (WANT & kWantColSums) {
-#pragma unroll
-        for (int it = 0; it < ITERS; ++it)
-#pragma unroll
-            for (int j = 0; j < V; ++j) colacc[it][j] = T(0);
-    }
-
-    auto load_row = [&](int64_t r, vec_t (&a)[ITERS]) __attribute__((always_inline)) {
-        const T *base = static_cast<const T *>(p.x) + r * p.x_rs;
-#pragma unroll
-        for (int it = 0; it < ITERS; ++it)
-            if (ok[it]) a[it] = __builtin_nontemporal_load(reinterpret_cast<const vec_t *>(base + col[it]));  // last reader
-    };
-    auto process_row = [&](int64_t r, const vec_t (&a)[ITERS]) __attribute__((always_inline)) {
-        const T sr = scale_row ? static_cast<const T *>(p.scale_vec)[r * p.scale_rs] : T(1);
-        const T hr = shift_row ? static_cast<const T *>(p.shift_vec)[r * p.shift_rs] : T(0);
-        const T ans_r = static_cast<const T *>(p.ans)[r * p.ans_rs];
-        const T g_r = static_cast<const T *>(p.g)[r * p.g_rs];
-        T rsum = T(0);
-#pragma unroll
-        for (int it = 0; it < ITERS; ++it) {
-            if (!ok[it]) continue;
-            vec_t o;
-#pragma unroll
-            for (int j = 0; j < V; ++j) {
-                T xv = a[it][j] * sc;
-                xv = xv * (scale_col ? sv[it][j] : sr);
-                xv = xv + sh;
-                xv = xv + (shift_col ? hv[it][j] : hr);
-                const T s = g_r * exp_of_nonpositive(xv - ans_r);
-                if (WANT & kWantRowSums) rsum += s;
-                if (WANT & kWantColSums) colacc[it][j] += a[it][j] * s;
-                if (WANT & kWantScaled) o[j] = fv[it][j] * s;
-            }
-            if (WANT & kWantScaled)
-                // a matrix-sized result that no kernel of this pass reads back: a streaming store (measured +4 %)
-                __builtin_nontemporal_store(o, reinterpret_cast<vec_t *>(static_cast<T *>(p.scaled) + r * p.scaled_rs + col[it]));
-        }
+        if ((WANT & kWantScaled) && ok)
+            // a matrix-sized result that no kernel of this pass reads back: a streaming store
+            __builtin_nontemporal_store(o, reinterpret_cast<vec_t *>(static_cast<T *>(p.scaled) + r * p.scaled_rs + col));
         if (WANT & kWantRowSums) {
+            if (!ok) rsum = T(0);
 #pragma unroll
             for (int m = 32; m > 0; m >>= 1) rsum += __shfl_xor(rsum, m, 64);
             if (lane == 0) wave_sums[r - row_begin][wave] = rsum;
         }
     };
 
-    // the loads of the next two rows are in flight while a row is worked on
-    vec_t a0[ITERS], a1[ITERS], a2[ITERS];
-    if (row_begin < row_end) load_row(row_begin, a0);
-    if (row_begin + 1 < row_end) load_row(row_begin + 1, a1);
-    for (int64_t r = row_begin; r < row_end; r += 3) {
-        if (r + 2 < row_end) load_row(r + 2, a2);
-        process_row(r, a0);
-        if (r + 1 < row_end) {
-            if (r + 3 < row_end) load_row(r + 3, a0);
-            process_row(r + 1, a1);
+    // D rows of loads are in flight while a row is worked on.  Whole groups of 16 rows run as straight-line code (no
+    // row tests between the loads and the arithmetic, so the compiler is free to order them); the pipeline is refilled
+    // at each group's start, which only tiles taller than one group notice.
+    vec_t a[D];
+    int64_t r = row_begin;
+    for (; r + kLseCotRowGroup <= row_end; r += kLseCotRowGroup) {
+        load_row_operands(r);
+#pragma unroll
+        for (int d = 0; d < D; ++d)
+            a[d] = __builtin_nontemporal_load(reinterpret_cast<const vec_t *>(static_cast<const T *>(p.x) + (r + d) * p.x_rs + col));
+#pragma unroll
+        for (int q = 0; q < kLseCotRowGroup; ++q) {
+            const vec_t cur = a[q % D];
+            if (q + D < kLseCotRowGroup)
+                a[q % D] = __builtin_nontemporal_load(reinterpret_cast<const vec_t *>(static_cast<const T *>(p.x) + (r + q + D) * p.x_rs + col));
+            process_row(r + q, q, cur);
         }
-        if (r + 2 < row_end) {
-            if (r + 4 < row_end) load_row(r + 4, a1);
-            process_row(r + 2, a2);
+    }
+    if (r < row_end) {  // the last rows of the matrix (fewer than 16)
+        load_row_operands(r);
+        const int64_t group = r;
+#pragma unroll
+        for (int d = 0; d < D; ++d) load_row(r + d, a[d]);
+        for (; r < row_end; r += D) {
+#pragma unroll
+            for (int d = 0; d < D; ++d) {
+                if (r + d < row_end) {  // the same for the whole block
+                    const vec_t cur = a[d];
+                    load_row(r + d + D, a[d]);
+                    process_row(r + d, static_cast<int>(r + d - group), cur);
+                }
+            }
         }
     }
 
@@ -169,36 +185,41 @@ __global__ __launch_bounds__(kBlock) void lse_cotangent_rows(const LseCotParams 
             T t = wave_sums[tid][0];
 #pragma unroll
             for (int w = 1; w < kBlock / 64; ++w) t += wave_sums[tid][w];
-            static_cast<T *>(p.row_sums)[r] = t;
+            if (gridDim.x == 1) static_cast<T *>(p.row_sums)[r] = t;
+            else static_cast<T *>(p.row_partials)[static_cast<int64_t>(blockIdx.x) * p.rows + r] = t;
         }
     }
-    if (WANT & kWantColSums) {
-        T *dst = static_cast<T *>(p.partials) + static_cast<int64_t>(blockIdx.x) * p.cols;
-#pragma unroll
-        for (int it = 0; it < ITERS; ++it) {
-            if (!ok[it]) continue;
-            vec_t v;
-#pragma unroll
-            for (int j = 0; j < V; ++j) v[j] = colacc[it][j];
-            *reinterpret_cast<vec_t *>(dst + col[it]) = v;
-        }
-    }
+    if ((WANT & kWantColSums) && ok)
+        *reinterpret_cast<vec_t *>(static_cast<T *>(p.partials) + static_cast<int64_t>(blockIdx.y) * p.cols + col) = colacc;
 }
 
-// out[k] = sum over blocks (in block order within each of the 16 walkers, walkers added in order) of partials[b][k]
+// Column blocks (the first `col_blocks`): out[k] = sum over bands of partials[band][k], in band order within each of 16
+// walkers, the walkers added in order.  Row blocks (the rest): out[r] = sum over tiles of row_partials[tile][r], in
+// tile order.
 constexpr int kFinishThreads = 1024;
 
 template <typename T>
-__global__ __launch_bounds__(kFinishThreads) void lse_cotangent_col_finish(const T *__restrict__ partials, int n_blocks, int64_t cols,
-                                                                   T *__restrict__ out) {
+__global__ __launch_bounds__(kFinishThreads) void lse_cotangent_finish(const T *__restrict__ partials, int n_bands, int64_t cols,
+                                                               T *__restrict__ col_out, int col_blocks,
+                                                               const T *__restrict__ row_partials, int n_tiles, int64_t rows,
+                                                               T *__restrict__ row_out) {
     constexpr int kCols = 64, kWalkers = kFinishThreads / kCols;
     __shared__ T part[kWalkers][kCols];
+    if (static_cast<int>(blockIdx.x) >= col_blocks) {  // the same for the whole block
+        const int64_t r = static_cast<int64_t>(blockIdx.x - col_blocks) * kFinishThreads + threadIdx.x;
+        if (r < rows) {
+            T t = row_partials[r];
+            for (int k = 1; k < n_tiles; ++k) t += row_partials[static_cast<int64_t>(k) * rows + r];
+            row_out[r] = t;
+        }
+        return;
+    }
     const int c = threadIdx.x % kCols, w = threadIdx.x / kCols;
     const int64_t k = static_cast<int64_t>(blockIdx.x) * kCols + c;
     T acc = T(0);
     if (k < cols) {
 #pragma unroll 8
-        for (int b = w; b < n_blocks; b += kWalkers) acc += partials[static_cast<int64_t>(b) * cols + k];
+        for (int b = w; b < n_bands; b += kWalkers) acc += partials[static_cast<int64_t>(b) * cols + k];
     }
     part[w][c] = acc;
     __syncthreads();
@@ -206,14 +227,14 @@ __global__ __launch_bounds__(kFinishThreads) void lse_cotangent_col_finish(const
         T t = part[0][c];
 #pragma unroll
         for (int i = 1; i < kWalkers; ++i) t += part[i][c];
-        out[k] = t;
+        col_out[k] = t;
     }
 }
 
-template <typename T, int ITERS>
-static void launch_rows(int want, const LseCotParams &p, unsigned blocks, hipStream_t s) {
+template <typename T>
+static void launch_tiles(int want, const LseCotParams &p, dim3 grid, hipStream_t s) {
 #define AGMI_LSECOT(W) \
-    case W: hipLaunchKernelGGL((lse_cotangent_rows<T, ITERS, W>), dim3(blocks), dim3(kBlock), 0, s, p); break;
+    case W: hipLaunchKernelGGL((lse_cotangent_tile<T, W>), grid, dim3(kBlock), 0, s, p); break;
     switch (want) {
         AGMI_LSECOT(1) AGMI_LSECOT(2) AGMI_LSECOT(3) AGMI_LSECOT(4) AGMI_LSECOT(5) AGMI_LSECOT(6) AGMI_LSECOT(7)
         default: break;
@@ -224,9 +245,8 @@ static void launch_rows(int want, const LseCotParams &p, unsigned blocks, hipStr
 template <typename T>
 static int launch_lse_cotangent(const agmi_lse_cotangent &c, void *workspace, size_t workspace_bytes, hipStream_t s) {
     constexpr int V = 16 / sizeof(T);
-    const int64_t max_cols = static_cast<int64_t>(kBlock) * V * kLseCotMaxIters;
-    if (c.cols % V != 0 || c.cols > max_cols) {
-        set_error("lse_cotangent: %lld columns (must be a multiple of %d and at most %lld)", (long long)c.cols, V, (long long)max_cols);
+    if (c.cols % V != 0) {
+        set_error("lse_cotangent: %lld columns (must be a multiple of %d)", (long long)c.cols, V);
         return AGMI_ERR_UNSUPPORTED;
     }
     int want = 0;
@@ -239,19 +259,21 @@ static int launch_lse_cotangent(const agmi_lse_cotangent &c, void *workspace, si
     p.x = c.x; p.x_rs = c.x_row_stride;
     p.scale = (c.affine & AGMI_AFFINE_SCALE) ? c.scale : 1.0;
     p.shift = (c.affine & AGMI_AFFINE_SHIFT) ? c.shift : 0.0;
+    // (the stride of an axis of extent 1 is never used: any value is as good as 0)
+    const int64_t scale_row_stride = c.rows == 1 ? 0 : c.scale_row_stride, shift_row_stride = c.rows == 1 ? 0 : c.shift_row_stride;
     if (c.affine & AGMI_AFFINE_SCALE_AUX) {
-        if (!c.scale_vec || (c.scale_col_stride != 0 && (c.scale_col_stride != 1 || c.scale_row_stride != 0))) {
+        if (!c.scale_vec || (c.scale_col_stride != 0 && (c.scale_col_stride != 1 || scale_row_stride != 0))) {
             set_error("lse_cotangent: the array factor must vary along rows only or along columns only (unit stride)");
             return AGMI_ERR_UNSUPPORTED;
         }
-        p.scale_vec = c.scale_vec; p.scale_rs = c.scale_row_stride; p.scale_by_col = c.scale_col_stride == 1;
+        p.scale_vec = c.scale_vec; p.scale_rs = scale_row_stride; p.scale_by_col = c.scale_col_stride == 1;
     }
     if (c.affine & AGMI_AFFINE_SHIFT_AUX) {
-        if (!c.shift_vec || (c.shift_col_stride != 0 && (c.shift_col_stride != 1 || c.shift_row_stride != 0))) {
+        if (!c.shift_vec || (c.shift_col_stride != 0 && (c.shift_col_stride != 1 || shift_row_stride != 0))) {
             set_error("lse_cotangent: the array offset must vary along rows only or along columns only (unit stride)");
             return AGMI_ERR_UNSUPPORTED;
         }
-        p.shift_vec = c.shift_vec; p.shift_rs = c.shift_row_stride; p.shift_by_col = c.shift_col_stride == 1;
+        p.shift_vec = c.shift_vec; p.shift_rs = shift_row_stride; p.shift_by_col = c.shift_col_stride == 1;
     }
     p.ans = c.ans; p.ans_rs = c.ans_stride;
     p.g = c.g; p.g_rs = c.g_stride;
@@ -261,49 +283,49 @@ static int launch_lse_cotangent(const agmi_lse_cotangent &c, void *workspace, si
         set_error("lse_cotangent: the scaled copy needs a column factor and a row stride >= cols");
         return AGMI_ERR_ARG;
     }
-    // 512 bands (two blocks of four waves per CU, each with two rows of loads in flight) measured best on
-    // 8192 x 4096: more bands make the column partials (one row per band) and their summation cost more
-    // than the extra waves gain, fewer leave CUs short of loads in flight
-    int64_t rpb = std::max<int64_t>(8, ceil_div(c.rows, 512));
-    if (want & kWantColSums) {
-        if (!workspace) {
-            set_error("lse_cotangent: column sums need a workspace");
-            return AGMI_ERR_WORKSPACE;
-        }
-        const int64_t fit = static_cast<int64_t>(workspace_bytes / (sizeof(T) * static_cast<size_t>(c.cols)));
-        if (fit < 1) {
-            set_error("lse_cotangent: workspace smaller than one row of partial sums");
-            return AGMI_ERR_WORKSPACE;
-        }
-        rpb = std::max(rpb, ceil_div(c.rows, fit));
+    const int64_t tiles_across = ceil_div(c.cols, static_cast<int64_t>(kBlock) * V);
+    const bool row_partials = (want & kWantRowSums) && tiles_across > 1;
+    // Tiles of 16 rows measured best on 8192 x 4096 (2048 blocks: 74 us for the forward reduction, this pass and its
+    // finish against 79 us with 512 long bands, 86 us with tiles of 32 rows); taller tiles only when the
+    // partial column sums (one row per band of rows) would not fit the workspace.
+    int64_t rpb = kLseCotRowGroup;
+    const auto staged = [&](int64_t rows_per_band, size_t *col_bytes) {
+        *col_bytes = (want & kWantColSums) ? static_cast<size_t>(ceil_div(c.rows, rows_per_band)) * static_cast<size_t>(c.cols) * sizeof(T) : 0;
+        *col_bytes = (*col_bytes + 255) / 256 * 256;
+        return *col_bytes + (row_partials ? static_cast<size_t>(tiles_across) * static_cast<size_t>(c.rows) * sizeof(T) : 0);
+    };
+    size_t col_bytes = 0;
+    size_t need = staged(rpb, &col_bytes);
+    while ((need > workspace_bytes || ceil_div(c.rows, rpb) > 65535) && rpb < kLseCotMaxRowsPerBlock) {  // (65535: the grid's y extent)
+        rpb += kLseCotRowGroup;
+        need = staged(rpb, &col_bytes);
     }
-    if (rpb > kLseCotMaxRowsPerBlock) {
-        // more rows than 512 (or the workspace allows) bands of 64: take more blocks, the band length is what LDS holds
-        rpb = kLseCotMaxRowsPerBlock;
-        if ((want & kWantColSums) &&
-            static_cast<size_t>(ceil_div(c.rows, rpb)) * static_cast<size_t>(c.cols) * sizeof(T) > workspace_bytes) {
-            set_error("lse_cotangent: workspace too small for %lld bands of partial sums", (long long)ceil_div(c.rows, rpb));
-            return AGMI_ERR_WORKSPACE;
-        }
+    if (need > 0 && !workspace) {
+        set_error("lse_cotangent: partial sums need a workspace (%zu bytes)", need);
+        return AGMI_ERR_WORKSPACE;
     }
-    const int64_t blocks = ceil_div(c.rows, rpb);
-    if (blocks > 0x7fffffffLL) {
-        set_error("lse_cotangent: too many rows");
+    if (need > workspace_bytes) {
+        set_error("lse_cotangent: workspace of %zu bytes is too small for the partial sums (%zu bytes)", workspace_bytes, need);
+        return AGMI_ERR_UNSUPPORTED;
+    }
+    const int64_t bands = ceil_div(c.rows, rpb);
+    if (bands > 65535 || tiles_across > 0x7fffffffLL) {
+        set_error("lse_cotangent: too many rows or columns for one launch");
         return AGMI_ERR_UNSUPPORTED;
     }
     p.rows_per_block = static_cast<int>(rpb);
     p.partials = workspace;
-    const int64_t need = ceil_div(c.cols, static_cast<int64_t>(kBlock) * V);
-    set_kernel_name("lse_cotangent_rows<%s%s%s>", (want & kWantScaled) ? "scaled," : "", (want & kWantRowSums) ? "rowsum," : "",
+    p.row_partials = row_partials ? static_cast<unsigned char *>(workspace) + col_bytes : nullptr;
+    set_kernel_name("lse_cotangent_tile<%s%s%s>", (want & kWantScaled) ? "scaled," : "", (want & kWantRowSums) ? "rowsum," : "",
                     (want & kWantColSums) ? "colsum" : "");
-    if (need <= 1) launch_rows<T, 1>(want, p, static_cast<unsigned>(blocks), s);
-    else if (need <= 2) launch_rows<T, 2>(want, p, static_cast<unsigned>(blocks), s);
-    else if (need <= 4) launch_rows<T, 4>(want, p, static_cast<unsigned>(blocks), s);
-    else launch_rows<T, 8>(want, p, static_cast<unsigned>(blocks), s);
+    launch_tiles<T>(want, p, dim3(static_cast<unsigned>(tiles_across), static_cast<unsigned>(bands)), s);
     if (int rc = hip_check(hipGetLastError(), "lse_cotangent launch")) return rc;
-    if (want & kWantColSums) {
-        hipLaunchKernelGGL(lse_cotangent_col_finish<T>, dim3(static_cast<unsigned>(ceil_div(c.cols, 64))), dim3(kFinishThreads), 0, s,
-                           static_cast<const T *>(workspace), static_cast<int>(blocks), c.cols, static_cast<T *>(c.col_sums));
+    const int col_blocks = (want & kWantColSums) ? static_cast<int>(ceil_div(c.cols, 64)) : 0;
+    const int row_blocks = row_partials ? static_cast<int>(ceil_div(c.rows, kFinishThreads)) : 0;
+    if (col_blocks + row_blocks > 0) {
+        hipLaunchKernelGGL(lse_cotangent_finish<T>, dim3(static_cast<unsigned>(col_blocks + row_blocks)), dim3(kFinishThreads), 0, s,
+                           static_cast<const T *>(workspace), static_cast<int>(bands), c.cols, static_cast<T *>(c.col_sums), col_blocks,
+                           static_cast<const T *>(p.row_partials), static_cast<int>(tiles_across), c.rows, static_cast<T *>(c.row_sums));
         return hip_check(hipGetLastError(), "lse_cotangent finish launch");
     }
     return 0;

@@ -319,7 +319,7 @@ class LseCotangent(DevArray):
             return False
         h = x._h()
         vec = 16 // dtype.itemsize
-        if h.shape[0] == 0 or h.shape[1] == 0 or h.shape[1] % vec or h.shape[1] > 256 * vec * 8 or h.stride(1) != 1:
+        if h.shape[0] == 0 or h.shape[1] == 0 or h.shape[1] % vec or h.stride(1) != 1:
             return False
         if type(x) is LazyDevArray:
             for aux in (x._ascale, x._shift):

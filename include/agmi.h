@@ -234,10 +234,13 @@ int agmi_map_reduce_static(int op, int red, int dtype, int ndim, const int64_t *
  *     col_sums[k]  = sum_r mem[r,k] * S[r,k]   multiply rule for the broadcast factor (80-83, 883-892)
  * mem is row-major with unit column stride; scale_vec / shift_vec vary along rows only (column
  * stride 0) or along columns only (row stride 0, column stride 1); cols must be a multiple of the
- * 16-byte vector (4 float32 / 2 float64) and at most 8192 float32 / 4096 float64.  Column sums
- * are staged per band of rows in `workspace` (cols * ceil(rows / 64) elements always suffice) and
- * added in a fixed order; nothing is atomic.  Returns AGMI_ERR_UNSUPPORTED for layouts outside
- * this (the caller then forms S with AGMI_OP_LSE_VJP and reduces it with agmi_map_reduce). */
+ * 16-byte vector (4 float32 / 2 float64).  The matrix is cut into tiles of 16 rows by 256 vectors;
+ * column sums are staged per band of rows and, when the matrix is more than one tile wide, row
+ * sums per tile, in `workspace` (cols * ceil(rows / 16) + rows * ceil(cols / 1024) float32 elements,
+ * / 512 for float64; a smaller workspace is met with bands of up to 64 rows) and added in a fixed
+ * order by a second kernel; nothing is atomic.  Returns AGMI_ERR_UNSUPPORTED for layouts outside
+ * this or a workspace that cannot hold the partial sums (the caller then forms S with
+ * AGMI_OP_LSE_VJP and reduces it with agmi_map_reduce). */
 typedef struct agmi_lse_cotangent {
     int64_t rows, cols;
     const void *x;              /* mem */
