@@ -443,7 +443,10 @@ __device__ __forceinline__ v4i raw_buffer(const void *base, uint32_t bytes) {
     return r;
 }
 
-template <int MODE_A, int MODE_B>
+// TAIL: K is not a multiple of 4 and an operand is contiguous along k, so the 16 bytes a lane fetches at the end of
+// a row run past k = K into whatever follows in memory (the next row); those elements are zeroed in LDS before
+// any wave reads the slab.
+template <int MODE_A, int MODE_B, bool TAIL>
 __global__ __launch_bounds__(kDirectThreads) void gemm_direct(const GemmParams p) {
     constexpr int BM = 64, BN = 64, BK = 32, NBUF = 4;
     constexpr int kOpFloats = 64 * BK;         // one operand slab
@@ -510,17 +513,44 @@ __global__ __launch_bounds__(kDirectThreads) void gemm_direct(const GemmParams p
         krem_b = (n0 + xl < p.N) ? static_cast<int>(k_limit - k_first) - 4 * k4 : 0;
     }
     const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));  // LDS byte address
+    // TAIL: where (float index in `lds`), in which slab and from which element on this lane's group runs past K
+    int fix_a_at = 0, fix_a_from = 4, fix_a_slab = -1, fix_b_at = 0, fix_b_from = 4, fix_b_slab = -1, issued = 0;
     auto issue_a = [&](int buf) __attribute__((always_inline)) {
+        if (TAIL && MODE_A == kKC && krem_a > 0 && krem_a < 4) {
+            fix_a_at = buf * kBufFloats + wave * 256 + lane * 4;
+            fix_a_from = krem_a;
+            fix_a_slab = issued;
+        }
         load_to_lds_16(rsrc_a, krem_a > 0 ? off_a : kDirectOob,
                        lds_base + static_cast<uint32_t>(buf * kBufFloats + wave * 256) * 4u);
         off_a += step_a;
         krem_a -= BK;
     };
     auto issue_b = [&](int buf) __attribute__((always_inline)) {
+        if (TAIL && MODE_B == kKC && krem_b > 0 && krem_b < 4) {
+            fix_b_at = buf * kBufFloats + kOpFloats + wave * 256 + lane * 4;
+            fix_b_from = krem_b;
+            fix_b_slab = issued;
+        }
         load_to_lds_16(rsrc_b, krem_b > 0 ? off_b : kDirectOob,
                        lds_base + static_cast<uint32_t>(buf * kBufFloats + kOpFloats + wave * 256) * 4u);
         off_b += step_b;
         krem_b -= BK;
+        ++issued;  // (a slab's A is always issued before its B)
+    };
+    // called once this lane's loads of `slab` have landed and before the barrier that publishes the slab
+    auto zero_tail = [&](int slab) __attribute__((always_inline)) {
+        if (!TAIL) return;
+        if (MODE_A == kKC && fix_a_slab == slab) {
+#pragma unroll
+            for (int j = 1; j < 4; ++j)
+                if (j >= fix_a_from) lds[fix_a_at + j] = 0.f;
+        }
+        if (MODE_B == kKC && fix_b_slab == slab) {
+#pragma unroll
+            for (int j = 1; j < 4; ++j)
+                if (j >= fix_b_from) lds[fix_b_at + j] = 0.f;
+        }
     };
 
     // fragment addresses (floats within one operand slab) of this wave's groups q = NQ * kgroup + qq
@@ -564,12 +594,14 @@ __global__ __launch_bounds__(kDirectThreads) void gemm_direct(const GemmParams p
         issue_b(d);
     }
     wait_vmcnt<(kDist - 1) * 2>();
+    zero_tail(0);
     __syncthreads();
 #pragma unroll
     for (int qq = 0; qq < NQ; ++qq) read_frag(0, 0, qq);
 
-    auto step = [&](const int tb /* t % NBUF */, const int f /* t % 2 */) __attribute__((always_inline)) {
+    auto step = [&](const int tb /* t % NBUF */, const int f /* t % 2 */, const int t) __attribute__((always_inline)) {
         wait_vmcnt<(kDist - 2) * 2>();  // all but the youngest slab's two loads: slab t+1 is in LDS
+        zero_tail(t + 1);
         __syncthreads();
 #pragma unroll
         for (int qq = 0; qq < NQ; ++qq) {
@@ -588,11 +620,11 @@ __global__ __launch_bounds__(kDirectThreads) void gemm_direct(const GemmParams p
     int t = 0;
     for (; t + NBUF <= n_slabs; t += NBUF) {
 #pragma unroll
-        for (int d = 0; d < NBUF; ++d) step(d, d & 1);
+        for (int d = 0; d < NBUF; ++d) step(d, d & 1, t + d);
     }
 #pragma unroll
     for (int d = 0; d < NBUF - 1; ++d)
-        if (t + d < n_slabs) step(d, d & 1);  // uniform across the block
+        if (t + d < n_slabs) step(d, d & 1, t + d);  // uniform across the block
 
     // the loads still in flight (zeros for slabs past the end) must land before LDS is reused
     wait_vmcnt<0>();
@@ -612,6 +644,9 @@ __global__ __launch_bounds__(kDirectThreads) void gemm_direct(const GemmParams p
     const int64_t row0 = m0 + wm0 + 4 * h;
     const bool interior = m0 + BM <= p.M && n0 + BN <= p.N;  // uniform: no per-element bounds tests
     if (p.splits > 1) {  // raw partial tile; gemm_split_finish applies alpha / beta
+        // (Adding the partial tiles up in the block that arrives last at a tile, behind an arrival counter, was
+        // measured: the device-wide fences it needs write back and invalidate a whole XCD's L2 per block, and the
+        // recurrent-net tape ran at half the rate.  The second kernel stays.)
         float *W = static_cast<float *>(p.ws) + (static_cast<int64_t>(blockIdx.z) * gridDim.y + batch) * p.M * p.N +
                    row0 * p.N + col;
 #pragma unroll
@@ -755,16 +790,16 @@ static int launch_gemm(GemmParams p, int64_t batch, hipStream_t s, void *ws = nu
     return hip_check(hipGetLastError(), "gemm launch");
 }
 
-// Operand layouts gemm_direct accepts: a unit stride along x or k, the other stride a positive
-// multiple of 4 elements, and whole 16-byte groups (so a lane's group is entirely inside the
-// matrix or entirely outside).  Returns kXC, kKC or -1.
+// Operand layouts gemm_direct accepts: a unit stride along x or k and a positive other stride.  Returns kXC, kKC
+// or -1.  Nothing needs 16-byte alignment: the loads take any 4-byte aligned address, the buffer range check is made
+// dword by dword (what lies past the operand's last element reads as zero), a group that runs past the last x only
+// feeds rows / columns of the tile that are never stored, and a group that runs past the last k is zeroed in LDS
+// (the TAIL instantiations).
 static int direct_mode(int64_t x_stride, int64_t k_stride, int64_t X, int64_t K) {
-    if (x_stride == 1 && X % 4 == 0 && (K == 1 || (k_stride > 0 && k_stride % 4 == 0))) return kXC;
-    if (k_stride == 1 && K % 4 == 0 && (X == 1 || (x_stride > 0 && x_stride % 4 == 0))) return kKC;
+    if (x_stride == 1 && (K == 1 || k_stride > 0)) return kXC;
+    if (k_stride == 1 && (X == 1 || x_stride > 0)) return kKC;
     return -1;
 }
-
-static bool aligned16(const void *ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
 
 // fp32 product through gemm_direct; returns 1 when the operands do not qualify (nothing launched).
 static int launch_direct(GemmParams p, int64_t batch, hipStream_t s, void *ws, size_t ws_bytes) {
@@ -773,8 +808,7 @@ static int launch_direct(GemmParams p, int64_t batch, hipStream_t s, void *ws, s
     const int mode_a = direct_mode(p.a_rs, p.a_cs, p.M, p.K);
     const int mode_b = direct_mode(p.b_cs, p.b_rs, p.N, p.K);
     if (mode_a < 0 || mode_b < 0) return 1;
-    if (!aligned16(p.A) || !aligned16(p.B)) return 1;
-    if (batch > 1 && (p.a_bs % 4 != 0 || p.b_bs % 4 != 0 || p.a_bs < 0 || p.b_bs < 0)) return 1;
+    if (batch > 1 && (p.a_bs < 0 || p.b_bs < 0)) return 1;
     const int64_t a_span = ((p.M - 1) * p.a_rs + (p.K - 1) * p.a_cs + 1) * 4;
     const int64_t b_span = ((p.K - 1) * p.b_rs + (p.N - 1) * p.b_cs + 1) * 4;
     if (a_span > kMaxSpan || b_span > kMaxSpan || BK * p.a_cs * 4 > kMaxSpan || BK * p.b_rs * 4 > kMaxSpan) return 1;
@@ -803,14 +837,21 @@ static int launch_direct(GemmParams p, int64_t batch, hipStream_t s, void *ws, s
         set_kernel_name("gemm_direct<f32,64,64,32,%s%s>", mode_name(mode_a), mode_name(mode_b));
     const dim3 grid((unsigned)(tm * tn), (unsigned)batch, (unsigned)p.splits);
     const dim3 block(kDirectThreads);
+    const bool tail = p.K % 4 != 0 && (mode_a == kKC || mode_b == kKC);
     if (mode_a == kXC && mode_b == kXC)
-        hipLaunchKernelGGL((gemm_direct<kXC, kXC>), grid, block, 0, s, p);
+        hipLaunchKernelGGL((gemm_direct<kXC, kXC, false>), grid, block, 0, s, p);
+    else if (mode_a == kXC && tail)
+        hipLaunchKernelGGL((gemm_direct<kXC, kKC, true>), grid, block, 0, s, p);
     else if (mode_a == kXC)
-        hipLaunchKernelGGL((gemm_direct<kXC, kKC>), grid, block, 0, s, p);
+        hipLaunchKernelGGL((gemm_direct<kXC, kKC, false>), grid, block, 0, s, p);
+    else if (mode_b == kXC && tail)
+        hipLaunchKernelGGL((gemm_direct<kKC, kXC, true>), grid, block, 0, s, p);
     else if (mode_b == kXC)
-        hipLaunchKernelGGL((gemm_direct<kKC, kXC>), grid, block, 0, s, p);
+        hipLaunchKernelGGL((gemm_direct<kKC, kXC, false>), grid, block, 0, s, p);
+    else if (tail)
+        hipLaunchKernelGGL((gemm_direct<kKC, kKC, true>), grid, block, 0, s, p);
     else
-        hipLaunchKernelGGL((gemm_direct<kKC, kKC>), grid, block, 0, s, p);
+        hipLaunchKernelGGL((gemm_direct<kKC, kKC, false>), grid, block, 0, s, p);
     if (int rc = hip_check(hipGetLastError(), "gemm launch")) return rc;
     if (p.splits > 1) {
         const int64_t n = batch * p.M * p.N;

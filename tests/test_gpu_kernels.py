@@ -356,6 +356,28 @@ def test_dot_all_operand_layouts(dnp, dtype, M, N, K):
               (a[::2, ::2].astype(F64) @ b[::2, ::2].astype(F64)).astype(dtype), rt)        # generic strides
 
 
+@pytest.mark.parametrize("K", [1, 2, 3, 5, 30, 33, 127, 641])
+def test_dot_rows_that_end_inside_a_vector_do_not_see_their_neighbours(dnp, K):
+    """An operand contiguous along k whose K is not a multiple of 4: the 16 bytes fetched at the end of a row run
+    into the next row.  Whatever lies there, an infinity included, must not reach the product (inf * 0 is NaN)."""
+    rs = onp.random.RandomState(K)
+    M, N = 70, 45
+    a, b = rs.randn(M, K).astype(F32), rs.randn(K, N).astype(F32)
+    bt = onp.ascontiguousarray(b.T)
+    a[5, 0] = a[33, min(1, K - 1)] = onp.inf      # the elements right after rows 4 and 32
+    bt[7, 0] = bt[20, min(2, K - 1)] = -onp.inf
+    with onp.errstate(invalid="ignore"):
+        want_nn = a.astype(F64) @ b.astype(F64)
+        want_nt = a.astype(F64) @ bt.T.astype(F64)
+    A, B, Bt = P(dnp, a), P(dnp, b), P(dnp, bt)
+    for got, want in ((dnp.dot(A, B).numpy(), want_nn), (dnp.dot(A, dnp.transpose(Bt)).numpy(), want_nt),
+                      (dnp.dot(Bt, dnp.transpose(A)).numpy(), want_nt.T)):
+        assert onp.array_equal(onp.isfinite(got), onp.isfinite(want))
+        assert onp.array_equal(onp.isnan(got), onp.isnan(want)) and onp.array_equal(onp.isposinf(got), onp.isposinf(want))
+        fin = onp.isfinite(want)
+        close(got[fin], want[fin].astype(F32), RT[F32] * max(1.0, onp.sqrt(K) / 8))
+
+
 def test_dot_small_integers_exact(dnp):
     rs = onp.random.RandomState(12)
     a = rs.randint(-4, 5, (200, 333)).astype(F32)
