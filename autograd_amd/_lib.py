@@ -184,6 +184,8 @@ def lib():
     L.agmi_sort_rows.argtypes = [c_i, c_p, c_i64, c_i64, c_p, c_p, c_p, c_p]
     L.agmi_cumsum.restype = c_i
     L.agmi_cumsum.argtypes = [c_i, c_p, c_i64, c_i64, c_i64, c_p, c_p]
+    L.agmi_concat.restype = c_i
+    L.agmi_concat.argtypes = [c_i, c_i64, c_i64, c_i, c_p, c_p, c_p]
     L.agmi_take_rows.restype = c_i
     L.agmi_take_rows.argtypes = [c_i, c_p, c_i64, c_i64, c_p, c_i64, c_p, c_p]
     L.agmi_scatter_add_rows.restype = c_i
@@ -201,7 +203,7 @@ def lib():
 EXPORTS = (
     "agmi_last_error agmi_version agmi_last_kernel agmi_elementwise agmi_compare agmi_cast agmi_map_reduce "
     "agmi_map_reduce_workspace_bytes agmi_map_reduce_static agmi_gemm agmi_fill agmi_take_rows agmi_sort_rows agmi_cumsum agmi_reverse agmi_triangle agmi_scatter_add_rows agmi_optimizer_step "
-    "agmi_correlate agmi_lse_cotangent_fused"
+    "agmi_correlate agmi_lse_cotangent_fused agmi_concat"
 ).split()
 
 
@@ -583,6 +585,29 @@ def fill(code, t, value):
     rc = _LIB.agmi_fill(code, t.data_ptr(), t.numel(), float(value), _stream())
     if rc:
         _check(rc, "agmi_fill")
+
+
+MAX_CONCAT = 8
+
+
+class AgmiConcatPiece(ctypes.Structure):
+    _fields_ = [("data", ctypes.c_void_p), ("extent", ctypes.c_int64), ("stride_outer", ctypes.c_int64),
+                ("stride_axis", ctypes.c_int64), ("stride_inner", ctypes.c_int64)]
+
+
+_concat_pieces = (AgmiConcatPiece * MAX_CONCAT)()
+
+
+def concat(code, outer, inner, pieces, out):
+    """``pieces``: (tensor, extent, stride_outer, stride_axis, stride_inner) per piece, joined along the middle axis
+    of the contiguous (outer, total, inner) tensor ``out`` in one launch."""
+    for k, (t, extent, so, sa, si) in enumerate(pieces):
+        slot = _concat_pieces[k]
+        slot.data, slot.extent, slot.stride_outer, slot.stride_axis, slot.stride_inner = t.data_ptr(), extent, so, sa, si
+    ev = _TIMER.begin(("concat",)) if _TIMER is not None else None
+    _check(_LIB.agmi_concat(code, outer, inner, len(pieces), _concat_pieces, out.data_ptr(), _stream()), "agmi_concat")
+    if ev is not None:
+        _TIMER.end(ev, ("concat",), 2 * out.numel() * out.element_size())
 
 
 def take_rows(code, src, n_rows, inner, index, n_index, out):

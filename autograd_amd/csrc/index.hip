@@ -322,9 +322,89 @@ __global__ __launch_bounds__(kBlock) void place_by_rank(const T *__restrict__ sr
     if (order) order[row * n + k] = i;
 }
 
+// ---- concatenation ------------------------------------------------------------------------------
+struct ConcatParams {
+    const void *data[AGMI_MAX_CONCAT];
+    int64_t end[AGMI_MAX_CONCAT];  // one past the piece's last position along the joined axis
+    int64_t so[AGMI_MAX_CONCAT], sa[AGMI_MAX_CONCAT], si[AGMI_MAX_CONCAT];
+    int n_pieces;
+    int64_t total, inner, n;
+};
+
+// one thread per element of the contiguous (outer, total, inner) result
+template <typename T>
+__global__ __launch_bounds__(kBlock) void concat_kernel(const ConcatParams p, T *__restrict__ out) {
+    const int64_t e = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (e >= p.n) return;
+    const int64_t i = e % p.inner, rest = e / p.inner;
+    const int64_t a = rest % p.total, o = rest / p.total;
+    int k = 0;
+    int64_t begin = 0;
+#pragma unroll
+    for (int j = 0; j < AGMI_MAX_CONCAT - 1; ++j) {
+        if (a >= p.end[j]) {
+            k = j + 1;
+            begin = p.end[j];
+        }
+    }
+    out[e] = static_cast<const T *>(p.data[k])[o * p.so[k] + (a - begin) * p.sa[k] + i * p.si[k]];
+}
+
 }  // namespace agmi
 
 using namespace agmi;
+
+extern "C" int agmi_concat(int dtype, int64_t outer, int64_t inner, int n_pieces, const agmi_concat_piece *pieces, void *out,
+                           void *stream) {
+    if (outer < 0 || inner < 0 || n_pieces < 0 || n_pieces > AGMI_MAX_CONCAT) {
+        set_error("concat: bad extents or more than %d pieces", AGMI_MAX_CONCAT);
+        return AGMI_ERR_ARG;
+    }
+    if (n_pieces > 0 && !pieces) {
+        set_error("concat: null piece table");
+        return AGMI_ERR_ARG;
+    }
+    ConcatParams p = {};
+    int64_t total = 0;
+    for (int k = 0; k < n_pieces; ++k) {
+        if (pieces[k].extent < 0 || (pieces[k].extent > 0 && outer > 0 && inner > 0 && !pieces[k].data)) {
+            set_error("concat: piece %d has a negative extent or no data", k);
+            return AGMI_ERR_ARG;
+        }
+        total += pieces[k].extent;
+        p.data[k] = pieces[k].data;
+        p.end[k] = total;
+        p.so[k] = pieces[k].stride_outer;
+        p.sa[k] = pieces[k].stride_axis;
+        p.si[k] = pieces[k].stride_inner;
+    }
+    for (int k = n_pieces; k < AGMI_MAX_CONCAT; ++k) p.end[k] = total;
+    p.n_pieces = n_pieces;
+    p.total = total;
+    p.inner = inner;
+    p.n = outer * total * inner;
+    if (p.n == 0) return 0;
+    if (!out) {
+        set_error("concat: null output");
+        return AGMI_ERR_ARG;
+    }
+    const int64_t blocks = ceil_div(p.n, kBlock);
+    if (blocks > 0x7fffffffLL) {
+        set_error("concat: too many elements");
+        return AGMI_ERR_UNSUPPORTED;
+    }
+    hipStream_t s = as_stream(stream);
+    set_kernel_name("concat_kernel");
+    if (dtype == AGMI_F32)
+        hipLaunchKernelGGL(concat_kernel<float>, dim3((unsigned)blocks), dim3(kBlock), 0, s, p, static_cast<float *>(out));
+    else if (dtype == AGMI_F64)
+        hipLaunchKernelGGL(concat_kernel<double>, dim3((unsigned)blocks), dim3(kBlock), 0, s, p, static_cast<double *>(out));
+    else {
+        set_error("concat: dtype %d is not a floating type", dtype);
+        return AGMI_ERR_ARG;
+    }
+    return hip_check(hipGetLastError(), "concat launch");
+}
 
 extern "C" int agmi_take_rows(int dtype, const void *src, int64_t n_rows, int64_t inner, const int64_t *index,
                               int64_t n_index, void *out, void *stream) {

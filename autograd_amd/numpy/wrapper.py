@@ -517,6 +517,44 @@ def repeat(x, repeats, axis=None):
     return DevArray(out._t.view(final), x.dtype)
 
 
+def _merged_stride(extents, strides):
+    """The one stride that walks axes of these extents and strides as if they were a single axis (0 for a
+    broadcast group), or None when there is none."""
+    stride, span = None, 1  # span: elements covered by the axes seen so far (innermost first)
+    for extent, st in zip(reversed(extents), reversed(strides)):
+        if extent == 1:
+            continue
+        if stride is None:
+            stride = st
+        elif st != stride * span:
+            return None
+        span *= extent
+    return 0 if stride is None else stride
+
+
+def _concat_pieces(arrs, axis, dt):
+    """The pieces of a concatenation as (tensor, extent, outer stride, axis stride, inner stride), or None when
+    a piece is not a plain strided view (a pending map that is not a launch-free constant, another dtype)."""
+    pieces = []
+    for a in arrs:
+        if a.dtype != dt:
+            return None
+        if type(a) is DevArray:
+            t = a._t
+        elif type(a) is D.LazyDevArray and a._scale == 1.0 and a._shift is None and a._ascale is None:
+            t = a._raw  # a constant: one shared element seen through stride-0 axes
+        else:
+            return None
+        extents, strides = tuple(t.shape), t.stride()
+        so = _merged_stride(extents[:axis], strides[:axis])
+        si = _merged_stride(extents[axis + 1:], strides[axis + 1:])
+        if so is None or si is None:
+            return None
+        if extents[axis]:
+            pieces.append((t, extents[axis], so, strides[axis], si))
+    return pieces if pieces else None
+
+
 @primitive
 def concatenate_args(axis, *args):
     arrs = [D.asarray(a) for a in args]
@@ -535,6 +573,14 @@ def concatenate_args(axis, *args):
         total += a.shape[axis]
     shape = arrs[0].shape[:axis] + (total,) + arrs[0].shape[axis + 1 :]
     out = D.empty(shape, dt)
+    if 2 <= len(arrs) <= _lib.MAX_CONCAT and dt in D._FLOATS and out.size:
+        pieces = _concat_pieces(arrs, axis, dt)
+        if pieces is not None:  # every piece is a strided (outer, extent, inner) view: one launch for all of them
+            outer = 1
+            for extent in shape[:axis]:
+                outer *= extent
+            _lib.concat(_lib.DTYPE_CODE[dt], outer, out.size // (outer * total), pieces, out._t)
+            return out
     start = 0
     for a in arrs:
         n = a.shape[axis]

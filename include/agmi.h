@@ -289,6 +289,19 @@ int agmi_fill(int dtype, void *ptr, int64_t n, double value, void *stream);
 int agmi_take_rows(int dtype, const void *src, int64_t n_rows, int64_t inner,
                    const int64_t *index, int64_t n_index, void *out, void *stream);
 
+/* numpy.concatenate (autograd/numpy/numpy_wrapper.py:58-62, concatenate_args) in one launch: the pieces are
+ * strided (outer, extent, inner) views that are laid one after another along the middle axis of the contiguous
+ * result (outer, sum of extents, inner).  A piece with all strides 0 is a constant column (the ones that
+ * examples/rnn.py:21 appends to its state).  At most AGMI_MAX_CONCAT pieces; none may overlap `out`. */
+#define AGMI_MAX_CONCAT 8
+typedef struct agmi_concat_piece {
+    const void *data;
+    int64_t extent;                                   /* along the joined axis */
+    int64_t stride_outer, stride_axis, stride_inner;  /* element strides */
+} agmi_concat_piece;
+int agmi_concat(int dtype, int64_t outer, int64_t inner, int n_pieces, const agmi_concat_piece *pieces,
+                void *out, void *stream);
+
 /* out[o, k, c] = src[o, n-1-k, c] on contiguous (outer, n, inner) arrays: numpy.flipud / fliplr / rot90
  * (numpy_vjps.py:202-204) and slices that step backwards, A[::-1] (numpy_boxes.py:16-18), whose
  * NumPy form is a view with a negative stride.  src and out must not overlap. */

@@ -378,6 +378,52 @@ def test_dot_rows_that_end_inside_a_vector_do_not_see_their_neighbours(dnp, K):
         close(got[fin], want[fin].astype(F32), RT[F32] * max(1.0, onp.sqrt(K) / 8))
 
 
+@pytest.mark.parametrize("dtype", [F32, F64])
+def test_concatenate_in_one_launch_is_a_copy(dnp, dtype):
+    """Pieces that are strided views (slices, transposes, broadcasts, launch-free constants) are joined by one kernel;
+    anything else (pending maps, other dtypes, more than eight pieces) goes piece by piece.  Either way the result
+    is NumPy's, bit for bit."""
+    from autograd_amd import _lib
+
+    rs = onp.random.RandomState(71)
+    a, b, c = rs.randn(6, 5, 4).astype(dtype), rs.randn(6, 3, 4).astype(dtype), rs.randn(6, 1, 4).astype(dtype)
+    A, B, C = P(dnp, a), P(dnp, b), P(dnp, c)
+    calls = []
+    real = _lib.concat
+    _lib.concat = lambda *args: (calls.append(len(args[3])), real(*args))[1]
+    try:
+        for axis in (0, 1, 2, -1):
+            if axis in (1,):
+                got, want = dnp.concatenate((A, B, C), axis=axis), onp.concatenate((a, b, c), axis=axis)
+            else:
+                got, want = dnp.concatenate((A, A[::-1][::-1], A * 1.0), axis=axis), onp.concatenate((a, a, a), axis=axis)
+            assert got.dtype == want.dtype and onp.array_equal(got.numpy(), want), axis
+        assert len(calls) == 4
+        x, h = rs.randn(7, 13).astype(dtype), rs.randn(7, 30).astype(dtype)
+        X, H = P(dnp, x), P(dnp, h)
+        got = dnp.hstack((X, H, dnp.ones((7, 1), dtype=dtype)))  # the recurrent net's state
+        assert onp.array_equal(got.numpy(), onp.hstack((x, h, onp.ones((7, 1), dtype)))) and calls[-1] == 3
+        got = dnp.hstack((X[:, ::2], dnp.transpose(P(dnp, onp.ascontiguousarray(h.T)))[:, 3:9], dnp.broadcast_to(X[:, :1], (7, 4))))
+        assert onp.array_equal(got.numpy(), onp.hstack((x[:, ::2], h[:, 3:9], onp.broadcast_to(x[:, :1], (7, 4)))))
+        assert onp.array_equal(dnp.vstack((X[1:3], X[5:], X[:0])).numpy(), onp.vstack((x[1:3], x[5:], x[:0])))
+        assert onp.array_equal(dnp.concatenate((X[:, 0], H[:, 1])).numpy(), onp.concatenate((x[:, 0], h[:, 1])))
+        assert onp.array_equal(dnp.stack((X, X * 2.0), axis=1).numpy(), onp.stack((x, x * dtype(2.0)), axis=1))
+        n = len(calls)
+        # not one launch: a pending map that is no constant, ten pieces, mixed precision
+        assert onp.array_equal(dnp.hstack((X, -H)).numpy(), onp.hstack((x, -h)))
+        assert onp.array_equal(dnp.hstack((X,) * 10).numpy(), onp.hstack((x,) * 10))
+        other = F64 if dtype == F32 else F32
+        mixed = dnp.hstack((X, P(dnp, h.astype(other))))
+        assert mixed.dtype == F64 and onp.array_equal(mixed.numpy(), onp.hstack((x, h.astype(other))))
+        assert len(calls) == n
+    finally:
+        _lib.concat = real
+    from autograd_amd.test_util import check_grads
+
+    check_grads(lambda u, v: dnp.hstack((u, v * v, dnp.ones((7, 1)))) ** 2, modes=["fwd", "rev"], order=2)(
+        dnp.asarray(rs.randn(7, 3)), dnp.asarray(rs.randn(7, 2)))
+
+
 def test_dot_small_integers_exact(dnp):
     rs = onp.random.RandomState(12)
     a = rs.randint(-4, 5, (200, 333)).astype(F32)
