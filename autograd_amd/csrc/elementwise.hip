@@ -199,7 +199,7 @@ __global__ __launch_bounds__(kBlock) void ew_rows(const EwParams p, const Index 
     const unsigned scalar_mask = p.scalar_mask;
     const AffineRegs<T, Fn::NIN> affine(p);
     const T *bases[NP];
-    bool broadcast[NP], once[NP];
+    bool broadcast[NP];
 #pragma unroll
     for (int k = 0; k < NP; ++k) {
         const int64_t outer = p.istr[k][0];
@@ -208,7 +208,6 @@ __global__ __launch_bounds__(kBlock) void ew_rows(const EwParams p, const Index 
         // keep the compiler from sinking these reads back behind the branches that use them
         asm volatile("" : : "v"(bases[k]), "s"(inner));
         broadcast[k] = inner == 0;
-        once[k] = outer != 0;  // not repeated for every row: read exactly once, stream it
     }
     T x[NP][V];
 #pragma unroll
@@ -225,7 +224,9 @@ __global__ __launch_bounds__(kBlock) void ew_rows(const EwParams p, const Index 
                 for (int j = 0; j < V; ++j) x[k][j] = s;
             } else if (full) {
                 const vec_t *src = reinterpret_cast<const vec_t *>(base + c0);
-                const vec_t v = once[k] ? __builtin_nontemporal_load(src) : *src;
+                // (an ordinary load: written as `once ? nontemporal : ordinary` the two loads are merged by the
+                // optimiser and the hint is lost, and rows of a matrix are often read again by the next rule)
+                const vec_t v = *src;
 #pragma unroll
                 for (int j = 0; j < V; ++j) x[k][j] = v[j];
             } else {
