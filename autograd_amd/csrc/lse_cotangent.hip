@@ -69,6 +69,9 @@ __device__ __forceinline__ double from_lane(double v, int q) {
     return __builtin_bit_cast(double, (static_cast<unsigned long long>(hi) << 32) | lo);
 }
 
+// Register use is left to the compiler on purpose: with the group's code in a straight line it hoists all 16 rows'
+// loads (192 VGPRs, two waves per SIMD) and that is the fastest form measured: bounding it to 3 / 4 / 6 / 8 waves per
+// SIMD took 43.6 -> 58 / 91 / 178 / 221 us on 8192 x 4096.
 template <typename T, int WANT>
 __global__ __launch_bounds__(kBlock) void lse_cotangent_tile(const LseCotParams p) {
     constexpr int V = 16 / sizeof(T);
@@ -117,7 +120,8 @@ __global__ __launch_bounds__(kBlock) void lse_cotangent_tile(const LseCotParams 
         if (scale_row) sr_v = static_cast<const T *>(p.scale_vec)[rr * p.scale_rs];
         if (shift_row) hr_v = static_cast<const T *>(p.shift_vec)[rr * p.shift_rs];
     };
-    const auto process_row = [&](int64_t r, int q, const vec_t &a) __attribute__((always_inline)) {
+    // process_row returns this lane's share of the row sum (zero for lanes past the last column)
+    const auto process_row = [&](int64_t r, int q, const vec_t &a) __attribute__((always_inline)) -> T {
         const T sr = from_lane(sr_v, q), hr = from_lane(hr_v, q), ans_r = from_lane(ans_v, q), g_r = from_lane(g_v, q);
         T rsum = T(0);
         vec_t o;
@@ -135,12 +139,31 @@ __global__ __launch_bounds__(kBlock) void lse_cotangent_tile(const LseCotParams 
         if ((WANT & kWantScaled) && ok)
             // a matrix-sized result that no kernel of this pass reads back: a streaming store
             __builtin_nontemporal_store(o, reinterpret_cast<vec_t *>(static_cast<T *>(p.scaled) + r * p.scaled_rs + col));
-        if (WANT & kWantRowSums) {
-            if (!ok) rsum = T(0);
+        return ok ? rsum : T(0);
+    };
+    // one row's sum over the wave, lane by lane (the short last group of the matrix)
+    const auto reduce_row = [&](int64_t r, T rsum) __attribute__((always_inline)) {
 #pragma unroll
-            for (int m = 32; m > 0; m >>= 1) rsum += __shfl_xor(rsum, m, 64);
-            if (lane == 0) wave_sums[r - row_begin][wave] = rsum;
-        }
+        for (int m = 32; m > 0; m >>= 1) rsum += __shfl_xor(rsum, m, 64);
+        if (lane == 0) wave_sums[r - row_begin][wave] = rsum;
+    };
+    // The sums of a whole group of 16 rows over the wave, together: at each of the first four exchanges a lane
+    // hands over the half of its rows that its partner keeps, so 8 + 4 + 2 + 1 values cross instead of 16 each
+    // time, and two plain exchanges finish the one row a lane is left with: 17 cross-lane moves for 16 rows, not
+    // 96.  Lane bits 5..2 say which row a lane ends up with; the order of the additions is fixed.
+    const auto reduce_group = [&](int64_t r0, T (&part)[kLseCotRowGroup]) __attribute__((always_inline)) {
+        T v8[8], v4[4], v2[2];
+        const bool b5 = (lane & 32) != 0, b4 = (lane & 16) != 0, b3 = (lane & 8) != 0, b2 = (lane & 4) != 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v8[i] = (b5 ? part[i + 8] : part[i]) + __shfl_xor(b5 ? part[i] : part[i + 8], 32, 64);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v4[i] = (b4 ? v8[i + 4] : v8[i]) + __shfl_xor(b4 ? v8[i] : v8[i + 4], 16, 64);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) v2[i] = (b3 ? v4[i + 2] : v4[i]) + __shfl_xor(b3 ? v4[i] : v4[i + 2], 8, 64);
+        T v = (b2 ? v2[1] : v2[0]) + __shfl_xor(b2 ? v2[0] : v2[1], 4, 64);
+        v += __shfl_xor(v, 2, 64);
+        v += __shfl_xor(v, 1, 64);
+        if ((lane & 3) == 0) wave_sums[(r0 - row_begin) + (lane >> 2)][wave] = v;
     };
 
     // D rows of loads are in flight while a row is worked on.  Whole groups of 16 rows run as straight-line code (no
@@ -153,13 +176,15 @@ __global__ __launch_bounds__(kBlock) void lse_cotangent_tile(const LseCotParams 
 #pragma unroll
         for (int d = 0; d < D; ++d)
             a[d] = __builtin_nontemporal_load(reinterpret_cast<const vec_t *>(static_cast<const T *>(p.x) + (r + d) * p.x_rs + col));
+        T part[kLseCotRowGroup];
 #pragma unroll
         for (int q = 0; q < kLseCotRowGroup; ++q) {
             const vec_t cur = a[q % D];
             if (q + D < kLseCotRowGroup)
                 a[q % D] = __builtin_nontemporal_load(reinterpret_cast<const vec_t *>(static_cast<const T *>(p.x) + (r + q + D) * p.x_rs + col));
-            process_row(r + q, q, cur);
+            part[q] = process_row(r + q, q, cur);
         }
+        if (WANT & kWantRowSums) reduce_group(r, part);
     }
     if (r < row_end) {  // the last rows of the matrix (fewer than 16)
         load_row_operands(r);
@@ -172,7 +197,8 @@ __global__ __launch_bounds__(kBlock) void lse_cotangent_tile(const LseCotParams 
                 if (r + d < row_end) {  // the same for the whole block
                     const vec_t cur = a[d];
                     load_row(r + d + D, a[d]);
-                    process_row(r + d, static_cast<int>(r + d - group), cur);
+                    const T part = process_row(r + d, static_cast<int>(r + d - group), cur);
+                    if (WANT & kWantRowSums) reduce_row(r + d, part);
                 }
             }
         }
