@@ -68,6 +68,8 @@ defjvp(
 )
 
 defjvp(anp.full, "same", argnums=(1,))  # numpy_jvps.py:33
+for _flat in (anp.imag, anp.angle):  # numpy_jvps.py:142-146 for a real argument: a zero tangent
+    defjvp(_flat, lambda g, ans, x: anp.zeros_like(ans))
 defjvp(  # numpy_jvps.py:169-173
     anp.linspace,
     lambda g, ans, start, stop, *args, **kwargs: anp.linspace(g, 0, *args, **kwargs),

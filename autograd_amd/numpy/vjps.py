@@ -673,6 +673,8 @@ defvjp(
 )
 for _identity in (anp.real, anp.real_if_close, anp.conjugate):
     defvjp(_identity, lambda ans, x: lambda g: g)
+for _flat in (anp.imag, anp.angle):  # numpy_vjps.py:220-224 evaluated for a real argument: nothing comes back
+    defvjp(_flat, lambda ans, x: lambda g: anp.zeros_like(x))
 
 
 # ---- dense contractions (numpy_vjps.py:552-747) ----------------------------------------------

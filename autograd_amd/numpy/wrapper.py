@@ -1835,6 +1835,81 @@ def synchronize():
     _lib.synchronize()
 
 
+# ---- what device arrays, being real, make trivial; and the functions whose result SHAPE depends on the data ----
+@primitive
+def imag(x):
+    """The imaginary part of a real array: zeros (its cotangent too, numpy_vjps.py:220)."""
+    s, _, dt, _ = _meta_of(x)
+    return D.constant(s, 0.0, D._float_dtype(dt))
+
+
+@primitive
+def angle(x):
+    """``numpy.angle`` of a real array: pi where it is negative, else 0 (piecewise constant: numpy_vjps.py:224
+    gives a zero cotangent for real arguments)."""
+    x = D.asarray(x)
+    dt = D._float_dtype(x.dtype)
+    return D.map_op(Op.WHERE, dt, D.astype(D.compare(Cmp.LT, x, 0.0), dt), float(onp.pi), 0.0)
+
+
+def isreal(x):
+    from ..tracer import getval
+
+    return D.full(_meta_of(getval(x))[0], True, onp.bool_)
+
+
+def iscomplex(x):
+    from ..tracer import getval
+
+    return D.full(_meta_of(getval(x))[0], False, onp.bool_)
+
+
+def floor_divide(a, b):
+    """``numpy.floor_divide`` (no derivative, numpy_vjps.py:13-68), the way NumPy forms it: the quotient of
+    ``a - remainder(a, b)`` and ``b`` is a whole number up to rounding, so it is rounded to the nearest; a zero
+    divisor gives ``a / b``."""
+    from ..tracer import getval
+
+    a, b = getval(a), getval(b)
+    whole = rint.fun(true_divide.fun(subtract.fun(a, remainder.fun(a, b)), b))
+    return _where3.fun(D.compare(Cmp.EQ, D.asarray(b) if isinstance(b, DevArray) else b, 0.0), true_divide.fun(a, b), whole)
+
+
+def array_equiv(a1, a2):
+    """A Python bool (reads one element back): the shapes broadcast and all elements are equal."""
+    from ..tracer import getval
+
+    a1, a2 = D.asarray(getval(a1)), D.asarray(getval(a2))
+    try:
+        D.broadcast_shapes(a1.shape, a2.shape)
+    except ValueError:
+        return False
+    hit = D.compare(Cmp.EQ, a1, a2)
+    return True if hit.size == 0 else bool(to_numpy(min.fun(D.astype(hit, onp.float64))) == 1.0)
+
+
+def _on_the_host(name):
+    """Functions whose result shape depends on the values (``nonzero`` and friends; none has a derivative,
+    numpy_vjps.py:13-68): the operands are read back, NumPy answers, the integer results are uploaded.  A
+    synchronising transfer, so they cannot be recorded into a graph."""
+    fun = getattr(onp, name)
+
+    def raw(*args, **kwargs):
+        from ..tracer import getval
+
+        host = [to_numpy(getval(a)) if isinstance(getval(a), DevArray) else getval(a) for a in args]
+        out = fun(*host, **kwargs)
+        if isinstance(out, tuple):
+            return tuple(D.from_numpy(onp.ascontiguousarray(o)) for o in out)
+        return D.from_numpy(onp.ascontiguousarray(out))
+
+    raw.__name__ = raw.__qualname__ = name
+    return raw
+
+
+nonzero, flatnonzero, argwhere, searchsorted = (_on_the_host(n) for n in ("nonzero", "flatnonzero", "argwhere", "searchsorted"))
+
+
 def allclose(a, b, rtol=1e-05, atol=1e-08):
     from ..tracer import getval
 

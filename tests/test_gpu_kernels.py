@@ -1095,6 +1095,41 @@ def test_sort_is_stable_and_puts_nans_last(dnp, dtype):
     close(h, (dtype(2.0) * want2 * w).astype(dtype), RT_EW[dtype] * 4)
 
 
+def test_real_array_trivia_and_data_dependent_shapes(dnp):
+    """The last names of the reference's rule table (numpy_vjps.py:13-68, 220-224): what is trivial for real
+    arrays (imag, angle, isreal, iscomplex), floor_divide, array_equiv, and the functions whose result shape
+    depends on the data (answered by NumPy on the host, indices uploaded)."""
+    import autograd_amd as ag
+
+    rs = onp.random.RandomState(62)
+    x = rs.randn(4, 5)
+    y = rs.uniform(0.3, 2.0, (4, 5)) * rs.choice([-1, 1], (4, 5))
+    X, Y = dnp.asarray(x), dnp.asarray(y)
+    assert onp.array_equal(dnp.imag(X).numpy(), onp.imag(x)) and onp.array_equal(dnp.angle(X).numpy(), onp.angle(x))
+    assert onp.array_equal(dnp.isreal(X).numpy(), onp.isreal(x)) and onp.array_equal(dnp.iscomplex(X).numpy(), onp.iscomplex(x))
+    assert onp.array_equal(dnp.floor_divide(X * 7, Y).numpy(), onp.floor_divide(x * 7, y))
+    assert onp.array_equal(dnp.floor_divide(X * 7, 0.7).numpy(), onp.floor_divide(x * 7, 0.7))
+    with onp.errstate(all="ignore"):
+        z = y.copy()
+        z[0, 0] = z[1, 1] = 0.0
+        assert onp.array_equal(dnp.floor_divide(X, dnp.asarray(z)).numpy(), onp.floor_divide(x, z), equal_nan=True)
+    assert dnp.array_equiv(X, X[:1] * 0 + X) and not dnp.array_equiv(X, Y)
+    assert dnp.array_equiv(dnp.asarray(onp.ones((3, 1))), dnp.asarray(onp.ones((1, 4)))) and not dnp.array_equiv(X, X[:, :3])
+    m = x > 0.3
+    assert all(onp.array_equal(a.numpy(), b) for a, b in zip(dnp.nonzero(X > 0.3), onp.nonzero(m)))
+    assert onp.array_equal(dnp.flatnonzero(X > 0.3).numpy(), onp.flatnonzero(m))
+    assert onp.array_equal(dnp.argwhere(X > 0.3).numpy(), onp.argwhere(m))
+    v = onp.sort(rs.randn(9))
+    assert onp.array_equal(dnp.searchsorted(dnp.asarray(v), X).numpy(), onp.searchsorted(v, x))
+    assert onp.array_equal(X[dnp.nonzero(X > 0.3)].numpy(), x[onp.nonzero(m)])
+    g = ag.grad(lambda a: dnp.sum(dnp.imag(a) + dnp.angle(a) * 3.0 + a))(X)
+    assert onp.array_equal(g.numpy(), onp.ones_like(x))
+    t = ag.make_jvp(lambda a: dnp.angle(a) + dnp.imag(a) + 2.0 * a)(X)(dnp.asarray(onp.ones_like(x)))[1]
+    assert onp.array_equal(t.numpy(), 2 * onp.ones_like(x))
+    g = ag.grad(lambda a: dnp.sum(a[dnp.nonzero(a > 0.3)] ** 2))(X)
+    assert onp.array_equal(g.numpy(), onp.where(m, 2 * x, 0.0))
+
+
 def test_truth_tests_and_closeness(dnp):
     rs = onp.random.RandomState(61)
     a = rs.randn(6, 9)
