@@ -904,15 +904,21 @@ extern "C" int agmi_gemm(int dtype, int64_t batch, int64_t M, int64_t N, int64_t
         return AGMI_ERR_ARG;
     }
     if (dtype == AGMI_F32) {
-        // 64x64 tiles, 8 waves (two K-groups), prefetch 4 slabs: best measured on the 1024-cubed
-        // contractions of the MLP workload (one tile per CU).  128x128 tiles only once they alone
-        // give every CU two tiles (less L2 traffic per flop for large problems).
+        // 64x64 tiles (the direct-to-LDS kernel): best measured on the 1024-cubed contractions of the MLP
+        // workload (one tile per CU).  128x128 tiles only once they alone give every CU two tiles (less L2
+        // traffic per flop for large problems) and fill their last round of CUs well enough.
         const int64_t big_tiles = ceil_div(M, 128) * ceil_div(N, 128) * batch;
-        if (big_tiles >= 512) return launch_gemm<MfmaF32x32, 128, 128, 16, 2, 1>(p, batch, s);
-        {
+        // Which tile: measured on full grids, the 128x128 kernel sustains about 117 TFLOP/s and the direct-to-LDS 64x64
+        // kernel about 107; each is then scaled by how well its tile count fills whole rounds of the 256 CUs
+        // (2944 x 2944: 529 big tiles are 2.07 rounds, i.e. three, 76 TFLOP/s; 2116 small ones are 8.3 rounds).
+        const int64_t small_tiles = ceil_div(M, 64) * ceil_div(N, 64) * batch;
+        const auto fill = [](int64_t tiles) { return static_cast<double>(tiles) / static_cast<double>(ceil_div(tiles, 256) * 256); };
+        const bool prefer_big = big_tiles >= 512 && 117.0 * fill(big_tiles) > 107.0 * fill(small_tiles);
+        if (!prefer_big) {
             const int rc = launch_direct(p, batch, s, workspace, workspace_bytes);
             if (rc != 1) return rc;  // launched (0) or failed; 1 = operands do not qualify
         }
+        if (big_tiles >= 512) return launch_gemm<MfmaF32x32, 128, 128, 16, 2, 1>(p, batch, s);
         return launch_gemm<MfmaF32x32, 64, 64, 32, 2, 2>(p, batch, s, workspace, workspace_bytes);
     }
     if (dtype == AGMI_F64) return launch_gemm<MfmaF64x16, 64, 64, 16, 2, 1>(p, batch, s, workspace, workspace_bytes);
