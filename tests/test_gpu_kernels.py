@@ -1238,6 +1238,42 @@ def test_lse_cotangent_fused_entry_point(dnp, dtype, rows, cols):
                     close(col_sums.cpu().numpy(), onp.sum(mem.astype(F64) * S, axis=0, keepdims=True).astype(dtype), RT[dtype]), label
 
 
+def test_lse_cotangent_tiles_grow_with_a_small_workspace(dnp):
+    """Partial column sums take one row per band of 16 rows; when the workspace cannot hold that many the bands get
+    taller (32, 48, 64 rows), and when even 64 do not fit the call reports the layout as unsupported."""
+    import torch
+
+    from autograd_amd import _lib
+
+    rs = onp.random.RandomState(5)
+    rows, cols = 200, 1028
+    dev = _lib.device()
+    code = _lib.DTYPE_CODE[onp.dtype(F32)]
+    mem = rs.randn(rows, cols).astype(F32)
+    by_col = rs.uniform(0.5, 1.5, (1, cols)).astype(F32)
+    g = rs.randn(rows, 1).astype(F32)
+    ans, S = _lse_cotangent_reference(mem, None, None, None, None, g.astype(F64))
+    put = lambda a: torch.from_numpy(onp.ascontiguousarray(a)).to(dev)
+    t_mem, t_col, t_ans, t_g = put(mem), put(by_col), put(ans.astype(F32)), put(g)
+    real = _lib._WORKSPACE_BYTES
+    try:
+        for limit in (real, 40 << 10, 26 << 10, 20 << 10):  # bands of 16, 32, 48 and 64 rows
+            _lib._WORKSPACE_BYTES = limit
+            row_sums = torch.full((rows, 1), float("nan"), device=dev)
+            scaled = torch.full((rows, cols), float("nan"), device=dev)
+            col_sums = torch.full((1, cols), float("nan"), device=dev)
+            assert _lib.lse_cotangent(code, t_mem, t_ans, t_g, row_sums=row_sums, col_factor=t_col.reshape(cols), scaled=scaled,
+                                      col_sums=col_sums), limit
+            close(scaled.cpu().numpy(), (by_col * S).astype(F32), RT[F32])
+            close(row_sums.cpu().numpy(), onp.sum(S, axis=1, keepdims=True).astype(F32), RT[F32])
+            close(col_sums.cpu().numpy(), onp.sum(mem.astype(F64) * S, axis=0, keepdims=True).astype(F32), RT[F32])
+        _lib._WORKSPACE_BYTES = 8 << 10
+        assert not _lib.lse_cotangent(code, t_mem, t_ans, t_g, row_sums=torch.zeros((rows, 1), device=dev),
+                                      col_sums=torch.zeros((1, cols), device=dev))
+    finally:
+        _lib._WORKSPACE_BYTES = real
+
+
 def test_lse_cotangent_layouts_outside_the_kernel_are_reported(dnp):
     import torch
 
