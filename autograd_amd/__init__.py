@@ -15,7 +15,7 @@ _host.install()  # an installed HIPS/autograd may host the value type instead of
 
 from . import differential_operators as _operators  # noqa: E402
 from .builtins import dict, isinstance, list, tuple, type  # noqa: A004,E402,F401
-from .extend import primitive  # noqa: E402,F401
+from .core import primitive_with_deprecation_warnings as primitive  # noqa: E402,F401
 from .graphs import capture  # noqa: E402,F401
 
 # the differential operators of autograd/__init__.py:1-22, under the same names

@@ -475,3 +475,50 @@ defvjp(func(VSpace.covector), None, lambda ans, vs, x: lambda g: vs.covector(g))
 for _bilinear in (func(VSpace.scalar_mul), func(VSpace.inner_prod)):
     defjvp(_bilinear, None, "same", "same")
 defjvp(func(VSpace.covector), None, "same")
+
+
+# ----------------------------------------------------------------------------------------------
+# The pre-1.2 way of attaching reverse rules, kept as warning shims (reference core.py:347-415):
+# a primitive obtained from THIS module, or from the package's top level (autograd/__init__.py:1), carries
+# ``defgrad`` / ``defvjp`` / ``defvjp_is_zero`` methods that translate to ``defvjp`` above.
+# ``extend.primitive`` is the plain one.
+# ----------------------------------------------------------------------------------------------
+_OLD_STYLE = ("The {} method is deprecated. See the update guide and tutorial:\n"
+              "https://github.com/HIPS/autograd/blob/master/docs/updateguide.md\n"
+              "https://github.com/HIPS/autograd/blob/master/docs/tutorial.md")
+_plain_primitive = primitive
+
+
+def _old_style_rules(wrapped):
+    """The three legacy registration methods of ``wrapped``; each call re-registers every rule given so far."""
+    import warnings
+
+    makers = {}  # argnum -> maker in today's form, or None for a zero cotangent
+
+    def register(method):
+        warnings.warn(_OLD_STYLE.format(method))
+        positions = sorted(makers)
+        defvjp(wrapped, *(makers[n] for n in positions), argnums=positions)
+
+    def defgrad(gradfun, argnum=0):  # already (ans, *args) -> (g -> cotangent)
+        makers[argnum] = gradfun
+        register("defgrad")
+
+    def defvjp_unstaged(rule, argnum=0):  # rule(g, ans, vs, gvs, *args): everything at once
+        makers[argnum] = lambda ans, *args, **kwargs: lambda g: rule(g, ans, vspace(args[argnum]), vspace(g), *args, **kwargs)
+        register("defvjp")
+
+    def defvjp_is_zero(argnums=(0,)):
+        makers.update((n, None) for n in argnums)
+        register("defvjp_is_zero")
+
+    return defgrad, defvjp_unstaged, defvjp_is_zero
+
+
+def primitive_with_deprecation_warnings(f_raw):
+    wrapped = _plain_primitive(f_raw)
+    wrapped.defgrad, wrapped.defvjp, wrapped.defvjp_is_zero = _old_style_rules(wrapped)
+    return wrapped
+
+
+primitive = primitive_with_deprecation_warnings  # (shadows the import on purpose, as reference core.py:415 does)

@@ -12,6 +12,7 @@ from .devarray import DevArray, from_numpy  # noqa: F401
 from .vspaces import DevArrayVSpace  # noqa: F401
 from .wrapper import *  # noqa: F401,F403
 from .wrapper import (  # noqa: F401
+    __version__,
     _array_from_scalar_or_array,
     _astype,
     _primitive_mean,

@@ -173,12 +173,17 @@ defjvp(anp.rad2deg, "same")  # numpy_jvps.py:78-81: the function itself applied 
 defjvp(anp.deg2rad, "same")
 defjvp(anp.clip, lambda g, ans, x, a_min, a_max: g * anp.logical_and(ans != a_min, ans != a_max))
 
+def _like_result(ans, tangent):
+    """A tangent of ``where`` in the result's shape, also when the other choice is what made the result larger."""
+    return tangent if anp.shape(tangent) == anp.shape(ans) else anp.broadcast_to(tangent, anp.shape(ans))
+
+
 defjvp(
     anp._where3,
     None,
     # numpy_jvps.py:150-151: float64 zeros, so a float32 tangent comes out float64
-    lambda g, ans, c, x, y: anp.where(c, g, _float64_zeros(anp.shape(g))),
-    lambda g, ans, c, x, y: anp.where(c, _float64_zeros(anp.shape(g)), g),
+    lambda g, ans, c, x, y: _like_result(ans, anp.where(c, g, _float64_zeros(anp.shape(g)))),
+    lambda g, ans, c, x, y: _like_result(ans, anp.where(c, _float64_zeros(anp.shape(g)), g)),
 )
 defjvp(anp.astype, lambda g, ans, A, dtype, *a, **k: anp.astype(g, dtype))
 defjvp(

@@ -318,12 +318,20 @@ def _float64_zeros(shape):
     return DevArray(_shared_zero(_F64)._t.expand(tuple(shape)), _F64) if all(shape) else D.zeros(shape, _F64)
 
 
+def _as_broadcast_from(operand, picked):
+    """``picked`` summed down to the shape of ``operand`` when the choice was broadcast (numpy_vjps.py:228-229 leaves the
+    cotangent in the shape of the result, which only fits an operand of that shape)."""
+    if anp.shape(picked)[BatchMode.active:] == anp.shape(operand):
+        return picked
+    return unbroadcast(picked, anp.metadata(operand))
+
+
 defvjp(
     anp._where3,
     None,
     # numpy_vjps.py:228-229: the zeros are float64 (anp.zeros(g.shape)), so a float32 cotangent comes out float64
-    lambda ans, c, x, y: lambda g: anp.where(c, g, _float64_zeros(anp.shape(g))),
-    lambda ans, c, x, y: lambda g: anp.where(c, _float64_zeros(anp.shape(g)), g),
+    lambda ans, c, x, y: lambda g: _as_broadcast_from(x, anp.where(c, g, _float64_zeros(anp.shape(g)))),
+    lambda ans, c, x, y: lambda g: _as_broadcast_from(y, anp.where(c, _float64_zeros(anp.shape(g)), g)),
 )
 defvjp(
     anp.astype,

@@ -21,8 +21,26 @@ from .devarray import DevArray
 # constants and dtypes
 pi, e, inf, nan, newaxis = onp.pi, onp.e, onp.inf, onp.nan, None
 euler_gamma = onp.euler_gamma
-float32, float64, int32, int64, bool_ = onp.float32, onp.float64, onp.int32, onp.int64, onp.bool_
+float32, float64, bool_ = onp.float32, onp.float64, onp.bool_
+dtype, __version__ = onp.dtype, onp.__version__
 ndarray = DevArray
+
+
+def _int_type(cls):
+    """NumPy's integer scalar type, which also casts a device array or a box around one (untraced: an integer
+    has no tangent).  The reference subclasses the integer types for the same reason, numpy_wrapper.py:18-22 and
+    42-43; as a dtype the subclass means its parent."""
+
+    def make(kind, value=0, *args):
+        from ..tracer import getval
+
+        value = getval(value)
+        return D.astype(value, cls) if isinstance(value, DevArray) else cls(value, *args)
+
+    return type(cls.__name__, (cls,), {"__new__": make, "__doc__": cls.__doc__})
+
+
+int8, int16, int32, int64 = onp.int8, onp.int16, _int_type(onp.int32), _int_type(onp.int64)  # (the device holds the last two)
 
 
 def _wrap(raw, name):
@@ -139,6 +157,8 @@ greater_equal = _compare(Cmp.GE, "greater_equal")
 @primitive
 def _where3(c, x, y):
     dt = D._float_dtype(D.result_dtype(x, y))
+    if isinstance(c, (list, tuple, onp.ndarray)):  # a host mask
+        c = D.asarray(onp.asarray(c))
     if isinstance(c, DevArray):
         c = D.astype(c, dt) if c.dtype != dt else c
     else:
@@ -146,16 +166,27 @@ def _where3(c, x, y):
     return D.map_op(Op.WHERE, dt, c, x, y)
 
 
-def where(condition, x, y):
-    """``numpy.where(c, x, y)``.  Keeps native Python types when no operand is an array or a
-    box, as the reference does (autograd/numpy/__init__.py:13-39): the ``power`` rule calls
-    ``where(y, y - 1, 1.0)`` with a Python exponent and needs a Python float back."""
+def where(condition, *args, **kwargs):
+    """``numpy.where(c, x, y)``, or ``numpy.nonzero(c)`` when called with the condition alone.  Keeps native Python
+    types when no operand is an array or a box, as the reference does (autograd/numpy/__init__.py:13-39): the
+    ``power`` rule calls ``where(y, y - 1, 1.0)`` with a Python exponent and needs a Python float back."""
     from ..tracer import isbox
 
+    if not args and not kwargs:
+        return nonzero(condition)
+    if len(args) + len(kwargs) != 2 or not set(kwargs) <= {"x", "y"}:
+        raise ValueError("either both or neither of x and y should be given")
+    x = args[0] if args else kwargs["x"]
+    y = args[1] if len(args) > 1 else kwargs["y"]
+
     def arrayish(v):
-        return isinstance(v, (DevArray, onp.ndarray, onp.generic)) or isbox(v)
+        if isinstance(v, (DevArray, onp.ndarray, onp.generic)) or isbox(v):
+            return True
+        return type(v) in (list, tuple) and builtins.any(arrayish(item) for item in v)
 
     if not (arrayish(condition) or arrayish(x) or arrayish(y)):
+        if type(condition) in (list, tuple) or type(x) in (list, tuple) or type(y) in (list, tuple):
+            return onp.where(condition, x, y).tolist()
         return x if condition else y
     return _where3(condition, x, y)
 
@@ -632,8 +663,12 @@ def array_from_args(array_args, array_kwargs, *args):
 
 def array(A, *args, **kwargs):
     """``numpy.array``: host data is uploaded; lists that contain boxes stay differentiable."""
-    from ..tracer import isbox
+    from ..tracer import getval, isbox
 
+    if isbox(A) and type(getval(A)) in (list, tuple):
+        # a traced sequence (the reference asks autograd.builtins.type, which sees through boxes,
+        # numpy_wrapper.py:83-88): its elements come out of the box one by one, traced
+        return array_from_args(args, kwargs, *map(array, A))
     if type(A) in (list, tuple):
         flat_has_dev = _contains_dev_or_box(A)
         if flat_has_dev:
@@ -675,6 +710,65 @@ def stack(arrays, axis=0):
     axis %= nd
     sl = (slice(None),) * axis + (None,)
     return concatenate([a[sl] for a in arrays], axis=axis)
+
+
+def column_stack(tup):
+    """1-d inputs become columns, the rest are joined along axis 1 (numpy_wrapper.py:73-80)."""
+    columns = []
+    for v in tup:
+        a = array(v)
+        columns.append(reshape(a, (-1, 1)) if ndim(a) < 2 else a)
+    return concatenate(columns, 1)
+
+
+def select(condlist, choicelist, default=0):
+    """``numpy.select``: the first condition that holds picks the choice (numpy_wrapper.py:58-60 assembles the result
+    element by element on the host; here it is a chain of ``where`` from the last condition to the first)."""
+    condlist, choicelist = list(condlist), list(choicelist)
+    if len(condlist) != len(choicelist):
+        raise ValueError("list of cases must be same length as list of conditions")
+    if not condlist:
+        raise ValueError("select with an empty condition list is not possible")
+    out = default
+    for cond, choice in zip(reversed(condlist), reversed(choicelist)):
+        out = where(array(cond), choice, out)
+    return out
+
+
+def append(arr, values, axis=None):
+    """``numpy.append`` through ``concatenate`` (numpy_wrapper.py:139-147): both flattened when no axis is given."""
+    arr = array(arr)
+    if axis is None:
+        arr = ravel(arr) if ndim(arr) != 1 else arr
+        values = ravel(array(values))
+        axis = 0
+    return concatenate((arr, values), axis=axis)
+
+
+class _Joiner:
+    """``r_[...]`` and ``c_[...]`` (numpy_wrapper.py:153-169) for arrays, scalars and ranges: ranges are expanded on
+    the host, every item is raised to ``min_ndim`` dimensions (new unit axes last) and the items are joined along
+    ``axis``.  The string directives of NumPy's index tricks are not taken."""
+
+    def __init__(self, name, axis, min_ndim):
+        self._name, self._axis, self._min_ndim = name, axis, min_ndim
+
+    def __getitem__(self, items):
+        items = items if type(items) is tuple else (items,)
+        pieces = []
+        for item in items:
+            if isinstance(item, str):
+                raise NotImplementedError(f"{self._name}[...] takes arrays, scalars and ranges, not string directives")
+            piece = D.from_numpy(onp.r_[item]) if type(item) is slice else array(item)
+            if ndim(piece) < self._min_ndim:
+                piece = reshape(piece, shape(piece) + (1,) * (self._min_ndim - ndim(piece)))
+            pieces.append(piece)
+        if not pieces:
+            return D.from_numpy(onp.r_[()])
+        return concatenate(pieces, axis=self._axis)
+
+
+r_, c_ = _Joiner("r_", 0, 1), _Joiner("c_", -1, 2)
 
 
 # ---- indexing -----------------------------------------------------------------------------------
@@ -1650,6 +1744,8 @@ def copy_if_input(x, inputs):
 def _meta_of(A):
     if isinstance(A, DevArray):
         return A.shape, A.ndim, A.dtype, False
+    if type(A) in (list, tuple):
+        A = onp.asarray(A)  # (result_type would read a nested list as a structured dtype)
     return onp.shape(A), onp.ndim(A), onp.result_type(A), onp.iscomplexobj(A)
 
 
@@ -1808,7 +1904,9 @@ def gradient(f, *varargs, axis=None, edge_order=1):
         outs.append(concatenate(pieces, axis=a))
     if len(axes) == 1 and (axis is None or isinstance(axis, numbers.Integral)):
         return outs[0]
-    return tuple(outs)
+    from ..builtins import tuple as traced_tuple  # (a traced container: the derivatives stay visible to the caller's trace)
+
+    return traced_tuple(outs)
 
 
 def arange(*args, **kwargs):

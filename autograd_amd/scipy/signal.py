@@ -113,6 +113,11 @@ def convolve(A, B, axes=None, dot_axes=None, mode="full", flip=_NO_FLIP):
         raise TypeError(f"convolve: {dtype} operands are not supported on the device")
     roles, shapes = _axis_roles(A.shape, B.shape, axes, dot_axes, mode)
     n_conv = len(roles["A"]["conv"])
+    if n_conv == 0:
+        # nothing slides: what is left is the contraction over dot_axes, free axes of A before those of B
+        from ..numpy.wrapper import _tensordot_raw
+
+        return _tensordot_raw(D.asarray(A, dtype), D.asarray(B, dtype), axes=(list(dot_axes[0]), list(dot_axes[1])))
     if not 1 <= n_conv <= 3:
         raise NotImplementedError(f"convolve over {n_conv} axes (1 to 3 are supported on the device)")
     if shapes["A"]["dot"] != shapes["B"]["dot"]:

@@ -95,3 +95,15 @@ def toposort(end_node, parents=_get_parents):
                 ready.append(parent)
             else:
                 pending_children[parent] = remaining - 1
+
+
+def quick_grad_check(fun, arg0, extra_args=(), kwargs=None, verbose=True, eps=1e-4, rtol=1e-4, atol=1e-6, rs=None):
+    """The retired name of a reverse-mode, first-order ``check_grads`` with respect to the first argument
+    (reference util.py:45-61); warns and delegates.  The tolerance arguments are accepted and ignored, as there."""
+    import warnings
+
+    warnings.warn("The quick_grad_check function is deprecated. See the update guide:\n"
+                  "https://github.com/HIPS/autograd/blob/master/docs/updateguide.md")
+    from .test_util import check_grads
+
+    check_grads(lambda first: fun(first, *extra_args, **(kwargs or {})), modes=["rev"], order=1)(arg0)
