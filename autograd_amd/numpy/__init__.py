@@ -24,3 +24,4 @@ from .wrapper import (  # noqa: F401
     sum,
 )
 from .vjps import untake  # noqa: F401
+from . import random  # noqa: E402,F401  (``np.random`` without a separate import, autograd/numpy/__init__.py:6)

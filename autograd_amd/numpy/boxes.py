@@ -108,3 +108,28 @@ DevArrayBox.register(PendingProduct)
 DevArrayBox.register(LseCotangent)
 DevArrayBox.register(FusedResult)
 DevArrayBox.register(float)
+
+
+def _box_host_value(value, trace, node):
+    """A host ``ndarray`` or NumPy scalar handed to a differential operator (``grad(f)(numpy_array)``, as callers such
+    as ``scipy.optimize.minimize`` do) is uploaded once where it enters the trace; everything downstream, the
+    gradient included, is a device array."""
+    from .devarray import from_numpy
+
+    import numpy as onp
+
+    return DevArrayBox(from_numpy(onp.asarray(value)), trace, node)
+
+
+def _register_host_values():
+    from .. import _host
+
+    if _host.HOST:
+        return  # the hosting package boxes host arrays itself, as host arrays
+    import numpy as onp
+
+    for host_type in (onp.ndarray, onp.float64, onp.float32):
+        Box.type_mappings[host_type] = _box_host_value
+
+
+_register_host_values()

@@ -36,8 +36,9 @@ class DevArray:
     def __init__(self, tensor, dtype=None):
         self._t = tensor
         self.dtype = dtype if dtype is not None else _lib.NUMPY_DTYPE[tensor.dtype]
-        # True on an accumulator that shares its memory with a cotangent it was initialised from
-        # (0 + g kept as g): in-place accumulation must then go to fresh memory instead
+        # True on an array whose memory another value reads: an accumulator initialised from a cotangent (0 + g kept
+        # as g), or the operand of arithmetic that is still pending.  In-place accumulation and item assignment
+        # then go to fresh memory instead
         self._borrowed = False
         self._shape_tuple = None  # filled by the first `shape` (asked many times per launch; arrays never change)
 
@@ -100,6 +101,11 @@ class DevArray:
     def __int__(self):
         return int(self.item())
 
+    def __index__(self):
+        if self.dtype.kind not in "iu" or self._t.numel() != 1:
+            raise TypeError("only integer scalar arrays can be converted to a scalar index")
+        return int(self.item())
+
     def __bool__(self):
         if self._t.numel() != 1:
             raise ValueError("The truth value of an array with more than one element is ambiguous.")
@@ -112,7 +118,9 @@ class DevArray:
     __hash__ = object.__hash__
 
     def __setitem__(self, idx, value):
-        raise TypeError("DevArray is immutable: item assignment is not supported")
+        from . import wrapper
+
+        wrapper.assign_items(self, idx, value)
 
     # ---- view helpers ---------------------------------------------------------------------
     def _h(self):
@@ -209,6 +217,8 @@ class LazyDevArray(DevArray):
         """The same view operation on the storage and on the array-valued steps (they have the
         storage's shape); when one of them cannot be viewed that way the value is written out."""
         asc, sh = self._ascale, self._shift
+        if sh is None and asc is None and self._scale == 1.0:
+            return DevArray(fn(self._raw), self.dtype)  # nothing pending (the value has been written out): a plain view
         try:
             return LazyDevArray(fn(self._raw), self.dtype, self._scale,
                                 fn(sh) if isinstance(sh, torch.Tensor) else sh,
@@ -600,6 +610,7 @@ def _fold(op, dtype, xs):
             t = -c
     else:
         return None
+    a._borrowed = True  # the result reads `a`'s memory when it is consumed: an item assignment into `a` must not reach it
     if s == 1.0 and t is None and asc is None:
         return DevArray(raw, dtype)
     return LazyDevArray(raw, dtype, s, t, asc)
@@ -618,15 +629,14 @@ def _fold_array(op, dtype, a, c, swapped):
     if type(c) is LazyDevArray or c.ndim > a.ndim:
         c = plain(c)
     vec = c._t.expand(a.shape)
+    if op == Op.MUL and asc is not None or op not in (Op.MUL, Op.ADD) and not (op == Op.SUB and swapped):
+        return None
+    a._borrowed = c._borrowed = True  # (both are read when the result is consumed; see `_fold`)
     if op == Op.MUL:
-        if asc is not None:
-            return None
         return LazyDevArray(raw, dtype, s, None, vec)
     if op == Op.ADD:
         return LazyDevArray(raw, dtype, s, vec, asc)
-    if op == Op.SUB and swapped:  # c - a = (-a) + c
-        return LazyDevArray(raw, dtype, -s, vec, asc)
-    return None
+    return LazyDevArray(raw, dtype, -s, vec, asc)  # c - a = (-a) + c
 
 
 _FOLDABLE = frozenset({Op.NEG, Op.MUL, Op.ADD, Op.SUB, Op.DIV})

@@ -163,3 +163,14 @@ DevArrayVSpace.register(D.PendingProduct)
 DevArrayVSpace.register(D.LseCotangent)
 DevArrayVSpace.register(D.FusedResult)
 DevArrayVSpace.register(float)
+
+
+def _register_host_values():
+    from .. import _host
+
+    if not _host.HOST:  # (under a hosting package host arrays keep that package's vector space)
+        for host_type in (onp.ndarray, onp.float64, onp.float32):
+            DevArrayVSpace.register(host_type)
+
+
+_register_host_values()

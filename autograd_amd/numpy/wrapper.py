@@ -14,6 +14,7 @@ import torch
 
 from .. import _lib
 from ..extend import notrace_primitive, primitive
+from ..tracer import trace_stack as _trace_stack
 from . import devarray as D
 from .._lib import Cmp, Op, Red
 from .devarray import DevArray
@@ -971,6 +972,8 @@ def take(A, idx):
     masks), driven by a device-resident table of flat positions that is built once per (shape, index)."""
     if _is_basic_index(idx):
         pidx, backwards = _positive_steps(_plain(idx), A.shape)
+        if type(A) is D.LazyDevArray and _trace_stack.top < 0 and not builtins.any(A._raw.stride()):
+            A._t  # outside any trace a lazy fill (zeros / ones) is written out before it is viewed: an item assignment through the view then reaches it
         picked = A._view(lambda t: t[pidx])
         return _reverse_axes(picked, backwards) if backwards else picked
     if A.ndim == 0:
@@ -983,6 +986,58 @@ def take(A, idx):
         return _gather(A, rows, A.shape[0], inner, (rows.size,) + A.shape[1:])
     plan = _index_plan(A.shape, idx)
     return _gather(A, plan.positions, A.size, 1, plan.shape)
+
+
+def assign_items(A, idx, value):
+    """``A[idx] = value`` on a plain device array: data preparation outside any trace, the way examples/rnn.py:86
+    fills its one-hot batches.  Basic indices with forward steps write through the strided view in one launch; a
+    boolean mask of the array's own shape with a scalar value is one in-place select.  Arrays that share their memory
+    by construction (broadcast views, borrowed accumulators) get a buffer of their own first.  Inside a traced
+    function arrays stay immutable, as in the reference: a box has no item assignment and a boxed value cannot be
+    stored into an array."""
+    from ..tracer import isbox
+    from .vspaces import is_broadcast_view
+
+    if isbox(value) or isbox(idx):
+        raise TypeError("a traced value cannot be assigned into an array: build the result with concatenate / where")
+    if type(A) is D.LazyDevArray:
+        A._t  # pending arithmetic (a lazy fill, say) is written out: from here on the array is its own buffer
+    elif type(A) is not DevArray:
+        raise TypeError("item assignment needs a plain device array; this one is a cotangent still being formed "
+                        "(np.settle gives a plain one)")
+    if A._borrowed or is_broadcast_view(A):
+        own = D.contiguous(D.copy(DevArray(A._t, A.dtype)))._t
+        A._t, A._borrowed = own, False
+        if type(A) is D.LazyDevArray:
+            A._raw = own
+    dtype = A.dtype
+    if _is_basic_index(idx):
+        pidx, backwards = _positive_steps(_plain(idx), A.shape)
+        if backwards:
+            raise NotImplementedError("item assignment through a slice that steps backwards")
+        target = DevArray(A._t[pidx], dtype)
+        source = D.asarray(value, dtype)
+        if type(source) is not DevArray:
+            source = D.plain(source)
+        if onp.broadcast_shapes(source.shape, target.shape) != target.shape:
+            raise ValueError(f"could not broadcast input array from shape {source.shape} into shape {target.shape}")
+        if target.size == 0:
+            return
+        if dtype in D._FLOATS:
+            D.map_op(Op.COPY, dtype, source, out=target)
+        else:
+            code = _lib.DTYPE_CODE[dtype]
+            _lib.cast(code, code, target.shape, target._t, source._t.expand(target.shape))
+        return
+    mask = idx if isinstance(idx, DevArray) else (onp.asarray(idx) if isinstance(idx, (list, onp.ndarray)) else None)
+    scalar = isinstance(value, (numbers.Number, onp.generic)) or (isinstance(value, (DevArray, onp.ndarray)) and value.ndim == 0)
+    if mask is not None and mask.dtype == onp.bool_ and tuple(mask.shape) == A.shape and scalar and dtype in D._FLOATS:
+        mask = D.astype(D.asarray(mask), dtype)
+        whole = DevArray(A._t, dtype)
+        D.map_op(Op.WHERE, dtype, mask, D.asarray(value, dtype) if not isinstance(value, numbers.Number) else float(value), whole, out=whole)
+        return
+    raise NotImplementedError("item assignment takes basic indices (integers, forward slices, newaxis, ellipsis) or a boolean "
+                              "mask of the array's shape with a scalar value")
 
 
 def _leading_rows(idx, shape):
@@ -2042,3 +2097,36 @@ def std(a, *args, **kwargs):
     if type(a) in (list, tuple):
         a = array(a)
     return _primitive_std(a, *args, **kwargs)
+
+
+# ---- names that never touch array data ---------------------------------------------------------------
+def meshgrid(*xi, copy=True, sparse=False, indexing="xy"):
+    """Coordinate matrices as broadcast views of the 1-d inputs (``numpy.meshgrid``; the reference wraps it without a
+    rule, here it differentiates through ``reshape`` and ``broadcast_to``).  ``copy`` is accepted for NumPy's
+    signature: device arrays are never written in place, so views serve either way."""
+    if indexing not in ("xy", "ij"):
+        raise ValueError("Valid values for `indexing` are 'xy' and 'ij'.")
+    nd = len(xi)
+    grids = []
+    for position, x in enumerate(xi):
+        extents = [1] * nd
+        extents[position] = -1
+        grids.append(reshape(ravel(array(x)), tuple(extents)))
+    if indexing == "xy" and nd > 1:
+        grids[0], grids[1] = reshape(grids[0], (1, -1) + (1,) * (nd - 2)), reshape(grids[1], (-1, 1) + (1,) * (nd - 2))
+    if not sparse:
+        full = onp.broadcast_shapes(*(shape(g) for g in grids)) if grids else ()
+        grids = [broadcast_to(g, full) for g in grids]
+    return tuple(grids)
+
+
+def identity(n, dtype=float):
+    return eye(n, dtype=dtype)
+
+
+# floating-point error state, printing, dtype arithmetic and index helpers are NumPy's own: they take no array data
+for _name in ("seterr geterr errstate set_printoptions get_printoptions printoptions finfo iinfo issubdtype promote_types "
+              "can_cast broadcast_shapes s_ index_exp iterable unravel_index ravel_multi_index generic number inexact "
+              "floating integer signedinteger unsignedinteger float16 double single uint8 uint16 uint32 uint64 intp int_").split():
+    globals()[_name] = getattr(onp, _name)
+del _name

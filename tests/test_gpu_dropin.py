@@ -289,3 +289,103 @@ def test_convolve_with_nothing_sliding_is_a_contraction(np):
         onp.testing.assert_allclose(_host(got), onp.tensordot(A, B, axes=([0], [0])), rtol=1e-12)
     check_grads(lambda a, b: convolve(a, b, axes=([], []), dot_axes=([0], [0])), argnum=(0, 1), modes=["rev"])(
         np.array(A), np.array(B))
+
+
+def test_item_assignment_outside_a_trace(ag, np):
+    """examples/rnn.py:86 fills its one-hot batches with ``seqs[:, ix, :] = ...``: plain device arrays take basic
+    indices and whole-array masks; arithmetic that was pending on the old contents keeps the old contents; a view
+    taken before the assignment sees it; traced values stay out."""
+    h = onp.arange(24.0).reshape(2, 3, 4)
+    d = np.array(h)
+    cases = [((slice(None), 1, slice(None)), onp.ones((2, 4))), (0, 7.0), ((1, slice(0, 3, 2)), onp.arange(4.0)),
+             ((Ellipsis, 2), -1.0), ((slice(None), None, 1), 5.0), ((1, 2, 3), 9.5), ((slice(0, 0),), 3.0)]
+    for idx, value in cases:
+        h[idx] = value
+        d[idx] = np.array(value) if isinstance(value, onp.ndarray) else value
+        onp.testing.assert_array_equal(_host(d), h)
+    mask = h > 10
+    h[mask] = 0.0
+    d[np.array(mask)] = 0.0
+    onp.testing.assert_array_equal(_host(d), h)
+
+    filled = np.zeros((3, 4))  # (a lazy fill until first written)
+    for row in range(3):
+        filled[row, row:] = float(row + 1)
+    onp.testing.assert_array_equal(_host(filled), onp.triu(onp.ones((3, 4))) * onp.arange(1.0, 4.0)[:, None])
+    counts = np.zeros(3, dtype=np.int64)
+    counts[1:] = np.array([4, 5])
+    onp.testing.assert_array_equal(_host(counts), [0, 4, 5])
+
+    x = np.ones(3)
+    doubled, negated = x * 2.0 + 1.0, -x
+    x[0] = 5.0
+    onp.testing.assert_array_equal(_host(doubled), [3.0, 3.0, 3.0])
+    onp.testing.assert_array_equal(_host(negated), [-1.0, -1.0, -1.0])
+    onp.testing.assert_array_equal(_host(x), [5.0, 1.0, 1.0])
+
+    z = np.zeros((2, 2))
+    first_row = z[0]
+    first_row[:] = 1.0
+    z.T[0, 1] = 4.0
+    onp.testing.assert_array_equal(_host(z), [[1.0, 1.0], [4.0, 0.0]])
+
+    with pytest.raises(NotImplementedError):
+        d[::-1] = 1.0
+    with pytest.raises(NotImplementedError):
+        d[[0, 1]] = 1.0
+    with pytest.raises(ValueError):
+        d[0] = onp.ones(5)
+    with pytest.raises(TypeError):
+        ag.grad(lambda v: (d.__setitem__(0, v), np.sum(d))[1])(np.ones(4))
+    with pytest.raises(TypeError):
+        ag.grad(lambda v: (v.__setitem__(0, 1.0), np.sum(v))[1])(np.ones(4))
+
+
+def test_integer_scalars_index_python_sequences(np):
+    """examples/rnn.py:74: ``chr(np.argmax(c))``."""
+    best = np.argmax(np.array([0.0, 70.0, 3.0]))
+    assert chr(best) == "\x01" and [10, 20, 30][best] == 20 and "abc"[best] == "b"
+    with pytest.raises(TypeError):
+        [10, 20][np.array(1.0)]
+
+
+def test_meshgrid(ag, np):
+    a, b, c = onp.arange(3.0), onp.arange(4.0) + 10, onp.arange(2.0) + 100
+    for kw in ({}, {"indexing": "ij"}, {"sparse": True}, {"indexing": "ij", "sparse": True}):
+        for args in ((a,), (a, b), (a, b, c)):
+            got = np.meshgrid(*[np.array(x) for x in args], **kw)
+            want = onp.meshgrid(*args, **kw)
+            assert len(got) == len(want)
+            for g, w in zip(got, want):
+                onp.testing.assert_array_equal(_host(g), w)
+    through = ag.grad(lambda x: np.sum(np.meshgrid(x, np.array(b))[0] ** 2))(np.array(a))
+    onp.testing.assert_array_equal(_host(through), 2 * a * 4)
+
+
+def test_host_arrays_enter_at_the_differential_operator(ag, np):
+    """examples/rosenbrock.py: ``scipy.optimize.minimize(value_and_grad(f), x0, jac=True)`` hands host arrays in and
+    reads the value and the gradient back through ``float()`` / ``numpy.asarray``."""
+    from scipy.optimize import minimize
+
+    def rosenbrock(x):
+        return 100 * (x[1] - x[0] ** 2) ** 2 + (1 - x[0]) ** 2
+
+    x0 = onp.array([0.5, -0.3])
+    g = ag.grad(rosenbrock)(x0)
+    onp.testing.assert_allclose(_host(g), [-400 * x0[0] * (x0[1] - x0[0] ** 2) - 2 * (1 - x0[0]), 200 * (x0[1] - x0[0] ** 2)],
+                                rtol=1e-12)
+    found = minimize(ag.value_and_grad(rosenbrock), onp.array([0.0, 0.0]), jac=True, method="CG")
+    onp.testing.assert_allclose(found.x, [1.0, 1.0], atol=1e-4)
+    assert float(_host(ag.grad(lambda t: np.sin(t) * t)(onp.float64(0.5)))) == onp.sin(0.5) + 0.5 * onp.cos(0.5)
+    assert _host(ag.grad(lambda t: np.sum(t * t))(onp.ones(3, dtype=onp.float32))).dtype == onp.float32
+
+
+def test_names_that_take_no_array_data(np):
+    assert np.random.RandomState(0).randn(2).shape == (2,)
+    with np.errstate(divide="ignore"):
+        old = np.seterr(over="ignore")
+    np.seterr(**old)
+    assert np.finfo(np.float32).eps == onp.finfo(onp.float32).eps and np.uint8 is onp.uint8
+    assert np.issubdtype(np.float64, np.floating) and np.broadcast_shapes((3, 1), (4,)) == (3, 4)
+    onp.testing.assert_array_equal(_host(np.identity(3)), onp.identity(3))
+    onp.testing.assert_array_equal(_host(np.arange(10.0)[np.s_[2:5]]), [2.0, 3.0, 4.0])

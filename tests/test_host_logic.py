@@ -122,8 +122,10 @@ def test_views_are_metadata_only():
     assert W.atleast_2d(meta((3,))).shape == (1, 3) and W.atleast_1d(meta(())).shape == (1,)
     assert x[1:, ::2].shape == (3, 3) and x[None, 2].shape == (1, 6)
     assert W.shape(x) == (4, 6) and W.ndim(x) == 2 and W.size(x) == 24 and W.result_type(x) == onp.float32
-    with pytest.raises(TypeError):
-        x[0] = 1.0
+    with pytest.raises(NotImplementedError):
+        x[::-1] = 1.0  # (item assignment takes forward-stepping basic indices; rejected before anything is launched)
+    with pytest.raises(ValueError):
+        x[0] = meta((5,))  # a shape that does not broadcast into the row
 
 
 def test_vspace_metadata_and_laziness():
