@@ -129,7 +129,9 @@ def _register_host_values():
     import numpy as onp
 
     for host_type in (onp.ndarray, onp.float64, onp.float32):
-        Box.type_mappings[host_type] = _box_host_value
+        # (only where nothing else has claimed host arrays as a value type of its own: a CPU array library
+        # registered on this tracer, before or after this import, keeps them)
+        Box.type_mappings.setdefault(host_type, _box_host_value)
 
 
 _register_host_values()

@@ -170,7 +170,7 @@ def _register_host_values():
 
     if not _host.HOST:  # (under a hosting package host arrays keep that package's vector space)
         for host_type in (onp.ndarray, onp.float64, onp.float32):
-            DevArrayVSpace.register(host_type)
+            VSpace.mappings.setdefault(host_type, DevArrayVSpace)  # (unless another array library on this tracer owns them)
 
 
 _register_host_values()

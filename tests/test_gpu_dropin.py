@@ -362,22 +362,55 @@ def test_meshgrid(ag, np):
     onp.testing.assert_array_equal(_host(through), 2 * a * 4)
 
 
-def test_host_arrays_enter_at_the_differential_operator(ag, np):
+HOST_ARRAY_PROGRAM = r"""
+import numpy as onp
+import autograd_amd as ag, autograd_amd.numpy as np
+from scipy.optimize import minimize
+
+def rosenbrock(x):
+    return 100 * (x[1] - x[0] ** 2) ** 2 + (1 - x[0]) ** 2
+
+x0 = onp.array([0.5, -0.3])
+g = ag.grad(rosenbrock)(x0)
+assert isinstance(g, np.DevArray)
+want = [-400 * x0[0] * (x0[1] - x0[0] ** 2) - 2 * (1 - x0[0]), 200 * (x0[1] - x0[0] ** 2)]
+onp.testing.assert_allclose(g.numpy(), want, rtol=1e-12)
+found = minimize(ag.value_and_grad(rosenbrock), onp.array([0.0, 0.0]), jac=True, method="CG")
+onp.testing.assert_allclose(found.x, [1.0, 1.0], atol=1e-4)
+d = ag.grad(lambda t: np.sin(t) * t)(onp.float64(0.5))
+assert abs(float(d) - (onp.sin(0.5) + 0.5 * onp.cos(0.5))) < 1e-15
+assert ag.grad(lambda t: np.sum(t * t))(onp.ones(3, dtype=onp.float32)).dtype == onp.float32
+J = ag.jacobian(lambda t: np.tanh(t) * 2.0)(onp.array([0.1, 0.2]))
+onp.testing.assert_allclose(J.numpy(), onp.diag(2.0 / onp.cosh([0.1, 0.2]) ** 2), rtol=1e-12)
+print("host arrays ok")
+"""
+
+
+def test_host_arrays_enter_at_the_differential_operator():
     """examples/rosenbrock.py: ``scipy.optimize.minimize(value_and_grad(f), x0, jac=True)`` hands host arrays in and
-    reads the value and the gradient back through ``float()`` / ``numpy.asarray``."""
-    from scipy.optimize import minimize
+    reads the value and the gradient back through ``float()`` / ``numpy.asarray``.  Host arrays are the device
+    namespace's only while no other array library on the tracer claims them (the CPU oracle of these tests does), so
+    the check runs in a process of its own."""
+    import os
+    import subprocess
+    import sys
 
-    def rosenbrock(x):
-        return 100 * (x[1] - x[0] ** 2) ** 2 + (1 - x[0]) ** 2
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, PYTHONPATH=root + os.pathsep + os.environ.get("PYTHONPATH", ""))
+    env.pop("AUTOGRAD_AMD_HOST", None)
+    done = subprocess.run([sys.executable, "-c", HOST_ARRAY_PROGRAM], env=env, capture_output=True, text=True, timeout=170)
+    assert done.returncode == 0 and "host arrays ok" in done.stdout, done.stdout + done.stderr
 
-    x0 = onp.array([0.5, -0.3])
-    g = ag.grad(rosenbrock)(x0)
-    onp.testing.assert_allclose(_host(g), [-400 * x0[0] * (x0[1] - x0[0] ** 2) - 2 * (1 - x0[0]), 200 * (x0[1] - x0[0] ** 2)],
-                                rtol=1e-12)
-    found = minimize(ag.value_and_grad(rosenbrock), onp.array([0.0, 0.0]), jac=True, method="CG")
-    onp.testing.assert_allclose(found.x, [1.0, 1.0], atol=1e-4)
-    assert float(_host(ag.grad(lambda t: np.sin(t) * t)(onp.float64(0.5)))) == onp.sin(0.5) + 0.5 * onp.cos(0.5)
-    assert _host(ag.grad(lambda t: np.sum(t * t))(onp.ones(3, dtype=onp.float32))).dtype == onp.float32
+
+def test_host_arrays_stay_with_an_array_library_that_claims_them(ag, np):
+    """The CPU oracle registers ``numpy.ndarray`` as its own value type: whichever is imported first, its programs
+    keep running on the host (a parity test that compared the device with itself would prove nothing)."""
+    import oracle.anp as anp
+    from autograd_amd.extend import Box, vspace
+
+    assert Box.type_mappings[onp.ndarray].__name__ == "ArrayBox"
+    got = ag.grad(lambda t: anp.sum(anp.sin(t)))(onp.array([0.1, 0.2]))
+    assert type(got) is onp.ndarray and type(vspace(onp.ones(2))).__name__ == "ArrayVSpace"
 
 
 def test_names_that_take_no_array_data(np):
