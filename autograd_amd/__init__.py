@@ -13,6 +13,10 @@ from . import _host
 
 _host.install()  # an installed HIPS/autograd may host the value type instead of this package's own tracer
 
+from . import _compiled  # noqa: E402
+
+_compiled.install()  # the host-side modules come from their compiled copies when those are built and current
+
 from . import differential_operators as _operators  # noqa: E402
 from .builtins import dict, isinstance, list, tuple, type  # noqa: A004,E402,F401
 from .core import primitive_with_deprecation_warnings as primitive  # noqa: E402,F401

@@ -12,11 +12,12 @@ call raises.
 
 import ctypes
 import os
+import sys
 
 import numpy as onp
 import torch
 
-_HERE = os.path.dirname(os.path.abspath(__file__))
+_HERE = os.path.dirname(os.path.abspath(sys.modules[__name__.rsplit(".", 1)[0]].__file__))  # the package's folder, wherever this module was loaded from
 LIB_PATH = os.environ.get("AGMI_LIBRARY", os.path.join(_HERE, "libagmi.so"))
 
 MAX_DIMS = 8

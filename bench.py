@@ -309,6 +309,10 @@ def main():
 
     be = configs.device_backend()
     fun, fun_args, config, dtype = make_workload(args.workload, be)
+    from autograd_amd import _compiled
+
+    # whether the tracer / rule tables / launch marshalling ran as compiled extension modules or interpreted
+    config = dict(config, host_modules=_compiled.status()["mode"])
     if args.graph:
         return main_graph(args, be, fun, fun_args, config, dtype)
 
