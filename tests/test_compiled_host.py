@@ -39,6 +39,7 @@ def test_compiled_modules_are_served_while_they_match_their_sources(monkeypatch)
     with open(MANIFEST) as f:
         manifest = json.load(f)
     assert set(manifest["modules"]) == {"autograd_amd." + name for name in build_host.MODULES}
+    monkeypatch.delenv("AUTOGRAD_AMD_PURE_PYTHON", raising=False)
     seen = _probe(AUTOGRAD_AMD_PURE_PYTHON="")
     table, reason = _compiled._usable()
     if table is None:  # a source was edited after the build: everything must come from the sources
@@ -53,3 +54,42 @@ def test_compiled_modules_are_served_while_they_match_their_sources(monkeypatch)
     assert table is None and "util.py changed" in reason
     monkeypatch.setenv("AUTOGRAD_AMD_PURE_PYTHON", "1")
     assert _compiled._usable() == (None, "AUTOGRAD_AMD_PURE_PYTHON is set")
+
+
+DIGEST = r"""
+import hashlib, json
+import numpy as onp
+import autograd_amd as ag, autograd_amd.numpy as np
+from autograd_amd import _compiled, configs
+from autograd_amd.scipy.special import logsumexp
+
+be = configs.device_backend()
+digest = hashlib.sha256()
+out = configs.run_config("bcast", be, configs.bcast_inputs(rows=96, cols=200))
+for key in sorted(out):
+    digest.update(onp.ascontiguousarray(out[key]).tobytes())
+inp = configs.rnn_inputs(seq_len=5, batch=3, input_size=4, state_size=6, output_size=4)
+grads = configs.rnn_program(be)["grad"](configs.tree_map(be.put, inp["params"]), be.put(inp["inputs"]), be.put(inp["targets"]))
+for key in sorted(grads):
+    digest.update(grads[key].numpy().tobytes())
+x = np.array(onp.linspace(-1.0, 1.0, 7))
+H = ag.hessian(lambda v: np.sum(np.tanh(v) * v[::-1]) + logsumexp(v * 2.0))(x)
+J = ag.make_jvp(lambda v: np.sin(v) @ v)(x)(np.ones(7))[1]
+digest.update(H.numpy().tobytes() + J.numpy().tobytes())
+print(json.dumps({"mode": _compiled.status()["mode"], "digest": digest.hexdigest()}))
+"""
+
+
+@pytest.mark.gpu
+@pytest.mark.skipif(not os.path.exists(MANIFEST), reason="host modules not compiled (python -m autograd_amd.build_host)")
+def test_compiled_and_interpreted_host_modules_give_the_same_bits():
+    """The same sources, compiled or interpreted, launch the same kernels on the same operands: gradients of the
+    broadcast + logsumexp workload and of a small recurrent net, a Hessian and a forward-mode product, bit for bit."""
+    seen = {}
+    for pure in ("", "1"):
+        env = dict(os.environ, PYTHONPATH=ROOT, AUTOGRAD_AMD_PURE_PYTHON=pure)
+        done = subprocess.run([sys.executable, "-W", "ignore", "-c", DIGEST], env=env, capture_output=True, text=True, timeout=170)
+        assert done.returncode == 0, done.stderr
+        result = json.loads(done.stdout.strip().splitlines()[-1])
+        seen[result["mode"]] = result["digest"]
+    assert set(seen) == {"compiled", "python"} and seen["compiled"] == seen["python"], seen
