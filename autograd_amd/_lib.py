@@ -261,14 +261,16 @@ class KernelTimer:
     """Times launches with HIP events recorded on the stream the kernels run on.
 
     ``with KernelTimer() as kt: ...`` brackets every launch whose ``(entry point, op)`` key is in
-    ``only`` (all launches when ``only`` is None).  ``summary()`` (after a device synchronise)
+    ``only`` (all launches when ``only`` is None; every ``every``-th of them when that is given: an event pair costs
+    the host a few microseconds and delays the launch behind it).  ``summary()`` (after a device synchronise)
     gives, per kernel name, the launch count, the average duration and the average algorithmic
     traffic: every distinct input element read once plus every output element written once
     (2*M*N*K flops for a contraction).
     """
 
-    def __init__(self, only=None, events=0):
+    def __init__(self, only=None, events=0, every=1):
         self.only = only
+        self.every, self._seen = every, 0  # `every` = n: only every n-th matching launch carries events
         self.records = []
         self._traffic = {}  # (key, shape of the first result) -> algorithmic bytes, computed once
         # events made ahead of time keep the cost inside a timed region to the two records per launch
@@ -295,6 +297,10 @@ class KernelTimer:
     def begin(self, key):
         if self.only is not None and key not in self.only:
             return None
+        if self.every > 1:
+            self._seen += 1
+            if self._seen % self.every:
+                return None
         return self._event()
 
     def end(self, ev0, key, nbytes, flops=0.0):
