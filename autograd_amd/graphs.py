@@ -73,6 +73,7 @@ class CapturedFunction:
                 leaf = D.from_numpy(leaf)
             self._static_in.append(_static_copy(leaf) if isinstance(leaf, DevArray) else leaf)
         self._last = [None] * len(leaves)  # the array object last copied into each input buffer
+        self._writes_seen = D.ITEM_WRITES  # value of the item-assignment counter at the last call
         args = _unflatten(self._in_struct, iter(self._static_in))
         for _ in range(max(int(warmup), 1)):
             # eager runs first: one-time allocations (shared zeros, the reduction workspace)
@@ -119,15 +120,17 @@ class CapturedFunction:
 
         Returns the recorded output arrays: the next call overwrites them, so copy what must
         outlive it.  An argument array that is the same object as in the previous call is not
-        copied again (device arrays are immutable)."""
+        copied again, unless some array has been written by item assignment since (``D.ITEM_WRITES``)."""
         leaves = []
         struct = _flatten(tuple(args), leaves)
         if struct != self._in_struct:
             raise TypeError("captured function called with a different argument structure than it was captured on")
         last = self._last
+        unwritten = self._writes_seen == D.ITEM_WRITES  # no item assignment anywhere since the last call
+        self._writes_seen = D.ITEM_WRITES
         for k, (leaf, static) in enumerate(zip(leaves, self._static_in)):
             if isinstance(static, DevArray):
-                if leaf is last[k] and isinstance(leaf, DevArray):
+                if leaf is last[k] and unwritten and isinstance(leaf, DevArray):
                     continue
                 src = D.from_numpy(leaf) if isinstance(leaf, onp.ndarray) else leaf
                 if not isinstance(src, DevArray) or src.shape != static.shape or src.dtype != static.dtype:

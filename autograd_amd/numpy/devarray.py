@@ -26,6 +26,9 @@ _BOOL = onp.dtype("bool")
 _I64 = onp.dtype("int64")
 
 
+ITEM_WRITES = 0  # counts item assignments (``x[idx] = v``): what caches an array by identity checks before trusting its contents
+
+
 class DevArray:
     """n-d array in GPU memory; arithmetic is hand-written HIP kernels."""
 

@@ -1000,6 +1000,7 @@ def assign_items(A, idx, value):
 
     if isbox(value) or isbox(idx):
         raise TypeError("a traced value cannot be assigned into an array: build the result with concatenate / where")
+    D.ITEM_WRITES += 1
     if type(A) is D.LazyDevArray:
         A._t  # pending arithmetic (a lazy fill, say) is written out: from here on the array is its own buffer
     elif type(A) is not DevArray:

@@ -184,3 +184,19 @@ def test_gather_and_ordered_scatter_replay_from_a_graph():
         onp.add.at(dM, onp.array([4, 0, 4, 2, 4]), w.numpy())
         onp.add.at(dM, (onp.array([1, 1, 3]), slice(1, None)), 3 * M0[[1, 1, 3], 1:] ** 2)
         assert onp.allclose(got[1], dM, rtol=1e-12)
+
+
+def test_an_argument_written_by_item_assignment_is_copied_again():
+    """A replay skips the copy of an argument that is the same object as last time; an item assignment in between
+    (``x[0] = ...`` outside any trace) must not be missed."""
+    import autograd_amd as ag
+    import autograd_amd.numpy as np
+
+    x = np.array(onp.arange(6.0))
+    g = ag.capture(ag.grad(lambda v: np.sum(np.sin(v) * v)), x)
+    want = lambda h: onp.cos(h) * h + onp.sin(h)  # noqa: E731
+    onp.testing.assert_allclose(g(x).numpy(), want(onp.arange(6.0)), rtol=1e-12)
+    onp.testing.assert_allclose(g(x).numpy(), want(onp.arange(6.0)), rtol=1e-12)
+    x[0] = 2.5
+    x[4:] = onp.array([-1.0, 0.5])
+    onp.testing.assert_allclose(g(x).numpy(), want(onp.array([2.5, 1.0, 2.0, 3.0, -1.0, 0.5])), rtol=1e-12)
