@@ -14,6 +14,7 @@ import torch
 
 from .. import _lib
 from ..extend import notrace_primitive, primitive
+from ..tracer import getval as _getval
 from ..tracer import trace_stack as _trace_stack
 from . import devarray as D
 from .._lib import Cmp, Op, Red
@@ -630,15 +631,21 @@ def concatenate(arr_list, axis=0):
     return concatenate_args(axis, *arr_list)
 
 
+def _with_rank(m, n, lift):
+    """``atleast_nd(m)``, skipping the call (and, for a traced array, the tape node of an identity) when ``m`` is an
+    array that has ``n`` dimensions already."""
+    return m if isinstance(_getval(m), DevArray) and ndim(m) >= n else lift(m)
+
+
 def vstack(tup):
-    return concatenate([atleast_2d(m) for m in tup], axis=0)
+    return concatenate([_with_rank(m, 2, atleast_2d) for m in tup], axis=0)
 
 
 row_stack = vstack
 
 
 def hstack(tup):
-    arrs = [atleast_1d(m) for m in tup]
+    arrs = [_with_rank(m, 1, atleast_1d) for m in tup]
     if arrs[0].ndim == 1:
         return concatenate(arrs, 0)
     return concatenate(arrs, 1)
