@@ -744,13 +744,10 @@ def select(condlist, choicelist, default=0):
 
 
 def append(arr, values, axis=None):
-    """``numpy.append`` through ``concatenate`` (numpy_wrapper.py:139-147): both flattened when no axis is given."""
-    arr = array(arr)
+    """``numpy.append`` through ``concatenate`` (numpy_wrapper.py:139-147): both operands flattened when no axis is given."""
     if axis is None:
-        arr = ravel(arr) if ndim(arr) != 1 else arr
-        values = ravel(array(values))
-        axis = 0
-    return concatenate((arr, values), axis=axis)
+        return concatenate((ravel(array(arr)), ravel(array(values))), axis=0)
+    return concatenate((array(arr), values), axis=axis)
 
 
 class _Joiner:
