@@ -739,6 +739,10 @@ def select(condlist, choicelist, default=0):
         raise ValueError("select with an empty condition list is not possible")
     out = default
     for cond, choice in zip(reversed(condlist), reversed(choicelist)):
+        if _getval(choice) is not choice:
+            # (a cast to its own dtype: the reference hands every traced choice its cotangent in the choice's dtype,
+            # where the rule of `where` alone would leave a float32 one in float64)
+            choice = astype(choice, result_type(choice))
         out = where(array(cond), choice, out)
     return out
 
@@ -770,6 +774,17 @@ class _Joiner:
             pieces.append(piece)
         if not pieces:
             return D.from_numpy(onp.r_[()])
+        traced = [_getval(item) is not item for item in items]
+        if builtins.any(traced):
+            # the reference lets NumPy build an object array around the boxes and unpacks it element by element
+            # (numpy_wrapper.py:91-97, 153-169).  Untraced items arrive there as Python numbers, which makes the
+            # result float64 even when every array was float32; and every traced item gets its cotangent back in
+            # its own dtype.  Casting the traced items first gives both.
+            final = onp.result_type(*[result_type(piece) for piece in pieces])
+            if not builtins.all(traced) and final == onp.float32:
+                final = onp.dtype(onp.float64)
+            pieces = [astype(piece, final) if is_traced and result_type(piece) != final else piece
+                      for piece, is_traced in zip(pieces, traced)]
         return concatenate(pieces, axis=self._axis)
 
 

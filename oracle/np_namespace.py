@@ -113,6 +113,49 @@ def stack(arrays, axis=0):
     return concatenate([a[sl] for a in arrays], axis=axis)
 
 
+def select(condlist, choicelist, default=0):  # numpy_wrapper.py:58-60: assembled element by element
+    raw_array = _np.select(list(condlist), list(choicelist), default=default)
+    return array(list(raw_array.ravel())).reshape(raw_array.shape)
+
+
+def column_stack(tup):  # numpy_wrapper.py:73-80
+    arrays = []
+    for v in tup:
+        arr = array(v)
+        if arr.ndim < 2:
+            arr = array(arr, ndmin=2).T
+        arrays.append(arr)
+    return concatenate(arrays, 1)
+
+
+def _wrap_if_boxes_inside(raw_array):  # numpy_wrapper.py:91-97 (without the warning)
+    if raw_array.dtype is _np.dtype("O"):
+        return array_from_args((), {}, *raw_array.ravel()).reshape(raw_array.shape)
+    return raw_array
+
+
+def append(arr, values, axis=None):  # numpy_wrapper.py:139-147
+    arr = array(arr)
+    if axis is None:
+        if ndim(arr) != 1:  # noqa: F821
+            arr = ravel(arr)  # noqa: F821
+        values = ravel(array(values))  # noqa: F821
+        axis = ndim(arr) - 1  # noqa: F821
+    return concatenate((arr, values), axis=axis)
+
+
+class _RClass:  # numpy_wrapper.py:153-159: NumPy builds an object array around the boxes, which is then unpacked
+    def __getitem__(self, args):
+        return _wrap_if_boxes_inside(_np.r_[args])
+
+
+class _CClass:  # numpy_wrapper.py:162-169
+    def __getitem__(self, args):
+        return _wrap_if_boxes_inside(_np.c_[args])
+
+
+r_, c_ = _RClass(), _CClass()
+
 _raw_where = where  # noqa: F821
 
 

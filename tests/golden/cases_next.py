@@ -446,4 +446,34 @@ def next_cases(be, ext):
             out[f"more/{name}_{tag}/jvp_tangent"] = be.make_jvp(f)(x)(tangent_in)[1]
             weights2 = P(onp.asarray(rs2.randn(*onp.shape(be.get(x)))).astype(dtype))
             out[f"more/{name}_{tag}/second"] = grad(lambda a: np.sum(grad(f)(a) * weights2))(x)  # noqa: B023
+    # ---- joins written with the index tricks and the list-taking helpers of numpy_wrapper.py:58-60, 73-80, 139-169
+    # (r_, c_, append, column_stack, select).  A generator of their own again. ----
+    rs3 = onp.random.RandomState(31)
+    h32, h32b, h3 = rs3.randn(3, 2), rs3.randn(3, 2), rs3.randn(3)
+    hsel = rs3.randn(3, 4)
+    c1, c2 = rs3.randn(3, 4) > 0.2, rs3.randn(3, 4) > -0.3
+    for dtype in (onp.float64, onp.float32):
+        tag = "f32" if dtype == onp.float32 else "f64"
+        X_, K_, V_, S_ = (P(h.astype(dtype)) for h in (h32, h32b, h3, hsel))
+        W62, W36, W34b = (P(rs3.randn(*shape).astype(dtype)) for shape in ((6, 2), (3, 6), (3, 4)))
+        w9, w8 = P(rs3.randn(9).astype(dtype)), P(rs3.randn(8).astype(dtype))
+        M1, M2 = P(c1), P(c2)
+        joins = {
+            "r_double": (lambda x: np.sum(np.r_[x, x] ** 2 * W62), X_),
+            "r_mixed": (lambda x: np.sum(np.sin(np.r_[x, K_]) * W62), X_),
+            "r_vector_and_range": (lambda v: np.sum(np.r_[v, V_, 1:4] ** 2 * w9), V_),
+            "c_mixed": (lambda x: np.sum(np.c_[x, K_, x] ** 3 * W36), X_),
+            "c_vectors": (lambda v: np.sum(np.c_[v, V_ * v] ** 2), V_),
+            "append_flat": (lambda x: np.sum(np.append(x, K_[0]) ** 2 * w8), X_),
+            "append_axis": (lambda x: np.sum(np.tanh(np.append(x, K_, axis=0)) * W62), X_),
+            "column_stack": (lambda v: np.sum(np.column_stack((v, K_, v * v)) ** 2), V_),
+            "select": (lambda a: np.sum(np.select([M1, M2], [a * a, np.sin(a)], default=0.5) * W34b), S_),
+        }
+        for name, (f, x) in joins.items():
+            out[f"joins/{name}_{tag}/value"] = f(x)
+            out[f"joins/{name}_{tag}/grad"] = grad(f)(x)
+            tangent_in = P(onp.asarray(rs3.randn(*onp.shape(be.get(x)))).astype(dtype))
+            out[f"joins/{name}_{tag}/jvp_tangent"] = be.make_jvp(f)(x)(tangent_in)[1]
+            weights2 = P(onp.asarray(rs3.randn(*onp.shape(be.get(x)))).astype(dtype))
+            out[f"joins/{name}_{tag}/second"] = grad(lambda a: np.sum(grad(f)(a) * weights2))(x)  # noqa: B023
     return out
