@@ -64,7 +64,7 @@ _METHODS["flatten"] = anp.ravel
 class DevArrayBox(Box):
     __slots__ = []
     __array_priority__ = 300.0
-    __array_ufunc__ = None  # ndarray <op> box defers to the box's reflected operator
+    __array_ufunc__ = DevArray.__array_ufunc__  # numpy.exp(box), ndarray <op> box: the namespace's (traced) function
     _namespace = staticmethod(lambda: __import__("autograd_amd.numpy", fromlist=["numpy"]))
 
     @primitive

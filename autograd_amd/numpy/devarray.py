@@ -33,8 +33,18 @@ class DevArray:
     """n-d array in GPU memory; arithmetic is hand-written HIP kernels."""
 
     __slots__ = ("_t", "dtype", "_borrowed", "_shape_tuple")
-    __array_ufunc__ = None  # NumPy binary operators defer to ours (ndarray * DevArray -> __rmul__)
     __array_priority__ = 200.0
+
+    def __array_ufunc__(self, ufunc, method, *inputs, **kwargs):
+        """A NumPy ufunc applied to a device array (``numpy.abs(x)``, ``host_array * x``, ``numpy.float64(2) * x``)
+        runs the namespace's function of the same name on the device; anything else (``out=``, ``.reduce`` ...)
+        is declined, which NumPy reports as a TypeError."""
+        if method != "__call__" or kwargs:
+            return NotImplemented
+        from . import wrapper
+
+        fn = getattr(wrapper, ufunc.__name__, None)
+        return NotImplemented if fn is None else fn(*inputs)
 
     def __init__(self, tensor, dtype=None):
         self._t = tensor

@@ -422,3 +422,25 @@ def test_names_that_take_no_array_data(np):
     assert np.issubdtype(np.float64, np.floating) and np.broadcast_shapes((3, 1), (4,)) == (3, 4)
     onp.testing.assert_array_equal(_host(np.identity(3)), onp.identity(3))
     onp.testing.assert_array_equal(_host(np.arange(10.0)[np.s_[2:5]]), [2.0, 3.0, 4.0])
+
+
+def test_numpy_ufuncs_called_on_device_arrays_and_boxes(ag, np):
+    """``numpy.abs(x)``, ``host * x``, ``numpy.float64(2) * x`` and ``numpy.sin(box)`` run the namespace's function of
+    the same name (tests/test_numpy.py:157-180 feeds ``npr.randn`` results to plain NumPy functions); forms the
+    namespace has no counterpart for are declined, which NumPy reports as a TypeError."""
+    h, g = onp.array([1.0, -2.0, 3.0]), onp.array([2.0, 2.0, 2.0])
+    x = np.array(h)
+    onp.testing.assert_array_equal(_host(onp.abs(x)), onp.abs(h))
+    onp.testing.assert_allclose(_host(onp.exp(x)), onp.exp(h), rtol=1e-15)
+    onp.testing.assert_array_equal(_host(g * x), g * h)
+    onp.testing.assert_array_equal(_host(g < x), g < h)
+    onp.testing.assert_array_equal(_host(onp.maximum(g, x)), onp.maximum(g, h))
+    x32 = np.array(h.astype(onp.float32))
+    assert (onp.float64(2.0) * x32).dtype == onp.float64 and (2.0 * x32).dtype == onp.float32
+    assert (g.astype(onp.float32) * x32).dtype == onp.float32
+    got = ag.grad(lambda v: np.sum(onp.sin(v) * g))(x)
+    onp.testing.assert_allclose(_host(got), onp.cos(h) * g, rtol=1e-15)
+    with pytest.raises(TypeError):
+        onp.add(x, x, out=onp.zeros(3))
+    with pytest.raises(TypeError):
+        onp.add.reduce(x)
