@@ -14,9 +14,10 @@ scattered into an owned dense buffer, which is zero-filled on first use or copie
 predecessor that was not owned.
 """
 
+import warnings
 from itertools import count
 
-from .tracer import Box, Node, getval, isbox, primitive, toposort, trace
+from .tracer import Box, Node, box_type_mappings, getval, isbox, new_box, primitive, toposort, trace, trace_stack
 from .util import collector_paused, func, subval
 
 
@@ -53,10 +54,50 @@ primitive_vjps = {}
 def make_vjp(fun, x):
     """Trace ``fun`` at ``x``; return ``(vjp, fun(x))``.  A result that does not depend on ``x``
     (nothing was traced) has the zero cotangent."""
+    if type(x) is tuple and x and all(type(element) in box_type_mappings for element in x):
+        return _make_vjp_by_element(fun, x)
     value, last = trace(VJPNode.new_root(), fun, x)
     if last is None:
         return (lambda g: vspace(x).zeros()), value
     return (lambda g: settle(backward_pass(g, last))), value
+
+
+def _make_vjp_by_element(fun, xs):
+    """``make_vjp`` for a tuple argument (several ``argnum`` s, or a tuple of parameters), every element traced
+    from a root of its own.
+
+    The reference boxes the tuple itself (autograd/builtins.py:37-96): each element then reaches ``fun`` through a
+    ``container_take`` node whose cotangent is scattered back into a tuple of zeros (builtins.py:24-34,
+    core.py:185-215).  Here ``fun`` receives a plain tuple of boxes, so those nodes, the sparse cotangents and the
+    tuple-level accumulation never exist; what they did to the values is applied once at the end: element ``i`` of
+    the result is ``vspace(xs[i]).mut_add(zeros, cotangent of root i)``, which is what gives a cotangent the dtype of
+    its argument (a float64 cotangent of a float32 argument comes back float32, unlike with a single ``argnum``) and
+    turns a ``-0.0`` into ``0.0``, exactly as the scattered form does."""
+    with trace_stack.new_trace() as level:
+        roots = [VJPNode.new_root() for _ in xs]
+        end_box = fun(tuple(new_box(x, level, root) for x, root in zip(xs, roots)))
+        traced = isbox(end_box) and end_box._trace == level
+    if not traced:
+        warnings.warn("Output seems independent of input.")
+        return (lambda g: vspace(xs).zeros()), end_box
+    end_node = end_box._node
+    position = {root: i for i, root in enumerate(roots)}
+
+    def pull_back(g):
+        table = {end_node: (g, False)}
+        found = {}
+        with collector_paused():
+            for node in toposort(end_node):
+                cotangent = table.pop(node)[0]
+                if node in position:
+                    found[position[node]] = cotangent
+                    continue
+                for parent, share in zip(node.parents, node.vjp(cotangent)):
+                    table[parent] = add_outgrads(table.get(parent), share)
+        spaces = [vspace(x) for x in xs]
+        return settle(tuple(space.mut_add(None, found[i]) if i in found else space.zeros() for i, space in enumerate(spaces)))
+
+    return pull_back, end_box._value
 
 
 def make_vjp_and_batched(fun, x):

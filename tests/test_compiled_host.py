@@ -51,7 +51,7 @@ def test_compiled_modules_are_served_while_they_match_their_sources(monkeypatch)
     real = _compiled.source_hash
     monkeypatch.setattr(_compiled, "source_hash", lambda path: "0" * 64 if path.endswith("util.py") else real(path))
     table, reason = _compiled._usable()
-    assert table is None and "util.py changed" in reason
+    assert table is None and "changed after it was compiled" in reason  # (names util.py, or a source edited since the build)
     monkeypatch.setenv("AUTOGRAD_AMD_PURE_PYTHON", "1")
     assert _compiled._usable() == (None, "AUTOGRAD_AMD_PURE_PYTHON is set")
 
