@@ -50,8 +50,24 @@ for _linear in (container_take, container_untake):
 class _ContainerBox(Box):
     """What tuples, lists and dicts share when boxed: traced item access, untraced size and membership."""
 
-    __slots__ = []
-    __getitem__ = container_take
+    __slots__ = ["_taken"]
+
+    def __getitem__(self, idx):
+        """Traced item access (builtins.py:37-40).  An item taken before is handed out again as the same box, so a
+        loop that reads ``params["W"]`` at every step leaves one ``container_take`` node on the tape instead of one
+        per step: the uses then share that node the way they would had the program kept the item in a variable,
+        and its cotangents are accumulated there (core.py:185-205) before ONE scattered add into the container."""
+        try:
+            taken = self._taken
+        except AttributeError:
+            taken = self._taken = {}
+        try:
+            return taken[idx]
+        except KeyError:
+            item = taken[idx] = container_take(self, idx)
+            return item
+        except TypeError:  # an index that cannot be a key (a slice)
+            return container_take(self, idx)
 
     def __len__(self):
         return len(self._value)

@@ -76,3 +76,31 @@ def test_higher_order_and_untraced_outputs():
     ga, gb = pull_back(onp.ones(2))
     onp.testing.assert_allclose(ga, onp.cos(x) * y, rtol=1e-15)
     onp.testing.assert_allclose(gb, onp.sin(x), rtol=1e-15)
+
+
+def test_repeated_item_access_shares_one_tape_node():
+    """``params["W"]`` read at every step of a loop (examples/rnn.py:38-44) hands out the box of the first read: the
+    gradient is, bit for bit, that of the program which keeps the item in a variable; slices are taken anew."""
+    rs = onp.random.RandomState(0)
+    params = {"W": rs.randn(4, 4), "b": rs.randn(4)}
+    x = rs.randn(3, 4)
+
+    def reads_every_step(p):
+        h = x
+        for _ in range(5):
+            h = np.tanh(np.dot(h, p["W"]) + p["b"])
+        return np.sum(h)
+
+    def reads_once(p):
+        W, b = p["W"], p["b"]
+        h = x
+        for _ in range(5):
+            h = np.tanh(np.dot(h, W) + b)
+        return np.sum(h)
+
+    a, b = ag.grad(reads_every_step)(params), ag.grad(reads_once)(params)
+    for key in params:
+        onp.testing.assert_array_equal(a[key], b[key])
+    seen = []
+    ag.grad(lambda t: (seen.append((t[0] is t[0], t[0:1] is t[0:1])) or np.sum(t[0])))([params["W"], params["b"]])
+    assert seen[-1] == (True, False)
