@@ -504,7 +504,7 @@ def extras(be):
     params = configs.tree_map(be.put, inp["params"])
     xs, ts = be.put(inp["inputs"]), be.put(inp["targets"])
     g4 = configs.rnn_program(be)["grad"]
-    ms = time_steps(lambda: g4(params, xs, ts), be.sync, 5, 1) * 1e3
+    ms = time_steps(lambda: g4(params, xs, ts), be.sync, 20, 3) * 1e3
     out["rnn_grad_evals_per_sec"] = 1e3 / ms
     out["rnn_grad_graph_evals_per_sec"] = graph_rate(g4, (params, xs, ts), be.sync, 5)
     # config 5: Rosenbrock HVP, f64
