@@ -54,7 +54,8 @@ primitive_vjps = {}
 def make_vjp(fun, x):
     """Trace ``fun`` at ``x``; return ``(vjp, fun(x))``.  A result that does not depend on ``x``
     (nothing was traced) has the zero cotangent."""
-    if type(x) is tuple and x and all(type(element) in box_type_mappings for element in x):
+    if (type(x) is tuple and x and getattr(fun, "unpacks_its_tuple", False)
+            and all(type(element) in box_type_mappings for element in x)):
         return _make_vjp_by_element(fun, x)
     value, last = trace(VJPNode.new_root(), fun, x)
     if last is None:
@@ -63,8 +64,11 @@ def make_vjp(fun, x):
 
 
 def _make_vjp_by_element(fun, xs):
-    """``make_vjp`` for a tuple argument (several ``argnum`` s, or a tuple of parameters), every element traced
-    from a root of its own.
+    """``make_vjp`` for the tuple of arguments that several ``argnum`` s select, every element traced from a root
+    of its own.  Only for a ``fun`` that declares ``unpacks_its_tuple`` (``wrap_util.unary_to_nary`` sets it on the
+    function it builds for several ``argnum`` s: that function does nothing with the tuple but unpack it).  A
+    tuple that a caller passes as ONE argument is boxed as a container, as in the reference: user code may hand it
+    to a primitive or return a slice of it, which needs the box.
 
     The reference boxes the tuple itself (autograd/builtins.py:37-96): each element then reaches ``fun`` through a
     ``container_take`` node whose cotangent is scattered back into a tuple of zeros (builtins.py:24-34,

@@ -56,6 +56,7 @@ def unary_to_nary(unary_operator):
                 pairs = [(argnum, x)] if single else zip(argnum, x)
                 return fun(*subvals(args, pairs), **kwargs)
 
+            unary_f.unpacks_its_tuple = not single  # (lets make_vjp trace the picked arguments one by one)
             x0 = args[argnum] if single else tuple(args[i] for i in argnum)
             with collector_paused():  # see util.collector_paused: tapes hold no cycles
                 return unary_operator(unary_f, x0, *op_args, **op_kwargs)

@@ -104,3 +104,23 @@ def test_repeated_item_access_shares_one_tape_node():
     seen = []
     ag.grad(lambda t: (seen.append((t[0] is t[0], t[0:1] is t[0:1])) or np.sum(t[0])))([params["W"], params["b"]])
     assert seen[-1] == (True, False)
+
+
+def test_a_tuple_passed_as_one_argument_stays_a_boxed_container():
+    """Only the tuple that several ``argnum`` s build is traced element by element; a caller's own tuple may be
+    sliced and returned, or handed to a primitive, which needs the box (autograd/builtins.py:37-96)."""
+    from autograd_amd.extend import defvjp, primitive
+
+    x, y, z = onp.array([1.0, 2.0]), onp.array([3.0]), onp.array([4.0, 5.0, 6.0])
+    pull_back, out = ag.make_vjp(lambda p: p[1:])((x, y, z))
+    assert isinstance(out, tuple) and len(out) == 2
+    got = pull_back((onp.array([7.0]), onp.array([1.0, 1.0, 1.0])))
+    assert not got[0].any() and got[1][0] == 7.0 and got[2].sum() == 3.0
+
+    @primitive
+    def total(parts):
+        return onp.float64(sum(float(onp.sum(part)) for part in parts))
+
+    defvjp(total, lambda ans, parts: lambda g: tuple(g * onp.ones_like(part) for part in parts))
+    grads = ag.grad(lambda p: total(p) * 2.0)((x, y, z))
+    assert [g.tolist() for g in grads] == [[2.0, 2.0], [2.0], [2.0, 2.0, 2.0]]
