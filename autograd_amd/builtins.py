@@ -21,7 +21,9 @@ type = notrace_primitive(type_)
 
 # ---- taking an element out of a container, and its cotangent (builtins.py:24-34, 99-109) ---------
 @primitive
-def container_take(A, idx):
+def container_take(A, idx, space=None):
+    """``A[idx]``.  ``space``: None, or a callable giving ``vspace(A)`` (boxes pass one that computes it once for all
+    the items taken from the same container, see ``_ContainerBox.__getitem__``); the value does not depend on it."""
     return A[idx]
 
 
@@ -40,13 +42,32 @@ def container_untake(x, idx, vs):
     return SparseObject(vs, lambda A: vs._subval(A, idx, merged(A[idx])))
 
 
-defvjp(container_take, lambda ans, A, idx: lambda g: container_untake(g, idx, vspace(A)))
+defvjp(container_take,
+       lambda ans, A, idx, space=None: lambda g: container_untake(g, idx, vspace(A) if space is None else space()))
 defvjp(container_untake, lambda ans, x, idx, _: lambda g: container_take(g, idx))
 for _linear in (container_take, container_untake):
     defjvp(_linear, "same")
 
 
 # ---- boxes (builtins.py:37-96) -------------------------------------------------------------------
+class _SpaceOnce:
+    """``vspace(value)``, computed at the first call: the cotangent rules of all the items taken from one container
+    need the container's vector space, which is as large as the container."""
+
+    __slots__ = ("value", "space")
+
+    def __init__(self, value):
+        self.value, self.space = value, None
+
+    def __call__(self):
+        if self.space is None:
+            self.space, self.value = vspace(self.value), None
+        return self.space
+
+
+_SPACE = object()  # key of the shared `_SpaceOnce` among a box's taken items (no index compares equal to it)
+
+
 class _ContainerBox(Box):
     """What tuples, lists and dicts share when boxed: traced item access, untraced size and membership."""
 
@@ -60,14 +81,14 @@ class _ContainerBox(Box):
         try:
             taken = self._taken
         except AttributeError:
-            taken = self._taken = {}
+            taken = self._taken = {_SPACE: _SpaceOnce(self._value)}
         try:
             return taken[idx]
         except KeyError:
-            item = taken[idx] = container_take(self, idx)
+            item = taken[idx] = container_take(self, idx, space=taken[_SPACE])
             return item
         except TypeError:  # an index that cannot be a key (a slice)
-            return container_take(self, idx)
+            return container_take(self, idx, space=taken[_SPACE])
 
     def __len__(self):
         return len(self._value)
