@@ -398,7 +398,7 @@ def test_host_arrays_enter_at_the_differential_operator():
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     env = dict(os.environ, PYTHONPATH=root + os.pathsep + os.environ.get("PYTHONPATH", ""))
     env.pop("AUTOGRAD_AMD_HOST", None)
-    done = subprocess.run([sys.executable, "-c", HOST_ARRAY_PROGRAM], env=env, capture_output=True, text=True, timeout=170)
+    done = subprocess.run([sys.executable, "-c", HOST_ARRAY_PROGRAM], env=env, capture_output=True, text=True, timeout=600)
     assert done.returncode == 0 and "host arrays ok" in done.stdout, done.stdout + done.stderr
 
 
