@@ -98,8 +98,16 @@ def _make_vjp_by_element(fun, xs):
                     continue
                 for parent, share in zip(node.parents, node.vjp(cotangent)):
                     table[parent] = add_outgrads(table.get(parent), share)
-        spaces = [vspace(x) for x in xs]
-        return settle(tuple(space.mut_add(None, found[i]) if i in found else space.zeros() for i, space in enumerate(spaces)))
+        out = []
+        for i, x in enumerate(xs):
+            space = vspace(x)
+            if i not in found:
+                out.append(space.zeros())
+            elif isbox(found[i]):  # this pull-back is itself being traced: through the primitive
+                out.append(space.mut_add(None, found[i]))
+            else:
+                out.append(space._mut_add(space.zeros(), found[i]))  # (what the primitive would run)
+        return settle(tuple(out))
 
     return pull_back, end_box._value
 

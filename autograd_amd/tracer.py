@@ -15,7 +15,6 @@ the call is recorded there as well), and re-boxes the result with a new node.
 
 import warnings
 from collections import defaultdict
-from contextlib import contextmanager
 
 from .util import subvals, toposort  # noqa: F401  (toposort re-exported as in the reference)
 from .wrap_util import wraps
@@ -60,19 +59,31 @@ class Node:
         return root
 
 
+class _OpenTrace:
+    """``with trace_stack.new_trace() as level``: one more nesting level for the duration of the block."""
+
+    __slots__ = ("stack",)
+
+    def __init__(self, stack):
+        self.stack = stack
+
+    def __enter__(self):
+        self.stack.top += 1
+        return self.stack.top
+
+    def __exit__(self, *exc):
+        self.stack.top -= 1
+        return False
+
+
 class TraceStack:
     """Process-global counter of nested traces (single-threaded by contract)."""
 
     def __init__(self):
         self.top = -1
 
-    @contextmanager
     def new_trace(self):
-        self.top += 1
-        try:
-            yield self.top
-        finally:
-            self.top -= 1
+        return _OpenTrace(self)
 
 
 trace_stack = TraceStack()

@@ -26,6 +26,12 @@ def wraps(fun, namestr="{fun}", docstr="{doc}", **fmt):
     """Decorator copying a (formatted) name and docstring from ``fun``."""
 
     def decorate(f):
+        if namestr == "{fun}" and docstr == "{doc}":  # a plain copy (made on every call of a differential operator)
+            try:
+                f.__name__, f.__doc__ = get_name(fun), get_doc(fun)
+            except AttributeError:
+                pass
+            return f
         with suppress(AttributeError, KeyError, ValueError):
             f.__name__ = namestr.format(fun=get_name(fun), **fmt)
             f.__doc__ = docstr.format(fun=get_name(fun), doc=get_doc(fun), **fmt)
