@@ -342,7 +342,8 @@ def main():
     # fourth of its launches (a pair costs the host about 7 us and delays the launch behind it: on the 140 us step
     # of the headline workload, events on every launch took 15-20 us per step)
     be.sync()
-    with _lib.KernelTimer(only={dom_key}, events=2 * args.steps * dom_launches, every=4) as kt:
+    every = max(4, dom_launches // 4)  # (a kernel launched hundreds of times per step carries about four pairs per step)
+    with _lib.KernelTimer(only={dom_key}, events=2 * args.steps * dom_launches, every=every) as kt:
         t0 = time.perf_counter()
         for _ in range(args.steps):
             step()
@@ -381,7 +382,7 @@ def main():
     roofline["timing"] = ("HIP events on the launch stream around every launch of this kernel over `steps` steps, the stream "
                           "kept busy ahead of each step so that the pair brackets GPU execution only; the pair's own cost "
                           "(measured live: 2 x pair around one 64 MiB fill - pair around two) is subtracted; "
-                          "avg_launch_ms_in_timed_region comes from events around every fourth launch inside the timed region, "
+                          "avg_launch_ms_in_timed_region comes from events around every fourth launch (of a kernel launched many times per step: about four launches per step) inside the timed region, "
                           "where the host sets the pace and the figure includes what the pair itself adds")
 
     result = {
