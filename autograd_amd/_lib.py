@@ -162,6 +162,9 @@ def lib():
     L.agmi_last_kernel.argtypes = []
     L.agmi_elementwise.restype = c_i
     L.agmi_elementwise.argtypes = [c_i, c_i, c_i, p_i64, c_i, p_arr, c_i, p_arr, p_d, c_p]
+    L.agmi_program.restype = c_i
+    L.agmi_program.argtypes = [c_i, c_i, p_i64, c_i, p_arr, c_i, p_arr, c_i, p_d, c_i, ctypes.POINTER(ctypes.c_uint32), c_i,
+                               c_p]
     L.agmi_compare.restype = c_i
     L.agmi_compare.argtypes = [c_i, c_i, c_i, p_i64, p_arr, p_arr, p_d, c_p]
     L.agmi_cast.restype = c_i
@@ -202,7 +205,7 @@ def lib():
 
 
 EXPORTS = (
-    "agmi_last_error agmi_version agmi_last_kernel agmi_elementwise agmi_compare agmi_cast agmi_map_reduce "
+    "agmi_last_error agmi_version agmi_last_kernel agmi_elementwise agmi_program agmi_compare agmi_cast agmi_map_reduce "
     "agmi_map_reduce_workspace_bytes agmi_map_reduce_static agmi_gemm agmi_fill agmi_take_rows agmi_sort_rows agmi_cumsum agmi_reverse agmi_triangle agmi_scatter_add_rows agmi_optimizer_step "
     "agmi_correlate agmi_lse_cotangent_fused agmi_concat"
 ).split()
@@ -455,6 +458,43 @@ def elementwise(op, code, shape, outs, ins):
         _check(rc, "agmi_elementwise")
     if ev is not None:
         _TIMER.end(ev, ("elementwise", op), (outs, ins))
+
+
+PROGRAM_MAX_LEAVES, PROGRAM_MAX_IMMEDIATES, PROGRAM_MAX_OUTPUTS, PROGRAM_MAX_INSTRUCTIONS = 6, 6, 4, 96
+PROGRAM_MAX_REGISTERS = 16
+PROGRAM_STORE = 255
+_prog_outs = (AgmiArray * PROGRAM_MAX_OUTPUTS)()
+_prog_leaves = (AgmiArray * PROGRAM_MAX_LEAVES)()
+_prog_imms = (ctypes.c_double * PROGRAM_MAX_IMMEDIATES)()
+_prog_code = (ctypes.c_uint32 * PROGRAM_MAX_INSTRUCTIONS)()
+
+
+def program(code, shape, outs, leaves, imms, words, n_regs):
+    """Run the elementwise program ``words`` (instruction words of ``agmi_program``) over ``shape``.
+
+    ``outs`` are tensors of exactly ``shape``; ``leaves`` tensors expanded to ``shape`` (stride 0 on
+    broadcast axes); ``imms`` Python floats.  Returns False when the layout is outside what the kernel
+    covers (the caller then evaluates the steps one by one)."""
+    nd = _set_shape(shape)
+    for k, t in enumerate(outs):
+        _set_array(_prog_outs[k], t)
+    for k, t in enumerate(leaves):
+        _set_array(_prog_leaves[k], t)
+    n_imm = len(imms)
+    if n_imm:
+        _prog_imms[:n_imm] = imms
+    n = len(words)
+    _prog_code[:n] = words
+    ev = _TIMER.begin(("program",)) if _TIMER is not None else None
+    rc = _LIB.agmi_program(code, nd, _shape, len(outs), _prog_outs, len(leaves), _prog_leaves, n_imm, _prog_imms, n,
+                           _prog_code, n_regs, _stream())
+    if rc == -2:  # AGMI_ERR_UNSUPPORTED
+        return False
+    if rc:
+        _check(rc, "agmi_program")
+    if ev is not None:
+        _TIMER.end(ev, ("program",), (outs, leaves))
+    return True
 
 
 def compare(cmp, code, shape, out, ins):

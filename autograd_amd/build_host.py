@@ -20,7 +20,7 @@ from . import _compiled
 # the tracer, the backward pass, the rule tables, the value type and the launch marshalling
 MODULES = (
     "tracer", "core", "util", "wrap_util", "builtins", "differential_operators", "_lib",
-    "numpy.devarray", "numpy.wrapper", "numpy.vjps", "numpy.jvps", "numpy.boxes", "numpy.vspaces",
+    "numpy.devarray", "numpy.fusion", "numpy.wrapper", "numpy.vjps", "numpy.jvps", "numpy.boxes", "numpy.vspaces",
     "scipy.special", "scipy.signal", "misc.flatten", "misc.optimizers",
 )
 _DIRECTIVES = ("language_level=3", "annotation_typing=False", "binding=True", "always_allow_keywords=True")

@@ -39,10 +39,28 @@ def settle(value):
     if finish is not None:
         return finish(value)
     if kind is tuple or kind is list:
+        _settle_together(value)
         return kind(settle(item) for item in value)
     if kind is dict:
+        _settle_together(value.values())
         return {key: settle(item) for key, item in value.items()}
     return value
+
+
+def _settle_together(items):
+    """Items of one container whose type can complete several values in one go (``_settle_group``:
+    the cotangents of several arguments usually share most of their arithmetic) are handed over together."""
+    groups = None
+    for item in items:
+        together = getattr(type(item), "_settle_group", None)
+        if together is not None:
+            if groups is None:
+                groups = {}
+            groups.setdefault(together, []).append(item)
+    if groups is not None:
+        for together, members in groups.items():
+            if len(members) > 1:
+                together(members)
 
 
 # ----------------------------------------------------------------------------------------------

@@ -14,7 +14,13 @@
 
 namespace agmi {
 
-// math on T in {float, double}
+// math on T in {float, double}.  The long library routines are inlined into the one-rule kernels; a
+// translation unit that holds many of them in one kernel (the program interpreter) defines
+// AGMI_HEAVY_MATH as `static __device__ __noinline__` before including this file, so that each is one
+// function called element by element and its temporaries do not add to the kernel's register budget.
+#ifndef AGMI_HEAVY_MATH
+#define AGMI_HEAVY_MATH __device__ __forceinline__
+#endif
 __device__ __forceinline__ float m_exp(float x) { return expf(x); }
 __device__ __forceinline__ double m_exp(double x) { return exp(x); }
 // exp(d) for d <= 0 (an element minus the logsumexp of its row) to within 1 ulp of expf, without the
@@ -32,51 +38,51 @@ __device__ __forceinline__ float exp_of_nonpositive(float d) {
 __device__ __forceinline__ double exp_of_nonpositive(double d) { return exp(d); }
 __device__ __forceinline__ float m_log(float x) { return logf(x); }
 __device__ __forceinline__ double m_log(double x) { return log(x); }
-__device__ __forceinline__ float m_log1p(float x) { return log1pf(x); }
-__device__ __forceinline__ double m_log1p(double x) { return log1p(x); }
-__device__ __forceinline__ float m_expm1(float x) { return expm1f(x); }
-__device__ __forceinline__ double m_expm1(double x) { return expm1(x); }
-__device__ __forceinline__ float m_tanh(float x) { return tanhf(x); }
-__device__ __forceinline__ double m_tanh(double x) { return tanh(x); }
-__device__ __forceinline__ float m_sinh(float x) { return sinhf(x); }
-__device__ __forceinline__ double m_sinh(double x) { return sinh(x); }
-__device__ __forceinline__ float m_cosh(float x) { return coshf(x); }
-__device__ __forceinline__ double m_cosh(double x) { return cosh(x); }
-__device__ __forceinline__ float m_sin(float x) { return sinf(x); }
-__device__ __forceinline__ double m_sin(double x) { return sin(x); }
-__device__ __forceinline__ float m_cos(float x) { return cosf(x); }
-__device__ __forceinline__ double m_cos(double x) { return cos(x); }
+AGMI_HEAVY_MATH float m_log1p(float x) { return log1pf(x); }
+AGMI_HEAVY_MATH double m_log1p(double x) { return log1p(x); }
+AGMI_HEAVY_MATH float m_expm1(float x) { return expm1f(x); }
+AGMI_HEAVY_MATH double m_expm1(double x) { return expm1(x); }
+AGMI_HEAVY_MATH float m_tanh(float x) { return tanhf(x); }
+AGMI_HEAVY_MATH double m_tanh(double x) { return tanh(x); }
+AGMI_HEAVY_MATH float m_sinh(float x) { return sinhf(x); }
+AGMI_HEAVY_MATH double m_sinh(double x) { return sinh(x); }
+AGMI_HEAVY_MATH float m_cosh(float x) { return coshf(x); }
+AGMI_HEAVY_MATH double m_cosh(double x) { return cosh(x); }
+AGMI_HEAVY_MATH float m_sin(float x) { return sinf(x); }
+AGMI_HEAVY_MATH double m_sin(double x) { return sin(x); }
+AGMI_HEAVY_MATH float m_cos(float x) { return cosf(x); }
+AGMI_HEAVY_MATH double m_cos(double x) { return cos(x); }
 __device__ __forceinline__ float m_sqrt(float x) { return sqrtf(x); }
 __device__ __forceinline__ double m_sqrt(double x) { return sqrt(x); }
 __device__ __forceinline__ float m_abs(float x) { return fabsf(x); }
 __device__ __forceinline__ double m_abs(double x) { return fabs(x); }
-__device__ __forceinline__ float m_pow(float x, float y) { return powf(x, y); }
-__device__ __forceinline__ double m_pow(double x, double y) { return pow(x, y); }
+AGMI_HEAVY_MATH float m_pow(float x, float y) { return powf(x, y); }
+AGMI_HEAVY_MATH double m_pow(double x, double y) { return pow(x, y); }
 
-__device__ __forceinline__ float m_exp2(float x) { return exp2f(x); }
-__device__ __forceinline__ double m_exp2(double x) { return exp2(x); }
+AGMI_HEAVY_MATH float m_exp2(float x) { return exp2f(x); }
+AGMI_HEAVY_MATH double m_exp2(double x) { return exp2(x); }
 __device__ __forceinline__ float m_log2(float x) { return log2f(x); }
 __device__ __forceinline__ double m_log2(double x) { return log2(x); }
 __device__ __forceinline__ float m_log10(float x) { return log10f(x); }
 __device__ __forceinline__ double m_log10(double x) { return log10(x); }
-__device__ __forceinline__ float m_tan(float x) { return tanf(x); }
-__device__ __forceinline__ double m_tan(double x) { return tan(x); }
-__device__ __forceinline__ float m_asin(float x) { return asinf(x); }
-__device__ __forceinline__ double m_asin(double x) { return asin(x); }
-__device__ __forceinline__ float m_acos(float x) { return acosf(x); }
-__device__ __forceinline__ double m_acos(double x) { return acos(x); }
-__device__ __forceinline__ float m_atan(float x) { return atanf(x); }
-__device__ __forceinline__ double m_atan(double x) { return atan(x); }
-__device__ __forceinline__ float m_asinh(float x) { return asinhf(x); }
-__device__ __forceinline__ double m_asinh(double x) { return asinh(x); }
-__device__ __forceinline__ float m_acosh(float x) { return acoshf(x); }
-__device__ __forceinline__ double m_acosh(double x) { return acosh(x); }
-__device__ __forceinline__ float m_atanh(float x) { return atanhf(x); }
-__device__ __forceinline__ double m_atanh(double x) { return atanh(x); }
-__device__ __forceinline__ float m_atan2(float y, float x) { return atan2f(y, x); }
-__device__ __forceinline__ double m_atan2(double y, double x) { return atan2(y, x); }
-__device__ __forceinline__ float m_hypot(float x, float y) { return hypotf(x, y); }
-__device__ __forceinline__ double m_hypot(double x, double y) { return hypot(x, y); }
+AGMI_HEAVY_MATH float m_tan(float x) { return tanf(x); }
+AGMI_HEAVY_MATH double m_tan(double x) { return tan(x); }
+AGMI_HEAVY_MATH float m_asin(float x) { return asinf(x); }
+AGMI_HEAVY_MATH double m_asin(double x) { return asin(x); }
+AGMI_HEAVY_MATH float m_acos(float x) { return acosf(x); }
+AGMI_HEAVY_MATH double m_acos(double x) { return acos(x); }
+AGMI_HEAVY_MATH float m_atan(float x) { return atanf(x); }
+AGMI_HEAVY_MATH double m_atan(double x) { return atan(x); }
+AGMI_HEAVY_MATH float m_asinh(float x) { return asinhf(x); }
+AGMI_HEAVY_MATH double m_asinh(double x) { return asinh(x); }
+AGMI_HEAVY_MATH float m_acosh(float x) { return acoshf(x); }
+AGMI_HEAVY_MATH double m_acosh(double x) { return acosh(x); }
+AGMI_HEAVY_MATH float m_atanh(float x) { return atanhf(x); }
+AGMI_HEAVY_MATH double m_atanh(double x) { return atanh(x); }
+AGMI_HEAVY_MATH float m_atan2(float y, float x) { return atan2f(y, x); }
+AGMI_HEAVY_MATH double m_atan2(double y, double x) { return atan2(y, x); }
+AGMI_HEAVY_MATH float m_hypot(float x, float y) { return hypotf(x, y); }
+AGMI_HEAVY_MATH double m_hypot(double x, double y) { return hypot(x, y); }
 
 // numpy.logaddexp (npy_math: equal operands -> x + log 2; otherwise the larger one plus log1p of
 // the exponential of the negative distance; a NaN distance is returned as it is)
@@ -102,8 +108,8 @@ __device__ __forceinline__ T logaddexp2_like_numpy(T x, T y) {
 
 // numpy.remainder for floating point (npy_divmod): fmod, then moved by one divisor when its sign
 // differs from the divisor's; an exact multiple gives a zero with the divisor's sign; b == 0 -> NaN.
-__device__ __forceinline__ float m_fmod(float a, float b) { return fmodf(a, b); }
-__device__ __forceinline__ double m_fmod(double a, double b) { return fmod(a, b); }
+AGMI_HEAVY_MATH float m_fmod(float a, float b) { return fmodf(a, b); }
+AGMI_HEAVY_MATH double m_fmod(double a, double b) { return fmod(a, b); }
 __device__ __forceinline__ float m_copysign(float a, float b) { return copysignf(a, b); }
 __device__ __forceinline__ double m_copysign(double a, double b) { return copysign(a, b); }
 template <typename T>
@@ -256,8 +262,8 @@ AGMI_FUNCTOR(FEqualAsFloat, 2, 1, o[0] = (x[0] == x[1]) ? T(1) : T(0);)
 // (g, x, ans, n): g * astype(x == ans, dtype) / n
 AGMI_FUNCTOR(FExtremumVjp, 4, 1, o[0] = (x[0] * ((x[1] == x[2]) ? T(1) : T(0))) / x[3];)
 
-// X(op enum, functor)
-#define AGMI_FOR_EACH_OP(X)                     \
+// X(op enum, functor): the operations with one result (what an elementwise program may contain)
+#define AGMI_FOR_EACH_PROGRAM_OP(X)             \
     X(AGMI_OP_COPY, FCopy)                      \
     X(AGMI_OP_NEG, FNeg)                        \
     X(AGMI_OP_EXP, FExp)                        \
@@ -320,9 +326,13 @@ AGMI_FUNCTOR(FExtremumVjp, 4, 1, o[0] = (x[0] * ((x[1] == x[2]) ? T(1) : T(0))) 
     X(AGMI_OP_CHOOSE_VJP, FChooseVjp)           \
     X(AGMI_OP_LOG1P_VJP, FLog1pVjp)             \
     X(AGMI_OP_EXPM1_VJP, FExpm1Vjp)             \
-    X(AGMI_OP_DIV_VJP_BOTH, FDivVjpBoth)        \
     X(AGMI_OP_MUL_ADD, FMulAdd)                 \
     X(AGMI_OP_EQUAL_AS_FLOAT, FEqualAsFloat)    \
     X(AGMI_OP_EXTREMUM_VJP, FExtremumVjp)
+
+// every operation of agmi_elementwise
+#define AGMI_FOR_EACH_OP(X)        \
+    AGMI_FOR_EACH_PROGRAM_OP(X)    \
+    X(AGMI_OP_DIV_VJP_BOTH, FDivVjpBoth)
 
 }  // namespace agmi

@@ -10,6 +10,7 @@ primitives (and therefore the same kernels).
 from ..extend import Box, primitive
 from . import wrapper as anp
 from .devarray import DevArray, FusedResult, LazyDevArray, LseCotangent, PendingProduct
+from .fusion import ExprArray
 
 
 def _route(name, swap=False):
@@ -107,6 +108,7 @@ DevArrayBox.register(LazyDevArray)
 DevArrayBox.register(PendingProduct)
 DevArrayBox.register(LseCotangent)
 DevArrayBox.register(FusedResult)
+DevArrayBox.register(ExprArray)
 DevArrayBox.register(float)
 
 

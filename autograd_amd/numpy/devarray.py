@@ -890,16 +890,33 @@ def _lift_scalars(operands, dtype):
     return (full((), operands[0], dtype)._t,) + tuple(operands[1:])
 
 
+_fusion = None  # the module that defers elementwise steps (``fusion.py`` sets it when it is imported)
+
+
 def map_op(op, dtype, *xs, out=None, n_out=1):
-    """Launch elementwise ``op`` on broadcast operands; returns DevArray (or a tuple).
+    """Elementwise ``op`` on broadcast operands; returns DevArray (or a tuple).
 
     Negation and arithmetic with one Python scalar launch nothing when the result can be kept as
-    a pending affine map of the operand (``_fold``)."""
+    a pending affine map of the operand (``_fold``); any other single-result step is returned as a
+    pending expression node (``fusion.ExprArray``) that is evaluated, together with the steps that
+    follow it, when something first needs its memory."""
     if out is None:
+        fuse = n_out == 1 and _fusion is not None and _fusion.ENABLED
+        if fuse:
+            for x in xs:
+                if type(x) is _fusion.ExprArray and x._args is not None:
+                    node = _fusion.make(op, dtype, xs)  # (an operand that is itself pending: no map can be folded into it)
+                    if node is not None:
+                        return node
+                    break
         if op in _FOLDABLE:
             folded = _fold(op, dtype, xs)
             if folded is not None:
                 return folded
+        if fuse:
+            node = _fusion.make(op, dtype, xs)
+            if node is not None:
+                return node
     elif type(out) is not DevArray:
         raise TypeError("map_op: `out` must be a plain device array")
     ops = _limit_aux(tuple(_operand(x, dtype) for x in xs), dtype)

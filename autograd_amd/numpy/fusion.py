@@ -1,0 +1,430 @@
+"""Deferred elementwise expressions: chains of rules evaluated as ONE kernel launch.
+
+The rules of a backward pass are mostly elementwise (autograd/numpy/numpy_vjps.py:76-93, 139-143,
+157-191 of the reference: ``y * g``, ``g / y``, ``-g * x / y**2``, ``ans * g``, and between them the
+cotangent sums of autograd/core.py:185-205).  ``devarray.map_op`` is the single door every such
+step goes through; instead of launching, it returns an :class:`ExprArray`: a node that names the
+operation and its operands.  Nothing runs until something needs the memory (a contraction, a
+reduction, a gather, a host transfer, ``core.settle`` at the end of a backward pass).  At that
+moment the pending nodes under the value are written down as a straight-line program over a small
+register file and handed to ``agmi_program``, which reads each leaf array once, keeps every
+intermediate in registers and writes only what was asked for.  Values that the forward pass saved
+for its rules are recomputed inside the program instead of being stored and read back.
+
+Every step of a program is the functor of the one-rule kernel, rounded on its own, so the result
+is bit for bit what the separate launches give (``ENABLED = False`` runs exactly those; the GPU
+tests compare the two).
+
+What ends a chain: an operand of another shape (a pending operand is written out before it is
+broadcast), another dtype, more pending nodes than ``MAX_CONE``, and anything that is not
+elementwise.
+"""
+
+import os
+import sys
+
+import numpy as onp
+
+from .. import _lib
+from .._lib import Op
+from . import devarray as D
+from .devarray import DevArray, LazyDevArray
+
+ENABLED = os.environ.get("AUTOGRAD_AMD_FUSE", "1").strip() not in ("0", "")
+MAX_CONE = 64  # pending nodes under one value before its largest pending operand is written out
+
+_F32 = onp.dtype("float32")
+
+# operands each op takes (single-result ops: everything a program may contain)
+ARITY = {}
+for _name in ("COPY NEG EXP LOG TANH SINH COSH SIN COS SQRT SQUARE ABS SIGN RECIPROCAL LOG1P EXPM1 EXP2 LOG2 LOG10 TAN "
+              "ARCSIN ARCCOS ARCTAN ARCSINH ARCCOSH ARCTANH FLOOR CEIL RINT TRUNC NAN_TO_NUM").split():
+    ARITY[getattr(Op, _name)] = 1
+for _name in ("ADD SUB MUL DIV POW MAXIMUM MINIMUM FMAX FMIN ARCTAN2 HYPOT LOGADDEXP REMAINDER LOGADDEXP2 TANH_VJP "
+              "RECIPROCAL_VJP SQRT_VJP SIN_VJP COS_VJP SINH_VJP COSH_VJP SQUARE_VJP LOG1P_VJP EXPM1_VJP "
+              "EQUAL_AS_FLOAT").split():
+    ARITY[getattr(Op, _name)] = 2
+for _name in "WHERE DIV_VJP1 POW_VJP0 POW_VJP1 ABS_VJP MUL_ADD".split():
+    ARITY[getattr(Op, _name)] = 3
+for _name in "LSE_VJP CHOOSE_VJP EXTREMUM_VJP".split():
+    ARITY[getattr(Op, _name)] = 4
+
+COUNTS = {"programs": 0, "instructions": 0, "single": 0, "unfused": 0}  # what ran (tests and profiles read it)
+
+
+class ExprArray(DevArray):
+    """``op(*args)`` not yet computed.  ``args`` are device arrays (plain, pending, or with a pending
+    affine map) of this node's dtype whose shapes broadcast to this node's, and Python floats.
+    Reading ``_t`` evaluates the node together with every pending node under it."""
+
+    __slots__ = ("_op", "_args", "_shape", "_out", "_cone")
+
+    def __init__(self, op, args, shape, dtype, cone):
+        self._op, self._args, self._shape = op, args, shape
+        self.dtype = dtype
+        self._borrowed = False
+        self._shape_tuple = shape
+        self._out = None
+        self._cone = cone  # upper bound on the number of pending nodes under (and including) this one
+
+    def __getattr__(self, name):
+        # only reached when a slot is unset: `_t` before the value has been computed
+        if name != "_t":
+            raise AttributeError(name)
+        evaluate((self,))
+        return self._out
+
+    def _buffer(self):
+        out = self._out
+        if out is None:
+            out = self._out = _lib.empty(self._shape, self.dtype)
+        return out
+
+    @property
+    def shape(self):
+        return self._shape
+
+    @property
+    def ndim(self):
+        return len(self._shape)
+
+    @property
+    def size(self):
+        n = 1
+        for s in self._shape:
+            n *= s
+        return n
+
+    @property
+    def strides(self):
+        item = self.dtype.itemsize
+        return tuple(s * item for s in self._buffer().stride())
+
+    def __len__(self):
+        if not self._shape:
+            raise TypeError("len() of unsized object")
+        return self._shape[0]
+
+    def __iter__(self):
+        if not self._shape:
+            raise TypeError("iteration over a 0-d array")
+        return (self[i] for i in range(self._shape[0]))
+
+    def _h(self):
+        return self._buffer()
+
+    def _settled(self):
+        return DevArray(self._t, self.dtype)
+
+    def _view(self, fn):
+        return DevArray(fn(self._t), self.dtype)
+
+    @staticmethod
+    def _settle_group(values):
+        evaluate(values)
+
+
+def pending(x):
+    return type(x) is ExprArray and x._args is not None
+
+
+def make(op, dtype, xs):
+    """``op(*xs)`` as a pending node, or None when the step has to run the ordinary way."""
+    arity = ARITY.get(op)
+    if arity is None or arity != len(xs) or dtype not in D._FLOATS:
+        return None
+    args = []
+    shape = None
+    for x in xs:
+        if isinstance(x, DevArray):
+            if x.dtype != dtype:
+                x = D.astype(x, dtype)
+            s = x.shape
+            if shape is None:
+                shape = s
+            elif s != shape:
+                shape = D.broadcast_shapes(shape, s)
+            args.append(x)
+        elif type(x) is float or type(x) is int or D.is_scalar(x):
+            args.append(float(x))
+        else:
+            return None
+    if shape is None or len(shape) > _lib.MAX_DIMS:
+        return None
+    wide = 0
+    for s in shape:
+        if s == 0:
+            return None
+        if s > 1:
+            wide += 1
+    if wide > 6:
+        return None  # more axes than the strided kernels index when none of them merge: said at once, by the ordinary path
+    cone = 1
+    for x in args:
+        if type(x) is float:
+            continue
+        if type(x) is ExprArray and x._args is not None:
+            if x._shape != shape:
+                x._t  # a pending operand is written out before it is broadcast: programs work on one shape
+            else:
+                cone += x._cone
+        x._borrowed = True  # read when the result is evaluated: in-place accumulation and item assignment must not reach it
+    if cone > MAX_CONE:
+        node = ExprArray(op, tuple(args), shape, dtype, cone)
+        cone = node._cone = len(_post_order((node,)))
+        while cone > MAX_CONE:
+            big = None
+            for x in args:
+                if pending(x) and (big is None or x._cone > big._cone):
+                    big = x
+            big._t
+            cone = node._cone = len(_post_order((node,)))
+        return node
+    return ExprArray(op, tuple(args), shape, dtype, cone)
+
+
+def _post_order(roots):
+    """The pending nodes under ``roots``, every node after the nodes it reads."""
+    order, seen = [], set()
+    stack = [(r, 0) for r in reversed(roots)]
+    while stack:
+        node, k = stack.pop()
+        if k == 0:
+            if id(node) in seen:
+                continue
+            seen.add(id(node))
+        args = node._args
+        n = len(args)
+        while k < n:
+            a = args[k]
+            k += 1
+            if type(a) is ExprArray and a._args is not None and id(a) not in seen:
+                stack.append((node, k))
+                stack.append((a, 0))
+                break
+        else:
+            order.append(node)
+    return order
+
+
+def evaluate(values):
+    """Compute every pending node among ``values`` (nodes of one shape and dtype share a launch)."""
+    groups = {}
+    for v in values:
+        if type(v) is ExprArray and v._args is not None:
+            groups.setdefault((v._shape, v.dtype), {})[id(v)] = v
+    for group in groups.values():
+        _run(list(group.values()))
+
+
+def _finish(node):
+    node._t = node._buffer()
+    node._args = None
+
+
+def _run(roots):
+    order = _post_order(roots)
+    if len(order) == 1:
+        _single(order[0])
+        return
+    if len(roots) > _lib.PROGRAM_MAX_OUTPUTS:
+        half = len(roots) // 2
+        _run(roots[:half])
+        _run([r for r in roots[half:] if r._args is not None])
+        return
+    program = _emit(order, roots)
+    if program is None:
+        # too long, too many leaves or too many live values for one program: write a node from the middle of the
+        # order out first (everything it needs comes before it), then try again with that node as a leaf
+        if len(roots) > 1:
+            half = len(roots) // 2
+            _run(roots[:half])
+            _run([r for r in roots[half:] if r._args is not None])
+            return
+        _run([order[(len(order) - 1) // 2]])
+        _run(roots)
+        return
+    leaves, imms, words, n_regs = program
+    root = roots[0]
+    shape, dtype = root._shape, root.dtype
+    outs = tuple(r._buffer() for r in roots)
+    leaves = tuple(t if tuple(t.shape) == shape else t.expand(shape) for t in leaves)
+    if _lib.program(_lib.DTYPE_CODE[dtype], shape, outs, leaves, imms, words, n_regs):
+        COUNTS["programs"] += 1
+        COUNTS["instructions"] += len(words)
+        for r in roots:
+            _finish(r)
+        return
+    # a layout the program kernel does not cover (more than two axes left after merging, a strided innermost
+    # axis): the steps run one by one
+    COUNTS["unfused"] += 1
+    for node in order:
+        if node._args is not None:
+            _single(node)
+
+
+def _single(node):
+    """One node by the ordinary elementwise kernel (its operands are computed first)."""
+    dtype = node.dtype
+    ops = D._limit_aux(tuple(D._operand(a, dtype) for a in node._args), dtype)
+    shape = node._shape
+    ops = tuple(D._expand(t, shape) for t in ops)
+    _lib.elementwise(node._op, _lib.DTYPE_CODE[dtype], shape, (node._buffer(),), ops)
+    COUNTS["single"] += 1
+    _finish(node)
+
+
+class _TooBig(Exception):
+    pass
+
+
+def _emit(order, roots):
+    """``(leaf tensors, immediates, instruction words, registers)`` of the program that computes ``roots``;
+    None when it does not fit the kernel's limits."""
+    dtype = roots[0].dtype
+    single = dtype == _F32
+    leaves, leaf_ids = [], {}
+    imms, imm_ids = [], {}
+    # a value is ("L", k) / ("I", k) / ("X", k): leaf k, immediate k, result of instruction k
+    instrs = []   # [op, (operand values...)]
+    numbered = {}  # (op, operand values) -> value: one instruction for equal subexpressions
+    node_value = {}
+
+    def leaf(t):
+        key = (t.data_ptr(), t.stride(), tuple(t.shape))
+        v = leaf_ids.get(key)
+        if v is None:
+            if len(leaves) >= _lib.PROGRAM_MAX_LEAVES:
+                raise _TooBig
+            v = leaf_ids[key] = ("L", len(leaves))
+            leaves.append(t)
+        return v
+
+    def imm(c):
+        c = float(onp.float32(c)) if single else float(c)
+        key = (c, onp.signbit(c)) if c == 0.0 else c  # -0.0 and 0.0 are different immediates; NaN never equals itself: not shared
+        v = imm_ids.get(key)
+        if v is None:
+            if len(imms) >= _lib.PROGRAM_MAX_IMMEDIATES:
+                raise _TooBig
+            v = ("I", len(imms))
+            if c == c:
+                imm_ids[key] = v
+            imms.append(c)
+        return v
+
+    def ins(op, *srcs):
+        key = (op, srcs)
+        v = numbered.get(key)
+        if v is None:
+            if len(instrs) >= _lib.PROGRAM_MAX_INSTRUCTIONS - len(roots):
+                raise _TooBig
+            v = numbered[key] = ("X", len(instrs))
+            instrs.append(key)
+        return v
+
+    def power(x, e):
+        """``pow_like_numpy(x, e)`` for an exponent known here: the short cuts NumPy takes become the plain
+        operations they are (same bits), so that the general routine stays out of the program."""
+        if e == 2.0:
+            return ins(Op.SQUARE, x)
+        if e == 1.0:
+            return x
+        if e == 0.0:
+            return imm(1.0)
+        if e == -1.0:
+            return ins(Op.RECIPROCAL, x)
+        if e == 0.5:
+            return ins(Op.SQRT, x)
+        return ins(Op.POW, x, imm(e))
+
+    def in_dtype(c):
+        return float(onp.float32(c)) if single else c
+
+    def operand(a):
+        if type(a) is float:
+            return imm(a)
+        if type(a) is ExprArray and a._args is not None:
+            return node_value[id(a)]
+        if type(a) is LazyDevArray:
+            raw, scale, ascale, shift = D._state(a)
+            v = leaf(raw)
+            if scale != 1.0:
+                v = ins(Op.MUL, v, imm(scale))
+            if ascale is not None:
+                v = ins(Op.MUL, v, leaf(ascale))
+            if shift is not None:
+                v = ins(Op.ADD, v, imm(shift) if type(shift) is float else leaf(shift))
+            return v
+        return leaf(a._t)
+
+    try:
+        for node in order:
+            op = node._op
+            srcs = tuple(operand(a) for a in node._args)
+            if op == Op.POW and srcs[1][0] == "I":
+                v = power(srcs[0], imms[srcs[1][1]])
+            elif op == Op.POW_VJP0 and srcs[2][0] == "I":
+                # (g * y) * x**where(y, y - 1, 1), the exponent formed in the array's precision as the functor does
+                y = imms[srcs[2][1]]
+                e = in_dtype(onp.float32(y) - onp.float32(1.0)) if single else y - 1.0
+                v = ins(Op.MUL, ins(Op.MUL, srcs[0], srcs[2]), power(srcs[1], float(e) if y != 0.0 else 1.0))
+            else:
+                v = ins(op, *srcs)
+            node_value[id(node)] = v
+        root_values = [node_value[id(r)] for r in roots]
+    except _TooBig:
+        return None
+    if not instrs:
+        # every root is a leaf or an immediate after the rewrites: one copy each keeps the kernel's contract simple
+        root_values = [ins(Op.COPY, v) for v in root_values]
+
+    n_leaf, n_imm, n_ins = len(leaves), len(imms), len(instrs)
+    # last use of every value (instruction index; stores come after all instructions)
+    last = {}
+    for k, (_op, srcs) in enumerate(instrs):
+        for s in srcs:
+            last[s] = k
+    for v in root_values:
+        last[v] = n_ins
+    for n_regs in ([16] if single else [8, 16]):  # (8 float32 registers are indexed by a chain of selects in the kernel: slower than 16)
+        if n_leaf + n_imm > n_regs:
+            continue
+        reg = {("L", k): k for k in range(n_leaf)}
+        for k in range(n_imm):
+            reg[("I", k)] = n_regs - 1 - k
+        free = list(range(n_regs - 1 - n_imm, n_leaf - 1, -1))  # popped from the low end
+        for k in range(n_leaf):
+            if ("L", k) not in last:
+                free.append(k)  # (a leaf that only a rewritten-away step read)
+        words = []
+        ok = True
+        for k, (op, srcs) in enumerate(instrs):
+            regs = [reg[s] for s in srcs]
+            for s in set(srcs):
+                if s[0] != "I" and last[s] == k:
+                    free.append(reg[s])
+            v = ("X", k)
+            if v not in last:
+                dst = regs[0]  # a value nobody reads (cannot happen for nodes under a root; kept harmless)
+            elif not free:
+                ok = False
+                break
+            else:
+                dst = free.pop()
+            reg[v] = dst
+            w = op | dst << 8
+            for pos, r in enumerate(regs):
+                w |= r << (12 + 4 * pos)
+            words.append(w)
+        if not ok:
+            continue
+        for out_index, v in enumerate(root_values):
+            r = reg[v]
+            words.append(_lib.PROGRAM_STORE | r << 8 | r << 12 | out_index << 16)
+        return leaves, imms, words, n_regs
+    return None
+
+
+D._DEFERRED = D._DEFERRED + (ExprArray,)
+D._fusion = sys.modules[__name__]

@@ -12,6 +12,7 @@ from .. import _lib
 from .._lib import Op, Red
 from ..extend import VSpace
 from . import devarray as D
+from . import fusion as _fusion
 from .devarray import DevArray, LazyDevArray
 
 
@@ -142,8 +143,8 @@ class DevArrayVSpace(VSpace):
             # adds in the promoted dtype and stores in x's: a float64 cotangent accumulated into a
             # float32 leaf comes out float32
             return D.astype(self._add(x, y), x.dtype)
-        if x._borrowed or type(x) is not DevArray or is_broadcast_view(x):
-            return self._add(x, y)
+        if x._borrowed or type(x) is not DevArray or is_broadcast_view(x) or _fusion.pending(y):
+            return self._add(x, y)  # (a pending addend: the sum joins its expression instead of forcing it into memory first)
         if isinstance(y, DevArray) and y.shape != x.shape and D.broadcast_shapes(x.shape, y.shape) != x.shape:
             return self._add(x, y)
         return D.map_op(Op.ADD, x.dtype, x, y, out=x)
@@ -162,6 +163,7 @@ DevArrayVSpace.register(LazyDevArray)
 DevArrayVSpace.register(D.PendingProduct)
 DevArrayVSpace.register(D.LseCotangent)
 DevArrayVSpace.register(D.FusedResult)
+DevArrayVSpace.register(_fusion.ExprArray)
 DevArrayVSpace.register(float)
 
 

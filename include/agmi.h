@@ -178,6 +178,34 @@ int agmi_elementwise(int op, int dtype, int ndim, const int64_t *shape,
                      int n_in, const agmi_array *ins, const double *scalars,
                      void *stream);
 
+/* A chain of elementwise rules evaluated in one pass: out[k][idx] = the value the straight-line
+ * program `code` leaves in the register it stores to output k, for every idx of `shape`.
+ * The program runs on a file of n_regs registers (at most AGMI_PROGRAM_MAX_REGISTERS) per point.
+ * When it starts, register i holds leaves[i][idx] (i < n_leaf: strided arrays, stride 0 on
+ * broadcast axes; pending maps are not applied) and register n - 1 - k holds imms[k] converted to
+ * `dtype` (k < n_imm; n = 8 when n_regs <= 8, else 16).  Instruction word:
+ *     op | dst << 8 | a << 12 | b << 16 | c << 20 | d << 24
+ * `op` is any single-result agmi_op: reg[dst] = op(reg[a], reg[b], reg[c], reg[d]) (as many operands
+ * as the op takes, in the order agmi_op lists them), rounded exactly as agmi_elementwise rounds
+ * it, so a program gives bit for bit what the same ops give as separate agmi_elementwise calls;
+ * op AGMI_PROGRAM_STORE writes reg[a] to output b (dst must equal a).  Every register read must
+ * have been written, every output stored, else AGMI_ERR_ARG and nothing is launched.
+ * Layout: after axis merging at most two axes may remain and every operand must have stride 1 or
+ * 0 (leaves only) along the innermost one; anything else returns AGMI_ERR_UNSUPPORTED.  Outputs
+ * may not overlap leaves unless they are the same view (in-place update).
+ * Replaces: the NumPy passes of consecutive elementwise rules of a backward or forward pass
+ * (autograd/numpy/numpy_vjps.py:76-93, 139-143, 157-191; numpy_jvps.py:60-120) together with the
+ * cotangent sums between them (autograd/core.py:185-205). */
+#define AGMI_PROGRAM_MAX_LEAVES 6
+#define AGMI_PROGRAM_MAX_IMMEDIATES 6
+#define AGMI_PROGRAM_MAX_OUTPUTS 4
+#define AGMI_PROGRAM_MAX_INSTRUCTIONS 96
+#define AGMI_PROGRAM_MAX_REGISTERS 16
+#define AGMI_PROGRAM_STORE 255
+int agmi_program(int dtype, int ndim, const int64_t *shape, int n_out, const agmi_array *outs,
+                 int n_leaf, const agmi_array *leaves, int n_imm, const double *imms,
+                 int n_instr, const uint32_t *code, int n_regs, void *stream);
+
 /* out[idx] = (in0[idx] <cmp> in1[idx]) as AGMI_BOOL; inputs as in agmi_elementwise. */
 int agmi_compare(int cmp, int dtype, int ndim, const int64_t *shape,
                  const agmi_array *out, const agmi_array *ins, const double *scalars,

@@ -500,12 +500,19 @@ def test_vspace_axioms(dnp):
     assert abs(float(vs.inner_prod(a, b)) - onp.sum(a.numpy() * b.numpy())) < 1e-12
     basis = list(vs.standard_basis())
     assert len(basis) == 12 and onp.array_equal(onp.sum([e.numpy() for e in basis], axis=0), onp.ones((4, 3)))
-    acc = vs.mut_add(None, a)          # 0 + a: borrows a's memory, never writes it
-    acc2 = vs.mut_add(acc, b)          # first real accumulation goes to fresh memory
-    acc3 = vs.mut_add(acc2, b)         # from then on in place
-    assert acc3 is acc2 and acc2 is not acc
-    assert onp.array_equal(acc.numpy(), a.numpy())
-    assert onp.array_equal(acc3.numpy(), ((0.0 + a.numpy()) + b.numpy()) + b.numpy())
+    from autograd_amd.numpy import fusion
+
+    for fused in (False, True):
+        was, fusion.ENABLED = fusion.ENABLED, fused
+        try:
+            acc = vs.mut_add(None, a)          # 0 + a: borrows a's memory, never writes it
+            acc2 = vs.mut_add(acc, b)          # first real accumulation goes to fresh memory (or stays an expression)
+            acc3 = vs.mut_add(acc2, b)         # from then on in place when the sums are launched one by one
+        finally:
+            fusion.ENABLED = was
+        assert acc2 is not acc and (fused or acc3 is acc2)
+        assert onp.array_equal(acc.numpy(), a.numpy())
+        assert onp.array_equal(acc3.numpy(), ((0.0 + a.numpy()) + b.numpy()) + b.numpy())
     assert vspace(dnp.ones((2,), dtype=F32)).dtype == onp.float32
 
 
