@@ -163,8 +163,8 @@ def lib():
     L.agmi_elementwise.restype = c_i
     L.agmi_elementwise.argtypes = [c_i, c_i, c_i, p_i64, c_i, p_arr, c_i, p_arr, p_d, c_p]
     L.agmi_program.restype = c_i
-    L.agmi_program.argtypes = [c_i, c_i, p_i64, c_i, p_arr, c_i, p_arr, c_i, p_d, c_i, ctypes.POINTER(ctypes.c_uint32), c_i,
-                               c_p]
+    L.agmi_program.argtypes = [c_i, c_i, p_i64, c_i, p_arr, c_i, p_arr, p_i64, c_i, p_d, c_i, p_i64, c_i,
+                               ctypes.POINTER(ctypes.c_uint32), c_i, c_p]
     L.agmi_compare.restype = c_i
     L.agmi_compare.argtypes = [c_i, c_i, c_i, p_i64, p_arr, p_arr, p_d, c_p]
     L.agmi_cast.restype = c_i
@@ -462,32 +462,51 @@ def elementwise(op, code, shape, outs, ins):
 
 PROGRAM_MAX_LEAVES, PROGRAM_MAX_IMMEDIATES, PROGRAM_MAX_OUTPUTS, PROGRAM_MAX_INSTRUCTIONS = 6, 6, 4, 96
 PROGRAM_MAX_REGISTERS = 16
-PROGRAM_STORE = 255
+PROGRAM_MAX_MASKS = 4
+PROGRAM_STORE, PROGRAM_MASK = 255, 254
+_prog_leaf_ranges = (ctypes.c_int64 * (2 * PROGRAM_MAX_LEAVES))()
+_prog_mask_ranges = (ctypes.c_int64 * (2 * PROGRAM_MAX_MASKS))()
 _prog_outs = (AgmiArray * PROGRAM_MAX_OUTPUTS)()
 _prog_leaves = (AgmiArray * PROGRAM_MAX_LEAVES)()
 _prog_imms = (ctypes.c_double * PROGRAM_MAX_IMMEDIATES)()
 _prog_code = (ctypes.c_uint32 * PROGRAM_MAX_INSTRUCTIONS)()
 
 
-def program(code, shape, outs, leaves, imms, words, n_regs):
+def program(code, shape, outs, leaves, imms, words, n_regs, shifted=None, masks=()):
     """Run the elementwise program ``words`` (instruction words of ``agmi_program``) over ``shape``.
 
     ``outs`` are tensors of exactly ``shape``; ``leaves`` tensors expanded to ``shape`` (stride 0 on
-    broadcast axes); ``imms`` Python floats.  Returns False when the layout is outside what the kernel
-    covers (the caller then evaluates the steps one by one)."""
+    broadcast axes); ``imms`` Python floats.  ``shifted`` (one-axis programs): per leaf ``(shift, lo, hi)``, the
+    leaf is read ``shift`` elements further on and only at indices in [lo, hi); ``masks``: the (lo, hi) ranges of
+    the program's mask instructions.  Returns False when the layout is outside what the kernel covers (the
+    caller then evaluates the steps one by one)."""
     nd = _set_shape(shape)
     for k, t in enumerate(outs):
         _set_array(_prog_outs[k], t)
-    for k, t in enumerate(leaves):
-        _set_array(_prog_leaves[k], t)
+    ranges = None
+    if shifted is None:
+        for k, t in enumerate(leaves):
+            _set_array(_prog_leaves[k], t)
+    else:
+        ranges = _prog_leaf_ranges
+        for k, t in enumerate(leaves):
+            slot = _prog_leaves[k]
+            shift, lo, hi = shifted[k]
+            _set_array(slot, t)
+            if shift:
+                slot.data = t.data_ptr() + shift * t.stride(0) * t.element_size()
+            ranges[2 * k], ranges[2 * k + 1] = lo, hi
+    n_mask = len(masks)
+    for k in range(n_mask):
+        _prog_mask_ranges[2 * k], _prog_mask_ranges[2 * k + 1] = masks[k]
     n_imm = len(imms)
     if n_imm:
         _prog_imms[:n_imm] = imms
     n = len(words)
     _prog_code[:n] = words
     ev = _TIMER.begin(("program",)) if _TIMER is not None else None
-    rc = _LIB.agmi_program(code, nd, _shape, len(outs), _prog_outs, len(leaves), _prog_leaves, n_imm, _prog_imms, n,
-                           _prog_code, n_regs, _stream())
+    rc = _LIB.agmi_program(code, nd, _shape, len(outs), _prog_outs, len(leaves), _prog_leaves, ranges, n_imm, _prog_imms,
+                           n_mask, _prog_mask_ranges, n, _prog_code, n_regs, _stream())
     if rc == -2:  # AGMI_ERR_UNSUPPORTED
         return False
     if rc:

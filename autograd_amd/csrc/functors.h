@@ -21,23 +21,23 @@ namespace agmi {
 #ifndef AGMI_HEAVY_MATH
 #define AGMI_HEAVY_MATH __device__ __forceinline__
 #endif
-__device__ __forceinline__ float m_exp(float x) { return expf(x); }
-__device__ __forceinline__ double m_exp(double x) { return exp(x); }
+AGMI_HEAVY_MATH float m_exp(float x) { return expf(x); }
+AGMI_HEAVY_MATH double m_exp(double x) { return exp(x); }
 // exp(d) for d <= 0 (an element minus the logsumexp of its row) to within 1 ulp of expf, without the
 // overflow handling: d*log2(e) is split into an integer n and a remainder whose rounding error is
 // recovered with fused multiply-adds (log2(e) as a float pair), the hardware exp2 sees |r| <= 1/2,
 // and ldexp scales, also into the subnormals.  n is clamped so that d = -inf (and anything whose exp
 // underflows) arrives at exp2(-inf) = 0; a NaN passes through the clamp's other operand into the fma.
-__device__ __forceinline__ float exp_of_nonpositive(float d) {
+AGMI_HEAVY_MATH float exp_of_nonpositive(float d) {
     const float kLog2eHi = 1.44269502162933349609375f, kLog2eLo = 1.92596299112661746e-8f;
     const float n = fmaxf(rintf(d * kLog2eHi), -160.0f);
     float r = __builtin_fmaf(d, kLog2eHi, -n);
     r = __builtin_fmaf(d, kLog2eLo, r);
     return ldexpf(__builtin_amdgcn_exp2f(r), static_cast<int>(n));
 }
-__device__ __forceinline__ double exp_of_nonpositive(double d) { return exp(d); }
-__device__ __forceinline__ float m_log(float x) { return logf(x); }
-__device__ __forceinline__ double m_log(double x) { return log(x); }
+AGMI_HEAVY_MATH double exp_of_nonpositive(double d) { return exp(d); }
+AGMI_HEAVY_MATH float m_log(float x) { return logf(x); }
+AGMI_HEAVY_MATH double m_log(double x) { return log(x); }
 AGMI_HEAVY_MATH float m_log1p(float x) { return log1pf(x); }
 AGMI_HEAVY_MATH double m_log1p(double x) { return log1p(x); }
 AGMI_HEAVY_MATH float m_expm1(float x) { return expm1f(x); }
@@ -61,10 +61,10 @@ AGMI_HEAVY_MATH double m_pow(double x, double y) { return pow(x, y); }
 
 AGMI_HEAVY_MATH float m_exp2(float x) { return exp2f(x); }
 AGMI_HEAVY_MATH double m_exp2(double x) { return exp2(x); }
-__device__ __forceinline__ float m_log2(float x) { return log2f(x); }
-__device__ __forceinline__ double m_log2(double x) { return log2(x); }
-__device__ __forceinline__ float m_log10(float x) { return log10f(x); }
-__device__ __forceinline__ double m_log10(double x) { return log10(x); }
+AGMI_HEAVY_MATH float m_log2(float x) { return log2f(x); }
+AGMI_HEAVY_MATH double m_log2(double x) { return log2(x); }
+AGMI_HEAVY_MATH float m_log10(float x) { return log10f(x); }
+AGMI_HEAVY_MATH double m_log10(double x) { return log10(x); }
 AGMI_HEAVY_MATH float m_tan(float x) { return tanf(x); }
 AGMI_HEAVY_MATH double m_tan(double x) { return tan(x); }
 AGMI_HEAVY_MATH float m_asin(float x) { return asinf(x); }

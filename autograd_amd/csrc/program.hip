@@ -19,11 +19,11 @@
 // Index space: (rows, cols) after axis merging, every leaf with column stride 1 or 0 (flat arrays
 // are one row).  Registers 0 .. n_leaf-1 hold the leaves when the program starts, registers
 // NREG-1, NREG-2, ... the immediates.
+#include <algorithm>
 #include <type_traits>
 
 #include "common.h"
 
-#define AGMI_HEAVY_MATH static __device__ __noinline__
 #include "functors.h"
 
 namespace agmi {
@@ -32,6 +32,7 @@ constexpr int kProgMaxLeaf = AGMI_PROGRAM_MAX_LEAVES;
 constexpr int kProgMaxImm = AGMI_PROGRAM_MAX_IMMEDIATES;
 constexpr int kProgMaxOut = AGMI_PROGRAM_MAX_OUTPUTS;
 constexpr int kProgMaxInstr = AGMI_PROGRAM_MAX_INSTRUCTIONS;
+constexpr int kProgMaxMask = AGMI_PROGRAM_MAX_MASKS;
 
 struct ProgParams {
     int64_t cols;
@@ -41,6 +42,10 @@ struct ProgParams {
     const void *leaf[kProgMaxLeaf];
     int64_t leaf_rs[kProgMaxLeaf];
     int32_t leaf_cs[kProgMaxLeaf];  // 0 or 1
+    // columns a leaf may be read at (one-row programs whose leaves are read at shifted positions); all columns otherwise
+    int64_t leaf_lo[kProgMaxLeaf], leaf_hi[kProgMaxLeaf];
+    int64_t safe_lo, safe_hi;  // the columns every leaf may be read at
+    int64_t mask_lo[kProgMaxMask], mask_hi[kProgMaxMask];
     void *out[kProgMaxOut];
     int64_t out_rs[kProgMaxOut];
     double imm[kProgMaxImm];
@@ -52,10 +57,96 @@ struct RegVec {
     typedef T type __attribute__((ext_vector_type(NREG)));
 };
 
+// Operations of a few instructions are expanded in place; every other functor is ONE function that the
+// interpreter calls element by element, so that the temporaries and constants of the long routines (exp, pow,
+// the trigonometric family) live in the callee's registers for the length of a call instead of adding to what
+// the kernel holds for its whole run: the register file of the program and the waves a SIMD keeps resident
+// depend on that.
+constexpr bool is_short_op(int op) {
+    switch (op) {
+        case AGMI_OP_COPY: case AGMI_OP_NEG: case AGMI_OP_SQUARE: case AGMI_OP_ABS:
+        case AGMI_OP_RECIPROCAL: case AGMI_OP_ADD: case AGMI_OP_SUB: case AGMI_OP_MUL: case AGMI_OP_DIV:
+        case AGMI_OP_MAXIMUM: case AGMI_OP_MINIMUM: case AGMI_OP_FMAX: case AGMI_OP_FMIN: case AGMI_OP_WHERE:
+        case AGMI_OP_DIV_VJP1: case AGMI_OP_RECIPROCAL_VJP: case AGMI_OP_SQUARE_VJP: case AGMI_OP_ABS_VJP:
+        case AGMI_OP_LOG1P_VJP: case AGMI_OP_EXPM1_VJP: case AGMI_OP_MUL_ADD: case AGMI_OP_EQUAL_AS_FLOAT:
+        case AGMI_OP_CHOOSE_VJP: case AGMI_OP_EXTREMUM_VJP: case AGMI_OP_FLOOR: case AGMI_OP_CEIL:
+        case AGMI_OP_RINT: case AGMI_OP_TRUNC:
+            return true;
+        default:
+            return false;
+    }
+}
+
+// The operations most chains are made of.  A program that uses nothing else runs on a kernel whose dispatch
+// holds only these (a shallower compare tree per instruction, fewer registers, exp / log / sqrt expanded in place).
+#define AGMI_FOR_EACH_LIGHT_OP(X)            \
+    X(AGMI_OP_COPY, FCopy)                   \
+    X(AGMI_OP_NEG, FNeg)                     \
+    X(AGMI_OP_EXP, FExp)                     \
+    X(AGMI_OP_LOG, FLog)                     \
+    X(AGMI_OP_SQRT, FSqrt)                   \
+    X(AGMI_OP_SQUARE, FSquare)               \
+    X(AGMI_OP_RECIPROCAL, FReciprocal)       \
+    X(AGMI_OP_TANH, FTanh)                   \
+    X(AGMI_OP_ADD, FAdd)                     \
+    X(AGMI_OP_SUB, FSub)                     \
+    X(AGMI_OP_MUL, FMul)                     \
+    X(AGMI_OP_DIV, FDiv)                     \
+    X(AGMI_OP_DIV_VJP1, FDivVjp1)            \
+    X(AGMI_OP_TANH_VJP, FTanhVjp)            \
+    X(AGMI_OP_MUL_ADD, FMulAdd)
+
+constexpr bool is_light_op(int op) {
+#define AGMI_LIGHT_CASE(OP, FN) case OP:
+    switch (op) {
+        AGMI_FOR_EACH_LIGHT_OP(AGMI_LIGHT_CASE)
+        case AGMI_PROGRAM_STORE:
+        case AGMI_PROGRAM_MASK:
+            return true;
+        default:
+            return false;
+    }
+#undef AGMI_LIGHT_CASE
+}
+
+// expanded in place by the light kernel (the full kernel calls them)
+constexpr bool is_light_inline_op(int op) {
+    return op == AGMI_OP_EXP || op == AGMI_OP_LOG || op == AGMI_OP_SQRT;
+}
+
+template <class Fn, typename T>
+static __device__ __noinline__ T apply_called(T a, T b, T c, T d) {
+    const T xi[4] = {a, b, c, d};
+    T oi[1];
+    Fn::apply(xi, oi);
+    return oi[0];
+}
+
+template <class Fn, typename T, bool SHORT>
+__device__ __forceinline__ T apply_one(const T (&xi)[4]) {
+    if constexpr (SHORT) {
+        T oi[1];
+        Fn::apply(xi, oi);
+        return oi[0];
+    } else {
+        return apply_called<Fn, T>(xi[0], Fn::NIN > 1 ? xi[1] : T(0), Fn::NIN > 2 ? xi[2] : T(0), Fn::NIN > 3 ? xi[3] : T(0));
+    }
+}
+
+// The last, partly filled vector of a row.  A function of its own: its per-lane branches would otherwise make
+// the compiler restructure the whole interpreter loop around them (every wave-uniform branch of the dispatch
+// would then cost several scalar instructions more).
+template <typename T, int VL>
+static __device__ __noinline__ void store_partial(T *base, int64_t c, int64_t cols, T __attribute__((ext_vector_type(VL))) v) {
+#pragma unroll
+    for (int j = 0; j < VL; ++j)
+        if (c + j < cols) base[c + j] = v[j];
+}
+
 // op | dst << 8 | a << 12 | b << 16 | c << 20 | d << 24
 __device__ __forceinline__ int field(uint32_t w, int shift, int mask) { return static_cast<int>(w >> shift) & mask; }
 
-template <typename T, int NREG, int U>
+template <typename T, int NREG, int U, bool LIGHT>
 __global__ __launch_bounds__(kBlock) void ew_program(const ProgParams p) {
     constexpr int VL = 16 / sizeof(T);
     constexpr int V = VL * U;
@@ -93,7 +184,9 @@ __global__ __launch_bounds__(kBlock) void ew_program(const ProgParams p) {
         // the tile's leaves go straight into the register file
         const uint32_t cur_row = row, cur_chunk = chunk;
         const int64_t c0 = static_cast<int64_t>(cur_chunk) * TW + lane * VL;
-        const bool interior = (static_cast<int64_t>(cur_chunk) + 1) * TW <= cols;
+        const int64_t tile_begin = static_cast<int64_t>(cur_chunk) * TW;
+        const bool interior = tile_begin + TW <= cols;
+        const bool readable = interior && tile_begin >= p.safe_lo && tile_begin + TW <= p.safe_hi;
         {
             vec_t L[kProgMaxLeaf][U];
 #pragma unroll
@@ -106,7 +199,7 @@ __global__ __launch_bounds__(kBlock) void ew_program(const ProgParams p) {
                         for (int u = 0; u < U; ++u)
 #pragma unroll
                             for (int j = 0; j < VL; ++j) L[k][u][j] = s;
-                    } else if (interior) {
+                    } else if (readable) {
 #pragma unroll
                         for (int u = 0; u < U; ++u)
                             L[k][u] = __builtin_nontemporal_load(reinterpret_cast<const vec_t *>(base + c0 + u * (64 * VL)));
@@ -116,7 +209,7 @@ __global__ __launch_bounds__(kBlock) void ew_program(const ProgParams p) {
 #pragma unroll
                             for (int j = 0; j < VL; ++j) {
                                 const int64_t c = c0 + u * (64 * VL) + j;
-                                L[k][u][j] = c < cols ? base[c] : T(1);
+                                L[k][u][j] = (c < cols && c >= p.leaf_lo[k] && c < p.leaf_hi[k]) ? base[c] : T(1);
                             }
                     }
                 }
@@ -155,7 +248,7 @@ __global__ __launch_bounds__(kBlock) void ew_program(const ProgParams p) {
 #pragma unroll
                     for (int u = 0; u < U; ++u) {
                         const int64_t c = n0 + u * (64 * VL);
-                        if (c < cols) touched[k] = base[c];
+                        if (c < cols && c >= p.leaf_lo[k] && c < p.leaf_hi[k]) touched[k] = base[c];
                     }
                 }
             }
@@ -173,15 +266,12 @@ __global__ __launch_bounds__(kBlock) void ew_program(const ProgParams p) {
             for (int j = 0; j < V; ++j) x[0][j] = r[j][a];
 #pragma unroll
             for (int j = 0; j < V; ++j) x[1][j] = r[j][b];
-#define AGMI_PROG_APPLY(FN)                                   \
-    {                                                         \
-        _Pragma("unroll") for (int j = 0; j < V; ++j) {       \
-            T xi[4] = {x[0][j], x[1][j], x[2][j], x[3][j]};   \
-            T oi[1];                                          \
-            FN<T>::apply(xi, oi);                             \
-            o[j] = oi[0];                                     \
-            __builtin_amdgcn_sched_barrier(0);                \
-        }                                                     \
+#define AGMI_PROG_APPLY(OP, FN)                                               \
+    {                                                                         \
+        _Pragma("unroll") for (int j = 0; j < V; ++j) {                       \
+            T xi[4] = {x[0][j], x[1][j], x[2][j], x[3][j]};                   \
+            o[j] = apply_one<FN<T>, T, is_short_op(OP) || (LIGHT && is_light_inline_op(OP))>(xi); \
+        }                                                                     \
     }
 #define AGMI_PROG_CASE(OP, FN)                                                        \
     case OP: {                                                                        \
@@ -191,37 +281,47 @@ __global__ __launch_bounds__(kBlock) void ew_program(const ProgParams p) {
         if (FN<T>::NIN >= 4) {                                                        \
             _Pragma("unroll") for (int j = 0; j < V; ++j) x[3][j] = r[j][d];          \
         }                                                                             \
-        AGMI_PROG_APPLY(FN)                                                           \
+        AGMI_PROG_APPLY(OP, FN)                                                       \
         break;                                                                        \
     }
-            switch (op) {
-                AGMI_FOR_EACH_PROGRAM_OP(AGMI_PROG_CASE)
-                case AGMI_PROGRAM_STORE: {
-                    T *base = static_cast<T *>(p.out[b]) + static_cast<int64_t>(cur_row) * p.out_rs[b];
-                    if (interior) {
-#pragma unroll
-                        for (int u = 0; u < U; ++u) {
-                            vec_t v;
-#pragma unroll
-                            for (int j = 0; j < VL; ++j) v[j] = x[0][u * VL + j];
-                            *reinterpret_cast<vec_t *>(base + c0 + u * (64 * VL)) = v;
-                        }
-                    } else {
-#pragma unroll
-                        for (int u = 0; u < U; ++u)
-#pragma unroll
-                            for (int j = 0; j < VL; ++j) {
-                                const int64_t cc = c0 + u * (64 * VL) + j;
-                                if (cc < cols) base[cc] = x[0][u * VL + j];
-                            }
-                    }
+#define AGMI_PROG_STORE_AND_DEFAULT                                                                        \
+    case AGMI_PROGRAM_MASK: {                                                                             \
+        const int64_t lo = p.mask_lo[b & (kProgMaxMask - 1)], hi = p.mask_hi[b & (kProgMaxMask - 1)];     \
+        _Pragma("unroll") for (int j = 0; j < V; ++j) x[2][j] = r[j][c];                                  \
+        _Pragma("unroll") for (int u = 0; u < U; ++u)                                                     \
+            _Pragma("unroll") for (int j = 0; j < VL; ++j) {                                              \
+                const int64_t cc = c0 + u * (64 * VL) + j;                                                \
+                o[u * VL + j] = (cc >= lo && cc < hi) ? x[0][u * VL + j] : x[2][u * VL + j];              \
+            }                                                                                             \
+        break;                                                                                            \
+    }                                                                                                     \
+    case AGMI_PROGRAM_STORE: {                                                                            \
+        T *base = static_cast<T *>(p.out[b]) + static_cast<int64_t>(cur_row) * p.out_rs[b];               \
+        _Pragma("unroll") for (int u = 0; u < U; ++u) {                                                   \
+            vec_t v;                                                                                      \
+            _Pragma("unroll") for (int j = 0; j < VL; ++j) v[j] = x[0][u * VL + j];                       \
+            if (interior)                                                                                 \
+                *reinterpret_cast<vec_t *>(base + c0 + u * (64 * VL)) = v;                                \
+            else                                                                                          \
+                store_partial<T, VL>(base, c0 + u * (64 * VL), cols, v);                                  \
+        }                                                                                                 \
+    }                                                                                                     \
+        [[fallthrough]];                                                                                  \
+    default:                                                                                              \
+        _Pragma("unroll") for (int j = 0; j < V; ++j) o[j] = x[0][j];                                     \
+        break;
+            if constexpr (LIGHT) {
+                switch (op) {
+                    AGMI_FOR_EACH_LIGHT_OP(AGMI_PROG_CASE)
+                    AGMI_PROG_STORE_AND_DEFAULT
                 }
-                    [[fallthrough]];
-                default:
-#pragma unroll
-                    for (int j = 0; j < V; ++j) o[j] = x[0][j];
-                    break;
+            } else {
+                switch (op) {
+                    AGMI_FOR_EACH_PROGRAM_OP(AGMI_PROG_CASE)
+                    AGMI_PROG_STORE_AND_DEFAULT
+                }
             }
+#undef AGMI_PROG_STORE_AND_DEFAULT
 #undef AGMI_PROG_CASE
 #undef AGMI_PROG_APPLY
 #pragma unroll
@@ -244,7 +344,7 @@ static int op_arity(int op) {
 #undef AGMI_ARITY_CASE
 }
 
-template <typename T, int NREG, int U>
+template <typename T, int NREG, int U, bool LIGHT>
 static int launch_program(const ProgParams &p0, int64_t rows, hipStream_t s) {
     ProgParams p = p0;
     constexpr int V = (16 / sizeof(T)) * U;
@@ -264,7 +364,7 @@ static int launch_program(const ProgParams &p0, int64_t rows, hipStream_t s) {
     p.n_tiles = static_cast<uint32_t>(n_tiles);
     p.step_rows = static_cast<uint32_t>(n_waves / tpr);
     p.step_chunks = static_cast<uint32_t>(n_waves % tpr);
-    hipLaunchKernelGGL((ew_program<T, NREG, U>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p);
+    hipLaunchKernelGGL((ew_program<T, NREG, U, LIGHT>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p);
     return hip_check(hipGetLastError(), "program launch");
 }
 
@@ -272,15 +372,22 @@ static int launch_program(const ProgParams &p0, int64_t rows, hipStream_t s) {
 #ifndef AGMI_PART
 #error "compile with -DAGMI_PART=32 or -DAGMI_PART=64"
 #endif
-int program_part_f32(int nreg, const ProgParams &p, int64_t rows, hipStream_t s);
-int program_part_f64(int nreg, const ProgParams &p, int64_t rows, hipStream_t s);
+int program_part_f32(int nreg, bool light, const ProgParams &p, int64_t rows, hipStream_t s);
+int program_part_f64(int nreg, bool light, const ProgParams &p, int64_t rows, hipStream_t s);
+// Two vectors per lane in every variant (measured on the 4M-element float64 tanh-gradient chain: 40 us against 42 with one;
+// the scalar unit's decode work per instruction is shared by twice the elements, which outweighs the lost occupancy).
+template <typename T>
+static int launch_variant(int nreg, bool light, const ProgParams &p, int64_t rows, hipStream_t s) {
+    if (light) return nreg == 8 ? launch_program<T, 8, 2, true>(p, rows, s) : launch_program<T, 16, 2, true>(p, rows, s);
+    return nreg == 8 ? launch_program<T, 8, 2, false>(p, rows, s) : launch_program<T, 16, 2, false>(p, rows, s);
+}
 #if AGMI_PART == 32
-int program_part_f32(int nreg, const ProgParams &p, int64_t rows, hipStream_t s) {
-    return nreg == 8 ? launch_program<float, 8, 2>(p, rows, s) : launch_program<float, 16, 2>(p, rows, s);
+int program_part_f32(int nreg, bool light, const ProgParams &p, int64_t rows, hipStream_t s) {
+    return launch_variant<float>(16, light, p, rows, s);
 }
 #else
-int program_part_f64(int nreg, const ProgParams &p, int64_t rows, hipStream_t s) {
-    return nreg == 8 ? launch_program<double, 8, 2>(p, rows, s) : launch_program<double, 16, 2>(p, rows, s);
+int program_part_f64(int nreg, bool light, const ProgParams &p, int64_t rows, hipStream_t s) {
+    return launch_variant<double>(nreg, light, p, rows, s);
 }
 #endif
 
@@ -290,10 +397,12 @@ using namespace agmi;
 
 #if AGMI_PART == 32
 extern "C" int agmi_program(int dtype, int ndim, const int64_t *shape, int n_out, const agmi_array *outs, int n_leaf,
-                            const agmi_array *leaves, int n_imm, const double *imms, int n_instr, const uint32_t *code,
-                            int n_regs, void *stream) {
+                            const agmi_array *leaves, const int64_t *leaf_ranges, int n_imm, const double *imms,
+                            int n_mask, const int64_t *mask_ranges, int n_instr, const uint32_t *code, int n_regs,
+                            void *stream) {
     if (n_out < 1 || n_out > kProgMaxOut || n_leaf < 0 || n_leaf > kProgMaxLeaf || n_imm < 0 || n_imm > kProgMaxImm ||
-        n_instr < 1 || n_instr > kProgMaxInstr || !outs || (n_leaf && !leaves) || (n_imm && !imms) || !code) {
+        n_instr < 1 || n_instr > kProgMaxInstr || n_mask < 0 || n_mask > kProgMaxMask || !outs || (n_leaf && !leaves) ||
+        (n_imm && !imms) || (n_mask && !mask_ranges) || !code) {
         set_error("program: bad counts (outputs %d, leaves %d, immediates %d, instructions %d) or null arrays", n_out,
                   n_leaf, n_imm, n_instr);
         return AGMI_ERR_ARG;
@@ -302,7 +411,7 @@ extern "C" int agmi_program(int dtype, int ndim, const int64_t *shape, int n_out
         set_error("program: dtype %d is not a floating type", dtype);
         return AGMI_ERR_ARG;
     }
-    const int nreg = n_regs <= 8 ? 8 : 16;
+    const int nreg = (n_regs <= 8 && dtype == AGMI_F64) ? 8 : 16;
     if (n_regs < 1 || n_regs > 16 || n_leaf + n_imm > nreg) {
         set_error("program: %d registers asked for (at most 16), %d leaves and %d immediates", n_regs, n_leaf, n_imm);
         return AGMI_ERR_ARG;
@@ -312,13 +421,25 @@ extern "C" int agmi_program(int dtype, int ndim, const int64_t *shape, int n_out
     for (int k = 0; k < n_leaf; ++k) defined |= 1u << k;
     for (int k = 0; k < n_imm; ++k) defined |= 1u << (nreg - 1 - k);
     uint32_t stored = 0;
+    bool light = true;
     for (int i = 0; i < n_instr; ++i) {
         const uint32_t w = code[i];
         const int op = w & 0xff, dst = (w >> 8) & 15;
+        light = light && is_light_op(op);
         const int src[4] = {int(w >> 12) & 15, int(w >> 16) & 15, int(w >> 20) & 15, int(w >> 24) & 15};
         if (w >> 28) {
             set_error("program: instruction %d has bits set above its fields", i);
             return AGMI_ERR_ARG;
+        }
+        if (op == AGMI_PROGRAM_MASK) {
+            if (src[0] >= nreg || !(defined >> src[0] & 1u) || src[2] >= nreg || !(defined >> src[2] & 1u) ||
+                src[1] >= n_mask || dst >= nreg) {
+                set_error("program: instruction %d selects between registers %d and %d by range %d of %d", i, src[0],
+                          src[2], src[1], n_mask);
+                return AGMI_ERR_ARG;
+            }
+            defined |= 1u << dst;
+            continue;
         }
         if (op == AGMI_PROGRAM_STORE) {
             if (src[0] >= nreg || !(defined >> src[0] & 1u) || src[1] >= n_out || dst != src[0]) {
@@ -397,6 +518,33 @@ extern "C" int agmi_program(int dtype, int ndim, const int64_t *shape, int n_out
         p.leaf_cs[k] = static_cast<int32_t>(cs);
         p.leaf_rs[k] = m.ndim == 2 ? m.stride[n_out + k][0] : 0;
     }
+    // Shifted reads: a leaf of a one-row program may come with the columns [lo, hi) at which its address is
+    // readable (its pointer is already moved by the shift, so columns outside would fall before or behind its
+    // storage); such columns read as 1 and the program masks them.  No range: every column.
+    p.safe_lo = 0;
+    p.safe_hi = p.cols;
+    for (int k = 0; k < n_leaf; ++k) {
+        p.leaf_lo[k] = 0;
+        p.leaf_hi[k] = p.cols;
+        if (leaf_ranges && p.leaf_cs[k] != 0) {
+            if (rows != 1) {
+                set_error("program: leaf ranges need a one-row index space");
+                return AGMI_ERR_UNSUPPORTED;
+            }
+            p.leaf_lo[k] = std::max<int64_t>(leaf_ranges[2 * k], 0);
+            p.leaf_hi[k] = std::min<int64_t>(leaf_ranges[2 * k + 1], p.cols);
+        }
+        p.safe_lo = std::max(p.safe_lo, p.leaf_lo[k]);
+        p.safe_hi = std::min(p.safe_hi, p.leaf_hi[k]);
+    }
+    for (int k = 0; k < n_mask; ++k) {
+        p.mask_lo[k] = mask_ranges[2 * k];
+        p.mask_hi[k] = mask_ranges[2 * k + 1];
+    }
+    if (n_mask && rows != 1) {
+        set_error("program: masks need a one-row index space");
+        return AGMI_ERR_UNSUPPORTED;
+    }
     p.n_leaf = n_leaf;
     p.n_imm = n_imm;
     p.n_instr = n_instr;
@@ -404,7 +552,7 @@ extern "C" int agmi_program(int dtype, int ndim, const int64_t *shape, int n_out
     for (int i = 0; i < n_instr; ++i) p.code[i] = code[i];
     p.code[n_instr] = 0;
     hipStream_t s = as_stream(stream);
-    set_kernel_name("ew_program<%s,%d>[%d]", dtype == AGMI_F32 ? "float" : "double", nreg, n_instr);
-    return dtype == AGMI_F32 ? program_part_f32(nreg, p, rows, s) : program_part_f64(nreg, p, rows, s);
+    set_kernel_name("ew_program<%s,%d,%s>[%d]", dtype == AGMI_F32 ? "float" : "double", nreg, light ? "light" : "full", n_instr);
+    return dtype == AGMI_F32 ? program_part_f32(nreg, light, p, rows, s) : program_part_f64(nreg, light, p, rows, s);
 }
 #endif  // AGMI_PART == 32

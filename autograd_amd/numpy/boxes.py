@@ -9,7 +9,7 @@ primitives (and therefore the same kernels).
 
 from ..extend import Box, primitive
 from . import wrapper as anp
-from .devarray import DevArray, FusedResult, LazyDevArray, LseCotangent, PendingProduct
+from .devarray import DevArray, FusedResult, LazyDevArray, LseCotangent, PendingProduct, PendingReduce
 from .fusion import ExprArray
 
 
@@ -109,6 +109,7 @@ DevArrayBox.register(PendingProduct)
 DevArrayBox.register(LseCotangent)
 DevArrayBox.register(FusedResult)
 DevArrayBox.register(ExprArray)
+DevArrayBox.register(PendingReduce)
 DevArrayBox.register(float)
 
 

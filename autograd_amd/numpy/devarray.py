@@ -730,6 +730,7 @@ def ones(shape, dtype=_F64):
 
 
 _CONSTANTS = {}
+KNOWN_SCALARS = {}  # data pointer of a one-element array that is never written -> its value (shared zeros / ones / constants)
 
 
 def constant(shape, value, dtype):
@@ -750,6 +751,7 @@ def constant(shape, value, dtype):
         if len(_CONSTANTS) > 64:
             return full(shape, value, dtype)
         one = _CONSTANTS[key] = full((), float(value), dtype)._t
+        KNOWN_SCALARS[one.data_ptr()] = float(value)
     return LazyDevArray(one.expand(shape), dtype, 1.0, None)
 
 
@@ -1005,8 +1007,87 @@ def reduce_shape(shape, axes, keepdims):
 _IDENTITY = {Red.SUM: 0.0, Red.PROD: 1.0}
 
 
+class PendingReduce(DevArray):
+    """A reduction of pending elementwise expressions, not yet run: the forward value of a traced ``sum`` is often
+    never read (``grad`` keeps the cotangents only), and running it would force its operand expression into memory
+    first.  Reading ``_t`` runs it."""
+
+    __slots__ = ("_call", "_shape")
+
+    def __init__(self, call, shape, dtype):
+        self._call, self._shape = call, shape
+        self.dtype = dtype
+        self._borrowed = False
+        self._shape_tuple = shape
+
+    def __getattr__(self, name):
+        if name != "_t":
+            raise AttributeError(name)
+        self._t = out = _map_reduce_now(*self._call)._t
+        self._call = None
+        return out
+
+    @property
+    def shape(self):
+        return self._shape
+
+    @property
+    def ndim(self):
+        return len(self._shape)
+
+    @property
+    def size(self):
+        n = 1
+        for s in self._shape:
+            n *= s
+        return n
+
+    @property
+    def strides(self):
+        return DevArray(self._t, self.dtype).strides
+
+    def __len__(self):
+        if not self._shape:
+            raise TypeError("len() of unsized object")
+        return self._shape[0]
+
+    def __iter__(self):
+        return (self[i] for i in range(len(self)))
+
+    def _h(self):
+        return self._t
+
+    def _settled(self):
+        return DevArray(self._t, self.dtype)
+
+    def _view(self, fn):
+        return DevArray(fn(self._t), self.dtype)
+
+
+_DEFERRED = _DEFERRED + (PendingReduce,)
+
+
 def map_reduce(op, red, dtype, xs, axes, keepdims, shape=None):
-    """``RED_axes op(xs...)`` with ``xs`` broadcast to ``shape`` (default: their broadcast)."""
+    """``RED_axes op(xs...)`` with ``xs`` broadcast to ``shape`` (default: their broadcast); left pending while an
+    operand is a pending expression (see :class:`PendingReduce`)."""
+    if _fusion is not None and _fusion.ENABLED:
+        for x in xs:
+            if type(x) is _fusion.ExprArray and x._args is not None:
+                full = shape
+                if full is None:
+                    full = ()
+                    for y in xs:
+                        if isinstance(y, DevArray) and y.shape != full:
+                            full = broadcast_shapes(full, y.shape)
+                for y in xs:
+                    if isinstance(y, DevArray):
+                        y._borrowed = True
+                axes = tuple(axes)
+                return PendingReduce((op, red, dtype, tuple(xs), axes, keepdims, shape), reduce_shape(full, axes, keepdims), dtype)
+    return _map_reduce_now(op, red, dtype, xs, axes, keepdims, shape)
+
+
+def _map_reduce_now(op, red, dtype, xs, axes, keepdims, shape=None):
     ops = _limit_aux(tuple(_operand(x, dtype) for x in xs), dtype)
     if shape is None:
         shape = _bshape(ops)
@@ -1034,7 +1115,7 @@ def map_reduce(op, red, dtype, xs, axes, keepdims, shape=None):
             # broadcast operands of pending maps can keep reduced axes from merging: write those out, retry
             settled = [LazyDevArray(t.t, dtype, t.scale, t.shift, t.ascale)._settled() if type(t) is _lib.Affine
                        else _rewrap(t, dtype) for t in ops]
-            return map_reduce(op, red, dtype, settled, axes, keepdims, shape=shape)
+            return _map_reduce_now(op, red, dtype, settled, axes, keepdims, shape=shape)
         # reduced axes interleaved with kept ones: one group of adjacent axes at a time
         if red == Red.LOGSUMEXP:
             raise NotImplementedError("logsumexp over non-adjacent axes of a non-contiguous layout")
@@ -1043,7 +1124,7 @@ def map_reduce(op, red, dtype, xs, axes, keepdims, shape=None):
         else:
             cur = map_op(op, dtype, *[_rewrap(t, dtype) for t in ops])
         for group in _adjacent_groups(axes):
-            cur = map_reduce(Op.COPY, red, dtype, (cur,), group, True)
+            cur = _map_reduce_now(Op.COPY, red, dtype, (cur,), group, True)
         out_t = cur._t
     out = DevArray(out_t, dtype)
     if not keepdims and axes:

@@ -31,7 +31,7 @@ from . import devarray as D
 from .devarray import DevArray, LazyDevArray
 
 ENABLED = os.environ.get("AUTOGRAD_AMD_FUSE", "1").strip() not in ("0", "")
-MAX_CONE = 64  # pending nodes under one value before its largest pending operand is written out
+MAX_CONE = 192  # pending nodes under one value before its largest pending operand is written out
 
 _F32 = onp.dtype("float32")
 
@@ -57,7 +57,7 @@ class ExprArray(DevArray):
     affine map) of this node's dtype whose shapes broadcast to this node's, and Python floats.
     Reading ``_t`` evaluates the node together with every pending node under it."""
 
-    __slots__ = ("_op", "_args", "_shape", "_out", "_cone")
+    __slots__ = ("_op", "_args", "_shape", "_out", "_cone", "_lo")
 
     def __init__(self, op, args, shape, dtype, cone):
         self._op, self._args, self._shape = op, args, shape
@@ -224,7 +224,7 @@ def _finish(node):
 
 def _run(roots):
     order = _post_order(roots)
-    if len(order) == 1:
+    if len(order) == 1 and order[0]._op != SHIFT:
         _single(order[0])
         return
     if len(roots) > _lib.PROGRAM_MAX_OUTPUTS:
@@ -232,7 +232,10 @@ def _run(roots):
         _run(roots[:half])
         _run([r for r in roots[half:] if r._args is not None])
         return
-    program = _emit(order, roots)
+    try:
+        program = _emit(roots)
+    except _Unsupported:
+        program = False
     if program is None:
         # too long, too many leaves or too many live values for one program: write a node from the middle of the
         # order out first (everything it needs comes before it), then try again with that node as a leaf
@@ -241,20 +244,29 @@ def _run(roots):
             _run(roots[:half])
             _run([r for r in roots[half:] if r._args is not None])
             return
-        _run([order[(len(order) - 1) // 2]])
-        _run(roots)
-        return
-    leaves, imms, words, n_regs = program
-    root = roots[0]
-    shape, dtype = root._shape, root.dtype
-    outs = tuple(r._buffer() for r in roots)
-    leaves = tuple(t if tuple(t.shape) == shape else t.expand(shape) for t in leaves)
-    if _lib.program(_lib.DTYPE_CODE[dtype], shape, outs, leaves, imms, words, n_regs):
-        COUNTS["programs"] += 1
-        COUNTS["instructions"] += len(words)
-        for r in roots:
-            _finish(r)
-        return
+        if len(order) > 1:
+            # the node whose own expression is closest to half of this one
+            half, pick = len(order) / 2.0, order[0]
+            for node in order[:-1]:
+                if abs(min(node._cone, len(order)) - half) < abs(min(pick._cone, len(order)) - half):
+                    pick = node
+            _run([pick])
+            _run(roots)
+            return
+        program = False
+    if program is not False:
+        leaves, imms, words, n_regs, shifted, masks = program
+        root = roots[0]
+        shape, dtype = root._shape, root.dtype
+        outs = tuple(r._buffer() for r in roots)
+        if shifted is None:
+            leaves = tuple(t if tuple(t.shape) == shape else t.expand(shape) for t in leaves)
+        if _lib.program(_lib.DTYPE_CODE[dtype], shape, outs, leaves, imms, words, n_regs, shifted, masks):
+            COUNTS["programs"] += 1
+            COUNTS["instructions"] += len(words)
+            for r in roots:
+                _finish(r)
+            return
     # a layout the program kernel does not cover (more than two axes left after merging, a strided innermost
     # axis): the steps run one by one
     COUNTS["unfused"] += 1
@@ -264,8 +276,11 @@ def _run(roots):
 
 
 def _single(node):
-    """One node by the ordinary elementwise kernel (its operands are computed first)."""
+    """One node by the ordinary kernels (its operands are computed first)."""
     dtype = node.dtype
+    if node._op == SHIFT:
+        _single_shift(node)
+        return
     ops = D._limit_aux(tuple(D._operand(a, dtype) for a in node._args), dtype)
     shape = node._shape
     ops = tuple(D._expand(t, shape) for t in ops)
@@ -274,35 +289,89 @@ def _single(node):
     _finish(node)
 
 
+def _single_shift(node):
+    """A shifted vector by the ordinary kernels: zeros outside, one copy inside."""
+    dtype = node.dtype
+    code = _lib.DTYPE_CODE[dtype]
+    src = D._operand(D.plain(node._args[0]), dtype)
+    if type(src) is _lib.Affine:
+        src = LazyDevArray(src.t, dtype, src.scale, src.shift, src.ascale)._t
+    out = node._buffer()
+    n, m, lo = node._shape[0], src.shape[0], node._lo
+    begin, end = max(lo, 0), min(lo + m, n)
+    end = max(end, begin)
+    outside = node._args[1]
+    if outside is not None:
+        rest = D.plain(outside)._t
+    for at, part in ((0, out[:begin]), (end, out[end:])):
+        if part.numel():
+            if outside is None:
+                _lib.fill(code, part, 0.0)
+            else:
+                _lib.elementwise(Op.COPY, code, tuple(part.shape), (part,), (rest[at:at + part.shape[0]],))
+    if end > begin:
+        _lib.elementwise(Op.COPY, code, (end - begin,), (out[begin:end],), (src[begin - lo:end - lo],))
+    COUNTS["single"] += 1
+    _finish(node)
+
+
 class _TooBig(Exception):
     pass
 
 
-def _emit(order, roots):
-    """``(leaf tensors, immediates, instruction words, registers)`` of the program that computes ``roots``;
-    None when it does not fit the kernel's limits."""
-    dtype = roots[0].dtype
-    single = dtype == _F32
-    leaves, leaf_ids = [], {}
-    imms, imm_ids = [], {}
-    # a value is ("L", k) / ("I", k) / ("X", k): leaf k, immediate k, result of instruction k
-    instrs = []   # [op, (operand values...)]
-    numbered = {}  # (op, operand values) -> value: one instruction for equal subexpressions
-    node_value = {}
+class _Unsupported(Exception):
+    pass
 
-    def leaf(t):
-        key = (t.data_ptr(), t.stride(), tuple(t.shape))
+
+def _emit(roots):
+    """``(leaf tensors, immediates, instruction words, registers, shifted, masks)`` of the program that computes
+    ``roots``; None when it does not fit the kernel's limits.  ``shifted`` is None, or per leaf ``(shift, lo,
+    hi)`` when some vector is read at a shifted position (see :func:`shifted`)."""
+    dtype = roots[0].dtype
+    KNOWN = D.KNOWN_SCALARS
+    n_out = roots[0]._shape[0] if len(roots[0]._shape) == 1 else None
+    single = dtype == _F32
+    itemsize = dtype.itemsize
+    leaves, leaf_ids, leaf_where = [], {}, []
+    imms, imm_ids = [], {}
+    masks = []
+    # a value is ("L", k) / ("I", k) / ("X", k): leaf k, immediate k, result of instruction k
+    instrs = []   # (op, operand values, mask index or None)
+    numbered = {}  # the same: one instruction for equal subexpressions
+    memo = {}      # (id(node), shift) -> value
+    any_shift = [False]
+
+    def leaf(t, shift):
+        if KNOWN:
+            c = KNOWN.get(t.data_ptr())
+            if c is not None and (t.numel() == 1 or builtins_all_zero(t.stride())):
+                return imm(c)  # a shared constant (the seed of elementwise_grad, a zeros / ones array): no load
+        vector = t.dim() == 1 and t.numel() > 1 and t.stride(0) == 1
+        if shift:
+            if not vector:
+                if t.numel() == 1 or builtins_all_zero(t.stride()):
+                    shift = 0  # one element for every index: nothing to shift
+                else:
+                    raise _Unsupported
+            else:
+                any_shift[0] = True
+        if vector and n_out is not None and t.shape[0] != n_out:
+            any_shift[0] = True  # (a slice that starts at index 0: read in place, but not over its whole extent)
+        # (unit-stride vectors are told apart by address alone: in a program all of them span the root's extent,
+        # or are read at shifted positions inside one storage)
+        key = (t.data_ptr() + shift * itemsize,) if vector else (t.data_ptr(), t.stride(), tuple(t.shape))
         v = leaf_ids.get(key)
         if v is None:
             if len(leaves) >= _lib.PROGRAM_MAX_LEAVES:
                 raise _TooBig
             v = leaf_ids[key] = ("L", len(leaves))
             leaves.append(t)
+            leaf_where.append(shift)
         return v
 
     def imm(c):
         c = float(onp.float32(c)) if single else float(c)
-        key = (c, onp.signbit(c)) if c == 0.0 else c  # -0.0 and 0.0 are different immediates; NaN never equals itself: not shared
+        key = (c, bool(onp.signbit(c))) if c == 0.0 else c  # -0.0 and 0.0 are different immediates; NaN never equals itself: not shared
         v = imm_ids.get(key)
         if v is None:
             if len(imms) >= _lib.PROGRAM_MAX_IMMEDIATES:
@@ -313,8 +382,16 @@ def _emit(order, roots):
             imms.append(c)
         return v
 
-    def ins(op, *srcs):
-        key = (op, srcs)
+    def ins(op, *srcs, mask=None):
+        if op == Op.MUL:
+            # x * 1.0 is x, bit for bit (the cotangent seeds of elementwise_grad are ones)
+            if srcs[1][0] == "I" and imms[srcs[1][1]] == 1.0:
+                return srcs[0]
+            if srcs[0][0] == "I" and imms[srcs[0][1]] == 1.0:
+                return srcs[1]
+        elif op == Op.DIV and srcs[1][0] == "I" and imms[srcs[1][1]] == 1.0:
+            return srcs[0]
+        key = (op, srcs, mask)
         v = numbered.get(key)
         if v is None:
             if len(instrs) >= _lib.PROGRAM_MAX_INSTRUCTIONS - len(roots):
@@ -322,6 +399,17 @@ def _emit(order, roots):
             v = numbered[key] = ("X", len(instrs))
             instrs.append(key)
         return v
+
+    def masked(v, rest, lo, hi):
+        rng = (lo, hi)
+        if rng in masks:
+            k = masks.index(rng)
+        else:
+            if len(masks) >= _lib.PROGRAM_MAX_MASKS:
+                raise _TooBig
+            k = len(masks)
+            masks.append(rng)
+        return ins(_lib.PROGRAM_MASK, v, rest, mask=k)
 
     def power(x, e):
         """``pow_like_numpy(x, e)`` for an exponent known here: the short cuts NumPy takes become the plain
@@ -338,51 +426,76 @@ def _emit(order, roots):
             return ins(Op.SQRT, x)
         return ins(Op.POW, x, imm(e))
 
-    def in_dtype(c):
-        return float(onp.float32(c)) if single else c
-
-    def operand(a):
+    def value(a, shift):
+        """The register value that holds ``a[i + shift]`` at output index ``i``."""
         if type(a) is float:
             return imm(a)
         if type(a) is ExprArray and a._args is not None:
-            return node_value[id(a)]
+            key = (id(a), shift)
+            v = memo.get(key)
+            if v is not None:
+                return v
+            op = a._op
+            if op == SHIFT:
+                src, outside = a._args
+                lo, m = a._lo, src.shape[0]
+                v = value(src, shift - lo)
+                first, behind = lo - shift, lo - shift + m  # the output indices that fall inside `src`
+                if first > 0 or behind < n_out:
+                    rest = imm(0.0) if outside is None else value(outside, shift)
+                    v = masked(v, rest, max(first, 0), min(behind, n_out))
+            else:
+                srcs = tuple(value(arg, shift) for arg in a._args)
+                if op == Op.POW and srcs[1][0] == "I":
+                    v = power(srcs[0], imms[srcs[1][1]])
+                elif op == Op.POW_VJP0 and srcs[2][0] == "I":
+                    # (g * y) * x**where(y, y - 1, 1), the exponent formed in the array's precision as the functor does
+                    y = imms[srcs[2][1]]
+                    e = float(onp.float32(y) - onp.float32(1.0)) if single else y - 1.0
+                    v = ins(Op.MUL, ins(Op.MUL, srcs[0], srcs[2]), power(srcs[1], e if y != 0.0 else 1.0))
+                else:
+                    v = ins(op, *srcs)
+            memo[key] = v
+            return v
         if type(a) is LazyDevArray:
-            raw, scale, ascale, shift = D._state(a)
-            v = leaf(raw)
+            raw, scale, ascale, offset = D._state(a)
+            v = leaf(raw, shift)
             if scale != 1.0:
                 v = ins(Op.MUL, v, imm(scale))
             if ascale is not None:
-                v = ins(Op.MUL, v, leaf(ascale))
-            if shift is not None:
-                v = ins(Op.ADD, v, imm(shift) if type(shift) is float else leaf(shift))
+                v = ins(Op.MUL, v, leaf(ascale, shift))
+            if offset is not None:
+                v = ins(Op.ADD, v, imm(offset) if type(offset) is float else leaf(offset, shift))
             return v
-        return leaf(a._t)
+        return leaf(a._t, shift)
 
     try:
-        for node in order:
-            op = node._op
-            srcs = tuple(operand(a) for a in node._args)
-            if op == Op.POW and srcs[1][0] == "I":
-                v = power(srcs[0], imms[srcs[1][1]])
-            elif op == Op.POW_VJP0 and srcs[2][0] == "I":
-                # (g * y) * x**where(y, y - 1, 1), the exponent formed in the array's precision as the functor does
-                y = imms[srcs[2][1]]
-                e = in_dtype(onp.float32(y) - onp.float32(1.0)) if single else y - 1.0
-                v = ins(Op.MUL, ins(Op.MUL, srcs[0], srcs[2]), power(srcs[1], float(e) if y != 0.0 else 1.0))
-            else:
-                v = ins(op, *srcs)
-            node_value[id(node)] = v
-        root_values = [node_value[id(r)] for r in roots]
+        root_values = [value(r, 0) for r in roots]
+        if not instrs:
+            # every root is a leaf or an immediate after the rewrites: one copy each keeps the kernel's contract simple
+            root_values = [ins(Op.COPY, v) for v in root_values]
     except _TooBig:
         return None
-    if not instrs:
-        # every root is a leaf or an immediate after the rewrites: one copy each keeps the kernel's contract simple
-        root_values = [ins(Op.COPY, v) for v in root_values]
 
     n_leaf, n_imm, n_ins = len(leaves), len(imms), len(instrs)
+    shifted_leaves = None
+    if any_shift[0] or masks:
+        # one-axis program with vectors read at shifted positions: every vector leaf comes with the indices at which its
+        # (moved) address stays inside its storage; whatever lies outside a vector's own extent is masked by the program
+        shifted_leaves = []
+        for t, shift in zip(leaves, leaf_where):
+            if t.dim() == 1 and t.numel() > 1 and t.stride(0) == 1:
+                first = t.storage_offset() + shift
+                total = t.untyped_storage().nbytes() // itemsize
+                shifted_leaves.append((shift, -first, total - first))
+            elif t.numel() == 1 or builtins_all_zero(t.stride()):
+                shifted_leaves.append((0, 0, n_out))
+            else:
+                raise _Unsupported
+        leaves = [t if (t.dim() == 1 and t.numel() > 1 and t.stride(0) == 1) else t.as_strided((n_out,), (0,)) for t in leaves]
     # last use of every value (instruction index; stores come after all instructions)
     last = {}
-    for k, (_op, srcs) in enumerate(instrs):
+    for k, (_op, srcs, _mask) in enumerate(instrs):
         for s in srcs:
             last[s] = k
     for v in root_values:
@@ -399,7 +512,7 @@ def _emit(order, roots):
                 free.append(k)  # (a leaf that only a rewritten-away step read)
         words = []
         ok = True
-        for k, (op, srcs) in enumerate(instrs):
+        for k, (op, srcs, mask) in enumerate(instrs):
             regs = [reg[s] for s in srcs]
             for s in set(srcs):
                 if s[0] != "I" and last[s] == k:
@@ -413,17 +526,72 @@ def _emit(order, roots):
             else:
                 dst = free.pop()
             reg[v] = dst
-            w = op | dst << 8
-            for pos, r in enumerate(regs):
-                w |= r << (12 + 4 * pos)
+            if mask is not None:
+                w = op | dst << 8 | regs[0] << 12 | mask << 16 | regs[1] << 20  # inside value, range, outside value
+            else:
+                w = op | dst << 8
+                for pos, r in enumerate(regs):
+                    w |= r << (12 + 4 * pos)
             words.append(w)
         if not ok:
             continue
         for out_index, v in enumerate(root_values):
             r = reg[v]
             words.append(_lib.PROGRAM_STORE | r << 8 | r << 12 | out_index << 16)
-        return leaves, imms, words, n_regs
+        return leaves, imms, words, n_regs, shifted_leaves, masks
     return None
+
+
+def slice_of(A, start, stop):
+    """``A[start:stop]`` of a pending vector ``A`` as a pending node (nothing is written out)."""
+    return shifted(A, -start, stop - start)
+
+
+def padded(x, start, n, dtype):
+    """``zeros(n)`` with ``0.0 + x`` added into ``[start : start + len(x)]`` (the cotangent of ``x = y[start:stop]``,
+    formed the way the scatter rule forms it, sign of zero included) as a pending node; None when ``x`` cannot
+    take part in a program."""
+    inner = make(Op.ADD, dtype, (0.0, x))
+    if inner is None or inner._shape != x.shape:
+        return None
+    return shifted(inner, start, n)
+
+
+def added_into(A, start, x, take):
+    """``A`` with ``x`` added into ``A[start : start + len(x)]`` (``numpy.add.at`` through a slice of a vector) as
+    a pending node; ``take(A, slice)`` gives that slice of ``A``.  None when the sum cannot take part in a program."""
+    m = x.shape[0]
+    inner = make(Op.ADD, A.dtype, (take(A, slice(start, start + m)), x))
+    if inner is None or inner._shape != (m,):
+        return None
+    return shifted(inner, start, A.shape[0], outside=A)
+
+
+def builtins_all_zero(strides):
+    for s in strides:
+        if s != 0:
+            return False
+    return True
+
+
+SHIFT = -1  # pseudo-op of a shifted vector
+
+
+def shifted(src, lo, n, outside=None):
+    """The vector of length ``n`` that holds ``src[i - lo]`` at index ``i`` where that exists and ``outside[i]`` (zero
+    when None) elsewhere, as a pending node: a slice of a pending vector (``lo = -start``) and the zero-padded vector that the cotangent of
+    a slice is (``untake`` of ``x[a:b]``, autograd/numpy/numpy_vjps.py:919-950: ``lo = a``) are both this.  The
+    program kernel reads the leaves under such a node at moved addresses, so ``x[1:]``, ``x[:-1]`` and the
+    cotangents scattered back through them cost no pass of their own."""
+    cone = 1 + (src._cone if pending(src) else 0)
+    src._borrowed = True
+    if outside is not None:
+        outside._borrowed = True
+        if pending(outside):
+            cone += outside._cone
+    node = ExprArray(SHIFT, (src, outside), (n,), src.dtype, cone)
+    node._lo = lo
+    return node
 
 
 D._DEFERRED = D._DEFERRED + (ExprArray,)

@@ -23,6 +23,7 @@ def _shared_zero(dtype):
     z = _ZEROS.get(dtype)
     if z is None:
         z = _ZEROS[dtype] = D.zeros((), dtype)
+        D.KNOWN_SCALARS[z._t.data_ptr()] = 0.0
     return z
 
 
@@ -33,6 +34,7 @@ def _shared_one(dtype):
     o = _ONES.get(dtype)
     if o is None:
         o = _ONES[dtype] = D.ones((), dtype)
+        D.KNOWN_SCALARS[o._t.data_ptr()] = 1.0
     return o
 
 
@@ -164,6 +166,7 @@ DevArrayVSpace.register(D.PendingProduct)
 DevArrayVSpace.register(D.LseCotangent)
 DevArrayVSpace.register(D.FusedResult)
 DevArrayVSpace.register(_fusion.ExprArray)
+DevArrayVSpace.register(D.PendingReduce)
 DevArrayVSpace.register(float)
 
 

@@ -993,6 +993,10 @@ def take(A, idx):
         pidx, backwards = _positive_steps(_plain(idx), A.shape)
         if type(A) is D.LazyDevArray and _trace_stack.top < 0 and not builtins.any(A._raw.stride()):
             A._t  # outside any trace a lazy fill (zeros / ones) is written out before it is viewed: an item assignment through the view then reaches it
+        if D._fusion.pending(A) and A.ndim == 1 and not backwards and D._fusion.ENABLED:
+            rows = _leading_rows(pidx, A.shape)
+            if rows is not None and rows[1] > rows[0]:
+                return D._fusion.slice_of(A, rows[0], rows[1])  # a slice of a vector that is still an expression stays one
         picked = A._view(lambda t: t[pidx])
         return _reverse_axes(picked, backwards) if backwards else picked
     if A.ndim == 0:
@@ -1089,6 +1093,13 @@ def scatter_add(A, idx, x):
         idx, backwards = _positive_steps(_plain(idx), A.shape)
         if backwards:  # A[::-1] += x  is  A[::1] += x reversed
             x = _reverse_axes(D.asarray(broadcast_to.fun(D.asarray(x, A.dtype), tuple(A._t[idx].shape))), backwards)
+    if (basic and A.ndim == 1 and D._fusion.ENABLED and A.dtype in D._FLOATS and isinstance(x, DevArray) and x.dtype == A.dtype
+            and not is_shared_zero(A)):
+        rows = _leading_rows(idx, A.shape)
+        if rows is not None and rows[1] > rows[0] and x.shape == (rows[1] - rows[0],):
+            node = D._fusion.added_into(A, rows[0], x, take)  # stays an expression: the sum joins whatever reads it
+            if node is not None:
+                return node
     if A._borrowed or type(A) is not DevArray or is_broadcast_view(A) or is_shared_zero(A):  # not this accumulator's own memory yet: allocate it
         if is_shared_zero(A):
             if basic:
@@ -1105,6 +1116,13 @@ def scatter_add(A, idx, x):
                     acc._borrowed = True
                     return acc
                 rows = None if full_cover else _leading_rows(idx, A.shape)
+                if (rows is not None and A.ndim == 1 and D._fusion.ENABLED and isinstance(x, DevArray) and x.dtype == A.dtype
+                        and A.dtype in D._FLOATS and x.shape == (rows[1] - rows[0],) and rows[1] > rows[0]):
+                    # a vector's x[a:b]: the padded cotangent stays an expression (its zeros are never written; the program
+                    # that finally needs it reads x's operands at moved addresses)
+                    node = D._fusion.padded(x, rows[0], A.shape[0], A.dtype)
+                    if node is not None:
+                        return node
                 if full_cover or rows is not None:
                     A = D.empty(A.shape, A.dtype)
                     if rows is not None:

@@ -190,6 +190,14 @@ int agmi_elementwise(int op, int dtype, int ndim, const int64_t *shape,
  * it, so a program gives bit for bit what the same ops give as separate agmi_elementwise calls;
  * op AGMI_PROGRAM_STORE writes reg[a] to output b (dst must equal a).  Every register read must
  * have been written, every output stored, else AGMI_ERR_ARG and nothing is launched.
+ * Shifted reads (slices of a vector and the zero-padded vectors their cotangents are:
+ * x[1:], x[:-1] and `untake`, autograd/numpy/numpy_vjps.py:919-950).  On a one-axis index space a
+ * leaf may be a vector read at a shifted position: its `data` then points at the element that
+ * index 0 reads (possibly before the vector's first element) and leaf_ranges[2i], leaf_ranges[2i+1]
+ * give the indices [lo, hi) at which that address may be dereferenced; outside them the register
+ * gets an unspecified finite value, which the program is expected to discard with op
+ * AGMI_PROGRAM_MASK: reg[dst] = (mask_ranges[2b] <= idx < mask_ranges[2b+1]) ? reg[a] : reg[c].
+ * leaf_ranges may be NULL (every index readable); n_mask <= AGMI_PROGRAM_MAX_MASKS.
  * Layout: after axis merging at most two axes may remain and every operand must have stride 1 or
  * 0 (leaves only) along the innermost one; anything else returns AGMI_ERR_UNSUPPORTED.  Outputs
  * may not overlap leaves unless they are the same view (in-place update).
@@ -201,9 +209,12 @@ int agmi_elementwise(int op, int dtype, int ndim, const int64_t *shape,
 #define AGMI_PROGRAM_MAX_OUTPUTS 4
 #define AGMI_PROGRAM_MAX_INSTRUCTIONS 96
 #define AGMI_PROGRAM_MAX_REGISTERS 16
+#define AGMI_PROGRAM_MAX_MASKS 4
 #define AGMI_PROGRAM_STORE 255
+#define AGMI_PROGRAM_MASK 254
 int agmi_program(int dtype, int ndim, const int64_t *shape, int n_out, const agmi_array *outs,
-                 int n_leaf, const agmi_array *leaves, int n_imm, const double *imms,
+                 int n_leaf, const agmi_array *leaves, const int64_t *leaf_ranges,
+                 int n_imm, const double *imms, int n_mask, const int64_t *mask_ranges,
                  int n_instr, const uint32_t *code, int n_regs, void *stream);
 
 /* out[idx] = (in0[idx] <cmp> in1[idx]) as AGMI_BOOL; inputs as in agmi_elementwise. */
