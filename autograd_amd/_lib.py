@@ -110,6 +110,11 @@ class AgmiCorrelation(ctypes.Structure):
                 ("out_strides", ctypes.c_int64 * 3)]
 
 
+class AgmiGemmEpilogue(ctypes.Structure):
+    _fields_ = [("kind", ctypes.c_int32), ("bias", ctypes.c_void_p), ("out", ctypes.c_void_p), ("out_ld", ctypes.c_int64),
+                ("x", ctypes.c_void_p), ("x_ld", ctypes.c_int64)]
+
+
 class AgmiLseCotangent(ctypes.Structure):
     _fields_ = [("rows", ctypes.c_int64), ("cols", ctypes.c_int64), ("x", ctypes.c_void_p), ("x_row_stride", ctypes.c_int64),
                 ("affine", ctypes.c_uint32), ("scale", ctypes.c_double), ("shift", ctypes.c_double),
@@ -178,6 +183,9 @@ def lib():
     L.agmi_gemm.restype = c_i
     L.agmi_gemm.argtypes = [c_i, c_i64, c_i64, c_i64, c_i64, c_d, c_p, c_i64, c_i64, c_i64, c_p, c_i64, c_i64,
                             c_i64, c_d, c_p, c_i64, c_i64, c_p, c_sz, c_p]
+    L.agmi_gemm_fused.restype = c_i
+    L.agmi_gemm_fused.argtypes = [c_i, c_i64, c_i64, c_i64, c_p, c_i64, c_i64, c_p, c_i64, c_i64, c_p, c_i64,
+                                  ctypes.POINTER(AgmiGemmEpilogue), c_p, c_sz, c_p]
     L.agmi_fill.restype = c_i
     L.agmi_fill.argtypes = [c_i, c_p, c_i64, c_d, c_p]
     L.agmi_reverse.restype = c_i
@@ -206,7 +214,7 @@ def lib():
 
 EXPORTS = (
     "agmi_last_error agmi_version agmi_last_kernel agmi_elementwise agmi_program agmi_compare agmi_cast agmi_map_reduce "
-    "agmi_map_reduce_workspace_bytes agmi_map_reduce_static agmi_gemm agmi_fill agmi_take_rows agmi_sort_rows agmi_cumsum agmi_reverse agmi_triangle agmi_scatter_add_rows agmi_optimizer_step "
+    "agmi_map_reduce_workspace_bytes agmi_map_reduce_static agmi_gemm agmi_gemm_fused agmi_fill agmi_take_rows agmi_sort_rows agmi_cumsum agmi_reverse agmi_triangle agmi_scatter_add_rows agmi_optimizer_step "
     "agmi_correlate agmi_lse_cotangent_fused agmi_concat"
 ).split()
 
@@ -644,6 +652,34 @@ def gemm(code, batch, M, N, K, alpha, A, a_rs, a_cs, a_bs, B, b_rs, b_cs, b_bs, 
     if ev is not None:
         es = A.element_size()
         _TIMER.end(ev, ("gemm",), batch * (M * K + K * N + M * N) * es, 2.0 * batch * M * N * K)
+
+
+EPILOGUE_BIAS_TANH, EPILOGUE_TANH_VJP = 1, 2
+_epilogue = AgmiGemmEpilogue()
+
+
+def gemm_fused(code, A, B, C, kind, bias=None, out=None, x=None):
+    """``agmi_gemm_fused``: ``A @ B`` (2-d tensors, any strides) into the contiguous ``C`` with a dense layer's
+    epilogue: ``out = tanh(C + bias)`` beside it, or ``C = (A @ B) / cosh(x + bias)**2`` (``bias``: contiguous
+    vector or None).  Returns False when the operands are outside what the fused kernel covers."""
+    M, K = A.shape
+    N = B.shape[1]
+    e = _epilogue
+    e.kind = kind
+    e.bias = bias.data_ptr() if bias is not None else None
+    e.out, e.out_ld = (out.data_ptr(), out.stride(0)) if out is not None else (None, 0)
+    e.x, e.x_ld = (x.data_ptr(), x.stride(0)) if x is not None else (None, 0)
+    ev = _TIMER.begin(("gemm",)) if _TIMER is not None else None
+    rc = _LIB.agmi_gemm_fused(code, M, N, K, A.data_ptr(), A.stride(0), A.stride(1), B.data_ptr(), B.stride(0), B.stride(1),
+                              C.data_ptr(), C.stride(0), ctypes.byref(e), _workspace().data_ptr(), _WORKSPACE_BYTES, _stream())
+    if rc == -2:  # AGMI_ERR_UNSUPPORTED
+        return False
+    if rc:
+        _check(rc, "agmi_gemm_fused")
+    if ev is not None:
+        es = A.element_size()
+        _TIMER.end(ev, ("gemm",), (M * K + K * N + 2 * M * N) * es, 2.0 * M * N * K)
+    return True
 
 
 def fill(code, t, value):

@@ -88,7 +88,30 @@ struct GemmParams {
     // gemm_direct only: bytes from element (0, 0) of one matrix of the batch to one past its last
     // element (the extent of the buffer descriptor the loads are range-checked against)
     uint32_t a_span_bytes, b_span_bytes;
+    // epilogue of the float32 direct kernel and of the split finish (agmi_gemm_fused):
+    //   1: beside C, epi_out[m, n] = tanh(C[m, n] + epi_bias[n])
+    //   2: C[m, n] = acc / cosh(epi_x[m, n] + epi_bias[n])**2 (the product itself is not stored)
+    // epi_bias may be null (nothing added)
+    int epi;
+    const float *epi_bias;
+    float *epi_out;
+    int64_t epi_ld;
+    const float *epi_x;
+    int64_t epi_x_ld;
 };
+
+// What follows the contraction in an evaluation of a dense layer and of its adjoint, applied to the accumulators
+// before they are stored.  The arithmetic is the one-rule kernels' (functors.h: FTanh, FTanhVjp; a pending
+// `+ bias` is one rounded add), so the results are the separate launches' bit for bit.
+__device__ __forceinline__ float epi_tanh(float acc, float bias, bool has_bias) {
+    const float z = has_bias ? acc + bias : acc;
+    return tanhf(z);
+}
+__device__ __forceinline__ float epi_tanh_vjp(float acc, float x, float bias, bool has_bias) {
+    const float z = has_bias ? x + bias : x;
+    const float c = coshf(z);
+    return acc / (c * c);
+}
 
 constexpr int kGroupM = 8;
 constexpr int kXcds = 8;
@@ -446,7 +469,7 @@ __device__ __forceinline__ v4i raw_buffer(const void *base, uint32_t bytes) {
 // TAIL: K is not a multiple of 4 and an operand is contiguous along k, so the 16 bytes a lane fetches at the end of
 // a row run past k = K into whatever follows in memory (the next row); those elements are zeroed in LDS before
 // any wave reads the slab.
-template <int MODE_A, int MODE_B, bool TAIL>
+template <int MODE_A, int MODE_B, bool TAIL, int EPI>
 __global__ __launch_bounds__(kDirectThreads) void gemm_direct(const GemmParams p) {
     constexpr int BM = 64, BN = 64, BK = 32, NBUF = 4;
     constexpr int kOpFloats = 64 * BK;         // one operand slab
@@ -672,6 +695,19 @@ __global__ __launch_bounds__(kDirectThreads) void gemm_direct(const GemmParams p
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[v] = acc[v] + beta * old[v];
     }
+    if constexpr (EPI == 2) {
+        const bool has_bias = p.epi_bias != nullptr;
+        const float bias = (has_bias && col < p.N) ? p.epi_bias[col] : 0.f;
+        const float *X = p.epi_x + row0 * p.epi_x_ld + col;
+        float xs[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int dr = 8 * (v / 4) + (v % 4);
+            xs[v] = (interior || (row0 + dr < p.M && col < p.N)) ? X[dr * p.epi_x_ld] : 0.f;
+        }
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[v] = epi_tanh_vjp(acc[v], xs[v], bias, has_bias);
+    }
     if (interior) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) C[(8 * (v / 4) + (v % 4)) * p.ldc] = acc[v];
@@ -680,6 +716,17 @@ __global__ __launch_bounds__(kDirectThreads) void gemm_direct(const GemmParams p
         for (int v = 0; v < 16; ++v) {
             const int dr = 8 * (v / 4) + (v % 4);
             if (row0 + dr < p.M && col < p.N) C[dr * p.ldc] = acc[v];
+        }
+    }
+    if constexpr (EPI == 1) {
+        const bool has_bias = p.epi_bias != nullptr;
+        const float bias = (has_bias && col < p.N) ? p.epi_bias[col] : 0.f;
+        float *Y = p.epi_out + row0 * p.epi_ld + col;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int dr = 8 * (v / 4) + (v % 4);
+            const float y = epi_tanh(acc[v], bias, has_bias);
+            if (interior || (row0 + dr < p.M && col < p.N)) Y[dr * p.epi_ld] = y;
         }
     }
 }
@@ -699,6 +746,24 @@ __global__ __launch_bounds__(kBlock) void gemm_split_finish(const T *__restrict_
     T v = alpha * acc;
     if (beta != T(0)) v = v + beta * *dst;
     *dst = v;
+}
+
+// the same with the dense-layer epilogues (one matrix, alpha = 1, beta = 0)
+template <int EPI>
+__global__ __launch_bounds__(kBlock) void gemm_split_finish_fused(const float *__restrict__ ws, float *__restrict__ C, int splits,
+                                                                  int64_t M, int64_t N, int64_t ldc, const float *bias,
+                                                                  float *out, int64_t out_ld, const float *x, int64_t x_ld) {
+    const int64_t e = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    const int64_t per = M * N;
+    if (e >= per) return;
+    const int64_t r = e / N, c = e - r * N;
+    float acc = ws[e];
+    for (int s = 1; s < splits; ++s) acc += ws[static_cast<int64_t>(s) * per + e];
+    const bool has_bias = bias != nullptr;
+    const float b = has_bias ? bias[c] : 0.f;
+    if (EPI == 2) acc = epi_tanh_vjp(acc, x[r * x_ld + c], b, has_bias);
+    C[r * ldc + c] = acc;
+    if (EPI == 1) out[r * out_ld + c] = epi_tanh(acc, b, has_bias);
 }
 
 // K == 0: the product is empty, C = beta * C.  Handled apart because the tile kernel's branch-free
@@ -834,25 +899,45 @@ static int launch_direct(GemmParams p, int64_t batch, hipStream_t s, void *ws, s
     if (p.splits > 1)
         set_kernel_name("gemm_direct<f32,64,64,32,%s%s>+split%d", mode_name(mode_a), mode_name(mode_b), p.splits);
     else
-        set_kernel_name("gemm_direct<f32,64,64,32,%s%s>", mode_name(mode_a), mode_name(mode_b));
+        set_kernel_name("gemm_direct<f32,64,64,32,%s%s%s>", mode_name(mode_a), mode_name(mode_b),
+                        p.epi == 1 ? ",+bias,tanh" : (p.epi == 2 ? ",tanh_vjp" : ""));
     const dim3 grid((unsigned)(tm * tn), (unsigned)batch, (unsigned)p.splits);
     const dim3 block(kDirectThreads);
     const bool tail = p.K % 4 != 0 && (mode_a == kKC || mode_b == kKC);
-    if (mode_a == kXC && mode_b == kXC)
-        hipLaunchKernelGGL((gemm_direct<kXC, kXC, false>), grid, block, 0, s, p);
-    else if (mode_a == kXC && tail)
-        hipLaunchKernelGGL((gemm_direct<kXC, kKC, true>), grid, block, 0, s, p);
-    else if (mode_a == kXC)
-        hipLaunchKernelGGL((gemm_direct<kXC, kKC, false>), grid, block, 0, s, p);
-    else if (mode_b == kXC && tail)
-        hipLaunchKernelGGL((gemm_direct<kKC, kXC, true>), grid, block, 0, s, p);
-    else if (mode_b == kXC)
-        hipLaunchKernelGGL((gemm_direct<kKC, kXC, false>), grid, block, 0, s, p);
-    else if (tail)
-        hipLaunchKernelGGL((gemm_direct<kKC, kKC, true>), grid, block, 0, s, p);
-    else
-        hipLaunchKernelGGL((gemm_direct<kKC, kKC, false>), grid, block, 0, s, p);
+    // (a product cut along K leaves raw partial tiles; its epilogue runs in the finishing kernel)
+    const int epi = p.splits > 1 ? 0 : p.epi;
+    const auto launch = [&](auto ma, auto mb, auto tl) {
+        constexpr int MA = decltype(ma)::value, MB = decltype(mb)::value;
+        constexpr bool TL = decltype(tl)::value;
+        if (epi == 1) hipLaunchKernelGGL((gemm_direct<MA, MB, TL, 1>), grid, block, 0, s, p);
+        else if (epi == 2) hipLaunchKernelGGL((gemm_direct<MA, MB, TL, 2>), grid, block, 0, s, p);
+        else hipLaunchKernelGGL((gemm_direct<MA, MB, TL, 0>), grid, block, 0, s, p);
+    };
+    using XC = std::integral_constant<int, kXC>;
+    using KC = std::integral_constant<int, kKC>;
+    using Yes = std::integral_constant<bool, true>;
+    using No = std::integral_constant<bool, false>;
+    if (mode_a == kXC && mode_b == kXC) launch(XC{}, XC{}, No{});
+    else if (mode_a == kXC && tail) launch(XC{}, KC{}, Yes{});
+    else if (mode_a == kXC) launch(XC{}, KC{}, No{});
+    else if (mode_b == kXC && tail) launch(KC{}, XC{}, Yes{});
+    else if (mode_b == kXC) launch(KC{}, XC{}, No{});
+    else if (tail) launch(KC{}, KC{}, Yes{});
+    else launch(KC{}, KC{}, No{});
     if (int rc = hip_check(hipGetLastError(), "gemm launch")) return rc;
+    if (p.splits > 1 && p.epi != 0) {
+        const int64_t n = p.M * p.N;
+        const dim3 fgrid((unsigned)ceil_div(n, kBlock));
+        if (p.epi == 1)
+            hipLaunchKernelGGL(gemm_split_finish_fused<1>, fgrid, dim3(kBlock), 0, s, static_cast<const float *>(p.ws),
+                               static_cast<float *>(p.C), p.splits, p.M, p.N, p.ldc, p.epi_bias, p.epi_out, p.epi_ld, p.epi_x,
+                               p.epi_x_ld);
+        else
+            hipLaunchKernelGGL(gemm_split_finish_fused<2>, fgrid, dim3(kBlock), 0, s, static_cast<const float *>(p.ws),
+                               static_cast<float *>(p.C), p.splits, p.M, p.N, p.ldc, p.epi_bias, p.epi_out, p.epi_ld, p.epi_x,
+                               p.epi_x_ld);
+        return hip_check(hipGetLastError(), "gemm launch");
+    }
     if (p.splits > 1) {
         const int64_t n = batch * p.M * p.N;
         hipLaunchKernelGGL(gemm_split_finish<float>, dim3((unsigned)ceil_div(n, kBlock)), dim3(kBlock), 0, s,
@@ -924,4 +1009,48 @@ extern "C" int agmi_gemm(int dtype, int64_t batch, int64_t M, int64_t N, int64_t
     if (dtype == AGMI_F64) return launch_gemm<MfmaF64x16, 64, 64, 16, 2, 1>(p, batch, s, workspace, workspace_bytes);
     set_error("gemm: dtype %d is not a floating type", dtype);
     return AGMI_ERR_ARG;
+}
+
+extern "C" int agmi_gemm_fused(int dtype, int64_t M, int64_t N, int64_t K, const void *A, int64_t a_rs, int64_t a_cs,
+                               const void *B, int64_t b_rs, int64_t b_cs, void *C, int64_t ldc,
+                               const agmi_gemm_epilogue *e, void *workspace, size_t workspace_bytes, void *stream) {
+    if (!e || (e->kind != AGMI_EPILOGUE_BIAS_TANH && e->kind != AGMI_EPILOGUE_TANH_VJP)) {
+        set_error("gemm_fused: unknown epilogue");
+        return AGMI_ERR_ARG;
+    }
+    if (M <= 0 || N <= 0 || K <= 0 || !A || !B || !C || ldc < N) {
+        set_error("gemm_fused: empty or null operands");
+        return AGMI_ERR_ARG;
+    }
+    if (e->kind == AGMI_EPILOGUE_BIAS_TANH && (!e->out || e->out_ld < N)) {
+        set_error("gemm_fused: the activation needs an output matrix");
+        return AGMI_ERR_ARG;
+    }
+    if (e->kind == AGMI_EPILOGUE_TANH_VJP && (!e->x || e->x_ld < N)) {
+        set_error("gemm_fused: the tanh cotangent needs the saved pre-activation");
+        return AGMI_ERR_ARG;
+    }
+    if (dtype != AGMI_F32) {
+        set_error("gemm_fused: float32 only");
+        return AGMI_ERR_UNSUPPORTED;
+    }
+    GemmParams p = {};
+    p.A = A; p.B = B; p.C = C;
+    p.M = M; p.N = N; p.K = K;
+    p.a_rs = a_rs; p.a_cs = a_cs;
+    p.b_rs = b_rs; p.b_cs = b_cs;
+    p.ldc = ldc;
+    p.alpha = 1.0; p.beta = 0.0;
+    p.epi = e->kind;
+    p.epi_bias = static_cast<const float *>(e->bias);
+    p.epi_out = static_cast<float *>(e->out);
+    p.epi_ld = e->out_ld;
+    p.epi_x = static_cast<const float *>(e->x);
+    p.epi_x_ld = e->x_ld;
+    const int rc = launch_direct(p, 1, as_stream(stream), workspace, workspace_bytes);
+    if (rc == 1) {
+        set_error("gemm_fused: operands outside the direct kernel's layouts (one unit stride each)");
+        return AGMI_ERR_UNSUPPORTED;
+    }
+    return rc;
 }

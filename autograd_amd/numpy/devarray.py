@@ -164,10 +164,14 @@ class LazyDevArray(DevArray):
     the value to a fresh buffer (one copy kernel) and keeps it.
     """
 
-    __slots__ = ("_raw", "_scale", "_shift", "_ascale")
+    __slots__ = ("_raw", "_scale", "_shift", "_ascale", "_producer")
 
-    def __init__(self, raw, dtype, scale, shift, ascale=None):
+    def __init__(self, raw, dtype, scale, shift, ascale=None, producer=None):
         self._raw = raw
+        # the matrix product whose (still empty) result buffer `raw` is, while that product has not run: whatever
+        # first needs this value runs it, possibly together with the pending steps (a dense layer's bias and
+        # activation go into the contraction's epilogue, see `fusion._dense_layer`)
+        self._producer = producer
         self.dtype = dtype
         self._borrowed = False
         self._scale = scale    # Python float, representable in dtype; 1.0 = no multiply
@@ -188,7 +192,14 @@ class LazyDevArray(DevArray):
         return out
 
     def _affine(self):
+        if self._producer is not None:
+            self._produce()
         return _lib.Affine(self._raw, self._scale, self._shift, self._ascale)
+
+    def _produce(self):
+        """Fill the storage (the matrix product it waits for runs now)."""
+        product, self._producer = self._producer, None
+        product._t
 
     @property
     def shape(self):
@@ -231,11 +242,13 @@ class LazyDevArray(DevArray):
         storage's shape); when one of them cannot be viewed that way the value is written out."""
         asc, sh = self._ascale, self._shift
         if sh is None and asc is None and self._scale == 1.0:
+            if self._producer is not None:
+                self._produce()
             return DevArray(fn(self._raw), self.dtype)  # nothing pending (the value has been written out): a plain view
         try:
             return LazyDevArray(fn(self._raw), self.dtype, self._scale,
                                 fn(sh) if isinstance(sh, torch.Tensor) else sh,
-                                fn(asc) if asc is not None else None)
+                                fn(asc) if asc is not None else None, self._producer)
         except RuntimeError:
             return DevArray(fn(self._t), self.dtype)
 
@@ -252,21 +265,58 @@ class PendingProduct(DevArray):
     ``DevArray``; the first such read computes the product and keeps it.
     """
 
-    __slots__ = ("_left", "_right", "_shape")
+    __slots__ = ("_left", "_right", "_shape", "_out")
 
     def __init__(self, left, right, dtype):
         self._left, self._right = left, right
         self._shape = (left.shape[0], right.shape[1])
         self.dtype = dtype
         self._borrowed = False
+        self._out = None
 
     def __getattr__(self, name):
         # only reached when a slot is unset: `_t` before the product has been computed
         if name != "_t":
             raise AttributeError(name)
-        self._t = out = gemm2d(self._left, self._right, self.dtype)
-        self._left = self._right = None
+        if self._out is None:
+            out = gemm2d(self._left, self._right, self.dtype)
+        else:
+            out = gemm2d(self._left, self._right, self.dtype, out=self._out)
+        self._t = out
+        self._left = self._right = self._out = None
         return out
+
+    def _buffer(self):
+        """The memory the product will be written to (allocated now, filled when the product runs)."""
+        if self._left is None:
+            return self._t
+        out = self._out
+        if out is None:
+            out = self._out = _lib.empty(self._shape, self.dtype)
+        return out
+
+    def _h(self):
+        return self._buffer()
+
+    def with_activation(self, bias, act_out):
+        """Run the product with ``act_out = tanh(product + bias)`` formed in the contraction's epilogue; False when the
+        fused kernel does not take these operands (nothing has run then)."""
+        if not self._shape[0] or not self._shape[1] or not self._left.shape[1]:
+            return False
+        out = self._buffer()
+        if not _lib.gemm_fused(_lib.DTYPE_CODE[self.dtype], self._left, self._right, out, _lib.EPILOGUE_BIAS_TANH, bias=bias,
+                               out=act_out):
+            return False
+        self._t = out
+        self._left = self._right = self._out = None
+        return True
+
+    def into_tanh_cotangent(self, x, bias, out):
+        """``out = (left @ right) / cosh(x + bias)**2`` in one launch (the product itself stays uncomputed); False when
+        the fused kernel does not take these operands."""
+        if not self._shape[0] or not self._shape[1] or not self._left.shape[1]:
+            return False
+        return _lib.gemm_fused(_lib.DTYPE_CODE[self.dtype], self._left, self._right, out, _lib.EPILOGUE_TANH_VJP, bias=bias, x=x)
 
     def computed(self):
         return self._left is None
@@ -544,8 +594,19 @@ def _representable(v, dtype):
 def _state(a):
     """(raw tensor, scalar scale, array scale, shift) of a device array."""
     if type(a) is LazyDevArray:
+        if a._producer is not None:
+            a._produce()
         return a._raw, a._scale, a._ascale, a._shift
     return a._t, 1.0, None, None
+
+
+def _state_and_producer(a):
+    """``_state`` without running a matrix product that has not run yet: its result buffer and the product."""
+    if type(a) is LazyDevArray:
+        return a._raw, a._scale, a._ascale, a._shift, a._producer
+    if type(a) is PendingProduct and not a.computed():
+        return a._buffer(), 1.0, None, None, a
+    return a._t, 1.0, None, None, None
 
 
 def _fold(op, dtype, xs):
@@ -584,7 +645,7 @@ def _fold(op, dtype, xs):
         return None
     if not isinstance(a, DevArray) or a.dtype != dtype:
         return None
-    raw, s, asc, t = _state(a)
+    raw, s, asc, t, producer = _state_and_producer(a)
     array_shift = isinstance(t, torch.Tensor)
     if c is not None:
         c = float(c) if dtype == _F64 else float(onp.float32(c))
@@ -624,9 +685,9 @@ def _fold(op, dtype, xs):
     else:
         return None
     a._borrowed = True  # the result reads `a`'s memory when it is consumed: an item assignment into `a` must not reach it
-    if s == 1.0 and t is None and asc is None:
+    if s == 1.0 and t is None and asc is None and producer is None:
         return DevArray(raw, dtype)
-    return LazyDevArray(raw, dtype, s, t, asc)
+    return LazyDevArray(raw, dtype, s, t, asc, producer)
 
 
 def _fold_array(op, dtype, a, c, swapped):
@@ -636,7 +697,7 @@ def _fold_array(op, dtype, a, c, swapped):
         return None
     if c.size >= a.size or a.size == 0 or broadcast_shapes(a.shape, c.shape) != a.shape:
         return None
-    raw, s, asc, t = _state(a)
+    raw, s, asc, t, producer = _state_and_producer(a)
     if t is not None:
         return None  # an offset is the last step
     if type(c) is LazyDevArray or c.ndim > a.ndim:
@@ -646,10 +707,10 @@ def _fold_array(op, dtype, a, c, swapped):
         return None
     a._borrowed = c._borrowed = True  # (both are read when the result is consumed; see `_fold`)
     if op == Op.MUL:
-        return LazyDevArray(raw, dtype, s, None, vec)
+        return LazyDevArray(raw, dtype, s, None, vec, producer)
     if op == Op.ADD:
-        return LazyDevArray(raw, dtype, s, vec, asc)
-    return LazyDevArray(raw, dtype, -s, vec, asc)  # c - a = (-a) + c
+        return LazyDevArray(raw, dtype, s, vec, asc, producer)
+    return LazyDevArray(raw, dtype, -s, vec, asc, producer)  # c - a = (-a) + c
 
 
 _FOLDABLE = frozenset({Op.NEG, Op.MUL, Op.ADD, Op.SUB, Op.DIV})

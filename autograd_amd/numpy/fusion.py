@@ -49,7 +49,7 @@ for _name in "WHERE DIV_VJP1 POW_VJP0 POW_VJP1 ABS_VJP MUL_ADD".split():
 for _name in "LSE_VJP CHOOSE_VJP EXTREMUM_VJP".split():
     ARITY[getattr(Op, _name)] = 4
 
-COUNTS = {"programs": 0, "instructions": 0, "single": 0, "unfused": 0}  # what ran (tests and profiles read it)
+COUNTS = {"programs": 0, "instructions": 0, "single": 0, "unfused": 0, "layers": 0}  # what ran (tests and profiles read it)
 
 
 class ExprArray(DevArray):
@@ -225,7 +225,8 @@ def _finish(node):
 def _run(roots):
     order = _post_order(roots)
     if len(order) == 1 and order[0]._op != SHIFT:
-        _single(order[0])
+        if not _dense_layer(order[0]):
+            _single(order[0])
         return
     if len(roots) > _lib.PROGRAM_MAX_OUTPUTS:
         half = len(roots) // 2
@@ -273,6 +274,69 @@ def _run(roots):
     for node in order:
         if node._args is not None:
             _single(node)
+
+
+def _row_vector(t, shape):
+    """The contiguous vector behind a tensor of ``shape`` that repeats one row (strides (0, 1)); None otherwise."""
+    if tuple(t.shape) != shape or t.stride(0) != 0 or (t.stride(1) != 1 and shape[1] != 1):
+        return None
+    return t[0]
+
+
+def _dense_layer(node):
+    """A lone ``tanh`` over a matrix product that has not run yet (plus a pending bias), or the tanh rule applied to
+    one (the cotangent ``G . W^T`` of examples/neural_net.py:33-35 under autograd/numpy/numpy_vjps.py:178, 615-624),
+    goes into the contraction's epilogue: one launch for the layer.  False: not that shape (nothing has run)."""
+    op = node._op
+    if node.dtype != _F32 or len(node._shape) != 2:
+        return False
+    if op == Op.TANH:
+        a = node._args[0]
+        if type(a) is D.PendingProduct and not a.computed():
+            product, bias = a, None
+        elif type(a) is LazyDevArray and a._producer is not None and a._scale == 1.0 and a._ascale is None:
+            product = a._producer
+            raw = a._raw
+            if product.computed() or raw.data_ptr() != product._buffer().data_ptr() or tuple(raw.shape) != product.shape \
+                    or not raw.is_contiguous():
+                return False
+            bias = a._shift
+            if bias is not None:
+                if type(bias) is float:
+                    return False
+                bias = _row_vector(bias, node._shape)
+                if bias is None:
+                    return False
+        else:
+            return False
+        if product.shape != node._shape or not product.with_activation(bias, node._buffer()):
+            return False
+        if type(a) is LazyDevArray:
+            a._producer = None
+    elif op == Op.TANH_VJP:
+        g, x = node._args
+        if type(g) is not D.PendingProduct or g.computed() or g.shape != node._shape:
+            return False
+        bias = None
+        if type(x) is DevArray:
+            xt = x._t
+        elif type(x) is LazyDevArray and x._scale == 1.0 and x._ascale is None and type(x._shift) is not float:
+            xt = D._state(x)[0]  # (runs the forward product first if it never ran)
+            if x._shift is not None:
+                bias = _row_vector(x._shift, node._shape)
+                if bias is None:
+                    return False
+        else:
+            return False
+        if tuple(xt.shape) != node._shape or (xt.stride(1) != 1 and node._shape[1] != 1) or xt.stride(0) < node._shape[1]:
+            return False
+        if not g.into_tanh_cotangent(xt, bias, node._buffer()):
+            return False
+    else:
+        return False
+    COUNTS["layers"] += 1
+    _finish(node)
+    return True
 
 
 def _single(node):

@@ -574,7 +574,7 @@ def _concat_pieces(arrs, axis, dt):
             return None
         if type(a) is DevArray:
             t = a._t
-        elif type(a) is D.LazyDevArray and a._scale == 1.0 and a._shift is None and a._ascale is None:
+        elif type(a) is D.LazyDevArray and a._scale == 1.0 and a._shift is None and a._ascale is None and a._producer is None:
             t = a._raw  # a constant: one shared element seen through stride-0 axes
         else:
             return None
@@ -1232,6 +1232,9 @@ def _dot_raw(a, b):
     if a.shape[-1] != b.shape[-2]:
         raise ValueError(f"shapes {a.shape} and {b.shape} not aligned: {a.shape[-1]} (dim {a.ndim - 1}) != {b.shape[-2]} (dim {b.ndim - 2})")
     if a.ndim == 2 and b.ndim == 2:
+        if D._fusion.ENABLED and a.shape[0] and b.shape[1]:
+            # left pending: a bias and an activation that follow can then ride in the contraction's epilogue
+            return D.PendingProduct(a._t, b._t, dt)
         return DevArray(D.gemm2d(a._t, b._t, dt), dt)
     # numpy.dot on higher ranks: sum over last axis of a and second-to-last of b
     return _tensordot_raw(a, b, axes=((a.ndim - 1,), (b.ndim - 2,)))

@@ -318,6 +318,31 @@ int agmi_gemm(int dtype, int64_t batch, int64_t M, int64_t N, int64_t K, double 
               double beta, void *C, int64_t ldc, int64_t c_bs,
               void *workspace, size_t workspace_bytes, void *stream);
 
+/* agmi_gemm (float32, one matrix, alpha = 1, beta = 0) with what follows the contraction in a dense layer
+ * applied to the accumulators before they are stored, so that the layer costs one launch:
+ *   AGMI_EPILOGUE_BIAS_TANH  C = A.B as agmi_gemm stores it, and beside it
+ *                            out[m,n] = tanh(C[m,n] + bias[n])          examples/neural_net.py:33-35
+ *   AGMI_EPILOGUE_TANH_VJP   C[m,n] = (A.B)[m,n] / cosh(x[m,n] + bias[n])**2: the tanh rule applied to the
+ *                            cotangent G.W^T while it is formed          autograd/numpy/numpy_vjps.py:178, 615-624
+ * bias may be NULL (nothing is added).  Each step is rounded as the separate kernels round it (the bias as a
+ * pending `+ bias`, tanh / cosh as AGMI_OP_TANH / AGMI_OP_TANH_VJP), so the results are theirs bit for bit.
+ * A and B as in agmi_gemm; each needs one unit stride and byte spans below 2 GiB, else AGMI_ERR_UNSUPPORTED (the
+ * caller then runs agmi_gemm and the elementwise kernel). */
+#define AGMI_EPILOGUE_BIAS_TANH 1
+#define AGMI_EPILOGUE_TANH_VJP 2
+typedef struct agmi_gemm_epilogue {
+    int32_t kind;
+    const void *bias;  /* [N], contiguous, or NULL */
+    void *out;         /* BIAS_TANH: [M][N] with leading dimension out_ld */
+    int64_t out_ld;
+    const void *x;     /* TANH_VJP: [M][N] with leading dimension x_ld */
+    int64_t x_ld;
+} agmi_gemm_epilogue;
+int agmi_gemm_fused(int dtype, int64_t M, int64_t N, int64_t K,
+                    const void *A, int64_t a_rs, int64_t a_cs, const void *B, int64_t b_rs, int64_t b_cs,
+                    void *C, int64_t ldc, const agmi_gemm_epilogue *e,
+                    void *workspace, size_t workspace_bytes, void *stream);
+
 /* ptr[0..n) = value (vspace zeros/ones, numpy_vspaces.py:21-25; sparse_add's zero fill,
  * core.py:212-215). */
 int agmi_fill(int dtype, void *ptr, int64_t n, double value, void *stream);

@@ -1449,3 +1449,44 @@ def test_device_resident_row_index_gathers_and_scatters_in_order(dnp, dtype):
         want = A.copy()
         onp.add.at(want, idx, x)
         assert onp.array_equal(W.scatter_add(dnp.asarray(A) + 0.0, d_idx, dnp.asarray(x)).numpy(), want), n
+
+
+# ---- dense-layer epilogues of the contraction ------------------------------------------------------
+@pytest.mark.parametrize("M,N,K", [(64, 64, 32), (200, 130, 70), (256, 512, 641), (1024, 1024, 784), (7, 3, 5)])
+def test_gemm_epilogues_equal_the_separate_kernels(dnp, M, N, K):
+    """``agmi_gemm_fused``: tanh(A.B + bias) and (G.W^T) / cosh(x + bias)**2 formed inside the contraction are, bit for
+    bit, what the product followed by the elementwise kernels gives (examples/neural_net.py:33-35,
+    autograd/numpy/numpy_vjps.py:178)."""
+    from autograd_amd import _lib
+    from autograd_amd._lib import Op
+    from autograd_amd.numpy import devarray as D
+
+    rs = onp.random.RandomState(M + N + K)
+    A = P(dnp, rs.randn(M, K).astype(F32))
+    B = P(dnp, (0.1 * rs.randn(K, N)).astype(F32))
+    bias = P(dnp, rs.randn(N).astype(F32))
+    x = P(dnp, rs.randn(M, N).astype(F32))
+    code = _lib.DTYPE_CODE[onp.dtype(F32)]
+    for operands in ((A._t, B._t), (P(dnp, rs.randn(K, M).astype(F32))._t.t(), B._t), (A._t, P(dnp, rs.randn(N, K).astype(F32))._t.t())):
+        a, b = operands
+        plain = DevArray_from(D.gemm2d(a, b, onp.dtype(F32)))
+        for with_bias in (True, False):
+            vec = bias._t if with_bias else None
+            z = D.map_op(Op.ADD, onp.dtype(F32), plain, bias) if with_bias else plain
+            want_act = D.plain(D.map_op(Op.TANH, onp.dtype(F32), z)).numpy()
+            C = _lib.empty((M, N), onp.dtype(F32))
+            act = _lib.empty((M, N), onp.dtype(F32))
+            assert _lib.gemm_fused(code, a, b, C, _lib.EPILOGUE_BIAS_TANH, bias=vec, out=act)
+            assert onp.array_equal(C.cpu().numpy(), plain.numpy())
+            assert onp.array_equal(act.cpu().numpy(), want_act)
+            zx = D.map_op(Op.ADD, onp.dtype(F32), x, bias) if with_bias else x
+            want_vjp = D.plain(D.map_op(Op.TANH_VJP, onp.dtype(F32), plain, zx)).numpy()
+            out = _lib.empty((M, N), onp.dtype(F32))
+            assert _lib.gemm_fused(code, a, b, out, _lib.EPILOGUE_TANH_VJP, bias=vec, x=x._t)
+            assert onp.array_equal(out.cpu().numpy(), want_vjp)
+
+
+def DevArray_from(t):
+    from autograd_amd.numpy.devarray import DevArray
+
+    return DevArray(t)
