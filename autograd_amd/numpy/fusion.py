@@ -160,15 +160,22 @@ def make(op, dtype, xs):
     if wide > 6:
         return None  # more axes than the strided kernels index when none of them merge: said at once, by the ordinary path
     cone = 1
-    for x in args:
-        if type(x) is float:
+    for k, x in enumerate(args):
+        kind = type(x)
+        if kind is float:
             continue
-        if type(x) is ExprArray and x._args is not None:
+        if kind is ExprArray and x._args is not None:
             if x._shape != shape:
                 x._t  # a pending operand is written out before it is broadcast: programs work on one shape
             else:
                 cone += x._cone
         x._borrowed = True  # read when the result is evaluated: in-place accumulation and item assignment must not reach it
+        # an item assignment into a borrowed array moves THAT handle to a buffer of its own: the node keeps a handle on
+        # the memory as it is now
+        if kind is DevArray:
+            args[k] = DevArray(x._t, dtype)
+        elif kind is LazyDevArray:
+            args[k] = LazyDevArray(x._raw, dtype, x._scale, x._shift, x._ascale, x._producer)
     if cone > MAX_CONE:
         node = ExprArray(op, tuple(args), shape, dtype, cone)
         cone = node._cone = len(_post_order((node,)))

@@ -1,0 +1,274 @@
+"""Elementwise chains evaluated as one launch (``agmi_program``, ``autograd_amd/numpy/fusion.py``).
+
+The fused evaluation must give, bit for bit, what the same steps give when every rule is launched on its own
+(``fusion.ENABLED = False``): each instruction of a program is the one-rule kernel's functor, rounded on its own.
+Checked here on the workloads the chains come from (config 1: tanh to third order, reference
+examples/tanh.py:22-23; config 5: Rosenbrock Hessian-vector products through ``x[1:]`` / ``x[:-1]`` and their scattered
+cotangents, autograd/numpy/numpy_vjps.py:919-950), on seeded random programs, and at the C ABI (argument checking,
+shifted leaves, range masks, row layouts, ragged extents).
+"""
+
+import numpy as onp
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+from cases_random import make_program  # noqa: E402  (tests/golden is on sys.path, see conftest.py)
+
+F32, F64 = onp.dtype("float32"), onp.dtype("float64")
+
+
+@pytest.fixture()
+def dnp():
+    import autograd_amd.numpy as dnp
+
+    return dnp
+
+
+class unfused:
+    """``with unfused(): ...``: every elementwise step is launched on its own, as before chains were deferred."""
+
+    def __enter__(self):
+        from autograd_amd.numpy import fusion
+
+        self.was, fusion.ENABLED = fusion.ENABLED, False
+
+    def __exit__(self, *exc):
+        from autograd_amd.numpy import fusion
+
+        fusion.ENABLED = self.was
+
+
+def _both_ways(fn):
+    from autograd_amd.numpy import fusion
+
+    assert fusion.ENABLED
+    before = dict(fusion.COUNTS)
+    fused = fn()
+    ran = {k: fusion.COUNTS[k] - before[k] for k in before}
+    with unfused():
+        plain = fn()
+    return fused, plain, ran
+
+
+def _same_bits(a, b):
+    a, b = onp.asarray(a), onp.asarray(b)
+    return a.shape == b.shape and a.dtype == b.dtype and onp.array_equal(a, b, equal_nan=True)
+
+
+# ---- the workloads ---------------------------------------------------------------------------------
+@pytest.mark.parametrize("order", ["d1", "d2", "d3"])
+@pytest.mark.parametrize("n", [4099, 1 << 20])
+def test_tanh_orders_fused_equal_unfused(order, n):
+    from autograd_amd import configs
+
+    be = configs.device_backend()
+    x = be.put(configs.tanh_inputs(n=n)["x"])
+    f = configs.tanh_program(be)[order]
+    fused, plain, ran = _both_ways(lambda: be.get(f(x)))
+    assert _same_bits(fused, plain)
+    # launches: one program for the first two orders, a handful for the third
+    assert ran["programs"] <= {"d1": 1, "d2": 1, "d3": 6}[order] and ran["single"] == 0 and ran["unfused"] == 0
+
+
+@pytest.mark.parametrize("which", ["grad", "hvp_rev", "hvp_fwd"])
+@pytest.mark.parametrize("n", [4097, 1 << 20])
+def test_rosenbrock_fused_equals_unfused(which, n):
+    from autograd_amd import configs
+
+    be = configs.device_backend()
+    inp = configs.rosen_inputs(n=n)
+    x, v = be.put(inp["x"]), be.put(inp["v"])
+    p = configs.rosen_program(be)
+    call = (lambda: be.get(p["grad"](x))) if which == "grad" else (lambda: be.get(p[which](x, v)))
+    fused, plain, ran = _both_ways(call)
+    assert _same_bits(fused, plain)
+    # slices of x and the cotangents scattered back through them stay inside ONE program
+    assert ran["programs"] == 1 and ran["single"] == 0 and ran["unfused"] == 0
+
+
+def test_mlp_gradient_fused_equals_unfused():
+    """Dense layers: bias + tanh in the forward contraction's epilogue, the tanh rule in the cotangent contraction's."""
+    from autograd_amd import configs
+    from autograd_amd.numpy import fusion
+
+    be = configs.device_backend()
+    inp = configs.mlp_inputs(batch=192, layer_sizes=(100, 256, 128, 10), seed=3)
+    rs = onp.random.RandomState(0)
+    params = [(be.put(W), be.put((0.1 * rs.randn(*b.shape)).astype(b.dtype))) for W, b in inp["params"]]
+    X, T = be.put(inp["X"]), be.put(inp["T"])
+    g = configs.mlp_program(be)["grad"]
+
+    def run():
+        return [tuple(be.get(a) for a in layer) for layer in g(params, X, T)]
+
+    fused, plain, ran = _both_ways(run)
+    assert ran["layers"] == 4  # two hidden layers forward, two backward
+    for lf, lp in zip(fused, plain):
+        for a, b in zip(lf, lp):
+            assert _same_bits(a, b)
+
+
+@pytest.mark.parametrize("dtype", [F64, F32])
+def test_random_programs_fused_equal_unfused(dtype, dnp):
+    import autograd_amd as ag
+    from autograd_amd.scipy.special import logsumexp as dlse
+
+    checked = 0
+    for seed in range(300, 380):
+        program, inputs = make_program(seed)
+        dev = [dnp.asarray(a.astype(dtype)) for a in inputs]
+        argnums = tuple(range(len(dev)))
+        call = lambda: [g.numpy() for g in ag.grad(lambda *xs: program(dnp, dlse, *xs), argnums)(*dev)]  # noqa: E731
+        fused, plain, _ = _both_ways(call)
+        for k, (a, b) in enumerate(zip(fused, plain)):
+            assert _same_bits(a, b), (seed, k)
+        checked += 1
+    assert checked == 80
+
+
+def test_forward_values_fused_equal_unfused(dnp):
+    """Values, not only cotangents: pending chains read by reductions, contractions, slices and the host."""
+    rs = onp.random.RandomState(5)
+    a, b = rs.randn(257, 130), rs.rand(130) + 0.5
+    A, B = dnp.asarray(a), dnp.asarray(b)
+
+    def run():
+        y = dnp.exp(-A * A) / (1.0 + dnp.sqrt(dnp.abs(A) + B))   # a chain with a broadcast row
+        z = dnp.tanh(y) * y - dnp.log1p(y * y)
+        return [z.numpy(), dnp.sum(z, axis=0).numpy(), dnp.dot(z, z.T)[:3].numpy(), (z[10:20] + 1.0).numpy(),
+                float(dnp.max(z)), dnp.where(z > 0.1, z, -z).numpy()]
+
+    fused, plain, ran = _both_ways(run)
+    assert ran["programs"] >= 1
+    for f, p in zip(fused, plain):
+        assert _same_bits(f, p)
+
+
+def test_a_long_chain_is_cut_into_programs(dnp):
+    from autograd_amd.numpy import fusion
+
+    x = dnp.asarray(onp.linspace(0.1, 1.0, 5000))
+
+    def run():
+        y = x
+        for k in range(400):  # more steps than one program holds
+            y = y * 1.01 + dnp.sin(y) if k % 7 == 0 else y * 0.99 + 0.001
+        return y.numpy()
+
+    fused, plain, ran = _both_ways(run)
+    assert _same_bits(fused, plain)
+    assert 2 <= ran["programs"] <= 40 and ran["instructions"] >= 400
+
+
+def test_leaves_are_not_written_while_an_expression_reads_them(dnp):
+    """A pending expression reads its operands when it is evaluated: item assignment into one of them in between
+    goes to a buffer of its own (NumPy semantics: ``y`` was computed before the write)."""
+    x = dnp.asarray(onp.arange(8.0))
+    y = dnp.exp(x) + x          # pending
+    x[0] = 100.0                # must not reach y
+    assert onp.array_equal(y.numpy(), onp.exp(onp.arange(8.0)) + onp.arange(8.0))
+    assert float(x[0]) == 100.0
+
+
+# ---- the entry point ---------------------------------------------------------------------------------
+def W(op, dst, a=0, b=0, c=0, d=0):
+    return op | dst << 8 | a << 12 | b << 16 | c << 20 | d << 24
+
+
+@pytest.mark.parametrize("dtype", [F64, F32])
+@pytest.mark.parametrize("shape", [(1,), (3, 7), (1000003,), (1024, 1000), (5, 3, 130), (513, 2)])
+def test_program_equals_the_one_rule_kernels(dtype, shape):
+    from autograd_amd import _lib
+    from autograd_amd._lib import Op
+    from autograd_amd.numpy import devarray as D
+
+    n = int(onp.prod(shape))
+    x = D.from_numpy(onp.linspace(-3, 3, n).astype(dtype).reshape(shape))
+    y = D.from_numpy(onp.random.RandomState(1).rand(*shape).astype(dtype) + 0.5)
+    nreg = 8 if dtype == F64 else 16
+    two, one = nreg - 1, nreg - 2
+    # r2 = exp(x * 2) ; r3 = (1 - r2) / y ; r2 = -1 * r3 * x / y**2 (div rule) ; out0 = r3 + r2, out1 = tanh(r3)
+    words = [W(Op.MUL, 2, 0, two), W(Op.EXP, 2, 2), W(Op.SUB, 3, one, 2), W(Op.DIV, 3, 3, 1), W(Op.DIV_VJP1, 2, one, 3, 1),
+             W(Op.ADD, 2, 3, 2), W(Op.TANH, 3, 3), W(_lib.PROGRAM_STORE, 2, 2, 0), W(_lib.PROGRAM_STORE, 3, 3, 1)]
+    out0, out1 = _lib.empty(shape, dtype), _lib.empty(shape, dtype)
+    assert _lib.program(_lib.DTYPE_CODE[dtype], shape, (out0, out1), (x._t, y._t), [2.0, 1.0], words, nreg)
+    from autograd_amd.numpy import fusion
+
+    with unfused():
+        m = lambda op, *xs: D.map_op(op, dtype, *xs)  # noqa: E731
+        r2 = m(Op.EXP, m(Op.MUL, x, D.full((), 2.0, dtype)))
+        r3 = m(Op.DIV, m(Op.SUB, D.full((), 1.0, dtype), r2), y)
+        want0 = m(Op.ADD, r3, m(Op.DIV_VJP1, D.full((), 1.0, dtype), r3, y)).numpy()
+        want1 = m(Op.TANH, r3).numpy()
+    assert fusion.ENABLED
+    assert onp.array_equal(out0.cpu().numpy(), want0) and onp.array_equal(out1.cpu().numpy(), want1)
+
+
+@pytest.mark.parametrize("dtype", [F64, F32])
+def test_program_row_and_column_broadcasts(dtype):
+    from autograd_amd import _lib
+    from autograd_amd._lib import Op
+    from autograd_amd.numpy import devarray as D
+
+    for rows, cols in ((512, 1024), (37, 1001), (4, 5), (1, 300), (300, 1)):
+        rs = onp.random.RandomState(rows + cols)
+        A = D.from_numpy(rs.randn(rows, cols).astype(dtype))
+        b = D.from_numpy(rs.randn(cols).astype(dtype))
+        c = D.from_numpy(rs.randn(rows, 1).astype(dtype))
+        with unfused():
+            want = D.map_op(Op.TANH, dtype, D.map_op(Op.ADD, dtype, D.map_op(Op.MUL, dtype, A, b), c)).numpy()
+        out = _lib.empty((rows, cols), dtype)
+        words = [W(Op.MUL, 0, 0, 1), W(Op.ADD, 0, 0, 2), W(Op.TANH, 0, 0), W(_lib.PROGRAM_STORE, 0, 0, 0)]
+        ok = _lib.program(_lib.DTYPE_CODE[dtype], (rows, cols), (out,), (A._t, b._t.expand(rows, cols), c._t.expand(rows, cols)), [],
+                          words, 8)
+        assert ok and onp.array_equal(out.cpu().numpy(), want)
+        # a transposed leaf has no unit stride along the rows: reported, nothing launched
+        At = D.from_numpy(rs.randn(cols, rows).astype(dtype))._t.t()
+        if rows > 1 and cols > 1:
+            assert not _lib.program(_lib.DTYPE_CODE[dtype], (rows, cols), (out,), (At, b._t.expand(rows, cols), c._t.expand(rows, cols)),
+                                    [], words, 8)
+
+
+@pytest.mark.parametrize("dtype", [F64, F32])
+@pytest.mark.parametrize("n", [5, 515, 4096, 100003])
+def test_program_shifted_leaves_and_masks(dtype, n):
+    """out[i] = x[i-1] * x[i+1] inside [1, n-1), and -x[i] outside: leaves read at moved addresses, one select."""
+    from autograd_amd import _lib
+    from autograd_amd._lib import Op
+    from autograd_amd.numpy import devarray as D
+
+    xh = onp.random.RandomState(n).randn(n).astype(dtype)
+    x = D.from_numpy(xh)
+    want = -xh.copy()
+    want[1:n - 1] = xh[:n - 2] * xh[2:]
+    words = [W(Op.MUL, 3, 0, 1), W(Op.NEG, 4, 2), W(_lib.PROGRAM_MASK, 3, 3, 0, 4), W(_lib.PROGRAM_STORE, 3, 3, 0)]
+    out = _lib.empty((n,), dtype)
+    t = x._t
+    shifted = [(-1, 1, n + 1), (1, -1, n - 1), (0, 0, n)]   # (shift, first readable index, one past the last)
+    assert _lib.program(_lib.DTYPE_CODE[dtype], (n,), (out,), (t, t, t), [], words, 8, shifted, [(1, n - 1)])
+    assert onp.array_equal(out.cpu().numpy(), want)
+
+
+def test_program_arguments_are_checked():
+    from autograd_amd import _lib
+    from autograd_amd._lib import AgmiError, Op
+    from autograd_amd.numpy import devarray as D
+
+    x = D.from_numpy(onp.ones(64))
+    out = _lib.empty((64,), F64)
+    code = _lib.DTYPE_CODE[F64]
+    store = W(_lib.PROGRAM_STORE, 1, 1, 0)
+    with pytest.raises(AgmiError, match="holds nothing"):      # reads a register nothing wrote
+        _lib.program(code, (64,), (out,), (x._t,), [], [W(Op.ADD, 1, 0, 5), store], 8)
+    with pytest.raises(AgmiError, match="unknown op"):
+        _lib.program(code, (64,), (out,), (x._t,), [], [W(200, 1, 0, 0), store], 8)
+    with pytest.raises(AgmiError, match="not every output"):
+        _lib.program(code, (64,), (out,), (x._t,), [], [W(Op.NEG, 1, 0)], 8)
+    with pytest.raises(AgmiError, match="range"):              # a mask that was not passed
+        _lib.program(code, (64,), (out,), (x._t,), [], [W(_lib.PROGRAM_MASK, 1, 0, 2, 0), store], 8)
+    with pytest.raises(AgmiError, match="registers"):          # more leaves and immediates than registers
+        _lib.program(code, (64,), (out,), (x._t,) * 5, [1.0] * 4, [W(Op.NEG, 1, 0), store], 8)
+    # what the checks let through runs
+    assert _lib.program(code, (64,), (out,), (x._t,), [], [W(Op.NEG, 1, 0), store], 8)
+    assert onp.array_equal(out.cpu().numpy(), -onp.ones(64))
