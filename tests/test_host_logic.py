@@ -169,11 +169,21 @@ def test_scalar_arithmetic_folds_into_a_pending_map_only_when_exact():
     # (a far power of two is exact by itself, but merged with its inverse it would hide the eager underflow:
     # (x * 2**-60) * 2**60 is 0 for a float32 1e-30 in NumPy, and must be two passes here too)
     assert state(x * 2.0**-60) == (2.0**-60, None)
+    from autograd_amd.numpy import fusion
+
     for expr in (lambda: (x * 3.0) * 5.0, lambda: (x + 1.0) * 3.0, lambda: (x + 1.0) + 1.0, lambda: 2.0 / x,
                  lambda: x / 3.0, lambda: x * onp.float64(3.0), lambda: (x * 2.0**-60) * 2.0**60,
                  lambda: (x * 3.0) * 2.0**40, lambda: (x + 1.0) * 2.0**9):
-        with pytest.raises(Exception):
-            expr()
+        # a step of its own: a pending expression node while chains are deferred (nothing is launched yet) ...
+        node = expr()
+        assert type(node) is fusion.ExprArray and node.shape == (4, 6) and node._cone == 1
+        # ... and an immediate launch otherwise
+        was, fusion.ENABLED = fusion.ENABLED, False
+        try:
+            with pytest.raises(Exception):
+                expr()
+        finally:
+            fusion.ENABLED = was
     # float32: scalars are rounded to the array's dtype first, as NumPy's weak scalars are
     y = meta((5,), torch.float32)
     assert state(y * 0.1) == (float(onp.float32(0.1)), None) and (y * 0.1).dtype == onp.float32
@@ -196,8 +206,16 @@ def test_accumulators_never_write_through_a_pending_map(monkeypatch):
     acc = vs._mut_add(vs.zeros(), g)  # 0 + g borrows g, pending map included
     assert type(acc) is LazyDevArray and acc._borrowed and acc._raw.data_ptr() == x._t.data_ptr()
     assert not is_shared_zero(acc)
-    with pytest.raises(Exception):  # next contribution goes out of place -> needs a launch -> no device here
-        vs._mut_add(acc, x)
+    from autograd_amd.numpy import fusion
+
+    later = vs._mut_add(acc, x)  # the next contribution goes out of place: a pending sum that reads both, writes neither
+    assert type(later) is fusion.ExprArray and later is not acc
+    was, fusion.ENABLED = fusion.ENABLED, False
+    try:
+        with pytest.raises(Exception):  # launched at once when chains are not deferred -> no device here
+            vs._mut_add(acc, x)
+    finally:
+        fusion.ENABLED = was
     with pytest.raises(TypeError):
         D.map_op(0, x.dtype, x, out=g)
 
@@ -229,10 +247,19 @@ def test_broadcast_operands_fold_into_pending_maps():
     V2 = W.reshape(A * b, (4, 2, 6))
     assert type(V2) is LazyDevArray and V2._ascale.stride() == (0, 0, 1)
     # not exact or not expressible in that order: these must launch (no device here -> raise)
+    from autograd_amd.numpy import fusion
+
     for expr in (lambda: (A * b) * 3.0, lambda: (A + c) * b, lambda: (A + c) + b, lambda: (A * b) * b, lambda: A - c,
-                 lambda: A / b, lambda: -(A + c), lambda: A * meta((8, 6), torch.float64), lambda: A * meta((6,), torch.float32)):
-        with pytest.raises(Exception):
-            expr()
+                 lambda: A / b, lambda: -(A + c), lambda: A * meta((8, 6), torch.float64)):
+        assert type(expr()) is fusion.ExprArray  # a step of its own: pending while chains are deferred
+    was, fusion.ENABLED = fusion.ENABLED, False
+    try:
+        for expr in (lambda: (A * b) * 3.0, lambda: (A + c) * b, lambda: (A + c) + b, lambda: (A * b) * b, lambda: A - c,
+                     lambda: A / b, lambda: -(A + c), lambda: A * meta((8, 6), torch.float64), lambda: A * meta((6,), torch.float32)):
+            with pytest.raises(Exception):
+                expr()
+    finally:
+        fusion.ENABLED = was
 
 
 def test_pending_products_are_contracted_into_an_accumulator_of_its_own(monkeypatch):
@@ -263,9 +290,15 @@ def test_pending_products_are_contracted_into_an_accumulator_of_its_own(monkeypa
     borrowed = D.alias(acc)
     borrowed._borrowed = True
     third = D.PendingProduct(left, right, onp.dtype("float64"))
-    with pytest.raises(Exception):  # the out-of-place add would launch a kernel: there is no CPU fallback
-        vs._mut_add(borrowed, third)
-    assert ("gemm", True, 1.0) not in calls[2:] and third.computed()
+    from autograd_amd.numpy import fusion
+
+    was, fusion.ENABLED = fusion.ENABLED, False
+    try:
+        with pytest.raises(Exception):  # the out-of-place add would launch a kernel: there is no CPU fallback
+            vs._mut_add(borrowed, third)
+    finally:
+        fusion.ENABLED = was
+    assert ("gemm", True, 1.0) not in calls[2:]
     # reading the value computes it once and keeps it
     fourth = D.PendingProduct(left, right, onp.dtype("float64"))
     n = len(calls)
