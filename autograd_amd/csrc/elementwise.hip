@@ -366,7 +366,7 @@ static int launch_ew(const char *fname, const Merged &m, int n_out, const agmi_a
     if (m.ndim == 1 && inner_unit) {
         const int64_t blocks = ceil_div(ceil_div(m.n, V), kBlock);
         if (int rc = check_blocks(blocks)) return rc;
-        set_kernel_name("ew_flat<%s>", fname);
+        set_kernel_name("ew_flat<%s>[%lld]", fname, (long long)m.n);
         with_naux([&](auto na) {
             hipLaunchKernelGGL((ew_flat<F, T, decltype(na)::value>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p);
         });
@@ -383,7 +383,7 @@ static int launch_ew(const char *fname, const Merged &m, int n_out, const agmi_a
             blocks = tiles * m.shape[0];
         }
         if (int rc = check_blocks(blocks)) return rc;
-        set_kernel_name("ew_rows<%s>", fname);
+        set_kernel_name("ew_rows<%s>[%lldx%lld]", fname, (long long)m.shape[0], (long long)m.shape[1]);
         if (total < 0x7fffffffLL)
             with_naux([&](auto na) {
                 hipLaunchKernelGGL((ew_rows<F, T, unsigned, decltype(na)::value>), dim3((unsigned)blocks), dim3(kBlock), 0,
@@ -397,7 +397,7 @@ static int launch_ew(const char *fname, const Merged &m, int n_out, const agmi_a
     } else {
         const int64_t blocks = ceil_div(m.n, kBlock);
         if (int rc = check_blocks(blocks)) return rc;
-        set_kernel_name("ew_nd<%s>", fname);
+        set_kernel_name("ew_nd<%s>[%lld]", fname, (long long)m.n);
         if (m.n < 0x7fffffffLL)
             with_naux([&](auto na) {
                 hipLaunchKernelGGL((ew_nd<F, T, unsigned, decltype(na)::value>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p);

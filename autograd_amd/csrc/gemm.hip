@@ -818,8 +818,8 @@ static int launch_gemm(GemmParams p, int64_t batch, hipStream_t s, void *ws = nu
     // how each operand's 4-element groups lie in memory (see SlabLoader)
     const int mode_a = (p.a_rs == 1 && p.M % 4 == 0) ? kXC : ((p.a_cs == 1 && p.K % 4 == 0) ? kKC : kGen);
     const int mode_b = (p.b_cs == 1 && p.N % 4 == 0) ? kXC : ((p.b_rs == 1 && p.K % 4 == 0) ? kKC : kGen);
-    set_kernel_name("gemm_mfma<%s,%d,%d,%d,%s%s>", sizeof(typename MF::elem_t) == 4 ? "f32" : "f64", BM, BN, BK, mode_name(mode_a),
-                    mode_name(mode_b));
+    set_kernel_name("gemm_mfma<%s,%d,%d,%d,%s%s>[%lldx%lldx%lld]", sizeof(typename MF::elem_t) == 4 ? "f32" : "f64", BM, BN, BK,
+                    mode_name(mode_a), mode_name(mode_b), (long long)p.M, (long long)p.N, (long long)p.K);
     // Few tiles but a long K (skinny outputs, small batches of a recurrent net): cut K across blocks so
     // the machine fills up; partial tiles go to the workspace and are summed in split order.
     p.splits = 1;
@@ -837,8 +837,8 @@ static int launch_gemm(GemmParams p, int64_t batch, hipStream_t s, void *ws = nu
     }
     const dim3 grid((unsigned)(tm * tn), (unsigned)batch, (unsigned)p.splits);
     if (p.splits > 1)
-        set_kernel_name("gemm_mfma<%s,%d,%d,%d,%s%s>+split%d", sizeof(T) == 4 ? "f32" : "f64", BM, BN, BK,
-                        mode_name(mode_a), mode_name(mode_b), p.splits);
+        set_kernel_name("gemm_mfma<%s,%d,%d,%d,%s%s>+split%d[%lldx%lldx%lld]", sizeof(T) == 4 ? "f32" : "f64", BM, BN, BK,
+                        mode_name(mode_a), mode_name(mode_b), p.splits, (long long)p.M, (long long)p.N, (long long)p.K);
     if (mode_a == kXC)
         launch_mode_b<MF, BM, BN, BK, DEPTH, KS, kXC>(mode_b, p, grid, s);
     else if (mode_a == kKC)
@@ -897,10 +897,12 @@ static int launch_direct(GemmParams p, int64_t batch, hipStream_t s, void *ws, s
         }
     }
     if (p.splits > 1)
-        set_kernel_name("gemm_direct<f32,64,64,32,%s%s>+split%d", mode_name(mode_a), mode_name(mode_b), p.splits);
+        set_kernel_name("gemm_direct<f32,64,64,32,%s%s>+split%d[%lldx%lldx%lld]", mode_name(mode_a), mode_name(mode_b), p.splits,
+                        (long long)p.M, (long long)p.N, (long long)p.K);
     else
-        set_kernel_name("gemm_direct<f32,64,64,32,%s%s%s>", mode_name(mode_a), mode_name(mode_b),
-                        p.epi == 1 ? ",+bias,tanh" : (p.epi == 2 ? ",tanh_vjp" : ""));
+        set_kernel_name("gemm_direct<f32,64,64,32,%s%s%s>[%lldx%lldx%lld]", mode_name(mode_a), mode_name(mode_b),
+                        p.epi == 1 ? ",+bias,tanh" : (p.epi == 2 ? ",tanh_vjp" : ""), (long long)p.M, (long long)p.N,
+                        (long long)p.K);
     const dim3 grid((unsigned)(tm * tn), (unsigned)batch, (unsigned)p.splits);
     const dim3 block(kDirectThreads);
     const bool tail = p.K % 4 != 0 && (mode_a == kKC || mode_b == kKC);

@@ -552,7 +552,8 @@ extern "C" int agmi_program(int dtype, int ndim, const int64_t *shape, int n_out
     for (int i = 0; i < n_instr; ++i) p.code[i] = code[i];
     p.code[n_instr] = 0;
     hipStream_t s = as_stream(stream);
-    set_kernel_name("ew_program<%s,%d,%s>[%d]", dtype == AGMI_F32 ? "float" : "double", nreg, light ? "light" : "full", n_instr);
+    set_kernel_name("ew_program<%s,%d,%s>[%d instr, %lldx%lld]", dtype == AGMI_F32 ? "float" : "double", nreg,
+                    light ? "light" : "full", n_instr, (long long)rows, (long long)p.cols);
     return dtype == AGMI_F32 ? program_part_f32(nreg, light, p, rows, s) : program_part_f64(nreg, light, p, rows, s);
 }
 #endif  // AGMI_PART == 32

@@ -627,7 +627,7 @@ static int launch_reduce(const char *fname, const RedParams &base, bool vec_ok, 
             set_error("map_reduce: too many rows");
             return AGMI_ERR_UNSUPPORTED;
         }
-        set_kernel_name("red_row_group<%s>", fname);
+        set_kernel_name("red_row_group<%s>[%lldx%lld]", fname, (long long)p.O, (long long)p.R);
         hipLaunchKernelGGL((red_row_group<F, AccT, T>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p, pl.G);
     } else if (pl.row_form) {
         if (p.O > 0x7fffffffLL) {
@@ -639,7 +639,7 @@ static int launch_reduce(const char *fname, const RedParams &base, bool vec_ok, 
             const bool unit = p.istr[0][1] == 1 || p.r_chunk == 1;
             const int v = (pl.V > 1 && unit) ? VEC : 1;
             if (!(p.scalar_mask & 1u) && p.r_chunk <= static_cast<int64_t>(kBlock) * v * kLseIters) {
-                set_kernel_name("lse_row_block%s", two_stage ? "+red_finish" : "");
+                set_kernel_name("lse_row_block%s[%lldx%lld]", two_stage ? "+red_finish" : "", (long long)p.O, (long long)p.R);
                 const int64_t need = ceil_div(p.r_chunk, static_cast<int64_t>(kBlock) * v);
                 // form of the pending map: auxiliary operands that vary along the reduced axis need registers
                 int mode = 0;
@@ -683,7 +683,7 @@ static int launch_reduce(const char *fname, const RedParams &base, bool vec_ok, 
                 goto launched;
             }
         }
-        set_kernel_name("red_row_block<%s>%s", fname, two_stage ? "+red_finish" : "");
+        set_kernel_name("red_row_block<%s>%s[%lldx%lld]", fname, two_stage ? "+red_finish" : "", (long long)p.O, (long long)p.R);
 #define AGMI_ROW(VV)                                                                                          \
     do {                                                                                                      \
         if (two_stage)                                                                                        \
@@ -703,7 +703,7 @@ static int launch_reduce(const char *fname, const RedParams &base, bool vec_ok, 
             set_error("map_reduce: too many outputs");
             return AGMI_ERR_UNSUPPORTED;
         }
-        set_kernel_name("red_short<%s>", fname);
+        set_kernel_name("red_short<%s>[%lldx%lldx%lld]", fname, (long long)p.O, (long long)p.R, (long long)p.I);
         if (pl.V > 1)
             hipLaunchKernelGGL((red_short<F, AccT, T, VEC>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p, i_vecs);
         else
@@ -716,7 +716,7 @@ static int launch_reduce(const char *fname, const RedParams &base, bool vec_ok, 
         }
         const dim3 grid((unsigned)blocks_x, (unsigned)(p.O * pl.n_chunks));
         const size_t smem = (kBlock / pl.TX > 1) ? sizeof(acc_t) * kBlock * pl.V : 0;
-        set_kernel_name("red_cols<%s>%s", fname, two_stage ? "+red_finish" : "");
+        set_kernel_name("red_cols<%s>%s[%lldx%lldx%lld]", fname, two_stage ? "+red_finish" : "", (long long)p.O, (long long)p.R, (long long)p.I);
 #define AGMI_COL(VV)                                                                                          \
     do {                                                                                                      \
         if (two_stage)                                                                                        \

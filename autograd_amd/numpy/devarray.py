@@ -573,6 +573,15 @@ def plain(x):
 _DEFERRED = (LazyDevArray, PendingProduct, LseCotangent, FusedResult)
 
 
+def in_memory(x):
+    """``x`` as a plain device array when its value already lies in memory (a deferred value that has been
+    computed: no launch, no copy); ``x`` itself otherwise."""
+    kind = type(x)
+    if kind is DevArray or kind is LazyDevArray or kind not in _DEFERRED:
+        return x
+    return DevArray(x._t, x.dtype) if _has_value(x) else x
+
+
 def alias(x):
     """A second handle on ``x``'s storage (and pending map)."""
     return x._view(lambda t: t)
@@ -967,8 +976,10 @@ def map_op(op, dtype, *xs, out=None, n_out=1):
         fuse = n_out == 1 and _fusion is not None and _fusion.ENABLED
         if fuse:
             for x in xs:
-                if type(x) is _fusion.ExprArray and x._args is not None:
-                    node = _fusion.make(op, dtype, xs)  # (an operand that is itself pending: no map can be folded into it)
+                if (type(x) is _fusion.ExprArray and x._args is not None) or (type(x) is PendingReduce and x._call is not None):
+                    # an operand that is itself pending (an expression, or a reduction of one: the value of a traced
+                    # loss, which `grad` never reads): no map can be folded into it
+                    node = _fusion.make(op, dtype, xs)
                     if node is not None:
                         return node
                     break
@@ -1026,7 +1037,7 @@ def astype_copy(x):
 
 
 def contiguous(x):
-    x = plain(x) if type(x) is PendingProduct else x  # a computed product is contiguous already
+    x = plain(x) if type(x) is PendingProduct else in_memory(x)  # a computed product is contiguous already
     return x if type(x) is DevArray and x._t.is_contiguous() else copy(x)
 
 

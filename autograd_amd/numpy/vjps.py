@@ -115,7 +115,7 @@ def _consume_lse_cotangent(op, target_shape, operands):
         out = s.row_sums()
         return out if target_shape == (rows, 1) else out._view(lambda t: t.reshape(rows))
     if op == Op.MUL and len(operands) == 2 and isinstance(operands[0], DevArray) and operands[0].dtype == s.dtype:
-        y = operands[0]
+        y = D.in_memory(operands[0])
         if target_shape == (rows, cols) and type(y) is DevArray and y.shape in ((1, cols), (cols,)):
             return s.scaled_by(y._t.reshape(1, cols).expand(rows, cols))
         if target_shape in ((1, cols), (cols,)) and y.shape == (rows, cols):

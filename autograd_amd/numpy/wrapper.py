@@ -572,6 +572,8 @@ def _concat_pieces(arrs, axis, dt):
     for a in arrs:
         if a.dtype != dt:
             return None
+        if type(a) is not DevArray and type(a) is not D.LazyDevArray:
+            a = D.plain(a)  # a pending expression, product or reduction: computed now, joined from where it lands
         if type(a) is DevArray:
             t = a._t
         elif type(a) is D.LazyDevArray and a._scale == 1.0 and a._shift is None and a._ascale is None and a._producer is None:

@@ -50,6 +50,13 @@ def parse():
     return ap.parse_args()
 
 
+def end_to_end(compulsory_bytes, evals_per_sec):
+    """The secondary roofline figure of a whole evaluation: the bytes it cannot avoid (its inputs read once, its
+    results written once) over the time one evaluation takes, against the HBM peak."""
+    gbps = compulsory_bytes * evals_per_sec / 1e9
+    return {"compulsory_bytes": compulsory_bytes, "achieved_GBps": gbps, "frac": gbps / HBM_PEAK_GBS}
+
+
 def time_steps(fn, sync, steps, warmup):
     for _ in range(warmup):
         fn()
@@ -422,6 +429,13 @@ def main():
     # no per-step Python tracing; reported beside the eager figure, never as `value`
     rate = graph_rate(fun, fun_args, be.sync, args.steps)
     result["graph_replay"] = {"value": rate, "unit": "grad evals/sec", "ms_per_step": 1e3 / rate}
+    if args.workload == "bcast":
+        # the whole evaluation against its compulsory traffic: A read once, dA written once, the vectors
+        compulsory = 2 * 8192 * 4096 * 4 + 2 * (8192 + 4096) * 4
+        roofline["end_to_end"] = dict(end_to_end(compulsory, result["value"]),
+                                      graph_replay=end_to_end(compulsory, rate),
+                                      what="inputs read once + results written once per evaluation, over the time of one "
+                                           "evaluation (eager: `value`; graph_replay: the recorded evaluation replayed)")
     if not args.no_extras and args.workload == "bcast":
         result["extras"] = extras(be)
     if not args.no_cpu_baseline:
@@ -573,6 +587,21 @@ def extras(be):
     be.sync()
     out["mlp_adam_training_graph_steps_per_sec"] = steps / (time.perf_counter() - t0)
     del graphed
+    # every workload against its compulsory bytes (inputs read once + results written once): what the per-kernel
+    # figures do not show is how many passes an evaluation makes
+    n1, n5 = 4194304, 1 << 24
+    out["end_to_end"] = {
+        **{f"tanh_{k}": {"eager": end_to_end(16 * n1, out[f"tanh_{k}_evals_per_sec"]),
+                         "graph_replay": end_to_end(16 * n1, out[f"tanh_{k}_graph_evals_per_sec"])} for k in ("d1", "d2", "d3")},
+        **{f"rosen_{k}": {"eager": end_to_end(24 * n5, out[f"rosen_{k}_evals_per_sec"]),
+                          "graph_replay": end_to_end(24 * n5, out[f"rosen_{k}_graph_evals_per_sec"])} for k in ("hvp_rev", "hvp_fwd")},
+        "mlp": {"flops_per_eval": 9.794e9,
+                "eager_frac_of_mfma_peak": 9.794e9 * out["mlp_grad_evals_per_sec"] / 1e12 / MFMA_F32_PEAK_TFLOPS,
+                "graph_replay_frac_of_mfma_peak": 9.794e9 * out["mlp_grad_graph_evals_per_sec"] / 1e12 / MFMA_F32_PEAK_TFLOPS},
+        "rnn": {"flops_per_eval": 38.8e9,
+                "eager_frac_of_mfma_peak": 38.8e9 * out["rnn_grad_evals_per_sec"] / 1e12 / MFMA_F32_PEAK_TFLOPS,
+                "graph_replay_frac_of_mfma_peak": 38.8e9 * out["rnn_grad_graph_evals_per_sec"] / 1e12 / MFMA_F32_PEAK_TFLOPS},
+    }
     return out
 
 
