@@ -397,7 +397,14 @@ class _Unsupported(Exception):
 def _emit(roots):
     """``(leaf tensors, immediates, instruction words, registers, shifted, masks)`` of the program that computes
     ``roots``; None when it does not fit the kernel's limits.  ``shifted`` is None, or per leaf ``(shift, lo,
-    hi)`` when some vector is read at a shifted position (see :func:`shifted`)."""
+    hi)`` when some vector is read at a shifted position (see :func:`shifted`).
+
+    The nodes are first written down in static single assignment form, one instruction per distinct
+    subexpression, with three rewrites that change no bit of any result: negations are carried as a sign on the
+    value and absorbed by the sums, products and quotients that consume them (``(-a) + b`` is ``b - a``,
+    ``(-a) * b`` is ``-(a * b)``, a negated immediate is another immediate); a product whose only reader is a sum
+    becomes one multiply-add instruction of two roundings; ``x * 1.0`` is ``x``.  Instructions nothing reads are
+    dropped, then registers are assigned by liveness."""
     dtype = roots[0].dtype
     KNOWN = D.KNOWN_SCALARS
     n_out = roots[0]._shape[0] if len(roots[0]._shape) == 1 else None
@@ -406,11 +413,12 @@ def _emit(roots):
     leaves, leaf_ids, leaf_where = [], {}, []
     imms, imm_ids = [], {}
     masks = []
-    # a value is ("L", k) / ("I", k) / ("X", k): leaf k, immediate k, result of instruction k
+    # a value is ("L", k) / ("I", k) / ("X", k): leaf k, immediate k, result of instruction k; ("N", v) is minus v
     instrs = []   # (op, operand values, mask index or None)
     numbered = {}  # the same: one instruction for equal subexpressions
     memo = {}      # (id(node), shift) -> value
     any_shift = [False]
+    limit = 4 * _lib.PROGRAM_MAX_INSTRUCTIONS  # (before dead instructions are dropped; bounds the work on a hopeless cone)
 
     def leaf(t, shift):
         if KNOWN:
@@ -433,7 +441,7 @@ def _emit(roots):
         key = (t.data_ptr() + shift * itemsize,) if vector else (t.data_ptr(), t.stride(), tuple(t.shape))
         v = leaf_ids.get(key)
         if v is None:
-            if len(leaves) >= _lib.PROGRAM_MAX_LEAVES:
+            if len(leaves) >= 4 * _lib.PROGRAM_MAX_LEAVES:
                 raise _TooBig
             v = leaf_ids[key] = ("L", len(leaves))
             leaves.append(t)
@@ -445,31 +453,95 @@ def _emit(roots):
         key = (c, bool(onp.signbit(c))) if c == 0.0 else c  # -0.0 and 0.0 are different immediates; NaN never equals itself: not shared
         v = imm_ids.get(key)
         if v is None:
-            if len(imms) >= _lib.PROGRAM_MAX_IMMEDIATES:
-                raise _TooBig
             v = ("I", len(imms))
             if c == c:
                 imm_ids[key] = v
             imms.append(c)
         return v
 
-    def ins(op, *srcs, mask=None):
-        if op == Op.MUL:
-            # x * 1.0 is x, bit for bit (the cotangent seeds of elementwise_grad are ones)
-            if srcs[1][0] == "I" and imms[srcs[1][1]] == 1.0:
-                return srcs[0]
-            if srcs[0][0] == "I" and imms[srcs[0][1]] == 1.0:
-                return srcs[1]
-        elif op == Op.DIV and srcs[1][0] == "I" and imms[srcs[1][1]] == 1.0:
-            return srcs[0]
+    def emit(op, *srcs, mask=None):
         key = (op, srcs, mask)
         v = numbered.get(key)
         if v is None:
-            if len(instrs) >= _lib.PROGRAM_MAX_INSTRUCTIONS - len(roots):
+            if len(instrs) >= limit:
                 raise _TooBig
             v = numbered[key] = ("X", len(instrs))
             instrs.append(key)
         return v
+
+    def real(v):
+        """``v`` as a value that exists: a carried sign becomes a negation (or the negated immediate)."""
+        if v[0] != "N":
+            return v
+        base = v[1]
+        return imm(-imms[base[1]]) if base[0] == "I" else emit(Op.NEG, base)
+
+    def minus(v):
+        if v[0] == "N":
+            return v[1]
+        if v[0] == "I":
+            return imm(-imms[v[1]])
+        return ("N", v)
+
+    def signed(negative, op, *bases):
+        """``op(bases)`` with the sign its operands carried; an immediate among them takes the sign."""
+        if negative:
+            for k, b in enumerate(bases):
+                if b[0] == "I" and (op != Op.DIV_VJP1 or k < 2):
+                    flipped = bases[:k] + (imm(-imms[b[1]]),) + bases[k + 1:]
+                    return ins_plain(op, *flipped)
+            return ("N", ins_plain(op, *bases))
+        return ins_plain(op, *bases)
+
+    def ins_plain(op, *srcs):
+        if op == Op.MUL:
+            # x * 1.0 is x, bit for bit (the cotangent seeds of elementwise_grad are ones); x * -1.0 is -x
+            for me, other in ((1, 0), (0, 1)):
+                if srcs[me][0] == "I":
+                    c = imms[srcs[me][1]]
+                    if c == 1.0:
+                        return srcs[other]
+                    if c == -1.0:
+                        return minus(srcs[other])
+        elif op == Op.DIV and srcs[1][0] == "I" and imms[srcs[1][1]] == 1.0:
+            return srcs[0]
+        return emit(op, *srcs)
+
+    def ins(op, *srcs, mask=None):
+        if mask is not None:
+            inside, rest = srcs
+            if inside[0] == "N" and (rest[0] == "N" or rest[0] == "I"):
+                # a select commutes with the sign when both sides carry it (minus an immediate is an immediate)
+                return ("N", emit(op, inside[1], minus(rest), mask=mask))
+            return emit(op, real(inside), real(rest), mask=mask)
+        if op == Op.NEG:
+            return minus(srcs[0])
+        na = srcs[0][0] == "N"
+        if op == Op.ADD or op == Op.SUB:
+            a, b = srcs
+            if op == Op.SUB:
+                b = minus(b)  # a - b is a + (-b), the very same operation
+            nb = b[0] == "N"
+            if not na and not nb:
+                return emit(Op.ADD, a, b)
+            if na and nb:
+                return emit(Op.SUB, real(a), b[1])   # (-a) + (-b): one negation stays, the other becomes the subtraction
+            if na:
+                return emit(Op.SUB, b, a[1])         # (-a) + b = b - a
+            return emit(Op.SUB, a, b[1])             # a + (-b) = a - b
+        if op == Op.MUL or op == Op.DIV:
+            a, b = srcs
+            nb = b[0] == "N"
+            return signed(na != nb, op, a[1] if na else a, b[1] if nb else b)
+        if op == Op.SQUARE or op == Op.ABS:
+            return emit(op, srcs[0][1] if na else srcs[0])
+        if op == Op.RECIPROCAL:
+            return signed(na, op, srcs[0][1] if na else srcs[0])
+        if op == Op.DIV_VJP1:  # ((-g) * x) / (y * y)
+            g, x, y = srcs
+            nx = x[0] == "N"
+            return signed(na != nx, op, g[1] if na else g, x[1] if nx else x, y[1] if y[0] == "N" else y)
+        return ins_plain(op, *[real(v) for v in srcs])
 
     def masked(v, rest, lo, hi):
         rng = (lo, hi)
@@ -541,12 +613,52 @@ def _emit(roots):
         return leaf(a._t, shift)
 
     try:
-        root_values = [value(r, 0) for r in roots]
-        if not instrs:
-            # every root is a leaf or an immediate after the rewrites: one copy each keeps the kernel's contract simple
-            root_values = [ins(Op.COPY, v) for v in root_values]
+        root_values = [real(value(r, 0)) for r in roots]
+        # every root is the result of an instruction of its own (a root that came out as a leaf, an immediate or
+        # another root's value gets a copy: the kernel stores registers, and each output once)
+        seen = set()
+        for k, v in enumerate(root_values):
+            if v[0] != "X" or v in seen:
+                root_values[k] = v = emit(Op.COPY, v, mask=("root", k))
+            seen.add(v)
     except _TooBig:
         return None
+
+    # a product that only one sum reads: one multiply-add (the product rounded, then the sum rounded)
+    uses = {}
+    for _op, srcs, _mask in instrs:
+        for v in srcs:
+            uses[v] = uses.get(v, 0) + 1
+    for v in root_values:
+        uses[v] = uses.get(v, 0) + 1
+    for k, (op, srcs, mask) in enumerate(instrs):
+        if op == Op.ADD:
+            for me, other in ((0, 1), (1, 0)):
+                p = srcs[me]
+                if p[0] == "X" and uses.get(p) == 1 and instrs[p[1]][0] == Op.MUL and instrs[p[1]][2] is None:
+                    a, b = instrs[p[1]][1]
+                    instrs[k] = (Op.MUL_ADD, (a, b, srcs[other]), None)
+                    uses[p] = 0
+                    break
+    # drop what nothing reads (from the roots backwards), then number leaves, immediates and instructions anew
+    needed = set(root_values)
+    for k in range(len(instrs) - 1, -1, -1):
+        if ("X", k) in needed:
+            needed.update(instrs[k][1])
+    kept = [k for k in range(len(instrs)) if ("X", k) in needed]
+    used_leaves = [k for k in range(len(leaves)) if ("L", k) in needed]
+    used_imms = [k for k in range(len(imms)) if ("I", k) in needed]
+    if (len(kept) > _lib.PROGRAM_MAX_INSTRUCTIONS - len(roots) or len(used_leaves) > _lib.PROGRAM_MAX_LEAVES
+            or len(used_imms) > _lib.PROGRAM_MAX_IMMEDIATES):
+        return None
+    rename = {("L", k): ("L", n) for n, k in enumerate(used_leaves)}
+    rename.update({("I", k): ("I", n) for n, k in enumerate(used_imms)})
+    rename.update({("X", k): ("X", n) for n, k in enumerate(kept)})
+    instrs = [(instrs[k][0], tuple(rename[v] for v in instrs[k][1]), instrs[k][2]) for k in kept]
+    root_values = [rename[v] for v in root_values]
+    leaf_where = [leaf_where[k] for k in used_leaves]
+    leaves = [leaves[k] for k in used_leaves]
+    imms = [imms[k] for k in used_imms]
 
     n_leaf, n_imm, n_ins = len(leaves), len(imms), len(instrs)
     shifted_leaves = None
@@ -578,9 +690,6 @@ def _emit(roots):
         for k in range(n_imm):
             reg[("I", k)] = n_regs - 1 - k
         free = list(range(n_regs - 1 - n_imm, n_leaf - 1, -1))  # popped from the low end
-        for k in range(n_leaf):
-            if ("L", k) not in last:
-                free.append(k)  # (a leaf that only a rewritten-away step read)
         words = []
         ok = True
         for k, (op, srcs, mask) in enumerate(instrs):
@@ -588,16 +697,12 @@ def _emit(roots):
             for s in set(srcs):
                 if s[0] != "I" and last[s] == k:
                     free.append(reg[s])
-            v = ("X", k)
-            if v not in last:
-                dst = regs[0]  # a value nobody reads (cannot happen for nodes under a root; kept harmless)
-            elif not free:
+            if not free:
                 ok = False
                 break
-            else:
-                dst = free.pop()
-            reg[v] = dst
-            if mask is not None:
+            dst = free.pop()
+            reg[("X", k)] = dst
+            if op == _lib.PROGRAM_MASK:
                 w = op | dst << 8 | regs[0] << 12 | mask << 16 | regs[1] << 20  # inside value, range, outside value
             else:
                 w = op | dst << 8
