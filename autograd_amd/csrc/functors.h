@@ -27,10 +27,11 @@ AGMI_HEAVY_MATH double m_exp(double x) { return exp(x); }
 // overflow handling: d*log2(e) is split into an integer n and a remainder whose rounding error is
 // recovered with fused multiply-adds (log2(e) as a float pair), the hardware exp2 sees |r| <= 1/2,
 // and ldexp scales, also into the subnormals.  n is clamped so that d = -inf (and anything whose exp
-// underflows) arrives at exp2(-inf) = 0; a NaN passes through the clamp's other operand into the fma.
+// underflows) arrives at exp2(-inf) = 0 and d = +inf (a weighted logsumexp whose maximum is infinite is shifted
+// by 0, not by its maximum) at inf; a NaN passes through the clamp's other operand into the fma.
 AGMI_HEAVY_MATH float exp_of_nonpositive(float d) {
     const float kLog2eHi = 1.44269502162933349609375f, kLog2eLo = 1.92596299112661746e-8f;
-    const float n = fmaxf(rintf(d * kLog2eHi), -160.0f);
+    const float n = fminf(fmaxf(rintf(d * kLog2eHi), -160.0f), 160.0f);  // (the upper clamp only matters for d = +inf: inf, not NaN)
     float r = __builtin_fmaf(d, kLog2eHi, -n);
     r = __builtin_fmaf(d, kLog2eLo, r);
     return ldexpf(__builtin_amdgcn_exp2f(r), static_cast<int>(n));

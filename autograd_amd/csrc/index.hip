@@ -10,9 +10,19 @@
 #include <algorithm>
 #include <cstdint>
 
+#include <type_traits>
+
 #include "common.h"
 
 namespace agmi {
+
+template <typename T>
+__device__ __forceinline__ T out_of_range_fill() {
+    if constexpr (std::is_floating_point<T>::value)
+        return static_cast<T>(__builtin_nanf(""));
+    else
+        return T(0);
+}
 
 template <typename T>
 __global__ __launch_bounds__(kBlock) void take_rows_kernel(const T *__restrict__ src, int64_t n_rows, int64_t inner,
@@ -23,6 +33,12 @@ __global__ __launch_bounds__(kBlock) void take_rows_kernel(const T *__restrict__
     const int64_t i = e / inner, c = e - i * inner;
     int64_t r = index[i];
     if (r < 0) r += n_rows;
+    // An index outside [-n_rows, n_rows) never reaches memory (NumPy raises IndexError; the values of a
+    // device-resident index are not known on the host): the row reads as NaN (zero for integer arrays).
+    if (static_cast<uint64_t>(r) >= static_cast<uint64_t>(n_rows)) {
+        out[e] = out_of_range_fill<T>();
+        return;
+    }
     out[e] = src[r * inner + c];
 }
 
@@ -40,6 +56,7 @@ __global__ __launch_bounds__(kBlock) void scatter_add_runs_kernel(T *__restrict_
     const int64_t pos = e / inner, c = e - pos * inner;
     int64_t r = index[order[pos]];
     if (r < 0) r += n_rows;
+    if (static_cast<uint64_t>(r) >= static_cast<uint64_t>(n_rows)) return;  // no such row: the addends are dropped, nothing is touched
     if (pos > 0) {
         int64_t before = index[order[pos - 1]];
         if (before < 0) before += n_rows;
@@ -67,6 +84,7 @@ __global__ __launch_bounds__(kBlock) void scatter_add_rows_kernel(T *__restrict_
     const int64_t begin = seg_start[seg], end = seg_start[seg + 1];
     int64_t r = index[order[begin]];
     if (r < 0) r += n_rows;
+    if (static_cast<uint64_t>(r) >= static_cast<uint64_t>(n_rows)) return;  // no such row: the addends are dropped
     T acc = dst[r * inner + c];
     for (int64_t k = begin; k < end; ++k) acc = acc + src[order[k] * inner + c];
     dst[r * inner + c] = acc;

@@ -164,7 +164,7 @@ class LazyDevArray(DevArray):
     the value to a fresh buffer (one copy kernel) and keeps it.
     """
 
-    __slots__ = ("_raw", "_scale", "_shift", "_ascale", "_producer")
+    __slots__ = ("_raw", "_scale", "_shift", "_ascale", "_producer", "_view_of_pending")
 
     def __init__(self, raw, dtype, scale, shift, ascale=None, producer=None):
         self._raw = raw
@@ -172,6 +172,7 @@ class LazyDevArray(DevArray):
         # first needs this value runs it, possibly together with the pending steps (a dense layer's bias and
         # activation go into the contraction's epilogue, see `fusion._dense_layer`)
         self._producer = producer
+        self._view_of_pending = False  # True on a view taken of an array whose arithmetic was still pending
         self.dtype = dtype
         self._borrowed = False
         self._scale = scale    # Python float, representable in dtype; 1.0 = no multiply
@@ -246,9 +247,11 @@ class LazyDevArray(DevArray):
                 self._produce()
             return DevArray(fn(self._raw), self.dtype)  # nothing pending (the value has been written out): a plain view
         try:
-            return LazyDevArray(fn(self._raw), self.dtype, self._scale,
+            view = LazyDevArray(fn(self._raw), self.dtype, self._scale,
                                 fn(sh) if isinstance(sh, torch.Tensor) else sh,
                                 fn(asc) if asc is not None else None, self._producer)
+            view._view_of_pending = True
+            return view
         except RuntimeError:
             return DevArray(fn(self._t), self.dtype)
 

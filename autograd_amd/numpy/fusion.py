@@ -30,7 +30,11 @@ from .._lib import Op
 from . import devarray as D
 from .devarray import DevArray, LazyDevArray
 
-ENABLED = os.environ.get("AUTOGRAD_AMD_FUSE", "1").strip() not in ("0", "")
+from .. import _host
+
+# off under a hosting `autograd` (AUTOGRAD_AMD_HOST): that package's make_vjp hands cotangents back as they are, and
+# never completes a pending expression for the caller
+ENABLED = os.environ.get("AUTOGRAD_AMD_FUSE", "1").strip() not in ("0", "") and not _host.HOST
 MAX_CONE = 192  # pending nodes under one value before its largest pending operand is written out
 
 _F32 = onp.dtype("float32")

@@ -874,33 +874,70 @@ def _flat_positions(shape, idx):
 
 
 class _IndexPlan:
-    """What ``A[idx]`` with an advanced index selects from an array of one shape: the flat position in ``A`` of
-    every element of the result, resident on the device, and the stable order of those positions that the
-    ordered scatter of the cotangent needs.  Built once per (shape, index) and kept, so repeated evaluations
-    and recorded graphs do no host work and no transfers for it."""
+    """What ``A[idx]`` with an advanced index selects from an array of one shape, resident on the device, and the
+    stable order of the selection that the ordered scatter of the cotangent needs.  Built once per (shape, index)
+    and kept while the cache has room, so repeated evaluations and recorded graphs do no host work and no
+    transfers for it.
 
-    __slots__ = ("shape", "positions", "n", "_order")
+    One integer vector on the leading axis (``X[batch_rows]``) is kept as rows: ``n`` row numbers and rows of
+    ``inner`` elements each.  Every other index form is the flat position of every selected ELEMENT (``inner`` = 1).
+    """
+
+    __slots__ = ("shape", "positions", "n", "_order", "n_rows", "inner", "nbytes")
 
     def __init__(self, shape, idx):
-        flat = _flat_positions(shape, idx)
-        self.shape = flat.shape
+        rows = idx if not isinstance(idx, tuple) else (idx[0] if len(idx) == 1 else None)
+        if isinstance(rows, onp.ndarray) and rows.ndim == 1 and rows.dtype.kind in "iu" and len(shape) >= 1:
+            extent = shape[0]
+            rows = rows.astype(onp.int64)
+            if rows.size and (rows.min() < -extent or rows.max() >= extent):
+                bad = rows[(rows < -extent) | (rows >= extent)][0]
+                raise IndexError(f"index {bad} is out of bounds for axis 0 with size {extent}")
+            flat = onp.where(rows < 0, rows + extent, rows)
+            inner = 1
+            for s in shape[1:]:
+                inner *= s
+            self.shape = (flat.size,) + tuple(shape[1:])
+            self.n_rows, self.inner = extent, inner
+        else:
+            flat = _flat_positions(shape, idx)
+            self.shape = flat.shape
+            total = 1
+            for s in shape:
+                total *= s
+            self.n_rows, self.inner = total, 1
         self.n = flat.size
         self.positions = D.from_numpy(flat.reshape(-1))
         # equal destinations keep their order of appearance, which is the order numpy.add.at adds them in
         self._order = D.from_numpy(onp.argsort(flat.reshape(-1), kind="stable").astype(onp.int64))
+        self.nbytes = 16 * flat.size
 
     def order(self):
         return self._order
 
 
+_INDEX_PLAN_BYTES = [0]
+_INDEX_PLAN_BUDGET = 64 << 20      # device memory the kept plans may hold
+_INDEX_PLAN_LARGEST = 8 << 20      # a plan beyond this is built, used and dropped (fresh minibatch rows every step)
+
+
 def _index_plan(shape, idx):
     idx = _to_host_index(idx)
+    big = builtins.sum(it.nbytes for it in (idx if isinstance(idx, tuple) else (idx,)) if isinstance(it, onp.ndarray)) > (1 << 20)
+    if big:
+        return _IndexPlan(tuple(shape), idx)  # (hashing a large index costs what building the plan costs)
     key = (tuple(shape), _index_key(idx))
-    plan = _INDEX_PLANS.get(key)
+    plan = _INDEX_PLANS.pop(key, None)
     if plan is None:
-        if len(_INDEX_PLANS) >= _INDEX_PLAN_LIMIT:
-            _INDEX_PLANS.clear()
-        plan = _INDEX_PLANS[key] = _IndexPlan(tuple(shape), idx)
+        plan = _IndexPlan(tuple(shape), idx)
+        if plan.nbytes > _INDEX_PLAN_LARGEST:
+            return plan
+        _INDEX_PLAN_BYTES[0] += plan.nbytes
+        # least recently used plans make room (a dict keeps insertion order; a hit re-inserts its key at the end)
+        while _INDEX_PLANS and (_INDEX_PLAN_BYTES[0] > _INDEX_PLAN_BUDGET or len(_INDEX_PLANS) >= _INDEX_PLAN_LIMIT):
+            oldest = next(iter(_INDEX_PLANS))
+            _INDEX_PLAN_BYTES[0] -= _INDEX_PLANS.pop(oldest).nbytes
+    _INDEX_PLANS[key] = plan
     return plan
 
 
@@ -1010,7 +1047,7 @@ def take(A, idx):
             inner *= s
         return _gather(A, rows, A.shape[0], inner, (rows.size,) + A.shape[1:])
     plan = _index_plan(A.shape, idx)
-    return _gather(A, plan.positions, A.size, 1, plan.shape)
+    return _gather(A, plan.positions, plan.n_rows, plan.inner, plan.shape)
 
 
 def assign_items(A, idx, value):
@@ -1027,6 +1064,11 @@ def assign_items(A, idx, value):
         raise TypeError("a traced value cannot be assigned into an array: build the result with concatenate / where")
     D.ITEM_WRITES += 1
     if type(A) is D.LazyDevArray:
+        if A._view_of_pending and (A._scale != 1.0 or A._shift is not None or A._ascale is not None) and builtins.any(A._raw.stride()):
+            # `y = 1 - x; v = y[1:]; v[:] = 0`: in NumPy the write reaches y; here y's value does not exist in memory yet and
+            # v would get a buffer of its own.  A wrong result without a word is worse than an error.
+            raise ValueError("item assignment into a view of an array whose arithmetic is still pending would not reach "
+                             "that array; assign into the array itself, or take the view of np.settle(array)")
         A._t  # pending arithmetic (a lazy fill, say) is written out: from here on the array is its own buffer
     elif type(A) is not DevArray:
         raise TypeError("item assignment needs a plain device array; this one is a cotangent still being formed "
@@ -1160,7 +1202,11 @@ def scatter_add(A, idx, x):
             inner *= s
         if n > 65536:
             raise NotImplementedError("scatter through a device-resident index of more than 65536 entries")
-        wrapped = D.map_op(Op.REMAINDER, D._F64, D.astype(rows, D._F64), float(A.shape[0]))  # negative rows count from the end
+        # negative rows count from the end; a row outside [-n, n) stays outside (the gather reads NaN for it, the
+        # scatter drops its addends: neither touches memory)
+        as_float = D.astype(rows, D._F64)
+        wrapped = D.map_op(Op.WHERE, D._F64, D.astype(D.compare(Cmp.LT, as_float, 0.0), D._F64),
+                           D.map_op(Op.ADD, D._F64, as_float, float(A.shape[0])), as_float)
         keys = D.astype(wrapped, D._I64)
         order = D.empty((n,), D._I64)
         _lib.sort_rows(_lib.DTYPE_CODE[D._F64], D.contiguous(wrapped)._t, 1, n, None, order._t, None)
@@ -1178,7 +1224,7 @@ def scatter_add(A, idx, x):
     if src.shape != plan.shape:
         src = broadcast_to.fun(src, plan.shape)
     src = D.contiguous(D.plain(src))
-    _lib.scatter_add_rows(code, A._t, A.size, 1, src._t, plan.positions._t, plan.order()._t, None, plan.n)
+    _lib.scatter_add_rows(code, A._t, plan.n_rows, plan.inner, src._t, plan.positions._t, plan.order()._t, None, plan.n)
     return A
 
 

@@ -348,7 +348,8 @@ int agmi_gemm_fused(int dtype, int64_t M, int64_t N, int64_t K,
 int agmi_fill(int dtype, void *ptr, int64_t n, double value, void *stream);
 
 /* Gather rows: out[i, :] = src[index[i], :] for i in [0, n_index); rows have `inner` elements,
- * src has `n_rows` rows.  Negative indices count from the end.  Forward of A[idx] with an
+ * src has `n_rows` rows.  Negative indices count from the end; an index outside [-n_rows, n_rows)
+ * reads nothing: its output row is NaN (0 for integer dtypes).  Forward of A[idx] with an
  * integer-array idx on the leading axis (numpy_boxes.py:16-18). */
 int agmi_take_rows(int dtype, const void *src, int64_t n_rows, int64_t inner,
                    const int64_t *index, int64_t n_index, void *out, void *stream);
@@ -402,7 +403,8 @@ int agmi_cumsum(int dtype, const void *src, int64_t outer, int64_t n, int64_t in
  * destination in that order (n_seg runs); both are device arrays prepared by the caller.
  * seg_start may be NULL: n_seg then counts the index entries and the runs are found on the device
  * (nothing about the index needs to be known on the host: agmi_sort_rows on the index values gives
- * `order`, so a device-resident index can be scattered from inside a recorded graph). */
+ * `order`, so a device-resident index can be scattered from inside a recorded graph).
+ * An index outside [-n_rows, n_rows) names no row: its addends are dropped. */
 int agmi_scatter_add_rows(int dtype, void *dst, int64_t n_rows, int64_t inner,
                           const void *src, const int64_t *index, const int64_t *order,
                           const int64_t *seg_start, int64_t n_seg, void *stream);

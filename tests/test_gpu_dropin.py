@@ -329,6 +329,14 @@ def test_item_assignment_outside_a_trace(ag, np):
     z.T[0, 1] = 4.0
     onp.testing.assert_array_equal(_host(z), [[1.0, 1.0], [4.0, 0.0]])
 
+    # a view of an array whose arithmetic is still pending: the write could not reach that array, so it is refused
+    y = 1.0 - np.array(onp.arange(4.0))
+    v = y[1:]
+    with pytest.raises(ValueError, match="still pending"):
+        v[:] = 0.0
+    y[1:] = 0.0  # assigning into the array itself is fine
+    onp.testing.assert_array_equal(_host(y), [1.0, 0.0, 0.0, 0.0])
+
     with pytest.raises(NotImplementedError):
         d[::-1] = 1.0
     with pytest.raises(NotImplementedError):

@@ -329,6 +329,15 @@ def test_weighted_logsumexp_follows_scipy(dnp):
     got = logsumexp(dnp.asarray(x32), axis=0, b=dnp.asarray(w32))
     assert got.dtype == onp.float32
     close(got.numpy(), scipy.special.logsumexp(x32, axis=0, b=w32), 1e-5)
+    # an infinite element with weights (no shift is applied then: exp(+inf) must come out inf, not NaN), both precisions
+    for dt in (onp.float32, onp.float64):
+        xi = onp.array([[0.5, onp.inf, -1.0], [0.25, -onp.inf, 2.0]], dt)
+        wi = onp.array([1.5, 0.5, 2.0], dt)
+        with onp.errstate(all="ignore"):
+            want = scipy.special.logsumexp(xi, axis=1, b=wi)
+        got = logsumexp(dnp.asarray(xi), axis=1, b=dnp.asarray(wi)).numpy()
+        assert want[0] == onp.inf and got[0] == onp.inf and got.dtype == dt
+        close(got[1:], want[1:], 1e-6 if dt == onp.float32 else 1e-13)
 
 
 # ---- contractions -------------------------------------------------------------------------------
@@ -1490,3 +1499,48 @@ def DevArray_from(t):
     from autograd_amd.numpy.devarray import DevArray
 
     return DevArray(t)
+
+
+def test_device_resident_row_index_out_of_range_reads_nothing(dnp):
+    """A row number held on the device is not known to the host, so NumPy's IndexError cannot be raised for it: the
+    gather gives NaN rows for indices outside [-n, n), the scatter of the cotangent drops them, and neither touches
+    memory outside the array."""
+    import autograd_amd as ag
+
+    x = onp.arange(12.0).reshape(4, 3)
+    rows = onp.array([0, 7, -1, -9, 3])
+    X, R = P(dnp, x), dnp.asarray(rows)
+    got = X[R].numpy()
+    assert onp.array_equal(got[[0, 2, 4]], x[[0, -1, 3]]) and onp.isnan(got[[1, 3]]).all()
+    g = ag.grad(lambda a: dnp.sum(dnp.nan_to_num(a[R]) * 2.0))(X).numpy()
+    want = onp.zeros_like(x)
+    onp.add.at(want, [0, -1, 3], 2.0)
+    assert onp.array_equal(g, want)
+    # host indices keep NumPy's error
+    with pytest.raises(IndexError):
+        X[onp.array([0, 7])]
+
+
+def test_row_gather_keeps_rows_and_the_plan_cache_is_bounded(dnp):
+    """``X[batch_rows]`` with host row numbers: n entries and rows of `inner` elements (not a position per element);
+    the plans kept on the device are bounded in bytes, least recently used first out."""
+    import autograd_amd as ag
+    from autograd_amd.numpy import wrapper
+
+    rs = onp.random.RandomState(0)
+    x = rs.randn(50, 7, 3)
+    X = P(dnp, x)
+    idx = rs.randint(-50, 50, 20)
+    plan = wrapper._index_plan(X.shape, idx)
+    assert plan.n == 20 and plan.inner == 21 and plan.n_rows == 50 and plan.shape == (20, 7, 3)
+    assert onp.array_equal(X[idx].numpy(), x[idx])
+    g = ag.grad(lambda a: dnp.sum(a[idx] * a[idx]))(X).numpy()
+    want = onp.zeros_like(x)
+    onp.add.at(want, idx, 2 * x[idx])
+    assert onp.array_equal(g, want)
+    for k in range(wrapper._INDEX_PLAN_LIMIT + 10):
+        wrapper._index_plan((1000,), onp.array([k % 1000, (k * 7) % 1000]))
+    assert len(wrapper._INDEX_PLANS) <= wrapper._INDEX_PLAN_LIMIT
+    assert 0 < wrapper._INDEX_PLAN_BYTES[0] <= wrapper._INDEX_PLAN_BUDGET
+    huge = onp.arange(300000) % 50
+    assert wrapper._index_plan(X.shape, huge) is not wrapper._index_plan(X.shape, huge)  # too large to keep

@@ -25,7 +25,13 @@ pytestmark = pytest.mark.gpu
 GOLD = onp.load(os.path.join(os.path.dirname(__file__), "golden", "reference_vectors.npz"))
 
 
-def check(name, got, want, rtol=None, exact=False):
+PURE = {}  # name -> fraction of elements inside the pure relative bound rtol * |ref| (filled by `check`)
+
+
+def check(name, got, want, rtol=None, exact=False, pure=None):
+    """``|got - ref| <= rtol * |ref| + rtol * max|ref|`` for every element (a pure relative bound is meaningless at the
+    zeros of a derivative); the fraction of elements that also meet the pure bound ``rtol * |ref|`` is recorded in
+    ``PURE[name]`` and, when ``pure`` is given, must reach it."""
     got, want = onp.asarray(got), onp.asarray(want)
     assert got.dtype == want.dtype, f"{name}: dtype {got.dtype} != {want.dtype}"
     assert got.shape == want.shape, f"{name}: shape {got.shape} != {want.shape}"
@@ -38,6 +44,9 @@ def check(name, got, want, rtol=None, exact=False):
     tol = rtol * onp.abs(w) + rtol * onp.max(onp.abs(w))
     err = onp.abs(g - w)
     assert onp.all(err <= tol), f"{name}: max err/tol {onp.max(err / (tol + 1e-300)):.3g}"
+    PURE[name] = float(onp.mean(err <= rtol * onp.abs(w))) if w.size else 1.0
+    if pure is not None:
+        assert PURE[name] >= pure, f"{name}: only {PURE[name]:.5f} of the elements are within rtol * |ref|"
 
 
 @pytest.fixture(scope="module")
@@ -103,7 +112,7 @@ def test_full_bcast(dev):
     want = configs.run_config("bcast", oracle_backend(), inputs)
     exact = cf.bcast_grads(**inputs)
     for k in ("dA", "db", "dc"):
-        check(f"bcast/{k} vs oracle", got[k], want[k])
+        check(f"bcast/{k} vs oracle", got[k], want[k], pure=0.999)
         check(f"bcast/{k} vs f64 closed form", got[k], exact[k].astype(onp.float32))
         # and the device result is at least as close to the float64 answer as NumPy's float32 one
         e_dev = onp.max(onp.abs(got[k].astype(onp.float64) - exact[k]))
@@ -120,6 +129,42 @@ def test_full_mlp(dev):
         for j, nm in enumerate(("W", "b")):
             check(f"mlp/{layer}/{nm} vs oracle", got[layer][j], want[layer][j])
             check(f"mlp/{layer}/{nm} vs f64 backprop", got[layer][j], exact[layer][j].astype(onp.float32))
+            # The pure bound rtol * |ref| element by element: a float32 contraction over 1024 terms summed in another
+            # order than the host BLAS differs from it by more than 1e-5 of a SMALL element (measured: 86 % of dW1 are
+            # inside); what can be asked is that the device is inside that bound of the float64 answer as often as
+            # NumPy's own float32 evaluation is.
+            check(f"mlp/{layer}/{nm} oracle vs f64 backprop", want[layer][j], exact[layer][j].astype(onp.float32))
+            assert PURE[f"mlp/{layer}/{nm} vs f64 backprop"] >= PURE[f"mlp/{layer}/{nm} oracle vs f64 backprop"] - 0.02, \
+                (layer, nm, PURE[f"mlp/{layer}/{nm} vs f64 backprop"], PURE[f"mlp/{layer}/{nm} oracle vs f64 backprop"])
+
+
+def test_full_size_slice_cotangents_are_bit_exact(dev):
+    """Index and scatter rules at config 5's full length (2^24): the cotangents of ``x[1:]`` and ``x[:-1]``, scattered back and
+    summed (``untake``, autograd/numpy/numpy_vjps.py:919-950 through ``add_outgrads``, autograd/core.py:185-205),
+    against ``numpy.add.at`` bit for bit: evaluated as one program (slices and scatters stay expressions) and by the
+    separate scatter launches."""
+    import autograd_amd as ag
+    from autograd_amd.numpy import fusion
+
+    np = dev.np
+    n = 1 << 24
+    rs = onp.random.RandomState(7)
+    w1, w2 = rs.randn(n - 1), rs.randn(n - 1)
+    w1[::1001] = -0.0  # signed zeros travel through `0.0 + g` as they do in NumPy
+    x = dev.put(rs.randn(n))
+    W1, W2 = dev.put(w1), dev.put(w2)
+    want = onp.zeros(n)
+    onp.add.at(want, slice(1, None), w1)
+    onp.add.at(want, slice(None, -1), w2)
+    f = lambda x: np.sum(x[1:] * W1) + np.sum(x[:-1] * W2)  # noqa: E731
+    for fused in (True, False):
+        was, fusion.ENABLED = fusion.ENABLED, fused
+        try:
+            got = dev.get(ag.grad(f)(x))
+        finally:
+            fusion.ENABLED = was
+        check(f"untake at 2^24 (fused={fused})", got, want, exact=True)
+        assert onp.array_equal(onp.signbit(got), onp.signbit(want))
 
 
 def test_full_rnn(dev):
