@@ -60,11 +60,17 @@ struct AccLse {
     typedef LsePair<T> type;
     __device__ __forceinline__ static type identity() { return {T(-INFINITY), T(0)}; }
     __device__ __forceinline__ static type lift(T v) { return {v, T(1)}; }
+    // value: the larger maximum, and its sum plus the other sum scaled by exp(difference of the maxima).  Written
+    // with selects and one exp, not one branch per case: lanes of a wave disagree on which side is larger, and with
+    // branches every step of a wave-wide reduction runs both exps one after the other.  Equal maxima (also both
+    // infinite) scale by exp(0) = 1 exactly; a NaN maximum gives NaN for both members.
     __device__ __forceinline__ static type combine(type a, type b) {
-        if (a.m == b.m) return {a.m, a.s + b.s};
-        if (a.m > b.m) return {a.m, a.s + b.s * m_exp(b.m - a.m)};
-        if (b.m > a.m) return {b.m, b.s + a.s * m_exp(a.m - b.m)};
-        return {a.m + b.m, a.s + b.s};  // a NaN is involved: propagate it
+        const bool a_larger = a.m >= b.m;
+        const T hi_m = a_larger ? a.m : b.m, lo_m = a_larger ? b.m : a.m;
+        const T hi_s = a_larger ? a.s : b.s, lo_s = a_larger ? b.s : a.s;
+        const T d = (a.m == b.m) ? T(0) : lo_m - hi_m;
+        const bool ordered = a.m == a.m && b.m == b.m;
+        return {ordered ? hi_m : a.m + b.m, ordered ? hi_s + lo_s * m_exp(d) : a.s + b.s};
     }
     __device__ __forceinline__ static T finish(type a) {
         if (a.s == T(0) || a.m == T(INFINITY)) return a.m;  // all -inf, or a +inf present
@@ -232,6 +238,8 @@ __global__ __launch_bounds__(kBlock) void red_row_block(const RedParams p) {
 // d * log2(e); the rounding of that product perturbs the term by at most |d| e^d 2^-24 <= 0.37 * 2^-24
 // of the sum, below the rounding of the sum itself, and results under the normal range flush to
 // zero (they are below 1e-38 of the sum).  double: the library routine.
+__device__ __forceinline__ float max_skipping_nan(float a, float b) { return __builtin_fmaxf(a, b); }
+__device__ __forceinline__ double max_skipping_nan(double a, double b) { return __builtin_fmax(a, b); }
 __device__ __forceinline__ float exp_nonpositive(float d) { return __builtin_amdgcn_exp2f(d * 1.44269504088896340736f); }
 __device__ __forceinline__ double exp_nonpositive(double d) { return exp(d); }
 
@@ -344,7 +352,17 @@ __global__ __launch_bounds__(kBlock) void lse_row_block(const RedParams p) {
         if (!VEC_B && p.shift_aux[0] >= 0) ub = static_cast<const T *>(p.in[p.shift_aux[0]])[o * p.istr[p.shift_aux[0]][0]];
         const T sc = (p.scale_mask & 1u) ? static_cast<T>(p.scale[0]) : T(1);
         const T sh = (p.shift_mask & 1u) ? static_cast<T>(p.shift[0]) : T(0);
-        if (n == static_cast<int64_t>(ITERS) * kBlock * V) {  // the chunk fills every lane: no padding to protect
+        if (n == static_cast<int64_t>(ITERS) * kBlock * V && !((p.scale_mask | p.shift_mask) & 1u)) {
+            // the same without the absent scalar steps (a block-wide choice; the VALU work of this kernel is
+            // not hidden behind its loads, every instruction per element shows in its duration)
+#pragma unroll
+            for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+                for (int j = 0; j < V; ++j) {
+                    const T v = x[it][j] * (VEC_A ? a[it][j] : ua);
+                    x[it][j] = v + (VEC_B ? b[it][j] : ub);
+                }
+        } else if (n == static_cast<int64_t>(ITERS) * kBlock * V) {  // the chunk fills every lane: no padding to protect
 #pragma unroll
             for (int it = 0; it < ITERS; ++it)
 #pragma unroll
@@ -369,11 +387,21 @@ __global__ __launch_bounds__(kBlock) void lse_row_block(const RedParams p) {
             }
         }
     }
+    // The maximum that skips NaNs is one instruction per element, the one that keeps them four.  A NaN among
+    // finite terms reaches the sum through exp(NaN - m); only where no exp is taken (m infinite) is it looked for.
     T m = T(-INFINITY);
 #pragma unroll
     for (int it = 0; it < ITERS; ++it)
 #pragma unroll
-        for (int j = 0; j < V; ++j) m = max_nan(x[it][j], m);
+        for (int j = 0; j < V; ++j) m = max_skipping_nan(x[it][j], m);
+    if (m == T(INFINITY) || m == T(-INFINITY)) {
+        bool any_nan = false;
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+            for (int j = 0; j < V; ++j) any_nan |= x[it][j] != x[it][j];
+        if (any_nan) m = T(NAN);
+    }
     T sum = T(0);
     if (m == T(INFINITY)) {
         sum = T(1);
