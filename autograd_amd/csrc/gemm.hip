@@ -731,6 +731,163 @@ __global__ __launch_bounds__(kDirectThreads) void gemm_direct(const GemmParams p
     }
 }
 
+// ---- small outputs, long K: the K split inside one block ---------------------------------------------------
+//
+// A product with few output tiles and a long K (the steps of a recurrent net: 256 x 512 from K = 641) cannot fill the
+// machine with one block per 64 x 64 tile; cutting K across blocks does, but leaves partial tiles in memory for a
+// second launch to add up, and at this size a launch costs as much as the arithmetic.  Here a block of up to 16 waves
+// owns one 32 x 32 tile of C and every wave a slice of K: a wave streams its slice of both operands from global memory
+// (they are a few hundred KB and sit in the L2) straight into the matrix core's operand registers, two chunks of
+// 32 k in flight, no LDS staging; the waves' accumulators meet in LDS and are added in wave order by the thread that
+// then applies alpha / beta or a dense-layer epilogue and stores the element.  One launch, nothing atomic, results
+// fixed by the shape.
+//
+// k order inside a chunk: instruction i of 16 multiplies k = 8 (i / 4) + 4 h + i % 4 for lane half h, so an operand
+// that is contiguous along k delivers a lane's four values of a group with one 16-byte load; an operand contiguous
+// along its other axis loads 4 bytes per instruction, 128 contiguous bytes per half wave.
+constexpr int kSmallTile = 32;
+constexpr int kSmallChunk = 32;
+constexpr int kSmallMaxWaves = 16;
+
+// An operand contiguous along k: plain 16-byte loads (four 64-bit addresses per chunk).  `row` points at the lane's
+// row (or column), `kc + 4 h` is the lane's first k of the chunk; only used where the whole chunk lies inside the slice.
+__device__ __forceinline__ void small_load_k(const float *__restrict__ row, int64_t kc, int h, float (&v)[16]) {
+    typedef float f4 __attribute__((ext_vector_type(4), aligned(4)));
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        const f4 t = *reinterpret_cast<const f4 *>(row + kc + 8 * g + 4 * h);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[4 * g + j] = t[j];
+    }
+}
+
+// Any other layout, and every operand in the last (partial) chunk of a slice: sixteen 4-byte loads through a buffer
+// descriptor.  The address is the descriptor's base + a wave-uniform offset (which k of which chunk: a scalar
+// register) + the lane's offset (its row or column and its half's 4 k: ONE vector register per operand) instead of a
+// 64-bit vector address per load; that is what lets two chunks of both operands stay in flight inside the 128
+// registers a wave of a 1024-thread block may hold.  Offsets past the operand's extent read as zero; k past the
+// wave's slice but inside the operand is zeroed by MASK.
+template <bool MASK>
+__device__ __forceinline__ void small_load_x(__amdgpu_buffer_rsrc_t rsrc, uint32_t lane_off, int64_t ks, int64_t kc, int64_t kend,
+                                             int h, float (&v)[16]) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+        v[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                             rsrc, lane_off, static_cast<uint32_t>((kc + 8 * (i / 4) + (i % 4)) * ks * 4), 0));
+    if (MASK) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v[i] = (kc + 8 * (i / 4) + 4 * h + (i % 4) < kend) ? v[i] : 0.f;
+    }
+}
+
+template <bool KCA, bool KCB>
+__global__ __launch_bounds__(kSmallMaxWaves * 64) void gemm_block_split(const GemmParams p) {
+    extern __shared__ float part_lds[];  // [waves][32 * 32]
+    float (*part)[kSmallTile * kSmallTile] = reinterpret_cast<float (*)[kSmallTile * kSmallTile]>(part_lds);
+    const int tid = threadIdx.x, lane = tid & 63, n_waves = blockDim.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // the same for the whole wave: offsets made of it are scalar
+    const int r = lane & 31, h = lane >> 5;
+    const int64_t tile_m = blockIdx.x / p.tiles_n, tile_n = blockIdx.x % p.tiles_n, batch = blockIdx.y;
+    const int64_t m0 = tile_m * kSmallTile, n0 = tile_n * kSmallTile;
+    // (the host admits only operands that span less than 2 GiB with non-negative strides: offsets fit 32 bits)
+    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float *>(static_cast<const float *>(p.A) + batch * p.a_bs), 0, p.a_span_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float *>(static_cast<const float *>(p.B) + batch * p.b_bs), 0, p.b_span_bytes, 0x00020000);
+    // rows / columns past the edge read the last one: their products land in elements that are never stored
+    const uint32_t a_lane = static_cast<uint32_t>((min(m0 + r, p.M - 1) * p.a_rs + 4 * h * p.a_cs) * 4);
+    const uint32_t b_lane = static_cast<uint32_t>((min(n0 + r, p.N - 1) * p.b_cs + 4 * h * p.b_rs) * 4);
+    const float *a_row = static_cast<const float *>(p.A) + batch * p.a_bs + min(m0 + r, p.M - 1) * p.a_rs;
+    const float *b_col = static_cast<const float *>(p.B) + batch * p.b_bs + min(n0 + r, p.N - 1) * p.b_cs;
+    const int64_t kbeg = wave * p.k_per_split, kend = min(p.K, kbeg + p.k_per_split);
+
+    v16f acc;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+    float a0[16], b0[16], a1[16], b1[16];
+    const auto load = [&](int64_t kc, float (&a)[16], float (&b)[16]) __attribute__((always_inline)) {
+        if (kc + kSmallChunk <= kend) {  // the same for the whole wave
+            if (KCA) small_load_k(a_row, kc, h, a);
+            else small_load_x<false>(rsrc_a, a_lane, p.a_cs, kc, kend, h, a);
+            if (KCB) small_load_k(b_col, kc, h, b);
+            else small_load_x<false>(rsrc_b, b_lane, p.b_rs, kc, kend, h, b);
+        } else {
+            small_load_x<true>(rsrc_a, a_lane, p.a_cs, kc, kend, h, a);
+            small_load_x<true>(rsrc_b, b_lane, p.b_rs, kc, kend, h, b);
+        }
+    };
+    const auto multiply = [&](const float (&a)[16], const float (&b)[16]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[i], acc, 0, 0, 0);
+    };
+    if (kbeg < kend) {
+        int64_t k = kbeg;
+        load(k, a0, b0);
+        while (true) {
+            if (k + kSmallChunk < kend) load(k + kSmallChunk, a1, b1);
+            multiply(a0, b0);
+            k += kSmallChunk;
+            if (k >= kend) break;
+            if (k + kSmallChunk < kend) load(k + kSmallChunk, a0, b0);
+            multiply(a1, b1);
+            k += kSmallChunk;
+            if (k >= kend) break;
+        }
+    }
+    // accumulator register v of lane (r, h) is C[8 (v/4) + 4 h + v%4][r] of the tile
+#pragma unroll
+    for (int v = 0; v < 16; ++v) part[wave][(8 * (v / 4) + 4 * h + (v % 4)) * kSmallTile + r] = acc[v];
+    __syncthreads();
+
+    const float alpha = static_cast<float>(p.alpha), beta = static_cast<float>(p.beta);
+    const bool has_bias = p.epi_bias != nullptr;
+    for (int e = tid; e < kSmallTile * kSmallTile; e += blockDim.x) {
+        const int64_t row = m0 + e / kSmallTile, col = n0 + e % kSmallTile;
+        if (row >= p.M || col >= p.N) continue;
+        float t = part[0][e];
+        for (int w = 1; w < n_waves; ++w) t += part[w][e];
+        float *C = static_cast<float *>(p.C) + batch * p.c_bs + row * p.ldc + col;
+        if (p.alpha != 1.0) t = alpha * t;
+        if (p.beta != 0.0) t = t + beta * *C;
+        const float bias = has_bias ? p.epi_bias[col] : 0.f;
+        if (p.epi == 2) t = epi_tanh_vjp(t, p.epi_x[row * p.epi_x_ld + col], bias, has_bias);
+        *C = t;
+        if (p.epi == 1) p.epi_out[row * p.epi_ld + col] = epi_tanh(t, bias, has_bias);
+    }
+}
+
+// Whether a float32 product goes to gemm_block_split: too few 64 x 64 tiles to fill the machine and a K long enough
+// to cut, but not so long that one block per 32 x 32 tile would be the slower way to cut it.
+static bool wants_block_split(const GemmParams &p, int64_t batch) {
+    const int64_t tiles64 = ceil_div(p.M, 64) * ceil_div(p.N, 64) * batch;
+    const int64_t tiles32 = ceil_div(p.M, kSmallTile) * ceil_div(p.N, kSmallTile) * batch;
+    const int64_t a_span = ((p.M - 1) * p.a_rs + (p.K - 1) * p.a_cs + 1) * 4, b_span = ((p.K - 1) * p.b_rs + (p.N - 1) * p.b_cs + 1) * 4;
+    const bool addressable = p.a_rs >= 0 && p.a_cs >= 0 && p.b_rs >= 0 && p.b_cs >= 0 && a_span < 0x7fff0000LL && b_span < 0x7fff0000LL;
+    return addressable && tiles64 < 128 && p.K >= 256 && (p.K <= 4096 || tiles32 >= 128) && tiles32 <= 0x7fffffffLL && batch <= 65535;
+}
+
+static int launch_block_split(GemmParams p, int64_t batch, hipStream_t s) {
+    const int64_t tm = ceil_div(p.M, kSmallTile), tn = ceil_div(p.N, kSmallTile);
+    p.tiles_m = static_cast<int>(tm);
+    p.tiles_n = static_cast<int>(tn);
+    // whole chunks per wave (only the slice that holds the end of K has a partial one), as many waves as there are chunks
+    const int waves = static_cast<int>(std::min<int64_t>(kSmallMaxWaves, ceil_div(p.K, kSmallChunk)));
+    p.splits = waves;
+    p.k_per_split = ceil_div(ceil_div(p.K, waves), kSmallChunk) * kSmallChunk;
+    p.a_span_bytes = static_cast<uint32_t>(((p.M - 1) * p.a_rs + (p.K - 1) * p.a_cs + 1) * 4);
+    p.b_span_bytes = static_cast<uint32_t>(((p.K - 1) * p.b_rs + (p.N - 1) * p.b_cs + 1) * 4);
+    const bool kca = p.a_cs == 1, kcb = p.b_rs == 1;
+    set_kernel_name("gemm_block_split<f32,32,32,%s%s%s>[%lldx%lldx%lld]", kca ? "k" : "x", kcb ? "k" : "x",
+                    p.epi == 1 ? ",+bias,tanh" : (p.epi == 2 ? ",tanh_vjp" : ""), (long long)p.M, (long long)p.N, (long long)p.K);
+    const dim3 grid((unsigned)(tm * tn), (unsigned)batch), block(waves * 64);
+    const size_t lds = static_cast<size_t>(waves) * kSmallTile * kSmallTile * sizeof(float);
+    if (kca && kcb) hipLaunchKernelGGL((gemm_block_split<true, true>), grid, block, lds, s, p);
+    else if (kca) hipLaunchKernelGGL((gemm_block_split<true, false>), grid, block, lds, s, p);
+    else if (kcb) hipLaunchKernelGGL((gemm_block_split<false, true>), grid, block, lds, s, p);
+    else hipLaunchKernelGGL((gemm_block_split<false, false>), grid, block, lds, s, p);
+    return hip_check(hipGetLastError(), "gemm launch");
+}
+
 // C = alpha * (sum over splits, in split order) + beta * C
 template <typename T>
 __global__ __launch_bounds__(kBlock) void gemm_split_finish(const T *__restrict__ ws, T *__restrict__ C, int splits,
@@ -1001,6 +1158,7 @@ extern "C" int agmi_gemm(int dtype, int64_t batch, int64_t M, int64_t N, int64_t
         const int64_t small_tiles = ceil_div(M, 64) * ceil_div(N, 64) * batch;
         const auto fill = [](int64_t tiles) { return static_cast<double>(tiles) / static_cast<double>(ceil_div(tiles, 256) * 256); };
         const bool prefer_big = big_tiles >= 512 && 117.0 * fill(big_tiles) > 107.0 * fill(small_tiles);
+        if (wants_block_split(p, batch)) return launch_block_split(p, batch, s);
         if (!prefer_big) {
             const int rc = launch_direct(p, batch, s, workspace, workspace_bytes);
             if (rc != 1) return rc;  // launched (0) or failed; 1 = operands do not qualify
@@ -1049,6 +1207,7 @@ extern "C" int agmi_gemm_fused(int dtype, int64_t M, int64_t N, int64_t K, const
     p.epi_ld = e->out_ld;
     p.epi_x = static_cast<const float *>(e->x);
     p.epi_x_ld = e->x_ld;
+    if (wants_block_split(p, 1)) return launch_block_split(p, 1, as_stream(stream));
     const int rc = launch_direct(p, 1, as_stream(stream), workspace, workspace_bytes);
     if (rc == 1) {
         set_error("gemm_fused: operands outside the direct kernel's layouts (one unit stride each)");

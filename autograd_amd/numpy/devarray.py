@@ -268,7 +268,7 @@ class PendingProduct(DevArray):
     ``DevArray``; the first such read computes the product and keeps it.
     """
 
-    __slots__ = ("_left", "_right", "_shape", "_out")
+    __slots__ = ("_left", "_right", "_shape", "_out", "_more")
 
     def __init__(self, left, right, dtype):
         self._left, self._right = left, right
@@ -276,18 +276,63 @@ class PendingProduct(DevArray):
         self.dtype = dtype
         self._borrowed = False
         self._out = None
+        self._more = None  # further (left, right) pairs whose products are added to this one (see `sum_started`)
 
     def __getattr__(self, name):
         # only reached when a slot is unset: `_t` before the product has been computed
         if name != "_t":
             raise AttributeError(name)
-        if self._out is None:
+        if self._more:
+            out = self._sum_of_products()
+        elif self._out is None:
             out = gemm2d(self._left, self._right, self.dtype)
         else:
             out = gemm2d(self._left, self._right, self.dtype, out=self._out)
         self._t = out
-        self._left = self._right = self._out = None
+        self._left = self._right = self._out = self._more = None
         return out
+
+    def sum_started(self):
+        """A new pending value that starts a sum of products with this one: the accumulator of a matrix cotangent.
+
+        A weight matrix used at every step of a recurrence receives one product per step, ``cat_t.T @ G_t``
+        (numpy_vjps.py:615-638 through core.py:185-205).  Run one by one they are as many small contractions as
+        there are steps, each a launch whose duration is mostly latency; the sum of all of them is ONE
+        contraction over the stacked operands, ``[cat_0; cat_1; ...].T @ [G_0; G_1; ...]``.  The accumulator
+        therefore only collects the operand pairs (``add_product``) and contracts when its value is read."""
+        acc = PendingProduct(self._left, self._right, self.dtype)
+        acc._more = list(self._more) if self._more else []
+        return acc
+
+    def add_product(self, other):
+        """``self += other`` for two pending products of one shape (``self`` came from ``sum_started``)."""
+        self._more.append((other._left, other._right))
+        if other._more:
+            self._more.extend(other._more)
+
+    def _sum_of_products(self):
+        terms = [(self._left, self._right)] + self._more
+        out = self._out if self._out is not None else _lib.empty(self._shape, self.dtype)
+        M, N = self._shape
+        # The stacked form: every left factor the transpose of a row-major (K_i, M) matrix, every right factor a
+        # row-major (K_i, N) matrix (the weight cotangents of `dot`), at least four of them.
+        stackable = len(terms) >= 4 and M and N and all(
+            l.stride(0) == 1 and l.stride(1) == M and r.is_contiguous() and l.shape[1] for l, r in terms)
+        if not stackable:
+            gemm2d(terms[0][0], terms[0][1], self.dtype, out=out)
+            for l, r in terms[1:]:
+                gemm2d(l, r, self.dtype, out=out, beta=1.0)
+            return out
+        total = sum(l.shape[1] for l, _ in terms)
+        lefts, rights = _lib.empty((total, M), self.dtype), _lib.empty((total, N), self.dtype)
+        code = _lib.DTYPE_CODE[self.dtype]
+        for k in range(0, len(terms), _lib.MAX_CONCAT):
+            group = terms[k:k + _lib.MAX_CONCAT]
+            begin = sum(l.shape[1] for l, _ in terms[:k])
+            rows = sum(l.shape[1] for l, _ in group)
+            _lib.concat(code, 1, M, [(l, l.shape[1], 0, M, 1) for l, _ in group], lefts[begin:begin + rows])
+            _lib.concat(code, 1, N, [(r, r.shape[0], 0, N, 1) for _, r in group], rights[begin:begin + rows])
+        return gemm2d(lefts.t(), rights, self.dtype, out=out)
 
     def _buffer(self):
         """The memory the product will be written to (allocated now, filled when the product runs)."""
@@ -304,7 +349,7 @@ class PendingProduct(DevArray):
     def with_activation(self, bias, act_out):
         """Run the product with ``act_out = tanh(product + bias)`` formed in the contraction's epilogue; False when the
         fused kernel does not take these operands (nothing has run then)."""
-        if not self._shape[0] or not self._shape[1] or not self._left.shape[1]:
+        if not self._shape[0] or not self._shape[1] or not self._left.shape[1] or self._more:
             return False
         out = self._buffer()
         if not _lib.gemm_fused(_lib.DTYPE_CODE[self.dtype], self._left, self._right, out, _lib.EPILOGUE_BIAS_TANH, bias=bias,
@@ -317,7 +362,7 @@ class PendingProduct(DevArray):
     def into_tanh_cotangent(self, x, bias, out):
         """``out = (left @ right) / cosh(x + bias)**2`` in one launch (the product itself stays uncomputed); False when
         the fused kernel does not take these operands."""
-        if not self._shape[0] or not self._shape[1] or not self._left.shape[1]:
+        if not self._shape[0] or not self._shape[1] or not self._left.shape[1] or self._more:
             return False
         return _lib.gemm_fused(_lib.DTYPE_CODE[self.dtype], self._left, self._right, out, _lib.EPILOGUE_TANH_VJP, bias=bias, x=x)
 
@@ -326,11 +371,18 @@ class PendingProduct(DevArray):
 
     def fresh(self):
         """The product in a buffer of the caller's own (nothing is kept here)."""
+        if self._more:
+            kept, self._out = self._out, None
+            out = self._sum_of_products()
+            self._out = kept
+            return DevArray(out, self.dtype)
         return DevArray(gemm2d(self._left, self._right, self.dtype), self.dtype)
 
     def add_into(self, acc):
         """``acc += left @ right`` for a contiguous tensor ``acc`` of this shape and dtype."""
         gemm2d(self._left, self._right, self.dtype, out=acc, beta=1.0)
+        for l, r in self._more or ():
+            gemm2d(l, r, self.dtype, out=acc, beta=1.0)
 
     @property
     def shape(self):

@@ -115,6 +115,11 @@ class DevArrayVSpace(VSpace):
         return D.from_numpy(onp.array(onp.random.randn(*self.shape)).astype(self.dtype))
 
     def _add(self, x, y):
+        if type(x) is D.PendingProduct and type(y) is D.PendingProduct and not x.computed() and not y.computed() \
+                and x.dtype == y.dtype and x.shape == y.shape:
+            acc = x.sum_started()  # two matrix cotangents whose contractions have not run: a sum of products (neither is touched)
+            acc.add_product(y)
+            return acc
         return D.map_op(Op.ADD, D._float_dtype(D.result_dtype(x, y)), x, y)
 
     def _mut_add(self, x, y):
@@ -129,7 +134,10 @@ class DevArrayVSpace(VSpace):
         if type(y) is D.PendingProduct and not y.computed() and y.dtype == x.dtype and y.shape == x.shape:
             # a matrix cotangent whose contraction has not run yet: run it into the accumulator
             if is_shared_zero(x):
-                return y.fresh()  # 0 + G: a buffer of the accumulator's own, so later contributions add in place
+                return y.sum_started()  # 0 + G: the accumulator collects the products and contracts once, when read
+            if type(x) is D.PendingProduct and not x.computed() and x._more is not None:
+                x.add_product(y)
+                return x
             if type(x) is DevArray and not x._borrowed and not is_broadcast_view(x) and x._t.is_contiguous():
                 y.add_into(x._t)
                 return x

@@ -342,7 +342,9 @@ def test_weighted_logsumexp_follows_scipy(dnp):
 
 # ---- contractions -------------------------------------------------------------------------------
 GEMM_SHAPES = [(1, 1, 1), (5, 7, 3), (64, 64, 16), (65, 63, 17), (130, 70, 33), (256, 128, 641), (1024, 10, 1024),
-               (10, 1024, 300), (300, 300, 1), (129, 257, 100), (512, 512, 512)]
+               (10, 1024, 300), (300, 300, 1), (129, 257, 100), (512, 512, 512),
+               # few output tiles and a long K (the K split inside one block): whole and partial chunks, ragged tiles
+               (256, 512, 641), (641, 512, 256), (33, 31, 257), (96, 40, 288), (64, 64, 5000), (200, 130, 4100)]
 
 
 @pytest.mark.parametrize("dtype", [F32, F64])
@@ -906,6 +908,47 @@ def test_matrix_cotangents_accumulate_inside_the_contraction(dnp, dtype, rows, i
     assert onp.array_equal(ag.grad(hm)(X1).numpy(), (dnp.dot(C1, V1.T) + dnp.dot(C2, V2.T)).numpy())
 
 
+@pytest.mark.parametrize("dtype", [F32, F64])
+@pytest.mark.parametrize("steps,rows,inner,cols", [(4, 16, 33, 10), (11, 64, 129, 48), (65, 256, 641, 128), (9, 7, 5, 3)])
+def test_many_products_into_one_weight_are_one_contraction(dnp, dtype, steps, rows, inner, cols):
+    """A weight used once per step of a loop (numpy_vjps.py:615-638 through core.py:185-205): from four
+    products on, the cotangent is ONE contraction over the stacked operands (one launch instead of one
+    per step, joined by a few copies).  The order of the additions is not the loop's, so the bound is the
+    floating-point one; the result does not change from run to run."""
+    import autograd_amd as ag
+    from autograd_amd import _lib
+
+    rs = onp.random.RandomState(steps)
+    xs = [rs.randn(rows + (t % 3), inner).astype(dtype) for t in range(steps)]  # (the steps need not be equally long)
+    cs = [rs.randn(rows + (t % 3), cols).astype(dtype) for t in range(steps)]
+    Xs, Cs = [P(dnp, x) for x in xs], [P(dnp, c) for c in cs]
+    W = P(dnp, rs.randn(inner, cols).astype(dtype))
+
+    def f(w):
+        total = 0.0
+        for X, C in zip(Xs, Cs):
+            total = total + dnp.sum(dnp.dot(X, w) * C)
+        return total
+
+    launches = []
+    was = _lib.gemm
+
+    def counting(*a, **k):
+        launches.append(a[2:5])
+        return was(*a, **k)
+
+    _lib.gemm = counting
+    try:
+        got = ag.grad(f)(W).numpy()
+    finally:
+        _lib.gemm = was
+    want = sum(x.astype(F64).T @ c.astype(F64) for x, c in zip(xs, cs))
+    close(got, want.astype(dtype), RT[dtype] * max(1.0, onp.sqrt(steps * rows) / 8))
+    backward = [l for l in launches if l[:2] == (inner, cols)]
+    assert len(backward) == 1 and backward[0][2] == sum(x.shape[0] for x in xs), launches
+    assert onp.array_equal(ag.grad(f)(W).numpy(), got)
+
+
 # ---- remainder, nan_to_num and the array functions built on views and copy kernels: bit-exact ---------------
 @pytest.mark.parametrize("dtype", [F32, F64])
 def test_remainder_and_nan_to_num_are_bit_exact(dnp, dtype):
@@ -1461,7 +1504,7 @@ def test_device_resident_row_index_gathers_and_scatters_in_order(dnp, dtype):
 
 
 # ---- dense-layer epilogues of the contraction ------------------------------------------------------
-@pytest.mark.parametrize("M,N,K", [(64, 64, 32), (200, 130, 70), (256, 512, 641), (1024, 1024, 784), (7, 3, 5)])
+@pytest.mark.parametrize("M,N,K", [(64, 64, 32), (200, 130, 70), (256, 512, 641), (1024, 1024, 784), (7, 3, 5), (70, 45, 300)])
 def test_gemm_epilogues_equal_the_separate_kernels(dnp, M, N, K):
     """``agmi_gemm_fused``: tanh(A.B + bias) and (G.W^T) / cosh(x + bias)**2 formed inside the contraction are, bit for
     bit, what the product followed by the elementwise kernels gives (examples/neural_net.py:33-35,

@@ -264,9 +264,10 @@ def test_broadcast_operands_fold_into_pending_maps():
 
 def test_pending_products_are_contracted_into_an_accumulator_of_its_own(monkeypatch):
     """The accumulation protocol for matrix cotangents, with the contraction replaced by a recorder:
-    0 + G computes G into a buffer the accumulator owns; an owned accumulator takes the next
-    product with beta = 1; a borrowed accumulator (it shares memory with a cotangent) is never
-    written, the product is computed on its own and added out of place."""
+    0 + G starts a sum of products that only collects operand pairs; further products join it; the sum is
+    contracted when its value is read (few terms: one by one with beta = 1 into the accumulator's own buffer);
+    a plain owned accumulator takes a product with beta = 1; a borrowed accumulator (it shares memory with a
+    cotangent) is never written, the product is computed on its own and added out of place."""
     from autograd_amd.numpy import vspaces
 
     calls = []
@@ -276,17 +277,23 @@ def test_pending_products_are_contracted_into_an_accumulator_of_its_own(monkeypa
         return out if out is not None else torch.zeros((a.shape[0], b.shape[1]), dtype=torch.float64)
 
     monkeypatch.setattr(D, "gemm2d", fake_gemm2d)
+    monkeypatch.setattr(D._lib, "empty", lambda shape, dtype: torch.zeros(tuple(shape), dtype=torch.float64))
     monkeypatch.setitem(vspaces._ZEROS, onp.dtype("float64"), DevArray(torch.zeros((), dtype=torch.float64)))
     left, right = torch.zeros((3, 5), dtype=torch.float64), torch.zeros((5, 4), dtype=torch.float64)
     vs = vspaces.DevArrayVSpace(DevArray(torch.zeros((3, 4), dtype=torch.float64)))
     first = D.PendingProduct(left, right, onp.dtype("float64"))
     assert first.shape == (3, 4) and first.ndim == 2 and first.size == 12 and not first.computed()
     acc = vs._mut_add(vs.zeros(), first)
-    assert type(acc) is DevArray and not acc._borrowed and calls == [("gemm", False, 0.0)]
-    assert not first.computed()  # the product went to the accumulator, nothing was cached on the cotangent
+    assert type(acc) is D.PendingProduct and acc is not first and not acc.computed() and calls == []
     second = D.PendingProduct(left, right, onp.dtype("float64"))
-    assert vs._mut_add(acc, second) is acc and calls[-1] == ("gemm", True, 1.0) and not second.computed()
+    assert vs._mut_add(acc, second) is acc and calls == [] and not second.computed() and not first.computed()
+    total = acc._t
+    assert calls == [("gemm", True, 0.0), ("gemm", True, 1.0)] and acc.computed() and acc._t is total
+    # an accumulator that is a plain array of its own takes the product with beta = 1
+    acc = DevArray(torch.zeros((3, 4), dtype=torch.float64))
+    assert vs._mut_add(acc, D.PendingProduct(left, right, onp.dtype("float64"))) is acc and calls[-1] == ("gemm", True, 1.0)
     # a borrowed accumulator must not be written: no beta = 1 call on it
+    n_before = len(calls)
     borrowed = D.alias(acc)
     borrowed._borrowed = True
     third = D.PendingProduct(left, right, onp.dtype("float64"))
@@ -298,7 +305,7 @@ def test_pending_products_are_contracted_into_an_accumulator_of_its_own(monkeypa
             vs._mut_add(borrowed, third)
     finally:
         fusion.ENABLED = was
-    assert ("gemm", True, 1.0) not in calls[2:]
+    assert ("gemm", True, 1.0) not in calls[n_before:]
     # reading the value computes it once and keeps it
     fourth = D.PendingProduct(left, right, onp.dtype("float64"))
     n = len(calls)
