@@ -689,7 +689,7 @@ def fill(code, t, value):
         _check(rc, "agmi_fill")
 
 
-MAX_CONCAT = 8
+MAX_CONCAT = 32
 
 
 class AgmiConcatPiece(ctypes.Structure):

@@ -358,8 +358,7 @@ __global__ __launch_bounds__(kBlock) void concat_kernel(const ConcatParams p, T 
     const int64_t a = rest % p.total, o = rest / p.total;
     int k = 0;
     int64_t begin = 0;
-#pragma unroll
-    for (int j = 0; j < AGMI_MAX_CONCAT - 1; ++j) {
+    for (int j = 0; j < p.n_pieces - 1; ++j) {  // (the same trip count for every thread; `end` is non-decreasing)
         if (a >= p.end[j]) {
             k = j + 1;
             begin = p.end[j];

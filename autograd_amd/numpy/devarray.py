@@ -1215,6 +1215,24 @@ def map_reduce(op, red, dtype, xs, axes, keepdims, shape=None):
 
 
 def _map_reduce_now(op, red, dtype, xs, axes, keepdims, shape=None):
+    if len(xs) == 1 and _fusion is not None and type(xs[0]) is _fusion.ExprArray and xs[0]._args is not None \
+            and red == Red.SUM and (op == Op.COPY or op == Op.NEG) and xs[0].dtype == dtype:
+        # The reduction of a pending `a * b` (or +, -, /) of arrays in memory: the reduction kernel forms the
+        # product itself, element by element as the elementwise kernel would, so the expression need not be
+        # written out for it (the sum's own rule, `-sum(g * t)` of a log-softmax, reads it once more at most,
+        # inside the program that consumes it).  -sum(x) = sum(-x) exactly.
+        inner = _fusion.lone_binary(xs[0])
+        if inner is not None and (shape is None or tuple(shape) == xs[0].shape):
+            iop, (a, b) = inner
+            if op == Op.NEG:  # the sign goes to the operands, where it is a pending factor of the load (exact)
+                neg = lambda v: -v if type(v) is float else map_op(Op.NEG, dtype, v)  # noqa: E731
+                if iop == Op.SUB:
+                    a, b = b, a
+                elif iop == Op.ADD:
+                    a, b = neg(a), neg(b)
+                else:
+                    a = neg(a)
+            return _map_reduce_now(iop, red, dtype, (a, b), axes, keepdims, shape=xs[0].shape)
     ops = _limit_aux(tuple(_operand(x, dtype) for x in xs), dtype)
     if shape is None:
         shape = _bshape(ops)
@@ -1249,7 +1267,7 @@ def _map_reduce_now(op, red, dtype, xs, axes, keepdims, shape=None):
         if op == Op.COPY and isinstance(ops[0], torch.Tensor) and ops[0].is_contiguous():
             cur = DevArray(ops[0], dtype)  # nothing to apply or lay out first: reduce the operand itself
         else:
-            cur = map_op(op, dtype, *[_rewrap(t, dtype) for t in ops])
+            cur = plain(map_op(op, dtype, *[_rewrap(t, dtype) for t in ops]))  # (written out: the reduction below must not take it apart again)
         for group in _adjacent_groups(axes):
             cur = _map_reduce_now(Op.COPY, red, dtype, (cur,), group, True)
         out_t = cur._t

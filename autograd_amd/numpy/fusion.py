@@ -132,6 +132,23 @@ def pending(x):
     return type(x) is ExprArray and x._args is not None
 
 
+_REDUCIBLE = (Op.MUL, Op.ADD, Op.SUB, Op.DIV)
+
+
+def lone_binary(x):
+    """(op, operands) when the pending expression ``x`` is one binary arithmetic rule over operands that are in memory
+    (or scalars), all of ``x``'s dtype; None otherwise."""
+    if x._op not in _REDUCIBLE or len(x._args) != 2:
+        return None
+    for a in x._args:
+        if isinstance(a, DevArray):
+            if pending(a) or a.dtype != x.dtype or type(a) not in (DevArray, LazyDevArray):
+                return None
+        elif type(a) is not float:
+            return None
+    return x._op, tuple(x._args)
+
+
 def make(op, dtype, xs):
     """``op(*xs)`` as a pending node, or None when the step has to run the ordinary way."""
     arity = ARITY.get(op)

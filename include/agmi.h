@@ -358,7 +358,7 @@ int agmi_take_rows(int dtype, const void *src, int64_t n_rows, int64_t inner,
  * strided (outer, extent, inner) views that are laid one after another along the middle axis of the contiguous
  * result (outer, sum of extents, inner).  A piece with all strides 0 is a constant column (the ones that
  * examples/rnn.py:21 appends to its state).  At most AGMI_MAX_CONCAT pieces; none may overlap `out`. */
-#define AGMI_MAX_CONCAT 8
+#define AGMI_MAX_CONCAT 32
 typedef struct agmi_concat_piece {
     const void *data;
     int64_t extent;                                   /* along the joined axis */

@@ -392,7 +392,7 @@ def test_dot_rows_that_end_inside_a_vector_do_not_see_their_neighbours(dnp, K):
 @pytest.mark.parametrize("dtype", [F32, F64])
 def test_concatenate_in_one_launch_is_a_copy(dnp, dtype):
     """Pieces that are strided views (slices, transposes, broadcasts, launch-free constants) are joined by one kernel;
-    anything else (pending maps, other dtypes, more than eight pieces) goes piece by piece.  Either way the result
+    anything else (pending maps, other dtypes, more pieces than one launch takes) goes piece by piece.  Either way the result
     is NumPy's, bit for bit."""
     from autograd_amd import _lib
 
@@ -420,9 +420,12 @@ def test_concatenate_in_one_launch_is_a_copy(dnp, dtype):
         assert onp.array_equal(dnp.concatenate((X[:, 0], H[:, 1])).numpy(), onp.concatenate((x[:, 0], h[:, 1])))
         assert onp.array_equal(dnp.stack((X, X * 2.0), axis=1).numpy(), onp.stack((x, x * dtype(2.0)), axis=1))
         n = len(calls)
-        # not one launch: a pending map that is no constant, ten pieces, mixed precision
+        # ten pieces are still one launch
+        assert onp.array_equal(dnp.hstack((X,) * 10).numpy(), onp.hstack((x,) * 10)) and calls[-1] == 10
+        n = len(calls)
+        # not one launch: a pending map that is no constant, more pieces than the kernel's table holds, mixed precision
         assert onp.array_equal(dnp.hstack((X, -H)).numpy(), onp.hstack((x, -h)))
-        assert onp.array_equal(dnp.hstack((X,) * 10).numpy(), onp.hstack((x,) * 10))
+        assert onp.array_equal(dnp.hstack((X,) * (_lib.MAX_CONCAT + 1)).numpy(), onp.hstack((x,) * (_lib.MAX_CONCAT + 1)))
         other = F64 if dtype == F32 else F32
         mixed = dnp.hstack((X, P(dnp, h.astype(other))))
         assert mixed.dtype == F64 and onp.array_equal(mixed.numpy(), onp.hstack((x, h.astype(other))))
