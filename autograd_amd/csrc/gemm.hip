@@ -787,7 +787,13 @@ __global__ __launch_bounds__(kSmallMaxWaves * 64) void gemm_block_split(const Ge
     const int tid = threadIdx.x, lane = tid & 63, n_waves = blockDim.x >> 6;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // the same for the whole wave: offsets made of it are scalar
     const int r = lane & 31, h = lane >> 5;
-    const int64_t tile_m = blockIdx.x / p.tiles_n, tile_n = blockIdx.x % p.tiles_n, batch = blockIdx.y;
+    // Workgroups go to the 8 XCDs in turn and each XCD has an L2 of its own: XCD x takes a contiguous range of the
+    // tiles in column-major order (a few columns of tiles, every row), so its L2 fetches all of A but only its
+    // columns of B, not both operands whole.
+    const int64_t n_tiles = static_cast<int64_t>(p.tiles_m) * p.tiles_n;
+    const int64_t xcd = blockIdx.x % kXcds, turn = blockIdx.x / kXcds;
+    const int64_t tile = xcd * (n_tiles / kXcds) + min(xcd, n_tiles % kXcds) + turn;
+    const int64_t tile_m = tile % p.tiles_m, tile_n = tile / p.tiles_m, batch = blockIdx.y;
     const int64_t m0 = tile_m * kSmallTile, n0 = tile_n * kSmallTile;
     // (the host admits only operands that span less than 2 GiB with non-negative strides: offsets fit 32 bits)
     const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(

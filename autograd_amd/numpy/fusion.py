@@ -20,6 +20,7 @@ broadcast), another dtype, more pending nodes than ``MAX_CONE``, and anything th
 elementwise.
 """
 
+import math
 import os
 import sys
 
@@ -261,10 +262,7 @@ def _run(roots):
         _run(roots[:half])
         _run([r for r in roots[half:] if r._args is not None])
         return
-    try:
-        program = _emit(roots)
-    except _Unsupported:
-        program = False
+    program = _program_for(roots, order)
     if program is None:
         # too long, too many leaves or too many live values for one program: write a node from the middle of the
         # order out first (everything it needs comes before it), then try again with that node as a leaf
@@ -416,9 +414,9 @@ class _Unsupported(Exception):
 
 
 def _emit(roots):
-    """``(leaf tensors, immediates, instruction words, registers, shifted, masks)`` of the program that computes
-    ``roots``; None when it does not fit the kernel's limits.  ``shifted`` is None, or per leaf ``(shift, lo,
-    hi)`` when some vector is read at a shifted position (see :func:`shifted`).
+    """``(leaf tensors, the shift each is read at, immediates, instruction words, registers, whether vectors are read at
+    shifted positions (see :func:`shifted`), masks)`` of the program that computes ``roots``; None when it does not fit
+    the kernel's limits.
 
     The nodes are first written down in static single assignment form, one instruction per distinct
     subexpression, with three rewrites that change no bit of any result: negations are carried as a sign on the
@@ -459,7 +457,10 @@ def _emit(roots):
             any_shift[0] = True  # (a slice that starts at index 0: read in place, but not over its whole extent)
         # (unit-stride vectors are told apart by address alone: in a program all of them span the root's extent,
         # or are read at shifted positions inside one storage)
-        key = (t.data_ptr() + shift * itemsize,) if vector else (t.data_ptr(), t.stride(), tuple(t.shape))
+        # (told apart by storage and position in it, not by address: two storages that happen to lie back to back
+        # must not look like one vector read at two shifts, or the program would depend on where the allocator put them)
+        key = (t.data_ptr() - t.storage_offset() * itemsize, t.storage_offset() + shift) if vector \
+            else (t.data_ptr(), t.stride(), tuple(t.shape))
         v = leaf_ids.get(key)
         if v is None:
             if len(leaves) >= 4 * _lib.PROGRAM_MAX_LEAVES:
@@ -682,21 +683,7 @@ def _emit(roots):
     imms = [imms[k] for k in used_imms]
 
     n_leaf, n_imm, n_ins = len(leaves), len(imms), len(instrs)
-    shifted_leaves = None
-    if any_shift[0] or masks:
-        # one-axis program with vectors read at shifted positions: every vector leaf comes with the indices at which its
-        # (moved) address stays inside its storage; whatever lies outside a vector's own extent is masked by the program
-        shifted_leaves = []
-        for t, shift in zip(leaves, leaf_where):
-            if t.dim() == 1 and t.numel() > 1 and t.stride(0) == 1:
-                first = t.storage_offset() + shift
-                total = t.untyped_storage().nbytes() // itemsize
-                shifted_leaves.append((shift, -first, total - first))
-            elif t.numel() == 1 or builtins_all_zero(t.stride()):
-                shifted_leaves.append((0, 0, n_out))
-            else:
-                raise _Unsupported
-        leaves = [t if (t.dim() == 1 and t.numel() > 1 and t.stride(0) == 1) else t.as_strided((n_out,), (0,)) for t in leaves]
+    need_shifted = bool(any_shift[0] or masks)
     # last use of every value (instruction index; stores come after all instructions)
     last = {}
     for k, (_op, srcs, _mask) in enumerate(instrs):
@@ -735,8 +722,161 @@ def _emit(roots):
         for out_index, v in enumerate(root_values):
             r = reg[v]
             words.append(_lib.PROGRAM_STORE | r << 8 | r << 12 | out_index << 16)
-        return leaves, imms, words, n_regs, shifted_leaves, masks
+        return leaves, leaf_where, imms, words, n_regs, need_shifted, masks
     return None
+
+
+def _bind(leaves, leaf_where, n_out, itemsize, need_shifted):
+    """The leaf tensors as the kernel takes them, and per leaf ``(shift, lo, hi)`` for a one-axis program with vectors read
+    at shifted positions (None otherwise): every vector leaf comes with the indices at which its (moved) address stays
+    inside its storage; whatever lies outside a vector's own extent is masked by the program."""
+    if not need_shifted:
+        return leaves, None
+    shifted_leaves, bound = [], []
+    for t, shift in zip(leaves, leaf_where):
+        if t.dim() == 1 and t.numel() > 1 and t.stride(0) == 1:
+            first = t.storage_offset() + shift
+            total = t.untyped_storage().nbytes() // itemsize
+            shifted_leaves.append((shift, -first, total - first))
+            bound.append(t)
+        elif t.numel() == 1 or builtins_all_zero(t.stride()):
+            shifted_leaves.append((0, 0, n_out))
+            bound.append(t.as_strided((n_out,), (0,)))
+        else:
+            raise _Unsupported
+    return bound, shifted_leaves
+
+
+# ---- emitted programs are kept ---------------------------------------------------------------------------------
+# Writing a program down (the walk, the rewrites, the register assignment) costs tens of microseconds for a three-step
+# expression and hundreds for a Hessian-vector product, every evaluation, although a loop evaluates the same
+# expressions over and over.  What the emitted program depends on is written down as a key: the nodes in order with
+# their operations and operands, where an operand is another node (by position), a scalar (by value), or an array in
+# memory (by shape, strides, which distinct array it is, and where it lies in which storage, since vectors of one
+# storage are merged when a shift makes them coincide).  Equal keys give equal programs; only the tensors differ, and
+# those are bound again from the walk.
+_PROGRAMS = {}
+_PROGRAM_LIMIT = 2048
+CACHE = os.environ.get("AUTOGRAD_AMD_FUSE_CACHE", "1").strip() not in ("0", "")
+VERIFY = os.environ.get("AUTOGRAD_AMD_FUSE_VERIFY", "").strip() not in ("0", "")  # re-emit on every hit and compare
+
+
+def _signature(roots, order):
+    """``(key, tensors)``: the key described above and the distinct leaf tensors in the order the key numbers them;
+    None when an operand is of a kind the key does not describe."""
+    KNOWN = D.KNOWN_SCALARS
+    itemsize = roots[0].dtype.itemsize
+    index = {}
+    for k, n in enumerate(order):
+        index[id(n)] = k
+    tensors, ident, bases = [], {}, {}
+
+    def leaf_desc(t):
+        ptr, stride, shape = t.data_ptr(), t.stride(), tuple(t.shape)
+        if KNOWN:
+            c = KNOWN.get(ptr)
+            if c is not None and (t.numel() == 1 or builtins_all_zero(stride)):
+                return ("k", c, math.copysign(1.0, c))
+        key = (ptr, stride, shape)
+        k = ident.get(key)
+        if k is None:
+            k = ident[key] = len(tensors)
+            tensors.append(t)
+        off = t.storage_offset()
+        base = ptr - off * itemsize
+        b = bases.get(base)
+        if b is None:
+            b = bases[base] = len(bases)
+        return ("l", k, shape, stride, b, off)
+
+    def desc(a):
+        kind = type(a)
+        if kind is float:
+            return ("f", a, math.copysign(1.0, a))
+        if a is None:
+            return None
+        if kind is ExprArray and a._args is not None:
+            return ("n", index[id(a)])
+        if kind is LazyDevArray:
+            raw, scale, ascale, offset = D._state(a)
+            if offset is not None:
+                offset = ("f", offset, math.copysign(1.0, offset)) if type(offset) is float else leaf_desc(offset)
+            return ("z", leaf_desc(raw), scale, None if ascale is None else leaf_desc(ascale), offset)
+        if not isinstance(a, DevArray):
+            raise _Unsupported
+        return leaf_desc(a._t)
+
+    parts = []
+    try:
+        for n in order:
+            parts.append((n._op, n._lo if n._op == SHIFT else 0, tuple([desc(a) for a in n._args])))
+        where = tuple([index[id(r)] for r in roots])
+    except (_Unsupported, KeyError, TypeError):
+        return None
+    for n in order:
+        if n._args is None:
+            return None  # reading a deferred operand ran part of this very expression: described as it no longer is
+    return (roots[0].dtype, roots[0]._shape, where, tuple(parts)), tensors
+
+
+def _program_for(roots, order):
+    """``_emit`` and ``_bind`` through the cache: ``(leaves, imms, words, n_regs, shifted, masks)``, None (does not fit
+    one program) or False (a layout the kernel does not cover)."""
+    root = roots[0]
+    n_out = root._shape[0] if len(root._shape) == 1 else None
+    itemsize = root.dtype.itemsize
+    sig = _signature(roots, order) if CACHE else None
+    if sig is not None:
+        key, tensors = sig
+        hit = _PROGRAMS.get(key)
+        if hit is not None:
+            if hit[0] != "ok":
+                return None if hit[0] == "none" else False
+            _, slots, where, imms, words, n_regs, need_shifted, masks = hit
+            leaves, shifted = _bind([tensors[k] for k in slots], where, n_out, itemsize, need_shifted)
+            if VERIFY:
+                _verify(roots, (leaves, imms, words, n_regs, shifted, masks), n_out, itemsize)
+            return leaves, imms, words, n_regs, shifted, masks
+    try:
+        emitted = _emit(roots)
+        if emitted is not None:
+            raw, where, imms, words, n_regs, need_shifted, masks = emitted
+            leaves, shifted = _bind(raw, where, n_out, itemsize, need_shifted)
+    except _Unsupported:
+        emitted = False
+    if sig is not None:
+        if len(_PROGRAMS) >= _PROGRAM_LIMIT:
+            _PROGRAMS.clear()
+        if emitted is None:
+            _PROGRAMS[key] = ("none",)
+        elif emitted is False:
+            _PROGRAMS[key] = ("unsupported",)
+        else:
+            ident = {}
+            for k, t in enumerate(tensors):
+                ident[(t.data_ptr(), t.stride(), tuple(t.shape))] = k
+            try:
+                slots = tuple([ident[(t.data_ptr(), t.stride(), tuple(t.shape))] for t in raw])
+            except KeyError:
+                slots = None  # (a leaf the key's walk did not see: leave this expression uncached)
+            if slots is not None:
+                _PROGRAMS[key] = ("ok", slots, tuple(where), list(imms), list(words), n_regs, need_shifted, list(masks))
+    if emitted is None or emitted is False:
+        return emitted
+    return leaves, imms, words, n_regs, shifted, masks
+
+
+def _verify(roots, bound, n_out, itemsize):
+    raw, where, imms, words, n_regs, need_shifted, masks = _emit(roots)
+    leaves, shifted = _bind(raw, where, n_out, itemsize, need_shifted)
+    got_leaves, got_imms, got_words, got_regs, got_shifted, got_masks = bound
+    same = (list(got_words) == list(words) and got_regs == n_regs and list(got_masks) == list(masks)
+            and [repr(c) for c in got_imms] == [repr(c) for c in imms] and got_shifted == shifted
+            and len(got_leaves) == len(leaves)
+            and all(a.data_ptr() == b.data_ptr() and a.stride() == b.stride() and a.shape == b.shape
+                    for a, b in zip(got_leaves, leaves)))
+    if not same:
+        raise AssertionError("a kept program differs from the one emitted for the same expression")
 
 
 def slice_of(A, start, stop):

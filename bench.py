@@ -282,6 +282,20 @@ def make_workload(name, be):
     return (lambda x, v: (prog["hvp_rev"](x, v), prog["hvp_fwd"](x, v))), (x, v), cfg, "f64"
 
 
+def priced(r, steps, overhead_ms):
+    """One row of `kernels_per_step`: launches per step, average duration, algorithmic MB (and GFLOP) per launch and
+    the rates they give against the published peaks."""
+    ms = max(r["avg_ms"] - overhead_ms, 1e-6)
+    row = {"launches": r["launches"] / steps, "avg_ms": round(ms, 5), "MB": round(r["avg_bytes"] / 1e6, 3),
+           "GB/s": round(r["avg_bytes"] / (ms * 1e-3) / 1e9, 1),
+           "frac_hbm": round(r["avg_bytes"] / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+    if r.get("avg_flops"):
+        row["GFLOP"] = round(r["avg_flops"] / 1e9, 4)
+        row["TFLOP/s"] = round(r["avg_flops"] / (ms * 1e-3) / 1e12, 2)
+        row["frac_mfma"] = round(r["avg_flops"] / (ms * 1e-3) / 1e12 / MFMA_F32_PEAK_TFLOPS, 4)
+    return row
+
+
 def measured_traffic(kernel):
     """HBM bytes per launch of ``kernel`` from the committed rocprofv3 counter summary
     (profiles/bcast_grad_hbm_traffic.md: FETCH_SIZE + WRITE_SIZE scaled by a plain copy) and where the figure
@@ -357,7 +371,8 @@ def main():
         be.sync()
         elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
-    dom_eager = kt.summary()[dominant]
+    # (kernels that share a launch key carry events in turn: a label launched once per step may have had none)
+    dom_eager = kt.summary().get(dominant, {"avg_ms": None, "launches": 0})
     # the same K steps again, each behind a busy stream: the events bracket GPU execution only
     with _lib.KernelTimer(only={dom_key}, events=2 * args.steps * dom_launches) as kt:
         for _ in range(args.steps):
@@ -407,12 +422,10 @@ def main():
         "data": "synthetic",
         "config": config,
         "roofline": roofline,
-        "kernels_per_step": {
-            # (averages over the probe steps, the event pair's own cost subtracted)
-            name: {"launches": r["launches"] / PROBE_STEPS, "avg_ms": round(max(r["avg_ms"] - overhead_ms, 1e-6), 5),
-                   "GB/s": round(r["avg_bytes"] / (max(r["avg_ms"] - overhead_ms, 1e-6) * 1e-3) / 1e9, 1)}
-            for name, r in sorted(per_kernel.items(), key=lambda kv: -kv[1]["ms"])
-        },
+        # (averages over the probe steps, the event pair's own cost subtracted; one row per kernel AND shape, with
+        # the algorithmic bytes / flops of one launch, so that every rate can be recomputed from the row)
+        "kernels_per_step": {name: priced(r, PROBE_STEPS, overhead_ms)
+                             for name, r in sorted(per_kernel.items(), key=lambda kv: -kv[1]["ms"])},
     }
 
     if args.calibrate_copy:
