@@ -176,6 +176,60 @@ def W(op, dst, a=0, b=0, c=0, d=0):
     return op | dst << 8 | a << 12 | b << 16 | c << 20 | d << 24
 
 
+def test_kept_programs_are_found_by_structure_and_bound_to_new_tensors(dnp):
+    """A loop evaluates the same expression again and again: its program is emitted once and found again by the
+    structure of the expression; what differs between two expressions of one structure (which arrays, which of them
+    are one and the same array, scalar values, the sign of a zero) either is bound anew or gives another program."""
+    from autograd_amd.numpy import fusion
+
+    rs = onp.random.RandomState(5)
+    n = 10007
+    fusion._PROGRAMS.clear()
+
+    def f(x, y, c):
+        return dnp.tanh(x * y + c) / (dnp.exp(x) + 2.0) - y
+
+    def ref(x, y, c):
+        return onp.tanh(x * y + c) / (onp.exp(x) + 2.0) - y
+
+    for k in range(6):
+        x, y = rs.randn(n), rs.randn(n)
+        got = f(dnp.asarray(x), dnp.asarray(y), 0.5).numpy()
+        with unfused():
+            want = f(dnp.asarray(x), dnp.asarray(y), 0.5).numpy()
+        assert onp.array_equal(got, want) and onp.allclose(got, ref(x, y, 0.5), rtol=1e-13, atol=0)
+        assert len(fusion._PROGRAMS) == 1, k
+    # the same array in both places is another structure (one leaf, not two), and so is another scalar
+    x = rs.randn(n)
+    X = dnp.asarray(x)
+    assert onp.array_equal(f(X, X, 0.5).numpy(), ref(x, x, 0.5)) or onp.allclose(f(X, X, 0.5).numpy(), ref(x, x, 0.5), rtol=1e-13)
+    assert len(fusion._PROGRAMS) == 2
+    y = rs.randn(n)
+    got = f(X, dnp.asarray(y), -0.25).numpy()
+    with unfused():
+        assert onp.array_equal(got, f(X, dnp.asarray(y), -0.25).numpy())
+    assert len(fusion._PROGRAMS) == 3
+    # 0.0 and -0.0 are different immediates: 1 / (x * 0.0) against 1 / (x * -0.0)
+    pos = (1.0 / (dnp.abs(X) * 0.0 + 0.0)).numpy()
+    neg = (1.0 / (dnp.abs(X) * -0.0 + -0.0)).numpy()
+    assert onp.all(pos == onp.inf) and onp.all(neg == -onp.inf)
+    # views of one array at different offsets (the Rosenbrock pattern) against two separate arrays of the same sizes
+    fusion._PROGRAMS.clear()
+    g = lambda a, b: (a * 3.0 + b * b).numpy()  # noqa: E731
+    z = rs.randn(n + 1)
+    Z = dnp.asarray(z)
+    assert onp.array_equal(g(Z[1:], Z[:-1]), z[1:] * 3.0 + z[:-1] * z[:-1])
+    u, v = rs.randn(n), rs.randn(n)
+    assert onp.array_equal(g(dnp.asarray(u), dnp.asarray(v)), u * 3.0 + v * v)
+    assert onp.array_equal(g(Z[1:], Z[:-1]), z[1:] * 3.0 + z[:-1] * z[:-1])
+    # with the cache off the same programs come out
+    was, fusion.CACHE = fusion.CACHE, False
+    try:
+        assert onp.array_equal(g(Z[1:], Z[:-1]), z[1:] * 3.0 + z[:-1] * z[:-1])
+    finally:
+        fusion.CACHE = was
+
+
 @pytest.mark.parametrize("dtype", [F64, F32])
 @pytest.mark.parametrize("shape", [(1,), (3, 7), (1000003,), (1024, 1000), (5, 3, 130), (513, 2)])
 def test_program_equals_the_one_rule_kernels(dtype, shape):
