@@ -63,7 +63,9 @@ def grad(fun, x):
 @unary_to_nary
 def value_and_grad(fun, x):
     """Like ``grad``, returning ``(fun's value, gradient)`` from the one forward pass."""
-    return _seeded_with_ones(fun, x, "value_and_grad")
+    value, gradient = _seeded_with_ones(fun, x, "value_and_grad")
+    settle = getattr(core, "settle", None)  # (a hosting package's core has none: values then stay as they are)
+    return (settle(value) if settle is not None else value), gradient  # deferred arithmetic is completed here, as the gradient's is
 
 
 @unary_to_nary
@@ -83,6 +85,9 @@ def deriv(fun, x):
     return core.make_jvp(fun, x)(vspace(x).ones())[1]
 
 
+JACOBIAN_BLOCK_BYTES = 4 << 30  # what the stacked cotangents of one replay of `jacobian` may hold (estimate, see there)
+
+
 @unary_to_nary
 def jacobian(fun, x):
     """Jacobian of an array-valued ``fun`` of an array (or scalar): output axes first, input axes
@@ -95,9 +100,19 @@ def jacobian(fun, x):
     out_space, in_space = vspace(ans), vspace(x)
     stacked_basis = getattr(out_space, "stacked_standard_basis", None)
     if pull_back_all is not None and stacked_basis is not None and out_space.size > 0 and type(in_space) is type(out_space):
-        # all basis cotangents in ONE replay of the tape, stacked along a leading axis
+        # all basis cotangents in ONE replay of the tape, stacked along a leading axis; every cotangent on the tape then
+        # carries that axis, so a large output space goes through in blocks of basis vectors that keep the stacked
+        # values within a byte budget (a tape is taken to hold a few values of about its larger end's size per vector)
+        n = out_space.size
+        per_vector = 16 * max(in_space.size, n, 1) * getattr(getattr(out_space, "dtype", None), "itemsize", 8)
+        block = max(1, min(n, JACOBIAN_BLOCK_BYTES // per_vector))
         try:
-            rows = pull_back_all(stacked_basis(), out_space.size, lambda value, i: value[i], np.stack)
+            basis = stacked_basis()
+            if block >= n:
+                rows = pull_back_all(basis, n, lambda value, i: value[i], np.stack)
+            else:
+                rows = np.concatenate([pull_back_all(basis[k:k + block], min(block, n - k), lambda value, i: value[i], np.stack)
+                                       for k in range(0, n, block)], axis=0)
             return np.reshape(rows, out_space.shape + in_space.shape)
         except core.NotBatchable:
             pass

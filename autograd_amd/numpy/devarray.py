@@ -1194,6 +1194,20 @@ class PendingReduce(DevArray):
 _DEFERRED = _DEFERRED + (PendingReduce,)
 
 
+def _kept(x):
+    """An operand as a deferred reduction keeps it: the array is marked as read by something pending (an item assignment
+    then moves the ARRAY's handle to a buffer of its own) and the reduction holds a handle of its own on the memory as it
+    is now."""
+    if isinstance(x, DevArray):
+        x._borrowed = True
+        kind = type(x)
+        if kind is DevArray:
+            return DevArray(x._t, x.dtype)
+        if kind is LazyDevArray:
+            return LazyDevArray(x._raw, x.dtype, x._scale, x._shift, x._ascale, x._producer)
+    return x
+
+
 def map_reduce(op, red, dtype, xs, axes, keepdims, shape=None):
     """``RED_axes op(xs...)`` with ``xs`` broadcast to ``shape`` (default: their broadcast); left pending while an
     operand is a pending expression (see :class:`PendingReduce`)."""
@@ -1206,11 +1220,16 @@ def map_reduce(op, red, dtype, xs, axes, keepdims, shape=None):
                     for y in xs:
                         if isinstance(y, DevArray) and y.shape != full:
                             full = broadcast_shapes(full, y.shape)
-                for y in xs:
-                    if isinstance(y, DevArray):
-                        y._borrowed = True
                 axes = tuple(axes)
-                return PendingReduce((op, red, dtype, tuple(xs), axes, keepdims, shape), reduce_shape(full, axes, keepdims), dtype)
+                return PendingReduce((op, red, dtype, tuple([_kept(y) for y in xs]), axes, keepdims, shape),
+                                     reduce_shape(full, axes, keepdims), dtype)
+        if red == Red.SUM and op == Op.COPY and len(xs) == 1 and shape is None and isinstance(xs[0], DevArray):
+            # The sum of a whole array, the last step of most losses: `grad` never reads its value (the cotangent of a sum
+            # needs none of it), so it runs when something does (`value_and_grad`, a print, arithmetic on the scalar).
+            x = xs[0]
+            axes = tuple(axes)
+            if len(axes) == x.ndim and x.size > 0:
+                return PendingReduce((op, red, dtype, (_kept(x),), axes, keepdims, None), reduce_shape(x.shape, axes, keepdims), dtype)
     return _map_reduce_now(op, red, dtype, xs, axes, keepdims, shape)
 
 

@@ -49,6 +49,26 @@ def test_jacobian_and_hessian_match_the_per_element_loop():
             assert onp.allclose(got_h, want_h, rtol=1e-10, atol=1e-10 * onp.max(onp.abs(want_h))), name
 
 
+def test_a_large_output_space_goes_through_in_blocks(monkeypatch):
+    """The stacked cotangents of one replay are kept within a byte budget: with a budget of a few basis vectors the
+    Jacobian comes out of several replays, row block by row block, and is the same array."""
+    import autograd_amd as ag
+    import autograd_amd.numpy as dnp
+    from autograd_amd import differential_operators as ops
+    from autograd_amd.scipy.special import logsumexp
+
+    progs = _programs(dnp, logsumexp, dnp.asarray)
+    for name in ("dense layer", "logsumexp", "broadcasts", "running sum", "two layers"):
+        f, x0 = progs[name]
+        x = dnp.asarray(x0)
+        whole = ag.jacobian(f)(x).numpy()
+        n_out, n_in = whole.size // max(x0.size, 1), x0.size
+        monkeypatch.setattr(ops, "JACOBIAN_BLOCK_BYTES", 3 * 16 * max(n_in, n_out) * 8)  # three basis vectors per replay
+        blocks = ag.jacobian(f)(x).numpy()
+        monkeypatch.undo()
+        assert onp.array_equal(blocks, whole), name
+
+
 def test_launch_count_of_a_jacobian_does_not_depend_on_the_output_size():
     import autograd_amd as ag
     import autograd_amd.numpy as dnp
