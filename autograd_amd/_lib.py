@@ -112,7 +112,7 @@ class AgmiCorrelation(ctypes.Structure):
 
 class AgmiGemmEpilogue(ctypes.Structure):
     _fields_ = [("kind", ctypes.c_int32), ("bias", ctypes.c_void_p), ("out", ctypes.c_void_p), ("out_ld", ctypes.c_int64),
-                ("x", ctypes.c_void_p), ("x_ld", ctypes.c_int64)]
+                ("x", ctypes.c_void_p), ("x_ld", ctypes.c_int64), ("beta", ctypes.c_double)]
 
 
 class AgmiLseCotangent(ctypes.Structure):
@@ -658,10 +658,11 @@ EPILOGUE_BIAS_TANH, EPILOGUE_TANH_VJP = 1, 2
 _epilogue = AgmiGemmEpilogue()
 
 
-def gemm_fused(code, A, B, C, kind, bias=None, out=None, x=None):
-    """``agmi_gemm_fused``: ``A @ B`` (2-d tensors, any strides) into the contiguous ``C`` with a dense layer's
-    epilogue: ``out = tanh(C + bias)`` beside it, or ``C = (A @ B) / cosh(x + bias)**2`` (``bias``: contiguous
-    vector or None).  Returns False when the operands are outside what the fused kernel covers."""
+def gemm_fused(code, A, B, C, kind, bias=None, out=None, x=None, beta=0.0):
+    """``agmi_gemm_fused``: ``A @ B`` (2-d tensors, any strides; plus ``beta`` times what ``C`` holds) into the
+    contiguous ``C`` with a dense layer's epilogue: ``out = tanh(C + bias)`` beside it, or
+    ``C = (A @ B + beta * C) / cosh(x + bias)**2`` (``bias``: contiguous vector or None).  Returns False when the
+    operands are outside what the fused kernel covers."""
     M, K = A.shape
     N = B.shape[1]
     e = _epilogue
@@ -669,6 +670,7 @@ def gemm_fused(code, A, B, C, kind, bias=None, out=None, x=None):
     e.bias = bias.data_ptr() if bias is not None else None
     e.out, e.out_ld = (out.data_ptr(), out.stride(0)) if out is not None else (None, 0)
     e.x, e.x_ld = (x.data_ptr(), x.stride(0)) if x is not None else (None, 0)
+    e.beta = beta
     ev = _TIMER.begin(("gemm",)) if _TIMER is not None else None
     rc = _LIB.agmi_gemm_fused(code, M, N, K, A.data_ptr(), A.stride(0), A.stride(1), B.data_ptr(), B.stride(0), B.stride(1),
                               C.data_ptr(), C.stride(0), ctypes.byref(e), _workspace().data_ptr(), _WORKSPACE_BYTES, _stream())

@@ -1059,6 +1059,10 @@ static int launch_direct(GemmParams p, int64_t batch, hipStream_t s, void *ws, s
             p.ws = ws;
         }
     }
+    if (p.splits > 1 && p.epi != 0 && p.beta != 0.0) {
+        set_error("gemm_fused: a product cut along K across blocks takes no beta together with an epilogue");
+        return AGMI_ERR_UNSUPPORTED;
+    }
     if (p.splits > 1)
         set_kernel_name("gemm_direct<f32,64,64,32,%s%s>+split%d[%lldx%lldx%lld]", mode_name(mode_a), mode_name(mode_b), p.splits,
                         (long long)p.M, (long long)p.N, (long long)p.K);
@@ -1206,7 +1210,7 @@ extern "C" int agmi_gemm_fused(int dtype, int64_t M, int64_t N, int64_t K, const
     p.a_rs = a_rs; p.a_cs = a_cs;
     p.b_rs = b_rs; p.b_cs = b_cs;
     p.ldc = ldc;
-    p.alpha = 1.0; p.beta = 0.0;
+    p.alpha = 1.0; p.beta = e->beta;
     p.epi = e->kind;
     p.epi_bias = static_cast<const float *>(e->bias);
     p.epi_out = static_cast<float *>(e->out);

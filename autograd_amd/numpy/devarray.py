@@ -362,9 +362,31 @@ class PendingProduct(DevArray):
     def into_tanh_cotangent(self, x, bias, out):
         """``out = (left @ right) / cosh(x + bias)**2`` in one launch (the product itself stays uncomputed); False when
         the fused kernel does not take these operands."""
-        if not self._shape[0] or not self._shape[1] or not self._left.shape[1] or self._more:
+        if not self._shape[0] or not self._shape[1] or not self._left.shape[1]:
             return False
-        return _lib.gemm_fused(_lib.DTYPE_CODE[self.dtype], self._left, self._right, out, _lib.EPILOGUE_TANH_VJP, bias=bias, x=x)
+        code = _lib.DTYPE_CODE[self.dtype]
+        if not self._more:
+            return _lib.gemm_fused(code, self._left, self._right, out, _lib.EPILOGUE_TANH_VJP, bias=bias, x=x)
+        # A sum of products (the state of a recurrent net receives one cotangent from the next step and one from the
+        # output head): all but the last are contracted into `out`, the last one adds what `out` holds to its
+        # accumulators (beta = 1) before the tanh rule is applied to them.
+        if len(self._more) > 3 or x.data_ptr() == out.data_ptr():
+            return False
+        terms = [(self._left, self._right)] + self._more
+        last_left, last_right = terms[-1]
+        M, N = self._shape
+        K = last_left.shape[1]
+        # (checked before anything runs, so that a refusal leaves nothing half done: the fused kernel wants a unit stride
+        # in each operand, spans below 2 GiB, and no cut of a very long K across blocks when it also reads C)
+        if not K or (last_left.stride(0) != 1 and last_left.stride(1) != 1) or (last_right.stride(0) != 1 and last_right.stride(1) != 1) \
+                or max(last_left.numel(), last_right.numel(), M * N) >= 1 << 28 or last_left.stride(0) < 0 or last_left.stride(1) < 0 \
+                or last_right.stride(0) < 0 or last_right.stride(1) < 0 or (K > 4096 and -(-M // 64) * -(-N // 64) < 128):
+            return False
+        for k, (l, r) in enumerate(terms[:-1]):
+            gemm2d(l, r, self.dtype, out=out, beta=1.0 if k else 0.0)
+        if not _lib.gemm_fused(code, last_left, last_right, out, _lib.EPILOGUE_TANH_VJP, bias=bias, x=x, beta=1.0):
+            raise RuntimeError("the fused contraction refused operands that were checked against its limits")
+        return True
 
     def computed(self):
         return self._left is None

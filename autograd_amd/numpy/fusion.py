@@ -343,6 +343,7 @@ def _dense_layer(node):
         g, x = node._args
         if type(g) is not D.PendingProduct or g.computed() or g.shape != node._shape:
             return False
+        x = D.in_memory(x)  # (a forward product that has run is a plain array by now)
         bias = None
         if type(x) is DevArray:
             xt = x._t

@@ -1036,6 +1036,10 @@ def take(A, idx):
             rows = _leading_rows(pidx, A.shape)
             if rows is not None and rows[1] > rows[0]:
                 return D._fusion.slice_of(A, rows[0], rows[1])  # a slice of a vector that is still an expression stays one
+        if type(A) is D.PendingProduct and not backwards and D._fusion.ENABLED:
+            part = _part_of_product(A, pidx)
+            if part is not None:
+                return part
         picked = A._view(lambda t: t[pidx])
         return _reverse_axes(picked, backwards) if backwards else picked
     if A.ndim == 0:
@@ -1048,6 +1052,30 @@ def take(A, idx):
         return _gather(A, rows, A.shape[0], inner, (rows.size,) + A.shape[1:])
     plan = _index_plan(A.shape, idx)
     return _gather(A, plan.positions, plan.n_rows, plan.inner, plan.shape)
+
+
+def _part_of_product(P, pidx):
+    """``P[r0:r1, c0:c1]`` of a matrix product that has not run yet, as the product of the factors' rows and columns
+    (nothing runs; None when this is not such a slice).  The cotangent of an `hstack` hands each piece its columns of the
+    stacked cotangent (numpy_vjps.py:783-788 `grad_concatenate_args`); when that cotangent is `G . W^T` only the columns
+    of a traced piece are ever read (a recurrent net's state between its input and the column of ones), so only they
+    are contracted, and the product stays one that a sum or a tanh rule can still take into its own launch.  Slices of
+    less than half of an axis are views of the whole product as before: several small pieces of one product are cheaper
+    contracted together."""
+    if P.computed() or P._more or P._out is not None:
+        return None
+    if type(pidx) is not tuple:
+        pidx = (pidx,)
+    if len(pidx) > 2 or not builtins.all(type(i) is slice for i in pidx):
+        return None
+    rows, cols = P.shape
+    r0, r1, rs = pidx[0].indices(rows)
+    c0, c1, cs = pidx[1].indices(cols) if len(pidx) == 2 else (0, cols, 1)
+    if rs != 1 or cs != 1 or r1 <= r0 or c1 <= c0 or (r1 - r0, c1 - c0) == (rows, cols):
+        return None
+    if 2 * (r1 - r0) < rows or 2 * (c1 - c0) < cols:
+        return None
+    return D.PendingProduct(P._left[r0:r1], P._right[:, c0:c1], P.dtype)
 
 
 def assign_items(A, idx, value):

@@ -318,14 +318,17 @@ int agmi_gemm(int dtype, int64_t batch, int64_t M, int64_t N, int64_t K, double 
               double beta, void *C, int64_t ldc, int64_t c_bs,
               void *workspace, size_t workspace_bytes, void *stream);
 
-/* agmi_gemm (float32, one matrix, alpha = 1, beta = 0) with what follows the contraction in a dense layer
+/* agmi_gemm (float32, one matrix, alpha = 1) with what follows the contraction in a dense layer
  * applied to the accumulators before they are stored, so that the layer costs one launch:
  *   AGMI_EPILOGUE_BIAS_TANH  C = A.B as agmi_gemm stores it, and beside it
  *                            out[m,n] = tanh(C[m,n] + bias[n])          examples/neural_net.py:33-35
  *   AGMI_EPILOGUE_TANH_VJP   C[m,n] = (A.B)[m,n] / cosh(x[m,n] + bias[n])**2: the tanh rule applied to the
  *                            cotangent G.W^T while it is formed          autograd/numpy/numpy_vjps.py:178, 615-624
- * bias may be NULL (nothing is added).  Each step is rounded as the separate kernels round it (the bias as a
- * pending `+ bias`, tanh / cosh as AGMI_OP_TANH / AGMI_OP_TANH_VJP), so the results are theirs bit for bit.
+ * bias may be NULL (nothing is added).  With beta != 0 the product is A.B + beta * C (what C held) before the
+ * epilogue: the cotangent that reaches a tanh is often the sum of two such products (the state of a recurrent net is
+ * read by the next step and by the output head, examples/rnn.py:37-50; core.py:185-205), the first of which has been
+ * stored in C.  Each step is rounded as the separate kernels round it (the bias as a pending `+ bias`, the sum as
+ * agmi_gemm's beta, tanh / cosh as AGMI_OP_TANH / AGMI_OP_TANH_VJP), so the results are theirs bit for bit.
  * A and B as in agmi_gemm; each needs one unit stride and byte spans below 2 GiB, else AGMI_ERR_UNSUPPORTED (the
  * caller then runs agmi_gemm and the elementwise kernel). */
 #define AGMI_EPILOGUE_BIAS_TANH 1
@@ -337,6 +340,7 @@ typedef struct agmi_gemm_epilogue {
     int64_t out_ld;
     const void *x;     /* TANH_VJP: [M][N] with leading dimension x_ld */
     int64_t x_ld;
+    double beta;       /* 0: C is only written */
 } agmi_gemm_epilogue;
 int agmi_gemm_fused(int dtype, int64_t M, int64_t N, int64_t K,
                     const void *A, int64_t a_rs, int64_t a_cs, const void *B, int64_t b_rs, int64_t b_cs,

@@ -1539,6 +1539,63 @@ def test_gemm_epilogues_equal_the_separate_kernels(dnp, M, N, K):
             out = _lib.empty((M, N), onp.dtype(F32))
             assert _lib.gemm_fused(code, a, b, out, _lib.EPILOGUE_TANH_VJP, bias=vec, x=x._t)
             assert onp.array_equal(out.cpu().numpy(), want_vjp)
+            # beta = 1: the product joins what the output holds (an earlier product) before the rule is applied
+            first = rs.randn(M, N).astype(F32)
+            summed = DevArray_from(D.gemm2d(a, b, onp.dtype(F32), out=P(dnp, first)._t.clone(), beta=1.0))
+            want_sum = D.plain(D.map_op(Op.TANH_VJP, onp.dtype(F32), summed, zx)).numpy()
+            out = P(dnp, first)._t.clone()
+            assert _lib.gemm_fused(code, a, b, out, _lib.EPILOGUE_TANH_VJP, bias=vec, x=x._t, beta=1.0)
+            assert onp.array_equal(out.cpu().numpy(), want_sum)
+
+
+def test_the_tanh_rule_over_a_sum_of_sliced_products_is_one_chain_of_contractions(dnp):
+    """The state of a recurrent net is read by the next step and by the output head (examples/rnn.py:37-50): its cotangent is
+    the sum of two `G . W^T` products, of each of which only the state's columns are wanted (the `hstack` rule slices
+    them out), and the tanh rule follows.  The slices stay products of the factors' columns, the sum stays a sum of
+    products, and the rule runs in the second contraction's epilogue: same bits as product, slice, add and rule one
+    by one."""
+    import autograd_amd as ag
+    from autograd_amd import _lib
+    from autograd_amd.numpy import devarray as D
+    from autograd_amd.numpy import fusion, wrapper
+
+    rs = onp.random.RandomState(12)
+    B_, I, H, O = 64, 24, 96, 20
+    Wc, Wp = P(dnp, (0.2 * rs.randn(I + H + 1, H)).astype(F32)), P(dnp, (0.2 * rs.randn(H + 1, O)).astype(F32))
+    x0, h0 = P(dnp, rs.randn(B_, I).astype(F32)), P(dnp, rs.randn(B_, H).astype(F32))
+    t1, t2 = P(dnp, rs.randn(B_, O).astype(F32)), P(dnp, rs.randn(B_, H).astype(F32))
+    ones = dnp.ones((B_, 1), dtype=F32)
+
+    def f(h):
+        h1 = dnp.tanh(dnp.dot(dnp.hstack((x0, h, ones)), Wc))
+        head = dnp.dot(dnp.hstack((h1, ones)), Wp)
+        h2 = dnp.tanh(dnp.dot(dnp.hstack((x0, h1, ones)), Wc))
+        return dnp.sum(head * t1) + dnp.sum(h2 * t2)
+
+    names = []
+    real_fused, real_gemm = _lib.gemm_fused, _lib.gemm
+    _lib.gemm_fused = lambda *a, **k: (names.append(("fused", k.get("beta", 0.0))), real_fused(*a, **k))[1]
+    _lib.gemm = lambda *a, **k: (names.append(("gemm", a[2:5])), real_gemm(*a, **k))[1]
+    try:
+        got = ag.grad(f)(h0).numpy()
+    finally:
+        _lib.gemm_fused, _lib.gemm = real_fused, real_gemm
+    assert ("fused", 1.0) in names                                   # the rule of h1 ran on a sum of two products
+    assert ("gemm", (B_, H, H)) in names and ("gemm", (B_, I + H + 1, H)) not in names   # only the state's columns were contracted
+    was, fusion.ENABLED = fusion.ENABLED, False
+    try:
+        want = ag.grad(f)(h0).numpy()
+    finally:
+        fusion.ENABLED = was
+    assert onp.array_equal(got, want)
+    # a slice of less than half of an axis is a view of the whole product
+    Pd = D.PendingProduct(x0._t, P(dnp, rs.randn(I, 50).astype(F32))._t, onp.dtype(F32))
+    small = wrapper.take(Pd, (slice(None), slice(0, 10)))
+    assert type(small) is not D.PendingProduct and Pd.computed()
+    Pd = D.PendingProduct(x0._t, P(dnp, rs.randn(I, 50).astype(F32))._t, onp.dtype(F32))
+    big = wrapper.take(Pd, (slice(8, None), slice(0, 40)))
+    assert type(big) is D.PendingProduct and not Pd.computed() and big.shape == (B_ - 8, 40)
+    assert onp.array_equal(big.numpy(), D.plain(Pd).numpy()[8:, :40])
 
 
 def DevArray_from(t):
