@@ -465,7 +465,7 @@ __global__ __launch_bounds__(kBlock) void red_cols(const RedParams p, const int 
 #pragma unroll
     for (int j = 0; j < V; ++j) acc[j] = Acc::identity();
     if (active) {
-#pragma unroll 4
+#pragma unroll 16
         for (int64_t r = r_begin + ty; r < r_end; r += TY) {
             T x[F<T>::NIN + AGMI_MAX_AUX][V];
             load_points<F, T, V, 2>(p, o, r, i0, x);
@@ -491,6 +491,70 @@ __global__ __launch_bounds__(kBlock) void red_cols(const RedParams p, const int 
     if (active && ty == 0) {
 #pragma unroll
         for (int j = 0; j < V; ++j) store_result<Acc, T, FINAL>(p, acc[j], o, i0 + j, chunk);
+    }
+}
+
+// Column sums of one plain operand with unit stride along i, whole extent of r in one block (the single-launch plan of
+// small operands).  The general kernel above decides per operand how to load (scalar, broadcast, pending map) inside
+// its row loop, and a load behind a condition is waited for where the branches join: a thread's rows went out one
+// round trip at a time (10 us for 1024 rows).  Here the loads carry no conditions and eight rows are in flight.
+// Same order of additions as the general kernel's single-chunk form.
+template <typename T, int V>
+__global__ __launch_bounds__(kBlock) void col_sums_plain(const T *__restrict__ x, int64_t R, int64_t I, int64_t x_o, int64_t x_r,
+                                                         T *__restrict__ out, int64_t out_o, int64_t out_i, const int TX) {
+    typedef T vec_t __attribute__((ext_vector_type(V > 1 ? V : 2), aligned(sizeof(T))));
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T *smem = reinterpret_cast<T *>(smem_raw);
+    const int TY = kBlock / TX;
+    const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
+    const int64_t i0 = (static_cast<int64_t>(blockIdx.x) * TX + tx) * V;
+    const int64_t o = blockIdx.y;
+    const bool active = i0 < I;  // (I % V == 0 when V > 1)
+    const T *col = x + o * x_o + (active ? i0 : 0);
+    T acc[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) acc[j] = T(0);
+    int64_t r = ty;
+    for (; r + 7 * static_cast<int64_t>(TY) < R; r += 8 * static_cast<int64_t>(TY)) {
+        T v[8][V];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const T *src = col + (r + u * static_cast<int64_t>(TY)) * x_r;
+            if (V > 1) {
+                const vec_t t = *reinterpret_cast<const vec_t *>(src);
+#pragma unroll
+                for (int j = 0; j < V; ++j) v[u][j] = t[j];
+            } else {
+                v[u][0] = *src;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+#pragma unroll
+            for (int j = 0; j < V; ++j) acc[j] = acc[j] + v[u][j];
+    }
+    for (; r < R; r += TY) {
+#pragma unroll
+        for (int j = 0; j < V; ++j) acc[j] = acc[j] + col[r * x_r + j];
+    }
+    if (TY > 1) {
+#pragma unroll
+        for (int j = 0; j < V; ++j) smem[(ty * TX + tx) * V + j] = acc[j];
+        __syncthreads();
+        for (int half = TY >> 1; half > 0; half >>= 1) {
+            if (ty < half) {
+#pragma unroll
+                for (int j = 0; j < V; ++j) {
+                    acc[j] = acc[j] + smem[((ty + half) * TX + tx) * V + j];
+                    smem[(ty * TX + tx) * V + j] = acc[j];
+                }
+            }
+            __syncthreads();
+        }
+    }
+    if (active && ty == 0) {
+#pragma unroll
+        for (int j = 0; j < V; ++j) out[o * out_o + (i0 + j) * out_i] = acc[j];
     }
 }
 
@@ -610,6 +674,13 @@ static RedPlan plan_reduce(int64_t O, int64_t R, int64_t I, int vec, bool vec_ok
         // block's threads walk different rows, so many blocks fit across I and few chunks are needed
         const int tx_full = std::max<int>(1, 256 / (pl.V * static_cast<int>(elem_size)));
         pl.TX = std::min<int>(tx_full, pow2_ceil(ceil_div(I, pl.V)));
+        // A small operand (the column sums of a 1024 x 1024 cotangent: a bias gradient) is one launch: cutting R into
+        // chunks would fill the machine, but the second kernel that adds the chunks costs more than the first one saves.
+        // Narrower thread rows (down to 64 bytes) put more blocks across I instead.
+        if (R <= 4096 && static_cast<size_t>(O * R * I) * elem_size <= (size_t(8) << 20)) {
+            while (pl.TX > 4 && ceil_div(ceil_div(I, pl.V), pl.TX) * O < 64) pl.TX >>= 1;
+            return pl;
+        }
         const int TY = kBlock / pl.TX;
         const int64_t blocks_x = ceil_div(ceil_div(I, pl.V), pl.TX);
         int64_t chunks = std::min<int64_t>(ceil_div(kTargetBlocks, blocks_x * O), ceil_div(R, static_cast<int64_t>(TY) * 8));
@@ -744,6 +815,22 @@ static int launch_reduce(const char *fname, const RedParams &base, bool vec_ok, 
         }
         const dim3 grid((unsigned)blocks_x, (unsigned)(p.O * pl.n_chunks));
         const size_t smem = (kBlock / pl.TX > 1) ? sizeof(acc_t) * kBlock * pl.V : 0;
+        if constexpr (std::is_same<AccT<T>, AccSum<T>>::value && std::is_same<F<T>, FCopy<T>>::value) {
+            // one plain operand, unit stride along i, one chunk: the kernel whose loads carry no conditions
+            if (!two_stage && !(p.scalar_mask & 1u) && !((p.scale_mask | p.shift_mask) & 1u) && p.n_aux == 0 && p.istr[0][2] == 1 &&
+                p.scale_aux[0] < 0 && p.shift_aux[0] < 0) {
+                set_kernel_name("col_sums_plain[%lldx%lldx%lld]", (long long)p.O, (long long)p.R, (long long)p.I);
+                const T *x = static_cast<const T *>(p.in[0]);
+                T *out = static_cast<T *>(p.out);
+                if (pl.V > 1)
+                    hipLaunchKernelGGL((col_sums_plain<T, VEC>), grid, dim3(kBlock), smem, s, x, p.R, p.I, p.istr[0][0], p.istr[0][1], out,
+                                       p.ostr_o, p.ostr_i, pl.TX);
+                else
+                    hipLaunchKernelGGL((col_sums_plain<T, 1>), grid, dim3(kBlock), smem, s, x, p.R, p.I, p.istr[0][0], p.istr[0][1], out,
+                                       p.ostr_o, p.ostr_i, pl.TX);
+                goto launched;
+            }
+        }
         set_kernel_name("red_cols<%s>%s[%lldx%lldx%lld]", fname, two_stage ? "+red_finish" : "", (long long)p.O, (long long)p.R, (long long)p.I);
 #define AGMI_COL(VV)                                                                                          \
     do {                                                                                                      \

@@ -460,6 +460,13 @@ def test_dot_vector_forms_matmul_tensordot(dnp, dtype):
     close(dnp.matmul(P(dnp, B3), P(dnp, C3[0])).numpy(), onp.matmul(B3, C3[0]), rt)
     close(dnp.matmul(P(dnp, A), P(dnp, C3)).numpy(), onp.matmul(A, C3), rt)
     close(dnp.matmul(P(dnp, B3), P(dnp, v)).numpy(), onp.matmul(B3, v), rt)
+    # batches of small outputs with a long K (float32: the K split inside one block, one block row of the grid per matrix)
+    B4, C4 = rs.randn(3, 40, 300).astype(dtype), rs.randn(3, 300, 50).astype(dtype)
+    long_k = rt * onp.sqrt(300) / 8
+    close(dnp.matmul(P(dnp, B4), P(dnp, C4)).numpy(), onp.matmul(B4, C4), long_k)
+    close(dnp.matmul(P(dnp, B4), P(dnp, C4[1])).numpy(), onp.matmul(B4, C4[1]), long_k)
+    close(dnp.matmul(dnp.swapaxes(P(dnp, onp.ascontiguousarray(B4.transpose(0, 2, 1))), 1, 2), P(dnp, C4)).numpy(),
+          onp.matmul(B4, C4), long_k)
     T1, T2 = rs.randn(2, 3, 5, 4).astype(dtype), rs.randn(5, 4, 2, 3).astype(dtype)
     close(dnp.tensordot(P(dnp, T1), P(dnp, T2), 2).numpy(), onp.tensordot(T1, T2, 2), rt)
     close(dnp.tensordot(P(dnp, T1), P(dnp, T2), [[0, 1], [2, 3]]).numpy(), onp.tensordot(T1, T2, [[0, 1], [2, 3]]), rt)
