@@ -165,6 +165,10 @@ def lib():
     L.agmi_version.argtypes = []
     L.agmi_last_kernel.restype = ctypes.c_char_p
     L.agmi_last_kernel.argtypes = []
+    L.agmi_probe_arm.restype = ctypes.c_int
+    L.agmi_probe_arm.argtypes = []
+    L.agmi_probe_elapsed.restype = ctypes.c_int
+    L.agmi_probe_elapsed.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_float)]
     L.agmi_elementwise.restype = c_i
     L.agmi_elementwise.argtypes = [c_i, c_i, c_i, p_i64, c_i, p_arr, c_i, p_arr, p_d, c_p]
     L.agmi_program.restype = c_i
@@ -215,7 +219,7 @@ def lib():
 EXPORTS = (
     "agmi_last_error agmi_version agmi_last_kernel agmi_elementwise agmi_program agmi_compare agmi_cast agmi_map_reduce "
     "agmi_map_reduce_workspace_bytes agmi_map_reduce_static agmi_gemm agmi_gemm_fused agmi_fill agmi_take_rows agmi_sort_rows agmi_cumsum agmi_reverse agmi_triangle agmi_scatter_add_rows agmi_optimizer_step "
-    "agmi_correlate agmi_lse_cotangent_fused agmi_concat"
+    "agmi_correlate agmi_lse_cotangent_fused agmi_concat agmi_probe_arm agmi_probe_elapsed"
 ).split()
 
 
@@ -314,8 +318,10 @@ class KernelTimer:
                 return None
         return self._event()
 
-    def end(self, ev0, key, nbytes, flops=0.0):
-        """``nbytes``: the algorithmic bytes, or ``(outs, ins)`` to have them counted (once per key and shape)."""
+    def end(self, ev0, key, nbytes, flops=0.0, probe=None):
+        """``nbytes``: the algorithmic bytes, or ``(outs, ins)`` to have them counted (once per key and shape).
+        ``probe``: index of the event pair the library itself recorded around the first kernel of an entry point that
+        launches several (``agmi_probe_arm``): that pair gives the kernel's duration, this one the whole call's."""
         ev1 = self._event()
         if type(nbytes) is tuple:
             outs, ins = nbytes
@@ -327,20 +333,28 @@ class KernelTimer:
                 if nbytes is None:
                     nbytes = self._traffic[sig] = _traffic(outs, ins)
         name = _LIB.agmi_last_kernel().decode()
-        self.records.append((name, key, ev0, ev1, nbytes, flops))
+        self.records.append((name, key, ev0, ev1, nbytes, flops, probe))
 
     def summary(self):
         synchronize()
         out = {}
-        for name, key, ev0, ev1, nbytes, flops in self.records:
-            r = out.setdefault(name, {"key": key, "launches": 0, "ms": 0.0, "bytes": 0.0, "flops": 0.0})
+        took = ctypes.c_float()
+        for name, key, ev0, ev1, nbytes, flops, probe in self.records:
+            r = out.setdefault(name, {"key": key, "launches": 0, "ms": 0.0, "bytes": 0.0, "flops": 0.0, "call_ms": 0.0})
             r["launches"] += 1
-            r["ms"] += ev0.elapsed_time(ev1)
+            whole = ev0.elapsed_time(ev1)
+            if probe is not None and _LIB.agmi_probe_elapsed(probe, ctypes.byref(took)) == 0:
+                r["ms"] += took.value   # the named kernel alone
+                r["call_ms"] += whole   # the entry point's call: that kernel and the one that adds up its partial results
+            else:
+                r["ms"] += whole
+                r["call_ms"] += whole
             r["bytes"] += nbytes
             r["flops"] += flops
         for r in out.values():
             n = r["launches"]
             r["avg_ms"], r["avg_bytes"], r["avg_flops"] = r["ms"] / n, r["bytes"] / n, r["flops"] / n
+            r["avg_call_ms"] = r["call_ms"] / n
         return out
 
 
@@ -632,6 +646,7 @@ def lse_cotangent(code, x, ans, g, row_sums=None, col_factor=None, scaled=None, 
     c.scaled_row_stride = scaled.stride(0) if scaled is not None else 0
     c.col_sums = col_sums.data_ptr() if col_sums is not None else None
     ev = _TIMER.begin(("lse_cotangent",)) if _TIMER is not None else None
+    probe = _LIB.agmi_probe_arm() if ev is not None else None  # (the tile kernel alone; `ev` brackets it and the finishing kernel)
     rc = _LIB.agmi_lse_cotangent_fused(code, ctypes.byref(c), _workspace().data_ptr(), _WORKSPACE_BYTES, _stream())
     if rc == -2:  # AGMI_ERR_UNSUPPORTED
         return False
@@ -639,7 +654,8 @@ def lse_cotangent(code, x, ans, g, row_sums=None, col_factor=None, scaled=None, 
         _check(rc, "agmi_lse_cotangent_fused")
     if ev is not None:
         outs = tuple(t for t in (row_sums, scaled, col_sums) if t is not None)
-        _TIMER.end(ev, ("lse_cotangent",), (outs, (x, ans, g) + ((col_factor,) if col_factor is not None else ())))
+        _TIMER.end(ev, ("lse_cotangent",), (outs, (x, ans, g) + ((col_factor,) if col_factor is not None else ())),
+                   probe=probe if probe is not None and probe >= 0 else None)
     return True
 
 

@@ -16,6 +16,9 @@ namespace agmi {
 void set_error(const char *fmt, ...);
 // name of the kernel family the last successful entry point launched (for profilers' labels)
 void set_kernel_name(const char *fmt, ...);
+// around the first kernel of an entry point that launches several (see agmi_probe_arm): no-ops unless armed
+void probe_begin(hipStream_t s);
+void probe_end(hipStream_t s);
 int hip_check(hipError_t e, const char *what);
 
 constexpr int kBlock = 256;        // 4 wavefronts of 64 lanes

@@ -121,9 +121,51 @@ static int launch_fill(void *ptr, int64_t n, double value, hipStream_t s) {
     return hip_check(hipGetLastError(), "fill launch");
 }
 
+// ---- event pairs around the first kernel of a multi-kernel entry point (agmi_probe_arm) -------------------------
+constexpr int kProbePairs = 4096;
+static hipEvent_t g_probe_ev[kProbePairs][2];
+static unsigned char g_probe_state[kProbePairs];  // 0: no events yet, 1: created, 2: filled
+static long long g_probe_serial[kProbePairs];
+static long long g_probe_next = 0;
+static int g_probe_armed = -1;
+
+void probe_begin(hipStream_t s) {
+    if (g_probe_armed >= 0) (void)hipEventRecord(g_probe_ev[g_probe_armed][0], s);
+}
+
+void probe_end(hipStream_t s) {
+    if (g_probe_armed >= 0) {
+        if (hipEventRecord(g_probe_ev[g_probe_armed][1], s) == hipSuccess) g_probe_state[g_probe_armed] = 2;
+        g_probe_armed = -1;
+    }
+}
+
 }  // namespace agmi
 
 using namespace agmi;
+
+extern "C" int agmi_probe_arm(void) {
+    const int slot = static_cast<int>(g_probe_next % kProbePairs);
+    if (g_probe_state[slot] == 0) {
+        if (int rc = hip_check(hipEventCreate(&g_probe_ev[slot][0]), "hipEventCreate")) return rc > 0 ? -rc : rc;
+        if (int rc = hip_check(hipEventCreate(&g_probe_ev[slot][1]), "hipEventCreate")) return rc > 0 ? -rc : rc;
+    }
+    g_probe_state[slot] = 1;
+    g_probe_serial[slot] = g_probe_next;
+    g_probe_armed = slot;
+    const long long index = g_probe_next++;
+    return static_cast<int>(index & 0x7fffffff);
+}
+
+extern "C" int agmi_probe_elapsed(int index, float *ms) {
+    const int slot = index % kProbePairs;
+    if (index < 0 || !ms || g_probe_state[slot] != 2 || (g_probe_serial[slot] & 0x7fffffff) != index) {
+        set_error("probe: pair %d was never filled (or has been overwritten)", index);
+        return AGMI_ERR_ARG;
+    }
+    if (int rc = hip_check(hipEventSynchronize(g_probe_ev[slot][1]), "hipEventSynchronize")) return rc;
+    return hip_check(hipEventElapsedTime(ms, g_probe_ev[slot][0], g_probe_ev[slot][1]), "hipEventElapsedTime");
+}
 
 extern "C" const char *agmi_last_error(void) { return g_error; }
 

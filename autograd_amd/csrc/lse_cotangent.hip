@@ -344,7 +344,9 @@ static int launch_lse_cotangent(const agmi_lse_cotangent &c, void *workspace, si
     p.row_partials = row_partials ? static_cast<unsigned char *>(workspace) + col_bytes : nullptr;
     set_kernel_name("lse_cotangent_tile<%s%s%s>", (want & kWantScaled) ? "scaled," : "", (want & kWantRowSums) ? "rowsum," : "",
                     (want & kWantColSums) ? "colsum" : "");
+    probe_begin(s);
     launch_tiles<T>(want, p, dim3(static_cast<unsigned>(tiles_across), static_cast<unsigned>(bands)), s);
+    probe_end(s);
     if (int rc = hip_check(hipGetLastError(), "lse_cotangent launch")) return rc;
     const int col_blocks = (want & kWantColSums) ? static_cast<int>(ceil_div(c.cols, 64)) : 0;
     const int row_blocks = row_partials ? static_cast<int>(ceil_div(c.rows, kFinishThreads)) : 0;

@@ -169,6 +169,15 @@ int agmi_version(void);
  * (static storage; for labelling profiles). */
 const char *agmi_last_kernel(void);
 
+/* Profiling aid with no counterpart in the reference.  An entry point that launches more than one kernel (the kernel
+ * that does the work, then one that adds up partial results) cannot be timed kernel by kernel from outside: events
+ * around the call bracket all of them.  agmi_probe_arm makes the NEXT such entry point (agmi_lse_cotangent_fused)
+ * record a pair of HIP events on its stream around the FIRST of its kernels and returns the index of that pair;
+ * agmi_probe_elapsed waits for the pair and gives the milliseconds between its events (AGMI_ERR_ARG for an index that
+ * was armed but never filled, or too old: the library keeps the last 4096 pairs).  Nothing is recorded unless armed. */
+int agmi_probe_arm(void);
+int agmi_probe_elapsed(int index, float *ms);
+
 /* out[k][idx] = op(in[0][idx], in[1][idx], ...) over the index space `shape` (rank `ndim`).
  * dtype is AGMI_F32 or AGMI_F64 for all operands.  An output may alias an input only when
  * both have identical strides (in-place update: VSpace._mut_add, core.py:262-264).

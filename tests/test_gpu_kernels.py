@@ -1262,6 +1262,35 @@ def _lse_cotangent_reference(mem, scale, svec, shift, hvec, g):
     return ans, g * onp.exp(x - ans)
 
 
+def test_the_probe_times_the_first_kernel_of_a_call_that_launches_two(dnp):
+    """``agmi_probe_arm``: the logsumexp-cotangent entry point launches its tile kernel and then a kernel that adds up
+    partial sums; events around the call bracket both, the library's own pair the first alone."""
+    import ctypes
+
+    import autograd_amd as ag
+    from autograd_amd import _lib
+    from autograd_amd.scipy.special import logsumexp
+
+    L = _lib.lib()
+    rs = onp.random.RandomState(2)
+    A, b, c = (P(dnp, rs.randn(*shape).astype(F32)) for shape in ((2048, 4096), (4096,), (2048,)))
+    g = ag.grad(lambda A, b, c: dnp.sum(logsumexp(A * b[None, :] + c[:, None], axis=1)), (0, 1, 2))
+    g(A, b, c)
+    with _lib.KernelTimer() as kt:
+        for _ in range(3):
+            g(A, b, c)
+    rows = {k: v for k, v in kt.summary().items() if k.startswith("lse_cotangent_tile")}
+    assert len(rows) == 1
+    (row,) = rows.values()
+    assert row["launches"] == 3 and 0.0 < row["avg_ms"] < row["avg_call_ms"]   # the tile kernel alone < tile + finish
+    took = ctypes.c_float()
+    never = L.agmi_probe_arm()                              # armed, but nothing runs before it is read
+    assert L.agmi_probe_elapsed(never, ctypes.byref(took)) == -1 and b"never filled" in L.agmi_last_error()
+    g(A, b, c)                                               # (fills the pair that is still armed)
+    assert L.agmi_probe_elapsed(never, ctypes.byref(took)) == 0 and took.value > 0.0
+    assert L.agmi_probe_elapsed(-5, ctypes.byref(took)) == -1
+
+
 @pytest.mark.parametrize("dtype", [F32, F64])
 @pytest.mark.parametrize("rows,cols", [(37, 8), (300, 64), (129, 1028), (1000, 4096), (64, 2), (1, 4), (15, 1024), (16, 1020),
                                        (17, 2052), (50, 9000)])
