@@ -14,6 +14,7 @@ import torch
 
 from .. import _lib
 from ..extend import notrace_primitive, primitive
+from ..tracer import box_types as _box_types
 from ..tracer import getval as _getval
 from ..tracer import trace_stack as _trace_stack
 from . import devarray as D
@@ -1921,19 +1922,33 @@ def _meta_of(A):
     return onp.shape(A), onp.ndim(A), onp.result_type(A), onp.iscomplexobj(A)
 
 
-@notrace_primitive
+# `metadata`, `shape` and `ndim` run dozens of times per step of a traced loop (every rule that reshapes or unbroadcasts
+# asks): they unbox and read the attributes themselves instead of going through the generic wrapper.
 def metadata(A):
+    while type(A) in _box_types:
+        A = A._value
+    if isinstance(A, DevArray):
+        return A.shape, A.ndim, A.dtype, False
     return _meta_of(A)
 
 
-@notrace_primitive
 def shape(A):
+    while type(A) in _box_types:
+        A = A._value
+    if isinstance(A, DevArray):
+        return A.shape
     return _meta_of(A)[0]
 
 
-@notrace_primitive
 def ndim(A):
+    while type(A) in _box_types:
+        A = A._value
+    if isinstance(A, DevArray):
+        return A.ndim
     return _meta_of(A)[1]
+
+
+metadata._is_primitive = shape._is_primitive = ndim._is_primitive = True
 
 
 @notrace_primitive
