@@ -311,3 +311,62 @@ def test_pending_products_are_contracted_into_an_accumulator_of_its_own(monkeypa
     n = len(calls)
     t = fourth._t
     assert fourth._t is t and len(calls) == n + 1 and fourth.computed() and D.plain(fourth)._t is t
+
+
+def test_program_keys_tell_apart_what_the_emitted_program_depends_on():
+    """The key under which an emitted program is kept (``fusion._signature``): equal for the same expression over other
+    arrays of the same layout, different when an operand is one and the same array in two places, when a scalar or its
+    sign differs, when a layout differs, and when two vectors are views of one storage (a shift could make them
+    coincide) instead of separate arrays."""
+    from autograd_amd.numpy import fusion
+
+    was, fusion.ENABLED = fusion.ENABLED, True
+    try:
+        def key(build):
+            root = build()
+            assert type(root) is fusion.ExprArray and root._args is not None
+            sig = fusion._signature([root], fusion._post_order([root]))
+            assert sig is not None
+            return sig[0], len(sig[1])
+
+        def arrays(n=3, shape=(8, 6)):
+            return [meta(shape, torch.float64) for _ in range(n)]
+
+        f = lambda a, b, c, s=0.5: (a * b + s) / (a - c)  # noqa: E731
+        k1, n1 = key(lambda: f(*arrays()))
+        k2, n2 = key(lambda: f(*arrays()))
+        assert k1 == k2 and n1 == n2 == 3 and hash(k1) == hash(k2)
+        a, b, c = arrays()
+        assert key(lambda: f(a, a, c))[0] != k1 and key(lambda: f(a, a, c))[1] == 2           # one array in two places
+        assert key(lambda: f(a, b, c, 0.25))[0] != k1                                          # another scalar
+        assert key(lambda: f(a, b, c, 0.0))[0] != key(lambda: f(a, b, c, -0.0))[0]              # the sign of a zero
+        assert key(lambda: f(a, b, DevArray(c._t.t().contiguous().t())))[0] != k1               # another layout
+        assert key(lambda: f(*arrays(shape=(8, 7))))[0] != k1                                   # another shape
+        assert key(lambda: f(*[meta((8, 6), torch.float32) for _ in range(3)]))[0] != k1        # another precision
+        # vectors: two views of one storage against two separate arrays
+        z = meta((101,), torch.float64)
+        u, v = meta((100,), torch.float64), meta((100,), torch.float64)
+        g = lambda p, q: p * 3.0 + q * q  # noqa: E731
+        assert key(lambda: g(z[1:], z[:-1]))[0] != key(lambda: g(u, v))[0]
+        z2 = meta((101,), torch.float64)
+        assert key(lambda: g(z[1:], z[:-1]))[0] == key(lambda: g(z2[1:], z2[:-1]))[0]
+    finally:
+        fusion.ENABLED = was
+
+
+def test_slices_of_a_pending_product_stay_products():
+    """``wrapper._part_of_product``: rows and columns of a product that has not run are taken from its factors when the
+    slice keeps at least half of each axis; anything else is left to the ordinary view of the whole product."""
+    left, right = torch.zeros((10, 7), dtype=torch.float64), torch.zeros((7, 12), dtype=torch.float64)
+    P = D.PendingProduct(left, right, onp.dtype("float64"))
+    part = W._part_of_product(P, (slice(None), slice(2, 11)))
+    assert type(part) is D.PendingProduct and part.shape == (10, 9) and not P.computed()
+    assert part._left.data_ptr() == left.data_ptr() and part._right.data_ptr() == right[:, 2:].data_ptr()
+    rows = W._part_of_product(P, (slice(4, None),))
+    assert rows.shape == (6, 12) and rows._left.data_ptr() == left[4:].data_ptr()
+    for idx in ((slice(None), slice(0, 5)), (slice(0, 4), slice(None)), (slice(None), slice(0, 12, 2)), (slice(None), slice(None)),
+                (slice(None), 3), (slice(None), slice(None), None)):
+        assert W._part_of_product(P, idx) is None
+    acc = P.sum_started()
+    acc.add_product(D.PendingProduct(left, right, onp.dtype("float64")))
+    assert W._part_of_product(acc, (slice(None), slice(2, 11))) is None  # a sum of products is sliced as a whole
