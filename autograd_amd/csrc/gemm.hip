@@ -869,7 +869,7 @@ static bool wants_block_split(const GemmParams &p, int64_t batch) {
     const int64_t tiles32 = ceil_div(p.M, kSmallTile) * ceil_div(p.N, kSmallTile) * batch;
     const int64_t a_span = ((p.M - 1) * p.a_rs + (p.K - 1) * p.a_cs + 1) * 4, b_span = ((p.K - 1) * p.b_rs + (p.N - 1) * p.b_cs + 1) * 4;
     const bool addressable = p.a_rs >= 0 && p.a_cs >= 0 && p.b_rs >= 0 && p.b_cs >= 0 && a_span < 0x7fff0000LL && b_span < 0x7fff0000LL;
-    return addressable && tiles64 < 128 && p.K >= 256 && p.K <= 4096 && tiles32 <= 0x7fffffffLL && batch <= 65535;
+    return addressable && tiles64 < 128 && p.K >= 128 && p.K <= 4096 && tiles32 <= 0x7fffffffLL && batch <= 65535;
 }
 
 static int launch_block_split(GemmParams p, int64_t batch, hipStream_t s) {

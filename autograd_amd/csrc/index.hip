@@ -349,22 +349,26 @@ struct ConcatParams {
     int64_t total, inner, n;
 };
 
-// one thread per element of the contiguous (outer, total, inner) result
-template <typename T>
+// one thread per element of the contiguous (outer, total, inner) result; I is the type the element's position is split
+// in (32-bit division is a handful of instructions, 64-bit a long routine that tiny joins spend most of their time in)
+template <typename T, typename I>
 __global__ __launch_bounds__(kBlock) void concat_kernel(const ConcatParams p, T *__restrict__ out) {
     const int64_t e = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
     if (e >= p.n) return;
-    const int64_t i = e % p.inner, rest = e / p.inner;
-    const int64_t a = rest % p.total, o = rest / p.total;
+    const I inner = static_cast<I>(p.inner), total = static_cast<I>(p.total);
+    const I rest = inner == 1 ? static_cast<I>(e) : static_cast<I>(e) / inner;
+    const I i = static_cast<I>(e) - rest * inner;
+    const I o = rest / total, a = rest - o * total;
     int k = 0;
     int64_t begin = 0;
     for (int j = 0; j < p.n_pieces - 1; ++j) {  // (the same trip count for every thread; `end` is non-decreasing)
-        if (a >= p.end[j]) {
+        if (static_cast<int64_t>(a) >= p.end[j]) {
             k = j + 1;
             begin = p.end[j];
         }
     }
-    out[e] = static_cast<const T *>(p.data[k])[o * p.so[k] + (a - begin) * p.sa[k] + i * p.si[k]];
+    out[e] = static_cast<const T *>(p.data[k])[static_cast<int64_t>(o) * p.so[k] + (static_cast<int64_t>(a) - begin) * p.sa[k] +
+                                               static_cast<int64_t>(i) * p.si[k]];
 }
 
 }  // namespace agmi
@@ -412,10 +416,15 @@ extern "C" int agmi_concat(int dtype, int64_t outer, int64_t inner, int n_pieces
     }
     hipStream_t s = as_stream(stream);
     set_kernel_name("concat_kernel");
-    if (dtype == AGMI_F32)
-        hipLaunchKernelGGL(concat_kernel<float>, dim3((unsigned)blocks), dim3(kBlock), 0, s, p, static_cast<float *>(out));
+    const bool narrow = p.n <= 0x7fffffffLL;
+    if (dtype == AGMI_F32 && narrow)
+        hipLaunchKernelGGL((concat_kernel<float, uint32_t>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p, static_cast<float *>(out));
+    else if (dtype == AGMI_F32)
+        hipLaunchKernelGGL((concat_kernel<float, int64_t>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p, static_cast<float *>(out));
+    else if (dtype == AGMI_F64 && narrow)
+        hipLaunchKernelGGL((concat_kernel<double, uint32_t>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p, static_cast<double *>(out));
     else if (dtype == AGMI_F64)
-        hipLaunchKernelGGL(concat_kernel<double>, dim3((unsigned)blocks), dim3(kBlock), 0, s, p, static_cast<double *>(out));
+        hipLaunchKernelGGL((concat_kernel<double, int64_t>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p, static_cast<double *>(out));
     else {
         set_error("concat: dtype %d is not a floating type", dtype);
         return AGMI_ERR_ARG;

@@ -39,6 +39,7 @@ struct ProgParams {
     uint32_t tiles_per_row, n_tiles;
     uint32_t step_rows, step_chunks;  // the wave stride (number of waves in the grid) split by tiles_per_row
     int32_t n_leaf, n_imm, n_instr;
+    int32_t row_group;  // programs with row sums: the lanes that share a row in the reduction kernel's order
     const void *leaf[kProgMaxLeaf];
     int64_t leaf_rs[kProgMaxLeaf];
     int32_t leaf_cs[kProgMaxLeaf];  // 0 or 1
@@ -146,11 +147,13 @@ static __device__ __noinline__ void store_partial(T *base, int64_t c, int64_t co
 // op | dst << 8 | a << 12 | b << 16 | c << 20 | d << 24
 __device__ __forceinline__ int field(uint32_t w, int shift, int mask) { return static_cast<int>(w >> shift) & mask; }
 
-template <typename T, int NREG, int U, bool LIGHT>
+// ROWS: the variant that knows AGMI_PROGRAM_ROWSUM (a row per tile; the row's values cross the wave through LDS)
+template <typename T, int NREG, int U, bool LIGHT, bool ROWS>
 __global__ __launch_bounds__(kBlock) void ew_program(const ProgParams p) {
     constexpr int VL = 16 / sizeof(T);
     constexpr int V = VL * U;
     constexpr int TW = 64 * V;  // columns per tile (one wave)
+    __shared__ __align__(16) T row_values[ROWS ? kBlock / 64 : 1][ROWS ? TW : 1];
     typedef T vec_t __attribute__((ext_vector_type(VL), aligned(sizeof(T))));
     using reg_t = typename RegVec<T, NREG>::type;
 
@@ -295,6 +298,32 @@ __global__ __launch_bounds__(kBlock) void ew_program(const ProgParams p) {
             }                                                                                             \
         break;                                                                                            \
     }                                                                                                     \
+    case AGMI_PROGRAM_ROWSUM: {                                                                           \
+        if constexpr (ROWS) {                                                                             \
+            /* the order of red_row_group: lane g of G adds up columns g, g + G, ... from zero, then the  \
+               lanes' sums meet in a butterfly; lane 0 holds what that kernel stores */                   \
+            T *mine = row_values[threadIdx.x >> 6];                                                       \
+            _Pragma("unroll") for (int u = 0; u < U; ++u) {                                               \
+                vec_t v;                                                                                  \
+                _Pragma("unroll") for (int j = 0; j < VL; ++j) v[j] = x[0][u * VL + j];                   \
+                *reinterpret_cast<vec_t *>(mine + u * (64 * VL) + lane * VL) = v;                         \
+            }                                                                                             \
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");                                        \
+            __builtin_amdgcn_wave_barrier();                                                              \
+            const int G = p.row_group;                                                                    \
+            T acc = T(0);                                                                                 \
+            if (static_cast<int>(lane) < G)                                                               \
+                for (int64_t rr = lane; rr < cols; rr += G) acc = acc + mine[rr];                         \
+            for (int m = G >> 1; m > 0; m >>= 1) acc = acc + __shfl_xor(acc, m, 64);                      \
+            acc = __shfl(acc, 0, 64);                                                                     \
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");                                        \
+            __builtin_amdgcn_wave_barrier();                                                              \
+            _Pragma("unroll") for (int j = 0; j < V; ++j) o[j] = acc;                                     \
+        } else {                                                                                          \
+            _Pragma("unroll") for (int j = 0; j < V; ++j) o[j] = x[0][j];                                 \
+        }                                                                                                 \
+        break;                                                                                            \
+    }                                                                                                     \
     case AGMI_PROGRAM_STORE: {                                                                            \
         T *base = static_cast<T *>(p.out[b]) + static_cast<int64_t>(cur_row) * p.out_rs[b];               \
         _Pragma("unroll") for (int u = 0; u < U; ++u) {                                                   \
@@ -344,7 +373,7 @@ static int op_arity(int op) {
 #undef AGMI_ARITY_CASE
 }
 
-template <typename T, int NREG, int U, bool LIGHT>
+template <typename T, int NREG, int U, bool LIGHT, bool ROWS = false>
 static int launch_program(const ProgParams &p0, int64_t rows, hipStream_t s) {
     ProgParams p = p0;
     constexpr int V = (16 / sizeof(T)) * U;
@@ -364,7 +393,11 @@ static int launch_program(const ProgParams &p0, int64_t rows, hipStream_t s) {
     p.n_tiles = static_cast<uint32_t>(n_tiles);
     p.step_rows = static_cast<uint32_t>(n_waves / tpr);
     p.step_chunks = static_cast<uint32_t>(n_waves % tpr);
-    hipLaunchKernelGGL((ew_program<T, NREG, U, LIGHT>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p);
+    if (ROWS && tpr != 1) {
+        set_error("program: a row sum needs rows of at most %lld columns", (long long)TW);
+        return AGMI_ERR_UNSUPPORTED;
+    }
+    hipLaunchKernelGGL((ew_program<T, NREG, U, LIGHT, ROWS>), dim3((unsigned)blocks), dim3(kBlock), 0, s, p);
     return hip_check(hipGetLastError(), "program launch");
 }
 
@@ -378,6 +411,7 @@ int program_part_f64(int nreg, bool light, const ProgParams &p, int64_t rows, hi
 // the scalar unit's decode work per instruction is shared by twice the elements, which outweighs the lost occupancy).
 template <typename T>
 static int launch_variant(int nreg, bool light, const ProgParams &p, int64_t rows, hipStream_t s) {
+    if (p.row_group > 0) return launch_program<T, 16, 2, false, true>(p, rows, s);
     if (light) return nreg == 8 ? launch_program<T, 8, 2, true>(p, rows, s) : launch_program<T, 16, 2, true>(p, rows, s);
     return nreg == 8 ? launch_program<T, 8, 2, false>(p, rows, s) : launch_program<T, 16, 2, false>(p, rows, s);
 }
@@ -422,6 +456,7 @@ extern "C" int agmi_program(int dtype, int ndim, const int64_t *shape, int n_out
     for (int k = 0; k < n_imm; ++k) defined |= 1u << (nreg - 1 - k);
     uint32_t stored = 0;
     bool light = true;
+    bool row_sums = false;
     for (int i = 0; i < n_instr; ++i) {
         const uint32_t w = code[i];
         const int op = w & 0xff, dst = (w >> 8) & 15;
@@ -438,6 +473,16 @@ extern "C" int agmi_program(int dtype, int ndim, const int64_t *shape, int n_out
                           src[2], src[1], n_mask);
                 return AGMI_ERR_ARG;
             }
+            defined |= 1u << dst;
+            continue;
+        }
+        if (op == AGMI_PROGRAM_ROWSUM) {
+            if (src[0] >= nreg || !(defined >> src[0] & 1u) || dst >= nreg) {
+                set_error("program: instruction %d sums register %d, which holds nothing, or writes register %d of %d", i,
+                          src[0], dst, nreg);
+                return AGMI_ERR_ARG;
+            }
+            row_sums = true;
             defined |= 1u << dst;
             continue;
         }
@@ -486,7 +531,30 @@ extern "C" int agmi_program(int dtype, int ndim, const int64_t *shape, int n_out
         strides[n_out + k] = leaves[k].strides;
     }
     Merged m;
-    if (!merge_axes(ndim, shape, nullptr, n_out + n_leaf, strides, &m)) return AGMI_ERR_ARG;
+    int row_group = 0;
+    if (row_sums) {
+        // rows stay rows: no merging, and only the shapes whose standalone row sums a group of lanes adds up
+        constexpr int64_t kRowMax[2] = {64 * 2 * 4, 64 * 2 * 2};  // a wave's tile in float32 / float64
+        const int64_t widest = kRowMax[dtype == AGMI_F32 ? 0 : 1];
+        if (ndim != 2 || shape[1] > widest || (shape[1] > 64 && shape[0] < 64) || n_regs != 16 || leaf_ranges || n_mask) {
+            set_error("program: row sums need a (rows, columns <= %lld) index space with at least 64 rows when the rows "
+                      "are longer than 64, 16 registers, no leaf ranges and no masks", (long long)widest);
+            return AGMI_ERR_UNSUPPORTED;
+        }
+        m.ndim = 2;
+        m.n = shape[0] * shape[1];
+        m.shape[0] = shape[0];
+        m.shape[1] = shape[1];
+        for (int k = 0; k < n_out + n_leaf; ++k) {
+            m.stride[k][0] = shape[0] == 1 ? 0 : strides[k][0];
+            m.stride[k][1] = shape[1] == 1 ? 0 : strides[k][1];
+        }
+        const int64_t quarter = (shape[1] + 3) / 4;
+        row_group = 1;
+        while (row_group < quarter && row_group < 64) row_group <<= 1;
+    } else if (!merge_axes(ndim, shape, nullptr, n_out + n_leaf, strides, &m)) {
+        return AGMI_ERR_ARG;
+    }
     if (m.n == 0) return 0;
     if (m.ndim > 2) {
         set_error("program: %d axes remain after merging, at most 2 are supported", m.ndim);
@@ -503,7 +571,7 @@ extern "C" int agmi_program(int dtype, int ndim, const int64_t *shape, int n_out
         }
         p.out[k] = outs[k].data;
         p.out_rs[k] = m.ndim == 2 ? m.stride[k][0] : 0;
-        if (m.ndim == 2 && p.out_rs[k] == 0) {
+        if (m.ndim == 2 && m.shape[0] > 1 && p.out_rs[k] == 0) {
             set_error("program: output %d has stride 0 on an axis of extent %lld", k, (long long)m.shape[0]);
             return AGMI_ERR_ARG;
         }
@@ -545,6 +613,7 @@ extern "C" int agmi_program(int dtype, int ndim, const int64_t *shape, int n_out
         set_error("program: masks need a one-row index space");
         return AGMI_ERR_UNSUPPORTED;
     }
+    p.row_group = row_group;
     p.n_leaf = n_leaf;
     p.n_imm = n_imm;
     p.n_instr = n_instr;
@@ -553,7 +622,7 @@ extern "C" int agmi_program(int dtype, int ndim, const int64_t *shape, int n_out
     p.code[n_instr] = 0;
     hipStream_t s = as_stream(stream);
     set_kernel_name("ew_program<%s,%d,%s>[%d instr, %lldx%lld]", dtype == AGMI_F32 ? "float" : "double", nreg,
-                    light ? "light" : "full", n_instr, (long long)rows, (long long)p.cols);
+                    row_group ? "rows" : (light ? "light" : "full"), n_instr, (long long)rows, (long long)p.cols);
     return dtype == AGMI_F32 ? program_part_f32(nreg, light, p, rows, s) : program_part_f64(nreg, light, p, rows, s);
 }
 #endif  // AGMI_PART == 32

@@ -27,7 +27,7 @@ import sys
 import numpy as onp
 
 from .. import _lib
-from .._lib import Op
+from .._lib import Op, Red
 from . import devarray as D
 from .devarray import DevArray, LazyDevArray
 
@@ -53,6 +53,11 @@ for _name in "WHERE DIV_VJP1 POW_VJP0 POW_VJP1 ABS_VJP MUL_ADD".split():
     ARITY[getattr(Op, _name)] = 3
 for _name in "LSE_VJP CHOOSE_VJP EXTREMUM_VJP".split():
     ARITY[getattr(Op, _name)] = 4
+
+# pseudo-op of a program: the sum of its operand over each row of a two-axis index space, at every index of the row
+ROWSUM = _lib.PROGRAM_ROWSUM
+ARITY[ROWSUM] = 1
+ROWSUM_WIDEST = {onp.dtype("float32"): 512, onp.dtype("float64"): 256}  # one wave's tile of the program kernel
 
 COUNTS = {"programs": 0, "instructions": 0, "single": 0, "unfused": 0, "layers": 0}  # what ran (tests and profiles read it)
 
@@ -186,6 +191,12 @@ def make(op, dtype, xs):
         kind = type(x)
         if kind is float:
             continue
+        if kind is D.PendingReduce and x._call is not None:
+            node = _row_sums(x, shape, dtype)
+            if node is not None:
+                args[k] = node
+                cone += node._cone
+                continue
         if kind is ExprArray and x._args is not None:
             if x._shape != shape:
                 x._t  # a pending operand is written out before it is broadcast: programs work on one shape
@@ -210,6 +221,28 @@ def make(op, dtype, xs):
             cone = node._cone = len(_post_order((node,)))
         return node
     return ExprArray(op, tuple(args), shape, dtype, cone)
+
+
+def _row_sums(x, shape, dtype):
+    """Row sums that have not run (``x``: a pending ``sum(e, axis=1, keepdims=True)``, the unbroadcast of a cotangent)
+    about to be broadcast back over the rows they came from: a node of the full shape that the program kernel forms
+    inside the chain (``g - exp(x - lse) * sum(g, axis=1)`` of a log-softmax is then one launch instead of a
+    reduction plus a program).  Only for the shapes whose rows the reduction kernel gives to a group of lanes: the
+    program adds in that kernel's order, so the value does not depend on which of the two ran.  None otherwise."""
+    op, red, rdtype, xs, axes, _keepdims, full = x._call
+    if red != Red.SUM or (op != Op.COPY and op != Op.NEG) or len(xs) != 1 or rdtype != dtype or len(shape) != 2:
+        return None
+    src = xs[0]
+    rows, cols = shape
+    if not isinstance(src, DevArray) or src.shape != shape or src.dtype != dtype or x.shape != (rows, 1) \
+            or tuple(axes) not in ((1,), (-1,)) or (full is not None and tuple(full) != shape):
+        return None
+    if cols < 2 or cols > ROWSUM_WIDEST[dtype] or (cols > 64 and rows < 64):
+        return None
+    node = ExprArray(ROWSUM, (src,), shape, dtype, 1 + (src._cone if pending(src) else 0))
+    if op == Op.NEG:
+        node = ExprArray(Op.NEG, (node,), shape, dtype, node._cone + 1)
+    return node
 
 
 def _post_order(roots):
@@ -371,6 +404,12 @@ def _single(node):
     dtype = node.dtype
     if node._op == SHIFT:
         _single_shift(node)
+        return
+    if node._op == ROWSUM:
+        sums = D._map_reduce_now(Op.COPY, Red.SUM, dtype, (node._args[0],), (1,), True)
+        _lib.elementwise(Op.COPY, _lib.DTYPE_CODE[dtype], node._shape, (node._buffer(),), (D._expand(sums._t, node._shape),))
+        COUNTS["single"] += 1
+        _finish(node)
         return
     ops = D._limit_aux(tuple(D._operand(a, dtype) for a in node._args), dtype)
     shape = node._shape
@@ -558,7 +597,7 @@ def _emit(roots):
             return signed(na != nb, op, a[1] if na else a, b[1] if nb else b)
         if op == Op.SQUARE or op == Op.ABS:
             return emit(op, srcs[0][1] if na else srcs[0])
-        if op == Op.RECIPROCAL:
+        if op == Op.RECIPROCAL or op == ROWSUM:  # (a row's sum of negated terms is minus its sum, bit for bit)
             return signed(na, op, srcs[0][1] if na else srcs[0])
         if op == Op.DIV_VJP1:  # ((-g) * x) / (y * y)
             g, x, y = srcs
@@ -692,7 +731,8 @@ def _emit(roots):
             last[s] = k
     for v in root_values:
         last[v] = n_ins
-    for n_regs in ([16] if single else [8, 16]):  # (8 float32 registers are indexed by a chain of selects in the kernel: slower than 16)
+    row_sums = builtins_any_rowsum(instrs)
+    for n_regs in ([16] if single or row_sums else [8, 16]):  # (8 float32 registers are indexed by a chain of selects in the kernel: slower than 16)
         if n_leaf + n_imm > n_regs:
             continue
         reg = {("L", k): k for k in range(n_leaf)}
@@ -903,6 +943,13 @@ def added_into(A, start, x, take):
     if inner is None or inner._shape != (m,):
         return None
     return shifted(inner, start, A.shape[0], outside=A)
+
+
+def builtins_any_rowsum(instrs):
+    for instr in instrs:
+        if instr[0] == ROWSUM:
+            return True
+    return False
 
 
 def builtins_all_zero(strides):

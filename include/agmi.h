@@ -207,6 +207,13 @@ int agmi_elementwise(int op, int dtype, int ndim, const int64_t *shape,
  * gets an unspecified finite value, which the program is expected to discard with op
  * AGMI_PROGRAM_MASK: reg[dst] = (mask_ranges[2b] <= idx < mask_ranges[2b+1]) ? reg[a] : reg[c].
  * leaf_ranges may be NULL (every index readable); n_mask <= AGMI_PROGRAM_MAX_MASKS.
+ * Row sums (the unbroadcast of a cotangent that a later rule of the same chain reads again, as in the
+ * log-softmax of examples/rnn.py:50-52: g - exp(x - lse) * sum(g, axis=1)): AGMI_PROGRAM_ROWSUM sets
+ * reg[dst], at every index of a row, to the sum of reg[a] over that row, added up in the order in which
+ * agmi_map_reduce adds a row of that length (bit for bit its result).  A program that holds one runs on
+ * `shape` as given: exactly two axes, the second at most 512 (float32) / 256 (float64) long and,
+ * beyond 64, at least 64 rows (the shapes for which agmi_map_reduce gives a row to a group of lanes);
+ * n_regs must be 16, no leaf ranges and no masks; else AGMI_ERR_UNSUPPORTED.
  * Layout: after axis merging at most two axes may remain and every operand must have stride 1 or
  * 0 (leaves only) along the innermost one; anything else returns AGMI_ERR_UNSUPPORTED.  Outputs
  * may not overlap leaves unless they are the same view (in-place update).
@@ -221,6 +228,7 @@ int agmi_elementwise(int op, int dtype, int ndim, const int64_t *shape,
 #define AGMI_PROGRAM_MAX_MASKS 4
 #define AGMI_PROGRAM_STORE 255
 #define AGMI_PROGRAM_MASK 254
+#define AGMI_PROGRAM_ROWSUM 253
 int agmi_program(int dtype, int ndim, const int64_t *shape, int n_out, const agmi_array *outs,
                  int n_leaf, const agmi_array *leaves, const int64_t *leaf_ranges,
                  int n_imm, const double *imms, int n_mask, const int64_t *mask_ranges,

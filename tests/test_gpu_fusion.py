@@ -333,6 +333,122 @@ def test_program_shifted_leaves_and_masks(dtype, n):
     assert onp.array_equal(out.cpu().numpy(), want)
 
 
+ROW_SUM_SHAPES = [(256, 128), (64, 512), (70, 256), (1000, 65), (100, 64), (1, 40), (7, 5), (3, 2), (300, 257)]
+
+
+@pytest.mark.parametrize("dtype", [F32, F64])
+@pytest.mark.parametrize("shape", ROW_SUM_SHAPES)
+def test_row_sums_read_back_by_the_chain_are_formed_inside_it(dtype, shape, dnp):
+    """``g - exp(x - lse) * sum(g, axis=1, keepdims=True)`` (the cotangent of a log-softmax, reference
+    examples/rnn.py:50-52 under autograd/numpy/numpy_vjps.py:76-93 and autograd/scipy/special.py:127-144): the row sums
+    of the pending ``g`` are formed by the program that reads them back, in the order the reduction kernel adds a row
+    of that length, so the chain is one launch and gives the separate launches' bits.  Shapes the reduction kernel
+    treats otherwise (rows longer than a wave's tile; long rows with few of them) keep the separate reduction."""
+    from autograd_amd import _lib
+    from autograd_amd._lib import Op, Red
+    from autograd_amd.numpy import devarray as D
+    from autograd_amd.numpy import fusion
+
+    rows, cols = shape
+    if dtype == F64 and cols > 256:
+        pytest.skip("wider than a float64 tile: covered by the float32 case of the same width")
+    rs = onp.random.RandomState(rows * 1000 + cols)
+    a, t = rs.randn(*shape).astype(dtype), rs.rand(*shape).astype(dtype)
+    x = (rs.randn(*shape) * 3).astype(dtype)
+    lse = onp.log(onp.sum(onp.exp(x.astype(F64)), axis=1, keepdims=True)).astype(dtype)
+    A, T, X, L = (dnp.asarray(v) for v in (a, t, x, lse))
+    reduced = []
+    real = _lib.map_reduce
+    _lib.map_reduce = lambda *args, **k: (reduced.append(args[0]), real(*args, **k))[1]
+
+    def chain(negated):
+        g = A * T
+        if negated:  # the unbroadcast of a subtraction's second cotangent negates inside the reduction
+            s = D.map_reduce(Op.NEG, Red.SUM, dtype, (g,), (1,), True)
+            return (g + dnp.exp(X - L) * s).numpy()
+        s = dnp.sum(g, axis=1, keepdims=True)
+        return (g - dnp.exp(X - L) * s).numpy()
+
+    try:
+        for negated in (False, True):
+            del reduced[:]
+            before = dict(fusion.COUNTS)
+            got = chain(negated)
+            inside = cols <= fusion.ROWSUM_WIDEST[dtype] and cols >= 2 and (cols <= 64 or rows >= 64)
+            assert len(reduced) == (0 if inside else 1), (reduced, inside)
+            assert fusion.COUNTS["programs"] - before["programs"] == 1 and fusion.COUNTS["unfused"] == before["unfused"]
+            with unfused():
+                want = chain(negated)
+            assert _same_bits(got, want)
+            g64 = a.astype(F64) * t
+            ref = g64 - onp.exp(x.astype(F64) - lse) * g64.sum(axis=1, keepdims=True)
+            assert onp.allclose(got, ref, rtol=1e-4 if dtype == F32 else 1e-11, atol=(1e-4 if dtype == F32 else 1e-11) * cols)
+    finally:
+        _lib.map_reduce = real
+
+
+def test_row_sums_of_special_values_and_of_an_array_in_memory(dnp):
+    """The in-chain row sum follows the reduction kernel on rows with infinities and NaNs, sums an operand that already
+    lies in memory just the same, and still gives the reduction's own result when that is read as well."""
+    rs = onp.random.RandomState(12)
+    g = rs.randn(128, 96)
+    g[3, 5], g[7, 0], g[9, 95] = onp.inf, onp.nan, -onp.inf
+    g[11, 2], g[11, 3] = onp.inf, -onp.inf
+    G, Y = dnp.asarray(g), dnp.asarray(rs.randn(128, 96))
+
+    def both():
+        s = dnp.sum(G, axis=1, keepdims=True)
+        return (Y * s + G).numpy(), s.numpy()
+
+    got, sums = both()
+    with unfused():
+        want, want_sums = both()
+    assert _same_bits(got, want) and _same_bits(sums, want_sums)
+    with onp.errstate(invalid="ignore"):
+        assert onp.allclose(sums, g.sum(axis=1, keepdims=True), equal_nan=True)
+
+
+def test_log_softmax_gradient_is_the_same_with_row_sums_inside_the_chain(dnp):
+    """The whole pattern through the tracer: gradient of ``-sum(log_softmax(x) * t)`` (reference examples/rnn.py:50-61,
+    examples/neural_net.py:24-28), fused against unfused bit for bit and against the closed form."""
+    import autograd_amd as ag
+    from autograd_amd.scipy.special import logsumexp
+
+    rs = onp.random.RandomState(3)
+    for dtype, shape in ((F32, (256, 128)), (F64, (100, 10)), (F32, (64, 300))):
+        x = rs.randn(*shape).astype(dtype)
+        t = onp.eye(shape[1], dtype=dtype)[rs.randint(0, shape[1], shape[0])]
+        X, T = dnp.asarray(x), dnp.asarray(t)
+
+        def loss(z):
+            return -dnp.sum((z - logsumexp(z, axis=1, keepdims=True)) * T)
+
+        fused, plain, ran = _both_ways(lambda: ag.grad(loss)(X).numpy())
+        assert _same_bits(fused, plain) and ran["unfused"] == 0
+        x64 = x.astype(F64)
+        soft = onp.exp(x64 - x64.max(axis=1, keepdims=True))
+        soft /= soft.sum(axis=1, keepdims=True)
+        assert onp.allclose(fused, soft - t, rtol=0, atol=2e-6 if dtype == F32 else 1e-14)
+
+
+def test_a_row_sum_outside_the_kernels_shapes_is_refused_at_the_library():
+    from autograd_amd import _lib
+    from autograd_amd._lib import Op
+    from autograd_amd.numpy import devarray as D
+
+    code = _lib.DTYPE_CODE[F32]
+    words = [W(_lib.PROGRAM_ROWSUM, 1, 0), W(Op.ADD, 2, 0, 1), W(_lib.PROGRAM_STORE, 2, 2, 0)]
+    for shape, fits in (((64, 512), True), ((64, 513), False), ((8, 100), False), ((8, 64), True)):
+        x = D.from_numpy(onp.ones(shape, F32))
+        out = _lib.empty(shape, F32)
+        assert _lib.program(code, shape, (out,), (x._t,), [], words, 16) == fits
+        if fits:
+            assert onp.array_equal(out.cpu().numpy(), onp.full(shape, shape[1] + 1.0, F32))
+    x = D.from_numpy(onp.ones((64, 64), F32))
+    out = _lib.empty((64, 64), F32)
+    assert not _lib.program(code, (64, 64), (out,), (x._t,), [], words, 8)  # the row-sum variant has 16 registers
+
+
 def test_program_arguments_are_checked():
     from autograd_amd import _lib
     from autograd_amd._lib import AgmiError, Op
