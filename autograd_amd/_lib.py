@@ -72,7 +72,12 @@ class Op:
         MUL_ADD,
         EQUAL_AS_FLOAT,
         EXTREMUM_VJP,
-    ) = range(96, 116)
+        MUL_MUL,   # the last five: two rules in one program instruction (programs only)
+        MUL_SUB,
+        MUL_RSUB,
+        ADD_MUL,
+        SUB_MUL,
+    ) = range(96, 121)
 
 
 class Cmp:

@@ -263,6 +263,19 @@ AGMI_FUNCTOR(FEqualAsFloat, 2, 1, o[0] = (x[0] == x[1]) ? T(1) : T(0);)
 // (g, x, ans, n): g * astype(x == ans, dtype) / n
 AGMI_FUNCTOR(FExtremumVjp, 4, 1, o[0] = (x[0] * ((x[1] == x[2]) ? T(1) : T(0))) / x[3];)
 
+// two rules in one program instruction, each rounded on its own
+AGMI_FUNCTOR(FMulMul, 3, 1, T t = x[0] * x[1]; o[0] = t * x[2];)
+AGMI_FUNCTOR(FMulSub, 3, 1, T t = x[0] * x[1]; o[0] = t - x[2];)
+AGMI_FUNCTOR(FMulRsub, 3, 1, T t = x[0] * x[1]; o[0] = x[2] - t;)
+AGMI_FUNCTOR(FAddMul, 3, 1, T t = x[0] + x[1]; o[0] = t * x[2];)
+AGMI_FUNCTOR(FSubMul, 3, 1, T t = x[0] - x[1]; o[0] = t * x[2];)
+#define AGMI_FOR_EACH_CHAINED_OP(X)   \
+    X(AGMI_OP_MUL_MUL, FMulMul)       \
+    X(AGMI_OP_MUL_SUB, FMulSub)       \
+    X(AGMI_OP_MUL_RSUB, FMulRsub)     \
+    X(AGMI_OP_ADD_MUL, FAddMul)       \
+    X(AGMI_OP_SUB_MUL, FSubMul)
+
 // X(op enum, functor): the operations with one result (what an elementwise program may contain)
 #define AGMI_FOR_EACH_PROGRAM_OP(X)             \
     X(AGMI_OP_COPY, FCopy)                      \

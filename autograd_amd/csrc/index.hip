@@ -359,16 +359,21 @@ __global__ __launch_bounds__(kBlock) void concat_kernel(const ConcatParams p, T 
     const I rest = inner == 1 ? static_cast<I>(e) : static_cast<I>(e) / inner;
     const I i = static_cast<I>(e) - rest * inner;
     const I o = rest / total, a = rest - o * total;
-    int k = 0;
-    int64_t begin = 0;
-    for (int j = 0; j < p.n_pieces - 1; ++j) {  // (the same trip count for every thread; `end` is non-decreasing)
-        if (static_cast<int64_t>(a) >= p.end[j]) {
-            k = j + 1;
-            begin = p.end[j];
+    // the piece's pointer and strides are picked by selects between values every lane loads at the same (scalar)
+    // addresses: no load waits on the piece number (indexing the table by it would be a second round trip to memory
+    // before the element's own)
+    const T *src = static_cast<const T *>(p.data[0]);
+    int64_t so = p.so[0], sa = p.sa[0], si = p.si[0], begin = 0;
+    for (int j = 1; j < p.n_pieces; ++j) {  // (the same trip count for every thread; `end` is non-decreasing)
+        if (static_cast<int64_t>(a) >= p.end[j - 1]) {
+            src = static_cast<const T *>(p.data[j]);
+            so = p.so[j];
+            sa = p.sa[j];
+            si = p.si[j];
+            begin = p.end[j - 1];
         }
     }
-    out[e] = static_cast<const T *>(p.data[k])[static_cast<int64_t>(o) * p.so[k] + (static_cast<int64_t>(a) - begin) * p.sa[k] +
-                                               static_cast<int64_t>(i) * p.si[k]];
+    out[e] = src[static_cast<int64_t>(o) * so + (static_cast<int64_t>(a) - begin) * sa + static_cast<int64_t>(i) * si];
 }
 
 }  // namespace agmi

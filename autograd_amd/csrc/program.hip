@@ -72,6 +72,7 @@ constexpr bool is_short_op(int op) {
         case AGMI_OP_LOG1P_VJP: case AGMI_OP_EXPM1_VJP: case AGMI_OP_MUL_ADD: case AGMI_OP_EQUAL_AS_FLOAT:
         case AGMI_OP_CHOOSE_VJP: case AGMI_OP_EXTREMUM_VJP: case AGMI_OP_FLOOR: case AGMI_OP_CEIL:
         case AGMI_OP_RINT: case AGMI_OP_TRUNC:
+        case AGMI_OP_MUL_MUL: case AGMI_OP_MUL_SUB: case AGMI_OP_MUL_RSUB: case AGMI_OP_ADD_MUL: case AGMI_OP_SUB_MUL:
             return true;
         default:
             return false;
@@ -95,7 +96,8 @@ constexpr bool is_short_op(int op) {
     X(AGMI_OP_DIV, FDiv)                     \
     X(AGMI_OP_DIV_VJP1, FDivVjp1)            \
     X(AGMI_OP_TANH_VJP, FTanhVjp)            \
-    X(AGMI_OP_MUL_ADD, FMulAdd)
+    X(AGMI_OP_MUL_ADD, FMulAdd)              \
+    AGMI_FOR_EACH_CHAINED_OP(X)
 
 constexpr bool is_light_op(int op) {
 #define AGMI_LIGHT_CASE(OP, FN) case OP:
@@ -347,6 +349,7 @@ __global__ __launch_bounds__(kBlock) void ew_program(const ProgParams p) {
             } else {
                 switch (op) {
                     AGMI_FOR_EACH_PROGRAM_OP(AGMI_PROG_CASE)
+                    AGMI_FOR_EACH_CHAINED_OP(AGMI_PROG_CASE)
                     AGMI_PROG_STORE_AND_DEFAULT
                 }
             }
@@ -368,6 +371,7 @@ static int op_arity(int op) {
     case OP: return FN<float>::NIN;
     switch (op) {
         AGMI_FOR_EACH_PROGRAM_OP(AGMI_ARITY_CASE)
+        AGMI_FOR_EACH_CHAINED_OP(AGMI_ARITY_CASE)
         default: return -1;
     }
 #undef AGMI_ARITY_CASE

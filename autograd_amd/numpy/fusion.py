@@ -49,7 +49,7 @@ for _name in ("ADD SUB MUL DIV POW MAXIMUM MINIMUM FMAX FMIN ARCTAN2 HYPOT LOGAD
               "RECIPROCAL_VJP SQRT_VJP SIN_VJP COS_VJP SINH_VJP COSH_VJP SQUARE_VJP LOG1P_VJP EXPM1_VJP "
               "EQUAL_AS_FLOAT").split():
     ARITY[getattr(Op, _name)] = 2
-for _name in "WHERE DIV_VJP1 POW_VJP0 POW_VJP1 ABS_VJP MUL_ADD".split():
+for _name in "WHERE DIV_VJP1 POW_VJP0 POW_VJP1 ABS_VJP MUL_ADD MUL_MUL MUL_SUB MUL_RSUB ADD_MUL SUB_MUL".split():
     ARITY[getattr(Op, _name)] = 3
 for _name in "LSE_VJP CHOOSE_VJP EXTREMUM_VJP".split():
     ARITY[getattr(Op, _name)] = 4
@@ -57,6 +57,8 @@ for _name in "LSE_VJP CHOOSE_VJP EXTREMUM_VJP".split():
 # pseudo-op of a program: the sum of its operand over each row of a two-axis index space, at every index of the row
 ROWSUM = _lib.PROGRAM_ROWSUM
 ARITY[ROWSUM] = 1
+_CHAINED_INTO_MUL = {Op.MUL: Op.MUL_MUL, Op.ADD: Op.ADD_MUL, Op.SUB: Op.SUB_MUL}
+CHAINED = os.environ.get("AUTOGRAD_AMD_FUSE_CHAINED", "1").strip() not in ("0", "")  # (off: for measurements)
 ROWSUM_WIDEST = {onp.dtype("float32"): 512, onp.dtype("float64"): 256}  # one wave's tile of the program kernel
 
 COUNTS = {"programs": 0, "instructions": 0, "single": 0, "unfused": 0, "layers": 0}  # what ran (tests and profiles read it)
@@ -686,22 +688,41 @@ def _emit(roots):
     except _TooBig:
         return None
 
-    # a product that only one sum reads: one multiply-add (the product rounded, then the sum rounded)
+    # A product, sum or difference that only one sum, difference or product reads travels with its reader: one
+    # instruction with three operands (the first rule rounded, then the second, as the two instructions would be).
+    # What an interpreted instruction costs is operand moves and dispatch, hardly the arithmetic.
     uses = {}
     for _op, srcs, _mask in instrs:
         for v in srcs:
             uses[v] = uses.get(v, 0) + 1
     for v in root_values:
         uses[v] = uses.get(v, 0) + 1
-    for k, (op, srcs, mask) in enumerate(instrs):
-        if op == Op.ADD:
+    if CHAINED:
+        for k, (op, srcs, mask) in enumerate(instrs):
+            if mask is not None or (op != Op.ADD and op != Op.SUB and op != Op.MUL):
+                continue
             for me, other in ((0, 1), (1, 0)):
                 p = srcs[me]
-                if p[0] == "X" and uses.get(p) == 1 and instrs[p[1]][0] == Op.MUL and instrs[p[1]][2] is None:
-                    a, b = instrs[p[1]][1]
-                    instrs[k] = (Op.MUL_ADD, (a, b, srcs[other]), None)
-                    uses[p] = 0
-                    break
+                if p[0] != "X" or uses.get(p) != 1:
+                    continue
+                pop, psrcs, pmask = instrs[p[1]]
+                if pmask is not None:
+                    continue
+                if pop == Op.SQUARE:
+                    pop, psrcs = Op.MUL, (psrcs[0], psrcs[0])  # x * x, the very same product
+                if op == Op.MUL:
+                    both = _CHAINED_INTO_MUL.get(pop)
+                elif pop != Op.MUL:
+                    continue
+                elif op == Op.ADD:
+                    both = Op.MUL_ADD
+                else:
+                    both = Op.MUL_SUB if me == 0 else Op.MUL_RSUB
+                if both is None:
+                    continue
+                instrs[k] = (both, (psrcs[0], psrcs[1], srcs[other]), None)
+                uses[p] = 0
+                break
     # drop what nothing reads (from the roots backwards), then number leaves, immediates and instructions anew
     needed = set(root_values)
     for k in range(len(instrs) - 1, -1, -1):

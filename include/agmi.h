@@ -147,8 +147,17 @@ typedef enum agmi_op {
     AGMI_OP_DIV_VJP_BOTH,  /* (g, x, y) -> two outputs: g / y and -g * x / y**2  (91-92)          */
     AGMI_OP_MUL_ADD,       /* (a, x, y)      a * x + y  (two roundings; scalar_mul + add)         */
     AGMI_OP_EQUAL_AS_FLOAT,/* (x, y)         1.0 where x == y else 0.0: astype(x == ans, dtype)   numpy_vjps.py:524 */
-    AGMI_OP_EXTREMUM_VJP   /* (g, x, ans, n) g * (x == ans) / n, n = number of positions that attain the
+    AGMI_OP_EXTREMUM_VJP,  /* (g, x, ans, n) g * (x == ans) / n, n = number of positions that attain the
                               extremum of their group (max / min over axes)  numpy_vjps.py:515-530 */
+    /* Two arithmetic rules in one instruction of agmi_program (each rounded on its own, as the two separate
+     * instructions would be).  An interpreted instruction costs far more in operand moves and dispatch than in
+     * arithmetic, so a product that only one sum, difference or product reads travels with its reader.  Programs
+     * only: agmi_elementwise and agmi_map_reduce do not know these. */
+    AGMI_OP_MUL_MUL,       /* (a, b, c)      (a * b) * c                                           */
+    AGMI_OP_MUL_SUB,       /* (a, b, c)      a * b - c                                             */
+    AGMI_OP_MUL_RSUB,      /* (a, b, c)      c - a * b                                             */
+    AGMI_OP_ADD_MUL,       /* (a, b, c)      (a + b) * c                                           */
+    AGMI_OP_SUB_MUL        /* (a, b, c)      (a - b) * c                                           */
 } agmi_op;
 
 /* comparison producing AGMI_BOOL: numpy.equal ... (non-differentiable, numpy_vjps.py:13-68) */

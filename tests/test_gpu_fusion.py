@@ -333,6 +333,54 @@ def test_program_shifted_leaves_and_masks(dtype, n):
     assert onp.array_equal(out.cpu().numpy(), want)
 
 
+@pytest.mark.parametrize("dtype", [F64, F32])
+def test_chained_instructions_equal_their_two_rules(dtype, dnp):
+    """``(a * b) * c``, ``a * b - c``, ``c - a * b``, ``(a + b) * c``, ``(a - b) * c`` as ONE instruction each give what the
+    two one-rule kernels give, and the emitter forms them (and ``a * b + c``) where a product, sum or difference is read
+    once, by a sum, difference or product: fewer interpreted instructions, same bits."""
+    from autograd_amd import _lib
+    from autograd_amd._lib import Op
+    from autograd_amd.numpy import devarray as D
+    from autograd_amd.numpy import fusion
+
+    rs = onp.random.RandomState(21)
+    n = 70001
+    a, b, c = (rs.randn(n).astype(dtype) for _ in range(3))
+    A, B, C = (D.from_numpy(v) for v in (a, b, c))
+    code = _lib.DTYPE_CODE[dtype]
+    two = {Op.MUL_MUL: (Op.MUL, Op.MUL, False), Op.MUL_SUB: (Op.MUL, Op.SUB, False), Op.MUL_RSUB: (Op.MUL, Op.SUB, True),
+           Op.ADD_MUL: (Op.ADD, Op.MUL, False), Op.SUB_MUL: (Op.SUB, Op.MUL, False), Op.MUL_ADD: (Op.MUL, Op.ADD, False)}
+    for both, (first, second, swapped) in two.items():
+        out = _lib.empty((n,), dtype)
+        assert _lib.program(code, (n,), (out,), (A._t, B._t, C._t), [], [W(both, 3, 0, 1, 2), W(_lib.PROGRAM_STORE, 3, 3, 0)], 8)
+        with unfused():
+            t = D.map_op(first, dtype, A, B)
+            want = (D.map_op(second, dtype, C, t) if swapped else D.map_op(second, dtype, t, C)).numpy()
+        assert onp.array_equal(out.cpu().numpy(), want), both
+    # through the emitter: seven rules, four instructions
+    X, Y, Z = (dnp.asarray(v) for v in (a, b, c))
+    seen = []
+    real = _lib.program
+    _lib.program = lambda *args, **k: (seen.append([w & 255 for w in args[5]]), real(*args, **k))[1]
+    try:
+        fusion._PROGRAMS.clear()
+        f = lambda: ((X * Y) * Z - (X - Y) * Z + (Z - X * X) * (Y + Z)).numpy()  # noqa: E731
+        got = f()
+    finally:
+        _lib.program = real
+    with unfused():
+        want = f()
+    assert onp.array_equal(got, want)
+    assert len(seen) == 1 and len(seen[0]) < 9 and any(op in two for op in seen[0]), seen
+    was, fusion.CHAINED = fusion.CHAINED, False
+    try:
+        fusion._PROGRAMS.clear()
+        assert onp.array_equal(f(), want)
+    finally:
+        fusion.CHAINED = was
+        fusion._PROGRAMS.clear()
+
+
 ROW_SUM_SHAPES = [(256, 128), (64, 512), (70, 256), (1000, 65), (100, 64), (1, 40), (7, 5), (3, 2), (300, 257)]
 
 
