@@ -354,6 +354,79 @@ def test_program_keys_tell_apart_what_the_emitted_program_depends_on():
         fusion.ENABLED = was
 
 
+def _ops_of(words):
+    return [w & 0xFF for w in words]
+
+
+def test_the_emitter_chains_a_value_read_once_into_its_reader():
+    """``fusion._emit``: a product, sum or difference with one reader that is a sum, difference or product becomes one
+    three-operand instruction (``x * x`` counts as a product); a value with two readers stays an instruction of its own."""
+    from autograd_amd._lib import Op, PROGRAM_STORE
+    from autograd_amd.numpy import fusion
+
+    was, fusion.ENABLED = fusion.ENABLED, True
+    try:
+        a, b, c = (meta((8, 6), torch.float64) for _ in range(3))
+
+        def ops(root):
+            emitted = fusion._emit([root])
+            assert emitted is not None
+            return _ops_of(emitted[3])
+
+        assert ops((a * b) * c) == [Op.MUL_MUL, PROGRAM_STORE]
+        assert ops(c * (a * b)) == [Op.MUL_MUL, PROGRAM_STORE]
+        assert ops(a * b - c) == [Op.MUL_SUB, PROGRAM_STORE]
+        assert ops(c - a * b) == [Op.MUL_RSUB, PROGRAM_STORE]
+        assert ops(c - D.map_op(Op.SQUARE, a.dtype, a)) == [Op.MUL_RSUB, PROGRAM_STORE]
+        assert ops((a + b) * c) == [Op.ADD_MUL, PROGRAM_STORE]
+        assert ops(c * (a - b)) == [Op.SUB_MUL, PROGRAM_STORE]
+        assert ops(a * b + c) == [Op.MUL_ADD, PROGRAM_STORE]
+        p = a * b
+        assert ops(p * c + p) == [Op.MUL, Op.MUL_ADD, PROGRAM_STORE]  # two readers of p: p * c travels, p stays
+        was_chained, fusion.CHAINED = fusion.CHAINED, False
+        try:
+            assert ops((a * b) * c) == [Op.MUL, Op.MUL, PROGRAM_STORE]
+        finally:
+            fusion.CHAINED = was_chained
+    finally:
+        fusion.ENABLED = was
+
+
+def test_pending_row_sums_broadcast_over_their_rows_join_the_chain():
+    """``fusion._row_sums``: ``sum(e, axis=1, keepdims=True)`` that has not run, multiplied back over the rows of ``e``,
+    becomes a row-sum instruction of the program (16 registers), for the shapes the reduction kernel gives to a group of
+    lanes; other shapes, other axes and sums that have run are ordinary operands."""
+    from autograd_amd._lib import Op, PROGRAM_ROWSUM, PROGRAM_STORE, Red
+    from autograd_amd.numpy import fusion
+
+    was, fusion.ENABLED = fusion.ENABLED, True
+    try:
+        def chain(shape, dtype=torch.float64, axes=(1,), op=Op.COPY):
+            g, t, y = (meta(shape, dtype) for _ in range(3))
+            e = g * t
+            s = D.map_reduce(op, Red.SUM, e.dtype, (e,), axes, True)
+            assert type(s) is D.PendingReduce and s._call is not None
+            return e, s, y
+
+        e, s, y = chain((256, 128))
+        root = e - y * s
+        assert type(root) is fusion.ExprArray and s._call is not None       # nothing ran
+        emitted = fusion._emit([root])
+        assert PROGRAM_ROWSUM in _ops_of(emitted[3]) and emitted[4] == 16 and _ops_of(emitted[3])[-1] == PROGRAM_STORE
+        assert len(emitted[0]) == 3                                          # g, t, y: the sums are no leaf
+        e, s, y = chain((256, 128), op=Op.NEG)                               # the unbroadcast of -g
+        assert PROGRAM_ROWSUM in _ops_of(fusion._emit([e + y * s])[3])
+        for shape, dtype in (((8, 100), torch.float64), ((256, 300), torch.float64), ((64, 600), torch.float32), ((5, 1), torch.float64)):
+            e, s, y = chain(shape, dtype)
+            assert fusion._row_sums(s, shape, e.dtype) is None, shape         # not a shape of the row-group kernel
+        e, s, y = chain((256, 128), axes=(0,))
+        assert fusion._row_sums(s, (256, 128), e.dtype) is None               # column sums
+        assert fusion._row_sums(chain((64, 512), torch.float32)[1], (64, 512), onp.dtype("float32")) is not None
+        assert fusion._row_sums(chain((7, 64))[1], (7, 64), onp.dtype("float64")) is not None
+    finally:
+        fusion.ENABLED = was
+
+
 def test_slices_of_a_pending_product_stay_products():
     """``wrapper._part_of_product``: rows and columns of a product that has not run are taken from its factors when the
     slice keeps at least half of each axis; anything else is left to the ordinary view of the whole product."""
