@@ -344,7 +344,9 @@ def test_weighted_logsumexp_follows_scipy(dnp):
 GEMM_SHAPES = [(1, 1, 1), (5, 7, 3), (64, 64, 16), (65, 63, 17), (130, 70, 33), (256, 128, 641), (1024, 10, 1024),
                (10, 1024, 300), (300, 300, 1), (129, 257, 100), (512, 512, 512),
                # few output tiles and a long K (the K split inside one block): whole and partial chunks, ragged tiles
-               (256, 512, 641), (641, 512, 256), (33, 31, 257), (96, 40, 288), (64, 64, 5000), (200, 130, 4100)]
+               (256, 512, 641), (641, 512, 256), (33, 31, 257), (96, 40, 288), (64, 64, 5000), (200, 130, 4100),
+               # the shortest K that is cut (four waves), around it, and K just short of a whole chunk
+               (256, 512, 128), (100, 70, 130), (33, 257, 200), (64, 64, 127), (70, 30, 159)]
 
 
 @pytest.mark.parametrize("dtype", [F32, F64])
@@ -1543,7 +1545,8 @@ def test_device_resident_row_index_gathers_and_scatters_in_order(dnp, dtype):
 
 
 # ---- dense-layer epilogues of the contraction ------------------------------------------------------
-@pytest.mark.parametrize("M,N,K", [(64, 64, 32), (200, 130, 70), (256, 512, 641), (1024, 1024, 784), (7, 3, 5), (70, 45, 300)])
+@pytest.mark.parametrize("M,N,K", [(64, 64, 32), (200, 130, 70), (256, 512, 641), (1024, 1024, 784), (7, 3, 5), (70, 45, 300),
+                                   (256, 512, 128), (90, 33, 150)])
 def test_gemm_epilogues_equal_the_separate_kernels(dnp, M, N, K):
     """``agmi_gemm_fused``: tanh(A.B + bias) and (G.W^T) / cosh(x + bias)**2 formed inside the contraction are, bit for
     bit, what the product followed by the elementwise kernels gives (examples/neural_net.py:33-35,
