@@ -179,6 +179,12 @@ def lib():
     L.agmi_program.restype = c_i
     L.agmi_program.argtypes = [c_i, c_i, p_i64, c_i, p_arr, c_i, p_arr, p_i64, c_i, p_d, c_i, p_i64, c_i,
                                ctypes.POINTER(ctypes.c_uint32), c_i, c_p]
+    L.agmi_program_specialize.restype = c_i
+    L.agmi_program_specialize.argtypes = [c_i]
+    L.agmi_program_specialized.restype = None
+    L.agmi_program_specialized.argtypes = [ctypes.POINTER(ctypes.c_longlong), ctypes.POINTER(ctypes.c_longlong)]
+    L.agmi_program_source.restype = ctypes.c_longlong
+    L.agmi_program_source.argtypes = [c_i, c_i, c_i, c_i, ctypes.POINTER(ctypes.c_uint32), c_i, c_i, ctypes.c_char_p, ctypes.c_size_t]
     L.agmi_compare.restype = c_i
     L.agmi_compare.argtypes = [c_i, c_i, c_i, p_i64, p_arr, p_arr, p_d, c_p]
     L.agmi_cast.restype = c_i
@@ -224,7 +230,8 @@ def lib():
 EXPORTS = (
     "agmi_last_error agmi_version agmi_last_kernel agmi_elementwise agmi_program agmi_compare agmi_cast agmi_map_reduce "
     "agmi_map_reduce_workspace_bytes agmi_map_reduce_static agmi_gemm agmi_gemm_fused agmi_fill agmi_take_rows agmi_sort_rows agmi_cumsum agmi_reverse agmi_triangle agmi_scatter_add_rows agmi_optimizer_step "
-    "agmi_correlate agmi_lse_cotangent_fused agmi_concat agmi_probe_arm agmi_probe_elapsed"
+    "agmi_correlate agmi_lse_cotangent_fused agmi_concat agmi_probe_arm agmi_probe_elapsed "
+    "agmi_program_specialize agmi_program_specialized agmi_program_source"
 ).split()
 
 
@@ -541,6 +548,32 @@ def program(code, shape, outs, leaves, imms, words, n_regs, shifted=None, masks=
     if ev is not None:
         _TIMER.end(ev, ("program",), (outs, leaves))
     return True
+
+
+def specialize_after(sightings):
+    """Programs handed to :func:`program` this many times get a kernel compiled for them (0: never; negative: only
+    ask).  Returns the previous setting."""
+    return lib().agmi_program_specialize(int(sightings))
+
+
+def specialized_programs():
+    """(programs compiled so far, launches they have served)."""
+    compiled, launches = ctypes.c_longlong(), ctypes.c_longlong()
+    lib().agmi_program_specialized(ctypes.byref(compiled), ctypes.byref(launches))
+    return compiled.value, launches.value
+
+
+def program_source(code, n_leaf, n_imm, words, n_regs, row_sums=False):
+    """The HIP source of the kernel a recurring program is specialised to."""
+    L = lib()
+    n = len(words)
+    arr = (ctypes.c_uint32 * n)(*words)
+    size = L.agmi_program_source(code, n_leaf, n_imm, n, arr, n_regs, 1 if row_sums else 0, None, 0)
+    if size < 0:
+        _check(int(size), "agmi_program_source")
+    text = ctypes.create_string_buffer(size + 1)
+    L.agmi_program_source(code, n_leaf, n_imm, n, arr, n_regs, 1 if row_sums else 0, text, size + 1)
+    return text.value.decode()
 
 
 def compare(cmp, code, shape, out, ins):

@@ -25,33 +25,9 @@
 #include "common.h"
 
 #include "functors.h"
+#include "program_params.h"
 
 namespace agmi {
-
-constexpr int kProgMaxLeaf = AGMI_PROGRAM_MAX_LEAVES;
-constexpr int kProgMaxImm = AGMI_PROGRAM_MAX_IMMEDIATES;
-constexpr int kProgMaxOut = AGMI_PROGRAM_MAX_OUTPUTS;
-constexpr int kProgMaxInstr = AGMI_PROGRAM_MAX_INSTRUCTIONS;
-constexpr int kProgMaxMask = AGMI_PROGRAM_MAX_MASKS;
-
-struct ProgParams {
-    int64_t cols;
-    uint32_t tiles_per_row, n_tiles;
-    uint32_t step_rows, step_chunks;  // the wave stride (number of waves in the grid) split by tiles_per_row
-    int32_t n_leaf, n_imm, n_instr;
-    int32_t row_group;  // programs with row sums: the lanes that share a row in the reduction kernel's order
-    const void *leaf[kProgMaxLeaf];
-    int64_t leaf_rs[kProgMaxLeaf];
-    int32_t leaf_cs[kProgMaxLeaf];  // 0 or 1
-    // columns a leaf may be read at (one-row programs whose leaves are read at shifted positions); all columns otherwise
-    int64_t leaf_lo[kProgMaxLeaf], leaf_hi[kProgMaxLeaf];
-    int64_t safe_lo, safe_hi;  // the columns every leaf may be read at
-    int64_t mask_lo[kProgMaxMask], mask_hi[kProgMaxMask];
-    void *out[kProgMaxOut];
-    int64_t out_rs[kProgMaxOut];
-    double imm[kProgMaxImm];
-    uint32_t code[kProgMaxInstr + 1];  // one word of padding: the fetch runs one instruction ahead
-};
 
 template <typename T, int NREG>
 struct RegVec {
@@ -134,16 +110,6 @@ __device__ __forceinline__ T apply_one(const T (&xi)[4]) {
     } else {
         return apply_called<Fn, T>(xi[0], Fn::NIN > 1 ? xi[1] : T(0), Fn::NIN > 2 ? xi[2] : T(0), Fn::NIN > 3 ? xi[3] : T(0));
     }
-}
-
-// The last, partly filled vector of a row.  A function of its own: its per-lane branches would otherwise make
-// the compiler restructure the whole interpreter loop around them (every wave-uniform branch of the dispatch
-// would then cost several scalar instructions more).
-template <typename T, int VL>
-static __device__ __noinline__ void store_partial(T *base, int64_t c, int64_t cols, T __attribute__((ext_vector_type(VL))) v) {
-#pragma unroll
-    for (int j = 0; j < VL; ++j)
-        if (c + j < cols) base[c + j] = v[j];
 }
 
 // op | dst << 8 | a << 12 | b << 16 | c << 20 | d << 24
@@ -409,6 +375,7 @@ static int launch_program(const ProgParams &p0, int64_t rows, hipStream_t s) {
 #ifndef AGMI_PART
 #error "compile with -DAGMI_PART=32 or -DAGMI_PART=64"
 #endif
+int launch_specialized(bool f32, int nreg, const ProgParams &p, int64_t rows, hipStream_t s);  // specialize.hip
 int program_part_f32(int nreg, bool light, const ProgParams &p, int64_t rows, hipStream_t s);
 int program_part_f64(int nreg, bool light, const ProgParams &p, int64_t rows, hipStream_t s);
 // Two vectors per lane in every variant (measured on the 4M-element float64 tanh-gradient chain: 40 us against 42 with one;
@@ -625,6 +592,9 @@ extern "C" int agmi_program(int dtype, int ndim, const int64_t *shape, int n_out
     for (int i = 0; i < n_instr; ++i) p.code[i] = code[i];
     p.code[n_instr] = 0;
     hipStream_t s = as_stream(stream);
+    // a program that keeps coming back runs on a kernel compiled for it (1: not this one, or not yet)
+    const int specialised = launch_specialized(dtype == AGMI_F32, nreg, p, rows, s);
+    if (specialised <= 0) return specialised;
     set_kernel_name("ew_program<%s,%d,%s>[%d instr, %lldx%lld]", dtype == AGMI_F32 ? "float" : "double", nreg,
                     row_group ? "rows" : (light ? "light" : "full"), n_instr, (long long)rows, (long long)p.cols);
     return dtype == AGMI_F32 ? program_part_f32(nreg, light, p, rows, s) : program_part_f64(nreg, light, p, rows, s);

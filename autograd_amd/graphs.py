@@ -75,10 +75,21 @@ class CapturedFunction:
         self._last = [None] * len(leaves)  # the array object last copied into each input buffer
         self._writes_seen = D.ITEM_WRITES  # value of the item-assignment counter at the last call
         args = _unflatten(self._in_struct, iter(self._static_in))
-        for _ in range(max(int(warmup), 1)):
-            # eager runs first: one-time allocations (shared zeros, the reduction workspace)
-            # happen outside the graph's memory pool, and unsupported programs fail here plainly
-            fun(*args)
+        # eager runs first: one-time allocations (shared zeros, the reduction workspace) happen outside the graph's
+        # memory pool, unsupported programs fail here plainly, and the elementwise programs of a function that is
+        # about to be replayed many times get their specialised kernels now (none can be compiled while recording)
+        sightings = _lib.specialize_after(-1)
+        if sightings > 0:
+            _lib.specialize_after(1)
+        try:
+            for _ in range(max(int(warmup), 1)):
+                warm = []
+                _flatten(fun(*args), warm)
+                for o in warm:
+                    if isinstance(o, DevArray):
+                        D.plain(o)  # (results still pending are written out, as the recording will)
+        finally:
+            _lib.specialize_after(sightings)
         _lib.synchronize()
         self._graph = torch.cuda.CUDAGraph()
         timer, _lib._TIMER = _lib._TIMER, None

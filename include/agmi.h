@@ -243,6 +243,25 @@ int agmi_program(int dtype, int ndim, const int64_t *shape, int n_out, const agm
                  int n_imm, const double *imms, int n_mask, const int64_t *mask_ranges,
                  int n_instr, const uint32_t *code, int n_regs, void *stream);
 
+/* Programs that recur are specialised: once agmi_program has been handed the same program (dtype, register
+ * count, leaf and immediate counts, instruction words) `after` times on a device, the library writes it out
+ * as straight-line HIP over the same functors, compiles it for gfx950 with the run-time compiler (the
+ * library's own flags: -ffp-contract=off, no packed float32 forms) and from then on launches that kernel
+ * in the interpreter's place: same argument block, same tiling, same bits, no decode and no register moves
+ * (config 1's first derivative: 41 us interpreted, 15 us specialised).  Nothing is compiled while the stream
+ * records a graph; a program whose compilation fails stays with the interpreter (agmi_last_error says why).
+ * agmi_program_specialize sets `after` (0: never; default 3, or AUTOGRAD_AMD_SPECIALIZE from the
+ * environment; negative: leave as is) and returns the previous value; agmi_program_specialized reports how
+ * many programs have been compiled and how many launches they have served.  No counterpart in the reference
+ * (its rules are NumPy calls). */
+int agmi_program_specialize(int after);
+void agmi_program_specialized(long long *compiled, long long *launches);
+/* The HIP source of the kernel a program is specialised to (for inspection and for checking, without a GPU, that
+ * it compiles): written to `text` (at most capacity - 1 characters and a terminating zero; may be NULL); returns
+ * its full length, or a negative error.  `row_sums`: the program holds AGMI_PROGRAM_ROWSUM. */
+long long agmi_program_source(int dtype, int n_leaf, int n_imm, int n_instr, const uint32_t *code, int n_regs,
+                              int row_sums, char *text, size_t capacity);
+
 /* out[idx] = (in0[idx] <cmp> in1[idx]) as AGMI_BOOL; inputs as in agmi_elementwise. */
 int agmi_compare(int cmp, int dtype, int ndim, const int64_t *shape,
                  const agmi_array *out, const agmi_array *ins, const double *scalars,

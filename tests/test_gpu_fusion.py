@@ -381,6 +381,92 @@ def test_chained_instructions_equal_their_two_rules(dtype, dnp):
         fusion._PROGRAMS.clear()
 
 
+# ---- recurring programs get a kernel of their own -------------------------------------------------------
+class specializing:
+    """``with specializing(n): ...``: programs seen ``n`` times are compiled (0: never)."""
+
+    def __init__(self, after):
+        self.after = after
+
+    def __enter__(self):
+        from autograd_amd import _lib
+
+        self.was = _lib.specialize_after(self.after)
+
+    def __exit__(self, *exc):
+        from autograd_amd import _lib
+
+        _lib.specialize_after(self.was)
+
+
+@pytest.mark.parametrize("dtype", [F64, F32])
+def test_a_specialised_kernel_gives_the_interpreters_bits(dtype, dnp):
+    """The same expression by the interpreter, by the kernel compiled for it, and rule by rule: the same bits, on
+    flat arrays with ragged ends, on row / column broadcasts, with shifted vectors and masks, and with a row sum
+    inside the chain; functions from every family of the functor table."""
+    from autograd_amd import _lib
+    from autograd_amd.numpy import fusion
+
+    rs = onp.random.RandomState(31)
+
+    def cases():
+        n = 100003
+        x, y = (rs.randn(n).astype(dtype) for _ in range(2))
+        X, Y = dnp.asarray(x), dnp.asarray(y)
+        yield lambda: (dnp.tanh(X * Y + 0.5) / (dnp.exp(X) + 2.0) - Y).numpy()
+        yield lambda: (dnp.sin(X) * dnp.log1p(dnp.abs(Y)) + dnp.sqrt(dnp.abs(X)) ** 1.5 - dnp.arctan2(X, Y)).numpy()
+        yield lambda: (X[1:] * X[:-1] - Y[1:] * 3.0 + (X[1:] - Y[:-1]) * Y[1:]).numpy()
+        a, b, c = rs.randn(300, 130).astype(dtype), rs.randn(130).astype(dtype), rs.randn(300, 1).astype(dtype)
+        A, B, C = dnp.asarray(a), dnp.asarray(b), dnp.asarray(c)
+        yield lambda: (dnp.tanh(A * B + C) * A - dnp.exp(C) * B).numpy()
+        yield lambda: ((A * B) - dnp.exp(A - C) * dnp.sum(A * B, axis=1, keepdims=True)).numpy()
+
+    for f in cases():
+        before = _lib.specialized_programs()
+        with specializing(0):
+            fusion._PROGRAMS.clear()
+            interpreted = f()
+        assert _lib.specialized_programs() == before
+        with specializing(1):
+            compiled = f()
+            again = f()
+        after = _lib.specialized_programs()
+        assert after[1] >= before[1] + 2, (before, after)      # both evaluations ran on the compiled kernel
+        with unfused():
+            plain = f()
+        assert _same_bits(compiled, interpreted) and _same_bits(again, interpreted) and _same_bits(interpreted, plain)
+
+
+def test_programs_are_specialised_after_a_few_sightings_and_never_while_a_graph_records(dnp):
+    import autograd_amd as ag
+    from autograd_amd import _lib, graphs
+
+    rs = onp.random.RandomState(8)
+    n = 50021
+    X = dnp.asarray(rs.randn(n))
+    f = lambda x: dnp.exp(x * 0.37) * x - dnp.cos(x) / (x * x + 1.25)  # noqa: E731  (an expression no other test uses)
+    with specializing(3):
+        c0, l0 = _lib.specialized_programs()
+        first = f(X).numpy()
+        second = f(X).numpy()
+        assert _lib.specialized_programs() == (c0, l0)                  # two sightings: the interpreter
+        third = f(X).numpy()
+        assert _lib.specialized_programs() == (c0 + 1, l0 + 1)          # compiled and used
+        assert onp.array_equal(first, second) and onp.array_equal(first, third)
+        # a function about to be recorded compiles its programs during the eager warm-up run, and replays them
+        g = lambda x: dnp.sinh(x * 0.21) - x / (dnp.exp(x) + 3.5)  # noqa: E731
+        eager = g(X).numpy()
+        c1, l1 = _lib.specialized_programs()
+        replayed = graphs.capture(g, X)
+        c2, l2 = _lib.specialized_programs()
+        assert c2 == c1 + 1 and l2 >= l1 + 2                             # warm-up and recording both ran it
+        for _ in range(3):
+            Z = dnp.asarray(rs.randn(n))
+            assert onp.array_equal(replayed(Z).numpy(), g(Z).numpy())
+        assert onp.array_equal(replayed(X).numpy(), eager)
+        assert _lib.specialize_after(-1) == 3                            # the recording put the setting back
+
+
 ROW_SUM_SHAPES = [(256, 128), (64, 512), (70, 256), (1000, 65), (100, 64), (1, 40), (7, 5), (3, 2), (300, 257)]
 
 

@@ -92,6 +92,45 @@ def test_argument_errors_are_reported_without_a_gpu(lib):
     assert lib.agmi_sort_rows(7, buf, i64(1), i64(8), buf, None, None, None) == -1 and b"floating" in lib.agmi_last_error()
 
 
+def test_the_source_of_a_specialised_program_compiles_for_gfx950():
+    """``agmi_program_source``: the straight-line kernel a recurring program is compiled to, here for a program with
+    one-rule, two-rule and long functors, a mask, a row sum and two outputs.  The run-time compiler needs no GPU, so
+    this checks on the CPU that the text the library generates (and the headers it carries inside) compiles for
+    gfx950 with the library's own flags."""
+    from autograd_amd import _lib
+    from autograd_amd._lib import Op
+
+    def W(op, dst, a=0, b=0, c=0, d=0):
+        return op | dst << 8 | a << 12 | b << 16 | c << 20 | d << 24
+
+    words = [W(Op.MUL, 2, 0, 1), W(Op.EXP, 3, 2), W(Op.MUL_ADD, 4, 3, 0, 15), W(_lib.PROGRAM_MASK, 5, 4, 0, 3),
+             W(_lib.PROGRAM_ROWSUM, 6, 5), W(Op.TANH, 7, 6), W(Op.POW, 8, 7, 14), W(Op.SUB_MUL, 9, 8, 0, 1),
+             W(Op.LSE_VJP, 10, 9, 0, 1, 2), W(_lib.PROGRAM_STORE, 10, 10, 0), W(_lib.PROGRAM_STORE, 7, 7, 1)]
+    try:
+        rtc = ctypes.CDLL("libhiprtc.so")
+    except OSError:
+        rtc = ctypes.CDLL("/opt/rocm/lib/libhiprtc.so")
+    for code, name in ((0, "float"), (1, "double")):
+        source = _lib.program_source(code, 2, 2, words, 16, row_sums=True)
+        assert f"typedef {name} T;" in source and "FLseVjp<T>::apply" in source and "row_values" in source
+        assert source.count("// instruction") == len(words)
+        prog = ctypes.c_void_p()
+        assert rtc.hiprtcCreateProgram(ctypes.byref(prog), source.encode(), b"agmi_specialized.hip", 0, None, None) == 0
+        options = [o.encode() for o in ("--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off",
+                                        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops")]
+        rc = rtc.hiprtcCompileProgram(prog, len(options), (ctypes.c_char_p * len(options))(*options))
+        n = ctypes.c_size_t()
+        rtc.hiprtcGetProgramLogSize(prog, ctypes.byref(n))
+        log = ctypes.create_string_buffer(n.value + 1)
+        rtc.hiprtcGetProgramLog(prog, log)
+        assert rc == 0, log.value.decode()[:2000]
+        rtc.hiprtcGetCodeSize(prog, ctypes.byref(n))
+        assert n.value > 1000
+        rtc.hiprtcDestroyProgram(ctypes.byref(prog))
+    with pytest.raises(_lib.AgmiError, match="unknown op"):
+        _lib.program_source(0, 1, 0, [W(200, 1, 0)], 16)
+
+
 def test_device_path_fails_loudly_without_gpu():
     import torch
 
