@@ -395,17 +395,37 @@ def _distinct_bytes(t):
 
 
 def _traffic(outs, ins):
+    """Algorithmic bytes of a launch: every result element written once, every distinct operand element read once
+    (views of one storage, such as a vector read at several shifts, count as the stretch of memory they cover
+    together, not once each)."""
     total = 0
     for t in outs:
         total += t.numel() * t.element_size()
+    by_storage = {}
+
+    def read(t):
+        es = t.element_size()
+        begin = t.data_ptr()
+        span = 1
+        for extent, stride in zip(t.shape, t.stride()):
+            if extent == 0:
+                return
+            span += (extent - 1) * abs(stride)
+        entry = by_storage.setdefault(begin - t.storage_offset() * es, [0, begin, begin])
+        entry[0] += _distinct_bytes(t)
+        entry[1] = min(entry[1], begin)
+        entry[2] = max(entry[2], begin + span * es)
+
     for t in ins:
         if type(t) is Affine:
             for aux in (t.ascale, t.shift):
                 if isinstance(aux, torch.Tensor):
-                    total += _distinct_bytes(aux)
+                    read(aux)
             t = t.t
         if isinstance(t, torch.Tensor):
-            total += _distinct_bytes(t)
+            read(t)
+    for distinct, begin, end in by_storage.values():
+        total += min(distinct, end - begin)
     return total
 
 

@@ -11,6 +11,7 @@
 #include <hip/hiprtc.h>
 
 #include <algorithm>
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <iterator>
@@ -37,6 +38,7 @@ struct SpecKernel {
     int state = 0;  // 0 not compiled, 1 ready, -1 failed
     hipModule_t module = nullptr;
     hipFunction_t function = nullptr;
+    std::string name;
 };
 
 static std::mutex g_spec_mutex;
@@ -68,14 +70,28 @@ static int functor_arity(int op) {
 #undef AGMI_ARITY_CASE
 }
 
-// The kernel's text.  Registers are plain local arrays with constant indices: the compiler keeps what is live.
-static std::string spec_source(bool f32, int nreg, const ProgParams &p) {
+// The kernel's name in traces: precision, instruction count and a hash of the instruction words, so that one
+// row of a kernel trace is one program.
+static std::string spec_name(bool f32, const ProgParams &p) {
+    uint32_t h = 2166136261u;
+    for (int i = 0; i < p.n_instr; ++i)
+        for (int b = 0; b < 4; ++b) h = (h ^ ((p.code[i] >> (8 * b)) & 0xffu)) * 16777619u;
+    char text[64];
+    std::snprintf(text, sizeof(text), "agmi_specialized_%s_%dinstr_%08x", f32 ? "f32" : "f64", p.n_instr, h);
+    return text;
+}
+
+// The kernel's text.  Leaves are read with plain loads (chains read one array at several shifts: the second and third
+// read of a line must find it in the cache, which the interpreter's non-temporal loads cost 20 us of a 95 us
+// Hessian-vector product), results leave with non-temporal stores (nothing in the kernel reads them back: 81 -> 62 us).
+//  Registers are plain local arrays with constant indices: the compiler keeps what is live.
+static std::string spec_source(bool f32, int nreg, const ProgParams &p, const std::string &name) {
     std::ostringstream o;
     o << "typedef signed long long int64_t;\ntypedef unsigned long long uint64_t;\ntypedef int int32_t;\n"
          "typedef unsigned int uint32_t;\ntypedef unsigned char uint8_t;\ntypedef unsigned long size_t;\n";
     for (const char *h : kSpecHeaders) o << h << "\n";
     o << "using namespace agmi;\n"
-         "extern \"C\" __global__ __launch_bounds__(256) void agmi_specialized(const agmi::ProgParams p) {\n"
+         "extern \"C\" __global__ __launch_bounds__(256) void " << name << "(const agmi::ProgParams p) {\n"
       << "    typedef " << (f32 ? "float" : "double") << " T;\n"
       << R"SRC(    constexpr int U = 2, VL = 16 / sizeof(T), V = VL * U, TW = 64 * V;
     typedef T vec_t __attribute__((ext_vector_type(VL), aligned(sizeof(T))));
@@ -100,7 +116,7 @@ static std::string spec_source(bool f32, int nreg, const ProgParams &p) {
           << k << "];\n            if (p.leaf_cs[" << k << "] == 0) {\n                const T s = *base;\n"
           << "                _Pragma(\"unroll\") for (int j = 0; j < V; ++j) r" << k << "[j] = s;\n"
           << "            } else if (readable) {\n                _Pragma(\"unroll\") for (int u = 0; u < U; ++u) {\n"
-          << "                    const vec_t v = __builtin_nontemporal_load(reinterpret_cast<const vec_t *>(base + c0 + u * (64 * VL)));\n"
+          << "                    const vec_t v = *reinterpret_cast<const vec_t *>(base + c0 + u * (64 * VL));\n"
           << "                    _Pragma(\"unroll\") for (int j = 0; j < VL; ++j) r" << k << "[u * VL + j] = v[j];\n                }\n"
           << "            } else {\n                _Pragma(\"unroll\") for (int u = 0; u < U; ++u)\n"
           << "                    _Pragma(\"unroll\") for (int j = 0; j < VL; ++j) {\n"
@@ -119,7 +135,7 @@ static std::string spec_source(bool f32, int nreg, const ProgParams &p) {
             o << "            T *base = static_cast<T *>(p.out[" << src[1] << "]) + static_cast<int64_t>(cur_row) * p.out_rs[" << src[1]
               << "];\n            _Pragma(\"unroll\") for (int u = 0; u < U; ++u) {\n                vec_t v;\n"
               << "                _Pragma(\"unroll\") for (int j = 0; j < VL; ++j) v[j] = r" << src[0] << "[u * VL + j];\n"
-              << "                if (interior) *reinterpret_cast<vec_t *>(base + c0 + u * (64 * VL)) = v;\n"
+              << "                if (interior) __builtin_nontemporal_store(v, reinterpret_cast<vec_t *>(base + c0 + u * (64 * VL)));\n"
               << "                else store_partial<T, VL>(base, c0 + u * (64 * VL), cols, v);\n            }\n        }\n";
             continue;
         }
@@ -170,7 +186,7 @@ static std::string spec_source(bool f32, int nreg, const ProgParams &p) {
     return o.str();
 }
 
-static bool spec_compile(const std::string &source, SpecKernel *k, std::string *log) {
+static bool spec_compile(const std::string &source, const std::string &name, SpecKernel *k, std::string *log) {
     hiprtcProgram prog = nullptr;
     if (hiprtcCreateProgram(&prog, source.c_str(), "agmi_specialized.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS) {
         *log = "hiprtcCreateProgram failed";
@@ -198,7 +214,7 @@ static bool spec_compile(const std::string &source, SpecKernel *k, std::string *
         *log = "hipModuleLoadData failed";
         return false;
     }
-    if (hipModuleGetFunction(&k->function, k->module, "agmi_specialized") != hipSuccess) {
+    if (hipModuleGetFunction(&k->function, k->module, name.c_str()) != hipSuccess) {
         (void)hipGetLastError();
         (void)hipModuleUnload(k->module);
         k->module = nullptr;
@@ -238,12 +254,14 @@ int launch_specialized(bool f32, int nreg, const ProgParams &p0, int64_t rows, h
         if (hipStreamIsCapturing(s, &capturing) != hipSuccess) (void)hipGetLastError();
         if (capturing != hipStreamCaptureStatusNone) return 1;  // a module cannot be loaded while a graph is recorded
         std::string log;
-        if (!spec_compile(spec_source(f32, nreg, p0), &k, &log)) {
+        const std::string name = spec_name(f32, p0);
+        if (!spec_compile(spec_source(f32, nreg, p0, name), name, &k, &log)) {
             k.state = -1;
             set_error("program: specialising a recurring program failed, the interpreter keeps running it: %.400s", log.c_str());
             return 1;
         }
         k.state = 1;
+        k.name = name;
         ++g_spec_compiled;
     }
     ProgParams p = p0;
@@ -260,7 +278,7 @@ int launch_specialized(bool f32, int nreg, const ProgParams &p0, int64_t rows, h
     p.step_chunks = static_cast<uint32_t>(n_waves % tpr);
     size_t size = sizeof(p);
     void *extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &p, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
-    set_kernel_name("ew_specialized<%s>[%d instr, %lldx%lld]", f32 ? "float" : "double", p.n_instr, (long long)rows, (long long)p.cols);
+    set_kernel_name("%s[%lldx%lld]", k.name.c_str(), (long long)rows, (long long)p.cols);
     const hipError_t rc = hipModuleLaunchKernel(k.function, static_cast<unsigned>(blocks), 1, 1, 256, 1, 1, 0, s, nullptr, extra);
     if (rc != hipSuccess) return hip_check(rc, "specialised program launch");
     ++g_spec_launches;
@@ -309,7 +327,7 @@ extern "C" long long agmi_program_source(int dtype, int n_leaf, int n_imm, int n
         p.code[i] = code[i];
     }
     const int nreg = (n_regs <= 8 && dtype == AGMI_F64) ? 8 : 16;
-    const std::string source = spec_source(dtype == AGMI_F32, nreg, p);
+    const std::string source = spec_source(dtype == AGMI_F32, nreg, p, spec_name(dtype == AGMI_F32, p));
     if (text && capacity > 0) {
         const size_t n = std::min(capacity - 1, source.size());
         std::memcpy(text, source.data(), n);
