@@ -764,7 +764,7 @@ def _emit(roots):
         ok = True
         for k, (op, srcs, mask) in enumerate(instrs):
             regs = [reg[s] for s in srcs]
-            for s in set(srcs):
+            for s in dict.fromkeys(srcs):  # (each once, in operand order: the same words in every process)
                 if s[0] != "I" and last[s] == k:
                     free.append(reg[s])
             if not free:

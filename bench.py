@@ -58,7 +58,9 @@ def end_to_end(compulsory_bytes, evals_per_sec):
 
 
 def time_steps(fn, sync, steps, warmup):
-    for _ in range(warmup):
+    # at least three untimed runs: an elementwise program handed over for the third time is compiled into a kernel
+    # of its own (a few tenths of a second, once), which belongs to the warm-up like the first run's allocations
+    for _ in range(max(warmup, 3)):
         fn()
     sync()
     t0 = time.perf_counter()
@@ -343,11 +345,14 @@ def main():
     # warm-up, then PROBE_STEPS steps with every launch timed (stream kept busy ahead of each step) to find
     # the kernel that dominates the step and to report every kernel's average duration
     PROBE_STEPS = 5
-    t0 = time.perf_counter()
-    for _ in range(max(1, args.warmup)):
+    for _ in range(max(3, args.warmup)):  # (three: a recurring elementwise program is compiled at its third sighting)
         step()
     be.sync()
-    host_ms = (time.perf_counter() - t0) / max(1, args.warmup) * 1e3
+    t0 = time.perf_counter()
+    for _ in range(2):
+        step()
+    be.sync()
+    host_ms = (time.perf_counter() - t0) / 2 * 1e3
     ahead = HeadStart()
     with _lib.KernelTimer() as probe:
         for _ in range(PROBE_STEPS):
@@ -499,9 +504,9 @@ def extras(be):
     x = be.put(configs.tanh_inputs()["x"])
     prog = configs.tanh_program(be)
     for k in ("d1", "d2", "d3"):
-        ms = time_steps(lambda: prog[k](x), be.sync, 10, 2) * 1e3
+        ms = time_steps(lambda: prog[k](x), be.sync, 40, 5) * 1e3
         out[f"tanh_{k}_evals_per_sec"] = 1e3 / ms
-        out[f"tanh_{k}_graph_evals_per_sec"] = graph_rate(prog[k], (x,), be.sync, 10)
+        out[f"tanh_{k}_graph_evals_per_sec"] = graph_rate(prog[k], (x,), be.sync, 40)
     # config 3: MLP gradient, f32; MFMA rate over the GEMMs whose dimensions are all >= 784
     inp = configs.mlp_inputs()
     params3 = configs.tree_map(be.put, inp["params"])
@@ -545,12 +550,12 @@ def extras(be):
     inp = configs.rosen_inputs()
     x5, v5 = be.put(inp["x"]), be.put(inp["v"])
     p5 = configs.rosen_program(be)
-    ms = time_steps(lambda: p5["hvp_rev"](x5, v5), be.sync, 5, 1) * 1e3
+    ms = time_steps(lambda: p5["hvp_rev"](x5, v5), be.sync, 30, 5) * 1e3
     out["rosen_hvp_rev_evals_per_sec"] = 1e3 / ms
-    out["rosen_hvp_rev_graph_evals_per_sec"] = graph_rate(p5["hvp_rev"], (x5, v5), be.sync, 5)
-    ms = time_steps(lambda: p5["hvp_fwd"](x5, v5), be.sync, 5, 1) * 1e3
+    out["rosen_hvp_rev_graph_evals_per_sec"] = graph_rate(p5["hvp_rev"], (x5, v5), be.sync, 30)
+    ms = time_steps(lambda: p5["hvp_fwd"](x5, v5), be.sync, 30, 5) * 1e3
     out["rosen_hvp_fwd_evals_per_sec"] = 1e3 / ms
-    out["rosen_hvp_fwd_graph_evals_per_sec"] = graph_rate(p5["hvp_fwd"], (x5, v5), be.sync, 5)
+    out["rosen_hvp_fwd_graph_evals_per_sec"] = graph_rate(p5["hvp_fwd"], (x5, v5), be.sync, 30)
     # training-loop residency: one fused Adam update of a flat 2^24-element float64 parameter vector
     # (reads x, g, m, v; writes m, v, x: 56 bytes per element), and whole MLP training steps
     # (gradient + flatten + update, nothing leaves HBM)
