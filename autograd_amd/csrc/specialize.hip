@@ -45,8 +45,8 @@ static std::mutex g_spec_mutex;
 static std::unordered_map<std::string, SpecKernel> g_spec;
 static int g_spec_after = -1;  // compile at this many sightings; 0: never; -1: read the environment first
 static long long g_spec_launches = 0, g_spec_compiled = 0;
-constexpr long long kSpecMaxKernels = 512;  // compiled programs kept (each a loaded code object)
-constexpr size_t kSpecMaxSeen = 4096;       // programs remembered, compiled or only counted
+constexpr long long kSpecMaxKernels = 4096;  // compiled programs kept (each a loaded code object of some tens of KB)
+constexpr size_t kSpecMaxSeen = 16384;        // programs remembered, compiled or only counted
 
 static const char *functor_name(int op) {
 #define AGMI_NAME_CASE(OP, FN) \
