@@ -38,6 +38,21 @@ def _shared_one(dtype):
     return o
 
 
+_SEED_VIEWS = {}
+
+
+def _seed_view(one, shape, dtype):
+    """The shared zero (or one) seen through ``shape``: a stride-0 view that nothing ever writes, so the view itself
+    is shared too (making one costs a few microseconds of a gradient evaluation that makes several)."""
+    key = (one, shape, dtype)
+    t = _SEED_VIEWS.get(key)
+    if t is None:
+        if len(_SEED_VIEWS) >= 1024:
+            _SEED_VIEWS.clear()
+        t = _SEED_VIEWS[key] = (_shared_one(dtype) if one else _shared_zero(dtype))._t.expand(shape)
+    return t
+
+
 def is_broadcast_view(x):
     """True when some axis of extent > 1 has stride 0: several indices share one element."""
     t = x._h()
@@ -85,7 +100,7 @@ class DevArrayVSpace(VSpace):
         ``_mut_add`` and the scatter rule allocate the real buffer when they meet it."""
         if self.size == 0:
             return D.zeros(self.shape, self.dtype)
-        return DevArray(_shared_zero(self.dtype)._t.expand(self.shape), self.dtype)
+        return DevArray(_seed_view(0, self.shape, self.dtype), self.dtype)
 
     def ones(self):
         """The seed cotangent of ``elementwise_grad`` (differential_operators.py:41-49 of the reference
@@ -93,7 +108,7 @@ class DevArrayVSpace(VSpace):
         backward pass writes nothing and the first rule reads the seed from a register."""
         if self.size == 0:
             return D.ones(self.shape, self.dtype)
-        return DevArray(_shared_one(self.dtype)._t.expand(self.shape), self.dtype)
+        return DevArray(_seed_view(1, self.shape, self.dtype), self.dtype)
 
     def standard_basis(self):
         for idxs in onp.ndindex(*self.shape):

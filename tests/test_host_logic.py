@@ -200,6 +200,7 @@ def test_accumulators_never_write_through_a_pending_map(monkeypatch):
     from autograd_amd.numpy.vspaces import DevArrayVSpace, is_shared_zero
 
     monkeypatch.setitem(vspaces._ZEROS, onp.dtype("float64"), DevArray(torch.zeros((), dtype=torch.float64)))
+    monkeypatch.setattr(vspaces, "_SEED_VIEWS", {})
     x = meta((3, 4), torch.float64)
     vs = DevArrayVSpace(x)
     g = W.negative(x)
@@ -279,6 +280,7 @@ def test_pending_products_are_contracted_into_an_accumulator_of_its_own(monkeypa
     monkeypatch.setattr(D, "gemm2d", fake_gemm2d)
     monkeypatch.setattr(D._lib, "empty", lambda shape, dtype: torch.zeros(tuple(shape), dtype=torch.float64))
     monkeypatch.setitem(vspaces._ZEROS, onp.dtype("float64"), DevArray(torch.zeros((), dtype=torch.float64)))
+    monkeypatch.setattr(vspaces, "_SEED_VIEWS", {})  # (views of the shared zero are kept: none of another zero's here)
     left, right = torch.zeros((3, 5), dtype=torch.float64), torch.zeros((5, 4), dtype=torch.float64)
     vs = vspaces.DevArrayVSpace(DevArray(torch.zeros((3, 4), dtype=torch.float64)))
     first = D.PendingProduct(left, right, onp.dtype("float64"))
