@@ -18,7 +18,13 @@
 //
 // Index space: (rows, cols) after axis merging, every leaf with column stride 1 or 0 (flat arrays
 // are one row).  Registers 0 .. n_leaf-1 hold the leaves when the program starts, registers
-// NREG-1, NREG-2, ... the immediates.
+// NREG-1, NREG-2, ... the immediates.  Beside the one-rule functors an instruction may hold two
+// rules (a * b + c and its kin: what an interpreted instruction costs is operand moves and dispatch,
+// not arithmetic), select by index range (the scattered cotangent of a slice), or sum its operand
+// over the row (the ROWS variant: programs whose rows fit one wave's tile).
+//
+// The interpreter runs whatever it is handed, at once.  A program that keeps coming back is
+// compiled into a kernel of its own (specialize.hip), which takes the same argument block.
 #include <algorithm>
 #include <type_traits>
 
