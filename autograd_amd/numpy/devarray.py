@@ -877,6 +877,7 @@ def ones(shape, dtype=_F64):
 
 
 _CONSTANTS = {}
+_CONSTANT_VIEWS = {}
 KNOWN_SCALARS = {}  # data pointer of a one-element array that is never written -> its value (shared zeros / ones / constants)
 
 
@@ -893,13 +894,21 @@ def constant(shape, value, dtype):
     if dtype not in _FLOATS or n == 0 or not shape:
         return full(shape, value, dtype)
     key = (dtype, float(value))
+    seen = _CONSTANT_VIEWS.get((key, shape))
+    if seen is not None:
+        return LazyDevArray(seen, dtype, 1.0, None)
     one = _CONSTANTS.get(key)
     if one is None:
         if len(_CONSTANTS) > 64:
             return full(shape, value, dtype)
         one = _CONSTANTS[key] = full((), float(value), dtype)._t
         KNOWN_SCALARS[one.data_ptr()] = float(value)
-    return LazyDevArray(one.expand(shape), dtype, 1.0, None)
+    if len(_CONSTANT_VIEWS) >= 1024:
+        _CONSTANT_VIEWS.clear()
+    # (the view of the shared element is shared as well: nothing ever writes through it, and a loop that makes the same
+    # column of ones at every step saves the view's few microseconds each time)
+    seen = _CONSTANT_VIEWS[(key, shape)] = one.expand(shape)
+    return LazyDevArray(seen, dtype, 1.0, None)
 
 
 # --------------------------------------------------------------------------------------------
