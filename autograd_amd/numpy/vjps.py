@@ -412,10 +412,21 @@ def repeat_to_match_shape(g, shape, dtype, axis, keepdims):
         return g, 1
     axes = D.normalize_axes(axis, len(shape))
     new_shape = tuple(1 if d in axes else s for d, s in enumerate(shape))
-    num_reps = onp.prod(onp.array(shape)[list(axes)])
+    reps = 1
+    for d in axes:
+        reps *= shape[d]
+    num_reps = onp.int64(reps)  # (what onp.prod(onp.array(shape)[axes]) gives, without three NumPy calls)
     if BatchMode.active:  # cotangents stacked along a leading axis: it is carried along
         n = anp.shape(g)[0]
         new_shape, shape = (n,) + new_shape, (n,) + shape
+    elif type(g) is DevArray and (g.dtype == dtype or g.dtype == _F64):
+        # the seed of `grad` (a shared one) or any other shared constant: the constant seen through the operand's
+        # shape is a kept view (no tensor views are made for the commonest cotangent of a loss's final sum)
+        t = g._t
+        if t.numel() == 1:
+            c = D.KNOWN_SCALARS.get(t.data_ptr())
+            if c is not None:
+                return D.constant(shape, c, g.dtype), num_reps
     if isinstance(g, DevArray) and (g.dtype == dtype or g.dtype == _F64):
         # a concrete cotangent that needs no promotion: the view itself, without the two primitive calls
         return g._view(lambda t: t.reshape(new_shape).expand(shape)), num_reps
