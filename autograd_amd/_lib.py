@@ -517,7 +517,7 @@ def elementwise(op, code, shape, outs, ins):
 PROGRAM_MAX_LEAVES, PROGRAM_MAX_IMMEDIATES, PROGRAM_MAX_OUTPUTS, PROGRAM_MAX_INSTRUCTIONS = 6, 6, 4, 96
 PROGRAM_MAX_REGISTERS = 16
 PROGRAM_MAX_MASKS = 4
-PROGRAM_STORE, PROGRAM_MASK, PROGRAM_ROWSUM = 255, 254, 253
+PROGRAM_STORE, PROGRAM_MASK, PROGRAM_ROWSUM, PROGRAM_ROWLSE = 255, 254, 253, 252
 _prog_leaf_ranges = (ctypes.c_int64 * (2 * PROGRAM_MAX_LEAVES))()
 _prog_mask_ranges = (ctypes.c_int64 * (2 * PROGRAM_MAX_MASKS))()
 _prog_outs = (AgmiArray * PROGRAM_MAX_OUTPUTS)()

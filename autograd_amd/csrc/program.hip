@@ -272,27 +272,13 @@ __global__ __launch_bounds__(kBlock) void ew_program(const ProgParams p) {
             }                                                                                             \
         break;                                                                                            \
     }                                                                                                     \
-    case AGMI_PROGRAM_ROWSUM: {                                                                           \
+    case AGMI_PROGRAM_ROWSUM:                                                                             \
+    case AGMI_PROGRAM_ROWLSE: {                                                                           \
         if constexpr (ROWS) {                                                                             \
-            /* the order of red_row_group: lane g of G adds up columns g, g + G, ... from zero, then the  \
-               lanes' sums meet in a butterfly; lane 0 holds what that kernel stores */                   \
-            T *mine = row_values[threadIdx.x >> 6];                                                       \
-            _Pragma("unroll") for (int u = 0; u < U; ++u) {                                               \
-                vec_t v;                                                                                  \
-                _Pragma("unroll") for (int j = 0; j < VL; ++j) v[j] = x[0][u * VL + j];                   \
-                *reinterpret_cast<vec_t *>(mine + u * (64 * VL) + lane * VL) = v;                         \
-            }                                                                                             \
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");                                        \
-            __builtin_amdgcn_wave_barrier();                                                              \
-            const int G = p.row_group;                                                                    \
-            T acc = T(0);                                                                                 \
-            if (static_cast<int>(lane) < G)                                                               \
-                for (int64_t rr = lane; rr < cols; rr += G) acc = acc + mine[rr];                         \
-            for (int m = G >> 1; m > 0; m >>= 1) acc = acc + __shfl_xor(acc, m, 64);                      \
-            acc = __shfl(acc, 0, 64);                                                                     \
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");                                        \
-            __builtin_amdgcn_wave_barrier();                                                              \
-            _Pragma("unroll") for (int j = 0; j < V; ++j) o[j] = acc;                                     \
+            const T total = op == AGMI_PROGRAM_ROWSUM                                                     \
+                ? program_row_reduce<AccSum<T>, T, VL, U>(row_values[threadIdx.x >> 6], lane, cols, p.row_group, x[0]) \
+                : program_row_reduce<AccLse<T>, T, VL, U>(row_values[threadIdx.x >> 6], lane, cols, p.row_group, x[0]); \
+            _Pragma("unroll") for (int j = 0; j < V; ++j) o[j] = total;                                   \
         } else {                                                                                          \
             _Pragma("unroll") for (int j = 0; j < V; ++j) o[j] = x[0][j];                                 \
         }                                                                                                 \
@@ -453,7 +439,7 @@ extern "C" int agmi_program(int dtype, int ndim, const int64_t *shape, int n_out
             defined |= 1u << dst;
             continue;
         }
-        if (op == AGMI_PROGRAM_ROWSUM) {
+        if (op == AGMI_PROGRAM_ROWSUM || op == AGMI_PROGRAM_ROWLSE) {
             if (src[0] >= nreg || !(defined >> src[0] & 1u) || dst >= nreg) {
                 set_error("program: instruction %d sums register %d, which holds nothing, or writes register %d of %d", i,
                           src[0], dst, nreg);

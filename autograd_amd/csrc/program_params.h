@@ -44,4 +44,31 @@ static __device__ __noinline__ void store_partial(T *base, int64_t c, int64_t co
         if (c + j < cols) base[c + j] = v[j];
 }
 
+// The reduction of a program register over a row that one wave holds (AGMI_PROGRAM_ROWSUM, AGMI_PROGRAM_ROWLSE), in
+// the order of the reduction kernel red_row_group for a row of that length: the wave writes the row to its stretch of
+// LDS, lane g of the first G adds up (combines) columns g, g + G, ... starting from the identity, the G partial results
+// meet in a butterfly, and lane 0 holds what that kernel would store; every lane gets it.  Bit for bit the reduction
+// kernel's result, so a value does not depend on whether a chain formed it inside or read it from memory.
+template <class Acc, typename T, int VL, int U>
+__device__ __forceinline__ T program_row_reduce(T *mine, uint32_t lane, int64_t cols, int G, const T (&v)[VL * U]) {
+    typedef T vec_t __attribute__((ext_vector_type(VL), aligned(sizeof(T))));
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        vec_t w;
+#pragma unroll
+        for (int j = 0; j < VL; ++j) w[j] = v[u * VL + j];
+        *reinterpret_cast<vec_t *>(mine + u * (64 * VL) + lane * VL) = w;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    typename Acc::type acc = Acc::identity();
+    if (static_cast<int>(lane) < G)
+        for (int64_t rr = lane; rr < cols; rr += G) acc = Acc::combine(acc, Acc::lift(mine[rr]));
+    for (int m = G >> 1; m > 0; m >>= 1) acc = Acc::combine(acc, Acc::shfl_xor(acc, m));
+    const T total = __shfl(Acc::finish(acc), 0, 64);
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    return total;
+}
+
 }  // namespace agmi

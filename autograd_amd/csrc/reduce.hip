@@ -23,63 +23,7 @@
 
 namespace agmi {
 
-// ---- accumulators ----------------------------------------------------------------------
-template <typename T>
-struct AccSum {
-    typedef T type;
-    __device__ __forceinline__ static T identity() { return T(0); }
-    __device__ __forceinline__ static T lift(T v) { return v; }
-    __device__ __forceinline__ static T combine(T a, T b) { return a + b; }
-    __device__ __forceinline__ static T finish(T a) { return a; }
-    __device__ __forceinline__ static T shfl_xor(T a, int m) { return __shfl_xor(a, m, 64); }
-};
-template <typename T>
-struct AccProd : AccSum<T> {
-    __device__ __forceinline__ static T identity() { return T(1); }
-    __device__ __forceinline__ static T combine(T a, T b) { return a * b; }
-};
-template <typename T>
-struct AccMax : AccSum<T> {
-    __device__ __forceinline__ static T identity() { return -INFINITY; }
-    __device__ __forceinline__ static T combine(T a, T b) { return max_nan(a, b); }
-};
-template <typename T>
-struct AccMin : AccSum<T> {
-    __device__ __forceinline__ static T identity() { return INFINITY; }
-    __device__ __forceinline__ static T combine(T a, T b) { return min_nan(a, b); }
-};
-
-// log-sum-exp as an associative reduction over (m, s) with value = m + log(s),
-// s = sum exp(x - m).  Infinite and equal maxima are combined without forming inf - inf.
-template <typename T>
-struct LsePair {
-    T m, s;
-};
-template <typename T>
-struct AccLse {
-    typedef LsePair<T> type;
-    __device__ __forceinline__ static type identity() { return {T(-INFINITY), T(0)}; }
-    __device__ __forceinline__ static type lift(T v) { return {v, T(1)}; }
-    // value: the larger maximum, and its sum plus the other sum scaled by exp(difference of the maxima).  Written
-    // with selects and one exp, not one branch per case: lanes of a wave disagree on which side is larger, and with
-    // branches every step of a wave-wide reduction runs both exps one after the other.  Equal maxima (also both
-    // infinite) scale by exp(0) = 1 exactly; a NaN maximum gives NaN for both members.
-    __device__ __forceinline__ static type combine(type a, type b) {
-        const bool a_larger = a.m >= b.m;
-        const T hi_m = a_larger ? a.m : b.m, lo_m = a_larger ? b.m : a.m;
-        const T hi_s = a_larger ? a.s : b.s, lo_s = a_larger ? b.s : a.s;
-        const T d = (a.m == b.m) ? T(0) : lo_m - hi_m;
-        const bool ordered = a.m == a.m && b.m == b.m;
-        return {ordered ? hi_m : a.m + b.m, ordered ? hi_s + lo_s * m_exp(d) : a.s + b.s};
-    }
-    __device__ __forceinline__ static T finish(type a) {
-        if (a.s == T(0) || a.m == T(INFINITY)) return a.m;  // all -inf, or a +inf present
-        return a.m + m_log(a.s);
-    }
-    __device__ __forceinline__ static type shfl_xor(type a, int m) {
-        return {__shfl_xor(a.m, m, 64), __shfl_xor(a.s, m, 64)};
-    }
-};
+// (the accumulators AccSum ... AccLse live in functors.h: the program kernels reduce rows with them too)
 
 struct RedParams {
     void *out;  // T* when final, Acc* (chunk-major) when partial

@@ -146,19 +146,10 @@ static std::string spec_source(bool f32, int nreg, const ProgParams &p, const st
               << "                    const int64_t cc = c0 + u * (64 * VL) + j;\n"
               << "                    o_[u * VL + j] = (cc >= lo && cc < hi) ? r" << src[0] << "[u * VL + j] : r" << src[2]
               << "[u * VL + j];\n                }\n";
-        } else if (op == AGMI_PROGRAM_ROWSUM) {
-            // the order of red_row_group (see the interpreter's case)
-            o << "            T *mine = row_values[threadIdx.x >> 6];\n"
-              << "            _Pragma(\"unroll\") for (int u = 0; u < U; ++u) {\n                vec_t v;\n"
-              << "                _Pragma(\"unroll\") for (int j = 0; j < VL; ++j) v[j] = r" << src[0] << "[u * VL + j];\n"
-              << "                *reinterpret_cast<vec_t *>(mine + u * (64 * VL) + lane * VL) = v;\n            }\n"
-              << "            __builtin_amdgcn_fence(__ATOMIC_RELEASE, \"wavefront\");\n            __builtin_amdgcn_wave_barrier();\n"
-              << "            const int G = p.row_group;\n            T acc = T(0);\n"
-              << "            if (static_cast<int>(lane) < G)\n                for (int64_t rr = lane; rr < cols; rr += G) acc = acc + mine[rr];\n"
-              << "            for (int m = G >> 1; m > 0; m >>= 1) acc = acc + __shfl_xor(acc, m, 64);\n"
-              << "            acc = __shfl(acc, 0, 64);\n"
-              << "            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, \"wavefront\");\n            __builtin_amdgcn_wave_barrier();\n"
-              << "            _Pragma(\"unroll\") for (int j = 0; j < V; ++j) o_[j] = acc;\n";
+        } else if (op == AGMI_PROGRAM_ROWSUM || op == AGMI_PROGRAM_ROWLSE) {
+            o << "            const T total = program_row_reduce<" << (op == AGMI_PROGRAM_ROWSUM ? "AccSum" : "AccLse")
+              << "<T>, T, VL, U>(row_values[threadIdx.x >> 6], lane, cols, p.row_group, r" << src[0] << ");\n"
+              << "            _Pragma(\"unroll\") for (int j = 0; j < V; ++j) o_[j] = total;\n";
         } else {
             const char *fn = functor_name(op);
             const int arity = functor_arity(op);
@@ -320,7 +311,8 @@ extern "C" long long agmi_program_source(int dtype, int n_leaf, int n_imm, int n
     p.row_group = row_sums ? 1 : 0;
     for (int i = 0; i < n_instr; ++i) {
         const int op = code[i] & 0xff;
-        if (op != AGMI_PROGRAM_STORE && op != AGMI_PROGRAM_MASK && op != AGMI_PROGRAM_ROWSUM && !functor_name(op)) {
+        if (op != AGMI_PROGRAM_STORE && op != AGMI_PROGRAM_MASK && op != AGMI_PROGRAM_ROWSUM && op != AGMI_PROGRAM_ROWLSE &&
+            !functor_name(op)) {
             set_error("program_source: instruction %d has unknown op %d", i, op);
             return AGMI_ERR_ARG;
         }

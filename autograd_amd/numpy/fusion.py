@@ -56,7 +56,8 @@ for _name in "LSE_VJP CHOOSE_VJP EXTREMUM_VJP".split():
 
 # pseudo-op of a program: the sum of its operand over each row of a two-axis index space, at every index of the row
 ROWSUM = _lib.PROGRAM_ROWSUM
-ARITY[ROWSUM] = 1
+ROWLSE = _lib.PROGRAM_ROWLSE  # the same for the logsumexp of a row
+ARITY[ROWSUM] = ARITY[ROWLSE] = 1
 _CHAINED_INTO_MUL = {Op.MUL: Op.MUL_MUL, Op.ADD: Op.ADD_MUL, Op.SUB: Op.SUB_MUL}
 CHAINED = os.environ.get("AUTOGRAD_AMD_FUSE_CHAINED", "1").strip() not in ("0", "")  # (off: for measurements)
 ROWSUM_WIDEST = {onp.dtype("float32"): 512, onp.dtype("float64"): 256}  # one wave's tile of the program kernel
@@ -225,6 +226,16 @@ def make(op, dtype, xs):
     return ExprArray(op, tuple(args), shape, dtype, cone)
 
 
+def rows_fit_a_wave(shape, dtype):
+    """Whether a reduction over the rows of ``shape`` can be formed inside a program: two axes, a row within one wave's
+    tile of the program kernel, and a shape whose rows the reduction kernel gives to a group of lanes (the order of
+    additions the program follows)."""
+    if len(shape) != 2 or dtype not in ROWSUM_WIDEST:
+        return False
+    rows, cols = shape
+    return 2 <= cols <= ROWSUM_WIDEST[dtype] and (cols <= 64 or rows >= 64)
+
+
 def _row_sums(x, shape, dtype):
     """Row sums that have not run (``x``: a pending ``sum(e, axis=1, keepdims=True)``, the unbroadcast of a cotangent)
     about to be broadcast back over the rows they came from: a node of the full shape that the program kernel forms
@@ -232,16 +243,18 @@ def _row_sums(x, shape, dtype):
     reduction plus a program).  Only for the shapes whose rows the reduction kernel gives to a group of lanes: the
     program adds in that kernel's order, so the value does not depend on which of the two ran.  None otherwise."""
     op, red, rdtype, xs, axes, _keepdims, full = x._call
-    if red != Red.SUM or (op != Op.COPY and op != Op.NEG) or len(xs) != 1 or rdtype != dtype or len(shape) != 2:
+    if len(xs) != 1 or rdtype != dtype or len(shape) != 2:
+        return None
+    if not (red == Red.SUM and (op == Op.COPY or op == Op.NEG)) and not (red == Red.LOGSUMEXP and op == Op.COPY):
         return None
     src = xs[0]
     rows, cols = shape
     if not isinstance(src, DevArray) or src.shape != shape or src.dtype != dtype or x.shape != (rows, 1) \
             or tuple(axes) not in ((1,), (-1,)) or (full is not None and tuple(full) != shape):
         return None
-    if cols < 2 or cols > ROWSUM_WIDEST[dtype] or (cols > 64 and rows < 64):
+    if not rows_fit_a_wave(shape, dtype):
         return None
-    node = ExprArray(ROWSUM, (src,), shape, dtype, 1 + (src._cone if pending(src) else 0))
+    node = ExprArray(ROWSUM if red == Red.SUM else ROWLSE, (src,), shape, dtype, 1 + (src._cone if pending(src) else 0))
     if op == Op.NEG:
         node = ExprArray(Op.NEG, (node,), shape, dtype, node._cone + 1)
     return node
@@ -407,8 +420,8 @@ def _single(node):
     if node._op == SHIFT:
         _single_shift(node)
         return
-    if node._op == ROWSUM:
-        sums = D._map_reduce_now(Op.COPY, Red.SUM, dtype, (node._args[0],), (1,), True)
+    if node._op == ROWSUM or node._op == ROWLSE:
+        sums = D._map_reduce_now(Op.COPY, Red.SUM if node._op == ROWSUM else Red.LOGSUMEXP, dtype, (node._args[0],), (1,), True)
         _lib.elementwise(Op.COPY, _lib.DTYPE_CODE[dtype], node._shape, (node._buffer(),), (D._expand(sums._t, node._shape),))
         COUNTS["single"] += 1
         _finish(node)
@@ -968,7 +981,7 @@ def added_into(A, start, x, take):
 
 def builtins_any_rowsum(instrs):
     for instr in instrs:
-        if instr[0] == ROWSUM:
+        if instr[0] == ROWSUM or instr[0] == ROWLSE:
             return True
     return False
 

@@ -14,6 +14,7 @@ from .._lib import Op, Red
 from ..core import BatchMode, batch_safe
 from ..extend import defjvp, defvjp, primitive
 from ..numpy import devarray as D
+from ..numpy import fusion
 from ..numpy import wrapper as np
 from ..numpy.vjps import _concrete, repeat_to_match_shape
 
@@ -23,7 +24,14 @@ def logsumexp(x, axis=None, b=1.0, keepdims=False):
     x = D.asarray(x)
     axes = D.normalize_axes(axis, x.ndim)
     if (type(b) is float or isinstance(b, numbers.Number)) and b == 1.0:
-        return D.map_reduce(Op.COPY, Red.LOGSUMEXP, D._float_dtype(x.dtype), (x,), axes, keepdims)
+        dt = D._float_dtype(x.dtype)
+        if keepdims and axes == (1,) and x.dtype == dt and fusion.ENABLED and fusion.rows_fit_a_wave(x.shape, dt):
+            # The log-softmax of a layer's rows (reference examples/rnn.py:50-52, examples/neural_net.py:24-28:
+            # x - logsumexp(x, axis=1, keepdims=True)): the value is only ever read back by the chains around it, the
+            # subtraction and the rule g * exp(x - ans), and a program forms the logsumexp of a short row itself
+            # (bit for bit the reduction kernel's value).  So nothing runs here; a reader of the value itself runs it.
+            return D.PendingReduce((Op.COPY, Red.LOGSUMEXP, dt, (D._kept(x),), axes, True, None), (x.shape[0], 1), dt)
+        return D.map_reduce(Op.COPY, Red.LOGSUMEXP, dt, (x,), axes, keepdims)
     # weighted form, the way scipy evaluates it: m = max(x), log(sum(b * exp(x - m))) + m, with weights of either
     # sign (a negative total gives NaN, as there).  Two passes over x: the maximum, then the weighted sum
     # fused into its reduction.

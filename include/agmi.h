@@ -222,7 +222,9 @@ int agmi_elementwise(int op, int dtype, int ndim, const int64_t *shape,
  * agmi_map_reduce adds a row of that length (bit for bit its result).  A program that holds one runs on
  * `shape` as given: exactly two axes, the second at most 512 (float32) / 256 (float64) long and,
  * beyond 64, at least 64 rows (the shapes for which agmi_map_reduce gives a row to a group of lanes);
- * n_regs must be 16, no leaf ranges and no masks; else AGMI_ERR_UNSUPPORTED.
+ * n_regs must be 16, no leaf ranges and no masks; else AGMI_ERR_UNSUPPORTED.  AGMI_PROGRAM_ROWLSE is the
+ * same for the logsumexp of a row (autograd/scipy/special.py:119-147: the log-softmax x - logsumexp(x) and its
+ * rule g * exp(x - logsumexp(x)) then need no reduction launch of their own), again in agmi_map_reduce's order.
  * Layout: after axis merging at most two axes may remain and every operand must have stride 1 or
  * 0 (leaves only) along the innermost one; anything else returns AGMI_ERR_UNSUPPORTED.  Outputs
  * may not overlap leaves unless they are the same view (in-place update).
@@ -238,6 +240,7 @@ int agmi_elementwise(int op, int dtype, int ndim, const int64_t *shape,
 #define AGMI_PROGRAM_STORE 255
 #define AGMI_PROGRAM_MASK 254
 #define AGMI_PROGRAM_ROWSUM 253
+#define AGMI_PROGRAM_ROWLSE 252
 int agmi_program(int dtype, int ndim, const int64_t *shape, int n_out, const agmi_array *outs,
                  int n_leaf, const agmi_array *leaves, const int64_t *leaf_ranges,
                  int n_imm, const double *imms, int n_mask, const int64_t *mask_ranges,

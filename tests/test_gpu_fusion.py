@@ -565,6 +565,56 @@ def test_log_softmax_gradient_is_the_same_with_row_sums_inside_the_chain(dnp):
         assert onp.allclose(fused, soft - t, rtol=0, atol=2e-6 if dtype == F32 else 1e-14)
 
 
+@pytest.mark.parametrize("dtype", [F32, F64])
+@pytest.mark.parametrize("shape", ROW_SUM_SHAPES)
+def test_the_logsumexp_of_short_rows_is_formed_by_the_chain_that_reads_it(dtype, shape, dnp):
+    """``x - logsumexp(x, axis=1, keepdims=True)`` (reference examples/rnn.py:50-52, examples/neural_net.py:24-28 over
+    autograd/scipy/special.py:119-147): for rows that fit a wave's tile nothing runs when the logsumexp is taken; the
+    log-softmax is one program that forms it (in the reduction kernel's order: the same bits as the separate
+    reduction, infinities, NaNs and all -inf rows included), and a reader of the value itself gets the reduction's."""
+    from autograd_amd import _lib
+    from autograd_amd.numpy import fusion
+    from autograd_amd.scipy.special import logsumexp
+
+    rows, cols = shape
+    if dtype == F64 and cols > 256:
+        pytest.skip("wider than a float64 tile: covered by the float32 case of the same width")
+    rs = onp.random.RandomState(rows + 7 * cols)
+    x = (rs.randn(*shape) * 4).astype(dtype)
+    x[0, 0] = onp.inf
+    if rows > 2:
+        x[1, :] = -onp.inf
+        x[2, cols - 1] = onp.nan
+    if rows > 4:
+        x[3, 0], x[3, 1] = 700.0, -700.0
+        x[4, :] = 3.25
+    X = dnp.asarray(x)
+    reduced = []
+    real = _lib.map_reduce
+    _lib.map_reduce = lambda *args, **k: (reduced.append(args[1]), real(*args, **k))[1]
+    try:
+        inside = fusion.rows_fit_a_wave(shape, dtype)
+        lse = logsumexp(X, axis=1, keepdims=True)
+        assert (reduced == []) == inside
+        got = (X - lse).numpy()
+        assert (reduced == []) == inside            # the chain formed it: still no reduction launched
+        value = lse.numpy()                         # a reader of the value itself
+        assert len(reduced) == 1
+    finally:
+        _lib.map_reduce = real
+    with unfused():
+        want_value = logsumexp(X, axis=1, keepdims=True).numpy()
+        want = (X - logsumexp(X, axis=1, keepdims=True)).numpy()
+    assert _same_bits(value, want_value) and _same_bits(got, want)
+    from scipy.special import logsumexp as host_lse
+
+    with onp.errstate(all="ignore"):
+        ref = host_lse(x.astype(F64), axis=1, keepdims=True)
+    ok = onp.isfinite(ref[:, 0])
+    assert onp.allclose(value[ok], ref[ok], rtol=2e-6 if dtype == F32 else 1e-13)
+    assert onp.array_equal(onp.isnan(value), onp.isnan(ref)) and onp.array_equal(onp.isinf(value), onp.isinf(ref))
+
+
 def test_a_row_sum_outside_the_kernels_shapes_is_refused_at_the_library():
     from autograd_amd import _lib
     from autograd_amd._lib import Op
