@@ -9,7 +9,9 @@
  * Conventions
  *  - Every pointer named "device" is GPU memory owned by the caller.  The library never
  *    allocates, frees or synchronises; work is enqueued on `stream` (a hipStream_t passed
- *    as void*, NULL = the default stream) and the call returns immediately.
+ *    as void*, NULL = the default stream) and the call returns immediately.  (One exception,
+ *    which agmi_program_specialize(0) switches off: agmi_program compiles a program that it
+ *    is handed for the third time and loads the code object; see there.)
  *  - Strides are in ELEMENTS, may be 0 (broadcast axis) and may be negative.
  *  - Return value: 0 on success; AGMI_ERR_* (negative) for a rejected argument, in which
  *    case nothing was launched; a positive value is a hipError_t from the launch.
