@@ -437,6 +437,40 @@ def test_a_specialised_kernel_gives_the_interpreters_bits(dtype, dnp):
         assert _same_bits(compiled, interpreted) and _same_bits(again, interpreted) and _same_bits(interpreted, plain)
 
 
+@pytest.mark.parametrize("dtype", [F64, F32])
+def test_a_specialised_kernel_treats_special_values_as_the_interpreter_does(dtype, dnp):
+    """Infinities, NaNs, signed zeros, subnormals and values at the edge of overflow through the long functors and the
+    two-rule instructions: interpreted, compiled and rule by rule give the same bits (the compiled kernel is built with
+    the library's floating-point flags: no contraction, no flushing of subnormals, no packed float32 forms)."""
+    from autograd_amd.numpy import fusion
+
+    tiny = onp.finfo(dtype).tiny
+    big = onp.finfo(dtype).max
+    special = onp.array([0.0, -0.0, onp.inf, -onp.inf, onp.nan, tiny, -tiny, tiny / 8, -tiny / 16, big, -big, big / 3, 1.0, -1.0,
+                         88.7, -87.3, 709.7, -745.1, 1e-30, 3.0e38, 0.5, 2.0], dtype=dtype)
+    a = onp.repeat(special, len(special))
+    b = onp.tile(special, len(special))
+    A, B = dnp.asarray(a), dnp.asarray(b)
+    chains = [
+        lambda: dnp.exp(A) * B - dnp.tanh(B) / (A + B),
+        lambda: dnp.sqrt(dnp.abs(A)) * B + dnp.log(dnp.abs(B) + dnp.abs(A)),
+        lambda: (A * B) * A - (A - B) * B + (A + B) * (B - A * A),
+        lambda: dnp.maximum(A, B) / dnp.minimum(A, B) + dnp.where(A > B, A, B) * 0.5,
+        lambda: dnp.power(dnp.abs(A), 0.3) * dnp.sin(B) + dnp.arctan2(A, B) - dnp.log1p(dnp.abs(B)) * dnp.expm1(A * 1e-3),
+    ]
+    for k, f in enumerate(chains):
+        with onp.errstate(all="ignore"):
+            with specializing(0):
+                fusion._PROGRAMS.clear()
+                interpreted = f().numpy()
+            with specializing(1):
+                compiled = f().numpy()
+            with unfused():
+                plain = f().numpy()
+        assert _same_bits(compiled, interpreted), k
+        assert _same_bits(interpreted, plain), k
+
+
 def test_programs_are_specialised_after_a_few_sightings_and_never_while_a_graph_records(dnp):
     import autograd_amd as ag
     from autograd_amd import _lib, graphs
