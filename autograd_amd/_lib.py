@@ -117,7 +117,9 @@ class AgmiCorrelation(ctypes.Structure):
 
 class AgmiGemmEpilogue(ctypes.Structure):
     _fields_ = [("kind", ctypes.c_int32), ("bias", ctypes.c_void_p), ("out", ctypes.c_void_p), ("out_ld", ctypes.c_int64),
-                ("x", ctypes.c_void_p), ("x_ld", ctypes.c_int64), ("beta", ctypes.c_double)]
+                ("x", ctypes.c_void_p), ("x_ld", ctypes.c_int64), ("beta", ctypes.c_double),
+                ("a2", ctypes.c_void_p), ("a2_rs", ctypes.c_int64), ("a2_cs", ctypes.c_int64),
+                ("b2", ctypes.c_void_p), ("b2_rs", ctypes.c_int64), ("b2_cs", ctypes.c_int64), ("k2", ctypes.c_int64)]
 
 
 class AgmiLseCotangent(ctypes.Structure):
@@ -732,11 +734,13 @@ EPILOGUE_BIAS_TANH, EPILOGUE_TANH_VJP = 1, 2
 _epilogue = AgmiGemmEpilogue()
 
 
-def gemm_fused(code, A, B, C, kind, bias=None, out=None, x=None, beta=0.0):
+def gemm_fused(code, A, B, C, kind, bias=None, out=None, x=None, beta=0.0, second=None):
     """``agmi_gemm_fused``: ``A @ B`` (2-d tensors, any strides; plus ``beta`` times what ``C`` holds) into the
     contiguous ``C`` with a dense layer's epilogue: ``out = tanh(C + bias)`` beside it, or
-    ``C = (A @ B + beta * C) / cosh(x + bias)**2`` (``bias``: contiguous vector or None).  Returns False when the
-    operands are outside what the fused kernel covers."""
+    ``C = (A @ B + beta * C) / cosh(x + bias)**2`` (``bias``: contiguous vector or None).  ``second``: a pair
+    ``(A2, B2)`` whose product is added before the tanh rule, in the same launch (bit for bit what running ``A @ B``
+    into ``C`` and then ``A2 @ B2`` with ``beta = 1`` gives).  Returns False when the operands are outside what the
+    fused kernel covers."""
     M, K = A.shape
     N = B.shape[1]
     e = _epilogue
@@ -745,6 +749,16 @@ def gemm_fused(code, A, B, C, kind, bias=None, out=None, x=None, beta=0.0):
     e.out, e.out_ld = (out.data_ptr(), out.stride(0)) if out is not None else (None, 0)
     e.x, e.x_ld = (x.data_ptr(), x.stride(0)) if x is not None else (None, 0)
     e.beta = beta
+    flops = 2.0 * M * N * K
+    if second is None:
+        e.a2 = e.b2 = None
+        e.k2 = 0
+    else:
+        A2, B2 = second
+        e.a2, e.a2_rs, e.a2_cs = A2.data_ptr(), A2.stride(0), A2.stride(1)
+        e.b2, e.b2_rs, e.b2_cs = B2.data_ptr(), B2.stride(0), B2.stride(1)
+        e.k2 = A2.shape[1]
+        flops += 2.0 * M * N * A2.shape[1]
     ev = _TIMER.begin(("gemm",)) if _TIMER is not None else None
     rc = _LIB.agmi_gemm_fused(code, M, N, K, A.data_ptr(), A.stride(0), A.stride(1), B.data_ptr(), B.stride(0), B.stride(1),
                               C.data_ptr(), C.stride(0), ctypes.byref(e), _workspace().data_ptr(), _WORKSPACE_BYTES, _stream())
@@ -754,7 +768,8 @@ def gemm_fused(code, A, B, C, kind, bias=None, out=None, x=None, beta=0.0):
         _check(rc, "agmi_gemm_fused")
     if ev is not None:
         es = A.element_size()
-        _TIMER.end(ev, ("gemm",), (M * K + K * N + 2 * M * N) * es, 2.0 * M * N * K)
+        k_all = K + (second[0].shape[1] if second is not None else 0)
+        _TIMER.end(ev, ("gemm",), (M * k_all + k_all * N + 2 * M * N) * es, flops)
     return True
 
 

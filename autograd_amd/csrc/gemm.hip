@@ -88,6 +88,11 @@ struct GemmParams {
     // gemm_direct only: bytes from element (0, 0) of one matrix of the batch to one past its last
     // element (the extent of the buffer descriptor the loads are range-checked against)
     uint32_t a_span_bytes, b_span_bytes;
+    // gemm_block_split only: a second product A2 . B2 (M x K2, K2 x N; no batch) added to the first before the epilogue
+    const void *A2, *B2;
+    int64_t K2, a2_rs, a2_cs, b2_rs, b2_cs, k_per_split2;
+    int splits2;
+    uint32_t a2_span_bytes, b2_span_bytes;
     // epilogue of the float32 direct kernel and of the split finish (agmi_gemm_fused):
     //   1: beside C, epi_out[m, n] = tanh(C[m, n] + epi_bias[n])
     //   2: C[m, n] = acc / cosh(epi_x[m, n] + epi_bias[n])**2 (the product itself is not stored)
@@ -784,7 +789,7 @@ template <bool KCA, bool KCB>
 __global__ __launch_bounds__(kSmallMaxWaves * 64) void gemm_block_split(const GemmParams p) {
     extern __shared__ float part_lds[];  // [waves][32 * 32]
     float (*part)[kSmallTile * kSmallTile] = reinterpret_cast<float (*)[kSmallTile * kSmallTile]>(part_lds);
-    const int tid = threadIdx.x, lane = tid & 63, n_waves = blockDim.x >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // the same for the whole wave: offsets made of it are scalar
     const int r = lane & 31, h = lane >> 5;
     // Workgroups go to the 8 XCDs in turn and each XCD has an L2 of its own: XCD x takes a contiguous range of the
@@ -795,54 +800,65 @@ __global__ __launch_bounds__(kSmallMaxWaves * 64) void gemm_block_split(const Ge
     const int64_t tile = xcd * (n_tiles / kXcds) + min(xcd, n_tiles % kXcds) + turn;
     const int64_t tile_m = tile % p.tiles_m, tile_n = tile / p.tiles_m, batch = blockIdx.y;
     const int64_t m0 = tile_m * kSmallTile, n0 = tile_n * kSmallTile;
-    // (the host admits only operands that span less than 2 GiB with non-negative strides: offsets fit 32 bits)
-    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<float *>(static_cast<const float *>(p.A) + batch * p.a_bs), 0, p.a_span_bytes, 0x00020000);
-    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<float *>(static_cast<const float *>(p.B) + batch * p.b_bs), 0, p.b_span_bytes, 0x00020000);
-    // rows / columns past the edge read the last one: their products land in elements that are never stored
-    const uint32_t a_lane = static_cast<uint32_t>((min(m0 + r, p.M - 1) * p.a_rs + 4 * h * p.a_cs) * 4);
-    const uint32_t b_lane = static_cast<uint32_t>((min(n0 + r, p.N - 1) * p.b_cs + 4 * h * p.b_rs) * 4);
-    const float *a_row = static_cast<const float *>(p.A) + batch * p.a_bs + min(m0 + r, p.M - 1) * p.a_rs;
-    const float *b_col = static_cast<const float *>(p.B) + batch * p.b_bs + min(n0 + r, p.N - 1) * p.b_cs;
-    const int64_t kbeg = wave * p.k_per_split, kend = min(p.K, kbeg + p.k_per_split);
+    // One product's share of this wave: the K slice [wave * k_per_split, ...) of A . B into `slot` of the LDS array.
+    const auto contract = [&](const float *A, const float *B, int64_t a_rs, int64_t a_cs, int64_t b_rs, int64_t b_cs, int64_t K,
+                              int64_t k_per_split, uint32_t a_span_bytes, uint32_t b_span_bytes,
+                              float *slot) __attribute__((always_inline)) {
+        // (the host admits only operands that span less than 2 GiB with non-negative strides: offsets fit 32 bits)
+        const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(A), 0, a_span_bytes, 0x00020000);
+        const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(B), 0, b_span_bytes, 0x00020000);
+        // rows / columns past the edge read the last one: their products land in elements that are never stored
+        const uint32_t a_lane = static_cast<uint32_t>((min(m0 + r, p.M - 1) * a_rs + 4 * h * a_cs) * 4);
+        const uint32_t b_lane = static_cast<uint32_t>((min(n0 + r, p.N - 1) * b_cs + 4 * h * b_rs) * 4);
+        const float *a_row = A + min(m0 + r, p.M - 1) * a_rs;
+        const float *b_col = B + min(n0 + r, p.N - 1) * b_cs;
+        const int64_t kbeg = wave * k_per_split, kend = min(K, kbeg + k_per_split);
 
-    v16f acc;
+        v16f acc;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) acc[v] = 0.f;
-    float a0[16], b0[16], a1[16], b1[16];
-    const auto load = [&](int64_t kc, float (&a)[16], float (&b)[16]) __attribute__((always_inline)) {
-        if (kc + kSmallChunk <= kend) {  // the same for the whole wave
-            if (KCA) small_load_k(a_row, kc, h, a);
-            else small_load_x<false>(rsrc_a, a_lane, p.a_cs, kc, kend, h, a);
-            if (KCB) small_load_k(b_col, kc, h, b);
-            else small_load_x<false>(rsrc_b, b_lane, p.b_rs, kc, kend, h, b);
-        } else {
-            small_load_x<true>(rsrc_a, a_lane, p.a_cs, kc, kend, h, a);
-            small_load_x<true>(rsrc_b, b_lane, p.b_rs, kc, kend, h, b);
+        for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+        float a0[16], b0[16], a1[16], b1[16];
+        const auto load = [&](int64_t kc, float (&a)[16], float (&b)[16]) __attribute__((always_inline)) {
+            if (kc + kSmallChunk <= kend) {  // the same for the whole wave
+                if (KCA) small_load_k(a_row, kc, h, a);
+                else small_load_x<false>(rsrc_a, a_lane, a_cs, kc, kend, h, a);
+                if (KCB) small_load_k(b_col, kc, h, b);
+                else small_load_x<false>(rsrc_b, b_lane, b_rs, kc, kend, h, b);
+            } else {
+                small_load_x<true>(rsrc_a, a_lane, a_cs, kc, kend, h, a);
+                small_load_x<true>(rsrc_b, b_lane, b_rs, kc, kend, h, b);
+            }
+        };
+        const auto multiply = [&](const float (&a)[16], const float (&b)[16]) __attribute__((always_inline)) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[i], acc, 0, 0, 0);
+        };
+        if (kbeg < kend) {
+            int64_t k = kbeg;
+            load(k, a0, b0);
+            while (true) {
+                if (k + kSmallChunk < kend) load(k + kSmallChunk, a1, b1);
+                multiply(a0, b0);
+                k += kSmallChunk;
+                if (k >= kend) break;
+                if (k + kSmallChunk < kend) load(k + kSmallChunk, a0, b0);
+                multiply(a1, b1);
+                k += kSmallChunk;
+                if (k >= kend) break;
+            }
         }
-    };
-    const auto multiply = [&](const float (&a)[16], const float (&b)[16]) __attribute__((always_inline)) {
+        // accumulator register v of lane (r, h) is C[8 (v/4) + 4 h + v%4][r] of the tile
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[i], acc, 0, 0, 0);
+        for (int v = 0; v < 16; ++v) slot[(8 * (v / 4) + 4 * h + (v % 4)) * kSmallTile + r] = acc[v];
     };
-    if (kbeg < kend) {
-        int64_t k = kbeg;
-        load(k, a0, b0);
-        while (true) {
-            if (k + kSmallChunk < kend) load(k + kSmallChunk, a1, b1);
-            multiply(a0, b0);
-            k += kSmallChunk;
-            if (k >= kend) break;
-            if (k + kSmallChunk < kend) load(k + kSmallChunk, a0, b0);
-            multiply(a1, b1);
-            k += kSmallChunk;
-            if (k >= kend) break;
-        }
-    }
-    // accumulator register v of lane (r, h) is C[8 (v/4) + 4 h + v%4][r] of the tile
-#pragma unroll
-    for (int v = 0; v < 16; ++v) part[wave][(8 * (v / 4) + 4 * h + (v % 4)) * kSmallTile + r] = acc[v];
+    if (wave < p.splits)
+        contract(static_cast<const float *>(p.A) + batch * p.a_bs, static_cast<const float *>(p.B) + batch * p.b_bs, p.a_rs, p.a_cs,
+                 p.b_rs, p.b_cs, p.K, p.k_per_split, p.a_span_bytes, p.b_span_bytes, part[wave]);
+    // A second product of the same shape (the other cotangent of a state that two consumers read) is contracted by the
+    // same block into slots of its own: the sum below is then what two launches, the second with beta = 1, would give.
+    if (p.A2 != nullptr && wave < p.splits2)
+        contract(static_cast<const float *>(p.A2), static_cast<const float *>(p.B2), p.a2_rs, p.a2_cs, p.b2_rs, p.b2_cs, p.K2,
+                 p.k_per_split2, p.a2_span_bytes, p.b2_span_bytes, part[p.splits + wave]);
     __syncthreads();
 
     const float alpha = static_cast<float>(p.alpha), beta = static_cast<float>(p.beta);
@@ -851,10 +867,16 @@ __global__ __launch_bounds__(kSmallMaxWaves * 64) void gemm_block_split(const Ge
         const int64_t row = m0 + e / kSmallTile, col = n0 + e % kSmallTile;
         if (row >= p.M || col >= p.N) continue;
         float t = part[0][e];
-        for (int w = 1; w < n_waves; ++w) t += part[w][e];
+        for (int w = 1; w < p.splits; ++w) t += part[w][e];
         float *C = static_cast<float *>(p.C) + batch * p.c_bs + row * p.ldc + col;
         if (p.alpha != 1.0) t = alpha * t;
         if (p.beta != 0.0) t = t + beta * *C;
+        if (p.A2 != nullptr) {  // (what the first launch would have stored, then the second's sum plus 1 * that)
+            const float first = t;
+            t = part[p.splits][e];
+            for (int w = 1; w < p.splits2; ++w) t += part[p.splits + w][e];
+            t = t + 1.0f * first;
+        }
         const float bias = has_bias ? p.epi_bias[col] : 0.f;
         if (p.epi == 2) t = epi_tanh_vjp(t, p.epi_x[row * p.epi_x_ld + col], bias, has_bias);
         *C = t;
@@ -884,9 +906,19 @@ static int launch_block_split(GemmParams p, int64_t batch, hipStream_t s) {
     p.b_span_bytes = static_cast<uint32_t>(((p.K - 1) * p.b_rs + (p.N - 1) * p.b_cs + 1) * 4);
     const bool kca = p.a_cs == 1, kcb = p.b_rs == 1;
     set_kernel_name("gemm_block_split<f32,32,32,%s%s%s>[%lldx%lldx%lld]", kca ? "k" : "x", kcb ? "k" : "x",
-                    p.epi == 1 ? ",+bias,tanh" : (p.epi == 2 ? ",tanh_vjp" : ""), (long long)p.M, (long long)p.N, (long long)p.K);
-    const dim3 grid((unsigned)(tm * tn), (unsigned)batch), block(waves * 64);
-    const size_t lds = static_cast<size_t>(waves) * kSmallTile * kSmallTile * sizeof(float);
+                    p.epi == 1 ? ",+bias,tanh" : (p.epi == 2 ? (p.A2 != nullptr ? ",two products,tanh_vjp" : ",tanh_vjp") : ""),
+                    (long long)p.M, (long long)p.N, (long long)(p.K + (p.A2 != nullptr ? p.K2 : 0)));
+    int block_waves = waves;
+    if (p.A2 != nullptr) {  // the second product of a pair: slices and extents of its own, the same block
+        const int waves2 = static_cast<int>(std::min<int64_t>(kSmallMaxWaves, ceil_div(p.K2, kSmallChunk)));
+        p.splits2 = waves2;
+        p.k_per_split2 = ceil_div(ceil_div(p.K2, waves2), kSmallChunk) * kSmallChunk;
+        p.a2_span_bytes = static_cast<uint32_t>(((p.M - 1) * p.a2_rs + (p.K2 - 1) * p.a2_cs + 1) * 4);
+        p.b2_span_bytes = static_cast<uint32_t>(((p.K2 - 1) * p.b2_rs + (p.N - 1) * p.b2_cs + 1) * 4);
+        block_waves = std::max(waves, waves2);
+    }
+    const dim3 grid((unsigned)(tm * tn), (unsigned)batch), block(block_waves * 64);
+    const size_t lds = static_cast<size_t>(waves + (p.A2 != nullptr ? p.splits2 : 0)) * kSmallTile * kSmallTile * sizeof(float);
     if (kca && kcb) hipLaunchKernelGGL((gemm_block_split<true, true>), grid, block, lds, s, p);
     else if (kca) hipLaunchKernelGGL((gemm_block_split<true, false>), grid, block, lds, s, p);
     else if (kcb) hipLaunchKernelGGL((gemm_block_split<false, true>), grid, block, lds, s, p);
@@ -1217,6 +1249,25 @@ extern "C" int agmi_gemm_fused(int dtype, int64_t M, int64_t N, int64_t K, const
     p.epi_ld = e->out_ld;
     p.epi_x = static_cast<const float *>(e->x);
     p.epi_x_ld = e->x_ld;
+    if (e->a2 != nullptr || e->b2 != nullptr) {
+        // Two products of one shape under one rule, in one launch, exactly when each alone would be cut over the waves
+        // of a block in the same way: the launch then gives what the two launches (the second adding to the first)
+        // give, bit for bit.  Anything else is the caller's to run one after the other.
+        GemmParams q = p;
+        q.A = e->a2; q.B = e->b2; q.K = e->k2;
+        q.a_rs = e->a2_rs; q.a_cs = e->a2_cs; q.b_rs = e->b2_rs; q.b_cs = e->b2_cs;
+        if (!e->a2 || !e->b2 || e->k2 <= 0 || e->kind != AGMI_EPILOGUE_TANH_VJP || e->beta != 0.0) {
+            set_error("gemm_fused: a second product needs both operands, the tanh rule and beta = 0");
+            return AGMI_ERR_ARG;
+        }
+        if (!wants_block_split(p, 1) || !wants_block_split(q, 1) || (p.a_cs == 1) != (q.a_cs == 1) || (p.b_rs == 1) != (q.b_rs == 1)) {
+            set_error("gemm_fused: the two products are not both cut inside a block, or differ in which operand is contiguous along k");
+            return AGMI_ERR_UNSUPPORTED;
+        }
+        p.A2 = e->a2; p.B2 = e->b2; p.K2 = e->k2;
+        p.a2_rs = e->a2_rs; p.a2_cs = e->a2_cs; p.b2_rs = e->b2_rs; p.b2_cs = e->b2_cs;
+        return launch_block_split(p, 1, as_stream(stream));
+    }
     if (wants_block_split(p, 1)) return launch_block_split(p, 1, as_stream(stream));
     const int rc = launch_direct(p, 1, as_stream(stream), workspace, workspace_bytes);
     if (rc == 1) {

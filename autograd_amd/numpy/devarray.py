@@ -382,6 +382,13 @@ class PendingProduct(DevArray):
                 or max(last_left.numel(), last_right.numel(), M * N) >= 1 << 28 or last_left.stride(0) < 0 or last_left.stride(1) < 0 \
                 or last_right.stride(0) < 0 or last_right.stride(1) < 0 or (K > 4096 and -(-M // 64) * -(-N // 64) < 128):
             return False
+        if len(terms) == 2:
+            # two products of one shape: one launch when each would be cut over the waves of a block (the kernel then
+            # gives the two launches' bits); refused for anything else, and nothing has run
+            first_left, first_right = terms[0]
+            if first_left.shape[1] and _lib.gemm_fused(code, first_left, first_right, out, _lib.EPILOGUE_TANH_VJP, bias=bias, x=x,
+                                                       second=(last_left, last_right)):
+                return True
         for k, (l, r) in enumerate(terms[:-1]):
             gemm2d(l, r, self.dtype, out=out, beta=1.0 if k else 0.0)
         if not _lib.gemm_fused(code, last_left, last_right, out, _lib.EPILOGUE_TANH_VJP, bias=bias, x=x, beta=1.0):

@@ -391,6 +391,16 @@ typedef struct agmi_gemm_epilogue {
     const void *x;     /* TANH_VJP: [M][N] with leading dimension x_ld */
     int64_t x_ld;
     double beta;       /* 0: C is only written */
+    /* TANH_VJP with beta = 0: a second product a2 (M x k2) . b2 (k2 x N) added before the rule (the state of a
+     * recurrent net has two readers, examples/rnn.py:37-50: its cotangent is the sum of two G . W^T products,
+     * core.py:185-205).  Taken only when each product alone would run on the kernel that cuts K over the waves of one
+     * block (AGMI_ERR_UNSUPPORTED otherwise: run them one after the other, the second with beta = 1); the result is
+     * bit for bit that of those two launches.  NULL: one product. */
+    const void *a2;
+    int64_t a2_rs, a2_cs;
+    const void *b2;
+    int64_t b2_rs, b2_cs;
+    int64_t k2;
 } agmi_gemm_epilogue;
 int agmi_gemm_fused(int dtype, int64_t M, int64_t N, int64_t K,
                     const void *A, int64_t a_rs, int64_t a_cs, const void *B, int64_t b_rs, int64_t b_cs,

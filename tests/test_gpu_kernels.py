@@ -1587,6 +1587,47 @@ def test_gemm_epilogues_equal_the_separate_kernels(dnp, M, N, K):
             assert onp.array_equal(out.cpu().numpy(), want_sum)
 
 
+@pytest.mark.parametrize("M,N,K1,K2,layout", [(256, 512, 512, 128, "kk"), (256, 512, 641, 128, "kx"), (64, 96, 130, 257, "xk"),
+                                             (33, 70, 128, 4000, "xx"), (256, 512, 128, 128, "kk")])
+def test_two_products_under_one_tanh_rule_in_one_launch_equal_the_two_launches(dnp, M, N, K1, K2, layout):
+    """``agmi_gemm_fused`` with a second product: ``(A1.B1 + A2.B2) / cosh(x + bias)**2`` from ONE launch is, bit for bit,
+    ``A1.B1`` written out followed by ``A2.B2`` added to it (beta = 1) under the rule (the cotangent of a recurrent net's
+    state, examples/rnn.py:37-50: two ``G . W^T`` products, core.py:185-205, then numpy_vjps.py:178); pairs the kernel
+    does not take are refused and nothing runs."""
+    from autograd_amd import _lib
+
+    rs = onp.random.RandomState(M + K1 + K2)
+    f32 = onp.dtype(F32)
+    code = _lib.DTYPE_CODE[f32]
+
+    def operand(rows, cols, contiguous_k_is_cols):
+        if contiguous_k_is_cols:
+            return P(dnp, rs.randn(rows, cols).astype(F32))._t
+        return P(dnp, rs.randn(cols, rows).astype(F32))._t.t()
+
+    ka, kb = layout[0] == "k", layout[1] == "k"
+    A1, A2 = operand(M, K1, ka), operand(M, K2, ka)          # K along the columns of A: contiguous when `ka`
+    B1, B2 = operand(K1, N, not kb), operand(K2, N, not kb)  # K along the rows of B: contiguous when `kb`
+    x = P(dnp, rs.randn(M, N).astype(F32))._t
+    bias = P(dnp, rs.randn(N).astype(F32))._t
+    one = _lib.empty((M, N), f32)
+    assert _lib.gemm_fused(code, A1, B1, one, _lib.EPILOGUE_TANH_VJP, bias=bias, x=x, second=(A2, B2))
+    two = _lib.empty((M, N), f32)
+    _lib.gemm(code, 1, M, N, K1, 1.0, A1, A1.stride(0), A1.stride(1), 0, B1, B1.stride(0), B1.stride(1), 0, 0.0, two, N, 0)
+    assert _lib.gemm_fused(code, A2, B2, two, _lib.EPILOGUE_TANH_VJP, bias=bias, x=x, beta=1.0)
+    assert onp.array_equal(one.cpu().numpy(), two.cpu().numpy())
+    want = (A1.cpu().numpy().astype(F64) @ B1.cpu().numpy() + A2.cpu().numpy().astype(F64) @ B2.cpu().numpy()) \
+        / onp.cosh(x.cpu().numpy().astype(F64) + bias.cpu().numpy()) ** 2
+    close(one.cpu().numpy(), want.astype(F32), RT[F32] * max(1.0, onp.sqrt(K1 + K2) / 8))
+    # refused: a product too short to be cut, operands that differ in which one is contiguous along k, a large output
+    short = operand(M, 64, ka)
+    assert not _lib.gemm_fused(code, A1, B1, one, _lib.EPILOGUE_TANH_VJP, bias=bias, x=x, second=(short, operand(64, N, not kb)))
+    assert not _lib.gemm_fused(code, A1, B1, one, _lib.EPILOGUE_TANH_VJP, bias=bias, x=x, second=(operand(M, K2, not ka), B2))
+    big = P(dnp, rs.randn(1024, 256).astype(F32))._t
+    assert not _lib.gemm_fused(code, big, P(dnp, rs.randn(256, 1024).astype(F32))._t, _lib.empty((1024, 1024), f32),
+                               _lib.EPILOGUE_TANH_VJP, x=P(dnp, rs.randn(1024, 1024).astype(F32))._t, second=(big, P(dnp, rs.randn(256, 1024).astype(F32))._t))
+
+
 def test_the_tanh_rule_over_a_sum_of_sliced_products_is_one_chain_of_contractions(dnp):
     """The state of a recurrent net is read by the next step and by the output head (examples/rnn.py:37-50): its cotangent is
     the sum of two `G . W^T` products, of each of which only the state's columns are wanted (the `hstack` rule slices
@@ -1613,13 +1654,14 @@ def test_the_tanh_rule_over_a_sum_of_sliced_products_is_one_chain_of_contraction
 
     names = []
     real_fused, real_gemm = _lib.gemm_fused, _lib.gemm
-    _lib.gemm_fused = lambda *a, **k: (names.append(("fused", k.get("beta", 0.0))), real_fused(*a, **k))[1]
+    _lib.gemm_fused = lambda *a, **k: (names.append(("fused", 1.0 if k.get("second") is not None else k.get("beta", 0.0))),
+                                       real_fused(*a, **k))[1]
     _lib.gemm = lambda *a, **k: (names.append(("gemm", a[2:5])), real_gemm(*a, **k))[1]
     try:
         got = ag.grad(f)(h0).numpy()
     finally:
         _lib.gemm_fused, _lib.gemm = real_fused, real_gemm
-    assert ("fused", 1.0) in names                                   # the rule of h1 ran on a sum of two products
+    assert ("fused", 1.0) in names                                   # the rule of h1 ran on a sum of two products (one launch, or two with beta = 1)
     assert ("gemm", (B_, H, H)) in names and ("gemm", (B_, I + H + 1, H)) not in names   # only the state's columns were contracted
     was, fusion.ENABLED = fusion.ENABLED, False
     try:
