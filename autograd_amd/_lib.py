@@ -119,7 +119,11 @@ class AgmiGemmEpilogue(ctypes.Structure):
     _fields_ = [("kind", ctypes.c_int32), ("bias", ctypes.c_void_p), ("out", ctypes.c_void_p), ("out_ld", ctypes.c_int64),
                 ("x", ctypes.c_void_p), ("x_ld", ctypes.c_int64), ("beta", ctypes.c_double),
                 ("a2", ctypes.c_void_p), ("a2_rs", ctypes.c_int64), ("a2_cs", ctypes.c_int64),
-                ("b2", ctypes.c_void_p), ("b2_rs", ctypes.c_int64), ("b2_cs", ctypes.c_int64), ("k2", ctypes.c_int64)]
+                ("b2", ctypes.c_void_p), ("b2_rs", ctypes.c_int64), ("b2_cs", ctypes.c_int64), ("k2", ctypes.c_int64),
+                ("with_a", ctypes.c_void_p), ("with_a_rs", ctypes.c_int64), ("with_a_cs", ctypes.c_int64),
+                ("with_b", ctypes.c_void_p), ("with_b_rs", ctypes.c_int64), ("with_b_cs", ctypes.c_int64),
+                ("with_c", ctypes.c_void_p), ("with_ldc", ctypes.c_int64), ("with_m", ctypes.c_int64),
+                ("with_n", ctypes.c_int64), ("with_k", ctypes.c_int64)]
 
 
 class AgmiLseCotangent(ctypes.Structure):
@@ -734,13 +738,14 @@ EPILOGUE_BIAS_TANH, EPILOGUE_TANH_VJP = 1, 2
 _epilogue = AgmiGemmEpilogue()
 
 
-def gemm_fused(code, A, B, C, kind, bias=None, out=None, x=None, beta=0.0, second=None):
+def gemm_fused(code, A, B, C, kind, bias=None, out=None, x=None, beta=0.0, second=None, beside=None):
     """``agmi_gemm_fused``: ``A @ B`` (2-d tensors, any strides; plus ``beta`` times what ``C`` holds) into the
     contiguous ``C`` with a dense layer's epilogue: ``out = tanh(C + bias)`` beside it, or
     ``C = (A @ B + beta * C) / cosh(x + bias)**2`` (``bias``: contiguous vector or None).  ``second``: a pair
     ``(A2, B2)`` whose product is added before the tanh rule, in the same launch (bit for bit what running ``A @ B``
-    into ``C`` and then ``A2 @ B2`` with ``beta = 1`` gives).  Returns False when the operands are outside what the
-    fused kernel covers."""
+    into ``C`` and then ``A2 @ B2`` with ``beta = 1`` gives).  ``beside``: ``(A3, B3, C3)``, an independent plain product
+    ``C3 = A3 @ B3`` computed by further blocks of the same launch.  Returns False when the operands are outside what
+    the fused kernel covers (nothing has run then)."""
     M, K = A.shape
     N = B.shape[1]
     e = _epilogue
@@ -759,6 +764,17 @@ def gemm_fused(code, A, B, C, kind, bias=None, out=None, x=None, beta=0.0, secon
         e.b2, e.b2_rs, e.b2_cs = B2.data_ptr(), B2.stride(0), B2.stride(1)
         e.k2 = A2.shape[1]
         flops += 2.0 * M * N * A2.shape[1]
+    nbytes = 0
+    if beside is None:
+        e.with_c = None
+    else:
+        A3, B3, C3 = beside
+        e.with_a, e.with_a_rs, e.with_a_cs = A3.data_ptr(), A3.stride(0), A3.stride(1)
+        e.with_b, e.with_b_rs, e.with_b_cs = B3.data_ptr(), B3.stride(0), B3.stride(1)
+        e.with_c, e.with_ldc = C3.data_ptr(), C3.stride(0)
+        e.with_m, e.with_n, e.with_k = A3.shape[0], B3.shape[1], A3.shape[1]
+        flops += 2.0 * A3.shape[0] * B3.shape[1] * A3.shape[1]
+        nbytes = (A3.numel() + B3.numel() + C3.numel()) * A3.element_size()
     ev = _TIMER.begin(("gemm",)) if _TIMER is not None else None
     rc = _LIB.agmi_gemm_fused(code, M, N, K, A.data_ptr(), A.stride(0), A.stride(1), B.data_ptr(), B.stride(0), B.stride(1),
                               C.data_ptr(), C.stride(0), ctypes.byref(e), _workspace().data_ptr(), _WORKSPACE_BYTES, _stream())
@@ -769,7 +785,7 @@ def gemm_fused(code, A, B, C, kind, bias=None, out=None, x=None, beta=0.0, secon
     if ev is not None:
         es = A.element_size()
         k_all = K + (second[0].shape[1] if second is not None else 0)
-        _TIMER.end(ev, ("gemm",), (M * k_all + k_all * N + 2 * M * N) * es, flops)
+        _TIMER.end(ev, ("gemm",), (M * k_all + k_all * N + 2 * M * N) * es + nbytes, flops)
     return True
 
 

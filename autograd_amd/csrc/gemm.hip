@@ -25,6 +25,8 @@
 // groups of kGroupM tile-rows, which keeps one XCD's A rows and B columns resident in its L2.
 #include <algorithm>
 
+#include <cstdio>
+
 #include "common.h"
 
 namespace agmi {
@@ -785,9 +787,9 @@ __device__ __forceinline__ void small_load_x(__amdgpu_buffer_rsrc_t rsrc, uint32
     }
 }
 
+// (the kernel's body: `bid` is the block's number among the blocks of the problem `p`, `batch` its matrix of the batch)
 template <bool KCA, bool KCB>
-__global__ __launch_bounds__(kSmallMaxWaves * 64) void gemm_block_split(const GemmParams p) {
-    extern __shared__ float part_lds[];  // [waves][32 * 32]
+__device__ __forceinline__ void block_split_tile(const GemmParams &p, const int64_t bid, const int64_t batch, float *part_lds) {
     float (*part)[kSmallTile * kSmallTile] = reinterpret_cast<float (*)[kSmallTile * kSmallTile]>(part_lds);
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // the same for the whole wave: offsets made of it are scalar
@@ -796,9 +798,9 @@ __global__ __launch_bounds__(kSmallMaxWaves * 64) void gemm_block_split(const Ge
     // tiles in column-major order (a few columns of tiles, every row), so its L2 fetches all of A but only its
     // columns of B, not both operands whole.
     const int64_t n_tiles = static_cast<int64_t>(p.tiles_m) * p.tiles_n;
-    const int64_t xcd = blockIdx.x % kXcds, turn = blockIdx.x / kXcds;
+    const int64_t xcd = bid % kXcds, turn = bid / kXcds;
     const int64_t tile = xcd * (n_tiles / kXcds) + min(xcd, n_tiles % kXcds) + turn;
-    const int64_t tile_m = tile % p.tiles_m, tile_n = tile / p.tiles_m, batch = blockIdx.y;
+    const int64_t tile_m = tile % p.tiles_m, tile_n = tile / p.tiles_m;
     const int64_t m0 = tile_m * kSmallTile, n0 = tile_n * kSmallTile;
     // One product's share of this wave: the K slice [wave * k_per_split, ...) of A . B into `slot` of the LDS array.
     const auto contract = [&](const float *A, const float *B, int64_t a_rs, int64_t a_cs, int64_t b_rs, int64_t b_cs, int64_t K,
@@ -884,6 +886,23 @@ __global__ __launch_bounds__(kSmallMaxWaves * 64) void gemm_block_split(const Ge
     }
 }
 
+template <bool KCA, bool KCB>
+__global__ __launch_bounds__(kSmallMaxWaves * 64) void gemm_block_split(const GemmParams p) {
+    extern __shared__ float part_lds[];  // [waves][32 * 32]
+    block_split_tile<KCA, KCB>(p, blockIdx.x, blockIdx.y, part_lds);
+}
+
+// Two independent problems in one launch: the first `blocks_p` blocks are the tiles of `p`, the others the tiles of `q`
+// (one matrix each).  Every block does exactly what it would do in a launch of its own problem.  For the contraction of
+// one time step of a recurrent net and the output head's contraction of the step before, which both wait for the same
+// state and not for each other (examples/rnn.py:37-50): one chain link instead of two.
+template <bool KCA, bool KCB>
+__global__ __launch_bounds__(kSmallMaxWaves * 64) void gemm_block_split_pair(const GemmParams p, const GemmParams q, const int blocks_p) {
+    extern __shared__ float part_lds[];
+    if (static_cast<int>(blockIdx.x) < blocks_p) block_split_tile<KCA, KCB>(p, blockIdx.x, 0, part_lds);
+    else block_split_tile<KCA, KCB>(q, static_cast<int64_t>(blockIdx.x) - blocks_p, 0, part_lds);
+}
+
 // Whether a float32 product goes to gemm_block_split: too few 64 x 64 tiles to fill the machine and a K long enough
 // to cut, but not so long that one block per 32 x 32 tile would be the slower way to cut it.
 static bool wants_block_split(const GemmParams &p, int64_t batch) {
@@ -894,20 +913,16 @@ static bool wants_block_split(const GemmParams &p, int64_t batch) {
     return addressable && tiles64 < 128 && p.K >= 128 && p.K <= 4096 && tiles32 <= 0x7fffffffLL && batch <= 65535;
 }
 
-static int launch_block_split(GemmParams p, int64_t batch, hipStream_t s) {
-    const int64_t tm = ceil_div(p.M, kSmallTile), tn = ceil_div(p.N, kSmallTile);
-    p.tiles_m = static_cast<int>(tm);
-    p.tiles_n = static_cast<int>(tn);
+// Tiles, slices and extents of a problem for gemm_block_split; returns the waves a block needs and, in *lds, its LDS bytes.
+static int plan_block_split(GemmParams &p, size_t *lds) {
+    p.tiles_m = static_cast<int>(ceil_div(p.M, kSmallTile));
+    p.tiles_n = static_cast<int>(ceil_div(p.N, kSmallTile));
     // whole chunks per wave (only the slice that holds the end of K has a partial one), as many waves as there are chunks
     const int waves = static_cast<int>(std::min<int64_t>(kSmallMaxWaves, ceil_div(p.K, kSmallChunk)));
     p.splits = waves;
     p.k_per_split = ceil_div(ceil_div(p.K, waves), kSmallChunk) * kSmallChunk;
     p.a_span_bytes = static_cast<uint32_t>(((p.M - 1) * p.a_rs + (p.K - 1) * p.a_cs + 1) * 4);
     p.b_span_bytes = static_cast<uint32_t>(((p.K - 1) * p.b_rs + (p.N - 1) * p.b_cs + 1) * 4);
-    const bool kca = p.a_cs == 1, kcb = p.b_rs == 1;
-    set_kernel_name("gemm_block_split<f32,32,32,%s%s%s>[%lldx%lldx%lld]", kca ? "k" : "x", kcb ? "k" : "x",
-                    p.epi == 1 ? ",+bias,tanh" : (p.epi == 2 ? (p.A2 != nullptr ? ",two products,tanh_vjp" : ",tanh_vjp") : ""),
-                    (long long)p.M, (long long)p.N, (long long)(p.K + (p.A2 != nullptr ? p.K2 : 0)));
     int block_waves = waves;
     if (p.A2 != nullptr) {  // the second product of a pair: slices and extents of its own, the same block
         const int waves2 = static_cast<int>(std::min<int64_t>(kSmallMaxWaves, ceil_div(p.K2, kSmallChunk)));
@@ -917,12 +932,48 @@ static int launch_block_split(GemmParams p, int64_t batch, hipStream_t s) {
         p.b2_span_bytes = static_cast<uint32_t>(((p.K2 - 1) * p.b2_rs + (p.N - 1) * p.b2_cs + 1) * 4);
         block_waves = std::max(waves, waves2);
     }
-    const dim3 grid((unsigned)(tm * tn), (unsigned)batch), block(block_waves * 64);
-    const size_t lds = static_cast<size_t>(waves + (p.A2 != nullptr ? p.splits2 : 0)) * kSmallTile * kSmallTile * sizeof(float);
+    *lds = static_cast<size_t>(waves + (p.A2 != nullptr ? p.splits2 : 0)) * kSmallTile * kSmallTile * sizeof(float);
+    return block_waves;
+}
+
+static void name_block_split(const GemmParams &p, char *text, size_t n) {
+    std::snprintf(text, n, "<f32,32,32,%s%s%s>[%lldx%lldx%lld]", p.a_cs == 1 ? "k" : "x", p.b_rs == 1 ? "k" : "x",
+                  p.epi == 1 ? ",+bias,tanh" : (p.epi == 2 ? (p.A2 != nullptr ? ",two products,tanh_vjp" : ",tanh_vjp") : ""),
+                  (long long)p.M, (long long)p.N, (long long)(p.K + (p.A2 != nullptr ? p.K2 : 0)));
+}
+
+static int launch_block_split(GemmParams p, int64_t batch, hipStream_t s) {
+    size_t lds = 0;
+    const int block_waves = plan_block_split(p, &lds);
+    const bool kca = p.a_cs == 1, kcb = p.b_rs == 1;
+    char name[160];
+    name_block_split(p, name, sizeof(name));
+    set_kernel_name("gemm_block_split%s", name);
+    const dim3 grid((unsigned)(static_cast<int64_t>(p.tiles_m) * p.tiles_n), (unsigned)batch), block(block_waves * 64);
     if (kca && kcb) hipLaunchKernelGGL((gemm_block_split<true, true>), grid, block, lds, s, p);
     else if (kca) hipLaunchKernelGGL((gemm_block_split<true, false>), grid, block, lds, s, p);
     else if (kcb) hipLaunchKernelGGL((gemm_block_split<false, true>), grid, block, lds, s, p);
     else hipLaunchKernelGGL((gemm_block_split<false, false>), grid, block, lds, s, p);
+    return hip_check(hipGetLastError(), "gemm launch");
+}
+
+// Two problems that are each gemm_block_split's, with the same operands contiguous along k, in one launch.
+static int launch_block_split_pair(GemmParams p, GemmParams q, hipStream_t s) {
+    size_t lds_p = 0, lds_q = 0;
+    const int waves_p = plan_block_split(p, &lds_p), waves_q = plan_block_split(q, &lds_q);
+    const bool kca = p.a_cs == 1, kcb = p.b_rs == 1;
+    char name_p[160], name_q[160];
+    name_block_split(p, name_p, sizeof(name_p));
+    name_block_split(q, name_q, sizeof(name_q));
+    set_kernel_name("gemm_block_split_pair%s+%s", name_p, name_q);
+    const int64_t blocks_p = static_cast<int64_t>(p.tiles_m) * p.tiles_n, blocks_q = static_cast<int64_t>(q.tiles_m) * q.tiles_n;
+    const dim3 grid((unsigned)(blocks_p + blocks_q)), block(std::max(waves_p, waves_q) * 64);
+    const size_t lds = std::max(lds_p, lds_q);
+    const int bp = static_cast<int>(blocks_p);
+    if (kca && kcb) hipLaunchKernelGGL((gemm_block_split_pair<true, true>), grid, block, lds, s, p, q, bp);
+    else if (kca) hipLaunchKernelGGL((gemm_block_split_pair<true, false>), grid, block, lds, s, p, q, bp);
+    else if (kcb) hipLaunchKernelGGL((gemm_block_split_pair<false, true>), grid, block, lds, s, p, q, bp);
+    else hipLaunchKernelGGL((gemm_block_split_pair<false, false>), grid, block, lds, s, p, q, bp);
     return hip_check(hipGetLastError(), "gemm launch");
 }
 
@@ -1249,6 +1300,24 @@ extern "C" int agmi_gemm_fused(int dtype, int64_t M, int64_t N, int64_t K, const
     p.epi_ld = e->out_ld;
     p.epi_x = static_cast<const float *>(e->x);
     p.epi_x_ld = e->x_ld;
+    if (e->with_c != nullptr) {
+        // An independent plain product computed by further blocks of the same launch (no second product then).
+        GemmParams q = {};
+        q.A = e->with_a; q.B = e->with_b; q.C = e->with_c;
+        q.M = e->with_m; q.N = e->with_n; q.K = e->with_k;
+        q.a_rs = e->with_a_rs; q.a_cs = e->with_a_cs; q.b_rs = e->with_b_rs; q.b_cs = e->with_b_cs;
+        q.ldc = e->with_ldc;
+        q.alpha = 1.0; q.beta = 0.0;
+        if (!e->with_a || !e->with_b || q.M <= 0 || q.N <= 0 || q.K <= 0 || q.ldc < q.N || e->a2 != nullptr || e->b2 != nullptr) {
+            set_error("gemm_fused: the accompanying product needs its operands and extents, and excludes a second product");
+            return AGMI_ERR_ARG;
+        }
+        if (!wants_block_split(p, 1) || !wants_block_split(q, 1) || (p.a_cs == 1) != (q.a_cs == 1) || (p.b_rs == 1) != (q.b_rs == 1)) {
+            set_error("gemm_fused: the two problems are not both cut inside a block, or differ in which operand is contiguous along k");
+            return AGMI_ERR_UNSUPPORTED;
+        }
+        return launch_block_split_pair(p, q, as_stream(stream));
+    }
     if (e->a2 != nullptr || e->b2 != nullptr) {
         // Two products of one shape under one rule, in one launch, exactly when each alone would be cut over the waves
         // of a block in the same way: the launch then gives what the two launches (the second adding to the first)

@@ -13,6 +13,7 @@ scalars are strong.
 
 import math
 import numbers
+import weakref
 
 import numpy as onp
 import torch
@@ -268,7 +269,7 @@ class PendingProduct(DevArray):
     ``DevArray``; the first such read computes the product and keeps it.
     """
 
-    __slots__ = ("_left", "_right", "_shape", "_out", "_more")
+    __slots__ = ("_left", "_right", "_shape", "_out", "_more", "__weakref__")
 
     def __init__(self, left, right, dtype):
         self._left, self._right = left, right
@@ -352,8 +353,21 @@ class PendingProduct(DevArray):
         if not self._shape[0] or not self._shape[1] or not self._left.shape[1] or self._more:
             return False
         out = self._buffer()
-        if not _lib.gemm_fused(_lib.DTYPE_CODE[self.dtype], self._left, self._right, out, _lib.EPILOGUE_BIAS_TANH, bias=bias,
-                               out=act_out):
+        code = _lib.DTYPE_CODE[self.dtype]
+        # Another forward product that has not run (the output head of the step before, which reads the state this
+        # layer reads): it waits for nothing this layer produces, so its tiles ride in this launch instead of
+        # being a link of their own in the chain of launches.  Refused unless both are the kernel's: nothing has run.
+        mate = _forward_mate(self)
+        if mate is not None:
+            mate_out = mate._buffer()
+            if _lib.gemm_fused(code, self._left, self._right, out, _lib.EPILOGUE_BIAS_TANH, bias=bias, out=act_out,
+                               beside=(mate._left, mate._right, mate_out)):
+                mate._t = mate_out
+                mate._left = mate._right = mate._out = mate._more = None
+                self._t = out
+                self._left = self._right = self._out = None
+                return True
+        if not _lib.gemm_fused(code, self._left, self._right, out, _lib.EPILOGUE_BIAS_TANH, bias=bias, out=act_out):
             return False
         self._t = out
         self._left = self._right = self._out = None
@@ -437,6 +451,31 @@ class PendingProduct(DevArray):
 
     def _settled(self):
         return DevArray(self._t, self.dtype)
+
+
+# the last few products that `dot` left pending (weakly held): candidates to ride in another layer's launch
+_FORWARD_PRODUCTS = []
+
+
+def note_forward_product(product):
+    """Remember a forward matrix product that has not run (see ``PendingProduct.with_activation``)."""
+    if len(_FORWARD_PRODUCTS) >= 3:
+        del _FORWARD_PRODUCTS[0]
+    _FORWARD_PRODUCTS.append(weakref.ref(product))
+    return product
+
+
+def _forward_mate(product):
+    for k in range(len(_FORWARD_PRODUCTS) - 1, -1, -1):
+        other = _FORWARD_PRODUCTS[k]()
+        if other is None or other.computed():
+            del _FORWARD_PRODUCTS[k]
+            continue
+        if other is not product and not other._more and other.dtype == product.dtype and other._shape[0] and other._shape[1] \
+                and other._left.shape[1]:
+            del _FORWARD_PRODUCTS[k]
+            return other
+    return None
 
 
 class LseCotangent(DevArray):

@@ -1311,7 +1311,7 @@ def _dot_raw(a, b):
     if a.ndim == 2 and b.ndim == 2:
         if D._fusion.ENABLED and a.shape[0] and b.shape[1]:
             # left pending: a bias and an activation that follow can then ride in the contraction's epilogue
-            return D.PendingProduct(a._t, b._t, dt)
+            return D.note_forward_product(D.PendingProduct(a._t, b._t, dt))
         return DevArray(D.gemm2d(a._t, b._t, dt), dt)
     # numpy.dot on higher ranks: sum over last axis of a and second-to-last of b
     return _tensordot_raw(a, b, axes=((a.ndim - 1,), (b.ndim - 2,)))

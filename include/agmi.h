@@ -401,6 +401,18 @@ typedef struct agmi_gemm_epilogue {
     const void *b2;
     int64_t b2_rs, b2_cs;
     int64_t k2;
+    /* An independent product with_c (with_m x with_n, leading dimension with_ldc) = with_a . with_b computed by further
+     * blocks of the same launch: a second problem that waits for the same inputs and not for this one (the output
+     * head of a recurrent net's previous step beside the recurrence of this step, examples/rnn.py:37-50) rides
+     * along instead of being a link of the chain of launches.  Taken only when both problems would run on the kernel
+     * that cuts K over the waves of one block (AGMI_ERR_UNSUPPORTED otherwise, nothing launched); each result is bit
+     * for bit that of its own launch.  with_c NULL: none.  Excludes a2 / b2. */
+    const void *with_a;
+    int64_t with_a_rs, with_a_cs;
+    const void *with_b;
+    int64_t with_b_rs, with_b_cs;
+    void *with_c;
+    int64_t with_ldc, with_m, with_n, with_k;
 } agmi_gemm_epilogue;
 int agmi_gemm_fused(int dtype, int64_t M, int64_t N, int64_t K,
                     const void *A, int64_t a_rs, int64_t a_cs, const void *B, int64_t b_rs, int64_t b_cs,

@@ -1628,6 +1628,54 @@ def test_two_products_under_one_tanh_rule_in_one_launch_equal_the_two_launches(d
                                _lib.EPILOGUE_TANH_VJP, x=P(dnp, rs.randn(1024, 1024).astype(F32))._t, second=(big, P(dnp, rs.randn(256, 1024).astype(F32))._t))
 
 
+def test_an_independent_product_rides_in_a_dense_layers_launch(dnp):
+    """``agmi_gemm_fused`` with an accompanying problem: the tiles of a second, independent product are computed by
+    further blocks of a dense layer's launch, each result bit for bit that of its own launch (the output head of a
+    recurrent net's previous step beside this step's recurrence, examples/rnn.py:37-50); and the host side: a forward
+    product left pending is taken along by the next dense layer, once, and read back as computed."""
+    from autograd_amd import _lib
+    from autograd_amd.numpy import devarray as D
+
+    rs = onp.random.RandomState(41)
+    f32 = onp.dtype(F32)
+    code = _lib.DTYPE_CODE[f32]
+    for (M, N, K), (M2, N2, K2) in (((256, 512, 641), (256, 128, 513)), ((64, 96, 300), (200, 33, 130)), ((33, 40, 128), (70, 257, 4000))):
+        A, B = P(dnp, rs.randn(M, K).astype(F32))._t, P(dnp, (0.1 * rs.randn(K, N)).astype(F32))._t
+        A2, B2 = P(dnp, rs.randn(M2, K2).astype(F32))._t, P(dnp, (0.1 * rs.randn(K2, N2)).astype(F32))._t
+        bias = P(dnp, rs.randn(N).astype(F32))._t
+        c1, t1, c2 = _lib.empty((M, N), f32), _lib.empty((M, N), f32), _lib.empty((M2, N2), f32)
+        assert _lib.gemm_fused(code, A, B, c1, _lib.EPILOGUE_BIAS_TANH, bias=bias, out=t1, beside=(A2, B2, c2))
+        d1, u1, d2 = _lib.empty((M, N), f32), _lib.empty((M, N), f32), _lib.empty((M2, N2), f32)
+        assert _lib.gemm_fused(code, A, B, d1, _lib.EPILOGUE_BIAS_TANH, bias=bias, out=u1)
+        _lib.gemm(code, 1, M2, N2, K2, 1.0, A2, A2.stride(0), A2.stride(1), 0, B2, B2.stride(0), B2.stride(1), 0, 0.0, d2, N2, 0)
+        for got, want in ((c1, d1), (t1, u1), (c2, d2)):
+            assert onp.array_equal(got.cpu().numpy(), want.cpu().numpy())
+        close(c2.cpu().numpy(), (A2.cpu().numpy().astype(F64) @ B2.cpu().numpy()).astype(F32), RT[F32] * max(1.0, onp.sqrt(K2) / 8))
+    # refused (nothing runs): a companion that is not the kernel's (a large output), or contiguous the other way round
+    big_a, big_b = P(dnp, rs.randn(1024, 256).astype(F32))._t, P(dnp, rs.randn(256, 1024).astype(F32))._t
+    assert not _lib.gemm_fused(code, A, B, c1, _lib.EPILOGUE_BIAS_TANH, bias=bias, out=t1, beside=(big_a, big_b, _lib.empty((1024, 1024), f32)))
+    At = P(dnp, rs.randn(K2, M2).astype(F32))._t.t()
+    assert not _lib.gemm_fused(code, A, B, c1, _lib.EPILOGUE_BIAS_TANH, bias=bias, out=t1, beside=(At, B2, c2))
+    # through the namespace: head = dot(h, Wp) stays pending and is computed by the launch of the next tanh(dot(...))
+    H, Wp = P(dnp, rs.randn(256, 513).astype(F32)), P(dnp, (0.1 * rs.randn(513, 128)).astype(F32))
+    X, Wc = P(dnp, rs.randn(256, 641).astype(F32)), P(dnp, (0.1 * rs.randn(641, 512)).astype(F32))
+    calls = []
+    real = _lib.gemm_fused
+    _lib.gemm_fused = lambda *a, **k: (calls.append(k.get("beside") is not None), real(*a, **k))[1]
+    try:
+        head = dnp.dot(H, Wp)
+        assert type(head) is D.PendingProduct and not head.computed()
+        state = dnp.tanh(dnp.dot(X, Wc)).numpy()
+        assert calls == [True] and head.computed()
+        got_head = head.numpy()
+        again = dnp.tanh(dnp.dot(X, Wc)).numpy()                   # nothing pending now: a launch of its own
+        assert calls == [True, False]
+    finally:
+        _lib.gemm_fused = real
+    assert onp.array_equal(again, state)
+    assert onp.array_equal(got_head, D.gemm2d(H._t, Wp._t, f32).cpu().numpy())
+
+
 def test_the_tanh_rule_over_a_sum_of_sliced_products_is_one_chain_of_contractions(dnp):
     """The state of a recurrent net is read by the next step and by the output head (examples/rnn.py:37-50): its cotangent is
     the sum of two `G . W^T` products, of each of which only the state's columns are wanted (the `hstack` rule slices
