@@ -461,18 +461,21 @@ def note_forward_product(product):
     """Remember a forward matrix product that has not run (see ``PendingProduct.with_activation``)."""
     if len(_FORWARD_PRODUCTS) >= 3:
         del _FORWARD_PRODUCTS[0]
-    _FORWARD_PRODUCTS.append(weakref.ref(product))
+    _FORWARD_PRODUCTS.append((weakref.ref(product), _lib.CAPTURING))
     return product
 
 
 def _forward_mate(product):
     for k in range(len(_FORWARD_PRODUCTS) - 1, -1, -1):
-        other = _FORWARD_PRODUCTS[k]()
+        ref, while_recording = _FORWARD_PRODUCTS[k]
+        other = ref()
         if other is None or other.computed():
             del _FORWARD_PRODUCTS[k]
             continue
-        if other is not product and not other._more and other.dtype == product.dtype and other._shape[0] and other._shape[1] \
-                and other._left.shape[1]:
+        # (a product from outside a graph that is being recorded is not taken into it: the recorded launch runs at the
+        # replays, and whoever reads the product outside would find a buffer that nothing has written yet)
+        if other is not product and while_recording == _lib.CAPTURING and not other._more and other.dtype == product.dtype \
+                and other._shape[0] and other._shape[1] and other._left.shape[1]:
             del _FORWARD_PRODUCTS[k]
             return other
     return None

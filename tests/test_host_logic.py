@@ -429,6 +429,35 @@ def test_pending_row_sums_broadcast_over_their_rows_join_the_chain():
         fusion.ENABLED = was
 
 
+def test_forward_products_left_pending_are_offered_once_and_not_across_a_recording(monkeypatch):
+    """``devarray.note_forward_product`` / ``_forward_mate``: the newest product that has not run is offered to the next
+    dense layer's launch, once; products that have run, have died, or were made on the other side of a graph recording
+    are not."""
+    import gc
+
+    f64 = onp.dtype("float64")
+    monkeypatch.setattr(D, "_FORWARD_PRODUCTS", [])
+    mk = lambda: D.PendingProduct(torch.zeros((4, 6), dtype=torch.float64), torch.zeros((6, 5), dtype=torch.float64), f64)  # noqa: E731
+    a, b, layer = D.note_forward_product(mk()), D.note_forward_product(mk()), D.note_forward_product(mk())
+    assert D._forward_mate(layer) is b            # the newest other one
+    assert D._forward_mate(layer) is a            # b is offered once
+    assert D._forward_mate(layer) is None
+    c = D.note_forward_product(mk())
+    c._left = None                                # it has run
+    assert c.computed() and D._forward_mate(layer) is None
+    d = D.note_forward_product(mk())
+    del d
+    gc.collect()
+    assert D._forward_mate(layer) is None         # it has died
+    e = D.note_forward_product(mk())
+    monkeypatch.setattr(D._lib, "CAPTURING", True)
+    assert D._forward_mate(layer) is None         # made outside the recording that is now running
+    inside = D.note_forward_product(mk())
+    assert D._forward_mate(layer) is inside
+    monkeypatch.setattr(D._lib, "CAPTURING", False)
+    assert D._forward_mate(layer) is e
+
+
 def test_slices_of_a_pending_product_stay_products():
     """``wrapper._part_of_product``: rows and columns of a product that has not run are taken from its factors when the
     slice keeps at least half of each axis; anything else is left to the ordinary view of the whole product."""
